@@ -1,0 +1,271 @@
+// TEST INFRASTRUCTURE ONLY -- never linked into, imported by or shipped with the product.
+//
+// C-ABI shim over the *reference* CPU forward.  It is compiled by oracle/Makefile together with
+// the reference's own sources where they lie under /root/reference (nothing is copied) into
+// oracle/_ref/libmsnh_ref.so.  The shim only drives public reference entry points:
+//   NetBuilder::buildNetFromMsnhNet   (src/net/MsnhNetBuilder.cpp:68-622)
+//   NetBuilder::loadWeightsFromMsnhBin (src/net/MsnhNetBuilder.cpp:624-663)
+//   the layer loop of runClassify/runYolo (src/net/MsnhNetBuilder.cpp:686-728, 763-806),
+//   restated here only so that every layer's output can be captured the way the reference's own
+//   setSaveLayerOutput dump does (src/net/MsnhNetBuilder.cpp:704-720).
+#include <vector>
+#include <string>
+#include <cstring>
+#include <cstdio>
+#include <memory>
+#include <exception>
+#include <sstream>
+#include <iostream>
+#include <map>
+#include <algorithm>
+#include <chrono>
+
+#define private public      // NetBuilder::_netState has no getter; the capture loop needs the pools
+#include "Msnhnet/net/MsnhNetBuilder.h"
+#undef private
+
+using namespace Msnhnet;
+
+namespace {
+struct RefNet
+{
+    NetBuilder                        *nb = nullptr;
+    std::vector<std::vector<float>>    captured;     // per top-level layer output of the last run
+    std::vector<std::vector<YoloBox>>  boxes;        // finalOut of the last run (yolo nets)
+    std::string                        detail;
+    double                             lastWallMs = 0;
+};
+
+void setErr(char *err, int errLen, const std::string &msg)
+{
+    if(err && errLen > 0)
+    {
+        std::snprintf(err, static_cast<size_t>(errLen), "%s", msg.c_str());
+    }
+}
+}
+
+extern "C" {
+
+// scalarMode!=0: BaseLayer::supportAvx/supportFma=false, i.e. the scalar branches of the reference
+// (the AVX max-pool branch is wrong for stride-1 padded pools, src/layers/MsnhMaxPoolLayer.cpp:517-544).
+void *ref_create(int scalarMode)
+{
+    RefNet *r = new RefNet();
+    std::streambuf *old = std::cout.rdbuf(nullptr);     // silence the SIMD banner (MsnhBaseLayer.cpp:21-59)
+    r->nb = new NetBuilder();
+    std::cout.rdbuf(old);
+    if(scalarMode)
+    {
+        BaseLayer::supportAvx = false;
+        BaseLayer::supportFma = false;
+    }
+    return r;
+}
+
+void ref_destroy(void *h)
+{
+    RefNet *r = static_cast<RefNet*>(h);
+    if(!r) return;
+    delete r->nb;
+    delete r;
+}
+
+int ref_build(void *h, const char *msnhnetPath, char *err, int errLen)
+{
+    RefNet *r = static_cast<RefNet*>(h);
+    try
+    {
+        r->nb->buildNetFromMsnhNet(msnhnetPath);
+    }
+    catch(const Exception &e)
+    {
+        setErr(err, errLen, e.what());
+        return -1;
+    }
+    catch(const std::exception &e)
+    {
+        setErr(err, errLen, std::string("std: ") + e.what());
+        return -2;
+    }
+    return 0;
+}
+
+int ref_load(void *h, const char *msnhbinPath, char *err, int errLen)
+{
+    RefNet *r = static_cast<RefNet*>(h);
+    try
+    {
+        r->nb->loadWeightsFromMsnhBin(msnhbinPath);
+    }
+    catch(const Exception &e)
+    {
+        setErr(err, errLen, e.what());
+        return -1;
+    }
+    catch(const std::exception &e)
+    {
+        setErr(err, errLen, std::string("std: ") + e.what());
+        return -2;
+    }
+    return 0;
+}
+
+int ref_num_layers(void *h)
+{
+    RefNet *r = static_cast<RefNet*>(h);
+    return static_cast<int>(r->nb->getNet()->layers.size());
+}
+
+// info[0..9] = type, outH, outW, outC, outputNum, inputNum, numWeights, memReUse, batch, activation
+int ref_layer_info(void *h, int i, long long *info, char *name, int nameLen)
+{
+    RefNet *r = static_cast<RefNet*>(h);
+    Network *net = r->nb->getNet();
+    if(i < 0 || i >= static_cast<int>(net->layers.size())) return -1;
+    BaseLayer *l = net->layers[static_cast<size_t>(i)];
+    info[0] = static_cast<long long>(l->type());
+    info[1] = l->getOutHeight();
+    info[2] = l->getOutWidth();
+    info[3] = l->getOutChannel();
+    info[4] = l->getOutputNum();
+    info[5] = l->getInputNum();
+    info[6] = static_cast<long long>(l->getNumWeights());
+    info[7] = l->getMemReUse();
+    info[8] = l->getBatch();
+    info[9] = static_cast<long long>(l->getActivation());
+    setErr(name, nameLen, l->getLayerName());
+    return 0;
+}
+
+long long ref_layer_detail(void *h, char *dst, long long cap)
+{
+    RefNet *r = static_cast<RefNet*>(h);
+    r->detail = r->nb->getLayerDetail();
+    long long n = static_cast<long long>(r->detail.size());
+    if(dst && cap > 0)
+    {
+        long long c = std::min(n, cap - 1);
+        std::memcpy(dst, r->detail.data(), static_cast<size_t>(c));
+        dst[c] = 0;
+    }
+    return n;
+}
+
+// One batch-1 forward with the reference's own layer loop.  capture!=0 keeps every top-level layer's
+// output.  Returns 0, or -1 with the reference's exception text.
+int ref_run(void *h, const float *img, long long n, int capture, char *err, int errLen)
+{
+    RefNet *r = static_cast<RefNet*>(h);
+    NetBuilder *nb = r->nb;
+    Network *net = nb->getNet();
+    NetworkState *st = nb->_netState;
+    try
+    {
+        std::vector<float> in(img, img + n);
+        r->captured.clear();
+        r->boxes.clear();
+        st->input    = in.data();
+        st->inputNum = static_cast<int>(in.size());
+        if(net->layers[0]->getInputNum() != st->inputNum)
+        {
+            throw Exception(1, "input image size err. Needed :" + std::to_string(net->layers[0]->getInputNum()) + " given :" +
+                            std::to_string(in.size()), __FILE__, __LINE__, __FUNCTION__);
+        }
+        auto t0 = std::chrono::steady_clock::now();
+        for(size_t i = 0; i < net->layers.size(); ++i)
+        {
+            BaseLayer *l = net->layers[i];
+            l->forward(*st);
+            if(l->getMemReUse() == 0)
+            {
+                st->input = l->getOutput();
+            }
+            st->inputNum = l->getOutputNum();
+            if(capture)
+            {
+                const float *p = (l->getMemReUse() == 1) ? st->getInput() : st->input;
+                r->captured.emplace_back(p, p + st->inputNum);
+            }
+        }
+        auto t1 = std::chrono::steady_clock::now();
+        r->lastWallMs = std::chrono::duration<double, std::milli>(t1 - t0).count();
+        BaseLayer *last = net->layers.back();
+        if(last->type() == LayerType::YOLO_OUT)
+        {
+            r->boxes = reinterpret_cast<YoloOutLayer*>(last)->finalOut;
+        }
+        if(!capture)
+        {
+            const float *p = (last->getMemReUse() == 1) ? st->getInput() : st->input;
+            r->captured.assign(net->layers.size(), std::vector<float>());
+            r->captured.back().assign(p, p + st->inputNum);
+        }
+    }
+    catch(const Exception &e)
+    {
+        setErr(err, errLen, e.what());
+        return -1;
+    }
+    catch(const std::exception &e)
+    {
+        setErr(err, errLen, std::string("std: ") + e.what());
+        return -2;
+    }
+    return 0;
+}
+
+double ref_last_wall_ms(void *h)
+{
+    return static_cast<RefNet*>(h)->lastWallMs;
+}
+
+// The reference's own sum of per-layer forward times (src/net/MsnhNetBuilder.cpp:1159-1168), ms.
+float ref_inference_time(void *h)
+{
+    return static_cast<RefNet*>(h)->nb->getInferenceTime();
+}
+
+long long ref_layer_output(void *h, int i, float *dst, long long cap)
+{
+    RefNet *r = static_cast<RefNet*>(h);
+    if(i < 0 || i >= static_cast<int>(r->captured.size())) return -1;
+    const std::vector<float> &v = r->captured[static_cast<size_t>(i)];
+    long long n = static_cast<long long>(v.size());
+    if(dst)
+    {
+        std::memcpy(dst, v.data(), sizeof(float) * static_cast<size_t>(std::min(n, cap)));
+    }
+    return n;
+}
+
+// Boxes of image 0 of the last run: rows of 7 floats  x y w h conf bestClsConf bestClsIdx.
+long long ref_boxes(void *h, float *dst, long long capBoxes)
+{
+    RefNet *r = static_cast<RefNet*>(h);
+    if(r->boxes.empty()) return 0;
+    const std::vector<YoloBox> &b = r->boxes[0];
+    long long n = static_cast<long long>(b.size());
+    if(dst)
+    {
+        for(long long i = 0; i < std::min(n, capBoxes); ++i)
+        {
+            const YoloBox &q = b[static_cast<size_t>(i)];
+            float *o = dst + 7 * i;
+            o[0] = q.xywhBox.x; o[1] = q.xywhBox.y; o[2] = q.xywhBox.w; o[3] = q.xywhBox.h;
+            o[4] = q.conf; o[5] = q.bestClsConf; o[6] = static_cast<float>(q.bestClsIdx);
+        }
+    }
+    return n;
+}
+
+void ref_set_threads_note(int *ompMax)
+{
+#ifdef USE_OMP
+    *ompMax = OMP_THREAD;
+#else
+    *ompMax = 1;
+#endif
+}
+
+}

@@ -1,0 +1,126 @@
+"""ctypes binding of oracle/_ref/libmsnh_ref.so (the reference's own CPU forward; checker only)."""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+REF_SO = os.path.join(_HERE, "..", "oracle", "_ref", "libmsnh_ref.so")
+
+LAYER_TYPE = {0: "conv", 2: "connect", 3: "maxpool", 4: "localavgpool", 8: "route", 13: "batchnorm",
+              15: "yolo", 16: "yoloout", 18: "upsample", 20: "empty", 27: "resblock", 28: "res2block",
+              29: "concatblock", 30: "addblock"}
+
+
+def available() -> bool:
+    return os.path.exists(REF_SO)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        L = ctypes.CDLL(REF_SO)
+        vp, cp, ci, ll = ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_longlong
+        fp = ctypes.POINTER(ctypes.c_float)
+        L.ref_create.restype = vp
+        L.ref_create.argtypes = [ci]
+        L.ref_destroy.argtypes = [vp]
+        L.ref_build.argtypes = [vp, cp, cp, ci]
+        L.ref_load.argtypes = [vp, cp, cp, ci]
+        L.ref_num_layers.argtypes = [vp]
+        L.ref_layer_info.argtypes = [vp, ci, ctypes.POINTER(ll), cp, ci]
+        L.ref_layer_detail.argtypes = [vp, cp, ll]
+        L.ref_layer_detail.restype = ll
+        L.ref_run.argtypes = [vp, fp, ll, ci, cp, ci]
+        L.ref_last_wall_ms.argtypes = [vp]
+        L.ref_last_wall_ms.restype = ctypes.c_double
+        L.ref_inference_time.argtypes = [vp]
+        L.ref_inference_time.restype = ctypes.c_float
+        L.ref_layer_output.argtypes = [vp, ci, fp, ll]
+        L.ref_layer_output.restype = ll
+        L.ref_boxes.argtypes = [vp, fp, ll]
+        L.ref_boxes.restype = ll
+        _lib = L
+    return _lib
+
+
+class RefError(RuntimeError):
+    pass
+
+
+class RefNet:
+    """One reference NetBuilder.  scalar=True runs the scalar (non-AVX) branches, the parity oracle."""
+
+    def __init__(self, msnhnet, msnhbin=None, scalar=True):
+        self.L = lib()
+        self.h = self.L.ref_create(1 if scalar else 0)
+        err = ctypes.create_string_buffer(1024)
+        if self.L.ref_build(self.h, msnhnet.encode(), err, 1024) != 0:
+            raise RefError(err.value.decode())
+        if msnhbin is not None:
+            if self.L.ref_load(self.h, msnhbin.encode(), err, 1024) != 0:
+                raise RefError(err.value.decode())
+
+    def close(self):
+        if self.h:
+            self.L.ref_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def num_layers(self):
+        return self.L.ref_num_layers(self.h)
+
+    def layer_info(self, i):
+        info = (ctypes.c_longlong * 10)()
+        name = ctypes.create_string_buffer(64)
+        self.L.ref_layer_info(self.h, i, info, name, 64)
+        keys = ["type", "outH", "outW", "outC", "outputNum", "inputNum", "numWeights", "memReUse", "batch", "act"]
+        d = dict(zip(keys, [int(v) for v in info]))
+        d["type"] = LAYER_TYPE.get(d["type"], str(d["type"]))
+        return d
+
+    def layer_infos(self):
+        return [self.layer_info(i) for i in range(self.num_layers())]
+
+    def detail(self):
+        n = self.L.ref_layer_detail(self.h, None, 0)
+        buf = ctypes.create_string_buffer(n + 1)
+        self.L.ref_layer_detail(self.h, buf, n + 1)
+        return buf.value.decode(errors="replace")
+
+    def run(self, img, capture=True):
+        """img: one CHW float32 image.  Returns list of per-top-level-layer outputs (flat arrays)."""
+        x = np.ascontiguousarray(img, dtype=np.float32).ravel()
+        err = ctypes.create_string_buffer(1024)
+        rc = self.L.ref_run(self.h, x.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), x.size, 1 if capture else 0, err, 1024)
+        if rc != 0:
+            raise RefError(err.value.decode())
+        outs = []
+        for i in range(self.num_layers()):
+            n = self.L.ref_layer_output(self.h, i, None, 0)
+            a = np.empty(max(n, 0), np.float32)
+            if n > 0:
+                self.L.ref_layer_output(self.h, i, a.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), n)
+            outs.append(a)
+        return outs
+
+    def boxes(self):
+        n = self.L.ref_boxes(self.h, None, 0)
+        a = np.empty((n, 7), np.float32)
+        if n:
+            self.L.ref_boxes(self.h, a.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), n)
+        return a
+
+    def wall_ms(self):
+        return self.L.ref_last_wall_ms(self.h)
+
+    def inference_time_ms(self):
+        return float(self.L.ref_inference_time(self.h))
