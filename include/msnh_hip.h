@@ -1,0 +1,203 @@
+/*
+ * msnh_hip.h -- C ABI of the MI355X (gfx950) kernel library `libmsnh_hip.so`.
+ *
+ * This is the drop-in boundary of the convolutional hot path: everything Msnhnet's layers do on the
+ * device (its CUDA kernels, cuBLAS and cuDNN calls) is reached through the plain-C entry points below.
+ * No C++ or framework types cross it: pointers are raw device (or, where stated, host) addresses, sizes
+ * are ints, streams/events/graphs are opaque `void*` handles owned by this library.
+ *
+ * Conventions
+ *   - Every function returns 0 on success and a non-zero code on failure; it never exits the process
+ *     (the reference prints and calls exit(), src/config/MsnhnetCuda.cpp:18-56).  The text of the last
+ *     failure on the calling thread is returned by msnh_hip_last_error().
+ *   - Activations live on the device in NHWC ("channels-last") order: element (n,y,x,c) of a tensor is at
+ *     data[((n*H + y)*W + x)*ld + c], ld >= C being the pixel stride in elements.  ld > C lets a tensor be
+ *     a channel slice of a wider buffer, which is how route/concat layers are planned away.  The reference
+ *     keeps NCHW (src/layers/MsnhConvolutionalLayer.cpp:645-760); NCHW float32 remains the layout of
+ *     everything that enters or leaves the library (msnh_hip_nchw_to_nhwc / msnh_hip_nhwc_to_nchw).
+ *   - dtype is MSNH_F32 or MSNH_F16 (IEEE half).  Arithmetic is always accumulated in float32.
+ *   - Shapes are validated on the host before any launch; a shape the kernels cannot run is an error,
+ *     never an out-of-bounds access.
+ */
+#ifndef MSNH_HIP_H
+#define MSNH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *msnh_stream_t;   /* hipStream_t; NULL = the library's default stream */
+typedef void *msnh_event_t;    /* hipEvent_t */
+typedef void *msnh_graph_t;    /* instantiated hipGraphExec_t */
+
+enum msnh_dtype { MSNH_F32 = 0, MSNH_F16 = 1 };
+
+/* Same numeric values as the reference's ActivationType (include/Msnhnet/config/MsnhnetCfg.h:95-120). */
+enum msnh_act
+{
+    MSNH_ACT_LOGISTIC = 0,
+    MSNH_ACT_RELU     = 1,
+    MSNH_ACT_RELU6    = 2,
+    MSNH_ACT_LEAKY    = 8,
+    MSNH_ACT_SWISH    = 16,
+    MSNH_ACT_MISH     = 18,
+    MSNH_ACT_NONE     = 22
+};
+
+enum msnh_conv_algo
+{
+    MSNH_CONV_AUTO      = 0,   /* let the library choose */
+    MSNH_CONV_DIRECT    = 1,   /* one thread per output element; any shape; the fallback */
+    MSNH_CONV_IGEMM     = 2,   /* implicit GEMM on MFMA, LDS-staged tiles; needs (in_c/groups) % 8 == 0 (f16) or % 4 (f32) */
+    MSNH_CONV_DEPTHWISE = 3,   /* groups == in_c == out_c, bandwidth-bound direct kernel */
+    MSNH_CONV_WINOGRAD  = 4,   /* F(2x2,3x3): ksize 3, stride 1, dilation 1, groups 1 */
+    MSNH_CONV_STEM      = 5    /* in_c <= 4 first layer: reads NCHW float32 input directly (cast fused) */
+};
+
+/* ------------------------------------------------------------------------------------------------
+ * Runtime plumbing.  Replaces the reference's `Cuda` helper class (src/config/MsnhnetCuda.cpp:105-239:
+ * cudaSetDevice, getCudaStream, mallocCudaArray/makeCudaArray, pushCudaArray/pullCudaArray, freeCuda).
+ * ---------------------------------------------------------------------------------------------- */
+const char *msnh_hip_last_error(void);
+int msnh_hip_init(int device);                                  /* selects the device, creates the default stream */
+int msnh_hip_device_count(int *count);
+int msnh_hip_device_name(char *dst, int cap, int *cu_count, size_t *total_mem);
+int msnh_hip_malloc(void **dptr, size_t bytes);
+int msnh_hip_free(void *dptr);
+int msnh_hip_host_alloc(void **hptr, size_t bytes);             /* pinned host memory */
+int msnh_hip_host_free(void *hptr);
+int msnh_hip_memcpy_h2d(void *dst, const void *src, size_t bytes, msnh_stream_t s);
+int msnh_hip_memcpy_d2h(void *dst, const void *src, size_t bytes, msnh_stream_t s);
+int msnh_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, msnh_stream_t s);
+int msnh_hip_fill_zero(void *dst, size_t bytes, msnh_stream_t s); /* a fill kernel, safe under graph capture */
+int msnh_hip_stream_create(msnh_stream_t *s);
+int msnh_hip_stream_destroy(msnh_stream_t s);
+int msnh_hip_stream_sync(msnh_stream_t s);
+int msnh_hip_event_create(msnh_event_t *e);
+int msnh_hip_event_destroy(msnh_event_t e);
+int msnh_hip_event_record(msnh_event_t e, msnh_stream_t s);
+int msnh_hip_event_sync(msnh_event_t e);
+int msnh_hip_event_elapsed_ms(msnh_event_t start, msnh_event_t stop, float *ms);
+/* Stream capture into a replayable graph: every kernel launched on `s` between begin and end is
+ * recorded instead of run.  No counterpart in the reference (it launches kernel by kernel,
+ * src/net/MsnhNetBuilder.cpp:847). */
+int msnh_hip_graph_begin(msnh_stream_t s);
+int msnh_hip_graph_end(msnh_stream_t s, msnh_graph_t *g);
+int msnh_hip_graph_launch(msnh_graph_t g, msnh_stream_t s);
+int msnh_hip_graph_destroy(msnh_graph_t g);
+
+/* ------------------------------------------------------------------------------------------------
+ * Convolution.  Replaces ConvolutionalLayer::forwardGPU (src/layers/MsnhConvolutionalLayer.cpp:914-1183):
+ * cudnnConvolutionForward (:995-1015) or im2ColExKernel + cublasSgemm (src/core/cuda/MsnhGemmGPU.cu:6-55,
+ * 136-145), then convBnKernel (src/layers/cuda/MsnhConvolutionalLayerGPU.cu:6-24) or addBiasKernel
+ * (src/core/cuda/MsnhBlasGPU.cu:656-688), then activateArrayKernel (src/layers/cuda/MsnhActivationsGPU.cu),
+ * and -- when has_residual -- the axpy + activation of the enclosing Res/Res2/Add block
+ * (src/layers/MsnhResBlockLayer.cpp:261-262, 264-293), all in one launch:
+ *
+ *     v = act( acc * scale[oc] + shift[oc] )                     acc = cross-correlation, float32
+ *     if has_residual:  v = act2( v + res_mul * residual )
+ *     y = out_mul * v
+ *
+ * Batch-norm is supplied folded: scale = gamma/sqrt(var+eps), shift = beta - gamma*mean/sqrt(var+eps)
+ * (src/layers/MsnhConvolutionalLayer.cpp:811-815); plain bias is scale = 1 (or scale == NULL), shift = bias.
+ * res_mul / out_mul are exact power-of-two rescalings used to keep float16 activations in range.
+ * Output size must satisfy out = (in + 2*pad - (dilation*(ksize-1)+1))/stride + 1 (:388-398).
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct msnh_conv_desc
+{
+    int   dtype;        /* of x, w and residual */
+    int   out_dtype;    /* of y */
+    int   batch, in_h, in_w, in_c, in_ld;
+    int   out_c, out_h, out_w, out_ld;
+    int   ksize, stride, pad, dilation, groups;
+    int   act;          /* msnh_act of the conv layer itself */
+    float act_param;    /* leaky slope */
+    int   has_residual;
+    int   res_ld;
+    int   act2;         /* msnh_act applied after the residual add */
+    float act2_param;
+    float res_mul;
+    float out_mul;
+    int   algo;         /* msnh_conv_algo */
+} msnh_conv_desc;
+
+/* Which algorithm MSNH_CONV_AUTO resolves to for this shape (never AUTO).  Pure host function. */
+int msnh_hip_conv2d_select_algo(const msnh_conv_desc *d);
+/* Number of elements (of d->dtype) of the packed weight buffer for `algo`.  Pure host function. */
+size_t msnh_hip_conv2d_packed_weight_elems(const msnh_conv_desc *d, int algo);
+/* Host-side weight packing from the `.msnhbin` order w[out_c][in_c/groups][k][k] float32
+ * (src/layers/MsnhConvolutionalLayer.cpp:1255-1257) into the layout `algo` reads:
+ *   DIRECT / IGEMM : [out_c][k*k][in_c/groups], tap-major, channel fastest
+ *   DEPTHWISE      : [k*k][channels]
+ *   WINOGRAD       : [16][out_c][in_c]  = G g G^T per (oc,ic), G of F(2x2,3x3)
+ *   STEM           : [k*k*in_c][out_c] float32 regardless of dtype
+ * `packed` is host memory of msnh_hip_conv2d_packed_weight_elems() elements; upload it afterwards. */
+int msnh_hip_conv2d_pack_weights(const msnh_conv_desc *d, int algo, const float *oihw, void *packed);
+/* Scratch bytes `workspace` must provide for `algo` (0 for all but WINOGRAD). */
+size_t msnh_hip_conv2d_workspace_bytes(const msnh_conv_desc *d, int algo);
+/* x: NHWC d->dtype (STEM: NCHW float32); w: packed for the resolved algo; scale/shift: float32[out_c] or NULL;
+ * residual: NHWC d->dtype with pixel stride res_ld, or NULL; y: NHWC d->out_dtype with pixel stride out_ld. */
+int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
+                    const void *residual, void *y, void *workspace, size_t workspace_bytes, msnh_stream_t s);
+
+/* ------------------------------------------------------------------------------------------------
+ * Element-wise / bandwidth-bound layers (all NHWC, any ld).
+ * ---------------------------------------------------------------------------------------------- */
+/* y = out_mul * act( x*scale[c] + shift[c] ).  Stand-alone BatchNormLayer::forwardGPU
+ * (src/layers/MsnhBatchNormLayer.cpp:284-398: copy + normKernel + scaleBias + addBias + activation). */
+int msnh_hip_affine_act(int dtype, int out_dtype, long long pixels, int c, const void *x, int x_ld, const float *scale,
+                        const float *shift, int act, float act_param, float out_mul, void *y, int y_ld, msnh_stream_t s);
+/* y = out_mul * act( a_mul*a + b_mul*b ).  Res/Res2/AddBlock tail when it cannot be fused into a conv
+ * (BlasGPU::gpuAxpy + gpuCopy + activation, src/layers/MsnhResBlockLayer.cpp:370-389). */
+int msnh_hip_add_act(int dtype, long long pixels, int c, const void *a, int a_ld, float a_mul, const void *b, int b_ld,
+                     float b_mul, int act, float act_param, float out_mul, void *y, int y_ld, msnh_stream_t s);
+/* y[.., 0:c] = mul * x[.., 0:c].  Route / ConcatBlock copies that could not be planned away
+ * (BlasGPU::gpuSimpleCopy, src/layers/MsnhRouteLayer.cpp:200-260). */
+int msnh_hip_copy_channels(int dtype, long long pixels, int c, const void *x, int x_ld, float mul, void *y, int y_ld,
+                           msnh_stream_t s);
+/* Max pooling, padding = -FLT_MAX (maxpoolNormalKernel, src/layers/cuda/MsnhMaxPoolLayerGPU.cu:35-90 /
+ * cudnnPoolingForward, src/layers/MsnhMaxPoolLayer.cpp:460-463). */
+int msnh_hip_maxpool(int dtype, int batch, int in_h, int in_w, int c, const void *x, int x_ld, int ksize, int stride,
+                     int pad, int out_h, int out_w, void *y, int y_ld, msnh_stream_t s);
+/* Average over the valid window elements (localAvgPoolNormalKernel, src/layers/cuda/MsnhLocalAvgPoolLayerGPU.cu:5;
+ * CPU semantics src/layers/MsnhLocalAvgPoolLayer.cpp:286-344).  y = out_mul * mean. */
+int msnh_hip_avgpool(int dtype, int out_dtype, int batch, int in_h, int in_w, int c, const void *x, int x_ld, int ksize,
+                     int stride, int pad, int out_h, int out_w, float out_mul, void *y, int y_ld, msnh_stream_t s);
+/* Nearest-neighbour upsample y[oy][ox] = scale * x[oy/stride][ox/stride] (upSampleKernel,
+ * src/core/cuda/MsnhBlasGPU.cu:541-578, without its fill + accumulate). */
+int msnh_hip_upsample_nearest(int dtype, int batch, int in_h, int in_w, int c, const void *x, int x_ld, int stride,
+                              float scale, void *y, int y_ld, msnh_stream_t s);
+/* Fully connected layer out[b][o] = act( sum_i x[b][i]*w[o][i] + bias[o] ) (cublasSgemm NT + bias,
+ * src/layers/MsnhConnectedLayer.cpp:300-360).  x: [batch][inputs] d-type; w: [outputs][inputs] dtype;
+ * y: float32 [batch][outputs].  x_mul undoes the input's power-of-two storage scale. */
+int msnh_hip_connected(int dtype, int batch, int inputs, int outputs, const void *x, float x_mul, const void *w,
+                       const float *bias, int act, float act_param, float *y, msnh_stream_t s);
+/* Layout/dtype conversion at the library boundary (fp32ToFp16Kernel / fp16ToFp32Kernel,
+ * src/config/cuda/MsnhnetCuda.cu:6-36, plus the transposition).  mul scales on the way. */
+int msnh_hip_nchw_to_nhwc(int out_dtype, int batch, int c, int h, int w, const float *x_nchw, float mul, void *y,
+                          int y_ld, msnh_stream_t s);
+int msnh_hip_nhwc_to_nchw(int dtype, int batch, int c, int h, int w, const void *x, int x_ld, float mul, float *y_nchw,
+                          msnh_stream_t s);
+
+/* ------------------------------------------------------------------------------------------------
+ * YOLO.  One launch per head replaces YoloLayer::forwardGPU's 15 launches (exSigmoidKernel, aExpTKernel,
+ * sigmoidKernel: src/layers/cuda/MsnhYoloLayerGPU.cu:4-54, src/layers/MsnhYoloLayer.cpp:164-185) and
+ * YoloOutLayer::forwardGPU's shuffleDataKernel + candidate threshold (src/layers/cuda/MsnhYoloOutLayerGPU.cu:5-21,
+ * src/layers/MsnhYoloOutLayer.cpp:216-260).
+ *   x        : head logits NHWC, channel = anchor*(5+classes)+m, times x_mul gives the true logit
+ *   decoded  : float32 [batch][3][h*w][5+classes]  (the reference's "shuffled" order), may not be NULL
+ *   cand_idx : optional int32 [batch][cand_cap]; receives (anchor*h*w + pixel) + cand_base of every entry
+ *              with objectness > conf_thresh, in no particular order;
+ *   cand_cnt : int32 [batch], incremented by the number of entries found (caller zeroes it).
+ * ---------------------------------------------------------------------------------------------- */
+int msnh_hip_yolo_decode(int dtype, int batch, int h, int w, int classes, const void *x, int x_ld, float x_mul,
+                         const float *anchors6, float ratio, float *decoded, float conf_thresh, int *cand_idx,
+                         int cand_cap, int cand_base, int *cand_cnt, msnh_stream_t s);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,74 @@
+"""Builds the two shared libraries of the package in-tree:
+
+  msnhnet_amd/lib/libmsnh_hip.so   HIP kernels + C ABI (include/msnh_hip.h), hipcc --offload-arch=gfx950
+  msnhnet_amd/lib/libMsnhnet.so    C++ host side (NetBuilder, Parser, layers) + C facade (include/msnhnet_c.h)
+
+Run as `python -m msnhnet_amd.build` or through `__graft_entry__.build()`.
+"""
+import glob
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "msnhnet_amd")
+LIB = os.path.join(PKG, "lib")
+OBJ = os.path.join(PKG, "build")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-Wno-unused-command-line-argument", "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(PKG, "csrc")]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-I" + os.path.join(ROOT, "include"),
+              "-I" + os.path.join(PKG, "host", "include")]
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("command failed: " + " ".join(cmd) + "\n" + out)
+    return out
+
+
+def _compile(src, obj, flags, compiler):
+    os.makedirs(os.path.dirname(obj), exist_ok=True)
+    return _run([compiler, *flags, "-c", src, "-o", obj])
+
+
+def build_hip(verbose=True):
+    srcs = sorted(glob.glob(os.path.join(PKG, "csrc", "*.hip")))
+    objs = [os.path.join(OBJ, "hip", os.path.basename(s) + ".o") for s in srcs]
+    with ThreadPoolExecutor(max_workers=8) as ex:
+        for out in ex.map(lambda so: _compile(so[0], so[1], HIP_FLAGS, HIPCC), zip(srcs, objs)):
+            if verbose and out.strip():
+                print(out)
+    os.makedirs(LIB, exist_ok=True)
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", os.path.join(LIB, "libmsnh_hip.so"), *objs])
+    return os.path.join(LIB, "libmsnh_hip.so")
+
+
+def build_host(verbose=True):
+    srcs = sorted(glob.glob(os.path.join(PKG, "host", "src", "*.cpp")))
+    if not srcs:
+        return None
+    objs = [os.path.join(OBJ, "host", os.path.basename(s) + ".o") for s in srcs]
+    with ThreadPoolExecutor(max_workers=8) as ex:
+        for out in ex.map(lambda so: _compile(so[0], so[1], HOST_FLAGS, "g++"), zip(srcs, objs)):
+            if verbose and out.strip():
+                print(out)
+    os.makedirs(LIB, exist_ok=True)
+    _run(["g++", "-shared", "-fPIC", "-o", os.path.join(LIB, "libMsnhnet.so"), *objs,
+          "-L" + LIB, "-lmsnh_hip", "-Wl,-rpath,$ORIGIN", "-lpthread"])
+    return os.path.join(LIB, "libMsnhnet.so")
+
+
+def build_all(verbose=True):
+    a = build_hip(verbose)
+    b = build_host(verbose)
+    return a, b
+
+
+if __name__ == "__main__":
+    print(build_all())

@@ -1,0 +1,376 @@
+// Convolution entry point of the C ABI plus the non-GEMM algorithms:
+//   DIRECT    : one thread per output element, any geometry -- the fallback every shape can use;
+//   DEPTHWISE : groups == channels; bandwidth-bound, one thread per (pixel, channel vector);
+//   STEM      : first layer with <= 4 input channels, reads the NCHW float32 network input directly
+//               (layout conversion and dtype cast fused) and writes NHWC.
+// Host-side weight packing and algorithm selection live here too.
+#include "common.hpp"
+#include <vector>
+
+namespace msnh {
+
+int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
+              const void *residual, void *y, hipStream_t st);
+int convWinograd(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
+                 const void *residual, void *y, void *ws, size_t wsBytes, hipStream_t st);
+size_t winogradWorkspaceBytes(const msnh_conv_desc *d);
+void   winogradPackWeights(const msnh_conv_desc *d, const float *oihw, void *packed);
+
+struct EpiArgs
+{
+    const float *scale;
+    const float *shift;
+    int   act, act2, hasRes;
+    float actParam, act2Param, resMul, outMul;
+};
+
+__device__ __forceinline__ float epilogue(const EpiArgs &e, float acc, int ch, float res)
+{
+    const float sc = e.scale ? e.scale[ch] : 1.f;
+    const float sh = e.shift ? e.shift[ch] : 0.f;
+    float v = activate(acc * sc + sh, e.act, e.actParam);
+    if (e.hasRes) v = activate(v + e.resMul * res, e.act2, e.act2Param);
+    return e.outMul * v;
+}
+
+// ---- DIRECT ---------------------------------------------------------------------------------------
+template <typename T, typename TOut>
+__global__ __launch_bounds__(256) void convDirectKernel(const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ res,
+                                                        TOut *__restrict__ y, EpiArgs e, int H, int W, int inLd, int OH, int OW,
+                                                        int outLd, int resLd, int cinG, int coutG, int outC, int ksize, int stride,
+                                                        int pad, int dil, long long total)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int oc = static_cast<int>(idx % outC);
+    long long p = idx / outC;
+    const int ox = static_cast<int>(p % OW);
+    long long t = p / OW;
+    const int oy = static_cast<int>(t % OH);
+    const int b  = static_cast<int>(t / OH);
+    const int g  = oc / coutG;
+    const T *wp = w + static_cast<size_t>(oc) * ksize * ksize * cinG;
+    float acc = 0.f;
+    for (int ki = 0; ki < ksize; ++ki)
+    {
+        const int iy = oy * stride - pad + ki * dil;
+        if (iy < 0 || iy >= H) continue;
+        for (int kj = 0; kj < ksize; ++kj)
+        {
+            const int ix = ox * stride - pad + kj * dil;
+            if (ix < 0 || ix >= W) continue;
+            const T *xp = x + ((static_cast<size_t>(b) * H + iy) * W + ix) * inLd + g * cinG;
+            const T *wt = wp + (ki * ksize + kj) * cinG;
+            for (int c = 0; c < cinG; ++c) acc += toF(xp[c]) * toF(wt[c]);
+        }
+    }
+    const float r = e.hasRes ? toF(res[static_cast<size_t>(p) * resLd + oc]) : 0.f;
+    y[static_cast<size_t>(p) * outLd + oc] = fromF<TOut>(epilogue(e, acc, oc, r));
+}
+
+// ---- DEPTHWISE ------------------------------------------------------------------------------------
+// weights [tap][C]; thread = (pixel, VEC channels).  VEC = 1 is the unaligned fallback.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void convDepthwiseKernel(const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ res,
+                                                           T *__restrict__ y, EpiArgs e, int H, int W, int inLd, int OH, int OW, int outLd,
+                                                           int resLd, int C, int ksize, int stride, int pad, int dil, long long total)
+{
+    typedef T V __attribute__((ext_vector_type(VEC)));
+    long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int cv = C / VEC;
+    const int c0 = static_cast<int>(idx % cv) * VEC;
+    long long p = idx / cv;
+    const int ox = static_cast<int>(p % OW);
+    long long t = p / OW;
+    const int oy = static_cast<int>(t % OH);
+    const int b  = static_cast<int>(t / OH);
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+    for (int ki = 0; ki < ksize; ++ki)
+    {
+        const int iy = oy * stride - pad + ki * dil;
+        if (iy < 0 || iy >= H) continue;
+        for (int kj = 0; kj < ksize; ++kj)
+        {
+            const int ix = ox * stride - pad + kj * dil;
+            if (ix < 0 || ix >= W) continue;
+            const V xv = *reinterpret_cast<const V *>(x + ((static_cast<size_t>(b) * H + iy) * W + ix) * inLd + c0);
+            const V wv = *reinterpret_cast<const V *>(w + static_cast<size_t>(ki * ksize + kj) * C + c0);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] += toF(xv[i]) * toF(wv[i]);
+        }
+    }
+    V rv;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) rv[i] = fromF<T>(0.f);
+    if (e.hasRes) rv = *reinterpret_cast<const V *>(res + static_cast<size_t>(p) * resLd + c0);
+    V o;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) o[i] = fromF<T>(epilogue(e, acc[i], c0 + i, toF(rv[i])));
+    *reinterpret_cast<V *>(y + static_cast<size_t>(p) * outLd + c0) = o;
+}
+
+// ---- STEM -----------------------------------------------------------------------------------------
+// x: NCHW float32 [B][Cin][H][W], Cin <= 4.  weights [tap*Cin + ci][outC] float32, staged in LDS.
+// thread = one output pixel x OCT consecutive output channels (blockIdx.y selects the channel chunk);
+// consecutive lanes take consecutive ox, so input reads are coalesced along W and every lane stores
+// OCT contiguous channels.
+template <typename TOut, int OCT>
+__global__ __launch_bounds__(256) void convStemKernel(const float *__restrict__ x, const float *__restrict__ w, TOut *__restrict__ y,
+                                                      EpiArgs e, int Cin, int H, int W, int OH, int OW, int outLd, int outC, int ksize,
+                                                      int stride, int pad, long long P)
+{
+    extern __shared__ float wl[];                         // [taps*Cin][OCT]
+    const int oc0 = blockIdx.y * OCT;
+    const int kTot = ksize * ksize * Cin;
+    for (int i = threadIdx.x; i < kTot * OCT; i += blockDim.x)
+        wl[i] = w[static_cast<size_t>(i / OCT) * outC + oc0 + (i % OCT)];
+    __syncthreads();
+    long long p = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (p >= P) return;
+    const int ox = static_cast<int>(p % OW);
+    long long t = p / OW;
+    const int oy = static_cast<int>(t % OH);
+    const int b  = static_cast<int>(t / OH);
+    float acc[OCT];
+#pragma unroll
+    for (int i = 0; i < OCT; ++i) acc[i] = 0.f;
+    for (int ki = 0; ki < ksize; ++ki)
+    {
+        const int iy = oy * stride - pad + ki;
+        if (iy < 0 || iy >= H) continue;
+        for (int kj = 0; kj < ksize; ++kj)
+        {
+            const int ix = ox * stride - pad + kj;
+            if (ix < 0 || ix >= W) continue;
+            for (int ci = 0; ci < Cin; ++ci)
+            {
+                const float xv = x[((static_cast<size_t>(b) * Cin + ci) * H + iy) * W + ix];
+                const float *wr = wl + ((ki * ksize + kj) * Cin + ci) * OCT;
+#pragma unroll
+                for (int i = 0; i < OCT; ++i) acc[i] += xv * wr[i];
+            }
+        }
+    }
+    TOut *yp = y + static_cast<size_t>(p) * outLd + oc0;
+    typedef TOut OutV __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int i = 0; i < OCT; i += 4)
+    {
+        OutV o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[j] = fromF<TOut>(epilogue(e, acc[i + j], oc0 + i + j, 0.f));
+        *reinterpret_cast<OutV *>(yp + i) = o;
+    }
+}
+
+// ---- host side ------------------------------------------------------------------------------------
+static int validate(const msnh_conv_desc *d)
+{
+    MSNH_REQUIRE(d != nullptr, "conv desc is NULL");
+    MSNH_REQUIRE(dtypeOk(d->dtype) && dtypeOk(d->out_dtype), "conv: bad dtype");
+    MSNH_REQUIRE(d->batch > 0 && d->in_h > 0 && d->in_w > 0 && d->in_c > 0 && d->out_c > 0, "conv: non-positive size");
+    MSNH_REQUIRE(d->ksize > 0 && d->stride > 0 && d->pad >= 0 && d->dilation > 0 && d->groups > 0, "conv: bad geometry");
+    MSNH_REQUIRE(d->in_c % d->groups == 0 && d->out_c % d->groups == 0, "conv: channels not divisible by groups");
+    const int ext = d->dilation * (d->ksize - 1) + 1;
+    MSNH_REQUIRE(d->in_h + 2 * d->pad >= ext && d->in_w + 2 * d->pad >= ext, "conv: kernel larger than padded input");
+    const int oh = (d->in_h + 2 * d->pad - ext) / d->stride + 1;
+    const int ow = (d->in_w + 2 * d->pad - ext) / d->stride + 1;
+    MSNH_REQUIRE(oh == d->out_h && ow == d->out_w, "conv: out size %dx%d does not match geometry (%dx%d)", d->out_h, d->out_w, oh, ow);
+    MSNH_REQUIRE(d->out_ld >= d->out_c, "conv: out_ld < out_c");
+    MSNH_REQUIRE(!d->has_residual || d->res_ld >= d->out_c, "conv: res_ld < out_c");
+    MSNH_REQUIRE(actOk(d->act) && (!d->has_residual || actOk(d->act2)), "conv: unsupported activation");
+    MSNH_REQUIRE(static_cast<long long>(d->batch) * d->out_h * d->out_w < (1LL << 31), "conv: too many output pixels");
+    return 0;
+}
+
+static bool igemmOk(const msnh_conv_desc *d)
+{
+    const int vec = d->dtype == MSNH_F16 ? 8 : 4;
+    if (d->dtype == MSNH_F32 && d->out_dtype != MSNH_F32) return false;
+    return (d->in_c / d->groups) % vec == 0 && d->in_ld % vec == 0;
+}
+
+static bool depthwiseOk(const msnh_conv_desc *d)
+{
+    return d->groups == d->in_c && d->out_c == d->in_c && d->groups > 1 && d->dtype == d->out_dtype;
+}
+
+static bool stemOk(const msnh_conv_desc *d)
+{
+    return d->in_c <= 4 && d->groups == 1 && d->dilation == 1 && d->out_c % 32 == 0 && d->out_ld % 4 == 0 &&
+           !d->has_residual && static_cast<size_t>(d->ksize) * d->ksize * d->in_c * 32 * 4 <= 60 * 1024;
+}
+
+static bool winogradOk(const msnh_conv_desc *d)
+{
+    return d->ksize == 3 && d->stride == 1 && d->dilation == 1 && d->groups == 1 && d->pad == 1 && d->dtype == MSNH_F16 &&
+           d->in_c % 8 == 0 && d->in_ld % 8 == 0 && d->out_c % 8 == 0;
+}
+
+} // namespace msnh
+
+using namespace msnh;
+
+extern "C" {
+
+int msnh_hip_conv2d_select_algo(const msnh_conv_desc *d)
+{
+    if (!d) return MSNH_CONV_DIRECT;
+    if (d->algo != MSNH_CONV_AUTO) return d->algo;
+    if (stemOk(d)) return MSNH_CONV_STEM;
+    if (depthwiseOk(d)) return MSNH_CONV_DEPTHWISE;
+    if (igemmOk(d)) return MSNH_CONV_IGEMM;
+    return MSNH_CONV_DIRECT;
+}
+
+size_t msnh_hip_conv2d_packed_weight_elems(const msnh_conv_desc *d, int algo)
+{
+    if (!d) return 0;
+    const size_t kk = static_cast<size_t>(d->ksize) * d->ksize;
+    const size_t cinG = static_cast<size_t>(d->in_c / d->groups);
+    if (algo == MSNH_CONV_WINOGRAD) return static_cast<size_t>(16) * d->out_c * d->in_c;
+    if (algo == MSNH_CONV_STEM) return kk * d->in_c * d->out_c * (d->dtype == MSNH_F16 ? 2 : 1);   // float32 payload
+    return static_cast<size_t>(d->out_c) * kk * cinG;
+}
+
+int msnh_hip_conv2d_pack_weights(const msnh_conv_desc *d, int algo, const float *oihw, void *packed)
+{
+    if (validate(d)) return 2;
+    MSNH_REQUIRE(oihw && packed, "pack_weights: NULL pointer");
+    const int kk = d->ksize * d->ksize;
+    const int cinG = d->in_c / d->groups;
+    auto put = [&](size_t i, float v) {
+        if (d->dtype == MSNH_F16) static_cast<_Float16 *>(packed)[i] = static_cast<_Float16>(v);
+        else static_cast<float *>(packed)[i] = v;
+    };
+    switch (algo)
+    {
+    case MSNH_CONV_DIRECT:
+    case MSNH_CONV_IGEMM:
+        for (int oc = 0; oc < d->out_c; ++oc)
+            for (int ci = 0; ci < cinG; ++ci)
+                for (int t = 0; t < kk; ++t)
+                    put((static_cast<size_t>(oc) * kk + t) * cinG + ci, oihw[(static_cast<size_t>(oc) * cinG + ci) * kk + t]);
+        return 0;
+    case MSNH_CONV_DEPTHWISE:
+        MSNH_REQUIRE(depthwiseOk(d), "pack_weights: not a depthwise convolution");
+        for (int c = 0; c < d->out_c; ++c)
+            for (int t = 0; t < kk; ++t) put(static_cast<size_t>(t) * d->out_c + c, oihw[static_cast<size_t>(c) * kk + t]);
+        return 0;
+    case MSNH_CONV_STEM:
+    {
+        MSNH_REQUIRE(stemOk(d), "pack_weights: shape not supported by the stem kernel");
+        float *o = static_cast<float *>(packed);
+        for (int oc = 0; oc < d->out_c; ++oc)
+            for (int ci = 0; ci < d->in_c; ++ci)
+                for (int t = 0; t < kk; ++t)
+                    o[(static_cast<size_t>(t) * d->in_c + ci) * d->out_c + oc] = oihw[(static_cast<size_t>(oc) * d->in_c + ci) * kk + t];
+        return 0;
+    }
+    case MSNH_CONV_WINOGRAD:
+        MSNH_REQUIRE(winogradOk(d), "pack_weights: shape not supported by the Winograd kernel");
+        winogradPackWeights(d, oihw, packed);
+        return 0;
+    default:
+        setError("pack_weights: unknown algo %d", algo);
+        return 2;
+    }
+}
+
+size_t msnh_hip_conv2d_workspace_bytes(const msnh_conv_desc *d, int algo)
+{
+    if (!d || algo != MSNH_CONV_WINOGRAD) return 0;
+    return winogradWorkspaceBytes(d);
+}
+
+int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
+                    const void *residual, void *y, void *workspace, size_t workspace_bytes, msnh_stream_t s)
+{
+    if (validate(d)) return 2;
+    MSNH_REQUIRE(x && w && y, "conv2d: NULL tensor pointer");
+    MSNH_REQUIRE(!d->has_residual || residual, "conv2d: has_residual without a residual tensor");
+    hipStream_t st = resolveStream(s);
+    const int algo = msnh_hip_conv2d_select_algo(d);
+    EpiArgs e;
+    e.scale = scale; e.shift = shift; e.act = d->act; e.act2 = d->act2; e.hasRes = d->has_residual ? 1 : 0;
+    e.actParam = d->act_param; e.act2Param = d->act2_param; e.resMul = d->res_mul; e.outMul = d->out_mul;
+    const int cinG = d->in_c / d->groups, coutG = d->out_c / d->groups;
+    const long long P = static_cast<long long>(d->batch) * d->out_h * d->out_w;
+    if (algo != MSNH_CONV_STEM) MSNH_REQUIRE(d->in_ld >= d->in_c, "conv2d: in_ld < in_c");
+
+    switch (algo)
+    {
+    case MSNH_CONV_IGEMM:
+        MSNH_REQUIRE(igemmOk(d), "conv2d: IGEMM needs (in_c/groups) and in_ld to be multiples of %d", d->dtype == MSNH_F16 ? 8 : 4);
+        MSNH_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0, "conv2d: IGEMM needs 16-byte aligned x and w");
+        return convIgemm(d, x, w, scale, shift, residual, y, st);
+    case MSNH_CONV_WINOGRAD:
+        MSNH_REQUIRE(winogradOk(d), "conv2d: shape not supported by the Winograd kernel");
+        return convWinograd(d, x, w, scale, shift, residual, y, workspace, workspace_bytes, st);
+    case MSNH_CONV_DEPTHWISE:
+    {
+        MSNH_REQUIRE(depthwiseOk(d), "conv2d: not a depthwise convolution");
+        const int C = d->in_c;
+        const int vec = d->dtype == MSNH_F16 ? 8 : 4;
+        const size_t el = dtypeSize(d->dtype);
+        const bool aligned = C % vec == 0 && d->in_ld % vec == 0 && d->out_ld % vec == 0 && (!d->has_residual || d->res_ld % vec == 0) &&
+                             reinterpret_cast<uintptr_t>(x) % (vec * el) == 0 && reinterpret_cast<uintptr_t>(y) % (vec * el) == 0 &&
+                             reinterpret_cast<uintptr_t>(w) % (vec * el) == 0 &&
+                             (!d->has_residual || reinterpret_cast<uintptr_t>(residual) % (vec * el) == 0);
+        const long long total = P * (aligned ? C / vec : C);
+        dim3 grid(gridFor(total, 256));
+#define MSNH_DW(T, V)                                                                                                   \
+    hipLaunchKernelGGL((convDepthwiseKernel<T, V>), grid, dim3(256), 0, st, static_cast<const T *>(x), static_cast<const T *>(w), \
+                       static_cast<const T *>(residual), static_cast<T *>(y), e, d->in_h, d->in_w, d->in_ld, d->out_h, d->out_w,    \
+                       d->out_ld, d->res_ld, C, d->ksize, d->stride, d->pad, d->dilation, total)
+        if (d->dtype == MSNH_F16) { if (aligned) MSNH_DW(f16, 8); else MSNH_DW(f16, 1); }
+        else                      { if (aligned) MSNH_DW(float, 4); else MSNH_DW(float, 1); }
+#undef MSNH_DW
+        MSNH_LAUNCH_CHECK();
+        return 0;
+    }
+    case MSNH_CONV_STEM:
+    {
+        MSNH_REQUIRE(stemOk(d), "conv2d: shape not supported by the stem kernel");
+        const size_t outEl = dtypeSize(d->out_dtype);
+        MSNH_REQUIRE(reinterpret_cast<uintptr_t>(y) % (4 * outEl) == 0, "conv2d: stem needs aligned output");
+        constexpr int OCT = 32;
+        dim3 grid(gridFor(P, 256), d->out_c / OCT);
+        const size_t smem = static_cast<size_t>(d->ksize) * d->ksize * d->in_c * OCT * sizeof(float);
+        if (d->out_dtype == MSNH_F16)
+            hipLaunchKernelGGL((convStemKernel<f16, OCT>), grid, dim3(256), smem, st, static_cast<const float *>(x), static_cast<const float *>(w),
+                               static_cast<f16 *>(y), e, d->in_c, d->in_h, d->in_w, d->out_h, d->out_w, d->out_ld, d->out_c, d->ksize, d->stride, d->pad, P);
+        else
+            hipLaunchKernelGGL((convStemKernel<float, OCT>), grid, dim3(256), smem, st, static_cast<const float *>(x), static_cast<const float *>(w),
+                               static_cast<float *>(y), e, d->in_c, d->in_h, d->in_w, d->out_h, d->out_w, d->out_ld, d->out_c, d->ksize, d->stride, d->pad, P);
+        MSNH_LAUNCH_CHECK();
+        return 0;
+    }
+    case MSNH_CONV_DIRECT:
+    {
+        const long long total = P * d->out_c;
+        dim3 grid(gridFor(total, 256));
+#define MSNH_DIRECT(T, TO)                                                                                              \
+    hipLaunchKernelGGL((convDirectKernel<T, TO>), grid, dim3(256), 0, st, static_cast<const T *>(x), static_cast<const T *>(w),  \
+                       static_cast<const T *>(residual), static_cast<TO *>(y), e, d->in_h, d->in_w, d->in_ld, d->out_h, d->out_w,  \
+                       d->out_ld, d->res_ld, cinG, coutG, d->out_c, d->ksize, d->stride, d->pad, d->dilation, total)
+        if (d->dtype == MSNH_F16) { if (d->out_dtype == MSNH_F16) MSNH_DIRECT(f16, f16); else MSNH_DIRECT(f16, float); }
+        else
+        {
+            MSNH_REQUIRE(d->out_dtype == MSNH_F32, "conv2d: float32 input needs float32 output");
+            MSNH_DIRECT(float, float);
+        }
+#undef MSNH_DIRECT
+        MSNH_LAUNCH_CHECK();
+        return 0;
+    }
+    default:
+        setError("conv2d: unknown algo %d", algo);
+        return 2;
+    }
+}
+
+}

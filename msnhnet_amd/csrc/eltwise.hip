@@ -1,0 +1,462 @@
+// Bandwidth-bound NHWC layers: stand-alone batch-norm affine, residual add, channel copy (concat),
+// max/avg pooling, nearest upsample, fully-connected, and the NCHW<->NHWC boundary conversions.
+// Every kernel maps consecutive lanes to consecutive channel vectors of a pixel (16-byte accesses when
+// the channel count, pixel strides and base addresses allow it, scalar otherwise), so global accesses
+// are coalesced along the contiguous NHWC channel axis.
+#include "common.hpp"
+
+namespace msnh {
+
+template <typename T, int VEC> struct VecOf { typedef T type __attribute__((ext_vector_type(VEC))); };
+template <typename T> struct VecOf<T, 1> { typedef T type; };
+
+template <typename T, int VEC> __device__ __forceinline__ void loadVec(const T *p, float (&v)[VEC])
+{
+    if constexpr (VEC == 1) { v[0] = toF(p[0]); }
+    else
+    {
+        typedef typename VecOf<T, VEC>::type V;
+        const V t = *reinterpret_cast<const V *>(p);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = toF(t[i]);
+    }
+}
+
+template <typename T, int VEC> __device__ __forceinline__ void storeVec(T *p, const float (&v)[VEC])
+{
+    if constexpr (VEC == 1) { p[0] = fromF<T>(v[0]); }
+    else
+    {
+        typedef typename VecOf<T, VEC>::type V;
+        V t;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) t[i] = fromF<T>(v[i]);
+        *reinterpret_cast<V *>(p) = t;
+    }
+}
+
+// ---- y = out_mul * act(x*scale[c] + shift[c]) ------------------------------------------------------
+template <typename T, typename TOut, int VEC>
+__global__ __launch_bounds__(256) void affineActKernel(const T *__restrict__ x, int xLd, const float *__restrict__ scale,
+                                                       const float *__restrict__ shift, int act, float actParam, float outMul,
+                                                       TOut *__restrict__ y, int yLd, int c, long long total)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int cv = c / VEC;
+    const int c0 = static_cast<int>(idx % cv) * VEC;
+    const long long p = idx / cv;
+    float v[VEC];
+    loadVec<T, VEC>(x + p * xLd + c0, v);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i)
+    {
+        const float sc = scale ? scale[c0 + i] : 1.f;
+        const float sh = shift ? shift[c0 + i] : 0.f;
+        v[i] = outMul * activate(v[i] * sc + sh, act, actParam);
+    }
+    storeVec<TOut, VEC>(y + p * yLd + c0, v);
+}
+
+// ---- y = out_mul * act(a_mul*a + b_mul*b) ----------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void addActKernel(const T *__restrict__ a, int aLd, float aMul, const T *__restrict__ b, int bLd,
+                                                    float bMul, int act, float actParam, float outMul, T *__restrict__ y, int yLd,
+                                                    int c, long long total)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int cv = c / VEC;
+    const int c0 = static_cast<int>(idx % cv) * VEC;
+    const long long p = idx / cv;
+    float va[VEC], vb[VEC];
+    loadVec<T, VEC>(a + p * aLd + c0, va);
+    loadVec<T, VEC>(b + p * bLd + c0, vb);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) va[i] = outMul * activate(aMul * va[i] + bMul * vb[i], act, actParam);
+    storeVec<T, VEC>(y + p * yLd + c0, va);
+}
+
+// ---- max pooling -----------------------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void maxPoolKernel(const T *__restrict__ x, int xLd, int H, int W, int c, int ksize, int stride,
+                                                     int pad, int OH, int OW, T *__restrict__ y, int yLd, long long total)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int cv = c / VEC;
+    const int c0 = static_cast<int>(idx % cv) * VEC;
+    const long long p = idx / cv;
+    const int ox = static_cast<int>(p % OW);
+    const long long t = p / OW;
+    const int oy = static_cast<int>(t % OH);
+    const long long b = t / OH;
+    float m[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) m[i] = -FLT_MAX;
+    const int y0 = oy * stride - pad, x0 = ox * stride - pad;
+    const int ya = y0 < 0 ? 0 : y0, yb = (y0 + ksize > H) ? H : y0 + ksize;
+    const int xa = x0 < 0 ? 0 : x0, xb = (x0 + ksize > W) ? W : x0 + ksize;
+    for (int iy = ya; iy < yb; ++iy)
+        for (int ix = xa; ix < xb; ++ix)
+        {
+            float v[VEC];
+            loadVec<T, VEC>(x + ((b * H + iy) * W + ix) * xLd + c0, v);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) m[i] = (v[i] > m[i]) ? v[i] : m[i];
+        }
+    if constexpr (sizeof(T) == 2)
+    {
+        // a window lying entirely in the padding yields -FLT_MAX in the reference; clamp to the half range
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) m[i] = m[i] < -65504.f ? -65504.f : m[i];
+    }
+    storeVec<T, VEC>(y + p * yLd + c0, m);
+}
+
+// ---- average pooling over valid elements -------------------------------------------------------------
+template <typename T, typename TOut, int VEC>
+__global__ __launch_bounds__(256) void avgPoolKernel(const T *__restrict__ x, int xLd, int H, int W, int c, int ksize, int stride,
+                                                     int pad, int OH, int OW, float outMul, TOut *__restrict__ y, int yLd, long long total)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int cv = c / VEC;
+    const int c0 = static_cast<int>(idx % cv) * VEC;
+    const long long p = idx / cv;
+    const int ox = static_cast<int>(p % OW);
+    const long long t = p / OW;
+    const int oy = static_cast<int>(t % OH);
+    const long long b = t / OH;
+    float sum[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) sum[i] = 0.f;
+    int count = 0;
+    for (int n = 0; n < ksize; ++n)
+        for (int m = 0; m < ksize; ++m)
+        {
+            const int iy = oy * stride - pad + n, ix = ox * stride - pad + m;
+            if (iy < 0 || iy >= H || ix < 0 || ix >= W) continue;
+            float v[VEC];
+            loadVec<T, VEC>(x + ((b * H + iy) * W + ix) * xLd + c0, v);
+            ++count;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) sum[i] += v[i];
+        }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) sum[i] = outMul * (sum[i] / static_cast<float>(count));
+    storeVec<TOut, VEC>(y + p * yLd + c0, sum);
+}
+
+// ---- nearest upsample / channel copy -------------------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void upsampleKernel(const T *__restrict__ x, int xLd, int H, int W, int c, int stride, float scale,
+                                                      T *__restrict__ y, int yLd, long long total)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int cv = c / VEC;
+    const int c0 = static_cast<int>(idx % cv) * VEC;
+    const long long p = idx / cv;
+    const int OW = W * stride, OH = H * stride;
+    const int ox = static_cast<int>(p % OW);
+    const long long t = p / OW;
+    const int oy = static_cast<int>(t % OH);
+    const long long b = t / OH;
+    float v[VEC];
+    loadVec<T, VEC>(x + ((b * H + oy / stride) * W + ox / stride) * xLd + c0, v);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = scale * v[i];
+    storeVec<T, VEC>(y + p * yLd + c0, v);
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void copyChannelsKernel(const T *__restrict__ x, int xLd, float mul, T *__restrict__ y, int yLd, int c,
+                                                          long long total)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int cv = c / VEC;
+    const int c0 = static_cast<int>(idx % cv) * VEC;
+    const long long p = idx / cv;
+    float v[VEC];
+    loadVec<T, VEC>(x + p * xLd + c0, v);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = mul * v[i];
+    storeVec<T, VEC>(y + p * yLd + c0, v);
+}
+
+// ---- fully connected: one wavefront per (batch row, output), wave-level reduction -------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void connectedKernel(const T *__restrict__ x, float xMul, const T *__restrict__ w,
+                                                       const float *__restrict__ bias, int act, float actParam, float *__restrict__ y,
+                                                       int batch, int inputs, int outputs)
+{
+    const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int lane = threadIdx.x & 63;
+    if (wave >= batch * outputs) return;
+    const int b = wave / outputs, o = wave - b * outputs;
+    const T *xp = x + static_cast<size_t>(b) * inputs;
+    const T *wp = w + static_cast<size_t>(o) * inputs;
+    float sum = 0.f;
+    for (int i = lane; i < inputs; i += 64) sum += toF(xp[i]) * toF(wp[i]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (lane == 0)
+    {
+        float v = sum * xMul + (bias ? bias[o] : 0.f);
+        y[static_cast<size_t>(b) * outputs + o] = activate(v, act, actParam);
+    }
+}
+
+// ---- boundary layout conversions (tiled transposes through LDS) --------------------------------------------
+// NCHW float32 -> NHWC T.  Block handles 32 pixels x 32 channels of one image.
+template <typename T>
+__global__ __launch_bounds__(256) void nchwToNhwcKernel(const float *__restrict__ x, float mul, T *__restrict__ y, int yLd, int C, int HW)
+{
+    __shared__ float tile[32][33];
+    const int b = blockIdx.z;
+    const int p0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;          // 32 x 8
+    for (int i = ty; i < 32; i += 8)
+    {
+        const int c = c0 + i, p = p0 + tx;
+        tile[i][tx] = (c < C && p < HW) ? x[(static_cast<size_t>(b) * C + c) * HW + p] : 0.f;
+    }
+    __syncthreads();
+    for (int i = ty; i < 32; i += 8)
+    {
+        const int p = p0 + i, c = c0 + tx;
+        if (p < HW && c < C) y[(static_cast<size_t>(b) * HW + p) * yLd + c] = fromF<T>(mul * tile[tx][i]);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void nhwcToNchwKernel(const T *__restrict__ x, int xLd, float mul, float *__restrict__ y, int C, int HW)
+{
+    __shared__ float tile[32][33];
+    const int b = blockIdx.z;
+    const int p0 = blockIdx.x * 32, c0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    for (int i = ty; i < 32; i += 8)
+    {
+        const int p = p0 + i, c = c0 + tx;
+        tile[i][tx] = (p < HW && c < C) ? toF(x[(static_cast<size_t>(b) * HW + p) * xLd + c]) : 0.f;
+    }
+    __syncthreads();
+    for (int i = ty; i < 32; i += 8)
+    {
+        const int c = c0 + i, p = p0 + tx;
+        if (c < C && p < HW) y[(static_cast<size_t>(b) * C + c) * HW + p] = mul * tile[tx][i];
+    }
+}
+
+// Picks the widest vector every participating tensor supports.
+static int pickVec(int dtype, int c, std::initializer_list<int> lds, std::initializer_list<const void *> ptrs)
+{
+    const int vec = dtype == MSNH_F16 ? 8 : 4;
+    if (c % vec) return 1;
+    for (int ld : lds) if (ld % vec) return 1;
+    for (const void *p : ptrs) if (p && reinterpret_cast<uintptr_t>(p) % 16) return 1;
+    return vec;
+}
+
+} // namespace msnh
+
+using namespace msnh;
+
+#define MSNH_CHECK_COMMON(name, pixels, c)                                                           \
+    MSNH_REQUIRE((pixels) > 0 && (c) > 0, name ": non-positive size");                              \
+    MSNH_REQUIRE(static_cast<long long>(pixels) * (c) < (1LL << 40), name ": tensor too large")
+
+extern "C" {
+
+int msnh_hip_affine_act(int dtype, int out_dtype, long long pixels, int c, const void *x, int x_ld, const float *scale,
+                        const float *shift, int act, float act_param, float out_mul, void *y, int y_ld, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype) && dtypeOk(out_dtype), "affine_act: bad dtype");
+    MSNH_CHECK_COMMON("affine_act", pixels, c);
+    MSNH_REQUIRE(x && y && x_ld >= c && y_ld >= c && actOk(act), "affine_act: bad argument");
+    hipStream_t st = resolveStream(s);
+    int vec = pickVec(dtype, c, {x_ld, y_ld}, {x, y});
+    if (dtype != out_dtype) vec = (vec > 1 && c % 8 == 0 && x_ld % 8 == 0 && y_ld % 8 == 0) ? 4 : 1;
+    const long long total = pixels * (c / vec);
+    dim3 grid(gridFor(total, 256));
+#define MSNH_AFF(T, TO, V)                                                                                                     \
+    hipLaunchKernelGGL((affineActKernel<T, TO, V>), grid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, scale, shift, act, \
+                       act_param, out_mul, static_cast<TO *>(y), y_ld, c, total)
+    if (dtype == MSNH_F16 && out_dtype == MSNH_F16) { if (vec == 8) MSNH_AFF(f16, f16, 8); else MSNH_AFF(f16, f16, 1); }
+    else if (dtype == MSNH_F32 && out_dtype == MSNH_F32) { if (vec == 4) MSNH_AFF(float, float, 4); else MSNH_AFF(float, float, 1); }
+    else if (dtype == MSNH_F16) { if (vec == 4) MSNH_AFF(f16, float, 4); else MSNH_AFF(f16, float, 1); }
+    else { if (vec == 4) MSNH_AFF(float, f16, 4); else MSNH_AFF(float, f16, 1); }
+#undef MSNH_AFF
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+int msnh_hip_add_act(int dtype, long long pixels, int c, const void *a, int a_ld, float a_mul, const void *b, int b_ld,
+                     float b_mul, int act, float act_param, float out_mul, void *y, int y_ld, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "add_act: bad dtype");
+    MSNH_CHECK_COMMON("add_act", pixels, c);
+    MSNH_REQUIRE(a && b && y && a_ld >= c && b_ld >= c && y_ld >= c && actOk(act), "add_act: bad argument");
+    hipStream_t st = resolveStream(s);
+    const int vec = pickVec(dtype, c, {a_ld, b_ld, y_ld}, {a, b, y});
+    const long long total = pixels * (c / vec);
+    dim3 grid(gridFor(total, 256));
+#define MSNH_ADD(T, V)                                                                                                          \
+    hipLaunchKernelGGL((addActKernel<T, V>), grid, dim3(256), 0, st, static_cast<const T *>(a), a_ld, a_mul, static_cast<const T *>(b), \
+                       b_ld, b_mul, act, act_param, out_mul, static_cast<T *>(y), y_ld, c, total)
+    if (dtype == MSNH_F16) { if (vec == 8) MSNH_ADD(f16, 8); else MSNH_ADD(f16, 1); }
+    else { if (vec == 4) MSNH_ADD(float, 4); else MSNH_ADD(float, 1); }
+#undef MSNH_ADD
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+int msnh_hip_copy_channels(int dtype, long long pixels, int c, const void *x, int x_ld, float mul, void *y, int y_ld,
+                           msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "copy_channels: bad dtype");
+    MSNH_CHECK_COMMON("copy_channels", pixels, c);
+    MSNH_REQUIRE(x && y && x_ld >= c && y_ld >= c, "copy_channels: bad argument");
+    hipStream_t st = resolveStream(s);
+    const int vec = pickVec(dtype, c, {x_ld, y_ld}, {x, y});
+    const long long total = pixels * (c / vec);
+    dim3 grid(gridFor(total, 256));
+#define MSNH_CPY(T, V)                                                                                                   \
+    hipLaunchKernelGGL((copyChannelsKernel<T, V>), grid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, mul, static_cast<T *>(y), \
+                       y_ld, c, total)
+    if (dtype == MSNH_F16) { if (vec == 8) MSNH_CPY(f16, 8); else MSNH_CPY(f16, 1); }
+    else { if (vec == 4) MSNH_CPY(float, 4); else MSNH_CPY(float, 1); }
+#undef MSNH_CPY
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+static int checkPool(const char *name, int batch, int in_h, int in_w, int c, int ksize, int stride, int pad, int out_h, int out_w)
+{
+    MSNH_REQUIRE(batch > 0 && in_h > 0 && in_w > 0 && c > 0 && ksize > 0 && stride > 0 && pad >= 0, "%s: bad geometry", name);
+    MSNH_REQUIRE(in_h + 2 * pad >= ksize && in_w + 2 * pad >= ksize, "%s: window larger than padded input", name);
+    MSNH_REQUIRE(out_h > 0 && out_w > 0, "%s: non-positive output size", name);
+    // every window must start inside the padded input (covers floor and ceil output sizes)
+    MSNH_REQUIRE((out_h - 1) * stride - pad < in_h && (out_w - 1) * stride - pad < in_w, "%s: output size too large", name);
+    return 0;
+}
+
+int msnh_hip_maxpool(int dtype, int batch, int in_h, int in_w, int c, const void *x, int x_ld, int ksize, int stride,
+                     int pad, int out_h, int out_w, void *y, int y_ld, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "maxpool: bad dtype");
+    if (checkPool("maxpool", batch, in_h, in_w, c, ksize, stride, pad, out_h, out_w)) return 2;
+    MSNH_REQUIRE(x && y && x_ld >= c && y_ld >= c, "maxpool: bad argument");
+    hipStream_t st = resolveStream(s);
+    const int vec = pickVec(dtype, c, {x_ld, y_ld}, {x, y});
+    const long long total = static_cast<long long>(batch) * out_h * out_w * (c / vec);
+    dim3 grid(gridFor(total, 256));
+#define MSNH_MP(T, V)                                                                                                  \
+    hipLaunchKernelGGL((maxPoolKernel<T, V>), grid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, in_h, in_w, c, ksize, stride, \
+                       pad, out_h, out_w, static_cast<T *>(y), y_ld, total)
+    if (dtype == MSNH_F16) { if (vec == 8) MSNH_MP(f16, 8); else MSNH_MP(f16, 1); }
+    else { if (vec == 4) MSNH_MP(float, 4); else MSNH_MP(float, 1); }
+#undef MSNH_MP
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+int msnh_hip_avgpool(int dtype, int out_dtype, int batch, int in_h, int in_w, int c, const void *x, int x_ld, int ksize,
+                     int stride, int pad, int out_h, int out_w, float out_mul, void *y, int y_ld, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype) && dtypeOk(out_dtype), "avgpool: bad dtype");
+    MSNH_REQUIRE(!(dtype == MSNH_F32 && out_dtype == MSNH_F16), "avgpool: float32 -> float16 not supported");
+    if (checkPool("avgpool", batch, in_h, in_w, c, ksize, stride, pad, out_h, out_w)) return 2;
+    MSNH_REQUIRE(x && y && x_ld >= c && y_ld >= c, "avgpool: bad argument");
+    hipStream_t st = resolveStream(s);
+    int vec = pickVec(dtype, c, {x_ld, y_ld}, {x, y});
+    if (dtype != out_dtype) vec = (vec > 1 && y_ld % 8 == 0) ? 4 : 1;
+    const long long total = static_cast<long long>(batch) * out_h * out_w * (c / vec);
+    dim3 grid(gridFor(total, 256));
+#define MSNH_AP(T, TO, V)                                                                                              \
+    hipLaunchKernelGGL((avgPoolKernel<T, TO, V>), grid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, in_h, in_w, c, ksize,  \
+                       stride, pad, out_h, out_w, out_mul, static_cast<TO *>(y), y_ld, total)
+    if (dtype == MSNH_F16 && out_dtype == MSNH_F16) { if (vec == 8) MSNH_AP(f16, f16, 8); else MSNH_AP(f16, f16, 1); }
+    else if (dtype == MSNH_F16) { if (vec == 4) MSNH_AP(f16, float, 4); else MSNH_AP(f16, float, 1); }
+    else { if (vec == 4) MSNH_AP(float, float, 4); else MSNH_AP(float, float, 1); }
+#undef MSNH_AP
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+int msnh_hip_upsample_nearest(int dtype, int batch, int in_h, int in_w, int c, const void *x, int x_ld, int stride,
+                              float scale, void *y, int y_ld, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "upsample: bad dtype");
+    MSNH_REQUIRE(batch > 0 && in_h > 0 && in_w > 0 && c > 0 && stride > 0, "upsample: bad geometry");
+    MSNH_REQUIRE(x && y && x_ld >= c && y_ld >= c, "upsample: bad argument");
+    hipStream_t st = resolveStream(s);
+    const int vec = pickVec(dtype, c, {x_ld, y_ld}, {x, y});
+    const long long total = static_cast<long long>(batch) * in_h * stride * in_w * stride * (c / vec);
+    dim3 grid(gridFor(total, 256));
+#define MSNH_UP(T, V)                                                                                                  \
+    hipLaunchKernelGGL((upsampleKernel<T, V>), grid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, in_h, in_w, c, stride, scale, \
+                       static_cast<T *>(y), y_ld, total)
+    if (dtype == MSNH_F16) { if (vec == 8) MSNH_UP(f16, 8); else MSNH_UP(f16, 1); }
+    else { if (vec == 4) MSNH_UP(float, 4); else MSNH_UP(float, 1); }
+#undef MSNH_UP
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+int msnh_hip_connected(int dtype, int batch, int inputs, int outputs, const void *x, float x_mul, const void *w,
+                       const float *bias, int act, float act_param, float *y, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "connected: bad dtype");
+    MSNH_REQUIRE(batch > 0 && inputs > 0 && outputs > 0 && x && w && y && actOk(act), "connected: bad argument");
+    hipStream_t st = resolveStream(s);
+    const long long waves = static_cast<long long>(batch) * outputs;
+    dim3 grid(gridFor(waves * 64, 256));
+    if (dtype == MSNH_F16)
+        hipLaunchKernelGGL((connectedKernel<f16>), grid, dim3(256), 0, st, static_cast<const f16 *>(x), x_mul, static_cast<const f16 *>(w),
+                           bias, act, act_param, y, batch, inputs, outputs);
+    else
+        hipLaunchKernelGGL((connectedKernel<float>), grid, dim3(256), 0, st, static_cast<const float *>(x), x_mul,
+                           static_cast<const float *>(w), bias, act, act_param, y, batch, inputs, outputs);
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+int msnh_hip_nchw_to_nhwc(int out_dtype, int batch, int c, int h, int w, const float *x_nchw, float mul, void *y,
+                          int y_ld, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(out_dtype), "nchw_to_nhwc: bad dtype");
+    MSNH_REQUIRE(batch > 0 && c > 0 && h > 0 && w > 0 && x_nchw && y && y_ld >= c, "nchw_to_nhwc: bad argument");
+    MSNH_REQUIRE(batch <= 65535 && (c + 31) / 32 <= 65535, "nchw_to_nhwc: grid too large");
+    hipStream_t st = resolveStream(s);
+    const int hw = h * w;
+    dim3 grid((hw + 31) / 32, (c + 31) / 32, batch);
+    if (out_dtype == MSNH_F16)
+        hipLaunchKernelGGL((nchwToNhwcKernel<f16>), grid, dim3(256), 0, st, x_nchw, mul, static_cast<f16 *>(y), y_ld, c, hw);
+    else
+        hipLaunchKernelGGL((nchwToNhwcKernel<float>), grid, dim3(256), 0, st, x_nchw, mul, static_cast<float *>(y), y_ld, c, hw);
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+int msnh_hip_nhwc_to_nchw(int dtype, int batch, int c, int h, int w, const void *x, int x_ld, float mul, float *y_nchw,
+                          msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "nhwc_to_nchw: bad dtype");
+    MSNH_REQUIRE(batch > 0 && c > 0 && h > 0 && w > 0 && x && y_nchw && x_ld >= c, "nhwc_to_nchw: bad argument");
+    MSNH_REQUIRE(batch <= 65535 && (c + 31) / 32 <= 65535, "nhwc_to_nchw: grid too large");
+    hipStream_t st = resolveStream(s);
+    const int hw = h * w;
+    dim3 grid((hw + 31) / 32, (c + 31) / 32, batch);
+    if (dtype == MSNH_F16)
+        hipLaunchKernelGGL((nhwcToNchwKernel<f16>), grid, dim3(256), 0, st, static_cast<const f16 *>(x), x_ld, mul, y_nchw, c, hw);
+    else
+        hipLaunchKernelGGL((nhwcToNchwKernel<float>), grid, dim3(256), 0, st, static_cast<const float *>(x), x_ld, mul, y_nchw, c, hw);
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+}

@@ -1,0 +1,389 @@
+/* TEST INFRASTRUCTURE ONLY -- see msnh_oracle.h.  Plain C restatement of the reference CPU path. */
+#include "msnh_oracle.h"
+#include <float.h>
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* Gemm::cpuIm2colEx, generic branch (src/core/MsnhGemm.cpp:156-292):
+ * col[((c*kH+kr)*kW+kc)*outH*outW + oy*outW + ox] = im[c][oy*sH-pH+kr*dH][ox*sW-pW+kc*dW] or 0. */
+void msnh_or_im2col(const float *im, int channels, int height, int width, int kH, int kW, int padH, int padW,
+                    int strideH, int strideW, int dilH, int dilW, float *col)
+{
+    const int outH = (height + 2 * padH - (dilH * (kH - 1) + 1)) / strideH + 1;
+    const int outW = (width + 2 * padW - (dilW * (kW - 1) + 1)) / strideW + 1;
+    for (int c = 0; c < channels; ++c)
+        for (int kr = 0; kr < kH; ++kr)
+            for (int kc = 0; kc < kW; ++kc)
+            {
+                float *dst = col + (((size_t)c * kH + kr) * kW + kc) * outH * outW;
+                for (int oy = 0; oy < outH; ++oy)
+                {
+                    const int iy = oy * strideH - padH + kr * dilH;
+                    for (int ox = 0; ox < outW; ++ox)
+                    {
+                        const int ix = ox * strideW - padW + kc * dilW;
+                        const int ok = iy >= 0 && iy < height && ix >= 0 && ix < width;
+                        dst[oy * outW + ox] = ok ? im[((size_t)c * height + iy) * width + ix] : 0.f;
+                    }
+                }
+            }
+}
+
+/* Gemm::cpuGemm(0,0,..,ALPHA=1,..,BETA=1,..) scalar branch -> cpuGemmNN row by row
+ * (src/core/MsnhGemm.cpp:888-935, 1071-1208): C[i][j] += A[i][k]*B[k][j], k ascending, float. */
+void msnh_or_gemm_nn(int M, int N, int K, const float *A, int lda, const float *B, int ldb, float *C, int ldc)
+{
+#pragma omp parallel for schedule(static)
+    for (int i = 0; i < M; ++i)
+        for (int k = 0; k < K; ++k)
+        {
+            const float a = A[(size_t)i * lda + k];
+            const float *b = B + (size_t)k * ldb;
+            float *c = C + (size_t)i * ldc;
+            for (int j = 0; j < N; ++j)
+                c[j] += a * b[j];
+        }
+}
+
+/* Gemm::cpuGemm(0,1,...) -> cpuGemmNT: C[i][j] += sum_k A[i][k]*B[j][k] (connected layer,
+ * src/layers/MsnhConnectedLayer.cpp:187). */
+void msnh_or_gemm_nt(int M, int N, int K, const float *A, int lda, const float *B, int ldb, float *C, int ldc)
+{
+#pragma omp parallel for schedule(static) collapse(2)
+    for (int i = 0; i < M; ++i)
+        for (int j = 0; j < N; ++j)
+        {
+            float sum = 0.f;
+            for (int k = 0; k < K; ++k)
+                sum += A[(size_t)i * lda + k] * B[(size_t)j * ldb + k];
+            C[(size_t)i * ldc + j] += sum;
+        }
+}
+
+/* Scalar activations (include/Msnhnet/layers/MsnhActivations.h:39-168). */
+static float softplus_thr(float x, float thr)
+{
+    if (x > thr) return x;
+    if (x < -thr) return expf(x);
+    return logf(expf(x) + 1);
+}
+
+float msnh_or_activate(float x, int act, float param)
+{
+    switch (act)
+    {
+    case MSNH_OR_ACT_LOGISTIC: return 1.f / (1.f + expf(-x));
+    case MSNH_OR_ACT_RELU:     return x * (x > 0);
+    case MSNH_OR_ACT_RELU6:    return (x > 0 ? x : 0) > 6 ? 6 : (x > 0 ? x : 0);
+    case MSNH_OR_ACT_LEAKY:    return (x > 0) ? x : param * x;
+    case MSNH_OR_ACT_SWISH:    return x * (1.f / (1.f + expf(-x)));
+    case MSNH_OR_ACT_MISH:     return x * tanhf(softplus_thr(x, 20.f));
+    default:                   return x;
+    }
+}
+
+void msnh_or_activate_array(float *x, long long n, int act, float param)
+{
+    if (act == MSNH_OR_ACT_NONE) return;
+#pragma omp parallel for schedule(static)
+    for (long long i = 0; i < n; ++i)
+        x[i] = msnh_or_activate(x[i], act, param);
+}
+
+/* Inference batch-norm as the reference evaluates it (src/layers/MsnhConvolutionalLayer.cpp:811-855,
+ * src/layers/MsnhBatchNormLayer.cpp:160-200): sqrtVal = sqrt(var+eps) (double sqrt of a float sum,
+ * rounded to float), scaleSqrt = g/sqrtVal, meanSqrt = -g*mean/sqrtVal, y = scaleSqrt*x + meanSqrt + b. */
+void msnh_or_bn_affine(float *x, int batch, int channels, int hw, const float *scales, const float *biases,
+                       const float *mean, const float *var, float eps)
+{
+    for (int b = 0; b < batch; ++b)
+#pragma omp parallel for schedule(static)
+        for (int c = 0; c < channels; ++c)
+        {
+            const float sqrtVal = (float)sqrt(var[c] + eps);
+            const float scaleSqrt = scales[c] / sqrtVal;
+            const float meanSqrt = -scales[c] * mean[c] / sqrtVal;
+            float *p = x + ((size_t)b * channels + c) * hw;
+            for (int i = 0; i < hw; ++i)
+                p[i] = scaleSqrt * p[i] + meanSqrt + biases[c];
+        }
+}
+
+/* ConvolutionalLayer::forward (src/layers/MsnhConvolutionalLayer.cpp:553-911): zero fill, per (batch,group)
+ * im2col (skipped for 1x1 s1 p0, :743-754) + GEMM M=filters/g N=outH*outW K=channels/g*k*k (:756),
+ * then BN or bias (:770-865), then activation (:891-900).  Output dims :388-398. */
+void msnh_or_conv(const float *in, int batch, int channels, int height, int width, const float *weights, int filters,
+                  int ksize, int stride, int pad, int dilation, int groups, const float *bn4, const float *bias,
+                  float eps, int act, float actParam, float *ws, float *out)
+{
+    const int outH = (height + 2 * pad - (dilation * (ksize - 1) + 1)) / stride + 1;
+    const int outW = (width + 2 * pad - (dilation * (ksize - 1) + 1)) / stride + 1;
+    const int m = filters / groups;
+    const int k = ksize * ksize * channels / groups;
+    const int n = outH * outW;
+    const size_t nWeights = (size_t)(channels / groups) * filters * ksize * ksize;
+    memset(out, 0, sizeof(float) * (size_t)batch * filters * n);
+    for (int b = 0; b < batch; ++b)
+        for (int g = 0; g < groups; ++g)
+        {
+            const float *a = weights + (size_t)g * nWeights / groups;
+            const float *im = in + ((size_t)b * groups + g) * (channels / groups) * height * width;
+            float *c = out + ((size_t)b * groups + g) * n * m;
+            const float *bm = im;
+            if (!(ksize == 1 && stride == 1 && pad == 0))
+            {
+                msnh_or_im2col(im, channels / groups, height, width, ksize, ksize, pad, pad, stride, stride,
+                               dilation, dilation, ws);
+                bm = ws;
+            }
+            msnh_or_gemm_nn(m, n, k, a, k, bm, n, c, n);
+        }
+    if (bn4)
+        msnh_or_bn_affine(out, batch, filters, n, bn4, bn4 + filters, bn4 + 2 * filters, bn4 + 3 * filters, eps);
+    else if (bias)
+        for (int b = 0; b < batch; ++b)
+            for (int f = 0; f < filters; ++f)
+            {
+                float *p = out + ((size_t)b * filters + f) * n;
+                for (int i = 0; i < n; ++i)
+                    p[i] += bias[f];
+            }
+    msnh_or_activate_array(out, (long long)batch * filters * n, act, actParam);
+}
+
+/* BatchNormLayer::forward (src/layers/MsnhBatchNormLayer.cpp:54-254). */
+void msnh_or_batchnorm(const float *in, int batch, int channels, int hw, const float *bn4, float eps, int act,
+                       float actParam, float *out)
+{
+    if (out != in)
+        memcpy(out, in, sizeof(float) * (size_t)batch * channels * hw);
+    msnh_or_bn_affine(out, batch, channels, hw, bn4, bn4 + channels, bn4 + 2 * channels, bn4 + 3 * channels, eps);
+    msnh_or_activate_array(out, (long long)batch * channels * hw, act, actParam);
+}
+
+/* MaxPoolLayer::forward scalar branch (src/layers/MsnhMaxPoolLayer.cpp:293-345): padding = -FLT_MAX. */
+void msnh_or_maxpool(const float *in, int batch, int channels, int height, int width, int ksize, int stride, int pad,
+                     int outH, int outW, float *out)
+{
+#pragma omp parallel for schedule(static) collapse(2)
+    for (int b = 0; b < batch; ++b)
+        for (int c = 0; c < channels; ++c)
+            for (int i = 0; i < outH; ++i)
+                for (int j = 0; j < outW; ++j)
+                {
+                    float mx = -FLT_MAX;
+                    for (int n = 0; n < ksize; ++n)
+                        for (int m = 0; m < ksize; ++m)
+                        {
+                            const int y = -pad + i * stride + n;
+                            const int x = -pad + j * stride + m;
+                            const int ok = y >= 0 && y < height && x >= 0 && x < width;
+                            const float v = ok ? in[(((size_t)b * channels + c) * height + y) * width + x] : -FLT_MAX;
+                            mx = (v > mx) ? v : mx;
+                        }
+                    out[(((size_t)b * channels + c) * outH + i) * outW + j] = mx;
+                }
+}
+
+/* LocalAvgPoolLayer::forward (src/layers/MsnhLocalAvgPoolLayer.cpp:286-344): mean over the valid
+ * window elements only, accumulated in row-major window order, divided by their count. */
+void msnh_or_avgpool(const float *in, int batch, int channels, int height, int width, int ksize, int stride, int pad,
+                     int outH, int outW, float *out)
+{
+    for (int b = 0; b < batch; ++b)
+        for (int c = 0; c < channels; ++c)
+            for (int i = 0; i < outH; ++i)
+                for (int j = 0; j < outW; ++j)
+                {
+                    float avg = 0;
+                    int counter = 0;
+                    for (int n = 0; n < ksize; ++n)
+                        for (int m = 0; m < ksize; ++m)
+                        {
+                            const int y = -pad + i * stride + n;
+                            const int x = -pad + j * stride + m;
+                            if (y >= 0 && y < height && x >= 0 && x < width)
+                            {
+                                counter++;
+                                avg += in[(((size_t)b * channels + c) * height + y) * width + x];
+                            }
+                        }
+                    out[(((size_t)b * channels + c) * outH + i) * outW + j] = avg / counter;
+                }
+}
+
+/* ConnectedLayer::forward without batch-norm (src/layers/MsnhConnectedLayer.cpp:176-240). */
+void msnh_or_connected(const float *in, int batch, int inputs, int outputs, const float *weights, const float *bias,
+                       int act, float actParam, float *out)
+{
+    memset(out, 0, sizeof(float) * (size_t)batch * outputs);
+    msnh_or_gemm_nt(batch, outputs, inputs, in, inputs, weights, inputs, out, outputs);
+    if (bias)
+        for (int b = 0; b < batch; ++b)
+            for (int o = 0; o < outputs; ++o)
+                out[(size_t)b * outputs + o] += bias[o];
+    msnh_or_activate_array(out, (long long)batch * outputs, act, actParam);
+}
+
+/* Blas::cpuUpSample (src/core/MsnhBlas.cpp:2354-2398): out[c][j][i] = scale*in[c][j/sy][i/sx]. */
+void msnh_or_upsample(const float *in, int batch, int channels, int height, int width, int strideX, int strideY,
+                      float scale, float *out)
+{
+    const int oh = height * strideY, ow = width * strideX;
+    for (int b = 0; b < batch; ++b)
+        for (int k = 0; k < channels; ++k)
+            for (int j = 0; j < oh; ++j)
+                for (int i = 0; i < ow; ++i)
+                    out[(((size_t)b * channels + k) * oh + j) * ow + i] =
+                        scale * in[(((size_t)b * channels + k) * height + j / strideY) * width + i / strideX];
+}
+
+/* Blas::cpuAxpy with unit strides (src/core/MsnhBlas.cpp:6-150): y += alpha*x. */
+void msnh_or_axpy(long long n, float alpha, const float *x, float *y)
+{
+    for (long long i = 0; i < n; ++i)
+        y[i] += alpha * x[i];
+}
+
+/* YoloLayer::forward for yolov3/yolov4 (src/layers/MsnhYoloLayer.cpp:61-142, helpers :217-284), in place:
+ * per anchor n: plane0 (sigmoid+col)*ratio, plane1 (sigmoid+row)*ratio, plane2 aw*exp, plane3 ah*exp,
+ * planes 4.. sigmoid. */
+void msnh_or_yolo_decode(float *data, int batch, int width, int height, int classNum, const float *anchors6, float ratio)
+{
+    const int hw = width * height;
+    const int per = 5 + classNum;
+    for (int b = 0; b < batch; ++b)
+        for (int n = 0; n < 3; ++n)
+        {
+            float *p = data + ((size_t)b * 3 + n) * per * hw;
+            for (int i = 0; i < hw; ++i)
+                p[i] = (1.f / (1.f + expf(-p[i])) + i % width) * ratio;
+            p += hw;
+            for (int i = 0; i < hw; ++i)
+                p[i] = (1.f / (1.f + expf(-p[i])) + i / width) * ratio;
+            p += hw;
+            for (int i = 0; i < hw; ++i)
+                p[i] = anchors6[n % 3 * 2] * expf(p[i]);
+            p += hw;
+            for (int i = 0; i < hw; ++i)
+                p[i] = anchors6[n % 3 * 2 + 1] * expf(p[i]);
+            p += hw;
+            for (long long i = 0; i < (long long)hw * (1 + classNum); ++i)
+                p[i] = 1.f / (1.f + expf(-p[i]));
+        }
+}
+
+/* Box::iou (include/Msnhnet/utils/MsnhTypes.h:104-140), including its +1 pixel convention. */
+float msnh_or_iou(const float *a, const float *b)
+{
+    const float ax1 = a[0] - a[2] / 2.f, ax2 = a[0] + a[2] / 2.f, ay1 = a[1] - a[3] / 2.f, ay2 = a[1] + a[3] / 2.f;
+    const float bx1 = b[0] - b[2] / 2.f, bx2 = b[0] + b[2] / 2.f, by1 = b[1] - b[3] / 2.f, by2 = b[1] + b[3] / 2.f;
+    /* std::max(a,b) = (a<b)?b:a ; std::min(a,b) = (b<a)?b:a  (NaN behaviour preserved) */
+    const float ix1 = (ax1 < bx1) ? bx1 : ax1;
+    const float iy1 = (ay1 < by1) ? by1 : ay1;
+    const float ix2 = (bx2 < ax2) ? bx2 : ax2;
+    const float iy2 = (by2 < ay2) ? by2 : ay2;
+    const float iw = ix2 - ix1 + 1;
+    const float ih = iy2 - iy1 + 1;
+    const float inter = (iw < 0 ? 0 : iw) * (ih < 0 ? 0 : ih);
+    const float a1 = (ax2 - ax1 + 1) * (ay2 - ay1 + 1);
+    const float a2 = (bx2 - bx1 + 1) * (by2 - by1 + 1);
+    return 1.f * inter / (a1 + a2 - inter);
+}
+
+typedef struct { float x, y, w, h, conf, best; int cls; float key; int order; } or_box;
+
+static int cmp_desc(const void *pa, const void *pb)
+{
+    const or_box *a = (const or_box *)pa, *b = (const or_box *)pb;
+    /* the reference sorts indices with the unstable std::sort on key ">" (include/Msnhnet/utils/MsnhExVector.h:58-74);
+     * ties are broken here by original order, callers compare box sets order-insensitively. */
+    if (a->key > b->key) return -1;
+    if (a->key < b->key) return 1;
+    return (a->order > b->order) - (a->order < b->order);
+}
+
+/* YoloOutLayer::forward for one image + YoloOutLayer::nms (src/layers/MsnhYoloOutLayer.cpp:79-203, 381-461):
+ * heads are visited in the given order, each transposed to [anchor][pixel][5+classes]; keep obj > confThresh;
+ * best class = first maximum; stable order by obj*bestCls descending; per class (in first-appearance order)
+ * greedy NMS picking the highest obj (first on ties) and erasing iou > nmsThresh; single-box classes pass. */
+long long msnh_or_yolo_out(const float *const *heads, const int *hw, int nHeads, int classNum, float confThresh,
+                           float nmsThresh, float *boxes, long long capBoxes)
+{
+    const int per = 5 + classNum;
+    long long total = 0;
+    for (int i = 0; i < nHeads; ++i) total += 3LL * hw[i];
+    or_box *cand = (or_box *)malloc(sizeof(or_box) * (size_t)(total > 0 ? total : 1));
+    long long n = 0;
+    for (int i = 0; i < nHeads; ++i)
+        for (int k = 0; k < 3; ++k)
+            for (int p = 0; p < hw[i]; ++p)
+            {
+                const float *base = heads[i] + (size_t)k * per * hw[i] + p;   /* element m at base[m*hw] */
+                const float obj = base[4 * (size_t)hw[i]];
+                if (obj > confThresh)
+                {
+                    or_box q;
+                    q.x = base[0]; q.y = base[(size_t)hw[i]]; q.w = base[2 * (size_t)hw[i]]; q.h = base[3 * (size_t)hw[i]];
+                    q.conf = obj;
+                    int best = 0;
+                    float bv = base[5 * (size_t)hw[i]];
+                    for (int m = 1; m < classNum; ++m)
+                    {
+                        const float v = base[(size_t)(5 + m) * hw[i]];
+                        if (bv < v) { bv = v; best = m; }      /* std::max_element: first maximum */
+                    }
+                    q.best = bv; q.cls = best; q.key = q.conf * q.best; q.order = (int)n;
+                    cand[n++] = q;
+                }
+            }
+    if (n > 0) qsort(cand, (size_t)n, sizeof(or_box), cmp_desc);
+
+    long long nOut = 0;
+    char *done = (char *)calloc((size_t)(n > 0 ? n : 1), 1);       /* class already processed */
+    or_box *cls = (or_box *)malloc(sizeof(or_box) * (size_t)(n > 0 ? n : 1));
+    for (long long i = 0; i < n; ++i)
+    {
+        if (done[i]) continue;
+        const int c = cand[i].cls;
+        long long m = 0;
+        for (long long j = i; j < n; ++j)
+            if (cand[j].cls == c) { cls[m++] = cand[j]; done[j] = 1; }
+        if (m == 1)
+        {
+            if (nOut < capBoxes && boxes)
+            {
+                float *o = boxes + 7 * nOut;
+                o[0] = cls[0].x; o[1] = cls[0].y; o[2] = cls[0].w; o[3] = cls[0].h; o[4] = cls[0].conf; o[5] = cls[0].best; o[6] = (float)c;
+            }
+            nOut++;
+            continue;
+        }
+        while (m > 0)
+        {
+            long long bi = 0;
+            float bc = -FLT_MAX;
+            for (long long j = 0; j < m; ++j)
+                if (cls[j].conf > bc) { bi = j; bc = cls[j].conf; }
+            const or_box best = cls[bi];
+            if (nOut < capBoxes && boxes)
+            {
+                float *o = boxes + 7 * nOut;
+                o[0] = best.x; o[1] = best.y; o[2] = best.w; o[3] = best.h; o[4] = best.conf; o[5] = best.best; o[6] = (float)c;
+            }
+            nOut++;
+            memmove(cls + bi, cls + bi + 1, sizeof(or_box) * (size_t)(m - bi - 1));
+            m--;
+            long long w = 0;
+            for (long long j = 0; j < m; ++j)
+            {
+                const float iou = msnh_or_iou(&cls[j].x, &best.x);
+                if (!(iou > nmsThresh)) cls[w++] = cls[j];
+            }
+            m = w;
+        }
+    }
+    free(cls); free(done); free(cand);
+    return nOut;
+}

@@ -1,0 +1,139 @@
+"""GPU parity of msnh_hip_conv2d (every algorithm) against the plain-C oracle convolution.
+
+Tolerances: float32 1e-5 of max|ref| (only the accumulation order differs); float16 2e-3 of max|ref| with the
+oracle fed the same float16-rounded inputs and weights (accumulation is float32, the output is rounded once)."""
+import numpy as np
+import pytest
+
+import msnh_oracle_net as on
+from msnhnet_amd import hipabi as abi
+
+pytestmark = pytest.mark.gpu
+
+TOL = {abi.F32: 1e-5, abi.F16: 2e-3}
+
+
+def _case(rng, b, c, h, w, oc, k, groups=1):
+    x = rng.standard_normal((b, c, h, w), dtype=np.float32)
+    wt = rng.standard_normal((oc, c // groups, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (c // groups * k * k)))
+    return x, wt
+
+
+def _ref(x, wt, stride, pad, dil, groups, scale, shift, act, act_param, residual, act2, res_mul, out_mul):
+    oc, _, k, _ = wt.shape
+    y = on.conv(x, wt, oc, k, stride, pad, dil, groups)
+    if scale is not None:
+        y = y * scale.reshape(1, -1, 1, 1)
+    if shift is not None:
+        y = y + shift.reshape(1, -1, 1, 1)
+    y = on.activate(y.astype(np.float32), act, act_param)
+    if residual is not None:
+        y = on.activate((y + np.float32(res_mul) * residual).astype(np.float32), act2, 0.1)
+    return (np.float32(out_mul) * y).astype(np.float32)
+
+
+CASES = [
+    # b, c, h, w, oc, k, stride, pad, dil, groups
+    (2, 16, 13, 11, 40, 3, 1, 1, 1, 1),
+    (1, 32, 19, 19, 255, 1, 1, 0, 1, 1),
+    (2, 24, 17, 15, 48, 3, 2, 1, 1, 1),
+    (1, 16, 20, 20, 32, 3, 1, 2, 2, 1),
+    (2, 32, 9, 9, 64, 3, 1, 1, 1, 2),
+    (1, 64, 14, 14, 128, 3, 1, 1, 1, 1),
+    (3, 128, 7, 7, 96, 1, 1, 0, 1, 1),
+    (1, 8, 5, 5, 8, 5, 1, 2, 1, 1),
+    (1, 72, 10, 12, 200, 3, 1, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("dtype", [abi.F32, abi.F16])
+@pytest.mark.parametrize("algo", ["igemm", "direct"])
+@pytest.mark.parametrize("case", CASES)
+def test_conv_plain(case, algo, dtype):
+    import gpuutil as gu
+    b, c, h, w, oc, k, stride, pad, dil, groups = case
+    rng = np.random.default_rng(hash(case) % (2 ** 31))
+    x, wt = _case(rng, b, c, h, w, oc, k, groups)
+    if dtype == abi.F16:
+        x, wt = gu.round_f16(x), gu.round_f16(wt)
+    print("case", case, algo, dtype, flush=True)
+    y, used = gu.conv2d(x, wt, dtype=dtype, stride=stride, pad=pad, dil=dil, groups=groups, algo=algo)
+    assert used == algo
+    ref = _ref(x, wt, stride, pad, dil, groups, None, None, "none", 0.1, None, "none", 1.0, 1.0)
+    assert gu.rel_err(y, ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", [abi.F32, abi.F16])
+@pytest.mark.parametrize("algo", ["igemm", "direct"])
+@pytest.mark.parametrize("act,act2", [("leaky", "none"), ("none", "relu"), ("mish", "none"), ("relu6", "leaky"), ("swish", "none")])
+def test_conv_epilogue(act, act2, algo, dtype):
+    """folded batch-norm, activation, residual add + second activation, power-of-two scales, channel-slice output."""
+    import gpuutil as gu
+    rng = np.random.default_rng(7)
+    x, wt = _case(rng, 2, 32, 12, 10, 48, 3)
+    res = rng.standard_normal((2, 48, 12, 10), dtype=np.float32)
+    scale = rng.uniform(0.5, 1.5, 48).astype(np.float32)
+    shift = (rng.standard_normal(48) * 0.1).astype(np.float32)
+    if dtype == abi.F16:
+        x, wt, res = gu.round_f16(x), gu.round_f16(wt), gu.round_f16(res)
+    print("epilogue", act, act2, algo, dtype, flush=True)
+    y, _ = gu.conv2d(x, wt, dtype=dtype, stride=1, pad=1, scale=scale, shift=shift, act=act, residual=res, act2=act2,
+                     res_mul=4.0, out_mul=0.25, algo=algo, in_ld=40, out_ld=64, res_ld=56)
+    ref = _ref(x, wt, 1, 1, 1, 1, scale, shift, act, 0.1, res, act2, 4.0, 0.25)
+    assert gu.rel_err(y, ref) <= TOL[dtype]
+
+
+def test_conv_f16_in_f32_out():
+    import gpuutil as gu
+    rng = np.random.default_rng(11)
+    x, wt = _case(rng, 2, 64, 8, 8, 255, 1)
+    x, wt = gu.round_f16(x), gu.round_f16(wt)
+    bias = rng.standard_normal(255).astype(np.float32)
+    y, used = gu.conv2d(x, wt, dtype=abi.F16, out_dtype=abi.F32, shift=bias, out_ld=256)
+    assert used == "igemm"
+    ref = _ref(x, wt, 1, 0, 1, 1, None, bias, "none", 0.1, None, "none", 1.0, 1.0)
+    assert gu.rel_err(y, ref) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", [abi.F32, abi.F16])
+@pytest.mark.parametrize("c,h,w,k,stride,pad", [(32, 14, 14, 3, 1, 1), (96, 15, 13, 3, 2, 1), (20, 9, 9, 3, 1, 1), (16, 8, 8, 5, 1, 2)])
+def test_conv_depthwise(c, h, w, k, stride, pad, dtype):
+    import gpuutil as gu
+    rng = np.random.default_rng(c)
+    x, wt = _case(rng, 2, c, h, w, c, k, groups=c)
+    scale = rng.uniform(0.5, 1.5, c).astype(np.float32)
+    shift = (rng.standard_normal(c) * 0.1).astype(np.float32)
+    if dtype == abi.F16:
+        x, wt = gu.round_f16(x), gu.round_f16(wt)
+    y, used = gu.conv2d(x, wt, dtype=dtype, stride=stride, pad=pad, groups=c, scale=scale, shift=shift, act="relu6")
+    assert used == "depthwise"
+    ref = _ref(x, wt, stride, pad, 1, c, scale, shift, "relu6", 0.1, None, "none", 1.0, 1.0)
+    assert gu.rel_err(y, ref) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("out_dtype", [abi.F32, abi.F16])
+@pytest.mark.parametrize("h,w,oc,k,stride,pad", [(33, 31, 32, 3, 1, 1), (40, 40, 64, 7, 2, 3), (25, 27, 32, 3, 2, 1)])
+def test_conv_stem(h, w, oc, k, stride, pad, out_dtype):
+    """first layer: NCHW float32 in, NHWC out, cast fused"""
+    import gpuutil as gu
+    rng = np.random.default_rng(oc + k)
+    x = rng.random((2, 3, h, w), dtype=np.float32)
+    wt = rng.standard_normal((oc, 3, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (3 * k * k)))
+    scale = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    shift = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    y, used = gu.conv2d(x, wt, dtype=out_dtype, stride=stride, pad=pad, scale=scale, shift=shift, act="leaky")
+    assert used == "stem"
+    ref = _ref(x, wt, stride, pad, 1, 1, scale, shift, "leaky", 0.1, None, "none", 1.0, 1.0)
+    assert gu.rel_err(y, ref) <= (1e-5 if out_dtype == abi.F32 else 1e-3)
+
+
+def test_conv_rejects_bad_shapes():
+    import ctypes
+    import gpuutil as gu
+    gu.init()
+    L = abi.lib()
+    d = abi.ConvDesc(abi.F16, abi.F16, 1, 8, 8, 12, 12, 16, 8, 8, 16, 3, 1, 1, 1, 1, 22, 0.1, 0, 16, 22, 0.1, 1.0, 1.0, abi.ALGO["igemm"])
+    assert L.msnh_hip_conv2d(ctypes.byref(d), 16, 16, None, None, None, 16, None, 0, None) != 0      # in_c % 8
+    assert b"IGEMM" in L.msnh_hip_last_error()
+    d = abi.ConvDesc(abi.F16, abi.F16, 1, 8, 8, 16, 16, 16, 9, 8, 16, 3, 1, 1, 1, 1, 22, 0.1, 0, 16, 22, 0.1, 1.0, 1.0, 0)
+    assert L.msnh_hip_conv2d(ctypes.byref(d), 16, 16, None, None, None, 16, None, 0, None) != 0      # wrong out_h
