@@ -188,14 +188,28 @@ int msnh_hip_nhwc_to_nchw(int dtype, int batch, int c, int h, int w, const void 
  * YoloOutLayer::forwardGPU's shuffleDataKernel + candidate threshold (src/layers/cuda/MsnhYoloOutLayerGPU.cu:5-21,
  * src/layers/MsnhYoloOutLayer.cpp:216-260).
  *   x        : head logits NHWC, channel = anchor*(5+classes)+m, times x_mul gives the true logit
- *   decoded  : float32 [batch][3][h*w][5+classes]  (the reference's "shuffled" order), may not be NULL
+ *   decoded  : float32, element (b,anchor,pixel,m) at decoded[b*decoded_batch_stride + ((anchor*h*w)+pixel)*(5+classes) + m]
+ *              (the reference's "shuffled" order; the stride lets all heads of an image share one buffer)
  *   cand_idx : optional int32 [batch][cand_cap]; receives (anchor*h*w + pixel) + cand_base of every entry
  *              with objectness > conf_thresh, in no particular order;
  *   cand_cnt : int32 [batch], incremented by the number of entries found (caller zeroes it).
  * ---------------------------------------------------------------------------------------------- */
 int msnh_hip_yolo_decode(int dtype, int batch, int h, int w, int classes, const void *x, int x_ld, float x_mul,
-                         const float *anchors6, float ratio, float *decoded, float conf_thresh, int *cand_idx,
-                         int cand_cap, int cand_base, int *cand_cnt, msnh_stream_t s);
+                         const float *anchors6, float ratio, float *decoded, long long decoded_batch_stride,
+                         float conf_thresh, int *cand_idx, int cand_cap, int cand_base, int *cand_cnt, msnh_stream_t s);
+/* Candidate compaction for YoloOutLayer (the per-box part of src/layers/MsnhYoloOutLayer.cpp:120-170 done on
+ * the device so that only surviving boxes cross PCIe): for image b and k < min(cand_cnt[b], cand_cap) reads
+ * the decoded row of cell cand_idx[b][k] (rows are `5+classes` floats, row r of image b at
+ * decoded + b*decoded_batch_stride + r*(5+classes)) and writes rows[b][k][0..7] =
+ * { x, y, w, h, objectness, best class score, best class index, cell index } (the two indices as float;
+ * best class = first maximum like std::max_element). */
+int msnh_hip_yolo_gather(int batch, int classes, const float *decoded, long long decoded_batch_stride, const int *cand_idx,
+                         int cand_cap, const int *cand_cnt, float *rows, msnh_stream_t s);
+
+/* max |x| over the finite elements of an NHWC tensor, combined into *result with an atomic max
+ * (caller zeroes *result).  Used once at load time to calibrate the power-of-two activation scales of the
+ * float16 plan; no counterpart in the reference. */
+int msnh_hip_absmax(int dtype, long long pixels, int c, const void *x, int x_ld, float *result, msnh_stream_t s);
 
 #ifdef __cplusplus
 }

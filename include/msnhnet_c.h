@@ -1,0 +1,94 @@
+/*
+ * msnhnet_c.h -- C ABI of the host library `libMsnhnet.so` (NetBuilder build / load / run).
+ *
+ * Part 1 keeps the names and argument meaning of the reference's C facade (src/c_api/MsnhnetLib.h:39-61), which
+ * drives one process-wide network.  Part 2 is a handle-based variant of the same calls (several networks,
+ * batches, per-layer dumps, device-resident inputs) used by the tests and the benchmark.
+ * All functions return 1 on success and -1 on failure like the reference's (MsnhnetLib.cpp:10-35) unless stated;
+ * the message of the last failure is kept in static storage (the reference returns a pointer into a destroyed
+ * local, src/c_api/MsnhnetLib.cpp:29-31).
+ */
+#ifndef MSNHNET_C_H
+#define MSNHNET_C_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MSNHNET_MAX_BBOX 1024          /* MaxBBoxNum, src/c_api/MsnhnetLib.h:9 */
+
+typedef struct BBox                    /* src/c_api/MsnhnetLib.h:22-32 */
+{
+    float    x, y, w, h;
+    float    conf;
+    float    bestClsConf;
+    uint32_t bestClsIdx;
+    float    angle;
+} BBox;
+
+typedef struct BBoxContainer           /* src/c_api/MsnhnetLib.h:34-37 */
+{
+    BBox boxes[MSNHNET_MAX_BBOX];
+} BBoxContainer;
+
+/* ---- part 1: the reference facade -------------------------------------------------------------------------------- */
+int initMsnhnet(void);                                                                  /* MsnhnetLib.h:39 */
+int buildMsnhnet(char **msg, const char *msnhnet, const char *msnhbin, int useFp16, int useCudaOnly);   /* :40 */
+/* data = one CHW float image (or batch*CHW when the graph's batch > 1); runGPU must be non-zero: the CPU path
+ * does not exist in this build and runGPU == 0 fails with "Gpu mode , can not run with cpu".            :49 */
+int runClassifyNoPred(char **msg, const float *data, const int len, int *bestIndex, int runGPU);
+/* Same contract for detection networks; fills at most MSNHNET_MAX_BBOX boxes of image 0.  The reference only
+ * offers the image-file / byte-image variants (runYoloFile / runYoloList, :51-54), whose pre-processing lives in
+ * its CV module outside the convolutional path. */
+int runYoloNoPred(char **msg, const float *data, const int len, BBoxContainer *bboxContainer, int *detectedNum, int runGPU);
+int dispose(void);                                                                      /* :56 */
+int withGPU(int *GPU);                                                                  /* :57 */
+int withCUDNN(int *CUDNN);                                                              /* :58, always 0 */
+int getCpuForwardTime(float *time);                                                     /* :59 */
+int getGpuForwardTime(float *time);                                                     /* :60 */
+int getInputDim(int *width, int *heigth, int *channel);                                 /* :61 */
+
+/* ---- part 2: handle-based API (0 = success, non-zero = failure; text via msnhnet_last_error) --------------------------- */
+typedef void *msnhnet_t;
+const char *msnhnet_last_error(void);
+int msnhnet_create(msnhnet_t *net);                       /* NetBuilder() */
+int msnhnet_destroy(msnhnet_t net);
+int msnhnet_set_use_fp16(int on);                         /* NetBuilder::setUseFp16, process-wide, before build */
+int msnhnet_set_keep_class_scores(int on);
+int msnhnet_set_save_layer_output(msnhnet_t net, int on); /* NetBuilder::setSaveLayerOutput */
+int msnhnet_build(msnhnet_t net, const char *msnhnet_path);      /* NetBuilder::buildNetFromMsnhNet */
+int msnhnet_load(msnhnet_t net, const char *msnhbin_path);       /* NetBuilder::loadWeightsFromMsnhBin */
+int msnhnet_load_from_memory(msnhnet_t net, const float *weights, size_t count);
+int msnhnet_input_dims(msnhnet_t net, int *batch, int *channels, int *height, int *width);
+int msnhnet_num_layers(msnhnet_t net);
+/* info[0..9] = type, outH, outW, outC, outputNum, inputNum, numWeights, memReUse, batch, activation */
+int msnhnet_layer_info(msnhnet_t net, int layer, long long *info, char *name, int name_cap);
+long long msnhnet_layer_detail(msnhnet_t net, char *dst, long long cap);      /* returns the full length */
+long long msnhnet_plan_detail(msnhnet_t net, char *dst, long long cap);
+double msnhnet_conv_flops(msnhnet_t net);
+/* NetBuilder::runClassify / runYolo (CPU): always fail with "Gpu mode , can not run with cpu". */
+int msnhnet_run_classify(msnhnet_t net, const float *img, long long n, float *out, long long cap, long long *n_out);
+/* NetBuilder::runClassifyGPU: img = batch*C*H*W floats; out receives batch*outputNum floats. */
+int msnhnet_run_classify_gpu(msnhnet_t net, const float *img, long long n, float *out, long long cap, long long *n_out);
+/* NetBuilder::runYoloGPU: counts[b] = boxes of image b; boxes = rows of 7 floats (x y w h conf bestClsConf
+ * bestClsIdx), images back to back, at most cap_boxes rows are written; *total = sum of counts. */
+int msnhnet_run_yolo_gpu(msnhnet_t net, const float *img, long long n, int *counts, float *boxes, long long cap_boxes, long long *total);
+/* Output of top-level layer `layer` from the last run with layer dumps on (batch-major NCHW). Returns its length. */
+long long msnhnet_layer_output(msnhnet_t net, int layer, float *dst, long long cap);
+/* Device-resident serving path: write the batch into the buffer returned by msnhnet_device_input (device memory,
+ * NCHW float32) or pass another device pointer, enqueue, then sync / fetch. */
+int msnhnet_device_input(msnhnet_t net, float **device_ptr);
+int msnhnet_enqueue(msnhnet_t net, const float *device_input);
+int msnhnet_sync(msnhnet_t net);
+int msnhnet_fetch_classify(msnhnet_t net, float *out, long long cap, long long *n_out);
+int msnhnet_fetch_yolo(msnhnet_t net, int *counts, float *boxes, long long cap_boxes, long long *total);
+float msnhnet_gpu_inference_time(msnhnet_t net);          /* NetBuilder::getGpuInferenceTime, ms */
+long long msnhnet_time_detail(msnhnet_t net, char *dst, long long cap);       /* NetBuilder::getTimeDetail */
+
+#ifdef __cplusplus
+}
+#endif
+#endif

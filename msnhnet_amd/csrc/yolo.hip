@@ -9,7 +9,7 @@ struct Anchors { float v[6]; };
 
 template <typename T>
 __global__ __launch_bounds__(256) void yoloDecodeKernel(const T *__restrict__ x, int xLd, float xMul, Anchors an, float ratio,
-                                                        float *__restrict__ decoded, float confThresh, int *__restrict__ candIdx,
+                                                        float *__restrict__ decoded, long long decStride, float confThresh, int *__restrict__ candIdx,
                                                         int candCap, int candBase, int *__restrict__ candCnt, int W, int HW, int per,
                                                         long long total)
 {
@@ -28,7 +28,7 @@ __global__ __launch_bounds__(256) void yoloDecodeKernel(const T *__restrict__ x,
     else if (m == 2) r = an.v[2 * a] * expf(v);
     else if (m == 3) r = an.v[2 * a + 1] * expf(v);
     else             r = 1.f / (1.f + expf(-v));
-    decoded[idx] = r;
+    decoded[static_cast<size_t>(b) * decStride + (static_cast<size_t>(a) * HW + p) * per + m] = r;
     if (m == 4 && candIdx != nullptr && r > confThresh)
     {
         const int pos = atomicAdd(candCnt + b, 1);
@@ -36,18 +36,64 @@ __global__ __launch_bounds__(256) void yoloDecodeKernel(const T *__restrict__ x,
     }
 }
 
+__global__ __launch_bounds__(256) void yoloGatherKernel(const float *__restrict__ decoded, long long decStride, const int *__restrict__ candIdx,
+                                                        int candCap, const int *__restrict__ candCnt, float *__restrict__ rows, int per,
+                                                        int batch)
+{
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    const int b = blockIdx.y;
+    if (b >= batch) return;
+    int n = candCnt[b];
+    n = n < candCap ? n : candCap;
+    if (k >= n) return;
+    const int cell = candIdx[static_cast<size_t>(b) * candCap + k];
+    const float *r = decoded + static_cast<size_t>(b) * decStride + static_cast<size_t>(cell) * per;
+    int best = 0;
+    float bv = r[5];
+    for (int m = 1; m < per - 5; ++m)
+    {
+        const float v = r[5 + m];
+        if (bv < v) { bv = v; best = m; }
+    }
+    float *o = rows + (static_cast<size_t>(b) * candCap + k) * 8;
+    o[0] = r[0]; o[1] = r[1]; o[2] = r[2]; o[3] = r[3]; o[4] = r[4];
+    o[5] = bv; o[6] = static_cast<float>(best); o[7] = static_cast<float>(cell);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void absMaxKernel(const T *__restrict__ x, int xLd, int c, long long total, float *__restrict__ result)
+{
+    float m = 0.f;
+    for (long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+         idx += static_cast<long long>(gridDim.x) * blockDim.x)
+    {
+        const long long p = idx / c;
+        const int ch = static_cast<int>(idx - p * c);
+        const float v = fabsf(toF(x[p * xLd + ch]));
+        if (v <= FLT_MAX && v > m) m = v;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1)
+    {
+        const float o = __shfl_xor(m, off, 64);
+        m = o > m ? o : m;
+    }
+    if ((threadIdx.x & 63) == 0 && m > 0.f) atomicMax(reinterpret_cast<int *>(result), __float_as_int(m));
+}
+
 } // namespace msnh
 
 using namespace msnh;
 
 extern "C" int msnh_hip_yolo_decode(int dtype, int batch, int h, int w, int classes, const void *x, int x_ld, float x_mul,
-                                    const float *anchors6, float ratio, float *decoded, float conf_thresh, int *cand_idx,
-                                    int cand_cap, int cand_base, int *cand_cnt, msnh_stream_t s)
+                                    const float *anchors6, float ratio, float *decoded, long long decoded_batch_stride,
+                                    float conf_thresh, int *cand_idx, int cand_cap, int cand_base, int *cand_cnt, msnh_stream_t s)
 {
     MSNH_REQUIRE(dtypeOk(dtype), "yolo_decode: bad dtype");
     MSNH_REQUIRE(batch > 0 && h > 0 && w > 0 && classes > 0, "yolo_decode: bad geometry");
     const int per = 5 + classes;
     MSNH_REQUIRE(x && decoded && anchors6 && x_ld >= 3 * per, "yolo_decode: bad argument");
+    MSNH_REQUIRE(decoded_batch_stride >= static_cast<long long>(3) * h * w * per, "yolo_decode: decoded_batch_stride too small");
     MSNH_REQUIRE(cand_idx == nullptr || (cand_cnt != nullptr && cand_cap > 0), "yolo_decode: candidate list without counter");
     Anchors an;
     for (int i = 0; i < 6; ++i) an.v[i] = anchors6[i];
@@ -56,10 +102,38 @@ extern "C" int msnh_hip_yolo_decode(int dtype, int batch, int h, int w, int clas
     hipStream_t st = resolveStream(s);
     if (dtype == MSNH_F16)
         hipLaunchKernelGGL((yoloDecodeKernel<f16>), grid, dim3(256), 0, st, static_cast<const f16 *>(x), x_ld, x_mul, an, ratio, decoded,
-                           conf_thresh, cand_idx, cand_cap, cand_base, cand_cnt, w, h * w, per, total);
+                           decoded_batch_stride, conf_thresh, cand_idx, cand_cap, cand_base, cand_cnt, w, h * w, per, total);
     else
         hipLaunchKernelGGL((yoloDecodeKernel<float>), grid, dim3(256), 0, st, static_cast<const float *>(x), x_ld, x_mul, an, ratio,
-                           decoded, conf_thresh, cand_idx, cand_cap, cand_base, cand_cnt, w, h * w, per, total);
+                           decoded, decoded_batch_stride, conf_thresh, cand_idx, cand_cap, cand_base, cand_cnt, w, h * w, per, total);
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int msnh_hip_yolo_gather(int batch, int classes, const float *decoded, long long decoded_batch_stride, const int *cand_idx,
+                                    int cand_cap, const int *cand_cnt, float *rows, msnh_stream_t s)
+{
+    MSNH_REQUIRE(batch > 0 && batch <= 65535 && classes > 0 && cand_cap > 0, "yolo_gather: bad geometry");
+    MSNH_REQUIRE(decoded && cand_idx && cand_cnt && rows, "yolo_gather: NULL pointer");
+    dim3 grid(gridFor(cand_cap, 256), batch);
+    hipLaunchKernelGGL(yoloGatherKernel, grid, dim3(256), 0, resolveStream(s), decoded, decoded_batch_stride, cand_idx, cand_cap, cand_cnt,
+                       rows, 5 + classes, batch);
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int msnh_hip_absmax(int dtype, long long pixels, int c, const void *x, int x_ld, float *result, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "absmax: bad dtype");
+    MSNH_REQUIRE(pixels > 0 && c > 0 && x && result && x_ld >= c, "absmax: bad argument");
+    const long long total = pixels * c;
+    long long blocks = (total + 255) / 256;
+    if (blocks > 2048) blocks = 2048;
+    dim3 grid(static_cast<unsigned>(blocks));
+    if (dtype == MSNH_F16)
+        hipLaunchKernelGGL((absMaxKernel<f16>), grid, dim3(256), 0, resolveStream(s), static_cast<const f16 *>(x), x_ld, c, total, result);
+    else
+        hipLaunchKernelGGL((absMaxKernel<float>), grid, dim3(256), 0, resolveStream(s), static_cast<const float *>(x), x_ld, c, total, result);
     MSNH_LAUNCH_CHECK();
     return 0;
 }

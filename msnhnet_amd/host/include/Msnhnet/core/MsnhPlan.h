@@ -1,0 +1,127 @@
+// The device plan of one network: the flat list of kernel launches ("ops") a graph lowers to, the tensors
+// they read and write, and the single device arena those tensors are placed in.
+//
+// The reference allocates per layer: two ping-pong pools sized for the largest output plus an own buffer
+// for every layer that is re-read later (src/net/MsnhNetBuilder.cpp:539-589), and its block layers
+// malloc/free a copy of their input on every forward (src/layers/MsnhResBlockLayer.cpp:319,391).  Here the
+// whole graph -- block internals included -- is lowered once, then
+//   1. fused   : conv + stand-alone batch-norm, conv + residual add (+ block activation) become one launch;
+//   2. aliased : route / concat-block inputs are placed directly inside the concatenated tensor (a channel
+//                slice with a larger pixel stride), so the concat copy disappears;
+//   3. scaled  : for float16, one float32 calibration pass fixes a power-of-two scale per tensor so that
+//                activations far outside the half range still fit (the scale is applied exactly in the
+//                float32 epilogues);
+//   4. placed  : tensor lifetimes over the op list drive a first-fit assignment of arena offsets.
+#pragma once
+#include <array>
+#include <memory>
+#include <string>
+#include <vector>
+#include "Msnhnet/config/MsnhnetCfg.h"
+#include "Msnhnet/core/MsnhDevice.h"
+
+namespace Msnhnet
+{
+class BaseLayer;
+
+struct PlanTensor
+{
+    enum Layout { NHWC = 0, NCHW_INPUT, FLAT };
+    int  n = 0, h = 0, w = 0, c = 0;
+    int  dtype = MSNH_F32;
+    Layout layout = NHWC;
+    int  parent = -1;          // >= 0: this tensor is channels [chanOffset, chanOffset+c) of `parent`
+    int  chanOffset = 0;
+    int  scaleExp = 0;         // stored value = true value * 2^-scaleExp
+    bool pinned = false;       // must stay a real tensor (top-level outputs while layer dumps are on, ...)
+    bool persistent = false;   // must survive until the end of the forward
+    int  ld = 0;               // pixel stride in elements (root tensors)
+    size_t bytes = 0;          // root tensors
+    size_t offset = 0;         // arena offset (root tensors)
+    bool external = false;     // storage provided outside the arena (the network input)
+    void *extPtr = nullptr;
+    float amax = 0.f;          // calibration result
+    std::string name;
+    size_t elems() const { return static_cast<size_t>(n) * h * w * c; }
+    long long pixels() const { return static_cast<long long>(n) * h * w; }
+};
+
+struct PlanOp
+{
+    enum Kind { CONV = 0, AFFINE, ADD, COPY, MAXPOOL, AVGPOOL, UPSAMPLE, CONNECTED, INPUT_CAST, YOLO_DECODE };
+    Kind kind = CONV;
+    int  in0 = -1, in1 = -1, out = -1;
+    bool dead = false;
+    int  layerIndex = -1;      // top-level layer this op belongs to
+    std::string name;
+
+    // geometry / epilogue
+    int  ksize = 1, stride = 1, pad = 0, dilation = 1, groups = 1;
+    ActivationType act = NONE, act2 = NONE;
+    float actParam = 0.1f, act2Param = 0.1f;
+    float upScale = 1.f;
+    int  dstChanOffset = 0;                 // COPY: channel offset inside `out`
+    int  algo = MSNH_CONV_AUTO;             // CONV: resolved at weight preparation
+    BaseLayer *src = nullptr;               // layer that owns the host weights of this op
+    BaseLayer *src2 = nullptr;              // batch-norm layer folded into a CONV
+
+    // YOLO_DECODE
+    std::array<float, 6> anchors{};
+    int   classes = 0;
+    float ratio = 1.f;
+    int   cellBase = 0;                     // first cell of this head inside an image's decoded rows
+    float confThresh = 0.f;
+
+    // device-side constants, filled by Plan::prepareWeights
+    DeviceBuffer wDev, scaleDev, shiftDev;
+    double flops = 0;                       // 2*MACs of this launch (conv / connected)
+};
+
+class Plan
+{
+public:
+    explicit Plan(int dtype) : computeDtype(dtype) {}
+
+    int computeDtype;
+    std::vector<PlanTensor> tensors;
+    std::vector<PlanOp>     ops;
+    std::vector<int>        layerOut;       // output tensor of each top-level layer
+    int inputTensor = -1;
+
+    // YOLO post-processing buffers (only for networks ending in a yoloout layer)
+    int  yoloCells = 0;                     // sum over heads of 3*H*W
+    int  yoloClasses = 0;
+    DeviceBuffer yoloDecoded, yoloCandIdx, yoloCandCnt, yoloRows;
+
+    int addTensor(int n, int h, int w, int c, int dtype, const std::string &name, PlanTensor::Layout layout = PlanTensor::NHWC);
+    PlanOp &addOp(PlanOp::Kind kind, int in0, int in1, int out, int layerIndex, const std::string &name);
+    int producerOf(int tensor) const;       // last live op writing `tensor`, or -1
+    int consumerCount(int tensor) const;
+
+    void fuse();                            // passes 1
+    void aliasConcats();                    // pass 2
+    void applyCalibration(const Plan &calibrated);   // pass 3: take amax from an executed float32 twin
+    void place();                           // pass 4 + arena allocation
+    void prepareWeights();                  // fold batch-norm, pick algorithms, pack and upload weights
+    void run(size_t opBegin, size_t opEnd, msnh_stream_t s);
+    void runAll(msnh_stream_t s) { run(0, ops.size(), s); }
+    void measureAmax(msnh_stream_t s);      // after an eager run: absmax of every live NHWC tensor
+
+    int   root(int t) const;
+    int   chanOffsetInRoot(int t) const;
+    void *ptr(int t) const;
+    int   ld(int t) const { return tensors[static_cast<size_t>(root(t))].ld; }
+    float mulOf(int t) const;               // 2^scaleExp
+    // Copies tensor `t` to the host as batch-major NCHW float32 true values.
+    void  exportTensor(int t, std::vector<float> &dst, msnh_stream_t s);
+
+    size_t arenaBytes() const { return _arena.bytes(); }
+    size_t liveOps() const;
+    double totalConvFlops() const;
+    std::string describe() const;           // one line per live op: kind, shapes, algorithm
+
+private:
+    void launch(PlanOp &op, msnh_stream_t s);
+    DeviceBuffer _arena, _exportScratch;
+};
+}

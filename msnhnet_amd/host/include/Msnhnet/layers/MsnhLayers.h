@@ -1,0 +1,260 @@
+// The concrete layer classes of the convolutional path.  Constructor parameter lists are the reference's
+// (so code that builds layers by hand keeps compiling); see the per-class citations.
+#pragma once
+#include "Msnhnet/io/MsnhParser.h"
+#include "Msnhnet/layers/MsnhBaseLayer.h"
+#include "Msnhnet/layers/MsnhYoloDef.h"
+
+namespace Msnhnet
+{
+class NetBuildParams
+{
+public:
+    int batch = 0, inputNums = 0, height = 0, width = 0, channels = 0;
+};
+
+// src/layers/MsnhConvolutionalLayer.cpp:5-319 (ctor, shapes, weight count), :1186-1434 (weights)
+class MsnhNet_API ConvolutionalLayer : public BaseLayer
+{
+public:
+    ConvolutionalLayer(const int &batch, const int &steps, const int &height, const int &width, const int &channel, const int &num,
+                       const int &groups, const int &kSizeX, const int &kSizeY, const int &strideX, const int &strideY,
+                       const int &dilationX, const int &dilationY, const int &paddingX, const int &paddingY,
+                       ActivationType activation, const std::vector<float> &actParams, const int &batchNorm, const float &bnEps,
+                       const int &useBias, const int &binary, const int &xnor, const int &useBinOutput, const int &groupIndex,
+                       const int &antialiasing, ConvolutionalLayer *const &shareLayer, const int &assistedExcitation, const int &deform);
+    int convOutHeight() const;
+    int convOutWidth() const;
+    void loadAllWeigths(std::vector<float> &weights) override;
+    int lower(Plan &plan, int in, int layerIndex) override;
+    const std::vector<float> &kernelWeights() const override { return _weights; }
+    void foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const override;
+
+    int getKSizeX() const { return _kSizeX; }
+    int getKSizeY() const { return _kSizeY; }
+    int getStride() const { return _strideX; }
+    int getStrideX() const { return _strideX; }
+    int getStrideY() const { return _strideY; }
+    int getPaddingX() const { return _paddingX; }
+    int getPaddingY() const { return _paddingY; }
+    int getDilationX() const { return _dilationX; }
+    int getDilationY() const { return _dilationY; }
+    int getGroups() const { return _groups; }
+    int getBatchNorm() const { return _batchNorm; }
+    int getUseBias() const { return _useBias; }
+    int getNBiases() const { return _nBiases; }
+    int getNWeights() const { return _nWeights; }
+    int getNScales() const { return _nScales; }
+    int getNRollMean() const { return _nRollMean; }
+    int getNRollVariance() const { return _nRollVariance; }
+
+private:
+    int _groups = 1, _kSizeX = 1, _kSizeY = 1, _strideX = 1, _strideY = 1, _dilationX = 1, _dilationY = 1, _paddingX = 0, _paddingY = 0;
+    int _batchNorm = 0, _useBias = 1;
+    float _bnEps = 0.00001f;
+    int _nWeights = 0, _nBiases = 0, _nScales = 0, _nRollMean = 0, _nRollVariance = 0;
+    std::vector<float> _weights, _biases, _scales, _rollMean, _rollVariance;
+};
+
+// src/layers/MsnhBatchNormLayer.cpp:5-52, 453-480
+class MsnhNet_API BatchNormLayer : public BaseLayer
+{
+public:
+    BatchNormLayer(const int &batch, const int &width, const int &height, const int &channel, const ActivationType &activation,
+                   const float &eps, const std::vector<float> &actParams);
+    void loadAllWeigths(std::vector<float> &weights) override;
+    int lower(Plan &plan, int in, int layerIndex) override;
+    void foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const override;
+
+private:
+    float _eps = 0.00001f;
+    std::vector<float> _scales, _biases, _rollMean, _rollVariance;
+};
+
+// src/layers/MsnhMaxPoolLayer.cpp:5-170
+class MsnhNet_API MaxPoolLayer : public BaseLayer
+{
+public:
+    MaxPoolLayer(const int &batch, const int &height, const int &width, const int &channel, const int &kSizeX, const int &kSizeY,
+                 const int &strideX, const int &strideY, const int &paddingX, const int &paddingY, const int &maxPoolDepth,
+                 const int &outChannelsMp, const int &ceilMode, const int &antialiasing);
+    int lower(Plan &plan, int in, int layerIndex) override;
+    int getKSizeX() const { return _kSizeX; }
+    int getStride() const { return _strideX; }
+    int getPaddingX() const { return _paddingX; }
+
+private:
+    int _kSizeX, _kSizeY, _strideX, _strideY, _paddingX, _paddingY, _ceilMode;
+};
+
+// src/layers/MsnhLocalAvgPoolLayer.cpp:5-150
+class MsnhNet_API LocalAvgPoolLayer : public BaseLayer
+{
+public:
+    LocalAvgPoolLayer(const int &batch, const int &height, const int &width, const int &channel, const int &kSizeX, const int &kSizeY,
+                      const int &strideX, const int &strideY, const int &paddingX, const int &paddingY, const int &ceilMode,
+                      const int &antialiasing);
+    int lower(Plan &plan, int in, int layerIndex) override;
+
+private:
+    int _kSizeX, _kSizeY, _strideX, _strideY, _paddingX, _paddingY, _ceilMode;
+};
+
+// src/layers/MsnhConnectedLayer.cpp:5-106, 495-540
+class MsnhNet_API ConnectedLayer : public BaseLayer
+{
+public:
+    ConnectedLayer(const int &batch, const int &steps, const int &inputNum, const int &outputNum, const ActivationType &activation,
+                   const std::vector<float> &actParams, const int &batchNorm, const float &bnEps, const int &useBias);
+    void loadAllWeigths(std::vector<float> &weights) override;
+    int lower(Plan &plan, int in, int layerIndex) override;
+    const std::vector<float> &kernelWeights() const override { return _weights; }
+    void foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const override;
+
+private:
+    int _batchNorm = 0, _useBias = 1;
+    int _nWeights = 0, _nBiases = 0;
+    std::vector<float> _weights, _biases;
+};
+
+// src/layers/MsnhUpSampleLayer.cpp:5-66
+class MsnhNet_API UpSampleLayer : public BaseLayer
+{
+public:
+    UpSampleLayer(const int &batch, const int &width, const int &height, const int &channel, const int &strideX, const int &strideY,
+                  const float &scaleX, const float &scaleY, UpSampleParams::UpsampleType upsampleType, const int &alignCorners);
+    int lower(Plan &plan, int in, int layerIndex) override;
+
+private:
+    int _strideX, _strideY;
+    float _scaleX, _scaleY;
+};
+
+// src/layers/MsnhEmptyLayer.cpp (identity)
+class MsnhNet_API EmptyLayer : public BaseLayer
+{
+public:
+    EmptyLayer(const int &batch, const int &width, const int &height, const int &channel);
+    int lower(Plan &plan, int in, int layerIndex) override;
+};
+
+// src/layers/MsnhRouteLayer.cpp:5-55; sizes are computed by NetBuilder (src/net/MsnhNetBuilder.cpp:205-334)
+class MsnhNet_API RouteLayer : public BaseLayer
+{
+public:
+    RouteLayer(const int &batch, std::vector<int> &inputLayerIndexes, std::vector<int> &inputLayerOutputs, const int &groups,
+               const int &groupIndex, const int &addModel, const ActivationType &activation, const std::vector<float> &actParams);
+    int lower(Plan &plan, int in, int layerIndex) override;
+    const std::vector<int> &inputLayerIndexes() const { return _inputLayerIndexes; }
+    std::vector<int> inputChannels;         // channels of each routed layer, set by NetBuilder
+
+private:
+    std::vector<int> _inputLayerIndexes, _inputLayerOutputs;
+    int _groups, _groupIndex, _addModel;
+};
+
+// Shared by the four block layers: builds the sub-layers of one branch exactly the way the reference's block
+// constructors do (same accepted node types, same exceptions), e.g. src/layers/MsnhResBlockLayer.cpp:23-150.
+class MsnhNet_API BlockLayer : public BaseLayer
+{
+public:
+    ~BlockLayer() override;
+    void loadAllWeigths(std::vector<float> &weights) override;
+
+protected:
+    std::vector<BaseLayer *> buildChain(NetBuildParams &params, std::vector<BaseParams *> &nodes, const char *blockName, bool allowEmpty);
+    int lowerChain(Plan &plan, const std::vector<BaseLayer *> &chain, int in, int layerIndex);
+    std::vector<std::vector<BaseLayer *>> _chains;      // weight order = chain order
+};
+
+// out = act(x + F(x))   src/layers/MsnhResBlockLayer.cpp:4-150, 215-302
+class MsnhNet_API ResBlockLayer : public BlockLayer
+{
+public:
+    ResBlockLayer(const int &batch, NetBuildParams &params, std::vector<BaseParams *> &baseParams, ActivationType &activation,
+                  const std::vector<float> &actParams);
+    int lower(Plan &plan, int in, int layerIndex) override;
+    std::vector<BaseLayer *> &baseLayers() { return _chains[0]; }
+};
+
+// out = act(base(x) + branch(x))   src/layers/MsnhRes2BlockLayer.cpp:4-260, 342-447
+class MsnhNet_API Res2BlockLayer : public BlockLayer
+{
+public:
+    Res2BlockLayer(const int &batch, NetBuildParams &params, std::vector<BaseParams *> &baseParams, std::vector<BaseParams *> &branchParams,
+                   ActivationType &activation, const std::vector<float> &actParams);
+    int lower(Plan &plan, int in, int layerIndex) override;
+};
+
+// out = act(sum of branches)   src/layers/MsnhAddBlockLayer.cpp:4-250, 255-357
+class MsnhNet_API AddBlockLayer : public BlockLayer
+{
+public:
+    AddBlockLayer(const int &batch, NetBuildParams &params, std::vector<std::vector<BaseParams *>> &branchParams, ActivationType &activation,
+                  const std::vector<float> &actParams);
+    int lower(Plan &plan, int in, int layerIndex) override;
+};
+
+// out = act(channel concat of branches)   src/layers/MsnhConcatBlockLayer.cpp:4-250, 255-355
+class MsnhNet_API ConcatBlockLayer : public BlockLayer
+{
+public:
+    ConcatBlockLayer(const int &batch, NetBuildParams &params, std::vector<std::vector<BaseParams *>> &branchParams, ActivationType &activation,
+                     const std::vector<float> &actParams);
+    int lower(Plan &plan, int in, int layerIndex) override;
+};
+
+// src/layers/MsnhYoloLayer.cpp:5-58
+class MsnhNet_API YoloLayer : public BaseLayer
+{
+public:
+    YoloLayer(const int &batch, const int &width, const int &height, const int &num, const int &orgWidth, const int &orgHeight,
+              const int &classNum, const std::vector<float> &anchors, const YoloType &yoloType);
+    int lower(Plan &plan, int in, int layerIndex) override;
+    int getClassNum() const { return _classNum; }
+    float getRatios() const { return _ratios; }
+    YoloType getYoloType() const { return _yoloType; }
+    std::vector<float> anchors;
+    int cellBase = 0;          // set by the YoloOutLayer that consumes this head
+    float confThresh = 2.f;    // likewise; 2 = "no candidate list" until a yoloout claims the head
+    size_t decodeOp = 0;
+
+private:
+    int _orgHeight, _orgWidth, _classNum;
+    float _ratios;
+    YoloType _yoloType;
+};
+
+// src/layers/MsnhYoloOutLayer.cpp:4-60 (ctor), :79-203 (candidate scan + sort), :381-461 (nms)
+class MsnhNet_API YoloOutLayer : public BaseLayer
+{
+public:
+    YoloOutLayer(const int &batch, const int &orgWidth, const int &orgHeight, std::vector<int> &yoloIndexes, std::vector<YoloInfo> &yoloLayersInfo,
+                 const float &confThresh, const float &nmsThresh, const int &useSotfNms, const YoloType &yoloType);
+    int lower(Plan &plan, int in, int layerIndex) override;
+    void forwardGPU(NetworkState &netState) override;      // device candidate compaction + host sort / NMS
+
+    static std::vector<YoloBox> nms(const std::vector<YoloBox> &bboxes, const float &nmsThresh, const bool &useSoftNms, const float &sigma = 0.3f);
+    float getConfThresh() const { return _confThresh; }
+    float getNmsThresh() const { return _nmsThresh; }
+    int   getUseSoftNms() const { return _useSoftNms; }
+    YoloType getYoloType() const { return _yoloType; }
+    const std::vector<int> &yoloIndexes() const { return _yoloIndexes; }
+
+    std::vector<bool> batchHasBox;
+    std::vector<std::vector<YoloBox>> finalOut;
+    static bool keepClassScores;           // also fill YoloBox::classesVal (costs an extra device->host copy)
+
+    // host post-processing of the compacted candidate rows of one image (8 floats per row, see msnh_hip_yolo_gather)
+    std::vector<YoloBox> boxesFromRows(const float *rows, int count, const float *decodedOfImage) const;
+
+private:
+    float _confThresh, _nmsThresh;
+    int _useSoftNms, _orgHeight, _orgWidth;
+    YoloType _yoloType;
+    std::vector<int> _yoloIndexes;
+    std::vector<YoloInfo> _yoloLayersInfo;
+    int _yoloAllInputNum = 0, _pixels = 0;
+    PinnedBuffer _hostCnt, _hostRows, _hostDecoded;
+};
+}

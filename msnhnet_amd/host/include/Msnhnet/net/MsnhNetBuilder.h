@@ -1,0 +1,93 @@
+// NetBuilder: build a network from a `.msnhnet` file, load `.msnhbin` weights, run it.
+// Public interface = the reference's (include/Msnhnet/net/MsnhNetBuilder.h:48-117) with the GPU entry points
+// unconditional.  Extensions, all optional: batches larger than one (the reference rejects them),
+// setKeepClassScores, the last-run accessors used by tests and the benchmark.
+#pragma once
+#include <string>
+#include <vector>
+#include "Msnhnet/io/MsnhParser.h"
+#include "Msnhnet/layers/MsnhLayers.h"
+#include "Msnhnet/net/MsnhNetwork.h"
+
+namespace Msnhnet
+{
+class MsnhNet_API NetBuilder
+{
+public:
+    NetBuilder();
+    ~NetBuilder();
+
+    static void setPreviewMode(const bool &mode);
+    static void setMemAlign(const bool &memAlign);
+    static void setOnlyGpu(const bool &onlyGpu);
+    static void setOnlyCpu(const bool &onlyCpu);
+    static void setUseFp16(const bool &useFp16);
+    static void setForceUseCuda(const bool &onlyUseCuda);
+    static void setKeepClassScores(const bool &keep);
+
+    void buildNetFromMsnhNet(const std::string &path);
+    void loadWeightsFromMsnhBin(const std::string &path);
+    void loadWeightsFromVector(const std::vector<float> &weights);     // same slicing, no file
+
+    // The reference's CPU entry points: this build has no CPU path, they throw "Gpu mode , can not run with cpu".
+    std::vector<float> runClassify(std::vector<float> img);
+    std::vector<std::vector<YoloBox>> runYolo(std::vector<float> img);
+    // img holds batch*C*H*W floats, batch-major NCHW (one image when the graph's batch is 1, as in the reference).
+    std::vector<float> runClassifyGPU(std::vector<float> img);
+    std::vector<std::vector<YoloBox>> runYoloGPU(std::vector<float> img);
+
+    // Steady-state serving path: the input already lives on the device (NCHW float32, batch*C*H*W floats).
+    // Enqueues one forward on the builder's stream; results are fetched with fetchClassify / fetchYolo.
+    void enqueueForward(const float *deviceInput);
+    void sync();
+    std::vector<float> fetchClassify();
+    std::vector<std::vector<YoloBox>> fetchYolo();
+    float *deviceInputBuffer();               // the builder's own device input buffer (batch*C*H*W floats)
+
+    Point2I getInputSize();
+    int getInputChannel();
+    int getBatch() const;
+    void clearLayers();
+    float getInferenceTime();
+    std::string getLayerDetail();
+    std::string getTimeDetail();
+    float getGpuInferenceTime() const;
+    Network *getNet() const;
+    int getLastLayerOutWidth() const;
+    int getLastLayerOutHeight() const;
+    int getLastLayerOutChannel() const;
+    size_t getLastLayerOutNum() const;
+    void setSaveLayerOutput(bool saveLayerOutput);
+    bool getSaveLayerWeights() const;
+    void setSaveLayerWeights(bool saveLayerWeights);
+
+    // When layer dumps are on, the last run's per-layer outputs are kept here (batch-major NCHW float32)
+    // instead of being written to "<i>gpu.txt" files only.
+    const std::vector<std::vector<float>> &layerOutputs() const { return _layerOutputs; }
+    void setWriteDumpFiles(bool on) { _writeDumpFiles = on; }
+    std::string getPlanDetail() const;
+    double getConvFlops() const;              // 2*MACs of all conv/connected launches of one forward (whole batch)
+
+private:
+    void finalizePlan();
+    std::unique_ptr<Plan> lowerNetwork(int dtype);
+    void uploadInput(const std::vector<float> &img);
+    void runLayersEager();
+    void checkInput(size_t given) const;
+
+    Parser       *_parser;
+    Network      *_net;
+    NetworkState *_netState;
+    float  _gpuInferenceTime = 0.f;
+    int    _lastLayerOutWidth = 0, _lastLayerOutHeight = 0, _lastLayerOutChannel = 0;
+    size_t _lastLayerOutNum = 0;
+    bool   _saveLayerOutput = false, _saveLayerWeights = false, _writeDumpFiles = false;
+    bool   _planReady = false;
+    std::vector<std::vector<float>> _layerOutputs;
+    DeviceBuffer _inputDev;
+    PinnedBuffer _inputPinned, _outputPinned;
+    msnh_stream_t _stream = nullptr;
+    msnh_graph_t  _graph = nullptr;
+    const float  *_graphInput = nullptr;
+};
+}

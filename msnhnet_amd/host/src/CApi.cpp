@@ -1,0 +1,323 @@
+// C ABI of the host library (include/msnhnet_c.h): the reference facade over one global NetBuilder plus the
+// handle-based variant.  Every entry point catches all exceptions; none of them lets one cross the boundary.
+#include "msnhnet_c.h"
+#include <algorithm>
+#include <cstring>
+#include <memory>
+#include <string>
+#include "Msnhnet/net/MsnhNetBuilder.h"
+
+using namespace Msnhnet;
+
+namespace
+{
+thread_local std::string g_lastError;
+std::unique_ptr<NetBuilder> g_net;
+
+char *keepError(const std::exception &e)
+{
+    g_lastError = e.what();
+    return const_cast<char *>(g_lastError.c_str());
+}
+
+template <typename F> int guarded(F &&f)
+{
+    try { f(); return 0; }
+    catch (const std::exception &e) { keepError(e); return 1; }
+    catch (...) { g_lastError = "unknown error"; return 1; }
+}
+
+template <typename F> int refStyle(char **msg, F &&f)
+{
+    try { f(); return 1; }
+    catch (const std::exception &e) { char *m = keepError(e); if (msg) *msg = m; return -1; }
+    catch (...) { g_lastError = "unknown error"; if (msg) *msg = const_cast<char *>(g_lastError.c_str()); return -1; }
+}
+
+NetBuilder &nb(msnhnet_t h)
+{
+    if (h == nullptr) MSNH_THROW("net handle is NULL");
+    return *static_cast<NetBuilder *>(h);
+}
+
+long long copyText(const std::string &s, char *dst, long long cap)
+{
+    if (dst && cap > 0)
+    {
+        const long long n = std::min<long long>(static_cast<long long>(s.size()), cap - 1);
+        std::memcpy(dst, s.data(), static_cast<size_t>(n));
+        dst[n] = 0;
+    }
+    return static_cast<long long>(s.size());
+}
+
+void packBoxes(const std::vector<std::vector<YoloBox>> &all, int *counts, float *boxes, long long cap, long long *total)
+{
+    long long w = 0, sum = 0;
+    for (size_t b = 0; b < all.size(); ++b)
+    {
+        if (counts) counts[b] = static_cast<int>(all[b].size());
+        sum += static_cast<long long>(all[b].size());
+        for (const YoloBox &q : all[b])
+        {
+            if (boxes && w < cap)
+            {
+                float *o = boxes + 7 * w;
+                o[0] = q.xywhBox.x; o[1] = q.xywhBox.y; o[2] = q.xywhBox.w; o[3] = q.xywhBox.h;
+                o[4] = q.conf; o[5] = q.bestClsConf; o[6] = static_cast<float>(q.bestClsIdx);
+            }
+            ++w;
+        }
+    }
+    if (total) *total = sum;
+}
+}
+
+extern "C" {
+
+// ---- part 1 -----------------------------------------------------------------------------------------------------------
+int initMsnhnet(void)
+{
+    try { g_net.reset(new NetBuilder()); return 1; }
+    catch (const std::exception &e) { keepError(e); return -1; }
+}
+
+int buildMsnhnet(char **msg, const char *msnhnet, const char *msnhbin, int useFp16, int useCudaOnly)
+{
+    return refStyle(msg, [&] {
+        if (!g_net) MSNH_THROW("initMsnhnet was not called");
+        if (!msnhnet || !msnhbin) MSNH_THROW("path is NULL");
+        NetBuilder::setUseFp16(useFp16 != 0);
+        NetBuilder::setForceUseCuda(useCudaOnly != 0);
+        g_net->buildNetFromMsnhNet(msnhnet);
+        g_net->loadWeightsFromMsnhBin(msnhbin);
+    });
+}
+
+int runClassifyNoPred(char **msg, const float *data, const int len, int *bestIndex, int runGPU)
+{
+    return refStyle(msg, [&] {
+        if (!g_net) MSNH_THROW("initMsnhnet was not called");
+        if (!data || !bestIndex || len <= 0) MSNH_THROW("bad argument");
+        std::vector<float> img(data, data + len);
+        const std::vector<float> out = runGPU ? g_net->runClassifyGPU(img) : g_net->runClassify(img);
+        const size_t per = g_net->getLastLayerOutNum();
+        *bestIndex = static_cast<int>(std::distance(out.begin(), std::max_element(out.begin(), out.begin() + static_cast<long long>(per))));
+    });
+}
+
+int runYoloNoPred(char **msg, const float *data, const int len, BBoxContainer *bboxContainer, int *detectedNum, int runGPU)
+{
+    return refStyle(msg, [&] {
+        if (!g_net) MSNH_THROW("initMsnhnet was not called");
+        if (!data || !bboxContainer || !detectedNum || len <= 0) MSNH_THROW("bad argument");
+        std::vector<float> img(data, data + len);
+        const std::vector<std::vector<YoloBox>> out = runGPU ? g_net->runYoloGPU(img) : g_net->runYolo(img);
+        const std::vector<YoloBox> &b0 = out.at(0);
+        const size_t n = std::min<size_t>(b0.size(), MSNHNET_MAX_BBOX);
+        for (size_t i = 0; i < n; ++i)
+        {
+            BBox &o = bboxContainer->boxes[i];
+            o.x = b0[i].xywhBox.x; o.y = b0[i].xywhBox.y; o.w = b0[i].xywhBox.w; o.h = b0[i].xywhBox.h;
+            o.conf = b0[i].conf; o.bestClsConf = b0[i].bestClsConf; o.bestClsIdx = static_cast<uint32_t>(b0[i].bestClsIdx); o.angle = b0[i].angle;
+        }
+        *detectedNum = static_cast<int>(n);
+    });
+}
+
+int dispose(void) { g_net.reset(); return 1; }
+
+int withGPU(int *GPU)
+{
+    if (!GPU) return -1;
+    int count = 0;
+    msnh_hip_device_count(&count);
+    *GPU = count > 0 ? 1 : 0;
+    return 1;
+}
+
+int withCUDNN(int *CUDNN)
+{
+    if (!CUDNN) return -1;
+    *CUDNN = 0;
+    return 1;
+}
+
+int getCpuForwardTime(float *time)
+{
+    if (!time || !g_net) return -1;
+    *time = g_net->getInferenceTime();
+    return 1;
+}
+
+int getGpuForwardTime(float *time)
+{
+    if (!time || !g_net) return -1;
+    *time = g_net->getGpuInferenceTime();
+    return 1;
+}
+
+int getInputDim(int *width, int *heigth, int *channel)
+{
+    return refStyle(nullptr, [&] {
+        if (!g_net || !width || !heigth || !channel) MSNH_THROW("bad argument");
+        const Point2I p = g_net->getInputSize();
+        *width = p.x; *heigth = p.y; *channel = g_net->getInputChannel();
+    });
+}
+
+// ---- part 2 -----------------------------------------------------------------------------------------------------------
+const char *msnhnet_last_error(void) { return g_lastError.c_str(); }
+
+int msnhnet_create(msnhnet_t *net)
+{
+    return guarded([&] { if (!net) MSNH_THROW("net pointer is NULL"); *net = new NetBuilder(); });
+}
+
+int msnhnet_destroy(msnhnet_t net)
+{
+    return guarded([&] { delete static_cast<NetBuilder *>(net); });
+}
+
+int msnhnet_set_use_fp16(int on) { return guarded([&] { NetBuilder::setUseFp16(on != 0); }); }
+int msnhnet_set_keep_class_scores(int on) { return guarded([&] { NetBuilder::setKeepClassScores(on != 0); }); }
+int msnhnet_set_save_layer_output(msnhnet_t net, int on) { return guarded([&] { nb(net).setSaveLayerOutput(on != 0); }); }
+int msnhnet_build(msnhnet_t net, const char *path) { return guarded([&] { if (!path) MSNH_THROW("path is NULL"); nb(net).buildNetFromMsnhNet(path); }); }
+int msnhnet_load(msnhnet_t net, const char *path) { return guarded([&] { if (!path) MSNH_THROW("path is NULL"); nb(net).loadWeightsFromMsnhBin(path); }); }
+
+int msnhnet_load_from_memory(msnhnet_t net, const float *weights, size_t count)
+{
+    return guarded([&] {
+        if (!weights && count) MSNH_THROW("weights is NULL");
+        nb(net).loadWeightsFromVector(std::vector<float>(weights, weights + count));
+    });
+}
+
+int msnhnet_input_dims(msnhnet_t net, int *batch, int *channels, int *height, int *width)
+{
+    return guarded([&] {
+        Network *n = nb(net).getNet();
+        if (batch) *batch = n->batch;
+        if (channels) *channels = n->channels;
+        if (height) *height = n->height;
+        if (width) *width = n->width;
+    });
+}
+
+int msnhnet_num_layers(msnhnet_t net)
+{
+    int n = -1;
+    guarded([&] { n = static_cast<int>(nb(net).getNet()->layers.size()); });
+    return n;
+}
+
+int msnhnet_layer_info(msnhnet_t net, int layer, long long *info, char *name, int name_cap)
+{
+    return guarded([&] {
+        Network *n = nb(net).getNet();
+        if (layer < 0 || static_cast<size_t>(layer) >= n->layers.size() || !info) MSNH_THROW("layer index out of range");
+        const BaseLayer *l = n->layers[static_cast<size_t>(layer)];
+        info[0] = static_cast<long long>(l->type()); info[1] = l->getOutHeight(); info[2] = l->getOutWidth(); info[3] = l->getOutChannel();
+        info[4] = l->getOutputNum(); info[5] = l->getInputNum(); info[6] = static_cast<long long>(l->getNumWeights()); info[7] = l->getMemReUse();
+        info[8] = l->getBatch(); info[9] = static_cast<long long>(l->getActivation());
+        copyText(l->getLayerName(), name, name_cap);
+    });
+}
+
+long long msnhnet_layer_detail(msnhnet_t net, char *dst, long long cap)
+{
+    long long n = -1;
+    guarded([&] { n = copyText(nb(net).getLayerDetail(), dst, cap); });
+    return n;
+}
+
+long long msnhnet_plan_detail(msnhnet_t net, char *dst, long long cap)
+{
+    long long n = -1;
+    guarded([&] { n = copyText(nb(net).getPlanDetail(), dst, cap); });
+    return n;
+}
+
+long long msnhnet_time_detail(msnhnet_t net, char *dst, long long cap)
+{
+    long long n = -1;
+    guarded([&] { n = copyText(nb(net).getTimeDetail(), dst, cap); });
+    return n;
+}
+
+double msnhnet_conv_flops(msnhnet_t net)
+{
+    double f = 0;
+    guarded([&] { f = nb(net).getConvFlops(); });
+    return f;
+}
+
+static void copyOut(const std::vector<float> &v, float *out, long long cap, long long *n_out)
+{
+    if (n_out) *n_out = static_cast<long long>(v.size());
+    if (out && cap > 0) std::memcpy(out, v.data(), sizeof(float) * static_cast<size_t>(std::min<long long>(cap, static_cast<long long>(v.size()))));
+}
+
+int msnhnet_run_classify(msnhnet_t net, const float *img, long long n, float *out, long long cap, long long *n_out)
+{
+    return guarded([&] {
+        if (!img || n <= 0) MSNH_THROW("bad argument");
+        copyOut(nb(net).runClassify(std::vector<float>(img, img + n)), out, cap, n_out);
+    });
+}
+
+int msnhnet_run_classify_gpu(msnhnet_t net, const float *img, long long n, float *out, long long cap, long long *n_out)
+{
+    return guarded([&] {
+        if (!img || n <= 0) MSNH_THROW("bad argument");
+        copyOut(nb(net).runClassifyGPU(std::vector<float>(img, img + n)), out, cap, n_out);
+    });
+}
+
+int msnhnet_run_yolo_gpu(msnhnet_t net, const float *img, long long n, int *counts, float *boxes, long long cap_boxes, long long *total)
+{
+    return guarded([&] {
+        if (!img || n <= 0) MSNH_THROW("bad argument");
+        packBoxes(nb(net).runYoloGPU(std::vector<float>(img, img + n)), counts, boxes, cap_boxes, total);
+    });
+}
+
+long long msnhnet_layer_output(msnhnet_t net, int layer, float *dst, long long cap)
+{
+    long long n = -1;
+    guarded([&] {
+        const std::vector<std::vector<float>> &outs = nb(net).layerOutputs();
+        if (layer < 0 || static_cast<size_t>(layer) >= outs.size()) MSNH_THROW("no dump for this layer (enable msnhnet_set_save_layer_output and run)");
+        const std::vector<float> &v = outs[static_cast<size_t>(layer)];
+        n = static_cast<long long>(v.size());
+        if (dst && cap > 0) std::memcpy(dst, v.data(), sizeof(float) * static_cast<size_t>(std::min(cap, n)));
+    });
+    return n;
+}
+
+int msnhnet_device_input(msnhnet_t net, float **device_ptr)
+{
+    return guarded([&] { if (!device_ptr) MSNH_THROW("pointer is NULL"); *device_ptr = nb(net).deviceInputBuffer(); });
+}
+
+int msnhnet_enqueue(msnhnet_t net, const float *device_input) { return guarded([&] { nb(net).enqueueForward(device_input); }); }
+int msnhnet_sync(msnhnet_t net) { return guarded([&] { nb(net).sync(); }); }
+
+int msnhnet_fetch_classify(msnhnet_t net, float *out, long long cap, long long *n_out)
+{
+    return guarded([&] { copyOut(nb(net).fetchClassify(), out, cap, n_out); });
+}
+
+int msnhnet_fetch_yolo(msnhnet_t net, int *counts, float *boxes, long long cap_boxes, long long *total)
+{
+    return guarded([&] { packBoxes(nb(net).fetchYolo(), counts, boxes, cap_boxes, total); });
+}
+
+float msnhnet_gpu_inference_time(msnhnet_t net)
+{
+    float t = -1.f;
+    guarded([&] { t = nb(net).getGpuInferenceTime(); });
+    return t;
+}
+
+}

@@ -1,0 +1,944 @@
+// Layer classes: shape inference, weight slicing and lowering into plan ops.
+// Shape rules, weight order and exception texts follow the reference's layer sources (cited per class in
+// MsnhLayers.h); none of its compute code exists here -- the arithmetic lives in the device kernels.
+#include "Msnhnet/layers/MsnhLayers.h"
+#include <algorithm>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include "Msnhnet/net/MsnhNetwork.h"
+#include "Msnhnet/utils/MsnhExVector.h"
+
+namespace Msnhnet
+{
+// ---- BaseLayer -------------------------------------------------------------------------------------------------
+bool BaseLayer::supportAvx = false;
+bool BaseLayer::supportFma = false;
+bool BaseLayer::isPreviewMode = false;
+bool BaseLayer::onlyUseCuda = false;
+bool BaseLayer::onlyUseCpu = false;
+bool BaseLayer::onlyUseGpu = true;          // there is no CPU compute path in this build
+bool BaseLayer::useFp16 = false;
+bool BaseLayer::convSingleOptim = false;
+
+BaseLayer::BaseLayer() {}
+BaseLayer::~BaseLayer() {}
+void BaseLayer::setPreviewMode(const bool &v) { isPreviewMode = v; }
+void BaseLayer::setMemAlign(const bool &) {}
+void BaseLayer::setForceUseCuda(const bool &v) { onlyUseCuda = v; }
+void BaseLayer::setUseFp16(const bool &v) { useFp16 = v; }
+void BaseLayer::setOnlyGpu(const bool &v) { onlyUseGpu = v; }
+void BaseLayer::setOnlyCpu(const bool &v) { onlyUseCpu = v; }
+void BaseLayer::initSimd() {}
+void BaseLayer::mallocMemory() { _memReUse = 0; _memoryMalloced = true; }
+
+void BaseLayer::forward(NetworkState &)
+{
+    MSNH_THROW("Gpu mode , can not run with cpu");
+}
+
+void BaseLayer::forwardGPU(NetworkState &netState)
+{
+    if (plan == nullptr) MSNH_THROW(_layerName + ": layer is not part of a planned network (build it with NetBuilder and load weights first)");
+    plan->run(opBegin, opEnd, netState.stream);
+}
+
+void BaseLayer::loadAllWeigths(std::vector<float> &weights)
+{
+    if (!weights.empty()) MSNH_THROW(_layerName + " has no weights");
+}
+
+void BaseLayer::saveAllWeights(const int &, const int &, const int &) {}
+
+int BaseLayer::lower(Plan &, int, int) { MSNH_THROW(_layerName + ": lowering is not implemented"); }
+
+const std::vector<float> &BaseLayer::kernelWeights() const
+{
+    static const std::vector<float> none;
+    return none;
+}
+
+void BaseLayer::foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const
+{
+    scale.clear();
+    shift.clear();
+}
+
+float *BaseLayer::getGpuOutput() const
+{
+    if (plan == nullptr || outTensor < 0) return nullptr;
+    return static_cast<float *>(plan->ptr(outTensor));
+}
+
+void BaseLayer::requireDeviceActivation(ActivationType act, const char *layer)
+{
+    if (!Activations::deviceSupported(act))
+        MSNH_THROW(std::string(layer) + ": activation '" + Activations::getActivationStr(act) + "' is outside the convolutional path this build implements");
+}
+
+static std::string fmt(const char *f, ...)
+{
+    char buf[256];
+    va_list ap;
+    va_start(ap, f);
+    vsnprintf(buf, sizeof(buf), f, ap);
+    va_end(ap);
+    return buf;
+}
+
+static int planDtype(const Plan &plan) { return plan.computeDtype; }
+
+// Batch-norm folded the way the reference evaluates it (src/layers/MsnhConvolutionalLayer.cpp:811-815):
+// sqrtVal = sqrt(var+eps); scale = gamma/sqrtVal; shift = -gamma*mean/sqrtVal + beta, all in float.
+static void foldBn(const std::vector<float> &g, const std::vector<float> &beta, const std::vector<float> &mean, const std::vector<float> &var,
+                   float eps, std::vector<float> &scale, std::vector<float> &shift)
+{
+    const size_t n = g.size();
+    scale.resize(n);
+    shift.resize(n);
+    for (size_t c = 0; c < n; ++c)
+    {
+        const float sqrtVal = static_cast<float>(std::sqrt(var[c] + eps));
+        const float scaleSqrt = g[c] / sqrtVal;
+        const float meanSqrt = -g[c] * mean[c] / sqrtVal;
+        scale[c] = scaleSqrt;
+        shift[c] = meanSqrt + (beta.empty() ? 0.f : beta[c]);
+    }
+}
+
+// ---- ConvolutionalLayer -------------------------------------------------------------------------------------------
+ConvolutionalLayer::ConvolutionalLayer(const int &batch, const int &steps, const int &height, const int &width, const int &channel, const int &num,
+                                       const int &groups, const int &kSizeX, const int &kSizeY, const int &strideX, const int &strideY,
+                                       const int &dilationX, const int &dilationY, const int &paddingX, const int &paddingY,
+                                       ActivationType activation, const std::vector<float> &actParams, const int &batchNorm, const float &bnEps,
+                                       const int &useBias, const int &binary, const int &xnor, const int &useBinOutput, const int &groupIndex,
+                                       const int &antialiasing, ConvolutionalLayer *const &shareLayer, const int &assistedExcitation, const int &deform)
+{
+    (void)steps; (void)useBinOutput; (void)groupIndex; (void)deform;
+    if (binary || xnor || shareLayer != nullptr || assistedExcitation || antialiasing)
+        MSNH_THROW("conv: binary/xnor/shared/assisted-excitation/antialiasing variants are outside the convolutional path this build implements");
+    if (activation == ActivationType::PRELU || activation == NORM_CHAN || activation == NORM_CHAN_SOFTMAX || activation == NORM_CHAN_SOFTMAX_MAXVAL)
+        MSNH_THROW("conv: prelu / channel-normalising activations are outside the convolutional path this build implements");
+    requireDeviceActivation(activation, "conv");
+    _type = LayerType::CONVOLUTIONAL;
+    _groups = groups < 1 ? 1 : groups;
+    _strideX = strideX; _strideY = strideY;
+    _height = height; _width = width; _channel = channel; _num = num; _batch = batch;
+    _dilationX = dilationX; _dilationY = dilationY; _kSizeX = kSizeX; _kSizeY = kSizeY; _paddingX = paddingX; _paddingY = paddingY;
+    _batchNorm = batchNorm; _useBias = useBias; _bnEps = bnEps;
+    if (num <= 0 || kSizeX <= 0 || kSizeY <= 0 || strideX <= 0 || strideY <= 0) MSNH_THROW("conv: filters, kSize and stride must be positive");
+    if (channel % _groups != 0 || num % _groups != 0) MSNH_THROW("conv: channels and filters must be divisible by groups");
+    // The reference feeds X-named sizes into the H slots of its im2col while the output size uses Y for the height
+    // (src/layers/MsnhConvolutionalLayer.cpp:750-752 vs :388-398), so only square geometry is self-consistent there.
+    if (kSizeX != kSizeY || strideX != strideY || paddingX != paddingY || dilationX != dilationY)
+        MSNH_THROW("conv: only square kernels / strides / paddings / dilations are supported");
+    _nWeights = (channel / groups) * num * kSizeX * kSizeY;
+    _nBiases = useBias ? num : 0;
+    if (batchNorm) { _nScales = num; _nRollMean = num; _nRollVariance = num; }
+    _outHeight = convOutHeight();
+    _outWidth = convOutWidth();
+    _outChannel = num;
+    if (_outHeight <= 0 || _outWidth <= 0) MSNH_THROW("conv: kernel larger than the padded input");
+    _outputNum = _outHeight * _outWidth * _outChannel;
+    _inputNum = height * width * channel;
+    _activation = activation;
+    _actParams = actParams;
+    _numWeights = static_cast<size_t>(_nWeights + _nScales + _nRollMean + _nRollVariance + _nBiases);
+    _workSpaceSize = 0;                       // implicit GEMM: no im2col scratch
+    _inputSpaceSize = static_cast<size_t>(_inputNum);
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _bFlops = (2.0f * _nWeights * _outHeight * _outWidth) / 1000000000.f;
+
+    const char *tag = "conv  ";
+    _layerName = "Conv            ";
+    if (_batchNorm) { _layerName = "ConvBN          "; tag = "convBN"; }
+    else if (_groups == _num) { _layerName = "ConvDW          "; tag = "convDW"; }
+    _layerDetail = tag;
+    _layerDetail += _groups > 1 ? fmt("%5d/%4d ", _num, _groups) : fmt("%5d      ", _num);
+    _layerDetail += _dilationX > 1 ? fmt("%2d x%2d/%2d(%1d)", _kSizeX, _kSizeY, _strideX, _dilationX) : fmt("%2d x%2d/%2d   ", _kSizeX, _kSizeY, _strideX);
+    _layerDetail += fmt("%4d x%4d x%4d -> %4d x%4d x%4d %5.3f BF\n", _width, _height, _channel, _outWidth, _outHeight, _outChannel,
+                        static_cast<double>(_bFlops));
+}
+
+int ConvolutionalLayer::convOutHeight() const { return (_height + 2 * _paddingY - (_dilationY * (_kSizeY - 1) + 1)) / _strideY + 1; }
+int ConvolutionalLayer::convOutWidth() const { return (_width + 2 * _paddingX - (_dilationX * (_kSizeX - 1) + 1)) / _strideX + 1; }
+
+void ConvolutionalLayer::loadAllWeigths(std::vector<float> &weights)
+{
+    if (weights.size() != _numWeights)
+        MSNH_THROW("Conv weights load err. needed : " + std::to_string(_numWeights) + " given : " + std::to_string(weights.size()));
+    if (BaseLayer::isPreviewMode) return;
+    const float *p = weights.data();
+    _weights.assign(p, p + _nWeights);
+    p += _nWeights;
+    if (_batchNorm)
+    {
+        // order: scales, biases (only when useBias), rollMean, rollVariance  (src/layers/MsnhConvolutionalLayer.cpp:1275-1288)
+        _scales.assign(p, p + _nScales); p += _nScales;
+        _biases.assign(p, p + _nBiases); p += _nBiases;
+        _rollMean.assign(p, p + _nRollMean); p += _nRollMean;
+        _rollVariance.assign(p, p + _nRollVariance);
+    }
+    else if (_useBias)
+    {
+        _biases.assign(p, p + _nBiases);
+    }
+    _weightsLoaded = true;
+}
+
+void ConvolutionalLayer::foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const
+{
+    scale.clear();
+    shift.clear();
+    if (_batchNorm) foldBn(_scales, _biases, _rollMean, _rollVariance, _bnEps, scale, shift);
+    else if (_useBias) shift = _biases;
+}
+
+int ConvolutionalLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    const int dtype = planDtype(plan);
+    const int out = plan.addTensor(_batch, _outHeight, _outWidth, _outChannel, dtype, "conv_out");
+    if (plan.tensors[static_cast<size_t>(in)].layout == PlanTensor::NCHW_INPUT)
+    {
+        // first layer: use the stem kernel (reads the NCHW float32 input directly) when the shape allows it
+        msnh_conv_desc d;
+        std::memset(&d, 0, sizeof(d));
+        d.dtype = dtype; d.out_dtype = dtype; d.batch = _batch; d.in_h = _height; d.in_w = _width; d.in_c = _channel; d.in_ld = _channel;
+        d.out_c = _outChannel; d.out_h = _outHeight; d.out_w = _outWidth; d.out_ld = (_outChannel + 7) / 8 * 8;
+        d.ksize = _kSizeX; d.stride = _strideX; d.pad = _paddingX; d.dilation = _dilationX; d.groups = _groups;
+        d.act = NONE; d.act2 = NONE; d.res_ld = d.out_c; d.res_mul = 1.f; d.out_mul = 1.f; d.algo = MSNH_CONV_AUTO;
+        if (msnh_hip_conv2d_select_algo(&d) != MSNH_CONV_STEM)
+        {
+            const int cast = plan.addTensor(_batch, _height, _width, _channel, dtype, "input_nhwc");
+            plan.addOp(PlanOp::INPUT_CAST, in, -1, cast, layerIndex, "input_cast");
+            in = cast;
+        }
+    }
+    PlanOp &op = plan.addOp(PlanOp::CONV, in, -1, out, layerIndex, "conv");
+    op.ksize = _kSizeX; op.stride = _strideX; op.pad = _paddingX; op.dilation = _dilationX; op.groups = _groups;
+    op.act = _activation; op.actParam = actParam();
+    op.src = this;
+    return out;
+}
+
+// ---- BatchNormLayer --------------------------------------------------------------------------------------------------
+BatchNormLayer::BatchNormLayer(const int &batch, const int &width, const int &height, const int &channel, const ActivationType &activation,
+                               const float &eps, const std::vector<float> &actParams)
+{
+    requireDeviceActivation(activation, "batchnorm");
+    _type = LayerType::BATCHNORM;
+    _layerName = "BatchNorm       ";
+    _activation = activation;
+    _actParams = actParams;
+    _eps = eps;
+    _batch = batch; _width = width; _height = height; _channel = channel;
+    _outWidth = width; _outHeight = height; _outChannel = channel;
+    _num = channel;
+    _inputNum = width * height * channel;
+    _outputNum = _inputNum;
+    _numWeights = static_cast<size_t>(4) * channel;
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _layerDetail = fmt("Batch Normalization Layer:     %d x %d x %d image\n", _width, _height, _channel);
+}
+
+void BatchNormLayer::loadAllWeigths(std::vector<float> &weights)
+{
+    if (weights.size() != _numWeights)
+        MSNH_THROW("BatchNorm weights load err. needed : " + std::to_string(_numWeights) + " given : " + std::to_string(weights.size()));
+    if (BaseLayer::isPreviewMode) return;
+    const float *p = weights.data();
+    const int c = _channel;
+    _scales.assign(p, p + c);               // scales, biases, rollMean, rollVariance (src/layers/MsnhBatchNormLayer.cpp:469-472)
+    _biases.assign(p + c, p + 2 * c);
+    _rollMean.assign(p + 2 * c, p + 3 * c);
+    _rollVariance.assign(p + 3 * c, p + 4 * c);
+    _weightsLoaded = true;
+}
+
+void BatchNormLayer::foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const
+{
+    foldBn(_scales, _biases, _rollMean, _rollVariance, _eps, scale, shift);
+}
+
+int BatchNormLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    const PlanTensor &ti = plan.tensors[static_cast<size_t>(in)];
+    if (ti.layout != PlanTensor::NHWC) MSNH_THROW("batchnorm can not be the first layer of a network");
+    const int out = plan.addTensor(_batch, _outHeight, _outWidth, _outChannel, planDtype(plan), "bn_out");
+    PlanOp &op = plan.addOp(PlanOp::AFFINE, in, -1, out, layerIndex, "batchnorm");
+    op.act = _activation; op.actParam = actParam();
+    op.src = this;
+    return out;
+}
+
+// ---- pooling ------------------------------------------------------------------------------------------------------------
+static int pooledSize(int in, int k, int s, int p, int ceilMode, const char *name)
+{
+    if (ceilMode == 1)
+    {
+        const int rem = (in + p * 2 - k) % s;
+        if (rem >= k) MSNH_THROW(std::string(name) + " padding error ");
+        return (in + p * 2 - k) / s + (rem <= p ? 1 : 2);
+    }
+    if (ceilMode == 0) return (in + p * 2 - k) / s + 1;
+    return (in + p - k) / s + 1;
+}
+
+MaxPoolLayer::MaxPoolLayer(const int &batch, const int &height, const int &width, const int &channel, const int &kSizeX, const int &kSizeY,
+                           const int &strideX, const int &strideY, const int &paddingX, const int &paddingY, const int &maxPoolDepth,
+                           const int &outChannelsMp, const int &ceilMode, const int &antialiasing)
+    : _kSizeX(kSizeX), _kSizeY(kSizeY), _strideX(strideX), _strideY(strideY), _paddingX(paddingX), _paddingY(paddingY), _ceilMode(ceilMode)
+{
+    (void)outChannelsMp; (void)antialiasing;
+    if (maxPoolDepth) MSNH_THROW("maxpool: depth mode is outside the convolutional path this build implements");
+    if (kSizeX != kSizeY || strideX != strideY || paddingX != paddingY) MSNH_THROW("maxpool: only square windows are supported");
+    if (kSizeX <= 0 || strideX <= 0) MSNH_THROW("maxpool: kSize and stride must be positive");
+    _type = LayerType::MAXPOOL;
+    _layerName = "MaxPool         ";
+    _batch = batch; _height = height; _width = width; _channel = channel;
+    _outWidth = pooledSize(width, kSizeX, strideX, paddingX, ceilMode, "maxpool");
+    _outHeight = pooledSize(height, kSizeY, strideY, paddingY, ceilMode, "maxpool");
+    _outChannel = channel;
+    _outputNum = _outHeight * _outWidth * _outChannel;
+    _inputNum = height * width * channel;
+    _bFlops = (_kSizeX * _kSizeY * _channel * _outHeight * _outWidth) / 1000000000.f;
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _layerDetail = fmt("max               %2dx%2d/%2d   %4d x%4d x%4d -> %4d x%4d x%4d %5.3f BF\n", _kSizeX, _kSizeY, _strideX, _width, _height,
+                       _channel, _outWidth, _outHeight, _outChannel, static_cast<double>(_bFlops));
+}
+
+int MaxPoolLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    if (plan.tensors[static_cast<size_t>(in)].layout != PlanTensor::NHWC) MSNH_THROW("maxpool can not be the first layer of a network");
+    const int out = plan.addTensor(_batch, _outHeight, _outWidth, _outChannel, plan.tensors[static_cast<size_t>(in)].dtype, "maxpool_out");
+    PlanOp &op = plan.addOp(PlanOp::MAXPOOL, in, -1, out, layerIndex, "maxpool");
+    op.ksize = _kSizeX; op.stride = _strideX; op.pad = _paddingX;
+    return out;
+}
+
+LocalAvgPoolLayer::LocalAvgPoolLayer(const int &batch, const int &height, const int &width, const int &channel, const int &kSizeX, const int &kSizeY,
+                                     const int &strideX, const int &strideY, const int &paddingX, const int &paddingY, const int &ceilMode,
+                                     const int &antialiasing)
+    : _kSizeX(kSizeX), _kSizeY(kSizeY), _strideX(strideX), _strideY(strideY), _paddingX(paddingX), _paddingY(paddingY), _ceilMode(ceilMode)
+{
+    (void)antialiasing;
+    if (kSizeX != kSizeY || strideX != strideY || paddingX != paddingY) MSNH_THROW("localavgpool: only square windows are supported");
+    if (kSizeX <= 0 || strideX <= 0) MSNH_THROW("localavgpool: kSize and stride must be positive");
+    _type = LayerType::LOCAL_AVGPOOL;
+    _layerName = "LocalAvgPool    ";
+    _batch = batch; _height = height; _width = width; _channel = channel;
+    _outWidth = pooledSize(width, kSizeX, strideX, paddingX, ceilMode, "localavgpool");
+    _outHeight = pooledSize(height, kSizeY, strideY, paddingY, ceilMode, "localavgpool");
+    _outChannel = channel;
+    _outputNum = _outHeight * _outWidth * _outChannel;
+    _inputNum = height * width * channel;
+    _bFlops = (_kSizeX * _kSizeY * _channel * _outHeight * _outWidth) / 1000000000.f;
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _layerDetail = fmt("avg               %2dx%2d/%2d   %4d x%4d x%4d -> %4d x%4d x%4d %5.3f BF\n", _kSizeX, _kSizeY, _strideX, _width, _height,
+                       _channel, _outWidth, _outHeight, _outChannel, static_cast<double>(_bFlops));
+}
+
+int LocalAvgPoolLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    if (plan.tensors[static_cast<size_t>(in)].layout != PlanTensor::NHWC) MSNH_THROW("localavgpool can not be the first layer of a network");
+    const int out = plan.addTensor(_batch, _outHeight, _outWidth, _outChannel, plan.tensors[static_cast<size_t>(in)].dtype, "avgpool_out");
+    PlanOp &op = plan.addOp(PlanOp::AVGPOOL, in, -1, out, layerIndex, "localavgpool");
+    op.ksize = _kSizeX; op.stride = _strideX; op.pad = _paddingX;
+    return out;
+}
+
+// ---- ConnectedLayer ---------------------------------------------------------------------------------------------------------
+ConnectedLayer::ConnectedLayer(const int &batch, const int &steps, const int &inputNum, const int &outputNum, const ActivationType &activation,
+                               const std::vector<float> &actParams, const int &batchNorm, const float &bnEps, const int &useBias)
+{
+    (void)steps; (void)bnEps;
+    if (batchNorm) MSNH_THROW("connect: batchNorm is outside the convolutional path this build implements");
+    requireDeviceActivation(activation, "connect");
+    if (inputNum <= 0 || outputNum <= 0) MSNH_THROW("connect: input and output sizes must be positive");
+    _type = LayerType::CONNECTED;
+    _layerName = "Connected       ";
+    _inputNum = inputNum; _outputNum = outputNum; _batch = batch; _batchNorm = batchNorm;
+    _height = 1; _width = 1; _channel = inputNum;
+    _outHeight = 1; _outWidth = 1; _outChannel = outputNum; _num = outputNum;
+    _activation = activation; _actParams = actParams; _useBias = useBias;
+    _nWeights = inputNum * outputNum;
+    _nBiases = useBias ? outputNum : 0;
+    _numWeights = static_cast<size_t>(_nWeights + _nBiases);
+    _inputSpaceSize = static_cast<size_t>(_inputNum);
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _layerDetail = fmt("connected                            %4d  ->  %4d\n", inputNum, outputNum);
+}
+
+void ConnectedLayer::loadAllWeigths(std::vector<float> &weights)
+{
+    if (weights.size() != _numWeights)
+        MSNH_THROW("Connect weights load err. needed : " + std::to_string(_numWeights) + " given : " + std::to_string(weights.size()));
+    if (BaseLayer::isPreviewMode) return;
+    _weights.assign(weights.begin(), weights.begin() + _nWeights);
+    if (_useBias) _biases.assign(weights.begin() + _nWeights, weights.end());
+    _weightsLoaded = true;
+}
+
+void ConnectedLayer::foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const
+{
+    scale.clear();
+    shift = _biases;
+}
+
+int ConnectedLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    const PlanTensor ti = plan.tensors[static_cast<size_t>(in)];
+    if (ti.layout == PlanTensor::NCHW_INPUT) MSNH_THROW("connect can not be the first layer of a network");
+    if (ti.layout == PlanTensor::NHWC && ti.h * ti.w != 1)
+        MSNH_THROW("connect: the input must be 1x1 spatially (put a pooling layer before it)");
+    // keep the classifier tail in float32: an average pool feeding the classifier writes float32
+    const int p = plan.producerOf(in);
+    if (p >= 0 && plan.ops[static_cast<size_t>(p)].kind == PlanOp::AVGPOOL && plan.consumerCount(in) == 0)
+        plan.tensors[static_cast<size_t>(in)].dtype = MSNH_F32;
+    const int out = plan.addTensor(_batch, 1, 1, _outputNum, MSNH_F32, "connected_out", PlanTensor::FLAT);
+    PlanOp &op = plan.addOp(PlanOp::CONNECTED, in, -1, out, layerIndex, "connected");
+    op.act = _activation; op.actParam = actParam();
+    op.src = this;
+    return out;
+}
+
+// ---- UpSample / Empty / Route ---------------------------------------------------------------------------------------------------
+UpSampleLayer::UpSampleLayer(const int &batch, const int &width, const int &height, const int &channel, const int &strideX, const int &strideY,
+                             const float &scaleX, const float &scaleY, UpSampleParams::UpsampleType upsampleType, const int &alignCorners)
+    : _strideX(strideX), _strideY(strideY), _scaleX(scaleX), _scaleY(scaleY)
+{
+    (void)alignCorners;
+    if (upsampleType != UpSampleParams::NEAREST) MSNH_THROW("upsample: bilinear mode is outside the convolutional path this build implements");
+    if (strideX != strideY || strideX <= 0) MSNH_THROW("upsample: strideX and strideY must be equal and positive");
+    _type = LayerType::UPSAMPLE;
+    _layerName = "UpSample        ";
+    _batch = batch; _width = width; _height = height; _channel = channel;
+    _outWidth = width * strideX; _outHeight = height * strideY; _outChannel = channel;
+    _outputNum = _outWidth * _outHeight * _outChannel;
+    _inputNum = width * height * channel;
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _layerDetail = fmt("upsample              %2dx%2d  %4d x%4d x%4d -> %4d x%4d x%4d\n", _strideX, _strideY, _width, _height, _channel, _outHeight,
+                       _outHeight, _outChannel);
+}
+
+int UpSampleLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    if (plan.tensors[static_cast<size_t>(in)].layout != PlanTensor::NHWC) MSNH_THROW("upsample can not be the first layer of a network");
+    const int out = plan.addTensor(_batch, _outHeight, _outWidth, _outChannel, plan.tensors[static_cast<size_t>(in)].dtype, "upsample_out");
+    PlanOp &op = plan.addOp(PlanOp::UPSAMPLE, in, -1, out, layerIndex, "upsample");
+    op.stride = _strideX;
+    op.upScale = _scaleX;          // Blas::cpuUpSample is called with scaleX only (src/layers/MsnhUpSampleLayer.cpp:106)
+    return out;
+}
+
+EmptyLayer::EmptyLayer(const int &batch, const int &width, const int &height, const int &channel)
+{
+    _type = LayerType::EMPTY;
+    _layerName = "Empty           ";
+    _batch = batch; _width = width; _height = height; _channel = channel;
+    _outWidth = width; _outHeight = height; _outChannel = channel;
+    _inputNum = width * height * channel;
+    _outputNum = _inputNum;
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _layerDetail = fmt("Empty Layer                  %4d x%4d x%4d -> %4d x%4d x%4d %5.3f BF\n", _width, _height, _channel, _outWidth, _outHeight,
+                       _outChannel, 0.0);
+}
+
+int EmptyLayer::lower(Plan &, int in, int) { return in; }        // identity: the reference copies, the plan aliases
+
+RouteLayer::RouteLayer(const int &batch, std::vector<int> &inputLayerIndexes, std::vector<int> &inputLayerOutputs, const int &groups,
+                       const int &groupIndex, const int &addModel, const ActivationType &activation, const std::vector<float> &actParams)
+    : _inputLayerIndexes(inputLayerIndexes), _inputLayerOutputs(inputLayerOutputs), _groups(groups), _groupIndex(groupIndex), _addModel(addModel)
+{
+    if (addModel == 1 || groups != 1) MSNH_THROW("route: addModel / groups are outside the convolutional path this build implements");
+    if (activation != ActivationType::NONE) MSNH_THROW("route: activation is outside the convolutional path this build implements");
+    _type = LayerType::ROUTE;
+    _layerName = "Route           ";
+    _batch = batch;
+    _activation = activation; _actParams = actParams;
+    _layerDetail = "route ";
+    int outputNum = 0;
+    for (size_t i = 0; i < inputLayerIndexes.size(); ++i)
+    {
+        _layerDetail += fmt(" %d", inputLayerIndexes[i]);
+        outputNum += inputLayerOutputs[i];
+    }
+    _layerDetail += "\n";
+    _outputNum = outputNum;
+    _inputNum = outputNum;
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+}
+
+int RouteLayer::lower(Plan &plan, int, int layerIndex)
+{
+    std::vector<int> srcs;
+    for (int idx : _inputLayerIndexes) srcs.push_back(plan.layerOut[static_cast<size_t>(idx)]);
+    if (srcs.size() == 1) return srcs[0];                        // a single routed layer is an alias, not a copy
+    const PlanTensor first = plan.tensors[static_cast<size_t>(srcs[0])];
+    int channels = 0;
+    for (int s : srcs) channels += plan.tensors[static_cast<size_t>(s)].c;
+    const int out = plan.addTensor(first.n, first.h, first.w, channels, first.dtype, "route_out");
+    int off = 0;
+    for (int s : srcs)
+    {
+        PlanOp &op = plan.addOp(PlanOp::COPY, s, -1, out, layerIndex, "route_copy");
+        op.dstChanOffset = off;
+        off += plan.tensors[static_cast<size_t>(s)].c;
+    }
+    return out;
+}
+
+// ---- blocks -----------------------------------------------------------------------------------------------------------------------
+BlockLayer::~BlockLayer()
+{
+    for (auto &chain : _chains)
+        for (BaseLayer *l : chain) delete l;
+}
+
+std::vector<BaseLayer *> BlockLayer::buildChain(NetBuildParams &params, std::vector<BaseParams *> &nodes, const char *blockName, bool allowEmpty)
+{
+    std::vector<BaseLayer *> chain;
+    try
+    {
+        for (size_t i = 0; i < nodes.size(); ++i)
+        {
+            BaseLayer *layer = nullptr;
+            BaseParams *bp = nodes[i];
+            if (bp->type == LayerType::CONVOLUTIONAL)
+            {
+                if (params.height == 0 || params.width == 0 || params.channels == 0) MSNH_THROW("Layer before convolutional layer must output image");
+                ConvParams *p = static_cast<ConvParams *>(bp);
+                layer = new ConvolutionalLayer(params.batch, 1, params.height, params.width, params.channels, p->filters, p->groups, p->kSizeX, p->kSizeY,
+                                               p->strideX, p->strideY, p->dilationX, p->dilationY, p->paddingX, p->paddingY, p->activation, p->actParams,
+                                               p->batchNorm, p->bnEps, p->useBias, 0, 0, 0, 0, p->antialiasing, nullptr, 0, 0);
+            }
+            else if (bp->type == LayerType::CONNECTED)
+            {
+                ConnectParams *p = static_cast<ConnectParams *>(bp);
+                layer = new ConnectedLayer(params.batch, 1, params.inputNums, p->output, p->activation, p->actParams, p->batchNorm, p->bnEps, p->useBias);
+            }
+            else if (bp->type == LayerType::MAXPOOL)
+            {
+                MaxPoolParams *p = static_cast<MaxPoolParams *>(bp);
+                layer = new MaxPoolLayer(params.batch, params.height, params.width, params.channels, p->kSizeX, p->kSizeY, p->strideX, p->strideY,
+                                         p->paddingX, p->paddingY, p->maxPoolDepth, p->outChannels, p->ceilMode, 0);
+            }
+            else if (bp->type == LayerType::LOCAL_AVGPOOL)
+            {
+                LocalAvgPoolParams *p = static_cast<LocalAvgPoolParams *>(bp);
+                layer = new LocalAvgPoolLayer(params.batch, params.height, params.width, params.channels, p->kSizeX, p->kSizeY, p->strideX, p->strideY,
+                                              p->paddingX, p->paddingY, p->ceilMode, 0);
+            }
+            else if (bp->type == LayerType::BATCHNORM)
+            {
+                BatchNormParams *p = static_cast<BatchNormParams *>(bp);
+                layer = new BatchNormLayer(params.batch, params.width, params.height, params.channels, p->activation, p->eps, p->actParams);
+            }
+            else if (allowEmpty && bp->type == LayerType::EMPTY)
+            {
+                layer = new EmptyLayer(params.batch, params.width, params.height, params.channels);
+            }
+            else
+            {
+                MSNH_THROW(std::string("layer type is not supported by [") + blockName + "]");
+            }
+            chain.push_back(layer);
+            params.height = layer->getOutHeight();
+            params.width = layer->getOutWidth();
+            params.channels = layer->getOutChannel();
+            params.inputNums = layer->getOutputNum();
+            _maxOutputNum = std::max(_maxOutputNum, layer->getMaxOutputNum());
+            _numWeights += layer->getNumWeights();
+            _bFlops += layer->getBFlops();
+            _layerDetail += layer->getLayerDetail();
+            if (_type == LayerType::CONCAT_BLOCK) _layerDetail += "nweights  :" + std::to_string(layer->getNumWeights()) + "\n";
+            layer->setIsBranchLayer(true);
+            layer->setBranchFirst(i == 0);
+            layer->setBranchLast(i + 1 == nodes.size());
+        }
+    }
+    catch (...)
+    {
+        for (BaseLayer *l : chain) delete l;
+        throw;
+    }
+    return chain;
+}
+
+void BlockLayer::loadAllWeigths(std::vector<float> &weights)
+{
+    if (weights.size() != _numWeights)
+        MSNH_THROW(ExString::trim(_layerName) + " weights load err. needed : " + std::to_string(_numWeights) + " given : " + std::to_string(weights.size()));
+    size_t ptr = 0;
+    for (auto &chain : _chains)
+        for (BaseLayer *l : chain)
+        {
+            const size_t n = l->getNumWeights();
+            if (n == 0) continue;
+            std::vector<float> part(weights.begin() + static_cast<long long>(ptr), weights.begin() + static_cast<long long>(ptr + n));
+            l->loadAllWeigths(part);
+            ptr += n;
+        }
+    _weightsLoaded = true;
+}
+
+int BlockLayer::lowerChain(Plan &plan, const std::vector<BaseLayer *> &chain, int in, int layerIndex)
+{
+    int t = in;
+    for (BaseLayer *l : chain) t = l->lower(plan, t, layerIndex);
+    return t;
+}
+
+static int lowerAdd(Plan &plan, int a, int b, ActivationType act, float actParam, int layerIndex)
+{
+    const PlanTensor ta = plan.tensors[static_cast<size_t>(a)];
+    const int out = plan.addTensor(ta.n, ta.h, ta.w, ta.c, ta.dtype, "add_out");
+    PlanOp &op = plan.addOp(PlanOp::ADD, a, b, out, layerIndex, "add");
+    op.act = act; op.actParam = actParam;
+    return out;
+}
+
+static void checkBlockActivation(ActivationType act, const char *name)
+{
+    if (act == ActivationType::PRELU) MSNH_THROW(std::string("prelu activation is not supported by ") + name + " ");
+    if (!Activations::deviceSupported(act)) MSNH_THROW(std::string(name) + ": activation is outside the convolutional path this build implements");
+}
+
+ResBlockLayer::ResBlockLayer(const int &batch, NetBuildParams &params, std::vector<BaseParams *> &baseParams, ActivationType &activation,
+                             const std::vector<float> &actParams)
+{
+    checkBlockActivation(activation, "ResBlock");
+    _type = LayerType::RES_BLOCK;
+    _layerName = "ResBlock        ";
+    _activation = activation; _actParams = actParams; _batch = batch;
+    _width = params.width; _height = params.height; _channel = params.channels;
+    _inputNum = params.width * params.height * params.channels;
+    if (baseParams.empty()) MSNH_THROW("resblock has no layers");
+    _layerDetail = "================================  ResBlock ================================\n";
+    _chains.push_back(buildChain(params, baseParams, "ResBlockLayer", false));
+    _outHeight = params.height; _outWidth = params.width; _outChannel = params.channels; _outputNum = params.inputNums;
+    if (_outputNum != _inputNum) MSNH_THROW("resblock: the output of the block must have the size of its input");
+    _layerDetail += "========================================================================\n";
+}
+
+int ResBlockLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    const int f = lowerChain(plan, _chains[0], in, layerIndex);
+    return lowerAdd(plan, f, in, _activation, actParam(), layerIndex);         // F(x) += x, then activation
+}
+
+Res2BlockLayer::Res2BlockLayer(const int &batch, NetBuildParams &params, std::vector<BaseParams *> &baseParams, std::vector<BaseParams *> &branchParams,
+                               ActivationType &activation, const std::vector<float> &actParams)
+{
+    checkBlockActivation(activation, "Res2Block");
+    _type = LayerType::RES_2_BLOCK;
+    _layerName = "Res2Block       ";
+    _activation = activation; _actParams = actParams; _batch = batch;
+    _width = params.width; _height = params.height; _channel = params.channels;
+    _inputNum = params.width * params.height * params.channels;
+    if (baseParams.empty() || branchParams.empty()) MSNH_THROW("res2block needs a base and a branch");
+    _layerDetail = "================================ Res2Block ================================\n";
+    NetBuildParams branchBuild = params;
+    _chains.push_back(buildChain(params, baseParams, "Res2BlockLayer", false));
+    _chains.push_back(buildChain(branchBuild, branchParams, "Res2BlockLayer", false));
+    if (params.height != branchBuild.height || params.width != branchBuild.width || params.channels != branchBuild.channels)
+        MSNH_THROW("base's outputs size is not equal with branch's outputs size");
+    _outHeight = params.height; _outWidth = params.width; _outChannel = params.channels; _outputNum = params.inputNums;
+    _layerDetail += "========================================================================\n";
+}
+
+int Res2BlockLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    const int base = lowerChain(plan, _chains[0], in, layerIndex);
+    const int branch = lowerChain(plan, _chains[1], in, layerIndex);
+    return lowerAdd(plan, branch, base, _activation, actParam(), layerIndex);  // branch += base, then activation
+}
+
+AddBlockLayer::AddBlockLayer(const int &batch, NetBuildParams &params, std::vector<std::vector<BaseParams *>> &branchParams, ActivationType &activation,
+                             const std::vector<float> &actParams)
+{
+    checkBlockActivation(activation, "AddBlock");
+    _type = LayerType::ADD_BLOCK;
+    _layerName = "AddBlock        ";
+    _activation = activation; _actParams = actParams; _batch = batch;
+    _width = params.width; _height = params.height; _channel = params.channels;
+    _inputNum = params.width * params.height * params.channels;
+    if (branchParams.empty()) MSNH_THROW("addblock has no branch");
+    if (branchParams.size() == 1 && activation != ActivationType::NONE)
+        MSNH_THROW("addblock: a single branch with a block activation is outside the convolutional path this build implements");
+    _layerDetail = "=============================== AddBlock ===============================\n";
+    NetBuildParams last = params;
+    for (size_t i = 0; i < branchParams.size(); ++i)
+    {
+        NetBuildParams bp = params;
+        if (branchParams[i].empty()) MSNH_THROW("addblock: empty branch");
+        _chains.push_back(buildChain(bp, branchParams[i], "AddBlockLayer", true));
+        _layerDetail += "\n";
+        if (i > 0 && (bp.height != last.height || bp.width != last.width || bp.channels != last.channels)) MSNH_THROW("branch's outputs size is not equal");
+        last = bp;
+    }
+    params = last;
+    _outHeight = last.height; _outWidth = last.width; _outChannel = last.channels; _outputNum = last.inputNums;
+    _layerDetail += "========================================================================\n";
+}
+
+int AddBlockLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    int acc = -1;
+    for (size_t i = 0; i < _chains.size(); ++i)
+    {
+        const int y = lowerChain(plan, _chains[i], in, layerIndex);
+        if (acc < 0) { acc = y; continue; }
+        const bool lastBranch = i + 1 == _chains.size();
+        acc = lowerAdd(plan, y, acc, lastBranch ? _activation : ActivationType::NONE, actParam(), layerIndex);      // b[i] += b[i-1]
+    }
+    return acc;
+}
+
+ConcatBlockLayer::ConcatBlockLayer(const int &batch, NetBuildParams &params, std::vector<std::vector<BaseParams *>> &branchParams,
+                                   ActivationType &activation, const std::vector<float> &actParams)
+{
+    if (activation != ActivationType::NONE) MSNH_THROW("concatblock: a block activation is outside the convolutional path this build implements");
+    _type = LayerType::CONCAT_BLOCK;
+    _layerName = "ConcatBlock     ";
+    _activation = activation; _actParams = actParams; _batch = batch;
+    _width = params.width; _height = params.height; _channel = params.channels;
+    _inputNum = params.width * params.height * params.channels;
+    if (branchParams.empty()) MSNH_THROW("concatblock has no branch");
+    _layerDetail = "=============================== ConcatBlock ===============================\n";
+    int channels = 0;
+    NetBuildParams last = params;
+    for (size_t i = 0; i < branchParams.size(); ++i)
+    {
+        NetBuildParams bp = params;
+        if (branchParams[i].empty()) MSNH_THROW("concatblock: empty branch");
+        _chains.push_back(buildChain(bp, branchParams[i], "ConcatBlockLayer", true));
+        _layerDetail += "\n";
+        if (i > 0 && (bp.height != last.height || bp.width != last.width)) MSNH_THROW("branch's outputs size is not equal");
+        channels += bp.channels;
+        last = bp;
+    }
+    _outHeight = last.height; _outWidth = last.width; _outChannel = channels;
+    _outputNum = _outHeight * _outWidth * _outChannel;
+    params.height = _outHeight; params.width = _outWidth; params.channels = _outChannel; params.inputNums = _outputNum;
+    _maxOutputNum = std::max(_maxOutputNum, static_cast<size_t>(_batch) * _outputNum);
+    _layerDetail += "===========================================================================\n";
+}
+
+int ConcatBlockLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    std::vector<int> outs;
+    for (auto &chain : _chains) outs.push_back(lowerChain(plan, chain, in, layerIndex));
+    const PlanTensor first = plan.tensors[static_cast<size_t>(outs[0])];
+    const int out = plan.addTensor(first.n, first.h, first.w, _outChannel, first.dtype, "concat_out");
+    int off = 0;
+    for (int s : outs)
+    {
+        PlanOp &op = plan.addOp(PlanOp::COPY, s, -1, out, layerIndex, "concat_copy");
+        op.dstChanOffset = off;
+        off += plan.tensors[static_cast<size_t>(s)].c;
+    }
+    return out;
+}
+
+// ---- YOLO ------------------------------------------------------------------------------------------------------------------------------
+YoloLayer::YoloLayer(const int &batch, const int &width, const int &height, const int &num, const int &orgWidth, const int &orgHeight,
+                     const int &classNum, const std::vector<float> &anchors, const YoloType &yoloType)
+    : anchors(anchors), _orgHeight(orgHeight), _orgWidth(orgWidth), _classNum(classNum), _yoloType(yoloType)
+{
+    _type = LayerType::YOLO;
+    _layerName = "Yolo            ";
+    _num = num; _batch = batch; _height = height; _width = width; _channel = num;
+    _outWidth = width; _outHeight = height; _outChannel = num;
+    _outputNum = height * width * num;
+    _inputNum = _outputNum;
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _ratios = 1.f * orgHeight / _outHeight;          // height only, used for both axes (src/layers/MsnhYoloLayer.cpp:34)
+    if (3 * (classNum + 4 + 1) != num) MSNH_THROW("class num error!");
+    if (this->anchors.size() != 6) MSNH_THROW("[yolo] anchor num should be 6");
+    if (static_cast<int>(yoloType) / 10 != 3 && static_cast<int>(yoloType) / 10 != 4) MSNH_THROW("yolo: only yolov3 / yolov4 decoding is implemented");
+    if (yoloType != YoloType::YoloV3 && yoloType != YoloType::YoloV4) MSNH_THROW("yolo: angle / gaussian variants are outside the convolutional path this build implements");
+    _memReUse = 0;
+    _layerDetail = "Yolo. class num : " + std::to_string(classNum) + "\n";
+}
+
+int YoloLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    if (layerIndex == 0) MSNH_THROW("Yolo layer should not be 0 layer");
+    // logits feeding the decode stay in float32: sigmoid / exp are evaluated on them exactly once
+    const int p = plan.producerOf(in);
+    if (p >= 0 && plan.ops[static_cast<size_t>(p)].kind == PlanOp::CONV && plan.consumerCount(in) == 0)
+        plan.tensors[static_cast<size_t>(in)].dtype = MSNH_F32;
+    const int out = plan.addTensor(_batch, _outHeight, _outWidth, _outChannel, MSNH_F32, "yolo_decoded", PlanTensor::FLAT);
+    plan.tensors[static_cast<size_t>(out)].external = true;      // lives in Plan::yoloDecoded
+    PlanOp &op = plan.addOp(PlanOp::YOLO_DECODE, in, -1, out, layerIndex, "yolo_decode");
+    for (int i = 0; i < 6; ++i) op.anchors[static_cast<size_t>(i)] = anchors[static_cast<size_t>(i)];
+    op.classes = _classNum;
+    op.ratio = _ratios;
+    op.confThresh = 2.f;
+    decodeOp = plan.ops.size() - 1;
+    return out;
+}
+
+bool YoloOutLayer::keepClassScores = false;
+
+YoloOutLayer::YoloOutLayer(const int &batch, const int &orgWidth, const int &orgHeight, std::vector<int> &yoloIndexes, std::vector<YoloInfo> &yoloLayersInfo,
+                           const float &confThresh, const float &nmsThresh, const int &useSotfNms, const YoloType &yoloType)
+    : _confThresh(confThresh), _nmsThresh(nmsThresh), _useSoftNms(useSotfNms), _orgHeight(orgHeight), _orgWidth(orgWidth), _yoloType(yoloType),
+      _yoloIndexes(yoloIndexes), _yoloLayersInfo(yoloLayersInfo)
+{
+    if (yoloType != YoloType::YoloV3 && yoloType != YoloType::YoloV4) MSNH_THROW("yoloout: only yolov3 / yolov4 are implemented");
+    _type = LayerType::YOLO_OUT;
+    _layerName = "YoloOut         ";
+    _batch = batch;
+    _layerDetail = "YoloOut    ";
+    for (size_t i = 0; i < yoloIndexes.size(); ++i)
+    {
+        _width += yoloLayersInfo[i].outWidth;
+        _height += yoloLayersInfo[i].outHeight;
+        _layerDetail += fmt(" %d", yoloIndexes[i]);
+        _yoloAllInputNum += yoloLayersInfo[i].getOutputNum();
+        if (yoloLayersInfo[i].outChannel != yoloLayersInfo[0].outChannel) MSNH_THROW("yoloout: heads disagree on the class count");
+    }
+    _channel = yoloLayersInfo[0].outChannel / 3;
+    _pixels = _yoloAllInputNum / _channel;
+    _layerDetail += "\n";
+    _memReUse = 0;
+}
+
+int YoloOutLayer::lower(Plan &plan, int, int layerIndex)
+{
+    // claim the heads: give each its cell range inside an image's decoded rows and switch its candidate list on
+    int cell = 0;
+    for (size_t i = 0; i < _yoloIndexes.size(); ++i)
+    {
+        const int t = plan.layerOut[static_cast<size_t>(_yoloIndexes[i])];
+        const int p = plan.producerOf(t);
+        if (p < 0 || plan.ops[static_cast<size_t>(p)].kind != PlanOp::YOLO_DECODE) MSNH_THROW("yoloout layer error, not a yolo layer");
+        PlanOp &op = plan.ops[static_cast<size_t>(p)];
+        op.cellBase = cell;
+        op.confThresh = _confThresh;
+        cell += 3 * _yoloLayersInfo[i].outHeight * _yoloLayersInfo[i].outWidth;
+    }
+    plan.yoloCells = cell;
+    plan.yoloClasses = _channel - 5;
+    (void)layerIndex;
+    return plan.addTensor(_batch, 1, 1, 0, MSNH_F32, "yoloout", PlanTensor::FLAT);
+}
+
+std::vector<YoloBox> YoloOutLayer::boxesFromRows(const float *rows, int count, const float *decodedOfImage) const
+{
+    // Candidates arrive in arbitrary order; the reference scans cells in ascending order
+    // (src/layers/MsnhYoloOutLayer.cpp:120-170), so restore that first.
+    std::vector<int> order(static_cast<size_t>(count));
+    for (int i = 0; i < count; ++i) order[static_cast<size_t>(i)] = i;
+    std::sort(order.begin(), order.end(), [rows](int a, int b) { return rows[a * 8 + 7] < rows[b * 8 + 7]; });
+    std::vector<YoloBox> boxes(static_cast<size_t>(count));
+    std::vector<float> keys(static_cast<size_t>(count));
+    for (int i = 0; i < count; ++i)
+    {
+        const float *r = rows + static_cast<size_t>(order[static_cast<size_t>(i)]) * 8;
+        YoloBox &b = boxes[static_cast<size_t>(i)];
+        b.xywhBox = Box::XYWHBox(r[0], r[1], r[2], r[3]);
+        b.conf = r[4];
+        b.bestClsConf = r[5];
+        b.bestClsIdx = static_cast<int>(r[6]);
+        if (decodedOfImage)
+        {
+            const float *row = decodedOfImage + static_cast<size_t>(r[7]) * _channel;
+            b.classesVal.assign(row + 5, row + _channel);
+        }
+        keys[static_cast<size_t>(i)] = b.conf * b.bestClsConf;
+    }
+    // descending by objectness * best class score (:175-194)
+    const std::vector<int> idx = ExVector::argsort(keys, true);
+    std::vector<YoloBox> sorted(static_cast<size_t>(count));
+    for (int i = 0; i < count; ++i) sorted[static_cast<size_t>(i)] = std::move(boxes[static_cast<size_t>(idx[static_cast<size_t>(i)])]);
+    return sorted;
+}
+
+// Per-class greedy NMS exactly as the reference runs it (src/layers/MsnhYoloOutLayer.cpp:381-461): classes in
+// first-appearance order, pick the highest objectness (first on ties), drop iou > thresh; a class with one
+// box passes through.  NaN IoU (boxes with infinite extent) never suppresses, like there.
+std::vector<YoloBox> YoloOutLayer::nms(const std::vector<YoloBox> &bboxes, const float &nmsThresh, const bool &useSoftNms, const float &sigma)
+{
+    std::vector<YoloBox> best;
+    std::vector<int> classes;
+    for (const YoloBox &b : bboxes)
+        if (!ExVector::contains<int>(classes, b.bestClsIdx)) classes.push_back(b.bestClsIdx);
+    std::vector<const YoloBox *> cur;
+    for (int cls : classes)
+    {
+        cur.clear();
+        for (const YoloBox &b : bboxes)
+            if (b.bestClsIdx == cls) cur.push_back(&b);
+        if (cur.size() == 1) { best.push_back(*cur[0]); continue; }
+        while (!cur.empty())
+        {
+            size_t bi = 0;
+            float bc = -FLT_MAX;
+            for (size_t j = 0; j < cur.size(); ++j)
+                if (cur[j]->conf > bc) { bi = j; bc = cur[j]->conf; }
+            const YoloBox *top = cur[bi];
+            best.push_back(*top);
+            cur.erase(cur.begin() + static_cast<long long>(bi));
+            size_t w = 0;
+            for (size_t j = 0; j < cur.size(); ++j)
+            {
+                const float iou = Box::iou(cur[j]->xywhBox, top->xywhBox);
+                bool drop;
+                if (useSoftNms) drop = cur[j]->conf * std::exp(-(1.f * iou * iou / sigma)) <= 0;
+                else drop = iou > nmsThresh;
+                if (!drop) cur[w++] = cur[j];
+            }
+            cur.resize(w);
+        }
+    }
+    return best;
+}
+
+void YoloOutLayer::forwardGPU(NetworkState &netState)
+{
+    if (plan == nullptr) MSNH_THROW("YoloOut: layer is not part of a planned network");
+    Plan &pl = *plan;
+    msnh_stream_t s = netState.stream;
+    const int cells = pl.yoloCells;
+    const int per = _channel;
+    MSNH_DEV(msnh_hip_yolo_gather(_batch, per - 5, pl.yoloDecoded.as<float>(), static_cast<long long>(cells) * per, pl.yoloCandIdx.as<int>(), cells,
+                                  pl.yoloCandCnt.as<int>(), pl.yoloRows.as<float>(), s));
+    _hostCnt.reserve(sizeof(int) * static_cast<size_t>(_batch));
+    MSNH_DEV(msnh_hip_memcpy_d2h(_hostCnt.ptr(), pl.yoloCandCnt.ptr(), sizeof(int) * static_cast<size_t>(_batch), s));
+    MSNH_DEV(msnh_hip_stream_sync(s));
+    const int *cnt = _hostCnt.as<int>();
+    _hostRows.reserve(sizeof(float) * 8 * static_cast<size_t>(cells) * static_cast<size_t>(_batch));
+    for (int b = 0; b < _batch; ++b)
+    {
+        const int n = std::min(cnt[b], cells);
+        if (n > 0)
+            MSNH_DEV(msnh_hip_memcpy_d2h(_hostRows.as<float>() + static_cast<size_t>(b) * cells * 8,
+                                         pl.yoloRows.as<float>() + static_cast<size_t>(b) * cells * 8, sizeof(float) * 8 * static_cast<size_t>(n), s));
+    }
+    const float *decodedHost = nullptr;
+    if (keepClassScores)
+    {
+        const size_t bytes = sizeof(float) * static_cast<size_t>(cells) * per * static_cast<size_t>(_batch);
+        _hostDecoded.reserve(bytes);
+        MSNH_DEV(msnh_hip_memcpy_d2h(_hostDecoded.ptr(), pl.yoloDecoded.ptr(), bytes, s));
+        decodedHost = _hostDecoded.as<float>();
+    }
+    MSNH_DEV(msnh_hip_stream_sync(s));
+
+    batchHasBox.assign(static_cast<size_t>(_batch), false);
+    finalOut.assign(static_cast<size_t>(_batch), std::vector<YoloBox>());
+#pragma omp parallel for schedule(dynamic)
+    for (int b = 0; b < _batch; ++b)
+    {
+        const int n = std::min(cnt[b], cells);
+        const float *dec = decodedHost ? decodedHost + static_cast<size_t>(b) * cells * per : nullptr;
+        std::vector<YoloBox> cand = boxesFromRows(_hostRows.as<float>() + static_cast<size_t>(b) * cells * 8, n, dec);
+        finalOut[static_cast<size_t>(b)] = nms(cand, _nmsThresh, _useSoftNms != 0);
+    }
+    for (int b = 0; b < _batch; ++b) batchHasBox[static_cast<size_t>(b)] = cnt[b] > 0;
+}
+}

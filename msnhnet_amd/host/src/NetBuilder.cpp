@@ -1,0 +1,614 @@
+// NetBuilder: graph construction, weight loading, planning and the run entry points.
+// Control flow and error texts follow src/net/MsnhNetBuilder.cpp of the reference (build :68-622, load :624-663,
+// run :820-1007); what happens underneath -- one planned device arena, fused launches, a captured graph --
+// is new.
+#include "Msnhnet/net/MsnhNetBuilder.h"
+#include <cmath>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+#include <sstream>
+
+namespace Msnhnet
+{
+void Network::forward(NetworkState &) { MSNH_THROW("Gpu mode , can not run with cpu"); }
+
+void Network::forwardGPU(NetworkState &netState)
+{
+    for (BaseLayer *l : layers) l->forwardGPU(netState);
+}
+
+NetBuilder::NetBuilder()
+{
+    _parser = new Parser();
+    _net = new Network();
+    _netState = new NetworkState();
+    _netState->net = _net;
+}
+
+NetBuilder::~NetBuilder()
+{
+    clearLayers();
+    if (_stream) msnh_hip_stream_destroy(_stream);
+    delete _netState;
+    delete _net;
+    delete _parser;
+}
+
+void NetBuilder::setPreviewMode(const bool &mode) { BaseLayer::setPreviewMode(mode); }
+void NetBuilder::setMemAlign(const bool &memAlign) { BaseLayer::setMemAlign(memAlign); }
+void NetBuilder::setOnlyGpu(const bool &onlyGpu) { BaseLayer::setOnlyGpu(onlyGpu); }
+void NetBuilder::setUseFp16(const bool &useFp16) { BaseLayer::setUseFp16(useFp16); }
+void NetBuilder::setForceUseCuda(const bool &v) { BaseLayer::setForceUseCuda(v); }
+void NetBuilder::setKeepClassScores(const bool &keep) { YoloOutLayer::keepClassScores = keep; }
+
+void NetBuilder::setOnlyCpu(const bool &onlyCpu)
+{
+    if (onlyCpu) MSNH_THROW("cpu only mode is not available: this build has no CPU compute path");
+    BaseLayer::setOnlyCpu(false);
+}
+
+void NetBuilder::clearLayers()
+{
+    if (_graph) { msnh_hip_graph_destroy(_graph); _graph = nullptr; }
+    _net->plan.reset();
+    for (BaseLayer *l : _net->layers) delete l;
+    _net->layers.clear();
+    _planReady = false;
+    _layerOutputs.clear();
+}
+
+// ---- build -----------------------------------------------------------------------------------------------------------
+void NetBuilder::buildNetFromMsnhNet(const std::string &path)
+{
+    _parser->readCfg(path);
+    clearLayers();
+    if (BaseLayer::onlyUseGpu && BaseLayer::onlyUseCpu) MSNH_THROW("Gpu only mode and cpu only mode can not use at the same time!");
+
+    NetBuildParams params;
+    for (size_t i = 0; i < _parser->params.size(); ++i)
+    {
+        BaseParams *bp = _parser->params[i];
+        BaseLayer *layer = nullptr;
+        if (i == 0)
+        {
+            if (bp->type != LayerType::CONFIG) MSNH_THROW("The first params must be config");
+            NetConfigParams *cfg = static_cast<NetConfigParams *>(bp);
+            if (cfg->height <= 0 || cfg->width <= 0 || cfg->channels <= 0 || cfg->batch <= 0) MSNH_THROW("net config params err, params = 0 or < 0");
+            _net->batch = cfg->batch; _net->channels = cfg->channels; _net->width = cfg->width; _net->height = cfg->height;
+            _net->inputNum = _net->batch * _net->channels * _net->width * _net->height;
+            params.height = _net->height; params.batch = _net->batch; params.width = _net->width; params.channels = _net->channels;
+            params.inputNums = _net->inputNum;
+            continue;
+        }
+        const size_t nLayers = _net->layers.size();
+        switch (bp->type)
+        {
+        case LayerType::CONVOLUTIONAL:
+        {
+            if (params.height == 0 || params.width == 0 || params.channels == 0) MSNH_THROW("Layer before convolutional layer must output image");
+            ConvParams *p = static_cast<ConvParams *>(bp);
+            layer = new ConvolutionalLayer(params.batch, 1, params.height, params.width, params.channels, p->filters, p->groups, p->kSizeX, p->kSizeY,
+                                           p->strideX, p->strideY, p->dilationX, p->dilationY, p->paddingX, p->paddingY, p->activation, p->actParams,
+                                           p->batchNorm, p->bnEps, p->useBias, 0, 0, 0, 0, p->antialiasing, nullptr, 0, 0);
+            break;
+        }
+        case LayerType::CONNECTED:
+        {
+            ConnectParams *p = static_cast<ConnectParams *>(bp);
+            // inputs of one sample (the reference's batch-1 files make params.inputNums exactly that)
+            layer = new ConnectedLayer(params.batch, 1, params.height * params.width * params.channels, p->output, p->activation, p->actParams,
+                                       p->batchNorm, p->bnEps, p->useBias);
+            break;
+        }
+        case LayerType::MAXPOOL:
+        {
+            MaxPoolParams *p = static_cast<MaxPoolParams *>(bp);
+            layer = new MaxPoolLayer(params.batch, params.height, params.width, params.channels, p->kSizeX, p->kSizeY, p->strideX, p->strideY, p->paddingX,
+                                     p->paddingY, p->maxPoolDepth, p->outChannels, p->ceilMode, 0);
+            break;
+        }
+        case LayerType::LOCAL_AVGPOOL:
+        {
+            LocalAvgPoolParams *p = static_cast<LocalAvgPoolParams *>(bp);
+            layer = new LocalAvgPoolLayer(params.batch, params.height, params.width, params.channels, p->kSizeX, p->kSizeY, p->strideX, p->strideY,
+                                          p->paddingX, p->paddingY, p->ceilMode, 0);
+            break;
+        }
+        case LayerType::BATCHNORM:
+        {
+            BatchNormParams *p = static_cast<BatchNormParams *>(bp);
+            layer = new BatchNormLayer(params.batch, params.width, params.height, params.channels, p->activation, p->eps, p->actParams);
+            break;
+        }
+        case LayerType::RES_BLOCK:
+        {
+            ResBlockParams *p = static_cast<ResBlockParams *>(bp);
+            layer = new ResBlockLayer(params.batch, params, p->baseParams, p->activation, p->actParams);
+            break;
+        }
+        case LayerType::RES_2_BLOCK:
+        {
+            Res2BlockParams *p = static_cast<Res2BlockParams *>(bp);
+            layer = new Res2BlockLayer(params.batch, params, p->baseParams, p->branchParams, p->activation, p->actParams);
+            break;
+        }
+        case LayerType::ADD_BLOCK:
+        {
+            AddBlockParams *p = static_cast<AddBlockParams *>(bp);
+            layer = new AddBlockLayer(params.batch, params, p->branchParams, p->activation, p->actParams);
+            break;
+        }
+        case LayerType::CONCAT_BLOCK:
+        {
+            ConcatBlockParams *p = static_cast<ConcatBlockParams *>(bp);
+            layer = new ConcatBlockLayer(params.batch, params, p->branchParams, p->activation, p->actParams);
+            break;
+        }
+        case LayerType::EMPTY:
+            layer = new EmptyLayer(params.batch, params.width, params.height, params.channels);
+            break;
+        case LayerType::ROUTE:
+        {
+            RouteParams *p = static_cast<RouteParams *>(bp);
+            if (p->layerIndexes.size() < 1) MSNH_THROW("route layer error, no route layers");
+            std::vector<int> outputs, chans;
+            int outC = 0, outH = 0, outW = 0;
+            for (size_t k = 0; k < p->layerIndexes.size(); ++k)
+            {
+                const int idx = p->layerIndexes[k];
+                if (idx < 0 || static_cast<size_t>(idx) >= nLayers) MSNH_THROW("route layer error, route layers index should < size of layers");
+                const BaseLayer *src = _net->layers[static_cast<size_t>(idx)];
+                if (k > 0 && (src->getOutHeight() != outH || src->getOutWidth() != outW))
+                {
+                    std::string indexes;
+                    for (int v : p->layerIndexes) indexes += std::to_string(v) + ", ";
+                    MSNH_THROW("[route] layers height or width not equal. layer: " + std::to_string(i - 1) + "  aux: " + indexes + "wh: " +
+                               std::to_string(outW) + ":" + std::to_string(src->getOutWidth()) + " , " + std::to_string(outH) + ":" +
+                               std::to_string(src->getOutHeight()) + " ");
+                }
+                outH = src->getOutHeight(); outW = src->getOutWidth();
+                outC += src->getOutChannel();
+                outputs.push_back(src->getOutputNum());
+                chans.push_back(src->getOutChannel());
+            }
+            RouteLayer *r = new RouteLayer(params.batch, p->layerIndexes, outputs, p->groups, p->groupsId, p->addModel, p->activation, p->actParams);
+            r->inputChannels = chans;
+            r->setOutChannel(outC); r->setOutWidth(outW); r->setOutHeight(outH);
+            layer = r;
+            break;
+        }
+        case LayerType::UPSAMPLE:
+        {
+            UpSampleParams *p = static_cast<UpSampleParams *>(bp);
+            layer = new UpSampleLayer(params.batch, params.width, params.height, params.channels, p->strideX, p->strideY, p->scaleX, p->scaleY,
+                                      p->upsampleType, p->alignCorners);
+            break;
+        }
+        case LayerType::YOLO:
+        {
+            YoloParams *p = static_cast<YoloParams *>(bp);
+            layer = new YoloLayer(params.batch, params.width, params.height, params.channels, p->orgWidth, p->orgHeight, p->classNum, p->anchors, p->yoloType);
+            break;
+        }
+        case LayerType::YOLO_OUT:
+        {
+            YoloOutParams *p = static_cast<YoloOutParams *>(bp);
+            if (p->layerIndexes.size() < 1) MSNH_THROW("yoloOut layer error, no yolo layers");
+            std::vector<YoloInfo> infos;
+            for (int idx : p->layerIndexes)
+            {
+                if (idx < 0 || static_cast<size_t>(idx) >= nLayers) MSNH_THROW("yoloout layer error, yolo layers index should < size of layers");
+                const BaseLayer *src = _net->layers[static_cast<size_t>(idx)];
+                if (src->type() != LayerType::YOLO) MSNH_THROW("yoloout layer error, not a yolo layer");
+                infos.push_back(YoloInfo(src->getOutHeight(), src->getOutWidth(), src->getOutChannel()));
+            }
+            layer = new YoloOutLayer(params.batch, p->orgWidth, p->orgHeight, p->layerIndexes, infos, p->confThresh, p->nmsThresh, p->useSoftNms, p->yoloType);
+            break;
+        }
+        default:
+            MSNH_THROW("layer type " + std::to_string(static_cast<int>(bp->type)) + " is outside the convolutional path this build implements");
+        }
+        params.height = layer->getOutHeight();
+        params.width = layer->getOutWidth();
+        params.channels = layer->getOutChannel();
+        params.inputNums = layer->getOutputNum();
+        layer->setLayerIndex(static_cast<int>(i) - 1);
+        _net->layers.push_back(layer);
+    }
+    if (_net->layers.empty()) MSNH_THROW("the network has no layers");
+    BaseLayer *last = _net->layers.back();
+    _lastLayerOutHeight = last->getOutHeight(); _lastLayerOutWidth = last->getOutWidth(); _lastLayerOutChannel = last->getOutChannel();
+    _lastLayerOutNum = static_cast<size_t>(last->getOutputNum());
+}
+
+// ---- weights ---------------------------------------------------------------------------------------------------------
+void NetBuilder::loadWeightsFromMsnhBin(const std::string &path)
+{
+    if (BaseLayer::isPreviewMode) MSNH_THROW("Can not load weights in preview mode !");
+    _parser->readMsnhBin(path);
+    loadWeightsFromVector(_parser->msnhF32Weights);
+    std::vector<float>().swap(_parser->msnhF32Weights);
+}
+
+void NetBuilder::loadWeightsFromVector(const std::vector<float> &all)
+{
+    if (BaseLayer::isPreviewMode) MSNH_THROW("Can not load weights in preview mode !");
+    size_t ptr = 0;
+    for (BaseLayer *l : _net->layers)
+    {
+        const LayerType t = l->type();
+        const bool has = t == CONVOLUTIONAL || t == CONNECTED || t == BATCHNORM || t == RES_BLOCK || t == RES_2_BLOCK || t == ADD_BLOCK || t == CONCAT_BLOCK;
+        if (!has) continue;
+        const size_t n = l->getNumWeights();
+        if (ptr + n > all.size())
+            MSNH_THROW("Load weights err, need > given. Needed :" + std::to_string(ptr + n) + " given :" + std::to_string(all.size()));
+        std::vector<float> part(all.begin() + static_cast<long long>(ptr), all.begin() + static_cast<long long>(ptr + n));
+        l->loadAllWeigths(part);
+        ptr += n;
+    }
+    if (ptr != all.size()) MSNH_THROW("Load weights err, need != given. Needed :" + std::to_string(ptr) + " given :" + std::to_string(all.size()));
+    finalizePlan();
+}
+
+// ---- planning --------------------------------------------------------------------------------------------------------
+std::unique_ptr<Plan> NetBuilder::lowerNetwork(int dtype)
+{
+    std::unique_ptr<Plan> plan(new Plan(dtype));
+    plan->inputTensor = plan->addTensor(_net->batch, _net->height, _net->width, _net->channels, MSNH_F32, "input", PlanTensor::NCHW_INPUT);
+    plan->tensors[static_cast<size_t>(plan->inputTensor)].external = true;
+    plan->tensors[static_cast<size_t>(plan->inputTensor)].extPtr = _inputDev.ptr();
+    int cur = plan->inputTensor;
+    for (size_t i = 0; i < _net->layers.size(); ++i)
+    {
+        BaseLayer *l = _net->layers[i];
+        const size_t before = plan->ops.size();
+        if (l->type() != LayerType::CONVOLUTIONAL && l->type() != LayerType::ROUTE && l->type() != LayerType::YOLO_OUT &&
+            plan->tensors[static_cast<size_t>(cur)].layout == PlanTensor::NCHW_INPUT)
+        {
+            // any first layer other than a conv reads NHWC: convert the input once
+            const int cast = plan->addTensor(_net->batch, _net->height, _net->width, _net->channels, dtype, "input_nhwc");
+            plan->addOp(PlanOp::INPUT_CAST, cur, -1, cast, static_cast<int>(i), "input_cast");
+            cur = cast;
+        }
+        cur = l->lower(*plan, cur, static_cast<int>(i));
+        plan->layerOut.push_back(cur);
+        (void)before;
+        if (_saveLayerOutput) plan->tensors[static_cast<size_t>(cur)].pinned = true;
+    }
+    // whatever the caller can still ask for after the forward must survive it
+    plan->tensors[static_cast<size_t>(plan->layerOut.back())].persistent = true;
+    for (size_t i = 0; i < _net->layers.size(); ++i)
+        if (_saveLayerOutput) plan->tensors[static_cast<size_t>(plan->layerOut[i])].persistent = true;
+    return plan;
+}
+
+static void setupYoloBuffers(Plan &plan, int batch)
+{
+    if (plan.yoloCells <= 0)
+    {
+        // yolo layers without a yoloout still need somewhere to decode into
+        int cells = 0;
+        for (PlanOp &op : plan.ops)
+            if (op.kind == PlanOp::YOLO_DECODE)
+            {
+                const PlanTensor &in = plan.tensors[static_cast<size_t>(op.in0)];
+                op.cellBase = cells;
+                cells += 3 * in.h * in.w;
+                plan.yoloClasses = op.classes;
+            }
+        plan.yoloCells = cells;
+    }
+    if (plan.yoloCells <= 0) return;
+    const size_t per = static_cast<size_t>(5 + plan.yoloClasses);
+    const size_t cells = static_cast<size_t>(plan.yoloCells);
+    plan.yoloDecoded.alloc(sizeof(float) * cells * per * static_cast<size_t>(batch));
+    plan.yoloCandIdx.alloc(sizeof(int) * cells * static_cast<size_t>(batch));
+    plan.yoloCandCnt.alloc(sizeof(int) * static_cast<size_t>(std::max(batch, 64)));
+    plan.yoloRows.alloc(sizeof(float) * 8 * cells * static_cast<size_t>(batch));
+}
+
+void NetBuilder::finalizePlan()
+{
+    Device::ensureInit();
+    if (_stream == nullptr) MSNH_DEV(msnh_hip_stream_create(&_stream));
+    _netState->stream = _stream;
+    const size_t inBytes = sizeof(float) * static_cast<size_t>(_net->inputNum);
+    if (_inputDev.bytes() < inBytes) _inputDev.alloc(inBytes);
+    _inputPinned.reserve(inBytes);
+    _netState->gpuInput = _inputDev.as<float>();
+    if (_graph) { msnh_hip_graph_destroy(_graph); _graph = nullptr; }
+
+    const int dtype = BaseLayer::useFp16 ? MSNH_F16 : MSNH_F32;
+    std::unique_ptr<Plan> plan = lowerNetwork(dtype);
+    plan->fuse();
+    plan->aliasConcats();
+
+    if (dtype == MSNH_F16)
+    {
+        // One float32 pass over a fixed pseudo-random U[0,1) input fixes the power-of-two scale of every
+        // float16 tensor.  The float32 twin is lowered and optimised identically, so tensor ids line up.
+        std::unique_ptr<Plan> cal = lowerNetwork(MSNH_F32);
+        cal->fuse();
+        cal->aliasConcats();
+        cal->place();
+        setupYoloBuffers(*cal, _net->batch);
+        cal->prepareWeights();
+        float *host = _inputPinned.as<float>();
+        uint32_t state = 0x9E3779B9u;
+        for (int i = 0; i < _net->inputNum; ++i)
+        {
+            state = state * 1664525u + 1013904223u;
+            host[i] = static_cast<float>(state >> 8) * (1.0f / 16777216.0f);
+        }
+        MSNH_DEV(msnh_hip_memcpy_h2d(_inputDev.ptr(), host, inBytes, _stream));
+        if (cal->yoloCandCnt.ptr()) MSNH_DEV(msnh_hip_fill_zero(cal->yoloCandCnt.ptr(), cal->yoloCandCnt.bytes(), _stream));
+        cal->runAll(_stream);
+        cal->measureAmax(_stream);
+        plan->applyCalibration(*cal);
+    }
+    plan->place();
+    setupYoloBuffers(*plan, _net->batch);
+    plan->prepareWeights();
+
+    // hand every layer its slice of the op list
+    for (size_t i = 0; i < _net->layers.size(); ++i)
+    {
+        BaseLayer *l = _net->layers[i];
+        l->plan = plan.get();
+        l->outTensor = plan->layerOut[i];
+        size_t b = plan->ops.size(), e = 0;
+        for (size_t k = 0; k < plan->ops.size(); ++k)
+            if (plan->ops[k].layerIndex == static_cast<int>(i)) { b = std::min(b, k); e = std::max(e, k + 1); }
+        if (e == 0) b = 0;
+        l->opBegin = b; l->opEnd = e;
+    }
+    _net->plan = std::move(plan);
+    _planReady = true;
+}
+
+// ---- run -------------------------------------------------------------------------------------------------------------
+void NetBuilder::checkInput(size_t given) const
+{
+    if (BaseLayer::isPreviewMode) MSNH_THROW("Can not infer in preview mode !");
+    if (_net->layers.empty()) MSNH_THROW("the network is not built");
+    const size_t need = static_cast<size_t>(_net->inputNum);
+    if (need != given) MSNH_THROW("input image size err. Needed :" + std::to_string(need) + " given :" + std::to_string(given));
+    if (!_planReady) MSNH_THROW("weights are not loaded");
+}
+
+std::vector<float> NetBuilder::runClassify(std::vector<float>) { MSNH_THROW("Gpu mode , can not run with cpu"); }
+std::vector<std::vector<YoloBox>> NetBuilder::runYolo(std::vector<float>) { MSNH_THROW("Gpu mode , can not run with cpu"); }
+
+void NetBuilder::uploadInput(const std::vector<float> &img)
+{
+    std::memcpy(_inputPinned.ptr(), img.data(), img.size() * sizeof(float));
+    MSNH_DEV(msnh_hip_memcpy_h2d(_inputDev.ptr(), _inputPinned.ptr(), img.size() * sizeof(float), _stream));
+}
+
+float *NetBuilder::deviceInputBuffer() { return _inputDev.as<float>(); }
+
+static std::vector<float> yoloLayerDump(Plan &plan, const YoloLayer *yl, const PlanOp &op, int batch, msnh_stream_t s)
+{
+    // decoded rows [cell][5+classes] of this head -> the reference's NCHW [anchor*(5+classes)+m][pixel] order
+    const int per = 5 + op.classes;
+    const int hw = yl->getOutHeight() * yl->getOutWidth();
+    std::vector<float> all(static_cast<size_t>(plan.yoloCells) * per * batch);
+    MSNH_DEV(msnh_hip_memcpy_d2h(all.data(), plan.yoloDecoded.ptr(), all.size() * sizeof(float), s));
+    MSNH_DEV(msnh_hip_stream_sync(s));
+    std::vector<float> out(static_cast<size_t>(batch) * 3 * per * hw);
+    for (int b = 0; b < batch; ++b)
+        for (int a = 0; a < 3; ++a)
+            for (int p = 0; p < hw; ++p)
+                for (int m = 0; m < per; ++m)
+                    out[((static_cast<size_t>(b) * 3 + a) * per + m) * hw + p] =
+                        all[(static_cast<size_t>(b) * plan.yoloCells + op.cellBase + static_cast<size_t>(a) * hw + p) * per + m];
+    return out;
+}
+
+void NetBuilder::runLayersEager()
+{
+    Plan &plan = *_net->plan;
+    if (plan.yoloCandCnt.ptr()) MSNH_DEV(msnh_hip_fill_zero(plan.yoloCandCnt.ptr(), plan.yoloCandCnt.bytes(), _stream));
+    _layerOutputs.assign(_net->layers.size(), std::vector<float>());
+    msnh_event_t e0 = nullptr, e1 = nullptr;
+    MSNH_DEV(msnh_hip_event_create(&e0));
+    MSNH_DEV(msnh_hip_event_create(&e1));
+    for (size_t i = 0; i < _net->layers.size(); ++i)
+    {
+        BaseLayer *l = _net->layers[i];
+        MSNH_DEV(msnh_hip_event_record(e0, _stream));
+        l->forwardGPU(*_netState);
+        MSNH_DEV(msnh_hip_event_record(e1, _stream));
+        MSNH_DEV(msnh_hip_event_sync(e1));
+        float ms = 0.f;
+        MSNH_DEV(msnh_hip_event_elapsed_ms(e0, e1, &ms));
+        l->setForwardTime(ms);
+        if (!_saveLayerOutput) continue;
+        if (l->type() == LayerType::YOLO)
+        {
+            const YoloLayer *yl = static_cast<const YoloLayer *>(l);
+            _layerOutputs[i] = yoloLayerDump(plan, yl, plan.ops[yl->decodeOp], _net->batch, _stream);
+        }
+        else if (l->type() != LayerType::YOLO_OUT)
+        {
+            plan.exportTensor(plan.layerOut[i], _layerOutputs[i], _stream);
+        }
+        if (_writeDumpFiles)
+        {
+            std::ofstream f(std::to_string(i) + "gpu.txt");
+            for (float v : _layerOutputs[i]) f << v << "\n";
+        }
+    }
+    msnh_hip_event_destroy(e0);
+    msnh_hip_event_destroy(e1);
+}
+
+void NetBuilder::enqueueForward(const float *deviceInput)
+{
+    if (!_planReady) MSNH_THROW("weights are not loaded");
+    Plan &plan = *_net->plan;
+    if (deviceInput != nullptr && deviceInput != _inputDev.as<float>())
+        MSNH_DEV(msnh_hip_memcpy_d2d(_inputDev.ptr(), deviceInput, sizeof(float) * static_cast<size_t>(_net->inputNum), _stream));
+    if (_graph == nullptr)
+    {
+        // Record the whole forward once; later calls replay it with a single launch.
+        MSNH_DEV(msnh_hip_graph_begin(_stream));
+        try
+        {
+            if (plan.yoloCandCnt.ptr()) MSNH_DEV(msnh_hip_fill_zero(plan.yoloCandCnt.ptr(), plan.yoloCandCnt.bytes(), _stream));
+            plan.runAll(_stream);
+            if (plan.yoloCells > 0 && _net->layers.back()->type() == LayerType::YOLO_OUT)
+            {
+                const int per = 5 + plan.yoloClasses;
+                MSNH_DEV(msnh_hip_yolo_gather(_net->batch, plan.yoloClasses, plan.yoloDecoded.as<float>(), static_cast<long long>(plan.yoloCells) * per,
+                                              plan.yoloCandIdx.as<int>(), plan.yoloCells, plan.yoloCandCnt.as<int>(), plan.yoloRows.as<float>(), _stream));
+            }
+        }
+        catch (...)
+        {
+            msnh_graph_t junk = nullptr;
+            msnh_hip_graph_end(_stream, &junk);
+            if (junk) msnh_hip_graph_destroy(junk);
+            throw;
+        }
+        MSNH_DEV(msnh_hip_graph_end(_stream, &_graph));
+    }
+    MSNH_DEV(msnh_hip_graph_launch(_graph, _stream));
+}
+
+void NetBuilder::sync() { MSNH_DEV(msnh_hip_stream_sync(_stream)); }
+
+std::vector<float> NetBuilder::fetchClassify()
+{
+    Plan &plan = *_net->plan;
+    std::vector<float> out;
+    plan.exportTensor(plan.layerOut.back(), out, _stream);
+    return out;
+}
+
+std::vector<std::vector<YoloBox>> NetBuilder::fetchYolo()
+{
+    BaseLayer *last = _net->layers.back();
+    if (last->type() != LayerType::YOLO_OUT) MSNH_THROW("not a yolo net");
+    // the captured graph already compacted the candidates; only the host half of YoloOut remains.  Calling the
+    // layer's forwardGPU repeats the (idempotent) gather and then does the copy-back, sort and NMS.
+    last->forwardGPU(*_netState);
+    return static_cast<YoloOutLayer *>(last)->finalOut;
+}
+
+std::vector<float> NetBuilder::runClassifyGPU(std::vector<float> img)
+{
+    checkInput(img.size());
+    auto st = TimeUtil::startRecord();
+    uploadInput(img);
+    std::vector<float> out;
+    if (_saveLayerOutput)
+    {
+        runLayersEager();
+        _net->plan->exportTensor(_net->plan->layerOut.back(), out, _stream);
+    }
+    else
+    {
+        enqueueForward(nullptr);
+        out = fetchClassify();
+    }
+    _gpuInferenceTime = TimeUtil::getElapsedTime(st);
+    return out;
+}
+
+std::vector<std::vector<YoloBox>> NetBuilder::runYoloGPU(std::vector<float> img)
+{
+    checkInput(img.size());
+    if (_net->layers.back()->type() != LayerType::YOLO_OUT) MSNH_THROW("not a yolo net");
+    auto st = TimeUtil::startRecord();
+    uploadInput(img);
+    std::vector<std::vector<YoloBox>> out;
+    if (_saveLayerOutput)
+    {
+        runLayersEager();
+        out = static_cast<YoloOutLayer *>(_net->layers.back())->finalOut;
+    }
+    else
+    {
+        enqueueForward(nullptr);
+        out = fetchYolo();
+    }
+    _gpuInferenceTime = TimeUtil::getElapsedTime(st);
+    return out;
+}
+
+// ---- getters ---------------------------------------------------------------------------------------------------------
+Point2I NetBuilder::getInputSize()
+{
+    if (_parser->params.empty()) MSNH_THROW("net param is empty");
+    if (_parser->params[0]->type != LayerType::CONFIG) MSNH_THROW("net param error");
+    NetConfigParams *cfg = static_cast<NetConfigParams *>(_parser->params[0]);
+    return Point2I(cfg->width, cfg->height);
+}
+
+int NetBuilder::getInputChannel()
+{
+    if (_parser->params.empty()) MSNH_THROW("net param is empty");
+    return static_cast<NetConfigParams *>(_parser->params[0])->channels;
+}
+
+int NetBuilder::getBatch() const { return _net->batch; }
+
+float NetBuilder::getInferenceTime()
+{
+    float t = 0.f;
+    for (BaseLayer *l : _net->layers) t += l->getForwardTime();
+    return t;
+}
+
+static std::string index3(size_t i)
+{
+    return i < 10 ? "00" + std::to_string(i) : (i < 100 ? "0" + std::to_string(i) : std::to_string(i));
+}
+
+std::string NetBuilder::getLayerDetail()
+{
+    std::string d;
+    for (size_t i = 0; i < _net->layers.size(); ++i)
+    {
+        d += "────────────────────────────────  " + index3(i) + " ─────────────────────────────────\n";
+        d += _net->layers[i]->getLayerDetail() + "weights : " + std::to_string(_net->layers[i]->getNumWeights()) + "\n\n";
+    }
+    return d;
+}
+
+std::string NetBuilder::getTimeDetail()
+{
+    const float total = getInferenceTime();
+    std::string d = "LAYER            INDEX       TIME         LAYER_t/TOTAL_t\r\n=========================================================\n";
+    for (size_t i = 0; i < _net->layers.size(); ++i)
+    {
+        const float t = _net->layers[i]->getForwardTime();
+        d += _net->layers[i]->getLayerName() + " : " + index3(i) + "     " + std::to_string(t).substr(0, 6) + " ms         " +
+             std::to_string(static_cast<int>(t / total * 1000) / 10.f).substr(0, 4) + "%\n";
+    }
+    d += "=========================================================\nMsnhnet inference time : " + std::to_string(total) + " ms";
+    return d;
+}
+
+float NetBuilder::getGpuInferenceTime() const { return _gpuInferenceTime; }
+Network *NetBuilder::getNet() const { return _net; }
+int NetBuilder::getLastLayerOutWidth() const { return _lastLayerOutWidth; }
+int NetBuilder::getLastLayerOutHeight() const { return _lastLayerOutHeight; }
+int NetBuilder::getLastLayerOutChannel() const { return _lastLayerOutChannel; }
+size_t NetBuilder::getLastLayerOutNum() const { return _lastLayerOutNum; }
+bool NetBuilder::getSaveLayerWeights() const { return _saveLayerWeights; }
+void NetBuilder::setSaveLayerWeights(bool v) { _saveLayerWeights = v; }
+
+void NetBuilder::setSaveLayerOutput(bool v)
+{
+    if (v == _saveLayerOutput) return;
+    _saveLayerOutput = v;
+    // dumps need every layer output as a real tensor: re-plan if a plan already exists
+    if (_planReady) finalizePlan();
+}
+
+std::string NetBuilder::getPlanDetail() const { return _net->plan ? _net->plan->describe() : std::string(); }
+double NetBuilder::getConvFlops() const { return _net->plan ? _net->plan->totalConvFlops() : 0.0; }
+}

@@ -1,0 +1,540 @@
+// Device plan: fusion, concat aliasing, float16 scale calibration, arena placement, weight preparation and
+// the launch of every op through the kernel library's C ABI.
+#include "Msnhnet/core/MsnhPlan.h"
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <functional>
+#include <limits>
+#include <mutex>
+#include <numeric>
+#include <sstream>
+#include "Msnhnet/layers/MsnhBaseLayer.h"
+
+namespace Msnhnet
+{
+// ---- Device ---------------------------------------------------------------------------------------------
+static bool g_deviceReady = false;
+static std::mutex g_deviceMutex;
+
+void Device::ensureInit()
+{
+    std::lock_guard<std::mutex> lock(g_deviceMutex);
+    if (g_deviceReady) return;
+    int count = 0;
+    msnh_hip_device_count(&count);
+    if (count <= 0) MSNH_THROW("no MI355X/HIP device is visible: this build has no CPU path");
+    MSNH_DEV(msnh_hip_init(0));
+    g_deviceReady = true;
+}
+
+bool Device::initialised() { return g_deviceReady; }
+
+// ---- construction -------------------------------------------------------------------------------------------
+int Plan::addTensor(int n, int h, int w, int c, int dtype, const std::string &name, PlanTensor::Layout layout)
+{
+    PlanTensor t;
+    t.n = n; t.h = h; t.w = w; t.c = c; t.dtype = dtype; t.name = name; t.layout = layout;
+    tensors.push_back(t);
+    return static_cast<int>(tensors.size()) - 1;
+}
+
+PlanOp &Plan::addOp(PlanOp::Kind kind, int in0, int in1, int out, int layerIndex, const std::string &name)
+{
+    ops.emplace_back();
+    PlanOp &op = ops.back();
+    op.kind = kind; op.in0 = in0; op.in1 = in1; op.out = out; op.layerIndex = layerIndex; op.name = name;
+    return op;
+}
+
+int Plan::producerOf(int tensor) const
+{
+    for (int i = static_cast<int>(ops.size()) - 1; i >= 0; --i)
+        if (!ops[static_cast<size_t>(i)].dead && ops[static_cast<size_t>(i)].out == tensor) return i;
+    return -1;
+}
+
+int Plan::consumerCount(int tensor) const
+{
+    int n = 0;
+    for (const PlanOp &op : ops)
+        if (!op.dead) n += (op.in0 == tensor) + (op.in1 == tensor);
+    return n;
+}
+
+size_t Plan::liveOps() const
+{
+    size_t n = 0;
+    for (const PlanOp &op : ops) n += op.dead ? 0 : 1;
+    return n;
+}
+
+double Plan::totalConvFlops() const
+{
+    double f = 0;
+    for (const PlanOp &op : ops)
+        if (!op.dead) f += op.flops;
+    return f;
+}
+
+int Plan::root(int t) const
+{
+    while (tensors[static_cast<size_t>(t)].parent >= 0) t = tensors[static_cast<size_t>(t)].parent;
+    return t;
+}
+
+int Plan::chanOffsetInRoot(int t) const
+{
+    int off = 0;
+    while (tensors[static_cast<size_t>(t)].parent >= 0)
+    {
+        off += tensors[static_cast<size_t>(t)].chanOffset;
+        t = tensors[static_cast<size_t>(t)].parent;
+    }
+    return off;
+}
+
+void *Plan::ptr(int t) const
+{
+    const PlanTensor &r = tensors[static_cast<size_t>(root(t))];
+    unsigned char *base = r.external ? static_cast<unsigned char *>(r.extPtr) : _arena.as<unsigned char>() + r.offset;
+    if (base == nullptr) MSNH_THROW("plan tensor '" + tensors[static_cast<size_t>(t)].name + "' has no storage");
+    const size_t el = r.dtype == MSNH_F16 ? 2 : 4;
+    return base + static_cast<size_t>(chanOffsetInRoot(t)) * el;
+}
+
+float Plan::mulOf(int t) const { return std::ldexp(1.f, tensors[static_cast<size_t>(t)].scaleExp); }
+
+// ---- pass 1: fusion ---------------------------------------------------------------------------------------------
+void Plan::fuse()
+{
+    // (a) CONV (no activation) -> AFFINE on the conv's only consumer : fold the affine into the conv epilogue.
+    for (size_t i = 0; i < ops.size(); ++i)
+    {
+        PlanOp &aff = ops[i];
+        if (aff.dead || aff.kind != PlanOp::AFFINE) continue;
+        const int p = producerOf(aff.in0);
+        if (p < 0) continue;
+        PlanOp &conv = ops[static_cast<size_t>(p)];
+        if (conv.kind != PlanOp::CONV || conv.act != NONE || conv.src2 != nullptr || conv.in1 >= 0) continue;
+        if (tensors[static_cast<size_t>(aff.in0)].pinned || consumerCount(aff.in0) != 1) continue;
+        conv.src2 = aff.src;
+        conv.act = aff.act;
+        conv.actParam = aff.actParam;
+        conv.out = aff.out;
+        aff.dead = true;
+    }
+    // (b) CONV -> ADD(conv output, other) : the add and the block activation move into the conv epilogue.
+    for (size_t i = 0; i < ops.size(); ++i)
+    {
+        PlanOp &add = ops[i];
+        if (add.dead || add.kind != PlanOp::ADD) continue;
+        for (int side = 0; side < 2; ++side)
+        {
+            const int mine = side == 0 ? add.in0 : add.in1;
+            const int other = side == 0 ? add.in1 : add.in0;
+            const int p = producerOf(mine);
+            if (p < 0 || mine == other) continue;
+            PlanOp &conv = ops[static_cast<size_t>(p)];
+            if (conv.kind != PlanOp::CONV || conv.in1 >= 0) continue;
+            if (tensors[static_cast<size_t>(mine)].pinned || consumerCount(mine) != 1) continue;
+            // the other operand must already exist when the conv runs
+            const int po = producerOf(other);
+            if (po >= p) continue;
+            conv.in1 = other;
+            conv.act2 = add.act;
+            conv.act2Param = add.actParam;
+            conv.out = add.out;
+            add.dead = true;
+            break;
+        }
+    }
+}
+
+// ---- pass 2: concat aliasing ---------------------------------------------------------------------------------------
+void Plan::aliasConcats()
+{
+    for (size_t i = 0; i < ops.size(); ++i)
+    {
+        PlanOp &cp = ops[i];
+        if (cp.dead || cp.kind != PlanOp::COPY) continue;
+        PlanTensor &src = tensors[static_cast<size_t>(cp.in0)];
+        const PlanTensor &dst = tensors[static_cast<size_t>(cp.out)];
+        if (src.parent >= 0 || src.external || src.layout != PlanTensor::NHWC || dst.layout != PlanTensor::NHWC) continue;
+        if (src.dtype != dst.dtype) continue;
+        if (cp.dstChanOffset % 8 != 0 || dst.c % 8 != 0 || src.c % 8 != 0) continue;     // keep 16-byte alignment for vector kernels
+        if (root(cp.out) == cp.in0) continue;
+        bool ok = true;
+        for (const PlanOp &op : ops)
+        {
+            if (op.dead) continue;
+            const bool reads = op.in0 == cp.in0 || op.in1 == cp.in0;
+            if (reads && op.kind == PlanOp::CONNECTED) ok = false;          // needs densely packed rows
+        }
+        const int p = producerOf(cp.in0);
+        if (p < 0 || static_cast<size_t>(p) > i) ok = false;
+        if (!ok) continue;
+        src.parent = cp.out;
+        src.chanOffset = cp.dstChanOffset;
+        cp.dead = true;
+    }
+}
+
+// ---- pass 3: calibration -------------------------------------------------------------------------------------------
+void Plan::measureAmax(msnh_stream_t s)
+{
+    DeviceBuffer res(sizeof(float) * tensors.size());
+    MSNH_DEV(msnh_hip_fill_zero(res.ptr(), sizeof(float) * tensors.size(), s));
+    std::vector<char> live(tensors.size(), 0);
+    for (const PlanOp &op : ops)
+        if (!op.dead && op.out >= 0) live[static_cast<size_t>(op.out)] = 1;
+    for (size_t t = 0; t < tensors.size(); ++t)
+    {
+        const PlanTensor &pt = tensors[t];
+        if (!live[t] || pt.layout != PlanTensor::NHWC) continue;
+        MSNH_DEV(msnh_hip_absmax(pt.dtype, pt.pixels(), pt.c, ptr(static_cast<int>(t)), ld(static_cast<int>(t)), res.as<float>() + t, s));
+    }
+    std::vector<float> host(tensors.size(), 0.f);
+    MSNH_DEV(msnh_hip_memcpy_d2h(host.data(), res.ptr(), sizeof(float) * tensors.size(), s));
+    MSNH_DEV(msnh_hip_stream_sync(s));
+    for (size_t t = 0; t < tensors.size(); ++t) tensors[t].amax = host[t];
+}
+
+void Plan::applyCalibration(const Plan &cal)
+{
+    if (cal.tensors.size() != tensors.size()) MSNH_THROW("calibration plan does not match");
+    // tensors that must share one scale: views with their parent, pooling / upsample inputs with outputs
+    std::vector<int> group(tensors.size());
+    std::iota(group.begin(), group.end(), 0);
+    std::function<int(int)> find = [&](int x) { return group[static_cast<size_t>(x)] == x ? x : group[static_cast<size_t>(x)] = find(group[static_cast<size_t>(x)]); };
+    auto unite = [&](int a, int b) { group[static_cast<size_t>(find(a))] = find(b); };
+    for (size_t t = 0; t < tensors.size(); ++t)
+        if (tensors[t].parent >= 0) unite(static_cast<int>(t), tensors[t].parent);
+    for (const PlanOp &op : ops)
+        if (!op.dead && (op.kind == PlanOp::MAXPOOL || op.kind == PlanOp::UPSAMPLE)) unite(op.in0, op.out);
+    std::vector<float> gmax(tensors.size(), 0.f);
+    for (size_t t = 0; t < tensors.size(); ++t)
+    {
+        const int g = find(static_cast<int>(t));
+        gmax[static_cast<size_t>(g)] = std::max(gmax[static_cast<size_t>(g)], cal.tensors[t].amax);
+    }
+    // Keep the calibrated maximum at or below 2^11: a 32x margin to the half maximum for inputs that run
+    // hotter than the calibration image, while staying far above the subnormal range.
+    const float target = 2048.f;
+    for (size_t t = 0; t < tensors.size(); ++t)
+    {
+        PlanTensor &pt = tensors[t];
+        pt.amax = cal.tensors[t].amax;
+        const float m = gmax[static_cast<size_t>(find(static_cast<int>(t)))];
+        pt.scaleExp = 0;
+        if (pt.dtype == MSNH_F16 && pt.layout == PlanTensor::NHWC && m > target)
+            pt.scaleExp = static_cast<int>(std::ceil(std::log2(m / target)));
+    }
+    // a float16 tensor sharing a group with a float32 one (possible for maxpool/upsample pairs) keeps exponent 0 on
+    // the float32 side only if the whole group is 0; otherwise force the group to 0 is unnecessary because such
+    // pairs always share the dtype in the plans this library builds.
+}
+
+// ---- pass 4: placement ---------------------------------------------------------------------------------------------
+void Plan::place()
+{
+    const int nT = static_cast<int>(tensors.size());
+    const int nOps = static_cast<int>(ops.size());
+    std::vector<int> first(static_cast<size_t>(nT), std::numeric_limits<int>::max()), last(static_cast<size_t>(nT), -1);
+    auto touch = [&](int t, int i) {
+        if (t < 0) return;
+        const int r = root(t);
+        first[static_cast<size_t>(r)] = std::min(first[static_cast<size_t>(r)], i);
+        last[static_cast<size_t>(r)] = std::max(last[static_cast<size_t>(r)], i);
+    };
+    for (int i = 0; i < nOps; ++i)
+    {
+        const PlanOp &op = ops[static_cast<size_t>(i)];
+        if (op.dead) continue;
+        touch(op.in0, i); touch(op.in1, i); touch(op.out, i);
+    }
+    for (int t = 0; t < nT; ++t)
+    {
+        if (!tensors[static_cast<size_t>(t)].persistent && !tensors[static_cast<size_t>(t)].pinned) continue;
+        const int r = root(t);
+        if (last[static_cast<size_t>(r)] >= 0 && tensors[static_cast<size_t>(t)].persistent) last[static_cast<size_t>(r)] = nOps;
+    }
+    struct Item { int t; size_t bytes; int first, last; size_t offset; };
+    std::vector<Item> items;
+    for (int t = 0; t < nT; ++t)
+    {
+        PlanTensor &pt = tensors[static_cast<size_t>(t)];
+        if (pt.parent >= 0) continue;
+        if (pt.layout == PlanTensor::NHWC) pt.ld = (pt.c + 7) / 8 * 8;
+        else pt.ld = pt.c;
+        if (pt.external || last[static_cast<size_t>(t)] < 0) continue;
+        const size_t el = pt.dtype == MSNH_F16 ? 2 : 4;
+        size_t bytes = static_cast<size_t>(pt.n) * pt.h * pt.w * pt.ld * el;
+        bytes = (bytes + 255) / 256 * 256;
+        pt.bytes = bytes;
+        items.push_back({t, bytes, first[static_cast<size_t>(t)], last[static_cast<size_t>(t)], 0});
+    }
+    std::sort(items.begin(), items.end(), [](const Item &a, const Item &b) { return a.first != b.first ? a.first < b.first : a.bytes > b.bytes; });
+    std::vector<Item> placed;
+    size_t total = 0;
+    for (Item &it : items)
+    {
+        // gaps between the tensors alive at the same time, lowest offset first
+        std::vector<std::pair<size_t, size_t>> busy;
+        for (const Item &p : placed)
+            if (!(p.last < it.first || p.first > it.last)) busy.emplace_back(p.offset, p.offset + p.bytes);
+        std::sort(busy.begin(), busy.end());
+        size_t at = 0;
+        for (const auto &b : busy)
+        {
+            if (at + it.bytes <= b.first) break;
+            at = std::max(at, b.second);
+        }
+        it.offset = at;
+        tensors[static_cast<size_t>(it.t)].offset = at;
+        total = std::max(total, at + it.bytes);
+        placed.push_back(it);
+    }
+    _arena.alloc(std::max<size_t>(total, 256));
+}
+
+// ---- weights -------------------------------------------------------------------------------------------------------
+static msnh_conv_desc convDesc(const Plan &plan, const PlanOp &op)
+{
+    const PlanTensor &in = plan.tensors[static_cast<size_t>(op.in0)];
+    const PlanTensor &out = plan.tensors[static_cast<size_t>(op.out)];
+    msnh_conv_desc d;
+    std::memset(&d, 0, sizeof(d));
+    const bool fromInput = in.layout == PlanTensor::NCHW_INPUT;
+    d.dtype = fromInput ? out.dtype : in.dtype;
+    d.out_dtype = out.dtype;
+    d.batch = in.n; d.in_h = in.h; d.in_w = in.w; d.in_c = in.c;
+    d.in_ld = fromInput ? in.c : plan.ld(op.in0);
+    d.out_c = out.c; d.out_h = out.h; d.out_w = out.w; d.out_ld = plan.ld(op.out);
+    d.ksize = op.ksize; d.stride = op.stride; d.pad = op.pad; d.dilation = op.dilation; d.groups = op.groups;
+    d.act = static_cast<int>(op.act); d.act_param = op.actParam;
+    d.has_residual = op.in1 >= 0 ? 1 : 0;
+    d.res_ld = op.in1 >= 0 ? plan.ld(op.in1) : out.c;
+    d.act2 = static_cast<int>(op.act2); d.act2_param = op.act2Param;
+    d.res_mul = op.in1 >= 0 ? plan.mulOf(op.in1) : 1.f;
+    d.out_mul = 1.f / plan.mulOf(op.out);
+    d.algo = op.algo;
+    return d;
+}
+
+static std::vector<uint16_t> toHalf(const std::vector<float> &v);
+
+void Plan::prepareWeights()
+{
+    for (PlanOp &op : ops)
+    {
+        if (op.dead) continue;
+        if (op.kind == PlanOp::CONV)
+        {
+            const PlanTensor &in = tensors[static_cast<size_t>(op.in0)];
+            msnh_conv_desc d = convDesc(*this, op);
+            if (in.layout == PlanTensor::NCHW_INPUT) d.algo = MSNH_CONV_STEM;
+            op.algo = msnh_hip_conv2d_select_algo(&d);
+            d.algo = op.algo;
+            const std::vector<float> &w = op.src->kernelWeights();
+            const size_t expect = static_cast<size_t>(d.out_c) * (d.in_c / d.groups) * d.ksize * d.ksize;
+            if (w.size() != expect) MSNH_THROW("conv weights are not loaded (" + op.name + ")");
+            const size_t elems = msnh_hip_conv2d_packed_weight_elems(&d, op.algo);
+            const size_t el = d.dtype == MSNH_F16 ? 2 : 4;
+            std::vector<unsigned char> packed(elems * el);
+            MSNH_DEV(msnh_hip_conv2d_pack_weights(&d, op.algo, w.data(), packed.data()));
+            op.wDev.upload(packed.data(), packed.size());
+
+            std::vector<float> scale, shift;
+            op.src->foldedAffine(scale, shift);
+            if (op.src2)
+            {
+                std::vector<float> s2, h2;
+                op.src2->foldedAffine(s2, h2);
+                if (scale.empty()) scale.assign(static_cast<size_t>(d.out_c), 1.f);
+                if (shift.empty()) shift.assign(static_cast<size_t>(d.out_c), 0.f);
+                for (int c = 0; c < d.out_c; ++c)
+                {
+                    const size_t i = static_cast<size_t>(c);
+                    scale[i] = s2[i] * scale[i];
+                    shift[i] = s2[i] * shift[i] + h2[i];
+                }
+            }
+            const float inMul = in.layout == PlanTensor::NCHW_INPUT ? 1.f : mulOf(op.in0);
+            if (inMul != 1.f)
+            {
+                if (scale.empty()) scale.assign(static_cast<size_t>(d.out_c), 1.f);
+                for (float &v : scale) v *= inMul;
+            }
+            if (!scale.empty()) op.scaleDev.upload(scale.data(), scale.size() * sizeof(float));
+            if (!shift.empty()) op.shiftDev.upload(shift.data(), shift.size() * sizeof(float));
+            op.flops = 2.0 * d.batch * d.out_c * d.out_h * d.out_w * (d.in_c / d.groups) * d.ksize * d.ksize;
+        }
+        else if (op.kind == PlanOp::AFFINE)
+        {
+            std::vector<float> scale, shift;
+            op.src->foldedAffine(scale, shift);
+            const float inMul = mulOf(op.in0);
+            for (float &v : scale) v *= inMul;
+            op.scaleDev.upload(scale.data(), scale.size() * sizeof(float));
+            op.shiftDev.upload(shift.data(), shift.size() * sizeof(float));
+        }
+        else if (op.kind == PlanOp::CONNECTED)
+        {
+            const PlanTensor &in = tensors[static_cast<size_t>(op.in0)];
+            const std::vector<float> &w = op.src->kernelWeights();
+            if (w.empty()) MSNH_THROW("connected weights are not loaded (" + op.name + ")");
+            if (in.dtype == MSNH_F16)
+            {
+                const std::vector<uint16_t> h = toHalf(w);
+                op.wDev.upload(h.data(), h.size() * 2);
+            }
+            else op.wDev.upload(w.data(), w.size() * sizeof(float));
+            std::vector<float> scale, shift;
+            op.src->foldedAffine(scale, shift);
+            if (!shift.empty()) op.shiftDev.upload(shift.data(), shift.size() * sizeof(float));
+            op.flops = 2.0 * static_cast<double>(w.size()) * in.n;
+        }
+    }
+}
+
+// round-to-nearest-even float -> IEEE half, host side
+static uint16_t halfBits(float f)
+{
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    x &= 0x7fffffffu;
+    if (x >= 0x7f800000u) return static_cast<uint16_t>(sign | 0x7c00u | ((x & 0x7fffffu) ? 0x200u : 0));
+    if (x >= 0x477ff000u) return static_cast<uint16_t>(sign | 0x7c00u);                 // rounds to >= 65520 -> inf
+    if (x < 0x33000001u) return static_cast<uint16_t>(sign);                            // < 2^-25 -> 0
+    int exp = static_cast<int>(x >> 23) - 127;
+    uint32_t man = (x & 0x7fffffu) | 0x800000u;
+    int shift;
+    uint32_t base;
+    if (exp < -14) { shift = 13 + (-14 - exp); base = 0; }
+    else { shift = 13; base = static_cast<uint32_t>(exp + 15) << 10; man &= 0x7fffffu; }
+    uint32_t h = man >> shift;
+    const uint32_t rem = man & ((1u << shift) - 1u);
+    const uint32_t halfway = 1u << (shift - 1);
+    if (rem > halfway || (rem == halfway && (h & 1u))) ++h;
+    return static_cast<uint16_t>(sign | (base + h));
+}
+
+static std::vector<uint16_t> toHalf(const std::vector<float> &v)
+{
+    std::vector<uint16_t> h(v.size());
+    for (size_t i = 0; i < v.size(); ++i) h[i] = halfBits(v[i]);
+    return h;
+}
+
+// ---- execution ---------------------------------------------------------------------------------------------------------
+void Plan::launch(PlanOp &op, msnh_stream_t s)
+{
+    const PlanTensor &in = tensors[static_cast<size_t>(op.in0)];
+    const PlanTensor &out = tensors[static_cast<size_t>(op.out)];
+    switch (op.kind)
+    {
+    case PlanOp::CONV:
+    {
+        const msnh_conv_desc d = convDesc(*this, op);
+        MSNH_DEV(msnh_hip_conv2d(&d, ptr(op.in0), op.wDev.ptr(), op.scaleDev.as<float>(), op.shiftDev.as<float>(),
+                                 op.in1 >= 0 ? ptr(op.in1) : nullptr, ptr(op.out), nullptr, 0, s));
+        break;
+    }
+    case PlanOp::AFFINE:
+        MSNH_DEV(msnh_hip_affine_act(in.dtype, out.dtype, in.pixels(), in.c, ptr(op.in0), ld(op.in0), op.scaleDev.as<float>(),
+                                     op.shiftDev.as<float>(), static_cast<int>(op.act), op.actParam, 1.f / mulOf(op.out), ptr(op.out), ld(op.out), s));
+        break;
+    case PlanOp::ADD:
+        MSNH_DEV(msnh_hip_add_act(in.dtype, in.pixels(), in.c, ptr(op.in0), ld(op.in0), mulOf(op.in0), ptr(op.in1), ld(op.in1), mulOf(op.in1),
+                                  static_cast<int>(op.act), op.actParam, 1.f / mulOf(op.out), ptr(op.out), ld(op.out), s));
+        break;
+    case PlanOp::COPY:
+    {
+        const size_t el = out.dtype == MSNH_F16 ? 2 : 4;
+        void *dst = static_cast<unsigned char *>(ptr(op.out)) + static_cast<size_t>(op.dstChanOffset) * el;
+        MSNH_DEV(msnh_hip_copy_channels(in.dtype, in.pixels(), in.c, ptr(op.in0), ld(op.in0), mulOf(op.in0) / mulOf(op.out), dst, ld(op.out), s));
+        break;
+    }
+    case PlanOp::MAXPOOL:
+        MSNH_DEV(msnh_hip_maxpool(in.dtype, in.n, in.h, in.w, in.c, ptr(op.in0), ld(op.in0), op.ksize, op.stride, op.pad, out.h, out.w,
+                                  ptr(op.out), ld(op.out), s));
+        break;
+    case PlanOp::AVGPOOL:
+        MSNH_DEV(msnh_hip_avgpool(in.dtype, out.dtype, in.n, in.h, in.w, in.c, ptr(op.in0), ld(op.in0), op.ksize, op.stride, op.pad, out.h,
+                                  out.w, mulOf(op.in0) / mulOf(op.out), ptr(op.out), ld(op.out), s));
+        break;
+    case PlanOp::UPSAMPLE:
+        MSNH_DEV(msnh_hip_upsample_nearest(in.dtype, in.n, in.h, in.w, in.c, ptr(op.in0), ld(op.in0), op.stride, op.upScale, ptr(op.out),
+                                           ld(op.out), s));
+        break;
+    case PlanOp::CONNECTED:
+        if (ld(op.in0) != in.c && in.n > 1 && in.h * in.w == 1) MSNH_THROW("connected input must be densely packed");
+        MSNH_DEV(msnh_hip_connected(in.dtype, in.n, in.h * in.w * in.c, out.c, ptr(op.in0), mulOf(op.in0), op.wDev.ptr(), op.shiftDev.as<float>(),
+                                    static_cast<int>(op.act), op.actParam, static_cast<float *>(ptr(op.out)), s));
+        break;
+    case PlanOp::INPUT_CAST:
+        MSNH_DEV(msnh_hip_nchw_to_nhwc(out.dtype, in.n, in.c, in.h, in.w, static_cast<const float *>(ptr(op.in0)), 1.f / mulOf(op.out),
+                                       ptr(op.out), ld(op.out), s));
+        break;
+    case PlanOp::YOLO_DECODE:
+    {
+        const int per = 5 + op.classes;
+        float *decoded = yoloDecoded.as<float>() + static_cast<size_t>(op.cellBase) * per;
+        const bool cand = op.confThresh < 1.5f;
+        MSNH_DEV(msnh_hip_yolo_decode(in.dtype, in.n, in.h, in.w, op.classes, ptr(op.in0), ld(op.in0), mulOf(op.in0), op.anchors.data(), op.ratio,
+                                      decoded, static_cast<long long>(yoloCells) * per, op.confThresh, cand ? yoloCandIdx.as<int>() : nullptr,
+                                      yoloCells, op.cellBase, cand ? yoloCandCnt.as<int>() : nullptr, s));
+        break;
+    }
+    }
+}
+
+void Plan::run(size_t opBegin, size_t opEnd, msnh_stream_t s)
+{
+    for (size_t i = opBegin; i < opEnd && i < ops.size(); ++i)
+        if (!ops[i].dead) launch(ops[i], s);
+}
+
+void Plan::exportTensor(int t, std::vector<float> &dst, msnh_stream_t s)
+{
+    const PlanTensor &pt = tensors[static_cast<size_t>(t)];
+    dst.resize(pt.elems());
+    if (dst.empty()) return;
+    if (pt.layout == PlanTensor::FLAT || pt.layout == PlanTensor::NCHW_INPUT)
+    {
+        MSNH_DEV(msnh_hip_memcpy_d2h(dst.data(), ptr(t), dst.size() * sizeof(float), s));
+        MSNH_DEV(msnh_hip_stream_sync(s));
+        return;
+    }
+    if (_exportScratch.bytes() < dst.size() * sizeof(float)) _exportScratch.alloc(dst.size() * sizeof(float));
+    MSNH_DEV(msnh_hip_nhwc_to_nchw(pt.dtype, pt.n, pt.c, pt.h, pt.w, ptr(t), ld(t), mulOf(t), _exportScratch.as<float>(), s));
+    MSNH_DEV(msnh_hip_memcpy_d2h(dst.data(), _exportScratch.ptr(), dst.size() * sizeof(float), s));
+    MSNH_DEV(msnh_hip_stream_sync(s));
+}
+
+std::string Plan::describe() const
+{
+    static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode"};
+    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem"};
+    std::ostringstream os;
+    os << "plan: " << liveOps() << " launches, " << tensors.size() << " tensors, arena " << _arena.bytes() / (1024.0 * 1024.0) << " MiB, dtype "
+       << (computeDtype == MSNH_F16 ? "f16" : "f32") << "\n";
+    for (size_t i = 0; i < ops.size(); ++i)
+    {
+        const PlanOp &op = ops[i];
+        if (op.dead) continue;
+        const PlanTensor &in = tensors[static_cast<size_t>(op.in0)];
+        const PlanTensor &out = tensors[static_cast<size_t>(op.out)];
+        os << "  L" << op.layerIndex << " " << kinds[op.kind];
+        if (op.kind == PlanOp::CONV)
+            os << "[" << algos[op.algo] << " k" << op.ksize << " s" << op.stride << " g" << op.groups << (op.in1 >= 0 ? " +res" : "") << (op.src2 ? " +bn" : "") << "]";
+        os << " " << in.n << "x" << in.h << "x" << in.w << "x" << in.c << " -> " << out.h << "x" << out.w << "x" << out.c
+           << (out.dtype == MSNH_F16 ? " f16" : " f32") << " e" << out.scaleExp;
+        if (out.parent >= 0) os << " (slice@" << chanOffsetInRoot(op.out) << " of " << tensors[static_cast<size_t>(root(op.out))].c << ")";
+        os << "\n";
+    }
+    return os.str();
+}
+}

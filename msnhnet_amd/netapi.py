@@ -1,0 +1,255 @@
+"""ctypes binding of the host library's C ABI (include/msnhnet_c.h): NetBuilder build / load / run.
+
+There is no CPU fallback: loading fails loudly if the libraries are not built, and every run entry point needs
+a GPU (the CPU entry points of the reference API exist and raise "Gpu mode , can not run with cpu").
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libMsnhnet.so")
+
+SYMBOLS = [
+    "initMsnhnet", "buildMsnhnet", "runClassifyNoPred", "runYoloNoPred", "dispose", "withGPU", "withCUDNN", "getCpuForwardTime",
+    "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16",
+    "msnhnet_set_keep_class_scores", "msnhnet_set_save_layer_output", "msnhnet_build", "msnhnet_load", "msnhnet_load_from_memory",
+    "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops",
+    "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
+    "msnhnet_enqueue", "msnhnet_sync", "msnhnet_fetch_classify", "msnhnet_fetch_yolo", "msnhnet_gpu_inference_time", "msnhnet_time_detail",
+]
+
+LAYER_TYPE = {0: "conv", 2: "connect", 3: "maxpool", 4: "localavgpool", 8: "route", 13: "batchnorm", 15: "yolo", 16: "yoloout",
+              18: "upsample", 20: "empty", 27: "resblock", 28: "res2block", 29: "concatblock", 30: "addblock"}
+
+
+class MsnhnetError(RuntimeError):
+    pass
+
+
+class BBox(ctypes.Structure):
+    _fields_ = [("x", ctypes.c_float), ("y", ctypes.c_float), ("w", ctypes.c_float), ("h", ctypes.c_float), ("conf", ctypes.c_float),
+                ("bestClsConf", ctypes.c_float), ("bestClsIdx", ctypes.c_uint32), ("angle", ctypes.c_float)]
+
+
+class BBoxContainer(ctypes.Structure):
+    _fields_ = [("boxes", BBox * 1024)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise MsnhnetError(f"{LIB_PATH} is missing: build it first (python -m msnhnet_amd.build)")
+    L = ctypes.CDLL(LIB_PATH)
+    vp, ci, ll, cp = ctypes.c_void_p, ctypes.c_int, ctypes.c_longlong, ctypes.c_char_p
+    fp = ctypes.POINTER(ctypes.c_float)
+    ip = ctypes.POINTER(ci)
+    llp = ctypes.POINTER(ll)
+    cpp = ctypes.POINTER(cp)
+    L.buildMsnhnet.argtypes = [cpp, cp, cp, ci, ci]
+    L.runClassifyNoPred.argtypes = [cpp, fp, ci, ip, ci]
+    L.runYoloNoPred.argtypes = [cpp, fp, ci, ctypes.POINTER(BBoxContainer), ip, ci]
+    L.withGPU.argtypes = [ip]
+    L.withCUDNN.argtypes = [ip]
+    L.getCpuForwardTime.argtypes = [fp]
+    L.getGpuForwardTime.argtypes = [fp]
+    L.getInputDim.argtypes = [ip, ip, ip]
+    L.msnhnet_last_error.restype = cp
+    L.msnhnet_create.argtypes = [ctypes.POINTER(vp)]
+    L.msnhnet_destroy.argtypes = [vp]
+    L.msnhnet_set_use_fp16.argtypes = [ci]
+    L.msnhnet_set_keep_class_scores.argtypes = [ci]
+    L.msnhnet_set_save_layer_output.argtypes = [vp, ci]
+    L.msnhnet_build.argtypes = [vp, cp]
+    L.msnhnet_load.argtypes = [vp, cp]
+    L.msnhnet_load_from_memory.argtypes = [vp, fp, ctypes.c_size_t]
+    L.msnhnet_input_dims.argtypes = [vp, ip, ip, ip, ip]
+    L.msnhnet_num_layers.argtypes = [vp]
+    L.msnhnet_layer_info.argtypes = [vp, ci, llp, cp, ci]
+    for n in ("msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_time_detail"):
+        getattr(L, n).argtypes = [vp, cp, ll]
+        getattr(L, n).restype = ll
+    L.msnhnet_conv_flops.argtypes = [vp]
+    L.msnhnet_conv_flops.restype = ctypes.c_double
+    L.msnhnet_run_classify.argtypes = [vp, fp, ll, fp, ll, llp]
+    L.msnhnet_run_classify_gpu.argtypes = [vp, fp, ll, fp, ll, llp]
+    L.msnhnet_run_yolo_gpu.argtypes = [vp, fp, ll, ip, fp, ll, llp]
+    L.msnhnet_layer_output.argtypes = [vp, ci, fp, ll]
+    L.msnhnet_layer_output.restype = ll
+    L.msnhnet_device_input.argtypes = [vp, ctypes.POINTER(fp)]
+    L.msnhnet_enqueue.argtypes = [vp, vp]
+    L.msnhnet_sync.argtypes = [vp]
+    L.msnhnet_fetch_classify.argtypes = [vp, fp, ll, llp]
+    L.msnhnet_fetch_yolo.argtypes = [vp, ip, fp, ll, llp]
+    L.msnhnet_gpu_inference_time.argtypes = [vp]
+    L.msnhnet_gpu_inference_time.restype = ctypes.c_float
+    _lib = L
+    return L
+
+
+def _check(rc):
+    if rc != 0:
+        raise MsnhnetError(lib().msnhnet_last_error().decode(errors="replace"))
+
+
+def _fp(a):
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+
+
+def set_use_fp16(on):
+    _check(lib().msnhnet_set_use_fp16(1 if on else 0))
+
+
+class Net:
+    """One NetBuilder.  `fp16` is the process-wide NetBuilder::setUseFp16 switch, applied before the build."""
+
+    def __init__(self, msnhnet_path=None, msnhbin_path=None, fp16=False, dump_layers=False):
+        self.L = lib()
+        self.h = ctypes.c_void_p()
+        _check(self.L.msnhnet_create(ctypes.byref(self.h)))
+        set_use_fp16(fp16)
+        if dump_layers:
+            _check(self.L.msnhnet_set_save_layer_output(self.h, 1))
+        if msnhnet_path:
+            self.build(msnhnet_path)
+        if msnhbin_path:
+            self.load(msnhbin_path)
+
+    def close(self):
+        if self.h:
+            self.L.msnhnet_destroy(self.h)
+            self.h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def build(self, path):
+        _check(self.L.msnhnet_build(self.h, path.encode()))
+
+    def load(self, path):
+        _check(self.L.msnhnet_load(self.h, path.encode()))
+
+    def load_array(self, w):
+        w = np.ascontiguousarray(w, np.float32)
+        _check(self.L.msnhnet_load_from_memory(self.h, _fp(w), w.size))
+
+    def dims(self):
+        v = [ctypes.c_int() for _ in range(4)]
+        _check(self.L.msnhnet_input_dims(self.h, *[ctypes.byref(x) for x in v]))
+        return tuple(x.value for x in v)          # batch, channels, height, width
+
+    def num_layers(self):
+        return self.L.msnhnet_num_layers(self.h)
+
+    def layer_info(self, i):
+        info = (ctypes.c_longlong * 10)()
+        name = ctypes.create_string_buffer(64)
+        _check(self.L.msnhnet_layer_info(self.h, i, info, name, 64))
+        keys = ["type", "outH", "outW", "outC", "outputNum", "inputNum", "numWeights", "memReUse", "batch", "act"]
+        d = dict(zip(keys, [int(v) for v in info]))
+        d["type"] = LAYER_TYPE.get(d["type"], str(d["type"]))
+        d["name"] = name.value.decode()
+        return d
+
+    def layer_infos(self):
+        return [self.layer_info(i) for i in range(self.num_layers())]
+
+    def _text(self, fn):
+        n = fn(self.h, None, 0)
+        if n < 0:
+            _check(1)
+        buf = ctypes.create_string_buffer(n + 1)
+        fn(self.h, buf, n + 1)
+        return buf.value.decode(errors="replace")
+
+    def layer_detail(self):
+        return self._text(self.L.msnhnet_layer_detail)
+
+    def plan_detail(self):
+        return self._text(self.L.msnhnet_plan_detail)
+
+    def time_detail(self):
+        return self._text(self.L.msnhnet_time_detail)
+
+    def conv_flops(self):
+        return float(self.L.msnhnet_conv_flops(self.h))
+
+    def run_classify_cpu(self, img):
+        x = np.ascontiguousarray(img, np.float32).ravel()
+        n = ctypes.c_longlong()
+        _check(self.L.msnhnet_run_classify(self.h, _fp(x), x.size, None, 0, ctypes.byref(n)))
+
+    def run_classify(self, img):
+        x = np.ascontiguousarray(img, np.float32).ravel()
+        b = self.dims()[0]
+        last = self.layer_info(self.num_layers() - 1)
+        out = np.empty(b * last["outputNum"], np.float32)
+        n = ctypes.c_longlong()
+        _check(self.L.msnhnet_run_classify_gpu(self.h, _fp(x), x.size, _fp(out), out.size, ctypes.byref(n)))
+        return out[:n.value].reshape(b, -1)
+
+    def _boxes(self, fn, *head):
+        b = self.dims()[0]
+        counts = (ctypes.c_int * b)()
+        total = ctypes.c_longlong()
+        cap = 4096
+        while True:
+            boxes = np.zeros((cap, 7), np.float32)
+            _check(fn(self.h, *head, counts, _fp(boxes), cap, ctypes.byref(total)))
+            if total.value <= cap:
+                break
+            cap = int(total.value)
+            if head:            # a run call: everything was computed, only the copy was truncated -> fetch again
+                fn, head = self.L.msnhnet_fetch_yolo, ()
+        out, at = [], 0
+        for i in range(b):
+            out.append(boxes[at:at + counts[i]].copy())
+            at += counts[i]
+        return out
+
+    def run_yolo(self, img):
+        x = np.ascontiguousarray(img, np.float32).ravel()
+        return self._boxes(self.L.msnhnet_run_yolo_gpu, _fp(x), x.size)
+
+    def layer_output(self, i):
+        n = self.L.msnhnet_layer_output(self.h, i, None, 0)
+        if n < 0:
+            _check(1)
+        a = np.empty(n, np.float32)
+        if n:
+            self.L.msnhnet_layer_output(self.h, i, _fp(a), n)
+        return a
+
+    def device_input_ptr(self):
+        p = ctypes.POINTER(ctypes.c_float)()
+        _check(self.L.msnhnet_device_input(self.h, ctypes.byref(p)))
+        return ctypes.cast(p, ctypes.c_void_p).value
+
+    def enqueue(self, device_ptr=None):
+        _check(self.L.msnhnet_enqueue(self.h, ctypes.c_void_p(device_ptr) if device_ptr else None))
+
+    def sync(self):
+        _check(self.L.msnhnet_sync(self.h))
+
+    def fetch_classify(self):
+        b = self.dims()[0]
+        last = self.layer_info(self.num_layers() - 1)
+        out = np.empty(b * last["outputNum"], np.float32)
+        n = ctypes.c_longlong()
+        _check(self.L.msnhnet_fetch_classify(self.h, _fp(out), out.size, ctypes.byref(n)))
+        return out[:n.value].reshape(b, -1)
+
+    def fetch_yolo(self):
+        return self._boxes(self.L.msnhnet_fetch_yolo)
+
+    def gpu_inference_time_ms(self):
+        return float(self.L.msnhnet_gpu_inference_time(self.h))

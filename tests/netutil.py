@@ -1,0 +1,75 @@
+"""Shared helpers of the network-level tests: model files in a temp dir, reference / oracle runs, comparisons."""
+import os
+import tempfile
+
+import numpy as np
+
+from msnhnet_amd import zoo
+
+_dir = None
+
+
+def workdir():
+    global _dir
+    if _dir is None:
+        _dir = tempfile.mkdtemp(prefix="msnh_models_")
+    return _dir
+
+
+def model(arch, batch, size, seed=1, **kw):
+    """Writes graph + seeded weights once per (arch,batch,size,seed); returns (msnhnet, msnhbin, GraphWriter)."""
+    net, binp, g = zoo.write_model(arch, workdir(), batch, size, seed=seed, **kw)
+    return net, binp, g
+
+
+def batch1_graph(arch, size, **kw):
+    g = zoo.ARCHS[arch](batch=1, size=size, **kw)
+    path = os.path.join(workdir(), f"{arch}_b1_{size}_oracle.msnhnet")
+    with open(path, "w") as f:
+        f.write(g.text())
+    return path
+
+
+def rel_err(a, b):
+    """max|a-b|/max|b| over entries finite in the reference; non-finite entries must agree in class and sign."""
+    a = np.asarray(a, np.float64).ravel()
+    b = np.asarray(b, np.float64).ravel()
+    assert a.shape == b.shape, (a.shape, b.shape)
+    fb = np.isfinite(b)
+    bad = ~fb
+    if bad.any():
+        assert (np.isnan(a[bad]) == np.isnan(b[bad])).all(), "NaN pattern differs"
+        inf = bad & ~np.isnan(b)
+        assert (a[inf] == b[inf]).all(), "inf pattern differs"
+    if not fb.any():
+        return 0.0
+    assert np.isfinite(a[fb]).all(), "non-finite value where the reference is finite"
+    return float(np.abs(a[fb] - b[fb]).max() / max(np.abs(b[fb]).max(), 1e-30))
+
+
+def sort_boxes(b):
+    b = np.asarray(b, np.float32).reshape(-1, 7)
+    if len(b) == 0:
+        return b
+    key = np.nan_to_num(b, nan=1e30, posinf=2e30, neginf=-2e30)
+    return b[np.lexsort(key.T[::-1])]
+
+
+def yolo_layer_err(got, ref, logits, channels_per_anchor, ratio):
+    """Error of a decoded yolo layer [3*per, H*W] in units of the logit error that explains it.
+
+    Every decoded value is a function of one logit t: (sigmoid(t)+cell)*ratio, anchor*exp(t) or sigmoid(t).  A logit
+    error d (itself bounded relative to max|t|) shows up as at most d/4 in a sigmoid plane and as a factor e^d in a
+    w,h plane, however small d/|t| is.  So: sigmoid planes -> absolute error (x,y divided by ratio), w,h planes ->
+    |log got - log ref|, all divided by max(1, max|t|)."""
+    per = channels_per_anchor
+    got = np.asarray(got, np.float64).reshape(3, per, -1)
+    ref = np.asarray(ref, np.float64).reshape(3, per, -1)
+    scale = max(np.abs(np.asarray(logits, np.float64)).max(), 1.0)
+    e_xy = np.abs(got[:, 0:2] - ref[:, 0:2]).max() / ratio
+    e_sig = np.abs(got[:, 4:] - ref[:, 4:]).max()
+    g, r = got[:, 2:4].ravel(), ref[:, 2:4].ravel()
+    fin = np.isfinite(r) & (r != 0)
+    assert (np.isfinite(g) == np.isfinite(r)).all() and ((g == 0) == (r == 0)).all(), "inf / underflow pattern differs"
+    e_wh = float(np.abs(np.log(np.abs(g[fin])) - np.log(np.abs(r[fin]))).max()) if fin.any() else 0.0
+    return float(max(e_xy, e_sig, e_wh) / scale)

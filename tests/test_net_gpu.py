@@ -1,0 +1,139 @@
+"""End-to-end GPU parity through the host library's C ABI (NetBuilder build / load / runClassifyGPU / runYoloGPU)
+against the reference's own CPU forward (oracle/_ref, scalar mode) when it is present, else the plain-C oracle.
+
+Tolerances (max|a-b| / max|ref| per layer output):
+  float32: 1e-4 on every top-level layer output (the reference's own FMA-contracted build and its plain-C
+           restatement already differ by up to 1.7e-4 on the deepest MobileNetV2 layers, so those use 5e-4;
+           decoded yolo layers are compared in units of the logit error that explains them, see netutil.yolo_layer_err);
+  float16: 2e-2 on the final logits / boxes; class indices and box counts are compared exactly where the margin
+           of the reference result is larger than the float16 error.
+"""
+import numpy as np
+import pytest
+
+import msnh_oracle_net as on
+import netutil as nu
+import refshim
+from msnhnet_amd import netapi, zoo
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle_layers(arch, size, binp, imgs, **kw):
+    """Per-image per-layer outputs from the reference (scalar mode) or, without it, the plain-C oracle."""
+    path = nu.batch1_graph(arch, size, **kw)
+    outs, boxes = [], []
+    if refshim.available():
+        r = refshim.RefNet(path, binp, scalar=True)
+        for x in imgs:
+            outs.append(r.run(x))
+            boxes.append(r.boxes())
+    else:
+        o = on.OracleNet(path, binp)
+        for x in imgs:
+            outs.append([v.ravel() for v in o.run(x)])
+            boxes.append(o.boxes if o.boxes is not None else np.zeros((0, 7), np.float32))
+    return outs, boxes
+
+
+SMALL = [("resnet18", 64, 2), ("resnet50", 64, 2), ("mobilenetv2", 64, 3), ("yolov3", 64, 2), ("yolov4", 64, 2)]
+
+
+@pytest.mark.parametrize("arch,size,batch", SMALL)
+def test_fp32_every_layer(arch, size, batch):
+    if arch in ("resnet18", "resnet50", "mobilenetv2"):
+        size = 224            # the 7x7 average pool needs the full-size feature map
+    net, binp, g = nu.model(arch, batch, size, seed=3)
+    x = zoo.seeded_input(batch, 3, size, size, seed=4)
+    ref, ref_boxes = _oracle_layers(arch, size, binp, x)
+    print("running", arch, size, batch, flush=True)
+    m = netapi.Net(net, binp, fp16=False, dump_layers=True)
+    if arch.startswith("yolo"):
+        boxes = m.run_yolo(x)
+    else:
+        logits = m.run_classify(x)
+    n_layers = m.num_layers()
+    assert n_layers == len(ref[0])
+    tol = 5e-4 if arch == "mobilenetv2" else 1e-4
+    worst = 0.0
+    for i in range(n_layers):
+        if m.layer_info(i)["type"] == "yoloout":
+            continue
+        got = m.layer_output(i).reshape(batch, -1)
+        is_yolo = m.layer_info(i)["type"] == "yolo"
+        lt = tol
+        for b in range(batch):
+            e = nu.yolo_layer_err(got[b], ref[b][i], ref[b][i - 1], 85, size / m.layer_info(i)['outH']) if is_yolo else nu.rel_err(got[b], ref[b][i])
+            worst = max(worst, e)
+            assert e <= lt, f"{arch} layer {i} ({m.layer_info(i)['type']}) image {b}: {e}"
+    print(arch, "worst layer error", worst)
+    if arch.startswith("yolo"):
+        for b in range(batch):
+            rb, gb = nu.sort_boxes(ref_boxes[b]), nu.sort_boxes(boxes[b])
+            assert len(rb) == len(gb), f"box count {len(gb)} vs {len(rb)}"
+            assert np.array_equal(rb[:, 6], gb[:, 6])
+            assert nu.rel_err(gb[:, :6], rb[:, :6]) <= 1e-4
+    else:
+        for b in range(batch):
+            assert int(np.argmax(logits[b])) == int(np.argmax(ref[b][-1]))
+
+
+@pytest.mark.parametrize("arch,size,batch", SMALL)
+def test_fused_graph_equals_layer_by_layer(arch, size, batch):
+    """The production path (fused launches, aliased concats, captured graph) must give what the dump path gives."""
+    if arch in ("resnet18", "resnet50", "mobilenetv2"):
+        size = 224
+    net, binp, g = nu.model(arch, batch, size, seed=3)
+    x = zoo.seeded_input(batch, 3, size, size, seed=4)
+    slow = netapi.Net(net, binp, fp16=False, dump_layers=True)
+    fast = netapi.Net(net, binp, fp16=False, dump_layers=False)
+    if arch.startswith("yolo"):
+        a, b1, b2 = slow.run_yolo(x), fast.run_yolo(x), fast.run_yolo(x)      # second call replays the graph
+        for i in range(batch):
+            for got in (b1[i], b2[i]):
+                assert len(got) == len(a[i])
+                assert nu.rel_err(nu.sort_boxes(got)[:, :6], nu.sort_boxes(a[i])[:, :6]) <= 1e-5
+    else:
+        a, b1, b2 = slow.run_classify(x), fast.run_classify(x), fast.run_classify(x)
+        assert nu.rel_err(b1, a) <= 1e-5 and np.array_equal(b1, b2)
+
+
+@pytest.mark.parametrize("arch,size,batch", SMALL)
+def test_fp16_final_outputs(arch, size, batch):
+    if arch in ("resnet18", "resnet50", "mobilenetv2"):
+        size = 224
+    net, binp, g = nu.model(arch, batch, size, seed=3)
+    x = zoo.seeded_input(batch, 3, size, size, seed=4)
+    ref, ref_boxes = _oracle_layers(arch, size, binp, x)
+    print("running fp16", arch, size, batch, flush=True)
+    m = netapi.Net(net, binp, fp16=True, dump_layers=True)
+    if arch.startswith("yolo"):
+        boxes = m.run_yolo(x)
+        # final logits = inputs of the yolo layers
+        for i in range(m.num_layers()):
+            if m.layer_info(i)["type"] != "yolo":
+                continue
+            got = m.layer_output(i - 1).reshape(batch, -1)
+            for b in range(batch):
+                e = nu.rel_err(got[b], ref[b][i - 1])
+                assert e <= 2e-2, f"{arch} head logits before layer {i}, image {b}: {e}"
+        for b in range(batch):
+            # objectness logits closer to the threshold than the float16 error may legitimately flip
+            assert abs(len(boxes[b]) - len(ref_boxes[b])) <= max(2, 0.02 * len(ref_boxes[b]))
+    else:
+        logits = m.run_classify(x)
+        for b in range(batch):
+            r = ref[b][-1]
+            assert nu.rel_err(logits[b], r) <= 2e-2
+            top2 = np.sort(r)[-2:]
+            if top2[1] - top2[0] > 4e-2 * np.abs(r).max():
+                assert int(np.argmax(logits[b])) == int(np.argmax(r))
+
+
+def test_cpu_entry_points_refuse():
+    net, binp, g = nu.model("resnet18", 1, 224, seed=3)
+    m = netapi.Net(net, binp)
+    with pytest.raises(netapi.MsnhnetError, match="Gpu mode , can not run with cpu"):
+        m.run_classify_cpu(np.zeros(3 * 224 * 224, np.float32))
+    with pytest.raises(netapi.MsnhnetError, match="input image size err. Needed :150528 given :10"):
+        m.run_classify(np.zeros(10, np.float32))

@@ -1,0 +1,216 @@
+"""GPU parity of the bandwidth-bound entry points of the C ABI against the plain-C oracle."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import msnh_oracle_net as on
+from msnhnet_amd import hipabi as abi
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [abi.F32, abi.F16]
+TOL = {abi.F32: 1e-6, abi.F16: 1.5e-3}
+
+
+def _x(rng, shape, dtype):
+    import gpuutil as gu
+    x = rng.standard_normal(shape, dtype=np.float32) * 3
+    return gu.round_f16(x) if dtype == abi.F16 else x
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("c,ld", [(16, 16), (24, 40), (13, 13), (255, 256)])
+@pytest.mark.parametrize("act", ["relu", "leaky", "mish", "none"])
+def test_affine_act(c, ld, act, dtype):
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(c)
+    x = _x(rng, (2, c, 7, 5), dtype)
+    bn4 = np.concatenate([rng.uniform(.5, 1.5, c), rng.standard_normal(c) * .1, rng.standard_normal(c) * .1, rng.uniform(.5, 1.5, c)]).astype(np.float32)
+    ref = on.batchnorm(x, bn4, 1e-5, act)
+    sq = np.sqrt(bn4[3 * c:] + np.float32(1e-5)).astype(np.float32)
+    scale = (bn4[:c] / sq).astype(np.float32)
+    shift = (-bn4[:c] * bn4[2 * c:3 * c] / sq + bn4[c:2 * c]).astype(np.float32)
+    xd = gu.nhwc_dev(x, dtype, ld)
+    yd = torch.full((2, 7, 5, ld), 3.0, dtype=gu.TORCH_DT[dtype]).cuda()
+    sd, hd = gu.dev(scale), gu.dev(shift)
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_affine_act(dtype, dtype, 2 * 7 * 5, c, gu.ptr(xd), ld, gu.ptr(sd), gu.ptr(hd), abi.ACT[act], 0.1, 1.0, gu.ptr(yd), ld, None))
+    gu.sync()
+    assert gu.rel_err(gu.nchw_host(yd, c), ref) <= max(TOL[dtype], 2e-6)
+    assert (yd[..., c:].float().cpu().numpy() == 3.0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("c", [32, 20])
+def test_add_act_and_copy(c, dtype):
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(c)
+    a, b = _x(rng, (2, c, 6, 6), dtype), _x(rng, (2, c, 6, 6), dtype)
+    ad, bd = gu.nhwc_dev(a, dtype, c + 8), gu.nhwc_dev(b, dtype, c)
+    yd = torch.full((2, 6, 6, c + 16), 3.0, dtype=gu.TORCH_DT[dtype]).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_add_act(dtype, 72, c, gu.ptr(ad), c + 8, 2.0, gu.ptr(bd), c, 0.5, abi.ACT["relu"], 0.1, 0.25, gu.ptr(yd), c + 16, None))
+    gu.sync()
+    ref = 0.25 * on.activate((2.0 * a + 0.5 * b).astype(np.float32), "relu")
+    assert gu.rel_err(gu.nchw_host(yd, c), ref) <= TOL[dtype]
+    # channel-slice copy into the middle of a wider tensor
+    zd = torch.full((2, 6, 6, 2 * c + 8), 3.0, dtype=gu.TORCH_DT[dtype]).cuda()
+    gu.sync()
+    off = 8
+    abi.check(abi.lib().msnh_hip_copy_channels(dtype, 72, c, gu.ptr(ad), c + 8, 1.0, ctypes.c_void_p(zd.data_ptr() + off * zd.element_size()), 2 * c + 8, None))
+    gu.sync()
+    z = zd.float().cpu().numpy()
+    assert np.array_equal(z[..., off:off + c].transpose(0, 3, 1, 2), a)
+    assert (z[..., :off] == 3.0).all() and (z[..., off + c:] == 3.0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("c,h,w,k,s,p", [(64, 28, 28, 3, 2, 1), (32, 19, 19, 5, 1, 2), (32, 19, 19, 9, 1, 4), (16, 19, 19, 13, 1, 6), (12, 10, 9, 2, 2, 0)])
+def test_maxpool(c, h, w, k, s, p, dtype):
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(k)
+    x = _x(rng, (2, c, h, w), dtype)
+    ref = on.maxpool(x, k, s, p)
+    oh, ow = ref.shape[2:]
+    xd = gu.nhwc_dev(x, dtype)
+    yd = torch.zeros((2, oh, ow, c), dtype=gu.TORCH_DT[dtype]).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_maxpool(dtype, 2, h, w, c, gu.ptr(xd), c, k, s, p, oh, ow, gu.ptr(yd), c, None))
+    gu.sync()
+    assert np.array_equal(gu.nchw_host(yd, c), ref)          # max is exact
+
+
+@pytest.mark.parametrize("dtype,out_dtype", [(abi.F32, abi.F32), (abi.F16, abi.F16), (abi.F16, abi.F32)])
+@pytest.mark.parametrize("c,h,w,k,s,p", [(512, 7, 7, 7, 1, 0), (24, 9, 9, 3, 2, 1)])
+def test_avgpool(c, h, w, k, s, p, dtype, out_dtype):
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(k)
+    x = _x(rng, (3, c, h, w), dtype)
+    ref = on.avgpool(x, k, s, p)
+    oh, ow = ref.shape[2:]
+    xd = gu.nhwc_dev(x, dtype)
+    yd = torch.zeros((3, oh, ow, c), dtype=gu.TORCH_DT[out_dtype]).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_avgpool(dtype, out_dtype, 3, h, w, c, gu.ptr(xd), c, k, s, p, oh, ow, 1.0, gu.ptr(yd), c, None))
+    gu.sync()
+    assert gu.rel_err(gu.nchw_host(yd, c), ref) <= (1e-6 if out_dtype == abi.F32 else 1e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_upsample(dtype):
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(1)
+    x = _x(rng, (2, 24, 5, 7), dtype)
+    ref = on.upsample(x, 2)
+    xd = gu.nhwc_dev(x, dtype)
+    yd = torch.full((2, 10, 14, 40), 3.0, dtype=gu.TORCH_DT[dtype]).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_upsample_nearest(dtype, 2, 5, 7, 24, gu.ptr(xd), 24, 2, 1.0, gu.ptr(yd), 40, None))
+    gu.sync()
+    assert np.array_equal(gu.nchw_host(yd, 24), ref)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_connected(dtype):
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(2)
+    x = _x(rng, (3, 512, 1, 1), dtype)
+    w = rng.uniform(-0.05, 0.05, (1000, 512)).astype(np.float32)
+    if dtype == abi.F16:
+        w = gu.round_f16(w)
+    bias = rng.uniform(-0.05, 0.05, 1000).astype(np.float32)
+    ref = on.connected(x, w, bias, 1000).reshape(3, 1000)
+    xd, wd, bd = gu.dev(x.reshape(3, 512), dtype), gu.dev(w, dtype), gu.dev(bias)
+    yd = torch.zeros((3, 1000), dtype=torch.float32).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_connected(dtype, 3, 512, 1000, gu.ptr(xd), 1.0, gu.ptr(wd), gu.ptr(bd), abi.ACT["none"], 0.1, gu.ptr(yd), None))
+    gu.sync()
+    assert gu.rel_err(yd.cpu().numpy(), ref) <= 2e-6
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_layout_roundtrip(dtype):
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(3)
+    x = _x(rng, (2, 37, 9, 11), dtype)
+    xd = gu.dev(x)
+    yd = torch.full((2, 9, 11, 40), 3.0, dtype=gu.TORCH_DT[dtype]).cuda()
+    zd = torch.zeros((2, 37, 9, 11), dtype=torch.float32).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_nchw_to_nhwc(dtype, 2, 37, 9, 11, gu.ptr(xd), 1.0, gu.ptr(yd), 40, None))
+    abi.check(abi.lib().msnh_hip_nhwc_to_nchw(dtype, 2, 37, 9, 11, gu.ptr(yd), 40, 1.0, gu.ptr(zd), None))
+    gu.sync()
+    assert np.array_equal(gu.nchw_host(yd, 37), x)
+    assert np.array_equal(zd.cpu().numpy(), x)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_yolo_decode(dtype):
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(4)
+    cls, h, w = 80, 7, 9
+    per = 5 + cls
+    x = (rng.standard_normal((2, 3 * per, h, w)) * 4).astype(np.float32)
+    x[0, 2, 0, 0] = 100.0          # exp overflow -> inf, as with the benchmark weights
+    x[1, 4, 3, 3] = -200.0
+    if dtype == abi.F16:
+        x = gu.round_f16(x)
+    anchors = np.array([10, 13, 16, 30, 33, 23], np.float32)
+    ratio = 32.0
+    ref = on.yolo_decode(x, cls, anchors, ratio)                       # [2][3*per][h][w]
+    ref_shuf = ref.reshape(2, 3, per, h * w).transpose(0, 1, 3, 2)    # [2][3][hw][per]
+    xd = gu.nhwc_dev(x, dtype, 256)
+    dd = torch.zeros((2, 3, h * w, per), dtype=torch.float32).cuda()
+    cap = 3 * h * w
+    ci = torch.full((2, cap), -1, dtype=torch.int32).cuda()
+    cc = torch.zeros(2, dtype=torch.int32).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_yolo_decode(dtype, 2, h, w, cls, gu.ptr(xd), 256, 1.0, anchors.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                                             ratio, gu.ptr(dd), 3 * h * w * per, 0.5, gu.ptr(ci), cap, 1000, gu.ptr(cc), None))
+    gu.sync()
+    out = dd.cpu().numpy()
+    assert gu.rel_err(out, ref_shuf) <= 2e-6
+    for b in range(2):
+        want = sorted(1000 + a * h * w + p for a in range(3) for p in range(h * w) if ref_shuf[b, a, p, 4] > 0.5)
+        n = int(cc[b])
+        assert sorted(ci[b, :n].cpu().numpy().tolist()) == want
+    # candidate compaction: box, objectness, first-maximum class
+    ci2 = (ci - 1000).clamp(min=0).contiguous()
+    rows = torch.zeros((2, cap, 8), dtype=torch.float32).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_yolo_gather(2, cls, gu.ptr(dd), 3 * h * w * per, gu.ptr(ci2), cap, gu.ptr(cc), gu.ptr(rows), None))
+    gu.sync()
+    rows = rows.cpu().numpy()
+    flat = ref_shuf.reshape(2, 3 * h * w, per)
+    for b in range(2):
+        for k in range(int(cc[b])):
+            cell = int(rows[b, k, 7])
+            r = flat[b, cell]
+            assert gu.rel_err(rows[b, k, :5], r[:5]) <= 2e-6
+            assert int(rows[b, k, 6]) == int(np.argmax(r[5:]))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_absmax(dtype):
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(5)
+    x = _x(rng, (2, 24, 9, 9), dtype)
+    x[1, 3, 2, 2] = np.inf if dtype == abi.F32 else 65504.0 * 4      # non-finite entries are ignored
+    xd = gu.nhwc_dev(x, dtype, 32, fill=1e4)                          # the padding channels must not be read
+    r = torch.zeros(1, dtype=torch.float32).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_absmax(dtype, 2 * 81, 24, gu.ptr(xd), 32, gu.ptr(r), None))
+    gu.sync()
+    xf = xd[..., :24].float().cpu().numpy()
+    assert float(r) == float(np.abs(xf[np.isfinite(xf)]).max())
