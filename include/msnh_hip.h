@@ -122,8 +122,13 @@ typedef struct msnh_conv_desc
     float res_mul;
     float out_mul;
     int   algo;         /* msnh_conv_algo */
+    int   tile;         /* IGEMM only: 0 = library default, 1..msnh_hip_conv2d_tile_count() = forced tile configuration */
 } msnh_conv_desc;
 
+/* Number of tile configurations of the IGEMM algorithm; any of them computes the same result, they differ in
+ * speed per shape.  The host library times them per layer at load (the reference asks cuDNN for the fastest
+ * algorithm the same way, src/layers/MsnhConvolutionalLayer.cpp:150-194). */
+int msnh_hip_conv2d_tile_count(void);
 /* Which algorithm MSNH_CONV_AUTO resolves to for this shape (never AUTO).  Pure host function. */
 int msnh_hip_conv2d_select_algo(const msnh_conv_desc *d);
 /* Number of elements (of d->dtype) of the packed weight buffer for `algo`.  Pure host function. */

@@ -85,6 +85,12 @@ int msnhnet_enqueue(msnhnet_t net, const float *device_input);
 int msnhnet_sync(msnhnet_t net);
 int msnhnet_fetch_classify(msnhnet_t net, float *out, long long cap, long long *n_out);
 int msnhnet_fetch_yolo(msnhnet_t net, int *counts, float *boxes, long long cap_boxes, long long *total);
+/* Device-event timing of `reps` eager passes over the plan's launches of one kind (0 conv, 1 affine, 2 add, 3 copy,
+ * 4 maxpool, 5 avgpool, 6 upsample, 7 connected, 8 input cast, 9 yolo decode, -1 all).  Outputs the total
+ * milliseconds, the number of launches timed and their algorithmic FLOPs (2*MACs; 0 for non-GEMM kinds). */
+int msnhnet_profile_ops(msnhnet_t net, int kind, int reps, float *ms_total, int *launches, double *flops);
+/* Per-launch timing table (text): every live launch of the plan timed on its own, `reps` repetitions each. */
+long long msnhnet_profile_each_op(msnhnet_t net, int reps, char *dst, long long cap);
 float msnhnet_gpu_inference_time(msnhnet_t net);          /* NetBuilder::getGpuInferenceTime, ms */
 long long msnhnet_time_detail(msnhnet_t net, char *dst, long long cap);       /* NetBuilder::getTimeDetail */
 

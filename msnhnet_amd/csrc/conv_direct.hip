@@ -11,6 +11,7 @@ namespace msnh {
 
 int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
               const void *residual, void *y, hipStream_t st);
+int igemmTileCount();
 int convWinograd(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
                  const void *residual, void *y, void *ws, size_t wsBytes, hipStream_t st);
 size_t winogradWorkspaceBytes(const msnh_conv_desc *d);
@@ -215,6 +216,8 @@ static bool winogradOk(const msnh_conv_desc *d)
 using namespace msnh;
 
 extern "C" {
+
+int msnh_hip_conv2d_tile_count(void) { return igemmTileCount(); }
 
 int msnh_hip_conv2d_select_algo(const msnh_conv_desc *d)
 {

@@ -1,0 +1,7 @@
+// Instantiations of the implicit-GEMM convolution kernel for f16 inputs and f16 outputs (one translation unit per
+// type pair so that they compile in parallel).
+#include "conv_igemm.hpp"
+
+namespace msnh {
+int igemmF16F16(IgemmArgs &a, int groups, int tile, hipStream_t st) { return igemmDispatch<f16, f16>(a, groups, tile, st); }
+}

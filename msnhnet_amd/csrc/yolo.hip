@@ -7,33 +7,48 @@ namespace msnh {
 
 struct Anchors { float v[6]; };
 
+// A workgroup decodes CHUNK consecutive values of one image.  Entries whose objectness passes the threshold are
+// first collected in LDS; one global atomic per workgroup then reserves their slots in the image's candidate list
+// (one atomic per candidate on a single counter would serialise half of all cells with the benchmark weights).
+constexpr int YOLO_CHUNK = 256 * 16;
+
 template <typename T>
 __global__ __launch_bounds__(256) void yoloDecodeKernel(const T *__restrict__ x, int xLd, float xMul, Anchors an, float ratio,
                                                         float *__restrict__ decoded, long long decStride, float confThresh, int *__restrict__ candIdx,
                                                         int candCap, int candBase, int *__restrict__ candCnt, int W, int HW, int per,
-                                                        long long total)
+                                                        int perImage)
 {
-    long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    const int m = static_cast<int>(idx % per);
-    long long t = idx / per;
-    const int p = static_cast<int>(t % HW);
-    t /= HW;
-    const int a = static_cast<int>(t % 3);
-    const int b = static_cast<int>(t / 3);
-    const float v = xMul * toF(x[(static_cast<size_t>(b) * HW + p) * xLd + a * per + m]);
-    float r;
-    if (m == 0)      r = (1.f / (1.f + expf(-v)) + static_cast<float>(p % W)) * ratio;
-    else if (m == 1) r = (1.f / (1.f + expf(-v)) + static_cast<float>(p / W)) * ratio;
-    else if (m == 2) r = an.v[2 * a] * expf(v);
-    else if (m == 3) r = an.v[2 * a + 1] * expf(v);
-    else             r = 1.f / (1.f + expf(-v));
-    decoded[static_cast<size_t>(b) * decStride + (static_cast<size_t>(a) * HW + p) * per + m] = r;
-    if (m == 4 && candIdx != nullptr && r > confThresh)
+    __shared__ int found[YOLO_CHUNK / 6 + 8];
+    __shared__ int nFound, base;
+    const int b = blockIdx.y;
+    if (threadIdx.x == 0) nFound = 0;
+    __syncthreads();
+    const int start = blockIdx.x * YOLO_CHUNK;
+#pragma unroll 4
+    for (int k = 0; k < YOLO_CHUNK / 256; ++k)
     {
-        const int pos = atomicAdd(candCnt + b, 1);
-        if (pos < candCap) candIdx[static_cast<size_t>(b) * candCap + pos] = candBase + a * HW + p;
+        const int idx = start + k * 256 + threadIdx.x;          // = (a*HW + p)*per + m inside the image
+        if (idx >= perImage) break;
+        const int m = idx % per;
+        const int cell = idx / per;
+        const int p = cell % HW;
+        const int a = cell / HW;
+        const float v = xMul * toF(x[(static_cast<size_t>(b) * HW + p) * xLd + a * per + m]);
+        float r;
+        if (m == 0)      r = (1.f / (1.f + expf(-v)) + static_cast<float>(p % W)) * ratio;
+        else if (m == 1) r = (1.f / (1.f + expf(-v)) + static_cast<float>(p / W)) * ratio;
+        else if (m == 2) r = an.v[2 * a] * expf(v);
+        else if (m == 3) r = an.v[2 * a + 1] * expf(v);
+        else             r = 1.f / (1.f + expf(-v));
+        decoded[static_cast<size_t>(b) * decStride + idx] = r;
+        if (m == 4 && candIdx != nullptr && r > confThresh) found[atomicAdd(&nFound, 1)] = candBase + cell;
     }
+    __syncthreads();
+    if (candIdx == nullptr || nFound == 0) return;
+    if (threadIdx.x == 0) base = atomicAdd(candCnt + b, nFound);
+    __syncthreads();
+    for (int i = threadIdx.x; i < nFound; i += 256)
+        if (base + i < candCap) candIdx[static_cast<size_t>(b) * candCap + base + i] = found[i];
 }
 
 __global__ __launch_bounds__(256) void yoloGatherKernel(const float *__restrict__ decoded, long long decStride, const int *__restrict__ candIdx,
@@ -97,15 +112,16 @@ extern "C" int msnh_hip_yolo_decode(int dtype, int batch, int h, int w, int clas
     MSNH_REQUIRE(cand_idx == nullptr || (cand_cnt != nullptr && cand_cap > 0), "yolo_decode: candidate list without counter");
     Anchors an;
     for (int i = 0; i < 6; ++i) an.v[i] = anchors6[i];
-    const long long total = static_cast<long long>(batch) * 3 * h * w * per;
-    dim3 grid(gridFor(total, 256));
+    MSNH_REQUIRE(per >= 6 && batch <= 65535, "yolo_decode: unsupported geometry");
+    const int perImage = 3 * h * w * per;
+    dim3 grid((perImage + YOLO_CHUNK - 1) / YOLO_CHUNK, batch);
     hipStream_t st = resolveStream(s);
     if (dtype == MSNH_F16)
         hipLaunchKernelGGL((yoloDecodeKernel<f16>), grid, dim3(256), 0, st, static_cast<const f16 *>(x), x_ld, x_mul, an, ratio, decoded,
-                           decoded_batch_stride, conf_thresh, cand_idx, cand_cap, cand_base, cand_cnt, w, h * w, per, total);
+                           decoded_batch_stride, conf_thresh, cand_idx, cand_cap, cand_base, cand_cnt, w, h * w, per, perImage);
     else
         hipLaunchKernelGGL((yoloDecodeKernel<float>), grid, dim3(256), 0, st, static_cast<const float *>(x), x_ld, x_mul, an, ratio,
-                           decoded, decoded_batch_stride, conf_thresh, cand_idx, cand_cap, cand_base, cand_cnt, w, h * w, per, total);
+                           decoded, decoded_batch_stride, conf_thresh, cand_idx, cand_cap, cand_base, cand_cnt, w, h * w, per, perImage);
     MSNH_LAUNCH_CHECK();
     return 0;
 }

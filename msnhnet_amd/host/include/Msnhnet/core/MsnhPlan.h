@@ -62,6 +62,7 @@ struct PlanOp
     float upScale = 1.f;
     int  dstChanOffset = 0;                 // COPY: channel offset inside `out`
     int  algo = MSNH_CONV_AUTO;             // CONV: resolved at weight preparation
+    int  tile = 0;                          // CONV/IGEMM: tile configuration chosen by Plan::tuneConvs (0 = library default)
     BaseLayer *src = nullptr;               // layer that owns the host weights of this op
     BaseLayer *src2 = nullptr;              // batch-norm layer folded into a CONV
 
@@ -103,6 +104,7 @@ public:
     void applyCalibration(const Plan &calibrated);   // pass 3: take amax from an executed float32 twin
     void place();                           // pass 4 + arena allocation
     void prepareWeights();                  // fold batch-norm, pick algorithms, pack and upload weights
+    void tuneConvs(msnh_stream_t s);        // time every IGEMM tile configuration per conv launch, keep the fastest
     void run(size_t opBegin, size_t opEnd, msnh_stream_t s);
     void runAll(msnh_stream_t s) { run(0, ops.size(), s); }
     void measureAmax(msnh_stream_t s);      // after an eager run: absmax of every live NHWC tensor

@@ -231,10 +231,18 @@ class MsnhNet_API YoloOutLayer : public BaseLayer
 public:
     YoloOutLayer(const int &batch, const int &orgWidth, const int &orgHeight, std::vector<int> &yoloIndexes, std::vector<YoloInfo> &yoloLayersInfo,
                  const float &confThresh, const float &nmsThresh, const int &useSotfNms, const YoloType &yoloType);
+    ~YoloOutLayer() override;
     int lower(Plan &plan, int in, int layerIndex) override;
     void forwardGPU(NetworkState &netState) override;      // device candidate compaction + host sort / NMS
+    // The three stages of forwardGPU, separately, so that a caller can overlap the host stage of one batch with
+    // the device work of the next (two copy-back slots):
+    void enqueueGather(msnh_stream_t s);                   // device: compact the candidate rows
+    void enqueueCopyBack(msnh_stream_t s, int slot);       // device -> pinned host, asynchronous
+    void finish(int slot);                                 // host: wait, sort, NMS -> finalOut
 
     static std::vector<YoloBox> nms(const std::vector<YoloBox> &bboxes, const float &nmsThresh, const bool &useSoftNms, const float &sigma = 0.3f);
+    // hard NMS with the same result as nms(), restructured for speed (see the definition)
+    static std::vector<YoloBox> nmsSorted(const std::vector<YoloBox> &bboxes, float nmsThresh);
     float getConfThresh() const { return _confThresh; }
     float getNmsThresh() const { return _nmsThresh; }
     int   getUseSoftNms() const { return _useSoftNms; }
@@ -255,6 +263,7 @@ private:
     std::vector<int> _yoloIndexes;
     std::vector<YoloInfo> _yoloLayersInfo;
     int _yoloAllInputNum = 0, _pixels = 0;
-    PinnedBuffer _hostCnt, _hostRows, _hostDecoded;
+    struct Slot { PinnedBuffer cnt, rows, decoded; msnh_event_t event = nullptr; bool pending = false; };
+    Slot _slots[2];
 };
 }

@@ -24,6 +24,9 @@ public:
     static void setUseFp16(const bool &useFp16);
     static void setForceUseCuda(const bool &onlyUseCuda);
     static void setKeepClassScores(const bool &keep);
+    // Per-layer search for the fastest convolution tile configuration at load time (default on).
+    static void setAutoTune(const bool &on);
+    static bool autoTune;
 
     void buildNetFromMsnhNet(const std::string &path);
     void loadWeightsFromMsnhBin(const std::string &path);
@@ -38,6 +41,8 @@ public:
 
     // Steady-state serving path: the input already lives on the device (NCHW float32, batch*C*H*W floats).
     // Enqueues one forward on the builder's stream; results are fetched with fetchClassify / fetchYolo.
+    // Detection networks may have two forwards in flight (enqueue, enqueue, fetch, enqueue, fetch, ...): the
+    // host-side sort / NMS of one batch then overlaps the device work of the next.
     void enqueueForward(const float *deviceInput);
     void sync();
     std::vector<float> fetchClassify();
@@ -67,6 +72,12 @@ public:
     void setWriteDumpFiles(bool on) { _writeDumpFiles = on; }
     std::string getPlanDetail() const;
     double getConvFlops() const;              // 2*MACs of all conv/connected launches of one forward (whole batch)
+    // Times `reps` eager passes over the live ops of one kind (PlanOp::Kind, or -1 for all) with device events on
+    // the builder's stream; returns the total milliseconds and the number of launches timed.  The ops run on
+    // whatever the buffers currently hold, so this is a timing tool, not a forward.
+    float profileOps(int kind, int reps, int *launches, double *flops);
+    // One line per live op: layer, kind, shapes, algorithm, microseconds per launch (mean of `reps`), TFLOP/s, GB/s.
+    std::string profileEachOp(int reps);
 
 private:
     void finalizePlan();
@@ -89,5 +100,6 @@ private:
     msnh_stream_t _stream = nullptr;
     msnh_graph_t  _graph = nullptr;
     const float  *_graphInput = nullptr;
+    int _nextSlot = 0, _inFlight = 0;          // copy-back slots of the detection post-processing
 };
 }

@@ -313,6 +313,26 @@ int msnhnet_fetch_yolo(msnhnet_t net, int *counts, float *boxes, long long cap_b
     return guarded([&] { packBoxes(nb(net).fetchYolo(), counts, boxes, cap_boxes, total); });
 }
 
+int msnhnet_profile_ops(msnhnet_t net, int kind, int reps, float *ms_total, int *launches, double *flops)
+{
+    return guarded([&] {
+        if (reps <= 0 || !ms_total) MSNH_THROW("bad argument");
+        *ms_total = nb(net).profileOps(kind, reps, launches, flops);
+    });
+}
+
+long long msnhnet_profile_each_op(msnhnet_t net, int reps, char *dst, long long cap)
+{
+    static thread_local std::string cache;
+    long long n = -1;
+    guarded([&] {
+        if (dst == nullptr || cache.empty()) cache = nb(net).profileEachOp(reps > 0 ? reps : 1);
+        n = copyText(cache, dst, cap);
+        if (dst != nullptr) cache.clear();
+    });
+    return n;
+}
+
 float msnhnet_gpu_inference_time(msnhnet_t net)
 {
     float t = -1.f;

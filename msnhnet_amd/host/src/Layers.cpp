@@ -898,37 +898,106 @@ std::vector<YoloBox> YoloOutLayer::nms(const std::vector<YoloBox> &bboxes, const
     return best;
 }
 
-void YoloOutLayer::forwardGPU(NetworkState &netState)
+// Same result as nms() for hard NMS, reorganised for speed: candidates of a class are visited in the order the
+// greedy loop would pick them (objectness descending, earlier position first on ties) and each is kept unless a
+// box kept before it overlaps it by more than the threshold -- that is exactly when the greedy loop would have
+// erased it.  The kept boxes are held as structure-of-arrays so the IoU test runs 8 wide.
+std::vector<YoloBox> YoloOutLayer::nmsSorted(const std::vector<YoloBox> &bboxes, float nmsThresh)
+{
+    const size_t n = bboxes.size();
+    std::vector<YoloBox> best;
+    if (n == 0) return best;
+    int maxCls = 0;
+    for (const YoloBox &b : bboxes) maxCls = std::max(maxCls, b.bestClsIdx);
+    std::vector<int> firstSeen;                                   // classes in first-appearance order
+    std::vector<int> slotOf(static_cast<size_t>(maxCls) + 1, -1);
+    std::vector<std::vector<int>> members;
+    for (size_t i = 0; i < n; ++i)
+    {
+        const int c = bboxes[i].bestClsIdx;
+        if (c < 0) MSNH_THROW("negative class index");
+        if (slotOf[static_cast<size_t>(c)] < 0)
+        {
+            slotOf[static_cast<size_t>(c)] = static_cast<int>(firstSeen.size());
+            firstSeen.push_back(c);
+            members.emplace_back();
+        }
+        members[static_cast<size_t>(slotOf[static_cast<size_t>(c)])].push_back(static_cast<int>(i));
+    }
+    best.reserve(n);
+    std::vector<float> kx1, ky1, kx2, ky2, karea;
+    for (std::vector<int> &m : members)
+    {
+        if (m.size() == 1) { best.push_back(bboxes[static_cast<size_t>(m[0])]); continue; }
+        std::stable_sort(m.begin(), m.end(), [&bboxes](int a, int b) { return bboxes[static_cast<size_t>(a)].conf > bboxes[static_cast<size_t>(b)].conf; });
+        kx1.clear(); ky1.clear(); kx2.clear(); ky2.clear(); karea.clear();
+        for (int j : m)
+        {
+            const Box::XYWHBox &q = bboxes[static_cast<size_t>(j)].xywhBox;
+            const float jx1 = q.x - q.w / 2.f, jx2 = q.x + q.w / 2.f, jy1 = q.y - q.h / 2.f, jy2 = q.y + q.h / 2.f;
+            const float jarea = (jx2 - jx1 + 1) * (jy2 - jy1 + 1);
+            const size_t nk = kx1.size();
+            int hit = 0;
+#pragma omp simd reduction(| : hit)
+            for (size_t k = 0; k < nk; ++k)
+            {
+                // Box::iou(candidate j, kept k) with std::min / std::max spelled out
+                const float ix2 = (kx2[k] < jx2) ? kx2[k] : jx2;
+                const float ix1 = (jx1 < kx1[k]) ? kx1[k] : jx1;
+                const float iy2 = (ky2[k] < jy2) ? ky2[k] : jy2;
+                const float iy1 = (jy1 < ky1[k]) ? ky1[k] : jy1;
+                const float iw = ix2 - ix1 + 1;
+                const float ih = iy2 - iy1 + 1;
+                const float inter = (iw < 0 ? 0 : iw) * (ih < 0 ? 0 : ih);
+                const float iou = 1.f * inter / (jarea + karea[k] - inter);
+                hit |= (iou > nmsThresh) ? 1 : 0;
+            }
+            if (hit) continue;
+            best.push_back(bboxes[static_cast<size_t>(j)]);
+            kx1.push_back(jx1); ky1.push_back(jy1); kx2.push_back(jx2); ky2.push_back(jy2); karea.push_back(jarea);
+        }
+    }
+    return best;
+}
+
+void YoloOutLayer::enqueueGather(msnh_stream_t s)
 {
     if (plan == nullptr) MSNH_THROW("YoloOut: layer is not part of a planned network");
     Plan &pl = *plan;
-    msnh_stream_t s = netState.stream;
-    const int cells = pl.yoloCells;
-    const int per = _channel;
-    MSNH_DEV(msnh_hip_yolo_gather(_batch, per - 5, pl.yoloDecoded.as<float>(), static_cast<long long>(cells) * per, pl.yoloCandIdx.as<int>(), cells,
-                                  pl.yoloCandCnt.as<int>(), pl.yoloRows.as<float>(), s));
-    _hostCnt.reserve(sizeof(int) * static_cast<size_t>(_batch));
-    MSNH_DEV(msnh_hip_memcpy_d2h(_hostCnt.ptr(), pl.yoloCandCnt.ptr(), sizeof(int) * static_cast<size_t>(_batch), s));
-    MSNH_DEV(msnh_hip_stream_sync(s));
-    const int *cnt = _hostCnt.as<int>();
-    _hostRows.reserve(sizeof(float) * 8 * static_cast<size_t>(cells) * static_cast<size_t>(_batch));
-    for (int b = 0; b < _batch; ++b)
-    {
-        const int n = std::min(cnt[b], cells);
-        if (n > 0)
-            MSNH_DEV(msnh_hip_memcpy_d2h(_hostRows.as<float>() + static_cast<size_t>(b) * cells * 8,
-                                         pl.yoloRows.as<float>() + static_cast<size_t>(b) * cells * 8, sizeof(float) * 8 * static_cast<size_t>(n), s));
-    }
-    const float *decodedHost = nullptr;
+    MSNH_DEV(msnh_hip_yolo_gather(_batch, _channel - 5, pl.yoloDecoded.as<float>(), static_cast<long long>(pl.yoloCells) * _channel,
+                                  pl.yoloCandIdx.as<int>(), pl.yoloCells, pl.yoloCandCnt.as<int>(), pl.yoloRows.as<float>(), s));
+}
+
+void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
+{
+    Plan &pl = *plan;
+    Slot &sl = _slots[slot & 1];
+    const size_t cells = static_cast<size_t>(pl.yoloCells);
+    sl.cnt.reserve(sizeof(int) * static_cast<size_t>(_batch));
+    sl.rows.reserve(sizeof(float) * 8 * cells * static_cast<size_t>(_batch));
+    if (sl.event == nullptr) MSNH_DEV(msnh_hip_event_create(&sl.event));
+    MSNH_DEV(msnh_hip_memcpy_d2h(sl.cnt.ptr(), pl.yoloCandCnt.ptr(), sizeof(int) * static_cast<size_t>(_batch), s));
+    MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.ptr(), pl.yoloRows.ptr(), sizeof(float) * 8 * cells * static_cast<size_t>(_batch), s));
     if (keepClassScores)
     {
-        const size_t bytes = sizeof(float) * static_cast<size_t>(cells) * per * static_cast<size_t>(_batch);
-        _hostDecoded.reserve(bytes);
-        MSNH_DEV(msnh_hip_memcpy_d2h(_hostDecoded.ptr(), pl.yoloDecoded.ptr(), bytes, s));
-        decodedHost = _hostDecoded.as<float>();
+        const size_t bytes = sizeof(float) * cells * static_cast<size_t>(_channel) * static_cast<size_t>(_batch);
+        sl.decoded.reserve(bytes);
+        MSNH_DEV(msnh_hip_memcpy_d2h(sl.decoded.ptr(), pl.yoloDecoded.ptr(), bytes, s));
     }
-    MSNH_DEV(msnh_hip_stream_sync(s));
+    MSNH_DEV(msnh_hip_event_record(sl.event, s));
+    sl.pending = true;
+}
 
+void YoloOutLayer::finish(int slot)
+{
+    Slot &sl = _slots[slot & 1];
+    if (!sl.pending) MSNH_THROW("YoloOut: nothing to fetch");
+    MSNH_DEV(msnh_hip_event_sync(sl.event));
+    sl.pending = false;
+    const int cells = plan->yoloCells;
+    const int per = _channel;
+    const int *cnt = sl.cnt.as<int>();
+    const float *decodedHost = keepClassScores ? sl.decoded.as<float>() : nullptr;
     batchHasBox.assign(static_cast<size_t>(_batch), false);
     finalOut.assign(static_cast<size_t>(_batch), std::vector<YoloBox>());
 #pragma omp parallel for schedule(dynamic)
@@ -936,9 +1005,22 @@ void YoloOutLayer::forwardGPU(NetworkState &netState)
     {
         const int n = std::min(cnt[b], cells);
         const float *dec = decodedHost ? decodedHost + static_cast<size_t>(b) * cells * per : nullptr;
-        std::vector<YoloBox> cand = boxesFromRows(_hostRows.as<float>() + static_cast<size_t>(b) * cells * 8, n, dec);
-        finalOut[static_cast<size_t>(b)] = nms(cand, _nmsThresh, _useSoftNms != 0);
+        std::vector<YoloBox> cand = boxesFromRows(sl.rows.as<float>() + static_cast<size_t>(b) * cells * 8, n, dec);
+        finalOut[static_cast<size_t>(b)] = _useSoftNms ? nms(cand, _nmsThresh, true) : nmsSorted(cand, _nmsThresh);
     }
     for (int b = 0; b < _batch; ++b) batchHasBox[static_cast<size_t>(b)] = cnt[b] > 0;
+}
+
+void YoloOutLayer::forwardGPU(NetworkState &netState)
+{
+    enqueueGather(netState.stream);
+    enqueueCopyBack(netState.stream, 0);
+    finish(0);
+}
+
+YoloOutLayer::~YoloOutLayer()
+{
+    for (Slot &sl : _slots)
+        if (sl.event) msnh_hip_event_destroy(sl.event);
 }
 }

@@ -41,6 +41,8 @@ void NetBuilder::setOnlyGpu(const bool &onlyGpu) { BaseLayer::setOnlyGpu(onlyGpu
 void NetBuilder::setUseFp16(const bool &useFp16) { BaseLayer::setUseFp16(useFp16); }
 void NetBuilder::setForceUseCuda(const bool &v) { BaseLayer::setForceUseCuda(v); }
 void NetBuilder::setKeepClassScores(const bool &keep) { YoloOutLayer::keepClassScores = keep; }
+bool NetBuilder::autoTune = true;
+void NetBuilder::setAutoTune(const bool &on) { autoTune = on; }
 
 void NetBuilder::setOnlyCpu(const bool &onlyCpu)
 {
@@ -56,6 +58,8 @@ void NetBuilder::clearLayers()
     _net->layers.clear();
     _planReady = false;
     _layerOutputs.clear();
+    _nextSlot = 0;
+    _inFlight = 0;
 }
 
 // ---- build -----------------------------------------------------------------------------------------------------------
@@ -318,6 +322,8 @@ void NetBuilder::finalizePlan()
     _inputPinned.reserve(inBytes);
     _netState->gpuInput = _inputDev.as<float>();
     if (_graph) { msnh_hip_graph_destroy(_graph); _graph = nullptr; }
+    _nextSlot = 0;
+    _inFlight = 0;
 
     const int dtype = BaseLayer::useFp16 ? MSNH_F16 : MSNH_F32;
     std::unique_ptr<Plan> plan = lowerNetwork(dtype);
@@ -350,6 +356,7 @@ void NetBuilder::finalizePlan()
     plan->place();
     setupYoloBuffers(*plan, _net->batch);
     plan->prepareWeights();
+    if (autoTune) plan->tuneConvs(_stream);
 
     // hand every layer its slice of the op list
     for (size_t i = 0; i < _net->layers.size(); ++i)
@@ -448,6 +455,8 @@ void NetBuilder::enqueueForward(const float *deviceInput)
 {
     if (!_planReady) MSNH_THROW("weights are not loaded");
     Plan &plan = *_net->plan;
+    YoloOutLayer *yout = _net->layers.back()->type() == LayerType::YOLO_OUT ? static_cast<YoloOutLayer *>(_net->layers.back()) : nullptr;
+    if (yout && _inFlight >= 2) MSNH_THROW("two forwards are already in flight: fetch a result first");
     if (deviceInput != nullptr && deviceInput != _inputDev.as<float>())
         MSNH_DEV(msnh_hip_memcpy_d2d(_inputDev.ptr(), deviceInput, sizeof(float) * static_cast<size_t>(_net->inputNum), _stream));
     if (_graph == nullptr)
@@ -458,12 +467,7 @@ void NetBuilder::enqueueForward(const float *deviceInput)
         {
             if (plan.yoloCandCnt.ptr()) MSNH_DEV(msnh_hip_fill_zero(plan.yoloCandCnt.ptr(), plan.yoloCandCnt.bytes(), _stream));
             plan.runAll(_stream);
-            if (plan.yoloCells > 0 && _net->layers.back()->type() == LayerType::YOLO_OUT)
-            {
-                const int per = 5 + plan.yoloClasses;
-                MSNH_DEV(msnh_hip_yolo_gather(_net->batch, plan.yoloClasses, plan.yoloDecoded.as<float>(), static_cast<long long>(plan.yoloCells) * per,
-                                              plan.yoloCandIdx.as<int>(), plan.yoloCells, plan.yoloCandCnt.as<int>(), plan.yoloRows.as<float>(), _stream));
-            }
+            if (yout) yout->enqueueGather(_stream);
         }
         catch (...)
         {
@@ -475,6 +479,13 @@ void NetBuilder::enqueueForward(const float *deviceInput)
         MSNH_DEV(msnh_hip_graph_end(_stream, &_graph));
     }
     MSNH_DEV(msnh_hip_graph_launch(_graph, _stream));
+    if (yout)
+    {
+        // results leave the device right behind the forward, so the next forward can start while the host sorts
+        yout->enqueueCopyBack(_stream, _nextSlot);
+        _nextSlot ^= 1;
+        ++_inFlight;
+    }
 }
 
 void NetBuilder::sync() { MSNH_DEV(msnh_hip_stream_sync(_stream)); }
@@ -491,10 +502,16 @@ std::vector<std::vector<YoloBox>> NetBuilder::fetchYolo()
 {
     BaseLayer *last = _net->layers.back();
     if (last->type() != LayerType::YOLO_OUT) MSNH_THROW("not a yolo net");
-    // the captured graph already compacted the candidates; only the host half of YoloOut remains.  Calling the
-    // layer's forwardGPU repeats the (idempotent) gather and then does the copy-back, sort and NMS.
-    last->forwardGPU(*_netState);
-    return static_cast<YoloOutLayer *>(last)->finalOut;
+    YoloOutLayer *yout = static_cast<YoloOutLayer *>(last);
+    if (_inFlight <= 0)
+    {
+        if (yout->finalOut.empty()) MSNH_THROW("no forward in flight");
+        return yout->finalOut;                                  // nothing new: the last result again
+    }
+    const int slot = (_nextSlot + 2 - _inFlight) & 1;          // oldest outstanding
+    yout->finish(slot);
+    --_inFlight;
+    return yout->finalOut;
 }
 
 std::vector<float> NetBuilder::runClassifyGPU(std::vector<float> img)
@@ -607,6 +624,76 @@ void NetBuilder::setSaveLayerOutput(bool v)
     _saveLayerOutput = v;
     // dumps need every layer output as a real tensor: re-plan if a plan already exists
     if (_planReady) finalizePlan();
+}
+
+float NetBuilder::profileOps(int kind, int reps, int *launches, double *flops)
+{
+    if (!_planReady) MSNH_THROW("weights are not loaded");
+    Plan &plan = *_net->plan;
+    msnh_event_t e0 = nullptr, e1 = nullptr;
+    MSNH_DEV(msnh_hip_event_create(&e0));
+    MSNH_DEV(msnh_hip_event_create(&e1));
+    int n = 0;
+    double f = 0;
+    MSNH_DEV(msnh_hip_event_record(e0, _stream));
+    for (int r = 0; r < reps; ++r)
+        for (size_t i = 0; i < plan.ops.size(); ++i)
+        {
+            const PlanOp &op = plan.ops[i];
+            if (op.dead || (kind >= 0 && static_cast<int>(op.kind) != kind)) continue;
+            plan.run(i, i + 1, _stream);
+            ++n;
+            f += op.flops;
+        }
+    MSNH_DEV(msnh_hip_event_record(e1, _stream));
+    MSNH_DEV(msnh_hip_event_sync(e1));
+    float ms = 0.f;
+    MSNH_DEV(msnh_hip_event_elapsed_ms(e0, e1, &ms));
+    msnh_hip_event_destroy(e0);
+    msnh_hip_event_destroy(e1);
+    if (launches) *launches = n;
+    if (flops) *flops = f;
+    return ms;
+}
+
+std::string NetBuilder::profileEachOp(int reps)
+{
+    if (!_planReady) MSNH_THROW("weights are not loaded");
+    Plan &plan = *_net->plan;
+    static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode"};
+    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem"};
+    msnh_event_t e0 = nullptr, e1 = nullptr;
+    MSNH_DEV(msnh_hip_event_create(&e0));
+    MSNH_DEV(msnh_hip_event_create(&e1));
+    std::ostringstream os;
+    double totalUs = 0;
+    for (size_t i = 0; i < plan.ops.size(); ++i)
+    {
+        const PlanOp &op = plan.ops[i];
+        if (op.dead) continue;
+        plan.run(i, i + 1, _stream);
+        MSNH_DEV(msnh_hip_event_record(e0, _stream));
+        for (int r = 0; r < reps; ++r) plan.run(i, i + 1, _stream);
+        MSNH_DEV(msnh_hip_event_record(e1, _stream));
+        MSNH_DEV(msnh_hip_event_sync(e1));
+        float ms = 0.f;
+        MSNH_DEV(msnh_hip_event_elapsed_ms(e0, e1, &ms));
+        const double us = ms * 1e3 / reps;
+        totalUs += us;
+        const PlanTensor &in = plan.tensors[static_cast<size_t>(op.in0)];
+        const PlanTensor &out = plan.tensors[static_cast<size_t>(op.out)];
+        const double bytes = static_cast<double>(in.elems()) * (in.dtype == MSNH_F16 ? 2 : 4) + static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4) +
+                             (op.in1 >= 0 ? static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4) : 0.0);
+        char line[320];
+        snprintf(line, sizeof(line), "L%-3d %-11s %-9s t%-2d k%d s%d g%-4d %4dx%4dx%4dx%4d -> %4dx%4dx%4d %s%s %9.2f us %8.2f TF/s %8.1f GB/s\n", op.layerIndex,
+                 kinds[op.kind], op.kind == PlanOp::CONV ? algos[op.algo] : "-", op.tile, op.ksize, op.stride, op.groups, in.n, in.h, in.w, in.c, out.h, out.w,
+                 out.c, out.dtype == MSNH_F16 ? "f16" : "f32", op.in1 >= 0 ? "+res" : "    ", us, op.flops / us * 1e-6, bytes / us * 1e-3);
+        os << line;
+    }
+    os << "total " << totalUs << " us over " << plan.liveOps() << " launches\n";
+    msnh_hip_event_destroy(e0);
+    msnh_hip_event_destroy(e1);
+    return os.str();
 }
 
 std::string NetBuilder::getPlanDetail() const { return _net->plan ? _net->plan->describe() : std::string(); }

@@ -319,6 +319,7 @@ static msnh_conv_desc convDesc(const Plan &plan, const PlanOp &op)
     d.res_mul = op.in1 >= 0 ? plan.mulOf(op.in1) : 1.f;
     d.out_mul = 1.f / plan.mulOf(op.out);
     d.algo = op.algo;
+    d.tile = op.tile;
     return d;
 }
 
@@ -396,6 +397,51 @@ void Plan::prepareWeights()
             op.flops = 2.0 * static_cast<double>(w.size()) * in.n;
         }
     }
+}
+
+// Per-layer search over the implicit-GEMM tile configurations: each candidate runs the real launch (same buffers,
+// same epilogue) a few times between two device events; the fastest wins.  Results do not depend on the choice.
+void Plan::tuneConvs(msnh_stream_t s)
+{
+    const int nTiles = msnh_hip_conv2d_tile_count();
+    msnh_event_t e0 = nullptr, e1 = nullptr;
+    MSNH_DEV(msnh_hip_event_create(&e0));
+    MSNH_DEV(msnh_hip_event_create(&e1));
+    struct Key { int b, h, w, c, oc, k, st, g, res, odt; bool operator==(const Key &o) const { return std::memcmp(this, &o, sizeof(Key)) == 0; } };
+    std::vector<std::pair<Key, int>> memo;         // identical shapes share one search
+    for (PlanOp &op : ops)
+    {
+        if (op.dead || op.kind != PlanOp::CONV || op.algo != MSNH_CONV_IGEMM) continue;
+        const PlanTensor &in = tensors[static_cast<size_t>(op.in0)];
+        const PlanTensor &out = tensors[static_cast<size_t>(op.out)];
+        Key key;
+        std::memset(&key, 0, sizeof(key));
+        key.b = in.n; key.h = in.h; key.w = in.w; key.c = in.c; key.oc = out.c; key.k = op.ksize; key.st = op.stride; key.g = op.groups;
+        key.res = op.in1 >= 0; key.odt = out.dtype;
+        bool found = false;
+        for (const auto &m : memo)
+            if (m.first == key) { op.tile = m.second; found = true; break; }
+        if (found) continue;
+        int best = 0;
+        float bestMs = std::numeric_limits<float>::max();
+        for (int tile = 0; tile <= nTiles; ++tile)
+        {
+            op.tile = tile;
+            const int reps = 3;
+            launch(op, s);                                       // warm-up (also surfaces launch errors for this tile)
+            MSNH_DEV(msnh_hip_event_record(e0, s));
+            for (int r = 0; r < reps; ++r) launch(op, s);
+            MSNH_DEV(msnh_hip_event_record(e1, s));
+            MSNH_DEV(msnh_hip_event_sync(e1));
+            float ms = 0.f;
+            MSNH_DEV(msnh_hip_event_elapsed_ms(e0, e1, &ms));
+            if (ms < bestMs) { bestMs = ms; best = tile; }
+        }
+        op.tile = best;
+        memo.emplace_back(key, best);
+    }
+    msnh_hip_event_destroy(e0);
+    msnh_hip_event_destroy(e1);
 }
 
 // round-to-nearest-even float -> IEEE half, host side
@@ -529,7 +575,7 @@ std::string Plan::describe() const
         const PlanTensor &out = tensors[static_cast<size_t>(op.out)];
         os << "  L" << op.layerIndex << " " << kinds[op.kind];
         if (op.kind == PlanOp::CONV)
-            os << "[" << algos[op.algo] << " k" << op.ksize << " s" << op.stride << " g" << op.groups << (op.in1 >= 0 ? " +res" : "") << (op.src2 ? " +bn" : "") << "]";
+            os << "[" << algos[op.algo] << (op.tile ? " t" + std::to_string(op.tile) : std::string()) << " k" << op.ksize << " s" << op.stride << " g" << op.groups << (op.in1 >= 0 ? " +res" : "") << (op.src2 ? " +bn" : "") << "]";
         os << " " << in.n << "x" << in.h << "x" << in.w << "x" << in.c << " -> " << out.h << "x" << out.w << "x" << out.c
            << (out.dtype == MSNH_F16 ? " f16" : " f32") << " e" << out.scaleExp;
         if (out.parent >= 0) os << " (slice@" << chanOffsetInRoot(op.out) << " of " << tensors[static_cast<size_t>(root(op.out))].c << ")";

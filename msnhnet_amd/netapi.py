@@ -18,6 +18,7 @@ SYMBOLS = [
     "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops",
     "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
     "msnhnet_enqueue", "msnhnet_sync", "msnhnet_fetch_classify", "msnhnet_fetch_yolo", "msnhnet_gpu_inference_time", "msnhnet_time_detail",
+    "msnhnet_profile_ops", "msnhnet_profile_each_op",
 ]
 
 LAYER_TYPE = {0: "conv", 2: "connect", 3: "maxpool", 4: "localavgpool", 8: "route", 13: "batchnorm", 15: "yolo", 16: "yoloout",
@@ -87,6 +88,9 @@ def lib():
     L.msnhnet_sync.argtypes = [vp]
     L.msnhnet_fetch_classify.argtypes = [vp, fp, ll, llp]
     L.msnhnet_fetch_yolo.argtypes = [vp, ip, fp, ll, llp]
+    L.msnhnet_profile_ops.argtypes = [vp, ci, ci, fp, ip, ctypes.POINTER(ctypes.c_double)]
+    L.msnhnet_profile_each_op.argtypes = [vp, ci, cp, ll]
+    L.msnhnet_profile_each_op.restype = ll
     L.msnhnet_gpu_inference_time.argtypes = [vp]
     L.msnhnet_gpu_inference_time.restype = ctypes.c_float
     _lib = L
@@ -250,6 +254,20 @@ class Net:
 
     def fetch_yolo(self):
         return self._boxes(self.L.msnhnet_fetch_yolo)
+
+    def profile_ops(self, kind, reps):
+        """-> (total ms, launches, algorithmic FLOPs) of `reps` eager passes over the launches of one kind (-1 = all)."""
+        ms, n, f = ctypes.c_float(), ctypes.c_int(), ctypes.c_double()
+        _check(self.L.msnhnet_profile_ops(self.h, kind, reps, ctypes.byref(ms), ctypes.byref(n), ctypes.byref(f)))
+        return ms.value, n.value, f.value
+
+    def profile_each_op(self, reps=20):
+        n = self.L.msnhnet_profile_each_op(self.h, reps, None, 0)
+        if n < 0:
+            _check(1)
+        buf = ctypes.create_string_buffer(n + 1)
+        self.L.msnhnet_profile_each_op(self.h, reps, buf, n + 1)
+        return buf.value.decode()
 
     def gpu_inference_time_ms(self):
         return float(self.L.msnhnet_gpu_inference_time(self.h))

@@ -67,7 +67,7 @@ def rel_err(a, b):
 
 def conv2d(x, w_oihw, *, dtype, out_dtype=None, stride=1, pad=0, dil=1, groups=1, scale=None, shift=None, act="none",
            act_param=0.1, residual=None, act2="none", act2_param=0.1, res_mul=1.0, out_mul=1.0, algo="auto",
-           in_ld=None, out_ld=None, res_ld=None):
+           in_ld=None, out_ld=None, res_ld=None, tile=0):
     """x: NCHW float32 numpy (for every algo; the stem algo is fed NCHW as is). Returns NCHW float32 numpy."""
     init()
     L = abi.lib()
@@ -79,7 +79,7 @@ def conv2d(x, w_oihw, *, dtype, out_dtype=None, stride=1, pad=0, dil=1, groups=1
     ow = (wd + 2 * pad - ext) // stride + 1
     d = abi.ConvDesc(dtype, out_dtype, b, h, wd, c, in_ld or c, oc, oh, ow, out_ld or oc, k, stride, pad, dil, groups,
                      abi.ACT[act], act_param, 1 if residual is not None else 0, res_ld or oc, abi.ACT[act2], act2_param,
-                     res_mul, out_mul, abi.ALGO[algo])
+                     res_mul, out_mul, abi.ALGO[algo], tile)
     resolved = L.msnh_hip_conv2d_select_algo(ctypes.byref(d))
     n = L.msnh_hip_conv2d_packed_weight_elems(ctypes.byref(d), resolved)
     host_dt = np.float32 if (dtype == abi.F32 or resolved == abi.ALGO["stem"]) else np.float16

@@ -83,6 +83,25 @@ def test_conv_epilogue(act, act2, algo, dtype):
     assert gu.rel_err(y, ref) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [abi.F32, abi.F16])
+def test_conv_every_tile_configuration(dtype):
+    """all tile configurations of the implicit GEMM give the same answer (odd sizes exercise every edge guard)"""
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(21)
+    x, wt = _case(rng, 2, 40, 21, 19, 136, 3)
+    res = rng.standard_normal((2, 136, 21, 19), dtype=np.float32)
+    if dtype == abi.F16:
+        x, wt, res = gu.round_f16(x), gu.round_f16(wt), gu.round_f16(res)
+    ref = _ref(x, wt, 1, 1, 1, 1, None, None, "leaky", 0.1, res, "none", 1.0, 1.0)
+    n = abi.lib().msnh_hip_conv2d_tile_count()
+    assert n >= 1
+    for tile in range(1, n + 1):
+        print("tile", tile, dtype, flush=True)
+        y, _ = gu.conv2d(x, wt, dtype=dtype, stride=1, pad=1, act="leaky", residual=res, algo="igemm", tile=tile)
+        assert gu.rel_err(y, ref) <= TOL[dtype], tile
+
+
 def test_conv_f16_in_f32_out():
     import gpuutil as gu
     rng = np.random.default_rng(11)
@@ -132,8 +151,8 @@ def test_conv_rejects_bad_shapes():
     import gpuutil as gu
     gu.init()
     L = abi.lib()
-    d = abi.ConvDesc(abi.F16, abi.F16, 1, 8, 8, 12, 12, 16, 8, 8, 16, 3, 1, 1, 1, 1, 22, 0.1, 0, 16, 22, 0.1, 1.0, 1.0, abi.ALGO["igemm"])
+    d = abi.ConvDesc(abi.F16, abi.F16, 1, 8, 8, 12, 12, 16, 8, 8, 16, 3, 1, 1, 1, 1, 22, 0.1, 0, 16, 22, 0.1, 1.0, 1.0, abi.ALGO["igemm"], 0)
     assert L.msnh_hip_conv2d(ctypes.byref(d), 16, 16, None, None, None, 16, None, 0, None) != 0      # in_c % 8
     assert b"IGEMM" in L.msnh_hip_last_error()
-    d = abi.ConvDesc(abi.F16, abi.F16, 1, 8, 8, 16, 16, 16, 9, 8, 16, 3, 1, 1, 1, 1, 22, 0.1, 0, 16, 22, 0.1, 1.0, 1.0, 0)
+    d = abi.ConvDesc(abi.F16, abi.F16, 1, 8, 8, 16, 16, 16, 9, 8, 16, 3, 1, 1, 1, 1, 22, 0.1, 0, 16, 22, 0.1, 1.0, 1.0, 0, 0)
     assert L.msnh_hip_conv2d(ctypes.byref(d), 16, 16, None, None, None, 16, None, 0, None) != 0      # wrong out_h
