@@ -72,6 +72,9 @@ def main():
     ap.add_argument("--workload", default="yolov3", choices=sorted(WORKLOADS))
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch a plain 256 MiB -> 256 MiB channel-copy kernel 5 times (a known-size reference for scaling "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no sharding, no collectives); use --gpus 1")
@@ -85,6 +88,18 @@ def main():
     netp, binp, g = zoo.write_model(a.workload, tmp, batch, size, seed=a.seed)
     net = netapi.Net(netp, binp, fp16=(dtype == "f16"))
     detect = a.workload.startswith("yolo")
+
+    if a.copy_probe:
+        import ctypes
+        from msnhnet_amd import hipabi
+        src = torch.ones(1 << 27, dtype=torch.float16).cuda()          # 256 MiB
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(5):
+            hipabi.check(hipabi.lib().msnh_hip_copy_channels(hipabi.F16, (1 << 27) // 256, 256, ctypes.c_void_p(src.data_ptr()), 256, 1.0,
+                                                             ctypes.c_void_p(dst.data_ptr()), 256, None))
+        hipabi.check(hipabi.lib().msnh_hip_stream_sync(None))
+        del src, dst
 
     x = torch.from_numpy(zoo.seeded_input(batch, 3, size, size, a.seed + 1)).cuda()
     torch.cuda.synchronize()

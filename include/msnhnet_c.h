@@ -85,6 +85,8 @@ int msnhnet_enqueue(msnhnet_t net, const float *device_input);
 int msnhnet_sync(msnhnet_t net);
 int msnhnet_fetch_classify(msnhnet_t net, float *out, long long cap, long long *n_out);
 int msnhnet_fetch_yolo(msnhnet_t net, int *counts, float *boxes, long long cap_boxes, long long *total);
+/* Upper bound of the boxes one run can return (batch * number of anchor cells); 0 for a non-detection network. */
+long long msnhnet_yolo_max_boxes(msnhnet_t net);
 /* Device-event timing of `reps` eager passes over the plan's launches of one kind (0 conv, 1 affine, 2 add, 3 copy,
  * 4 maxpool, 5 avgpool, 6 upsample, 7 connected, 8 input cast, 9 yolo decode, -1 all).  Outputs the total
  * milliseconds, the number of launches timed and their algorithmic FLOPs (2*MACs; 0 for non-GEMM kinds). */

@@ -31,6 +31,7 @@ struct IgemmArgs
     int P;                  // batch*OH*OW
     int cChunks;            // ceil(cinG / BK)
     int nIter;              // taps * cChunks
+    int mTiles;             // ceil(coutG / BM)
     int act, act2, hasRes, vecOk;
     float actParam, act2Param, resMul, outMul;
 };
@@ -83,8 +84,17 @@ __global__ __launch_bounds__(256) void convIgemmKernel(IgemmArgs a)
     const int wm   = wave / WN;
     const int wn   = wave % WN;
     const int g    = blockIdx.z;
-    const int m0   = blockIdx.y * BM;
-    const int p0   = blockIdx.x * BN;
+    // Workgroup -> tile mapping.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its own
+    // L2.  Ids are therefore first regrouped per XCD (id % 8 selects the XCD, id / 8 the position inside it), and
+    // inside an XCD the channel tiles of one pixel tile run back to back, so an input pixel is fetched into one L2
+    // once instead of once per channel tile and XCD.
+    const int nTilesP = (a.P + BN - 1) / BN;
+    const int total   = a.mTiles * nTilesP;
+    const int perXcd  = (total + 7) / 8;
+    const int logical = (blockIdx.x % 8) * perXcd + blockIdx.x / 8;
+    if (logical >= total) return;                     // padding ids of the last round
+    const int m0   = (logical % a.mTiles) * BM;
+    const int p0   = (logical / a.mTiles) * BN;
 
     const T *xg = static_cast<const T *>(a.x) + static_cast<size_t>(g) * a.cinG;
     const T *wg = static_cast<const T *>(a.w) + static_cast<size_t>(g) * a.coutG * a.taps * a.cinG;
@@ -300,7 +310,9 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
     const size_t smemLoop = static_cast<size_t>(2) * (BM + BN) * LDK * sizeof(T);
     const size_t smemEpi  = static_cast<size_t>(4) * (BN / WN) * (BM / WM + 4) * sizeof(float);
     const size_t smem = smemLoop > smemEpi ? smemLoop : smemEpi;
-    dim3 grid((a.P + BN - 1) / BN, (a.coutG + BM - 1) / BM, groups);
+    a.mTiles = (a.coutG + BM - 1) / BM;
+    const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
+    dim3 grid((tiles + 7) / 8 * 8, 1, groups);
     auto kern = convIgemmKernel<T, TOut, BM, BN, KV, WM, WN>;
     if (smem > 48 * 1024)
     {

@@ -333,6 +333,19 @@ long long msnhnet_profile_each_op(msnhnet_t net, int reps, char *dst, long long 
     return n;
 }
 
+long long msnhnet_yolo_max_boxes(msnhnet_t net)
+{
+    long long n = 0;
+    guarded([&] {
+        Network *nw = nb(net).getNet();
+        long long cells = 0;
+        for (const BaseLayer *l : nw->layers)
+            if (l->type() == LayerType::YOLO) cells += 3LL * l->getOutHeight() * l->getOutWidth();
+        n = cells * nw->batch;
+    });
+    return n;
+}
+
 float msnhnet_gpu_inference_time(msnhnet_t net)
 {
     float t = -1.f;

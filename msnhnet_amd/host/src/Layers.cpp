@@ -6,6 +6,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include "Msnhnet/net/MsnhNetwork.h"
 #include "Msnhnet/utils/MsnhExVector.h"
@@ -992,7 +993,9 @@ void YoloOutLayer::finish(int slot)
 {
     Slot &sl = _slots[slot & 1];
     if (!sl.pending) MSNH_THROW("YoloOut: nothing to fetch");
+    auto dbg0 = TimeUtil::startRecord();
     MSNH_DEV(msnh_hip_event_sync(sl.event));
+    const float dbgWait = TimeUtil::getElapsedTime(dbg0);
     sl.pending = false;
     const int cells = plan->yoloCells;
     const int per = _channel;
@@ -1009,6 +1012,7 @@ void YoloOutLayer::finish(int slot)
         finalOut[static_cast<size_t>(b)] = _useSoftNms ? nms(cand, _nmsThresh, true) : nmsSorted(cand, _nmsThresh);
     }
     for (int b = 0; b < _batch; ++b) batchHasBox[static_cast<size_t>(b)] = cnt[b] > 0;
+    if (std::getenv("MSNH_DEBUG_TIMING")) std::fprintf(stderr, "yoloout finish: wait %.3f ms, host %.3f ms\n", dbgWait, TimeUtil::getElapsedTime(dbg0) - dbgWait);
 }
 
 void YoloOutLayer::forwardGPU(NetworkState &netState)

@@ -18,7 +18,7 @@ SYMBOLS = [
     "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops",
     "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
     "msnhnet_enqueue", "msnhnet_sync", "msnhnet_fetch_classify", "msnhnet_fetch_yolo", "msnhnet_gpu_inference_time", "msnhnet_time_detail",
-    "msnhnet_profile_ops", "msnhnet_profile_each_op",
+    "msnhnet_profile_ops", "msnhnet_profile_each_op", "msnhnet_yolo_max_boxes",
 ]
 
 LAYER_TYPE = {0: "conv", 2: "connect", 3: "maxpool", 4: "localavgpool", 8: "route", 13: "batchnorm", 15: "yolo", 16: "yoloout",
@@ -91,6 +91,8 @@ def lib():
     L.msnhnet_profile_ops.argtypes = [vp, ci, ci, fp, ip, ctypes.POINTER(ctypes.c_double)]
     L.msnhnet_profile_each_op.argtypes = [vp, ci, cp, ll]
     L.msnhnet_profile_each_op.restype = ll
+    L.msnhnet_yolo_max_boxes.argtypes = [vp]
+    L.msnhnet_yolo_max_boxes.restype = ll
     L.msnhnet_gpu_inference_time.argtypes = [vp]
     L.msnhnet_gpu_inference_time.restype = ctypes.c_float
     _lib = L
@@ -205,15 +207,10 @@ class Net:
         b = self.dims()[0]
         counts = (ctypes.c_int * b)()
         total = ctypes.c_longlong()
-        cap = 4096
-        while True:
-            boxes = np.zeros((cap, 7), np.float32)
-            _check(fn(self.h, *head, counts, _fp(boxes), cap, ctypes.byref(total)))
-            if total.value <= cap:
-                break
-            cap = int(total.value)
-            if head:            # a run call: everything was computed, only the copy was truncated -> fetch again
-                fn, head = self.L.msnhnet_fetch_yolo, ()
+        if getattr(self, "_box_buf", None) is None:
+            self._box_buf = np.zeros((max(int(self.L.msnhnet_yolo_max_boxes(self.h)), 1), 7), np.float32)
+        boxes = self._box_buf
+        _check(fn(self.h, *head, counts, _fp(boxes), boxes.shape[0], ctypes.byref(total)))
         out, at = [], 0
         for i in range(b):
             out.append(boxes[at:at + counts[i]].copy())
