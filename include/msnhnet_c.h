@@ -94,6 +94,10 @@ int msnhnet_profile_ops(msnhnet_t net, int kind, int reps, float *ms_total, int 
 /* Per-launch timing table (text): every live launch of the plan timed on its own, `reps` repetitions each. */
 long long msnhnet_profile_each_op(msnhnet_t net, int reps, char *dst, long long cap);
 float msnhnet_gpu_inference_time(msnhnet_t net);          /* NetBuilder::getGpuInferenceTime, ms */
+/* YoloOutLayer::nms on its own (pure host code, no GPU needed): rows of 7 floats in (x y w h conf bestClsConf
+ * bestClsIdx), already in the order the layer would pass them; fast = 0 runs the reference-shaped greedy loop,
+ * fast = 1 the sorted variant the library uses.  Writes at most cap rows, *n_out = number of surviving boxes. */
+int msnhnet_nms(const float *rows, long long n, float nms_thresh, int fast, float *out, long long cap, long long *n_out);
 long long msnhnet_time_detail(msnhnet_t net, char *dst, long long cap);       /* NetBuilder::getTimeDetail */
 
 #ifdef __cplusplus

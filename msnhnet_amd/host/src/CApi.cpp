@@ -346,6 +346,24 @@ long long msnhnet_yolo_max_boxes(msnhnet_t net)
     return n;
 }
 
+int msnhnet_nms(const float *rows, long long n, float nms_thresh, int fast, float *out, long long cap, long long *n_out)
+{
+    return guarded([&] {
+        if ((!rows && n > 0) || n < 0) MSNH_THROW("bad argument");
+        std::vector<YoloBox> in(static_cast<size_t>(n));
+        for (long long i = 0; i < n; ++i)
+        {
+            const float *r = rows + 7 * i;
+            YoloBox &b = in[static_cast<size_t>(i)];
+            b.xywhBox = Box::XYWHBox(r[0], r[1], r[2], r[3]);
+            b.conf = r[4]; b.bestClsConf = r[5]; b.bestClsIdx = static_cast<int>(r[6]);
+        }
+        std::vector<std::vector<YoloBox>> res(1);
+        res[0] = fast ? YoloOutLayer::nmsSorted(in, nms_thresh) : YoloOutLayer::nms(in, nms_thresh, false);
+        packBoxes(res, nullptr, out, cap, n_out);
+    });
+}
+
 float msnhnet_gpu_inference_time(msnhnet_t net)
 {
     float t = -1.f;

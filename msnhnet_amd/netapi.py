@@ -18,7 +18,7 @@ SYMBOLS = [
     "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops",
     "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
     "msnhnet_enqueue", "msnhnet_sync", "msnhnet_fetch_classify", "msnhnet_fetch_yolo", "msnhnet_gpu_inference_time", "msnhnet_time_detail",
-    "msnhnet_profile_ops", "msnhnet_profile_each_op", "msnhnet_yolo_max_boxes",
+    "msnhnet_profile_ops", "msnhnet_profile_each_op", "msnhnet_yolo_max_boxes", "msnhnet_nms",
 ]
 
 LAYER_TYPE = {0: "conv", 2: "connect", 3: "maxpool", 4: "localavgpool", 8: "route", 13: "batchnorm", 15: "yolo", 16: "yoloout",
@@ -91,6 +91,7 @@ def lib():
     L.msnhnet_profile_ops.argtypes = [vp, ci, ci, fp, ip, ctypes.POINTER(ctypes.c_double)]
     L.msnhnet_profile_each_op.argtypes = [vp, ci, cp, ll]
     L.msnhnet_profile_each_op.restype = ll
+    L.msnhnet_nms.argtypes = [fp, ll, ctypes.c_float, ci, fp, ll, llp]
     L.msnhnet_yolo_max_boxes.argtypes = [vp]
     L.msnhnet_yolo_max_boxes.restype = ll
     L.msnhnet_gpu_inference_time.argtypes = [vp]
@@ -110,6 +111,15 @@ def _fp(a):
 
 def set_use_fp16(on):
     _check(lib().msnhnet_set_use_fp16(1 if on else 0))
+
+
+def nms(rows, thresh, fast=True):
+    """YoloOutLayer::nms on rows of (x y w h conf bestClsConf bestClsIdx); host only."""
+    rows = np.ascontiguousarray(rows, np.float32).reshape(-1, 7)
+    out = np.zeros_like(rows)
+    n = ctypes.c_longlong()
+    _check(lib().msnhnet_nms(_fp(rows), len(rows), thresh, 1 if fast else 0, _fp(out), len(rows), ctypes.byref(n)))
+    return out[:n.value]
 
 
 class Net:

@@ -1,0 +1,302 @@
+"""Pins the oracle (oracle/msnh_oracle.c + oracle/msnh_oracle_net.py) without a GPU:
+
+  1. against golden vectors produced by the reference's own CPU forward (tests/golden/ref_golden.npz, written by
+     tests/golden/make_golden.py from oracle/_ref): whole tensors for 20 micro graphs covering every op and block
+     type, per-layer statistics + final outputs for the five benchmark architectures;
+  2. live against oracle/_ref when that library is present (layer by layer);
+  3. against what the mathematics fixes: brute-force double-precision cross-correlation, identity kernels,
+     1x1 conv == matrix product, depthwise == per-channel correlation, brute-force pooling, closed forms for
+     batch-norm / activations / YOLO decode, hand-computed IoU and NMS cases.
+A dropped term, a transposed operand or a wrong index in any oracle function fails at least one of these.
+"""
+import os
+import tempfile
+
+import numpy as np
+import pytest
+
+import msnh_oracle_net as on
+import netutil as nu
+import refshim
+from msnhnet_amd import zoo
+
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_golden.npz"))
+MICRO = bytes(GOLD["micro/names"]).decode().split("\n")
+
+
+def _write(tmp, name, text, weights):
+    netp = os.path.join(tmp, name + ".msnhnet")
+    binp = os.path.join(tmp, name + ".msnhbin")
+    with open(netp, "w") as f:
+        f.write(text)
+    np.asarray(weights, np.float32).tofile(binp)
+    return netp, binp
+
+
+@pytest.mark.parametrize("name", MICRO)
+def test_oracle_matches_reference_golden_micro(name, tmp_path):
+    text = bytes(GOLD[f"micro/{name}/graph"]).decode()
+    netp, binp = _write(str(tmp_path), name, text, GOLD[f"micro/{name}/weights"])
+    o = on.OracleNet(netp, binp)
+    outs = o.run(GOLD[f"micro/{name}/input"])
+    for i, got in enumerate(outs):
+        ref = GOLD[f"micro/{name}/out{i}"]
+        if ref.size == 0:
+            continue
+        assert nu.rel_err(got.ravel(), ref) <= 3e-6, (name, i)
+    ref_boxes = GOLD[f"micro/{name}/boxes"]
+    if len(ref_boxes):
+        assert len(o.boxes) == len(ref_boxes)
+        assert nu.rel_err(nu.sort_boxes(o.boxes), nu.sort_boxes(ref_boxes)) <= 3e-6
+
+
+def _stats(a):
+    a = np.asarray(a, np.float64).ravel()
+    fin = np.isfinite(a)
+    v = a[fin]
+    idx = (np.arange(16) * 7919) % max(a.size, 1)
+    return np.array([a.size, fin.sum(), v.sum() if v.size else 0, np.abs(v).sum() if v.size else 0, v.max() if v.size else 0,
+                     v.min() if v.size else 0] + [a[i] if a.size else 0 for i in idx], np.float64)
+
+
+@pytest.mark.parametrize("arch", ["resnet18", "resnet50", "mobilenetv2", "yolov3", "yolov4"])
+def test_oracle_matches_reference_golden_nets(arch, tmp_path):
+    size = int(GOLD[f"net/{arch}/size"][0])
+    netp, binp, gw = zoo.write_model(arch, str(tmp_path), 1, size, seed=11)
+    x = zoo.seeded_input(1, 3, size, size, 12)[0]
+    # the fixture is only meaningful if the seeded data is what it was generated from
+    assert abs(x.astype(np.float64).sum() - GOLD[f"net/{arch}/input_sum"][0]) < 1e-6
+    assert abs(np.fromfile(binp, np.float32).astype(np.float64).sum() - GOLD[f"net/{arch}/weights_sum"][0]) < 1e-6
+    o = on.OracleNet(netp, binp)
+    outs = o.run(x)
+    gold = GOLD[f"net/{arch}/stats"]
+    assert len(outs) == len(gold)
+    tol = 5e-4 if arch == "mobilenetv2" else 5e-5       # FMA contraction in the reference build vs none here
+    for i, got in enumerate(outs):
+        s, g = _stats(got), gold[i]
+        assert s[0] == g[0] and s[1] == g[1], (arch, i, "size / finite count")
+        if g[0] == 0:
+            continue
+        scale = max(abs(g[4]), abs(g[5]), 1e-30)
+        assert abs(s[3] - g[3]) <= tol * max(g[3], 1e-30), (arch, i, "abs-sum")
+        assert abs(s[4] - g[4]) <= tol * scale and abs(s[5] - g[5]) <= tol * scale, (arch, i, "max / min")
+        fin = np.isfinite(g[6:])
+        assert (np.isfinite(s[6:]) == fin).all()
+        assert np.abs(s[6:][fin] - g[6:][fin]).max() <= 20 * tol * scale, (arch, i, "samples")
+    if arch.startswith("yolo"):
+        rb = GOLD[f"net/{arch}/boxes"]
+        assert abs(len(o.boxes) - len(rb)) <= 1
+    else:
+        assert int(np.argmax(outs[-1])) == int(np.argmax(GOLD[f"net/{arch}/final"]))
+        assert nu.rel_err(outs[-1].ravel(), GOLD[f"net/{arch}/final"]) <= 10 * tol
+
+
+@pytest.mark.skipif(not refshim.available(), reason="oracle/_ref is not built here")
+@pytest.mark.parametrize("arch,size", [("resnet18", 224), ("mobilenetv2", 224), ("yolov3", 64), ("yolov4", 64)])
+def test_oracle_matches_reference_live(arch, size, tmp_path):
+    netp, binp, gw = zoo.write_model(arch, str(tmp_path), 1, size, seed=21)
+    x = zoo.seeded_input(1, 3, size, size, 22)[0]
+    r = refshim.RefNet(netp, binp, scalar=True)
+    ro = r.run(x)
+    o = on.OracleNet(netp, binp)
+    oo = o.run(x)
+    tol = 5e-4 if arch == "mobilenetv2" else 2e-5
+    infos = r.layer_infos()
+    for i, (a, b) in enumerate(zip(ro, oo)):
+        if not a.size:
+            continue
+        if infos[i]["type"] == "yolo":      # decoded values amplify the logit error, see netutil.yolo_layer_err
+            assert nu.yolo_layer_err(b.ravel(), a, ro[i - 1], 85, size / infos[i]["outH"]) <= tol, (arch, i)
+        else:
+            assert nu.rel_err(b.ravel(), a) <= tol, (arch, i)
+    if arch.startswith("yolo"):
+        assert len(r.boxes()) == len(o.boxes)
+
+
+# ---- what the mathematics fixes ------------------------------------------------------------------------------------
+def _brute_conv(x, w, stride, pad, dil, groups):
+    b, c, h, wd = x.shape
+    oc, cg, k, _ = w.shape
+    ext = dil * (k - 1) + 1
+    oh, ow = (h + 2 * pad - ext) // stride + 1, (wd + 2 * pad - ext) // stride + 1
+    xp = np.zeros((b, c, h + 2 * pad, wd + 2 * pad), np.float64)
+    xp[:, :, pad:pad + h, pad:pad + wd] = x
+    out = np.zeros((b, oc, oh, ow), np.float64)
+    ocg = oc // groups
+    for o in range(oc):
+        g = o // ocg
+        for i in range(k):
+            for j in range(k):
+                patch = xp[:, g * cg:(g + 1) * cg, i * dil:i * dil + (oh - 1) * stride + 1:stride, j * dil:j * dil + (ow - 1) * stride + 1:stride]
+                out[:, o] += np.einsum("bchw,c->bhw", patch, w[o, :, i, j].astype(np.float64))
+    return out
+
+
+@pytest.mark.parametrize("c,oc,k,stride,pad,dil,groups", [(3, 4, 3, 1, 1, 1, 1), (4, 6, 3, 2, 0, 1, 2), (2, 2, 5, 1, 2, 1, 1), (4, 4, 3, 1, 2, 2, 1),
+                                                          (6, 6, 3, 1, 1, 1, 6), (5, 3, 1, 1, 0, 1, 1), (3, 2, 7, 2, 3, 1, 1)])
+def test_conv_is_cross_correlation(c, oc, k, stride, pad, dil, groups):
+    rng = np.random.default_rng(k * 10 + c)
+    x = rng.standard_normal((2, c, 9, 8)).astype(np.float32)
+    w = rng.standard_normal((oc, c // groups, k, k)).astype(np.float32)
+    got = on.conv(x, w, oc, k, stride, pad, dil, groups)
+    ref = _brute_conv(x, w, stride, pad, dil, groups)
+    assert got.shape == ref.shape
+    assert nu.rel_err(got, ref) <= 2e-6
+
+
+def test_conv_identity_and_shift_kernels():
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((1, 3, 6, 7)).astype(np.float32)
+    w = np.zeros((3, 3, 3, 3), np.float32)
+    for ch in range(3):
+        w[ch, ch, 1, 1] = 1                      # centre tap: identity
+    assert np.array_equal(on.conv(x, w, 3, 3, 1, 1), x)
+    w[:] = 0
+    for ch in range(3):
+        w[ch, ch, 1, 2] = 1                      # tap to the right: out[y][x] = in[y][x+1] (no kernel flip)
+    y = on.conv(x, w, 3, 3, 1, 1)
+    assert np.array_equal(y[..., :-1], x[..., 1:]) and (y[..., -1] == 0).all()
+    w[:] = 0
+    for ch in range(3):
+        w[ch, ch, 2, 1] = 1                      # tap below: out[y][x] = in[y+1][x]
+    y = on.conv(x, w, 3, 3, 1, 1)
+    assert np.array_equal(y[:, :, :-1], x[:, :, 1:]) and (y[:, :, -1] == 0).all()
+
+
+def test_conv_1x1_is_matrix_product_and_bias_bn_closed_form():
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((2, 5, 4, 3)).astype(np.float32)
+    w = rng.standard_normal((7, 5, 1, 1)).astype(np.float32)
+    bias = rng.standard_normal(7).astype(np.float32)
+    ref = np.einsum("oc,bchw->bohw", w[:, :, 0, 0].astype(np.float64), x.astype(np.float64))
+    assert nu.rel_err(on.conv(x, w, 7, 1, bias=bias), ref + bias.reshape(1, -1, 1, 1)) <= 1e-6
+    g, beta, mean, var = [rng.uniform(0.5, 1.5, 7).astype(np.float32) for _ in range(4)]
+    bn = ((ref - mean.reshape(1, -1, 1, 1)) / np.sqrt(var.reshape(1, -1, 1, 1).astype(np.float64) + 1e-5)) * g.reshape(1, -1, 1, 1) + beta.reshape(1, -1, 1, 1)
+    got = on.conv(x, w, 7, 1, bn4=np.concatenate([g, beta, mean, var]), act="leaky", act_param=0.1)
+    assert nu.rel_err(got, np.where(bn > 0, bn, 0.1 * bn)) <= 2e-6
+
+
+def test_activation_special_values():
+    f = lambda v, a, p=0.1: float(on.activate(np.array([v], np.float32), a, p)[0])
+    assert f(0, "relu6") == 0 and f(6, "relu6") == 6 and f(7.5, "relu6") == 6 and f(-1, "relu6") == 0 and f(3, "relu6") == 3
+    assert f(-2, "leaky") == pytest.approx(-0.2) and f(-2, "leaky", 0.25) == pytest.approx(-0.5) and f(2, "leaky") == 2
+    assert f(-3, "relu") == 0 and f(3, "relu") == 3
+    assert f(0, "mish") == 0 and f(0, "swish") == 0 and f(0, "logistic") == 0.5
+    assert f(25, "mish") == pytest.approx(25.0)                      # softplus threshold +20: tanh(x) == 1
+    assert f(-25, "mish") == pytest.approx(-25 * np.tanh(np.exp(-25.0)), rel=1e-5)
+    assert f(1, "mish") == pytest.approx(1 * np.tanh(np.log1p(np.exp(1.0))), rel=1e-6)
+    assert f(2, "swish") == pytest.approx(2 / (1 + np.exp(-2.0)), rel=1e-6)
+    assert f(5, "none") == 5
+
+
+def test_pooling_and_upsample_brute_force():
+    rng = np.random.default_rng(2)
+    x = rng.standard_normal((2, 3, 7, 9)).astype(np.float32)
+    for k, s, p in ((2, 2, 0), (3, 2, 1), (5, 1, 2), (3, 1, 1)):
+        oh, ow = (7 + 2 * p - k) // s + 1, (9 + 2 * p - k) // s + 1
+        mx = np.empty((2, 3, oh, ow), np.float32)
+        av = np.empty((2, 3, oh, ow), np.float64)
+        for i in range(oh):
+            for j in range(ow):
+                ys = [y for y in range(i * s - p, i * s - p + k) if 0 <= y < 7]
+                xs = [v for v in range(j * s - p, j * s - p + k) if 0 <= v < 9]
+                win = x[:, :, ys][:, :, :, xs]
+                mx[:, :, i, j] = win.max(axis=(2, 3))
+                av[:, :, i, j] = win.astype(np.float64).mean(axis=(2, 3))          # divides by the VALID count
+        assert np.array_equal(on.maxpool(x, k, s, p), mx)
+        assert nu.rel_err(on.avgpool(x, k, s, p), av) <= 1e-6
+    up = on.upsample(x, 2)
+    assert up.shape == (2, 3, 14, 18)
+    for j in range(14):
+        for i in range(18):
+            assert np.array_equal(up[:, :, j, i], x[:, :, j // 2, i // 2])
+    assert np.array_equal(on.upsample(x, 3, 0.5), 0.5 * np.repeat(np.repeat(x, 3, axis=2), 3, axis=3))
+
+
+def test_connected_is_matrix_vector():
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((3, 20, 1, 1)).astype(np.float32)
+    w = rng.standard_normal((6, 20)).astype(np.float32)
+    b = rng.standard_normal(6).astype(np.float32)
+    ref = x.reshape(3, 20).astype(np.float64) @ w.T.astype(np.float64) + b
+    assert nu.rel_err(on.connected(x, w, b, 6).reshape(3, 6), ref) <= 1e-6
+
+
+def test_yolo_decode_closed_form():
+    rng = np.random.default_rng(4)
+    cls, h, w = 3, 4, 5
+    per = 5 + cls
+    x = rng.standard_normal((1, 3 * per, h, w)).astype(np.float32) * 2
+    anchors = np.array([10, 14, 23, 27, 37, 58], np.float32)
+    out = on.yolo_decode(x, cls, anchors, 8.0)
+    sig = lambda v: 1 / (1 + np.exp(-v.astype(np.float64)))
+    cols, rows = np.meshgrid(np.arange(w), np.arange(h))
+    for a in range(3):
+        p = x[0, a * per:(a + 1) * per]
+        assert nu.rel_err(out[0, a * per + 0], (sig(p[0]) + cols) * 8.0) <= 1e-6
+        assert nu.rel_err(out[0, a * per + 1], (sig(p[1]) + rows) * 8.0) <= 1e-6
+        assert nu.rel_err(out[0, a * per + 2], anchors[2 * a] * np.exp(p[2].astype(np.float64))) <= 1e-6
+        assert nu.rel_err(out[0, a * per + 3], anchors[2 * a + 1] * np.exp(p[3].astype(np.float64))) <= 1e-6
+        assert nu.rel_err(out[0, a * per + 4:(a + 1) * per], sig(p[4:])) <= 1e-6
+    big = np.full((1, 3 * per, 1, 1), 100.0, np.float32)            # exp overflow -> +inf, like the benchmark weights
+    o = on.yolo_decode(big, cls, anchors, 32.0)
+    assert np.isinf(o[0, 2, 0, 0]) and o[0, 4, 0, 0] == 1.0
+
+
+def test_iou_plus_one_convention_and_nan():
+    # boxes [0,10]x[0,10] and [5,15]x[0,10] with the inclusive-pixel +1: inter = 6*11, areas 11*11
+    a, b = [5, 5, 10, 10], [10, 5, 10, 10]
+    assert on.iou(a, b) == pytest.approx(66 / (121 + 121 - 66))
+    assert on.iou(a, a) == pytest.approx(1.0)
+    assert on.iou([0, 0, 2, 2], [100, 100, 2, 2]) == 0.0
+    # touching boxes still overlap by one "pixel" column under the +1 convention
+    assert on.iou([0, 0, 2, 2], [2, 0, 2, 2]) == pytest.approx(3 / (9 + 9 - 3))
+    assert np.isnan(on.iou([5, 5, np.inf, np.inf], [5, 5, np.inf, np.inf]))
+
+
+def _head(boxes, cls_num, hw):
+    """builds one decoded head [3*(5+cls), hw] holding the given (anchor, pixel) -> (x,y,w,h,obj,scores...) entries"""
+    per = 5 + cls_num
+    t = np.zeros((3 * per, hw, 1), np.float32)
+    for (a, p), v in boxes.items():
+        t[a * per:(a + 1) * per, p, 0] = v
+    return t
+
+
+def test_yolo_out_hand_cases():
+    cls = 3
+    big = [50, 50, 40, 40]
+    near = [52, 50, 40, 40]          # IoU with big ~ 0.9 -> suppressed when same class
+    far = [150, 150, 40, 40]
+    entries = {
+        (0, 0): big + [0.9, 0.1, 0.8, 0.1],       # class 1, kept (highest objectness of class 1)
+        (0, 1): near + [0.8, 0.1, 0.9, 0.1],      # class 1, suppressed by the first although its obj*cls key is equal
+        (1, 0): near + [0.7, 0.9, 0.1, 0.1],      # class 0, alone in its class -> passes through
+        (1, 2): far + [0.6, 0.2, 0.7, 0.1],       # class 1, far away -> kept
+        (2, 3): big + [0.3, 0.9, 0.9, 0.9],       # objectness below the threshold -> never a candidate
+        (2, 1): big + [0.5, 0.9, 0.9, 0.9],       # objectness == threshold: strict '>' drops it
+    }
+    out = on.yolo_out([_head(entries, cls, 4)], cls, 0.5, 0.45)
+    got = sorted((round(float(b[4]), 3), int(b[6])) for b in out)
+    assert got == sorted([(0.9, 1), (0.7, 0), (0.6, 1)])
+    # NMS ranks by objectness, not by objectness*class score: swap which of the overlapping pair has more objectness
+    entries[(0, 0)] = big + [0.8, 0.1, 0.99, 0.1]
+    entries[(0, 1)] = near + [0.9, 0.1, 0.6, 0.1]
+    out = on.yolo_out([_head(entries, cls, 4)], cls, 0.5, 0.45)
+    assert sorted(round(float(b[4]), 3) for b in out if int(b[6]) == 1) == [0.6, 0.9]
+    # threshold is strict: iou exactly at the threshold is kept
+    e2 = {(0, 0): [5, 5, 10, 10, 0.9, 1, 0, 0], (0, 1): [10, 5, 10, 10, 0.8, 1, 0, 0]}
+    thr = on.iou([10, 5, 10, 10], [5, 5, 10, 10])
+    assert len(on.yolo_out([_head(e2, cls, 2)], cls, 0.5, thr)) == 2
+    assert len(on.yolo_out([_head(e2, cls, 2)], cls, 0.5, np.nextafter(np.float32(thr), np.float32(0)))) == 1
+    assert len(on.yolo_out([_head({}, cls, 2)], cls, 0.5, 0.5)) == 0
+
+
+def test_parse_msnhnet_duplicate_keys_and_expansion(tmp_path):
+    g = zoo.yolov3(batch=1, size=64)
+    netp = os.path.join(str(tmp_path), "y.msnhnet")
+    with open(netp, "w") as f:
+        f.write(g.text())
+    o = on.OracleNet(netp)
+    assert len(o.top) == 53                      # 23 residual blocks expanded from 5 `size:` entries
+    assert [k for k, _ in o.top].count("resblock") == 23
