@@ -129,6 +129,9 @@ typedef struct msnh_conv_desc
  * speed per shape.  The host library times them per layer at load (the reference asks cuDNN for the fastest
  * algorithm the same way, src/layers/MsnhConvolutionalLayer.cpp:150-194). */
 int msnh_hip_conv2d_tile_count(void);
+/* 1 if IGEMM tile configuration `tile` can run this shape (some configurations are specialised, e.g. for 3x3
+ * stride-1 layers whose input patch fits in LDS), else 0.  Pure host function. */
+int msnh_hip_conv2d_tile_supported(const msnh_conv_desc *d, int tile);
 /* Which algorithm MSNH_CONV_AUTO resolves to for this shape (never AUTO).  Pure host function. */
 int msnh_hip_conv2d_select_algo(const msnh_conv_desc *d);
 /* Number of elements (of d->dtype) of the packed weight buffer for `algo`.  Pure host function. */

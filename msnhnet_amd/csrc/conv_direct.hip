@@ -10,7 +10,7 @@
 namespace msnh {
 
 int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
-              const void *residual, void *y, hipStream_t st);
+              const void *residual, void *y, hipStream_t st, bool dryRun);
 int igemmTileCount();
 int convWinograd(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
                  const void *residual, void *y, void *ws, size_t wsBytes, hipStream_t st);
@@ -219,6 +219,15 @@ extern "C" {
 
 int msnh_hip_conv2d_tile_count(void) { return igemmTileCount(); }
 
+int msnh_hip_conv2d_tile_supported(const msnh_conv_desc *d, int tile)
+{
+    if (!d || validate(d) || !igemmOk(d) || tile < 0 || tile > igemmTileCount()) return 0;
+    if (tile == 0) return 1;
+    msnh_conv_desc t = *d;
+    t.tile = tile;
+    return convIgemm(&t, d, d, nullptr, nullptr, nullptr, &t, nullptr, true) == 0 ? 1 : 0;      // pointers unused in a dry run
+}
+
 int msnh_hip_conv2d_select_algo(const msnh_conv_desc *d)
 {
     if (!d) return MSNH_CONV_DIRECT;
@@ -309,7 +318,7 @@ int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const
     case MSNH_CONV_IGEMM:
         MSNH_REQUIRE(igemmOk(d), "conv2d: IGEMM needs (in_c/groups) and in_ld to be multiples of %d", d->dtype == MSNH_F16 ? 8 : 4);
         MSNH_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0, "conv2d: IGEMM needs 16-byte aligned x and w");
-        return convIgemm(d, x, w, scale, shift, residual, y, st);
+        return convIgemm(d, x, w, scale, shift, residual, y, st, false);
     case MSNH_CONV_WINOGRAD:
         MSNH_REQUIRE(winogradOk(d), "conv2d: shape not supported by the Winograd kernel");
         return convWinograd(d, x, w, scale, shift, residual, y, workspace, workspace_bytes, st);

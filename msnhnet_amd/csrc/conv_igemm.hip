@@ -18,7 +18,7 @@ int igemmHeuristicTile(const msnh_conv_desc *d)
 int igemmTileCount() { return kIgemmTiles; }
 
 int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
-              const void *residual, void *y, hipStream_t st)
+              const void *residual, void *y, hipStream_t st, bool dryRun)
 {
     IgemmArgs a;
     a.x = x; a.w = w; a.scale = scale; a.shift = shift; a.res = residual; a.y = y;
@@ -27,6 +27,9 @@ int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float
     a.cinG = d->in_c / d->groups; a.coutG = d->out_c / d->groups;
     a.taps = d->ksize * d->ksize; a.ksize = d->ksize; a.stride = d->stride; a.pad = d->pad; a.dil = d->dilation;
     a.P = d->batch * d->out_h * d->out_w;
+    a.patchOk = (d->ksize == 3 && d->stride == 1 && d->pad == 1 && d->dilation == 1 && d->groups == 1 && d->out_h == d->in_h && d->out_w == d->in_w) ? 1 : 0;
+    a.patchRows = 0; a.mTiles = 0; a.cChunks = 0; a.nIter = 0;
+    a.dryRun = dryRun ? 1 : 0;
     a.act = d->act; a.act2 = d->act2; a.hasRes = (d->has_residual && residual) ? 1 : 0;
     a.actParam = d->act_param; a.act2Param = d->act2_param; a.resMul = d->res_mul; a.outMul = d->out_mul;
     const size_t outEl = dtypeSize(d->out_dtype);

@@ -32,6 +32,9 @@ struct IgemmArgs
     int cChunks;            // ceil(cinG / BK)
     int nIter;              // taps * cChunks
     int mTiles;             // ceil(coutG / BM)
+    int patchRows;          // patch kernel: input pixels staged per tile = BN + 2*W + 2
+    int patchOk;            // geometry is 3x3 stride 1 pad 1 dilation 1, ungrouped, same-size output
+    int dryRun;             // validate the tile for this shape, launch nothing
     int act, act2, hasRes, vecOk;
     float actParam, act2Param, resMul, outMul;
 };
@@ -54,6 +57,101 @@ __device__ __forceinline__ void mfmaBlock(const f32x4 &a, const f32x4 &b, f32x16
     c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[1], b[1], c, 0, 0, 0);
     c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2], b[2], c, 0, 0, 0);
     c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[3], b[3], c, 0, 0, 0);
+}
+
+// Shared epilogue of the GEMM-shaped convolution kernels:
+// 1. folded batch-norm / bias + activation on the float32 accumulators, in registers;
+// 2. each wavefront stages its TM x TN sub-tile as float32 in LDS, pixel-major (the main loop's LDS is free after
+//    its last barrier), so that
+// 3. every lane then owns 8 consecutive channels of a pixel: 16-byte residual loads and output stores, 8 lanes
+//    covering a contiguous run of 64 channels.
+template <typename T, typename TOut, int TM, int TN>
+__device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[TM / 32][TN / 32], unsigned char *smemRaw, int m0, int p0,
+                                              int wm, int wn, int wave, int lane, int g)
+{
+    constexpr int MB = TM / 32;
+    constexpr int NB = TN / 32;
+    constexpr int LDE = TM + 4;                       // padded staging row (floats)
+    float *stage = reinterpret_cast<float *>(smemRaw) + wave * (TN * LDE);
+    const int chBase = g * a.coutG;
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                const int ml = i * 32 + q * 8 + (lane >> 5) * 4;           // channel inside the wave tile
+                const int m = m0 + wm * TM + ml;
+                f32x4 v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                {
+                    const int ch = chBase + m + e;
+                    const bool ok = m + e < a.coutG;
+                    const float sc = (ok && a.scale) ? a.scale[ch] : 1.f;
+                    const float sh = (ok && a.shift) ? a.shift[ch] : 0.f;
+                    v[e] = activate(acc[i][j][q * 4 + e] * sc + sh, a.act, a.actParam);
+                }
+                *reinterpret_cast<f32x4 *>(stage + (j * 32 + (lane & 31)) * LDE + ml) = v;
+            }
+    __syncthreads();
+
+    const T *resg = static_cast<const T *>(a.res);
+    TOut    *yg   = static_cast<TOut *>(a.y);
+    constexpr int VPR = TM / 8;                       // 8-channel vectors per staged row
+    constexpr int RPI = 64 / VPR;                     // rows covered per pass of the wave
+    const int vcol = (lane % VPR) * 8;
+    const int mv   = m0 + wm * TM + vcol;             // first channel of this lane's vector (within the group)
+    if (mv < a.coutG)
+    {
+        const bool full = a.vecOk && (mv + 7 < a.coutG);
+#pragma unroll
+        for (int t = 0; t < TN / RPI; ++t)
+        {
+            const int row = t * RPI + lane / VPR;
+            const int p = p0 + wn * TN + row;
+            if (p >= a.P) continue;
+            float v[8];
+            const f32x4 lo = *reinterpret_cast<const f32x4 *>(stage + row * LDE + vcol);
+            const f32x4 hi = *reinterpret_cast<const f32x4 *>(stage + row * LDE + vcol + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[4 + e] = hi[e]; }
+            const size_t ch = static_cast<size_t>(chBase + mv);
+            if (a.hasRes)
+            {
+                const T *rp = resg + static_cast<size_t>(p) * a.resLd + ch;
+                if (full)
+                {
+                    typedef T ResV __attribute__((ext_vector_type(8)));
+                    const ResV r = *reinterpret_cast<const ResV *>(rp);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[e] = activate(v[e] + a.resMul * toF(r[e]), a.act2, a.act2Param);
+                }
+                else
+                {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (mv + e < a.coutG) v[e] = activate(v[e] + a.resMul * toF(rp[e]), a.act2, a.act2Param);
+                }
+            }
+            TOut *yp = yg + static_cast<size_t>(p) * a.outLd + ch;
+            if (full)
+            {
+                typedef TOut OutV __attribute__((ext_vector_type(8)));
+                OutV o;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = fromF<TOut>(a.outMul * v[e]);
+                *reinterpret_cast<OutV *>(yp) = o;
+            }
+            else
+            {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (mv + e < a.coutG) yp[e] = fromF<TOut>(a.outMul * v[e]);
+            }
+        }
+    }
 }
 
 template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN>
@@ -210,93 +308,7 @@ __global__ __launch_bounds__(256) void convIgemmKernel(IgemmArgs a)
         __syncthreads();
     }
 
-    // ---- epilogue -------------------------------------------------------------------------------------
-    // 1. folded batch-norm / bias + activation on the float32 accumulators, in registers;
-    // 2. each wavefront stages its TM x TN sub-tile as float32 in LDS, pixel-major (the main loop's LDS is free
-    //    after its last barrier), so that
-    // 3. every lane then owns 8 consecutive channels of a pixel: 16-byte residual loads and output stores,
-    //    8 lanes covering a contiguous run of 64 channels.
-    constexpr int LDE = TM + 4;                       // padded staging row (floats)
-    float *stage = reinterpret_cast<float *>(smemRaw) + wave * (TN * LDE);
-    const int chBase = g * a.coutG;
-#pragma unroll
-    for (int j = 0; j < NB; ++j)
-#pragma unroll
-        for (int i = 0; i < MB; ++i)
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-            {
-                const int ml = i * 32 + q * 8 + (lane >> 5) * 4;           // channel inside the wave tile
-                const int m = m0 + wm * TM + ml;
-                f32x4 v;
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                {
-                    const int ch = chBase + m + e;
-                    const bool ok = m + e < a.coutG;
-                    const float sc = (ok && a.scale) ? a.scale[ch] : 1.f;
-                    const float sh = (ok && a.shift) ? a.shift[ch] : 0.f;
-                    v[e] = activate(acc[i][j][q * 4 + e] * sc + sh, a.act, a.actParam);
-                }
-                *reinterpret_cast<f32x4 *>(stage + (j * 32 + (lane & 31)) * LDE + ml) = v;
-            }
-    __syncthreads();
-
-    const T *resg = static_cast<const T *>(a.res);
-    TOut    *yg   = static_cast<TOut *>(a.y);
-    constexpr int VPR = TM / 8;                       // 8-channel vectors per staged row
-    constexpr int RPI = 64 / VPR;                     // rows covered per pass of the wave
-    const int vcol = (lane % VPR) * 8;
-    const int mv   = m0 + wm * TM + vcol;             // first channel of this lane's vector (within the group)
-    if (mv < a.coutG)
-    {
-        const bool full = a.vecOk && (mv + 7 < a.coutG);
-#pragma unroll
-        for (int t = 0; t < TN / RPI; ++t)
-        {
-            const int row = t * RPI + lane / VPR;
-            const int p = p0 + wn * TN + row;
-            if (p >= a.P) continue;
-            float v[8];
-            const f32x4 lo = *reinterpret_cast<const f32x4 *>(stage + row * LDE + vcol);
-            const f32x4 hi = *reinterpret_cast<const f32x4 *>(stage + row * LDE + vcol + 4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[4 + e] = hi[e]; }
-            const size_t ch = static_cast<size_t>(chBase + mv);
-            if (a.hasRes)
-            {
-                const T *rp = resg + static_cast<size_t>(p) * a.resLd + ch;
-                if (full)
-                {
-                    typedef T ResV __attribute__((ext_vector_type(8)));
-                    const ResV r = *reinterpret_cast<const ResV *>(rp);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) v[e] = activate(v[e] + a.resMul * toF(r[e]), a.act2, a.act2Param);
-                }
-                else
-                {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (mv + e < a.coutG) v[e] = activate(v[e] + a.resMul * toF(rp[e]), a.act2, a.act2Param);
-                }
-            }
-            TOut *yp = yg + static_cast<size_t>(p) * a.outLd + ch;
-            if (full)
-            {
-                typedef TOut OutV __attribute__((ext_vector_type(8)));
-                OutV o;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) o[e] = fromF<TOut>(a.outMul * v[e]);
-                *reinterpret_cast<OutV *>(yp) = o;
-            }
-            else
-            {
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (mv + e < a.coutG) yp[e] = fromF<TOut>(a.outMul * v[e]);
-            }
-        }
-    }
+    igemmEpilogue<T, TOut, TM, TN>(a, acc, smemRaw, m0, p0, wm, wn, wave, lane, g);
 }
 
 template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN>
@@ -313,6 +325,7 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
     a.mTiles = (a.coutG + BM - 1) / BM;
     const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
     dim3 grid((tiles + 7) / 8 * 8, 1, groups);
+    if (a.dryRun) return 0;
     auto kern = convIgemmKernel<T, TOut, BM, BN, KV, WM, WN>;
     if (smem > 48 * 1024)
     {
@@ -325,10 +338,16 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
     return 0;
 }
 
+} // namespace msnh
+
+#include "conv_patch.hpp"
+
+namespace msnh {
+
 // Tile configurations (BM x BN output tile, KV 16-byte vectors of K per step, WM x WN wavefront grid).
 // Index 0 is "choose for me"; the others can be forced through msnh_conv_desc::tile, which is how the host
 // library's per-layer search picks the fastest one at load time.
-constexpr int kIgemmTiles = 13;
+constexpr int kIgemmTiles = 19;
 
 template <typename T, typename TOut>
 int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
@@ -348,6 +367,13 @@ int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
     case 11: return launchIgemm<T, TOut, 64, 128, 4, 1, 4>(a, groups, st);
     case 12: return launchIgemm<T, TOut, 64, 64, 8, 2, 2>(a, groups, st);
     case 13: return launchIgemm<T, TOut, 256, 128, 8, 2, 2>(a, groups, st);
+    // 3x3 stride-1 pad-1 only: input patch resident in LDS, weights streamed per tap
+    case 14: return launchPatch<T, TOut, 128, 128, 8, 2, 2>(a, groups, st);
+    case 15: return launchPatch<T, TOut, 128, 128, 4, 2, 2>(a, groups, st);
+    case 16: return launchPatch<T, TOut, 64, 128, 8, 1, 4>(a, groups, st);
+    case 17: return launchPatch<T, TOut, 64, 128, 4, 1, 4>(a, groups, st);
+    case 18: return launchPatch<T, TOut, 256, 128, 4, 2, 2>(a, groups, st);
+    case 19: return launchPatch<T, TOut, 128, 64, 8, 2, 2>(a, groups, st);
     default: break;
     }
     setError("igemm: unknown tile %d", tile);

@@ -427,6 +427,10 @@ void Plan::tuneConvs(msnh_stream_t s)
         for (int tile = 0; tile <= nTiles; ++tile)
         {
             op.tile = tile;
+            {
+                const msnh_conv_desc probe = convDesc(*this, op);
+                if (!msnh_hip_conv2d_tile_supported(&probe, tile)) continue;
+            }
             const int reps = 3;
             launch(op, s);                                       // warm-up (also surfaces launch errors for this tile)
             MSNH_DEV(msnh_hip_event_record(e0, s));

@@ -96,10 +96,45 @@ def test_conv_every_tile_configuration(dtype):
     ref = _ref(x, wt, 1, 1, 1, 1, None, None, "leaky", 0.1, res, "none", 1.0, 1.0)
     n = abi.lib().msnh_hip_conv2d_tile_count()
     assert n >= 1
+    ran = 0
     for tile in range(1, n + 1):
         print("tile", tile, dtype, flush=True)
-        y, _ = gu.conv2d(x, wt, dtype=dtype, stride=1, pad=1, act="leaky", residual=res, algo="igemm", tile=tile)
+        try:
+            y, _ = gu.conv2d(x, wt, dtype=dtype, stride=1, pad=1, act="leaky", residual=res, algo="igemm", tile=tile)
+        except abi.HipError as e:
+            assert "this tile needs" in str(e)
+            continue
+        ran += 1
         assert gu.rel_err(y, ref) <= TOL[dtype], tile
+    assert ran >= 16            # 3x3 stride 1: the LDS-patch configurations apply too
+
+
+@pytest.mark.parametrize("dtype", [abi.F32, abi.F16])
+@pytest.mark.parametrize("shape", [(2, 16, 19, 19, 40), (1, 64, 38, 38, 96), (3, 8, 7, 5, 16), (1, 32, 76, 76, 64), (2, 72, 13, 11, 136)])
+def test_conv_patch_tiles(shape, dtype):
+    """3x3 stride-1 layers with the input patch resident in LDS: image borders, batch seams, ragged channel chunks"""
+    import ctypes
+    import gpuutil as gu
+    gu.init()
+    b, c, h, w, oc = shape
+    rng = np.random.default_rng(sum(shape))
+    x, wt = _case(rng, b, c, h, w, oc, 3)
+    scale = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    shift = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    if dtype == abi.F16:
+        x, wt = gu.round_f16(x), gu.round_f16(wt)
+    ref = _ref(x, wt, 1, 1, 1, 1, scale, shift, "leaky", 0.1, None, "none", 1.0, 1.0)
+    ran = 0
+    for tile in range(14, abi.lib().msnh_hip_conv2d_tile_count() + 1):
+        print("patch tile", tile, shape, dtype, flush=True)
+        try:
+            y, _ = gu.conv2d(x, wt, dtype=dtype, stride=1, pad=1, scale=scale, shift=shift, act="leaky", algo="igemm", tile=tile)
+        except abi.HipError as e:
+            assert "this tile needs" in str(e)
+            continue
+        ran += 1
+        assert gu.rel_err(y, ref) <= TOL[dtype], tile
+    assert ran >= 3
 
 
 def test_conv_f16_in_f32_out():
