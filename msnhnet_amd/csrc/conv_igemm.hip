@@ -30,6 +30,15 @@ int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float
     a.patchOk = (d->ksize == 3 && d->stride == 1 && d->pad == 1 && d->dilation == 1 && d->groups == 1 && d->out_h == d->in_h && d->out_w == d->in_w) ? 1 : 0;
     a.patchRows = 0; a.mTiles = 0; a.cChunks = 0; a.nIter = 0;
     a.dryRun = dryRun ? 1 : 0;
+    {
+        const unsigned long long es = dtypeSize(d->dtype);
+        const unsigned long long xb = ((static_cast<unsigned long long>(d->batch) * d->in_h * d->in_w - 1) * d->in_ld + d->in_c) * es;
+        const unsigned long long wb = static_cast<unsigned long long>(d->out_c) * a.taps * a.cinG * es;
+        a.buffersOk = xb < 0x7fffffffull && wb < 0x7fffffffull;
+        a.xBytes = static_cast<unsigned>(xb);
+        a.wBytes = static_cast<unsigned>(wb);
+        a.ragged = 0;
+    }
     a.act = d->act; a.act2 = d->act2; a.hasRes = (d->has_residual && residual) ? 1 : 0;
     a.actParam = d->act_param; a.act2Param = d->act2_param; a.resMul = d->res_mul; a.outMul = d->out_mul;
     const size_t outEl = dtypeSize(d->out_dtype);

@@ -14,6 +14,7 @@
 // power-of-two output scale on the float32 accumulators and stores 4 consecutive channels per lane.
 #pragma once
 #include "common.hpp"
+#include <type_traits>
 
 namespace msnh {
 
@@ -35,6 +36,9 @@ struct IgemmArgs
     int patchRows;          // patch kernel: input pixels staged per tile = BN + 2*W + 2
     int patchOk;            // geometry is 3x3 stride 1 pad 1 dilation 1, ungrouped, same-size output
     int dryRun;             // validate the tile for this shape, launch nothing
+    unsigned xBytes, wBytes; // extent of the input tensor / packed weights in bytes (buffer resources; < 2 GiB)
+    int ragged;             // cinG is not a multiple of the tile's K step
+    int buffersOk;          // both extents fit a buffer resource
     int act, act2, hasRes, vecOk;
     float actParam, act2Param, resMul, outMul;
 };
@@ -59,99 +63,231 @@ __device__ __forceinline__ void mfmaBlock(const f32x4 &a, const f32x4 &b, f32x16
     c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[3], b[3], c, 0, 0, 0);
 }
 
-// Shared epilogue of the GEMM-shaped convolution kernels:
-// 1. folded batch-norm / bias + activation on the float32 accumulators, in registers;
-// 2. each wavefront stages its TM x TN sub-tile as float32 in LDS, pixel-major (the main loop's LDS is free after
-//    its last barrier), so that
-// 3. every lane then owns 8 consecutive channels of a pixel: 16-byte residual loads and output stores, 8 lanes
-//    covering a contiguous run of 64 channels.
-template <typename T, typename TOut, int TM, int TN>
-__device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[TM / 32][TN / 32], unsigned char *smemRaw, int m0, int p0,
-                                              int wm, int wn, int wave, int lane, int g)
+// 16-byte load through a buffer resource: the address is base + voffset + soffset with a hardware range check of
+// voffset against the resource size, so a lane whose row, tap or channel falls outside the tensor simply carries an
+// out-of-range voffset and reads zeros -- no branches, no 64-bit address arithmetic in the loop.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+constexpr unsigned kOobOffset = 0x80000000u;      // beyond any resource this kernel accepts (sizes are < 2 GiB)
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t makeRsrc(const void *base, unsigned bytes)
 {
-    constexpr int MB = TM / 32;
-    constexpr int NB = TN / 32;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+template <typename V> __device__ __forceinline__ V bufferLoad16(__amdgpu_buffer_rsrc_t r, unsigned voffset, unsigned soffset)
+{
+    const i32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, static_cast<int>(voffset), static_cast<int>(soffset), 0);
+    return __builtin_bit_cast(V, v);
+}
+
+// Shared epilogue of the GEMM-shaped convolution kernels.  Nothing in it waits on a global load issued inside it
+// except the residual, and that one is issued a whole staging pass ahead:
+// 1. the per-channel affine (folded batch-norm / bias) was fetched before the main loop, one channel per thread,
+//    and is now spread through LDS;
+// 2. per 32-pixel column block the wavefront applies affine + activation on its float32 accumulators and stages
+//    them pixel-major in LDS (the main loop's LDS is free after its last barrier), so that
+// 3. every lane then owns 8 consecutive channels of a pixel: 16-byte residual loads and output stores through
+//    range-checked buffer resources (pixels past the end of the tensor are dropped by the hardware), the lanes of
+//    a pixel covering a contiguous run of channels.
+template <typename T> struct Raw8;               // 8 consecutive elements as loaded / stored
+template <> struct Raw8<f16>
+{
+    i32x4 r[1];
+    __device__ __forceinline__ void toFloat(float (&v)[8]) const
+    {
+        const f16x8 h = __builtin_bit_cast(f16x8, r[0]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = static_cast<float>(h[e]);
+    }
+    __device__ __forceinline__ void fromFloat(const float (&v)[8])
+    {
+        f16x8 h;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) h[e] = static_cast<f16>(v[e]);
+        r[0] = __builtin_bit_cast(i32x4, h);
+    }
+};
+template <> struct Raw8<float>
+{
+    i32x4 r[2];
+    __device__ __forceinline__ void toFloat(float (&v)[8]) const
+    {
+        const f32x4 lo = __builtin_bit_cast(f32x4, r[0]), hi = __builtin_bit_cast(f32x4, r[1]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[4 + e] = hi[e]; }
+    }
+    __device__ __forceinline__ void fromFloat(const float (&v)[8])
+    {
+        f32x4 lo, hi;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { lo[e] = v[e]; hi[e] = v[4 + e]; }
+        r[0] = __builtin_bit_cast(i32x4, lo);
+        r[1] = __builtin_bit_cast(i32x4, hi);
+    }
+};
+
+template <typename T> __device__ __forceinline__ Raw8<T> bufferLoad8(__amdgpu_buffer_rsrc_t rs, unsigned voffset)
+{
+    Raw8<T> o;
+#pragma unroll
+    for (int h = 0; h < static_cast<int>(sizeof(T)) / 2; ++h)
+        o.r[h] = __builtin_amdgcn_raw_buffer_load_b128(rs, static_cast<int>(voffset + 16 * h), 0, 0);
+    return o;
+}
+
+template <typename T> __device__ __forceinline__ void bufferStore8(const Raw8<T> &o, __amdgpu_buffer_rsrc_t rs, unsigned voffset)
+{
+#pragma unroll
+    for (int h = 0; h < static_cast<int>(sizeof(T)) / 2; ++h)
+        __builtin_amdgcn_raw_buffer_store_b128(o.r[h], rs, static_cast<int>(voffset + 16 * h), 0, 0);
+}
+
+// The affine of channel m0 + tid of group g, fetched by thread tid ahead of the main loop.
+__device__ __forceinline__ void loadChannelAffine(const IgemmArgs &a, int g, int m0, int tid, int bm, float &sc, float &sh)
+{
+    sc = 1.f;
+    sh = 0.f;
+    const int m = m0 + tid;
+    if (tid < bm && m < a.coutG)
+    {
+        if (a.scale) sc = a.scale[g * a.coutG + m];
+        if (a.shift) sh = a.shift[g * a.coutG + m];
+    }
+}
+
+// relu, leaky and identity are x > 0 ? x : slope * x with slope 0, param, 1
+__device__ __forceinline__ bool actIsSlope(int act, float param, float &slope)
+{
+    slope = act == MSNH_ACT_LEAKY ? param : (act == MSNH_ACT_RELU ? 0.f : 1.f);
+    return act == MSNH_ACT_LEAKY || act == MSNH_ACT_RELU || act == MSNH_ACT_NONE;
+}
+
+template <bool SLOPE> __device__ __forceinline__ float activateSel(float x, float slope, int act, float param)
+{
+    if (SLOPE) return x > 0.f ? x : slope * x;
+    return activate(x, act, param);
+}
+
+// Loop whose index is a compile-time constant in the body (accumulator arrays must never be indexed dynamically,
+// or they are demoted from registers to scratch memory).
+template <int I, int N, typename F> __device__ __forceinline__ void staticFor(F &&f)
+{
+    if constexpr (I < N)
+    {
+        f(std::integral_constant<int, I>());
+        staticFor<I + 1, N>(f);
+    }
+}
+
+template <int BM, int TM> constexpr size_t igemmEpilogueLds() { return (2 * BM + 4 * 32 * (TM + 4)) * sizeof(float); }
+
+template <typename T, typename TOut, int BM, int BN, int TM, int TN>
+__device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[TM / 32][TN / 32], unsigned char *smemRaw, float chScale,
+                                              float chShift, int m0, int p0, int wm, int wn, int wave, int lane, int g)
+{
+    constexpr int MB  = TM / 32;
+    constexpr int NB  = TN / 32;
     constexpr int LDE = TM + 4;                       // padded staging row (floats)
-    float *stage = reinterpret_cast<float *>(smemRaw) + wave * (TN * LDE);
-    const int chBase = g * a.coutG;
-#pragma unroll
-    for (int j = 0; j < NB; ++j)
-#pragma unroll
-        for (int i = 0; i < MB; ++i)
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-            {
-                const int ml = i * 32 + q * 8 + (lane >> 5) * 4;           // channel inside the wave tile
-                const int m = m0 + wm * TM + ml;
-                f32x4 v;
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                {
-                    const int ch = chBase + m + e;
-                    const bool ok = m + e < a.coutG;
-                    const float sc = (ok && a.scale) ? a.scale[ch] : 1.f;
-                    const float sh = (ok && a.shift) ? a.shift[ch] : 0.f;
-                    v[e] = activate(acc[i][j][q * 4 + e] * sc + sh, a.act, a.actParam);
-                }
-                *reinterpret_cast<f32x4 *>(stage + (j * 32 + (lane & 31)) * LDE + ml) = v;
-            }
+    constexpr int VPR = TM / 8;                       // lanes (8-channel vectors) per staged pixel
+    constexpr int RPI = 64 / VPR;                     // pixels covered per pass of the wave
+    constexpr int PASSES = 32 / RPI;
+    static_assert(BM <= 256 && VPR <= 32, "epilogue geometry");
+    float *ss    = reinterpret_cast<float *>(smemRaw);                 // [BM] scale, [BM] shift
+    float *stage = ss + 2 * BM + wave * (32 * LDE);
+    const int tid = wave * 64 + lane;
+    if (tid < BM) { ss[tid] = chScale; ss[BM + tid] = chShift; }
     __syncthreads();
 
-    const T *resg = static_cast<const T *>(a.res);
-    TOut    *yg   = static_cast<TOut *>(a.y);
-    constexpr int VPR = TM / 8;                       // 8-channel vectors per staged row
-    constexpr int RPI = 64 / VPR;                     // rows covered per pass of the wave
+    const int chBase = g * a.coutG;
     const int vcol = (lane % VPR) * 8;
     const int mv   = m0 + wm * TM + vcol;             // first channel of this lane's vector (within the group)
-    if (mv < a.coutG)
-    {
-        const bool full = a.vecOk && (mv + 7 < a.coutG);
-#pragma unroll
-        for (int t = 0; t < TN / RPI; ++t)
+    const bool chOk = mv < a.coutG;
+    const bool full = a.vecOk && (mv + 7 < a.coutG);
+    const unsigned ch = static_cast<unsigned>(chBase + mv);
+    const int npix = min(a.P - p0, BN);
+    TOut    *yBlock = static_cast<TOut *>(a.y) + static_cast<size_t>(p0) * a.outLd;
+    const T *rBlock = static_cast<const T *>(a.res) + static_cast<size_t>(p0) * a.resLd;
+    const __amdgpu_buffer_rsrc_t ry = makeRsrc(yBlock, static_cast<unsigned>(npix) * a.outLd * sizeof(TOut));
+    const __amdgpu_buffer_rsrc_t rr = makeRsrc(a.hasRes ? rBlock : nullptr, a.hasRes ? static_cast<unsigned>(npix) * a.resLd * sizeof(T) : 0u);
+    float slope1, slope2;
+    const bool lin1 = actIsSlope(a.act, a.actParam, slope1);
+    const bool lin2 = actIsSlope(a.act2, a.act2Param, slope2);
+
+    staticFor<0, NB>([&](auto jTag) {
+        constexpr int j = decltype(jTag)::value;
+        const int pixBase = wn * TN + j * 32;         // first pixel of this column block inside the tile
+        Raw8<T> resRaw[PASSES];
+        if (a.hasRes)
         {
-            const int row = t * RPI + lane / VPR;
-            const int p = p0 + wn * TN + row;
-            if (p >= a.P) continue;
-            float v[8];
-            const f32x4 lo = *reinterpret_cast<const f32x4 *>(stage + row * LDE + vcol);
-            const f32x4 hi = *reinterpret_cast<const f32x4 *>(stage + row * LDE + vcol + 4);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[4 + e] = hi[e]; }
-            const size_t ch = static_cast<size_t>(chBase + mv);
-            if (a.hasRes)
+            for (int t = 0; t < PASSES; ++t)
             {
-                const T *rp = resg + static_cast<size_t>(p) * a.resLd + ch;
-                if (full)
-                {
-                    typedef T ResV __attribute__((ext_vector_type(8)));
-                    const ResV r = *reinterpret_cast<const ResV *>(rp);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) v[e] = activate(v[e] + a.resMul * toF(r[e]), a.act2, a.act2Param);
-                }
-                else
-                {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (mv + e < a.coutG) v[e] = activate(v[e] + a.resMul * toF(rp[e]), a.act2, a.act2Param);
-                }
-            }
-            TOut *yp = yg + static_cast<size_t>(p) * a.outLd + ch;
-            if (full)
-            {
-                typedef TOut OutV __attribute__((ext_vector_type(8)));
-                OutV o;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) o[e] = fromF<TOut>(a.outMul * v[e]);
-                *reinterpret_cast<OutV *>(yp) = o;
-            }
-            else
-            {
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (mv + e < a.coutG) yp[e] = fromF<TOut>(a.outMul * v[e]);
+                const unsigned pl = pixBase + t * RPI + lane / VPR;
+                resRaw[t] = bufferLoad8<T>(rr, full ? (pl * a.resLd + ch) * static_cast<unsigned>(sizeof(T)) : kOobOffset);
             }
         }
-    }
+        auto stageBlock = [&](auto slopeTag) {
+            constexpr bool SL = decltype(slopeTag)::value;
+            staticFor<0, MB * 4>([&](auto iqTag) {
+                    constexpr int i = decltype(iqTag)::value / 4;
+                    constexpr int q = decltype(iqTag)::value % 4;
+                    const int ml = i * 32 + q * 8 + (lane >> 5) * 4;       // channel inside the wave tile
+                    const f32x4 sc = *reinterpret_cast<const f32x4 *>(ss + wm * TM + ml);
+                    const f32x4 sh = *reinterpret_cast<const f32x4 *>(ss + BM + wm * TM + ml);
+                    f32x4 v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = activateSel<SL>(acc[i][j][q * 4 + e] * sc[e] + sh[e], slope1, a.act, a.actParam);
+                    *reinterpret_cast<f32x4 *>(stage + (lane & 31) * LDE + ml) = v;
+            });
+        };
+        if (lin1) stageBlock(std::true_type()); else stageBlock(std::false_type());
+        __syncthreads();
+
+        auto storeBlock = [&](auto slopeTag) {
+            constexpr bool SL = decltype(slopeTag)::value;
+#pragma unroll
+            for (int t = 0; t < PASSES; ++t)
+            {
+                const int row = t * RPI + lane / VPR;
+                const unsigned pl = pixBase + row;
+                float v[8];
+                const f32x4 lo = *reinterpret_cast<const f32x4 *>(stage + row * LDE + vcol);
+                const f32x4 hi = *reinterpret_cast<const f32x4 *>(stage + row * LDE + vcol + 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { v[e] = lo[e]; v[4 + e] = hi[e]; }
+                if (full)
+                {
+                    if (a.hasRes)
+                    {
+                        float r[8];
+                        resRaw[t].toFloat(r);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) v[e] = activateSel<SL>(v[e] + a.resMul * r[e], slope2, a.act2, a.act2Param);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[e] *= a.outMul;
+                    Raw8<TOut> o;
+                    o.fromFloat(v);
+                    bufferStore8<TOut>(o, ry, (pl * a.outLd + ch) * static_cast<unsigned>(sizeof(TOut)));
+                }
+                else if (chOk && static_cast<int>(pl) < npix)
+                {
+                    const T *rp = rBlock + static_cast<size_t>(pl) * a.resLd + ch;
+                    TOut *yp = yBlock + static_cast<size_t>(pl) * a.outLd + ch;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (mv + e < a.coutG)
+                        {
+                            float o = v[e];
+                            if (a.hasRes) o = activateSel<SL>(o + a.resMul * toF(rp[e]), slope2, a.act2, a.act2Param);
+                            yp[e] = fromF<TOut>(a.outMul * o);
+                        }
+                }
+            }
+        };
+        if (lin2) storeBlock(std::true_type()); else storeBlock(std::false_type());
+        if (j + 1 < NB) __syncthreads();
+    });
 }
 
 template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN>
@@ -169,6 +305,7 @@ __global__ __launch_bounds__(256) void convIgemmKernel(IgemmArgs a)
     constexpr int MB    = TM / 32;
     constexpr int NB    = TN / 32;
     constexpr int KBLK  = KV / 2;                 // k-blocks per step
+    constexpr unsigned ES = sizeof(T);
     static_assert((BM % RPP == 0 || BM < RPP) && BN % RPP == 0, "tile rows must be a multiple of rows per pass");
     static_assert(TM % 32 == 0 && TN % 32 == 0 && WM * WN == 4, "wave grid");
 
@@ -194,78 +331,86 @@ __global__ __launch_bounds__(256) void convIgemmKernel(IgemmArgs a)
     const int m0   = (logical % a.mTiles) * BM;
     const int p0   = (logical / a.mTiles) * BN;
 
-    const T *xg = static_cast<const T *>(a.x) + static_cast<size_t>(g) * a.cinG;
-    const T *wg = static_cast<const T *>(a.w) + static_cast<size_t>(g) * a.coutG * a.taps * a.cinG;
+    const unsigned gx = static_cast<unsigned>(g) * a.cinG * ES;
+    const unsigned gw = static_cast<unsigned>(g) * a.coutG * a.taps * a.cinG * ES;
+    const __amdgpu_buffer_rsrc_t rx = makeRsrc(static_cast<const unsigned char *>(a.x) + gx, a.xBytes - gx);
+    const __amdgpu_buffer_rsrc_t rw = makeRsrc(static_cast<const unsigned char *>(a.w) + gw, a.wBytes - gw);
+
+    float chScale, chShift;
+    loadChannelAffine(a, g, m0, tid, BM, chScale, chShift);
 
     const int ldRow = tid / KV;
     const int ldVec = tid % KV;
 
-    // per-thread row metadata, fixed over the K loop
-    int    bIy0[BROWS], bIx0[BROWS];
-    size_t bBase[BROWS];
-    bool   bOk[BROWS];
+    // Per-thread row state, fixed over the K loop: byte offset of the row's first tap (may be "negative", it wraps
+    // back into range once a valid tap offset is added) and one bit per tap telling whether that tap lies inside
+    // the image for this output pixel.
+    unsigned bOff[BROWS];
+    unsigned long long bMask[BROWS];
 #pragma unroll
     for (int i = 0; i < BROWS; ++i)
     {
         const int p = p0 + ldRow + i * RPP;
-        bOk[i] = p < a.P;
-        const int pp = bOk[i] ? p : 0;
+        const bool ok = p < a.P;
+        const int pp = ok ? p : 0;
         const int ox = pp % a.OW;
         const int t  = pp / a.OW;
         const int oy = t % a.OH;
         const int b  = t / a.OH;
-        bIy0[i]  = oy * a.stride - a.pad;
-        bIx0[i]  = ox * a.stride - a.pad;
-        bBase[i] = static_cast<size_t>(b) * a.H * a.W;
+        const int iy0 = oy * a.stride - a.pad;
+        const int ix0 = ox * a.stride - a.pad;
+        const long long pix = (static_cast<long long>(b) * a.H + iy0) * a.W + ix0;
+        bOff[i] = static_cast<unsigned>((pix * a.inLd + ldVec * VEC) * static_cast<long long>(ES));
+        unsigned long long mask = 0;
+        if (ok)
+            for (int ki = 0; ki < a.ksize; ++ki)
+                for (int kj = 0; kj < a.ksize; ++kj)
+                {
+                    const int iy = iy0 + ki * a.dil, ix = ix0 + kj * a.dil;
+                    if (iy >= 0 && iy < a.H && ix >= 0 && ix < a.W) mask |= 1ull << (ki * a.ksize + kj);
+                }
+        bMask[i] = mask;
     }
-    size_t aBase[AROWS];
-    bool   aOk[AROWS];
+    unsigned aOff[AROWS];
 #pragma unroll
     for (int i = 0; i < AROWS; ++i)
     {
-        const int m = m0 + ldRow + i * RPP;
-        aOk[i]   = m < a.coutG && (ldRow + i * RPP) < BM;
-        aBase[i] = static_cast<size_t>(aOk[i] ? m : 0) * a.taps * a.cinG;
+        const int row = ldRow + i * RPP;
+        const int m = m0 + row;
+        aOff[i] = (m < a.coutG && row < BM) ? (static_cast<unsigned>(m) * a.taps * a.cinG + ldVec * VEC) * ES : kOobOffset;
     }
 
     V regA[AROWS], regB[BROWS];
+    unsigned bVoff[BROWS];                       // B offsets of the tap being loaded
 
-    auto loadGlobal = [&](int it) {
-        const int tap = it / a.cChunks;
-        const int c   = (it - tap * a.cChunks) * BK + ldVec * VEC;
-        const bool cOk = c < a.cinG;
+    auto setTap = [&](int tap) {
         const int ki = tap / a.ksize;
         const int kj = tap - ki * a.ksize;
+        const unsigned tapOff = static_cast<unsigned>((ki * a.dil * a.W + kj * a.dil) * a.inLd) * ES;
 #pragma unroll
-        for (int i = 0; i < AROWS; ++i)
-        {
-            V v = {0};
-            if (aOk[i] && cOk)
-                v = *reinterpret_cast<const V *>(wg + aBase[i] + static_cast<size_t>(tap) * a.cinG + c);
-            regA[i] = v;
-        }
+        for (int i = 0; i < BROWS; ++i) bVoff[i] = ((bMask[i] >> tap) & 1ull) ? bOff[i] + tapOff : kOobOffset;
+    };
+    // loads step (tap, chunk); `ragged` (cinG not a multiple of BK) additionally blanks lanes past the last channel
+    auto loadGlobal = [&](int tap, int chunk) {
+        const unsigned sA = (static_cast<unsigned>(tap) * a.cinG + chunk * BK) * ES;
+        const unsigned sB = static_cast<unsigned>(chunk * BK) * ES;
+        const bool cut = a.ragged && (chunk * BK + ldVec * VEC >= a.cinG);
 #pragma unroll
-        for (int i = 0; i < BROWS; ++i)
-        {
-            const int iy = bIy0[i] + ki * a.dil;
-            const int ix = bIx0[i] + kj * a.dil;
-            V v = {0};
-            if (bOk[i] && cOk && iy >= 0 && iy < a.H && ix >= 0 && ix < a.W)
-                v = *reinterpret_cast<const V *>(xg + (bBase[i] + static_cast<size_t>(iy) * a.W + ix) * a.inLd + c);
-            regB[i] = v;
-        }
+        for (int i = 0; i < AROWS; ++i) regA[i] = bufferLoad16<V>(rw, cut ? kOobOffset : aOff[i], sA);
+#pragma unroll
+        for (int i = 0; i < BROWS; ++i) regB[i] = bufferLoad16<V>(rx, cut ? kOobOffset : bVoff[i], sB);
     };
 
+    T *aDst = As + ldRow * LDK + ldVec * VEC;
+    T *bDst = Bs + ldRow * LDK + ldVec * VEC;
     auto storeLds = [&](int buf) {
-        T *ad = As + buf * BM * LDK;
-        T *bd = Bs + buf * BN * LDK;
 #pragma unroll
         for (int i = 0; i < AROWS; ++i)
             if (BM % RPP == 0 || ldRow + i * RPP < BM)
-                *reinterpret_cast<V *>(ad + (ldRow + i * RPP) * LDK + ldVec * VEC) = regA[i];
+                *reinterpret_cast<V *>(aDst + (buf * BM + i * RPP) * LDK) = regA[i];
 #pragma unroll
         for (int i = 0; i < BROWS; ++i)
-            *reinterpret_cast<V *>(bd + (ldRow + i * RPP) * LDK + ldVec * VEC) = regB[i];
+            *reinterpret_cast<V *>(bDst + (buf * BN + i * RPP) * LDK) = regB[i];
     };
 
     f32x16 acc[MB][NB];
@@ -276,20 +421,29 @@ __global__ __launch_bounds__(256) void convIgemmKernel(IgemmArgs a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    loadGlobal(0);
+    int tapNext = 0, chunkNext = 0;              // the step whose loads are issued next
+    setTap(0);
+    loadGlobal(0, 0);
     storeLds(0);
     __syncthreads();
 
     const int fragRow = lane & 31;
     const int fragCol = (lane >> 5) * VEC;
+    const T *aFrag = As + (wm * TM + fragRow) * LDK + fragCol;
+    const T *bFrag = Bs + (wn * TN + fragRow) * LDK + fragCol;
 
     for (int it = 0; it < a.nIter; ++it)
     {
         const int buf = it & 1;
-        if (it + 1 < a.nIter) loadGlobal(it + 1);
+        const bool more = it + 1 < a.nIter;
+        if (more)
+        {
+            if (++chunkNext == a.cChunks) { chunkNext = 0; setTap(++tapNext); }
+            loadGlobal(tapNext, chunkNext);
+        }
 
-        const T *ab = As + buf * BM * LDK + (wm * TM + fragRow) * LDK + fragCol;
-        const T *bb = Bs + buf * BN * LDK + (wn * TN + fragRow) * LDK + fragCol;
+        const T *ab = aFrag + buf * BM * LDK;
+        const T *bb = bFrag + buf * BN * LDK;
 #pragma unroll
         for (int kb = 0; kb < KBLK; ++kb)
         {
@@ -304,11 +458,11 @@ __global__ __launch_bounds__(256) void convIgemmKernel(IgemmArgs a)
                 for (int j = 0; j < NB; ++j) mfmaBlock(fa[i], fb[j], acc[i][j]);
         }
 
-        if (it + 1 < a.nIter) storeLds(buf ^ 1);
+        if (more) storeLds(buf ^ 1);
         __syncthreads();
     }
 
-    igemmEpilogue<T, TOut, TM, TN>(a, acc, smemRaw, m0, p0, wm, wn, wave, lane, g);
+    igemmEpilogue<T, TOut, BM, BN, TM, TN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, wave, lane, g);
 }
 
 template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN>
@@ -319,8 +473,14 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
     constexpr int LDK = BK + VEC;
     a.cChunks = (a.cinG + BK - 1) / BK;
     a.nIter   = a.taps * a.cChunks;
+    a.ragged  = (a.cinG % BK) != 0;
+    if (a.taps > 64 || !a.buffersOk)
+    {
+        setError("conv2d: the implicit GEMM needs at most 64 filter taps and tensors below 2 GiB");
+        return 3;
+    }
     const size_t smemLoop = static_cast<size_t>(2) * (BM + BN) * LDK * sizeof(T);
-    const size_t smemEpi  = static_cast<size_t>(4) * (BN / WN) * (BM / WM + 4) * sizeof(float);
+    const size_t smemEpi  = igemmEpilogueLds<BM, BM / WM>();
     const size_t smem = smemLoop > smemEpi ? smemLoop : smemEpi;
     a.mTiles = (a.coutG + BM - 1) / BM;
     const int tiles = a.mTiles * ((a.P + BN - 1) / BN);

@@ -47,6 +47,9 @@ __global__ __launch_bounds__(256) void convPatch3x3Kernel(IgemmArgs a)
     const int m0 = (logical % a.mTiles) * BM;
     const int p0 = (logical / a.mTiles) * BN;
 
+    float chScale, chShift;
+    loadChannelAffine(a, 0, m0, tid, BM, chScale, chShift);
+
     const T *xg = static_cast<const T *>(a.x);
     const T *wg = static_cast<const T *>(a.w);
     const int W = a.W, H = a.H;
@@ -183,7 +186,7 @@ __global__ __launch_bounds__(256) void convPatch3x3Kernel(IgemmArgs a)
         __syncthreads();
     }
 
-    igemmEpilogue<T, TOut, TM, TN>(a, acc, smemRaw, m0, p0, wm, wn, wave, lane, 0);
+    igemmEpilogue<T, TOut, BM, BN, TM, TN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, wave, lane, 0);
 }
 
 // Host-side check shared by launch and tile enumeration.
@@ -194,7 +197,7 @@ inline bool patchFits(const IgemmArgs &a, size_t *smemOut)
     constexpr int LDK = KV * VEC + VEC;
     const int R = BN + 2 * a.W + 2;
     const size_t loop = (static_cast<size_t>(2) * R + 2 * BM) * LDK * sizeof(T);
-    const size_t epi = static_cast<size_t>(4) * (BN / WN) * (BM / WM + 4) * sizeof(float);
+    const size_t epi = igemmEpilogueLds<BM, BM / WM>();
     const size_t smem = loop > epi ? loop : epi;
     if (smemOut) *smemOut = smem;
     const int sv = (R * KV + 7) / 8;
@@ -216,6 +219,7 @@ inline int launchPatch(IgemmArgs &a, int groups, hipStream_t st)
     a.patchRows = BN + 2 * a.W + 2;
     a.cChunks = (a.cinG + BK - 1) / BK;
     a.nIter   = 9 * a.cChunks;
+    a.ragged  = (a.cinG % BK) != 0;
     a.mTiles  = (a.coutG + BM - 1) / BM;
     const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
     dim3 grid((tiles + 7) / 8 * 8, 1, 1);
