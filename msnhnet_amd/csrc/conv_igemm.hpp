@@ -6,12 +6,14 @@
 //     k = (tap, channel); the B operand is gathered on the fly from the NHWC input: for one tap the
 //         cin_g channels of an input pixel are contiguous, so a 16-byte vector load per lane feeds the
 //         MFMA operand registers without any transposition.
-// A workgroup of 256 threads (4 wavefronts in a WM x WN grid) owns a BM x BN tile of D.  Per K step each
-// thread moves 16-byte vectors global -> registers -> LDS (two LDS buffers, one barrier per step) while
-// the wavefronts issue 32x32 MFMA blocks from the other buffer.  LDS rows are padded by 16 bytes so the
-// 128-bit fragment reads of 8 neighbouring lanes fall into distinct banks.
+// A workgroup of 256 threads (4 wavefronts in a WM x WN grid) owns a BM x BN tile of D.  Per K step every
+// wavefront issues 16-byte-per-lane buffer loads that deliver straight into LDS (no registers, no LDS store
+// instructions); three LDS stages rotate so that the loads run two steps ahead of the MFMAs, with one barrier
+// per step.  LDS rows are unpadded and XOR-swizzled so that both the 1 KiB deliveries and the 128-bit fragment
+// reads are bank-conflict free.  Lanes outside the image, the channel range or the tensor carry an out-of-range
+// offset and the hardware fills zeros.
 // The epilogue applies folded batch-norm / bias, activation, residual add + second activation and the
-// power-of-two output scale on the float32 accumulators and stores 4 consecutive channels per lane.
+// power-of-two output scale on the float32 accumulators and stores 8 consecutive channels per lane.
 #pragma once
 #include "common.hpp"
 #include <type_traits>
@@ -290,32 +292,68 @@ __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[
     });
 }
 
+// Register budget: two workgroups per CU (one wave of each per SIMD) so that one workgroup's barrier and epilogue
+// are covered by the other's MFMAs; smaller tiles get three or four.
+constexpr int igemmWavesPerSimd(int bm, int bn) { return bm * bn > 128 * 128 ? 2 : (bm * bn > 64 * 64 ? 3 : 4); }
+
+// 16-byte-per-lane load from a buffer resource straight into LDS: the 64 lanes of the wave fill 1 KiB starting at
+// ldsAddr (lane l at ldsAddr + 16 * l); lanes whose voffset is out of range store zeros.  No VGPRs and no LDS store
+// instructions are involved (the LDS store path moves a quarter of what the load path delivers).  Written as inline
+// assembly so that the compiler does not serialise later LDS reads of *other* stages behind it; completion is
+// awaited explicitly with dmaWait<N>() (at most N younger loads of this wave still in flight).
+__device__ __forceinline__ void dmaLoad16(i32x4 rsrc, unsigned voffset, unsigned soffset, unsigned ldsAddr)
+{
+    asm volatile("s_mov_b32 m0, %3\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voffset), "s"(rsrc), "s"(soffset), "s"(ldsAddr) : "memory");
+}
+
+template <int N> __device__ __forceinline__ void dmaWait()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+__device__ __forceinline__ i32x4 makeRsrcWords(const void *base, unsigned bytes)
+{
+    const unsigned long long p = reinterpret_cast<unsigned long long>(base);
+    i32x4 r;
+    r[0] = static_cast<int>(static_cast<unsigned>(p));
+    r[1] = static_cast<int>(static_cast<unsigned>(p >> 32) & 0xffffu);
+    r[2] = static_cast<int>(bytes);
+    r[3] = 0x00020000;
+    return r;
+}
+
+constexpr int kIgemmStages = 3;
+
 template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN>
-__global__ __launch_bounds__(256) void convIgemmKernel(IgemmArgs a)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(igemmWavesPerSimd(BM, BN), igemmWavesPerSimd(BM, BN))))
+void convIgemmKernel(IgemmArgs a)
 {
     typedef typename Frag<T>::V V;
     constexpr int VEC   = Frag<T>::VEC;
-    constexpr int BK    = KV * VEC;               // K elements per step
-    constexpr int LDK   = BK + VEC;               // padded LDS row (elements)
-    constexpr int RPP   = 256 / KV;               // rows loaded per pass
-    constexpr int AROWS = (BM + RPP - 1) / RPP;   // A rows per thread (BM < RPP: only some threads load A)
+    constexpr int BK    = KV * VEC;               // K elements per tile step
+    constexpr int RPP   = 256 / KV;               // rows loaded per pass of the workgroup
+    constexpr int AROWS = BM / RPP;               // A rows (16-byte chunks) per thread per tile step
     constexpr int BROWS = BN / RPP;               // B rows per thread
+    constexpr int NL    = AROWS + BROWS;          // loads per thread per tile step
     constexpr int TM    = BM / WM;                // wave tile
     constexpr int TN    = BN / WN;
     constexpr int MB    = TM / 32;
     constexpr int NB    = TN / 32;
-    constexpr int KBLK  = KV / 2;                 // k-blocks per step
+    constexpr int S     = KV / 2;                 // MFMA k-steps per tile step (one k-block = two 16-byte chunks)
     constexpr unsigned ES = sizeof(T);
-    static_assert((BM % RPP == 0 || BM < RPP) && BN % RPP == 0, "tile rows must be a multiple of rows per pass");
-    static_assert(TM % 32 == 0 && TN % 32 == 0 && WM * WN == 4, "wave grid");
+    constexpr int ROWB  = KV * 16;                // bytes per LDS row: unpadded
+    constexpr int SWDIV = 16 / KV;                // rows per 256 bytes of LDS
+    constexpr int A_BYTES = BM * ROWB;
+    constexpr unsigned STAGE = (BM + BN) * ROWB;  // one LDS stage: A rows, then B rows
+    static_assert(BM % RPP == 0 && BN % RPP == 0, "tile rows must be a multiple of rows per pass");
+    static_assert(TM % 32 == 0 && TN % 32 == 0 && WM * WN == 4 && S % 2 == 0, "wave grid");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smemRaw[];
-    T *As = reinterpret_cast<T *>(smemRaw);                       // [2][BM][LDK]
-    T *Bs = As + 2 * BM * LDK;                                    // [2][BN][LDK]
+    const unsigned ldsBase = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char *)smemRaw));
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm   = wave / WN;
     const int wn   = wave % WN;
     const int g    = blockIdx.z;
@@ -333,14 +371,18 @@ __global__ __launch_bounds__(256) void convIgemmKernel(IgemmArgs a)
 
     const unsigned gx = static_cast<unsigned>(g) * a.cinG * ES;
     const unsigned gw = static_cast<unsigned>(g) * a.coutG * a.taps * a.cinG * ES;
-    const __amdgpu_buffer_rsrc_t rx = makeRsrc(static_cast<const unsigned char *>(a.x) + gx, a.xBytes - gx);
-    const __amdgpu_buffer_rsrc_t rw = makeRsrc(static_cast<const unsigned char *>(a.w) + gw, a.wBytes - gw);
+    const i32x4 rx = makeRsrcWords(static_cast<const unsigned char *>(a.x) + gx, a.xBytes - gx);
+    const i32x4 rw = makeRsrcWords(static_cast<const unsigned char *>(a.w) + gw, a.wBytes - gw);
 
     float chScale, chShift;
     loadChannelAffine(a, g, m0, tid, BM, chScale, chShift);
 
+    // LDS layout of a stage: rows of KV 16-byte chunks without padding; chunk c of row r sits at chunk position
+    // c ^ ((r / SWDIV) % KV).  With that XOR the 16 lanes the LDS serves per cycle hit 16 different 16-byte bank
+    // groups when a wave reads one chunk column of 32 rows, while a wave's load fills 64 consecutive chunk
+    // positions.  Thread tid owns chunk position tid % KV of row tid / KV (+ RPP rows per pass): byte tid * 16.
     const int ldRow = tid / KV;
-    const int ldVec = tid % KV;
+    const int ldVec = (tid % KV) ^ ((ldRow / SWDIV) % KV);   // the logical chunk this thread fetches
 
     // Per-thread row state, fixed over the K loop: byte offset of the row's first tap (may be "negative", it wraps
     // back into range once a valid tap offset is added) and one bit per tap telling whether that tap lies inside
@@ -375,14 +417,11 @@ __global__ __launch_bounds__(256) void convIgemmKernel(IgemmArgs a)
 #pragma unroll
     for (int i = 0; i < AROWS; ++i)
     {
-        const int row = ldRow + i * RPP;
-        const int m = m0 + row;
-        aOff[i] = (m < a.coutG && row < BM) ? (static_cast<unsigned>(m) * a.taps * a.cinG + ldVec * VEC) * ES : kOobOffset;
+        const int m = m0 + ldRow + i * RPP;
+        aOff[i] = m < a.coutG ? (static_cast<unsigned>(m) * a.taps * a.cinG + ldVec * VEC) * ES : kOobOffset;
     }
 
-    V regA[AROWS], regB[BROWS];
     unsigned bVoff[BROWS];                       // B offsets of the tap being loaded
-
     auto setTap = [&](int tap) {
         const int ki = tap / a.ksize;
         const int kj = tap - ki * a.ksize;
@@ -390,27 +429,45 @@ __global__ __launch_bounds__(256) void convIgemmKernel(IgemmArgs a)
 #pragma unroll
         for (int i = 0; i < BROWS; ++i) bVoff[i] = ((bMask[i] >> tap) & 1ull) ? bOff[i] + tapOff : kOobOffset;
     };
-    // loads step (tap, chunk); `ragged` (cinG not a multiple of BK) additionally blanks lanes past the last channel
-    auto loadGlobal = [&](int tap, int chunk) {
+    // Issues the NL loads of tile step (tap, chunk) into the LDS stage at byte offset stageOff; `ragged` (cinG not
+    // a multiple of BK) additionally blanks lanes past the last channel.
+    const unsigned waveLds = ldsBase + wave * 1024;
+    auto issueLoads = [&](int tap, int chunk, unsigned stageOff) {
         const unsigned sA = (static_cast<unsigned>(tap) * a.cinG + chunk * BK) * ES;
         const unsigned sB = static_cast<unsigned>(chunk * BK) * ES;
         const bool cut = a.ragged && (chunk * BK + ldVec * VEC >= a.cinG);
 #pragma unroll
-        for (int i = 0; i < AROWS; ++i) regA[i] = bufferLoad16<V>(rw, cut ? kOobOffset : aOff[i], sA);
+        for (int i = 0; i < AROWS; ++i) dmaLoad16(rw, cut ? kOobOffset : aOff[i], sA, waveLds + stageOff + i * RPP * ROWB);
 #pragma unroll
-        for (int i = 0; i < BROWS; ++i) regB[i] = bufferLoad16<V>(rx, cut ? kOobOffset : bVoff[i], sB);
+        for (int i = 0; i < BROWS; ++i) dmaLoad16(rx, cut ? kOobOffset : bVoff[i], sB, waveLds + stageOff + A_BYTES + i * RPP * ROWB);
+    };
+    int tapNext = 0, chunkNext = 0;              // the tile step whose loads were issued last
+    auto issueNext = [&](unsigned stageOff) {
+        if (++chunkNext == a.cChunks) { chunkNext = 0; setTap(++tapNext); }
+        issueLoads(tapNext, chunkNext, stageOff);
     };
 
-    T *aDst = As + ldRow * LDK + ldVec * VEC;
-    T *bDst = Bs + ldRow * LDK + ldVec * VEC;
-    auto storeLds = [&](int buf) {
+    // fragment addresses: lane l feeds MFMA row l % 32 with chunk 2 * kb + l / 32 of k-step kb
+    const int fragRow = lane & 31;
+    const int fragSw  = (fragRow / SWDIV) % KV;
+    unsigned aAddr[S], bAddr[S];
 #pragma unroll
-        for (int i = 0; i < AROWS; ++i)
-            if (BM % RPP == 0 || ldRow + i * RPP < BM)
-                *reinterpret_cast<V *>(aDst + (buf * BM + i * RPP) * LDK) = regA[i];
+    for (int kb = 0; kb < S; ++kb)
+    {
+        const unsigned off = fragRow * ROWB + (((2 * kb + (lane >> 5)) ^ fragSw) * 16);
+        aAddr[kb] = wm * TM * ROWB + off;
+        bAddr[kb] = A_BYTES + wn * TN * ROWB + off;
+    }
+
+    V fa[2][MB], fb[2][NB];                      // fragments of k-step s live in buffer s % 2
+    auto readFrags = [&](unsigned stageOff, auto kbTag) {
+        constexpr int kb = decltype(kbTag)::value;
+        const unsigned char *ap = smemRaw + (aAddr[kb] + stageOff);
+        const unsigned char *bp = smemRaw + (bAddr[kb] + stageOff);
 #pragma unroll
-        for (int i = 0; i < BROWS; ++i)
-            *reinterpret_cast<V *>(bDst + (buf * BN + i * RPP) * LDK) = regB[i];
+        for (int i = 0; i < MB; ++i) fa[kb % 2][i] = *reinterpret_cast<const V *>(ap + i * 32 * ROWB);
+#pragma unroll
+        for (int j = 0; j < NB; ++j) fb[kb % 2][j] = *reinterpret_cast<const V *>(bp + j * 32 * ROWB);
     };
 
     f32x16 acc[MB][NB];
@@ -421,46 +478,58 @@ __global__ __launch_bounds__(256) void convIgemmKernel(IgemmArgs a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    int tapNext = 0, chunkNext = 0;              // the step whose loads are issued next
+    auto mfmaStep = [&](auto kbTag) {
+        constexpr int buf = decltype(kbTag)::value % 2;
+        staticFor<0, MB * NB>([&](auto ijTag) {
+            constexpr int i = decltype(ijTag)::value / NB;
+            constexpr int j = decltype(ijTag)::value % NB;
+            mfmaBlock(fa[buf][i], fb[buf][j], acc[i][j]);
+        });
+    };
+
+    // Three LDS stages rotate: while tile step `it` is multiplied out of stage `cur`, step it+1 is already (being)
+    // delivered into `nxt` and the loads of step it+2 are issued into `nn`, whose last readers all passed the
+    // previous barrier.  Inside a step the LDS reads for k-step s+1 are issued before the MFMAs of k-step s, and
+    // the single barrier sits before the last k-step, whose MFMAs cover the first fragment reads of step it+1.
     setTap(0);
-    loadGlobal(0, 0);
-    storeLds(0);
+    issueLoads(0, 0, 0);
+    if (a.nIter > 1)
+    {
+        issueNext(STAGE);
+        dmaWait<NL>();
+    }
+    else
+        dmaWait<0>();
     __syncthreads();
+    readFrags(0, std::integral_constant<int, 0>());
 
-    const int fragRow = lane & 31;
-    const int fragCol = (lane >> 5) * VEC;
-    const T *aFrag = As + (wm * TM + fragRow) * LDK + fragCol;
-    const T *bFrag = Bs + (wn * TN + fragRow) * LDK + fragCol;
-
+    unsigned cur = 0, nxt = STAGE, nn = 2 * STAGE;
     for (int it = 0; it < a.nIter; ++it)
     {
-        const int buf = it & 1;
-        const bool more = it + 1 < a.nIter;
-        if (more)
-        {
-            if (++chunkNext == a.cChunks) { chunkNext = 0; setTap(++tapNext); }
-            loadGlobal(tapNext, chunkNext);
-        }
-
-        const T *ab = aFrag + buf * BM * LDK;
-        const T *bb = bFrag + buf * BN * LDK;
-#pragma unroll
-        for (int kb = 0; kb < KBLK; ++kb)
-        {
-            V fa[MB], fb[NB];
-#pragma unroll
-            for (int i = 0; i < MB; ++i) fa[i] = *reinterpret_cast<const V *>(ab + i * 32 * LDK + kb * 2 * VEC);
-#pragma unroll
-            for (int j = 0; j < NB; ++j) fb[j] = *reinterpret_cast<const V *>(bb + j * 32 * LDK + kb * 2 * VEC);
-#pragma unroll
-            for (int i = 0; i < MB; ++i)
-#pragma unroll
-                for (int j = 0; j < NB; ++j) mfmaBlock(fa[i], fb[j], acc[i][j]);
-        }
-
-        if (more) storeLds(buf ^ 1);
-        __syncthreads();
+        const bool more1 = it + 1 < a.nIter;
+        const bool more2 = it + 2 < a.nIter;
+        readFrags(cur, std::integral_constant<int, 1>());
+        if (more2) issueNext(nn);
+        __builtin_amdgcn_sched_barrier(0);
+        mfmaStep(std::integral_constant<int, 0>());
+        staticFor<1, S - 1>([&](auto sTag) {
+            constexpr int s = decltype(sTag)::value;
+            readFrags(cur, std::integral_constant<int, s + 1>());
+            __builtin_amdgcn_sched_barrier(0);
+            mfmaStep(sTag);
+        });
+        __builtin_amdgcn_sched_barrier(0);
+        if (more2) dmaWait<NL>(); else dmaWait<0>();      // this wave's part of step it+1 has landed
+        __syncthreads();                                  // ... and everybody else's
+        if (more1) readFrags(nxt, std::integral_constant<int, 0>());
+        __builtin_amdgcn_sched_barrier(0);
+        mfmaStep(std::integral_constant<int, S - 1>());
+        const unsigned t = cur;
+        cur = nxt;
+        nxt = nn;
+        nn = t;
     }
+    __syncthreads();
 
     igemmEpilogue<T, TOut, BM, BN, TM, TN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, wave, lane, g);
 }
@@ -470,7 +539,6 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
 {
     constexpr int VEC = Frag<T>::VEC;
     constexpr int BK  = KV * VEC;
-    constexpr int LDK = BK + VEC;
     a.cChunks = (a.cinG + BK - 1) / BK;
     a.nIter   = a.taps * a.cChunks;
     a.ragged  = (a.cinG % BK) != 0;
@@ -479,7 +547,7 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
         setError("conv2d: the implicit GEMM needs at most 64 filter taps and tensors below 2 GiB");
         return 3;
     }
-    const size_t smemLoop = static_cast<size_t>(2) * (BM + BN) * LDK * sizeof(T);
+    const size_t smemLoop = static_cast<size_t>(kIgemmStages) * (BM + BN) * KV * 16;
     const size_t smemEpi  = igemmEpilogueLds<BM, BM / WM>();
     const size_t smem = smemLoop > smemEpi ? smemLoop : smemEpi;
     a.mTiles = (a.coutG + BM - 1) / BM;
@@ -519,14 +587,14 @@ int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
     case 3:  return launchIgemm<T, TOut, 64, 256, 8, 1, 4>(a, groups, st);
     case 4:  return launchIgemm<T, TOut, 64, 256, 4, 1, 4>(a, groups, st);
     case 5:  return launchIgemm<T, TOut, 32, 256, 8, 1, 4>(a, groups, st);
-    case 6:  return launchIgemm<T, TOut, 32, 256, 4, 1, 4>(a, groups, st);
+    case 6:  return launchIgemm<T, TOut, 64, 64, 4, 2, 2>(a, groups, st);
     case 7:  return launchIgemm<T, TOut, 256, 128, 4, 2, 2>(a, groups, st);
     case 8:  return launchIgemm<T, TOut, 128, 64, 8, 2, 2>(a, groups, st);
     case 9:  return launchIgemm<T, TOut, 128, 64, 4, 2, 2>(a, groups, st);
     case 10: return launchIgemm<T, TOut, 64, 128, 8, 1, 4>(a, groups, st);
     case 11: return launchIgemm<T, TOut, 64, 128, 4, 1, 4>(a, groups, st);
     case 12: return launchIgemm<T, TOut, 64, 64, 8, 2, 2>(a, groups, st);
-    case 13: return launchIgemm<T, TOut, 256, 128, 8, 2, 2>(a, groups, st);
+    case 13: return launchIgemm<T, TOut, 128, 256, 4, 2, 2>(a, groups, st);
     // 3x3 stride-1 pad-1 only: input patch resident in LDS, weights streamed per tap
     case 14: return launchPatch<T, TOut, 128, 128, 8, 2, 2>(a, groups, st);
     case 15: return launchPatch<T, TOut, 128, 128, 4, 2, 2>(a, groups, st);
