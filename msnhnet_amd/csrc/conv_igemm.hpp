@@ -322,9 +322,7 @@ __device__ __forceinline__ i32x4 makeRsrcWords(const void *base, unsigned bytes)
     return r;
 }
 
-constexpr int kIgemmStages = 3;
-
-template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN>
+template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int NS>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(igemmWavesPerSimd(BM, BN), igemmWavesPerSimd(BM, BN))))
 void convIgemmKernel(IgemmArgs a)
 {
@@ -347,6 +345,7 @@ void convIgemmKernel(IgemmArgs a)
     constexpr unsigned STAGE = (BM + BN) * ROWB;  // one LDS stage: A rows, then B rows
     static_assert(BM % RPP == 0 && BN % RPP == 0, "tile rows must be a multiple of rows per pass");
     static_assert(TM % 32 == 0 && TN % 32 == 0 && WM * WN == 4 && S % 2 == 0, "wave grid");
+    static_assert(NS >= 2 && NS <= 8, "LDS stages");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smemRaw[];
     const unsigned ldsBase = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char *)smemRaw));
@@ -429,22 +428,24 @@ void convIgemmKernel(IgemmArgs a)
 #pragma unroll
         for (int i = 0; i < BROWS; ++i) bVoff[i] = ((bMask[i] >> tap) & 1ull) ? bOff[i] + tapOff : kOobOffset;
     };
-    // Issues the NL loads of tile step (tap, chunk) into the LDS stage at byte offset stageOff; `ragged` (cinG not
-    // a multiple of BK) additionally blanks lanes past the last channel.
+    // Load l of a tile step (A rows first, then B rows) into the LDS stage at byte offset stageOff.  `cut` blanks
+    // the lane: past the last channel of a ragged K chunk, or a step past the end of K.
     const unsigned waveLds = ldsBase + wave * 1024;
-    auto issueLoads = [&](int tap, int chunk, unsigned stageOff) {
-        const unsigned sA = (static_cast<unsigned>(tap) * a.cinG + chunk * BK) * ES;
-        const unsigned sB = static_cast<unsigned>(chunk * BK) * ES;
-        const bool cut = a.ragged && (chunk * BK + ldVec * VEC >= a.cinG);
-#pragma unroll
-        for (int i = 0; i < AROWS; ++i) dmaLoad16(rw, cut ? kOobOffset : aOff[i], sA, waveLds + stageOff + i * RPP * ROWB);
-#pragma unroll
-        for (int i = 0; i < BROWS; ++i) dmaLoad16(rx, cut ? kOobOffset : bVoff[i], sB, waveLds + stageOff + A_BYTES + i * RPP * ROWB);
+    auto issueLoad = [&](auto lTag, unsigned sA, unsigned sB, bool cut, unsigned stageOff) {
+        constexpr int l = decltype(lTag)::value;
+        if constexpr (l < AROWS)
+            dmaLoad16(rw, cut ? kOobOffset : aOff[l], sA, waveLds + stageOff + l * RPP * ROWB);
+        else
+            dmaLoad16(rx, cut ? kOobOffset : bVoff[l - AROWS], sB, waveLds + stageOff + A_BYTES + (l - AROWS) * RPP * ROWB);
     };
     int tapNext = 0, chunkNext = 0;              // the tile step whose loads were issued last
-    auto issueNext = [&](unsigned stageOff) {
-        if (++chunkNext == a.cChunks) { chunkNext = 0; setTap(++tapNext); }
-        issueLoads(tapNext, chunkNext, stageOff);
+    unsigned sANext = 0, sBNext = 0;
+    bool cutNext = false;
+    auto advance = [&](bool pastEnd) {
+        if (++chunkNext == a.cChunks) { chunkNext = 0; ++tapNext; if (tapNext < a.taps) setTap(tapNext); }
+        sANext = (static_cast<unsigned>(tapNext) * a.cinG + chunkNext * BK) * ES;
+        sBNext = static_cast<unsigned>(chunkNext * BK) * ES;
+        cutNext = pastEnd || (a.ragged && (chunkNext * BK + ldVec * VEC >= a.cinG));
     };
 
     // fragment addresses: lane l feeds MFMA row l % 32 with chunk 2 * kb + l / 32 of k-step kb
@@ -478,63 +479,81 @@ void convIgemmKernel(IgemmArgs a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    auto mfmaStep = [&](auto kbTag) {
-        constexpr int buf = decltype(kbTag)::value % 2;
-        staticFor<0, MB * NB>([&](auto ijTag) {
-            constexpr int i = decltype(ijTag)::value / NB;
-            constexpr int j = decltype(ijTag)::value % NB;
-            mfmaBlock(fa[buf][i], fb[buf][j], acc[i][j]);
-        });
-    };
-
-    // Three LDS stages rotate: while tile step `it` is multiplied out of stage `cur`, step it+1 is already (being)
-    // delivered into `nxt` and the loads of step it+2 are issued into `nn`, whose last readers all passed the
-    // previous barrier.  Inside a step the LDS reads for k-step s+1 are issued before the MFMAs of k-step s, and
+    // NS >= 3 LDS stages rotate: while tile step `it` is multiplied out of stage `cur`, steps it+1 .. it+NS-2 are
+    // already (being) delivered into the following stages and the loads of step it+NS-1 go into the stage before
+    // `cur`, whose last readers all passed the previous barrier.  How far ahead the loads must run is set by
+    // Little's law: a CU has to keep (bytes per step) / (MFMA time per step) x (L2 latency) in flight, tens of KiB.
+    // The NL loads of a step are spread evenly between the step's MFMAs (issued back to back they fill the memory
+    // pipeline's queue and the wave, stuck on the issue, stops feeding the matrix core).
+    // NS = 2: step it+2 goes into `cur` itself, which is free once the barrier of step `it` is passed, so all NL
+    // loads follow that barrier, among the MFMAs of the last k-step, and must have landed by the next barrier.
+    // Steps past the end of K are issued all the same with every lane out of range, so the count of loads in
+    // flight is the same in every step.  LDS reads for k-step s+1 are issued before the MFMAs of k-step s, and
     // the single barrier sits before the last k-step, whose MFMAs cover the first fragment reads of step it+1.
+    constexpr int PER  = MB * NB;                // MFMAs per k-step
+    constexpr int TOT  = PER * S;                // MFMAs per tile step
+    // NS >= 3: load l follows MFMA number l * TOT / NL, NPRE of them ahead of the barrier (numbers < TOT - PER);
+    // NS = 2: load l follows MFMA number TOT - PER + l * PER / NL
+    constexpr int NPRE = NS >= 3 ? ((TOT - PER) * NL + TOT - 1) / TOT : 0;
+    constexpr int LBASE = NS >= 3 ? 0 : TOT - PER;
+    constexpr int LSPAN = NS >= 3 ? TOT : PER;
+    constexpr int AHEAD = NS >= 3 ? NS - 1 : 2;  // the loads issued during step `it` belong to step it + AHEAD
+    constexpr int INFLIGHT = NS >= 3 ? (NS - 3) * NL + NPRE : 0;   // loads younger than step it+1's at the barrier
+
     setTap(0);
-    issueLoads(0, 0, 0);
-    if (a.nIter > 1)
-    {
-        issueNext(STAGE);
-        dmaWait<NL>();
-    }
-    else
-        dmaWait<0>();
+    staticFor<0, NL>([&](auto lTag) { issueLoad(lTag, 0u, 0u, a.ragged && (ldVec * VEC >= a.cinG), 0u); });
+    staticFor<1, AHEAD>([&](auto stTag) {
+        constexpr int st = decltype(stTag)::value;
+        advance(a.nIter <= st);
+        staticFor<0, NL>([&](auto lTag) { issueLoad(lTag, sANext, sBNext, cutNext, st * STAGE); });
+    });
+    dmaWait<(AHEAD - 1) * NL>();                 // step 0 has landed
     __syncthreads();
     readFrags(0, std::integral_constant<int, 0>());
 
-    unsigned cur = 0, nxt = STAGE, nn = 2 * STAGE;
+    // cur: stage of step it; nxt: of step it+1; nn: where the loads issued during step it go
+    unsigned cur = 0, nxt = STAGE, nn = NS >= 3 ? (NS - 1) * STAGE : 0;
     for (int it = 0; it < a.nIter; ++it)
     {
-        const bool more1 = it + 1 < a.nIter;
-        const bool more2 = it + 2 < a.nIter;
+        advance(it + AHEAD >= a.nIter);          // sANext / sBNext / cutNext now describe step it + AHEAD
         readFrags(cur, std::integral_constant<int, 1>());
-        if (more2) issueNext(nn);
         __builtin_amdgcn_sched_barrier(0);
-        mfmaStep(std::integral_constant<int, 0>());
-        staticFor<1, S - 1>([&](auto sTag) {
-            constexpr int s = decltype(sTag)::value;
-            readFrags(cur, std::integral_constant<int, s + 1>());
+        staticFor<0, TOT>([&](auto gTag) {
+            constexpr int gi = decltype(gTag)::value;
+            constexpr int ks = gi / PER;
+            if constexpr (gi % PER == 0 && ks >= 1)
+            {
+                if constexpr (ks < S - 1)
+                    readFrags(cur, std::integral_constant<int, ks + 1>());
+                else
+                {
+                    dmaWait<INFLIGHT>();         // all of step it+1 has landed; younger loads may be in flight
+                    __syncthreads();
+                    readFrags(nxt, std::integral_constant<int, 0>());
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            mfmaBlock(fa[ks % 2][(gi % PER) / NB], fb[ks % 2][(gi % PER) % NB], acc[(gi % PER) / NB][(gi % PER) % NB]);
+            if constexpr (gi >= LBASE)
+            {
+                // loads l with LBASE + l * LSPAN / NL == gi
+                constexpr int first = ((gi - LBASE) * NL + LSPAN - 1) / LSPAN;
+                constexpr int last  = ((gi - LBASE + 1) * NL + LSPAN - 1) / LSPAN;
+                staticFor<first, last>([&](auto lTag) { issueLoad(lTag, sANext, sBNext, cutNext, nn); });
+            }
             __builtin_amdgcn_sched_barrier(0);
-            mfmaStep(sTag);
         });
-        __builtin_amdgcn_sched_barrier(0);
-        if (more2) dmaWait<NL>(); else dmaWait<0>();      // this wave's part of step it+1 has landed
-        __syncthreads();                                  // ... and everybody else's
-        if (more1) readFrags(nxt, std::integral_constant<int, 0>());
-        __builtin_amdgcn_sched_barrier(0);
-        mfmaStep(std::integral_constant<int, S - 1>());
-        const unsigned t = cur;
+        nn = NS >= 3 ? cur : nxt;
         cur = nxt;
-        nxt = nn;
-        nn = t;
+        nxt = nxt + STAGE == NS * STAGE ? 0u : nxt + STAGE;
     }
+    dmaWait<0>();
     __syncthreads();
 
     igemmEpilogue<T, TOut, BM, BN, TM, TN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, wave, lane, g);
 }
 
-template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN>
+template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int NS = 3>
 inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
 {
     constexpr int VEC = Frag<T>::VEC;
@@ -547,14 +566,14 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
         setError("conv2d: the implicit GEMM needs at most 64 filter taps and tensors below 2 GiB");
         return 3;
     }
-    const size_t smemLoop = static_cast<size_t>(kIgemmStages) * (BM + BN) * KV * 16;
+    const size_t smemLoop = static_cast<size_t>(NS) * (BM + BN) * KV * 16;
     const size_t smemEpi  = igemmEpilogueLds<BM, BM / WM>();
     const size_t smem = smemLoop > smemEpi ? smemLoop : smemEpi;
     a.mTiles = (a.coutG + BM - 1) / BM;
     const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
     dim3 grid((tiles + 7) / 8 * 8, 1, groups);
     if (a.dryRun) return 0;
-    auto kern = convIgemmKernel<T, TOut, BM, BN, KV, WM, WN>;
+    auto kern = convIgemmKernel<T, TOut, BM, BN, KV, WM, WN, NS>;
     if (smem > 48 * 1024)
     {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -575,7 +594,7 @@ namespace msnh {
 // Tile configurations (BM x BN output tile, KV 16-byte vectors of K per step, WM x WN wavefront grid).
 // Index 0 is "choose for me"; the others can be forced through msnh_conv_desc::tile, which is how the host
 // library's per-layer search picks the fastest one at load time.
-constexpr int kIgemmTiles = 19;
+constexpr int kIgemmTiles = 28;
 
 template <typename T, typename TOut>
 int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
@@ -595,13 +614,25 @@ int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
     case 11: return launchIgemm<T, TOut, 64, 128, 4, 1, 4>(a, groups, st);
     case 12: return launchIgemm<T, TOut, 64, 64, 8, 2, 2>(a, groups, st);
     case 13: return launchIgemm<T, TOut, 128, 256, 4, 2, 2>(a, groups, st);
-    // 3x3 stride-1 pad-1 only: input patch resident in LDS, weights streamed per tap
-    case 14: return launchPatch<T, TOut, 128, 128, 8, 2, 2>(a, groups, st);
-    case 15: return launchPatch<T, TOut, 128, 128, 4, 2, 2>(a, groups, st);
-    case 16: return launchPatch<T, TOut, 64, 128, 8, 1, 4>(a, groups, st);
-    case 17: return launchPatch<T, TOut, 64, 128, 4, 1, 4>(a, groups, st);
-    case 18: return launchPatch<T, TOut, 256, 128, 4, 2, 2>(a, groups, st);
-    case 19: return launchPatch<T, TOut, 128, 64, 8, 2, 2>(a, groups, st);
+    // 3x3 stride-1 pad-1 only: input patch resident in LDS, weights streamed per tap (last number: patch slices
+    // per wave and step, 2 for wide images)
+    case 14: return launchPatch<T, TOut, 128, 256, 4, 2, 2, 1>(a, groups, st);
+    case 15: return launchPatch<T, TOut, 128, 256, 4, 2, 2, 2>(a, groups, st);
+    case 16: return launchPatch<T, TOut, 128, 128, 4, 2, 2, 1>(a, groups, st);
+    case 17: return launchPatch<T, TOut, 256, 128, 4, 2, 2, 1>(a, groups, st);
+    case 18: return launchPatch<T, TOut, 64, 256, 4, 1, 4, 1>(a, groups, st);
+    case 19: return launchPatch<T, TOut, 128, 128, 4, 2, 2, 2>(a, groups, st);
+    // two LDS stages, 128-byte rows
+    case 20: return launchIgemm<T, TOut, 128, 128, 8, 2, 2, 2>(a, groups, st);
+    case 21: return launchIgemm<T, TOut, 256, 128, 8, 2, 2, 2>(a, groups, st);
+    case 22: return launchIgemm<T, TOut, 128, 256, 8, 2, 2, 2>(a, groups, st);
+    case 23: return launchIgemm<T, TOut, 128, 64, 8, 2, 2, 2>(a, groups, st);
+    case 24: return launchIgemm<T, TOut, 64, 128, 8, 1, 4, 2>(a, groups, st);
+    // deeper prefetch
+    case 25: return launchIgemm<T, TOut, 128, 128, 4, 2, 2, 4>(a, groups, st);
+    case 26: return launchIgemm<T, TOut, 256, 128, 4, 2, 2, 6>(a, groups, st);
+    case 27: return launchIgemm<T, TOut, 128, 128, 8, 2, 2, 4>(a, groups, st);
+    case 28: return launchIgemm<T, TOut, 128, 128, 4, 2, 2, 5>(a, groups, st);
     default: break;
     }
     setError("igemm: unknown tile %d", tile);

@@ -1,42 +1,58 @@
 // 3x3 stride-1 pad-1 convolution with the input patch resident in LDS.
 //
 // The generic implicit GEMM gathers the B operand (pixels x K) from global memory once per filter tap, so every
-// input pixel crosses the L2 -> CU path nine times per channel tile.  Here a tile of BN consecutive output pixels
-// (flattened over the batch) stages the contiguous run of BN + 2W + 2 input pixels it can touch -- one row above,
-// one below, one pixel either side -- ONCE per channel chunk; the nine taps then read their operand fragments
-// from that patch at a row offset of ti*W + tj, with lanes whose tap falls outside the image zeroed.  Only the
-// weight tile of the current (chunk, tap) is streamed per step.  The next chunk's patch is brought in in eight
-// slices interleaved with the tap steps (second LDS buffer), the next weight tile one step ahead.
+// input pixel crosses the L2 -> CU path nine times per channel chunk, and it is the L2's request rate, not the
+// matrix cores, that bounds those kernels.  Here a tile of BN consecutive output pixels (flattened over the
+// batch) stages the contiguous run of R = BN + 2W + 2 input pixels it can touch -- one image row above, one
+// below, one pixel either side -- ONCE per channel chunk; the nine taps then read their operand fragments from
+// that patch at a row offset of ky*W + kx, and lanes whose tap falls outside the image read a zero chunk instead.
+// Only the weight tile of the current (chunk, tap) is streamed per step.
+//
+// Data movement is the implicit GEMM's: 16-byte-per-lane buffer loads straight into LDS, XOR-swizzled unpadded
+// rows, three rotating stages for the weight tile.  The patch has two stages; the patch of chunk c+1 arrives in
+// 1 KiB slices (one wave instruction each), PS per wave and tap step over taps 0..7 of chunk c.  Every step
+// issues the same number of loads per wave -- slices that do not exist go, out of range and therefore as
+// zeros without touching memory, into a 1 KiB dump area that doubles as the zero chunk -- so the count of loads
+// in flight at each barrier is a compile-time constant.
 #pragma once
 #include "conv_igemm.hpp"
 
 namespace msnh {
 
-constexpr int kPatchSliceMax = 3;       // patch vectors a thread moves per tap step (upper bound)
-
-template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN>
-__global__ __launch_bounds__(256) void convPatch3x3Kernel(IgemmArgs a)
+template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int PS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void convPatch3x3Kernel(IgemmArgs a)
 {
     typedef typename Frag<T>::V V;
-    constexpr int VEC  = Frag<T>::VEC;
-    constexpr int BK   = KV * VEC;
-    constexpr int LDK  = BK + VEC;
-    constexpr int TM   = BM / WM;
-    constexpr int TN   = BN / WN;
-    constexpr int MB   = TM / 32;
-    constexpr int NB   = TN / 32;
-    constexpr int KBLK = KV / 2;
-    constexpr int AV   = BM * KV / 256;           // weight vectors per thread per step
-    static_assert(BM * KV % 256 == 0 && TM % 32 == 0 && TN % 32 == 0 && WM * WN == 4, "tile shape");
+    constexpr int VEC   = Frag<T>::VEC;
+    constexpr int BK    = KV * VEC;
+    constexpr int RPP   = 256 / KV;
+    constexpr int AL    = BM / RPP;               // weight loads per thread per step
+    constexpr int NL    = AL + PS;                // loads per thread per step
+    constexpr int TM    = BM / WM;
+    constexpr int TN    = BN / WN;
+    constexpr int MB    = TM / 32;
+    constexpr int NB    = TN / 32;
+    constexpr int S     = KV / 2;
+    constexpr unsigned ES = sizeof(T);
+    constexpr int ROWB  = KV * 16;
+    constexpr int SWDIV = 16 / KV;
+    constexpr unsigned A_STAGE = BM * ROWB;
+    constexpr int RPS   = 64 / KV;                // patch rows per 1 KiB slice
+    static_assert(KV == 4 && S == 2, "the slice arithmetic below assumes 64-byte rows");
+    static_assert(BM % RPP == 0 && TM % 32 == 0 && TN % 32 == 0 && WM * WN == 4, "tile shape");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smemRaw[];
-    const int R = a.patchRows;
-    T *Ps = reinterpret_cast<T *>(smemRaw);               // [2][R][LDK]
-    T *As = Ps + 2 * R * LDK;                              // [2][BM][LDK]
+    const unsigned ldsBase = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char *)smemRaw));
+    // LDS: three weight stages | patch stage 0 | patch stage 1 | dump / zero area (1 KiB)
+    const int nSlices = a.patchRows;              // 1 KiB slices per patch stage (host: ceil(R * KV / 64))
+    const unsigned patchBytes = static_cast<unsigned>(nSlices) * 1024u;
+    const unsigned patchOff0 = 3 * A_STAGE;
+    const unsigned dumpOff = patchOff0 + 2 * patchBytes;
 
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm   = wave / WN;
     const int wn   = wave % WN;
     const int nTilesP = (a.P + BN - 1) / BN;
@@ -47,87 +63,100 @@ __global__ __launch_bounds__(256) void convPatch3x3Kernel(IgemmArgs a)
     const int m0 = (logical % a.mTiles) * BM;
     const int p0 = (logical / a.mTiles) * BN;
 
+    const i32x4 rx = makeRsrcWords(a.x, a.xBytes);
+    const i32x4 rw = makeRsrcWords(a.w, a.wBytes);
+
     float chScale, chShift;
     loadChannelAffine(a, 0, m0, tid, BM, chScale, chShift);
 
-    const T *xg = static_cast<const T *>(a.x);
-    const T *wg = static_cast<const T *>(a.w);
+    if (tid < 64) *reinterpret_cast<f32x4 *>(smemRaw + dumpOff + tid * 16) = f32x4{0.f, 0.f, 0.f, 0.f};
+
     const int W = a.W, H = a.H;
-    const int q0 = p0 - W - 1;                            // input pixel held by patch row 0
-    const int PV = R * KV;                                // vectors per patch chunk
-    const int SV = (PV + 7) / 8;                          // vectors per slice
 
-    // ---- loaders ----------------------------------------------------------------------------------------
-    auto patchVec = [&](int idx, int chunk) -> V {
-        const int r = idx / KV, v = idx - r * KV;
-        const int q = q0 + r;
-        const int c = chunk * BK + v * VEC;
-        V val = {0};
-        if (q >= 0 && q < a.P && c < a.cinG) val = *reinterpret_cast<const V *>(xg + static_cast<size_t>(q) * a.inLd + c);
-        return val;
-    };
-    auto patchDst = [&](int idx, int buf) -> V * {
-        const int r = idx / KV, v = idx - r * KV;
-        return reinterpret_cast<V *>(Ps + (static_cast<size_t>(buf) * R + r) * LDK + v * VEC);
-    };
-    V regA[AV], regP[kPatchSliceMax];
-    auto loadA = [&](int it) {
-        const int chunk = it / 9, tap = it - chunk * 9;
+    // ---- weight tile: thread tid owns chunk position tid % KV of row tid / KV (+ RPP rows per load) -----------
+    const int ldRow = tid / KV;
+    const int ldVec = (tid % KV) ^ ((ldRow / SWDIV) % KV);
+    unsigned aOff[AL];
 #pragma unroll
-        for (int i = 0; i < AV; ++i)
-        {
-            const int va = tid + i * 256;
-            const int row = va / KV, v = va - row * KV;
-            const int m = m0 + row;
-            const int c = chunk * BK + v * VEC;
-            V val = {0};
-            if (m < a.coutG && c < a.cinG) val = *reinterpret_cast<const V *>(wg + (static_cast<size_t>(m) * 9 + tap) * a.cinG + c);
-            regA[i] = val;
-        }
+    for (int i = 0; i < AL; ++i)
+    {
+        const int m = m0 + ldRow + i * RPP;
+        aOff[i] = m < a.coutG ? (static_cast<unsigned>(m) * 9u * a.cinG + ldVec * VEC) * ES : kOobOffset;
+    }
+    // ---- patch: slice s holds patch rows s*RPS .. s*RPS+RPS-1; lane l of the slice's load owns chunk position
+    // l % KV of row s*RPS + l / KV, i.e. input pixel q0 + that row.  Pixels before the tensor give a negative
+    // offset, which as unsigned is out of range like the pixels behind the tensor: zeros, no test needed.
+    const int q0 = p0 - W - 1;                                  // input pixel of patch row 0
+    const int pRow = lane / KV;
+    const int pVec = (lane % KV) ^ ((pRow / SWDIV) % KV);       // (s*RPS + pRow) / SWDIV % KV does not depend on s
+    const unsigned pBase = static_cast<unsigned>((static_cast<long long>(q0 + pRow) * a.inLd + pVec * VEC) * static_cast<long long>(ES));
+    const unsigned sliceStride = static_cast<unsigned>(RPS) * a.inLd * ES;
+    const unsigned waveDump = ldsBase + dumpOff;
+
+    // slice number i of this wave (slices wave, wave+4, ...) of the patch of channel chunk `chunk` into stage `st`
+    auto issuePatch = [&](int i, int chunk, unsigned stOff) {
+        const int s = wave + 4 * i;
+        const bool real = s < nSlices && chunk < a.cChunks;
+        const bool cut = a.ragged && (chunk * BK + pVec * VEC >= a.cinG);
+        const unsigned voff = (real && !cut) ? pBase + static_cast<unsigned>(s) * sliceStride : kOobOffset;
+        dmaLoad16(rx, voff, static_cast<unsigned>(chunk * BK) * ES, real ? ldsBase + stOff + static_cast<unsigned>(s) * 1024u : waveDump);
     };
-    auto storeA = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < AV; ++i)
-        {
-            const int va = tid + i * 256;
-            const int row = va / KV, v = va - row * KV;
-            *reinterpret_cast<V *>(As + (buf * BM + row) * LDK + v * VEC) = regA[i];
-        }
-    };
-    auto loadSlice = [&](int slice, int chunk) {
-        const int end = (slice + 1) * SV < PV ? (slice + 1) * SV : PV;
-#pragma unroll
-        for (int j = 0; j < kPatchSliceMax; ++j)
-        {
-            const int idx = slice * SV + tid + j * 256;
-            V val = {0};
-            if (idx < end) val = patchVec(idx, chunk);
-            regP[j] = val;
-        }
-    };
-    auto storeSlice = [&](int slice, int buf) {
-        const int end = (slice + 1) * SV < PV ? (slice + 1) * SV : PV;
-#pragma unroll
-        for (int j = 0; j < kPatchSliceMax; ++j)
-        {
-            const int idx = slice * SV + tid + j * 256;
-            if (idx < end) *patchDst(idx, buf) = regP[j];
-        }
+    const unsigned waveLds = ldsBase + wave * 1024;
+    auto issueA = [&](auto lTag, unsigned sA, bool cut, unsigned stageOff) {
+        constexpr int l = decltype(lTag)::value;
+        dmaLoad16(rw, cut ? kOobOffset : aOff[l], sA, waveLds + stageOff + l * RPP * ROWB);
     };
 
-    // ---- per-lane pixel metadata for the B fragments -----------------------------------------------------------
-    int  nLocal[NB], oy[NB], ox[NB];
-    bool pOk[NB];
+    // ---- fragments ------------------------------------------------------------------------------------------
+    const int fragRow = lane & 31;
+    const int fragSw  = (fragRow / SWDIV) % KV;
+    unsigned aAddr[S];
+#pragma unroll
+    for (int kb = 0; kb < S; ++kb) aAddr[kb] = wm * TM * ROWB + fragRow * ROWB + (((2 * kb + (lane >> 5)) ^ fragSw) * 16);
+    // per 32-pixel block j of the wave tile: which of the nine taps lie inside the image for this lane's pixel
+    unsigned tapOk[NB];
 #pragma unroll
     for (int j = 0; j < NB; ++j)
     {
-        nLocal[j] = wn * TN + j * 32 + (lane & 31);
-        const int p = p0 + nLocal[j];
-        pOk[j] = p < a.P;
-        const int pp = pOk[j] ? p : 0;
-        ox[j] = pp % W;
-        oy[j] = (pp / W) % H;
+        const int p = p0 + wn * TN + j * 32 + fragRow;
+        unsigned m = 0;
+        if (p < a.P)
+        {
+            const int x = p % W;
+            const int y = (p / W) % H;
+#pragma unroll
+            for (int t = 0; t < 9; ++t)
+            {
+                const int yy = y + t / 3 - 1, xx = x + t % 3 - 1;
+                if (yy >= 0 && yy < H && xx >= 0 && xx < W) m |= 1u << t;
+            }
+        }
+        tapOk[j] = m;
     }
+    const unsigned bRow0 = wn * TN + fragRow;     // patch row of this lane's pixel for tap (0,0), block 0
+
+    V fa[2][MB], fb[2][NB];
+    auto readA = [&](unsigned stageOff, auto kbTag) {
+        constexpr int kb = decltype(kbTag)::value;
+        const unsigned char *ap = smemRaw + (aAddr[kb] + stageOff);
+#pragma unroll
+        for (int i = 0; i < MB; ++i) fa[kb % 2][i] = *reinterpret_cast<const V *>(ap + i * 32 * ROWB);
+    };
+    // B fragments of tap `tap` from the patch stage at pOff
+    auto readB = [&](unsigned pOff, int tap, auto kbTag) {
+        constexpr int kb = decltype(kbTag)::value;
+        const int ky = tap / 3;
+        const unsigned row = bRow0 + static_cast<unsigned>(ky * W + (tap - 3 * ky));
+        const unsigned sw = (row / SWDIV) % KV;   // rows 32 apart share it
+        const unsigned addr = pOff + row * ROWB + (((2 * kb + (lane >> 5)) ^ sw) * 16);
+        const unsigned bit = 1u << tap;
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+        {
+            const unsigned aj = (tapOk[j] & bit) ? addr + j * 32 * ROWB : dumpOff;
+            fb[kb % 2][j] = *reinterpret_cast<const V *>(smemRaw + aj);
+        }
+    };
 
     f32x16 acc[MB][NB];
 #pragma unroll
@@ -137,93 +166,122 @@ __global__ __launch_bounds__(256) void convPatch3x3Kernel(IgemmArgs a)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // ---- prologue: whole patch of chunk 0, weight tile of step 0 -------------------------------------------------------
-    for (int idx = tid; idx < PV; idx += 256) *patchDst(idx, 0) = patchVec(idx, 0);
-    loadA(0);
-    storeA(0);
+    constexpr int PER = MB * NB;
+    // all NL loads of a step are issued among the MFMAs of its first k-step, ahead of the barrier
+    // ---- prologue: whole patch of chunk 0, weight tiles of steps 0 and 1 ----------------------------------------
+    for (int i = 0; wave + 4 * i < nSlices; ++i) issuePatch(i, 0, patchOff0);
+    staticFor<0, AL>([&](auto lTag) { issueA(lTag, 0u, a.ragged && (ldVec * VEC >= a.cinG), 0u); });
+    {
+        const bool pastEnd = a.nIter < 2;         // never: nIter >= 9
+        staticFor<0, AL>([&](auto lTag) { issueA(lTag, static_cast<unsigned>(a.cinG) * ES, pastEnd || (a.ragged && (ldVec * VEC >= a.cinG)), A_STAGE); });
+    }
+    dmaWait<0>();
     __syncthreads();
+    readA(0, std::integral_constant<int, 0>());
+    readB(patchOff0, 0, std::integral_constant<int, 0>());
 
-    const int fragRow = lane & 31;
-    const int fragCol = (lane >> 5) * VEC;
-    const int chunks = a.cChunks;
-
+    // step it = chunk * 9 + tap; weight stage of step it is (it % 3) * A_STAGE; patch stage of chunk is chunk % 2
+    unsigned curA = 0, nxtA = A_STAGE, nnA = 2 * A_STAGE;
+    unsigned curP = patchOff0, othP = patchOff0 + patchBytes;
+    int tap = 0, chunk = 0;
+    int tapL = 1, chunkL = 0;                     // (tap, chunk) of the step whose weight tile was issued last
     for (int it = 0; it < a.nIter; ++it)
     {
-        const int chunk = it / 9, tap = it - chunk * 9;
-        const int ti = tap / 3, tj = tap - ti * 3;
-        const bool moreChunks = chunk + 1 < chunks;
-        if (it + 1 < a.nIter) loadA(it + 1);
-        if (moreChunks && tap < 8) loadSlice(tap, chunk + 1);
+        // the weight tile of step it+2
+        if (++tapL == 9) { tapL = 0; ++chunkL; }
+        const unsigned sA = (static_cast<unsigned>(tapL) * a.cinG + chunkL * BK) * ES;
+        const bool cutA = it + 2 >= a.nIter || (a.ragged && (chunkL * BK + ldVec * VEC >= a.cinG));
+        // the next step's tap and patch stage
+        const int tapN = tap == 8 ? 0 : tap + 1;
+        const unsigned nextP = tap == 8 ? othP : curP;
 
-        const T *ab = As + ((it & 1) * BM + wm * TM + fragRow) * LDK + fragCol;
-        const T *pb = Ps + static_cast<size_t>(chunk & 1) * R * LDK + static_cast<size_t>(ti * W + tj) * LDK + fragCol;
-        bool ok[NB];
-#pragma unroll
-        for (int j = 0; j < NB; ++j)
-            ok[j] = pOk[j] && static_cast<unsigned>(oy[j] + ti - 1) < static_cast<unsigned>(H) &&
-                    static_cast<unsigned>(ox[j] + tj - 1) < static_cast<unsigned>(W);
-#pragma unroll
-        for (int kb = 0; kb < KBLK; ++kb)
-        {
-            V fa[MB], fb[NB];
-#pragma unroll
-            for (int i = 0; i < MB; ++i) fa[i] = *reinterpret_cast<const V *>(ab + i * 32 * LDK + kb * 2 * VEC);
-#pragma unroll
-            for (int j = 0; j < NB; ++j)
+        readA(curA, std::integral_constant<int, 1>());
+        readB(curP, tap, std::integral_constant<int, 1>());
+        __builtin_amdgcn_sched_barrier(0);
+        staticFor<0, 2 * PER>([&](auto gTag) {
+            constexpr int gi = decltype(gTag)::value;
+            constexpr int ks = gi / PER;
+            if constexpr (gi == PER)
             {
-                V v = *reinterpret_cast<const V *>(pb + static_cast<size_t>(nLocal[j]) * LDK + kb * 2 * VEC);
-                if (!ok[j]) v = V{0};
-                fb[j] = v;
+                dmaWait<NL>();                    // everything issued before this step has landed
+                __syncthreads();
+                readA(nxtA, std::integral_constant<int, 0>());
+                readB(nextP, tapN, std::integral_constant<int, 0>());
+                __builtin_amdgcn_sched_barrier(0);
             }
-#pragma unroll
-            for (int i = 0; i < MB; ++i)
-#pragma unroll
-                for (int j = 0; j < NB; ++j) mfmaBlock(fa[i], fb[j], acc[i][j]);
+            mfmaBlock(fa[ks % 2][(gi % PER) / NB], fb[ks % 2][(gi % PER) % NB], acc[(gi % PER) / NB][(gi % PER) % NB]);
+            if constexpr (gi < PER)
+            {
+                // loads l with l * PER / NL == gi: patch slices first, then the weight rows
+                constexpr int first = (gi * NL + PER - 1) / PER;
+                constexpr int last  = ((gi + 1) * NL + PER - 1) / PER;
+                staticFor<first, last>([&](auto lTag) {
+                    constexpr int l = decltype(lTag)::value;
+                    if constexpr (l < PS)
+                        issuePatch(tap == 8 ? (1 << 20) : tap * PS + l, chunk + 1, othP);
+                    else
+                        issueA(std::integral_constant<int, l - PS>(), sA, cutA, nnA);
+                });
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        const unsigned t = curA;
+        curA = nxtA;
+        nxtA = nnA;
+        nnA = t;
+        if (tap == 8)
+        {
+            tap = 0;
+            ++chunk;
+            const unsigned tp = curP;
+            curP = othP;
+            othP = tp;
         }
-
-        if (it + 1 < a.nIter) storeA((it + 1) & 1);
-        if (moreChunks && tap < 8) storeSlice(tap, (chunk + 1) & 1);
-        __syncthreads();
+        else
+            ++tap;
     }
+    dmaWait<0>();
+    __syncthreads();
 
     igemmEpilogue<T, TOut, BM, BN, TM, TN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, wave, lane, 0);
 }
 
 // Host-side check shared by launch and tile enumeration.
-template <typename T, int BM, int BN, int KV, int WM, int WN>
-inline bool patchFits(const IgemmArgs &a, size_t *smemOut)
+template <typename T, int BM, int BN, int KV, int WM, int WN, int PS>
+inline bool patchFits(const IgemmArgs &a, size_t *smemOut, int *slicesOut)
 {
-    constexpr int VEC = Frag<T>::VEC;
-    constexpr int LDK = KV * VEC + VEC;
     const int R = BN + 2 * a.W + 2;
-    const size_t loop = (static_cast<size_t>(2) * R + 2 * BM) * LDK * sizeof(T);
+    const int slices = (R * KV + 63) / 64;
+    const size_t loop = static_cast<size_t>(3) * BM * KV * 16 + static_cast<size_t>(2) * slices * 1024 + 1024;
     const size_t epi = igemmEpilogueLds<BM, BM / WM>();
     const size_t smem = loop > epi ? loop : epi;
     if (smemOut) *smemOut = smem;
-    const int sv = (R * KV + 7) / 8;
-    return a.patchOk && smem <= 160 * 1024 && (sv + 255) / 256 <= kPatchSliceMax;
+    if (slicesOut) *slicesOut = slices;
+    // taps 0..7 of a chunk bring in the next patch: 8 * PS slices per wave, 4 waves
+    return a.patchOk && a.buffersOk && smem <= 160 * 1024 && slices <= 32 * PS;
 }
 
-template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN>
+template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int PS>
 inline int launchPatch(IgemmArgs &a, int groups, hipStream_t st)
 {
     constexpr int VEC = Frag<T>::VEC;
     constexpr int BK  = KV * VEC;
     size_t smem = 0;
-    if (groups != 1 || !patchFits<T, BM, BN, KV, WM, WN>(a, &smem))
+    int slices = 0;
+    if (groups != 1 || !patchFits<T, BM, BN, KV, WM, WN, PS>(a, &smem, &slices))
     {
         setError("conv2d: this tile needs a 3x3 stride-1 pad-1 ungrouped convolution whose input patch fits in LDS");
         return 3;
     }
     if (a.dryRun) return 0;
-    a.patchRows = BN + 2 * a.W + 2;
+    a.patchRows = slices;
     a.cChunks = (a.cinG + BK - 1) / BK;
     a.nIter   = 9 * a.cChunks;
     a.ragged  = (a.cinG % BK) != 0;
     a.mTiles  = (a.coutG + BM - 1) / BM;
     const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
     dim3 grid((tiles + 7) / 8 * 8, 1, 1);
-    auto kern = convPatch3x3Kernel<T, TOut, BM, BN, KV, WM, WN>;
+    auto kern = convPatch3x3Kernel<T, TOut, BM, BN, KV, WM, WN, PS>;
     if (smem > 48 * 1024)
     {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
