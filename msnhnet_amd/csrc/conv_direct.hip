@@ -16,6 +16,10 @@ int convWinograd(const msnh_conv_desc *d, const void *x, const void *w, const fl
                  const void *residual, void *y, void *ws, size_t wsBytes, hipStream_t st);
 size_t winogradWorkspaceBytes(const msnh_conv_desc *d);
 void   winogradPackWeights(const msnh_conv_desc *d, const float *oihw, void *packed);
+bool   stemMfmaOk(const msnh_conv_desc *d);
+size_t stemMfmaElems(const msnh_conv_desc *d);
+void   stemMfmaPack(const msnh_conv_desc *d, const float *oihw, _Float16 *packed);
+int    convStemMfma(const msnh_conv_desc *d, const float *x, const _Float16 *wA, const float *scale, const float *shift, void *y, hipStream_t st);
 
 struct EpiArgs
 {
@@ -244,7 +248,8 @@ size_t msnh_hip_conv2d_packed_weight_elems(const msnh_conv_desc *d, int algo)
     const size_t kk = static_cast<size_t>(d->ksize) * d->ksize;
     const size_t cinG = static_cast<size_t>(d->in_c / d->groups);
     if (algo == MSNH_CONV_WINOGRAD) return static_cast<size_t>(16) * d->out_c * d->in_c;
-    if (algo == MSNH_CONV_STEM) return kk * d->in_c * d->out_c * (d->dtype == MSNH_F16 ? 2 : 1);   // float32 payload
+    // float32 payload for the scalar kernel, followed (float16 plans) by the MFMA operand fragments
+    if (algo == MSNH_CONV_STEM) return kk * d->in_c * d->out_c * (d->dtype == MSNH_F16 ? 2 : 1) + (stemMfmaOk(d) ? stemMfmaElems(d) : 0);
     return static_cast<size_t>(d->out_c) * kk * cinG;
 }
 
@@ -280,6 +285,7 @@ int msnh_hip_conv2d_pack_weights(const msnh_conv_desc *d, int algo, const float 
             for (int ci = 0; ci < d->in_c; ++ci)
                 for (int t = 0; t < kk; ++t)
                     o[(static_cast<size_t>(t) * d->in_c + ci) * d->out_c + oc] = oihw[(static_cast<size_t>(oc) * d->in_c + ci) * kk + t];
+        if (stemMfmaOk(d)) stemMfmaPack(d, oihw, static_cast<_Float16 *>(packed) + static_cast<size_t>(kk) * d->in_c * d->out_c * 2);
         return 0;
     }
     case MSNH_CONV_WINOGRAD:
@@ -349,6 +355,9 @@ int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const
         MSNH_REQUIRE(stemOk(d), "conv2d: shape not supported by the stem kernel");
         const size_t outEl = dtypeSize(d->out_dtype);
         MSNH_REQUIRE(reinterpret_cast<uintptr_t>(y) % (4 * outEl) == 0, "conv2d: stem needs aligned output");
+        if (stemMfmaOk(d))
+            return convStemMfma(d, static_cast<const float *>(x), static_cast<const _Float16 *>(w) + static_cast<size_t>(d->ksize) * d->ksize * d->in_c * d->out_c * 2,
+                                scale, shift, y, st);
         constexpr int OCT = 32;
         dim3 grid(gridFor(P, 256), d->out_c / OCT);
         const size_t smem = static_cast<size_t>(d->ksize) * d->ksize * d->in_c * OCT * sizeof(float);
