@@ -10,7 +10,12 @@ struct Anchors { float v[6]; };
 // A workgroup decodes CHUNK consecutive values of one image.  Entries whose objectness passes the threshold are
 // first collected in LDS; one global atomic per workgroup then reserves their slots in the image's candidate list
 // (one atomic per candidate on a single counter would serialise half of all cells with the benchmark weights).
-constexpr int YOLO_CHUNK = 256 * 16;
+constexpr int YOLO_CHUNK = 256 * 8;
+
+// logistic with the hardware exp2 / reciprocal (about 1e-6 relative, against 1e-7 for expf and a full division):
+// the 5 + classes logistics per cell are what the kernel computes most of, and with library precision they, not
+// the memory traffic, set its run time.  Box width and height keep expf.
+__device__ __forceinline__ float fastLogistic(float v) { return __builtin_amdgcn_rcpf(1.f + __expf(-v)); }
 
 template <typename T>
 __global__ __launch_bounds__(256) void yoloDecodeKernel(const T *__restrict__ x, int xLd, float xMul, Anchors an, float ratio,
@@ -24,24 +29,47 @@ __global__ __launch_bounds__(256) void yoloDecodeKernel(const T *__restrict__ x,
     if (threadIdx.x == 0) nFound = 0;
     __syncthreads();
     const int start = blockIdx.x * YOLO_CHUNK;
+    // idx = (a*HW + p)*per + m inside the image; a thread's idx advances by 256 per step, so (m, p, a) are carried
+    // along with adds and compares instead of being recovered by three divisions per element
+    int idx = start + threadIdx.x;
+    int m = idx % per;
+    int cell = idx / per;
+    int p = cell % HW;
+    int a = cell / HW;
+    int px = p % W, py = p / W;
+    const int stepCell = 256 / per, stepM = 256 % per;
+    const int stepY = stepCell / W, stepX = stepCell % W;
+    const T *xb = x + static_cast<size_t>(b) * HW * xLd;
+    float *db = decoded + static_cast<size_t>(b) * decStride;
 #pragma unroll 4
     for (int k = 0; k < YOLO_CHUNK / 256; ++k)
     {
-        const int idx = start + k * 256 + threadIdx.x;          // = (a*HW + p)*per + m inside the image
-        if (idx >= perImage) break;
-        const int m = idx % per;
-        const int cell = idx / per;
-        const int p = cell % HW;
-        const int a = cell / HW;
-        const float v = xMul * toF(x[(static_cast<size_t>(b) * HW + p) * xLd + a * per + m]);
+        const bool live = idx < perImage;          // predicate, not an exit: the unrolled loads can then be issued together
+        const float v = live ? xMul * toF(xb[static_cast<size_t>(p) * xLd + a * per + m]) : 0.f;
         float r;
-        if (m == 0)      r = (1.f / (1.f + expf(-v)) + static_cast<float>(p % W)) * ratio;
-        else if (m == 1) r = (1.f / (1.f + expf(-v)) + static_cast<float>(p / W)) * ratio;
-        else if (m == 2) r = an.v[2 * a] * expf(v);
-        else if (m == 3) r = an.v[2 * a + 1] * expf(v);
-        else             r = 1.f / (1.f + expf(-v));
-        decoded[static_cast<size_t>(b) * decStride + idx] = r;
-        if (m == 4 && candIdx != nullptr && r > confThresh) found[atomicAdd(&nFound, 1)] = candBase + cell;
+        if (m == 0)      r = (fastLogistic(v) + static_cast<float>(px)) * ratio;
+        else if (m == 1) r = (fastLogistic(v) + static_cast<float>(py)) * ratio;
+        else if (m == 2) r = an.v[(2 * a) % 6] * expf(v);
+        else if (m == 3) r = an.v[(2 * a + 1) % 6] * expf(v);
+        else             r = fastLogistic(v);
+        if (live) db[idx] = r;
+        if (live && m == 4 && candIdx != nullptr && r > confThresh) found[atomicAdd(&nFound, 1)] = candBase + a * HW + p;
+        idx += 256;
+        m += stepM;
+        int dc = stepCell;
+        if (m >= per) { m -= per; ++dc; }
+        // advance the pixel by dc cells: dc = stepCell or stepCell + 1
+        px += stepX + (dc - stepCell);
+        py += stepY;
+        p += dc;
+        if (px >= W) { px -= W; ++py; }
+        if (px >= W) { px -= W; ++py; }
+        if (p >= HW)
+        {
+            do { p -= HW; ++a; } while (p >= HW);
+            py = p / W;
+            px = p - py * W;
+        }
     }
     __syncthreads();
     if (candIdx == nullptr || nFound == 0) return;
