@@ -16,6 +16,7 @@ int convWinograd(const msnh_conv_desc *d, const void *x, const void *w, const fl
                  const void *residual, void *y, void *ws, size_t wsBytes, hipStream_t st);
 size_t winogradWorkspaceBytes(const msnh_conv_desc *d);
 void   winogradPackWeights(const msnh_conv_desc *d, const float *oihw, void *packed);
+void   winogradGemmDesc(const msnh_conv_desc *d, msnh_conv_desc *gd);
 bool   stemMfmaOk(const msnh_conv_desc *d);
 size_t stemMfmaElems(const msnh_conv_desc *d);
 void   stemMfmaPack(const msnh_conv_desc *d, const float *oihw, _Float16 *packed);
@@ -212,7 +213,7 @@ static bool stemOk(const msnh_conv_desc *d)
 static bool winogradOk(const msnh_conv_desc *d)
 {
     return d->ksize == 3 && d->stride == 1 && d->dilation == 1 && d->groups == 1 && d->pad == 1 && d->dtype == MSNH_F16 &&
-           d->in_c % 8 == 0 && d->in_ld % 8 == 0 && d->out_c % 8 == 0;
+           d->in_c % 8 == 0 && d->in_ld % 8 == 0 && d->out_c % 8 == 0 && d->out_ld % 8 == 0;
 }
 
 } // namespace msnh
@@ -225,9 +226,16 @@ int msnh_hip_conv2d_tile_count(void) { return igemmTileCount(); }
 
 int msnh_hip_conv2d_tile_supported(const msnh_conv_desc *d, int tile)
 {
-    if (!d || validate(d) || !igemmOk(d) || tile < 0 || tile > igemmTileCount()) return 0;
-    if (tile == 0) return 1;
+    if (!d || validate(d) || tile < 0 || tile > igemmTileCount()) return 0;
     msnh_conv_desc t = *d;
+    if (d->algo == MSNH_CONV_WINOGRAD)
+    {
+        // the tile applies to the 16 transformed-domain GEMMs
+        if (!winogradOk(d) || static_cast<long long>(d->batch) * ((d->out_h + 1) / 2) * ((d->out_w + 1) / 2) * 16 * d->in_c * 2 >= (1LL << 31)) return 0;
+        winogradGemmDesc(d, &t);
+    }
+    else if (!igemmOk(d)) return 0;
+    if (tile == 0) return 1;
     t.tile = tile;
     return convIgemm(&t, d, d, nullptr, nullptr, nullptr, &t, nullptr, true) == 0 ? 1 : 0;      // pointers unused in a dry run
 }

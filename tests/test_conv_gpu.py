@@ -184,6 +184,49 @@ def test_conv_stem(h, w, oc, k, stride, pad, out_dtype):
     assert gu.rel_err(y, ref) <= (1e-5 if out_dtype == abi.F32 else 1e-3)
 
 
+@pytest.mark.parametrize("b,c,h,w,oc", [(2, 16, 12, 10, 24), (1, 32, 19, 19, 64), (3, 8, 7, 9, 8), (1, 64, 38, 38, 128)])
+@pytest.mark.parametrize("with_res", [False, True])
+def test_conv_winograd(b, c, h, w, oc, with_res):
+    """Winograd F(2x2,3x3): same result as the direct form (odd sizes exercise the partial tiles), full epilogue."""
+    import gpuutil as gu
+    rng = np.random.default_rng(b * 100 + c)
+    x, wt = _case(rng, b, c, h, w, oc, 3)
+    res = rng.standard_normal((b, oc, h, w), dtype=np.float32) if with_res else None
+    scale = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    shift = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    x, wt = gu.round_f16(x), gu.round_f16(wt)
+    if with_res:
+        res = gu.round_f16(res)
+    y, used = gu.conv2d(x, wt, dtype=abi.F16, stride=1, pad=1, scale=scale, shift=shift, act="leaky", residual=res, act2="none",
+                        res_mul=2.0, out_mul=0.5, algo="winograd", out_ld=oc + 8, res_ld=oc + 8 if with_res else None)
+    assert used == "winograd"
+    ref = _ref(x, wt, 1, 1, 1, 1, scale, shift, "leaky", 0.1, res, "none", 2.0, 0.5)
+    # the transformed weights are rounded to float16 a second time: a little above the direct kernel's tolerance
+    assert gu.rel_err(y, ref) <= 3 * TOL[abi.F16]
+    # every tile configuration of the transformed-domain GEMM that accepts the shape gives the same answer
+    L = abi.lib()
+    for tile in (2, 8, 12):
+        y2, _ = gu.conv2d(x, wt, dtype=abi.F16, stride=1, pad=1, scale=scale, shift=shift, act="leaky", residual=res, act2="none",
+                          res_mul=2.0, out_mul=0.5, algo="winograd", out_ld=oc + 8, res_ld=oc + 8 if with_res else None, tile=tile)
+        assert gu.rel_err(y2, ref) <= 3 * TOL[abi.F16]
+
+
+def test_conv_winograd_rejects():
+    import ctypes
+    import gpuutil as gu
+    gu.init()
+    L = abi.lib()
+    # stride 2 is not a Winograd shape
+    d = abi.ConvDesc(abi.F16, abi.F16, 1, 8, 8, 16, 16, 16, 4, 4, 16, 3, 2, 1, 1, 1, 22, 0.1, 0, 16, 22, 0.1, 1.0, 1.0, abi.ALGO["winograd"], 0)
+    assert L.msnh_hip_conv2d(ctypes.byref(d), 16, 16, None, None, None, 16, 256, 1 << 20, None) != 0
+    assert b"Winograd" in L.msnh_hip_last_error()
+    # a good shape without its workspace
+    d = abi.ConvDesc(abi.F16, abi.F16, 1, 8, 8, 16, 16, 16, 8, 8, 16, 3, 1, 1, 1, 1, 22, 0.1, 0, 16, 22, 0.1, 1.0, 1.0, abi.ALGO["winograd"], 0)
+    assert L.msnh_hip_conv2d_workspace_bytes(ctypes.byref(d), abi.ALGO["winograd"]) > 0
+    assert L.msnh_hip_conv2d(ctypes.byref(d), 256, 256, None, None, None, 256, None, 0, None) != 0
+    assert b"workspace" in L.msnh_hip_last_error()
+
+
 def test_conv_rejects_bad_shapes():
     import ctypes
     import gpuutil as gu
