@@ -57,6 +57,9 @@ const char *msnhnet_last_error(void);
 int msnhnet_create(msnhnet_t *net);                       /* NetBuilder() */
 int msnhnet_destroy(msnhnet_t net);
 int msnhnet_set_use_fp16(int on);                         /* NetBuilder::setUseFp16, process-wide, before build */
+int msnhnet_set_use_winograd(int on);                     /* float16 builds: 3x3 stride-1 convolutions through Winograd F(2x2,3x3);
+                                                             the reference keeps its own (ARM NEON, commented out) Winograd switch at
+                                                             src/layers/MsnhConvolutionalLayer.cpp:1262 */
 int msnhnet_set_keep_class_scores(int on);
 int msnhnet_set_save_layer_output(msnhnet_t net, int on); /* NetBuilder::setSaveLayerOutput */
 int msnhnet_build(msnhnet_t net, const char *msnhnet_path);      /* NetBuilder::buildNetFromMsnhNet */

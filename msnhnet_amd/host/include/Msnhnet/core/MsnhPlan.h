@@ -84,6 +84,7 @@ public:
     explicit Plan(int dtype) : computeDtype(dtype) {}
 
     int computeDtype;
+    bool preferWinograd = false;            // 3x3 stride-1 float16 convs take the Winograd path where the kernel accepts the shape
     std::vector<PlanTensor> tensors;
     std::vector<PlanOp>     ops;
     std::vector<int>        layerOut;       // output tensor of each top-level layer
@@ -124,6 +125,6 @@ public:
 
 private:
     void launch(PlanOp &op, msnh_stream_t s);
-    DeviceBuffer _arena, _exportScratch;
+    DeviceBuffer _arena, _exportScratch, _convWorkspace;
 };
 }

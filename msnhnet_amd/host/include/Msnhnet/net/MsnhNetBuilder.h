@@ -26,6 +26,8 @@ public:
     static void setKeepClassScores(const bool &keep);
     // Per-layer search for the fastest convolution tile configuration at load time (default on).
     static void setAutoTune(const bool &on);
+    static void setUseWinograd(const bool &on);   // float16 plans: 3x3 stride-1 convolutions through Winograd F(2x2,3x3)
+    static bool useWinograd;
     static bool autoTune;
 
     void buildNetFromMsnhNet(const std::string &path);

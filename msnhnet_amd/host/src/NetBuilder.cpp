@@ -43,6 +43,8 @@ void NetBuilder::setForceUseCuda(const bool &v) { BaseLayer::setForceUseCuda(v);
 void NetBuilder::setKeepClassScores(const bool &keep) { YoloOutLayer::keepClassScores = keep; }
 bool NetBuilder::autoTune = true;
 void NetBuilder::setAutoTune(const bool &on) { autoTune = on; }
+bool NetBuilder::useWinograd = false;
+void NetBuilder::setUseWinograd(const bool &on) { useWinograd = on; }
 
 void NetBuilder::setOnlyCpu(const bool &onlyCpu)
 {
@@ -355,6 +357,7 @@ void NetBuilder::finalizePlan()
     }
     plan->place();
     setupYoloBuffers(*plan, _net->batch);
+    plan->preferWinograd = useWinograd && dtype == MSNH_F16;
     plan->prepareWeights();
     if (autoTune) plan->tuneConvs(_stream);
 

@@ -327,6 +327,7 @@ static std::vector<uint16_t> toHalf(const std::vector<float> &v);
 
 void Plan::prepareWeights()
 {
+    size_t workspace = 0;
     for (PlanOp &op : ops)
     {
         if (op.dead) continue;
@@ -336,7 +337,14 @@ void Plan::prepareWeights()
             msnh_conv_desc d = convDesc(*this, op);
             if (in.layout == PlanTensor::NCHW_INPUT) d.algo = MSNH_CONV_STEM;
             op.algo = msnh_hip_conv2d_select_algo(&d);
+            if (preferWinograd && op.algo == MSNH_CONV_IGEMM)
+            {
+                msnh_conv_desc wd = d;
+                wd.algo = MSNH_CONV_WINOGRAD;
+                if (msnh_hip_conv2d_tile_supported(&wd, 0)) op.algo = MSNH_CONV_WINOGRAD;
+            }
             d.algo = op.algo;
+            workspace = std::max(workspace, msnh_hip_conv2d_workspace_bytes(&d, op.algo));
             const std::vector<float> &w = op.src->kernelWeights();
             const size_t expect = static_cast<size_t>(d.out_c) * (d.in_c / d.groups) * d.ksize * d.ksize;
             if (w.size() != expect) MSNH_THROW("conv weights are not loaded (" + op.name + ")");
@@ -397,6 +405,7 @@ void Plan::prepareWeights()
             op.flops = 2.0 * static_cast<double>(w.size()) * in.n;
         }
     }
+    if (workspace > _convWorkspace.bytes()) _convWorkspace.alloc(workspace);
 }
 
 // Per-layer search over the implicit-GEMM tile configurations: each candidate runs the real launch (same buffers,
@@ -407,17 +416,17 @@ void Plan::tuneConvs(msnh_stream_t s)
     msnh_event_t e0 = nullptr, e1 = nullptr;
     MSNH_DEV(msnh_hip_event_create(&e0));
     MSNH_DEV(msnh_hip_event_create(&e1));
-    struct Key { int b, h, w, c, oc, k, st, g, res, odt; bool operator==(const Key &o) const { return std::memcmp(this, &o, sizeof(Key)) == 0; } };
+    struct Key { int b, h, w, c, oc, k, st, g, res, odt, algo; bool operator==(const Key &o) const { return std::memcmp(this, &o, sizeof(Key)) == 0; } };
     std::vector<std::pair<Key, int>> memo;         // identical shapes share one search
     for (PlanOp &op : ops)
     {
-        if (op.dead || op.kind != PlanOp::CONV || op.algo != MSNH_CONV_IGEMM) continue;
+        if (op.dead || op.kind != PlanOp::CONV || (op.algo != MSNH_CONV_IGEMM && op.algo != MSNH_CONV_WINOGRAD)) continue;
         const PlanTensor &in = tensors[static_cast<size_t>(op.in0)];
         const PlanTensor &out = tensors[static_cast<size_t>(op.out)];
         Key key;
         std::memset(&key, 0, sizeof(key));
         key.b = in.n; key.h = in.h; key.w = in.w; key.c = in.c; key.oc = out.c; key.k = op.ksize; key.st = op.stride; key.g = op.groups;
-        key.res = op.in1 >= 0; key.odt = out.dtype;
+        key.res = op.in1 >= 0; key.odt = out.dtype; key.algo = op.algo;
         bool found = false;
         for (const auto &m : memo)
             if (m.first == key) { op.tile = m.second; found = true; break; }
@@ -489,7 +498,7 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
     {
         const msnh_conv_desc d = convDesc(*this, op);
         MSNH_DEV(msnh_hip_conv2d(&d, ptr(op.in0), op.wDev.ptr(), op.scaleDev.as<float>(), op.shiftDev.as<float>(),
-                                 op.in1 >= 0 ? ptr(op.in1) : nullptr, ptr(op.out), nullptr, 0, s));
+                                 op.in1 >= 0 ? ptr(op.in1) : nullptr, ptr(op.out), _convWorkspace.ptr(), _convWorkspace.bytes(), s));
         break;
     }
     case PlanOp::AFFINE:

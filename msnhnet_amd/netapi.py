@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libMsnhnet.so")
 
 SYMBOLS = [
     "initMsnhnet", "buildMsnhnet", "runClassifyNoPred", "runYoloNoPred", "dispose", "withGPU", "withCUDNN", "getCpuForwardTime",
-    "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16",
+    "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16", "msnhnet_set_use_winograd",
     "msnhnet_set_keep_class_scores", "msnhnet_set_save_layer_output", "msnhnet_build", "msnhnet_load", "msnhnet_load_from_memory",
     "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops",
     "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
@@ -65,6 +65,7 @@ def lib():
     L.msnhnet_create.argtypes = [ctypes.POINTER(vp)]
     L.msnhnet_destroy.argtypes = [vp]
     L.msnhnet_set_use_fp16.argtypes = [ci]
+    L.msnhnet_set_use_winograd.argtypes = [ci]
     L.msnhnet_set_keep_class_scores.argtypes = [ci]
     L.msnhnet_set_save_layer_output.argtypes = [vp, ci]
     L.msnhnet_build.argtypes = [vp, cp]
@@ -111,6 +112,10 @@ def _fp(a):
 
 def set_use_fp16(on):
     _check(lib().msnhnet_set_use_fp16(1 if on else 0))
+
+
+def set_use_winograd(on):
+    _check(lib().msnhnet_set_use_winograd(1 if on else 0))
 
 
 def nms(rows, thresh, fast=True):

@@ -130,6 +130,36 @@ def test_fp16_final_outputs(arch, size, batch):
                 assert int(np.argmax(logits[b])) == int(np.argmax(r))
 
 
+@pytest.mark.parametrize("arch,size,batch", [("resnet18", 224, 1), ("yolov3", 224, 2)])
+def test_fp16_winograd_network(arch, size, batch):
+    """every 3x3 stride-1 convolution through Winograd F(2x2,3x3): same final outputs within the float16 tolerance"""
+    net, binp, g = nu.model(arch, batch, size, seed=3)
+    x = zoo.seeded_input(batch, 3, size, size, seed=4)
+    ref, ref_boxes = _oracle_layers(arch, size, binp, x)
+    print("running fp16 winograd", arch, size, batch, flush=True)
+    netapi.set_use_winograd(True)
+    try:
+        m = netapi.Net(net, binp, fp16=True, dump_layers=True)
+    finally:
+        netapi.set_use_winograd(False)
+    assert "winograd" in m.plan_detail()
+    if arch.startswith("yolo"):
+        boxes = m.run_yolo(x)
+        for i in range(m.num_layers()):
+            if m.layer_info(i)["type"] != "yolo":
+                continue
+            got = m.layer_output(i - 1).reshape(batch, -1)
+            for b in range(batch):
+                e = nu.rel_err(got[b], ref[b][i - 1])
+                assert e <= 2e-2, f"{arch} head logits before layer {i}, image {b}: {e}"
+        for b in range(batch):
+            assert abs(len(boxes[b]) - len(ref_boxes[b])) <= max(2, 0.02 * len(ref_boxes[b]))
+    else:
+        logits = m.run_classify(x)
+        for b in range(batch):
+            assert nu.rel_err(logits[b], ref[b][-1]) <= 2e-2
+
+
 def test_cpu_entry_points_refuse():
     net, binp, g = nu.model("resnet18", 1, 224, seed=3)
     m = netapi.Net(net, binp)
