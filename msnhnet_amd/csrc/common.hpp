@@ -62,24 +62,35 @@ template <typename T> __device__ __forceinline__ T fromF(float v);
 template <> __device__ __forceinline__ float fromF<float>(float v) { return v; }
 template <> __device__ __forceinline__ f16 fromF<f16>(float v) { return static_cast<f16>(v); }
 
-// ---- activations: the reference's scalar formulas (include/Msnhnet/layers/MsnhActivations.h:39-168) ----
-__device__ __forceinline__ float softplusThr(float x, float thr)
+// ---- activations: the reference's scalar formulas (include/Msnhnet/layers/MsnhActivations.h:39-168), with the
+// transcendental ones rearranged so that each costs one hardware exp2 and one hardware reciprocal (about 1e-6
+// relative; on the epilogue of a bandwidth-bound convolution the library expf / logf / tanhf sequence of mish
+// otherwise takes longer than the memory traffic):
+//   logistic(x) = 1 / (1 + e^-x)
+//   mish(x)     = x * tanh(softplus(x)) = x * n / (n + 2),  n = w (w + 2),  w = e^x
+//                 (tanh(ln(1 + w)) = ((1+w)^2 - 1) / ((1+w)^2 + 1)); the reference's softplus thresholds at +-20 only
+//                 guard its own overflow: beyond +20 the quotient is 1 to float precision, below -20 it is w
+__device__ __forceinline__ float fastRcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+__device__ __forceinline__ float logisticF(float x) { return fastRcp(1.f + __expf(-x)); }
+
+__device__ __forceinline__ float mishF(float x)
 {
-    if (x > thr) return x;
-    if (x < -thr) return expf(x);
-    return logf(expf(x) + 1.f);
+    const float w = __expf(x < 20.f ? x : 20.f);
+    const float n = w * (w + 2.f);
+    return x * (n * fastRcp(n + 2.f));
 }
 
 __device__ __forceinline__ float activate(float x, int act, float param)
 {
     switch (act)
     {
-    case MSNH_ACT_LOGISTIC: return 1.f / (1.f + expf(-x));
+    case MSNH_ACT_LOGISTIC: return logisticF(x);
     case MSNH_ACT_RELU:     return x > 0.f ? x : 0.f * x;          // x*(x>0): keeps NaN, -0
     case MSNH_ACT_RELU6:    return (x > 0.f ? x : 0.f) > 6.f ? 6.f : (x > 0.f ? x : 0.f);
     case MSNH_ACT_LEAKY:    return x > 0.f ? x : param * x;
-    case MSNH_ACT_SWISH:    return x * (1.f / (1.f + expf(-x)));
-    case MSNH_ACT_MISH:     return x * tanhf(softplusThr(x, 20.f));
+    case MSNH_ACT_SWISH:    return x * logisticF(x);
+    case MSNH_ACT_MISH:     return mishF(x);
     default:                return x;
     }
 }

@@ -12,11 +12,8 @@ struct Anchors { float v[6]; };
 // (one atomic per candidate on a single counter would serialise half of all cells with the benchmark weights).
 constexpr int YOLO_CHUNK = 256 * 8;
 
-// logistic with the hardware exp2 / reciprocal (about 1e-6 relative, against 1e-7 for expf and a full division):
-// the 5 + classes logistics per cell are what the kernel computes most of, and with library precision they, not
-// the memory traffic, set its run time.  Box width and height keep expf.
-__device__ __forceinline__ float fastLogistic(float v) { return __builtin_amdgcn_rcpf(1.f + __expf(-v)); }
-
+// The 5 + classes logistics per cell are what the kernel computes most of (logisticF: hardware exp2 and
+// reciprocal); box width and height keep expf.
 template <typename T>
 __global__ __launch_bounds__(256) void yoloDecodeKernel(const T *__restrict__ x, int xLd, float xMul, Anchors an, float ratio,
                                                         float *__restrict__ decoded, long long decStride, float confThresh, int *__restrict__ candIdx,
@@ -47,11 +44,11 @@ __global__ __launch_bounds__(256) void yoloDecodeKernel(const T *__restrict__ x,
         const bool live = idx < perImage;          // predicate, not an exit: the unrolled loads can then be issued together
         const float v = live ? xMul * toF(xb[static_cast<size_t>(p) * xLd + a * per + m]) : 0.f;
         float r;
-        if (m == 0)      r = (fastLogistic(v) + static_cast<float>(px)) * ratio;
-        else if (m == 1) r = (fastLogistic(v) + static_cast<float>(py)) * ratio;
+        if (m == 0)      r = (logisticF(v) + static_cast<float>(px)) * ratio;
+        else if (m == 1) r = (logisticF(v) + static_cast<float>(py)) * ratio;
         else if (m == 2) r = an.v[(2 * a) % 6] * expf(v);
         else if (m == 3) r = an.v[(2 * a + 1) % 6] * expf(v);
-        else             r = fastLogistic(v);
+        else             r = logisticF(v);
         if (live) db[idx] = r;
         if (live && m == 4 && candIdx != nullptr && r > confThresh) found[atomicAdd(&nFound, 1)] = candBase + a * HW + p;
         idx += 256;
