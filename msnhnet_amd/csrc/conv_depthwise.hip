@@ -1,0 +1,142 @@
+// Depthwise 3x3 convolution (groups == channels), float16 NHWC, stride 1 or 2: the bandwidth kernel of the
+// MobileNet family.  A thread owns 8 channels of a strip of 4 consecutive output pixels of one row:
+//   * the nine filter taps of its 8 channels are loaded once (weights [tap][C]) instead of once per output pixel;
+//   * per input row the strip needs 6 (stride 1) or 9 (stride 2) 16-byte pixel vectors, each used by up to three
+//     outputs: 4.5 / 6.75 loads per output pixel instead of 9, all of them issued before the first use;
+//   * loads go through a buffer resource, so pixels outside the image are an out-of-range offset that reads zeros:
+//     no branches around the taps.
+// Consecutive lanes take consecutive channel vectors of the same strip, so every load instruction of a wavefront
+// covers whole pixels.
+#include "common.hpp"
+
+namespace msnh {
+
+namespace {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+constexpr unsigned kOob = 0x80000000u;
+
+struct DwArgs
+{
+    const f16 *x;
+    const f16 *w;
+    const float *scale;
+    const float *shift;
+    f16 *y;
+    int H, W, inLd, OH, OW, outLd, C, pad;
+    int strips;             // ceil(OW / 4)
+    long long total;        // B * OH * strips * (C / 8)
+    unsigned xBytes;
+    int act;
+    float actParam, outMul;
+};
+
+template <int STRIDE>
+__global__ __launch_bounds__(256) void convDepthwise3x3Kernel(DwArgs a)
+{
+    constexpr int COLS = 3 * STRIDE + 3;          // input columns feeding 4 outputs: (4 - 1) * STRIDE + 3
+    const long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= a.total) return;
+    const int cv = a.C / 8;
+    const int c0 = static_cast<int>(idx % cv) * 8;
+    long long t = idx / cv;
+    const int sx = static_cast<int>(t % a.strips);
+    t /= a.strips;
+    const int oy = static_cast<int>(t % a.OH);
+    const int b  = static_cast<int>(t / a.OH);
+    const int ox0 = sx * 4;
+    const int iy0 = oy * STRIDE - a.pad;
+    const int ix0 = ox0 * STRIDE - a.pad;
+
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<f16 *>(a.x), 0, static_cast<int>(a.xBytes), 0x00020000);
+
+    f16x8 wv[9];
+#pragma unroll
+    for (int k = 0; k < 9; ++k) wv[k] = *reinterpret_cast<const f16x8 *>(a.w + static_cast<size_t>(k) * a.C + c0);
+
+    // byte offset of input pixel (iy0, ix0), channel c0; may be "negative": it wraps back once a valid tap is added
+    const unsigned base = static_cast<unsigned>(((static_cast<long long>(b) * a.H + iy0) * a.W + ix0) * a.inLd + c0) * 2u;
+    unsigned colOff[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c)
+    {
+        const int ix = ix0 + c;
+        colOff[c] = (ix >= 0 && ix < a.W) ? base + static_cast<unsigned>(c * a.inLd) * 2u : kOob;
+    }
+    float acc[4][8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
+
+    f16x8 xv[3][COLS];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+    {
+        const int iy = iy0 + r;
+        const bool rowOk = iy >= 0 && iy < a.H;
+        const unsigned rowOff = static_cast<unsigned>(r * a.W * a.inLd) * 2u;
+#pragma unroll
+        for (int c = 0; c < COLS; ++c)
+        {
+            const unsigned off = (rowOk && colOff[c] != kOob) ? colOff[c] + rowOff : kOob;
+            xv[r][c] = __builtin_bit_cast(f16x8, __builtin_amdgcn_raw_buffer_load_b128(rx, static_cast<int>(off), 0, 0));
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int kx = 0; kx < 3; ++kx)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    acc[j][e] += static_cast<float>(xv[r][j * STRIDE + kx][e]) * static_cast<float>(wv[r * 3 + kx][e]);
+
+    float sc[8], sh[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+    {
+        sc[e] = a.scale ? a.scale[c0 + e] : 1.f;
+        sh[e] = a.shift ? a.shift[c0 + e] : 0.f;
+    }
+    const size_t prow = (static_cast<size_t>(b) * a.OH + oy) * a.OW;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        if (ox0 + j >= a.OW) break;
+        f16x8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = static_cast<f16>(a.outMul * activate(acc[j][e] * sc[e] + sh[e], a.act, a.actParam));
+        *reinterpret_cast<f16x8 *>(a.y + (prow + ox0 + j) * a.outLd + c0) = o;
+    }
+}
+
+} // namespace
+
+bool depthwise3x3Ok(const msnh_conv_desc *d, const void *x, const void *w, const void *y)
+{
+    const unsigned long long xb = ((static_cast<unsigned long long>(d->batch) * d->in_h * d->in_w - 1) * d->in_ld + d->in_c) * 2ull;
+    return d->dtype == MSNH_F16 && d->out_dtype == MSNH_F16 && d->ksize == 3 && (d->stride == 1 || d->stride == 2) && d->dilation == 1 &&
+           d->groups == d->in_c && d->out_c == d->in_c && d->in_c % 8 == 0 && d->in_ld % 8 == 0 && d->out_ld % 8 == 0 && !d->has_residual &&
+           xb < 0x7fffffffull && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 &&
+           reinterpret_cast<uintptr_t>(y) % 16 == 0;
+}
+
+int convDepthwise3x3(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift, void *y, hipStream_t st)
+{
+    DwArgs a;
+    a.x = static_cast<const f16 *>(x); a.w = static_cast<const f16 *>(w); a.scale = scale; a.shift = shift; a.y = static_cast<f16 *>(y);
+    a.H = d->in_h; a.W = d->in_w; a.inLd = d->in_ld; a.OH = d->out_h; a.OW = d->out_w; a.outLd = d->out_ld; a.C = d->in_c; a.pad = d->pad;
+    a.strips = (d->out_w + 3) / 4;
+    a.total = static_cast<long long>(d->batch) * d->out_h * a.strips * (d->in_c / 8);
+    a.xBytes = static_cast<unsigned>(((static_cast<unsigned long long>(d->batch) * d->in_h * d->in_w - 1) * d->in_ld + d->in_c) * 2ull);
+    a.act = d->act; a.actParam = d->act_param; a.outMul = d->out_mul;
+    const dim3 grid(gridFor(a.total, 256));
+    if (d->stride == 1) hipLaunchKernelGGL(convDepthwise3x3Kernel<1>, grid, dim3(256), 0, st, a);
+    else                hipLaunchKernelGGL(convDepthwise3x3Kernel<2>, grid, dim3(256), 0, st, a);
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+} // namespace msnh

@@ -17,6 +17,8 @@ int convWinograd(const msnh_conv_desc *d, const void *x, const void *w, const fl
 size_t winogradWorkspaceBytes(const msnh_conv_desc *d);
 void   winogradPackWeights(const msnh_conv_desc *d, const float *oihw, void *packed);
 void   winogradGemmDesc(const msnh_conv_desc *d, msnh_conv_desc *gd);
+bool   depthwise3x3Ok(const msnh_conv_desc *d, const void *x, const void *w, const void *y);
+int    convDepthwise3x3(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift, void *y, hipStream_t st);
 bool   stemMfmaOk(const msnh_conv_desc *d);
 size_t stemMfmaElems(const msnh_conv_desc *d);
 void   stemMfmaPack(const msnh_conv_desc *d, const float *oihw, _Float16 *packed);
@@ -339,6 +341,7 @@ int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const
     case MSNH_CONV_DEPTHWISE:
     {
         MSNH_REQUIRE(depthwiseOk(d), "conv2d: not a depthwise convolution");
+        if (depthwise3x3Ok(d, x, w, y)) return convDepthwise3x3(d, x, w, scale, shift, y, st);
         const int C = d->in_c;
         const int vec = d->dtype == MSNH_F16 ? 8 : 4;
         const size_t el = dtypeSize(d->dtype);
