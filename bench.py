@@ -64,6 +64,12 @@ def cpu_baseline(arch, size, tmp, seed, budget_s=30.0):
                       f"({best:.2f} s per image incl. its NMS)"}
 
 
+# HBM bytes per convolution launch (fetch + write), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script,
+# each scaled by what the same counter reads for a plain copy kernel of known size (fetch x2.0, write x1.0); the runs
+# and their summary are in profiles/conv_igemm_yolov3_608_f16_b8.md.  None for workloads that were not profiled.
+HBM_BYTES_PER_CONV_LAUNCH = {("yolov3", "f16", 8): int((39.86 + 17.43) * 2**20)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -141,7 +147,7 @@ def main():
     conv_ms, launches, flops = net.profile_ops(0, 10)
     achieved = flops / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else 0.0
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK[dtype], "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK[dtype], 4), "traffic": None,
+                "frac": round(achieved / PEAK[dtype], 4), "traffic": HBM_BYTES_PER_CONV_LAUNCH.get((a.workload, dtype, batch)),
                 "kernel": "convolution launches (implicit-GEMM MFMA + stem)", "launches_per_step": launches // 10,
                 "avg_launch_us": round(conv_ms * 1e3 / max(launches, 1), 2), "flops_per_step": flops / 10}
 
