@@ -2,6 +2,7 @@
 // Control flow and error texts follow src/net/MsnhNetBuilder.cpp of the reference (build :68-622, load :624-663,
 // run :820-1007); what happens underneath -- one planned device arena, fused launches, a captured graph --
 // is new.
+#include <cstdlib>
 #include "Msnhnet/net/MsnhNetBuilder.h"
 #include <cmath>
 #include <cstring>
@@ -462,7 +463,14 @@ void NetBuilder::enqueueForward(const float *deviceInput)
     if (yout && _inFlight >= 2) MSNH_THROW("two forwards are already in flight: fetch a result first");
     if (deviceInput != nullptr && deviceInput != _inputDev.as<float>())
         MSNH_DEV(msnh_hip_memcpy_d2d(_inputDev.ptr(), deviceInput, sizeof(float) * static_cast<size_t>(_net->inputNum), _stream));
-    if (_graph == nullptr)
+    static const bool eager = std::getenv("MSNH_EAGER") != nullptr;
+    if (eager)
+    {
+        if (plan.yoloCandCnt.ptr()) MSNH_DEV(msnh_hip_fill_zero(plan.yoloCandCnt.ptr(), plan.yoloCandCnt.bytes(), _stream));
+        plan.runAll(_stream);
+        if (yout) yout->enqueueGather(_stream);
+    }
+    else if (_graph == nullptr)
     {
         // Record the whole forward once; later calls replay it with a single launch.
         MSNH_DEV(msnh_hip_graph_begin(_stream));
@@ -481,7 +489,7 @@ void NetBuilder::enqueueForward(const float *deviceInput)
         }
         MSNH_DEV(msnh_hip_graph_end(_stream, &_graph));
     }
-    MSNH_DEV(msnh_hip_graph_launch(_graph, _stream));
+    if (!eager) MSNH_DEV(msnh_hip_graph_launch(_graph, _stream));
     if (yout)
     {
         // results leave the device right behind the forward, so the next forward can start while the host sorts
