@@ -79,6 +79,7 @@ int msnh_hip_stream_sync(msnh_stream_t s);
 int msnh_hip_event_create(msnh_event_t *e);
 int msnh_hip_event_destroy(msnh_event_t e);
 int msnh_hip_event_record(msnh_event_t e, msnh_stream_t s);
+int msnh_hip_stream_wait_event(msnh_stream_t s, msnh_event_t e);   /* work queued on s afterwards starts once e has fired */
 int msnh_hip_event_sync(msnh_event_t e);
 int msnh_hip_event_elapsed_ms(msnh_event_t start, msnh_event_t stop, float *ms);
 /* Stream capture into a replayable graph: every kernel launched on `s` between begin and end is

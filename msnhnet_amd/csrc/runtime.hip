@@ -182,6 +182,13 @@ int msnh_hip_event_record(msnh_event_t e, msnh_stream_t s)
     return 0;
 }
 
+int msnh_hip_stream_wait_event(msnh_stream_t s, msnh_event_t e)
+{
+    MSNH_REQUIRE(e != nullptr, "event is NULL");
+    MSNH_HIP_CHECK(hipStreamWaitEvent(resolveStream(s), static_cast<hipEvent_t>(e), 0));
+    return 0;
+}
+
 int msnh_hip_event_sync(msnh_event_t e)
 {
     MSNH_REQUIRE(e != nullptr, "event is NULL");

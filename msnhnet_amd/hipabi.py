@@ -35,7 +35,7 @@ SYMBOLS = [
     "msnh_hip_last_error", "msnh_hip_init", "msnh_hip_device_count", "msnh_hip_device_name", "msnh_hip_malloc", "msnh_hip_free",
     "msnh_hip_host_alloc", "msnh_hip_host_free", "msnh_hip_memcpy_h2d", "msnh_hip_memcpy_d2h", "msnh_hip_memcpy_d2d",
     "msnh_hip_fill_zero", "msnh_hip_stream_create", "msnh_hip_stream_destroy", "msnh_hip_stream_sync", "msnh_hip_event_create",
-    "msnh_hip_event_destroy", "msnh_hip_event_record", "msnh_hip_event_sync", "msnh_hip_event_elapsed_ms", "msnh_hip_graph_begin",
+    "msnh_hip_event_destroy", "msnh_hip_event_record", "msnh_hip_stream_wait_event", "msnh_hip_event_sync", "msnh_hip_event_elapsed_ms", "msnh_hip_graph_begin",
     "msnh_hip_graph_end", "msnh_hip_graph_launch", "msnh_hip_graph_destroy", "msnh_hip_conv2d_tile_count", "msnh_hip_conv2d_tile_supported", "msnh_hip_conv2d_select_algo",
     "msnh_hip_conv2d_packed_weight_elems", "msnh_hip_conv2d_pack_weights", "msnh_hip_conv2d_workspace_bytes", "msnh_hip_conv2d",
     "msnh_hip_affine_act", "msnh_hip_add_act", "msnh_hip_copy_channels", "msnh_hip_maxpool", "msnh_hip_avgpool",
@@ -71,6 +71,7 @@ def lib():
     L.msnh_hip_event_create.argtypes = [ctypes.POINTER(vp)]
     L.msnh_hip_event_destroy.argtypes = [vp]
     L.msnh_hip_event_record.argtypes = [vp, vp]
+    L.msnh_hip_stream_wait_event.argtypes = [vp, vp]
     L.msnh_hip_event_sync.argtypes = [vp]
     L.msnh_hip_event_elapsed_ms.argtypes = [vp, vp, fp]
     L.msnh_hip_graph_begin.argtypes = [vp]

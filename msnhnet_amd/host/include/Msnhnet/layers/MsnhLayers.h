@@ -263,7 +263,10 @@ private:
     std::vector<int> _yoloIndexes;
     std::vector<YoloInfo> _yoloLayersInfo;
     int _yoloAllInputNum = 0, _pixels = 0;
-    struct Slot { PinnedBuffer cnt, rows, decoded; msnh_event_t event = nullptr; bool pending = false; };
+    // devCnt / devRows: device-side snapshot of one forward's candidates, so the copy to the host can run on its own
+    // stream while the next forward already overwrites the plan's buffers
+    struct Slot { PinnedBuffer cnt, rows, decoded; DeviceBuffer devCnt, devRows; msnh_event_t event = nullptr, ready = nullptr; bool pending = false; };
+    msnh_stream_t _copyStream = nullptr;
     Slot _slots[2];
 };
 }

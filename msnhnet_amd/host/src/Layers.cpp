@@ -977,15 +977,33 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
     sl.cnt.reserve(sizeof(int) * static_cast<size_t>(_batch));
     sl.rows.reserve(sizeof(float) * 8 * cells * static_cast<size_t>(_batch));
     if (sl.event == nullptr) MSNH_DEV(msnh_hip_event_create(&sl.event));
-    MSNH_DEV(msnh_hip_memcpy_d2h(sl.cnt.ptr(), pl.yoloCandCnt.ptr(), sizeof(int) * static_cast<size_t>(_batch), s));
-    MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.ptr(), pl.yoloRows.ptr(), sizeof(float) * 8 * cells * static_cast<size_t>(_batch), s));
+    const size_t cntBytes = sizeof(int) * static_cast<size_t>(_batch);
+    const size_t rowBytes = sizeof(float) * 8 * cells * static_cast<size_t>(_batch);
     if (keepClassScores)
     {
+        // the decoded tensor is too large to snapshot: everything leaves on the forward's own stream
+        MSNH_DEV(msnh_hip_memcpy_d2h(sl.cnt.ptr(), pl.yoloCandCnt.ptr(), cntBytes, s));
+        MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.ptr(), pl.yoloRows.ptr(), rowBytes, s));
         const size_t bytes = sizeof(float) * cells * static_cast<size_t>(_channel) * static_cast<size_t>(_batch);
         sl.decoded.reserve(bytes);
         MSNH_DEV(msnh_hip_memcpy_d2h(sl.decoded.ptr(), pl.yoloDecoded.ptr(), bytes, s));
+        MSNH_DEV(msnh_hip_event_record(sl.event, s));
+        sl.pending = true;
+        return;
     }
-    MSNH_DEV(msnh_hip_event_record(sl.event, s));
+    // Snapshot on the device (microseconds), then cross PCIe on a second stream: the next forward does not wait for
+    // the copy (several MiB: every cell has a row slot, the count is only known on the device).
+    if (_copyStream == nullptr) MSNH_DEV(msnh_hip_stream_create(&_copyStream));
+    if (sl.ready == nullptr) MSNH_DEV(msnh_hip_event_create(&sl.ready));
+    if (sl.devCnt.bytes() < cntBytes) sl.devCnt.alloc(cntBytes);
+    if (sl.devRows.bytes() < rowBytes) sl.devRows.alloc(rowBytes);
+    MSNH_DEV(msnh_hip_memcpy_d2d(sl.devCnt.ptr(), pl.yoloCandCnt.ptr(), cntBytes, s));
+    MSNH_DEV(msnh_hip_memcpy_d2d(sl.devRows.ptr(), pl.yoloRows.ptr(), rowBytes, s));
+    MSNH_DEV(msnh_hip_event_record(sl.ready, s));
+    MSNH_DEV(msnh_hip_stream_wait_event(_copyStream, sl.ready));
+    MSNH_DEV(msnh_hip_memcpy_d2h(sl.cnt.ptr(), sl.devCnt.ptr(), cntBytes, _copyStream));
+    MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.ptr(), sl.devRows.ptr(), rowBytes, _copyStream));
+    MSNH_DEV(msnh_hip_event_record(sl.event, _copyStream));
     sl.pending = true;
 }
 
@@ -1025,6 +1043,10 @@ void YoloOutLayer::forwardGPU(NetworkState &netState)
 YoloOutLayer::~YoloOutLayer()
 {
     for (Slot &sl : _slots)
+    {
         if (sl.event) msnh_hip_event_destroy(sl.event);
+        if (sl.ready) msnh_hip_event_destroy(sl.ready);
+    }
+    if (_copyStream) msnh_hip_stream_destroy(_copyStream);
 }
 }
