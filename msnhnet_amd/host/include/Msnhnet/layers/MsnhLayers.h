@@ -255,6 +255,8 @@ public:
 
     // host post-processing of the compacted candidate rows of one image (8 floats per row, see msnh_hip_yolo_gather)
     std::vector<YoloBox> boxesFromRows(const float *rows, int count, const float *decodedOfImage) const;
+    static std::vector<std::vector<int>> groupByClass(const std::vector<YoloBox> &bboxes);
+    static void nmsClass(const std::vector<YoloBox> &bboxes, std::vector<int> &members, float nmsThresh);
 
 private:
     float _confThresh, _nmsThresh;

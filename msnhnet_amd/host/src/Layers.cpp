@@ -905,60 +905,72 @@ std::vector<YoloBox> YoloOutLayer::nms(const std::vector<YoloBox> &bboxes, const
 // erased it.  The kept boxes are held as structure-of-arrays so the IoU test runs 8 wide.
 std::vector<YoloBox> YoloOutLayer::nmsSorted(const std::vector<YoloBox> &bboxes, float nmsThresh)
 {
-    const size_t n = bboxes.size();
     std::vector<YoloBox> best;
-    if (n == 0) return best;
+    if (bboxes.empty()) return best;
+    std::vector<std::vector<int>> members = groupByClass(bboxes);
+    best.reserve(bboxes.size());
+    for (std::vector<int> &m : members)
+    {
+        nmsClass(bboxes, m, nmsThresh);
+        for (int j : m) best.push_back(bboxes[static_cast<size_t>(j)]);
+    }
+    return best;
+}
+
+// indices of the candidates of each class, classes in first-appearance order
+std::vector<std::vector<int>> YoloOutLayer::groupByClass(const std::vector<YoloBox> &bboxes)
+{
     int maxCls = 0;
     for (const YoloBox &b : bboxes) maxCls = std::max(maxCls, b.bestClsIdx);
-    std::vector<int> firstSeen;                                   // classes in first-appearance order
     std::vector<int> slotOf(static_cast<size_t>(maxCls) + 1, -1);
     std::vector<std::vector<int>> members;
-    for (size_t i = 0; i < n; ++i)
+    for (size_t i = 0; i < bboxes.size(); ++i)
     {
         const int c = bboxes[i].bestClsIdx;
         if (c < 0) MSNH_THROW("negative class index");
         if (slotOf[static_cast<size_t>(c)] < 0)
         {
-            slotOf[static_cast<size_t>(c)] = static_cast<int>(firstSeen.size());
-            firstSeen.push_back(c);
+            slotOf[static_cast<size_t>(c)] = static_cast<int>(members.size());
             members.emplace_back();
         }
         members[static_cast<size_t>(slotOf[static_cast<size_t>(c)])].push_back(static_cast<int>(i));
     }
-    best.reserve(n);
+    return members;
+}
+
+// greedy NMS inside one class: on return m holds the kept candidates in pick order
+void YoloOutLayer::nmsClass(const std::vector<YoloBox> &bboxes, std::vector<int> &m, float nmsThresh)
+{
+    if (m.size() <= 1) return;
+    std::stable_sort(m.begin(), m.end(), [&bboxes](int a, int b) { return bboxes[static_cast<size_t>(a)].conf > bboxes[static_cast<size_t>(b)].conf; });
     std::vector<float> kx1, ky1, kx2, ky2, karea;
-    for (std::vector<int> &m : members)
+    size_t w = 0;
+    for (int j : m)
     {
-        if (m.size() == 1) { best.push_back(bboxes[static_cast<size_t>(m[0])]); continue; }
-        std::stable_sort(m.begin(), m.end(), [&bboxes](int a, int b) { return bboxes[static_cast<size_t>(a)].conf > bboxes[static_cast<size_t>(b)].conf; });
-        kx1.clear(); ky1.clear(); kx2.clear(); ky2.clear(); karea.clear();
-        for (int j : m)
-        {
-            const Box::XYWHBox &q = bboxes[static_cast<size_t>(j)].xywhBox;
-            const float jx1 = q.x - q.w / 2.f, jx2 = q.x + q.w / 2.f, jy1 = q.y - q.h / 2.f, jy2 = q.y + q.h / 2.f;
-            const float jarea = (jx2 - jx1 + 1) * (jy2 - jy1 + 1);
-            const size_t nk = kx1.size();
-            int hit = 0;
+        const Box::XYWHBox &q = bboxes[static_cast<size_t>(j)].xywhBox;
+        const float jx1 = q.x - q.w / 2.f, jx2 = q.x + q.w / 2.f, jy1 = q.y - q.h / 2.f, jy2 = q.y + q.h / 2.f;
+        const float jarea = (jx2 - jx1 + 1) * (jy2 - jy1 + 1);
+        const size_t nk = kx1.size();
+        int hit = 0;
 #pragma omp simd reduction(| : hit)
-            for (size_t k = 0; k < nk; ++k)
-            {
-                // Box::iou(candidate j, kept k) with std::min / std::max spelled out
-                const float ix2 = (kx2[k] < jx2) ? kx2[k] : jx2;
-                const float ix1 = (jx1 < kx1[k]) ? kx1[k] : jx1;
-                const float iy2 = (ky2[k] < jy2) ? ky2[k] : jy2;
-                const float iy1 = (jy1 < ky1[k]) ? ky1[k] : jy1;
-                const float iw = ix2 - ix1 + 1;
-                const float ih = iy2 - iy1 + 1;
-                const float inter = (iw < 0 ? 0 : iw) * (ih < 0 ? 0 : ih);
-                const float iou = 1.f * inter / (jarea + karea[k] - inter);
-                hit |= (iou > nmsThresh) ? 1 : 0;
-            }
-            if (hit) continue;
-            best.push_back(bboxes[static_cast<size_t>(j)]);
-            kx1.push_back(jx1); ky1.push_back(jy1); kx2.push_back(jx2); ky2.push_back(jy2); karea.push_back(jarea);
+        for (size_t k = 0; k < nk; ++k)
+        {
+            // Box::iou(candidate j, kept k) with std::min / std::max spelled out
+            const float ix2 = (kx2[k] < jx2) ? kx2[k] : jx2;
+            const float ix1 = (jx1 < kx1[k]) ? kx1[k] : jx1;
+            const float iy2 = (ky2[k] < jy2) ? ky2[k] : jy2;
+            const float iy1 = (jy1 < ky1[k]) ? ky1[k] : jy1;
+            const float iw = ix2 - ix1 + 1;
+            const float ih = iy2 - iy1 + 1;
+            const float inter = (iw < 0 ? 0 : iw) * (ih < 0 ? 0 : ih);
+            const float iou = 1.f * inter / (jarea + karea[k] - inter);
+            hit |= (iou > nmsThresh) ? 1 : 0;
         }
+        if (hit) continue;
+        m[w++] = j;
+        kx1.push_back(jx1); ky1.push_back(jy1); kx2.push_back(jx2); ky2.push_back(jy2); karea.push_back(jarea);
     }
-    return best;
+    m.resize(w);
 }
 
 void YoloOutLayer::enqueueGather(msnh_stream_t s)
@@ -1021,13 +1033,38 @@ void YoloOutLayer::finish(int slot)
     const float *decodedHost = keepClassScores ? sl.decoded.as<float>() : nullptr;
     batchHasBox.assign(static_cast<size_t>(_batch), false);
     finalOut.assign(static_cast<size_t>(_batch), std::vector<YoloBox>());
+    // three flat parallel phases: candidates per image; NMS per (image, class) -- the classes of an image are
+    // independent, and a batch has far fewer images than the host has cores; concatenation per image
+    std::vector<std::vector<YoloBox>> cand(static_cast<size_t>(_batch));
+    std::vector<std::vector<std::vector<int>>> groups(static_cast<size_t>(_batch));
 #pragma omp parallel for schedule(dynamic)
     for (int b = 0; b < _batch; ++b)
     {
         const int n = std::min(cnt[b], cells);
         const float *dec = decodedHost ? decodedHost + static_cast<size_t>(b) * cells * per : nullptr;
-        std::vector<YoloBox> cand = boxesFromRows(sl.rows.as<float>() + static_cast<size_t>(b) * cells * 8, n, dec);
-        finalOut[static_cast<size_t>(b)] = _useSoftNms ? nms(cand, _nmsThresh, true) : nmsSorted(cand, _nmsThresh);
+        cand[static_cast<size_t>(b)] = boxesFromRows(sl.rows.as<float>() + static_cast<size_t>(b) * cells * 8, n, dec);
+        if (_useSoftNms) finalOut[static_cast<size_t>(b)] = nms(cand[static_cast<size_t>(b)], _nmsThresh, true);
+        else groups[static_cast<size_t>(b)] = groupByClass(cand[static_cast<size_t>(b)]);
+    }
+    if (!_useSoftNms)
+    {
+        std::vector<std::pair<int, int>> tasks;
+        for (int b = 0; b < _batch; ++b)
+            for (size_t g = 0; g < groups[static_cast<size_t>(b)].size(); ++g) tasks.emplace_back(b, static_cast<int>(g));
+        const int nTasks = static_cast<int>(tasks.size());
+#pragma omp parallel for schedule(dynamic, 4)
+        for (int t = 0; t < nTasks; ++t)
+        {
+            const size_t b = static_cast<size_t>(tasks[static_cast<size_t>(t)].first);
+            nmsClass(cand[b], groups[b][static_cast<size_t>(tasks[static_cast<size_t>(t)].second)], _nmsThresh);
+        }
+#pragma omp parallel for schedule(dynamic)
+        for (int b = 0; b < _batch; ++b)
+        {
+            std::vector<YoloBox> &out = finalOut[static_cast<size_t>(b)];
+            for (const std::vector<int> &m : groups[static_cast<size_t>(b)])
+                for (int j : m) out.push_back(cand[static_cast<size_t>(b)][static_cast<size_t>(j)]);
+        }
     }
     for (int b = 0; b < _batch; ++b) batchHasBox[static_cast<size_t>(b)] = cnt[b] > 0;
     if (std::getenv("MSNH_DEBUG_TIMING")) std::fprintf(stderr, "yoloout finish: wait %.3f ms, host %.3f ms\n", dbgWait, TimeUtil::getElapsedTime(dbg0) - dbgWait);
