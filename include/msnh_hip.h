@@ -191,6 +191,12 @@ int msnh_hip_nchw_to_nhwc(int out_dtype, int batch, int c, int h, int w, const f
 int msnh_hip_nhwc_to_nchw(int dtype, int batch, int c, int h, int w, const void *x, int x_ld, float mul, float *y_nchw,
                           msnh_stream_t s);
 
+/* Letterbox of one 8-bit RGB image (HWC, device memory) into the network's NCHW float32 input: pad to a square with
+ * 127, bilinear resize, optional R<->B swap, scale to [0,1] (half_init 0) or [-1,1].  Replaces
+ * CVUtil::getPaddingZeroF32C3 (src/utils/MsnhCVUtil.cpp:203-261) + the host-to-device copy of the float image. */
+int msnh_hip_letterbox_u8(const unsigned char *rgb_hwc, int width, int height, int net_w, int net_h, int half_init,
+                          int shuffle_rgb, float *out_chw, msnh_stream_t s);
+
 /* ------------------------------------------------------------------------------------------------
  * YOLO.  One launch per head replaces YoloLayer::forwardGPU's 15 launches (exSigmoidKernel, aExpTKernel,
  * sigmoidKernel: src/layers/cuda/MsnhYoloLayerGPU.cu:4-54, src/layers/MsnhYoloLayer.cpp:164-185) and

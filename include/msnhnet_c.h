@@ -101,6 +101,16 @@ float msnhnet_gpu_inference_time(msnhnet_t net);          /* NetBuilder::getGpuI
  * bestClsIdx), already in the order the layer would pass them; fast = 0 runs the reference-shaped greedy loop,
  * fast = 1 the sorted variant the library uses.  Writes at most cap rows, *n_out = number of surviving boxes. */
 int msnhnet_nms(const float *rows, long long n, float nms_thresh, int fast, float *out, long long cap, long long *n_out);
+
+/* The step either side of the graph.
+ * msnhnet_set_input_image_u8: letterbox one 8-bit RGB image (HWC, host memory) on the device into slot `index` of the
+ *   input batch -- CVUtil::getPaddingZeroF32C3 (src/utils/MsnhCVUtil.cpp:203-261) fused with the upload; run with
+ *   msnhnet_enqueue(net, NULL) afterwards.
+ * msnhnet_boxes_to_image: boxes (rows of 7 floats as returned by the run / fetch calls) from network-input pixels back
+ *   to the original image -- YoloOutLayer::bboxResize2Org (padded != 0) / bboxResize2OrgNoPad
+ *   (src/layers/MsnhYoloOutLayer.cpp:321-379). */
+int msnhnet_set_input_image_u8(msnhnet_t net, int index, const unsigned char *rgb_hwc, int width, int height, int half_init, int shuffle_rgb);
+int msnhnet_boxes_to_image(float *boxes, long long count, int net_w, int net_h, int org_w, int org_h, int padded);
 long long msnhnet_time_detail(msnhnet_t net, char *dst, long long cap);       /* NetBuilder::getTimeDetail */
 
 #ifdef __cplusplus

@@ -243,6 +243,9 @@ public:
     static std::vector<YoloBox> nms(const std::vector<YoloBox> &bboxes, const float &nmsThresh, const bool &useSoftNms, const float &sigma = 0.3f);
     // hard NMS with the same result as nms(), restructured for speed (see the definition)
     static std::vector<YoloBox> nmsSorted(const std::vector<YoloBox> &bboxes, float nmsThresh);
+    // boxes from network-input pixels back to the original image (reference: MsnhYoloOutLayer.cpp:321-379)
+    static YoloBox bboxResize2Org(YoloBox &box, const Point2I &currentShape, const Point2I &orgShape);
+    static YoloBox bboxResize2OrgNoPad(YoloBox &box, const Point2I &currentShape, const Point2I &orgShape);
     float getConfThresh() const { return _confThresh; }
     float getNmsThresh() const { return _nmsThresh; }
     int   getUseSoftNms() const { return _useSoftNms; }

@@ -50,6 +50,10 @@ public:
     std::vector<float> fetchClassify();
     std::vector<std::vector<YoloBox>> fetchYolo();
     float *deviceInputBuffer();               // the builder's own device input buffer (batch*C*H*W floats)
+    // Letterboxes one 8-bit RGB image (HWC, host memory) on the device into slot `index` of the input batch: what
+    // CVUtil::getPaddingZeroF32C3 + the float upload do in the reference (MsnhCVUtil.cpp:203-261); then
+    // enqueueForward(nullptr) runs on it.
+    void setInputImageU8(int index, const unsigned char *rgbHwc, int width, int height, bool halfInit = false, bool shuffleRGB = false);
 
     Point2I getInputSize();
     int getInputChannel();
@@ -97,7 +101,8 @@ private:
     bool   _saveLayerOutput = false, _saveLayerWeights = false, _writeDumpFiles = false;
     bool   _planReady = false;
     std::vector<std::vector<float>> _layerOutputs;
-    DeviceBuffer _inputDev;
+    DeviceBuffer _inputDev, _imageDev;
+    PinnedBuffer _imagePinned;
     PinnedBuffer _inputPinned, _outputPinned;
     msnh_stream_t _stream = nullptr;
     msnh_graph_t  _graph = nullptr;

@@ -347,6 +347,27 @@ long long msnhnet_yolo_max_boxes(msnhnet_t net)
     return n;
 }
 
+int msnhnet_set_input_image_u8(msnhnet_t net, int index, const unsigned char *rgb_hwc, int width, int height, int half_init, int shuffle_rgb)
+{
+    return guarded([&] { nb(net).setInputImageU8(index, rgb_hwc, width, height, half_init != 0, shuffle_rgb != 0); });
+}
+
+int msnhnet_boxes_to_image(float *boxes, long long count, int net_w, int net_h, int org_w, int org_h, int padded)
+{
+    return guarded([&] {
+        if (count < 0 || (count > 0 && boxes == nullptr) || net_w <= 0 || net_h <= 0 || org_w <= 0 || org_h <= 0) MSNH_THROW("bad argument");
+        for (long long i = 0; i < count; ++i)
+        {
+            float *r = boxes + 7 * i;
+            YoloBox b;
+            b.xywhBox = Box::XYWHBox(r[0], r[1], r[2], r[3]);
+            if (padded) YoloOutLayer::bboxResize2Org(b, Point2I(net_w, net_h), Point2I(org_w, org_h));
+            else        YoloOutLayer::bboxResize2OrgNoPad(b, Point2I(net_w, net_h), Point2I(org_w, org_h));
+            r[0] = b.xywhBox.x; r[1] = b.xywhBox.y; r[2] = b.xywhBox.w; r[3] = b.xywhBox.h;
+        }
+    });
+}
+
 int msnhnet_nms(const float *rows, long long n, float nms_thresh, int fast, float *out, long long cap, long long *n_out)
 {
     return guarded([&] {

@@ -973,6 +973,43 @@ void YoloOutLayer::nmsClass(const std::vector<YoloBox> &bboxes, std::vector<int>
     m.resize(w);
 }
 
+// Undo the letterbox (square padding + uniform scale): the padding is on the short side of the original image.
+YoloBox YoloOutLayer::bboxResize2Org(YoloBox &box, const Point2I &currentShape, const Point2I &orgShape)
+{
+    const int orgW = orgShape.x, orgH = orgShape.y, curW = currentShape.x, curH = currentShape.y;
+    if (orgW > orgH)
+    {
+        const float ratio = 1.0f * curW / orgW;
+        const int padUp = static_cast<int>((curH - orgH * ratio) / 2);
+        box.xywhBox.x = box.xywhBox.x / ratio;
+        box.xywhBox.w = box.xywhBox.w / ratio;
+        box.xywhBox.y = (box.xywhBox.y - padUp) / ratio;
+        box.xywhBox.h = box.xywhBox.h / ratio;
+    }
+    else
+    {
+        const float ratio = 1.0f * curH / orgH;
+        const int padLeft = static_cast<int>((curW - orgW * ratio) / 2);
+        box.xywhBox.x = (box.xywhBox.x - padLeft) / ratio;
+        box.xywhBox.w = box.xywhBox.w / ratio;
+        box.xywhBox.y = box.xywhBox.y / ratio;
+        box.xywhBox.h = box.xywhBox.h / ratio;
+    }
+    return box;
+}
+
+// Undo a plain resize that did not keep the aspect ratio.
+YoloBox YoloOutLayer::bboxResize2OrgNoPad(YoloBox &box, const Point2I &currentShape, const Point2I &orgShape)
+{
+    const float ratioW = 1.0f * currentShape.x / orgShape.x;
+    const float ratioH = 1.0f * currentShape.y / orgShape.y;
+    box.xywhBox.x = box.xywhBox.x / ratioW;
+    box.xywhBox.w = box.xywhBox.w / ratioW;
+    box.xywhBox.y = box.xywhBox.y / ratioH;
+    box.xywhBox.h = box.xywhBox.h / ratioH;
+    return box;
+}
+
 void YoloOutLayer::enqueueGather(msnh_stream_t s)
 {
     if (plan == nullptr) MSNH_THROW("YoloOut: layer is not part of a planned network");

@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libMsnhnet.so")
 
 SYMBOLS = [
     "initMsnhnet", "buildMsnhnet", "runClassifyNoPred", "runYoloNoPred", "dispose", "withGPU", "withCUDNN", "getCpuForwardTime",
-    "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16", "msnhnet_set_use_winograd",
+    "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16", "msnhnet_set_use_winograd", "msnhnet_set_input_image_u8", "msnhnet_boxes_to_image",
     "msnhnet_set_keep_class_scores", "msnhnet_set_save_layer_output", "msnhnet_build", "msnhnet_load", "msnhnet_load_from_memory",
     "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops",
     "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
@@ -66,6 +66,8 @@ def lib():
     L.msnhnet_destroy.argtypes = [vp]
     L.msnhnet_set_use_fp16.argtypes = [ci]
     L.msnhnet_set_use_winograd.argtypes = [ci]
+    L.msnhnet_set_input_image_u8.argtypes = [vp, ci, ctypes.POINTER(ctypes.c_ubyte), ci, ci, ci, ci]
+    L.msnhnet_boxes_to_image.argtypes = [fp, ll, ci, ci, ci, ci, ci]
     L.msnhnet_set_keep_class_scores.argtypes = [ci]
     L.msnhnet_set_save_layer_output.argtypes = [vp, ci]
     L.msnhnet_build.argtypes = [vp, cp]
@@ -112,6 +114,13 @@ def _fp(a):
 
 def set_use_fp16(on):
     _check(lib().msnhnet_set_use_fp16(1 if on else 0))
+
+
+def boxes_to_image(boxes, net_w, net_h, org_w, org_h, padded=True):
+    """rows of 7 floats (x y w h conf clsConf cls) from network-input pixels to original-image pixels; returns a copy"""
+    b = np.ascontiguousarray(boxes, np.float32).reshape(-1, 7).copy()
+    _check(lib().msnhnet_boxes_to_image(_fp(b), len(b), net_w, net_h, org_w, org_h, int(padded)))
+    return b
 
 
 def set_use_winograd(on):
@@ -266,6 +275,15 @@ class Net:
 
     def fetch_yolo(self):
         return self._boxes(self.L.msnhnet_fetch_yolo)
+
+    def set_input_image_u8(self, index, img, half_init=False, shuffle_rgb=False):
+        """img: HWC uint8, 3 channels; letterboxed on the device into slot `index` of the input batch."""
+        a = np.ascontiguousarray(img, np.uint8)
+        h, w, c = a.shape
+        if c != 3:
+            raise ValueError("3-channel image expected")
+        _check(self.L.msnhnet_set_input_image_u8(self.h, index, a.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte)), w, h,
+                                                 int(half_init), int(shuffle_rgb)))
 
     def profile_ops(self, kind, reps):
         """-> (total ms, launches, algorithmic FLOPs) of `reps` eager passes over the launches of one kind (-1 = all)."""

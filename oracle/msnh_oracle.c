@@ -387,3 +387,100 @@ long long msnh_or_yolo_out(const float *const *heads, const int *hw, int nHeads,
     free(cls); free(done); free(cand);
     return nOut;
 }
+
+/* ---- pre / post-processing around the graph ------------------------------------------------------------------- */
+
+/* CVUtil::getPaddingZeroF32C3 for a 3-channel 8-bit image (src/utils/MsnhCVUtil.cpp:203-261):
+ *   - pad the shorter side to a square with (127,127,127): top/left = diff/2, bottom/right = diff - diff/2
+ *     (:216-225; MatOp::copyMakeBorder, include/Msnhnet/cv/MsnhCVMatOp.h:18-54);
+ *   - MatOp::resize to (netW, netH), bilinear, MAT_RGB_U8 branch (src/cv/MsnhCVMatOp.cpp:142-160, 404-437): no resize
+ *     when the size already matches (:152-156); source coordinate (i+0.5)*f-0.5 clamped below at 0 only; second
+ *     sample index min(i0+1, n-1); weights (i1 - s) and (s - i0), which sum to 0 where i1 == i0 (the reference's
+ *     behaviour when enlarging: the last rows/columns come out 0); float arithmetic in the order written there,
+ *     truncation to uint16 and a clamp at 255;
+ *   - cvtColor RGB2BGR when asked (:232-233);
+ *   - v/255 or (v-127.5)/127.5, HWC -> CHW (:243-257). */
+void msnh_or_letterbox_u8(const unsigned char *img, int width, int height, int netW, int netH, int halfInit,
+                          int shuffleRGB, float *out)
+{
+    const int diff = abs(width - height);
+    const int top = width > height ? diff / 2 : 0;
+    const int left = width < height ? diff / 2 : 0;
+    const int S = width > height ? width : height;
+    unsigned char *sq = (unsigned char *)malloc((size_t)S * S * 3);
+    memset(sq, 127, (size_t)S * S * 3);
+    for (int y = 0; y < height; ++y)
+        memcpy(sq + ((size_t)(y + top) * S + left) * 3, img + (size_t)y * width * 3, (size_t)width * 3);
+
+    unsigned char *rs = sq;
+    if (!(netW == S && netH == S))
+    {
+        rs = (unsigned char *)calloc((size_t)netW * netH * 3, 1);
+        const float fx = 1.f * S / netW;
+        const float fy = 1.f * S / netH;
+        for (int i = 0; i < netH; ++i)
+        {
+            float sh = (i + 0.5f) * fy - 0.5f;
+            sh = sh < 0 ? 0 : sh;
+            const int h0 = (int)sh;
+            const int h1 = h0 + 1 < S - 1 ? h0 + 1 : S - 1;
+            for (int j = 0; j < netW; ++j)
+            {
+                float sw = (j + 0.5f) * fx - 0.5f;
+                sw = sw < 0 ? 0 : sw;
+                const int w0 = (int)sw;
+                const int w1 = w0 + 1 < S - 1 ? w0 + 1 : S - 1;
+                for (int k = 0; k < 3; ++k)
+                {
+                    const float v = (h1 - sh) * ((w1 - sw) * sq[3 * ((size_t)h0 * S + w0) + k] + (sw - w0) * sq[3 * ((size_t)h0 * S + w1) + k]) +
+                                    (sh - h0) * ((w1 - sw) * sq[3 * ((size_t)h1 * S + w0) + k] + (sw - w0) * sq[3 * ((size_t)h1 * S + w1) + k]);
+                    const unsigned short r = (unsigned short)v;
+                    rs[3 * ((size_t)i * netW + j) + k] = (unsigned char)(r > 255 ? 255 : r);
+                }
+            }
+        }
+    }
+    for (int y = 0; y < netH; ++y)
+        for (int k = 0; k < 3; ++k)
+            for (int x = 0; x < netW; ++x)
+            {
+                const unsigned char u = rs[3 * ((size_t)y * netW + x) + (shuffleRGB ? 2 - k : k)];
+                out[(size_t)k * netW * netH + (size_t)y * netW + x] = halfInit ? (u - 127.5f) / 127.5f : u / 255.0f;
+            }
+    if (rs != sq) free(rs);
+    free(sq);
+}
+
+/* YoloOutLayer::bboxResize2Org (src/layers/MsnhYoloOutLayer.cpp:321-361): undo the letterbox */
+void msnh_or_bbox_resize2org(float *b, int curW, int curH, int orgW, int orgH)
+{
+    if (orgW > orgH)
+    {
+        const float scaledRatio = 1.0f * curW / orgW;
+        const int padUp = (int)((curH - orgH * scaledRatio) / 2);
+        b[0] = b[0] / scaledRatio;
+        b[2] = b[2] / scaledRatio;
+        b[1] = (b[1] - padUp) / scaledRatio;
+        b[3] = b[3] / scaledRatio;
+    }
+    else
+    {
+        const float scaledRatio = 1.0f * curH / orgH;
+        const int padLeft = (int)((curW - orgW * scaledRatio) / 2);
+        b[0] = (b[0] - padLeft) / scaledRatio;
+        b[2] = b[2] / scaledRatio;
+        b[1] = b[1] / scaledRatio;
+        b[3] = b[3] / scaledRatio;
+    }
+}
+
+/* YoloOutLayer::bboxResize2OrgNoPad (:363-379): undo a plain (aspect-changing) resize */
+void msnh_or_bbox_resize2org_nopad(float *b, int curW, int curH, int orgW, int orgH)
+{
+    const float scaledRatioW = 1.0f * curW / orgW;
+    const float scaledRatioH = 1.0f * curH / orgH;
+    b[0] = b[0] / scaledRatioW;
+    b[2] = b[2] / scaledRatioW;
+    b[1] = b[1] / scaledRatioH;
+    b[3] = b[3] / scaledRatioH;
+}

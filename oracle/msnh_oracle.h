@@ -51,6 +51,15 @@ float msnh_or_iou(const float *xywh1, const float *xywh2);
 long long msnh_or_yolo_out(const float *const *heads, const int *hw, int nHeads, int classNum, float confThresh,
                            float nmsThresh, float *boxes, long long capBoxes);
 
+/* The step either side of the graph.
+ * Letterbox of one 3-channel 8-bit HWC image to the network input: pad to a square with 127, bilinear resize,
+ * optional R<->B swap, scale to [0,1] (half_init 0) or [-1,1] (half_init 1), HWC -> CHW float. */
+void  msnh_or_letterbox_u8(const unsigned char *img, int width, int height, int netW, int netH, int halfInit,
+                           int shuffleRGB, float *out);
+/* Box (x y w h, centre form, network-input pixels) back to the original image; in place. */
+void  msnh_or_bbox_resize2org(float *xywh, int curW, int curH, int orgW, int orgH);
+void  msnh_or_bbox_resize2org_nopad(float *xywh, int curW, int curH, int orgW, int orgH);
+
 #ifdef __cplusplus
 }
 #endif

@@ -43,6 +43,9 @@ def lib():
         L.msnh_or_iou.argtypes = [_fp, _fp]
         L.msnh_or_iou.restype = cf
         L.msnh_or_yolo_out.argtypes = [ctypes.POINTER(_fp), ctypes.POINTER(ci), ci, ci, cf, cf, _fp, ll]
+        L.msnh_or_letterbox_u8.argtypes = [ctypes.POINTER(ctypes.c_ubyte), ci, ci, ci, ci, ci, ci, _fp]
+        L.msnh_or_bbox_resize2org.argtypes = [_fp, ci, ci, ci, ci]
+        L.msnh_or_bbox_resize2org_nopad.argtypes = [_fp, ci, ci, ci, ci]
         L.msnh_or_yolo_out.restype = ll
         L.msnh_or_im2col.argtypes = [_fp, ci, ci, ci, ci, ci, ci, ci, ci, ci, ci, ci, _fp]
         L.msnh_or_gemm_nn.argtypes = [ci, ci, ci, _fp, ci, _fp, ci, _fp, ci]
@@ -142,6 +145,22 @@ def yolo_decode(x, class_num, anchors6, ratio):
 def iou(b1, b2):
     a, b = _f32(b1), _f32(b2)
     return float(lib().msnh_or_iou(_p(a), _p(b)))
+
+
+def letterbox_u8(img, net_w, net_h, half_init=False, shuffle_rgb=False):
+    """img: HWC uint8 with 3 channels -> CHW float32 network input (pad to square with 127, bilinear resize)."""
+    a = np.ascontiguousarray(img, np.uint8)
+    h, w, c = a.shape
+    assert c == 3
+    out = np.empty((3, net_h, net_w), np.float32)
+    lib().msnh_or_letterbox_u8(a.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte)), w, h, net_w, net_h, int(half_init), int(shuffle_rgb), _p(out))
+    return out
+
+
+def bbox_resize2org(xywh, cur_w, cur_h, org_w, org_h, no_pad=False):
+    b = _f32(xywh).copy()
+    (lib().msnh_or_bbox_resize2org_nopad if no_pad else lib().msnh_or_bbox_resize2org)(_p(b), cur_w, cur_h, org_w, org_h)
+    return b
 
 
 def yolo_out(heads, class_num, conf, nms):

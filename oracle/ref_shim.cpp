@@ -22,6 +22,7 @@
 
 #define private public      // NetBuilder::_netState has no getter; the capture loop needs the pools
 #include "Msnhnet/net/MsnhNetBuilder.h"
+#include "Msnhnet/utils/MsnhCVUtil.h"
 #undef private
 
 using namespace Msnhnet;
@@ -257,6 +258,34 @@ long long ref_boxes(void *h, float *dst, long long capBoxes)
         }
     }
     return n;
+}
+
+// CVUtil::getPaddingZeroF32C3 on a 3-channel 8-bit HWC image; dst holds 3*netW*netH floats (CHW).
+int ref_letterbox_u8(const unsigned char *img, int width, int height, int netW, int netH, int halfInit, int shuffleRGB,
+                     float *dst, char *err, int errCap)
+{
+    try
+    {
+        Mat mat(width, height, MAT_RGB_U8, const_cast<unsigned char*>(img));
+        std::vector<float> v = CVUtil::getPaddingZeroF32C3(mat, Vec2I32(netW, netH), halfInit != 0 ? 1.f : 0.f, shuffleRGB != 0);
+        std::memcpy(dst, v.data(), v.size() * sizeof(float));
+        return 0;
+    }
+    catch(Exception &e)
+    {
+        std::snprintf(err, static_cast<size_t>(errCap), "%s", e.what());
+        return 1;
+    }
+}
+
+// YoloOutLayer::bboxResize2Org / bboxResize2OrgNoPad on one box given as x y w h; in place.
+void ref_bbox_resize2org(float *xywh, int curW, int curH, int orgW, int orgH, int noPad)
+{
+    YoloBox b;
+    b.xywhBox = Box::XYWHBox(xywh[0], xywh[1], xywh[2], xywh[3]);
+    if(noPad) YoloOutLayer::bboxResize2OrgNoPad(b, Point2I(curW, curH), Point2I(orgW, orgH));
+    else      YoloOutLayer::bboxResize2Org(b, Point2I(curW, curH), Point2I(orgW, orgH));
+    xywh[0] = b.xywhBox.x; xywh[1] = b.xywhBox.y; xywh[2] = b.xywhBox.w; xywh[3] = b.xywhBox.h;
 }
 
 void ref_set_threads_note(int *ompMax)

@@ -24,6 +24,9 @@ TMP = "/tmp/msnh_golden"
 os.makedirs(TMP, exist_ok=True)
 
 
+LETTERBOX_CASES = [(48, 64, 40, 40, 1), (70, 50, 64, 64, 2), (30, 30, 52, 52, 3), (36, 36, 36, 36, 4)]
+
+
 def layer_stats(a):
     a = np.asarray(a, np.float64)
     fin = np.isfinite(a)
@@ -131,6 +134,22 @@ def main():
         store[f"shape/{arch}/types"] = np.frombuffer("\n".join(i["type"] for i in infos).encode(), np.uint8)
         store[f"shape/{arch}/detail"] = np.frombuffer(r.detail().encode(), np.uint8)
         r.close()
+    # pre / post-processing around the graph: CVUtil::getPaddingZeroF32C3 on seeded 8-bit images (stored as the 8-bit
+    # values it scales, i.e. round(out * 255)), YoloOutLayer::bboxResize2Org[NoPad] on seeded boxes
+    for idx, (h, w, nw, nh, seed) in enumerate(LETTERBOX_CASES):
+        img = np.random.default_rng(seed).integers(0, 256, (h, w, 3), dtype=np.uint8)
+        for shuffle in (0, 1):
+            out = refshim.letterbox_u8(img, nw, nh, False, bool(shuffle))
+            store[f"letterbox/{idx}/shuffle{shuffle}"] = np.rint(out * 255.0).astype(np.uint8)
+        store[f"letterbox/{idx}/case"] = np.array([h, w, nw, nh, seed], np.int64)
+    rng = np.random.default_rng(77)
+    rows = []
+    for _ in range(40):
+        box = rng.uniform(0, 600, 4).astype(np.float32)
+        cw, ch, ow, oh = (int(v) for v in rng.integers(32, 2000, 4))
+        rows.append(np.concatenate([box, [cw, ch, ow, oh], refshim.bbox_resize2org(box, cw, ch, ow, oh, False),
+                                    refshim.bbox_resize2org(box, cw, ch, ow, oh, True)]).astype(np.float64))
+    store["bbox/rows"] = np.array(rows)
     np.savez_compressed(OUT, **store)
     print("wrote", OUT, os.path.getsize(OUT), "bytes,", len(store), "arrays")
 

@@ -43,6 +43,9 @@ def lib():
         L.ref_layer_output.restype = ll
         L.ref_boxes.argtypes = [vp, fp, ll]
         L.ref_boxes.restype = ll
+        u8p = ctypes.POINTER(ctypes.c_ubyte)
+        L.ref_letterbox_u8.argtypes = [u8p, ci, ci, ci, ci, ci, ci, fp, cp, ci]
+        L.ref_bbox_resize2org.argtypes = [fp, ci, ci, ci, ci, ci]
         _lib = L
     return _lib
 
@@ -124,3 +127,25 @@ class RefNet:
 
     def inference_time_ms(self):
         return float(self.L.ref_inference_time(self.h))
+
+
+def letterbox_u8(img, net_w, net_h, half_init=False, shuffle_rgb=False):
+    """img: HWC uint8, 3 channels.  CVUtil::getPaddingZeroF32C3 -> CHW float32."""
+    import numpy as np
+    a = np.ascontiguousarray(img, np.uint8)
+    h, w, c = a.shape
+    assert c == 3
+    out = np.empty((3, net_h, net_w), np.float32)
+    err = ctypes.create_string_buffer(1024)
+    rc = lib().ref_letterbox_u8(a.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte)), w, h, net_w, net_h, int(half_init), int(shuffle_rgb),
+                                out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), err, 1024)
+    if rc != 0:
+        raise RefError(err.value.decode())
+    return out
+
+
+def bbox_resize2org(xywh, cur_w, cur_h, org_w, org_h, no_pad=False):
+    import numpy as np
+    b = np.array(xywh, np.float32)
+    lib().ref_bbox_resize2org(b.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), cur_w, cur_h, org_w, org_h, int(no_pad))
+    return b

@@ -179,3 +179,18 @@ def test_nms_variants_agree(seed):
     assert np.array_equal(a, b, equal_nan=True)
     assert np.array_equal(a, c, equal_nan=True)
     assert 0 < len(a) < n
+
+
+def test_boxes_to_image_matches_the_oracle():
+    import msnh_oracle_net as on
+    rng = np.random.default_rng(8)
+    boxes = rng.uniform(0, 600, (40, 7)).astype(np.float32)
+    for (nw, nh, ow, oh) in [(608, 608, 1280, 720), (608, 608, 480, 640), (416, 416, 416, 416), (320, 224, 1000, 333)]:
+        for padded in (True, False):
+            got = netapi.boxes_to_image(boxes, nw, nh, ow, oh, padded)
+            for i in range(len(boxes)):
+                want = on.bbox_resize2org(boxes[i, :4], nw, nh, ow, oh, no_pad=not padded)
+                assert np.array_equal(got[i, :4], want)
+                assert np.array_equal(got[i, 4:], boxes[i, 4:])
+    with pytest.raises(netapi.MsnhnetError):
+        netapi.boxes_to_image(boxes, 0, 608, 10, 10)

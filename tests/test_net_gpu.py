@@ -160,6 +160,29 @@ def test_fp16_winograd_network(arch, size, batch):
             assert nu.rel_err(logits[b], ref[b][-1]) <= 2e-2
 
 
+def test_image_in_boxes_out():
+    """8-bit images of different shapes -> device letterbox -> forward -> boxes in original-image pixels: equals the
+    float path fed with the restatement's letterbox, followed by the restatement's rescale."""
+    size, batch = 96, 2
+    net, binp, g = nu.model("yolov3", batch, size, seed=3)
+    rng = np.random.default_rng(12)
+    imgs = [rng.integers(0, 256, (120, 200, 3), dtype=np.uint8), rng.integers(0, 256, (150, 90, 3), dtype=np.uint8)]
+    m = netapi.Net(net, binp)
+    for i, im in enumerate(imgs):
+        m.set_input_image_u8(i, im)
+    m.enqueue(None)
+    got = m.fetch_yolo()
+    x = np.stack([on.letterbox_u8(im, size, size) for im in imgs])
+    want = m.run_yolo(x)
+    for i, im in enumerate(imgs):
+        assert np.array_equal(got[i], want[i])
+        back = netapi.boxes_to_image(got[i], size, size, im.shape[1], im.shape[0])
+        for k in range(len(back)):
+            assert np.array_equal(back[k, :4], on.bbox_resize2org(got[i][k, :4], size, size, im.shape[1], im.shape[0]))
+    with pytest.raises(netapi.MsnhnetError):
+        m.set_input_image_u8(2, imgs[0])
+
+
 def test_cpu_entry_points_refuse():
     net, binp, g = nu.model("resnet18", 1, 224, seed=3)
     m = netapi.Net(net, binp)

@@ -214,3 +214,23 @@ def test_absmax(dtype):
     gu.sync()
     xf = xd[..., :24].float().cpu().numpy()
     assert float(r) == float(np.abs(xf[np.isfinite(xf)]).max())
+
+
+@pytest.mark.parametrize("h,w,nw,nh", [(480, 640, 608, 608), (640, 480, 416, 416), (300, 300, 608, 608), (100, 37, 64, 64),
+                                       (608, 608, 608, 608), (50, 80, 224, 224), (33, 33, 32, 32), (720, 1280, 608, 608)])
+def test_letterbox_u8(h, w, nw, nh):
+    """device letterbox == the restatement of CVUtil::getPaddingZeroF32C3, bit for bit (no fused multiply-add in either)"""
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(h + 3 * w)
+    img = rng.integers(0, 256, (h, w, 3), dtype=np.uint8)
+    src = torch.from_numpy(img).cuda()
+    for half in (0, 1):
+        for shuffle in (0, 1):
+            dst = torch.full((3, nh, nw), -5.0, dtype=torch.float32).cuda()
+            gu.sync()
+            abi.check(abi.lib().msnh_hip_letterbox_u8(gu.ptr(src), w, h, nw, nh, half, shuffle, gu.ptr(dst), None))
+            gu.sync()
+            assert np.array_equal(dst.cpu().numpy(), on.letterbox_u8(img, nw, nh, bool(half), bool(shuffle)))
+    assert abi.lib().msnh_hip_letterbox_u8(gu.ptr(src), w, h, 0, nh, 0, 0, gu.ptr(dst), None) != 0
+    assert b"letterbox" in abi.lib().msnh_hip_last_error()

@@ -300,3 +300,97 @@ def test_parse_msnhnet_duplicate_keys_and_expansion(tmp_path):
     o = on.OracleNet(netp)
     assert len(o.top) == 53                      # 23 residual blocks expanded from 5 `size:` entries
     assert [k for k, _ in o.top].count("resblock") == 23
+
+
+# ---- pre / post-processing around the graph ------------------------------------------------------------------------
+LETTERBOX_SHAPES = [(480, 640, 608, 608), (640, 480, 416, 416), (300, 300, 608, 608), (720, 1280, 608, 608), (100, 37, 64, 64),
+                    (608, 608, 608, 608), (50, 80, 224, 224), (33, 33, 32, 32)]
+
+
+@pytest.mark.parametrize("h,w,nw,nh", LETTERBOX_SHAPES)
+def test_letterbox_against_reference(h, w, nw, nh):
+    """The restatement against CVUtil::getPaddingZeroF32C3 itself.  The reference build lets the compiler fuse
+    multiply-adds in the interpolation, the restatement does not: a few pixels per million land one 8-bit step apart."""
+    if not refshim.available():
+        pytest.skip("reference build not present")
+    rng = np.random.default_rng(h * 7 + w)
+    img = rng.integers(0, 256, (h, w, 3), dtype=np.uint8)
+    for half in (False, True):
+        for shuffle in (False, True):
+            a = on.letterbox_u8(img, nw, nh, half, shuffle)
+            b = refshim.letterbox_u8(img, nw, nh, half, shuffle)
+            step = 1 / 127.5 if half else 1 / 255.0
+            d = np.abs(a - b)
+            assert d.max() <= step * 1.001
+            assert (d > 1e-7).mean() <= 1e-4
+
+
+def test_letterbox_mathematics():
+    rng = np.random.default_rng(11)
+    # same size: a pure layout change and scale
+    img = rng.integers(0, 256, (24, 24, 3), dtype=np.uint8)
+    out = on.letterbox_u8(img, 24, 24)
+    assert np.array_equal(out, img.transpose(2, 0, 1).astype(np.float32) / np.float32(255.0))
+    assert np.array_equal(on.letterbox_u8(img, 24, 24, shuffle_rgb=True), out[::-1])
+    assert np.array_equal(on.letterbox_u8(img, 24, 24, half_init=True),
+                          (img.transpose(2, 0, 1).astype(np.float32) - np.float32(127.5)) / np.float32(127.5))
+    # padding: a wide image gets rows of 127 above (diff/2) and below (diff - diff/2)
+    wide = rng.integers(0, 256, (10, 15, 3), dtype=np.uint8)
+    o = on.letterbox_u8(wide, 15, 15)
+    assert np.all(o[:, :2] == np.float32(127 / 255.0)) and np.all(o[:, 12:] == np.float32(127 / 255.0))
+    assert np.array_equal(o[:, 2:12], wide.transpose(2, 0, 1).astype(np.float32) / np.float32(255.0))
+    tall = rng.integers(0, 256, (15, 10, 3), dtype=np.uint8)
+    o = on.letterbox_u8(tall, 15, 15)
+    assert np.all(o[:, :, :2] == np.float32(127 / 255.0)) and np.all(o[:, :, 12:] == np.float32(127 / 255.0))
+    # halving an image whose 2x2 blocks are constant returns the block values (samples fall half-way between equal pixels)
+    small = rng.integers(0, 256, (16, 16, 3), dtype=np.uint8)
+    big = np.repeat(np.repeat(small, 2, axis=0), 2, axis=1)
+    assert np.array_equal(on.letterbox_u8(big, 16, 16), small.transpose(2, 0, 1).astype(np.float32) / np.float32(255.0))
+    # against a library bilinear resize (half-pixel centres, no corner alignment) when shrinking: truncation of two
+    # float evaluations of the same real number may differ by one step, never more
+    import torch
+    src = rng.integers(0, 256, (90, 90, 3), dtype=np.uint8)
+    ours = on.letterbox_u8(src, 40, 40) * 255.0
+    t = torch.from_numpy(src.transpose(2, 0, 1).astype(np.float32))[None]
+    lib = torch.nn.functional.interpolate(t, size=(40, 40), mode="bilinear", align_corners=False)[0].numpy()
+    assert np.abs(ours - np.floor(lib)).max() <= 1.0
+    assert (np.abs(ours - np.floor(lib)) > 0).mean() < 0.02
+    # enlarging: the reference's weights sum to zero on the last row and column (second sample index clamped, first not)
+    up = on.letterbox_u8(np.full((8, 8, 3), 200, np.uint8), 16, 16) * 255.0
+    assert np.all(up[:, :15, :15] == 200) and np.all(up[:, 15, :] == 0) and np.all(up[:, :, 15] == 0)
+
+
+def test_bbox_back_to_image():
+    # 1280x720 letterboxed into 608x608: scale 0.475, 133 rows of padding above; the centre maps to the centre
+    b = on.bbox_resize2org([304.0, 304.0, 95.0, 47.5], 608, 608, 1280, 720)
+    assert np.allclose(b, [640.0, 360.0, 200.0, 100.0], rtol=1e-6)
+    b = on.bbox_resize2org([304.0, 304.0, 95.0, 47.5], 608, 608, 720, 1280)
+    assert np.allclose(b, [360.0, 640.0, 200.0, 100.0], rtol=1e-6)
+    b = on.bbox_resize2org([100.0, 50.0, 10.0, 20.0], 416, 416, 832, 416, no_pad=True)
+    assert np.allclose(b, [200.0, 50.0, 20.0, 20.0], rtol=1e-6)
+    if refshim.available():
+        rng = np.random.default_rng(5)
+        for _ in range(50):
+            box = rng.uniform(0, 600, 4).astype(np.float32)
+            cw, ch, ow, oh = (int(v) for v in rng.integers(32, 2000, 4))
+            for no_pad in (False, True):
+                assert np.array_equal(on.bbox_resize2org(box, cw, ch, ow, oh, no_pad), refshim.bbox_resize2org(box, cw, ch, ow, oh, no_pad))
+
+
+def test_letterbox_and_bbox_against_golden():
+    """the same two comparisons against vectors the reference build wrote (present also where the build is not)"""
+    idx = 0
+    while f"letterbox/{idx}/case" in GOLD.files:
+        h, w, nw, nh, seed = (int(v) for v in GOLD[f"letterbox/{idx}/case"])
+        img = np.random.default_rng(seed).integers(0, 256, (h, w, 3), dtype=np.uint8)
+        for shuffle in (0, 1):
+            want = GOLD[f"letterbox/{idx}/shuffle{shuffle}"].astype(np.int32)
+            got = np.rint(on.letterbox_u8(img, nw, nh, False, bool(shuffle)) * 255.0).astype(np.int32)
+            assert np.abs(got - want).max() <= 1 and (got != want).mean() <= 1e-3
+        idx += 1
+    assert idx >= 4
+    for row in GOLD["bbox/rows"]:
+        box = row[:4].astype(np.float32)
+        cw, ch, ow, oh = (int(v) for v in row[4:8])
+        assert np.array_equal(on.bbox_resize2org(box, cw, ch, ow, oh, False), row[8:12].astype(np.float32))
+        assert np.array_equal(on.bbox_resize2org(box, cw, ch, ow, oh, True), row[12:16].astype(np.float32))
