@@ -7,6 +7,10 @@
 
 namespace msnh {
 
+int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
+              const void *residual, void *y, hipStream_t st, bool dryRun);
+
+
 template <typename T, int VEC> struct VecOf { typedef T type __attribute__((ext_vector_type(VEC))); };
 template <typename T> struct VecOf<T, 1> { typedef T type; };
 
@@ -413,6 +417,22 @@ int msnh_hip_connected(int dtype, int batch, int inputs, int outputs, const void
     MSNH_REQUIRE(dtypeOk(dtype), "connected: bad dtype");
     MSNH_REQUIRE(batch > 0 && inputs > 0 && outputs > 0 && x && w && y && actOk(act), "connected: bad argument");
     hipStream_t st = resolveStream(s);
+    // With a real batch this is a GEMM [outputs x inputs] x [inputs x batch]: the 1x1 case of the implicit-GEMM
+    // convolution (batch "pixels"), which reads the weights once instead of once per image.
+    const int vec = dtype == MSNH_F16 ? 8 : 4;
+    if (batch >= 8 && x_mul == 1.f && inputs % vec == 0 && outputs % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 32 == 0)
+    {
+        msnh_conv_desc d;
+        d.dtype = dtype; d.out_dtype = MSNH_F32;
+        d.batch = batch; d.in_h = 1; d.in_w = 1; d.in_c = inputs; d.in_ld = inputs;
+        d.out_c = outputs; d.out_h = 1; d.out_w = 1; d.out_ld = outputs;
+        d.ksize = 1; d.stride = 1; d.pad = 0; d.dilation = 1; d.groups = 1;
+        d.act = act; d.act_param = act_param; d.has_residual = 0; d.res_ld = outputs; d.act2 = MSNH_ACT_NONE; d.act2_param = 0.f;
+        d.res_mul = 1.f; d.out_mul = 1.f; d.algo = MSNH_CONV_IGEMM;
+        d.tile = batch <= 64 ? 12 : 0;           // 64 x 64 tile for small batches, else the default by output count
+        return convIgemm(&d, x, w, nullptr, bias, nullptr, y, st, false);
+    }
     const long long waves = static_cast<long long>(batch) * outputs;
     dim3 grid(gridFor(waves * 64, 256));
     if (dtype == MSNH_F16)

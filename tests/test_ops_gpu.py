@@ -137,6 +137,27 @@ def test_connected(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("batch,inputs,outputs,act", [(32, 2048, 1000, "none"), (64, 1280, 1000, "relu"), (9, 64, 24, "leaky")])
+def test_connected_batched(dtype, batch, inputs, outputs, act):
+    """with a real batch the fully connected layer runs as the 1x1 case of the MFMA implicit GEMM"""
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(batch)
+    x = _x(rng, (batch, inputs, 1, 1), dtype)
+    w = rng.uniform(-0.05, 0.05, (outputs, inputs)).astype(np.float32)
+    if dtype == abi.F16:
+        w = gu.round_f16(w)
+    bias = rng.uniform(-0.05, 0.05, outputs).astype(np.float32)
+    ref = on.connected(x, w, bias, outputs, act=act).reshape(batch, outputs)
+    xd, wd, bd = gu.dev(x.reshape(batch, inputs), dtype), gu.dev(w, dtype), gu.dev(bias)
+    yd = torch.zeros((batch, outputs), dtype=torch.float32).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_connected(dtype, batch, inputs, outputs, gu.ptr(xd), 1.0, gu.ptr(wd), gu.ptr(bd), abi.ACT[act], 0.1, gu.ptr(yd), None))
+    gu.sync()
+    assert gu.rel_err(yd.cpu().numpy(), ref) <= 5e-6
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_layout_roundtrip(dtype):
     import gpuutil as gu
     gu.init()
