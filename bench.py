@@ -78,6 +78,10 @@ def main():
     ap.add_argument("--workload", default="yolov3", choices=sorted(WORKLOADS))
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--input", default="device", choices=["device", "host_f32", "host_u8"],
+                    help="device (default, the headline figure): the batch is resident in HBM when the clock starts.  host_f32: the "
+                         "reference's own calling convention, a host float image per call (runYoloGPU / runClassifyGPU), PCIe "
+                         "inclusive.  host_u8: 8-bit host images, letterboxed on the device, PCIe inclusive.")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch a plain 256 MiB -> 256 MiB channel-copy kernel 5 times (a known-size reference for scaling "
                          "the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
@@ -111,19 +115,36 @@ def main():
     torch.cuda.synchronize()
     dev_in = x.data_ptr()
 
+    host_x = zoo.seeded_input(batch, 3, size, size, a.seed + 1) if a.input == "host_f32" else None
+    host_u8 = None
+    if a.input == "host_u8":
+        import numpy as np
+        host_u8 = np.random.default_rng(a.seed + 2).integers(0, 256, (batch, size, size, 3), dtype=np.uint8)
+
+    def feed():
+        if host_u8 is not None:
+            for i in range(batch):
+                net.set_input_image_u8(i, host_u8[i])
+            net.enqueue(None)
+        else:
+            net.enqueue(dev_in)
+
     def run_steps(k):
         """k forwards + k result fetches.  Detection keeps two batches in flight: while the host sorts and
         suppresses the boxes of batch i the device already runs batch i+1."""
         out = None
-        if detect:
-            net.enqueue(dev_in)
+        if host_x is not None:
+            for _ in range(k):
+                out = net.run_yolo(host_x) if detect else net.run_classify(host_x)
+        elif detect:
+            feed()
             for _ in range(k - 1):
-                net.enqueue(dev_in)
+                feed()
                 out = net.fetch_yolo()
             out = net.fetch_yolo()
         else:
             for _ in range(k):
-                net.enqueue(dev_in)
+                feed()
                 out = net.fetch_classify()
         return out
 
@@ -155,8 +176,8 @@ def main():
            "unit": "images/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4),
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
            "config": {"workload": f"{a.workload}-{size} {dtype} batch {batch}, seeded He-normal weights, U[0,1) input, "
-                                  f"device-resident input -> {'boxes' if detect else 'logits'} on host",
-                      "seed": a.seed, "device_launches_per_step": n_all // 10, "device_ms_per_step_eager": round(gpu_only_ms, 4)},
+                                  f"{'device-resident' if a.input == 'device' else a.input} input -> {'boxes' if detect else 'logits'} on host",
+                      "input": a.input, "seed": a.seed, "device_launches_per_step": n_all // 10, "device_ms_per_step_eager": round(gpu_only_ms, 4)},
            "roofline": roofline}
     if detect:
         res["config"]["boxes_per_image"] = [int(len(b)) for b in out]
