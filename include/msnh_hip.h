@@ -54,7 +54,10 @@ enum msnh_conv_algo
     MSNH_CONV_IGEMM     = 2,   /* implicit GEMM on MFMA, LDS-staged tiles; needs (in_c/groups) % 8 == 0 (f16) or % 4 (f32) */
     MSNH_CONV_DEPTHWISE = 3,   /* groups == in_c == out_c, bandwidth-bound direct kernel */
     MSNH_CONV_WINOGRAD  = 4,   /* F(2x2,3x3): ksize 3, stride 1, dilation 1, groups 1 */
-    MSNH_CONV_STEM      = 5    /* in_c <= 4 first layer: reads NCHW float32 input directly (cast fused) */
+    MSNH_CONV_STEM      = 5,   /* in_c <= 4 first layer: reads NCHW float32 input directly (cast fused) */
+    MSNH_CONV_IGEMM_SPLITK = 6 /* IGEMM with the K loop cut into up to 8 slices on separate workgroups, float32 partial sums in
+                                  the workspace summed in slice order (deterministic); for launches with few output tiles.
+                                  Same weight packing as IGEMM.  Never chosen by AUTO. */
 };
 
 /* ------------------------------------------------------------------------------------------------

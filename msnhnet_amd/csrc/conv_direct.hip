@@ -11,6 +11,9 @@ namespace msnh {
 
 int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
               const void *residual, void *y, hipStream_t st, bool dryRun);
+int convIgemmWs(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
+                const void *residual, void *y, hipStream_t st, bool dryRun, void *splitWs, size_t splitWsBytes);
+size_t igemmSplitKWorkspaceBytes(const msnh_conv_desc *d);
 int igemmTileCount();
 int convWinograd(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
                  const void *residual, void *y, void *ws, size_t wsBytes, hipStream_t st);
@@ -237,7 +240,7 @@ int msnh_hip_conv2d_tile_supported(const msnh_conv_desc *d, int tile)
         winogradGemmDesc(d, &t);
     }
     else if (!igemmOk(d)) return 0;
-    if (tile == 0) return 1;
+    if (tile == 0 && d->algo != MSNH_CONV_IGEMM_SPLITK) return 1;
     t.tile = tile;
     return convIgemm(&t, d, d, nullptr, nullptr, nullptr, &t, nullptr, true) == 0 ? 1 : 0;      // pointers unused in a dry run
 }
@@ -277,6 +280,7 @@ int msnh_hip_conv2d_pack_weights(const msnh_conv_desc *d, int algo, const float 
     {
     case MSNH_CONV_DIRECT:
     case MSNH_CONV_IGEMM:
+    case MSNH_CONV_IGEMM_SPLITK:
         for (int oc = 0; oc < d->out_c; ++oc)
             for (int ci = 0; ci < cinG; ++ci)
                 for (int t = 0; t < kk; ++t)
@@ -310,8 +314,9 @@ int msnh_hip_conv2d_pack_weights(const msnh_conv_desc *d, int algo, const float 
 
 size_t msnh_hip_conv2d_workspace_bytes(const msnh_conv_desc *d, int algo)
 {
-    if (!d || algo != MSNH_CONV_WINOGRAD) return 0;
-    return winogradWorkspaceBytes(d);
+    if (!d) return 0;
+    if (algo == MSNH_CONV_IGEMM_SPLITK) return igemmSplitKWorkspaceBytes(d);
+    return algo == MSNH_CONV_WINOGRAD ? winogradWorkspaceBytes(d) : 0;
 }
 
 int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
@@ -335,6 +340,10 @@ int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const
         MSNH_REQUIRE(igemmOk(d), "conv2d: IGEMM needs (in_c/groups) and in_ld to be multiples of %d", d->dtype == MSNH_F16 ? 8 : 4);
         MSNH_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0, "conv2d: IGEMM needs 16-byte aligned x and w");
         return convIgemm(d, x, w, scale, shift, residual, y, st, false);
+    case MSNH_CONV_IGEMM_SPLITK:
+        MSNH_REQUIRE(igemmOk(d), "conv2d: IGEMM needs (in_c/groups) and in_ld to be multiples of %d", d->dtype == MSNH_F16 ? 8 : 4);
+        MSNH_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0, "conv2d: IGEMM needs 16-byte aligned x and w");
+        return convIgemmWs(d, x, w, scale, shift, residual, y, st, false, workspace, workspace_bytes);
     case MSNH_CONV_WINOGRAD:
         MSNH_REQUIRE(winogradOk(d), "conv2d: shape not supported by the Winograd kernel");
         return convWinograd(d, x, w, scale, shift, residual, y, workspace, workspace_bytes, st);

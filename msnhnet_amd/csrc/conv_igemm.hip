@@ -17,8 +17,13 @@ int igemmHeuristicTile(const msnh_conv_desc *d)
 
 int igemmTileCount() { return kIgemmTiles; }
 
-int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
-              const void *residual, void *y, hipStream_t st, bool dryRun)
+size_t igemmSplitKWorkspaceBytes(const msnh_conv_desc *d)
+{
+    return static_cast<size_t>(kSplitKMax) * d->batch * d->out_h * d->out_w * d->out_c * sizeof(float);
+}
+
+int convIgemmWs(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
+                const void *residual, void *y, hipStream_t st, bool dryRun, void *splitWs, size_t splitWsBytes)
 {
     IgemmArgs a;
     a.x = x; a.w = w; a.scale = scale; a.shift = shift; a.res = residual; a.y = y;
@@ -46,12 +51,30 @@ int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float
     a.vecOk = (d->out_ld % 8 == 0) && ((d->out_c / d->groups) % 8 == 0 || d->groups == 1) &&
               (reinterpret_cast<uintptr_t>(y) % (8 * outEl) == 0) &&
               (!a.hasRes || (d->res_ld % 8 == 0 && reinterpret_cast<uintptr_t>(residual) % 16 == 0));
+    a.splitMax = 0; a.splitK = 1; a.ws = nullptr; a.wsLd = d->out_c;
+    if (d->algo == MSNH_CONV_IGEMM_SPLITK)
+    {
+        MSNH_REQUIRE(d->out_c % 4 == 0, "conv2d: split-K needs out_c to be a multiple of 4");
+        if (!dryRun)
+        {
+            MSNH_REQUIRE(splitWs && reinterpret_cast<uintptr_t>(splitWs) % 16 == 0 && splitWsBytes >= igemmSplitKWorkspaceBytes(d),
+                         "conv2d: split-K needs a 16-byte aligned workspace of msnh_hip_conv2d_workspace_bytes() bytes");
+        }
+        a.splitMax = kSplitKMax;
+        a.ws = static_cast<float *>(splitWs);
+    }
     int tile = d->tile;
     if (tile <= 0 || tile > kIgemmTiles) tile = igemmHeuristicTile(d);
     if (d->dtype == MSNH_F16)
         return d->out_dtype == MSNH_F16 ? igemmF16F16(a, d->groups, tile, st) : igemmF16F32(a, d->groups, tile, st);
     MSNH_REQUIRE(d->out_dtype == MSNH_F32, "igemm: float32 input needs float32 output");
     return igemmF32F32(a, d->groups, tile, st);
+}
+
+int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
+              const void *residual, void *y, hipStream_t st, bool dryRun)
+{
+    return convIgemmWs(d, x, w, scale, shift, residual, y, st, dryRun, nullptr, 0);
 }
 
 } // namespace msnh

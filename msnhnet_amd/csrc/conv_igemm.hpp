@@ -40,6 +40,10 @@ struct IgemmArgs
     int dryRun;             // validate the tile for this shape, launch nothing
     unsigned xBytes, wBytes; // extent of the input tensor / packed weights in bytes (buffer resources; < 2 GiB)
     int ragged;             // cinG is not a multiple of the tile's K step
+    int splitMax;           // > 1: split-K requested, at most this many slices of the K loop (grid y)
+    int splitK;             // slices actually used by the launch
+    float *ws;              // split-K: float32 partial sums [slice][pixel][out_c]
+    int wsLd;               // = out_c of the whole convolution
     int buffersOk;          // both extents fit a buffer resource
     int act, act2, hasRes, vecOk;
     float actParam, act2Param, resMul, outMul;
@@ -500,11 +504,15 @@ void convIgemmKernel(IgemmArgs a)
     constexpr int AHEAD = NS >= 3 ? NS - 1 : 2;  // the loads issued during step `it` belong to step it + AHEAD
     constexpr int INFLIGHT = NS >= 3 ? (NS - 3) * NL + NPRE : 0;   // loads younger than step it+1's at the barrier
 
-    setTap(0);
-    staticFor<0, NL>([&](auto lTag) { issueLoad(lTag, 0u, 0u, a.ragged && (ldVec * VEC >= a.cinG), 0u); });
-    staticFor<1, AHEAD>([&](auto stTag) {
+    // split-K: this workgroup multiplies tile steps [itBegin, itBegin + nLocal) of the K loop
+    const int itBegin = a.splitK > 1 ? static_cast<int>(static_cast<long long>(blockIdx.y) * a.nIter / a.splitK) : 0;
+    const int nLocal  = a.splitK > 1 ? static_cast<int>(static_cast<long long>(blockIdx.y + 1) * a.nIter / a.splitK) - itBegin : a.nIter;
+    tapNext = itBegin / a.cChunks;
+    chunkNext = itBegin - tapNext * a.cChunks - 1;            // advance() steps onto the first tile step
+    setTap(tapNext);
+    staticFor<0, AHEAD>([&](auto stTag) {
         constexpr int st = decltype(stTag)::value;
-        advance(a.nIter <= st);
+        advance(nLocal <= st);
         staticFor<0, NL>([&](auto lTag) { issueLoad(lTag, sANext, sBNext, cutNext, st * STAGE); });
     });
     dmaWait<(AHEAD - 1) * NL>();                 // step 0 has landed
@@ -513,9 +521,9 @@ void convIgemmKernel(IgemmArgs a)
 
     // cur: stage of step it; nxt: of step it+1; nn: where the loads issued during step it go
     unsigned cur = 0, nxt = STAGE, nn = NS >= 3 ? (NS - 1) * STAGE : 0;
-    for (int it = 0; it < a.nIter; ++it)
+    for (int it = 0; it < nLocal; ++it)
     {
-        advance(it + AHEAD >= a.nIter);          // sANext / sBNext / cutNext now describe step it + AHEAD
+        advance(it + AHEAD >= nLocal);          // sANext / sBNext / cutNext now describe step it + AHEAD
         readFrags(cur, std::integral_constant<int, 1>());
         __builtin_amdgcn_sched_barrier(0);
         staticFor<0, TOT>([&](auto gTag) {
@@ -550,8 +558,47 @@ void convIgemmKernel(IgemmArgs a)
     dmaWait<0>();
     __syncthreads();
 
+    if (a.splitK > 1)
+    {
+        // raw float32 partial sums of this K slice; affine, activation and residual follow in the reduction pass
+        IgemmArgs e = a;
+        e.act = MSNH_ACT_NONE; e.hasRes = 0; e.outMul = 1.f;
+        e.y = a.ws + static_cast<size_t>(blockIdx.y) * a.P * a.wsLd;
+        e.outLd = a.wsLd;
+        e.vecOk = (a.wsLd % 8 == 0) && (a.coutG % 8 == 0 || gridDim.z == 1);
+        igemmEpilogue<T, float, BM, BN, TM, TN>(e, acc, smemRaw, 1.f, 0.f, m0, p0, wm, wn, wave, lane, g);
+        return;
+    }
     igemmEpilogue<T, TOut, BM, BN, TM, TN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, wave, lane, g);
 }
+
+// Split-K reduction: sums the K slices in slice order (so the result does not depend on timing) and applies the
+// convolution's epilogue.  One thread per (pixel, 4 channels).
+template <typename T, typename TOut>
+__global__ __launch_bounds__(256) void splitKReduceKernel(IgemmArgs a, int outC, long long total)
+{
+    const long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int cq = outC / 4;
+    const int c = static_cast<int>(idx % cq) * 4;
+    const long long p = idx / cq;
+    const float *w = a.ws + static_cast<size_t>(p) * a.wsLd + c;
+    f32x4 acc = *reinterpret_cast<const f32x4 *>(w);
+    for (int s = 1; s < a.splitK; ++s) acc += *reinterpret_cast<const f32x4 *>(w + static_cast<size_t>(s) * a.P * a.wsLd);
+    const T *res = static_cast<const T *>(a.res);
+    TOut *y = static_cast<TOut *>(a.y);
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+    {
+        const float sc = a.scale ? a.scale[c + k] : 1.f;
+        const float sh = a.shift ? a.shift[c + k] : 0.f;
+        float v = activate(acc[k] * sc + sh, a.act, a.actParam);
+        if (a.hasRes) v = activate(v + a.resMul * toF(res[static_cast<size_t>(p) * a.resLd + c + k]), a.act2, a.act2Param);
+        y[static_cast<size_t>(p) * a.outLd + c + k] = fromF<TOut>(a.outMul * v);
+    }
+}
+
+constexpr int kSplitKMax = 8;
 
 template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int NS = 3>
 inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
@@ -571,7 +618,21 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
     const size_t smem = smemLoop > smemEpi ? smemLoop : smemEpi;
     a.mTiles = (a.coutG + BM - 1) / BM;
     const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
-    dim3 grid((tiles + 7) / 8 * 8, 1, groups);
+    a.splitK = 1;
+    if (a.splitMax > 1)
+    {
+        // enough slices to give every CU two workgroups, each slice at least four tile steps long
+        int want = (512 + tiles * groups - 1) / (tiles * groups);
+        if (want > a.splitMax) want = a.splitMax;
+        if (want > a.nIter / 4) want = a.nIter / 4;
+        if (want < 2 || a.wsLd % 4 != 0)
+        {
+            setError("conv2d: split-K does not apply to this shape and tile");
+            return 3;
+        }
+        a.splitK = want;
+    }
+    dim3 grid((tiles + 7) / 8 * 8, a.splitK, groups);
     if (a.dryRun) return 0;
     auto kern = convIgemmKernel<T, TOut, BM, BN, KV, WM, WN, NS>;
     if (smem > 48 * 1024)
@@ -582,6 +643,13 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
     }
     hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a);
     MSNH_LAUNCH_CHECK();
+    if (a.splitK > 1)
+    {
+        const int outC = a.coutG * groups;
+        const long long total = static_cast<long long>(a.P) * (outC / 4);
+        hipLaunchKernelGGL((splitKReduceKernel<T, TOut>), dim3(gridFor(total, 256)), dim3(256), 0, st, a, outC, total);
+        MSNH_LAUNCH_CHECK();
+    }
     return 0;
 }
 

@@ -268,7 +268,7 @@ inline int launchPatch(IgemmArgs &a, int groups, hipStream_t st)
     constexpr int BK  = KV * VEC;
     size_t smem = 0;
     int slices = 0;
-    if (groups != 1 || !patchFits<T, BM, BN, KV, WM, WN, PS>(a, &smem, &slices))
+    if (groups != 1 || a.splitMax > 1 || !patchFits<T, BM, BN, KV, WM, WN, PS>(a, &smem, &slices))
     {
         setError("conv2d: this tile needs a 3x3 stride-1 pad-1 ungrouped convolution whose input patch fits in LDS");
         return 3;
@@ -279,6 +279,7 @@ inline int launchPatch(IgemmArgs &a, int groups, hipStream_t st)
     a.nIter   = 9 * a.cChunks;
     a.ragged  = (a.cinG % BK) != 0;
     a.mTiles  = (a.coutG + BM - 1) / BM;
+    a.splitK  = 1;
     const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
     dim3 grid((tiles + 7) / 8 * 8, 1, 1);
     auto kern = convPatch3x3Kernel<T, TOut, BM, BN, KV, WM, WN, PS>;

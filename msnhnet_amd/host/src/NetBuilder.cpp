@@ -690,7 +690,7 @@ std::string NetBuilder::profileEachOp(int reps)
     if (!_planReady) MSNH_THROW("weights are not loaded");
     Plan &plan = *_net->plan;
     static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode"};
-    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem"};
+    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk"};
     msnh_event_t e0 = nullptr, e1 = nullptr;
     MSNH_DEV(msnh_hip_event_create(&e0));
     MSNH_DEV(msnh_hip_event_create(&e1));
@@ -715,7 +715,7 @@ std::string NetBuilder::profileEachOp(int reps)
                              (op.in1 >= 0 ? static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4) : 0.0);
         char line[320];
         snprintf(line, sizeof(line), "L%-3d %-11s %-9s t%-2d k%d s%d g%-4d %4dx%4dx%4dx%4d -> %4dx%4dx%4d %s%s %9.2f us %8.2f TF/s %8.1f GB/s\n", op.layerIndex,
-                 kinds[op.kind], op.kind == PlanOp::CONV ? algos[op.algo] : "-", op.tile, op.ksize, op.stride, op.groups, in.n, in.h, in.w, in.c, out.h, out.w,
+                 kinds[op.kind], (op.kind == PlanOp::CONV || op.algo != MSNH_CONV_AUTO) ? algos[op.algo] : "-", op.tile, op.ksize, op.stride, op.groups, in.n, in.h, in.w, in.c, out.h, out.w,
                  out.c, out.dtype == MSNH_F16 ? "f16" : "f32", op.in1 >= 0 ? "+res" : "    ", us, op.flops / us * 1e-6, bytes / us * 1e-3);
         os << line;
     }

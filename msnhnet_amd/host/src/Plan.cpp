@@ -403,13 +403,24 @@ void Plan::prepareWeights()
             op.src->foldedAffine(scale, shift);
             if (!shift.empty()) op.shiftDev.upload(shift.data(), shift.size() * sizeof(float));
             op.flops = 2.0 * static_cast<double>(w.size()) * in.n;
+            // a real batch is a GEMM: run it as the 1x1 convolution of a 1x1 image, so that the tile search (and its
+            // split-K variant, which suits the few output tiles of a classifier) covers it
+            const int vec = in.dtype == MSNH_F16 ? 8 : 4;
+            op.algo = MSNH_CONV_AUTO;
+            if (in.n >= 8 && in.h * in.w == 1 && in.c % vec == 0 && ld(op.in0) % vec == 0 && mulOf(op.in0) == 1.f && !shift.empty())
+            {
+                op.ksize = 1; op.stride = 1; op.pad = 0; op.dilation = 1; op.groups = 1;
+                op.algo = MSNH_CONV_IGEMM;
+                op.tile = in.n <= 64 ? 12 : 0;
+            }
         }
     }
     if (workspace > _convWorkspace.bytes()) _convWorkspace.alloc(workspace);
 }
 
 // Per-layer search over the implicit-GEMM tile configurations: each candidate runs the real launch (same buffers,
-// same epilogue) a few times between two device events; the fastest wins.  Results do not depend on the choice.
+// same epilogue) a few times between two device events; the fastest wins.  Tiles change the result by nothing but the
+// float32 summation order, and so does the split-K variant tried for layers with few output tiles.
 void Plan::tuneConvs(msnh_stream_t s)
 {
     const int nTiles = msnh_hip_conv2d_tile_count();
@@ -420,7 +431,7 @@ void Plan::tuneConvs(msnh_stream_t s)
     std::vector<std::pair<Key, int>> memo;         // identical shapes share one search
     for (PlanOp &op : ops)
     {
-        if (op.dead || op.kind != PlanOp::CONV || (op.algo != MSNH_CONV_IGEMM && op.algo != MSNH_CONV_WINOGRAD)) continue;
+        if (op.dead || (op.kind != PlanOp::CONV && op.kind != PlanOp::CONNECTED) || (op.algo != MSNH_CONV_IGEMM && op.algo != MSNH_CONV_WINOGRAD)) continue;
         const PlanTensor &in = tensors[static_cast<size_t>(op.in0)];
         const PlanTensor &out = tensors[static_cast<size_t>(op.out)];
         Key key;
@@ -429,29 +440,48 @@ void Plan::tuneConvs(msnh_stream_t s)
         key.res = op.in1 >= 0; key.odt = out.dtype; key.algo = op.algo;
         bool found = false;
         for (const auto &m : memo)
-            if (m.first == key) { op.tile = m.second; found = true; break; }
+            if (m.first == key) { op.algo = m.second / 1000; op.tile = m.second % 1000; found = true; break; }
         if (found) continue;
-        int best = 0;
+        int best = 0, bestAlgo = op.algo;
         float bestMs = std::numeric_limits<float>::max();
-        for (int tile = 0; tile <= nTiles; ++tile)
-        {
-            op.tile = tile;
+        auto search = [&](int algo) {
+            op.algo = algo;
+            for (int tile = 0; tile <= nTiles; ++tile)
             {
-                const msnh_conv_desc probe = convDesc(*this, op);
-                if (!msnh_hip_conv2d_tile_supported(&probe, tile)) continue;
+                op.tile = tile;
+                {
+                    const msnh_conv_desc probe = convDesc(*this, op);
+                    if (!msnh_hip_conv2d_tile_supported(&probe, tile)) continue;
+                }
+                const int reps = 3;
+                launch(op, s);                                       // warm-up (also surfaces launch errors for this tile)
+                MSNH_DEV(msnh_hip_event_record(e0, s));
+                for (int r = 0; r < reps; ++r) launch(op, s);
+                MSNH_DEV(msnh_hip_event_record(e1, s));
+                MSNH_DEV(msnh_hip_event_sync(e1));
+                float ms = 0.f;
+                MSNH_DEV(msnh_hip_event_elapsed_ms(e0, e1, &ms));
+                if (ms < bestMs) { bestMs = ms; best = tile; bestAlgo = algo; }
             }
-            const int reps = 3;
-            launch(op, s);                                       // warm-up (also surfaces launch errors for this tile)
-            MSNH_DEV(msnh_hip_event_record(e0, s));
-            for (int r = 0; r < reps; ++r) launch(op, s);
-            MSNH_DEV(msnh_hip_event_record(e1, s));
-            MSNH_DEV(msnh_hip_event_sync(e1));
-            float ms = 0.f;
-            MSNH_DEV(msnh_hip_event_elapsed_ms(e0, e1, &ms));
-            if (ms < bestMs) { bestMs = ms; best = tile; }
+        };
+        const int baseAlgo = op.algo;
+        search(baseAlgo);
+        if (baseAlgo == MSNH_CONV_IGEMM)
+        {
+            // layers with few output tiles: the K loop cut over several workgroups, if its workspace is modest
+            op.tile = 0;
+            const msnh_conv_desc d = convDesc(*this, op);
+            const size_t need = msnh_hip_conv2d_workspace_bytes(&d, MSNH_CONV_IGEMM_SPLITK);
+            if (out.c % 4 == 0 && need <= (static_cast<size_t>(256) << 20))
+            {
+                MSNH_DEV(msnh_hip_stream_sync(s));
+                if (need > _convWorkspace.bytes()) _convWorkspace.alloc(need);
+                search(MSNH_CONV_IGEMM_SPLITK);
+            }
         }
+        op.algo = bestAlgo;
         op.tile = best;
-        memo.emplace_back(key, best);
+        memo.emplace_back(key, bestAlgo * 1000 + best);
     }
     msnh_hip_event_destroy(e0);
     msnh_hip_event_destroy(e1);
@@ -529,6 +559,13 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
                                            ld(op.out), s));
         break;
     case PlanOp::CONNECTED:
+        if (op.algo == MSNH_CONV_IGEMM || op.algo == MSNH_CONV_IGEMM_SPLITK)
+        {
+            const msnh_conv_desc d = convDesc(*this, op);
+            MSNH_DEV(msnh_hip_conv2d(&d, ptr(op.in0), op.wDev.ptr(), nullptr, op.shiftDev.as<float>(), nullptr, ptr(op.out),
+                                     _convWorkspace.ptr(), _convWorkspace.bytes(), s));
+            break;
+        }
         if (ld(op.in0) != in.c && in.n > 1 && in.h * in.w == 1) MSNH_THROW("connected input must be densely packed");
         MSNH_DEV(msnh_hip_connected(in.dtype, in.n, in.h * in.w * in.c, out.c, ptr(op.in0), mulOf(op.in0), op.wDev.ptr(), op.shiftDev.as<float>(),
                                     static_cast<int>(op.act), op.actParam, static_cast<float *>(ptr(op.out)), s));
@@ -576,7 +613,7 @@ void Plan::exportTensor(int t, std::vector<float> &dst, msnh_stream_t s)
 std::string Plan::describe() const
 {
     static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode"};
-    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem"};
+    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk"};
     std::ostringstream os;
     os << "plan: " << liveOps() << " launches, " << tensors.size() << " tensors, arena " << _arena.bytes() / (1024.0 * 1024.0) << " MiB, dtype "
        << (computeDtype == MSNH_F16 ? "f16" : "f32") << "\n";

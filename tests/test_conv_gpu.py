@@ -211,6 +211,75 @@ def test_conv_winograd(b, c, h, w, oc, with_res):
         assert gu.rel_err(y2, ref) <= 3 * TOL[abi.F16]
 
 
+SPLITK_CASES = [
+    # b, c, h, w, oc, k, stride, pad, groups
+    (1, 512, 7, 7, 512, 3, 1, 1, 1),
+    (2, 256, 14, 14, 512, 3, 2, 1, 1),
+    (1, 1024, 7, 7, 256, 1, 1, 0, 1),
+    (1, 72, 10, 12, 200, 3, 1, 1, 1),       # ragged K chunks and a partial channel tile
+    (2, 128, 9, 9, 64, 3, 1, 1, 2),
+    (16, 2048, 1, 1, 1000, 1, 1, 0, 1),     # a fully connected layer
+]
+
+
+@pytest.mark.parametrize("dtype", [abi.F32, abi.F16])
+@pytest.mark.parametrize("case", SPLITK_CASES)
+def test_conv_split_k(case, dtype):
+    """Split-K implicit GEMM: the K loop cut over several workgroups, partial sums added in slice order.  Same result
+    as the oracle to the one-pass kernel's tolerance, with the full epilogue, for every tile configuration that takes
+    the shape, and bit-identical from run to run."""
+    import ctypes
+    import gpuutil as gu
+    b, c, h, w, oc, k, stride, pad, groups = case
+    rng = np.random.default_rng(sum(case))
+    x, wt = _case(rng, b, c, h, w, oc, k, groups)
+    oh = (h + 2 * pad - k) // stride + 1
+    ow = (w + 2 * pad - k) // stride + 1
+    res = rng.standard_normal((b, oc, oh, ow), dtype=np.float32)
+    scale = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    shift = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    if dtype == abi.F16:
+        x, wt, res = gu.round_f16(x), gu.round_f16(wt), gu.round_f16(res)
+    ref = _ref(x, wt, stride, pad, 1, groups, scale, shift, "leaky", 0.1, res, "relu", 2.0, 0.5)
+    kw = dict(dtype=dtype, stride=stride, pad=pad, groups=groups, scale=scale, shift=shift, act="leaky", residual=res, act2="relu",
+              res_mul=2.0, out_mul=0.5, algo="igemm_splitk", out_ld=oc + 8, res_ld=oc + 8)
+    L = abi.lib()
+    d = abi.ConvDesc(dtype, dtype, b, h, w, c, c, oc, oh, ow, oc + 8, k, stride, pad, 1, groups, abi.ACT["leaky"], 0.1, 1, oc + 8, abi.ACT["relu"], 0.1, 2.0, 0.5,
+                     abi.ALGO["igemm_splitk"], 0)
+    tried = 0
+    for tile in range(0, L.msnh_hip_conv2d_tile_count() + 1):
+        d.tile = tile
+        if not L.msnh_hip_conv2d_tile_supported(ctypes.byref(d), tile):
+            continue
+        y, used = gu.conv2d(x, wt, tile=tile, **kw)
+        assert used == "igemm_splitk"
+        assert gu.rel_err(y, ref) <= TOL[dtype], (tile, gu.rel_err(y, ref))
+        if tried % 4 == 0:
+            y2, _ = gu.conv2d(x, wt, tile=tile, **kw)
+            assert np.array_equal(y, y2), tile
+        tried += 1
+    assert tried >= 3
+
+
+def test_conv_split_k_rejects():
+    """Split-K needs its workspace, a K loop long enough to cut, and few enough output tiles to be worth cutting."""
+    import ctypes
+    L = abi.lib()
+    # a 1x1 layer over 16 channels has a single tile step
+    d = abi.ConvDesc(abi.F16, abi.F16, 1, 8, 8, 16, 16, 16, 8, 8, 16, 1, 1, 0, 1, 1, 22, 0.1, 0, 16, 22, 0.1, 1.0, 1.0, abi.ALGO["igemm_splitk"], 0)
+    assert all(L.msnh_hip_conv2d_tile_supported(ctypes.byref(d), t) == 0 for t in range(0, L.msnh_hip_conv2d_tile_count() + 1))
+    # a launch that already fills the chip
+    d = abi.ConvDesc(abi.F16, abi.F16, 8, 76, 76, 256, 256, 256, 76, 76, 256, 3, 1, 1, 1, 1, 22, 0.1, 0, 256, 22, 0.1, 1.0, 1.0, abi.ALGO["igemm_splitk"], 1)
+    assert L.msnh_hip_conv2d_tile_supported(ctypes.byref(d), 1) == 0
+    # a good shape without its workspace
+    d = abi.ConvDesc(abi.F16, abi.F16, 1, 7, 7, 512, 512, 512, 7, 7, 512, 3, 1, 1, 1, 1, 22, 0.1, 0, 512, 22, 0.1, 1.0, 1.0, abi.ALGO["igemm_splitk"], 1)
+    assert L.msnh_hip_conv2d_tile_supported(ctypes.byref(d), 1) == 1
+    assert L.msnh_hip_conv2d_workspace_bytes(ctypes.byref(d), abi.ALGO["igemm_splitk"]) == 8 * 49 * 512 * 4
+    buf = ctypes.c_void_p(256)
+    assert L.msnh_hip_conv2d(ctypes.byref(d), buf, buf, None, None, None, buf, None, 0, None) != 0
+    assert b"workspace" in L.msnh_hip_last_error()
+
+
 def test_conv_winograd_rejects():
     import ctypes
     import gpuutil as gu
