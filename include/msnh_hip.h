@@ -43,6 +43,7 @@ enum msnh_act
     MSNH_ACT_RELU6    = 2,
     MSNH_ACT_LEAKY    = 8,
     MSNH_ACT_SWISH    = 16,
+    MSNH_ACT_HARD_SWISH = 17,
     MSNH_ACT_MISH     = 18,
     MSNH_ACT_NONE     = 22
 };
@@ -182,6 +183,23 @@ int msnh_hip_avgpool(int dtype, int out_dtype, int batch, int in_h, int in_w, in
  * src/core/cuda/MsnhBlasGPU.cu:541-578, without its fill + accumulate). */
 int msnh_hip_upsample_nearest(int dtype, int batch, int in_h, int in_w, int c, const void *x, int x_ld, int stride,
                               float scale, void *y, int y_ld, msnh_stream_t s);
+/* Constant padding of the two image axes (PaddingLayer::forward, src/layers/MsnhPaddingLayer.cpp:143-177):
+ * y[oy][ox] = mul * x[oy-top][ox-left] inside the image, `value` outside.  out_h/out_w = in + top + down / left + right. */
+int msnh_hip_pad(int dtype, int batch, int in_h, int in_w, int c, const void *x, int x_ld, int top, int left, int out_h,
+                 int out_w, float mul, float value, void *y, int y_ld, msnh_stream_t s);
+/* Strided slice of channels, rows and columns (SliceLayer::forward, src/layers/MsnhSliceLayer.cpp:120-147):
+ * y[oc][oy][ox] = mul * x[c0 + oc*cs][h0 + oy*hs][w0 + ox*ws]. */
+int msnh_hip_slice(int dtype, int batch, int in_h, int in_w, const void *x, int x_ld, int c0, int cs, int h0, int hs, int w0,
+                   int ws, int out_c, int out_h, int out_w, float mul, void *y, int y_ld, msnh_stream_t s);
+/* Bilinear resize, source index (o + 0.5) * in/out - 0.5 clamped at 0 (align_corners 0) or o * (in-1)/(out-1)
+ * (align_corners 1), float32 weights (Blas::cpuBilinearResize, src/core/MsnhBlas.cpp:2400-2465).  y = mul * value. */
+int msnh_hip_upsample_bilinear(int dtype, int batch, int in_h, int in_w, int c, const void *x, int x_ld, int out_h, int out_w,
+                               int align_corners, float mul, void *y, int y_ld, msnh_stream_t s);
+/* Softmax over all pixels*c values of each image: e_i = exp(x_i/T - max/T), y_i = y_mul * e_i / sum e
+ * (SoftMaxLayer::forward with groups 1, src/layers/MsnhSoftMaxLayer.cpp:60-93; Blas::softmax, src/core/MsnhBlas.cpp:1970-2110).
+ * x_mul undoes the input's power-of-two storage scale. */
+int msnh_hip_softmax(int dtype, int batch, int pixels, int c, const void *x, int x_ld, float x_mul, float temperature, void *y,
+                     int y_ld, float y_mul, msnh_stream_t s);
 /* Fully connected layer out[b][o] = act( sum_i x[b][i]*w[o][i] + bias[o] ) (cublasSgemm NT + bias,
  * src/layers/MsnhConnectedLayer.cpp:300-360).  x: [batch][inputs] d-type; w: [outputs][inputs] dtype;
  * y: float32 [batch][outputs].  x_mul undoes the input's power-of-two storage scale. */
@@ -208,12 +226,14 @@ int msnh_hip_letterbox_u8(const unsigned char *rgb_hwc, int width, int height, i
  *   x        : head logits NHWC, channel = anchor*(5+classes)+m, times x_mul gives the true logit
  *   decoded  : float32, element (b,anchor,pixel,m) at decoded[b*decoded_batch_stride + ((anchor*h*w)+pixel)*(5+classes) + m]
  *              (the reference's "shuffled" order; the stride lets all heads of an image share one buffer)
+ *   yolo_version : 3 or 4: centre (s + cell)*ratio, size anchor*e^t; 5: centre (2s - 0.5 + cell)*ratio, size anchor*(2s)^2
+ *              (src/layers/MsnhYoloLayer.cpp:84-136)
  *   cand_idx : optional int32 [batch][cand_cap]; receives (anchor*h*w + pixel) + cand_base of every entry
  *              with objectness > conf_thresh, in no particular order;
  *   cand_cnt : int32 [batch], incremented by the number of entries found (caller zeroes it).
  * ---------------------------------------------------------------------------------------------- */
 int msnh_hip_yolo_decode(int dtype, int batch, int h, int w, int classes, const void *x, int x_ld, float x_mul,
-                         const float *anchors6, float ratio, float *decoded, long long decoded_batch_stride,
+                         const float *anchors6, float ratio, int yolo_version, float *decoded, long long decoded_batch_stride,
                          float conf_thresh, int *cand_idx, int cand_cap, int cand_base, int *cand_cnt, msnh_stream_t s);
 /* Candidate compaction for YoloOutLayer (the per-box part of src/layers/MsnhYoloOutLayer.cpp:120-170 done on
  * the device so that only surviving boxes cross PCIe): for image b and k < min(cand_cnt[b], cand_cap) reads

@@ -32,8 +32,21 @@ def _run(cmd):
     return out
 
 
+# `python -m msnhnet_amd.build --changed` (a developer convenience; build_all() itself always compiles everything) skips a
+# source whose object is newer than the source and every header of the tree.
+ONLY_CHANGED = False
+
+
+def _newest_header():
+    hs = glob.glob(os.path.join(PKG, "csrc", "*.hpp")) + glob.glob(os.path.join(ROOT, "include", "*.h")) + \
+        glob.glob(os.path.join(PKG, "host", "include", "**", "*.h"), recursive=True)
+    return max(os.path.getmtime(h) for h in hs)
+
+
 def _compile(src, obj, flags, compiler):
     os.makedirs(os.path.dirname(obj), exist_ok=True)
+    if ONLY_CHANGED and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), _newest_header()):
+        return ""
     return _run([compiler, *flags, "-c", src, "-o", obj])
 
 
@@ -71,4 +84,6 @@ def build_all(verbose=True):
 
 
 if __name__ == "__main__":
+    import sys
+    ONLY_CHANGED = "--changed" in sys.argv[1:]
     print(build_all())

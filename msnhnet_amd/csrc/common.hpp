@@ -90,6 +90,12 @@ __device__ __forceinline__ float activate(float x, int act, float param)
     case MSNH_ACT_RELU6:    return (x > 0.f ? x : 0.f) > 6.f ? 6.f : (x > 0.f ? x : 0.f);
     case MSNH_ACT_LEAKY:    return x > 0.f ? x : param * x;
     case MSNH_ACT_SWISH:    return x * logisticF(x);
+    case MSNH_ACT_HARD_SWISH:
+    {
+        const float t = x + 3.f;
+        const float r = (t > 0.f ? t : 0.f) > 6.f ? 6.f : (t > 0.f ? t : 0.f);
+        return x * r / 6.f;                                     // x*relu6(x+3)/6, evaluated in that order
+    }
     case MSNH_ACT_MISH:     return mishF(x);
     default:                return x;
     }
@@ -98,7 +104,7 @@ __device__ __forceinline__ float activate(float x, int act, float param)
 inline bool actOk(int act)
 {
     return act == MSNH_ACT_LOGISTIC || act == MSNH_ACT_RELU || act == MSNH_ACT_RELU6 || act == MSNH_ACT_LEAKY ||
-           act == MSNH_ACT_SWISH || act == MSNH_ACT_MISH || act == MSNH_ACT_NONE;
+           act == MSNH_ACT_SWISH || act == MSNH_ACT_HARD_SWISH || act == MSNH_ACT_MISH || act == MSNH_ACT_NONE;
 }
 
 inline unsigned gridFor(long long n, int block)

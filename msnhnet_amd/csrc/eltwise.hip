@@ -190,6 +190,137 @@ __global__ __launch_bounds__(256) void copyChannelsKernel(const T *__restrict__ 
     storeVec<T, VEC>(y + p * yLd + c0, v);
 }
 
+// ---- constant padding / strided slice / bilinear resize ---------------------------------------------------------
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void padKernel(const T *__restrict__ x, int xLd, int H, int W, int c, int top, int left, int OH, int OW,
+                                                 float mul, float value, T *__restrict__ y, int yLd, long long total)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int cv = c / VEC;
+    const int c0 = static_cast<int>(idx % cv) * VEC;
+    const long long p = idx / cv;
+    const int ox = static_cast<int>(p % OW);
+    const long long t = p / OW;
+    const int oy = static_cast<int>(t % OH);
+    const long long b = t / OH;
+    const int iy = oy - top, ix = ox - left;
+    float v[VEC];
+    if (iy >= 0 && iy < H && ix >= 0 && ix < W)
+    {
+        loadVec<T, VEC>(x + ((b * H + iy) * W + ix) * xLd + c0, v);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = mul * v[i];
+    }
+    else
+    {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = value;
+    }
+    storeVec<T, VEC>(y + p * yLd + c0, v);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void sliceKernel(const T *__restrict__ x, int xLd, int H, int W, int c0, int cs, int h0, int hs, int w0, int ws,
+                                                   int OC, int OH, int OW, float mul, T *__restrict__ y, int yLd, long long total)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int oc = static_cast<int>(idx % OC);
+    const long long p = idx / OC;
+    const int ox = static_cast<int>(p % OW);
+    const long long t = p / OW;
+    const int oy = static_cast<int>(t % OH);
+    const long long b = t / OH;
+    const float v = toF(x[((b * H + h0 + oy * hs) * W + w0 + ox * ws) * xLd + c0 + oc * cs]);
+    y[p * yLd + oc] = fromF<T>(mul * v);
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void bilinearKernel(const T *__restrict__ x, int xLd, int H, int W, int c, int OH, int OW, int alignCorners,
+                                                      float rH, float rW, float mul, T *__restrict__ y, int yLd, long long total)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int cv = c / VEC;
+    const int c0 = static_cast<int>(idx % cv) * VEC;
+    const long long p = idx / cv;
+    const int ox = static_cast<int>(p % OW);
+    const long long t = p / OW;
+    const int oy = static_cast<int>(t % OH);
+    const long long b = t / OH;
+    float h1r, w1r;
+    if (alignCorners == 0)
+    {
+        const float ih = rH * (oy + 0.5f) - 0.5f;
+        const float iw = rW * (ox + 0.5f) - 0.5f;
+        h1r = ih < 0 ? 0 : ih;
+        w1r = iw < 0 ? 0 : iw;
+    }
+    else
+    {
+        h1r = rH * oy;
+        w1r = rW * ox;
+    }
+    const int h1 = static_cast<int>(h1r), w1 = static_cast<int>(w1r);
+    const int h1p = h1 < H - 1 ? 1 : 0, w1p = w1 < W - 1 ? 1 : 0;
+    const float h1L = h1r - h1, h0L = 1.f - h1L, w1L = w1r - w1, w0L = 1.f - w1L;
+    const T *base = x + ((b * H + h1) * W + w1) * xLd + c0;
+    float v00[VEC], v01[VEC], v10[VEC], v11[VEC], o[VEC];
+    loadVec<T, VEC>(base, v00);
+    loadVec<T, VEC>(base + static_cast<long long>(w1p) * xLd, v01);
+    loadVec<T, VEC>(base + static_cast<long long>(h1p) * W * xLd, v10);
+    loadVec<T, VEC>(base + (static_cast<long long>(h1p) * W + w1p) * xLd, v11);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i)
+        o[i] = mul * (h0L * (w0L * v00[i] + w1L * v01[i]) + h1L * (w0L * v10[i] + w1L * v11[i]));
+    storeVec<T, VEC>(y + p * yLd + c0, o);
+}
+
+// ---- softmax over all values of one image --------------------------------------------------------------------
+// One workgroup per image: maximum, sum of exp((x - max) / T), quotient (Blas::softmax, src/core/MsnhBlas.cpp:1970-2110).
+template <typename T>
+__global__ __launch_bounds__(256) void softmaxKernel(const T *__restrict__ x, int xLd, float xMul, int pixels, int c, float temperature,
+                                                     T *__restrict__ y, int yLd, float yMul)
+{
+    __shared__ float red[256];
+    const int b = blockIdx.x;
+    const long long n = static_cast<long long>(pixels) * c;
+    const T *xb = x + static_cast<size_t>(b) * pixels * xLd;
+    T *yb = y + static_cast<size_t>(b) * pixels * yLd;
+    float m = -3.402823466e38f;
+    for (long long i = threadIdx.x; i < n; i += 256)
+    {
+        const float v = xMul * toF(xb[(i / c) * xLd + (i % c)]);
+        m = v > m ? v : m;
+    }
+    red[threadIdx.x] = m;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1)
+    {
+        if (threadIdx.x < s) red[threadIdx.x] = red[threadIdx.x + s] > red[threadIdx.x] ? red[threadIdx.x + s] : red[threadIdx.x];
+        __syncthreads();
+    }
+    const float largest = red[0];
+    __syncthreads();
+    float sum = 0.f;
+    for (long long i = threadIdx.x; i < n; i += 256)
+        sum += expf(xMul * toF(xb[(i / c) * xLd + (i % c)]) / temperature - largest / temperature);
+    red[threadIdx.x] = sum;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1)
+    {
+        if (threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+        __syncthreads();
+    }
+    const float total = red[0];
+    for (long long i = threadIdx.x; i < n; i += 256)
+    {
+        const float e = expf(xMul * toF(xb[(i / c) * xLd + (i % c)]) / temperature - largest / temperature);
+        yb[(i / c) * yLd + (i % c)] = fromF<T>(yMul * (e / total));
+    }
+}
+
 // ---- fully connected: one wavefront per (batch row, output), wave-level reduction -------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void connectedKernel(const T *__restrict__ x, float xMul, const T *__restrict__ w,
@@ -341,7 +472,9 @@ int msnh_hip_copy_channels(int dtype, long long pixels, int c, const void *x, in
 static int checkPool(const char *name, int batch, int in_h, int in_w, int c, int ksize, int stride, int pad, int out_h, int out_w)
 {
     MSNH_REQUIRE(batch > 0 && in_h > 0 && in_w > 0 && c > 0 && ksize > 0 && stride > 0 && pad >= 0, "%s: bad geometry", name);
-    MSNH_REQUIRE(in_h + 2 * pad >= ksize && in_w + 2 * pad >= ksize, "%s: window larger than padded input", name);
+    // (a single window that covers the whole plane may overhang the shorter axis: the global mean of a non-square plane)
+    MSNH_REQUIRE((in_h + 2 * pad >= ksize && in_w + 2 * pad >= ksize) || (out_h == 1 && out_w == 1 && pad == 0),
+                 "%s: window larger than padded input", name);
     MSNH_REQUIRE(out_h > 0 && out_w > 0, "%s: non-positive output size", name);
     // every window must start inside the padded input (covers floor and ceil output sizes)
     MSNH_REQUIRE((out_h - 1) * stride - pad < in_h && (out_w - 1) * stride - pad < in_w, "%s: output size too large", name);
@@ -407,6 +540,85 @@ int msnh_hip_upsample_nearest(int dtype, int batch, int in_h, int in_w, int c, c
     if (dtype == MSNH_F16) { if (vec == 8) MSNH_UP(f16, 8); else MSNH_UP(f16, 1); }
     else { if (vec == 4) MSNH_UP(float, 4); else MSNH_UP(float, 1); }
 #undef MSNH_UP
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+int msnh_hip_pad(int dtype, int batch, int in_h, int in_w, int c, const void *x, int x_ld, int top, int left, int out_h,
+                 int out_w, float mul, float value, void *y, int y_ld, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "pad: bad dtype");
+    MSNH_REQUIRE(batch > 0 && in_h > 0 && in_w > 0 && c > 0 && top >= 0 && left >= 0 && out_h >= in_h + top && out_w >= in_w + left, "pad: bad geometry");
+    MSNH_REQUIRE(x && y && x_ld >= c && y_ld >= c, "pad: bad argument");
+    hipStream_t st = resolveStream(s);
+    const int vec = pickVec(dtype, c, {x_ld, y_ld}, {x, y});
+    const long long total = static_cast<long long>(batch) * out_h * out_w * (c / vec);
+    dim3 grid(gridFor(total, 256));
+#define MSNH_PAD(T, V)                                                                                                 \
+    hipLaunchKernelGGL((padKernel<T, V>), grid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, in_h, in_w, c, top, left, out_h, out_w, \
+                       mul, value, static_cast<T *>(y), y_ld, total)
+    if (dtype == MSNH_F16) { if (vec == 8) MSNH_PAD(f16, 8); else MSNH_PAD(f16, 1); }
+    else { if (vec == 4) MSNH_PAD(float, 4); else MSNH_PAD(float, 1); }
+#undef MSNH_PAD
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+int msnh_hip_slice(int dtype, int batch, int in_h, int in_w, const void *x, int x_ld, int c0, int cs, int h0, int hs, int w0,
+                   int ws, int out_c, int out_h, int out_w, float mul, void *y, int y_ld, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "slice: bad dtype");
+    MSNH_REQUIRE(batch > 0 && in_h > 0 && in_w > 0 && out_c > 0 && out_h > 0 && out_w > 0 && c0 >= 0 && h0 >= 0 && w0 >= 0 && cs > 0 && hs > 0 && ws > 0,
+                 "slice: bad geometry");
+    MSNH_REQUIRE(h0 + (out_h - 1) * hs < in_h && w0 + (out_w - 1) * ws < in_w && c0 + (out_c - 1) * cs < x_ld, "slice: window leaves the tensor");
+    MSNH_REQUIRE(x && y && y_ld >= out_c, "slice: bad argument");
+    hipStream_t st = resolveStream(s);
+    const long long total = static_cast<long long>(batch) * out_h * out_w * out_c;
+    dim3 grid(gridFor(total, 256));
+    if (dtype == MSNH_F16)
+        hipLaunchKernelGGL((sliceKernel<f16>), grid, dim3(256), 0, st, static_cast<const f16 *>(x), x_ld, in_h, in_w, c0, cs, h0, hs, w0, ws, out_c, out_h,
+                           out_w, mul, static_cast<f16 *>(y), y_ld, total);
+    else
+        hipLaunchKernelGGL((sliceKernel<float>), grid, dim3(256), 0, st, static_cast<const float *>(x), x_ld, in_h, in_w, c0, cs, h0, hs, w0, ws, out_c,
+                           out_h, out_w, mul, static_cast<float *>(y), y_ld, total);
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+int msnh_hip_upsample_bilinear(int dtype, int batch, int in_h, int in_w, int c, const void *x, int x_ld, int out_h, int out_w,
+                               int align_corners, float mul, void *y, int y_ld, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "bilinear: bad dtype");
+    MSNH_REQUIRE(batch > 0 && in_h > 0 && in_w > 0 && c > 0 && out_h > 0 && out_w > 0, "bilinear: w*x and outw*outx must > 1");
+    MSNH_REQUIRE(x && y && x_ld >= c && y_ld >= c, "bilinear: bad argument");
+    hipStream_t st = resolveStream(s);
+    const float rH = align_corners == 0 ? 1.0f * in_h / out_h : 1.0f * (in_h - 1) / (out_h - 1);
+    const float rW = align_corners == 0 ? 1.0f * in_w / out_w : 1.0f * (in_w - 1) / (out_w - 1);
+    const int vec = pickVec(dtype, c, {x_ld, y_ld}, {x, y});
+    const long long total = static_cast<long long>(batch) * out_h * out_w * (c / vec);
+    dim3 grid(gridFor(total, 256));
+#define MSNH_BIL(T, V)                                                                                                 \
+    hipLaunchKernelGGL((bilinearKernel<T, V>), grid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, in_h, in_w, c, out_h, out_w, align_corners, \
+                       rH, rW, mul, static_cast<T *>(y), y_ld, total)
+    if (dtype == MSNH_F16) { if (vec == 8) MSNH_BIL(f16, 8); else MSNH_BIL(f16, 1); }
+    else { if (vec == 4) MSNH_BIL(float, 4); else MSNH_BIL(float, 1); }
+#undef MSNH_BIL
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+int msnh_hip_softmax(int dtype, int batch, int pixels, int c, const void *x, int x_ld, float x_mul, float temperature, void *y,
+                     int y_ld, float y_mul, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "softmax: bad dtype");
+    MSNH_REQUIRE(batch > 0 && pixels > 0 && c > 0 && x && y && x_ld >= c && y_ld >= c && temperature != 0.f, "softmax: bad argument");
+    hipStream_t st = resolveStream(s);
+    if (dtype == MSNH_F16)
+        hipLaunchKernelGGL((softmaxKernel<f16>), dim3(batch), dim3(256), 0, st, static_cast<const f16 *>(x), x_ld, x_mul, pixels, c, temperature,
+                           static_cast<f16 *>(y), y_ld, y_mul);
+    else
+        hipLaunchKernelGGL((softmaxKernel<float>), dim3(batch), dim3(256), 0, st, static_cast<const float *>(x), x_ld, x_mul, pixels, c, temperature,
+                           static_cast<float *>(y), y_ld, y_mul);
     MSNH_LAUNCH_CHECK();
     return 0;
 }

@@ -1,4 +1,4 @@
-// YOLO v3/v4 head decode fused with the [anchor][channel][pixel] -> [anchor][pixel][channel] reordering and
+// YOLO v3/v4/v5 head decode fused with the [anchor][channel][pixel] -> [anchor][pixel][channel] reordering and
 // the objectness threshold.  The NHWC head tensor already stores the (5+classes) values of one anchor of
 // one pixel contiguously, so both the read and the write of a wavefront are contiguous runs.
 #include "common.hpp"
@@ -14,7 +14,7 @@ constexpr int YOLO_CHUNK = 256 * 8;
 
 // The 5 + classes logistics per cell are what the kernel computes most of (logisticF: hardware exp2 and
 // reciprocal); box width and height keep expf.
-template <typename T>
+template <typename T, bool V5>
 __global__ __launch_bounds__(256) void yoloDecodeKernel(const T *__restrict__ x, int xLd, float xMul, Anchors an, float ratio,
                                                         float *__restrict__ decoded, long long decStride, float confThresh, int *__restrict__ candIdx,
                                                         int candCap, int candBase, int *__restrict__ candCnt, int W, int HW, int per,
@@ -44,7 +44,17 @@ __global__ __launch_bounds__(256) void yoloDecodeKernel(const T *__restrict__ x,
         const bool live = idx < perImage;          // predicate, not an exit: the unrolled loads can then be issued together
         const float v = live ? xMul * toF(xb[static_cast<size_t>(p) * xLd + a * per + m]) : 0.f;
         float r;
-        if (m == 0)      r = (logisticF(v) + static_cast<float>(px)) * ratio;
+        if (V5)
+        {
+            // yolov5: centre (2s - 0.5 + cell) * ratio, size anchor * (2s)^2, s = logistic (src/layers/MsnhYoloLayer.cpp:250-296)
+            const float s2 = 2.f * logisticF(v);
+            if (m == 0)      r = (s2 - 0.5f + static_cast<float>(px)) * ratio;
+            else if (m == 1) r = (s2 - 0.5f + static_cast<float>(py)) * ratio;
+            else if (m == 2) r = an.v[(2 * a) % 6] * (s2 * s2);
+            else if (m == 3) r = an.v[(2 * a + 1) % 6] * (s2 * s2);
+            else             r = 0.5f * s2;
+        }
+        else if (m == 0) r = (logisticF(v) + static_cast<float>(px)) * ratio;
         else if (m == 1) r = (logisticF(v) + static_cast<float>(py)) * ratio;
         else if (m == 2) r = an.v[(2 * a) % 6] * expf(v);
         else if (m == 3) r = an.v[(2 * a + 1) % 6] * expf(v);
@@ -126,11 +136,12 @@ __global__ __launch_bounds__(256) void absMaxKernel(const T *__restrict__ x, int
 using namespace msnh;
 
 extern "C" int msnh_hip_yolo_decode(int dtype, int batch, int h, int w, int classes, const void *x, int x_ld, float x_mul,
-                                    const float *anchors6, float ratio, float *decoded, long long decoded_batch_stride,
+                                    const float *anchors6, float ratio, int yolo_version, float *decoded, long long decoded_batch_stride,
                                     float conf_thresh, int *cand_idx, int cand_cap, int cand_base, int *cand_cnt, msnh_stream_t s)
 {
     MSNH_REQUIRE(dtypeOk(dtype), "yolo_decode: bad dtype");
     MSNH_REQUIRE(batch > 0 && h > 0 && w > 0 && classes > 0, "yolo_decode: bad geometry");
+    MSNH_REQUIRE(yolo_version == 3 || yolo_version == 4 || yolo_version == 5, "yolo_decode: yolo_version must be 3, 4 or 5");
     const int per = 5 + classes;
     MSNH_REQUIRE(x && decoded && anchors6 && x_ld >= 3 * per, "yolo_decode: bad argument");
     MSNH_REQUIRE(decoded_batch_stride >= static_cast<long long>(3) * h * w * per, "yolo_decode: decoded_batch_stride too small");
@@ -141,12 +152,12 @@ extern "C" int msnh_hip_yolo_decode(int dtype, int batch, int h, int w, int clas
     const int perImage = 3 * h * w * per;
     dim3 grid((perImage + YOLO_CHUNK - 1) / YOLO_CHUNK, batch);
     hipStream_t st = resolveStream(s);
-    if (dtype == MSNH_F16)
-        hipLaunchKernelGGL((yoloDecodeKernel<f16>), grid, dim3(256), 0, st, static_cast<const f16 *>(x), x_ld, x_mul, an, ratio, decoded,
-                           decoded_batch_stride, conf_thresh, cand_idx, cand_cap, cand_base, cand_cnt, w, h * w, per, perImage);
-    else
-        hipLaunchKernelGGL((yoloDecodeKernel<float>), grid, dim3(256), 0, st, static_cast<const float *>(x), x_ld, x_mul, an, ratio,
-                           decoded, decoded_batch_stride, conf_thresh, cand_idx, cand_cap, cand_base, cand_cnt, w, h * w, per, perImage);
+#define MSNH_YOLO(T, V5)                                                                                                \
+    hipLaunchKernelGGL((yoloDecodeKernel<T, V5>), grid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, x_mul, an, ratio, decoded, \
+                       decoded_batch_stride, conf_thresh, cand_idx, cand_cap, cand_base, cand_cnt, w, h * w, per, perImage)
+    if (dtype == MSNH_F16) { if (yolo_version == 5) MSNH_YOLO(f16, true); else MSNH_YOLO(f16, false); }
+    else { if (yolo_version == 5) MSNH_YOLO(float, true); else MSNH_YOLO(float, false); }
+#undef MSNH_YOLO
     MSNH_LAUNCH_CHECK();
     return 0;
 }

@@ -48,7 +48,7 @@ struct PlanTensor
 
 struct PlanOp
 {
-    enum Kind { CONV = 0, AFFINE, ADD, COPY, MAXPOOL, AVGPOOL, UPSAMPLE, CONNECTED, INPUT_CAST, YOLO_DECODE };
+    enum Kind { CONV = 0, AFFINE, ADD, COPY, MAXPOOL, AVGPOOL, UPSAMPLE, CONNECTED, INPUT_CAST, YOLO_DECODE, PAD, SLICE, BILINEAR, SOFTMAX };
     Kind kind = CONV;
     int  in0 = -1, in1 = -1, out = -1;
     bool dead = false;
@@ -59,8 +59,15 @@ struct PlanOp
     int  ksize = 1, stride = 1, pad = 0, dilation = 1, groups = 1;
     ActivationType act = NONE, act2 = NONE;
     float actParam = 0.1f, act2Param = 0.1f;
-    float upScale = 1.f;
+    float upScale = 1.f;                    // UPSAMPLE: value scale; SOFTMAX: temperature
     int  dstChanOffset = 0;                 // COPY: channel offset inside `out`
+    bool pureAct = false;                   // AFFINE with identity scale and shift: only the activation matters
+    float in1Sign = 1.f;                    // ADD: out = act(in0 + in1Sign * in1)
+    int  padTop = 0, padLeft = 0;           // PAD
+    float padValue = 0.f;
+    int  slice[6] = {0, 1, 0, 1, 0, 1};     // SLICE: start / step of channels, rows, columns
+    int  alignCorners = 0;                  // BILINEAR
+    int  yoloVersion = 3;                   // YOLO_DECODE: 3, 4 or 5
     int  algo = MSNH_CONV_AUTO;             // CONV: resolved at weight preparation
     int  tile = 0;                          // CONV/IGEMM: tile configuration chosen by Plan::tuneConvs (0 = library default)
     BaseLayer *src = nullptr;               // layer that owns the host weights of this op
@@ -89,6 +96,7 @@ public:
     std::vector<PlanOp>     ops;
     std::vector<int>        layerOut;       // output tensor of each top-level layer
     int inputTensor = -1;
+    int inputNhwc = -1;                     // NHWC copy of the network input, made on first use by a non-convolution first layer
 
     // YOLO post-processing buffers (only for networks ending in a yoloout layer)
     int  yoloCells = 0;                     // sum over heads of 3*H*W
@@ -98,6 +106,7 @@ public:
     int addTensor(int n, int h, int w, int c, int dtype, const std::string &name, PlanTensor::Layout layout = PlanTensor::NHWC);
     PlanOp &addOp(PlanOp::Kind kind, int in0, int in1, int out, int layerIndex, const std::string &name);
     int producerOf(int tensor) const;       // last live op writing `tensor`, or -1
+    int nhwcOf(int tensor, int layerIndex); // `tensor` itself, or (for the NCHW network input) its NHWC copy in the compute dtype
     int consumerCount(int tensor) const;
 
     void fuse();                            // passes 1

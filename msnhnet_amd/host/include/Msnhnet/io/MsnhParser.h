@@ -145,6 +145,61 @@ public:
     std::vector<float> actParams;
 };
 
+class MsnhNet_API GlobalAvgPoolParams : public BaseParams
+{
+public:
+    explicit GlobalAvgPoolParams(bool inc) : BaseParams(inc) { type = LayerType::GLOBAL_AVGPOOL; }
+};
+
+class MsnhNet_API SoftMaxParams : public BaseParams
+{
+public:
+    explicit SoftMaxParams(bool inc) : BaseParams(inc) { type = LayerType::SOFTMAX; }
+    int groups = 1;
+    float temperature = 1;
+};
+
+class MsnhNet_API ActivationParams : public BaseParams
+{
+public:
+    explicit ActivationParams(bool inc) : BaseParams(inc) { type = LayerType::ACTIVE; }
+    ActivationType activation = ActivationType::NONE;
+    std::vector<float> actParams;
+};
+
+class MsnhNet_API PaddingParams : public BaseParams
+{
+public:
+    explicit PaddingParams(bool inc) : BaseParams(inc) { type = LayerType::PADDING; }
+    int top = 0, down = 0, left = 0, right = 0;
+    float paddingVal = 0;
+};
+
+class MsnhNet_API SliceParams : public BaseParams
+{
+public:
+    explicit SliceParams(bool inc) : BaseParams(inc) { type = LayerType::SLICE; }
+    int start0 = 0, step0 = 1, start1 = 0, step1 = 1, start2 = 0, step2 = 1;
+};
+
+class MsnhNet_API VariableOpParams : public BaseParams
+{
+public:
+    enum VarOpType
+    {
+        VAR_OP_ADD = 0, VAR_OP_SUB, VAR_OP_SUB_INV, VAR_OP_MUL, VAR_OP_DIV, VAR_OP_DIV_INV,
+        VAR_OP_ADD_CONST, VAR_OP_SUB_CONST, VAR_OP_SUB_CONST_INV, VAR_OP_MUL_CONST, VAR_OP_DIV_CONST, VAR_OP_DIV_CONST_INV,
+        VAR_OP_ABS, VAR_OP_ACOS, VAR_OP_ASIN, VAR_OP_ATAN, VAR_OP_COS, VAR_OP_COSH, VAR_OP_SIN, VAR_OP_SINH, VAR_OP_TAN, VAR_OP_TANH,
+        VAR_OP_EXP, VAR_OP_POW, VAR_OP_LOG, VAR_OP_LOG10, VAR_OP_SQRT
+    };
+    explicit VariableOpParams(bool inc) : BaseParams(inc) { type = LayerType::VARIABLE_OP; }
+    std::vector<int> layerIndexes;
+    VarOpType varOpType = VAR_OP_ADD;
+    float constVal = 0;
+    static VarOpType getVarOpTypeFromStr(const std::string &s);
+    static std::string getStrFromVarOpType(const VarOpType &t);
+};
+
 class MsnhNet_API UpSampleParams : public BaseParams
 {
 public:

@@ -128,6 +128,80 @@ public:
 private:
     int _strideX, _strideY;
     float _scaleX, _scaleY;
+    UpSampleParams::UpsampleType _upsampleType;
+    int _alignCorners;
+};
+
+// src/layers/MsnhGlobalAvgPoolLayer.cpp:5-30, 152-168: mean of every channel plane
+class MsnhNet_API GlobalAvgPoolLayer : public BaseLayer
+{
+public:
+    GlobalAvgPoolLayer(const int &batch, const int &height, const int &width, const int &channel);
+    int lower(Plan &plan, int in, int layerIndex) override;
+};
+
+// src/layers/MsnhSoftMaxLayer.cpp:5-30, 60-93 (groups == 1: one softmax over all values of an image)
+class MsnhNet_API SoftMaxLayer : public BaseLayer
+{
+public:
+    SoftMaxLayer(const int &batch, const int &inputNum, const int &groups, const float &temperature);
+    int lower(Plan &plan, int in, int layerIndex) override;
+
+private:
+    int _groups;
+    float _temperature;
+};
+
+// src/layers/MsnhActivationLayer.cpp:5-40 (stand-alone activation; PReLU, which owns weights, is not implemented)
+class MsnhNet_API ActivationLayer : public BaseLayer
+{
+public:
+    ActivationLayer(const int &batch, const int &width, const int &height, const int &channel, const int &inputNum,
+                    const ActivationType &activation, const std::vector<float> &actParams);
+    int lower(Plan &plan, int in, int layerIndex) override;
+    void foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const override;
+};
+
+// src/layers/MsnhPaddingLayer.cpp:5-45
+class MsnhNet_API PaddingLayer : public BaseLayer
+{
+public:
+    PaddingLayer(const int &batch, const int &height, const int &width, const int &channel, const int &top, const int &down,
+                 const int &left, const int &right, const float &paddingVal);
+    int lower(Plan &plan, int in, int layerIndex) override;
+
+private:
+    int _top, _down, _left, _right;
+    float _paddingVal;
+};
+
+// src/layers/MsnhSliceLayer.cpp:5-70
+class MsnhNet_API SliceLayer : public BaseLayer
+{
+public:
+    SliceLayer(const int &batch, const int &height, const int &width, const int &channel, const int &start0, const int &step0,
+               const int &start1, const int &step1, const int &start2, const int &step2);
+    int lower(Plan &plan, int in, int layerIndex) override;
+
+private:
+    int _start0, _step0, _start1, _step1, _start2, _step2;
+};
+
+// src/layers/MsnhVariableOpLayer.cpp:5-60.  Implemented: add / sub / subInv of two tensors and the constant forms
+// addConst / subConst / subConstInv / mulConst / divConst.
+class MsnhNet_API VariableOpLayer : public BaseLayer
+{
+public:
+    VariableOpLayer(const int &batch, const int &width, const int &height, const int &channel, std::vector<int> &inputLayerIndexes,
+                    const VariableOpParams::VarOpType &varOpType, const float &constVal);
+    int lower(Plan &plan, int in, int layerIndex) override;
+    void foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const override;
+    const std::vector<int> &inputLayerIndexes() const { return _inputLayerIndexes; }
+
+private:
+    std::vector<int> _inputLayerIndexes;
+    VariableOpParams::VarOpType _varOpType;
+    float _constVal;
 };
 
 // src/layers/MsnhEmptyLayer.cpp (identity)
@@ -145,6 +219,7 @@ public:
     RouteLayer(const int &batch, std::vector<int> &inputLayerIndexes, std::vector<int> &inputLayerOutputs, const int &groups,
                const int &groupIndex, const int &addModel, const ActivationType &activation, const std::vector<float> &actParams);
     int lower(Plan &plan, int in, int layerIndex) override;
+    void foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const override;
     const std::vector<int> &inputLayerIndexes() const { return _inputLayerIndexes; }
     std::vector<int> inputChannels;         // channels of each routed layer, set by NetBuilder
 

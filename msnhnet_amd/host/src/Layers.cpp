@@ -407,29 +407,254 @@ int ConnectedLayer::lower(Plan &plan, int in, int layerIndex)
 // ---- UpSample / Empty / Route ---------------------------------------------------------------------------------------------------
 UpSampleLayer::UpSampleLayer(const int &batch, const int &width, const int &height, const int &channel, const int &strideX, const int &strideY,
                              const float &scaleX, const float &scaleY, UpSampleParams::UpsampleType upsampleType, const int &alignCorners)
-    : _strideX(strideX), _strideY(strideY), _scaleX(scaleX), _scaleY(scaleY)
+    : _strideX(strideX), _strideY(strideY), _scaleX(scaleX), _scaleY(scaleY), _upsampleType(upsampleType), _alignCorners(alignCorners)
 {
-    (void)alignCorners;
-    if (upsampleType != UpSampleParams::NEAREST) MSNH_THROW("upsample: bilinear mode is outside the convolutional path this build implements");
-    if (strideX != strideY || strideX <= 0) MSNH_THROW("upsample: strideX and strideY must be equal and positive");
     _type = LayerType::UPSAMPLE;
     _layerName = "UpSample        ";
     _batch = batch; _width = width; _height = height; _channel = channel;
-    _outWidth = width * strideX; _outHeight = height * strideY; _outChannel = channel;
+    if (upsampleType == UpSampleParams::NEAREST)
+    {
+        if (strideX != strideY || strideX <= 0) MSNH_THROW("upsample: strideX and strideY must be equal and positive");
+        _outWidth = width * strideX; _outHeight = height * strideY;
+    }
+    else
+    {
+        // src/layers/MsnhUpSampleLayer.cpp:20-24
+        _outWidth = static_cast<int>(width * scaleX); _outHeight = static_cast<int>(height * scaleY);
+        if (_outWidth < 1 || _outHeight < 1) MSNH_THROW("w*x and outw*outx must > 1");
+    }
+    _outChannel = channel;
     _outputNum = _outWidth * _outHeight * _outChannel;
     _inputNum = width * height * channel;
     _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
-    _layerDetail = fmt("upsample              %2dx%2d  %4d x%4d x%4d -> %4d x%4d x%4d\n", _strideX, _strideY, _width, _height, _channel, _outHeight,
-                       _outHeight, _outChannel);
+    if (upsampleType == UpSampleParams::NEAREST)
+        _layerDetail = fmt("upsample              %2dx%2d  %4d x%4d x%4d -> %4d x%4d x%4d\n", _strideX, _strideY, _width, _height, _channel, _outHeight,
+                           _outHeight, _outChannel);
+    else
+        _layerDetail = fmt("upsample          %4fx%4f  %4d x%4d x%4d -> %4d x%4d x%4d\n", _scaleX, _scaleY, _width, _height, _channel, _outHeight,
+                           _outHeight, _outChannel);
 }
 
 int UpSampleLayer::lower(Plan &plan, int in, int layerIndex)
 {
-    if (plan.tensors[static_cast<size_t>(in)].layout != PlanTensor::NHWC) MSNH_THROW("upsample can not be the first layer of a network");
+    in = plan.nhwcOf(in, layerIndex);
     const int out = plan.addTensor(_batch, _outHeight, _outWidth, _outChannel, plan.tensors[static_cast<size_t>(in)].dtype, "upsample_out");
+    if (_upsampleType == UpSampleParams::BILINEAR)
+    {
+        PlanOp &op = plan.addOp(PlanOp::BILINEAR, in, -1, out, layerIndex, "upsample_bilinear");
+        op.alignCorners = _alignCorners;
+        return out;
+    }
     PlanOp &op = plan.addOp(PlanOp::UPSAMPLE, in, -1, out, layerIndex, "upsample");
     op.stride = _strideX;
     op.upScale = _scaleX;          // Blas::cpuUpSample is called with scaleX only (src/layers/MsnhUpSampleLayer.cpp:106)
+    return out;
+}
+
+GlobalAvgPoolLayer::GlobalAvgPoolLayer(const int &batch, const int &height, const int &width, const int &channel)
+{
+    _type = LayerType::GLOBAL_AVGPOOL;
+    _layerName = "GlobalAvgPool   ";
+    _batch = batch; _height = height; _width = width; _channel = channel;
+    _outWidth = 1; _outHeight = 1; _outChannel = channel;
+    _inputNum = height * width * channel;
+    _outputNum = channel;
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _layerDetail = fmt("GlobalAvgPool                %4d x%4d x%4d ->   %4d\n", _width, _height, _channel, _outChannel);
+}
+
+int GlobalAvgPoolLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    in = plan.nhwcOf(in, layerIndex);
+    const PlanTensor ti = plan.tensors[static_cast<size_t>(in)];
+    if (ti.layout != PlanTensor::NHWC) MSNH_THROW("globalavgpool: the input must be an image tensor");
+    const int out = plan.addTensor(ti.n, 1, 1, ti.c, ti.dtype, "globalavgpool_out");
+    // the local average pool divides by the number of valid window elements: a window covering the whole plane is the global mean
+    PlanOp &op = plan.addOp(PlanOp::AVGPOOL, in, -1, out, layerIndex, "globalavgpool");
+    op.ksize = std::max(ti.h, ti.w); op.stride = 1; op.pad = 0;
+    return out;
+}
+
+SoftMaxLayer::SoftMaxLayer(const int &batch, const int &inputNum, const int &groups, const float &temperature)
+    : _groups(groups), _temperature(temperature)
+{
+    if (groups != 1) MSNH_THROW("softmax: groups are outside the convolutional path this build implements");
+    if (temperature == 0.f) MSNH_THROW("softmax: temperature must not be 0");
+    _type = LayerType::SOFTMAX;
+    _layerName = "SoftMax         ";
+    _batch = batch;
+    _inputNum = inputNum; _outputNum = inputNum;
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _layerDetail = fmt("softmax                                        %4d\n", inputNum);
+}
+
+int SoftMaxLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    in = plan.nhwcOf(in, layerIndex);
+    const PlanTensor ti = plan.tensors[static_cast<size_t>(in)];
+    _outHeight = ti.h; _outWidth = ti.w; _outChannel = ti.c;
+    const int out = plan.addTensor(ti.n, ti.h, ti.w, ti.c, ti.dtype, "softmax_out", ti.layout);
+    PlanOp &op = plan.addOp(PlanOp::SOFTMAX, in, -1, out, layerIndex, "softmax");
+    op.upScale = _temperature;
+    return out;
+}
+
+// ---- stand-alone activation / padding / slice / variable op --------------------------------------------------------------------
+ActivationLayer::ActivationLayer(const int &batch, const int &width, const int &height, const int &channel, const int &inputNum,
+                                 const ActivationType &activation, const std::vector<float> &actParams)
+{
+    if (activation == ActivationType::PRELU) MSNH_THROW("act: prelu is outside the convolutional path this build implements");
+    requireDeviceActivation(activation, "act");
+    _type = LayerType::ACTIVE;
+    _layerName = "Activate        ";
+    _batch = batch; _width = width; _height = height; _channel = channel;
+    _outWidth = width; _outHeight = height; _outChannel = channel;
+    _inputNum = inputNum; _outputNum = inputNum;
+    _activation = activation; _actParams = actParams;
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _layerDetail = "Activate Layer: " + Activations::getActivationStr(activation) + "\n";
+}
+
+void ActivationLayer::foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const
+{
+    scale.assign(static_cast<size_t>(_channel), 1.f);
+    shift.assign(static_cast<size_t>(_channel), 0.f);
+}
+
+int ActivationLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    if (_activation == ActivationType::NONE) return in;          // identity: the reference copies, the plan aliases
+    in = plan.nhwcOf(in, layerIndex);
+    const PlanTensor ti = plan.tensors[static_cast<size_t>(in)];
+    if (ti.layout != PlanTensor::NHWC) MSNH_THROW("act: the input must be an image tensor");
+    const int out = plan.addTensor(ti.n, ti.h, ti.w, ti.c, ti.dtype, "act_out");
+    PlanOp &op = plan.addOp(PlanOp::AFFINE, in, -1, out, layerIndex, "act");
+    op.act = _activation; op.actParam = actParam();
+    op.pureAct = true;
+    op.src = this;
+    return out;
+}
+
+PaddingLayer::PaddingLayer(const int &batch, const int &height, const int &width, const int &channel, const int &top, const int &down,
+                           const int &left, const int &right, const float &paddingVal)
+    : _top(top), _down(down), _left(left), _right(right), _paddingVal(paddingVal)
+{
+    if (top < 0 || down < 0 || left < 0 || right < 0) MSNH_THROW("padding: negative padding");
+    _type = LayerType::PADDING;
+    _layerName = "Padding         ";
+    _batch = batch; _height = height; _width = width; _channel = channel;
+    _inputNum = width * height * channel;
+    _outHeight = height + top + down; _outWidth = width + left + right; _outChannel = channel;
+    _outputNum = _outHeight * _outWidth * _outChannel;
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _layerDetail = fmt("Padding                      %4d x%4d x%4d -> %4d x%4d x%4d %5.3f BF\n", _width, _height, _channel, _outWidth, _outHeight,
+                       _outChannel, 0.0);
+}
+
+int PaddingLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    in = plan.nhwcOf(in, layerIndex);
+    const PlanTensor ti = plan.tensors[static_cast<size_t>(in)];
+    if (ti.layout != PlanTensor::NHWC) MSNH_THROW("padding: the input must be an image tensor");
+    const int out = plan.addTensor(ti.n, _outHeight, _outWidth, ti.c, ti.dtype, "padding_out");
+    PlanOp &op = plan.addOp(PlanOp::PAD, in, -1, out, layerIndex, "padding");
+    op.padTop = _top; op.padLeft = _left; op.padValue = _paddingVal;
+    return out;
+}
+
+SliceLayer::SliceLayer(const int &batch, const int &height, const int &width, const int &channel, const int &start0, const int &step0,
+                       const int &start1, const int &step1, const int &start2, const int &step2)
+    : _start0(start0), _step0(step0), _start1(start1), _step1(step1), _start2(start2), _step2(step2)
+{
+    if (step0 <= 0 || step1 <= 0 || step2 <= 0 || start0 < 0 || start1 < 0 || start2 < 0) MSNH_THROW("slice: start must be >= 0 and step > 0");
+    _type = LayerType::SLICE;
+    _layerName = "Slice           ";
+    _batch = batch; _height = height; _width = width; _channel = channel;
+    if (start0 > channel - 1) MSNH_THROW("slice c start error");
+    _outChannel = (channel - start0) / step0 + ((channel - start0) % step0 == 0 ? 0 : 1);
+    if (start1 > height - 1) MSNH_THROW("slice h start error");
+    _outHeight = (height - start1) / step1 + ((height - start1) % step1 == 0 ? 0 : 1);
+    if (start2 > width - 1) MSNH_THROW("slice w start error");
+    _outWidth = (width - start2) / step2 + ((width - start2) % step2 == 0 ? 0 : 1);
+    _inputNum = width * height * channel;
+    _outputNum = _outWidth * _outHeight * _outChannel;
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _layerDetail = fmt("Slice                        %4d x%4d x%4d -> %4d x%4d x%4d %5.3f BF\n", _width, _height, _channel, _outWidth, _outHeight,
+                       _outChannel, 0.0);
+}
+
+int SliceLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    in = plan.nhwcOf(in, layerIndex);
+    const PlanTensor ti = plan.tensors[static_cast<size_t>(in)];
+    if (ti.layout != PlanTensor::NHWC) MSNH_THROW("slice: the input must be an image tensor");
+    const int out = plan.addTensor(ti.n, _outHeight, _outWidth, _outChannel, ti.dtype, "slice_out");
+    PlanOp &op = plan.addOp(PlanOp::SLICE, in, -1, out, layerIndex, "slice");
+    op.slice[0] = _start0; op.slice[1] = _step0; op.slice[2] = _start1; op.slice[3] = _step1; op.slice[4] = _start2; op.slice[5] = _step2;
+    return out;
+}
+
+VariableOpLayer::VariableOpLayer(const int &batch, const int &width, const int &height, const int &channel, std::vector<int> &inputLayerIndexes,
+                                 const VariableOpParams::VarOpType &varOpType, const float &constVal)
+    : _inputLayerIndexes(inputLayerIndexes), _varOpType(varOpType), _constVal(constVal)
+{
+    const bool two = varOpType == VariableOpParams::VAR_OP_ADD || varOpType == VariableOpParams::VAR_OP_SUB || varOpType == VariableOpParams::VAR_OP_SUB_INV;
+    const bool con = varOpType == VariableOpParams::VAR_OP_ADD_CONST || varOpType == VariableOpParams::VAR_OP_SUB_CONST ||
+                     varOpType == VariableOpParams::VAR_OP_SUB_CONST_INV || varOpType == VariableOpParams::VAR_OP_MUL_CONST ||
+                     varOpType == VariableOpParams::VAR_OP_DIV_CONST;
+    if (!two && !con)
+        MSNH_THROW("varop: " + VariableOpParams::getStrFromVarOpType(varOpType) + " is outside the convolutional path this build implements");
+    if (two && (inputLayerIndexes.size() < 1 || inputLayerIndexes.size() > 2)) MSNH_THROW("varop: one or two input layers are needed");
+    if (con && !inputLayerIndexes.empty()) MSNH_THROW("varop: constant forms take the previous layer as their input");
+    if (varOpType == VariableOpParams::VAR_OP_DIV_CONST && constVal == 0.f) MSNH_THROW("varop: division by zero");
+    _type = LayerType::VARIABLE_OP;
+    _layerName = "VarOp           ";
+    _batch = batch; _width = width; _height = height; _channel = channel;
+    _outWidth = width; _outHeight = height; _outChannel = channel;
+    _inputNum = width * height * channel; _outputNum = _inputNum;
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _layerDetail = "VarOp Layer: " + VariableOpParams::getStrFromVarOpType(varOpType) + "\n";
+}
+
+void VariableOpLayer::foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const
+{
+    float a = 1.f, b = 0.f;
+    switch (_varOpType)
+    {
+    case VariableOpParams::VAR_OP_ADD_CONST:     b = _constVal; break;
+    case VariableOpParams::VAR_OP_SUB_CONST:     b = -_constVal; break;
+    case VariableOpParams::VAR_OP_SUB_CONST_INV: a = -1.f; b = _constVal; break;
+    case VariableOpParams::VAR_OP_MUL_CONST:     a = _constVal; break;
+    case VariableOpParams::VAR_OP_DIV_CONST:     a = 1.f / _constVal; break;
+    default: break;
+    }
+    scale.assign(static_cast<size_t>(_channel), a);
+    shift.assign(static_cast<size_t>(_channel), b);
+}
+
+int VariableOpLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    if (_inputLayerIndexes.empty())
+    {
+        in = plan.nhwcOf(in, layerIndex);
+        const PlanTensor ti = plan.tensors[static_cast<size_t>(in)];
+        if (ti.layout != PlanTensor::NHWC) MSNH_THROW("varop: the input must be an image tensor");
+        const int out = plan.addTensor(ti.n, ti.h, ti.w, ti.c, ti.dtype, "varop_out");
+        PlanOp &op = plan.addOp(PlanOp::AFFINE, in, -1, out, layerIndex, "varop_const");
+        op.src = this;
+        return out;
+    }
+    // one listed layer: A = previous layer, B = it; two: A, B = the listed layers (src/layers/MsnhVariableOpLayer.cpp:78-158)
+    int a = in, b = plan.layerOut[static_cast<size_t>(_inputLayerIndexes[0])];
+    if (_inputLayerIndexes.size() == 2) { a = b; b = plan.layerOut[static_cast<size_t>(_inputLayerIndexes[1])]; }
+    a = plan.nhwcOf(a, layerIndex); b = plan.nhwcOf(b, layerIndex);
+    const PlanTensor ta = plan.tensors[static_cast<size_t>(a)], tb = plan.tensors[static_cast<size_t>(b)];
+    if (ta.layout != PlanTensor::NHWC || tb.layout != PlanTensor::NHWC || ta.h != tb.h || ta.w != tb.w || ta.c != tb.c)
+        MSNH_THROW("varop: the two inputs must be image tensors of the same shape");
+    if (_varOpType == VariableOpParams::VAR_OP_SUB_INV) std::swap(a, b);
+    const int out = plan.addTensor(ta.n, ta.h, ta.w, ta.c, ta.dtype, "varop_out");
+    PlanOp &op = plan.addOp(PlanOp::ADD, a, b, out, layerIndex, "varop");
+    op.in1Sign = _varOpType == VariableOpParams::VAR_OP_ADD ? 1.f : -1.f;
     return out;
 }
 
@@ -452,8 +677,9 @@ RouteLayer::RouteLayer(const int &batch, std::vector<int> &inputLayerIndexes, st
                        const int &groupIndex, const int &addModel, const ActivationType &activation, const std::vector<float> &actParams)
     : _inputLayerIndexes(inputLayerIndexes), _inputLayerOutputs(inputLayerOutputs), _groups(groups), _groupIndex(groupIndex), _addModel(addModel)
 {
-    if (addModel == 1 || groups != 1) MSNH_THROW("route: addModel / groups are outside the convolutional path this build implements");
-    if (activation != ActivationType::NONE) MSNH_THROW("route: activation is outside the convolutional path this build implements");
+    if (groups != 1) MSNH_THROW("route: groups are outside the convolutional path this build implements");
+    if (addModel == 1 && inputLayerIndexes.size() < 2) MSNH_THROW("route layer error, add model must have at least 2 layers ");
+    requireDeviceActivation(activation, "route");
     _type = LayerType::ROUTE;
     _layerName = "Route           ";
     _batch = batch;
@@ -466,6 +692,7 @@ RouteLayer::RouteLayer(const int &batch, std::vector<int> &inputLayerIndexes, st
         outputNum += inputLayerOutputs[i];
     }
     _layerDetail += "\n";
+    if (addModel == 1) outputNum = inputLayerOutputs[0];
     _outputNum = outputNum;
     _inputNum = outputNum;
     _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
@@ -474,20 +701,55 @@ RouteLayer::RouteLayer(const int &batch, std::vector<int> &inputLayerIndexes, st
 int RouteLayer::lower(Plan &plan, int, int layerIndex)
 {
     std::vector<int> srcs;
-    for (int idx : _inputLayerIndexes) srcs.push_back(plan.layerOut[static_cast<size_t>(idx)]);
-    if (srcs.size() == 1) return srcs[0];                        // a single routed layer is an alias, not a copy
+    for (int idx : _inputLayerIndexes) srcs.push_back(plan.nhwcOf(plan.layerOut[static_cast<size_t>(idx)], layerIndex));
     const PlanTensor first = plan.tensors[static_cast<size_t>(srcs[0])];
-    int channels = 0;
-    for (int s : srcs) channels += plan.tensors[static_cast<size_t>(s)].c;
-    const int out = plan.addTensor(first.n, first.h, first.w, channels, first.dtype, "route_out");
-    int off = 0;
-    for (int s : srcs)
+    int result;
+    if (_addModel == 1)
     {
-        PlanOp &op = plan.addOp(PlanOp::COPY, s, -1, out, layerIndex, "route_copy");
-        op.dstChanOffset = off;
-        off += plan.tensors[static_cast<size_t>(s)].c;
+        // zero-filled output, then += every listed layer in list order (src/layers/MsnhRouteLayer.cpp:77-115); the last add takes the activation
+        int acc = srcs[0];
+        for (size_t i = 1; i < srcs.size(); ++i)
+        {
+            const PlanTensor t = plan.tensors[static_cast<size_t>(srcs[i])];
+            if (t.h != first.h || t.w != first.w || t.c != first.c) MSNH_THROW("[route] layers height or width not equal.");
+            const int out = plan.addTensor(first.n, first.h, first.w, first.c, first.dtype, "route_sum");
+            PlanOp &op = plan.addOp(PlanOp::ADD, acc, srcs[i], out, layerIndex, "route_add");
+            if (i + 1 == srcs.size()) { op.act = _activation; op.actParam = actParam(); }
+            acc = out;
+        }
+        return acc;
     }
-    return out;
+    if (srcs.size() == 1) result = srcs[0];                      // a single routed layer is an alias, not a copy
+    else
+    {
+        int channels = 0;
+        for (int s : srcs) channels += plan.tensors[static_cast<size_t>(s)].c;
+        result = plan.addTensor(first.n, first.h, first.w, channels, first.dtype, "route_out");
+        int off = 0;
+        for (int s : srcs)
+        {
+            PlanOp &op = plan.addOp(PlanOp::COPY, s, -1, result, layerIndex, "route_copy");
+            op.dstChanOffset = off;
+            off += plan.tensors[static_cast<size_t>(s)].c;
+        }
+    }
+    if (_activation != ActivationType::NONE)
+    {
+        const PlanTensor tr = plan.tensors[static_cast<size_t>(result)];
+        const int out = plan.addTensor(tr.n, tr.h, tr.w, tr.c, tr.dtype, "route_act");
+        PlanOp &op = plan.addOp(PlanOp::AFFINE, result, -1, out, layerIndex, "route_act");
+        op.act = _activation; op.actParam = actParam();
+        op.pureAct = true;
+        op.src = this;
+        result = out;
+    }
+    return result;
+}
+
+void RouteLayer::foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const
+{
+    scale.assign(static_cast<size_t>(_outChannel), 1.f);
+    shift.assign(static_cast<size_t>(_outChannel), 0.f);
 }
 
 // ---- blocks -----------------------------------------------------------------------------------------------------------------------
@@ -758,8 +1020,8 @@ YoloLayer::YoloLayer(const int &batch, const int &width, const int &height, cons
     _ratios = 1.f * orgHeight / _outHeight;          // height only, used for both axes (src/layers/MsnhYoloLayer.cpp:34)
     if (3 * (classNum + 4 + 1) != num) MSNH_THROW("class num error!");
     if (this->anchors.size() != 6) MSNH_THROW("[yolo] anchor num should be 6");
-    if (static_cast<int>(yoloType) / 10 != 3 && static_cast<int>(yoloType) / 10 != 4) MSNH_THROW("yolo: only yolov3 / yolov4 decoding is implemented");
-    if (yoloType != YoloType::YoloV3 && yoloType != YoloType::YoloV4) MSNH_THROW("yolo: angle / gaussian variants are outside the convolutional path this build implements");
+    if (yoloType != YoloType::YoloV3 && yoloType != YoloType::YoloV4 && yoloType != YoloType::YoloV5)
+        MSNH_THROW("yolo: angle / gaussian variants are outside the convolutional path this build implements");
     _memReUse = 0;
     _layerDetail = "Yolo. class num : " + std::to_string(classNum) + "\n";
 }
@@ -777,6 +1039,7 @@ int YoloLayer::lower(Plan &plan, int in, int layerIndex)
     for (int i = 0; i < 6; ++i) op.anchors[static_cast<size_t>(i)] = anchors[static_cast<size_t>(i)];
     op.classes = _classNum;
     op.ratio = _ratios;
+    op.yoloVersion = static_cast<int>(_yoloType) / 10;
     op.confThresh = 2.f;
     decodeOp = plan.ops.size() - 1;
     return out;
@@ -789,7 +1052,7 @@ YoloOutLayer::YoloOutLayer(const int &batch, const int &orgWidth, const int &org
     : _confThresh(confThresh), _nmsThresh(nmsThresh), _useSoftNms(useSotfNms), _orgHeight(orgHeight), _orgWidth(orgWidth), _yoloType(yoloType),
       _yoloIndexes(yoloIndexes), _yoloLayersInfo(yoloLayersInfo)
 {
-    if (yoloType != YoloType::YoloV3 && yoloType != YoloType::YoloV4) MSNH_THROW("yoloout: only yolov3 / yolov4 are implemented");
+    if (yoloType != YoloType::YoloV3 && yoloType != YoloType::YoloV4 && yoloType != YoloType::YoloV5) MSNH_THROW("yoloout: only yolov3 / yolov4 / yolov5 are implemented");
     _type = LayerType::YOLO_OUT;
     _layerName = "YoloOut         ";
     _batch = batch;

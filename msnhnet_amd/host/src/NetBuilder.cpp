@@ -174,8 +174,12 @@ void NetBuilder::buildNetFromMsnhNet(const std::string &path)
                                std::to_string(outW) + ":" + std::to_string(src->getOutWidth()) + " , " + std::to_string(outH) + ":" +
                                std::to_string(src->getOutHeight()) + " ");
                 }
+                if (p->addModel == 1 && k > 0 && src->getOutChannel() != outC)
+                    MSNH_THROW("[route] layers height or width not equal. layer: " + std::to_string(i - 1) + " whc: channels " + std::to_string(outC) + ":" +
+                               std::to_string(src->getOutChannel()));
                 outH = src->getOutHeight(); outW = src->getOutWidth();
-                outC += src->getOutChannel();
+                if (p->addModel == 1) outC = src->getOutChannel();
+                else outC += src->getOutChannel();
                 outputs.push_back(src->getOutputNum());
                 chans.push_back(src->getOutChannel());
             }
@@ -183,6 +187,41 @@ void NetBuilder::buildNetFromMsnhNet(const std::string &path)
             r->inputChannels = chans;
             r->setOutChannel(outC); r->setOutWidth(outW); r->setOutHeight(outH);
             layer = r;
+            break;
+        }
+        case LayerType::GLOBAL_AVGPOOL:
+            layer = new GlobalAvgPoolLayer(params.batch, params.height, params.width, params.channels);
+            break;
+        case LayerType::SOFTMAX:
+        {
+            SoftMaxParams *p = static_cast<SoftMaxParams *>(bp);
+            layer = new SoftMaxLayer(params.batch, params.inputNums, p->groups, p->temperature);
+            break;
+        }
+        case LayerType::ACTIVE:
+        {
+            ActivationParams *p = static_cast<ActivationParams *>(bp);
+            layer = new ActivationLayer(params.batch, params.width, params.height, params.channels, params.inputNums, p->activation, p->actParams);
+            break;
+        }
+        case LayerType::PADDING:
+        {
+            PaddingParams *p = static_cast<PaddingParams *>(bp);
+            layer = new PaddingLayer(params.batch, params.height, params.width, params.channels, p->top, p->down, p->left, p->right, p->paddingVal);
+            break;
+        }
+        case LayerType::SLICE:
+        {
+            SliceParams *p = static_cast<SliceParams *>(bp);
+            layer = new SliceLayer(params.batch, params.height, params.width, params.channels, p->start0, p->step0, p->start1, p->step1, p->start2, p->step2);
+            break;
+        }
+        case LayerType::VARIABLE_OP:
+        {
+            VariableOpParams *p = static_cast<VariableOpParams *>(bp);
+            for (int idx : p->layerIndexes)
+                if (idx < 0 || static_cast<size_t>(idx) >= nLayers) MSNH_THROW("varop layer error, layers index should < size of layers");
+            layer = new VariableOpLayer(params.batch, params.width, params.height, params.channels, p->layerIndexes, p->varOpType, p->constVal);
             break;
         }
         case LayerType::UPSAMPLE:
@@ -689,7 +728,7 @@ std::string NetBuilder::profileEachOp(int reps)
 {
     if (!_planReady) MSNH_THROW("weights are not loaded");
     Plan &plan = *_net->plan;
-    static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode"};
+    static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode", "pad", "slice", "bilinear", "softmax"};
     static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk"};
     msnh_event_t e0 = nullptr, e1 = nullptr;
     MSNH_DEV(msnh_hip_event_create(&e0));

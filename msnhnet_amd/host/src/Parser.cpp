@@ -112,7 +112,7 @@ std::string Activations::getActivationStr(const ActivationType &type)
 
 bool Activations::deviceSupported(const ActivationType &t)
 {
-    return t == NONE || t == RELU || t == RELU6 || t == LEAKY || t == MISH || t == SWISH || t == LOGISTIC;
+    return t == NONE || t == RELU || t == RELU6 || t == LEAKY || t == MISH || t == SWISH || t == HARD_SWISH || t == LOGISTIC;
 }
 
 // ---- params ownership -------------------------------------------------------------------------------------
@@ -261,10 +261,37 @@ void Parser::parseSubNodes(const std::vector<MsnhNode> &nodes, const char *owner
     }
 }
 
+static const std::pair<const char *, VariableOpParams::VarOpType> kVarOps[] = {
+    {"add", VariableOpParams::VAR_OP_ADD}, {"sub", VariableOpParams::VAR_OP_SUB}, {"subInv", VariableOpParams::VAR_OP_SUB_INV},
+    {"mul", VariableOpParams::VAR_OP_MUL}, {"div", VariableOpParams::VAR_OP_DIV}, {"divInv", VariableOpParams::VAR_OP_DIV_INV},
+    {"addConst", VariableOpParams::VAR_OP_ADD_CONST}, {"subConst", VariableOpParams::VAR_OP_SUB_CONST},
+    {"subConstInv", VariableOpParams::VAR_OP_SUB_CONST_INV}, {"mulConst", VariableOpParams::VAR_OP_MUL_CONST},
+    {"divConst", VariableOpParams::VAR_OP_DIV_CONST}, {"divConstInv", VariableOpParams::VAR_OP_DIV_CONST_INV},
+    {"abs", VariableOpParams::VAR_OP_ABS}, {"acos", VariableOpParams::VAR_OP_ACOS}, {"asin", VariableOpParams::VAR_OP_ASIN},
+    {"atan", VariableOpParams::VAR_OP_ATAN}, {"cos", VariableOpParams::VAR_OP_COS}, {"cosh", VariableOpParams::VAR_OP_COSH},
+    {"sin", VariableOpParams::VAR_OP_SIN}, {"sinh", VariableOpParams::VAR_OP_SINH}, {"tan", VariableOpParams::VAR_OP_TAN},
+    {"tanh", VariableOpParams::VAR_OP_TANH}, {"exp", VariableOpParams::VAR_OP_EXP}, {"pow", VariableOpParams::VAR_OP_POW},
+    {"log", VariableOpParams::VAR_OP_LOG}, {"log10", VariableOpParams::VAR_OP_LOG10}, {"sqrt", VariableOpParams::VAR_OP_SQRT}};
+
+// src/io/MsnhParser.cpp:2278-2392
+VariableOpParams::VarOpType VariableOpParams::getVarOpTypeFromStr(const std::string &s)
+{
+    for (const auto &e : kVarOps)
+        if (s == e.first) return e.second;
+    MSNH_THROW("[varop] var op no supported : " + s);
+}
+
+std::string VariableOpParams::getStrFromVarOpType(const VarOpType &t)
+{
+    for (const auto &e : kVarOps)
+        if (t == e.second) return e.first;
+    return "unknown";
+}
+
 BaseParams *Parser::parseNode(const MsnhNode &node, bool top, const NetConfigParams &cfg)
 {
     const std::string &k = node.key;
-    if (k != "empty" && !node.isBlock) MSNH_THROW("[" + k + "] content error");
+    if (k != "empty" && k != "globalavgpool" && !node.isBlock) MSNH_THROW("[" + k + "] content error");
 
     if (k == "conv")
     {
@@ -388,6 +415,69 @@ BaseParams *Parser::parseNode(const MsnhNode &node, bool top, const NetConfigPar
             else if (n.key == "addModel") toInt(n, "route", p->addModel);
             else if (n.key == "activation") toActivation(n, p->activation, p->actParams);
             else unsupportedKey(n, "route");
+        }
+        return p.release();
+    }
+    if (k == "globalavgpool") return new GlobalAvgPoolParams(top);
+    if (k == "softmax")
+    {
+        std::unique_ptr<SoftMaxParams> p(new SoftMaxParams(top));
+        for (const MsnhNode &n : node.children)
+        {
+            if (n.key == "groups") toInt(n, "softmax", p->groups);
+            else if (n.key == "temperature") toFloat(n, "softmax", p->temperature);
+            else unsupportedKey(n, "softmax");
+        }
+        return p.release();
+    }
+    if (k == "act")
+    {
+        std::unique_ptr<ActivationParams> p(new ActivationParams(top));
+        for (const MsnhNode &n : node.children)
+        {
+            if (n.key == "activation") toActivation(n, p->activation, p->actParams);
+            else unsupportedKey(n, "act");
+        }
+        return p.release();
+    }
+    if (k == "padding")
+    {
+        std::unique_ptr<PaddingParams> p(new PaddingParams(top));
+        for (const MsnhNode &n : node.children)
+        {
+            if (n.key == "top") toInt(n, "padding", p->top);
+            else if (n.key == "down") toInt(n, "padding", p->down);
+            else if (n.key == "left") toInt(n, "padding", p->left);
+            else if (n.key == "right") toInt(n, "padding", p->right);
+            else if (n.key == "paddingVal") toFloat(n, "padding", p->paddingVal);
+            else unsupportedKey(n, "padding");
+        }
+        return p.release();
+    }
+    if (k == "slice")
+    {
+        std::unique_ptr<SliceParams> p(new SliceParams(top));
+        for (const MsnhNode &n : node.children)
+        {
+            if (n.key == "start0") toInt(n, "slice", p->start0);
+            else if (n.key == "step0") toInt(n, "slice", p->step0);
+            else if (n.key == "start1") toInt(n, "slice", p->start1);
+            else if (n.key == "step1") toInt(n, "slice", p->step1);
+            else if (n.key == "start2") toInt(n, "slice", p->start2);
+            else if (n.key == "step2") toInt(n, "slice", p->step2);
+            else unsupportedKey(n, "slice");
+        }
+        return p.release();
+    }
+    if (k == "varop")
+    {
+        std::unique_ptr<VariableOpParams> p(new VariableOpParams(top));
+        for (const MsnhNode &n : node.children)
+        {
+            if (n.key == "layers") p->layerIndexes = layerList(n, "varop", BaseParams::index);
+            else if (n.key == "type") p->varOpType = VariableOpParams::getVarOpTypeFromStr(n.value);
+            else if (n.key == "constVal") toFloat(n, "varop", p->constVal);
+            else unsupportedKey(n, "varop");
         }
         return p.release();
     }

@@ -47,6 +47,18 @@ PlanOp &Plan::addOp(PlanOp::Kind kind, int in0, int in1, int out, int layerIndex
     return op;
 }
 
+int Plan::nhwcOf(int tensor, int layerIndex)
+{
+    const PlanTensor t = tensors[static_cast<size_t>(tensor)];
+    if (t.layout != PlanTensor::NCHW_INPUT) return tensor;
+    if (inputNhwc < 0)
+    {
+        inputNhwc = addTensor(t.n, t.h, t.w, t.c, computeDtype, "input_nhwc");
+        addOp(PlanOp::INPUT_CAST, tensor, -1, inputNhwc, layerIndex, "input_cast");
+    }
+    return inputNhwc;
+}
+
 int Plan::producerOf(int tensor) const
 {
     for (int i = static_cast<int>(ops.size()) - 1; i >= 0; --i)
@@ -115,6 +127,26 @@ void Plan::fuse()
         if (aff.dead || aff.kind != PlanOp::AFFINE) continue;
         const int p = producerOf(aff.in0);
         if (p < 0) continue;
+        if (aff.pureAct)
+        {
+            // a stand-alone activation moves into whatever produced its input, if that has no activation of its own yet
+            PlanOp &prod = ops[static_cast<size_t>(p)];
+            if (tensors[static_cast<size_t>(aff.in0)].pinned || consumerCount(aff.in0) != 1) continue;
+            if (prod.kind == PlanOp::CONV && prod.in1 >= 0)
+            {
+                if (prod.act2 != NONE) continue;
+                prod.act2 = aff.act; prod.act2Param = aff.actParam;
+            }
+            else if (prod.kind == PlanOp::CONV || prod.kind == PlanOp::AFFINE || prod.kind == PlanOp::ADD)
+            {
+                if (prod.act != NONE) continue;
+                prod.act = aff.act; prod.actParam = aff.actParam;
+            }
+            else continue;
+            prod.out = aff.out;
+            aff.dead = true;
+            continue;
+        }
         PlanOp &conv = ops[static_cast<size_t>(p)];
         if (conv.kind != PlanOp::CONV || conv.act != NONE || conv.src2 != nullptr || conv.in1 >= 0) continue;
         if (tensors[static_cast<size_t>(aff.in0)].pinned || consumerCount(aff.in0) != 1) continue;
@@ -536,7 +568,7 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
                                      op.shiftDev.as<float>(), static_cast<int>(op.act), op.actParam, 1.f / mulOf(op.out), ptr(op.out), ld(op.out), s));
         break;
     case PlanOp::ADD:
-        MSNH_DEV(msnh_hip_add_act(in.dtype, in.pixels(), in.c, ptr(op.in0), ld(op.in0), mulOf(op.in0), ptr(op.in1), ld(op.in1), mulOf(op.in1),
+        MSNH_DEV(msnh_hip_add_act(in.dtype, in.pixels(), in.c, ptr(op.in0), ld(op.in0), mulOf(op.in0), ptr(op.in1), ld(op.in1), op.in1Sign * mulOf(op.in1),
                                   static_cast<int>(op.act), op.actParam, 1.f / mulOf(op.out), ptr(op.out), ld(op.out), s));
         break;
     case PlanOp::COPY:
@@ -557,6 +589,22 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
     case PlanOp::UPSAMPLE:
         MSNH_DEV(msnh_hip_upsample_nearest(in.dtype, in.n, in.h, in.w, in.c, ptr(op.in0), ld(op.in0), op.stride, op.upScale, ptr(op.out),
                                            ld(op.out), s));
+        break;
+    case PlanOp::PAD:
+        MSNH_DEV(msnh_hip_pad(in.dtype, in.n, in.h, in.w, in.c, ptr(op.in0), ld(op.in0), op.padTop, op.padLeft, out.h, out.w, mulOf(op.in0) / mulOf(op.out),
+                              op.padValue / mulOf(op.out), ptr(op.out), ld(op.out), s));
+        break;
+    case PlanOp::SLICE:
+        MSNH_DEV(msnh_hip_slice(in.dtype, in.n, in.h, in.w, ptr(op.in0), ld(op.in0), op.slice[0], op.slice[1], op.slice[2], op.slice[3], op.slice[4],
+                                op.slice[5], out.c, out.h, out.w, mulOf(op.in0) / mulOf(op.out), ptr(op.out), ld(op.out), s));
+        break;
+    case PlanOp::SOFTMAX:
+        MSNH_DEV(msnh_hip_softmax(in.dtype, in.n, in.h * in.w, in.c, ptr(op.in0), in.layout == PlanTensor::FLAT ? in.c : ld(op.in0), mulOf(op.in0),
+                                  op.upScale, ptr(op.out), out.layout == PlanTensor::FLAT ? out.c : ld(op.out), 1.f / mulOf(op.out), s));
+        break;
+    case PlanOp::BILINEAR:
+        MSNH_DEV(msnh_hip_upsample_bilinear(in.dtype, in.n, in.h, in.w, in.c, ptr(op.in0), ld(op.in0), out.h, out.w, op.alignCorners,
+                                            mulOf(op.in0) / mulOf(op.out), ptr(op.out), ld(op.out), s));
         break;
     case PlanOp::CONNECTED:
         if (op.algo == MSNH_CONV_IGEMM || op.algo == MSNH_CONV_IGEMM_SPLITK)
@@ -580,7 +628,7 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
         float *decoded = yoloDecoded.as<float>() + static_cast<size_t>(op.cellBase) * per;
         const bool cand = op.confThresh < 1.5f;
         MSNH_DEV(msnh_hip_yolo_decode(in.dtype, in.n, in.h, in.w, op.classes, ptr(op.in0), ld(op.in0), mulOf(op.in0), op.anchors.data(), op.ratio,
-                                      decoded, static_cast<long long>(yoloCells) * per, op.confThresh, cand ? yoloCandIdx.as<int>() : nullptr,
+                                      op.yoloVersion, decoded, static_cast<long long>(yoloCells) * per, op.confThresh, cand ? yoloCandIdx.as<int>() : nullptr,
                                       yoloCells, op.cellBase, cand ? yoloCandCnt.as<int>() : nullptr, s));
         break;
     }
@@ -612,7 +660,7 @@ void Plan::exportTensor(int t, std::vector<float> &dst, msnh_stream_t s)
 
 std::string Plan::describe() const
 {
-    static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode"};
+    static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode", "pad", "slice", "bilinear", "softmax"};
     static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk"};
     std::ostringstream os;
     os << "plan: " << liveOps() << " launches, " << tensors.size() << " tensors, arena " << _arena.bytes() / (1024.0 * 1024.0) << " MiB, dtype "

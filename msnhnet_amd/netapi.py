@@ -21,8 +21,9 @@ SYMBOLS = [
     "msnhnet_profile_ops", "msnhnet_profile_each_op", "msnhnet_yolo_max_boxes", "msnhnet_nms",
 ]
 
-LAYER_TYPE = {0: "conv", 2: "connect", 3: "maxpool", 4: "localavgpool", 8: "route", 13: "batchnorm", 15: "yolo", 16: "yoloout",
-              18: "upsample", 20: "empty", 27: "resblock", 28: "res2block", 29: "concatblock", 30: "addblock"}
+LAYER_TYPE = {0: "conv", 1: "deconv", 2: "connect", 3: "maxpool", 4: "localavgpool", 5: "globalavgpool", 6: "softmax", 8: "route", 9: "varop",
+              12: "act", 13: "batchnorm", 15: "yolo", 16: "yoloout", 18: "upsample", 20: "empty", 24: "slice", 27: "resblock", 28: "res2block",
+              29: "concatblock", 30: "addblock", 31: "padding"}
 
 
 class MsnhnetError(RuntimeError):

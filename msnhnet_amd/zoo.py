@@ -169,13 +169,69 @@ class GraphWriter:
         self.shape = _Shape(s.c, s.h * stride, s.w * stride)
         self._top_done()
 
-    def route(self, layers: List[int]):
+    def route(self, layers: List[int], add_model: bool = False, act: Optional[str] = None):
         """`layers` as written in the file: negative = relative to this route layer."""
         self._emit("route:")
         self._emit("  layers: " + ",".join(str(v) for v in layers))
+        if add_model:
+            self._emit("  addModel: 1")
+        if act:
+            self._emit(f"  activation: {act}")
         idx = [v if v >= 0 else self.n_top + v for v in layers]
         shp = [self.top_shapes[i] for i in idx]
-        self.shape = _Shape(sum(s.c for s in shp), shp[0].h, shp[0].w)
+        self.shape = _Shape(shp[0].c if add_model else sum(s.c for s in shp), shp[0].h, shp[0].w)
+        self._top_done()
+
+    def act(self, act: str):
+        self._emit("act:")
+        self._emit(f"  activation: {act}")
+        self._top_done()
+
+    def padding(self, top, down, left, right, value=0.0):
+        self._emit("padding:")
+        for k, v in (("top", top), ("down", down), ("left", left), ("right", right)):
+            self._emit(f"  {k}: {v}")
+        self._emit(f"  paddingVal: {value}")
+        s = self.shape
+        self.shape = _Shape(s.c, s.h + top + down, s.w + left + right)
+        self._top_done()
+
+    def slice(self, start0, step0, start1, step1, start2, step2):
+        self._emit("slice:")
+        for k, v in (("start0", start0), ("step0", step0), ("start1", start1), ("step1", step1), ("start2", start2), ("step2", step2)):
+            self._emit(f"  {k}: {v}")
+        s = self.shape
+        ext = lambda n, st, sp: (n - st) // sp + (1 if (n - st) % sp else 0)
+        self.shape = _Shape(ext(s.c, start0, step0), ext(s.h, start1, step1), ext(s.w, start2, step2))
+        self._top_done()
+
+    def varop(self, kind: str, layers: Optional[List[int]] = None, const: float = 0.0):
+        self._emit("varop:")
+        if layers:
+            self._emit("  layers: " + ",".join(str(v) for v in layers))
+        self._emit(f"  type: {kind}")
+        self._emit(f"  constVal: {const}")
+        self._top_done()
+
+    def softmax(self, temperature: float = 1.0):
+        self._emit("softmax:")
+        self._emit("  groups: 1")
+        self._emit(f"  temperature: {temperature}")
+        self._top_done()
+
+    def globalavgpool(self):
+        self._emit("globalavgpool:")
+        self.shape = _Shape(self.shape.c, 1, 1)
+        self._top_done()
+
+    def upsample_bilinear(self, scale_x: float, scale_y: float, align_corners: int = 0):
+        self._emit("upsample:")
+        self._emit("  type: bilinear")
+        self._emit(f"  scaleX: {scale_x}")
+        self._emit(f"  scaleY: {scale_y}")
+        self._emit(f"  alignCorners: {align_corners}")
+        s = self.shape
+        self.shape = _Shape(s.c, int(np.float32(s.h) * np.float32(scale_y)), int(np.float32(s.w) * np.float32(scale_x)))
         self._top_done()
 
     def yolo(self, anchors: List[int], class_num=80, yolo_type: Optional[str] = None):

@@ -78,6 +78,12 @@ float msnh_or_activate(float x, int act, float param)
     case MSNH_OR_ACT_RELU6:    return (x > 0 ? x : 0) > 6 ? 6 : (x > 0 ? x : 0);
     case MSNH_OR_ACT_LEAKY:    return (x > 0) ? x : param * x;
     case MSNH_OR_ACT_SWISH:    return x * (1.f / (1.f + expf(-x)));
+    case MSNH_OR_ACT_HARD_SWISH:
+    {
+        const float t = x + 3.f;                 /* x*relu6Activate(x+3.f)/6.f (MsnhActivations.h:59-62) */
+        const float r = (t > 0 ? t : 0) > 6 ? 6 : (t > 0 ? t : 0);
+        return x * r / 6.f;
+    }
     case MSNH_OR_ACT_MISH:     return x * tanhf(softplus_thr(x, 20.f));
     default:                   return x;
     }
@@ -246,10 +252,12 @@ void msnh_or_axpy(long long n, float alpha, const float *x, float *y)
         y[i] += alpha * x[i];
 }
 
-/* YoloLayer::forward for yolov3/yolov4 (src/layers/MsnhYoloLayer.cpp:61-142, helpers :217-284), in place:
- * per anchor n: plane0 (sigmoid+col)*ratio, plane1 (sigmoid+row)*ratio, plane2 aw*exp, plane3 ah*exp,
- * planes 4.. sigmoid. */
-void msnh_or_yolo_decode(float *data, int batch, int width, int height, int classNum, const float *anchors6, float ratio)
+/* YoloLayer::forward (src/layers/MsnhYoloLayer.cpp:61-142, helpers :217-296), in place.  Per anchor n:
+ *   yolov3 / yolov4 (version 3, 4): plane0 (sigmoid+col)*ratio, plane1 (sigmoid+row)*ratio, plane2 aw*exp, plane3 ah*exp;
+ *   yolov5 (version 5): plane0 (2*sigmoid-0.5+col)*ratio, plane1 likewise with row, planes 2,3 a*powf(2*sigmoid, 2);
+ *   planes 4.. sigmoid in both. */
+void msnh_or_yolo_decode(float *data, int batch, int width, int height, int classNum, const float *anchors6, float ratio,
+                         int version)
 {
     const int hw = width * height;
     const int per = 5 + classNum;
@@ -257,20 +265,142 @@ void msnh_or_yolo_decode(float *data, int batch, int width, int height, int clas
         for (int n = 0; n < 3; ++n)
         {
             float *p = data + ((size_t)b * 3 + n) * per * hw;
-            for (int i = 0; i < hw; ++i)
-                p[i] = (1.f / (1.f + expf(-p[i])) + i % width) * ratio;
-            p += hw;
-            for (int i = 0; i < hw; ++i)
-                p[i] = (1.f / (1.f + expf(-p[i])) + i / width) * ratio;
-            p += hw;
-            for (int i = 0; i < hw; ++i)
-                p[i] = anchors6[n % 3 * 2] * expf(p[i]);
-            p += hw;
-            for (int i = 0; i < hw; ++i)
-                p[i] = anchors6[n % 3 * 2 + 1] * expf(p[i]);
-            p += hw;
+            if (version == 5)
+            {
+                for (int i = 0; i < hw; ++i)
+                    p[i] = (2.f / (1.f + expf(-p[i])) - 0.5f + i % width) * ratio;
+                p += hw;
+                for (int i = 0; i < hw; ++i)
+                    p[i] = (2.f / (1.f + expf(-p[i])) - 0.5f + i / width) * ratio;
+                p += hw;
+                for (int i = 0; i < hw; ++i)
+                    p[i] = anchors6[n % 3 * 2] * powf(2.f / (1.f + expf(-p[i])), 2.f);
+                p += hw;
+                for (int i = 0; i < hw; ++i)
+                    p[i] = anchors6[n % 3 * 2 + 1] * powf(2.f / (1.f + expf(-p[i])), 2.f);
+                p += hw;
+            }
+            else
+            {
+                for (int i = 0; i < hw; ++i)
+                    p[i] = (1.f / (1.f + expf(-p[i])) + i % width) * ratio;
+                p += hw;
+                for (int i = 0; i < hw; ++i)
+                    p[i] = (1.f / (1.f + expf(-p[i])) + i / width) * ratio;
+                p += hw;
+                for (int i = 0; i < hw; ++i)
+                    p[i] = anchors6[n % 3 * 2] * expf(p[i]);
+                p += hw;
+                for (int i = 0; i < hw; ++i)
+                    p[i] = anchors6[n % 3 * 2 + 1] * expf(p[i]);
+                p += hw;
+            }
             for (long long i = 0; i < (long long)hw * (1 + classNum); ++i)
                 p[i] = 1.f / (1.f + expf(-p[i]));
+        }
+}
+
+/* PaddingLayer::forward (src/layers/MsnhPaddingLayer.cpp:143-177): constant border around every channel plane. */
+void msnh_or_pad(const float *in, int batch, int channels, int height, int width, int top, int down, int left, int right,
+                 float value, float *out)
+{
+    const int oh = height + top + down, ow = width + left + right;
+    for (int i = 0; i < batch; ++i)
+        for (int j = 0; j < channels; ++j)
+            for (int m = 0; m < oh; ++m)
+                for (int n = 0; n < ow; ++n)
+                {
+                    float val;
+                    if (m < top || m >= height + top) val = value;
+                    else if (n < left || n >= width + left) val = value;
+                    else val = in[(((size_t)i * channels + j) * height + (m - top)) * width + (n - left)];
+                    out[(((size_t)i * channels + j) * oh + m) * ow + n] = val;
+                }
+}
+
+/* SliceLayer::forward (src/layers/MsnhSliceLayer.cpp:120-147): out[c][h][w] = in[c*step0+start0][h*step1+start1][w*step2+start2],
+ * output extents ceil((extent - start) / step) (ctor, :28-48). */
+void msnh_or_slice(const float *in, int batch, int channels, int height, int width, int start0, int step0, int start1, int step1,
+                   int start2, int step2, float *out)
+{
+    const int oc = (channels - start0) / step0 + ((channels - start0) % step0 ? 1 : 0);
+    const int oh = (height - start1) / step1 + ((height - start1) % step1 ? 1 : 0);
+    const int ow = (width - start2) / step2 + ((width - start2) % step2 ? 1 : 0);
+    for (int b = 0; b < batch; ++b)
+        for (int c = 0; c < oc; ++c)
+            for (int h = 0; h < oh; ++h)
+                for (int w = 0; w < ow; ++w)
+                    out[(((size_t)b * oc + c) * oh + h) * ow + w] =
+                        in[(((size_t)b * channels + c * step0 + start0) * height + h * step1 + start1) * width + w * step2 + start2];
+}
+
+/* Blas::cpuBilinearResize (src/core/MsnhBlas.cpp:2400-2465). */
+void msnh_or_bilinear(const float *in, int batch, int channels, int height, int width, int outH, int outW, int alignCorners,
+                      float *out)
+{
+    const float rH = alignCorners == 0 ? 1.0f * height / outH : 1.0f * (height - 1) / (outH - 1);
+    const float rW = alignCorners == 0 ? 1.0f * width / outW : 1.0f * (width - 1) / (outW - 1);
+    const size_t inSize = (size_t)width * height, outSize = (size_t)outW * outH;
+    for (size_t i = 0; i < outSize; ++i)
+    {
+        const int h2 = (int)(i / outW), w2 = (int)(i % outW);
+        float h1r, w1r;
+        if (alignCorners == 0)
+        {
+            const float ih = rH * (h2 + 0.5f) - 0.5f;
+            const float iw = rW * (w2 + 0.5f) - 0.5f;
+            h1r = ih < 0 ? 0 : ih;
+            w1r = iw < 0 ? 0 : iw;
+        }
+        else
+        {
+            h1r = rH * h2;
+            w1r = rW * w2;
+        }
+        const int h1 = (int)h1r, w1 = (int)w1r;
+        const int h1p = h1 < height - 1 ? 1 : 0, w1p = w1 < width - 1 ? 1 : 0;
+        const float h1L = h1r - h1, h0L = 1.0f - h1L, w1L = w1r - w1, w0L = 1.0f - w1L;
+        const float *ip = in + (size_t)h1 * width + w1;
+        for (int c = 0; c < channels * batch; ++c)
+        {
+            const float *t = ip + c * inSize;
+            out[i + c * outSize] = h0L * (w0L * t[0] + w1L * t[w1p]) + h1L * (w0L * t[h1p * width] + w1L * t[h1p * width + w1p]);
+        }
+    }
+}
+
+/* SoftMaxLayer::forward with groups == 1 (src/layers/MsnhSoftMaxLayer.cpp:60-93): Blas::softmax over all inputNum values
+ * of each image, scalar path (src/core/MsnhBlas.cpp:2076-2110): e = exp(x/T - max/T) in double, rounded to float. */
+void msnh_or_softmax(const float *in, int batch, int num, float temperature, float *out)
+{
+    for (int b = 0; b < batch; ++b)
+    {
+        const float *x = in + (size_t)b * num;
+        float *y = out + (size_t)b * num;
+        float largest = -FLT_MAX, sum = 0;
+        for (int i = 0; i < num; ++i)
+            if (x[i] > largest) largest = x[i];
+        for (int i = 0; i < num; ++i)
+        {
+            const float e = (float)exp(x[i] / temperature - largest / temperature);
+            sum += e;
+            y[i] = e;
+        }
+        for (int i = 0; i < num; ++i)
+            y[i] /= sum;
+    }
+}
+
+/* GlobalAvgPoolLayer::forward (src/layers/MsnhGlobalAvgPoolLayer.cpp:152-168): running float sum over the plane, / (h*w). */
+void msnh_or_global_avgpool(const float *in, int batch, int channels, int hw, float *out)
+{
+    for (int b = 0; b < batch; ++b)
+        for (int k = 0; k < channels; ++k)
+        {
+            float acc = 0;
+            for (int i = 0; i < hw; ++i)
+                acc += in[((size_t)b * channels + k) * hw + i];
+            out[(size_t)b * channels + k] = acc / hw;
         }
 }
 

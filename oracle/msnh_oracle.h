@@ -18,7 +18,7 @@ extern "C" {
 
 /* values of the reference's ActivationType (include/Msnhnet/config/MsnhnetCfg.h:95-120) */
 enum { MSNH_OR_ACT_LOGISTIC = 0, MSNH_OR_ACT_RELU = 1, MSNH_OR_ACT_RELU6 = 2, MSNH_OR_ACT_LEAKY = 8,
-       MSNH_OR_ACT_SWISH = 16, MSNH_OR_ACT_MISH = 18, MSNH_OR_ACT_NONE = 22 };
+       MSNH_OR_ACT_SWISH = 16, MSNH_OR_ACT_HARD_SWISH = 17, MSNH_OR_ACT_MISH = 18, MSNH_OR_ACT_NONE = 22 };
 
 void  msnh_or_im2col(const float *im, int channels, int height, int width, int kH, int kW, int padH, int padW,
                      int strideH, int strideW, int dilH, int dilW, float *col);
@@ -44,7 +44,17 @@ void  msnh_or_connected(const float *in, int batch, int inputs, int outputs, con
 void  msnh_or_upsample(const float *in, int batch, int channels, int height, int width, int strideX, int strideY,
                        float scale, float *out);
 void  msnh_or_axpy(long long n, float alpha, const float *x, float *y);
-void  msnh_or_yolo_decode(float *data, int batch, int width, int height, int classNum, const float *anchors6, float ratio);
+/* version 3 / 4: yolov3 and yolov4 decoding; 5: yolov5 */
+void  msnh_or_yolo_decode(float *data, int batch, int width, int height, int classNum, const float *anchors6, float ratio,
+                          int version);
+void  msnh_or_pad(const float *in, int batch, int channels, int height, int width, int top, int down, int left, int right,
+                  float value, float *out);
+void  msnh_or_slice(const float *in, int batch, int channels, int height, int width, int start0, int step0, int start1, int step1,
+                    int start2, int step2, float *out);
+void  msnh_or_softmax(const float *in, int batch, int num, float temperature, float *out);
+void  msnh_or_global_avgpool(const float *in, int batch, int channels, int hw, float *out);
+void  msnh_or_bilinear(const float *in, int batch, int channels, int height, int width, int outH, int outW, int alignCorners,
+                       float *out);
 float msnh_or_iou(const float *xywh1, const float *xywh2);
 /* One image.  heads[i] points at a decoded head [3*(5+classes)][hw[i]]; boxes out as rows of
  * 7 floats (x y w h conf bestClsConf bestClsIdx).  Returns the box count (may exceed capBoxes). */

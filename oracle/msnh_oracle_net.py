@@ -20,7 +20,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libmsnh_oracle.so")
 
-ACT = {"logistic": 0, "relu": 1, "relu6": 2, "leaky": 8, "swish": 16, "mish": 18, "none": 22}
+ACT = {"logistic": 0, "relu": 1, "relu6": 2, "leaky": 8, "swish": 16, "hardswish": 17, "mish": 18, "none": 22}
 _fp = ctypes.POINTER(ctypes.c_float)
 _lib = None
 
@@ -39,7 +39,12 @@ def lib():
         L.msnh_or_activate_array.argtypes = [_fp, ll, ci, cf]
         L.msnh_or_activate.argtypes = [cf, ci, cf]
         L.msnh_or_activate.restype = cf
-        L.msnh_or_yolo_decode.argtypes = [_fp, ci, ci, ci, ci, _fp, cf]
+        L.msnh_or_yolo_decode.argtypes = [_fp, ci, ci, ci, ci, _fp, cf, ci]
+        L.msnh_or_pad.argtypes = [_fp, ci, ci, ci, ci, ci, ci, ci, ci, cf, _fp]
+        L.msnh_or_slice.argtypes = [_fp, ci, ci, ci, ci, ci, ci, ci, ci, ci, ci, _fp]
+        L.msnh_or_bilinear.argtypes = [_fp, ci, ci, ci, ci, ci, ci, ci, _fp]
+        L.msnh_or_softmax.argtypes = [_fp, ci, ci, cf, _fp]
+        L.msnh_or_global_avgpool.argtypes = [_fp, ci, ci, ci, _fp]
         L.msnh_or_iou.argtypes = [_fp, _fp]
         L.msnh_or_iou.restype = cf
         L.msnh_or_yolo_out.argtypes = [ctypes.POINTER(_fp), ctypes.POINTER(ci), ci, ci, cf, cf, _fp, ll]
@@ -134,11 +139,51 @@ def activate(x, act, act_param=0.1):
     return out
 
 
-def yolo_decode(x, class_num, anchors6, ratio):
+def yolo_decode(x, class_num, anchors6, ratio, version=3):
     out = _f32(x).copy()
     b, c, h, w = out.shape
     a = _f32(anchors6)
-    lib().msnh_or_yolo_decode(_p(out), b, w, h, class_num, _p(a), ratio)
+    lib().msnh_or_yolo_decode(_p(out), b, w, h, class_num, _p(a), ratio, version)
+    return out
+
+
+def pad(x, top, down, left, right, value=0.0):
+    x = _f32(x)
+    b, c, h, w = x.shape
+    out = np.empty((b, c, h + top + down, w + left + right), np.float32)
+    lib().msnh_or_pad(_p(x), b, c, h, w, top, down, left, right, value, _p(out))
+    return out
+
+
+def slice_(x, start0, step0, start1, step1, start2, step2):
+    x = _f32(x)
+    b, c, h, w = x.shape
+    ext = lambda n, st, sp: (n - st) // sp + (1 if (n - st) % sp else 0)
+    out = np.empty((b, ext(c, start0, step0), ext(h, start1, step1), ext(w, start2, step2)), np.float32)
+    lib().msnh_or_slice(_p(x), b, c, h, w, start0, step0, start1, step1, start2, step2, _p(out))
+    return out
+
+
+def softmax(x, temperature=1.0):
+    x = _f32(x)
+    out = np.empty_like(x)
+    lib().msnh_or_softmax(_p(x), x.shape[0], x.size // x.shape[0], temperature, _p(out))
+    return out
+
+
+def global_avgpool(x):
+    x = _f32(x)
+    b, c, h, w = x.shape
+    out = np.empty((b, c, 1, 1), np.float32)
+    lib().msnh_or_global_avgpool(_p(x), b, c, h * w, _p(out))
+    return out
+
+
+def bilinear(x, out_h, out_w, align_corners=0):
+    x = _f32(x)
+    b, c, h, w = x.shape
+    out = np.empty((b, c, out_h, out_w), np.float32)
+    lib().msnh_or_bilinear(_p(x), b, c, h, w, out_h, out_w, align_corners, _p(out))
     return out
 
 
@@ -284,7 +329,26 @@ class OracleNet:
         if key == "empty":
             return x.copy()
         if key == "upsample":
-            return upsample(x, int(d.get("stride", 1)), float(d.get("scale", 1.0)))
+            if d.get("type", "nearest").strip() == "bilinear":
+                # output extent int(extent * scale) (src/layers/MsnhUpSampleLayer.cpp:20-24)
+                sx = float(d.get("scaleX", d.get("scale", 1.0))); sy = float(d.get("scaleY", d.get("scale", 1.0)))
+                return bilinear(x, int(x.shape[2] * np.float32(sy)), int(x.shape[3] * np.float32(sx)), int(d.get("alignCorners", 0)))
+            return upsample(x, int(d.get("stride", d.get("strideX", 1))), float(d.get("scale", d.get("scaleX", 1.0))))
+        if key == "softmax":
+            if int(d.get("groups", 1)) != 1:
+                raise ValueError("softmax groups")
+            return softmax(x, float(d.get("temperature", 1.0)))
+        if key == "globalavgpool":
+            return global_avgpool(x)
+        if key == "act":
+            act, ap = _act(d)
+            return activate(x, act, ap)
+        if key == "padding":
+            return pad(x, int(d.get("top", 0)), int(d.get("down", 0)), int(d.get("left", 0)), int(d.get("right", 0)),
+                       float(d.get("paddingVal", 0)))
+        if key == "slice":
+            return slice_(x, int(d.get("start0", 0)), int(d.get("step0", 1)), int(d.get("start1", 0)), int(d.get("step1", 1)),
+                          int(d.get("start2", 0)), int(d.get("step2", 1)))
         raise ValueError(f"{key} is not supported")
 
     def _seq(self, nodes, x):
@@ -325,13 +389,38 @@ class OracleNet:
             elif key == "route":
                 idx = [int(t) for t in d["layers"].split(",") if t.strip() != ""]
                 idx = [i if i >= 0 else li + i for i in idx]
-                x = np.concatenate([outs[i] for i in idx], axis=1)
+                if int(d.get("addModel", 0)) == 1:
+                    # zero-filled output, then += each listed layer in list order (src/layers/MsnhRouteLayer.cpp:77-115)
+                    x = np.zeros_like(outs[idx[0]])
+                    for i in idx:
+                        x = (x + outs[i]).astype(np.float32)
+                else:
+                    x = np.concatenate([outs[i] for i in idx], axis=1)
+                act, ap = _act(d)
+                if act != "none":
+                    x = activate(x, act, ap)
+            elif key == "varop":
+                # one listed layer: A = previous layer, B = it; two: A, B = the listed layers
+                # (src/layers/MsnhVariableOpLayer.cpp:78-165); constant forms use A and constVal (:166-240)
+                idx = [int(t) for t in d.get("layers", "").split(",") if t.strip() != ""]
+                idx = [i if i >= 0 else li + i for i in idx]
+                kind = d.get("type", "add").strip()
+                cv = np.float32(float(d.get("constVal", 0)))
+                if kind.endswith("Const") or kind.endswith("ConstInv"):
+                    a = x if not idx else outs[idx[0]]
+                    x = {"addConst": lambda: a + cv, "subConst": lambda: a - cv, "subConstInv": lambda: cv - a, "mulConst": lambda: a * cv,
+                         "divConst": lambda: a / cv, "divConstInv": lambda: cv / a}[kind]().astype(np.float32)
+                else:
+                    a, b = (x, outs[idx[0]]) if len(idx) == 1 else (outs[idx[0]], outs[idx[1]])
+                    x = {"add": lambda: a + b, "sub": lambda: a - b, "subInv": lambda: b - a, "mul": lambda: a * b, "div": lambda: a / b,
+                         "divInv": lambda: b / a}[kind]().astype(np.float32)
             elif key == "yolo":
                 anchors = [float(t) for t in d["anchors"].split(",")]
                 cls = int(d.get("classNum", 1))
                 if 3 * (cls + 5) != x.shape[1]:
                     raise ValueError("class num error!")
-                x = yolo_decode(x, cls, anchors, self.h / x.shape[2])
+                version = 5 if d.get("yoloType", "yolov3").strip().startswith("yolov5") else 3
+                x = yolo_decode(x, cls, anchors, self.h / x.shape[2], version)
                 heads[li] = (x, cls)
             elif key == "yoloout":
                 idx = [int(t) for t in d["layers"].split(",") if t.strip() != ""]

@@ -71,6 +71,28 @@ def micro_cases():
         #  largest tensor of the net: a wide conv in front keeps it from overrunning the pool)
         "concatblock_spp": lambda: g(4, 9, 9, lambda q: (q.conv(32, 1, 1, 0, bn=1, act="leaky"), q.conv(8, 1, 1, 0, bn=1, act="leaky"),
                                                         q.concatblock([lambda: q.maxpool_node(5, 1, 2), lambda: q.maxpool_node(3, 1, 1), None]))),
+        # ---- layer types of the other shipped graphs --------------------------------------------------------------
+        "conv_hardswish": lambda: g(6, 7, 8, lambda q: q.conv(9, 3, 1, 1, bn=1, act="hardswish")),
+        "act_after_bn": lambda: g(5, 8, 8, lambda q: (q.conv(8, 3, 1, 1, bn=0, act="none"), q.batchnorm("none"), q.act("hardswish"),
+                                                      q.maxpool(2, 2, 0), q.act("leaky"))),
+        "padding_then_pool": lambda: g(4, 7, 9, lambda q: (q.conv(8, 3, 1, 1, bn=1, act="leaky"), q.padding(0, 1, 0, 1, 0.0), q.maxpool(2, 1, 0))),
+        "padding_first": lambda: g(3, 14, 12, lambda q: (q.padding(3, 3, 3, 3, 0.0), q.conv(8, 7, 2, 0, bn=0, act="relu"), q.padding(1, 0, 2, 1, -1.5))),
+        "route_add": lambda: g(4, 6, 6, lambda q: (q.conv(8, 3, 1, 1, bn=1, act="leaky"), q.conv(8, 1, 1, 0, bn=1, act="none"),
+                                                   q.conv(8, 3, 1, 1, bn=1, act="none"), q.route([-1, -3], add_model=True),
+                                                   q.route([-1, 1, 0], add_model=True, act="relu"))),
+        "varop": lambda: g(4, 5, 7, lambda q: (q.conv(6, 3, 1, 1, bn=0, act="none"), q.conv(6, 1, 1, 0, bn=0, act="relu"), q.varop("add", [0]),
+                                               q.act("relu"), q.varop("sub", [0, 1]), q.varop("subInv", [0]), q.varop("mulConst", None, 0.75),
+                                               q.varop("subConstInv", None, 2.0), q.varop("addConst", None, -0.5))),
+        "slice_focus": lambda: g(3, 10, 12, lambda q: (q.act("none"), q.slice(0, 1, 0, 2, 0, 2), q.route([-2]), q.slice(0, 1, 1, 2, 0, 2),
+                                                       q.route([-4]), q.slice(0, 1, 0, 2, 1, 2), q.route([-6]), q.slice(0, 1, 1, 2, 1, 2),
+                                                       q.route([-7, -5, -3, -1]), q.conv(8, 3, 1, 1, bn=1, act="hardswish"))),
+        "slice_channels": lambda: g(3, 6, 6, lambda q: (q.conv(10, 1, 1, 0, bn=0, act="none"), q.slice(1, 3, 1, 1, 2, 3))),
+        "globalavg_fc_softmax": lambda: g(3, 6, 5, lambda q: (q.conv(12, 3, 1, 1, bn=0, act="relu"), q.globalavgpool(), q.connect(7), q.softmax())),
+        "softmax_map": lambda: g(3, 5, 6, lambda q: (q.conv(2, 3, 1, 1, bn=0, act="none"), q.softmax(2.0))),
+        "bilinear_x2": lambda: g(3, 5, 6, lambda q: (q.conv(6, 3, 1, 1, bn=0, act="none"), q.upsample_bilinear(2.0, 2.0, 0))),
+        "bilinear_align": lambda: g(3, 6, 4, lambda q: (q.conv(6, 1, 1, 0, bn=0, act="none"), q.upsample_bilinear(2.5, 1.5, 1))),
+        "yolo5_head": lambda: g(8, 6, 6, lambda q: (q.conv(21, 1, 1, 0, bn=0, act="none"), q.yolo([10, 13, 16, 30, 33, 23], class_num=2, yolo_type="yolov5"),
+                                                   q.yoloout([1], 0.3, 0.45, yolo_type="yolov5"))),
         "yolo_head": lambda: g(8, 6, 6, lambda q: (q.conv(21, 1, 1, 0, bn=0, act="none"), q.yolo([10, 13, 16, 30, 33, 23], class_num=2),
                                                   q.yoloout([1], 0.3, 0.45))),
     }
@@ -95,7 +117,7 @@ def main():
         r = refshim.RefNet(netp, binp, scalar=True)
         c0 = int(gw.text().split("channels:")[1].split()[0]); h0 = int(gw.text().split("height:")[1].split()[0]); w0 = int(gw.text().split("width:")[1].split()[0])
         x = zoo.seeded_input(1, c0, h0, w0, seed + 1)[0]
-        if name == "yolo_head":
+        if name in ("yolo_head", "yolo5_head"):
             x = (x - 0.5) * 8          # spread the logits so some boxes pass the threshold and some do not
         outs = r.run(x)
         store[f"micro/{name}/graph"] = np.frombuffer(gw.text().encode(), np.uint8)

@@ -63,6 +63,37 @@ def test_graph_construction_matches_reference_tables(arch, dtype, batch, size, t
     assert sum(i["numWeights"] for i in infos) == sum(s.count for s in g.slots)
 
 
+SHIPPED = sorted(__import__("glob").glob("/root/reference/models/*/*.msnhnet"))
+# graphs this build refuses, with the reason: transposed convolution is not implemented; yolov3_spp.msnhnet uses node names
+# ("yolov3", "yolov3out") that the reference's own parser rejects too
+REFUSED = {"fcns.msnhnet": r"\[deconv\]", "yolov3_spp.msnhnet": r"\[yolov3\]"}
+
+
+@pytest.mark.skipif(not SHIPPED, reason="the reference's model files are not present")
+@pytest.mark.parametrize("path", SHIPPED, ids=[os.path.basename(p) for p in SHIPPED])
+def test_shipped_graphs_build_like_the_reference(path):
+    """Every .msnhnet file the reference ships builds here, layer for layer with the shapes and weight counts the reference's own
+    NetBuilder derives (when its library is present)."""
+    import refshim
+    name = os.path.basename(path)
+    if name in REFUSED:
+        with pytest.raises(netapi.MsnhnetError, match=REFUSED[name]):
+            netapi.Net(path)
+        return
+    infos = netapi.Net(path).layer_infos()
+    assert len(infos) > 0
+    if not refshim.available():
+        return
+    r = refshim.RefNet(path)
+    ref = r.layer_infos()
+    r.close()
+    assert len(infos) == len(ref)
+    for i, (a, b) in enumerate(zip(infos, ref)):
+        # (a softmax layer leaves its image shape unset in the reference: compare the element counts only)
+        keys = ["outputNum", "numWeights"] if b["type"] in ("6", "softmax") else ["outH", "outW", "outC", "outputNum", "numWeights"]
+        assert [a[k] for k in keys] == [b[k] for k in keys], (name, i, a, b)
+
+
 def test_zoo_totals():
     want = {"resnet18": 11699112, "resnet50": 25610152, "mobilenetv2": 3538984, "yolov3": 62001757, "yolov4": 64429405}
     gf = {"resnet18": 3.63, "resnet50": 8.18, "mobilenetv2": 0.605, "yolov3": 140.7, "yolov4": 128.4}

@@ -130,6 +130,54 @@ def test_fp16_final_outputs(arch, size, batch):
                 assert int(np.argmax(logits[b])) == int(np.argmax(r))
 
 
+import os
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_golden.npz"))
+MICRO = bytes(GOLD["micro/names"]).decode().split("\n")
+
+
+@pytest.mark.parametrize("fp16", [False, True])
+@pytest.mark.parametrize("name", MICRO)
+def test_micro_graphs_against_reference_golden(name, fp16, tmp_path):
+    """Every micro graph of the golden file (one per op / block / layer type, outputs written by the reference's own CPU
+    forward) through NetBuilder on the device: every layer output in float32 to 1e-4, in float16 to 2e-2 of the layer's range;
+    boxes of the yolo heads as sets."""
+    text = bytes(GOLD[f"micro/{name}/graph"]).decode()
+    netp = str(tmp_path / (name + ".msnhnet"))
+    binp = str(tmp_path / (name + ".msnhbin"))
+    with open(netp, "w") as f:
+        f.write(text)
+    np.asarray(GOLD[f"micro/{name}/weights"], np.float32).tofile(binp)
+    x = GOLD[f"micro/{name}/input"][None]
+    print("running micro", name, "fp16" if fp16 else "fp32", flush=True)
+    m = netapi.Net(netp, binp, fp16=fp16, dump_layers=True)
+    is_yolo = any(m.layer_info(i)["type"] == "yoloout" for i in range(m.num_layers()))
+    boxes = m.run_yolo(x) if is_yolo else None
+    if not is_yolo:
+        m.run_classify(x)
+    tol = 2e-2 if fp16 else 1e-4
+    for i in range(m.num_layers()):
+        ref = GOLD[f"micro/{name}/out{i}"]
+        t = m.layer_info(i)["type"]
+        if ref.size == 0 or t == "yoloout" or (fp16 and t == "yolo"):
+            continue
+        got = m.layer_output(i).ravel()
+        assert got.size == ref.size, (name, i, t, got.size, ref.size)
+        assert nu.rel_err(got, ref) <= tol, (name, i, t, nu.rel_err(got, ref))
+    if is_yolo and not fp16:
+        rb, gb = nu.sort_boxes(GOLD[f"micro/{name}/boxes"]), nu.sort_boxes(boxes[0])
+        assert len(rb) == len(gb)
+        assert nu.rel_err(gb[:, :6], rb[:, :6]) <= 1e-4
+    # the production path (fused launches, captured graph) gives what the layer-by-layer path gave
+    fast = netapi.Net(netp, binp, fp16=fp16, dump_layers=False)
+    if is_yolo:
+        fb = fast.run_yolo(x)
+        if not fp16:
+            assert len(fb[0]) == len(boxes[0])
+    else:
+        a, b = m.run_classify(x), fast.run_classify(x)
+        assert nu.rel_err(b, a) <= (1e-5 if not fp16 else 2e-2)
+
+
 @pytest.mark.parametrize("arch,size,batch", [("resnet18", 224, 1), ("yolov3", 224, 2)])
 def test_fp16_winograd_network(arch, size, batch):
     """every 3x3 stride-1 convolution through Winograd F(2x2,3x3): same final outputs within the float16 tolerance"""

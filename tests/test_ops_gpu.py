@@ -118,6 +118,80 @@ def test_upsample(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("c", [24, 5])
+def test_pad(dtype, c):
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(3)
+    x = _x(rng, (2, c, 5, 7), dtype)
+    ref = on.pad(x, 1, 2, 0, 3, -1.5)
+    ld = (c + 7) // 8 * 8
+    xd = gu.nhwc_dev(x, dtype, ld)
+    yd = torch.full((2, 8, 10, ld + 8), 3.0, dtype=gu.TORCH_DT[dtype]).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_pad(dtype, 2, 5, 7, c, gu.ptr(xd), ld, 1, 0, 8, 10, 1.0, -1.5, gu.ptr(yd), ld + 8, None))
+    gu.sync()
+    assert np.array_equal(gu.nchw_host(yd, c), ref)
+    assert (yd[..., c:].float().cpu().numpy() == 3.0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_slice(dtype):
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(4)
+    x = _x(rng, (2, 10, 9, 11), dtype)
+    for args in ((0, 1, 0, 2, 1, 2), (1, 3, 1, 1, 2, 3), (9, 1, 8, 5, 0, 11)):
+        ref = on.slice_(x, *args)
+        oc, oh, ow = ref.shape[1:]
+        xd = gu.nhwc_dev(x, dtype, 16)
+        yd = torch.full((2, oh, ow, 16), 3.0, dtype=gu.TORCH_DT[dtype]).cuda()
+        gu.sync()
+        abi.check(abi.lib().msnh_hip_slice(dtype, 2, 9, 11, gu.ptr(xd), 16, *args, oc, oh, ow, 1.0, gu.ptr(yd), 16, None))
+        gu.sync()
+        assert np.array_equal(gu.nchw_host(yd, oc), ref)
+        assert (yd[..., oc:].float().cpu().numpy() == 3.0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("oh,ow,align", [(10, 14, 0), (12, 9, 1), (3, 4, 0), (5, 7, 1)])
+def test_upsample_bilinear(dtype, oh, ow, align):
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(5)
+    x = _x(rng, (2, 24, 5, 7), dtype)
+    ref = on.bilinear(x, oh, ow, align)
+    xd = gu.nhwc_dev(x, dtype)
+    yd = torch.full((2, oh, ow, 32), 3.0, dtype=gu.TORCH_DT[dtype]).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_upsample_bilinear(dtype, 2, 5, 7, 24, gu.ptr(xd), 24, oh, ow, align, 1.0, gu.ptr(yd), 32, None))
+    gu.sync()
+    # same float32 expression; the compiler may contract its multiply-adds
+    assert gu.rel_err(gu.nchw_host(yd, 24), ref) <= (2e-6 if dtype == abi.F32 else 1e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("c,h,w,temp", [(1000, 1, 1, 1.0), (2, 9, 11, 2.0), (21, 4, 4, 0.5)])
+def test_softmax(dtype, c, h, w, temp):
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(6)
+    x = _x(rng, (3, c, h, w), dtype) * 4
+    if dtype == abi.F16:
+        x = gu.round_f16(x)
+    ref = on.softmax(x, temp)
+    ld = (c + 7) // 8 * 8
+    xd = gu.nhwc_dev(x, dtype, ld)
+    yd = torch.zeros((3, h, w, ld), dtype=gu.TORCH_DT[dtype]).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_softmax(dtype, 3, h * w, c, gu.ptr(xd), ld, 1.0, temp, gu.ptr(yd), ld, 1.0, None))
+    gu.sync()
+    got = gu.nchw_host(yd, c)
+    assert gu.rel_err(got, ref) <= (1e-5 if dtype == abi.F32 else 2e-3)
+    assert np.allclose(got.reshape(3, -1).sum(1), 1.0, atol=1e-5 if dtype == abi.F32 else 5e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_connected(dtype):
     import gpuutil as gu
     gu.init()
@@ -175,7 +249,8 @@ def test_layout_roundtrip(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_yolo_decode(dtype):
+@pytest.mark.parametrize("version", [3, 5])
+def test_yolo_decode(dtype, version):
     import gpuutil as gu
     gu.init()
     rng = np.random.default_rng(4)
@@ -188,7 +263,7 @@ def test_yolo_decode(dtype):
         x = gu.round_f16(x)
     anchors = np.array([10, 13, 16, 30, 33, 23], np.float32)
     ratio = 32.0
-    ref = on.yolo_decode(x, cls, anchors, ratio)                       # [2][3*per][h][w]
+    ref = on.yolo_decode(x, cls, anchors, ratio, version)              # [2][3*per][h][w]
     ref_shuf = ref.reshape(2, 3, per, h * w).transpose(0, 1, 3, 2)    # [2][3][hw][per]
     xd = gu.nhwc_dev(x, dtype, 256)
     dd = torch.zeros((2, 3, h * w, per), dtype=torch.float32).cuda()
@@ -197,7 +272,7 @@ def test_yolo_decode(dtype):
     cc = torch.zeros(2, dtype=torch.int32).cuda()
     gu.sync()
     abi.check(abi.lib().msnh_hip_yolo_decode(dtype, 2, h, w, cls, gu.ptr(xd), 256, 1.0, anchors.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
-                                             ratio, gu.ptr(dd), 3 * h * w * per, 0.5, gu.ptr(ci), cap, 1000, gu.ptr(cc), None))
+                                             ratio, version, gu.ptr(dd), 3 * h * w * per, 0.5, gu.ptr(ci), cap, 1000, gu.ptr(cc), None))
     gu.sync()
     out = dd.cpu().numpy()
     assert gu.rel_err(out, ref_shuf) <= 2e-6
