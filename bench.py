@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the convolutional hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload yolov3|yolov4|resnet50|mobilenetv2|resnet18]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload yolov3|yolov4|resnet50|mobilenetv2|resnet18|yolov3_tiny|yolov5s]
 
 A step is one forward of one batch through NetBuilder's device-resident path (input already in HBM): every
 launch of the planned graph, and for detection networks the candidate compaction on the device plus copy-back,
@@ -23,7 +23,9 @@ from msnhnet_amd import netapi, zoo  # noqa: E402
 
 # workload -> (dtype, batch, input size) : the benchmark configurations
 WORKLOADS = {"resnet18": ("f32", 1, 224), "resnet50": ("f16", 32, 224), "mobilenetv2": ("f16", 64, 224),
-             "yolov3": ("f16", 8, 608), "yolov4": ("f16", 16, 608)}
+             "yolov3": ("f16", 8, 608), "yolov4": ("f16", 16, 608),
+             # two of the reference's other shipped detectors, at the input size of their own graph files
+             "yolov3_tiny": ("f16", 8, 416), "yolov5s": ("f16", 8, 512)}
 PEAK = {"f16": 2500.0, "f32": 157.3}        # dense MFMA peak, TFLOP/s
 
 

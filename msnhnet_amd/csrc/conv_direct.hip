@@ -79,6 +79,113 @@ __global__ __launch_bounds__(256) void convDirectKernel(const T *__restrict__ x,
     y[static_cast<size_t>(p) * outLd + oc] = fromF<TOut>(epilogue(e, acc, oc, r));
 }
 
+// Register-blocked variant for out_c/groups % 8 == 0: a lane owns one output pixel and 8 consecutive output channels
+// (blockIdx.y picks the channel block, so the weight addresses are uniform over a wavefront and every input value
+// fetched feeds 8 multiply-adds); one 8-channel NHWC store per lane.
+template <typename T, typename TOut>
+__global__ __launch_bounds__(256) void convDirectBlockedKernel(const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ res,
+                                                               TOut *__restrict__ y, EpiArgs e, int H, int W, int inLd, int OH, int OW,
+                                                               int outLd, int resLd, int cinG, int coutG, int ksize, int stride,
+                                                               int pad, int dil, long long pixels)
+{
+    constexpr int OCB = 8;
+    const long long p = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (p >= pixels) return;
+    const int oc0 = blockIdx.y * OCB;
+    const int g = oc0 / coutG;
+    const int ox = static_cast<int>(p % OW);
+    const long long t = p / OW;
+    const int oy = static_cast<int>(t % OH);
+    const int b  = static_cast<int>(t / OH);
+    const int K = ksize * ksize * cinG;
+    const T *wp = w + static_cast<size_t>(oc0) * K;
+    float acc[OCB];
+#pragma unroll
+    for (int j = 0; j < OCB; ++j) acc[j] = 0.f;
+    for (int ki = 0; ki < ksize; ++ki)
+    {
+        const int iy = oy * stride - pad + ki * dil;
+        for (int kj = 0; kj < ksize; ++kj)
+        {
+            const int ix = ox * stride - pad + kj * dil;
+            const bool in = iy >= 0 && iy < H && ix >= 0 && ix < W;
+            const T *xp = x + ((static_cast<size_t>(b) * H + (in ? iy : 0)) * W + (in ? ix : 0)) * inLd + g * cinG;
+            const T *wt = wp + (ki * ksize + kj) * cinG;
+            for (int c = 0; c < cinG; ++c)
+            {
+                const float xv = in ? toF(xp[c]) : 0.f;
+#pragma unroll
+                for (int j = 0; j < OCB; ++j) acc[j] += xv * toF(wt[static_cast<size_t>(j) * K + c]);
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < OCB; ++j)
+    {
+        const float r = e.hasRes ? toF(res[static_cast<size_t>(p) * resLd + oc0 + j]) : 0.f;
+        y[static_cast<size_t>(p) * outLd + oc0 + j] = fromF<TOut>(epilogue(e, acc[j], oc0 + j, r));
+    }
+}
+
+// Wider variant for small K = ksize^2 * (in_c/groups): the OCB x K weight block of the workgroup sits in LDS as float32,
+// [k][OCB], so that the inner loop is one input load, OCB/4 broadcast 16-byte LDS reads and OCB multiply-adds.
+template <typename T, typename TOut, int OCB>
+__global__ __launch_bounds__(256) void convDirectLdsKernel(const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ res,
+                                                           TOut *__restrict__ y, EpiArgs e, int H, int W, int inLd, int OH, int OW,
+                                                           int outLd, int resLd, int cinG, int coutG, int ksize, int stride,
+                                                           int pad, int dil, long long pixels)
+{
+    extern __shared__ __attribute__((aligned(16))) float wl[];
+    const int oc0 = blockIdx.y * OCB;
+    const int g = oc0 / coutG;
+    const int K = ksize * ksize * cinG;
+    for (int i = threadIdx.x; i < K * OCB; i += 256)
+    {
+        const int k = i / OCB, j = i - k * OCB;
+        wl[i] = toF(w[static_cast<size_t>(oc0 + j) * K + k]);
+    }
+    __syncthreads();
+    const long long p = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (p >= pixels) return;
+    const int ox = static_cast<int>(p % OW);
+    const long long t = p / OW;
+    const int oy = static_cast<int>(t % OH);
+    const int b  = static_cast<int>(t / OH);
+    float acc[OCB];
+#pragma unroll
+    for (int j = 0; j < OCB; ++j) acc[j] = 0.f;
+    for (int ki = 0; ki < ksize; ++ki)
+    {
+        const int iy = oy * stride - pad + ki * dil;
+        for (int kj = 0; kj < ksize; ++kj)
+        {
+            const int ix = ox * stride - pad + kj * dil;
+            const bool in = iy >= 0 && iy < H && ix >= 0 && ix < W;
+            const T *xp = x + ((static_cast<size_t>(b) * H + (in ? iy : 0)) * W + (in ? ix : 0)) * inLd + g * cinG;
+            const f32x4 *wr = reinterpret_cast<const f32x4 *>(wl + static_cast<size_t>(ki * ksize + kj) * cinG * OCB);
+            for (int c = 0; c < cinG; ++c)
+            {
+                const float xv = in ? toF(xp[c]) : 0.f;
+#pragma unroll
+                for (int j4 = 0; j4 < OCB / 4; ++j4)
+                {
+                    const f32x4 w4 = wr[c * (OCB / 4) + j4];
+                    acc[4 * j4 + 0] += xv * w4[0];
+                    acc[4 * j4 + 1] += xv * w4[1];
+                    acc[4 * j4 + 2] += xv * w4[2];
+                    acc[4 * j4 + 3] += xv * w4[3];
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < OCB; ++j)
+    {
+        const float r = e.hasRes ? toF(res[static_cast<size_t>(p) * resLd + oc0 + j]) : 0.f;
+        y[static_cast<size_t>(p) * outLd + oc0 + j] = fromF<TOut>(epilogue(e, acc[j], oc0 + j, r));
+    }
+}
+
 // ---- DEPTHWISE ------------------------------------------------------------------------------------
 // weights [tap][C]; thread = (pixel, VEC channels).  VEC = 1 is the unaligned fallback.
 template <typename T, int VEC>
@@ -392,6 +499,45 @@ int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const
     }
     case MSNH_CONV_DIRECT:
     {
+        const int Kdir = d->ksize * d->ksize * cinG;
+        const int ocb = coutG % 32 == 0 ? 32 : (coutG % 16 == 0 ? 16 : 0);
+        if (ocb && static_cast<size_t>(Kdir) * ocb * sizeof(float) <= 48 * 1024 && d->out_c / ocb <= 65535)
+        {
+            dim3 lgrid(gridFor(P, 256), d->out_c / ocb);
+            const size_t lds = static_cast<size_t>(Kdir) * ocb * sizeof(float);
+#define MSNH_DIRECTL(T, TO, B)                                                                                          \
+    hipLaunchKernelGGL((convDirectLdsKernel<T, TO, B>), lgrid, dim3(256), lds, st, static_cast<const T *>(x), static_cast<const T *>(w),  \
+                       static_cast<const T *>(residual), static_cast<TO *>(y), e, d->in_h, d->in_w, d->in_ld, d->out_h, d->out_w,  \
+                       d->out_ld, d->res_ld, cinG, coutG, d->ksize, d->stride, d->pad, d->dilation, P)
+#define MSNH_DIRECTL2(T, TO) do { if (ocb == 32) MSNH_DIRECTL(T, TO, 32); else MSNH_DIRECTL(T, TO, 16); } while (0)
+            if (d->dtype == MSNH_F16) { if (d->out_dtype == MSNH_F16) MSNH_DIRECTL2(f16, f16); else MSNH_DIRECTL2(f16, float); }
+            else
+            {
+                MSNH_REQUIRE(d->out_dtype == MSNH_F32, "conv2d: float32 input needs float32 output");
+                MSNH_DIRECTL2(float, float);
+            }
+#undef MSNH_DIRECTL2
+#undef MSNH_DIRECTL
+            MSNH_LAUNCH_CHECK();
+            return 0;
+        }
+        if (coutG % 8 == 0 && d->out_c / 8 <= 65535)
+        {
+            dim3 bgrid(gridFor(P, 256), d->out_c / 8);
+#define MSNH_DIRECTB(T, TO)                                                                                             \
+    hipLaunchKernelGGL((convDirectBlockedKernel<T, TO>), bgrid, dim3(256), 0, st, static_cast<const T *>(x), static_cast<const T *>(w),  \
+                       static_cast<const T *>(residual), static_cast<TO *>(y), e, d->in_h, d->in_w, d->in_ld, d->out_h, d->out_w,  \
+                       d->out_ld, d->res_ld, cinG, coutG, d->ksize, d->stride, d->pad, d->dilation, P)
+            if (d->dtype == MSNH_F16) { if (d->out_dtype == MSNH_F16) MSNH_DIRECTB(f16, f16); else MSNH_DIRECTB(f16, float); }
+            else
+            {
+                MSNH_REQUIRE(d->out_dtype == MSNH_F32, "conv2d: float32 input needs float32 output");
+                MSNH_DIRECTB(float, float);
+            }
+#undef MSNH_DIRECTB
+            MSNH_LAUNCH_CHECK();
+            return 0;
+        }
         const long long total = P * d->out_c;
         dim3 grid(gridFor(total, 256));
 #define MSNH_DIRECT(T, TO)                                                                                              \

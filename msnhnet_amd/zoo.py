@@ -115,9 +115,11 @@ class GraphWriter:
         self._emit(f"  activation: {act}")
         self._conv_apply(filters, k, stride, pad, groups, bn, True if bias is None else bias)
 
-    def bn_node(self, act="none"):
+    def bn_node(self, act="none", eps=None):
         self._emit("batchnorm:")
         self._emit(f"  activation: {act}")
+        if eps is not None:
+            self._emit(f"  eps: {eps}")
         self._bn_apply()
 
     def maxpool_node(self, k, stride, pad):
@@ -133,8 +135,8 @@ class GraphWriter:
         self.conv_node(*a, **kw)
         self._top_done()
 
-    def batchnorm(self, act="none"):
-        self.bn_node(act)
+    def batchnorm(self, act="none", eps=None):
+        self.bn_node(act, eps)
         self._top_done()
 
     def maxpool(self, k, stride, pad):
@@ -552,8 +554,102 @@ def yolov4(batch=1, size=608, conf=0.5, nms=0.5) -> GraphWriter:
     return g
 
 
+def yolov3_tiny(batch=1, size=416, conf=0.2, nms=0.2) -> GraphWriter:
+    """The reference's yolov3_tiny graph (models/yolov3_tiny/yolov3_tiny.msnhnet): six conv + max-pool stages, the last
+    pool with stride 1 behind a one-pixel padding layer, two heads."""
+    g = GraphWriter(batch, 3, size, size)
+    lk = "leaky"
+    for i, c in enumerate((16, 32, 64, 128, 256)):
+        g.conv(c, 3, 1, 1, act=lk)
+        g.maxpool(2, 2, 0)
+    g.conv(512, 3, 1, 1, act=lk)                 # layer 10
+    g.padding(0, 1, 0, 1, 0.0)
+    g.maxpool(2, 1, 0)
+    g.conv(1024, 3, 1, 1, act=lk)
+    g.conv(256, 1, 1, 0, act=lk)                 # layer 14
+    g.conv(512, 3, 1, 1, act=lk)
+    g.conv(255, 1, 1, 0, bn=0, act="none")
+    yolos = []
+    g.yolo([81, 82, 135, 169, 344, 319]); yolos.append(g.n_top - 1)
+    g.route([-4])
+    g.conv(128, 1, 1, 0, act=lk)
+    g.upsample(2)
+    g.route([-1, 8])
+    g.conv(256, 3, 1, 1, act=lk)
+    g.conv(255, 1, 1, 0, bn=0, act="none")
+    g.yolo([10, 14, 23, 27, 37, 58]); yolos.append(g.n_top - 1)
+    g.yoloout(yolos, conf, nms)
+    return g
+
+
+def yolov5s(batch=1, size=512, conf=0.5, nms=0.5) -> GraphWriter:
+    """YOLOv5s in the node vocabulary of the reference's exported graph (models/yolov5s/yolov5s.msnhnet): focus slices,
+    bias-less conv + batchnorm(eps 1e-3) + stand-alone hardswish, CSP stages whose residuals are `varop: add`, SPP, three
+    yolov5 heads."""
+    g = GraphWriter(batch, 3, size, size)
+
+    def cbh(c, k, s):
+        g.conv(c, k, s, k // 2, bn=0, bias=False, act="none")
+        g.batchnorm("none", 0.001)
+        g.act("hardswish")
+
+    def csp(c, n, shortcut=True):
+        start = g.n_top - 1                       # the layer feeding the stage
+        h = c // 2
+        cbh(h, 1, 1)
+        for _ in range(n):
+            inp = g.n_top - 1
+            cbh(h, 1, 1)
+            cbh(h, 3, 1)
+            if shortcut:
+                g.varop("add", [inp])
+        g.conv(h, 1, 1, 0, bn=0, bias=False, act="none")
+        a = g.n_top - 1
+        g.route([start])
+        g.conv(h, 1, 1, 0, bn=0, bias=False, act="none")
+        b = g.n_top - 1
+        g.route([a, b])
+        g.batchnorm("none", 0.001)
+        g.act("leaky,0.1")
+        cbh(c, 1, 1)
+
+    # focus
+    g.act("none")
+    g.slice(0, 1, 0, 2, 0, 2); g.route([-2])
+    g.slice(0, 1, 1, 2, 0, 2); g.route([-4])
+    g.slice(0, 1, 0, 2, 1, 2); g.route([-6])
+    g.slice(0, 1, 1, 2, 1, 2)
+    g.route([-7, -5, -3, -1])
+    cbh(32, 3, 1)
+    cbh(64, 3, 2); csp(64, 1)
+    cbh(128, 3, 2); csp(128, 3); p3 = g.n_top - 1
+    cbh(256, 3, 2); csp(256, 3); p4 = g.n_top - 1
+    cbh(512, 3, 2)
+    # SPP
+    cbh(256, 1, 1); x = g.n_top - 1
+    g.maxpool(5, 1, 2); m5 = g.n_top - 1
+    g.route([x]); g.maxpool(9, 1, 4); m9 = g.n_top - 1
+    g.route([x]); g.maxpool(13, 1, 6); m13 = g.n_top - 1
+    g.route([x, m5, m9, m13])
+    cbh(512, 1, 1)
+    csp(512, 1, False)
+    cbh(256, 1, 1); h5 = g.n_top - 1
+    g.upsample(2); g.route([-1, p4]); csp(256, 1, False)
+    cbh(128, 1, 1); h4 = g.n_top - 1
+    g.upsample(2); g.route([-1, p3]); csp(128, 1, False); o3 = g.n_top - 1
+    cbh(128, 3, 2); g.route([-1, h4]); csp(256, 1, False); o4 = g.n_top - 1
+    cbh(256, 3, 2); g.route([-1, h5]); csp(512, 1, False); o5 = g.n_top - 1
+    yolos = []
+    for src, anchors in ((o3, [10, 13, 16, 30, 33, 23]), (o4, [30, 61, 62, 45, 59, 119]), (o5, [116, 90, 156, 198, 373, 326])):
+        g.route([src])
+        g.conv(255, 1, 1, 0, bn=0, act="none")
+        g.yolo(anchors, yolo_type="yolov5"); yolos.append(g.n_top - 1)
+    g.yoloout(yolos, conf, nms, "yolov5")
+    return g
+
+
 ARCHS = {"resnet18": resnet18, "resnet50": resnet50, "mobilenetv2": mobilenetv2,
-         "yolov3": yolov3, "yolov4": yolov4}
+         "yolov3": yolov3, "yolov4": yolov4, "yolov3_tiny": yolov3_tiny, "yolov5s": yolov5s}
 
 # The benchmark configurations: (architecture, compute dtype, batch, input size)
 CONFIGS = [

@@ -55,13 +55,14 @@ def sort_boxes(b):
     return b[np.lexsort(key.T[::-1])]
 
 
-def yolo_layer_err(got, ref, logits, channels_per_anchor, ratio):
+def yolo_layer_err(got, ref, logits, channels_per_anchor, ratio, version=3):
     """Error of a decoded yolo layer [3*per, H*W] in units of the logit error that explains it.
 
     Every decoded value is a function of one logit t: (sigmoid(t)+cell)*ratio, anchor*exp(t) or sigmoid(t).  A logit
     error d (itself bounded relative to max|t|) shows up as at most d/4 in a sigmoid plane and as a factor e^d in a
     w,h plane, however small d/|t| is.  So: sigmoid planes -> absolute error (x,y divided by ratio), w,h planes ->
-    |log got - log ref|, all divided by max(1, max|t|)."""
+    |log got - log ref|, all divided by max(1, max|t|).  yolov5 (version 5) decodes with 2*sigmoid and (2*sigmoid)^2: its
+    x,y and w,h errors are twice as sensitive, and a squared sigmoid underflows gradually instead of overflowing."""
     per = channels_per_anchor
     got = np.asarray(got, np.float64).reshape(3, per, -1)
     ref = np.asarray(ref, np.float64).reshape(3, per, -1)
@@ -70,6 +71,14 @@ def yolo_layer_err(got, ref, logits, channels_per_anchor, ratio):
     e_sig = np.abs(got[:, 4:] - ref[:, 4:]).max()
     g, r = got[:, 2:4].ravel(), ref[:, 2:4].ravel()
     fin = np.isfinite(r) & (r != 0)
-    assert (np.isfinite(g) == np.isfinite(r)).all() and ((g == 0) == (r == 0)).all(), "inf / underflow pattern differs"
+    if version == 5:
+        tiny = 1e-30                      # (2*sigmoid)^2 below this is in or next to the subnormal range: only require both to be tiny
+        assert np.isfinite(g).all() and np.isfinite(r).all() and (np.abs(g[np.abs(r) < tiny]) < 1e-25).all() and (np.abs(r[np.abs(g) < tiny]) < 1e-25).all()
+        fin = (np.abs(r) >= tiny) & (np.abs(g) >= tiny)
+        e_xy /= 2.0
+    else:
+        assert (np.isfinite(g) == np.isfinite(r)).all() and ((g == 0) == (r == 0)).all(), "inf / underflow pattern differs"
     e_wh = float(np.abs(np.log(np.abs(g[fin])) - np.log(np.abs(r[fin]))).max()) if fin.any() else 0.0
+    if version == 5:
+        e_wh /= 2.0
     return float(max(e_xy, e_sig, e_wh) / scale)

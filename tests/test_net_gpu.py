@@ -36,7 +36,8 @@ def _oracle_layers(arch, size, binp, imgs, **kw):
     return outs, boxes
 
 
-SMALL = [("resnet18", 64, 2), ("resnet50", 64, 2), ("mobilenetv2", 64, 3), ("yolov3", 64, 2), ("yolov4", 64, 2)]
+SMALL = [("resnet18", 64, 2), ("resnet50", 64, 2), ("mobilenetv2", 64, 3), ("yolov3", 64, 2), ("yolov4", 64, 2), ("yolov3_tiny", 96, 2),
+         ("yolov5s", 64, 2)]
 
 
 @pytest.mark.parametrize("arch,size,batch", SMALL)
@@ -63,7 +64,8 @@ def test_fp32_every_layer(arch, size, batch):
         is_yolo = m.layer_info(i)["type"] == "yolo"
         lt = tol
         for b in range(batch):
-            e = nu.yolo_layer_err(got[b], ref[b][i], ref[b][i - 1], 85, size / m.layer_info(i)['outH']) if is_yolo else nu.rel_err(got[b], ref[b][i])
+            e = (nu.yolo_layer_err(got[b], ref[b][i], ref[b][i - 1], 85, size / m.layer_info(i)['outH'], 5 if arch == "yolov5s" else 3)
+                 if is_yolo else nu.rel_err(got[b], ref[b][i]))
             worst = max(worst, e)
             assert e <= lt, f"{arch} layer {i} ({m.layer_info(i)['type']}) image {b}: {e}"
     print(arch, "worst layer error", worst)

@@ -92,7 +92,7 @@ def test_oracle_matches_reference_golden_nets(arch, tmp_path):
 
 
 @pytest.mark.skipif(not refshim.available(), reason="oracle/_ref is not built here")
-@pytest.mark.parametrize("arch,size", [("resnet18", 224), ("mobilenetv2", 224), ("yolov3", 64), ("yolov4", 64)])
+@pytest.mark.parametrize("arch,size", [("resnet18", 224), ("mobilenetv2", 224), ("yolov3", 64), ("yolov4", 64), ("yolov3_tiny", 96), ("yolov5s", 64)])
 def test_oracle_matches_reference_live(arch, size, tmp_path):
     netp, binp, gw = zoo.write_model(arch, str(tmp_path), 1, size, seed=21)
     x = zoo.seeded_input(1, 3, size, size, 22)[0]
@@ -106,7 +106,7 @@ def test_oracle_matches_reference_live(arch, size, tmp_path):
         if not a.size:
             continue
         if infos[i]["type"] == "yolo":      # decoded values amplify the logit error, see netutil.yolo_layer_err
-            assert nu.yolo_layer_err(b.ravel(), a, ro[i - 1], 85, size / infos[i]["outH"]) <= tol, (arch, i)
+            assert nu.yolo_layer_err(b.ravel(), a, ro[i - 1], 85, size / infos[i]["outH"], 5 if arch == "yolov5s" else 3) <= tol, (arch, i)
         else:
             assert nu.rel_err(b.ravel(), a) <= tol, (arch, i)
     if arch.startswith("yolo"):
