@@ -200,6 +200,14 @@ int msnh_hip_upsample_bilinear(int dtype, int batch, int in_h, int in_w, int c, 
  * x_mul undoes the input's power-of-two storage scale. */
 int msnh_hip_softmax(int dtype, int batch, int pixels, int c, const void *x, int x_ld, float x_mul, float temperature, void *y,
                      int y_ld, float y_mul, msnh_stream_t s);
+/* Second half of a transposed convolution (the first half is a 1x1 msnh_hip_conv2d with ksize*ksize*c output channels,
+ * channel = (ky*ksize + kx)*c + oc, weights W1[that channel][ic] = W[ic][oc][ky][kx]): output pixel (oy, ox) sums the taps whose
+ * source pixel ((oy + pad - ky)/stride, (ox + pad - kx)/stride) exists, then y = out_mul * act(cols_mul * sum + bias)
+ * (Gemm::cpuCol2Im, src/core/MsnhGemm.cpp:115-154; DeConvolutionalLayer::forward, src/layers/MsnhDeConvolutionalLayer.cpp:140-200).
+ * out_h = (in_h - 1)*stride - 2*pad + ksize. */
+int msnh_hip_deconv_col2im(int dtype, int batch, int in_h, int in_w, int c, int ksize, int stride, int pad, const void *cols, int cols_ld,
+                           float cols_mul, const float *bias, int act, float act_param, int out_h, int out_w, float out_mul, void *y,
+                           int y_ld, msnh_stream_t s);
 /* Fully connected layer out[b][o] = act( sum_i x[b][i]*w[o][i] + bias[o] ) (cublasSgemm NT + bias,
  * src/layers/MsnhConnectedLayer.cpp:300-360).  x: [batch][inputs] d-type; w: [outputs][inputs] dtype;
  * y: float32 [batch][outputs].  x_mul undoes the input's power-of-two storage scale. */

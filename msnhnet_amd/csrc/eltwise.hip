@@ -321,6 +321,48 @@ __global__ __launch_bounds__(256) void softmaxKernel(const T *__restrict__ x, in
     }
 }
 
+// ---- transposed convolution, second half: gather of the per-tap products ------------------------------------------
+// cols[b][y][x][(ky*k + kx)*C + c] holds, for input pixel (y, x), the product of the input vector with the weights of tap
+// (ky, kx) (a 1x1 convolution with k*k*C outputs).  Output pixel (oy, ox) sums the taps whose source pixel
+// ((oy + pad - ky) / stride, (ox + pad - kx) / stride) exists, in (ky, kx) order -- the order in which
+// Gemm::cpuCol2Im accumulates them (src/core/MsnhGemm.cpp:115-154) -- then bias and activation
+// (DeConvolutionalLayer::forward, src/layers/MsnhDeConvolutionalLayer.cpp:140-200).
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void col2imKernel(const T *__restrict__ cols, int colsLd, float colsMul, int H, int W, int c, int ksize, int stride,
+                                                    int pad, int OH, int OW, const float *__restrict__ bias, int act, float actParam, float outMul,
+                                                    T *__restrict__ y, int yLd, long long total)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int cv = c / VEC;
+    const int c0 = static_cast<int>(idx % cv) * VEC;
+    const long long p = idx / cv;
+    const int ox = static_cast<int>(p % OW);
+    const long long t = p / OW;
+    const int oy = static_cast<int>(t % OH);
+    const long long b = t / OH;
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+    for (int ky = 0; ky < ksize; ++ky)
+    {
+        const int ny = oy + pad - ky;
+        if (ny < 0 || ny % stride != 0 || ny / stride >= H) continue;
+        for (int kx = 0; kx < ksize; ++kx)
+        {
+            const int nx = ox + pad - kx;
+            if (nx < 0 || nx % stride != 0 || nx / stride >= W) continue;
+            float v[VEC];
+            loadVec<T, VEC>(cols + ((b * H + ny / stride) * W + nx / stride) * colsLd + (ky * ksize + kx) * c + c0, v);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] += v[i];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = outMul * activate(colsMul * acc[i] + (bias ? bias[c0 + i] : 0.f), act, actParam);
+    storeVec<T, VEC>(y + p * yLd + c0, acc);
+}
+
 // ---- fully connected: one wavefront per (batch row, output), wave-level reduction -------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void connectedKernel(const T *__restrict__ x, float xMul, const T *__restrict__ w,
@@ -619,6 +661,29 @@ int msnh_hip_softmax(int dtype, int batch, int pixels, int c, const void *x, int
     else
         hipLaunchKernelGGL((softmaxKernel<float>), dim3(batch), dim3(256), 0, st, static_cast<const float *>(x), x_ld, x_mul, pixels, c, temperature,
                            static_cast<float *>(y), y_ld, y_mul);
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+int msnh_hip_deconv_col2im(int dtype, int batch, int in_h, int in_w, int c, int ksize, int stride, int pad, const void *cols, int cols_ld,
+                           float cols_mul, const float *bias, int act, float act_param, int out_h, int out_w, float out_mul, void *y,
+                           int y_ld, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "deconv_col2im: bad dtype");
+    MSNH_REQUIRE(batch > 0 && in_h > 0 && in_w > 0 && c > 0 && ksize > 0 && stride > 0 && pad >= 0 && actOk(act), "deconv_col2im: bad geometry");
+    MSNH_REQUIRE(out_h == (in_h - 1) * stride - 2 * pad + ksize && out_w == (in_w - 1) * stride - 2 * pad + ksize && out_h > 0 && out_w > 0,
+                 "deconv_col2im: out size does not match geometry");
+    MSNH_REQUIRE(cols && y && cols_ld >= ksize * ksize * c && y_ld >= c, "deconv_col2im: bad argument");
+    hipStream_t st = resolveStream(s);
+    const int vec = pickVec(dtype, c, {cols_ld, y_ld}, {cols, y});
+    const long long total = static_cast<long long>(batch) * out_h * out_w * (c / vec);
+    dim3 grid(gridFor(total, 256));
+#define MSNH_C2I(T, V)                                                                                                 \
+    hipLaunchKernelGGL((col2imKernel<T, V>), grid, dim3(256), 0, st, static_cast<const T *>(cols), cols_ld, cols_mul, in_h, in_w, c, ksize, stride, \
+                       pad, out_h, out_w, bias, act, act_param, out_mul, static_cast<T *>(y), y_ld, total)
+    if (dtype == MSNH_F16) { if (vec == 8) MSNH_C2I(f16, 8); else MSNH_C2I(f16, 1); }
+    else { if (vec == 4) MSNH_C2I(float, 4); else MSNH_C2I(float, 1); }
+#undef MSNH_C2I
     MSNH_LAUNCH_CHECK();
     return 0;
 }

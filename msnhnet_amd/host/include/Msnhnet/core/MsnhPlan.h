@@ -48,7 +48,7 @@ struct PlanTensor
 
 struct PlanOp
 {
-    enum Kind { CONV = 0, AFFINE, ADD, COPY, MAXPOOL, AVGPOOL, UPSAMPLE, CONNECTED, INPUT_CAST, YOLO_DECODE, PAD, SLICE, BILINEAR, SOFTMAX };
+    enum Kind { CONV = 0, AFFINE, ADD, COPY, MAXPOOL, AVGPOOL, UPSAMPLE, CONNECTED, INPUT_CAST, YOLO_DECODE, PAD, SLICE, BILINEAR, SOFTMAX, COL2IM };
     Kind kind = CONV;
     int  in0 = -1, in1 = -1, out = -1;
     bool dead = false;

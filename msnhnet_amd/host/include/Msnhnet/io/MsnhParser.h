@@ -55,6 +55,18 @@ public:
     float bnEps = 0.00001f;
 };
 
+class MsnhNet_API DeConvParams : public BaseParams
+{
+public:
+    explicit DeConvParams(bool inc) : BaseParams(inc) { type = LayerType::DECONVOLUTIONAL; }
+    int filters = 1, groups = 1, useBias = 1;
+    int kSize = 1, kSizeX = -1, kSizeY = -1;
+    int stride = 1, strideX = -1, strideY = -1;
+    int padding = 0, paddingX = -1, paddingY = -1;
+    ActivationType activation = ActivationType::NONE;
+    std::vector<float> actParams;
+};
+
 class MsnhNet_API MaxPoolParams : public BaseParams
 {
 public:

@@ -132,6 +132,29 @@ private:
     int _alignCorners;
 };
 
+// Transposed convolution (src/layers/MsnhDeConvolutionalLayer.cpp:4-70 ctor, :140-200 forward), groups == 1, square geometry.
+// Lowered to a 1x1 convolution with kSize^2 * filters output channels (the reference's transposed GEMM) and a gather of the
+// taps (its col2im) that also adds the bias and applies the activation.
+class MsnhNet_API DeConvolutionalLayer : public BaseLayer
+{
+public:
+    DeConvolutionalLayer(const int &batch, const int &height, const int &width, const int &channel, const int &num, const int &kSizeX,
+                         const int &kSizeY, const int &strideX, const int &strideY, const int &paddingX, const int &paddingY, const int &groups,
+                         const ActivationType &activation, const std::vector<float> &actParams, const int &useBias);
+    ~DeConvolutionalLayer() override;
+    int deConvOutHeight() const { return (_height - 1) * _strideY - 2 * _paddingY + _kSizeY; }
+    int deConvOutWidth() const { return (_width - 1) * _strideX - 2 * _paddingX + _kSizeX; }
+    void loadAllWeigths(std::vector<float> &weights) override;
+    int lower(Plan &plan, int in, int layerIndex) override;
+    void foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const override;      // the bias, for the gather launch
+
+private:
+    int _kSizeX, _kSizeY, _strideX, _strideY, _paddingX, _paddingY, _useBias;
+    int _nWeights = 0, _nBiases = 0;
+    std::vector<float> _biases;
+    BaseLayer *_gemm = nullptr;            // owner of the rearranged [k*k*filters][channel] weights of the 1x1 convolution
+};
+
 // src/layers/MsnhGlobalAvgPoolLayer.cpp:5-30, 152-168: mean of every channel plane
 class MsnhNet_API GlobalAvgPoolLayer : public BaseLayer
 {

@@ -451,6 +451,88 @@ int UpSampleLayer::lower(Plan &plan, int in, int layerIndex)
     return out;
 }
 
+// ---- DeConvolutionalLayer -----------------------------------------------------------------------------------------------
+namespace
+{
+// weights of the 1x1 convolution a transposed convolution lowers to; no affine of its own
+class DeconvGemmWeights : public BaseLayer
+{
+public:
+    std::vector<float> w;
+    const std::vector<float> &kernelWeights() const override { return w; }
+    void foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const override { scale.clear(); shift.clear(); }
+};
+}
+
+DeConvolutionalLayer::DeConvolutionalLayer(const int &batch, const int &height, const int &width, const int &channel, const int &num, const int &kSizeX,
+                                           const int &kSizeY, const int &strideX, const int &strideY, const int &paddingX, const int &paddingY,
+                                           const int &groups, const ActivationType &activation, const std::vector<float> &actParams, const int &useBias)
+    : _kSizeX(kSizeX), _kSizeY(kSizeY), _strideX(strideX), _strideY(strideY), _paddingX(paddingX), _paddingY(paddingY), _useBias(useBias)
+{
+    requireDeviceActivation(activation, "deconv");
+    if (groups > 1) MSNH_THROW("deconv: groups are outside the convolutional path this build implements");
+    if (kSizeX != kSizeY || strideX != strideY || paddingX != paddingY) MSNH_THROW("deconv: only square kernels, strides and paddings are supported");
+    if (kSizeX <= 0 || strideX <= 0 || paddingX < 0 || num <= 0) MSNH_THROW("deconv: bad geometry");
+    _type = LayerType::DECONVOLUTIONAL;
+    _layerName = "DeConv          ";
+    _batch = batch; _height = height; _width = width; _channel = channel; _num = num;
+    _activation = activation; _actParams = actParams;
+    _outHeight = deConvOutHeight(); _outWidth = deConvOutWidth(); _outChannel = num;
+    if (_outHeight <= 0 || _outWidth <= 0) MSNH_THROW("deconv: non-positive output size");
+    _outputNum = _outWidth * _outHeight * _outChannel;
+    _inputNum = width * width * channel;                                 // (sic, src/layers/MsnhDeConvolutionalLayer.cpp:46)
+    _nWeights = channel * num * kSizeX * kSizeY;
+    _nBiases = useBias ? num : 0;
+    _numWeights = static_cast<size_t>(_nWeights + _nBiases);
+    _maxOutputNum = static_cast<size_t>(_batch) * _outputNum;
+    _layerDetail = fmt("Deconvolutional Layer: %d x %d x %d image, %d filters -> %d x %d x %d image\n", _height, _width, _channel, _num, _outHeight,
+                       _outWidth, _num);
+    _gemm = new DeconvGemmWeights();
+}
+
+DeConvolutionalLayer::~DeConvolutionalLayer() { delete _gemm; }
+
+void DeConvolutionalLayer::loadAllWeigths(std::vector<float> &weights)
+{
+    if (weights.size() != _numWeights)
+        MSNH_THROW("Deconv weights load err. needed : " + std::to_string(_numWeights) + " given : " + std::to_string(weights.size()));
+    if (BaseLayer::isPreviewMode) return;
+    // file order [channel][filters][ky][kx] -> rows of the 1x1 convolution [(ky*k + kx)*filters + oc][channel]
+    const int kk = _kSizeX * _kSizeY;
+    std::vector<float> &w = static_cast<DeconvGemmWeights *>(_gemm)->w;
+    w.assign(static_cast<size_t>(_nWeights), 0.f);
+    for (int ic = 0; ic < _channel; ++ic)
+        for (int oc = 0; oc < _num; ++oc)
+            for (int t = 0; t < kk; ++t)
+                w[(static_cast<size_t>(t) * _num + oc) * _channel + ic] = weights[(static_cast<size_t>(ic) * _num + oc) * kk + t];
+    if (_useBias) _biases.assign(weights.begin() + _nWeights, weights.end());
+    _weightsLoaded = true;
+}
+
+void DeConvolutionalLayer::foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const
+{
+    scale.clear();
+    shift = _biases;
+}
+
+int DeConvolutionalLayer::lower(Plan &plan, int in, int layerIndex)
+{
+    in = plan.nhwcOf(in, layerIndex);
+    const PlanTensor ti = plan.tensors[static_cast<size_t>(in)];
+    if (ti.layout != PlanTensor::NHWC) MSNH_THROW("Layer before deconvolutional layer must output image");
+    const int kk = _kSizeX * _kSizeY;
+    const int cols = plan.addTensor(ti.n, ti.h, ti.w, kk * _num, ti.dtype, "deconv_cols");
+    PlanOp &gemm = plan.addOp(PlanOp::CONV, in, -1, cols, layerIndex, "deconv_gemm");
+    gemm.ksize = 1; gemm.stride = 1; gemm.pad = 0; gemm.dilation = 1; gemm.groups = 1;
+    gemm.src = _gemm;
+    const int out = plan.addTensor(ti.n, _outHeight, _outWidth, _num, ti.dtype, "deconv_out");
+    PlanOp &op = plan.addOp(PlanOp::COL2IM, cols, -1, out, layerIndex, "deconv_col2im");
+    op.ksize = _kSizeX; op.stride = _strideX; op.pad = _paddingX;
+    op.act = _activation; op.actParam = actParam();
+    op.src = this;
+    return out;
+}
+
 GlobalAvgPoolLayer::GlobalAvgPoolLayer(const int &batch, const int &height, const int &width, const int &channel)
 {
     _type = LayerType::GLOBAL_AVGPOOL;

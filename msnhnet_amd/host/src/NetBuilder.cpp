@@ -189,6 +189,14 @@ void NetBuilder::buildNetFromMsnhNet(const std::string &path)
             layer = r;
             break;
         }
+        case LayerType::DECONVOLUTIONAL:
+        {
+            if (params.height == 0 || params.width == 0 || params.channels == 0) MSNH_THROW("Layer before deconvolutional layer must output image");
+            DeConvParams *p = static_cast<DeConvParams *>(bp);
+            layer = new DeConvolutionalLayer(params.batch, params.height, params.width, params.channels, p->filters, p->kSizeX, p->kSizeY, p->strideX,
+                                             p->strideY, p->paddingX, p->paddingY, p->groups, p->activation, p->actParams, p->useBias);
+            break;
+        }
         case LayerType::GLOBAL_AVGPOOL:
             layer = new GlobalAvgPoolLayer(params.batch, params.height, params.width, params.channels);
             break;
@@ -284,7 +292,7 @@ void NetBuilder::loadWeightsFromVector(const std::vector<float> &all)
     for (BaseLayer *l : _net->layers)
     {
         const LayerType t = l->type();
-        const bool has = t == CONVOLUTIONAL || t == CONNECTED || t == BATCHNORM || t == RES_BLOCK || t == RES_2_BLOCK || t == ADD_BLOCK || t == CONCAT_BLOCK;
+        const bool has = t == CONVOLUTIONAL || t == DECONVOLUTIONAL || t == CONNECTED || t == BATCHNORM || t == RES_BLOCK || t == RES_2_BLOCK || t == ADD_BLOCK || t == CONCAT_BLOCK;
         if (!has) continue;
         const size_t n = l->getNumWeights();
         if (ptr + n > all.size())
@@ -728,7 +736,7 @@ std::string NetBuilder::profileEachOp(int reps)
 {
     if (!_planReady) MSNH_THROW("weights are not loaded");
     Plan &plan = *_net->plan;
-    static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode", "pad", "slice", "bilinear", "softmax"};
+    static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode", "pad", "slice", "bilinear", "softmax", "col2im"};
     static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk"};
     msnh_event_t e0 = nullptr, e1 = nullptr;
     MSNH_DEV(msnh_hip_event_create(&e0));

@@ -327,6 +327,31 @@ BaseParams *Parser::parseNode(const MsnhNode &node, bool top, const NetConfigPar
         if (p->kSizeY == 1 && p->dilationY > 1) p->dilationY = 1;
         return p.release();
     }
+    if (k == "deconv")
+    {
+        std::unique_ptr<DeConvParams> p(new DeConvParams(top));
+        for (const MsnhNode &n : node.children)
+        {
+            if (n.key == "filters") toInt(n, "deconv", p->filters);
+            else if (n.key == "kSize") toInt(n, "deconv", p->kSize);
+            else if (n.key == "kSizeX") toInt(n, "deconv", p->kSizeX);
+            else if (n.key == "kSizeY") toInt(n, "deconv", p->kSizeY);
+            else if (n.key == "stride") toInt(n, "deconv", p->stride);
+            else if (n.key == "strideX") toInt(n, "deconv", p->strideX);
+            else if (n.key == "strideY") toInt(n, "deconv", p->strideY);
+            else if (n.key == "padding") toInt(n, "deconv", p->padding);
+            else if (n.key == "paddingX") toInt(n, "deconv", p->paddingX);
+            else if (n.key == "paddingY") toInt(n, "deconv", p->paddingY);
+            else if (n.key == "useBias") toInt(n, "deconv", p->useBias);
+            else if (n.key == "groups") toInt(n, "deconv", p->groups);
+            else if (n.key == "activation") toActivation(n, p->activation, p->actParams);
+            else unsupportedKey(n, "deconv");
+        }
+        spread(p->stride, p->strideX, p->strideY);
+        spread(p->kSize, p->kSizeX, p->kSizeY);
+        spread(p->padding, p->paddingX, p->paddingY);
+        return p.release();
+    }
     if (k == "batchnorm")
     {
         std::unique_ptr<BatchNormParams> p(new BatchNormParams(top));

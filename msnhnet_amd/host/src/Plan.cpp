@@ -411,6 +411,12 @@ void Plan::prepareWeights()
             if (!shift.empty()) op.shiftDev.upload(shift.data(), shift.size() * sizeof(float));
             op.flops = 2.0 * d.batch * d.out_c * d.out_h * d.out_w * (d.in_c / d.groups) * d.ksize * d.ksize;
         }
+        else if (op.kind == PlanOp::COL2IM)
+        {
+            std::vector<float> scale, shift;
+            op.src->foldedAffine(scale, shift);
+            if (!shift.empty()) op.shiftDev.upload(shift.data(), shift.size() * sizeof(float));
+        }
         else if (op.kind == PlanOp::AFFINE)
         {
             std::vector<float> scale, shift;
@@ -598,6 +604,11 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
         MSNH_DEV(msnh_hip_slice(in.dtype, in.n, in.h, in.w, ptr(op.in0), ld(op.in0), op.slice[0], op.slice[1], op.slice[2], op.slice[3], op.slice[4],
                                 op.slice[5], out.c, out.h, out.w, mulOf(op.in0) / mulOf(op.out), ptr(op.out), ld(op.out), s));
         break;
+    case PlanOp::COL2IM:
+        MSNH_DEV(msnh_hip_deconv_col2im(in.dtype, in.n, in.h, in.w, out.c, op.ksize, op.stride, op.pad, ptr(op.in0), ld(op.in0), mulOf(op.in0),
+                                        op.shiftDev.as<float>(), static_cast<int>(op.act), op.actParam, out.h, out.w, 1.f / mulOf(op.out), ptr(op.out),
+                                        ld(op.out), s));
+        break;
     case PlanOp::SOFTMAX:
         MSNH_DEV(msnh_hip_softmax(in.dtype, in.n, in.h * in.w, in.c, ptr(op.in0), in.layout == PlanTensor::FLAT ? in.c : ld(op.in0), mulOf(op.in0),
                                   op.upScale, ptr(op.out), out.layout == PlanTensor::FLAT ? out.c : ld(op.out), 1.f / mulOf(op.out), s));
@@ -660,7 +671,7 @@ void Plan::exportTensor(int t, std::vector<float> &dst, msnh_stream_t s)
 
 std::string Plan::describe() const
 {
-    static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode", "pad", "slice", "bilinear", "softmax"};
+    static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode", "pad", "slice", "bilinear", "softmax", "col2im"};
     static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk"};
     std::ostringstream os;
     os << "plan: " << liveOps() << " launches, " << tensors.size() << " tensors, arena " << _arena.bytes() / (1024.0 * 1024.0) << " MiB, dtype "

@@ -215,6 +215,24 @@ class GraphWriter:
         self._emit(f"  constVal: {const}")
         self._top_done()
 
+    def deconv(self, filters, k, stride, pad=0, bias=True, act="none"):
+        self._emit("deconv:")
+        self._emit(f"  filters: {filters}")
+        self._emit(f"  kSize: {k}")
+        self._emit(f"  stride: {stride}")
+        if pad:
+            self._emit(f"  padding: {pad}")
+        if not bias:
+            self._emit("  useBias: 0")
+        self._emit(f"  activation: {act}")
+        s = self.shape
+        self.slots.append(WeightSlot("conv_w", s.c * filters * k * k, s.c * k * k))
+        if bias:
+            self.slots.append(WeightSlot("bias", filters, s.c * k * k))
+        self.conv_flops += 2 * s.c * filters * k * k * s.h * s.w
+        self.shape = _Shape(filters, (s.h - 1) * stride - 2 * pad + k, (s.w - 1) * stride - 2 * pad + k)
+        self._top_done()
+
     def softmax(self, temperature: float = 1.0):
         self._emit("softmax:")
         self._emit("  groups: 1")

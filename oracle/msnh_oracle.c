@@ -404,6 +404,52 @@ void msnh_or_global_avgpool(const float *in, int batch, int channels, int hw, fl
         }
 }
 
+/* DeConvolutionalLayer::forward, groups == 1 (src/layers/MsnhDeConvolutionalLayer.cpp:140-200): per image
+ * col[m][n] = sum_ic W[ic][m] * in[ic][n]  (cpuGemm with A transposed; m = (oc*k + ky)*k + kx, n = pixel), then
+ * Gemm::cpuCol2Im (src/core/MsnhGemm.cpp:115-154) accumulates col into the zero-filled output, then bias, activation.
+ * weights: [channels][filters][k][k]. */
+void msnh_or_deconv(const float *in, int batch, int channels, int height, int width, const float *weights, int filters, int ksize,
+                    int stride, int pad, const float *bias, int act, float actParam, float *out)
+{
+    const int oh = (height - 1) * stride - 2 * pad + ksize, ow = (width - 1) * stride - 2 * pad + ksize;
+    const int m = ksize * ksize * filters, n = height * width;
+    float *col = (float *)malloc((size_t)m * n * sizeof(float));
+    for (int b = 0; b < batch; ++b)
+    {
+        const float *x = in + (size_t)b * channels * n;
+        float *y = out + (size_t)b * filters * oh * ow;
+        memset(y, 0, (size_t)filters * oh * ow * sizeof(float));
+#pragma omp parallel for schedule(static)
+        for (int i = 0; i < m; ++i)
+            for (int j = 0; j < n; ++j)
+            {
+                float sum = 0;
+                for (int k = 0; k < channels; ++k)
+                    sum += weights[(size_t)k * m + i] * x[(size_t)k * n + j];
+                col[(size_t)i * n + j] = sum;
+            }
+        for (int c = 0; c < m; ++c)
+        {
+            const int wOff = c % ksize, hOff = (c / ksize) % ksize, cIm = c / ksize / ksize;
+            for (int h = 0; h < height; ++h)
+                for (int w = 0; w < width; ++w)
+                {
+                    const int r = hOff + h * stride - pad, q = wOff + w * stride - pad;
+                    if (r < 0 || q < 0 || r >= oh || q >= ow) continue;
+                    y[q + (size_t)ow * (r + (size_t)oh * cIm)] += col[((size_t)c * height + h) * width + w];
+                }
+        }
+        for (int f = 0; f < filters; ++f)
+            for (int i = 0; i < oh * ow; ++i)
+            {
+                float v = y[(size_t)f * oh * ow + i];
+                if (bias) v += bias[f];
+                y[(size_t)f * oh * ow + i] = msnh_or_activate(v, act, actParam);
+            }
+    }
+    free(col);
+}
+
 /* Box::iou (include/Msnhnet/utils/MsnhTypes.h:104-140), including its +1 pixel convention. */
 float msnh_or_iou(const float *a, const float *b)
 {

@@ -51,6 +51,8 @@ void  msnh_or_pad(const float *in, int batch, int channels, int height, int widt
                   float value, float *out);
 void  msnh_or_slice(const float *in, int batch, int channels, int height, int width, int start0, int step0, int start1, int step1,
                     int start2, int step2, float *out);
+void  msnh_or_deconv(const float *in, int batch, int channels, int height, int width, const float *weights, int filters, int ksize,
+                     int stride, int pad, const float *bias, int act, float actParam, float *out);
 void  msnh_or_softmax(const float *in, int batch, int num, float temperature, float *out);
 void  msnh_or_global_avgpool(const float *in, int batch, int channels, int hw, float *out);
 void  msnh_or_bilinear(const float *in, int batch, int channels, int height, int width, int outH, int outW, int alignCorners,

@@ -44,6 +44,7 @@ def lib():
         L.msnh_or_slice.argtypes = [_fp, ci, ci, ci, ci, ci, ci, ci, ci, ci, ci, _fp]
         L.msnh_or_bilinear.argtypes = [_fp, ci, ci, ci, ci, ci, ci, ci, _fp]
         L.msnh_or_softmax.argtypes = [_fp, ci, ci, cf, _fp]
+        L.msnh_or_deconv.argtypes = [_fp, ci, ci, ci, ci, _fp, ci, ci, ci, ci, _fp, ci, cf, _fp]
         L.msnh_or_global_avgpool.argtypes = [_fp, ci, ci, ci, _fp]
         L.msnh_or_iou.argtypes = [_fp, _fp]
         L.msnh_or_iou.restype = cf
@@ -161,6 +162,18 @@ def slice_(x, start0, step0, start1, step1, start2, step2):
     ext = lambda n, st, sp: (n - st) // sp + (1 if (n - st) % sp else 0)
     out = np.empty((b, ext(c, start0, step0), ext(h, start1, step1), ext(w, start2, step2)), np.float32)
     lib().msnh_or_slice(_p(x), b, c, h, w, start0, step0, start1, step1, start2, step2, _p(out))
+    return out
+
+
+def deconv(x, w, filters, k, stride, pad, bias=None, act="none", act_param=0.1):
+    """w: [in_c][filters][k][k] flat"""
+    x = _f32(x)
+    b, c, h, wd = x.shape
+    oh, ow = (h - 1) * stride - 2 * pad + k, (wd - 1) * stride - 2 * pad + k
+    out = np.empty((b, filters, oh, ow), np.float32)
+    w = _f32(w)
+    bias = _f32(bias) if bias is not None else None
+    lib().msnh_or_deconv(_p(x), b, c, h, wd, _p(w), filters, k, stride, pad, _p(bias), ACT[act], act_param, _p(out))
     return out
 
 
@@ -334,6 +347,12 @@ class OracleNet:
                 sx = float(d.get("scaleX", d.get("scale", 1.0))); sy = float(d.get("scaleY", d.get("scale", 1.0)))
                 return bilinear(x, int(x.shape[2] * np.float32(sy)), int(x.shape[3] * np.float32(sx)), int(d.get("alignCorners", 0)))
             return upsample(x, int(d.get("stride", d.get("strideX", 1))), float(d.get("scale", d.get("scaleX", 1.0))))
+        if key == "deconv":
+            filters = int(d.get("filters", 1)); k = int(d.get("kSize", 1)); st = int(d.get("stride", 1)); p = int(d.get("padding", 0))
+            act, ap = _act(d)
+            w = self._take(x.shape[1] * filters * k * k)
+            bias = self._take(filters) if int(d.get("useBias", 1)) else None
+            return deconv(x, w, filters, k, st, p, bias, act, ap)
         if key == "softmax":
             if int(d.get("groups", 1)) != 1:
                 raise ValueError("softmax groups")

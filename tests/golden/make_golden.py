@@ -91,6 +91,10 @@ def micro_cases():
         "softmax_map": lambda: g(3, 5, 6, lambda q: (q.conv(2, 3, 1, 1, bn=0, act="none"), q.softmax(2.0))),
         "bilinear_x2": lambda: g(3, 5, 6, lambda q: (q.conv(6, 3, 1, 1, bn=0, act="none"), q.upsample_bilinear(2.0, 2.0, 0))),
         "bilinear_align": lambda: g(3, 6, 4, lambda q: (q.conv(6, 1, 1, 0, bn=0, act="none"), q.upsample_bilinear(2.5, 1.5, 1))),
+        "deconv_k2s2": lambda: g(6, 5, 7, lambda q: (q.conv(8, 3, 1, 1, bn=1, act="relu"), q.deconv(8, 2, 2, 0, act="relu"), q.batchnorm("none"),
+                                                     q.conv(8, 3, 2, 1, bn=0, act="none"), q.route([-1, 0], add_model=True))),
+        "deconv_k3s2p1": lambda: g(4, 6, 5, lambda q: (q.conv(8, 1, 1, 0, bn=0, act="none"), q.deconv(5, 3, 2, 1, act="leaky"))),
+        "deconv_k4s2p1_nobias": lambda: g(3, 4, 6, lambda q: (q.conv(16, 3, 1, 1, bn=0, act="relu"), q.deconv(8, 4, 2, 1, bias=False, act="none"))),
         "yolo5_head": lambda: g(8, 6, 6, lambda q: (q.conv(21, 1, 1, 0, bn=0, act="none"), q.yolo([10, 13, 16, 30, 33, 23], class_num=2, yolo_type="yolov5"),
                                                    q.yoloout([1], 0.3, 0.45, yolo_type="yolov5"))),
         "yolo_head": lambda: g(8, 6, 6, lambda q: (q.conv(21, 1, 1, 0, bn=0, act="none"), q.yolo([10, 13, 16, 30, 33, 23], class_num=2),

@@ -64,9 +64,8 @@ def test_graph_construction_matches_reference_tables(arch, dtype, batch, size, t
 
 
 SHIPPED = sorted(__import__("glob").glob("/root/reference/models/*/*.msnhnet"))
-# graphs this build refuses, with the reason: transposed convolution is not implemented; yolov3_spp.msnhnet uses node names
-# ("yolov3", "yolov3out") that the reference's own parser rejects too
-REFUSED = {"fcns.msnhnet": r"\[deconv\]", "yolov3_spp.msnhnet": r"\[yolov3\]"}
+# the one graph this build refuses: yolov3_spp.msnhnet uses node names ("yolov3", "yolov3out") that the reference's own parser rejects too
+REFUSED = {"yolov3_spp.msnhnet": r"\[yolov3\]"}
 
 
 @pytest.mark.skipif(not SHIPPED, reason="the reference's model files are not present")
@@ -124,7 +123,7 @@ CFG = "config:\n  batch: 1\n  width: 8\n  height: 8\n  channels: 3\n"
     (CFG + "conv:\n  filters: 4\nyoloout:\n  layers: 0\n", "yoloout layer error, not a yolo layer"),
     ("config:\n  batch: 1\n  width: 0\n  height: 8\n  channels: 3\nconv:\n  filters: 4\n", "net config params err, params = 0 or < 0"),
     (CFG + "conv:\n  filters: 4\n  kSize: 3\n  kSizeY: 5\n", "only square kernels"),
-    (CFG + "deconv:\n  filters: 4\n", "outside the convolutional path"),
+    (CFG + "deconv:\n  filters: 4\n  groups: 2\n", "outside the convolutional path"),
     (CFG + "conv:\n  filters: 4\nconcatblock:\n  size: 1\n  branch:\n    empty:\n", r"size is not supported in \[concatblock\]"),
     (CFG + "conv:\n  filters: 4\nresblock:\n  size: 1\n  upsample:\n    stride: 2\n", r"upsample is not supported by \[ResBlockLayer\]"),
     (CFG + "conv:\n  filters: 4\nres2block:\n  base:\n    conv:\n      filters: 6\n  branch:\n    conv:\n      filters: 8\n", "base's outputs size is not equal"),

@@ -192,6 +192,34 @@ def test_softmax(dtype, c, h, w, temp):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("c,oc,h,w,k,s,p,bias", [(16, 8, 5, 7, 2, 2, 0, True), (8, 5, 6, 5, 3, 2, 1, True), (16, 8, 4, 6, 4, 2, 1, False), (8, 16, 3, 3, 3, 1, 1, True)])
+def test_deconv(dtype, c, oc, h, w, k, s, p, bias):
+    """Transposed convolution = 1x1 convolution to k*k*oc channels + msnh_hip_deconv_col2im, against the oracle's GEMM + col2im."""
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(k * 10 + s)
+    x = _x(rng, (2, c, h, w), dtype)
+    wt = (rng.standard_normal((c, oc, k, k)) * 0.2).astype(np.float32)
+    b = (rng.standard_normal(oc) * 0.1).astype(np.float32) if bias else None
+    if dtype == abi.F16:
+        x, wt = gu.round_f16(x), gu.round_f16(wt)
+    ref = on.deconv(x, wt.ravel(), oc, k, s, p, b, "leaky", 0.1)
+    oh, ow = ref.shape[2:]
+    # first half: [k*k*oc][c] weights as a 1x1 convolution
+    w1 = np.ascontiguousarray(wt.transpose(2, 3, 1, 0).reshape(k * k * oc, c, 1, 1))
+    cols, _ = gu.conv2d(x, w1, dtype=dtype, algo="auto")                    # NCHW float32 [2][k*k*oc][h][w]
+    cd = gu.nhwc_dev(cols, dtype)
+    yd = torch.full((2, oh, ow, oc + 8), 3.0, dtype=gu.TORCH_DT[dtype]).cuda()
+    bd = gu.dev(b) if bias else None
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_deconv_col2im(dtype, 2, h, w, oc, k, s, p, gu.ptr(cd), k * k * oc, 1.0, gu.ptr(bd) if bias else None, abi.ACT["leaky"], 0.1,
+                                               oh, ow, 1.0, gu.ptr(yd), oc + 8, None))
+    gu.sync()
+    assert gu.rel_err(gu.nchw_host(yd, oc), ref) <= (1e-5 if dtype == abi.F32 else 4e-3)
+    assert (yd[..., oc:].float().cpu().numpy() == 3.0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_connected(dtype):
     import gpuutil as gu
     gu.init()
