@@ -297,8 +297,8 @@ __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[
 }
 
 // Register budget: two workgroups per CU (one wave of each per SIMD) so that one workgroup's barrier and epilogue
-// are covered by the other's MFMAs; smaller tiles get three or four.
-constexpr int igemmWavesPerSimd(int bm, int bn) { return bm * bn > 128 * 128 ? 2 : (bm * bn > 64 * 64 ? 3 : 4); }
+// are covered by the other's MFMAs; smaller tiles, which serve the short-K bandwidth-bound layers, get three to six.
+constexpr int igemmWavesPerSimd(int bm, int bn) { return bm * bn > 128 * 128 ? 2 : (bm * bn > 64 * 128 ? 3 : (bm * bn > 64 * 64 ? 4 : 6)); }
 
 // 16-byte-per-lane load from a buffer resource straight into LDS: the 64 lanes of the wave fill 1 KiB starting at
 // ldsAddr (lane l at ldsAddr + 16 * l); lanes whose voffset is out of range store zeros.  No VGPRs and no LDS store

@@ -14,6 +14,27 @@ constexpr int YOLO_CHUNK = 256 * 8;
 
 // The 5 + classes logistics per cell are what the kernel computes most of (logisticF: hardware exp2 and
 // reciprocal); box width and height keep expf.
+// One decoded value: m = index inside the cell's 5 + classes values, (px, py) = cell, a = anchor.
+template <bool V5>
+__device__ __forceinline__ float yoloDecodeOne(float v, int m, int px, int py, int a, const Anchors &an, float ratio)
+{
+    if (V5)
+    {
+        // yolov5: centre (2s - 0.5 + cell) * ratio, size anchor * (2s)^2, s = logistic (src/layers/MsnhYoloLayer.cpp:250-296)
+        const float s2 = 2.f * logisticF(v);
+        if (m == 0) return (s2 - 0.5f + static_cast<float>(px)) * ratio;
+        if (m == 1) return (s2 - 0.5f + static_cast<float>(py)) * ratio;
+        if (m == 2) return an.v[(2 * a) % 6] * (s2 * s2);
+        if (m == 3) return an.v[(2 * a + 1) % 6] * (s2 * s2);
+        return 0.5f * s2;
+    }
+    if (m == 0) return (logisticF(v) + static_cast<float>(px)) * ratio;
+    if (m == 1) return (logisticF(v) + static_cast<float>(py)) * ratio;
+    if (m == 2) return an.v[(2 * a) % 6] * expf(v);
+    if (m == 3) return an.v[(2 * a + 1) % 6] * expf(v);
+    return logisticF(v);
+}
+
 template <typename T, bool V5>
 __global__ __launch_bounds__(256) void yoloDecodeKernel(const T *__restrict__ x, int xLd, float xMul, Anchors an, float ratio,
                                                         float *__restrict__ decoded, long long decStride, float confThresh, int *__restrict__ candIdx,
@@ -43,22 +64,7 @@ __global__ __launch_bounds__(256) void yoloDecodeKernel(const T *__restrict__ x,
     {
         const bool live = idx < perImage;          // predicate, not an exit: the unrolled loads can then be issued together
         const float v = live ? xMul * toF(xb[static_cast<size_t>(p) * xLd + a * per + m]) : 0.f;
-        float r;
-        if (V5)
-        {
-            // yolov5: centre (2s - 0.5 + cell) * ratio, size anchor * (2s)^2, s = logistic (src/layers/MsnhYoloLayer.cpp:250-296)
-            const float s2 = 2.f * logisticF(v);
-            if (m == 0)      r = (s2 - 0.5f + static_cast<float>(px)) * ratio;
-            else if (m == 1) r = (s2 - 0.5f + static_cast<float>(py)) * ratio;
-            else if (m == 2) r = an.v[(2 * a) % 6] * (s2 * s2);
-            else if (m == 3) r = an.v[(2 * a + 1) % 6] * (s2 * s2);
-            else             r = 0.5f * s2;
-        }
-        else if (m == 0) r = (logisticF(v) + static_cast<float>(px)) * ratio;
-        else if (m == 1) r = (logisticF(v) + static_cast<float>(py)) * ratio;
-        else if (m == 2) r = an.v[(2 * a) % 6] * expf(v);
-        else if (m == 3) r = an.v[(2 * a + 1) % 6] * expf(v);
-        else             r = logisticF(v);
+        const float r = yoloDecodeOne<V5>(v, m, px, py, a, an, ratio);
         if (live) db[idx] = r;
         if (live && m == 4 && candIdx != nullptr && r > confThresh) found[atomicAdd(&nFound, 1)] = candBase + a * HW + p;
         idx += 256;
@@ -84,6 +90,53 @@ __global__ __launch_bounds__(256) void yoloDecodeKernel(const T *__restrict__ x,
     __syncthreads();
     for (int i = threadIdx.x; i < nFound; i += 256)
         if (base + i < candCap) candIdx[static_cast<size_t>(b) * candCap + base + i] = found[i];
+}
+
+// Objectness only: the candidate list of a head without materialising its decoded tensor.  One lane per cell
+// (anchor, pixel); same logistic and same threshold test as the full decode, so the list is identical.
+template <typename T>
+__global__ __launch_bounds__(256) void yoloScanKernel(const T *__restrict__ x, int xLd, float xMul, float confThresh, int *__restrict__ candIdx,
+                                                      int candCap, int candBase, int *__restrict__ candCnt, int HW, int per)
+{
+    __shared__ int found[256];
+    __shared__ int nFound, base;
+    const int b = blockIdx.y;
+    if (threadIdx.x == 0) nFound = 0;
+    __syncthreads();
+    const int cell = blockIdx.x * 256 + threadIdx.x;             // a * HW + p
+    if (cell < 3 * HW)
+    {
+        const int a = cell / HW, p = cell - a * HW;
+        const float v = xMul * toF(x[(static_cast<size_t>(b) * HW + p) * xLd + a * per + 4]);
+        if (logisticF(v) > confThresh) found[atomicAdd(&nFound, 1)] = candBase + cell;
+    }
+    __syncthreads();
+    if (nFound == 0) return;
+    if (threadIdx.x == 0) base = atomicAdd(candCnt + b, nFound);
+    __syncthreads();
+    if (static_cast<int>(threadIdx.x) < nFound && base + static_cast<int>(threadIdx.x) < candCap)
+        candIdx[static_cast<size_t>(b) * candCap + base + threadIdx.x] = found[threadIdx.x];
+}
+
+// Decodes the rows of the listed candidates that belong to this head into their places of the decoded buffer.
+template <typename T, bool V5>
+__global__ __launch_bounds__(128) void yoloRowsKernel(const T *__restrict__ x, int xLd, float xMul, Anchors an, float ratio,
+                                                      float *__restrict__ decoded, long long decStride, const int *__restrict__ candIdx, int candCap,
+                                                      int candBase, const int *__restrict__ candCnt, int W, int HW, int per)
+{
+    const int b = blockIdx.y;
+    int n = candCnt[b];
+    n = n < candCap ? n : candCap;
+    for (int k = blockIdx.x; k < n; k += gridDim.x)
+    {
+        const int cell = candIdx[static_cast<size_t>(b) * candCap + k] - candBase;
+        if (cell < 0 || cell >= 3 * HW) continue;                // another head's candidate
+        const int a = cell / HW, p = cell - a * HW;
+        const int py = p / W, px = p - py * W;
+        const T *xr = x + (static_cast<size_t>(b) * HW + p) * xLd + a * per;
+        float *dr = decoded + static_cast<size_t>(b) * decStride + static_cast<size_t>(cell) * per;
+        for (int m = threadIdx.x; m < per; m += 128) dr[m] = yoloDecodeOne<V5>(xMul * toF(xr[m]), m, px, py, a, an, ratio);
+    }
 }
 
 __global__ __launch_bounds__(256) void yoloGatherKernel(const float *__restrict__ decoded, long long decStride, const int *__restrict__ candIdx,
@@ -158,6 +211,39 @@ extern "C" int msnh_hip_yolo_decode(int dtype, int batch, int h, int w, int clas
     if (dtype == MSNH_F16) { if (yolo_version == 5) MSNH_YOLO(f16, true); else MSNH_YOLO(f16, false); }
     else { if (yolo_version == 5) MSNH_YOLO(float, true); else MSNH_YOLO(float, false); }
 #undef MSNH_YOLO
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int msnh_hip_yolo_decode_candidates(int dtype, int batch, int h, int w, int classes, const void *x, int x_ld, float x_mul,
+                                               const float *anchors6, float ratio, int yolo_version, float *decoded,
+                                               long long decoded_batch_stride, float conf_thresh, int *cand_idx, int cand_cap, int cand_base,
+                                               int *cand_cnt, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "yolo_decode_candidates: bad dtype");
+    MSNH_REQUIRE(batch > 0 && batch <= 65535 && h > 0 && w > 0 && classes > 0, "yolo_decode_candidates: bad geometry");
+    MSNH_REQUIRE(yolo_version == 3 || yolo_version == 4 || yolo_version == 5, "yolo_decode_candidates: yolo_version must be 3, 4 or 5");
+    const int per = 5 + classes;
+    MSNH_REQUIRE(x && decoded && anchors6 && cand_idx && cand_cnt && cand_cap > 0 && x_ld >= 3 * per, "yolo_decode_candidates: bad argument");
+    MSNH_REQUIRE(decoded_batch_stride >= static_cast<long long>(3) * h * w * per, "yolo_decode_candidates: decoded_batch_stride too small");
+    Anchors an;
+    for (int i = 0; i < 6; ++i) an.v[i] = anchors6[i];
+    hipStream_t st = resolveStream(s);
+    const int HW = h * w;
+    dim3 sgrid((3 * HW + 255) / 256, batch), rgrid(64, batch);
+#define MSNH_YC(T)                                                                                                      \
+    do {                                                                                                                \
+        hipLaunchKernelGGL((yoloScanKernel<T>), sgrid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, x_mul, conf_thresh, cand_idx, cand_cap,  \
+                           cand_base, cand_cnt, HW, per);                                                               \
+        if (yolo_version == 5)                                                                                          \
+            hipLaunchKernelGGL((yoloRowsKernel<T, true>), rgrid, dim3(128), 0, st, static_cast<const T *>(x), x_ld, x_mul, an, ratio, decoded,  \
+                               decoded_batch_stride, cand_idx, cand_cap, cand_base, cand_cnt, w, HW, per);              \
+        else                                                                                                            \
+            hipLaunchKernelGGL((yoloRowsKernel<T, false>), rgrid, dim3(128), 0, st, static_cast<const T *>(x), x_ld, x_mul, an, ratio, decoded, \
+                               decoded_batch_stride, cand_idx, cand_cap, cand_base, cand_cnt, w, HW, per);              \
+    } while (0)
+    if (dtype == MSNH_F16) MSNH_YC(f16); else MSNH_YC(float);
+#undef MSNH_YC
     MSNH_LAUNCH_CHECK();
     return 0;
 }

@@ -91,6 +91,7 @@ public:
     explicit Plan(int dtype) : computeDtype(dtype) {}
 
     int computeDtype;
+    bool sparseYolo = false;                // yolo heads decode only the rows of their candidates (nobody reads the full decoded tensors)
     bool preferWinograd = false;            // 3x3 stride-1 float16 convs take the Winograd path where the kernel accepts the shape
     std::vector<PlanTensor> tensors;
     std::vector<PlanOp>     ops;

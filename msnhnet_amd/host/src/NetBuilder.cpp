@@ -406,6 +406,7 @@ void NetBuilder::finalizePlan()
     plan->place();
     setupYoloBuffers(*plan, _net->batch);
     plan->preferWinograd = useWinograd && dtype == MSNH_F16;
+    plan->sparseYolo = !_saveLayerOutput;         // layer dumps read the whole decoded tensors
     plan->prepareWeights();
     if (autoTune) plan->tuneConvs(_stream);
 
@@ -748,8 +749,14 @@ std::string NetBuilder::profileEachOp(int reps)
         const PlanOp &op = plan.ops[i];
         if (op.dead) continue;
         plan.run(i, i + 1, _stream);
+        const bool yolo = op.kind == PlanOp::YOLO_DECODE && plan.yoloCandCnt.ptr();
         MSNH_DEV(msnh_hip_event_record(e0, _stream));
-        for (int r = 0; r < reps; ++r) plan.run(i, i + 1, _stream);
+        for (int r = 0; r < reps; ++r)
+        {
+            // (a head appends to the candidate list: start every repetition from an empty one, as a forward does)
+            if (yolo) MSNH_DEV(msnh_hip_fill_zero(plan.yoloCandCnt.ptr(), plan.yoloCandCnt.bytes(), _stream));
+            plan.run(i, i + 1, _stream);
+        }
         MSNH_DEV(msnh_hip_event_record(e1, _stream));
         MSNH_DEV(msnh_hip_event_sync(e1));
         float ms = 0.f;

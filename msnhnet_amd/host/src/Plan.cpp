@@ -638,9 +638,14 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
         const int per = 5 + op.classes;
         float *decoded = yoloDecoded.as<float>() + static_cast<size_t>(op.cellBase) * per;
         const bool cand = op.confThresh < 1.5f;
-        MSNH_DEV(msnh_hip_yolo_decode(in.dtype, in.n, in.h, in.w, op.classes, ptr(op.in0), ld(op.in0), mulOf(op.in0), op.anchors.data(), op.ratio,
-                                      op.yoloVersion, decoded, static_cast<long long>(yoloCells) * per, op.confThresh, cand ? yoloCandIdx.as<int>() : nullptr,
-                                      yoloCells, op.cellBase, cand ? yoloCandCnt.as<int>() : nullptr, s));
+        if (sparseYolo && cand)
+            MSNH_DEV(msnh_hip_yolo_decode_candidates(in.dtype, in.n, in.h, in.w, op.classes, ptr(op.in0), ld(op.in0), mulOf(op.in0), op.anchors.data(),
+                                                     op.ratio, op.yoloVersion, decoded, static_cast<long long>(yoloCells) * per, op.confThresh,
+                                                     yoloCandIdx.as<int>(), yoloCells, op.cellBase, yoloCandCnt.as<int>(), s));
+        else
+            MSNH_DEV(msnh_hip_yolo_decode(in.dtype, in.n, in.h, in.w, op.classes, ptr(op.in0), ld(op.in0), mulOf(op.in0), op.anchors.data(), op.ratio,
+                                          op.yoloVersion, decoded, static_cast<long long>(yoloCells) * per, op.confThresh,
+                                          cand ? yoloCandIdx.as<int>() : nullptr, yoloCells, op.cellBase, cand ? yoloCandCnt.as<int>() : nullptr, s));
         break;
     }
     }

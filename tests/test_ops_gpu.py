@@ -308,6 +308,24 @@ def test_yolo_decode(dtype, version):
         want = sorted(1000 + a * h * w + p for a in range(3) for p in range(h * w) if ref_shuf[b, a, p, 4] > 0.5)
         n = int(cc[b])
         assert sorted(ci[b, :n].cpu().numpy().tolist()) == want
+    # candidate-only decode: the same list, the candidates' rows bit for bit, every other row untouched
+    dd2 = torch.full((2, 3, h * w, per), -7.0, dtype=torch.float32).cuda()
+    ci3 = torch.full((2, cap), -1, dtype=torch.int32).cuda()
+    cc3 = torch.zeros(2, dtype=torch.int32).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_yolo_decode_candidates(dtype, 2, h, w, cls, gu.ptr(xd), 256, 1.0, anchors.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                                                        ratio, version, gu.ptr(dd2), 3 * h * w * per, 0.5, gu.ptr(ci3), cap, 1000, gu.ptr(cc3), None))
+    gu.sync()
+    out2 = dd2.cpu().numpy().reshape(2, 3 * h * w, per)
+    full = out.reshape(2, 3 * h * w, per)
+    for b in range(2):
+        n = int(cc3[b])
+        got = sorted(ci3[b, :n].cpu().numpy().tolist())
+        assert got == sorted(ci[b, :int(cc[b])].cpu().numpy().tolist())
+        rows_in = np.zeros(3 * h * w, bool)
+        rows_in[np.array(got, np.int64) - 1000] = True
+        assert np.array_equal(out2[b][rows_in], full[b][rows_in])
+        assert (out2[b][~rows_in] == -7.0).all()
     # candidate compaction: box, objectness, first-maximum class
     ci2 = (ci - 1000).clamp(min=0).contiguous()
     rows = torch.zeros((2, cap, 8), dtype=torch.float32).cuda()
