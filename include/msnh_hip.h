@@ -56,6 +56,9 @@ enum msnh_conv_algo
     MSNH_CONV_DEPTHWISE = 3,   /* groups == in_c == out_c, bandwidth-bound direct kernel */
     MSNH_CONV_WINOGRAD  = 4,   /* F(2x2,3x3): ksize 3, stride 1, dilation 1, groups 1 */
     MSNH_CONV_STEM      = 5,   /* in_c <= 4 first layer: reads NCHW float32 input directly (cast fused) */
+    MSNH_CONV_POINTWISE = 7,   /* 1x1 stride 1, float16, in_c and out_c <= 128 and multiples of 8: weights resident in LDS, pixels
+                                  straight from memory into MFMA fragments, no tiles (tile must be 0).  IGEMM weight packing.
+                                  Never chosen by AUTO. */
     MSNH_CONV_IGEMM_SPLITK = 6 /* IGEMM with the K loop cut into up to 8 slices on separate workgroups, float32 partial sums in
                                   the workspace summed in slice order (deterministic); for launches with few output tiles.
                                   Same weight packing as IGEMM.  Never chosen by AUTO. */

@@ -14,6 +14,9 @@ int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float
 int convIgemmWs(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
                 const void *residual, void *y, hipStream_t st, bool dryRun, void *splitWs, size_t splitWsBytes);
 size_t igemmSplitKWorkspaceBytes(const msnh_conv_desc *d);
+bool pointwiseOk(const msnh_conv_desc *d);
+int convPointwise(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift, const void *residual,
+                  void *y, hipStream_t st);
 int igemmTileCount();
 int convWinograd(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
                  const void *residual, void *y, void *ws, size_t wsBytes, hipStream_t st);
@@ -340,6 +343,7 @@ int msnh_hip_conv2d_tile_supported(const msnh_conv_desc *d, int tile)
 {
     if (!d || validate(d) || tile < 0 || tile > igemmTileCount()) return 0;
     msnh_conv_desc t = *d;
+    if (d->algo == MSNH_CONV_POINTWISE) return tile == 0 && pointwiseOk(d) ? 1 : 0;
     if (d->algo == MSNH_CONV_WINOGRAD)
     {
         // the tile applies to the 16 transformed-domain GEMMs
@@ -388,6 +392,7 @@ int msnh_hip_conv2d_pack_weights(const msnh_conv_desc *d, int algo, const float 
     case MSNH_CONV_DIRECT:
     case MSNH_CONV_IGEMM:
     case MSNH_CONV_IGEMM_SPLITK:
+    case MSNH_CONV_POINTWISE:
         for (int oc = 0; oc < d->out_c; ++oc)
             for (int ci = 0; ci < cinG; ++ci)
                 for (int t = 0; t < kk; ++t)
@@ -451,6 +456,8 @@ int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const
         MSNH_REQUIRE(igemmOk(d), "conv2d: IGEMM needs (in_c/groups) and in_ld to be multiples of %d", d->dtype == MSNH_F16 ? 8 : 4);
         MSNH_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0, "conv2d: IGEMM needs 16-byte aligned x and w");
         return convIgemmWs(d, x, w, scale, shift, residual, y, st, false, workspace, workspace_bytes);
+    case MSNH_CONV_POINTWISE:
+        return convPointwise(d, x, w, scale, shift, residual, y, st);
     case MSNH_CONV_WINOGRAD:
         MSNH_REQUIRE(winogradOk(d), "conv2d: shape not supported by the Winograd kernel");
         return convWinograd(d, x, w, scale, shift, residual, y, workspace, workspace_bytes, st);

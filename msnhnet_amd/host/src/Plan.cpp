@@ -517,6 +517,7 @@ void Plan::tuneConvs(msnh_stream_t s)
                 search(MSNH_CONV_IGEMM_SPLITK);
             }
         }
+        if (baseAlgo == MSNH_CONV_IGEMM && op.kind == PlanOp::CONV) search(MSNH_CONV_POINTWISE);      // (refused by the library unless the shape fits)
         op.algo = bestAlgo;
         op.tile = best;
         memo.emplace_back(key, bestAlgo * 1000 + best);
@@ -677,7 +678,7 @@ void Plan::exportTensor(int t, std::vector<float> &dst, msnh_stream_t s)
 std::string Plan::describe() const
 {
     static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode", "pad", "slice", "bilinear", "softmax", "col2im"};
-    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk"};
+    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk", "pointwise"};
     std::ostringstream os;
     os << "plan: " << liveOps() << " launches, " << tensors.size() << " tensors, arena " << _arena.bytes() / (1024.0 * 1024.0) << " MiB, dtype "
        << (computeDtype == MSNH_F16 ? "f16" : "f32") << "\n";

@@ -280,6 +280,44 @@ def test_conv_split_k_rejects():
     assert b"workspace" in L.msnh_hip_last_error()
 
 
+@pytest.mark.parametrize("b,c,h,w,oc", [(2, 64, 19, 17, 32), (1, 16, 30, 30, 96), (3, 24, 9, 11, 144 - 16), (2, 128, 13, 13, 64), (1, 96, 7, 7, 24),
+                                         (2, 32, 8, 8, 16), (1, 128, 20, 21, 128), (4, 8, 5, 5, 8), (1, 80, 12, 9, 40)])
+@pytest.mark.parametrize("with_res", [False, True])
+def test_conv_pointwise(b, c, h, w, oc, with_res):
+    """1x1 convolution with the weights resident in LDS and pixels loaded straight into MFMA fragments: every combination of
+    channel-block counts, ragged K (in_c % 16 == 8), partial last blocks (out_c % 32 != 0), pixel tails, full epilogue."""
+    import gpuutil as gu
+    rng = np.random.default_rng(b * 1000 + c + oc)
+    x, wt = _case(rng, b, c, h, w, oc, 1)
+    res = rng.standard_normal((b, oc, h, w), dtype=np.float32) if with_res else None
+    scale = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    shift = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    x, wt = gu.round_f16(x), gu.round_f16(wt)
+    if with_res:
+        res = gu.round_f16(res)
+    y, used = gu.conv2d(x, wt, dtype=abi.F16, scale=scale, shift=shift, act="leaky", residual=res, act2="relu6", res_mul=2.0, out_mul=0.5,
+                        algo="pointwise", in_ld=c + 8, out_ld=oc + 8, res_ld=oc + 16 if with_res else None)
+    assert used == "pointwise"
+    ref = _ref(x, wt, 1, 0, 1, 1, scale, shift, "leaky", 0.1, res, "relu6", 2.0, 0.5)
+    assert gu.rel_err(y, ref) <= TOL[abi.F16]
+    # without the affine
+    y, _ = gu.conv2d(x, wt, dtype=abi.F16, act="none", algo="pointwise")
+    assert gu.rel_err(y, _ref(x, wt, 1, 0, 1, 1, None, None, "none", 0.1, None, "none", 1.0, 1.0)) <= TOL[abi.F16]
+
+
+def test_conv_pointwise_rejects():
+    import ctypes
+    L = abi.lib()
+    mk = lambda **kw: abi.ConvDesc(**{**dict(dtype=abi.F16, out_dtype=abi.F16, batch=1, in_h=8, in_w=8, in_c=16, in_ld=16, out_c=16, out_h=8, out_w=8, out_ld=16,
+                                             ksize=1, stride=1, pad=0, dilation=1, groups=1, act=22, act_param=0.1, has_residual=0, res_ld=16, act2=22,
+                                             act2_param=0.1, res_mul=1.0, out_mul=1.0, algo=abi.ALGO["pointwise"], tile=0), **kw})
+    assert L.msnh_hip_conv2d_tile_supported(ctypes.byref(mk()), 0) == 1
+    assert L.msnh_hip_conv2d_tile_supported(ctypes.byref(mk()), 1) == 0
+    for bad in (dict(in_c=136, in_ld=136), dict(out_c=136, out_ld=136), dict(in_c=12, in_ld=16), dict(dtype=abi.F32, out_dtype=abi.F32),
+                dict(ksize=3, pad=1), dict(stride=2, out_h=4, out_w=4), dict(groups=2)):
+        assert L.msnh_hip_conv2d_tile_supported(ctypes.byref(mk(**bad)), 0) == 0, bad
+
+
 def test_conv_winograd_rejects():
     import ctypes
     import gpuutil as gu
