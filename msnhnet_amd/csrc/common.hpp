@@ -101,6 +101,45 @@ __device__ __forceinline__ float activate(float x, int act, float param)
     }
 }
 
+// The same over a register array with the choice of the activation made once, outside the element loop: a kernel that
+// calls activate() per element of an unrolled epilogue carries one copy of the whole switch per element.
+template <int N> __device__ __forceinline__ void activateArray(float (&v)[N], int act, float param)
+{
+    switch (act)
+    {
+    case MSNH_ACT_NONE: break;
+    case MSNH_ACT_RELU:
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = v[i] > 0.f ? v[i] : 0.f * v[i];
+        break;
+    case MSNH_ACT_LEAKY:
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = v[i] > 0.f ? v[i] : param * v[i];
+        break;
+    case MSNH_ACT_RELU6:
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = activate(v[i], MSNH_ACT_RELU6, param);
+        break;
+    case MSNH_ACT_LOGISTIC:
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = logisticF(v[i]);
+        break;
+    case MSNH_ACT_SWISH:
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = v[i] * logisticF(v[i]);
+        break;
+    case MSNH_ACT_HARD_SWISH:
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = activate(v[i], MSNH_ACT_HARD_SWISH, param);
+        break;
+    case MSNH_ACT_MISH:
+#pragma unroll
+        for (int i = 0; i < N; ++i) v[i] = mishF(v[i]);
+        break;
+    default: break;
+    }
+}
+
 inline bool actOk(int act)
 {
     return act == MSNH_ACT_LOGISTIC || act == MSNH_ACT_RELU || act == MSNH_ACT_RELU6 || act == MSNH_ACT_LEAKY ||

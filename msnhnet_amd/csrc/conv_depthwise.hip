@@ -1,5 +1,5 @@
 // Depthwise 3x3 convolution (groups == channels), float16 NHWC, stride 1 or 2: the bandwidth kernel of the
-// MobileNet family.  A thread owns 8 channels of a strip of 4 consecutive output pixels of one row:
+// MobileNet family.  A thread owns 2 (4, 8) channels of a strip of 4 consecutive output pixels of one row:
 //   * the nine filter taps of its 8 channels are loaded once (weights [tap][C]) instead of once per output pixel;
 //   * per input row the strip needs 6 (stride 1) or 9 (stride 2) 16-byte pixel vectors, each used by up to three
 //     outputs: 4.5 / 6.75 loads per output pixel instead of 9, all of them issued before the first use;
@@ -25,20 +25,21 @@ struct DwArgs
     f16 *y;
     int H, W, inLd, OH, OW, outLd, C, pad;
     int strips;             // ceil(OW / 4)
-    long long total;        // B * OH * strips * (C / 8)
+    long long total;        // B * OH * strips * (C / channels per lane)
     unsigned xBytes;
     int act;
     float actParam, outMul;
 };
 
-template <int STRIDE>
+template <int STRIDE, int CPL>
 __global__ __launch_bounds__(256) void convDepthwise3x3Kernel(DwArgs a)
 {
     constexpr int COLS = 3 * STRIDE + 3;          // input columns feeding 4 outputs: (4 - 1) * STRIDE + 3
+    typedef f16 HV __attribute__((ext_vector_type(CPL)));          // CPL channels per lane: one 16-, 8- or 4-byte access
     const long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
     if (idx >= a.total) return;
-    const int cv = a.C / 8;
-    const int c0 = static_cast<int>(idx % cv) * 8;
+    const int cv = a.C / CPL;
+    const int c0 = static_cast<int>(idx % cv) * CPL;
     long long t = idx / cv;
     const int sx = static_cast<int>(t % a.strips);
     t /= a.strips;
@@ -50,9 +51,9 @@ __global__ __launch_bounds__(256) void convDepthwise3x3Kernel(DwArgs a)
 
     const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<f16 *>(a.x), 0, static_cast<int>(a.xBytes), 0x00020000);
 
-    f16x8 wv[9];
+    HV wv[9];
 #pragma unroll
-    for (int k = 0; k < 9; ++k) wv[k] = *reinterpret_cast<const f16x8 *>(a.w + static_cast<size_t>(k) * a.C + c0);
+    for (int k = 0; k < 9; ++k) wv[k] = *reinterpret_cast<const HV *>(a.w + static_cast<size_t>(k) * a.C + c0);
 
     // byte offset of input pixel (iy0, ix0), channel c0; may be "negative": it wraps back once a valid tap is added
     const unsigned base = static_cast<unsigned>(((static_cast<long long>(b) * a.H + iy0) * a.W + ix0) * a.inLd + c0) * 2u;
@@ -63,13 +64,13 @@ __global__ __launch_bounds__(256) void convDepthwise3x3Kernel(DwArgs a)
         const int ix = ix0 + c;
         colOff[c] = (ix >= 0 && ix < a.W) ? base + static_cast<unsigned>(c * a.inLd) * 2u : kOob;
     }
-    float acc[4][8];
+    float acc[4][CPL];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
+        for (int e = 0; e < CPL; ++e) acc[j][e] = 0.f;
 
-    f16x8 xv[3][COLS];
+    HV xv[3][COLS];
 #pragma unroll
     for (int r = 0; r < 3; ++r)
     {
@@ -80,7 +81,9 @@ __global__ __launch_bounds__(256) void convDepthwise3x3Kernel(DwArgs a)
         for (int c = 0; c < COLS; ++c)
         {
             const unsigned off = (rowOk && colOff[c] != kOob) ? colOff[c] + rowOff : kOob;
-            xv[r][c] = __builtin_bit_cast(f16x8, __builtin_amdgcn_raw_buffer_load_b128(rx, static_cast<int>(off), 0, 0));
+            if constexpr (CPL == 8) xv[r][c] = __builtin_bit_cast(HV, __builtin_amdgcn_raw_buffer_load_b128(rx, static_cast<int>(off), 0, 0));
+            else if constexpr (CPL == 4) xv[r][c] = __builtin_bit_cast(HV, __builtin_amdgcn_raw_buffer_load_b64(rx, static_cast<int>(off), 0, 0));
+            else xv[r][c] = __builtin_bit_cast(HV, __builtin_amdgcn_raw_buffer_load_b32(rx, static_cast<int>(off), 0, 0));
         }
     }
 #pragma unroll
@@ -90,25 +93,31 @@ __global__ __launch_bounds__(256) void convDepthwise3x3Kernel(DwArgs a)
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
+                for (int e = 0; e < CPL; ++e)
                     acc[j][e] += static_cast<float>(xv[r][j * STRIDE + kx][e]) * static_cast<float>(wv[r * 3 + kx][e]);
 
-    float sc[8], sh[8];
+    float sc[CPL], sh[CPL];
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
+    for (int e = 0; e < CPL; ++e)
     {
         sc[e] = a.scale ? a.scale[c0 + e] : 1.f;
         sh[e] = a.shift ? a.shift[c0 + e] : 0.f;
     }
     const size_t prow = (static_cast<size_t>(b) * a.OH + oy) * a.OW;
+    float v[4 * CPL];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) v[j * CPL + e] = acc[j][e] * sc[e] + sh[e];
+    activateArray<4 * CPL>(v, a.act, a.actParam);
 #pragma unroll
     for (int j = 0; j < 4; ++j)
     {
         if (ox0 + j >= a.OW) break;
-        f16x8 o;
+        HV o;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = static_cast<f16>(a.outMul * activate(acc[j][e] * sc[e] + sh[e], a.act, a.actParam));
-        *reinterpret_cast<f16x8 *>(a.y + (prow + ox0 + j) * a.outLd + c0) = o;
+        for (int e = 0; e < CPL; ++e) o[e] = static_cast<f16>(a.outMul * v[j * CPL + e]);
+        *reinterpret_cast<HV *>(a.y + (prow + ox0 + j) * a.outLd + c0) = o;
     }
 }
 
@@ -129,12 +138,16 @@ int convDepthwise3x3(const msnh_conv_desc *d, const void *x, const void *w, cons
     a.x = static_cast<const f16 *>(x); a.w = static_cast<const f16 *>(w); a.scale = scale; a.shift = shift; a.y = static_cast<f16 *>(y);
     a.H = d->in_h; a.W = d->in_w; a.inLd = d->in_ld; a.OH = d->out_h; a.OW = d->out_w; a.outLd = d->out_ld; a.C = d->in_c; a.pad = d->pad;
     a.strips = (d->out_w + 3) / 4;
-    a.total = static_cast<long long>(d->batch) * d->out_h * a.strips * (d->in_c / 8);
+    // 2 channels per lane: a quarter of the registers of 8 (78 instead of 192), four times the wavefronts in flight -- the kernel
+    // is bound by load latency, not by the number of load instructions (measured over MobileNetV2's 17 layers at batch 64:
+    // 447 us with 8, 287 us with 4, 237 us with 2)
+    constexpr int CPL = 2;
+    a.total = static_cast<long long>(d->batch) * d->out_h * a.strips * (d->in_c / CPL);
     a.xBytes = static_cast<unsigned>(((static_cast<unsigned long long>(d->batch) * d->in_h * d->in_w - 1) * d->in_ld + d->in_c) * 2ull);
     a.act = d->act; a.actParam = d->act_param; a.outMul = d->out_mul;
     const dim3 grid(gridFor(a.total, 256));
-    if (d->stride == 1) hipLaunchKernelGGL(convDepthwise3x3Kernel<1>, grid, dim3(256), 0, st, a);
-    else                hipLaunchKernelGGL(convDepthwise3x3Kernel<2>, grid, dim3(256), 0, st, a);
+    if (d->stride == 1) hipLaunchKernelGGL((convDepthwise3x3Kernel<1, CPL>), grid, dim3(256), 0, st, a);
+    else                hipLaunchKernelGGL((convDepthwise3x3Kernel<2, CPL>), grid, dim3(256), 0, st, a);
     MSNH_LAUNCH_CHECK();
     return 0;
 }

@@ -132,14 +132,16 @@ void convPointwiseKernel(PwArgs a)
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                     {
-                        v[e]     = activate(acc[i][j][8 * g + e] * s0[e] + h0[e], a.act, a.actParam);
-                        v[4 + e] = activate(acc[i][j][8 * g + 4 + e] * s1[e] + h1[e], a.act, a.actParam);
+                        v[e]     = acc[i][j][8 * g + e] * s0[e] + h0[e];
+                        v[4 + e] = acc[i][j][8 * g + 4 + e] * s1[e] + h1[e];
                     }
+                    activateArray<8>(v, a.act, a.actParam);
                     if (a.hasRes)
                     {
                         const f16x8 r = *reinterpret_cast<const f16x8 *>(a.res + static_cast<size_t>(p) * a.resLd + c0);
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) v[e] = activate(v[e] + a.resMul * static_cast<float>(r[e]), a.act2, a.act2Param);
+                        for (int e = 0; e < 8; ++e) v[e] += a.resMul * static_cast<float>(r[e]);
+                        activateArray<8>(v, a.act2, a.act2Param);
                     }
                     f16x8 o;
 #pragma unroll
