@@ -234,17 +234,41 @@ __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[
         }
         auto stageBlock = [&](auto slopeTag) {
             constexpr bool SL = decltype(slopeTag)::value;
-            staticFor<0, MB * 4>([&](auto iqTag) {
-                    constexpr int i = decltype(iqTag)::value / 4;
-                    constexpr int q = decltype(iqTag)::value % 4;
-                    const int ml = i * 32 + q * 8 + (lane >> 5) * 4;       // channel inside the wave tile
-                    const f32x4 sc = *reinterpret_cast<const f32x4 *>(ss + wm * TM + ml);
-                    const f32x4 sh = *reinterpret_cast<const f32x4 *>(ss + BM + wm * TM + ml);
-                    f32x4 v;
+            if constexpr (SL)
+            {
+                staticFor<0, MB * 4>([&](auto iqTag) {
+                        constexpr int i = decltype(iqTag)::value / 4;
+                        constexpr int q = decltype(iqTag)::value % 4;
+                        const int ml = i * 32 + q * 8 + (lane >> 5) * 4;       // channel inside the wave tile
+                        const f32x4 sc = *reinterpret_cast<const f32x4 *>(ss + wm * TM + ml);
+                        const f32x4 sh = *reinterpret_cast<const f32x4 *>(ss + BM + wm * TM + ml);
+                        f32x4 v;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = activateSel<SL>(acc[i][j][q * 4 + e] * sc[e] + sh[e], slope1, a.act, a.actParam);
-                    *reinterpret_cast<f32x4 *>(stage + (lane & 31) * LDE + ml) = v;
-            });
+                        for (int e = 0; e < 4; ++e) v[e] = activateSel<true>(acc[i][j][q * 4 + e] * sc[e] + sh[e], slope1, a.act, a.actParam);
+                        *reinterpret_cast<f32x4 *>(stage + (lane & 31) * LDE + ml) = v;
+                });
+            }
+            else
+            {
+                // transcendental activations: affine on every accumulator first, then ONE choice of the activation for all of them
+                float t[MB * 16];
+                staticFor<0, MB * 4>([&](auto iqTag) {
+                        constexpr int iq = decltype(iqTag)::value;
+                        constexpr int i = iq / 4, q = iq % 4;
+                        const int ml = i * 32 + q * 8 + (lane >> 5) * 4;
+                        const f32x4 sc = *reinterpret_cast<const f32x4 *>(ss + wm * TM + ml);
+                        const f32x4 sh = *reinterpret_cast<const f32x4 *>(ss + BM + wm * TM + ml);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) t[iq * 4 + e] = acc[i][j][q * 4 + e] * sc[e] + sh[e];
+                });
+                activateArray<MB * 16>(t, a.act, a.actParam);
+                staticFor<0, MB * 4>([&](auto iqTag) {
+                        constexpr int iq = decltype(iqTag)::value;
+                        constexpr int i = iq / 4, q = iq % 4;
+                        const int ml = i * 32 + q * 8 + (lane >> 5) * 4;
+                        *reinterpret_cast<f32x4 *>(stage + (lane & 31) * LDE + ml) = f32x4{t[iq * 4], t[iq * 4 + 1], t[iq * 4 + 2], t[iq * 4 + 3]};
+                });
+            }
         };
         if (lin1) stageBlock(std::true_type()); else stageBlock(std::false_type());
         __syncthreads();
@@ -267,8 +291,17 @@ __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[
                     {
                         float r[8];
                         resRaw[t].toFloat(r);
+                        if constexpr (SL)
+                        {
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) v[e] = activateSel<SL>(v[e] + a.resMul * r[e], slope2, a.act2, a.act2Param);
+                            for (int e = 0; e < 8; ++e) v[e] = activateSel<true>(v[e] + a.resMul * r[e], slope2, a.act2, a.act2Param);
+                        }
+                        else
+                        {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) v[e] += a.resMul * r[e];
+                            activateArray<8>(v, a.act2, a.act2Param);
+                        }
                     }
 #pragma unroll
                     for (int e = 0; e < 8; ++e) v[e] *= a.outMul;

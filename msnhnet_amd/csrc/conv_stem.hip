@@ -139,13 +139,20 @@ __global__ __launch_bounds__(256) void convStemMfmaKernel(StemArgs a)
                 const float *scp = ssl + mb * 32 + (hi ? 16 : 0);
                 const float *shp = scp + MBLK * 32;
                 f16x8 o0, o1;
+                float t[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) t[r] = acc[mb][r] * scp[r] + shp[r];
+                if (lin)
+                {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) t[r] = t[r] > 0.f ? t[r] : slope * t[r];
+                }
+                else activateArray<16>(t, a.act, a.actParam);       // one choice of the activation for the 16 values
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                 {
-                    float t = acc[mb][r] * scp[r] + shp[r];
-                    t = lin ? (t > 0.f ? t : slope * t) : activate(t, a.act, a.actParam);
-                    t *= a.outMul;
-                    if (r < 8) o0[r] = static_cast<f16>(t); else o1[r - 8] = static_cast<f16>(t);
+                    const float u = t[r] * a.outMul;
+                    if (r < 8) o0[r] = static_cast<f16>(u); else o1[r - 8] = static_cast<f16>(u);
                 }
                 *reinterpret_cast<f16x8 *>(yp + mb * 32) = o0;
                 *reinterpret_cast<f16x8 *>(yp + mb * 32 + 8) = o1;

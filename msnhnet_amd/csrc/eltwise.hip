@@ -57,8 +57,11 @@ __global__ __launch_bounds__(256) void affineActKernel(const T *__restrict__ x, 
     {
         const float sc = scale ? scale[c0 + i] : 1.f;
         const float sh = shift ? shift[c0 + i] : 0.f;
-        v[i] = outMul * activate(v[i] * sc + sh, act, actParam);
+        v[i] = v[i] * sc + sh;
     }
+    activateArray<VEC>(v, act, actParam);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] *= outMul;
     storeVec<TOut, VEC>(y + p * yLd + c0, v);
 }
 
@@ -77,7 +80,10 @@ __global__ __launch_bounds__(256) void addActKernel(const T *__restrict__ a, int
     loadVec<T, VEC>(a + p * aLd + c0, va);
     loadVec<T, VEC>(b + p * bLd + c0, vb);
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) va[i] = outMul * activate(aMul * va[i] + bMul * vb[i], act, actParam);
+    for (int i = 0; i < VEC; ++i) va[i] = aMul * va[i] + bMul * vb[i];
+    activateArray<VEC>(va, act, actParam);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) va[i] *= outMul;
     storeVec<T, VEC>(y + p * yLd + c0, va);
 }
 
@@ -359,7 +365,10 @@ __global__ __launch_bounds__(256) void col2imKernel(const T *__restrict__ cols, 
         }
     }
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[i] = outMul * activate(colsMul * acc[i] + (bias ? bias[c0 + i] : 0.f), act, actParam);
+    for (int i = 0; i < VEC; ++i) acc[i] = colsMul * acc[i] + (bias ? bias[c0 + i] : 0.f);
+    activateArray<VEC>(acc, act, actParam);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] *= outMul;
     storeVec<T, VEC>(y + p * yLd + c0, acc);
 }
 
