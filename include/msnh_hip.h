@@ -248,12 +248,13 @@ int msnh_hip_yolo_decode(int dtype, int batch, int h, int w, int classes, const 
                          float conf_thresh, int *cand_idx, int cand_cap, int cand_base, int *cand_cnt, msnh_stream_t s);
 /* The same candidate list as msnh_hip_yolo_decode, but only the rows of the candidates are decoded (into the places the full
  * decode would give them; the rest of `decoded` is left as it is): an objectness scan over the head, then one row per
- * candidate.  For callers that only consume the candidates (msnh_hip_yolo_gather).  Arguments as for msnh_hip_yolo_decode;
- * cand_idx and cand_cnt are required. */
+ * candidate.  For callers that only consume the candidates.  Arguments as for msnh_hip_yolo_decode; cand_idx and cand_cnt are
+ * required.  rows, if not NULL: [batch][cand_cap][8] float32; the compact row of every candidate of this head is written at the
+ * candidate's position in the list, exactly what msnh_hip_yolo_gather would produce for it (that call is then unnecessary). */
 int msnh_hip_yolo_decode_candidates(int dtype, int batch, int h, int w, int classes, const void *x, int x_ld, float x_mul,
                                     const float *anchors6, float ratio, int yolo_version, float *decoded,
                                     long long decoded_batch_stride, float conf_thresh, int *cand_idx, int cand_cap, int cand_base,
-                                    int *cand_cnt, msnh_stream_t s);
+                                    int *cand_cnt, float *rows, msnh_stream_t s);
 /* Candidate compaction for YoloOutLayer (the per-box part of src/layers/MsnhYoloOutLayer.cpp:120-170 done on
  * the device so that only surviving boxes cross PCIe): for image b and k < min(cand_cnt[b], cand_cap) reads
  * the decoded row of cell cand_idx[b][k] (rows are `5+classes` floats, row r of image b at

@@ -118,24 +118,56 @@ __global__ __launch_bounds__(256) void yoloScanKernel(const T *__restrict__ x, i
         candIdx[static_cast<size_t>(b) * candCap + base + threadIdx.x] = found[threadIdx.x];
 }
 
-// Decodes the rows of the listed candidates that belong to this head into their places of the decoded buffer.
+// Decodes the rows of the listed candidates that belong to this head into their places of the decoded buffer and, when
+// `rows` is given, writes the candidate's compact row { x, y, w, h, objectness, best class score, best class index, cell }
+// (what yoloGatherKernel derives from the decoded row).  One wavefront per candidate: lane l decodes values l, l + 64, ...;
+// the best class is the first maximum in channel order, found with a wavefront reduction on (score, index).
 template <typename T, bool V5>
-__global__ __launch_bounds__(128) void yoloRowsKernel(const T *__restrict__ x, int xLd, float xMul, Anchors an, float ratio,
+__global__ __launch_bounds__(256) void yoloRowsKernel(const T *__restrict__ x, int xLd, float xMul, Anchors an, float ratio,
                                                       float *__restrict__ decoded, long long decStride, const int *__restrict__ candIdx, int candCap,
-                                                      int candBase, const int *__restrict__ candCnt, int W, int HW, int per)
+                                                      int candBase, const int *__restrict__ candCnt, float *__restrict__ rows, int W, int HW, int per)
 {
     const int b = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
     int n = candCnt[b];
     n = n < candCap ? n : candCap;
-    for (int k = blockIdx.x; k < n; k += gridDim.x)
+    for (int k = blockIdx.x * 4 + wave; k < n; k += gridDim.x * 4)
     {
-        const int cell = candIdx[static_cast<size_t>(b) * candCap + k] - candBase;
+        const int cellG = candIdx[static_cast<size_t>(b) * candCap + k];
+        const int cell = cellG - candBase;
         if (cell < 0 || cell >= 3 * HW) continue;                // another head's candidate
         const int a = cell / HW, p = cell - a * HW;
         const int py = p / W, px = p - py * W;
         const T *xr = x + (static_cast<size_t>(b) * HW + p) * xLd + a * per;
         float *dr = decoded + static_cast<size_t>(b) * decStride + static_cast<size_t>(cell) * per;
-        for (int m = threadIdx.x; m < per; m += 128) dr[m] = yoloDecodeOne<V5>(xMul * toF(xr[m]), m, px, py, a, an, ratio);
+        float first = 0.f;                                       // this lane's value of m = lane (box and objectness live in lanes 0..4)
+        float bv = -3.402823466e38f * 2.f;                       // -inf: NaN scores are never selected
+        int bi = 0x7fffffff;
+        for (int m = lane; m < per; m += 64)
+        {
+            const float v = yoloDecodeOne<V5>(xMul * toF(xr[m]), m, px, py, a, an, ratio);
+            dr[m] = v;
+            if (m == lane) first = v;
+            if (m >= 5 && v > bv) { bv = v; bi = m - 5; }
+        }
+        if (rows == nullptr) continue;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1)
+        {
+            const float ov = __shfl_xor(bv, off, 64);
+            const int oi = __shfl_xor(bi, off, 64);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
+        // a NaN score of class 0 absorbs the sequential scan of the reference (nothing compares greater than it)
+        const float c0v = __shfl(first, 5, 64);
+        if (c0v != c0v) { bv = c0v; bi = 0; }
+        if (bi == 0x7fffffff) bi = 0;
+        float *o = rows + (static_cast<size_t>(b) * candCap + k) * 8;
+        if (lane < 5) o[lane] = first;
+        else if (lane == 5) o[5] = bv;
+        else if (lane == 6) o[6] = static_cast<float>(bi);
+        else if (lane == 7) o[7] = static_cast<float>(cellG);
     }
 }
 
@@ -218,7 +250,7 @@ extern "C" int msnh_hip_yolo_decode(int dtype, int batch, int h, int w, int clas
 extern "C" int msnh_hip_yolo_decode_candidates(int dtype, int batch, int h, int w, int classes, const void *x, int x_ld, float x_mul,
                                                const float *anchors6, float ratio, int yolo_version, float *decoded,
                                                long long decoded_batch_stride, float conf_thresh, int *cand_idx, int cand_cap, int cand_base,
-                                               int *cand_cnt, msnh_stream_t s)
+                                               int *cand_cnt, float *rows, msnh_stream_t s)
 {
     MSNH_REQUIRE(dtypeOk(dtype), "yolo_decode_candidates: bad dtype");
     MSNH_REQUIRE(batch > 0 && batch <= 65535 && h > 0 && w > 0 && classes > 0, "yolo_decode_candidates: bad geometry");
@@ -230,17 +262,17 @@ extern "C" int msnh_hip_yolo_decode_candidates(int dtype, int batch, int h, int 
     for (int i = 0; i < 6; ++i) an.v[i] = anchors6[i];
     hipStream_t st = resolveStream(s);
     const int HW = h * w;
-    dim3 sgrid((3 * HW + 255) / 256, batch), rgrid(64, batch);
+    dim3 sgrid((3 * HW + 255) / 256, batch), rgrid(128, batch);
 #define MSNH_YC(T)                                                                                                      \
     do {                                                                                                                \
         hipLaunchKernelGGL((yoloScanKernel<T>), sgrid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, x_mul, conf_thresh, cand_idx, cand_cap,  \
                            cand_base, cand_cnt, HW, per);                                                               \
         if (yolo_version == 5)                                                                                          \
-            hipLaunchKernelGGL((yoloRowsKernel<T, true>), rgrid, dim3(128), 0, st, static_cast<const T *>(x), x_ld, x_mul, an, ratio, decoded,  \
-                               decoded_batch_stride, cand_idx, cand_cap, cand_base, cand_cnt, w, HW, per);              \
+            hipLaunchKernelGGL((yoloRowsKernel<T, true>), rgrid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, x_mul, an, ratio, decoded,  \
+                               decoded_batch_stride, cand_idx, cand_cap, cand_base, cand_cnt, rows, w, HW, per);        \
         else                                                                                                            \
-            hipLaunchKernelGGL((yoloRowsKernel<T, false>), rgrid, dim3(128), 0, st, static_cast<const T *>(x), x_ld, x_mul, an, ratio, decoded, \
-                               decoded_batch_stride, cand_idx, cand_cap, cand_base, cand_cnt, w, HW, per);              \
+            hipLaunchKernelGGL((yoloRowsKernel<T, false>), rgrid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, x_mul, an, ratio, decoded, \
+                               decoded_batch_stride, cand_idx, cand_cap, cand_base, cand_cnt, rows, w, HW, per);        \
     } while (0)
     if (dtype == MSNH_F16) MSNH_YC(f16); else MSNH_YC(float);
 #undef MSNH_YC

@@ -102,7 +102,7 @@ def lib():
     L.msnh_hip_nchw_to_nhwc.argtypes = [ci, ci, ci, ci, ci, vp, cf, vp, ci, vp]
     L.msnh_hip_nhwc_to_nchw.argtypes = [ci, ci, ci, ci, ci, vp, ci, cf, vp, vp]
     L.msnh_hip_yolo_decode.argtypes = [ci, ci, ci, ci, ci, vp, ci, cf, fp, cf, ci, vp, ll, cf, vp, ci, ci, vp, vp]
-    L.msnh_hip_yolo_decode_candidates.argtypes = [ci, ci, ci, ci, ci, vp, ci, cf, fp, cf, ci, vp, ll, cf, vp, ci, ci, vp, vp]
+    L.msnh_hip_yolo_decode_candidates.argtypes = [ci, ci, ci, ci, ci, vp, ci, cf, fp, cf, ci, vp, ll, cf, vp, ci, ci, vp, vp, vp]
     L.msnh_hip_yolo_gather.argtypes = [ci, ci, vp, ll, vp, ci, vp, vp, vp]
     L.msnh_hip_absmax.argtypes = [ci, ll, ci, vp, ci, vp, vp]
     _lib = L

@@ -1359,6 +1359,7 @@ void YoloOutLayer::enqueueGather(msnh_stream_t s)
 {
     if (plan == nullptr) MSNH_THROW("YoloOut: layer is not part of a planned network");
     Plan &pl = *plan;
+    if (pl.sparseYolo) return;          // the heads' candidate-only decode already wrote the compact rows
     MSNH_DEV(msnh_hip_yolo_gather(_batch, _channel - 5, pl.yoloDecoded.as<float>(), static_cast<long long>(pl.yoloCells) * _channel,
                                   pl.yoloCandIdx.as<int>(), pl.yoloCells, pl.yoloCandCnt.as<int>(), pl.yoloRows.as<float>(), s));
 }

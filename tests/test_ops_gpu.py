@@ -312,9 +312,10 @@ def test_yolo_decode(dtype, version):
     dd2 = torch.full((2, 3, h * w, per), -7.0, dtype=torch.float32).cuda()
     ci3 = torch.full((2, cap), -1, dtype=torch.int32).cuda()
     cc3 = torch.zeros(2, dtype=torch.int32).cuda()
+    rows3 = torch.zeros((2, cap, 8), dtype=torch.float32).cuda()
     gu.sync()
     abi.check(abi.lib().msnh_hip_yolo_decode_candidates(dtype, 2, h, w, cls, gu.ptr(xd), 256, 1.0, anchors.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
-                                                        ratio, version, gu.ptr(dd2), 3 * h * w * per, 0.5, gu.ptr(ci3), cap, 1000, gu.ptr(cc3), None))
+                                                        ratio, version, gu.ptr(dd2), 3 * h * w * per, 0.5, gu.ptr(ci3), cap, 1000, gu.ptr(cc3), gu.ptr(rows3), None))
     gu.sync()
     out2 = dd2.cpu().numpy().reshape(2, 3 * h * w, per)
     full = out.reshape(2, 3 * h * w, per)
@@ -326,6 +327,12 @@ def test_yolo_decode(dtype, version):
         rows_in[np.array(got, np.int64) - 1000] = True
         assert np.array_equal(out2[b][rows_in], full[b][rows_in])
         assert (out2[b][~rows_in] == -7.0).all()
+        # ... and its compact rows are what the gather kernel derives from the decoded rows
+        r3 = rows3[b, :n].cpu().numpy()
+        cells = ci3[b, :n].cpu().numpy() - 1000
+        assert np.array_equal(r3[:, :5], full[b][cells][:, :5])
+        assert np.array_equal(r3[:, 5], full[b][cells][:, 5:].max(1)) and np.array_equal(r3[:, 6], full[b][cells][:, 5:].argmax(1).astype(np.float32))
+        assert np.array_equal(r3[:, 7], (cells + 1000).astype(np.float32))
     # candidate compaction: box, objectness, first-maximum class
     ci2 = (ci - 1000).clamp(min=0).contiguous()
     rows = torch.zeros((2, cap, 8), dtype=torch.float32).cuda()
