@@ -331,7 +331,13 @@ __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[
 
 // Register budget: two workgroups per CU (one wave of each per SIMD) so that one workgroup's barrier and epilogue
 // are covered by the other's MFMAs; smaller tiles, which serve the short-K bandwidth-bound layers, get three to six.
-constexpr int igemmWavesPerSimd(int bm, int bn) { return bm * bn > 128 * 128 ? 2 : (bm * bn > 64 * 128 ? 3 : (bm * bn > 64 * 64 ? 4 : 6)); }
+constexpr int igemmWavesPerSimd(int bm, int bn, int kv = 8, int ns = 3)
+{
+    // (two-stage 64-byte-row variants of the small tiles: LDS for six to eight workgroups per CU, for the short-K layers that
+    // live on memory bandwidth)
+    if (ns == 2 && kv == 4 && bm * bn <= 64 * 128) return bm * bn > 64 * 64 ? 6 : 8;
+    return bm * bn > 128 * 128 ? 2 : (bm * bn > 64 * 128 ? 3 : (bm * bn > 64 * 64 ? 4 : 6));
+}
 
 // 16-byte-per-lane load from a buffer resource straight into LDS: the 64 lanes of the wave fill 1 KiB starting at
 // ldsAddr (lane l at ldsAddr + 16 * l); lanes whose voffset is out of range store zeros.  No VGPRs and no LDS store
@@ -360,7 +366,7 @@ __device__ __forceinline__ i32x4 makeRsrcWords(const void *base, unsigned bytes)
 }
 
 template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int NS>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(igemmWavesPerSimd(BM, BN), igemmWavesPerSimd(BM, BN))))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(igemmWavesPerSimd(BM, BN, KV, NS), igemmWavesPerSimd(BM, BN, KV, NS))))
 void convIgemmKernel(IgemmArgs a)
 {
     typedef typename Frag<T>::V V;
@@ -695,7 +701,7 @@ namespace msnh {
 // Tile configurations (BM x BN output tile, KV 16-byte vectors of K per step, WM x WN wavefront grid).
 // Index 0 is "choose for me"; the others can be forced through msnh_conv_desc::tile, which is how the host
 // library's per-layer search picks the fastest one at load time.
-constexpr int kIgemmTiles = 28;
+constexpr int kIgemmTiles = 31;
 
 template <typename T, typename TOut>
 int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
@@ -734,6 +740,10 @@ int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
     case 26: return launchIgemm<T, TOut, 256, 128, 4, 2, 2, 6>(a, groups, st);
     case 27: return launchIgemm<T, TOut, 128, 128, 8, 2, 2, 4>(a, groups, st);
     case 28: return launchIgemm<T, TOut, 128, 128, 4, 2, 2, 5>(a, groups, st);
+    // small tiles at high occupancy for bandwidth-bound short-K layers
+    case 29: return launchIgemm<T, TOut, 64, 128, 4, 1, 4, 2>(a, groups, st);
+    case 30: return launchIgemm<T, TOut, 64, 64, 4, 2, 2, 2>(a, groups, st);
+    case 31: return launchIgemm<T, TOut, 128, 64, 4, 2, 2, 2>(a, groups, st);
     default: break;
     }
     setError("igemm: unknown tile %d", tile);
