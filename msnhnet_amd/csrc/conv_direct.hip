@@ -492,15 +492,19 @@ int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const
         if (stemMfmaOk(d))
             return convStemMfma(d, static_cast<const float *>(x), static_cast<const _Float16 *>(w) + static_cast<size_t>(d->ksize) * d->ksize * d->in_c * d->out_c * 2,
                                 scale, shift, y, st);
-        constexpr int OCT = 32;
-        dim3 grid(gridFor(P, 256), d->out_c / OCT);
-        const size_t smem = static_cast<size_t>(d->ksize) * d->ksize * d->in_c * OCT * sizeof(float);
-        if (d->out_dtype == MSNH_F16)
-            hipLaunchKernelGGL((convStemKernel<f16, OCT>), grid, dim3(256), smem, st, static_cast<const float *>(x), static_cast<const float *>(w),
-                               static_cast<f16 *>(y), e, d->in_c, d->in_h, d->in_w, d->out_h, d->out_w, d->out_ld, d->out_c, d->ksize, d->stride, d->pad, P);
-        else
-            hipLaunchKernelGGL((convStemKernel<float, OCT>), grid, dim3(256), smem, st, static_cast<const float *>(x), static_cast<const float *>(w),
-                               static_cast<float *>(y), e, d->in_c, d->in_h, d->in_w, d->out_h, d->out_w, d->out_ld, d->out_c, d->ksize, d->stride, d->pad, P);
+        // a lane owns one pixel and OCT output channels: 32 when there are pixels enough to fill the chip, 8 for small images
+        // (a single 224 x 224 image gives 98 workgroups at 32 channels per lane, 392 at 8)
+#define MSNH_STEM(TO, OCT)                                                                                              \
+    do {                                                                                                                \
+        dim3 grid(gridFor(P, 256), d->out_c / OCT);                                                                     \
+        const size_t smem = static_cast<size_t>(d->ksize) * d->ksize * d->in_c * OCT * sizeof(float);                  \
+        hipLaunchKernelGGL((convStemKernel<TO, OCT>), grid, dim3(256), smem, st, static_cast<const float *>(x), static_cast<const float *>(w), \
+                           static_cast<TO *>(y), e, d->in_c, d->in_h, d->in_w, d->out_h, d->out_w, d->out_ld, d->out_c, d->ksize, d->stride, d->pad, P); \
+    } while (0)
+        const bool few = P * (d->out_c / 32) < 256LL * 512;
+        if (d->out_dtype == MSNH_F16) { if (few) MSNH_STEM(f16, 8); else MSNH_STEM(f16, 32); }
+        else                          { if (few) MSNH_STEM(float, 8); else MSNH_STEM(float, 32); }
+#undef MSNH_STEM
         MSNH_LAUNCH_CHECK();
         return 0;
     }
