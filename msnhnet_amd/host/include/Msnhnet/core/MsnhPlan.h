@@ -115,7 +115,9 @@ public:
     void applyCalibration(const Plan &calibrated);   // pass 3: take amax from an executed float32 twin
     void place();                           // pass 4 + arena allocation
     void prepareWeights();                  // fold batch-norm, pick algorithms, pack and upload weights
-    void tuneConvs(msnh_stream_t s);        // time every IGEMM tile configuration per conv launch, keep the fastest
+    // time every tile configuration / algorithm variant per conv launch, keep the fastest.  cacheFile (may be empty): choices of an
+    // earlier search for the same plan on the same device are read from it instead of being timed again, and written to it otherwise
+    void tuneConvs(msnh_stream_t s, const std::string &cacheFile = std::string());
     void run(size_t opBegin, size_t opEnd, msnh_stream_t s);
     void runAll(msnh_stream_t s) { run(0, ops.size(), s); }
     void measureAmax(msnh_stream_t s);      // after an eager run: absmax of every live NHWC tensor

@@ -26,6 +26,10 @@ public:
     static void setKeepClassScores(const bool &keep);
     // Per-layer search for the fastest convolution tile configuration at load time (default on).
     static void setAutoTune(const bool &on);
+    // keep the per-layer tile / algorithm choices next to the weights file ("<path>.msnhbin.tune"): the next load of the same
+    // graph on the same device skips the search.  Off by default (the library then writes no files).
+    static void setTuneCache(const bool &on);
+    static bool tuneCache;
     static void setUseWinograd(const bool &on);   // float16 plans: 3x3 stride-1 convolutions through Winograd F(2x2,3x3)
     static bool useWinograd;
     static bool autoTune;
@@ -87,6 +91,7 @@ public:
 
 private:
     void finalizePlan();
+    std::string _weightsPath;               // set while loadWeightsFromMsnhBin runs: where the tune cache goes
     std::unique_ptr<Plan> lowerNetwork(int dtype);
     void uploadInput(const std::vector<float> &img);
     void runLayersEager();

@@ -44,6 +44,8 @@ void NetBuilder::setForceUseCuda(const bool &v) { BaseLayer::setForceUseCuda(v);
 void NetBuilder::setKeepClassScores(const bool &keep) { YoloOutLayer::keepClassScores = keep; }
 bool NetBuilder::autoTune = true;
 void NetBuilder::setAutoTune(const bool &on) { autoTune = on; }
+bool NetBuilder::tuneCache = false;
+void NetBuilder::setTuneCache(const bool &on) { tuneCache = on; }
 bool NetBuilder::useWinograd = false;
 void NetBuilder::setUseWinograd(const bool &on) { useWinograd = on; }
 
@@ -281,7 +283,9 @@ void NetBuilder::loadWeightsFromMsnhBin(const std::string &path)
 {
     if (BaseLayer::isPreviewMode) MSNH_THROW("Can not load weights in preview mode !");
     _parser->readMsnhBin(path);
+    _weightsPath = path;
     loadWeightsFromVector(_parser->msnhF32Weights);
+    _weightsPath.clear();
     std::vector<float>().swap(_parser->msnhF32Weights);
 }
 
@@ -408,7 +412,7 @@ void NetBuilder::finalizePlan()
     plan->preferWinograd = useWinograd && dtype == MSNH_F16;
     plan->sparseYolo = !_saveLayerOutput;         // layer dumps read the whole decoded tensors
     plan->prepareWeights();
-    if (autoTune) plan->tuneConvs(_stream);
+    if (autoTune) plan->tuneConvs(_stream, (tuneCache && !_weightsPath.empty()) ? _weightsPath + (dtype == MSNH_F16 ? ".f16.tune" : ".f32.tune") : std::string());
 
     // hand every layer its slice of the op list
     for (size_t i = 0; i < _net->layers.size(); ++i)

@@ -4,6 +4,8 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <cstdio>
+#include <fstream>
 #include <functional>
 #include <limits>
 #include <mutex>
@@ -456,12 +458,83 @@ void Plan::prepareWeights()
     if (workspace > _convWorkspace.bytes()) _convWorkspace.alloc(workspace);
 }
 
+// Tune cache, one line per tuned launch: what identifies the launch (shape, dtype, epilogue kind) and what the search chose for it.
+static std::string tuneSignature(const Plan &plan, const PlanOp &op)
+{
+    const PlanTensor &in = plan.tensors[static_cast<size_t>(op.in0)];
+    const PlanTensor &out = plan.tensors[static_cast<size_t>(op.out)];
+    std::ostringstream os;
+    os << static_cast<int>(op.kind) << ' ' << in.n << ' ' << in.h << ' ' << in.w << ' ' << in.c << ' ' << plan.ld(op.in0) << ' ' << out.c << ' '
+       << plan.ld(op.out) << ' ' << op.ksize << ' ' << op.stride << ' ' << op.pad << ' ' << op.dilation << ' ' << op.groups << ' ' << (op.in1 >= 0) << ' '
+       << in.dtype << ' ' << out.dtype;
+    return os.str();
+}
+
+static std::string tuneHeader(int nTiles)
+{
+    char name[256] = {0};
+    int cus = 0;
+    size_t mem = 0;
+    msnh_hip_device_name(name, sizeof(name), &cus, &mem);
+    std::string dev(name);
+    for (char &ch : dev)
+        if (ch == ' ' || ch == '\n') ch = '_';
+    return "msnhtune 1 " + (dev.empty() ? std::string("device") : dev) + " cus " + std::to_string(cus) + " tiles " + std::to_string(nTiles);
+}
+
 // Per-layer search over the implicit-GEMM tile configurations: each candidate runs the real launch (same buffers,
 // same epilogue) a few times between two device events; the fastest wins.  Tiles change the result by nothing but the
 // float32 summation order, and so does the split-K variant tried for layers with few output tiles.
-void Plan::tuneConvs(msnh_stream_t s)
+// With a cache file: a file written by an earlier search over the same launches on the same device replaces the search.
+void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
 {
     const int nTiles = msnh_hip_conv2d_tile_count();
+    const auto tunable = [](const PlanOp &op) {
+        return !op.dead && (op.kind == PlanOp::CONV || op.kind == PlanOp::CONNECTED) && (op.algo == MSNH_CONV_IGEMM || op.algo == MSNH_CONV_WINOGRAD);
+    };
+    std::vector<size_t> tunedOps;
+    for (size_t i = 0; i < ops.size(); ++i)
+        if (tunable(ops[i])) tunedOps.push_back(i);
+    if (!cacheFile.empty())
+    {
+        // file: header, then "<signature> | <algo> <tile>" per tunable launch in plan order; any mismatch discards the file
+        std::ifstream f(cacheFile);
+        std::string line;
+        std::vector<std::pair<int, int>> picks;
+        bool ok = f.is_open() && std::getline(f, line) && line == tuneHeader(nTiles);
+        for (size_t k = 0; ok && k < tunedOps.size(); ++k)
+        {
+            ok = static_cast<bool>(std::getline(f, line));
+            const size_t bar = ok ? line.find(" | ") : std::string::npos;
+            ok = ok && bar != std::string::npos && line.substr(0, bar) == tuneSignature(*this, ops[tunedOps[k]]);
+            int algo = 0, tile = 0;
+            ok = ok && std::sscanf(line.c_str() + bar + 3, "%d %d", &algo, &tile) == 2 && tile >= 0 && tile <= nTiles &&
+                 (algo == MSNH_CONV_IGEMM || algo == MSNH_CONV_WINOGRAD || algo == MSNH_CONV_IGEMM_SPLITK || algo == MSNH_CONV_POINTWISE);
+            if (ok) picks.emplace_back(algo, tile);
+        }
+        if (ok)
+        {
+            // the library must still accept every recorded choice; otherwise the defaults come back and the search runs
+            std::vector<std::pair<int, int>> before;
+            size_t need = 0;
+            for (size_t k = 0; k < tunedOps.size(); ++k)
+            {
+                PlanOp &op = ops[tunedOps[k]];
+                before.emplace_back(op.algo, op.tile);
+                op.algo = picks[k].first; op.tile = picks[k].second;
+                const msnh_conv_desc d = convDesc(*this, op);
+                if (!msnh_hip_conv2d_tile_supported(&d, op.tile)) ok = false;
+                need = std::max(need, msnh_hip_conv2d_workspace_bytes(&d, op.algo));
+            }
+            if (ok)
+            {
+                if (need > _convWorkspace.bytes()) _convWorkspace.alloc(need);
+                return;
+            }
+            for (size_t k = 0; k < tunedOps.size(); ++k) { ops[tunedOps[k]].algo = before[k].first; ops[tunedOps[k]].tile = before[k].second; }
+        }
+    }
+
     msnh_event_t e0 = nullptr, e1 = nullptr;
     MSNH_DEV(msnh_hip_event_create(&e0));
     MSNH_DEV(msnh_hip_event_create(&e1));
@@ -524,6 +597,19 @@ void Plan::tuneConvs(msnh_stream_t s)
     }
     msnh_hip_event_destroy(e0);
     msnh_hip_event_destroy(e1);
+    if (!cacheFile.empty())
+    {
+        std::ofstream f(cacheFile, std::ios::trunc);
+        if (f.is_open())
+        {
+            f << tuneHeader(nTiles) << "\n";
+            for (size_t i : tunedOps)
+            {
+                // (the signature is taken with the searched choice in place: it does not depend on algo / tile)
+                f << tuneSignature(*this, ops[i]) << " | " << ops[i].algo << ' ' << ops[i].tile << "\n";
+            }
+        }
+    }
 }
 
 // round-to-nearest-even float -> IEEE half, host side

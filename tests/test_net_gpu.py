@@ -210,6 +210,61 @@ def test_fp16_winograd_network(arch, size, batch):
             assert nu.rel_err(logits[b], ref[b][-1]) <= 2e-2
 
 
+def test_tune_cache(tmp_path):
+    """the per-layer search result is kept beside the weights file when asked for: the next load takes the same choices
+    from the file (same plan, bit-identical outputs), a file that does not fit is ignored and rewritten, and nothing is
+    written unless the switch is on"""
+    import shutil
+    import time
+    arch, size, batch = "yolov3", 96, 2
+    net0, bin0, g = nu.model(arch, batch, size, seed=3)
+    net, binp = str(tmp_path / "m.msnhnet"), str(tmp_path / "m.msnhbin")
+    shutil.copy(net0, net)
+    shutil.copy(bin0, binp)
+    x = zoo.seeded_input(batch, 3, size, size, seed=4)
+    cache = binp + ".f16.tune"
+    netapi.Net(net, binp, fp16=True)
+    assert not os.path.exists(cache) and not os.path.exists(binp + ".f32.tune")
+    netapi.set_tune_cache(True)
+    try:
+        t0 = time.perf_counter()
+        a = netapi.Net(net, binp, fp16=True)
+        t1 = time.perf_counter()
+        assert os.path.exists(cache)
+        text = open(cache).read()
+        lines = text.splitlines()
+        assert lines[0].startswith("msnhtune 1 ") and len(lines) > 10 and all(" | " in ln for ln in lines[1:])
+        b = netapi.Net(net, binp, fp16=True)
+        t2 = time.perf_counter()
+        print(f"load with search {t1 - t0:.3f} s, from the file {t2 - t1:.3f} s", flush=True)
+        assert b.plan_detail() == a.plan_detail()
+        assert open(cache).read() == text
+        ya, yb = a.run_yolo(x), b.run_yolo(x)
+        for i in range(batch):
+            assert np.array_equal(ya[i], yb[i])
+        # a line that names another launch: the whole file is dropped, the search runs and writes a fresh one
+        bad = lines[:]
+        bad[3] = "9 " + bad[3]
+        open(cache, "w").write("\n".join(bad) + "\n")
+        c = netapi.Net(net, binp, fp16=True)
+        fresh = open(cache).read().splitlines()
+        assert [ln.split(" | ")[0] for ln in fresh] == [ln.split(" | ")[0] for ln in lines]
+        yc = c.run_yolo(x)
+        for i in range(batch):
+            assert abs(len(yc[i]) - len(ya[i])) <= max(2, 0.02 * len(ya[i]))
+        # a choice the library refuses for the launch (a tile number past the table): same
+        bad = fresh[:]
+        bad[2] = bad[2].split(" | ")[0] + " | 1 999"
+        open(cache, "w").write("\n".join(bad) + "\n")
+        netapi.Net(net, binp, fp16=True)
+        assert " | 1 999" not in open(cache).read()
+        # float32 plans keep their own file
+        netapi.Net(net, binp, fp16=False)
+        assert os.path.exists(binp + ".f32.tune")
+    finally:
+        netapi.set_tune_cache(False)
+
+
 def test_image_in_boxes_out():
     """8-bit images of different shapes -> device letterbox -> forward -> boxes in original-image pixels: equals the
     float path fed with the restatement's letterbox, followed by the restatement's rescale."""
