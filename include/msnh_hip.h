@@ -263,6 +263,20 @@ int msnh_hip_yolo_decode_candidates(int dtype, int batch, int h, int w, int clas
  * best class = first maximum like std::max_element). */
 int msnh_hip_yolo_gather(int batch, int classes, const float *decoded, long long decoded_batch_stride, const int *cand_idx,
                          int cand_cap, const int *cand_cnt, float *rows, msnh_stream_t s);
+/* Per-class greedy NMS over the compact rows (src/layers/MsnhYoloOutLayer.cpp:175-194 and :381-461 on the device, so that
+ * only the boxes that survive cross PCIe).  rows / cand_cap / cand_cnt as written by msnh_hip_yolo_gather or
+ * msnh_hip_yolo_decode_candidates.  kept: [kept_cap][12] float32, 16-byte aligned; kept_cnt: int32 [1 + batch], zeroed by
+ * the caller.  workspace: msnh_hip_yolo_nms_workspace_bytes() bytes of device memory (contents irrelevant), or NULL.
+ * On return kept_cnt[0] is the number of records written (kept_cap >= batch * cand_cap can never overflow) and
+ * kept_cnt[1 + b] != 0 says that image b was NOT processed completely: a class with more candidates in that image than the
+ * kernels take (6144 with a workspace, 1024 without) or a NaN score.  The caller then runs the reference's procedure on
+ * that image's rows itself and ignores its records.
+ * A record = { row[0..7], score of the class's best-scoring candidate, that candidate's cell index, pick order inside the
+ * class, image index }, in no particular order.  The reference's output order of an image is: classes by (record[8]
+ * descending, record[9] ascending), inside a class by record[10] ascending. */
+size_t msnh_hip_yolo_nms_workspace_bytes(int batch, int classes, int cand_cap);
+int msnh_hip_yolo_nms(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept,
+                      int kept_cap, int *kept_cnt, void *workspace, size_t workspace_bytes, msnh_stream_t s);
 
 /* max |x| over the finite elements of an NHWC tensor, combined into *result with an atomic max
  * (caller zeroes *result).  Used once at load time to calibrate the power-of-two activation scales of the

@@ -57,6 +57,8 @@ const char *msnhnet_last_error(void);
 int msnhnet_create(msnhnet_t *net);                       /* NetBuilder() */
 int msnhnet_destroy(msnhnet_t net);
 int msnhnet_set_use_fp16(int on);                         /* NetBuilder::setUseFp16, process-wide, before build */
+int msnhnet_set_device_nms(int mode);                     /* hard NMS: 0 = candidates copied back, sort + NMS on the host; 2 = on the device, only kept boxes cross
+                                                              PCIe; 1 (default) = on the device while the previous result had <= 2048 candidates per image */
 int msnhnet_set_tune_cache(int on);                       /* keep the per-layer tile search result in "<weights>.f16.tune" / ".f32.tune" next to the
                                                               .msnhbin file and reuse it on the next load (same graph, same device); off by default */
 int msnhnet_set_use_winograd(int on);                     /* float16 builds: 3x3 stride-1 convolutions through Winograd F(2x2,3x3);

@@ -171,6 +171,289 @@ __global__ __launch_bounds__(256) void yoloRowsKernel(const T *__restrict__ x, i
     }
 }
 
+// ---- per-class greedy NMS on the device (src/layers/MsnhYoloOutLayer.cpp:175-194 sort, :381-461 nms) -------------------
+// One workgroup per (class, image).  The reference sorts all candidates of an image by objectness * best class score
+// (descending; here ties keep cell order), visits the classes in the order of their first appearance in that list and,
+// inside a class, repeatedly picks the highest objectness (first of the list on ties) and erases what overlaps it by more
+// than the threshold.  Per class that is: order the members by (objectness, score, cell) and keep a member unless one kept
+// before it overlaps it.  The workgroup collects the members of its class, ranks them by counting, runs the greedy pass in
+// its first wavefront (lanes test the later members against the pick in parallel) and appends one record per kept box:
+// the compact row, the (score, cell) of the class's first member in the global list -- the host orders classes by it --,
+// the pick order inside the class and the image index.
+constexpr int NMS_CAP = 1024;           // members of one class in one image; more -> the image is flagged for the caller
+
+__device__ __forceinline__ unsigned orderedBits(float f)
+{
+    const unsigned u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// Box::iou(candidate, pick) > thr (include/Msnhnet/utils/MsnhTypes.h:123-140: corners from centre and size, "+ 1" extents,
+// min / max spelled out so that NaN behaves alike), decided without the division wherever the product form is clear of
+// rounding: inter / uni > thr is certain when inter > (thr * uni)(1 + 1e-5) and impossible when inter < (thr * uni)(1 - 1e-5)
+// for positive finite operands; everything else (and every NaN / infinity / zero-union case) takes the division itself.
+__device__ __forceinline__ bool iouAbove(float kx1, float ky1, float kx2, float ky2, float karea, float jx1, float jy1, float jx2, float jy2,
+                                         float jarea, float thr)
+{
+#pragma clang fp contract(off)
+    const float ix2 = (kx2 < jx2) ? kx2 : jx2;
+    const float ix1 = (jx1 < kx1) ? kx1 : jx1;
+    const float iy2 = (ky2 < jy2) ? ky2 : jy2;
+    const float iy1 = (jy1 < ky1) ? ky1 : jy1;
+    const float iw = ix2 - ix1 + 1;
+    const float ih = iy2 - iy1 + 1;
+    const float inter = (iw < 0 ? 0 : iw) * (ih < 0 ? 0 : ih);
+    const float uni = jarea + karea - inter;
+    if (thr >= 0.f && thr <= 1e3f && uni > 1e-20f && uni < 1e30f && inter < 1e30f)
+    {
+        if (inter == 0.f) return false;
+        const float p = thr * uni;
+        if (p > 1e-20f)
+        {
+            if (inter > p * 1.00001f) return true;
+            if (inter < p * 0.99999f) return false;
+        }
+    }
+    return 1.f * inter / uni > thr;
+}
+
+__global__ __launch_bounds__(256) void yoloNmsKernel(const float *__restrict__ rows, int candCap, const int *__restrict__ candCnt, float thr,
+                                                     float *__restrict__ kept, int keptCap, int *__restrict__ keptCnt, int *__restrict__ bigCnt,
+                                                     int *__restrict__ wsUsed)
+{
+#pragma clang fp contract(off)
+    __shared__ unsigned long long keyA[NMS_CAP];
+    __shared__ unsigned keyB[NMS_CAP];
+    __shared__ int member[NMS_CAP], sorted[NMS_CAP];
+    __shared__ float x1[NMS_CAP], y1[NMS_CAP], x2[NMS_CAP], y2[NMS_CAP], area[NMS_CAP];
+    __shared__ unsigned short pickOf[NMS_CAP];
+    __shared__ unsigned char gone[NMS_CAP];
+    __shared__ unsigned long long top;
+    __shared__ int nMem, bad, nKept, base;
+    const int cls = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    int n = candCnt[b];
+    n = n < candCap ? n : candCap;
+    const float *r = rows + static_cast<size_t>(b) * candCap * 8;
+    if (tid == 0) { nMem = 0; bad = 0; top = 0ull; nKept = 0; }
+    if (wsUsed != nullptr && cls == 0 && tid == 0) wsUsed[b] = 0;       // yoloNmsBigKernel's cursor into the image's workspace
+    __syncthreads();
+    for (int k = tid; k < n; k += 256)
+        if (static_cast<int>(r[static_cast<size_t>(k) * 8 + 6]) == cls)
+        {
+            const int slot = atomicAdd(&nMem, 1);
+            if (slot < NMS_CAP) member[slot] = k;
+        }
+    __syncthreads();
+    const int m = nMem;
+    if (bigCnt != nullptr && tid == 0) bigCnt[b * gridDim.x + cls] = m;
+    if (m == 0) return;
+    if (m > NMS_CAP)
+    {
+        if (bigCnt == nullptr && tid == 0) atomicOr(&keptCnt[1 + b], 1);    // (else yoloNmsBigKernel takes the class)
+        return;
+    }
+    for (int i = tid; i < m; i += 256)
+    {
+        const float *q = r + static_cast<size_t>(member[i]) * 8;
+        const float conf = q[4];
+        const float score = conf * q[5];
+        if (!(score == score) || !(conf == conf)) bad = 1;
+        const unsigned sb = orderedBits(score), cell = ~static_cast<unsigned>(q[7]);
+        keyA[i] = (static_cast<unsigned long long>(orderedBits(conf)) << 32) | sb;
+        keyB[i] = cell;
+        atomicMax(&top, (static_cast<unsigned long long>(sb) << 32) | cell);
+    }
+    __syncthreads();
+    if (bad)
+    {
+        if (tid == 0) atomicOr(&keptCnt[1 + b], 2);    // the order of NaN scores is whatever the caller's sort makes of them
+        return;
+    }
+    for (int i = tid; i < m; i += 256)
+    {
+        const unsigned long long a = keyA[i];
+        const unsigned bk = keyB[i];
+        int rank = 0;
+        for (int j = 0; j < m; ++j)
+        {
+            const unsigned long long oa = keyA[j];
+            rank += (oa > a || (oa == a && keyB[j] > bk)) ? 1 : 0;
+        }
+        const float *q = r + static_cast<size_t>(member[i]) * 8;
+        const float bx = q[0], by = q[1], bw = q[2], bh = q[3];
+        const float ax1 = bx - bw / 2.f, ax2 = bx + bw / 2.f, ay1 = by - bh / 2.f, ay2 = by + bh / 2.f;
+        sorted[rank] = member[i];
+        x1[rank] = ax1; x2[rank] = ax2; y1[rank] = ay1; y2[rank] = ay2;
+        area[rank] = (ax2 - ax1 + 1) * (ay2 - ay1 + 1);
+        gone[rank] = 0;
+    }
+    __syncthreads();
+    {
+        volatile unsigned char *g = gone;           // written by other threads between two reads; the barrier orders them
+        int picks = 0;
+        for (int i = 0; i < m; ++i)
+        {
+            if (g[i]) continue;                          // same answer in every thread
+            const float kx1 = x1[i], ky1 = y1[i], kx2 = x2[i], ky2 = y2[i], karea = area[i];
+            for (int j = i + 1 + tid; j < m; j += 256)
+                if (!g[j] && iouAbove(kx1, ky1, kx2, ky2, karea, x1[j], y1[j], x2[j], y2[j], area[j], thr)) g[j] = 1;
+            if (tid == 0) pickOf[i] = static_cast<unsigned short>(picks);
+            ++picks;
+            __syncthreads();
+        }
+        if (tid == 0) { nKept = picks; base = atomicAdd(&keptCnt[0], picks); }
+    }
+    __syncthreads();
+    const unsigned long long t = top;
+    const float topScore = __uint_as_float((static_cast<unsigned>(t >> 32) & 0x80000000u) ? (static_cast<unsigned>(t >> 32) & 0x7fffffffu) : ~static_cast<unsigned>(t >> 32));
+    const float topCell = static_cast<float>(~static_cast<unsigned>(t & 0xffffffffull));
+    for (int i = tid; i < m; i += 256)
+    {
+        if (gone[i]) continue;
+        const int pos = base + pickOf[i];
+        if (pos >= keptCap) continue;                    // (cannot happen with keptCap >= batch * candCap)
+        const float4 *q = reinterpret_cast<const float4 *>(r + static_cast<size_t>(sorted[i]) * 8);
+        float4 *o = reinterpret_cast<float4 *>(kept + static_cast<size_t>(pos) * 12);
+        o[0] = q[0]; o[1] = q[1];
+        o[2] = make_float4(topScore, topCell, static_cast<float>(pickOf[i]), static_cast<float>(b));
+    }
+}
+
+// The same procedure for a class with more than NMS_CAP members in an image (up to NMS_BIG): the members are sorted by a
+// bitonic network in LDS (keys and row indices, 128 KiB), the sorted row indices go to the workspace, then the corner
+// coordinates of all members take the keys' place in LDS and the whole workgroup runs the greedy pass (one barrier per pick).
+// state[i]: 0xffff = erased, 0xfffe = not visited yet, else the pick order.
+constexpr int NMS_BIG = 6144, NMS_SORT = 8192, NMS_SLOTS = NMS_BIG / 256;
+constexpr int NMS_BIG_LDS = NMS_SORT * 16 + NMS_BIG * 2;        // max(sort: 8+4+4 bytes per slot, boxes: 20 bytes per member) + state
+
+__global__ __launch_bounds__(256) void yoloNmsBigKernel(const float *__restrict__ rows, int candCap, const int *__restrict__ candCnt, float thr,
+                                                        float *__restrict__ kept, int keptCap, int *__restrict__ keptCnt,
+                                                        const int *__restrict__ bigCnt, int *__restrict__ wsSorted, int *__restrict__ wsUsed)
+{
+#pragma clang fp contract(off)
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    __shared__ unsigned long long top;
+    __shared__ int nMem, bad, base, off;
+    const int cls = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const int m = bigCnt[b * gridDim.x + cls];
+    if (m <= NMS_CAP) return;
+    if (m > NMS_BIG)
+    {
+        if (tid == 0) atomicOr(&keptCnt[1 + b], 1);
+        return;
+    }
+    unsigned long long *kA = reinterpret_cast<unsigned long long *>(smem);
+    unsigned *kB = reinterpret_cast<unsigned *>(smem + NMS_SORT * 8);
+    int *ix = reinterpret_cast<int *>(smem + NMS_SORT * 12);
+    int n = candCnt[b];
+    n = n < candCap ? n : candCap;
+    const float *r = rows + static_cast<size_t>(b) * candCap * 8;
+    if (tid == 0) { nMem = 0; bad = 0; top = 0ull; off = atomicAdd(&wsUsed[b], m); }
+    __syncthreads();
+    for (int k = tid; k < n; k += 256)
+    {
+        const float *q = r + static_cast<size_t>(k) * 8;
+        if (static_cast<int>(q[6]) != cls) continue;
+        const int slot = atomicAdd(&nMem, 1);
+        if (slot >= NMS_SORT) continue;
+        const float conf = q[4];
+        const float score = conf * q[5];
+        if (!(score == score) || !(conf == conf)) bad = 1;
+        const unsigned sb = orderedBits(score), cell = ~static_cast<unsigned>(q[7]);
+        kA[slot] = (static_cast<unsigned long long>(orderedBits(conf)) << 32) | sb;
+        kB[slot] = cell;
+        ix[slot] = k;
+        atomicMax(&top, (static_cast<unsigned long long>(sb) << 32) | cell);
+    }
+    __syncthreads();
+    if (bad || nMem != m || off + m > candCap)
+    {
+        if (tid == 0) atomicOr(&keptCnt[1 + b], bad ? 2 : 4);
+        return;
+    }
+    int S = 2048;
+    while (S < m) S <<= 1;
+    for (int i = m + tid; i < S; i += 256) { kA[i] = 0ull; kB[i] = 0u; ix[i] = -1; }       // below every real key (objectness > 0)
+    for (int k2 = 2; k2 <= S; k2 <<= 1)
+        for (int j = k2 >> 1; j > 0; j >>= 1)
+        {
+            __syncthreads();
+            for (int t = tid; t < S / 2; t += 256)
+            {
+                const int lo = ((t / j) * 2 * j) + (t % j), hi = lo + j;
+                const unsigned long long a0 = kA[lo], a1 = kA[hi];
+                const unsigned b0 = kB[lo], b1 = kB[hi];
+                const bool loLess = a0 < a1 || (a0 == a1 && b0 < b1);
+                const bool descending = (lo & k2) == 0;
+                if (loLess == descending)
+                {
+                    kA[lo] = a1; kA[hi] = a0; kB[lo] = b1; kB[hi] = b0;
+                    const int t0 = ix[lo]; ix[lo] = ix[hi]; ix[hi] = t0;
+                }
+            }
+        }
+    __syncthreads();
+    int *sortedRow = wsSorted + static_cast<size_t>(b) * candCap + off;
+    for (int i = tid; i < m; i += 256) sortedRow[i] = ix[i];
+    __syncthreads();                                             // the keys are dead from here on
+    float *x1 = reinterpret_cast<float *>(smem), *y1 = x1 + NMS_BIG, *x2 = y1 + NMS_BIG, *y2 = x2 + NMS_BIG, *area = y2 + NMS_BIG;
+    volatile unsigned short *state = reinterpret_cast<unsigned short *>(smem + NMS_SORT * 16);
+    // Every thread keeps its members (sorted positions tid, tid + 256, ...) in registers, so that the test against a pick is
+    // arithmetic only; LDS holds the same coordinates for the broadcast of the pick and the erased / picked state.
+    float rx1[NMS_SLOTS], ry1[NMS_SLOTS], rx2[NMS_SLOTS], ry2[NMS_SLOTS], rar[NMS_SLOTS];
+    unsigned alive = 0u;
+#pragma unroll
+    for (int t = 0; t < NMS_SLOTS; ++t)
+    {
+        const int i = t * 256 + tid;
+        rx1[t] = ry1[t] = rx2[t] = ry2[t] = rar[t] = 0.f;
+        if (i >= m) continue;
+        const float *q = r + static_cast<size_t>(sortedRow[i]) * 8;
+        const float bx = q[0], by = q[1], bw = q[2], bh = q[3];
+        const float ax1 = bx - bw / 2.f, ax2 = bx + bw / 2.f, ay1 = by - bh / 2.f, ay2 = by + bh / 2.f;
+        const float ar = (ax2 - ax1 + 1) * (ay2 - ay1 + 1);
+        x1[i] = ax1; x2[i] = ax2; y1[i] = ay1; y2[i] = ay2; area[i] = ar;
+        rx1[t] = ax1; rx2[t] = ax2; ry1[t] = ay1; ry2[t] = ay2; rar[t] = ar;
+        state[i] = 0xfffe;
+        alive |= 1u << t;
+    }
+    __syncthreads();
+    int picks = 0;
+    for (int i = 0;; ++i)
+    {
+        while (i < m && state[i] == 0xffff) ++i;                 // same answer in every thread: writes end at the barrier below
+        if (i >= m) break;
+        const float kx1 = x1[i], ky1 = y1[i], kx2 = x2[i], ky2 = y2[i], karea = area[i];
+#pragma unroll
+        for (int t = 0; t < NMS_SLOTS; ++t)
+        {
+            if (t * 256 + 255 <= i || t * 256 >= m) continue;    // (uniform) nothing of this slot lies behind the pick
+            const int j = t * 256 + tid;
+            if (j <= i || !((alive >> t) & 1u)) continue;
+            if (iouAbove(kx1, ky1, kx2, ky2, karea, rx1[t], ry1[t], rx2[t], ry2[t], rar[t], thr)) { alive &= ~(1u << t); state[j] = 0xffff; }
+        }
+        __syncthreads();
+        if (tid == 0) state[i] = static_cast<unsigned short>(picks);
+        ++picks;
+    }
+    if (tid == 0) base = atomicAdd(&keptCnt[0], picks);
+    __syncthreads();
+    const unsigned long long t = top;
+    const float topScore = __uint_as_float((static_cast<unsigned>(t >> 32) & 0x80000000u) ? (static_cast<unsigned>(t >> 32) & 0x7fffffffu) : ~static_cast<unsigned>(t >> 32));
+    const float topCell = static_cast<float>(~static_cast<unsigned>(t & 0xffffffffull));
+    for (int i = tid; i < m; i += 256)
+    {
+        const unsigned short st = state[i];
+        if (st == 0xffff) continue;
+        const int pos = base + st;
+        if (pos >= keptCap) continue;
+        const float4 *q = reinterpret_cast<const float4 *>(r + static_cast<size_t>(sortedRow[i]) * 8);
+        float4 *o = reinterpret_cast<float4 *>(kept + static_cast<size_t>(pos) * 12);
+        o[0] = q[0]; o[1] = q[1];
+        o[2] = make_float4(topScore, topCell, static_cast<float>(st), static_cast<float>(b));
+    }
+}
+
 __global__ __launch_bounds__(256) void yoloGatherKernel(const float *__restrict__ decoded, long long decStride, const int *__restrict__ candIdx,
                                                         int candCap, const int *__restrict__ candCnt, float *__restrict__ rows, int per,
                                                         int batch)
@@ -288,6 +571,35 @@ extern "C" int msnh_hip_yolo_gather(int batch, int classes, const float *decoded
     dim3 grid(gridFor(cand_cap, 256), batch);
     hipLaunchKernelGGL(yoloGatherKernel, grid, dim3(256), 0, resolveStream(s), decoded, decoded_batch_stride, cand_idx, cand_cap, cand_cnt,
                        rows, 5 + classes, batch);
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" size_t msnh_hip_yolo_nms_workspace_bytes(int batch, int classes, int cand_cap)
+{
+    if (batch <= 0 || classes <= 0 || cand_cap <= 0) return 0;
+    return sizeof(int) * (static_cast<size_t>(batch) * classes + static_cast<size_t>(batch) * cand_cap + static_cast<size_t>(batch));
+}
+
+extern "C" int msnh_hip_yolo_nms(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept,
+                                 int kept_cap, int *kept_cnt, void *workspace, size_t workspace_bytes, msnh_stream_t s)
+{
+    MSNH_REQUIRE(batch > 0 && batch <= 65535 && classes > 0 && cand_cap > 0 && cand_cap <= (1 << 24) && kept_cap > 0, "yolo_nms: bad geometry");
+    MSNH_REQUIRE(rows && cand_cnt && kept && kept_cnt, "yolo_nms: NULL pointer");
+    MSNH_REQUIRE(reinterpret_cast<uintptr_t>(rows) % 16 == 0 && reinterpret_cast<uintptr_t>(kept) % 16 == 0, "yolo_nms: rows and kept must be 16-byte aligned");
+    MSNH_REQUIRE(workspace == nullptr || (workspace_bytes >= msnh_hip_yolo_nms_workspace_bytes(batch, classes, cand_cap) && reinterpret_cast<uintptr_t>(workspace) % 4 == 0),
+                 "yolo_nms: workspace too small (msnh_hip_yolo_nms_workspace_bytes)");
+    hipStream_t st = resolveStream(s);
+    int *bigCnt = static_cast<int *>(workspace);
+    int *wsSorted = bigCnt ? bigCnt + static_cast<size_t>(batch) * classes : nullptr;
+    int *wsUsed = bigCnt ? wsSorted + static_cast<size_t>(batch) * cand_cap : nullptr;
+    hipLaunchKernelGGL(yoloNmsKernel, dim3(classes, batch), dim3(256), 0, st, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, bigCnt, wsUsed);
+    MSNH_LAUNCH_CHECK();
+    if (workspace == nullptr) return 0;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsBigKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_BIG_LDS);
+    if (e != hipSuccess) { setError("hipFuncSetAttribute: %s", hipGetErrorString(e)); return 1; }
+    hipLaunchKernelGGL(yoloNmsBigKernel, dim3(classes, batch), dim3(256), NMS_BIG_LDS, st, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt,
+                       bigCnt, wsSorted, wsUsed);
     MSNH_LAUNCH_CHECK();
     return 0;
 }

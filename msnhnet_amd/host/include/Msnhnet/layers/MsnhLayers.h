@@ -353,6 +353,12 @@ public:
     std::vector<bool> batchHasBox;
     std::vector<std::vector<YoloBox>> finalOut;
     static bool keepClassScores;           // also fill YoloBox::classesVal (costs an extra device->host copy)
+    // hard NMS on the device (only the kept boxes are copied back): 0 = never (sort + NMS on the host), 2 = always,
+    // 1 = while the previous result of this network had at most kDeviceNmsCandidates candidates in every image (default): the
+    // device kernels give one workgroup to a class of an image, which beats the host for the hundreds of candidates real
+    // detections have and loses to its threads when a class has thousands.
+    static int deviceNms;
+    static const int kDeviceNmsCandidates = 2048;
 
     // host post-processing of the compacted candidate rows of one image (8 floats per row, see msnh_hip_yolo_gather)
     std::vector<YoloBox> boxesFromRows(const float *rows, int count, const float *decodedOfImage) const;
@@ -368,8 +374,16 @@ private:
     int _yoloAllInputNum = 0, _pixels = 0;
     // devCnt / devRows: device-side snapshot of one forward's candidates, so the copy to the host can run on its own
     // stream while the next forward already overwrites the plan's buffers
-    struct Slot { PinnedBuffer cnt, rows, decoded; DeviceBuffer devCnt, devRows; msnh_event_t event = nullptr, ready = nullptr; bool pending = false; };
-    msnh_stream_t _copyStream = nullptr;
+    struct Slot
+    {
+        PinnedBuffer cnt, rows, decoded, kept, keptCnt;
+        DeviceBuffer devCnt, devRows, devKept, devKeptCnt, devNmsWs;
+        msnh_event_t event = nullptr, ready = nullptr;
+        bool pending = false, onDevice = false;
+    };
+    std::vector<YoloBox> boxesFromKept(std::vector<const float *> &records) const;
+    msnh_stream_t _copyStream = nullptr, _fetchStream = nullptr;
+    int _lastMaxCandidates = 0;            // largest per-image candidate count of the previous result
     Slot _slots[2];
 };
 }

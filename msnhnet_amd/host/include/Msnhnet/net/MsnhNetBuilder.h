@@ -28,6 +28,9 @@ public:
     static void setAutoTune(const bool &on);
     // keep the per-layer tile / algorithm choices next to the weights file ("<path>.msnhbin.tune"): the next load of the same
     // graph on the same device skips the search.  Off by default (the library then writes no files).
+    // hard NMS of detection networks: 0 = candidates are copied back and sorted / suppressed on the host, 2 = on the device (only
+    // kept boxes are copied back), 1 (default) = on the device while the previous result had at most 2048 candidates per image
+    static void setDeviceNms(const int &mode);
     static void setTuneCache(const bool &on);
     static bool tuneCache;
     static void setUseWinograd(const bool &on);   // float16 plans: 3x3 stride-1 convolutions through Winograd F(2x2,3x3)

@@ -181,6 +181,7 @@ int msnhnet_destroy(msnhnet_t net)
 
 int msnhnet_set_use_fp16(int on) { return guarded([&] { NetBuilder::setUseFp16(on != 0); }); }
 int msnhnet_set_use_winograd(int on) { return guarded([&] { NetBuilder::setUseWinograd(on != 0); }); }
+int msnhnet_set_device_nms(int mode) { return guarded([&] { NetBuilder::setDeviceNms(mode); }); }
 int msnhnet_set_tune_cache(int on) { return guarded([&] { NetBuilder::setTuneCache(on != 0); }); }
 int msnhnet_set_keep_class_scores(int on) { return guarded([&] { NetBuilder::setKeepClassScores(on != 0); }); }
 int msnhnet_set_save_layer_output(msnhnet_t net, int on) { return guarded([&] { nb(net).setSaveLayerOutput(on != 0); }); }

@@ -1128,6 +1128,9 @@ int YoloLayer::lower(Plan &plan, int in, int layerIndex)
 }
 
 bool YoloOutLayer::keepClassScores = false;
+int YoloOutLayer::deviceNms = 1;
+static const size_t kRecordBytes = 12 * sizeof(float);     // one record of msnh_hip_yolo_nms
+static const size_t kQuickRecords = 2048;                   // records copied back with the counters, before their number is known
 
 YoloOutLayer::YoloOutLayer(const int &batch, const int &orgWidth, const int &orgHeight, std::vector<int> &yoloIndexes, std::vector<YoloInfo> &yoloLayersInfo,
                            const float &confThresh, const float &nmsThresh, const int &useSotfNms, const YoloType &yoloType)
@@ -1397,9 +1400,51 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
     MSNH_DEV(msnh_hip_event_record(sl.ready, s));
     MSNH_DEV(msnh_hip_stream_wait_event(_copyStream, sl.ready));
     MSNH_DEV(msnh_hip_memcpy_d2h(sl.cnt.ptr(), sl.devCnt.ptr(), cntBytes, _copyStream));
-    MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.ptr(), sl.devRows.ptr(), rowBytes, _copyStream));
+    sl.onDevice = !_useSoftNms && (deviceNms == 2 || (deviceNms == 1 && _lastMaxCandidates <= kDeviceNmsCandidates));
+    if (sl.onDevice)
+    {
+        // NMS on the snapshot, on the copy stream: it overlaps the next forward, and what crosses PCIe is the kept boxes
+        // (the first kQuickRecords of them with the counters; finish() fetches the rest if there are more)
+        const size_t keptCntBytes = sizeof(int) * (1 + static_cast<size_t>(_batch));
+        const size_t keptCap = cells * static_cast<size_t>(_batch);
+        if (sl.devKeptCnt.bytes() < keptCntBytes) sl.devKeptCnt.alloc(keptCntBytes);
+        if (sl.devKept.bytes() < keptCap * kRecordBytes) sl.devKept.alloc(keptCap * kRecordBytes);
+        sl.keptCnt.reserve(keptCntBytes);
+        sl.kept.reserve(std::min(keptCap, kQuickRecords) * kRecordBytes);
+        MSNH_DEV(msnh_hip_fill_zero(sl.devKeptCnt.ptr(), keptCntBytes, _copyStream));
+        const size_t wsBytes = msnh_hip_yolo_nms_workspace_bytes(_batch, _channel - 5, pl.yoloCells);
+        if (sl.devNmsWs.bytes() < wsBytes) sl.devNmsWs.alloc(wsBytes);
+        MSNH_DEV(msnh_hip_yolo_nms(_batch, _channel - 5, sl.devRows.as<float>(), pl.yoloCells, sl.devCnt.as<int>(), _nmsThresh, sl.devKept.as<float>(),
+                                   static_cast<int>(keptCap), sl.devKeptCnt.as<int>(), sl.devNmsWs.ptr(), wsBytes, _copyStream));
+        MSNH_DEV(msnh_hip_memcpy_d2h(sl.keptCnt.ptr(), sl.devKeptCnt.ptr(), keptCntBytes, _copyStream));
+        MSNH_DEV(msnh_hip_memcpy_d2h(sl.kept.ptr(), sl.devKept.ptr(), std::min(keptCap, kQuickRecords) * kRecordBytes, _copyStream));
+    }
+    else
+        MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.ptr(), sl.devRows.ptr(), rowBytes, _copyStream));
     MSNH_DEV(msnh_hip_event_record(sl.event, _copyStream));
     sl.pending = true;
+}
+
+// Boxes of one image from the device's NMS records, in the reference's output order: classes by the first appearance in
+// the score-sorted candidate list (= by their best-scoring candidate), inside a class in pick order.
+std::vector<YoloBox> YoloOutLayer::boxesFromKept(std::vector<const float *> &records) const
+{
+    std::sort(records.begin(), records.end(), [](const float *a, const float *b) {
+        if (a[8] != b[8]) return a[8] > b[8];
+        if (a[9] != b[9]) return a[9] < b[9];
+        return a[10] < b[10];
+    });
+    std::vector<YoloBox> out(records.size());
+    for (size_t i = 0; i < records.size(); ++i)
+    {
+        const float *r = records[i];
+        YoloBox &b = out[i];
+        b.xywhBox = Box::XYWHBox(r[0], r[1], r[2], r[3]);
+        b.conf = r[4];
+        b.bestClsConf = r[5];
+        b.bestClsIdx = static_cast<int>(r[6]);
+    }
+    return out;
 }
 
 void YoloOutLayer::finish(int slot)
@@ -1413,6 +1458,49 @@ void YoloOutLayer::finish(int slot)
     const int cells = plan->yoloCells;
     const int per = _channel;
     const int *cnt = sl.cnt.as<int>();
+    _lastMaxCandidates = 0;
+    for (int b = 0; b < _batch; ++b) _lastMaxCandidates = std::max(_lastMaxCandidates, std::min(cnt[b], cells));
+    if (sl.onDevice)
+    {
+        const int *keptCnt = sl.keptCnt.as<int>();
+        const size_t total = static_cast<size_t>(keptCnt[0]);
+        // (its own stream: the copy stream may already hold the next forward's work)
+        if (_fetchStream == nullptr) MSNH_DEV(msnh_hip_stream_create(&_fetchStream));
+        if (total > kQuickRecords)
+        {
+            PinnedBuffer &rest = sl.rows;                                  // the host path's buffer doubles as the overflow area
+            rest.reserve((total - kQuickRecords) * kRecordBytes);
+            MSNH_DEV(msnh_hip_memcpy_d2h(rest.ptr(), sl.devKept.as<char>() + kQuickRecords * kRecordBytes, (total - kQuickRecords) * kRecordBytes, _fetchStream));
+            MSNH_DEV(msnh_hip_stream_sync(_fetchStream));
+        }
+        std::vector<std::vector<const float *>> perImage(static_cast<size_t>(_batch));
+        for (size_t i = 0; i < total; ++i)
+        {
+            const float *r = i < kQuickRecords ? sl.kept.as<float>() + i * 12 : sl.rows.as<float>() + (i - kQuickRecords) * 12;
+            const int b = static_cast<int>(r[11]);
+            if (b < 0 || b >= _batch) MSNH_THROW("YoloOut: device NMS record names image " + std::to_string(b));
+            perImage[static_cast<size_t>(b)].push_back(r);
+        }
+        batchHasBox.assign(static_cast<size_t>(_batch), false);
+        finalOut.assign(static_cast<size_t>(_batch), std::vector<YoloBox>());
+#pragma omp parallel for schedule(dynamic)
+        for (int b = 0; b < _batch; ++b)
+            if (keptCnt[1 + b] == 0) finalOut[static_cast<size_t>(b)] = boxesFromKept(perImage[static_cast<size_t>(b)]);
+        std::vector<float> hostRows;
+        for (int b = 0; b < _batch; ++b)
+        {
+            batchHasBox[static_cast<size_t>(b)] = cnt[b] > 0;
+            if (keptCnt[1 + b] == 0) continue;
+            // the device left this image to the host (a class with very many candidates, or NaN scores): the snapshot still holds its rows
+            const int n = std::min(cnt[b], cells);
+            hostRows.resize(static_cast<size_t>(n) * 8);
+            MSNH_DEV(msnh_hip_memcpy_d2h(hostRows.data(), sl.devRows.as<float>() + static_cast<size_t>(b) * cells * 8, hostRows.size() * sizeof(float), _fetchStream));
+            MSNH_DEV(msnh_hip_stream_sync(_fetchStream));
+            finalOut[static_cast<size_t>(b)] = nmsSorted(boxesFromRows(hostRows.data(), n, nullptr), _nmsThresh);
+        }
+        if (std::getenv("MSNH_DEBUG_TIMING")) std::fprintf(stderr, "yoloout finish (device NMS, %zu boxes): wait %.3f ms, host %.3f ms\n", total, dbgWait, TimeUtil::getElapsedTime(dbg0) - dbgWait);
+        return;
+    }
     const float *decodedHost = keepClassScores ? sl.decoded.as<float>() : nullptr;
     batchHasBox.assign(static_cast<size_t>(_batch), false);
     finalOut.assign(static_cast<size_t>(_batch), std::vector<YoloBox>());
@@ -1468,5 +1556,6 @@ YoloOutLayer::~YoloOutLayer()
         if (sl.ready) msnh_hip_event_destroy(sl.ready);
     }
     if (_copyStream) msnh_hip_stream_destroy(_copyStream);
+    if (_fetchStream) msnh_hip_stream_destroy(_fetchStream);
 }
 }

@@ -42,6 +42,11 @@ void NetBuilder::setOnlyGpu(const bool &onlyGpu) { BaseLayer::setOnlyGpu(onlyGpu
 void NetBuilder::setUseFp16(const bool &useFp16) { BaseLayer::setUseFp16(useFp16); }
 void NetBuilder::setForceUseCuda(const bool &v) { BaseLayer::setForceUseCuda(v); }
 void NetBuilder::setKeepClassScores(const bool &keep) { YoloOutLayer::keepClassScores = keep; }
+void NetBuilder::setDeviceNms(const int &mode)
+{
+    if (mode < 0 || mode > 2) throw Exception(1, "setDeviceNms: mode must be 0 (host), 1 (by candidate count) or 2 (device)", __FILE__, __LINE__, __FUNCTION__);
+    YoloOutLayer::deviceNms = mode;
+}
 bool NetBuilder::autoTune = true;
 void NetBuilder::setAutoTune(const bool &on) { autoTune = on; }
 bool NetBuilder::tuneCache = false;

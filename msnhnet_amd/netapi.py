@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libMsnhnet.so")
 
 SYMBOLS = [
     "initMsnhnet", "buildMsnhnet", "runClassifyNoPred", "runYoloNoPred", "dispose", "withGPU", "withCUDNN", "getCpuForwardTime",
-    "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16", "msnhnet_set_use_winograd", "msnhnet_set_tune_cache", "msnhnet_set_input_image_u8", "msnhnet_boxes_to_image",
+    "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16", "msnhnet_set_use_winograd", "msnhnet_set_tune_cache", "msnhnet_set_device_nms", "msnhnet_set_input_image_u8", "msnhnet_boxes_to_image",
     "msnhnet_set_keep_class_scores", "msnhnet_set_save_layer_output", "msnhnet_build", "msnhnet_load", "msnhnet_load_from_memory",
     "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops",
     "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
@@ -68,6 +68,7 @@ def lib():
     L.msnhnet_set_use_fp16.argtypes = [ci]
     L.msnhnet_set_use_winograd.argtypes = [ci]
     L.msnhnet_set_tune_cache.argtypes = [ci]
+    L.msnhnet_set_device_nms.argtypes = [ci]
     L.msnhnet_set_input_image_u8.argtypes = [vp, ci, ctypes.POINTER(ctypes.c_ubyte), ci, ci, ci, ci]
     L.msnhnet_boxes_to_image.argtypes = [fp, ll, ci, ci, ci, ci, ci]
     L.msnhnet_set_keep_class_scores.argtypes = [ci]
@@ -123,6 +124,11 @@ def boxes_to_image(boxes, net_w, net_h, org_w, org_h, padded=True):
     b = np.ascontiguousarray(boxes, np.float32).reshape(-1, 7).copy()
     _check(lib().msnhnet_boxes_to_image(_fp(b), len(b), net_w, net_h, org_w, org_h, int(padded)))
     return b
+
+
+def set_device_nms(mode):
+    """0 host, 1 by the previous result's candidate count (default), 2 device"""
+    _check(lib().msnhnet_set_device_nms(int(mode)))
 
 
 def set_tune_cache(on):

@@ -265,6 +265,33 @@ def test_tune_cache(tmp_path):
         netapi.set_tune_cache(False)
 
 
+@pytest.mark.parametrize("arch,size,batch", [("yolov3", 224, 3), ("yolov3_tiny", 160, 2), ("yolov5s", 128, 2)])
+def test_device_nms_equals_host_nms(arch, size, batch):
+    """same network, same input: boxes from the device's NMS (the default) and from the host's sort + NMS are identical,
+    eagerly and with two forwards in flight"""
+    net, binp, g = nu.model(arch, batch, size, seed=3)
+    xs = [zoo.seeded_input(batch, 3, size, size, seed=s) for s in (4, 5, 6)]
+    print("device nms", arch, size, batch, flush=True)
+    m = netapi.Net(net, binp, fp16=True)
+    try:
+        netapi.set_device_nms(2)
+        got = [m.run_yolo(x) for x in xs]
+        netapi.set_device_nms(0)
+        want = [m.run_yolo(x) for x in xs]
+        netapi.set_device_nms(1)
+        auto = [m.run_yolo(x) for x in xs]
+        with pytest.raises(netapi.MsnhnetError):
+            netapi.set_device_nms(3)
+    finally:
+        netapi.set_device_nms(1)
+    got += auto
+    want += want
+    assert sum(len(b) for w in want for b in w) > 0
+    for g_, w_ in zip(got, want):
+        for b in range(batch):
+            assert np.array_equal(g_[b], w_[b], equal_nan=True)
+
+
 def test_image_in_boxes_out():
     """8-bit images of different shapes -> device letterbox -> forward -> boxes in original-image pixels: equals the
     float path fed with the restatement's letterbox, followed by the restatement's rescale."""

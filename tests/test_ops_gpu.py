@@ -349,6 +349,87 @@ def test_yolo_decode(dtype, version):
             assert int(rows[b, k, 6]) == int(np.argmax(r[5:]))
 
 
+def _ordered_records(kept, total, image):
+    rec = kept[:total]
+    rec = rec[rec[:, 11] == image]
+    order = sorted(range(len(rec)), key=lambda i: (-rec[i, 8], rec[i, 9], rec[i, 10]))
+    return rec[order]
+
+
+def test_yolo_nms():
+    """device NMS records, put in the documented order, are the reference procedure's boxes bit for bit: objectness and
+    class scores on a coarse grid (many exact ties in both sort keys), heavy overlap, boxes of infinite extent (NaN IoU
+    never suppresses), an empty image, a sparse image, and an image with 1200 / 6100 members in one class (the large-class
+    kernel, which needs the workspace); an image with more members than that, an image with a NaN score -- and without a
+    workspace every image with more than 1024 members in a class -- are flagged instead"""
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(21)
+    cls, h, w = 6, 48, 48
+    per, hw = 5 + cls, 48 * 48
+    cells = 3 * hw                     # 6912
+    conf_t, nms_t = 0.5, 0.45
+    heads = []
+    for b in range(7):
+        d = np.zeros((3 * per, h, w), np.float32)
+        v = d.reshape(3, per, hw)
+        v[:, 0] = rng.uniform(0, 400, (3, hw)); v[:, 1] = rng.uniform(0, 400, (3, hw))
+        v[:, 2] = rng.uniform(10, 70, (3, hw)); v[:, 3] = rng.uniform(10, 70, (3, hw))
+        v[:, 4] = rng.integers(0, 17, (3, hw)) / 16.0
+        v[:, 5:] = rng.integers(0, 9, (3, cls, hw)) / 8.0
+        if b == 0:
+            v[1, 2, 5:9] = np.inf
+        if b in (1, 5, 6):             # one class holds 1200 / 6100 / 6912 candidates, the other classes a few
+            keep = {1: 1200, 5: 6100, 6: cells}[b]
+            v[:, 5] = 2.0
+            obj = np.zeros(cells, np.float32)
+            obj[rng.permutation(cells)[:keep]] = rng.integers(9, 17, keep) / 16.0
+            v[:, 4] = obj.reshape(3, hw)
+            v[0, 5, :7] = 0.0; v[0, 6, :7] = 3.0
+        if b == 2:
+            v[:, 4] = 0.0              # no candidate at all
+        if b == 4:
+            v[:, 4] = np.where(rng.uniform(size=(3, hw)) < 0.01, 0.8, 0.1)    # a sparse image, like real detections
+        heads.append(d)
+    rows = np.zeros((7, cells, 8), np.float32)
+    cnt = np.zeros(7, np.int32)
+    for b, d in enumerate(heads):
+        flat = d.reshape(3, per, hw).transpose(0, 2, 1).reshape(cells, per)
+        cand = np.nonzero(flat[:, 4] > conf_t)[0]
+        rng.shuffle(cand)
+        cnt[b] = len(cand)
+        r = rows[b, :len(cand)]
+        r[:, :5] = flat[cand, :5]
+        r[:, 5] = flat[cand, 5:].max(1); r[:, 6] = flat[cand, 5:].argmax(1); r[:, 7] = cand
+    rows[3, 7, 5] = np.nan             # image 3: a NaN class score
+    rd, cd = gu.dev(rows), gu.dev(cnt)
+    nbytes = abi.lib().msnh_hip_yolo_nms_workspace_bytes(7, cls, cells)
+    ws = torch.full((nbytes // 4,), 0x55555555, dtype=torch.int32).cuda()
+    print("yolo_nms", cnt.tolist(), flush=True)
+    for with_ws, flags in ((True, [0, 0, 0, 2, 0, 0, 1]), (False, [0, 1, 0, 2, 0, 1, 1])):
+        keptd = torch.zeros((7 * cells, 12), dtype=torch.float32).cuda()
+        kcd = torch.zeros(8, dtype=torch.int32).cuda()
+        gu.sync()
+        abi.check(abi.lib().msnh_hip_yolo_nms(7, cls, gu.ptr(rd), cells, gu.ptr(cd), nms_t, gu.ptr(keptd), 7 * cells, gu.ptr(kcd),
+                                              gu.ptr(ws) if with_ws else None, nbytes if with_ws else 0, None))
+        gu.sync()
+        kc = kcd.cpu().numpy()
+        kept = keptd.cpu().numpy()
+        assert kc[1:].tolist() == flags, kc
+        total = int(kc[0])
+        for b in range(7):
+            if flags[b]:
+                continue
+            want = on.yolo_out([heads[b]], cls, conf_t, nms_t)
+            got = _ordered_records(kept, total, b)
+            assert len(want) == len(got), (b, len(want), len(got))
+            assert np.array_equal(got[:, :7], want, equal_nan=True), b
+            assert (b == 2) == (len(got) == 0)
+    assert len(on.yolo_out([heads[0]], cls, conf_t, nms_t)) > 100
+    with pytest.raises(abi.HipError):
+        abi.check(abi.lib().msnh_hip_yolo_nms(5, cls, gu.ptr(rd), cells, gu.ptr(cd), nms_t, None, 7 * cells, gu.ptr(kcd), None, 0, None))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_absmax(dtype):
     import gpuutil as gu
