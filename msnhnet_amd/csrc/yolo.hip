@@ -229,12 +229,12 @@ __global__ __launch_bounds__(256) void yoloNmsKernel(const float *__restrict__ r
     __shared__ unsigned short pickOf[NMS_CAP];
     __shared__ unsigned char gone[NMS_CAP];
     __shared__ unsigned long long top;
-    __shared__ int nMem, bad, nKept, base;
+    __shared__ int nMem, bad, base;
     const int cls = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
     int n = candCnt[b];
     n = n < candCap ? n : candCap;
     const float *r = rows + static_cast<size_t>(b) * candCap * 8;
-    if (tid == 0) { nMem = 0; bad = 0; top = 0ull; nKept = 0; }
+    if (tid == 0) { nMem = 0; bad = 0; top = 0ull; }
     if (wsUsed != nullptr && cls == 0 && tid == 0) wsUsed[b] = 0;       // yoloNmsBigKernel's cursor into the image's workspace
     __syncthreads();
     for (int k = tid; k < n; k += 256)
@@ -301,7 +301,7 @@ __global__ __launch_bounds__(256) void yoloNmsKernel(const float *__restrict__ r
             ++picks;
             __syncthreads();
         }
-        if (tid == 0) { nKept = picks; base = atomicAdd(&keptCnt[0], picks); }
+        if (tid == 0) base = atomicAdd(&keptCnt[0], picks);
     }
     __syncthreads();
     const unsigned long long t = top;
