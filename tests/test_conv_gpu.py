@@ -166,7 +166,9 @@ def test_conv_depthwise(c, h, w, k, stride, pad, dtype):
 
 
 @pytest.mark.parametrize("out_dtype", [abi.F32, abi.F16])
-@pytest.mark.parametrize("h,w,oc,k,stride,pad", [(33, 31, 32, 3, 1, 1), (40, 40, 64, 7, 2, 3), (25, 27, 32, 3, 2, 1), (70, 100, 64, 3, 1, 1)])
+@pytest.mark.parametrize("h,w,oc,k,stride,pad", [(33, 31, 32, 3, 1, 1), (40, 40, 64, 7, 2, 3), (25, 27, 32, 3, 2, 1), (70, 100, 64, 3, 1, 1),
+                                                 (37, 45, 64, 7, 2, 3), (30, 70, 32, 7, 1, 3), (21, 19, 128, 7, 2, 0), (224, 224, 64, 7, 2, 3),
+                                                 (9, 150, 64, 7, 2, 5), (31, 33, 64, 5, 2, 2)])
 def test_conv_stem(h, w, oc, k, stride, pad, out_dtype):
     """first layer: NCHW float32 in, NHWC out, cast fused"""
     import gpuutil as gu
