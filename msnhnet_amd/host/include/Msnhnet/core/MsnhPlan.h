@@ -111,6 +111,7 @@ public:
     int consumerCount(int tensor) const;
 
     void fuse();                            // passes 1
+    void chainMaxPools();                   // stride-1 max-pools of one tensor (SPP): each larger window reads the next smaller one's result
     void aliasConcats();                    // pass 2
     void applyCalibration(const Plan &calibrated);   // pass 3: take amax from an executed float32 twin
     void place();                           // pass 4 + arena allocation

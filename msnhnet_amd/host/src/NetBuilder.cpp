@@ -387,6 +387,7 @@ void NetBuilder::finalizePlan()
     const int dtype = BaseLayer::useFp16 ? MSNH_F16 : MSNH_F32;
     std::unique_ptr<Plan> plan = lowerNetwork(dtype);
     plan->fuse();
+    plan->chainMaxPools();
     plan->aliasConcats();
 
     if (dtype == MSNH_F16)
@@ -395,6 +396,7 @@ void NetBuilder::finalizePlan()
         // float16 tensor.  The float32 twin is lowered and optimised identically, so tensor ids line up.
         std::unique_ptr<Plan> cal = lowerNetwork(MSNH_F32);
         cal->fuse();
+        cal->chainMaxPools();
         cal->aliasConcats();
         cal->place();
         setupYoloBuffers(*cal, _net->batch);

@@ -185,6 +185,57 @@ void Plan::fuse()
     }
 }
 
+// ---- pass 1b: stride-1 max-pools over one tensor (SPP blocks: 5, 9, 13) ---------------------------------------------
+// With -FLT_MAX padding and stride 1, a window of a + b - 1 is the window b over the result of the window a, exactly
+// (max is associative and the clipped windows compose).  So the pools of one input run smallest first and each larger one
+// reads its predecessor through the difference window: 5, 5 over 5, 5 over 9 -- 75 taps per output instead of 275.
+void Plan::chainMaxPools()
+{
+    const auto eligible = [&](const PlanOp &op) {
+        return !op.dead && op.kind == PlanOp::MAXPOOL && op.stride == 1 && op.ksize % 2 == 1 && op.pad == op.ksize / 2;
+    };
+    std::vector<bool> done(ops.size(), false);
+    for (size_t i = 0; i < ops.size(); ++i)
+    {
+        if (done[i] || !eligible(ops[i])) continue;
+        std::vector<size_t> slots;
+        for (size_t j = i; j < ops.size(); ++j)
+            if (!done[j] && eligible(ops[j]) && ops[j].in0 == ops[i].in0) { slots.push_back(j); done[j] = true; }
+        if (slots.size() < 2) continue;
+        // the members change places inside their own slots only; nothing between them may read one of them, and with
+        // per-layer outputs kept (pinned) every member must belong to the same layer, whose ops run as one unit
+        bool ok = true;
+        for (size_t k = slots.front(); k <= slots.back() && ok; ++k)
+        {
+            if (std::find(slots.begin(), slots.end(), k) != slots.end() || ops[k].dead) continue;
+            for (size_t m : slots)
+                if (ops[k].in0 == ops[m].out || ops[k].in1 == ops[m].out) ok = false;
+        }
+        for (size_t m : slots)
+        {
+            if (ops[m].layerIndex != ops[slots.front()].layerIndex && (tensors[static_cast<size_t>(ops[m].out)].pinned || tensors[static_cast<size_t>(ops[slots.front()].out)].pinned)) ok = false;
+            for (size_t m2 : slots)
+                if (m2 != m && ops[m2].ksize == ops[m].ksize) ok = false;
+        }
+        if (!ok) continue;
+        std::vector<size_t> byK(slots);
+        std::sort(byK.begin(), byK.end(), [&](size_t a, size_t b) { return ops[a].ksize < ops[b].ksize; });
+        std::vector<PlanOp> moved;
+        for (size_t m : byK) moved.push_back(std::move(ops[m]));
+        for (size_t q = 0; q < slots.size(); ++q) ops[slots[q]] = std::move(moved[q]);
+        int prevK = ops[slots[0]].ksize;
+        for (size_t q = 1; q < slots.size(); ++q)
+        {
+            PlanOp &cur = ops[slots[q]];
+            const int k = cur.ksize;
+            cur.in0 = ops[slots[q - 1]].out;
+            cur.ksize = k - prevK + 1;
+            cur.pad = cur.ksize / 2;
+            prevK = k;
+        }
+    }
+}
+
 // ---- pass 2: concat aliasing ---------------------------------------------------------------------------------------
 void Plan::aliasConcats()
 {
@@ -777,6 +828,7 @@ std::string Plan::describe() const
         os << "  L" << op.layerIndex << " " << kinds[op.kind];
         if (op.kind == PlanOp::CONV)
             os << "[" << algos[op.algo] << (op.tile ? " t" + std::to_string(op.tile) : std::string()) << " k" << op.ksize << " s" << op.stride << " g" << op.groups << (op.in1 >= 0 ? " +res" : "") << (op.src2 ? " +bn" : "") << "]";
+        if (op.kind == PlanOp::MAXPOOL || op.kind == PlanOp::AVGPOOL) os << "[k" << op.ksize << " s" << op.stride << " p" << op.pad << "]";
         os << " " << in.n << "x" << in.h << "x" << in.w << "x" << in.c << " -> " << out.h << "x" << out.w << "x" << out.c
            << (out.dtype == MSNH_F16 ? " f16" : " f32") << " e" << out.scaleExp;
         if (out.parent >= 0) os << " (slice@" << chanOffsetInRoot(op.out) << " of " << tensors[static_cast<size_t>(root(op.out))].c << ")";

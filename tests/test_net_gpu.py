@@ -292,6 +292,16 @@ def test_device_nms_equals_host_nms(arch, size, batch):
             assert np.array_equal(g_[b], w_[b], equal_nan=True)
 
 
+def test_spp_maxpools_run_as_a_chain():
+    """the 5 / 9 / 13 pools of an SPP block become three 5-wide pools, each reading the one before (same results: the
+    per-layer and final-output parity tests of yolov4 and yolov5s run through this plan)"""
+    for arch, size in (("yolov4", 160), ("yolov5s", 160)):
+        net, binp, g = nu.model(arch, 1, size, seed=3)
+        m = netapi.Net(net, binp, fp16=True)
+        pools = [ln for ln in m.plan_detail().splitlines() if " maxpool[" in ln and " s1 " in ln]
+        assert len(pools) == 3 and all("[k5 s1 p2]" in ln for ln in pools), pools
+
+
 def test_image_in_boxes_out():
     """8-bit images of different shapes -> device letterbox -> forward -> boxes in original-image pixels: equals the
     float path fed with the restatement's letterbox, followed by the restatement's rescale."""

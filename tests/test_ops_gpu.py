@@ -85,6 +85,30 @@ def test_maxpool(c, h, w, k, s, p, dtype):
     assert np.array_equal(gu.nchw_host(yd, c), ref)          # max is exact
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("h,w", [(19, 19), (7, 5), (2, 2)])
+def test_maxpool_windows_compose(h, w, dtype):
+    """stride 1, -FLT_MAX padding: the 9 and 13 windows equal a 5 window over the 5 and the 9 result bit for bit (what the
+    plan relies on when it runs the pools of an SPP block as a chain)"""
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(h * 31 + w)
+    c = 24
+    x = _x(rng, (2, c, h, w), dtype)
+    xd = gu.nhwc_dev(x, dtype)
+    out = {}
+    for name, src, k in (("5", xd, 5), ("9", xd, 9), ("13", xd, 13)):
+        out[name] = torch.zeros((2, h, w, c), dtype=gu.TORCH_DT[dtype]).cuda()
+        abi.check(abi.lib().msnh_hip_maxpool(dtype, 2, h, w, c, gu.ptr(src), c, k, 1, k // 2, h, w, gu.ptr(out[name]), c, None))
+    for name, src in (("5o5", out["5"]), ("5o9", out["9"])):
+        out[name] = torch.zeros((2, h, w, c), dtype=gu.TORCH_DT[dtype]).cuda()
+        gu.sync()
+        abi.check(abi.lib().msnh_hip_maxpool(dtype, 2, h, w, c, gu.ptr(src), c, 5, 1, 2, h, w, gu.ptr(out[name]), c, None))
+    gu.sync()
+    assert np.array_equal(gu.nchw_host(out["13"], c), on.maxpool(x, 13, 1, 6))
+    assert torch.equal(out["5o5"], out["9"]) and torch.equal(out["5o9"], out["13"])
+
+
 @pytest.mark.parametrize("dtype,out_dtype", [(abi.F32, abi.F32), (abi.F16, abi.F16), (abi.F16, abi.F32)])
 @pytest.mark.parametrize("c,h,w,k,s,p", [(512, 7, 7, 7, 1, 0), (24, 9, 9, 3, 2, 1)])
 def test_avgpool(c, h, w, k, s, p, dtype, out_dtype):
