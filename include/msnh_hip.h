@@ -250,7 +250,8 @@ int msnh_hip_yolo_decode(int dtype, int batch, int h, int w, int classes, const 
  * decode would give them; the rest of `decoded` is left as it is): an objectness scan over the head, then one row per
  * candidate.  For callers that only consume the candidates.  Arguments as for msnh_hip_yolo_decode; cand_idx and cand_cnt are
  * required.  rows, if not NULL: [batch][cand_cap][8] float32; the compact row of every candidate of this head is written at the
- * candidate's position in the list, exactly what msnh_hip_yolo_gather would produce for it (that call is then unnecessary). */
+ * candidate's position in the list, exactly what msnh_hip_yolo_gather would produce for it (that call is then unnecessary).
+ * decoded may be NULL when rows is given: nothing but the compact rows is written then. */
 int msnh_hip_yolo_decode_candidates(int dtype, int batch, int h, int w, int classes, const void *x, int x_ld, float x_mul,
                                     const float *anchors6, float ratio, int yolo_version, float *decoded,
                                     long long decoded_batch_stride, float conf_thresh, int *cand_idx, int cand_cap, int cand_base,

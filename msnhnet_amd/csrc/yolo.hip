@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void yoloRowsKernel(const T *__restrict__ x, i
         for (int m = lane; m < per; m += 64)
         {
             const float v = yoloDecodeOne<V5>(xMul * toF(xr[m]), m, px, py, a, an, ratio);
-            dr[m] = v;
+            if (decoded != nullptr) dr[m] = v;
             if (m == lane) first = v;
             if (m >= 5 && v > bv) { bv = v; bi = m - 5; }
         }
@@ -539,7 +539,7 @@ extern "C" int msnh_hip_yolo_decode_candidates(int dtype, int batch, int h, int 
     MSNH_REQUIRE(batch > 0 && batch <= 65535 && h > 0 && w > 0 && classes > 0, "yolo_decode_candidates: bad geometry");
     MSNH_REQUIRE(yolo_version == 3 || yolo_version == 4 || yolo_version == 5, "yolo_decode_candidates: yolo_version must be 3, 4 or 5");
     const int per = 5 + classes;
-    MSNH_REQUIRE(x && decoded && anchors6 && cand_idx && cand_cnt && cand_cap > 0 && x_ld >= 3 * per, "yolo_decode_candidates: bad argument");
+    MSNH_REQUIRE(x && (decoded || rows) && anchors6 && cand_idx && cand_cnt && cand_cap > 0 && x_ld >= 3 * per, "yolo_decode_candidates: bad argument");
     MSNH_REQUIRE(decoded_batch_stride >= static_cast<long long>(3) * h * w * per, "yolo_decode_candidates: decoded_batch_stride too small");
     Anchors an;
     for (int i = 0; i < 6; ++i) an.v[i] = anchors6[i];

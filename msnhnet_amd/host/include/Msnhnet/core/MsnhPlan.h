@@ -92,6 +92,7 @@ public:
 
     int computeDtype;
     bool sparseYolo = false;                // yolo heads decode only the rows of their candidates (nobody reads the full decoded tensors)
+    bool yoloKeepDecoded = true;            // sparseYolo: also write the candidates' full decoded rows (only YoloBox::classesVal needs them)
     bool preferWinograd = false;            // 3x3 stride-1 float16 convs take the Winograd path where the kernel accepts the shape
     std::vector<PlanTensor> tensors;
     std::vector<PlanOp>     ops;

@@ -540,6 +540,12 @@ void NetBuilder::enqueueForward(const float *deviceInput)
     if (yout && _inFlight >= 2) MSNH_THROW("two forwards are already in flight: fetch a result first");
     if (deviceInput != nullptr && deviceInput != _inputDev.as<float>())
         MSNH_DEV(msnh_hip_memcpy_d2d(_inputDev.ptr(), deviceInput, sizeof(float) * static_cast<size_t>(_net->inputNum), _stream));
+    if (yout && plan.sparseYolo && plan.yoloKeepDecoded != YoloOutLayer::keepClassScores)
+    {
+        // the full decoded rows are only written for YoloBox::classesVal; the recorded launches carry the choice
+        plan.yoloKeepDecoded = YoloOutLayer::keepClassScores;
+        if (_graph) { msnh_hip_graph_destroy(_graph); _graph = nullptr; }
+    }
     static const bool eager = std::getenv("MSNH_EAGER") != nullptr;
     if (eager)
     {

@@ -778,7 +778,7 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
         const bool cand = op.confThresh < 1.5f;
         if (sparseYolo && cand)
             MSNH_DEV(msnh_hip_yolo_decode_candidates(in.dtype, in.n, in.h, in.w, op.classes, ptr(op.in0), ld(op.in0), mulOf(op.in0), op.anchors.data(),
-                                                     op.ratio, op.yoloVersion, decoded, static_cast<long long>(yoloCells) * per, op.confThresh,
+                                                     op.ratio, op.yoloVersion, yoloKeepDecoded ? decoded : nullptr, static_cast<long long>(yoloCells) * per, op.confThresh,
                                                      yoloCandIdx.as<int>(), yoloCells, op.cellBase, yoloCandCnt.as<int>(), yoloRows.as<float>(), s));
         else
             MSNH_DEV(msnh_hip_yolo_decode(in.dtype, in.n, in.h, in.w, op.classes, ptr(op.in0), ld(op.in0), mulOf(op.in0), op.anchors.data(), op.ratio,

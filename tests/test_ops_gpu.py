@@ -357,6 +357,19 @@ def test_yolo_decode(dtype, version):
         assert np.array_equal(r3[:, :5], full[b][cells][:, :5])
         assert np.array_equal(r3[:, 5], full[b][cells][:, 5:].max(1)) and np.array_equal(r3[:, 6], full[b][cells][:, 5:].argmax(1).astype(np.float32))
         assert np.array_equal(r3[:, 7], (cells + 1000).astype(np.float32))
+    # ... and without a decoded buffer the same compact rows are all it writes
+    ci4 = torch.full((2, cap), -1, dtype=torch.int32).cuda()
+    cc4 = torch.zeros(2, dtype=torch.int32).cuda()
+    rows4 = torch.zeros((2, cap, 8), dtype=torch.float32).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_yolo_decode_candidates(dtype, 2, h, w, cls, gu.ptr(xd), 256, 1.0, anchors.ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                                                        ratio, version, None, 3 * h * w * per, 0.5, gu.ptr(ci4), cap, 1000, gu.ptr(cc4), gu.ptr(rows4), None))
+    gu.sync()
+    for b in range(2):
+        n = int(cc4[b])
+        assert n == int(cc3[b])
+        a4 = rows4[b, :n].cpu().numpy(); a3 = rows3[b, :n].cpu().numpy()
+        assert np.array_equal(a4[np.argsort(a4[:, 7])], a3[np.argsort(a3[:, 7])], equal_nan=True)
     # candidate compaction: box, objectness, first-maximum class
     ci2 = (ci - 1000).clamp(min=0).contiguous()
     rows = torch.zeros((2, cap, 8), dtype=torch.float32).cuda()
