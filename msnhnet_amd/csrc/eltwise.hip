@@ -158,6 +158,41 @@ __global__ __launch_bounds__(256) void avgPoolKernel(const T *__restrict__ x, in
     storeVec<TOut, VEC>(y + p * yLd + c0, sum);
 }
 
+// One window that covers the whole image (the classifier heads: 7x7 -> 1x1): a thread per output would walk all H*W
+// pixels alone, with only batch * c / VEC threads on the device.  Here a workgroup takes 16 channel vectors of one image,
+// 16 threads share the pixels of each (pixel p, p + 16, ...) and their partial sums are added in a fixed order through LDS.
+template <typename T, typename TOut, int VEC>
+__global__ __launch_bounds__(256) void avgPoolGlobalKernel(const T *__restrict__ x, int xLd, int HW, int c, float outMul, TOut *__restrict__ y, int yLd)
+{
+    __shared__ float part[16][16][VEC];
+    const int cl = threadIdx.x & 15, pl = threadIdx.x >> 4;
+    const int cv = blockIdx.x * 16 + cl;
+    const long long b = blockIdx.y;
+    const bool live = cv * VEC < c;
+    float sum[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) sum[i] = 0.f;
+    if (live)
+        for (int p = pl; p < HW; p += 16)
+        {
+            float v[VEC];
+            loadVec<T, VEC>(x + (b * HW + p) * xLd + cv * VEC, v);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) sum[i] += v[i];
+        }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) part[pl][cl][i] = sum[i];
+    __syncthreads();
+    if (pl != 0 || !live) return;
+#pragma unroll
+    for (int q = 1; q < 16; ++q)
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) sum[i] += part[q][cl][i];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) sum[i] = outMul * (sum[i] / static_cast<float>(HW));
+    storeVec<TOut, VEC>(y + b * yLd + cv * VEC, sum);
+}
+
 // ---- nearest upsample / channel copy -------------------------------------------------------------------
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void upsampleKernel(const T *__restrict__ x, int xLd, int H, int W, int c, int stride, float scale,
@@ -562,6 +597,19 @@ int msnh_hip_avgpool(int dtype, int out_dtype, int batch, int in_h, int in_w, in
     hipStream_t st = resolveStream(s);
     int vec = pickVec(dtype, c, {x_ld, y_ld}, {x, y});
     if (dtype != out_dtype) vec = (vec > 1 && y_ld % 8 == 0) ? 4 : 1;
+    if (out_h == 1 && out_w == 1 && pad == 0 && ksize >= in_h && ksize >= in_w && batch <= 65535)
+    {
+        dim3 ggrid((c / vec + 15) / 16, batch);
+#define MSNH_APG(T, TO, V)                                                                                             \
+        hipLaunchKernelGGL((avgPoolGlobalKernel<T, TO, V>), ggrid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, in_h * in_w, c, out_mul,  \
+                           static_cast<TO *>(y), y_ld)
+        if (dtype == MSNH_F16 && out_dtype == MSNH_F16) { if (vec == 8) MSNH_APG(f16, f16, 8); else MSNH_APG(f16, f16, 1); }
+        else if (dtype == MSNH_F16) { if (vec == 4) MSNH_APG(f16, float, 4); else MSNH_APG(f16, float, 1); }
+        else { if (vec == 4) MSNH_APG(float, float, 4); else MSNH_APG(float, float, 1); }
+#undef MSNH_APG
+        MSNH_LAUNCH_CHECK();
+        return 0;
+    }
     const long long total = static_cast<long long>(batch) * out_h * out_w * (c / vec);
     dim3 grid(gridFor(total, 256));
 #define MSNH_AP(T, TO, V)                                                                                              \

@@ -126,6 +126,23 @@ def test_avgpool(c, h, w, k, s, p, dtype, out_dtype):
     assert gu.rel_err(gu.nchw_host(yd, c), ref) <= (1e-6 if out_dtype == abi.F32 else 1e-3)
 
 
+@pytest.mark.parametrize("dtype,out_dtype", [(abi.F32, abi.F32), (abi.F16, abi.F16), (abi.F16, abi.F32)])
+@pytest.mark.parametrize("c,h,w", [(1280, 7, 7), (20, 5, 7), (7, 3, 3), (2048, 1, 1), (264, 19, 17)])
+def test_avgpool_whole_image(c, h, w, dtype, out_dtype):
+    """one window over the whole image (classifier heads, globalavgpool): the mean of every channel"""
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(c + h)
+    x = _x(rng, (3, c, h, w), dtype)
+    ref = x.astype(np.float64).mean(axis=(2, 3), keepdims=True)
+    xd = gu.nhwc_dev(x, dtype)
+    yd = torch.zeros((3, 1, 1, c), dtype=gu.TORCH_DT[out_dtype]).cuda()
+    gu.sync()
+    abi.check(abi.lib().msnh_hip_avgpool(dtype, out_dtype, 3, h, w, c, gu.ptr(xd), c, max(h, w), 1, 0, 1, 1, 1.0, gu.ptr(yd), c, None))
+    gu.sync()
+    assert gu.rel_err(gu.nchw_host(yd, c), ref) <= (1e-6 if out_dtype == abi.F32 else 1e-3)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_upsample(dtype):
     import gpuutil as gu
