@@ -6,7 +6,7 @@
 //     k = (tap, channel); the B operand is gathered on the fly from the NHWC input: for one tap the
 //         cin_g channels of an input pixel are contiguous, so a 16-byte vector load per lane feeds the
 //         MFMA operand registers without any transposition.
-// A workgroup of 256 threads (4 wavefronts in a WM x WN grid) owns a BM x BN tile of D.  Per K step every
+// A workgroup of 256, 512 or 768 threads (4, 8 or 12 wavefronts in a WM x WN grid) owns a BM x BN tile of D.  Per K step every
 // wavefront issues 16-byte-per-lane buffer loads that deliver straight into LDS (no registers, no LDS store
 // instructions); three LDS stages rotate so that the loads run two steps ahead of the MFMAs, with one barrier
 // per step.  LDS rows are unpadded and XOR-swizzled so that both the 1 KiB deliveries and the 128-bit fragment
@@ -185,7 +185,7 @@ template <int I, int N, typename F> __device__ __forceinline__ void staticFor(F 
     }
 }
 
-template <int BM, int TM> constexpr size_t igemmEpilogueLds() { return (2 * BM + 4 * 32 * (TM + 4)) * sizeof(float); }
+template <int BM, int TM, int NW = 4> constexpr size_t igemmEpilogueLds() { return (2 * BM + NW * 32 * (TM + 4)) * sizeof(float); }
 
 template <typename T, typename TOut, int BM, int BN, int TM, int TN>
 __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[TM / 32][TN / 32], unsigned char *smemRaw, float chScale,
@@ -331,8 +331,12 @@ __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[
 
 // Register budget: two workgroups per CU (one wave of each per SIMD) so that one workgroup's barrier and epilogue
 // are covered by the other's MFMAs; smaller tiles, which serve the short-K bandwidth-bound layers, get three to six.
-constexpr int igemmWavesPerSimd(int bm, int bn, int kv = 8, int ns = 3)
+constexpr int igemmWavesPerSimd(int bm, int bn, int kv = 8, int ns = 3, int nw = 4)
 {
+    // eight-wavefront workgroups put two waves on every SIMD: one workgroup per CU, or two where registers (64 x 64 wave tile)
+    // and LDS (at most 80 KiB) allow it
+    if (nw == 12) return 3;
+    if (nw == 8) return (bm * bn <= 256 * 128 && static_cast<size_t>(ns) * (bm + bn) * kv * 16 <= 80 * 1024) ? 4 : 2;
     // (two-stage 64-byte-row variants of the small tiles: LDS for six to eight workgroups per CU, for the short-K layers that
     // live on memory bandwidth)
     if (ns == 2 && kv == 4 && bm * bn <= 64 * 128) return bm * bn > 64 * 64 ? 6 : 8;
@@ -366,15 +370,19 @@ __device__ __forceinline__ i32x4 makeRsrcWords(const void *base, unsigned bytes)
 }
 
 template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int NS>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(igemmWavesPerSimd(BM, BN, KV, NS), igemmWavesPerSimd(BM, BN, KV, NS))))
+__global__ __launch_bounds__(64 * WM * WN)
+__attribute__((amdgpu_waves_per_eu(igemmWavesPerSimd(BM, BN, KV, NS, WM * WN), igemmWavesPerSimd(BM, BN, KV, NS, WM * WN))))
 void convIgemmKernel(IgemmArgs a)
 {
     typedef typename Frag<T>::V V;
     constexpr int VEC   = Frag<T>::VEC;
     constexpr int BK    = KV * VEC;               // K elements per tile step
-    constexpr int RPP   = 256 / KV;               // rows loaded per pass of the workgroup
-    constexpr int AROWS = BM / RPP;               // A rows (16-byte chunks) per thread per tile step
-    constexpr int BROWS = BN / RPP;               // B rows per thread
+    constexpr int NT    = 64 * WM * WN;           // threads: 4, 8 or 12 wavefronts
+    constexpr int RPP   = NT / KV;                // rows loaded per pass of the workgroup
+    constexpr int BML   = (BM + RPP - 1) / RPP * RPP; // A rows held in LDS: BM rounded up to whole passes (the surplus rows load nothing)
+    constexpr int AROWS = BML / RPP;              // A rows (16-byte chunks) per thread per tile step
+    constexpr int BNL   = (BN + RPP - 1) / RPP * RPP; // B rows held in LDS: BN rounded up to whole passes (the surplus rows load nothing)
+    constexpr int BROWS = BNL / RPP;              // B rows per thread
     constexpr int NL    = AROWS + BROWS;          // loads per thread per tile step
     constexpr int TM    = BM / WM;                // wave tile
     constexpr int TN    = BN / WN;
@@ -384,10 +392,9 @@ void convIgemmKernel(IgemmArgs a)
     constexpr unsigned ES = sizeof(T);
     constexpr int ROWB  = KV * 16;                // bytes per LDS row: unpadded
     constexpr int SWDIV = 16 / KV;                // rows per 256 bytes of LDS
-    constexpr int A_BYTES = BM * ROWB;
-    constexpr unsigned STAGE = (BM + BN) * ROWB;  // one LDS stage: A rows, then B rows
-    static_assert(BM % RPP == 0 && BN % RPP == 0, "tile rows must be a multiple of rows per pass");
-    static_assert(TM % 32 == 0 && TN % 32 == 0 && WM * WN == 4 && S % 2 == 0, "wave grid");
+    constexpr int A_BYTES = BML * ROWB;
+    constexpr unsigned STAGE = (BML + BNL) * ROWB; // one LDS stage: A rows, then B rows
+    static_assert(TM % 32 == 0 && TN % 32 == 0 && (WM * WN == 4 || WM * WN == 8 || WM * WN == 12) && S % 2 == 0, "wave grid");
     static_assert(NS >= 2 && NS <= 8, "LDS stages");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smemRaw[];
@@ -435,7 +442,7 @@ void convIgemmKernel(IgemmArgs a)
     for (int i = 0; i < BROWS; ++i)
     {
         const int p = p0 + ldRow + i * RPP;
-        const bool ok = p < a.P;
+        const bool ok = p < a.P && ldRow + i * RPP < BN;
         const int pp = ok ? p : 0;
         const int ox = pp % a.OW;
         const int t  = pp / a.OW;
@@ -460,7 +467,7 @@ void convIgemmKernel(IgemmArgs a)
     for (int i = 0; i < AROWS; ++i)
     {
         const int m = m0 + ldRow + i * RPP;
-        aOff[i] = m < a.coutG ? (static_cast<unsigned>(m) * a.taps * a.cinG + ldVec * VEC) * ES : kOobOffset;
+        aOff[i] = (m < a.coutG && ldRow + i * RPP < BM) ? (static_cast<unsigned>(m) * a.taps * a.cinG + ldVec * VEC) * ES : kOobOffset;
     }
 
     unsigned bVoff[BROWS];                       // B offsets of the tap being loaded
@@ -652,8 +659,9 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
         setError("conv2d: the implicit GEMM needs at most 64 filter taps and tensors below 2 GiB");
         return 3;
     }
-    const size_t smemLoop = static_cast<size_t>(NS) * (BM + BN) * KV * 16;
-    const size_t smemEpi  = igemmEpilogueLds<BM, BM / WM>();
+    constexpr int RPP = 64 * WM * WN / KV;
+    const size_t smemLoop = static_cast<size_t>(NS) * ((BM + RPP - 1) / RPP * RPP + (BN + RPP - 1) / RPP * RPP) * KV * 16;
+    const size_t smemEpi  = igemmEpilogueLds<BM, BM / WM, WM * WN>();
     const size_t smem = smemLoop > smemEpi ? smemLoop : smemEpi;
     a.mTiles = (a.coutG + BM - 1) / BM;
     const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
@@ -680,7 +688,7 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
                                            static_cast<int>(smem));
         if (e != hipSuccess) { setError("hipFuncSetAttribute: %s", hipGetErrorString(e)); return 1; }
     }
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * WM * WN), smem, st, a);
     MSNH_LAUNCH_CHECK();
     if (a.splitK > 1)
     {
@@ -701,7 +709,7 @@ namespace msnh {
 // Tile configurations (BM x BN output tile, KV 16-byte vectors of K per step, WM x WN wavefront grid).
 // Index 0 is "choose for me"; the others can be forced through msnh_conv_desc::tile, which is how the host
 // library's per-layer search picks the fastest one at load time.
-constexpr int kIgemmTiles = 31;
+constexpr int kIgemmTiles = 40;
 
 template <typename T, typename TOut>
 int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
@@ -744,6 +752,20 @@ int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
     case 29: return launchIgemm<T, TOut, 64, 128, 4, 1, 4, 2>(a, groups, st);
     case 30: return launchIgemm<T, TOut, 64, 64, 4, 2, 2, 2>(a, groups, st);
     case 31: return launchIgemm<T, TOut, 128, 64, 4, 2, 2, 2>(a, groups, st);
+    // eight wavefronts (512 threads, two per SIMD): a second wave per SIMD covers the first one's barrier and LDS waits where
+    // the launch has at most one workgroup per CU; pixel tiles of 192 and 96 bring the tile count of the 76x76 and 38x38
+    // layers at batch 8 just under the CU count (241 and 242 tiles instead of 361 and 182)
+    case 32: return launchIgemm<T, TOut, 256, 128, 8, 4, 2, 3>(a, groups, st);
+    case 33: return launchIgemm<T, TOut, 128, 128, 8, 2, 4, 4>(a, groups, st);
+    case 34: return launchIgemm<T, TOut, 256, 192, 8, 4, 2, 2>(a, groups, st);
+    case 35: return launchIgemm<T, TOut, 256, 192, 4, 4, 2, 4>(a, groups, st);
+    case 36: return launchIgemm<T, TOut, 256, 96, 8, 8, 1, 3>(a, groups, st);
+    // twelve wavefronts (768 threads, three per SIMD) over 192-pixel tiles: 64 x 64 and 32 x 64 wave tiles
+    case 37: return launchIgemm<T, TOut, 256, 192, 8, 4, 3, 2>(a, groups, st);
+    case 38: return launchIgemm<T, TOut, 128, 192, 8, 4, 3, 3>(a, groups, st);
+    // the LDS-patch kernel with eight wavefronts
+    case 39: return launchPatch<T, TOut, 128, 384, 4, 2, 4, 1>(a, groups, st);
+    case 40: return launchIgemm<T, TOut, 128, 128, 8, 2, 4, 3>(a, groups, st);
     default: break;
     }
     setError("igemm: unknown tile %d", tile);

@@ -20,13 +20,14 @@
 namespace msnh {
 
 template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int PS>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(64 * WM * WN) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void convPatch3x3Kernel(IgemmArgs a)
 {
     typedef typename Frag<T>::V V;
     constexpr int VEC   = Frag<T>::VEC;
     constexpr int BK    = KV * VEC;
-    constexpr int RPP   = 256 / KV;
+    constexpr int NW    = WM * WN;                // wavefronts: 4 or 8
+    constexpr int RPP   = 64 * NW / KV;
     constexpr int AL    = BM / RPP;               // weight loads per thread per step
     constexpr int NL    = AL + PS;                // loads per thread per step
     constexpr int TM    = BM / WM;
@@ -40,7 +41,7 @@ void convPatch3x3Kernel(IgemmArgs a)
     constexpr unsigned A_STAGE = BM * ROWB;
     constexpr int RPS   = 64 / KV;                // patch rows per 1 KiB slice
     static_assert(KV == 4 && S == 2, "the slice arithmetic below assumes 64-byte rows");
-    static_assert(BM % RPP == 0 && TM % 32 == 0 && TN % 32 == 0 && WM * WN == 4, "tile shape");
+    static_assert(BM % RPP == 0 && TM % 32 == 0 && TN % 32 == 0 && (NW == 4 || NW == 8), "tile shape");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smemRaw[];
     const unsigned ldsBase = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char *)smemRaw));
@@ -93,9 +94,9 @@ void convPatch3x3Kernel(IgemmArgs a)
     const unsigned sliceStride = static_cast<unsigned>(RPS) * a.inLd * ES;
     const unsigned waveDump = ldsBase + dumpOff;
 
-    // slice number i of this wave (slices wave, wave+4, ...) of the patch of channel chunk `chunk` into stage `st`
+    // slice number i of this wave (slices wave, wave+NW, ...) of the patch of channel chunk `chunk` into stage `st`
     auto issuePatch = [&](int i, int chunk, unsigned stOff) {
-        const int s = wave + 4 * i;
+        const int s = wave + NW * i;
         const bool real = s < nSlices && chunk < a.cChunks;
         const bool cut = a.ragged && (chunk * BK + pVec * VEC >= a.cinG);
         const unsigned voff = (real && !cut) ? pBase + static_cast<unsigned>(s) * sliceStride : kOobOffset;
@@ -169,7 +170,7 @@ void convPatch3x3Kernel(IgemmArgs a)
     constexpr int PER = MB * NB;
     // all NL loads of a step are issued among the MFMAs of its first k-step, ahead of the barrier
     // ---- prologue: whole patch of chunk 0, weight tiles of steps 0 and 1 ----------------------------------------
-    for (int i = 0; wave + 4 * i < nSlices; ++i) issuePatch(i, 0, patchOff0);
+    for (int i = 0; wave + NW * i < nSlices; ++i) issuePatch(i, 0, patchOff0);
     staticFor<0, AL>([&](auto lTag) { issueA(lTag, 0u, a.ragged && (ldVec * VEC >= a.cinG), 0u); });
     {
         const bool pastEnd = a.nIter < 2;         // never: nIter >= 9
@@ -253,12 +254,12 @@ inline bool patchFits(const IgemmArgs &a, size_t *smemOut, int *slicesOut)
     const int R = BN + 2 * a.W + 2;
     const int slices = (R * KV + 63) / 64;
     const size_t loop = static_cast<size_t>(3) * BM * KV * 16 + static_cast<size_t>(2) * slices * 1024 + 1024;
-    const size_t epi = igemmEpilogueLds<BM, BM / WM>();
+    const size_t epi = igemmEpilogueLds<BM, BM / WM, WM * WN>();
     const size_t smem = loop > epi ? loop : epi;
     if (smemOut) *smemOut = smem;
     if (slicesOut) *slicesOut = slices;
-    // taps 0..7 of a chunk bring in the next patch: 8 * PS slices per wave, 4 waves
-    return a.patchOk && a.buffersOk && smem <= 160 * 1024 && slices <= 32 * PS;
+    // taps 0..7 of a chunk bring in the next patch: 8 * PS slices per wave
+    return a.patchOk && a.buffersOk && smem <= 160 * 1024 && slices <= 8 * WM * WN * PS;
 }
 
 template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int PS>
@@ -288,7 +289,7 @@ inline int launchPatch(IgemmArgs &a, int groups, hipStream_t st)
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
         if (e != hipSuccess) { setError("hipFuncSetAttribute: %s", hipGetErrorString(e)); return 1; }
     }
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, a);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * WM * WN), smem, st, a);
     MSNH_LAUNCH_CHECK();
     return 0;
 }
