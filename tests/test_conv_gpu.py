@@ -110,6 +110,38 @@ def test_conv_every_tile_configuration(dtype):
 
 
 @pytest.mark.parametrize("dtype", [abi.F32, abi.F16])
+@pytest.mark.parametrize("k,stride", [(3, 1), (3, 2), (1, 1)])
+def test_conv_multi_wavefront_tiles(k, stride, dtype):
+    """The 8- and 12-wavefront tile configurations over several channel tiles and pixel tiles: 520 output channels (three 256-row
+    tiles, the last one 8 rows), pixel counts that are no multiple of 192, 128 or 96, a ragged last channel chunk, residual add."""
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(100 + 10 * k + stride)
+    b, c, h, w, oc = 3, 72, 25, 23, 520
+    x, wt = _case(rng, b, c, h, w, oc, k)
+    pad = k // 2
+    oh, ow = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
+    res = rng.standard_normal((b, oc, oh, ow), dtype=np.float32)
+    scale = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    shift = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    if dtype == abi.F16:
+        x, wt, res = gu.round_f16(x), gu.round_f16(wt), gu.round_f16(res)
+    ref = _ref(x, wt, stride, pad, 1, 1, scale, shift, "leaky", 0.1, res, "relu", 1.0, 1.0)
+    ran = 0
+    for tile in range(32, abi.lib().msnh_hip_conv2d_tile_count() + 1):
+        print("multi-wavefront tile", tile, k, stride, dtype, flush=True)
+        try:
+            y, _ = gu.conv2d(x, wt, dtype=dtype, stride=stride, pad=pad, scale=scale, shift=shift, act="leaky", residual=res, act2="relu",
+                             algo="igemm", tile=tile)
+        except abi.HipError as e:
+            assert "this tile needs" in str(e)
+            continue
+        ran += 1
+        assert gu.rel_err(y, ref) <= TOL[dtype], tile
+    assert ran >= 8
+
+
+@pytest.mark.parametrize("dtype", [abi.F32, abi.F16])
 @pytest.mark.parametrize("shape", [(2, 16, 19, 19, 40), (1, 64, 38, 38, 96), (3, 8, 7, 5, 16), (1, 32, 76, 76, 64), (2, 72, 13, 11, 136)])
 def test_conv_patch_tiles(shape, dtype):
     """3x3 stride-1 layers with the input patch resident in LDS: image borders, batch seams, ragged channel chunks"""
