@@ -1300,19 +1300,25 @@ void YoloOutLayer::nmsClass(const std::vector<YoloBox> &bboxes, std::vector<int>
         const float jarea = (jx2 - jx1 + 1) * (jy2 - jy1 + 1);
         const size_t nk = kx1.size();
         int hit = 0;
-#pragma omp simd reduction(| : hit)
-        for (size_t k = 0; k < nk; ++k)
+        // the kept boxes are tested in blocks: most candidates of a crowded class are erased by one of the first
+        // (highest-objectness) kept boxes, and any hit decides
+        for (size_t k0 = 0; k0 < nk && !hit; k0 += 64)
         {
-            // Box::iou(candidate j, kept k) with std::min / std::max spelled out
-            const float ix2 = (kx2[k] < jx2) ? kx2[k] : jx2;
-            const float ix1 = (jx1 < kx1[k]) ? kx1[k] : jx1;
-            const float iy2 = (ky2[k] < jy2) ? ky2[k] : jy2;
-            const float iy1 = (jy1 < ky1[k]) ? ky1[k] : jy1;
-            const float iw = ix2 - ix1 + 1;
-            const float ih = iy2 - iy1 + 1;
-            const float inter = (iw < 0 ? 0 : iw) * (ih < 0 ? 0 : ih);
-            const float iou = 1.f * inter / (jarea + karea[k] - inter);
-            hit |= (iou > nmsThresh) ? 1 : 0;
+            const size_t k1 = std::min(nk, k0 + 64);
+#pragma omp simd reduction(| : hit)
+            for (size_t k = k0; k < k1; ++k)
+            {
+                // Box::iou(candidate j, kept k) with std::min / std::max spelled out
+                const float ix2 = (kx2[k] < jx2) ? kx2[k] : jx2;
+                const float ix1 = (jx1 < kx1[k]) ? kx1[k] : jx1;
+                const float iy2 = (ky2[k] < jy2) ? ky2[k] : jy2;
+                const float iy1 = (jy1 < ky1[k]) ? ky1[k] : jy1;
+                const float iw = ix2 - ix1 + 1;
+                const float ih = iy2 - iy1 + 1;
+                const float inter = (iw < 0 ? 0 : iw) * (ih < 0 ? 0 : ih);
+                const float iou = 1.f * inter / (jarea + karea[k] - inter);
+                hit |= (iou > nmsThresh) ? 1 : 0;
+            }
         }
         if (hit) continue;
         m[w++] = j;
@@ -1517,18 +1523,25 @@ void YoloOutLayer::finish(int slot)
         if (_useSoftNms) finalOut[static_cast<size_t>(b)] = nms(cand[static_cast<size_t>(b)], _nmsThresh, true);
         else groups[static_cast<size_t>(b)] = groupByClass(cand[static_cast<size_t>(b)]);
     }
+    const double dbgA = TimeUtil::getElapsedTime(dbg0);
+    double dbgB = dbgA;
     if (!_useSoftNms)
     {
         std::vector<std::pair<int, int>> tasks;
         for (int b = 0; b < _batch; ++b)
             for (size_t g = 0; g < groups[static_cast<size_t>(b)].size(); ++g) tasks.emplace_back(b, static_cast<int>(g));
+        // largest classes first, one task at a time: a crowded class costs as much as all the small ones together
+        std::stable_sort(tasks.begin(), tasks.end(), [&groups](const std::pair<int, int> &x, const std::pair<int, int> &y) {
+            return groups[static_cast<size_t>(x.first)][static_cast<size_t>(x.second)].size() > groups[static_cast<size_t>(y.first)][static_cast<size_t>(y.second)].size();
+        });
         const int nTasks = static_cast<int>(tasks.size());
-#pragma omp parallel for schedule(dynamic, 4)
+#pragma omp parallel for schedule(dynamic, 1)
         for (int t = 0; t < nTasks; ++t)
         {
             const size_t b = static_cast<size_t>(tasks[static_cast<size_t>(t)].first);
             nmsClass(cand[b], groups[b][static_cast<size_t>(tasks[static_cast<size_t>(t)].second)], _nmsThresh);
         }
+        dbgB = TimeUtil::getElapsedTime(dbg0);
 #pragma omp parallel for schedule(dynamic)
         for (int b = 0; b < _batch; ++b)
         {
@@ -1538,7 +1551,9 @@ void YoloOutLayer::finish(int slot)
         }
     }
     for (int b = 0; b < _batch; ++b) batchHasBox[static_cast<size_t>(b)] = cnt[b] > 0;
-    if (std::getenv("MSNH_DEBUG_TIMING")) std::fprintf(stderr, "yoloout finish: wait %.3f ms, host %.3f ms\n", dbgWait, TimeUtil::getElapsedTime(dbg0) - dbgWait);
+    if (std::getenv("MSNH_DEBUG_TIMING"))
+        std::fprintf(stderr, "yoloout finish: wait %.3f ms, host %.3f ms (candidates %.3f, suppression %.3f, output %.3f)\n", dbgWait,
+                     TimeUtil::getElapsedTime(dbg0) - dbgWait, dbgA - dbgWait, dbgB - dbgA, TimeUtil::getElapsedTime(dbg0) - dbgB);
 }
 
 void YoloOutLayer::forwardGPU(NetworkState &netState)

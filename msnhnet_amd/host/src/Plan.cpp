@@ -604,8 +604,22 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
         for (const auto &m : memo)
             if (m.first == key) { op.algo = m.second / 1000; op.tile = m.second % 1000; found = true; break; }
         if (found) continue;
-        int best = 0, bestAlgo = op.algo;
-        float bestMs = std::numeric_limits<float>::max();
+        // Two passes: every candidate is timed over a few launches, then the four fastest are timed again over many more and the
+        // best of those wins (a single short timing of a 10-40 us kernel is too noisy to separate candidates a few percent apart).
+        struct Cand { float ms; int algo, tile; };
+        std::vector<Cand> cands;
+        auto timeOne = [&](int algo, int tile, int warm, int reps) {
+            op.algo = algo;
+            op.tile = tile;
+            for (int r = 0; r < warm; ++r) launch(op, s);            // warm-up (also surfaces launch errors for this tile)
+            MSNH_DEV(msnh_hip_event_record(e0, s));
+            for (int r = 0; r < reps; ++r) launch(op, s);
+            MSNH_DEV(msnh_hip_event_record(e1, s));
+            MSNH_DEV(msnh_hip_event_sync(e1));
+            float ms = 0.f;
+            MSNH_DEV(msnh_hip_event_elapsed_ms(e0, e1, &ms));
+            return ms / static_cast<float>(reps);
+        };
         auto search = [&](int algo) {
             op.algo = algo;
             for (int tile = 0; tile <= nTiles; ++tile)
@@ -615,15 +629,7 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
                     const msnh_conv_desc probe = convDesc(*this, op);
                     if (!msnh_hip_conv2d_tile_supported(&probe, tile)) continue;
                 }
-                const int reps = 3;
-                launch(op, s);                                       // warm-up (also surfaces launch errors for this tile)
-                MSNH_DEV(msnh_hip_event_record(e0, s));
-                for (int r = 0; r < reps; ++r) launch(op, s);
-                MSNH_DEV(msnh_hip_event_record(e1, s));
-                MSNH_DEV(msnh_hip_event_sync(e1));
-                float ms = 0.f;
-                MSNH_DEV(msnh_hip_event_elapsed_ms(e0, e1, &ms));
-                if (ms < bestMs) { bestMs = ms; best = tile; bestAlgo = algo; }
+                cands.push_back({timeOne(algo, tile, 1, 3), algo, tile});
             }
         };
         const int baseAlgo = op.algo;
@@ -632,6 +638,7 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
         {
             // layers with few output tiles: the K loop cut over several workgroups, if its workspace is modest
             op.tile = 0;
+            op.algo = baseAlgo;
             const msnh_conv_desc d = convDesc(*this, op);
             const size_t need = msnh_hip_conv2d_workspace_bytes(&d, MSNH_CONV_IGEMM_SPLITK);
             if (out.c % 4 == 0 && need <= (static_cast<size_t>(256) << 20))
@@ -642,6 +649,18 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
             }
         }
         if (baseAlgo == MSNH_CONV_IGEMM && op.kind == PlanOp::CONV) search(MSNH_CONV_POINTWISE);      // (refused by the library unless the shape fits)
+        int best = 0, bestAlgo = baseAlgo;
+        if (!cands.empty())
+        {
+            std::sort(cands.begin(), cands.end(), [](const Cand &x, const Cand &y) { return x.ms < y.ms; });
+            const size_t finalists = std::min<size_t>(cands.size(), 4);
+            float bestMs = std::numeric_limits<float>::max();
+            for (size_t i = 0; i < finalists; ++i)
+            {
+                const float ms = finalists > 1 ? timeOne(cands[i].algo, cands[i].tile, 2, 16) : cands[i].ms;
+                if (ms < bestMs) { bestMs = ms; best = cands[i].tile; bestAlgo = cands[i].algo; }
+            }
+        }
         op.algo = bestAlgo;
         op.tile = best;
         memo.emplace_back(key, bestAlgo * 1000 + best);
