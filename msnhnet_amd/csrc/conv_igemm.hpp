@@ -709,7 +709,7 @@ namespace msnh {
 // Tile configurations (BM x BN output tile, KV 16-byte vectors of K per step, WM x WN wavefront grid).
 // Index 0 is "choose for me"; the others can be forced through msnh_conv_desc::tile, which is how the host
 // library's per-layer search picks the fastest one at load time.
-constexpr int kIgemmTiles = 40;
+constexpr int kIgemmTiles = 41;
 
 template <typename T, typename TOut>
 int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
@@ -766,6 +766,8 @@ int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
     // the LDS-patch kernel with eight wavefronts
     case 39: return launchPatch<T, TOut, 128, 384, 4, 2, 4, 1>(a, groups, st);
     case 40: return launchIgemm<T, TOut, 128, 128, 8, 2, 4, 3>(a, groups, st);
+    // 64 channels x 256 pixels with eight wavefronts side by side, for the first layers of the detectors (32 -> 64 channels)
+    case 41: return launchIgemm<T, TOut, 64, 256, 4, 1, 8, 3>(a, groups, st);
     default: break;
     }
     setError("igemm: unknown tile %d", tile);
