@@ -120,8 +120,10 @@ __global__ __launch_bounds__(256) void yoloScanKernel(const T *__restrict__ x, i
 
 // Decodes the rows of the listed candidates that belong to this head into their places of the decoded buffer and, when
 // `rows` is given, writes the candidate's compact row { x, y, w, h, objectness, best class score, best class index, cell }
-// (what yoloGatherKernel derives from the decoded row).  One wavefront per candidate: lane l decodes values l, l + 64, ...;
-// the best class is the first maximum in channel order, found with a wavefront reduction on (score, index).
+// (what yoloGatherKernel derives from the decoded row).  Sixteen lanes per candidate, four candidates per wavefront (the
+// kernel lives on the latency of its dependent loads, so candidates in flight count, not lanes per candidate): lane s of a
+// group decodes values s, s + 16, ...; the best class is the first maximum in channel order, found with a reduction on
+// (score, index) over the group's lanes.
 template <typename T, bool V5>
 __global__ __launch_bounds__(256) void yoloRowsKernel(const T *__restrict__ x, int xLd, float xMul, Anchors an, float ratio,
                                                       float *__restrict__ decoded, long long decStride, const int *__restrict__ candIdx, int candCap,
@@ -129,10 +131,12 @@ __global__ __launch_bounds__(256) void yoloRowsKernel(const T *__restrict__ x, i
 {
     const int b = blockIdx.y;
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int sub = lane & 15;                                   // lane inside the candidate's group
+    const int groupLane0 = lane & 48;                            // first lane of the group
+    const int group = threadIdx.x >> 4;                          // 16 groups per workgroup
     int n = candCnt[b];
     n = n < candCap ? n : candCap;
-    for (int k = blockIdx.x * 4 + wave; k < n; k += gridDim.x * 4)
+    for (int k = blockIdx.x * 16 + group; k < n; k += gridDim.x * 16)
     {
         const int cellG = candIdx[static_cast<size_t>(b) * candCap + k];
         const int cell = cellG - candBase;
@@ -141,33 +145,33 @@ __global__ __launch_bounds__(256) void yoloRowsKernel(const T *__restrict__ x, i
         const int py = p / W, px = p - py * W;
         const T *xr = x + (static_cast<size_t>(b) * HW + p) * xLd + a * per;
         float *dr = decoded + static_cast<size_t>(b) * decStride + static_cast<size_t>(cell) * per;
-        float first = 0.f;                                       // this lane's value of m = lane (box and objectness live in lanes 0..4)
+        float first = 0.f;                                       // this lane's value of m = sub (box and objectness live in lanes 0..4 of the group)
         float bv = -3.402823466e38f * 2.f;                       // -inf: NaN scores are never selected
         int bi = 0x7fffffff;
-        for (int m = lane; m < per; m += 64)
+        for (int m = sub; m < per; m += 16)
         {
             const float v = yoloDecodeOne<V5>(xMul * toF(xr[m]), m, px, py, a, an, ratio);
             if (decoded != nullptr) dr[m] = v;
-            if (m == lane) first = v;
+            if (m == sub) first = v;
             if (m >= 5 && v > bv) { bv = v; bi = m - 5; }
         }
         if (rows == nullptr) continue;
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1)
+        for (int off = 8; off > 0; off >>= 1)
         {
             const float ov = __shfl_xor(bv, off, 64);
             const int oi = __shfl_xor(bi, off, 64);
             if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
         }
         // a NaN score of class 0 absorbs the sequential scan of the reference (nothing compares greater than it)
-        const float c0v = __shfl(first, 5, 64);
+        const float c0v = __shfl(first, groupLane0 + 5, 64);
         if (c0v != c0v) { bv = c0v; bi = 0; }
         if (bi == 0x7fffffff) bi = 0;
         float *o = rows + (static_cast<size_t>(b) * candCap + k) * 8;
-        if (lane < 5) o[lane] = first;
-        else if (lane == 5) o[5] = bv;
-        else if (lane == 6) o[6] = static_cast<float>(bi);
-        else if (lane == 7) o[7] = static_cast<float>(cellG);
+        if (sub < 5) o[sub] = first;
+        else if (sub == 5) o[5] = bv;
+        else if (sub == 6) o[6] = static_cast<float>(bi);
+        else if (sub == 7) o[7] = static_cast<float>(cellG);
     }
 }
 
@@ -545,7 +549,7 @@ extern "C" int msnh_hip_yolo_decode_candidates(int dtype, int batch, int h, int 
     for (int i = 0; i < 6; ++i) an.v[i] = anchors6[i];
     hipStream_t st = resolveStream(s);
     const int HW = h * w;
-    dim3 sgrid((3 * HW + 255) / 256, batch), rgrid(128, batch);
+    dim3 sgrid((3 * HW + 255) / 256, batch), rgrid(256, batch);
 #define MSNH_YC(T)                                                                                                      \
     do {                                                                                                                \
         hipLaunchKernelGGL((yoloScanKernel<T>), sgrid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, x_mul, conf_thresh, cand_idx, cand_cap,  \
