@@ -69,7 +69,7 @@ def cpu_baseline(arch, size, tmp, seed, budget_s=30.0):
 # HBM bytes per convolution launch (fetch + write), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script,
 # each scaled by what the same counter reads for a plain copy kernel of known size (fetch x2.0, write x1.0); the runs
 # and their summary are in profiles/conv_igemm_yolov3_608_f16_b8.md.  None for workloads that were not profiled.
-HBM_BYTES_PER_CONV_LAUNCH = {("yolov3", "f16", 8): int((39.51 + 19.08) * 2**20)}
+HBM_BYTES_PER_CONV_LAUNCH = {("yolov3", "f16", 8): int((40.24 + 19.06) * 2**20)}
 
 
 def main():
