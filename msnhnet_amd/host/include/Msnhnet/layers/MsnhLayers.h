@@ -380,6 +380,7 @@ private:
         DeviceBuffer devCnt, devRows, devKept, devKeptCnt, devNmsWs;
         msnh_event_t event = nullptr, ready = nullptr;
         bool pending = false, onDevice = false;
+        size_t rowsCopied = 0;             // row slots per image that the asynchronous copy brings to the host
     };
     std::vector<YoloBox> boxesFromKept(std::vector<const float *> &records) const;
     msnh_stream_t _copyStream = nullptr, _fetchStream = nullptr;

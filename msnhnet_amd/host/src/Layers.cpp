@@ -1393,6 +1393,7 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
         MSNH_DEV(msnh_hip_memcpy_d2h(sl.decoded.ptr(), pl.yoloDecoded.ptr(), bytes, s));
         MSNH_DEV(msnh_hip_event_record(sl.event, s));
         sl.pending = true;
+        sl.rowsCopied = cells;
         return;
     }
     // Snapshot on the device (microseconds), then cross PCIe on a second stream: the next forward does not wait for
@@ -1426,7 +1427,21 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
         MSNH_DEV(msnh_hip_memcpy_d2h(sl.kept.ptr(), sl.devKept.ptr(), std::min(keptCap, kQuickRecords) * kRecordBytes, _copyStream));
     }
     else
-        MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.ptr(), sl.devRows.ptr(), rowBytes, _copyStream));
+    {
+        // Every cell has a row slot and the count is known only on the device; all slots are several MiB and their copy sits
+        // between the end of a forward and the host stage of its batch.  So only a prefix of every image's slots is copied ahead
+        // of time, sized from the previous result (half as much again, + 1024); finish() fetches what an image has beyond it.
+        const size_t guess = _lastMaxCandidates > 0 ? static_cast<size_t>(_lastMaxCandidates) + static_cast<size_t>(_lastMaxCandidates) / 2 + 1024 : cells;
+        sl.rowsCopied = std::min(guess, cells);
+        if (sl.rowsCopied == cells)
+            MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.ptr(), sl.devRows.ptr(), rowBytes, _copyStream));
+        else
+            for (int b = 0; b < _batch; ++b)
+            {
+                const size_t off = static_cast<size_t>(b) * cells * 8;
+                MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.as<float>() + off, sl.devRows.as<float>() + off, sizeof(float) * 8 * sl.rowsCopied, _copyStream));
+            }
+    }
     MSNH_DEV(msnh_hip_event_record(sl.event, _copyStream));
     sl.pending = true;
 }
@@ -1506,6 +1521,20 @@ void YoloOutLayer::finish(int slot)
         }
         if (std::getenv("MSNH_DEBUG_TIMING")) std::fprintf(stderr, "yoloout finish (device NMS, %zu boxes): wait %.3f ms, host %.3f ms\n", total, dbgWait, TimeUtil::getElapsedTime(dbg0) - dbgWait);
         return;
+    }
+    {
+        // rows beyond the prefix that was copied ahead of time (the device snapshot of this slot is still intact)
+        bool more = false;
+        for (int b = 0; b < _batch; ++b)
+        {
+            const size_t n = static_cast<size_t>(std::min(cnt[b], cells));
+            if (n <= sl.rowsCopied) continue;
+            if (_fetchStream == nullptr) MSNH_DEV(msnh_hip_stream_create(&_fetchStream));
+            const size_t off = (static_cast<size_t>(b) * static_cast<size_t>(cells) + sl.rowsCopied) * 8;
+            MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.as<float>() + off, sl.devRows.as<float>() + off, sizeof(float) * 8 * (n - sl.rowsCopied), _fetchStream));
+            more = true;
+        }
+        if (more) MSNH_DEV(msnh_hip_stream_sync(_fetchStream));
     }
     const float *decodedHost = keepClassScores ? sl.decoded.as<float>() : nullptr;
     batchHasBox.assign(static_cast<size_t>(_batch), false);
