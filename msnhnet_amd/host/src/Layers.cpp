@@ -1431,7 +1431,8 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
         // Every cell has a row slot and the count is known only on the device; all slots are several MiB and their copy sits
         // between the end of a forward and the host stage of its batch.  So only a prefix of every image's slots is copied ahead
         // of time, sized from the previous result (half as much again, + 1024); finish() fetches what an image has beyond it.
-        const size_t guess = _lastMaxCandidates > 0 ? static_cast<size_t>(_lastMaxCandidates) + static_cast<size_t>(_lastMaxCandidates) / 2 + 1024 : cells;
+        size_t guess = _lastMaxCandidates > 0 ? static_cast<size_t>(_lastMaxCandidates) + static_cast<size_t>(_lastMaxCandidates) / 2 + 1024 : cells;
+        if (const char *forced = std::getenv("MSNH_YOLO_ROWS_PREFIX")) guess = static_cast<size_t>(std::max(1L, std::atol(forced)));    // (tests)
         sl.rowsCopied = std::min(guess, cells);
         if (sl.rowsCopied == cells)
             MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.ptr(), sl.devRows.ptr(), rowBytes, _copyStream));

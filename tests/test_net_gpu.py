@@ -292,6 +292,38 @@ def test_device_nms_equals_host_nms(arch, size, batch):
             assert np.array_equal(g_[b], w_[b], equal_nan=True)
 
 
+def test_yolo_rows_copied_in_part():
+    """The host path copies only a prefix of the candidate row slots ahead of time, sized from the previous result, and fetches
+    the remainder on demand: a network that saw few candidates and then many (and the other way round) returns what a fresh
+    network returns for each input."""
+    size, batch = 320, 2
+    net, binp, g = nu.model("yolov3", batch, size, seed=8)
+    few = np.zeros((batch, 3, size, size), np.float32)
+    many = zoo.seeded_input(batch, 3, size, size, seed=9)
+    try:
+        netapi.set_device_nms(0)
+        want_few = netapi.Net(net, binp, fp16=True).run_yolo(few)
+        want_many = netapi.Net(net, binp, fp16=True).run_yolo(many)
+        m = netapi.Net(net, binp, fp16=True)
+        seq = [few, many, many, few, few, many]
+        got = [m.run_yolo(x) for x in seq]
+        # with these weights most cells are candidates whatever the input, so the prefix is also forced to be short:
+        # 100 rows ahead of time, thousands on demand; 3000: some images need more, some do not
+        for forced in ("100", "3000"):
+            os.environ["MSNH_YOLO_ROWS_PREFIX"] = forced
+            got += [m.run_yolo(x) for x in seq]
+    finally:
+        os.environ.pop("MSNH_YOLO_ROWS_PREFIX", None)
+        netapi.set_device_nms(1)
+    seq = seq * 3
+    print("boxes: few", [len(b) for b in want_few], "many", [len(b) for b in want_many], flush=True)
+    assert sum(len(b) for b in want_many) > 0
+    for x, g_ in zip(seq, got):
+        w_ = want_few if x is few else want_many
+        for b in range(batch):
+            assert np.array_equal(g_[b], w_[b], equal_nan=True)
+
+
 def test_spp_maxpools_run_as_a_chain():
     """the 5 / 9 / 13 pools of an SPP block become three 5-wide pools, each reading the one before (same results: the
     per-layer and final-output parity tests of yolov4 and yolov5s run through this plan)"""
