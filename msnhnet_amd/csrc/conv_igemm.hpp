@@ -709,7 +709,7 @@ namespace msnh {
 // Tile configurations (BM x BN output tile, KV 16-byte vectors of K per step, WM x WN wavefront grid).
 // Index 0 is "choose for me"; the others can be forced through msnh_conv_desc::tile, which is how the host
 // library's per-layer search picks the fastest one at load time.
-constexpr int kIgemmTiles = 41;
+constexpr int kIgemmTiles = 42;
 
 template <typename T, typename TOut>
 int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
@@ -768,6 +768,8 @@ int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
     case 40: return launchIgemm<T, TOut, 128, 128, 8, 2, 4, 3>(a, groups, st);
     // 64 channels x 256 pixels with eight wavefronts side by side, for the first layers of the detectors (32 -> 64 channels)
     case 41: return launchIgemm<T, TOut, 64, 256, 4, 1, 8, 3>(a, groups, st);
+    // 128 channels x 384 pixels with twelve wavefronts: one round of tiles for 128-filter layers over many pixels
+    case 42: return launchIgemm<T, TOut, 128, 384, 8, 2, 6, 2>(a, groups, st);
     default: break;
     }
     setError("igemm: unknown tile %d", tile);
