@@ -62,7 +62,7 @@ struct PlanOp
     float upScale = 1.f;                    // UPSAMPLE: value scale; SOFTMAX: temperature
     int  dstChanOffset = 0;                 // COPY: channel offset inside `out`
     bool pureAct = false;                   // AFFINE with identity scale and shift: only the activation matters
-    float in1Sign = 1.f;                    // ADD: out = act(in0 + in1Sign * in1)
+    float in1Sign = 1.f;                    // ADD: out = act(in0 + in1Sign * in1); CONV with a fused add: sign of the residual
     int  padTop = 0, padLeft = 0;           // PAD
     float padValue = 0.f;
     int  slice[6] = {0, 1, 0, 1, 0, 1};     // SLICE: start / step of channels, rows, columns

@@ -1377,6 +1377,8 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
 {
     Plan &pl = *plan;
     Slot &sl = _slots[slot & 1];
+    if (sl.pending) MSNH_THROW("YoloOut: the results of the previous forward in this slot were not fetched");
+    sl.onDevice = false;
     const size_t cells = static_cast<size_t>(pl.yoloCells);
     sl.cnt.reserve(sizeof(int) * static_cast<size_t>(_batch));
     sl.rows.reserve(sizeof(float) * 8 * cells * static_cast<size_t>(_batch));

@@ -172,10 +172,14 @@ void Plan::fuse()
             PlanOp &conv = ops[static_cast<size_t>(p)];
             if (conv.kind != PlanOp::CONV || conv.in1 >= 0) continue;
             if (tensors[static_cast<size_t>(mine)].pinned || consumerCount(mine) != 1) continue;
+            // a subtraction (in0 - in1) only moves into the epilogue of the conv that produces in0: the sign then rides
+            // on the residual multiplier; -conv + other has no epilogue form
+            if (side == 1 && add.in1Sign != 1.f) continue;
             // the other operand must already exist when the conv runs
             const int po = producerOf(other);
             if (po >= p) continue;
             conv.in1 = other;
+            conv.in1Sign = side == 0 ? add.in1Sign : 1.f;
             conv.act2 = add.act;
             conv.act2Param = add.actParam;
             conv.out = add.out;
@@ -401,7 +405,7 @@ static msnh_conv_desc convDesc(const Plan &plan, const PlanOp &op)
     d.has_residual = op.in1 >= 0 ? 1 : 0;
     d.res_ld = op.in1 >= 0 ? plan.ld(op.in1) : out.c;
     d.act2 = static_cast<int>(op.act2); d.act2_param = op.act2Param;
-    d.res_mul = op.in1 >= 0 ? plan.mulOf(op.in1) : 1.f;
+    d.res_mul = op.in1 >= 0 ? op.in1Sign * plan.mulOf(op.in1) : 1.f;
     d.out_mul = 1.f / plan.mulOf(op.out);
     d.algo = op.algo;
     d.tile = op.tile;
@@ -521,7 +525,7 @@ static std::string tuneSignature(const Plan &plan, const PlanOp &op)
     return os.str();
 }
 
-static std::string tuneHeader(int nTiles)
+static std::string tuneHeader(int nTiles, bool preferWinograd)
 {
     char name[256] = {0};
     int cus = 0;
@@ -530,7 +534,10 @@ static std::string tuneHeader(int nTiles)
     std::string dev(name);
     for (char &ch : dev)
         if (ch == ' ' || ch == '\n') ch = '_';
-    return "msnhtune 1 " + (dev.empty() ? std::string("device") : dev) + " cus " + std::to_string(cus) + " tiles " + std::to_string(nTiles);
+    // the weights are packed for the algorithm family chosen before the search (Winograd or not), so a file written under the other
+    // preference must not be applied
+    return "msnhtune 2 " + (dev.empty() ? std::string("device") : dev) + " cus " + std::to_string(cus) + " tiles " + std::to_string(nTiles) + " winograd " +
+           std::to_string(preferWinograd ? 1 : 0);
 }
 
 // Per-layer search over the implicit-GEMM tile configurations: each candidate runs the real launch (same buffers,
@@ -552,7 +559,7 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
         std::ifstream f(cacheFile);
         std::string line;
         std::vector<std::pair<int, int>> picks;
-        bool ok = f.is_open() && std::getline(f, line) && line == tuneHeader(nTiles);
+        bool ok = f.is_open() && std::getline(f, line) && line == tuneHeader(nTiles, preferWinograd);
         for (size_t k = 0; ok && k < tunedOps.size(); ++k)
         {
             ok = static_cast<bool>(std::getline(f, line));
@@ -572,9 +579,13 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
             {
                 PlanOp &op = ops[tunedOps[k]];
                 before.emplace_back(op.algo, op.tile);
+                // the packed weights on the device are laid out for the algorithm resolved at weight preparation: a recorded choice
+                // from the other family (Winograd's transformed filters against the tap-major layout) would read them wrongly
+                if ((picks[k].first == MSNH_CONV_WINOGRAD) != (op.algo == MSNH_CONV_WINOGRAD)) ok = false;
                 op.algo = picks[k].first; op.tile = picks[k].second;
                 const msnh_conv_desc d = convDesc(*this, op);
                 if (!msnh_hip_conv2d_tile_supported(&d, op.tile)) ok = false;
+                if (op.kind == PlanOp::CONV && op.wDev.bytes() != msnh_hip_conv2d_packed_weight_elems(&d, op.algo) * (d.dtype == MSNH_F16 ? 2u : 4u)) ok = false;
                 need = std::max(need, msnh_hip_conv2d_workspace_bytes(&d, op.algo));
             }
             if (ok)
@@ -589,7 +600,7 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
     msnh_event_t e0 = nullptr, e1 = nullptr;
     MSNH_DEV(msnh_hip_event_create(&e0));
     MSNH_DEV(msnh_hip_event_create(&e1));
-    struct Key { int b, h, w, c, oc, k, st, g, res, odt, algo; bool operator==(const Key &o) const { return std::memcmp(this, &o, sizeof(Key)) == 0; } };
+    struct Key { int kind, b, h, w, c, inLd, oc, outLd, k, st, pad, dil, g, res, odt, algo; bool operator==(const Key &o) const { return std::memcmp(this, &o, sizeof(Key)) == 0; } };
     std::vector<std::pair<Key, int>> memo;         // identical shapes share one search
     for (PlanOp &op : ops)
     {
@@ -598,11 +609,22 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
         const PlanTensor &out = tensors[static_cast<size_t>(op.out)];
         Key key;
         std::memset(&key, 0, sizeof(key));
-        key.b = in.n; key.h = in.h; key.w = in.w; key.c = in.c; key.oc = out.c; key.k = op.ksize; key.st = op.stride; key.g = op.groups;
+        key.kind = static_cast<int>(op.kind);
+        key.b = in.n; key.h = in.h; key.w = in.w; key.c = in.c; key.inLd = ld(op.in0); key.oc = out.c; key.outLd = ld(op.out);
+        key.k = op.ksize; key.st = op.stride; key.pad = op.pad; key.dil = op.dilation; key.g = op.groups;
         key.res = op.in1 >= 0; key.odt = out.dtype; key.algo = op.algo;
         bool found = false;
         for (const auto &m : memo)
-            if (m.first == key) { op.algo = m.second / 1000; op.tile = m.second % 1000; found = true; break; }
+        {
+            if (!(m.first == key)) continue;
+            // same launch as one searched before: take its result, if the library accepts it for this op as well
+            const int wasAlgo = op.algo, wasTile = op.tile;
+            op.algo = m.second / 1000; op.tile = m.second % 1000;
+            const msnh_conv_desc d = convDesc(*this, op);
+            if (msnh_hip_conv2d_tile_supported(&d, op.tile) && msnh_hip_conv2d_workspace_bytes(&d, op.algo) <= _convWorkspace.bytes()) found = true;
+            else { op.algo = wasAlgo; op.tile = wasTile; }
+            break;
+        }
         if (found) continue;
         // Two passes: every candidate is timed over a few launches, then the four fastest are timed again over many more and the
         // best of those wins (a single short timing of a 10-40 us kernel is too noisy to separate candidates a few percent apart).
@@ -672,7 +694,7 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
         std::ofstream f(cacheFile, std::ios::trunc);
         if (f.is_open())
         {
-            f << tuneHeader(nTiles) << "\n";
+            f << tuneHeader(nTiles, preferWinograd) << "\n";
             for (size_t i : tunedOps)
             {
                 // (the signature is taken with the searched choice in place: it does not depend on algo / tile)
@@ -722,6 +744,8 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
     case PlanOp::CONV:
     {
         const msnh_conv_desc d = convDesc(*this, op);
+        if (op.wDev.bytes() != msnh_hip_conv2d_packed_weight_elems(&d, op.algo) * (d.dtype == MSNH_F16 ? 2u : 4u))
+            MSNH_THROW("conv weights on the device are not packed for the algorithm of this launch (" + op.name + ")");
         MSNH_DEV(msnh_hip_conv2d(&d, ptr(op.in0), op.wDev.ptr(), op.scaleDev.as<float>(), op.shiftDev.as<float>(),
                                  op.in1 >= 0 ? ptr(op.in1) : nullptr, ptr(op.out), _convWorkspace.ptr(), _convWorkspace.bytes(), s));
         break;

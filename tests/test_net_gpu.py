@@ -233,7 +233,7 @@ def test_tune_cache(tmp_path):
         assert os.path.exists(cache)
         text = open(cache).read()
         lines = text.splitlines()
-        assert lines[0].startswith("msnhtune 1 ") and len(lines) > 10 and all(" | " in ln for ln in lines[1:])
+        assert lines[0].startswith("msnhtune 2 ") and lines[0].endswith(" winograd 0") and len(lines) > 10 and all(" | " in ln for ln in lines[1:])
         b = netapi.Net(net, binp, fp16=True)
         t2 = time.perf_counter()
         print(f"load with search {t1 - t0:.3f} s, from the file {t2 - t1:.3f} s", flush=True)
@@ -261,6 +261,31 @@ def test_tune_cache(tmp_path):
         # float32 plans keep their own file
         netapi.Net(net, binp, fp16=False)
         assert os.path.exists(binp + ".f32.tune")
+        # a file written under the other Winograd preference is not applied: the weights on the device are packed for the algorithm
+        # family chosen before the search, and a Winograd choice on tap-major weights (or the reverse) would read them wrongly
+        plain = open(cache).read()
+        netapi.set_use_winograd(True)
+        try:
+            w = netapi.Net(net, binp, fp16=True)
+            wino = open(cache).read()
+            assert wino.splitlines()[0].endswith(" winograd 1") and "winograd" in w.plan_detail()
+            yw = w.run_yolo(x)
+        finally:
+            netapi.set_use_winograd(False)
+        d = netapi.Net(net, binp, fp16=True)
+        assert open(cache).read().splitlines()[0].endswith(" winograd 0") and "winograd" not in d.plan_detail()
+        yd = d.run_yolo(x)
+        for i in range(batch):
+            assert abs(len(yd[i]) - len(ya[i])) <= max(2, 0.02 * len(ya[i])) and abs(len(yw[i]) - len(ya[i])) <= max(2, 0.02 * len(ya[i]))
+        # the same header with a Winograd choice spliced into a plain file: refused line by line as well
+        lines_d = open(cache).read().splitlines()
+        k3 = next(i for i, ln in enumerate(lines_d[1:], 1) if ln.split()[8] == "3" and ln.split()[9] == "1")
+        forged = lines_d[:]
+        forged[k3] = forged[k3].split(" | ")[0] + " | 4 0"
+        open(cache, "w").write("\n".join(forged) + "\n")
+        e = netapi.Net(net, binp, fp16=True)
+        assert "winograd" not in e.plan_detail() and " | 4 0" not in open(cache).read()
+        del plain
     finally:
         netapi.set_tune_cache(False)
 
