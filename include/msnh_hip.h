@@ -228,6 +228,23 @@ int msnh_hip_nhwc_to_nchw(int dtype, int batch, int c, int h, int w, const void 
  * CVUtil::getPaddingZeroF32C3 (src/utils/MsnhCVUtil.cpp:203-261) + the host-to-device copy of the float image. */
 int msnh_hip_letterbox_u8(const unsigned char *rgb_hwc, int width, int height, int net_w, int net_h, int half_init,
                           int shuffle_rgb, float *out_chw, msnh_stream_t s);
+/* The reference's other 8-bit image -> network input variants (the PredDataType values of its C facade,
+ * src/c_api/MsnhnetLib.h:11-20, each a CVUtil function): plain bilinear resize to (net_w, net_h) (MatOp::resize,
+ * src/cv/MsnhCVMatOp.cpp:142-160, 404-437), optional R<->B swap, then per channel k
+ *   MSNH_PRE_F32C3        u / 255                                       CVUtil::getImgDataF32C3, src/utils/MsnhCVUtil.cpp:91-138
+ *   MSNH_PRE_F32C3_HALF   (u - 127.5) / 127.5                           the same with halfInit
+ *   MSNH_PRE_GOOGLENET    u / 255 * (std_k / 0.5) + (mean_k - 0.5) / 0.5 with the ImageNet constants, getGoogLenetF32C3, :146-195
+ *   MSNH_PRE_TRANSFORMED  (u / 255 - mean3[k]) / std3[k]                getTransformedF32C3, :269-318
+ *   MSNH_PRE_CAFFE        u - {123.68, 116.779, 103.939}[k]             getCaffeModeF32C3, :326-375
+ *   MSNH_PRE_PADDING_ZERO / _HALF   the letterbox above (msnh_hip_letterbox_u8 with half_init 0 / 1).
+ * mean3 / std3 are host pointers, read at the call; only MSNH_PRE_TRANSFORMED needs them. */
+enum msnh_preproc
+{
+    MSNH_PRE_F32C3 = 0, MSNH_PRE_F32C3_HALF = 1, MSNH_PRE_GOOGLENET = 2, MSNH_PRE_TRANSFORMED = 3, MSNH_PRE_CAFFE = 4,
+    MSNH_PRE_PADDING_ZERO = 5, MSNH_PRE_PADDING_ZERO_HALF = 6
+};
+int msnh_hip_image_u8_to_input(const unsigned char *rgb_hwc, int width, int height, int net_w, int net_h, int kind,
+                               const float *mean3, const float *std3, int shuffle_rgb, float *out_chw, msnh_stream_t s);
 
 /* ------------------------------------------------------------------------------------------------
  * YOLO.  One launch per head replaces YoloLayer::forwardGPU's 15 launches (exSigmoidKernel, aExpTKernel,

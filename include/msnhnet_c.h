@@ -34,6 +34,18 @@ typedef struct BBoxContainer           /* src/c_api/MsnhnetLib.h:34-37 */
     BBox boxes[MSNHNET_MAX_BBOX];
 } BBoxContainer;
 
+/* PredDataType, src/c_api/MsnhnetLib.h:11-20 */
+enum PredDataType
+{
+    PRE_DATA_NONE = 0,
+    PRE_DATA_FC32_C1,
+    PRE_DATA_FC32_C3,
+    PRE_DATA_GOOGLENET_FC3,
+    PRE_DATA_PADDING_ZERO_FC3,
+    PRE_DATA_TRANSFORMED_FC3,
+    PRE_DATA_CAFFE_FC3
+};
+
 /* ---- part 1: the reference facade -------------------------------------------------------------------------------- */
 int initMsnhnet(void);                                                                  /* MsnhnetLib.h:39 */
 int buildMsnhnet(char **msg, const char *msnhnet, const char *msnhbin, int useFp16, int useCudaOnly);   /* :40 */
@@ -44,6 +56,19 @@ int runClassifyNoPred(char **msg, const float *data, const int len, int *bestInd
  * offers the image-file / byte-image variants (runYoloFile / runYoloList, :51-54), whose pre-processing lives in
  * its CV module outside the convolutional path. */
 int runYoloNoPred(char **msg, const float *data, const int len, BBoxContainer *bboxContainer, int *detectedNum, int runGPU);
+/* One 8-bit image (HWC, `channel` bytes per pixel, host memory) -> pre-processing named by preDataType (a PredDataType) on the
+ * device -> forward -> index of the largest logit.  MsnhnetLib.h:44-46; the reference's own implementation needs its OpenCV
+ * build (MsnhnetLib.cpp:97-...), here the in-tree CVUtil variants are followed (src/utils/MsnhCVUtil.cpp:91-375).  swapRGB
+ * exchanges the first and third channel.  mean / std: three floats each, read only by PRE_DATA_TRANSFORMED_FC3.  Errors as the
+ * reference's: "channel must be 1 or 3", "channel 1 must preprocess with F32_C1", "preDataType can't be none",
+ * "mean or std can't be null"; 1-channel images and runGPU == 0 fail (no gray path, no CPU path in this build). */
+int runClassifyList(char **msg, unsigned char *imageData, const int width, const int height, const int channel, int *bestIndex,
+                    int preDataType, const int swapRGB, int runGPU, const float *mean, const float *std);
+/* One 8-bit image -> letterbox (CVUtil::getPaddingZeroF32C3) -> forward -> boxes of the image in network-input pixels.
+ * MsnhnetLib.h:53-54.  More than MSNHNET_MAX_BBOX boxes fail with the reference's "BBox buffer is not enough, ..." */
+int runYoloList(char **msg, unsigned char *imageData, const int width, const int height, const int channel, BBoxContainer *bboxContainer,
+                int *detectedNum, const int swapRGB, const int runGPU);
+/* runClassifyFile / runYoloFile (MsnhnetLib.h:41-42, 51) decode image files and are not part of this library. */
 int dispose(void);                                                                      /* :56 */
 int withGPU(int *GPU);                                                                  /* :57 */
 int withCUDNN(int *CUDNN);                                                              /* :58, always 0 */
@@ -114,6 +139,9 @@ int msnhnet_nms(const float *rows, long long n, float nms_thresh, int fast, floa
  *   to the original image -- YoloOutLayer::bboxResize2Org (padded != 0) / bboxResize2OrgNoPad
  *   (src/layers/MsnhYoloOutLayer.cpp:321-379). */
 int msnhnet_set_input_image_u8(msnhnet_t net, int index, const unsigned char *rgb_hwc, int width, int height, int half_init, int shuffle_rgb);
+/* The same with any pre-processing variant of msnh_hip.h's msnh_preproc (plain resize + normalisation, or the letterbox). */
+int msnhnet_set_input_image(msnhnet_t net, int index, const unsigned char *rgb_hwc, int width, int height, int preproc, const float *mean3,
+                            const float *std3, int shuffle_rgb);
 int msnhnet_boxes_to_image(float *boxes, long long count, int net_w, int net_h, int org_w, int org_h, int padded);
 long long msnhnet_time_detail(msnhnet_t net, char *dst, long long cap);       /* NetBuilder::getTimeDetail */
 

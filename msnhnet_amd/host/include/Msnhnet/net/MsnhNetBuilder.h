@@ -61,6 +61,10 @@ public:
     // CVUtil::getPaddingZeroF32C3 + the float upload do in the reference (MsnhCVUtil.cpp:203-261); then
     // enqueueForward(nullptr) runs on it.
     void setInputImageU8(int index, const unsigned char *rgbHwc, int width, int height, bool halfInit = false, bool shuffleRGB = false);
+    // The same with any of the reference's 8-bit pre-processing variants (msnh_preproc: CVUtil::getImgDataF32C3,
+    // getGoogLenetF32C3, getTransformedF32C3, getCaffeModeF32C3 or the letterbox; MsnhCVUtil.cpp:91-375) resized to the
+    // network's input size on the device.  mean / std: three floats each, only read by MSNH_PRE_TRANSFORMED.
+    void setInputImage(int index, const unsigned char *rgbHwc, int width, int height, int preproc, const float *mean, const float *std, bool shuffleRGB);
 
     Point2I getInputSize();
     int getInputChannel();

@@ -125,6 +125,69 @@ int runYoloNoPred(char **msg, const float *data, const int len, BBoxContainer *b
     });
 }
 
+// The byte-image entry points: pre-processing on the device (msnh_hip_image_u8_to_input), then the forward on what it wrote.
+static int preprocOf(int preDataType, int channel)
+{
+    if (channel != 1 && channel != 3) MSNH_THROW("channel must be 1 or 3");
+    if (channel == 1 && preDataType != PRE_DATA_FC32_C1) MSNH_THROW("channel 1 must preprocess with F32_C1");
+    if (channel == 3 && preDataType == PRE_DATA_FC32_C1) MSNH_THROW("channel 1 can't preprocess with F32_C1");
+    // (the reference's own gray-image loop reads the resized image with the extent of the original one,
+    //  src/utils/MsnhCVUtil.cpp:47-82; this build takes 3-channel images only)
+    if (channel == 1) MSNH_THROW("1-channel images are outside the convolutional path this build implements");
+    switch (preDataType)
+    {
+    case PRE_DATA_FC32_C3:          return MSNH_PRE_F32C3;
+    case PRE_DATA_GOOGLENET_FC3:    return MSNH_PRE_GOOGLENET;
+    case PRE_DATA_PADDING_ZERO_FC3: return MSNH_PRE_PADDING_ZERO;
+    case PRE_DATA_TRANSFORMED_FC3:  return MSNH_PRE_TRANSFORMED;
+    case PRE_DATA_CAFFE_FC3:        return MSNH_PRE_CAFFE;
+    default: break;
+    }
+    MSNH_THROW("preDataType can't be none");
+}
+
+int runClassifyList(char **msg, unsigned char *imageData, const int width, const int height, const int channel, int *bestIndex, int preDataType,
+                    const int swapRGB, int runGPU, const float *mean, const float *std)
+{
+    return refStyle(msg, [&] {
+        if (!g_net) MSNH_THROW("initMsnhnet was not called");
+        if (!imageData || !bestIndex) MSNH_THROW("bad argument");
+        const int kind = preprocOf(preDataType, channel);
+        if (kind == MSNH_PRE_TRANSFORMED && (mean == nullptr || std == nullptr)) MSNH_THROW("mean or std can't be null");
+        if (!runGPU) g_net->runClassify(std::vector<float>());           // throws: this build has no CPU path
+        if (g_net->getBatch() != 1) MSNH_THROW("runClassifyList takes one image: build the graph with batch 1");
+        g_net->setInputImage(0, imageData, width, height, kind, mean, std, swapRGB != 0);
+        g_net->enqueueForward(nullptr);
+        const std::vector<float> out = g_net->fetchClassify();
+        *bestIndex = static_cast<int>(std::distance(out.begin(), std::max_element(out.begin(), out.end())));
+    });
+}
+
+int runYoloList(char **msg, unsigned char *imageData, const int width, const int height, const int channel, BBoxContainer *bboxContainer,
+                int *detectedNum, const int swapRGB, const int runGPU)
+{
+    return refStyle(msg, [&] {
+        if (!g_net) MSNH_THROW("initMsnhnet was not called");
+        if (!imageData || !bboxContainer || !detectedNum) MSNH_THROW("bad argument");
+        if (channel != 1 && channel != 3) MSNH_THROW("channel must be 1 or 3");
+        if (channel == 1) MSNH_THROW("1-channel images are outside the convolutional path this build implements");
+        if (!runGPU) g_net->runYolo(std::vector<float>());               // throws: this build has no CPU path
+        if (g_net->getBatch() != 1) MSNH_THROW("runYoloList takes one image: build the graph with batch 1");
+        g_net->setInputImage(0, imageData, width, height, MSNH_PRE_PADDING_ZERO, nullptr, nullptr, swapRGB != 0);
+        g_net->enqueueForward(nullptr);
+        const std::vector<std::vector<YoloBox>> out = g_net->fetchYolo();
+        const std::vector<YoloBox> &b0 = out.at(0);
+        if (b0.size() > MSNHNET_MAX_BBOX) MSNH_THROW("BBox buffer is not enough, please change MaxBBoxNum and rebuild");
+        *detectedNum = static_cast<int>(b0.size());
+        for (size_t i = 0; i < b0.size(); ++i)
+        {
+            BBox &o = bboxContainer->boxes[i];
+            o.x = b0[i].xywhBox.x; o.y = b0[i].xywhBox.y; o.w = b0[i].xywhBox.w; o.h = b0[i].xywhBox.h;
+            o.conf = b0[i].conf; o.bestClsConf = b0[i].bestClsConf; o.bestClsIdx = static_cast<uint32_t>(b0[i].bestClsIdx); o.angle = b0[i].angle;
+        }
+    });
+}
+
 int dispose(void) { g_net.reset(); return 1; }
 
 int withGPU(int *GPU)
@@ -352,6 +415,12 @@ long long msnhnet_yolo_max_boxes(msnhnet_t net)
 int msnhnet_set_input_image_u8(msnhnet_t net, int index, const unsigned char *rgb_hwc, int width, int height, int half_init, int shuffle_rgb)
 {
     return guarded([&] { nb(net).setInputImageU8(index, rgb_hwc, width, height, half_init != 0, shuffle_rgb != 0); });
+}
+
+int msnhnet_set_input_image(msnhnet_t net, int index, const unsigned char *rgb_hwc, int width, int height, int preproc, const float *mean3,
+                            const float *std3, int shuffle_rgb)
+{
+    return guarded([&] { nb(net).setInputImage(index, rgb_hwc, width, height, preproc, mean3, std3, shuffle_rgb != 0); });
 }
 
 int msnhnet_boxes_to_image(float *boxes, long long count, int net_w, int net_h, int org_w, int org_h, int padded)

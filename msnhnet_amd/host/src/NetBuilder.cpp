@@ -460,10 +460,16 @@ float *NetBuilder::deviceInputBuffer() { return _inputDev.as<float>(); }
 
 void NetBuilder::setInputImageU8(int index, const unsigned char *rgbHwc, int width, int height, bool halfInit, bool shuffleRGB)
 {
+    setInputImage(index, rgbHwc, width, height, halfInit ? MSNH_PRE_PADDING_ZERO_HALF : MSNH_PRE_PADDING_ZERO, nullptr, nullptr, shuffleRGB);
+}
+
+void NetBuilder::setInputImage(int index, const unsigned char *rgbHwc, int width, int height, int preproc, const float *mean, const float *std, bool shuffleRGB)
+{
     if (!_planReady) MSNH_THROW("weights are not loaded");
     if (rgbHwc == nullptr || width <= 0 || height <= 0) MSNH_THROW("img empty");
     if (_net->channels != 3) MSNH_THROW("the network does not take 3-channel images");
     if (index < 0 || index >= _net->batch) MSNH_THROW("image index outside the batch");
+    if (preproc == MSNH_PRE_TRANSFORMED && (mean == nullptr || std == nullptr)) MSNH_THROW("mean or std can't be null");
     const size_t bytes = static_cast<size_t>(width) * height * 3;
     // the pinned staging buffer is reused by the next call: wait for the previous upload before overwriting it
     MSNH_DEV(msnh_hip_stream_sync(_stream));
@@ -472,8 +478,8 @@ void NetBuilder::setInputImageU8(int index, const unsigned char *rgbHwc, int wid
     std::memcpy(_imagePinned.ptr(), rgbHwc, bytes);
     MSNH_DEV(msnh_hip_memcpy_h2d(_imageDev.ptr(), _imagePinned.ptr(), bytes, _stream));
     float *dst = _inputDev.as<float>() + static_cast<size_t>(index) * 3 * _net->height * _net->width;
-    MSNH_DEV(msnh_hip_letterbox_u8(static_cast<const unsigned char *>(_imageDev.ptr()), width, height, _net->width, _net->height,
-                                   halfInit ? 1 : 0, shuffleRGB ? 1 : 0, dst, _stream));
+    MSNH_DEV(msnh_hip_image_u8_to_input(static_cast<const unsigned char *>(_imageDev.ptr()), width, height, _net->width, _net->height, preproc, mean, std,
+                                        shuffleRGB ? 1 : 0, dst, _stream));
 }
 
 static std::vector<float> yoloLayerDump(Plan &plan, const YoloLayer *yl, const PlanOp &op, int batch, msnh_stream_t s)

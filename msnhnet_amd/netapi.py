@@ -12,8 +12,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libMsnhnet.so")
 
 SYMBOLS = [
-    "initMsnhnet", "buildMsnhnet", "runClassifyNoPred", "runYoloNoPred", "dispose", "withGPU", "withCUDNN", "getCpuForwardTime",
-    "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16", "msnhnet_set_use_winograd", "msnhnet_set_tune_cache", "msnhnet_set_device_nms", "msnhnet_set_input_image_u8", "msnhnet_boxes_to_image",
+    "initMsnhnet", "buildMsnhnet", "runClassifyNoPred", "runYoloNoPred", "runClassifyList", "runYoloList", "dispose", "withGPU", "withCUDNN", "getCpuForwardTime",
+    "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16", "msnhnet_set_use_winograd", "msnhnet_set_tune_cache", "msnhnet_set_device_nms", "msnhnet_set_input_image_u8", "msnhnet_set_input_image", "msnhnet_boxes_to_image",
     "msnhnet_set_keep_class_scores", "msnhnet_set_save_layer_output", "msnhnet_build", "msnhnet_load", "msnhnet_load_from_memory",
     "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops",
     "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
@@ -57,6 +57,9 @@ def lib():
     L.buildMsnhnet.argtypes = [cpp, cp, cp, ci, ci]
     L.runClassifyNoPred.argtypes = [cpp, fp, ci, ip, ci]
     L.runYoloNoPred.argtypes = [cpp, fp, ci, ctypes.POINTER(BBoxContainer), ip, ci]
+    u8p = ctypes.POINTER(ctypes.c_ubyte)
+    L.runClassifyList.argtypes = [cpp, u8p, ci, ci, ci, ip, ci, ci, ci, fp, fp]
+    L.runYoloList.argtypes = [cpp, u8p, ci, ci, ci, ctypes.POINTER(BBoxContainer), ip, ci, ci]
     L.withGPU.argtypes = [ip]
     L.withCUDNN.argtypes = [ip]
     L.getCpuForwardTime.argtypes = [fp]
@@ -70,6 +73,7 @@ def lib():
     L.msnhnet_set_tune_cache.argtypes = [ci]
     L.msnhnet_set_device_nms.argtypes = [ci]
     L.msnhnet_set_input_image_u8.argtypes = [vp, ci, ctypes.POINTER(ctypes.c_ubyte), ci, ci, ci, ci]
+    L.msnhnet_set_input_image.argtypes = [vp, ci, ctypes.POINTER(ctypes.c_ubyte), ci, ci, ci, fp, fp, ci]
     L.msnhnet_boxes_to_image.argtypes = [fp, ll, ci, ci, ci, ci, ci]
     L.msnhnet_set_keep_class_scores.argtypes = [ci]
     L.msnhnet_set_save_layer_output.argtypes = [vp, ci]
@@ -296,6 +300,17 @@ class Net:
             raise ValueError("3-channel image expected")
         _check(self.L.msnhnet_set_input_image_u8(self.h, index, a.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte)), w, h,
                                                  int(half_init), int(shuffle_rgb)))
+
+    def set_input_image(self, index, img, preproc, mean=None, std=None, shuffle_rgb=False):
+        """img: HWC uint8, 3 channels; pre-processed on the device (preproc: a msnh_preproc value of include/msnh_hip.h) into slot `index`."""
+        a = np.ascontiguousarray(img, np.uint8)
+        h, w, c = a.shape
+        if c != 3:
+            raise ValueError("3-channel image expected")
+        m = np.ascontiguousarray(mean, np.float32) if mean is not None else None
+        sd = np.ascontiguousarray(std, np.float32) if std is not None else None
+        _check(self.L.msnhnet_set_input_image(self.h, index, a.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte)), w, h, int(preproc),
+                                              _fp(m) if m is not None else None, _fp(sd) if sd is not None else None, int(shuffle_rgb)))
 
     def profile_ops(self, kind, reps):
         """-> (total ms, launches, algorithmic FLOPs) of `reps` eager passes over the launches of one kind (-1 = all)."""

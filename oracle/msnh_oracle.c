@@ -627,6 +627,68 @@ void msnh_or_letterbox_u8(const unsigned char *img, int width, int height, int n
     free(sq);
 }
 
+/* The plain-resize pre-processing variants of CVUtil for a 3-channel 8-bit image (src/utils/MsnhCVUtil.cpp):
+ *   kind 0  getImgDataF32C3, halfInit 0 (:91-138)      u / 255
+ *   kind 1  getImgDataF32C3, halfInit 1                 (u - 127.5) / 127.5
+ *   kind 2  getGoogLenetF32C3 (:146-195)                u / 255 * (std_k / 0.5) + (mean_k - 0.5) / 0.5  with the ImageNet constants written there
+ *   kind 3  getTransformedF32C3 (:269-318)              (u / 255 - mean[k]) / std[k]
+ *   kind 4  getCaffeModeF32C3 (:326-375)                u - {123.68, 116.779, 103.939}[k]
+ * all after MatOp::resize to (netW, netH) (src/cv/MsnhCVMatOp.cpp:142-160, 404-437: fx = srcW / dstW, fy = srcH / dstH, see
+ * msnh_or_letterbox_u8 for the arithmetic; no resize when the size already matches) and the optional RGB2BGR swap; HWC -> CHW. */
+void msnh_or_preproc_u8(const unsigned char *img, int width, int height, int netW, int netH, int kind, const float *mean,
+                        const float *stdv, int shuffleRGB, float *out)
+{
+    const unsigned char *rs = img;
+    unsigned char *tmp = NULL;
+    if (!(netW == width && netH == height))
+    {
+        tmp = (unsigned char *)calloc((size_t)netW * netH * 3, 1);
+        const float fx = 1.f * width / netW;
+        const float fy = 1.f * height / netH;
+        for (int i = 0; i < netH; ++i)
+        {
+            float sh = (i + 0.5f) * fy - 0.5f;
+            sh = sh < 0 ? 0 : sh;
+            const int h0 = (int)sh;
+            const int h1 = h0 + 1 < height - 1 ? h0 + 1 : height - 1;
+            for (int j = 0; j < netW; ++j)
+            {
+                float sw = (j + 0.5f) * fx - 0.5f;
+                sw = sw < 0 ? 0 : sw;
+                const int w0 = (int)sw;
+                const int w1 = w0 + 1 < width - 1 ? w0 + 1 : width - 1;
+                for (int k = 0; k < 3; ++k)
+                {
+                    const float v = (h1 - sh) * ((w1 - sw) * img[3 * ((size_t)h0 * width + w0) + k] + (sw - w0) * img[3 * ((size_t)h0 * width + w1) + k]) +
+                                    (sh - h0) * ((w1 - sw) * img[3 * ((size_t)h1 * width + w0) + k] + (sw - w0) * img[3 * ((size_t)h1 * width + w1) + k]);
+                    const unsigned short r = (unsigned short)v;
+                    tmp[3 * ((size_t)i * netW + j) + k] = (unsigned char)(r > 255 ? 255 : r);
+                }
+            }
+        }
+        rs = tmp;
+    }
+    static const float gStd[3] = {0.229f, 0.224f, 0.225f}, gMean[3] = {0.485f, 0.456f, 0.406f};
+    static const float caffe[3] = {123.68f, 116.779f, 103.939f};
+    for (int y = 0; y < netH; ++y)
+        for (int k = 0; k < 3; ++k)
+            for (int x = 0; x < netW; ++x)
+            {
+                const unsigned char u = rs[3 * ((size_t)y * netW + x) + (shuffleRGB ? 2 - k : k)];
+                float v;
+                switch (kind)
+                {
+                case 1:  v = (u - 127.5f) / 127.5f; break;
+                case 2:  v = u / 255.0f * (gStd[k] / 0.5f) + (gMean[k] - 0.5f) / 0.5f; break;
+                case 3:  v = ((u / 255.0f) - mean[k]) / stdv[k]; break;
+                case 4:  v = (u) - caffe[k]; break;
+                default: v = u / 255.0f; break;
+                }
+                out[(size_t)k * netW * netH + (size_t)y * netW + x] = v;
+            }
+    free(tmp);
+}
+
 /* YoloOutLayer::bboxResize2Org (src/layers/MsnhYoloOutLayer.cpp:321-361): undo the letterbox */
 void msnh_or_bbox_resize2org(float *b, int curW, int curH, int orgW, int orgH)
 {

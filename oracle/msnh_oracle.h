@@ -68,6 +68,8 @@ long long msnh_or_yolo_out(const float *const *heads, const int *hw, int nHeads,
  * optional R<->B swap, scale to [0,1] (half_init 0) or [-1,1] (half_init 1), HWC -> CHW float. */
 void  msnh_or_letterbox_u8(const unsigned char *img, int width, int height, int netW, int netH, int halfInit,
                            int shuffleRGB, float *out);
+void  msnh_or_preproc_u8(const unsigned char *img, int width, int height, int netW, int netH, int kind, const float *mean,
+                          const float *stdv, int shuffleRGB, float *out);
 /* Box (x y w h, centre form, network-input pixels) back to the original image; in place. */
 void  msnh_or_bbox_resize2org(float *xywh, int curW, int curH, int orgW, int orgH);
 void  msnh_or_bbox_resize2org_nopad(float *xywh, int curW, int curH, int orgW, int orgH);

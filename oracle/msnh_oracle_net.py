@@ -50,6 +50,7 @@ def lib():
         L.msnh_or_iou.restype = cf
         L.msnh_or_yolo_out.argtypes = [ctypes.POINTER(_fp), ctypes.POINTER(ci), ci, ci, cf, cf, _fp, ll]
         L.msnh_or_letterbox_u8.argtypes = [ctypes.POINTER(ctypes.c_ubyte), ci, ci, ci, ci, ci, ci, _fp]
+        L.msnh_or_preproc_u8.argtypes = [ctypes.POINTER(ctypes.c_ubyte), ci, ci, ci, ci, ci, _fp, _fp, ci, _fp]
         L.msnh_or_bbox_resize2org.argtypes = [_fp, ci, ci, ci, ci]
         L.msnh_or_bbox_resize2org_nopad.argtypes = [_fp, ci, ci, ci, ci]
         L.msnh_or_yolo_out.restype = ll
@@ -212,6 +213,20 @@ def letterbox_u8(img, net_w, net_h, half_init=False, shuffle_rgb=False):
     assert c == 3
     out = np.empty((3, net_h, net_w), np.float32)
     lib().msnh_or_letterbox_u8(a.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte)), w, h, net_w, net_h, int(half_init), int(shuffle_rgb), _p(out))
+    return out
+
+
+PREPROC_KINDS = {"f32c3": 0, "f32c3_half": 1, "googlenet": 2, "transformed": 3, "caffe": 4}
+
+
+def preproc_u8(img, net_w, net_h, kind="f32c3", mean=(0, 0, 0), std=(1, 1, 1), shuffle_rgb=False):
+    """img: HWC uint8 with 3 channels -> CHW float32 network input by plain bilinear resize + one of the reference's normalisations."""
+    a = np.ascontiguousarray(img, np.uint8)
+    h, w, c = a.shape
+    assert c == 3
+    out = np.empty((3, net_h, net_w), np.float32)
+    m, sd = _f32(mean), _f32(std)
+    lib().msnh_or_preproc_u8(a.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte)), w, h, net_w, net_h, PREPROC_KINDS[kind], _p(m), _p(sd), int(shuffle_rgb), _p(out))
     return out
 
 

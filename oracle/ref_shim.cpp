@@ -278,6 +278,35 @@ int ref_letterbox_u8(const unsigned char *img, int width, int height, int netW, 
     }
 }
 
+// The plain-resize pre-processing variants of CVUtil on a 3-channel 8-bit HWC image; dst holds 3*netW*netH floats (CHW).
+// kind: 0 getImgDataF32C3, 1 the same with halfInit, 2 getGoogLenetF32C3, 3 getTransformedF32C3(mean, std), 4 getCaffeModeF32C3.
+int ref_preproc_u8(const unsigned char *img, int width, int height, int netW, int netH, int kind, const float *mean, const float *stdv,
+                   int shuffleRGB, float *dst, char *err, int errCap)
+{
+    try
+    {
+        Mat mat(width, height, MAT_RGB_U8, const_cast<unsigned char*>(img));
+        std::vector<float> v;
+        const Vec2I32 size(netW, netH);
+        switch(kind)
+        {
+        case 0: v = CVUtil::getImgDataF32C3(mat, size, false, shuffleRGB != 0); break;
+        case 1: v = CVUtil::getImgDataF32C3(mat, size, true, shuffleRGB != 0); break;
+        case 2: v = CVUtil::getGoogLenetF32C3(mat, size, shuffleRGB != 0); break;
+        case 3: v = CVUtil::getTransformedF32C3(mat, size, Vec3F32(mean[0], mean[1], mean[2]), Vec3F32(stdv[0], stdv[1], stdv[2]), shuffleRGB != 0); break;
+        case 4: v = CVUtil::getCaffeModeF32C3(mat, size, shuffleRGB != 0); break;
+        default: throw Exception(1, "unknown kind", __FILE__, __LINE__, __FUNCTION__);
+        }
+        std::memcpy(dst, v.data(), v.size() * sizeof(float));
+        return 0;
+    }
+    catch(Exception &e)
+    {
+        std::snprintf(err, static_cast<size_t>(errCap), "%s", e.what());
+        return 1;
+    }
+}
+
 // YoloOutLayer::bboxResize2Org / bboxResize2OrgNoPad on one box given as x y w h; in place.
 void ref_bbox_resize2org(float *xywh, int curW, int curH, int orgW, int orgH, int noPad)
 {

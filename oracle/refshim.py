@@ -1,11 +1,13 @@
-"""ctypes binding of oracle/_ref/libmsnh_ref.so (the reference's own CPU forward; checker only)."""
+"""TEST INFRASTRUCTURE ONLY.  ctypes binding of oracle/_ref/libmsnh_ref.so (the reference's own CPU forward, built by
+oracle/Makefile from the reference sources where they lie): the checker of the parity tests and the timed CPU baseline of
+bench.py.  Nothing in the product package imports it."""
 import ctypes
 import os
 
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-REF_SO = os.path.join(_HERE, "..", "oracle", "_ref", "libmsnh_ref.so")
+REF_SO = os.path.join(_HERE, "_ref", "libmsnh_ref.so")
 
 LAYER_TYPE = {0: "conv", 2: "connect", 3: "maxpool", 4: "localavgpool", 8: "route", 13: "batchnorm",
               15: "yolo", 16: "yoloout", 18: "upsample", 20: "empty", 27: "resblock", 28: "res2block",
@@ -46,6 +48,7 @@ def lib():
         u8p = ctypes.POINTER(ctypes.c_ubyte)
         L.ref_letterbox_u8.argtypes = [u8p, ci, ci, ci, ci, ci, ci, fp, cp, ci]
         L.ref_bbox_resize2org.argtypes = [fp, ci, ci, ci, ci, ci]
+        L.ref_preproc_u8.argtypes = [u8p, ci, ci, ci, ci, ci, fp, fp, ci, fp, cp, ci]
         _lib = L
     return _lib
 
@@ -139,6 +142,27 @@ def letterbox_u8(img, net_w, net_h, half_init=False, shuffle_rgb=False):
     err = ctypes.create_string_buffer(1024)
     rc = lib().ref_letterbox_u8(a.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte)), w, h, net_w, net_h, int(half_init), int(shuffle_rgb),
                                 out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), err, 1024)
+    if rc != 0:
+        raise RefError(err.value.decode())
+    return out
+
+
+PREPROC_KINDS = {"f32c3": 0, "f32c3_half": 1, "googlenet": 2, "transformed": 3, "caffe": 4}
+
+
+def preproc_u8(img, net_w, net_h, kind="f32c3", mean=(0, 0, 0), std=(1, 1, 1), shuffle_rgb=False):
+    """img: HWC uint8, 3 channels.  CVUtil::getImgDataF32C3 / getGoogLenetF32C3 / getTransformedF32C3 / getCaffeModeF32C3 -> CHW float32."""
+    import numpy as np
+    a = np.ascontiguousarray(img, np.uint8)
+    h, w, c = a.shape
+    assert c == 3
+    out = np.empty((3, net_h, net_w), np.float32)
+    m = np.ascontiguousarray(mean, np.float32)
+    sd = np.ascontiguousarray(std, np.float32)
+    fp = ctypes.POINTER(ctypes.c_float)
+    err = ctypes.create_string_buffer(1024)
+    rc = lib().ref_preproc_u8(a.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte)), w, h, net_w, net_h, PREPROC_KINDS[kind], m.ctypes.data_as(fp),
+                              sd.ctypes.data_as(fp), int(shuffle_rgb), out.ctypes.data_as(fp), err, 1024)
     if rc != 0:
         raise RefError(err.value.decode())
     return out

@@ -13,7 +13,7 @@ import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
-for p in (ROOT, os.path.join(ROOT, "tests")):
+for p in (ROOT, os.path.join(ROOT, "tests"), os.path.join(ROOT, "oracle")):
     sys.path.insert(0, p)
 
 import refshim  # noqa: E402
@@ -24,6 +24,7 @@ TMP = "/tmp/msnh_golden"
 os.makedirs(TMP, exist_ok=True)
 
 
+PREPROC_CASES = [(40, 56, 32, 24, 11), (31, 20, 40, 40, 12), (24, 24, 24, 24, 13)]
 LETTERBOX_CASES = [(48, 64, 40, 40, 1), (70, 50, 64, 64, 2), (30, 30, 52, 52, 3), (36, 36, 36, 36, 4)]
 
 
@@ -99,6 +100,15 @@ def micro_cases():
                                                    q.yoloout([1], 0.3, 0.45, yolo_type="yolov5"))),
         "yolo_head": lambda: g(8, 6, 6, lambda q: (q.conv(21, 1, 1, 0, bn=0, act="none"), q.yolo([10, 13, 16, 30, 33, 23], class_num=2),
                                                   q.yoloout([1], 0.3, 0.45))),
+        # a subtraction whose minuend / subtrahend is a convolution nobody else reads (the add moves into that convolution's launch
+        # where the arithmetic allows it): previous layer - layer 0, layer 0 - previous layer, layer 0 - layer 2
+        "varop_sub_conv": lambda: g(4, 6, 7, lambda q: (q.conv(6, 3, 1, 1, bn=0, act="none"), q.conv(6, 1, 1, 0, bn=0, act="relu"),
+                                                       q.conv(6, 3, 1, 1, bn=1, act="leaky"), q.varop("sub", [0]), q.act("relu"))),
+        "varop_subinv_conv": lambda: g(4, 6, 7, lambda q: (q.conv(6, 3, 1, 1, bn=0, act="none"), q.conv(6, 1, 1, 0, bn=0, act="relu"),
+                                                          q.conv(6, 3, 1, 1, bn=1, act="leaky"), q.varop("subInv", [0]), q.act("relu"))),
+        "varop_sub_conv_second": lambda: g(4, 6, 7, lambda q: (q.conv(6, 3, 1, 1, bn=0, act="none"), q.conv(6, 1, 1, 0, bn=0, act="relu"),
+                                                              q.conv(6, 3, 1, 1, bn=1, act="leaky"), q.conv(6, 1, 1, 0, bn=0, act="none"),
+                                                              q.varop("sub", [0, 2]))),
     }
     return cases
 
@@ -147,6 +157,32 @@ def main():
         store[f"net/{arch}/weights_sum"] = np.array([np.float64(np.fromfile(binp, np.float32).astype(np.float64).sum())])
         r.close()
 
+    # YOLOv4 at its full benchmark size: 70 s per image on the scalar build, so the GPU tests cannot run the reference there.  First and
+    # last image of the batch of 16 the full-size test feeds (weights seed 5, input seed 6): per-layer statistics, samples of the three
+    # head logit tensors, and the boxes (count, class histogram, every 8th box of the sorted list).
+    netp, binp, gw = zoo.write_model("yolov4", TMP, 1, 608, seed=5)
+    xs = zoo.seeded_input(16, 3, 608, 608, 6)
+    r = refshim.RefNet(netp, binp, scalar=True)
+    heads = [i - 1 for i in range(r.num_layers()) if r.layer_info(i)["type"] == "yolo"]
+    for slot in (0, 15):
+        outs = r.run(xs[slot])
+        key = f"full/yolov4/slot{slot}"
+        store[f"{key}/stats"] = np.stack([layer_stats(o) for o in outs])
+        for k, li in enumerate(heads):
+            idx = (np.arange(4096, dtype=np.int64) * 104729) % outs[li].size
+            store[f"{key}/head{k}_idx"] = idx
+            store[f"{key}/head{k}_val"] = outs[li][idx]
+            store[f"{key}/head{k}_absmax"] = np.array([np.abs(outs[li]).max()], np.float64)
+        b = r.boxes()
+        key7 = np.nan_to_num(b, nan=1e30, posinf=2e30, neginf=-2e30)
+        b = b[np.lexsort(key7.T[::-1])] if len(b) else b
+        store[f"{key}/box_count"] = np.array([len(b)], np.int64)
+        store[f"{key}/class_hist"] = np.bincount(b[:, 6].astype(np.int64), minlength=80) if len(b) else np.zeros(80, np.int64)
+        store[f"{key}/boxes_every8"] = b[::8]
+        print("yolov4-608 slot", slot, "boxes", len(b), "wall ms", r.wall_ms(), flush=True)
+    store["full/yolov4/heads"] = np.array(heads, np.int64)
+    r.close()
+
     # full-size shape tables and the reference's own layer-detail text
     for arch, dtype, batch, size in zoo.CONFIGS:
         gw = zoo.ARCHS[arch](batch=1, size=size)
@@ -168,6 +204,15 @@ def main():
             out = refshim.letterbox_u8(img, nw, nh, False, bool(shuffle))
             store[f"letterbox/{idx}/shuffle{shuffle}"] = np.rint(out * 255.0).astype(np.uint8)
         store[f"letterbox/{idx}/case"] = np.array([h, w, nw, nh, seed], np.int64)
+    # the plain-resize variants (CVUtil::getImgDataF32C3, getGoogLenetF32C3, getTransformedF32C3, getCaffeModeF32C3)
+    for idx, (h, w, nw, nh, seed) in enumerate(PREPROC_CASES):
+        img = np.random.default_rng(seed).integers(0, 256, (h, w, 3), dtype=np.uint8)
+        mean, std = np.array([0.4, 0.5, 0.6], np.float32), np.array([0.2, 0.3, 0.25], np.float32)
+        for kind in refshim.PREPROC_KINDS:
+            store[f"preproc/{idx}/{kind}"] = refshim.preproc_u8(img, nw, nh, kind, mean, std, bool(idx % 2))
+        store[f"preproc/{idx}/case"] = np.array([h, w, nw, nh, seed], np.int64)
+        store[f"preproc/{idx}/mean"] = mean
+        store[f"preproc/{idx}/std"] = std
     rng = np.random.default_rng(77)
     rows = []
     for _ in range(40):

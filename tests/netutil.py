@@ -55,6 +55,65 @@ def sort_boxes(b):
     return b[np.lexsort(key.T[::-1])]
 
 
+def _box_embedding(b):
+    """rows of 7 floats -> points whose Euclidean neighbours are the boxes that nearly equal them (sizes on a log scale: they
+    overflow to inf with the seeded weights; the class index far apart)"""
+    k = np.asarray(b, np.float64).reshape(-1, 7).copy()
+    wh = k[:, 2:4]
+    wh = np.where(np.isnan(wh), 400.0, np.sign(wh) * np.log1p(np.minimum(np.abs(wh), 1e300)))
+    k[:, 2:4] = np.where(np.isinf(k[:, 2:4]), np.sign(k[:, 2:4]) * 800.0, wh)
+    k[:, 0:2] = np.nan_to_num(k[:, 0:2], nan=1e6, posinf=2e6, neginf=-2e6)
+    k[:, 4:6] = np.nan_to_num(k[:, 4:6], nan=50.0) * 100.0
+    k[:, 6] *= 1e4
+    return k
+
+
+def boxes_one_sided_err(sub, full):
+    """every box of `sub` has a box of `full` next to it: returns the largest column-wise deviation |sub - nearest| / max|full| over the
+    finite entries (non-finite entries and the class index must agree exactly).  Unlike a comparison of two sorted lists this does not
+    depend on how boxes that differ in the last bits are ordered."""
+    from scipy.spatial import cKDTree
+    sub = np.asarray(sub, np.float32).reshape(-1, 7)
+    full = np.asarray(full, np.float32).reshape(-1, 7)
+    if len(sub) == 0:
+        return 0.0
+    assert len(full) > 0, "no boxes to match against"
+    _, idx = cKDTree(_box_embedding(full)).query(_box_embedding(sub))
+    near = full[idx]
+    assert np.array_equal(sub[:, 6], near[:, 6]), "class of the nearest box differs"
+    return rel_err(sub[:, :6], near[:, :6])
+
+
+def boxes_matched_fraction(got, ref, tol):
+    """fraction of the boxes of `got` that have a box of `ref` of the same class within tol * max|ref| in every finite column.  For
+    comparisons across two builds of a plan: with the seeded weights most objectness values saturate at exactly 1, suppression among
+    such ties depends on the last bit of the few values that do not, and two tile choices differ in exactly those bits -- so a few
+    boxes of a crowded image may legitimately be replaced by their neighbours."""
+    from scipy.spatial import cKDTree
+    got = np.asarray(got, np.float32).reshape(-1, 7)
+    ref = np.asarray(ref, np.float32).reshape(-1, 7)
+    if len(got) == 0 or len(ref) == 0:
+        return 1.0 if len(got) == len(ref) else 0.0
+    _, idx = cKDTree(_box_embedding(ref)).query(_box_embedding(got))
+    near = ref[idx].astype(np.float64)
+    g = got.astype(np.float64)
+    fin = np.isfinite(near[:, :6])
+    scale = max(np.abs(near[:, :6][fin]).max(), 1e-30) if fin.any() else 1.0
+    with np.errstate(invalid="ignore"):
+        ok_fin = np.where(fin, np.abs(g[:, :6] - near[:, :6]) <= tol * scale, True)
+        ok_inf = np.where(fin, True, (g[:, :6] == near[:, :6]) | (np.isnan(g[:, :6]) & np.isnan(near[:, :6])))
+    ok = ok_fin.all(1) & ok_inf.all(1) & (g[:, 6] == near[:, 6])
+    return float(ok.mean())
+
+
+def boxes_err(got, ref):
+    """two box sets agree: same count, and each box of either set has a box of the other next to it (see boxes_one_sided_err)"""
+    got = np.asarray(got, np.float32).reshape(-1, 7)
+    ref = np.asarray(ref, np.float32).reshape(-1, 7)
+    assert len(got) == len(ref), f"box count {len(got)} vs {len(ref)}"
+    return max(boxes_one_sided_err(got, ref), boxes_one_sided_err(ref, got))
+
+
 def yolo_layer_err(got, ref, logits, channels_per_anchor, ratio, version=3):
     """Error of a decoded yolo layer [3*per, H*W] in units of the logit error that explains it.
 

@@ -19,7 +19,7 @@ GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_golden.npz
 def _declared(header):
     text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b((?:msnh_hip_|msnhnet_)\w+|initMsnhnet|buildMsnhnet|runClassifyNoPred|runYoloNoPred|dispose|withGPU|withCUDNN|"
+    return sorted(set(re.findall(r"\b((?:msnh_hip_|msnhnet_)\w+|initMsnhnet|buildMsnhnet|runClassifyNoPred|runYoloNoPred|runClassifyList|runYoloList|dispose|withGPU|withCUDNN|"
                                  r"getCpuForwardTime|getGpuForwardTime|getInputDim)\s*\(", text)))
 
 

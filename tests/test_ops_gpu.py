@@ -518,3 +518,32 @@ def test_letterbox_u8(h, w, nw, nh):
             assert np.array_equal(dst.cpu().numpy(), on.letterbox_u8(img, nw, nh, bool(half), bool(shuffle)))
     assert abi.lib().msnh_hip_letterbox_u8(gu.ptr(src), w, h, 0, nh, 0, 0, gu.ptr(dst), None) != 0
     assert b"letterbox" in abi.lib().msnh_hip_last_error()
+
+
+@pytest.mark.parametrize("h,w,nw,nh", [(480, 640, 224, 224), (50, 80, 64, 48), (33, 33, 32, 32), (224, 224, 224, 224), (20, 33, 96, 96)])
+def test_image_u8_to_input(h, w, nw, nh):
+    """device resize + normalisation == the restatement of the reference's CVUtil variants, bit for bit (no fused multiply-add in either)"""
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(h + 5 * w)
+    img = rng.integers(0, 256, (h, w, 3), dtype=np.uint8)
+    src = torch.from_numpy(img).cuda()
+    mean, std = np.array([0.4, 0.5, 0.6], np.float32), np.array([0.2, 0.3, 0.25], np.float32)
+    fp = ctypes.POINTER(ctypes.c_float)
+    kinds = {"f32c3": 0, "f32c3_half": 1, "googlenet": 2, "transformed": 3, "caffe": 4}
+    for kind, code in kinds.items():
+        for shuffle in (0, 1):
+            dst = torch.full((3, nh, nw), -5.0, dtype=torch.float32).cuda()
+            gu.sync()
+            abi.check(abi.lib().msnh_hip_image_u8_to_input(gu.ptr(src), w, h, nw, nh, code, mean.ctypes.data_as(fp), std.ctypes.data_as(fp), shuffle, gu.ptr(dst), None))
+            gu.sync()
+            assert np.array_equal(dst.cpu().numpy(), on.preproc_u8(img, nw, nh, kind, mean, std, bool(shuffle))), (kind, shuffle)
+    for code, half in ((5, False), (6, True)):
+        dst = torch.full((3, nh, nw), -5.0, dtype=torch.float32).cuda()
+        gu.sync()
+        abi.check(abi.lib().msnh_hip_image_u8_to_input(gu.ptr(src), w, h, nw, nh, code, None, None, 0, gu.ptr(dst), None))
+        gu.sync()
+        assert np.array_equal(dst.cpu().numpy(), on.letterbox_u8(img, nw, nh, half, False))
+    assert abi.lib().msnh_hip_image_u8_to_input(gu.ptr(src), w, h, nw, nh, 3, None, None, 0, gu.ptr(dst), None) != 0
+    assert b"mean or std" in abi.lib().msnh_hip_last_error()
+    assert abi.lib().msnh_hip_image_u8_to_input(gu.ptr(src), w, h, nw, nh, 9, None, None, 0, gu.ptr(dst), None) != 0

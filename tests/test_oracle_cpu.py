@@ -360,6 +360,81 @@ def test_letterbox_mathematics():
     assert np.all(up[:, :15, :15] == 200) and np.all(up[:, 15, :] == 0) and np.all(up[:, :, 15] == 0)
 
 
+PREPROC_SHAPES = [(480, 640, 224, 224), (50, 80, 64, 48), (33, 33, 32, 32), (224, 224, 224, 224), (20, 33, 96, 96)]
+
+
+@pytest.mark.parametrize("h,w,nw,nh", PREPROC_SHAPES)
+def test_preproc_against_reference(h, w, nw, nh):
+    """The plain-resize variants against CVUtil::getImgDataF32C3 / getGoogLenetF32C3 / getTransformedF32C3 / getCaffeModeF32C3
+    themselves.  As for the letterbox, the reference build fuses multiply-adds: a few pixels per million land one 8-bit step
+    apart, and the GoogLeNet form differs by an ulp."""
+    if not refshim.available():
+        pytest.skip("reference build not present")
+    rng = np.random.default_rng(h * 5 + w)
+    img = rng.integers(0, 256, (h, w, 3), dtype=np.uint8)
+    mean, std = (0.4, 0.5, 0.6), (0.2, 0.3, 0.25)
+    step = {"f32c3": 1 / 255.0, "f32c3_half": 1 / 127.5, "googlenet": 0.458 / 255.0, "transformed": 1 / 255.0 / 0.2, "caffe": 1.0}
+    for kind in on.PREPROC_KINDS:
+        for shuffle in (False, True):
+            a = on.preproc_u8(img, nw, nh, kind, mean, std, shuffle)
+            b = refshim.preproc_u8(img, nw, nh, kind, mean, std, shuffle)
+            d = np.abs(a - b)
+            assert d.max() <= step[kind] * 1.001, (kind, d.max())
+            assert (d > 1e-6).mean() <= 1e-3, (kind, (d > 1e-6).mean())
+
+
+def test_preproc_mathematics():
+    rng = np.random.default_rng(21)
+    img = rng.integers(0, 256, (12, 17, 3), dtype=np.uint8)
+    chw = img.transpose(2, 0, 1).astype(np.float32)
+    f = np.float32
+    # same size: only the normalisation, in the reference's float expressions
+    assert np.array_equal(on.preproc_u8(img, 17, 12, "f32c3"), chw / f(255.0))
+    assert np.array_equal(on.preproc_u8(img, 17, 12, "f32c3", shuffle_rgb=True), (chw / f(255.0))[::-1])
+    assert np.array_equal(on.preproc_u8(img, 17, 12, "f32c3_half"), (chw - f(127.5)) / f(127.5))
+    gs, gm = np.array([0.229, 0.224, 0.225], f), np.array([0.485, 0.456, 0.406], f)
+    want = chw / f(255.0) * (gs / f(0.5))[:, None, None] + ((gm - f(0.5)) / f(0.5))[:, None, None]
+    assert np.array_equal(on.preproc_u8(img, 17, 12, "googlenet"), want.astype(f))
+    mean, std = np.array([0.4, 0.5, 0.6], f), np.array([0.2, 0.3, 0.25], f)
+    assert np.array_equal(on.preproc_u8(img, 17, 12, "transformed", mean, std), ((chw / f(255.0)) - mean[:, None, None]) / std[:, None, None])
+    assert np.array_equal(on.preproc_u8(img, 17, 12, "caffe"), chw - np.array([123.68, 116.779, 103.939], f)[:, None, None])
+    # the GoogLeNet form is the ImageNet normalisation re-expressed for a net trained on (x - 0.5) / 0.5 inputs (closed form, double)
+    x = chw.astype(np.float64) / 255.0
+    ident = (x * gs.astype(np.float64)[:, None, None] + gm.astype(np.float64)[:, None, None] - 0.5) / 0.5
+    assert np.abs(on.preproc_u8(img, 17, 12, "googlenet") - ident).max() < 1e-6
+    # a square image: plain resize == letterbox (nothing to pad)
+    sq = rng.integers(0, 256, (30, 30, 3), dtype=np.uint8)
+    assert np.array_equal(on.preproc_u8(sq, 20, 20, "f32c3"), on.letterbox_u8(sq, 20, 20))
+    # separate scale factors per axis: halving only the width of an image whose column pairs are equal returns the pair values.
+    # Along the axis that keeps its size the reference's weights (i1 - s) and (s - i0) are both zero on the last row / column
+    # (second sample index clamped to the first): that line comes out 0, as it does when enlarging.
+    small = rng.integers(0, 256, (9, 8, 3), dtype=np.uint8)
+    want = small.transpose(2, 0, 1).astype(f) / f(255.0)
+    wide = np.repeat(small, 2, axis=1)
+    got = on.preproc_u8(wide, 8, 9, "f32c3")
+    assert np.array_equal(got[:, :8], want[:, :8]) and np.all(got[:, 8] == 0)
+    tall = np.repeat(small, 2, axis=0)
+    got = on.preproc_u8(tall, 8, 9, "f32c3")
+    assert np.array_equal(got[:, :, :7], want[:, :, :7]) and np.all(got[:, :, 7] == 0)
+
+
+def test_preproc_against_golden():
+    """vectors written by the reference build (present also where the build is not)"""
+    idx = 0
+    while f"preproc/{idx}/case" in GOLD.files:
+        h, w, nw, nh, seed = (int(v) for v in GOLD[f"preproc/{idx}/case"])
+        img = np.random.default_rng(seed).integers(0, 256, (h, w, 3), dtype=np.uint8)
+        mean, std = GOLD[f"preproc/{idx}/mean"], GOLD[f"preproc/{idx}/std"]
+        for kind in on.PREPROC_KINDS:
+            want = GOLD[f"preproc/{idx}/{kind}"]
+            got = on.preproc_u8(img, nw, nh, kind, mean, std, bool(idx % 2))
+            scale = {"f32c3": 255.0, "f32c3_half": 127.5, "googlenet": 255.0 / 0.44, "transformed": 255.0 * float(std.min()), "caffe": 1.0}[kind]
+            d = np.abs(got - want) * scale
+            assert d.max() <= 1.05 and (d > 1e-3).mean() <= 1e-3, (idx, kind, d.max())
+        idx += 1
+    assert idx >= 3
+
+
 def test_bbox_back_to_image():
     # 1280x720 letterboxed into 608x608: scale 0.475, 133 rows of padding above; the centre maps to the centre
     b = on.bbox_resize2org([304.0, 304.0, 95.0, 47.5], 608, 608, 1280, 720)
