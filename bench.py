@@ -6,6 +6,13 @@
 A step is one forward of one batch through NetBuilder's device-resident path (input already in HBM): every
 launch of the planned graph, and for detection networks the candidate compaction on the device plus copy-back,
 sort and NMS on the host, so that a step ends with the boxes (or logits) in host memory.  Prints ONE JSON line.
+`value` is the whole-job rate over the K timed steps; the median of the per-step times is reported beside it.
+
+    python bench.py --conv-shape b,c,h,w,oc,k,stride [--tile n] [--reps 20] [--residual] [--conv-dtype f16|f32]
+
+times one convolution shape through the kernel C ABI instead: with every implicit-GEMM tile configuration that accepts
+it (microseconds and TFLOP/s per tile), or, with --tile, launches that configuration --reps times and nothing else,
+which is the form to put behind `rocprofv3 --pmc ... --` when the counters of one kernel are wanted.
 """
 import argparse
 import json
@@ -32,7 +39,6 @@ PEAK = {"f16": 2500.0, "f32": 157.3}        # dense MFMA peak, TFLOP/s
 def cpu_baseline(arch, size, tmp, seed, budget_s=30.0):
     """Reference CPU forward (its own code, as shipped: AVX2+FMA, all OpenMP threads) on a bounded sample of the
     same workload: batch-1 forwards of the same graph and weights, repeated while they fit the time budget."""
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import refshim
     g = zoo.ARCHS[arch](batch=1, size=size)
@@ -72,11 +78,80 @@ def cpu_baseline(arch, size, tmp, seed, budget_s=30.0):
 HBM_BYTES_PER_CONV_LAUNCH = {("yolov3", "f16", 8): int((40.24 + 19.06) * 2**20)}
 
 
+def conv_shape_mode(a):
+    """One convolution shape through msnh_hip_conv2d: every tile configuration timed with device events, or one forced
+    configuration launched --reps times (nothing else runs then: the form for a counter run).  Random inputs; results
+    are not checked here (the parity tests do that)."""
+    import ctypes
+
+    import torch
+
+    from msnhnet_amd import hipabi as abi
+    b, c, h, w, oc, k, stride = (int(v) for v in a.conv_shape.split(","))
+    pad = k // 2
+    oh, ow = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
+    dt = abi.F16 if a.conv_dtype == "f16" else abi.F32
+    tdt = torch.float16 if a.conv_dtype == "f16" else torch.float32
+    L = abi.lib()
+    abi.check(L.msnh_hip_init(0))
+    d = abi.ConvDesc(dt, dt, b, h, w, c, c, oc, oh, ow, oc, k, stride, pad, 1, 1, abi.ACT["leaky"], 0.1, 1 if a.residual else 0, oc,
+                     abi.ACT["none"], 0.1, 1.0, 1.0, abi.ALGO["igemm"], 0)
+    x = torch.randn(b, h, w, c, dtype=tdt, device="cuda")
+    wt = torch.randn(oc, k * k, c, dtype=tdt, device="cuda") * 0.05
+    y = torch.empty(b, oh, ow, oc, dtype=tdt, device="cuda")
+    res = torch.randn(b, oh, ow, oc, dtype=tdt, device="cuda") if a.residual else None
+    sc = torch.ones(oc, device="cuda")
+    sh = torch.zeros(oc, device="cuda")
+
+    def ptr(t):
+        return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+    def run():
+        abi.check(L.msnh_hip_conv2d(ctypes.byref(d), ptr(x), ptr(wt), ptr(sc), ptr(sh), ptr(res), ptr(y), None, 0, None))
+
+    torch.cuda.synchronize()
+    if a.tile > 0:
+        d.tile = a.tile
+        if not L.msnh_hip_conv2d_tile_supported(ctypes.byref(d), a.tile):
+            sys.exit(f"tile {a.tile} does not take this shape")
+        for _ in range(a.reps):
+            run()
+        abi.check(L.msnh_hip_stream_sync(None))
+        print(f"tile {a.tile}: {a.reps} launches of {a.conv_shape}")
+        return
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    abi.check(L.msnh_hip_event_create(ctypes.byref(e0)))
+    abi.check(L.msnh_hip_event_create(ctypes.byref(e1)))
+    flops = 2.0 * b * oc * oh * ow * c * k * k
+    for tile in range(1, L.msnh_hip_conv2d_tile_count() + 1):
+        d.tile = tile
+        if not L.msnh_hip_conv2d_tile_supported(ctypes.byref(d), tile):
+            continue
+        run()
+        run()
+        abi.check(L.msnh_hip_event_record(e0, None))
+        for _ in range(a.reps):
+            run()
+        abi.check(L.msnh_hip_event_record(e1, None))
+        abi.check(L.msnh_hip_event_sync(e1))
+        ms = ctypes.c_float()
+        abi.check(L.msnh_hip_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+        us = ms.value * 1e3 / a.reps
+        print(f"tile {tile:2d}: {us:8.2f} us  {flops / us * 1e-6:7.1f} TFLOP/s", flush=True)
+    L.msnh_hip_event_destroy(e0)
+    L.msnh_hip_event_destroy(e1)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--conv-shape", default=None, help="b,c,h,w,oc,k,stride: time this one convolution shape instead of a workload")
+    ap.add_argument("--tile", type=int, default=0, help="--conv-shape: launch only this tile configuration, --reps times, untimed")
+    ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--residual", action="store_true", help="--conv-shape: with a fused residual add")
+    ap.add_argument("--conv-dtype", default="f16", choices=["f16", "f32"])
     ap.add_argument("--workload", default="yolov3", choices=sorted(WORKLOADS))
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -97,6 +172,9 @@ def main():
     import torch          # device memory for the synthetic input only
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the hot path has no CPU fallback")
+    if a.conv_shape:
+        conv_shape_mode(a)
+        return
 
     dtype, batch, size = WORKLOADS[a.workload]
     tmp = tempfile.mkdtemp(prefix="msnh_bench_")
@@ -144,40 +222,60 @@ def main():
         else:
             net.enqueue(dev_in)
 
-    def run_steps(k):
+    def run_steps(k, stamps=None, host=None):
         """k forwards + k result fetches.  Detection keeps two batches in flight: while the host sorts and
-        suppresses the boxes of batch i the device already runs batch i+1."""
+        suppresses the boxes of batch i the device already runs batch i+1.  stamps collects the time at which each
+        step's result reached the host."""
         out = None
-        if host_x is not None:
+        tick = (lambda: stamps.append(time.perf_counter())) if stamps is not None else (lambda: None)
+        if host is not None:
             for _ in range(k):
-                out = net.run_yolo(host_x) if detect else net.run_classify(host_x)
+                out = net.run_yolo(host) if detect else net.run_classify(host)
+                tick()
         elif detect:
             feed()
             for _ in range(k - 1):
                 feed()
                 out = net.fetch_yolo()
+                tick()
             out = net.fetch_yolo()
+            tick()
         else:
             for _ in range(k):
                 feed()
                 out = net.fetch_classify()
+                tick()
         return out
 
     # set-up, not warm-up: the first forwards allocate the two copy-back slots (pinned host and device snapshots) and start the
     # host worker threads; they belong to building the network like the plan and the tile search
-    run_steps(4)
+    run_steps(4, host=host_x)
     if a.warmup > 0:
-        run_steps(a.warmup)
+        run_steps(a.warmup, host=host_x)
     net.sync()
     marker()
     torch.cuda.synchronize()
+    stamps = []
     t0 = time.perf_counter()
-    out = run_steps(a.steps)
+    out = run_steps(a.steps, stamps, host=host_x)
     net.sync()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     marker()
     ms_per_step = dt / a.steps * 1e3
+    per_step = np.diff(np.array([t0] + stamps)) * 1e3
+    # (pipelined detection: the first interval holds two forwards, every later one is a steady-state step)
+    ms_median = float(np.median(per_step[1:])) if len(per_step) > 1 else float(per_step[0])
+
+    # the reference's own calling convention beside the headline: one synchronous run*GPU(std::vector<float>) per batch, the float
+    # host image uploaded inside the call (PCIe inclusive; never `value`)
+    host_rate = None
+    if a.input == "device" and not a.copy_probe:
+        hx = zoo.seeded_input(batch, 3, size, size, a.seed + 1)
+        run_steps(2, host=hx)
+        th = time.perf_counter()
+        run_steps(5, host=hx)
+        host_rate = round(batch * 5 / (time.perf_counter() - th), 2)
 
     # device-only time of the captured forward (no host post-processing), for orientation
     all_ms, n_all, _ = net.profile_ops(-1, 10)
@@ -199,7 +297,8 @@ def main():
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
            "config": {"workload": f"{a.workload}-{size} {dtype} batch {batch}, seeded He-normal weights, U[0,1) input, "
                                   f"{'device-resident' if a.input == 'device' else a.input} input -> {'boxes' if detect else 'logits'} on host",
-                      "input": a.input, "seed": a.seed, "device_launches_per_step": n_all // 10, "device_ms_per_step_eager": round(gpu_only_ms, 4)},
+                      "input": a.input, "seed": a.seed, "ms_per_step_median": round(ms_median, 4), "device_launches_per_step": n_all // 10,
+                      "device_ms_per_step_eager": round(gpu_only_ms, 4), "host_f32_images_per_s": host_rate},
            "roofline": roofline}
     if detect:
         res["config"]["boxes_per_image"] = [int(len(b)) for b in out]
