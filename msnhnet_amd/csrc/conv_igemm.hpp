@@ -703,13 +703,14 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
 } // namespace msnh
 
 #include "conv_patch.hpp"
+#include "conv_patch8.hpp"
 
 namespace msnh {
 
 // Tile configurations (BM x BN output tile, KV 16-byte vectors of K per step, WM x WN wavefront grid).
 // Index 0 is "choose for me"; the others can be forced through msnh_conv_desc::tile, which is how the host
 // library's per-layer search picks the fastest one at load time.
-constexpr int kIgemmTiles = 42;
+constexpr int kIgemmTiles = 51;
 
 template <typename T, typename TOut>
 int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
@@ -770,6 +771,17 @@ int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
     case 41: return launchIgemm<T, TOut, 64, 256, 4, 1, 8, 3>(a, groups, st);
     // 128 channels x 384 pixels with twelve wavefronts: one round of tiles for 128-filter layers over many pixels
     case 42: return launchIgemm<T, TOut, 128, 384, 8, 2, 6, 2>(a, groups, st);
+    // 3x3 stride-1 pad-1 only: input patch resident in LDS with 128-byte rows (last three numbers: wavefront grid rows x columns,
+    // weight stages, patch slices per wavefront and tap step)
+    case 43: return launchPatch8<T, TOut, 128, 192, 4, 3, 3, 1>(a, groups, st);
+    case 44: return launchPatch8<T, TOut, 128, 192, 4, 2, 4, 1>(a, groups, st);
+    case 45: return launchPatch8<T, TOut, 128, 192, 2, 2, 4, 2>(a, groups, st);
+    case 46: return launchPatch8<T, TOut, 64, 384, 2, 6, 3, 1>(a, groups, st);
+    case 47: return launchPatch8<T, TOut, 64, 384, 2, 4, 4, 2>(a, groups, st);
+    case 48: return launchPatch8<T, TOut, 64, 256, 2, 4, 4, 1>(a, groups, st);
+    case 49: return launchPatch8<T, TOut, 128, 256, 4, 2, 3, 1>(a, groups, st);
+    case 50: return launchPatch8<T, TOut, 64, 192, 2, 2, 4, 2>(a, groups, st);
+    case 51: return launchPatch8<T, TOut, 128, 384, 2, 4, 3, 2>(a, groups, st);
     default: break;
     }
     setError("igemm: unknown tile %d", tile);

@@ -1,0 +1,335 @@
+// 3x3 stride-1 pad-1 convolution with the input patch resident in LDS, 128-byte rows, 4 / 8 / 12 wavefronts.
+//
+// Why: the 3x3 layers of the detectors at 76x76 ... 19x19 are bound by what a CU can draw out of the L2 (about 20 bytes per
+// clock and CU, measured), not by the matrix cores.  The generic implicit GEMM delivers (BM + BN) x 128 bytes to LDS per 64-deep
+// K step and multiplies BM x BN x 64 with it; per filter tap it fetches the same input pixels again, shifted by one.  Here the
+// run of BN + 2W + 2 input pixels that a tile of BN consecutive output pixels (flattened over the batch) can touch is delivered
+// ONCE per 64-channel chunk and the nine taps read their B fragments from it at a row offset of ky*W + kx; only the weight tile
+// (BM rows) streams per tap.  Bytes per MFMA fall by 2 - 2.8x against the generic kernel at the same tile, and the best shape
+// moves to few channels x many pixels (the weights are what is left to stream, and they are amortised over the pixels).
+// conv_patch.hpp is the same idea with 64-byte rows and four wavefronts; it loses to the generic kernel because its L2 requests
+// are 64 bytes long (the L2 serves requests, not bytes), its weight tile arrives one step ahead only, and a single wavefront per
+// SIMD has nothing to cover the barrier with.  This kernel differs in exactly those three points.
+//
+// LDS: NSA weight stages of BM x 128 B | patch of the current chunk | patch of the next chunk | 1 KiB of zeros.
+// Data movement as in conv_igemm.hpp: 16-byte-per-lane buffer loads straight into LDS, XOR-swizzled unpadded rows, explicit
+// vmcnt waits, one barrier per tap step.  The patch of chunk c+1 arrives in 1 KiB slices (8 pixels x 128 B, one wave
+// instruction each), PS per wavefront and tap step over the first 11 - NSA taps of chunk c; every tap step issues the same number
+// of loads per wavefront (slices that do not exist go, out of range and therefore as zeros, into the zero area), so the count
+// of loads in flight at each barrier is a compile-time constant.
+#pragma once
+#include "conv_igemm.hpp"
+
+namespace msnh {
+
+// DBG (timing experiments only, results are then meaningless; 0 in every instantiation the library ships): bit 0 leaves out the
+// loads of the main loop, bit 1 its LDS fragment reads, bit 2 its barrier, bit 3 its MFMAs.
+template <typename T, typename TOut, int BM, int BN, int WM, int WN, int NSA, int PS, int DBG = 0>
+__global__ __launch_bounds__(64 * WM * WN) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, WM * WN / 4)))
+void convPatch8Kernel(IgemmArgs a)
+{
+    typedef typename Frag<T>::V V;
+    constexpr int VEC   = Frag<T>::VEC;
+    constexpr int KV    = 8;
+    constexpr int BK    = KV * VEC;
+    constexpr int NW    = WM * WN;
+    constexpr int NT    = 64 * NW;
+    constexpr int RPP   = NT / KV;                    // weight rows per load pass of the workgroup
+    constexpr int BML   = (BM + RPP - 1) / RPP * RPP; // weight rows held in LDS (whole passes; the surplus rows load nothing)
+    constexpr int AL    = BML / RPP;                  // weight loads per thread per tap step
+    constexpr int NL    = AL + PS;                    // loads per thread per tap step
+    constexpr int TM    = BM / WM;
+    constexpr int TN    = BN / WN;
+    constexpr int MB    = TM / 32;
+    constexpr int NB    = TN / 32;
+    constexpr int S     = KV / 2;                     // MFMA k-blocks per tap step
+    constexpr unsigned ES = sizeof(T);
+    constexpr int ROWB  = KV * 16;
+    constexpr unsigned A_STAGE = BML * ROWB;
+    constexpr int PSTEPS = 11 - NSA;                  // tap steps of a chunk that bring in slices of the next chunk's patch
+    static_assert(TM % 32 == 0 && TN % 32 == 0 && (NW == 4 || NW == 8 || NW == 12), "tile shape");
+    static_assert(NSA >= 3 && NSA <= 5, "weight stages");
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smemRaw[];
+    const unsigned ldsBase = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char *)smemRaw));
+    const int nSlices = a.patchRows;                  // 1 KiB slices per patch stage (host: ceil((BN + 2W + 2) / 8))
+    const unsigned patchBytes = static_cast<unsigned>(nSlices) * 1024u;
+    const unsigned patchOff0 = NSA * A_STAGE;
+    const unsigned patchStages = a.cChunks > 1 ? 2u : 1u;     // a single channel chunk never loads a second patch
+    const unsigned dumpOff = patchOff0 + patchStages * patchBytes;
+
+    const int tid  = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm   = wave / WN;
+    const int wn   = wave % WN;
+    const int nTilesP = (a.P + BN - 1) / BN;
+    const int total   = a.mTiles * nTilesP;
+    const int perXcd  = (total + 7) / 8;
+    const int logical = (blockIdx.x % 8) * perXcd + blockIdx.x / 8;
+    if (logical >= total) return;
+    const int m0 = (logical % a.mTiles) * BM;
+    const int p0 = (logical / a.mTiles) * BN;
+
+    const i32x4 rx = makeRsrcWords(a.x, a.xBytes);
+    const i32x4 rw = makeRsrcWords(a.w, a.wBytes);
+
+    float chScale, chShift;
+    loadChannelAffine(a, 0, m0, tid, BM, chScale, chShift);
+
+    if (tid < 64) *reinterpret_cast<f32x4 *>(smemRaw + dumpOff + tid * 16) = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int W = a.W, H = a.H;
+
+    // ---- weight tile: thread tid owns chunk position tid % 8 of row tid / 8 (+ RPP rows per pass); row r keeps logical chunk c
+    // at position c ^ ((r / 2) % 8) ------------------------------------------------------------------------------------------
+    const int ldRow = tid / KV;
+    const int ldVec = (tid % KV) ^ ((ldRow / 2) % KV);
+    unsigned aOff[AL];
+#pragma unroll
+    for (int i = 0; i < AL; ++i)
+    {
+        const int m = m0 + ldRow + i * RPP;
+        aOff[i] = (m < a.coutG && ldRow + i * RPP < BM) ? (static_cast<unsigned>(m) * 9u * a.cinG + ldVec * VEC) * ES : kOobOffset;
+    }
+    // ---- patch: slice s holds patch rows 8s .. 8s+7 = input pixels q0 + 8s ..; lane l of the slice's load owns chunk position
+    // l % 8 of row 8s + l / 8, whose swizzle is ((8s + l/8) / 2) % 8 = (l / 16) ^ 4*(s & 1).  A wavefront's slices are
+    // wave, wave + NW, ...: NW is even, so the parity of s is the wavefront's and one base offset serves all its slices.
+    // Pixels in front of the tensor give a negative offset, which as unsigned is out of range like the pixels behind it.
+    const int q0 = p0 - W - 1;
+    const int pRow = lane / KV;
+    const int pVec = (lane % KV) ^ (lane / 16) ^ (4 * (wave & 1));
+    const unsigned pBase = static_cast<unsigned>((static_cast<long long>(q0 + pRow) * a.inLd + pVec * VEC) * static_cast<long long>(ES));
+    const unsigned sliceStride = 8u * static_cast<unsigned>(a.inLd) * ES;
+    const unsigned waveDump = ldsBase + dumpOff;
+    const bool pCutAlways = false;
+
+    auto issuePatch = [&](int i, int chunk, unsigned stOff) {
+        const int s = wave + NW * i;
+        const bool real = s < nSlices && chunk < a.cChunks;
+        const bool cut = a.ragged && (chunk * BK + pVec * VEC >= a.cinG);
+        const unsigned voff = (real && !cut && !pCutAlways) ? pBase + static_cast<unsigned>(s) * sliceStride : kOobOffset;
+        dmaLoad16(rx, voff, static_cast<unsigned>(chunk * BK) * ES, real ? ldsBase + stOff + static_cast<unsigned>(s) * 1024u : waveDump);
+    };
+    const unsigned waveLds = ldsBase + wave * 1024;
+    auto issueA = [&](auto lTag, unsigned sA, bool cut, unsigned stageOff) {
+        constexpr int l = decltype(lTag)::value;
+        dmaLoad16(rw, cut ? kOobOffset : aOff[l], sA, waveLds + stageOff + l * RPP * ROWB);
+    };
+
+    // ---- fragments ----------------------------------------------------------------------------------------------------------
+    const int fragRow = lane & 31;
+    const int fragSw  = (fragRow / 2) % KV;
+    unsigned aAddr[S];
+#pragma unroll
+    for (int kb = 0; kb < S; ++kb) aAddr[kb] = wm * TM * ROWB + fragRow * ROWB + (((2 * kb + (lane >> 5)) ^ fragSw) * 16);
+    // per 32-pixel block j of the wave tile: which of the nine taps lie inside the image for this lane's pixel
+    unsigned tapOk[NB];
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+    {
+        const int p = p0 + wn * TN + j * 32 + fragRow;
+        unsigned m = 0;
+        if (p < a.P)
+        {
+            const int x = p % W;
+            const int y = (p / W) % H;
+#pragma unroll
+            for (int t = 0; t < 9; ++t)
+            {
+                const int yy = y + t / 3 - 1, xx = x + t % 3 - 1;
+                if (yy >= 0 && yy < H && xx >= 0 && xx < W) m |= 1u << t;
+            }
+        }
+        tapOk[j] = m;
+    }
+    const unsigned bRow0 = wn * TN + fragRow;         // patch row of this lane's pixel for tap (0,0), block 0
+    const unsigned zeroAddr = dumpOff + lane * 16;
+
+    V fa[2][MB], fb[2][NB];
+    auto readA = [&](unsigned stageOff, auto kbTag) {
+        constexpr int kb = decltype(kbTag)::value;
+        const unsigned char *ap = smemRaw + (aAddr[kb] + stageOff);
+#pragma unroll
+        for (int i = 0; i < MB; ++i) fa[kb % 2][i] = *reinterpret_cast<const V *>(ap + i * 32 * ROWB);
+    };
+    // B fragments of tap `tap` (row offset tapRow = ky*W + kx) from the patch stage at pOff; rows 32 apart share the swizzle
+    auto readB = [&](unsigned pOff, int tap, unsigned tapRow, auto kbTag) {
+        constexpr int kb = decltype(kbTag)::value;
+        const unsigned row = bRow0 + tapRow;
+        const unsigned sw = (row / 2) % KV;
+        const unsigned addr = pOff + row * ROWB + (((2 * kb + (lane >> 5)) ^ sw) * 16);
+        const unsigned bit = 1u << tap;
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+        {
+            const unsigned aj = (tapOk[j] & bit) ? addr + j * 32 * ROWB : zeroAddr;
+            fb[kb % 2][j] = *reinterpret_cast<const V *>(smemRaw + aj);
+        }
+    };
+
+    f32x16 acc[MB][NB];
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    constexpr int PER = MB * NB;                      // MFMAs per k-block
+    constexpr int TOT = PER * S;
+    constexpr int LSPAN = TOT - PER;                  // the loads of a step follow its MFMAs 0 .. LSPAN-1, ahead of the barrier
+    // At the barrier of step `it` the weight tile of step it+1 must have landed: it was issued during step it+2-NSA, and the
+    // loads of the NSA-2 steps since then may still be in flight.  Patch slices are issued during taps 0 .. PSTEPS-1 = 10-NSA and
+    // are needed from the barrier of tap 8 on, NSA-2 steps later: covered by the same count.
+    constexpr int INFLIGHT = (NSA - 2) * NL;
+
+    // ---- prologue: whole patch of chunk 0, weight tiles of steps 0 .. NSA-2 -----------------------------------------------------
+    for (int i = 0; wave + NW * i < nSlices; ++i) issuePatch(i, 0, patchOff0);
+    int tapL = -1, chunkL = 0;                        // (tap, chunk) of the step whose weight tile was issued last
+    auto advanceA = [&](unsigned &sA, bool &cutA, int stepIndex) {
+        if (++tapL == 9) { tapL = 0; ++chunkL; }
+        sA = (static_cast<unsigned>(tapL) * a.cinG + chunkL * BK) * ES;
+        cutA = stepIndex >= a.nIter || (a.ragged && (chunkL * BK + ldVec * VEC >= a.cinG));
+    };
+    staticFor<0, NSA - 1>([&](auto stTag) {
+        constexpr int st = decltype(stTag)::value;
+        unsigned sA; bool cutA;
+        advanceA(sA, cutA, st);
+        staticFor<0, AL>([&](auto lTag) { issueA(lTag, sA, cutA, st * A_STAGE); });
+    });
+    dmaWait<0>();
+    __syncthreads();
+    readA(0, std::integral_constant<int, 0>());
+    readB(patchOff0, 0, 0u, std::integral_constant<int, 0>());
+
+    unsigned curA = 0, nxtA = A_STAGE, nnA = (NSA - 1) * A_STAGE;
+    unsigned curP = patchOff0, othP = patchStages > 1 ? patchOff0 + patchBytes : patchOff0;
+    int it = 0;
+    for (int chunk = 0; chunk < a.cChunks; ++chunk)
+    {
+        staticFor<0, 9>([&](auto tapTag) {
+            constexpr int tap = decltype(tapTag)::value;
+            constexpr int tapN = tap == 8 ? 0 : tap + 1;
+            const unsigned tapRow = static_cast<unsigned>((tap / 3) * W + tap % 3);
+            const unsigned tapRowN = static_cast<unsigned>((tapN / 3) * W + tapN % 3);
+            const unsigned nextP = tap == 8 ? othP : curP;
+            unsigned sA; bool cutA;
+            advanceA(sA, cutA, it + NSA - 1);         // the weight tile of step it + NSA - 1
+
+            if constexpr (!(DBG & 2))
+            {
+                readA(curA, std::integral_constant<int, 1>());
+                readB(curP, tap, tapRow, std::integral_constant<int, 1>());
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            staticFor<0, TOT>([&](auto gTag) {
+                constexpr int gi = decltype(gTag)::value;
+                constexpr int ks = gi / PER;
+                if constexpr (gi % PER == 0 && ks >= 1)
+                {
+                    if constexpr (ks < S - 1)
+                    {
+                        if constexpr (!(DBG & 2))
+                        {
+                            readA(curA, std::integral_constant<int, ks + 1>());
+                            readB(curP, tap, tapRow, std::integral_constant<int, ks + 1>());
+                        }
+                    }
+                    else
+                    {
+                        if constexpr (!(DBG & 1)) dmaWait<INFLIGHT>();
+                        if constexpr (!(DBG & 4)) __syncthreads();
+                        if constexpr (!(DBG & 2))
+                        {
+                            readA(nxtA, std::integral_constant<int, 0>());
+                            readB(nextP, tapN, tapRowN, std::integral_constant<int, 0>());
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if constexpr (!(DBG & 8)) mfmaBlock(fa[ks % 2][(gi % PER) / NB], fb[ks % 2][(gi % PER) % NB], acc[(gi % PER) / NB][(gi % PER) % NB]);
+                else asm volatile("" : "+v"(fa[ks % 2][(gi % PER) / NB]), "+v"(fb[ks % 2][(gi % PER) % NB]));
+                if constexpr (gi < LSPAN && !(DBG & 1))
+                {
+                    // loads l with l * LSPAN / NL == gi: patch slices first, then the weight rows
+                    constexpr int first = (gi * NL + LSPAN - 1) / LSPAN;
+                    constexpr int last  = ((gi + 1) * NL + LSPAN - 1) / LSPAN;
+                    staticFor<first, last>([&](auto lTag) {
+                        constexpr int l = decltype(lTag)::value;
+                        if constexpr (l < PS)
+                            issuePatch(tap < PSTEPS ? tap * PS + l : (1 << 20), chunk + 1, othP);
+                        else
+                            issueA(std::integral_constant<int, l - PS>(), sA, cutA, nnA);
+                    });
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            nnA = curA;
+            curA = nxtA;
+            nxtA = nxtA + A_STAGE == NSA * A_STAGE ? 0u : nxtA + A_STAGE;
+            ++it;
+        });
+        const unsigned tp = curP;
+        curP = othP;
+        othP = tp;
+    }
+    dmaWait<0>();
+    __syncthreads();
+
+    igemmEpilogue<T, TOut, BM, BN, TM, TN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, wave, lane, 0);
+}
+
+// Host-side check shared by launch and tile enumeration.
+template <typename T, int BM, int BN, int WM, int WN, int NSA, int PS>
+inline bool patch8Fits(const IgemmArgs &a, size_t *smemOut, int *slicesOut)
+{
+    constexpr int NW = WM * WN;
+    constexpr int RPP = 64 * NW / 8;
+    constexpr int BML = (BM + RPP - 1) / RPP * RPP;
+    constexpr int BK = 8 * Frag<T>::VEC;
+    const int R = BN + 2 * a.W + 2;
+    const int slices = (R + 7) / 8;
+    const int stages = a.cinG > BK ? 2 : 1;
+    const size_t loop = static_cast<size_t>(NSA) * BML * 128 + static_cast<size_t>(stages) * slices * 1024 + 1024;
+    const size_t epi = igemmEpilogueLds<BM, BM / WM, NW>();
+    const size_t smem = loop > epi ? loop : epi;
+    if (smemOut) *smemOut = smem;
+    if (slicesOut) *slicesOut = slices;
+    // the first 11 - NSA taps of a chunk bring in the next patch: (11 - NSA) * PS slices per wavefront
+    return a.patchOk && a.buffersOk && smem <= 160 * 1024 && (stages == 1 || slices <= (11 - NSA) * NW * PS);
+}
+
+template <typename T, typename TOut, int BM, int BN, int WM, int WN, int NSA, int PS, int DBG = 0>
+inline int launchPatch8(IgemmArgs &a, int groups, hipStream_t st)
+{
+    constexpr int VEC = Frag<T>::VEC;
+    constexpr int BK  = 8 * VEC;
+    size_t smem = 0;
+    int slices = 0;
+    if (groups != 1 || a.splitMax > 1 || !patch8Fits<T, BM, BN, WM, WN, NSA, PS>(a, &smem, &slices))
+    {
+        setError("conv2d: this tile needs a 3x3 stride-1 pad-1 ungrouped convolution whose input patch fits in LDS");
+        return 3;
+    }
+    if (a.dryRun) return 0;
+    a.patchRows = slices;
+    a.cChunks = (a.cinG + BK - 1) / BK;
+    a.nIter   = 9 * a.cChunks;
+    a.ragged  = (a.cinG % BK) != 0;
+    a.mTiles  = (a.coutG + BM - 1) / BM;
+    a.splitK  = 1;
+    const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
+    dim3 grid((tiles + 7) / 8 * 8, 1, 1);
+    auto kern = convPatch8Kernel<T, TOut, BM, BN, WM, WN, NSA, PS, DBG>;
+    if (smem > 48 * 1024)
+    {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
+        if (e != hipSuccess) { setError("hipFuncSetAttribute: %s", hipGetErrorString(e)); return 1; }
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(64 * WM * WN), smem, st, a);
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+} // namespace msnh
