@@ -296,6 +296,17 @@ size_t msnh_hip_yolo_nms_workspace_bytes(int batch, int classes, int cand_cap);
 int msnh_hip_yolo_nms(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept,
                       int kept_cap, int *kept_cnt, void *workspace, size_t workspace_bytes, msnh_stream_t s);
 
+/* msnh_hip_yolo_nms for callers that cannot allocate device memory (code under graph capture, tight serving loops, harnesses that
+ * forbid it).  No counterpart in the reference.  Same arguments, results and flags as msnh_hip_yolo_nms called with a workspace, but
+ * the workspace is a device array inside the library: msnh_hip_yolo_nms_static_max_bytes() = 4 MiB per GPU the library runs on, held
+ * until the process ends.  A geometry whose msnh_hip_yolo_nms_workspace_bytes() exceeds that is refused with an error (YOLOv3 / YOLOv4
+ * at 608 x 608 with 80 classes, 22743 candidate slots per image, fit up to batch 45).  The call itself allocates and frees nothing; its one-time set-up per device runs
+ * in msnh_hip_init (or in the first call on a device that msnh_hip_init did not select).  Every call on a GPU shares that GPU's
+ * array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream follow each other safely. */
+size_t msnh_hip_yolo_nms_static_max_bytes(void);
+int msnh_hip_yolo_nms_static(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept,
+                             int kept_cap, int *kept_cnt, msnh_stream_t s);
+
 /* max |x| over the finite elements of an NHWC tensor, combined into *result with an atomic max
  * (caller zeroes *result).  Used once at load time to calibrate the power-of-two activation scales of the
  * float16 plan; no counterpart in the reference. */

@@ -13,6 +13,7 @@ namespace msnh {
 // ---- error reporting ------------------------------------------------------------------------------
 void setError(const char *fmt, ...);
 hipStream_t resolveStream(msnh_stream_t s);
+int yoloNmsSetupDevice();            // per-device set-up of msnh_hip_yolo_nms_static (csrc/yolo.hip), on the current device
 
 #define MSNH_HIP_CHECK(expr)                                                                      \
     do {                                                                                          \

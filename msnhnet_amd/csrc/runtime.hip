@@ -50,7 +50,7 @@ int msnh_hip_init(int device)
         MSNH_HIP_CHECK(hipStreamCreateWithFlags(&g_defaultStream, hipStreamNonBlocking));
         g_device = device;
     }
-    return 0;
+    return yoloNmsSetupDevice();
 }
 
 int msnh_hip_device_count(int *count)

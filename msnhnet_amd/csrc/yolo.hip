@@ -2,6 +2,7 @@
 // the objectness threshold.  The NHWC head tensor already stores the (5+classes) values of one anchor of
 // one pixel contiguously, so both the read and the write of a wavefront are contiguous runs.
 #include "common.hpp"
+#include <mutex>
 
 namespace msnh {
 
@@ -585,27 +586,92 @@ extern "C" size_t msnh_hip_yolo_nms_workspace_bytes(int batch, int classes, int 
     return sizeof(int) * (static_cast<size_t>(batch) * classes + static_cast<size_t>(batch) * cand_cap + static_cast<size_t>(batch));
 }
 
-extern "C" int msnh_hip_yolo_nms(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept,
-                                 int kept_cap, int *kept_cnt, void *workspace, size_t workspace_bytes, msnh_stream_t s)
+// The two launches of the device NMS; ws = [batch*classes] class sizes | [batch*cand_cap] sorted rows | [batch] cursors, or NULL
+// (small classes only).
+static int launchYoloNms(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept, int kept_cap,
+                         int *kept_cnt, int *ws, bool bigKernelReady, hipStream_t st)
 {
-    MSNH_REQUIRE(batch > 0 && batch <= 65535 && classes > 0 && cand_cap > 0 && cand_cap <= (1 << 24) && kept_cap > 0, "yolo_nms: bad geometry");
-    MSNH_REQUIRE(rows && cand_cnt && kept && kept_cnt, "yolo_nms: NULL pointer");
-    MSNH_REQUIRE(reinterpret_cast<uintptr_t>(rows) % 16 == 0 && reinterpret_cast<uintptr_t>(kept) % 16 == 0, "yolo_nms: rows and kept must be 16-byte aligned");
-    MSNH_REQUIRE(workspace == nullptr || (workspace_bytes >= msnh_hip_yolo_nms_workspace_bytes(batch, classes, cand_cap) && reinterpret_cast<uintptr_t>(workspace) % 4 == 0),
-                 "yolo_nms: workspace too small (msnh_hip_yolo_nms_workspace_bytes)");
-    hipStream_t st = resolveStream(s);
-    int *bigCnt = static_cast<int *>(workspace);
+    int *bigCnt = ws;
     int *wsSorted = bigCnt ? bigCnt + static_cast<size_t>(batch) * classes : nullptr;
     int *wsUsed = bigCnt ? wsSorted + static_cast<size_t>(batch) * cand_cap : nullptr;
     hipLaunchKernelGGL(yoloNmsKernel, dim3(classes, batch), dim3(256), 0, st, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, bigCnt, wsUsed);
     MSNH_LAUNCH_CHECK();
-    if (workspace == nullptr) return 0;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsBigKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_BIG_LDS);
-    if (e != hipSuccess) { setError("hipFuncSetAttribute: %s", hipGetErrorString(e)); return 1; }
+    if (ws == nullptr) return 0;
+    if (!bigKernelReady)
+    {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsBigKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_BIG_LDS);
+        if (e != hipSuccess) { setError("hipFuncSetAttribute: %s", hipGetErrorString(e)); return 1; }
+    }
     hipLaunchKernelGGL(yoloNmsBigKernel, dim3(classes, batch), dim3(256), NMS_BIG_LDS, st, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt,
                        bigCnt, wsSorted, wsUsed);
     MSNH_LAUNCH_CHECK();
     return 0;
+}
+
+static int checkYoloNmsArgs(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, const float *kept, int kept_cap, const int *kept_cnt)
+{
+    MSNH_REQUIRE(batch > 0 && batch <= 65535 && classes > 0 && cand_cap > 0 && cand_cap <= (1 << 24) && kept_cap > 0, "yolo_nms: bad geometry");
+    MSNH_REQUIRE(rows && cand_cnt && kept && kept_cnt, "yolo_nms: NULL pointer");
+    MSNH_REQUIRE(reinterpret_cast<uintptr_t>(rows) % 16 == 0 && reinterpret_cast<uintptr_t>(kept) % 16 == 0, "yolo_nms: rows and kept must be 16-byte aligned");
+    return 0;
+}
+
+extern "C" int msnh_hip_yolo_nms(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept,
+                                 int kept_cap, int *kept_cnt, void *workspace, size_t workspace_bytes, msnh_stream_t s)
+{
+    if (int rc = checkYoloNmsArgs(batch, classes, rows, cand_cap, cand_cnt, kept, kept_cap, kept_cnt)) return rc;
+    MSNH_REQUIRE(workspace == nullptr || (workspace_bytes >= msnh_hip_yolo_nms_workspace_bytes(batch, classes, cand_cap) && reinterpret_cast<uintptr_t>(workspace) % 4 == 0),
+                 "yolo_nms: workspace too small (msnh_hip_yolo_nms_workspace_bytes)");
+    return launchYoloNms(batch, classes, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, static_cast<int *>(workspace), false, resolveStream(s));
+}
+
+// ---- the same call for callers that cannot allocate ------------------------------------------------------------------------------
+// The workspace lives in a device array of this module: 4 MiB per GPU the library runs on, held until the process ends.  The
+// array's name is only a host-side stand-in; its device address is asked for once per device and kept.
+namespace {
+constexpr size_t kNmsScratchInts = static_cast<size_t>(1) << 20;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) int scratch[kNmsScratchInts];
+int *g_scratchPtr[kMaxDevices] = {};
+std::mutex g_scratchMutex;
+}
+
+namespace msnh {
+// One-time set-up on the current device: the scratch array's address there, and the large-class kernel's LDS limit.
+int yoloNmsSetupDevice()
+{
+    int dev = -1;
+    MSNH_HIP_CHECK(hipGetDevice(&dev));
+    MSNH_REQUIRE(dev >= 0 && dev < kMaxDevices, "yolo_nms_static: device index %d is beyond the %d this library keeps state for", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratchMutex);
+    if (g_scratchPtr[dev] != nullptr) return 0;
+    void *p = nullptr;
+    MSNH_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    MSNH_REQUIRE(p != nullptr, "yolo_nms_static: the scratch array has no address on device %d", dev);
+    MSNH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsBigKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_BIG_LDS));
+    g_scratchPtr[dev] = static_cast<int *>(p);
+    return 0;
+}
+}
+
+extern "C" size_t msnh_hip_yolo_nms_static_max_bytes(void) { return kNmsScratchInts * sizeof(int); }
+
+extern "C" int msnh_hip_yolo_nms_static(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept,
+                                        int kept_cap, int *kept_cnt, msnh_stream_t s)
+{
+    if (int rc = checkYoloNmsArgs(batch, classes, rows, cand_cap, cand_cnt, kept, kept_cap, kept_cnt)) return rc;
+    const size_t need = msnh_hip_yolo_nms_workspace_bytes(batch, classes, cand_cap);
+    MSNH_REQUIRE(need <= kNmsScratchInts * sizeof(int),
+                 "yolo_nms_static: batch %d x (%d classes + %d candidate slots + 1) needs %zu bytes of workspace, the built-in one holds %zu; "
+                 "use msnh_hip_yolo_nms with a workspace of the caller", batch, classes, cand_cap, need, kNmsScratchInts * sizeof(int));
+    int dev = -1;
+    MSNH_HIP_CHECK(hipGetDevice(&dev));
+    MSNH_REQUIRE(dev >= 0 && dev < kMaxDevices, "yolo_nms_static: device index %d is beyond the %d this library keeps state for", dev, kMaxDevices);
+    if (g_scratchPtr[dev] == nullptr)
+        if (int rc = yoloNmsSetupDevice()) return rc;        // (msnh_hip_init does this for the device it selects)
+    // Nothing in the workspace has to start at zero: the first kernel writes every class size and resets every image's cursor,
+    // and the sorted rows are written before they are read.
+    return launchYoloNms(batch, classes, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, g_scratchPtr[dev], true, resolveStream(s));
 }
 
 extern "C" int msnh_hip_absmax(int dtype, long long pixels, int c, const void *x, int x_ld, float *result, msnh_stream_t s)
