@@ -211,7 +211,6 @@ def main():
     host_x = zoo.seeded_input(batch, 3, size, size, a.seed + 1) if a.input == "host_f32" else None
     host_u8 = None
     if a.input == "host_u8":
-        import numpy as np
         host_u8 = np.random.default_rng(a.seed + 2).integers(0, 256, (batch, size, size, 3), dtype=np.uint8)
 
     def feed():

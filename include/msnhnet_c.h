@@ -100,6 +100,11 @@ int msnhnet_num_layers(msnhnet_t net);
 int msnhnet_layer_info(msnhnet_t net, int layer, long long *info, char *name, int name_cap);
 long long msnhnet_layer_detail(msnhnet_t net, char *dst, long long cap);      /* returns the full length */
 long long msnhnet_plan_detail(msnhnet_t net, char *dst, long long cap);
+/* The parts of the weights file this graph expects, in `.msnhbin` order (NetBuilder::loadWeightsFromMsnhBin,
+ * src/net/MsnhNetBuilder.cpp:624-663, and each layer's loadAllWeigths).  parts receives up to cap triples { what, count, fan_in }:
+ * what = 0 convolution / deconvolution kernel, 1 batch-norm scale, 2 batch-norm shift, 3 running mean, 4 running variance,
+ * 5 bias, 6 connected weights.  Returns the number of parts (call with parts == NULL first).  Works on a built graph without weights. */
+long long msnhnet_weight_layout(msnhnet_t net, long long *parts, long long cap);
 double msnhnet_conv_flops(msnhnet_t net);
 /* NetBuilder::runClassify / runYolo (CPU): always fail with "Gpu mode , can not run with cpu". */
 int msnhnet_run_classify(msnhnet_t net, const float *img, long long n, float *out, long long cap, long long *n_out);

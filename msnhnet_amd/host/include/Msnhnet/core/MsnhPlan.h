@@ -122,7 +122,7 @@ public:
     void tuneConvs(msnh_stream_t s, const std::string &cacheFile = std::string());
     void run(size_t opBegin, size_t opEnd, msnh_stream_t s);
     void runAll(msnh_stream_t s) { run(0, ops.size(), s); }
-    void measureAmax(msnh_stream_t s);      // after an eager run: absmax of every live NHWC tensor
+    void runCalibration(msnh_stream_t s);   // one eager run; absmax of every NHWC tensor taken right behind the launch that writes it
 
     int   root(int t) const;
     int   chanOffsetInRoot(int t) const;

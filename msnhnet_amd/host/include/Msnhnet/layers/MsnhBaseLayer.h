@@ -53,6 +53,10 @@ public:
     // Constants of the ops this layer owns (conv / batchnorm / connected override these).
     virtual const std::vector<float> &kernelWeights() const;
     virtual void foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const;
+    // The parts this layer's weights consist of, in `.msnhbin` order.  Each part is three numbers: what it is (0 convolution /
+    // deconvolution kernel, 1 batch-norm scale, 2 batch-norm shift, 3 running mean, 4 running variance, 5 bias, 6 connected
+    // weights), how many floats, and the fan-in of a kernel or connected part.  Lets a caller synthesise a weights file for any graph.
+    virtual void weightLayout(std::vector<long long> &parts) const;
 
     LayerType type() const { return _type; }
     ActivationType activation() const { return _activation; }

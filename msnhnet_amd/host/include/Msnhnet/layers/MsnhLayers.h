@@ -26,6 +26,7 @@ public:
     int convOutHeight() const;
     int convOutWidth() const;
     void loadAllWeigths(std::vector<float> &weights) override;
+    void weightLayout(std::vector<long long> &parts) const override;
     int lower(Plan &plan, int in, int layerIndex) override;
     const std::vector<float> &kernelWeights() const override { return _weights; }
     void foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const override;
@@ -63,6 +64,7 @@ public:
     BatchNormLayer(const int &batch, const int &width, const int &height, const int &channel, const ActivationType &activation,
                    const float &eps, const std::vector<float> &actParams);
     void loadAllWeigths(std::vector<float> &weights) override;
+    void weightLayout(std::vector<long long> &parts) const override;
     int lower(Plan &plan, int in, int layerIndex) override;
     void foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const override;
 
@@ -107,6 +109,7 @@ public:
     ConnectedLayer(const int &batch, const int &steps, const int &inputNum, const int &outputNum, const ActivationType &activation,
                    const std::vector<float> &actParams, const int &batchNorm, const float &bnEps, const int &useBias);
     void loadAllWeigths(std::vector<float> &weights) override;
+    void weightLayout(std::vector<long long> &parts) const override;
     int lower(Plan &plan, int in, int layerIndex) override;
     const std::vector<float> &kernelWeights() const override { return _weights; }
     void foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const override;
@@ -145,6 +148,7 @@ public:
     int deConvOutHeight() const { return (_height - 1) * _strideY - 2 * _paddingY + _kSizeY; }
     int deConvOutWidth() const { return (_width - 1) * _strideX - 2 * _paddingX + _kSizeX; }
     void loadAllWeigths(std::vector<float> &weights) override;
+    void weightLayout(std::vector<long long> &parts) const override;
     int lower(Plan &plan, int in, int layerIndex) override;
     void foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const override;      // the bias, for the gather launch
 
@@ -258,6 +262,7 @@ class MsnhNet_API BlockLayer : public BaseLayer
 public:
     ~BlockLayer() override;
     void loadAllWeigths(std::vector<float> &weights) override;
+    void weightLayout(std::vector<long long> &parts) const override;
 
 protected:
     std::vector<BaseLayer *> buildChain(NetBuildParams &params, std::vector<BaseParams *> &nodes, const char *blockName, bool allowEmpty);

@@ -311,6 +311,18 @@ long long msnhnet_time_detail(msnhnet_t net, char *dst, long long cap)
     return n;
 }
 
+long long msnhnet_weight_layout(msnhnet_t net, long long *parts, long long cap)
+{
+    long long n = -1;
+    guarded([&] {
+        std::vector<long long> all;
+        for (const BaseLayer *l : nb(net).getNet()->layers) l->weightLayout(all);
+        n = static_cast<long long>(all.size() / 3);
+        if (parts && cap > 0) std::memcpy(parts, all.data(), sizeof(long long) * static_cast<size_t>(std::min<long long>(cap, n) * 3));
+    });
+    return n;
+}
+
 double msnhnet_conv_flops(msnhnet_t net)
 {
     double f = 0;

@@ -52,6 +52,14 @@ void BaseLayer::loadAllWeigths(std::vector<float> &weights)
 
 void BaseLayer::saveAllWeights(const int &, const int &, const int &) {}
 
+void BaseLayer::weightLayout(std::vector<long long> &) const {}
+
+static void addPart(std::vector<long long> &parts, int what, long long count, long long fanIn = 0)
+{
+    if (count <= 0) return;
+    parts.push_back(what); parts.push_back(count); parts.push_back(fanIn);
+}
+
 int BaseLayer::lower(Plan &, int, int) { MSNH_THROW(_layerName + ": lowering is not implemented"); }
 
 const std::vector<float> &BaseLayer::kernelWeights() const
@@ -188,6 +196,16 @@ void ConvolutionalLayer::loadAllWeigths(std::vector<float> &weights)
     _weightsLoaded = true;
 }
 
+void ConvolutionalLayer::weightLayout(std::vector<long long> &parts) const
+{
+    addPart(parts, 0, _nWeights, static_cast<long long>(_channel / _groups) * _kSizeX * _kSizeY);
+    if (_batchNorm)
+    {
+        addPart(parts, 1, _nScales); addPart(parts, 2, _nBiases); addPart(parts, 3, _nRollMean); addPart(parts, 4, _nRollVariance);
+    }
+    else if (_useBias) addPart(parts, 5, _nBiases, static_cast<long long>(_channel / _groups) * _kSizeX * _kSizeY);
+}
+
 void ConvolutionalLayer::foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const
 {
     scale.clear();
@@ -255,6 +273,11 @@ void BatchNormLayer::loadAllWeigths(std::vector<float> &weights)
     _rollMean.assign(p + 2 * c, p + 3 * c);
     _rollVariance.assign(p + 3 * c, p + 4 * c);
     _weightsLoaded = true;
+}
+
+void BatchNormLayer::weightLayout(std::vector<long long> &parts) const
+{
+    for (int what = 1; what <= 4; ++what) addPart(parts, what, _channel);
 }
 
 void BatchNormLayer::foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const
@@ -381,6 +404,12 @@ void ConnectedLayer::loadAllWeigths(std::vector<float> &weights)
     _weightsLoaded = true;
 }
 
+void ConnectedLayer::weightLayout(std::vector<long long> &parts) const
+{
+    addPart(parts, 6, _nWeights, _inputNum);
+    if (_useBias) addPart(parts, 5, static_cast<long long>(_numWeights) - _nWeights, _inputNum);
+}
+
 void ConnectedLayer::foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const
 {
     scale.clear();
@@ -391,8 +420,8 @@ int ConnectedLayer::lower(Plan &plan, int in, int layerIndex)
 {
     const PlanTensor ti = plan.tensors[static_cast<size_t>(in)];
     if (ti.layout == PlanTensor::NCHW_INPUT) MSNH_THROW("connect can not be the first layer of a network");
-    if (ti.layout == PlanTensor::NHWC && ti.h * ti.w != 1)
-        MSNH_THROW("connect: the input must be 1x1 spatially (put a pooling layer before it)");
+    // (an image tensor with more than one pixel is flattened in the reference's channel-major order: the weights are permuted to
+    //  the device's pixel-major order when they are uploaded, Plan::prepareWeights)
     // keep the classifier tail in float32: an average pool feeding the classifier writes float32
     const int p = plan.producerOf(in);
     if (p >= 0 && plan.ops[static_cast<size_t>(p)].kind == PlanOp::AVGPOOL && plan.consumerCount(in) == 0)
@@ -509,6 +538,12 @@ void DeConvolutionalLayer::loadAllWeigths(std::vector<float> &weights)
     _weightsLoaded = true;
 }
 
+void DeConvolutionalLayer::weightLayout(std::vector<long long> &parts) const
+{
+    addPart(parts, 0, _nWeights, static_cast<long long>(_channel) * _kSizeX * _kSizeY);
+    if (_useBias) addPart(parts, 5, static_cast<long long>(_numWeights) - _nWeights, static_cast<long long>(_channel) * _kSizeX * _kSizeY);
+}
+
 void DeConvolutionalLayer::foldedAffine(std::vector<float> &scale, std::vector<float> &shift) const
 {
     scale.clear();
@@ -608,8 +643,8 @@ int ActivationLayer::lower(Plan &plan, int in, int layerIndex)
     if (_activation == ActivationType::NONE) return in;          // identity: the reference copies, the plan aliases
     in = plan.nhwcOf(in, layerIndex);
     const PlanTensor ti = plan.tensors[static_cast<size_t>(in)];
-    if (ti.layout != PlanTensor::NHWC) MSNH_THROW("act: the input must be an image tensor");
-    const int out = plan.addTensor(ti.n, ti.h, ti.w, ti.c, ti.dtype, "act_out");
+    // (the flat float32 vector a connected layer writes is a 1 x 1 image of `outputs` channels to the element-wise kernel)
+    const int out = plan.addTensor(ti.n, ti.h, ti.w, ti.c, ti.dtype, "act_out", ti.layout);
     PlanOp &op = plan.addOp(PlanOp::AFFINE, in, -1, out, layerIndex, "act");
     op.act = _activation; op.actParam = actParam();
     op.pureAct = true;
@@ -926,6 +961,12 @@ void BlockLayer::loadAllWeigths(std::vector<float> &weights)
             ptr += n;
         }
     _weightsLoaded = true;
+}
+
+void BlockLayer::weightLayout(std::vector<long long> &parts) const
+{
+    for (const auto &chain : _chains)
+        for (const BaseLayer *l : chain) l->weightLayout(parts);
 }
 
 int BlockLayer::lowerChain(Plan &plan, const std::vector<BaseLayer *> &chain, int in, int layerIndex)

@@ -410,8 +410,7 @@ void NetBuilder::finalizePlan()
         }
         MSNH_DEV(msnh_hip_memcpy_h2d(_inputDev.ptr(), host, inBytes, _stream));
         if (cal->yoloCandCnt.ptr()) MSNH_DEV(msnh_hip_fill_zero(cal->yoloCandCnt.ptr(), cal->yoloCandCnt.bytes(), _stream));
-        cal->runAll(_stream);
-        cal->measureAmax(_stream);
+        cal->runCalibration(_stream);
         plan->applyCalibration(*cal);
     }
     plan->place();

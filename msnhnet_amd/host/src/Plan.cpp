@@ -139,7 +139,7 @@ void Plan::fuse()
                 if (prod.act2 != NONE) continue;
                 prod.act2 = aff.act; prod.act2Param = aff.actParam;
             }
-            else if (prod.kind == PlanOp::CONV || prod.kind == PlanOp::AFFINE || prod.kind == PlanOp::ADD)
+            else if (prod.kind == PlanOp::CONV || prod.kind == PlanOp::AFFINE || prod.kind == PlanOp::ADD || prod.kind == PlanOp::CONNECTED)
             {
                 if (prod.act != NONE) continue;
                 prod.act = aff.act; prod.actParam = aff.actParam;
@@ -270,18 +270,29 @@ void Plan::aliasConcats()
 }
 
 // ---- pass 3: calibration -------------------------------------------------------------------------------------------
-void Plan::measureAmax(msnh_stream_t s)
+// Runs the plan once and takes max|x| of every tensor right behind the launch that writes it.  (Measuring after the whole forward
+// would read arena space that later tensors have reused: a tensor of the first layers would then be given the magnitude of whatever
+// ended up in its place, and with it a scale that flushes its own values to zero.)
+void Plan::runCalibration(msnh_stream_t s)
 {
     DeviceBuffer res(sizeof(float) * tensors.size());
     MSNH_DEV(msnh_hip_fill_zero(res.ptr(), sizeof(float) * tensors.size(), s));
-    std::vector<char> live(tensors.size(), 0);
-    for (const PlanOp &op : ops)
-        if (!op.dead && op.out >= 0) live[static_cast<size_t>(op.out)] = 1;
-    for (size_t t = 0; t < tensors.size(); ++t)
+    for (PlanOp &op : ops)
     {
-        const PlanTensor &pt = tensors[t];
-        if (!live[t] || pt.layout != PlanTensor::NHWC) continue;
-        MSNH_DEV(msnh_hip_absmax(pt.dtype, pt.pixels(), pt.c, ptr(static_cast<int>(t)), ld(static_cast<int>(t)), res.as<float>() + t, s));
+        if (op.dead) continue;
+        launch(op, s);
+        if (op.out < 0) continue;
+        const PlanTensor &pt = tensors[static_cast<size_t>(op.out)];
+        if (pt.layout != PlanTensor::NHWC) continue;
+        if (op.kind == PlanOp::COPY)
+        {
+            // a copy fills a channel slice of its output; the other slices may not have been written yet
+            const size_t el = pt.dtype == MSNH_F16 ? 2 : 4;
+            const void *slice = static_cast<const unsigned char *>(ptr(op.out)) + static_cast<size_t>(op.dstChanOffset) * el;
+            MSNH_DEV(msnh_hip_absmax(pt.dtype, pt.pixels(), tensors[static_cast<size_t>(op.in0)].c, slice, ld(op.out), res.as<float>() + op.out, s));
+            continue;
+        }
+        MSNH_DEV(msnh_hip_absmax(pt.dtype, pt.pixels(), pt.c, ptr(op.out), ld(op.out), res.as<float>() + op.out, s));
     }
     std::vector<float> host(tensors.size(), 0.f);
     MSNH_DEV(msnh_hip_memcpy_d2h(host.data(), res.ptr(), sizeof(float) * tensors.size(), s));
@@ -426,6 +437,14 @@ void Plan::prepareWeights()
             msnh_conv_desc d = convDesc(*this, op);
             if (in.layout == PlanTensor::NCHW_INPUT) d.algo = MSNH_CONV_STEM;
             op.algo = msnh_hip_conv2d_select_algo(&d);
+            if (op.algo == MSNH_CONV_STEM && in.layout != PlanTensor::NCHW_INPUT)
+            {
+                // the first-layer kernel reads the network's NCHW float32 input; a few-channel image tensor made on the device (a
+                // padding or slice layer in front of the first convolution) is NHWC like every other
+                msnh_conv_desc nd = d;
+                nd.algo = MSNH_CONV_IGEMM;
+                op.algo = msnh_hip_conv2d_tile_supported(&nd, 0) ? MSNH_CONV_IGEMM : MSNH_CONV_DIRECT;
+            }
             if (preferWinograd && op.algo == MSNH_CONV_IGEMM)
             {
                 msnh_conv_desc wd = d;
@@ -486,8 +505,25 @@ void Plan::prepareWeights()
         else if (op.kind == PlanOp::CONNECTED)
         {
             const PlanTensor &in = tensors[static_cast<size_t>(op.in0)];
-            const std::vector<float> &w = op.src->kernelWeights();
-            if (w.empty()) MSNH_THROW("connected weights are not loaded (" + op.name + ")");
+            const std::vector<float> &w0 = op.src->kernelWeights();
+            if (w0.empty()) MSNH_THROW("connected weights are not loaded (" + op.name + ")");
+            // The reference flattens an image tensor channel-major, input index = (ch * H + y) * W + x
+            // (src/layers/MsnhConnectedLayer.cpp:187 on an NCHW buffer); on the device the pixel's channels are contiguous.
+            std::vector<float> permuted;
+            const int hw = in.layout == PlanTensor::NHWC ? in.h * in.w : 1;
+            if (hw > 1)
+            {
+                if (ld(op.in0) != in.c) MSNH_THROW("connect: an image input needs a channel count that is a multiple of 8 (" + op.name + ")");
+                const size_t inputs = static_cast<size_t>(hw) * in.c;
+                if (w0.size() % inputs != 0) MSNH_THROW("connect: weight count does not match the input (" + op.name + ")");
+                const size_t outputs = w0.size() / inputs;
+                permuted.resize(w0.size());
+                for (size_t o = 0; o < outputs; ++o)
+                    for (int ch = 0; ch < in.c; ++ch)
+                        for (int p = 0; p < hw; ++p)
+                            permuted[o * inputs + static_cast<size_t>(p) * in.c + ch] = w0[o * inputs + static_cast<size_t>(ch) * hw + p];
+            }
+            const std::vector<float> &w = hw > 1 ? permuted : w0;
             if (in.dtype == MSNH_F16)
             {
                 const std::vector<uint16_t> h = toHalf(w);

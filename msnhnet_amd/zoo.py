@@ -702,6 +702,15 @@ def seeded_weights(slots: List[WeightSlot], seed: int) -> np.ndarray:
     return np.concatenate(parts) if parts else np.zeros(0, np.float32)
 
 
+_LAYOUT_KINDS = {0: "conv_w", 1: "bn_gamma", 2: "bn_beta", 3: "bn_mean", 4: "bn_var", 5: "bias", 6: "fc_w"}
+
+
+def slots_from_layout(layout) -> List[WeightSlot]:
+    """(what, count, fan_in) triples of netapi.Net.weight_layout -> weight slots for seeded_weights: a seeded weights file for any graph
+    the host library can build, not only the ones this module emits."""
+    return [WeightSlot(_LAYOUT_KINDS[w], n, max(f, 1)) for w, n, f in layout]
+
+
 def seeded_input(batch: int, channels: int, height: int, width: int, seed: int) -> np.ndarray:
     """NCHW float32 ~U[0,1)."""
     rng = np.random.Generator(np.random.PCG64(seed))

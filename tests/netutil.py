@@ -141,3 +141,26 @@ def yolo_layer_err(got, ref, logits, channels_per_anchor, ratio, version=3):
     if version == 5:
         e_wh /= 2.0
     return float(max(e_xy, e_sig, e_wh) / scale)
+
+
+def layer_stats(a):
+    """the 22 numbers the golden files keep per layer output: size, finite count, sum, abs-sum, max, min, 16 sampled values"""
+    a = np.asarray(a, np.float64).ravel()
+    fin = np.isfinite(a)
+    v = a[fin]
+    idx = (np.arange(16) * 7919) % max(a.size, 1)
+    return np.array([a.size, fin.sum(), v.sum() if v.size else 0, np.abs(v).sum() if v.size else 0, v.max() if v.size else 0,
+                     v.min() if v.size else 0] + [a[i] if a.size else 0 for i in idx], np.float64)
+
+
+def stats_err(got, want):
+    """layer statistics against stored ones, relative to the layer's range (sums relative to the abs-sum)"""
+    size, nfin, s, sabs, mx, mn = want[:6]
+    assert got[0] == size and got[1] == nfin, ("element / finite count differs", got[:2], want[:2])
+    rng = max(abs(mx), abs(mn), 1e-30)
+    e = max(abs(got[4] - mx), abs(got[5] - mn)) / rng
+    e = max(e, abs(got[2] - s) / max(sabs, 1e-30), abs(got[3] - sabs) / max(sabs, 1e-30))
+    ok = np.isfinite(want[6:])
+    if ok.any():
+        e = max(e, float(np.abs(got[6:][ok] - want[6:][ok]).max()) / rng)
+    return float(e)

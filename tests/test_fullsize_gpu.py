@@ -41,28 +41,6 @@ def _head_logits(m, batch):
     return outs
 
 
-def _stats_err(got, want):
-    """per-layer statistics (sum, abs-sum, max, min and 16 sampled values) against the stored ones, relative to the layer's range"""
-    size, nfin, s, sabs, mx, mn = want[:6]
-    assert got[0] == size and got[1] == nfin, "element / finite count differs"
-    rng = max(abs(mx), abs(mn), 1e-30)
-    e = max(abs(got[4] - mx), abs(got[5] - mn)) / rng
-    e = max(e, abs(got[2] - s) / max(sabs, 1e-30), abs(got[3] - sabs) / max(sabs, 1e-30))
-    samp_ok = np.isfinite(want[6:])
-    if samp_ok.any():
-        e = max(e, float(np.abs(got[6:][samp_ok] - want[6:][samp_ok]).max()) / rng)
-    return e
-
-
-def _layer_stats(a):
-    a = np.asarray(a, np.float64)
-    fin = np.isfinite(a)
-    v = a[fin]
-    idx = (np.arange(16) * 7919) % max(a.size, 1)
-    return np.array([a.size, fin.sum(), v.sum() if v.size else 0, np.abs(v).sum() if v.size else 0, v.max() if v.size else 0,
-                     v.min() if v.size else 0] + [a[i] if a.size else 0 for i in idx], np.float64)
-
-
 @pytest.mark.parametrize("arch,size,batch,fp16", FULL)
 def test_full_size_configuration(arch, size, batch, fp16):
     net, binp, g = nu.model(arch, batch, size, seed=5)
@@ -98,7 +76,7 @@ def test_full_size_configuration(arch, size, batch, fp16):
         final = [ls]
     yolo_stats = None
     if arch == "yolov4":
-        yolo_stats = {s: [_layer_stats(slow.layer_output(i).reshape(batch, -1)[s]) if slow.layer_info(i)["type"] not in ("yolo", "yoloout") else None
+        yolo_stats = {s: [nu.layer_stats(slow.layer_output(i).reshape(batch, -1)[s]) if slow.layer_info(i)["type"] not in ("yolo", "yoloout") else None
                           for i in range(slow.num_layers())] for s in (0, batch - 1)}
     del slow
 
@@ -130,7 +108,7 @@ def test_full_size_configuration(arch, size, batch, fp16):
             for i, st in enumerate(yolo_stats[s]):
                 if st is None or want_stats[i][0] == 0:
                     continue
-                worst = max(worst, _stats_err(st, want_stats[i]))
+                worst = max(worst, nu.stats_err(st, want_stats[i]))
             print(f"FULLSIZE yolov4 slot {s} worst per-layer statistic vs reference: {worst:.3e}", flush=True)
             assert worst <= 2e-2
             n_ref = int(GOLD[f"{key}/box_count"][0])
@@ -200,7 +178,7 @@ def test_fp32_full_size_yolov4_against_reference_vectors():
         for i in range(m.num_layers()):
             if m.layer_info(i)["type"] in ("yolo", "yoloout") or want_stats[i][0] == 0:
                 continue
-            e = _stats_err(_layer_stats(m.layer_output(i).reshape(2, -1)[j]), want_stats[i])
+            e = nu.stats_err(nu.layer_stats(m.layer_output(i).reshape(2, -1)[j]), want_stats[i])
             worst = max(worst, e)
             assert e <= 1e-4, (s, i, m.layer_info(i)["type"], e)
         for k in range(3):
