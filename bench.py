@@ -162,6 +162,9 @@ def main():
     ap.add_argument("--nms", default="auto", choices=["host", "auto", "device"],
                     help="detection workloads: sort + NMS on the host, on the device, or (library default) on the device while the "
                          "previous result had at most 2048 candidates per image -- the seeded weights give 11k, so auto means host here")
+    ap.add_argument("--per-op", default=None, metavar="FILE",
+                    help="also write the per-launch table (every launch of the plan timed on its own with device events: microseconds, "
+                         "algorithmic TFLOP/s and GB/s with every tensor counted once) to FILE")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch a plain 256 MiB -> 256 MiB channel-copy kernel 5 times (a known-size reference for scaling "
                          "the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
@@ -302,6 +305,9 @@ def main():
     if detect:
         res["config"]["boxes_per_image"] = [int(len(b)) for b in out]
         res["config"]["nms"] = a.nms
+    if a.per_op:
+        with open(a.per_op, "w") as f:
+            f.write(net.profile_each_op(20))
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(a.workload, size, tmp, a.seed)
     print(json.dumps(res))

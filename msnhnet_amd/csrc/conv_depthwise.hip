@@ -32,11 +32,17 @@ struct DwArgs
 };
 
 template <int STRIDE, int CPL>
-__global__ __launch_bounds__(256) void convDepthwise3x3Kernel(DwArgs a)
+__global__ __launch_bounds__(256) void convDepthwise3x3Kernel(DwArgs a, int blocks)
 {
     constexpr int COLS = 3 * STRIDE + 3;          // input columns feeding 4 outputs: (4 - 1) * STRIDE + 3
     typedef f16 HV __attribute__((ext_vector_type(CPL)));          // CPL channels per lane: one 16-, 8- or 4-byte access
-    const long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+    // Consecutive hardware workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  Regrouped so that an XCD
+    // works on one contiguous run of rows: the input rows an output row shares with the rows above and below it are then found
+    // in the same L2 instead of being fetched from memory by three of them.
+    const int perXcd = (blocks + 7) / 8;
+    const int logical = static_cast<int>(blockIdx.x % 8) * perXcd + static_cast<int>(blockIdx.x / 8);
+    if (logical >= blocks) return;
+    const long long idx = static_cast<long long>(logical) * 256 + threadIdx.x;
     if (idx >= a.total) return;
     const int cv = a.C / CPL;
     const int c0 = static_cast<int>(idx % cv) * CPL;
@@ -145,9 +151,10 @@ int convDepthwise3x3(const msnh_conv_desc *d, const void *x, const void *w, cons
     a.total = static_cast<long long>(d->batch) * d->out_h * a.strips * (d->in_c / CPL);
     a.xBytes = static_cast<unsigned>(((static_cast<unsigned long long>(d->batch) * d->in_h * d->in_w - 1) * d->in_ld + d->in_c) * 2ull);
     a.act = d->act; a.actParam = d->act_param; a.outMul = d->out_mul;
-    const dim3 grid(gridFor(a.total, 256));
-    if (d->stride == 1) hipLaunchKernelGGL((convDepthwise3x3Kernel<1, CPL>), grid, dim3(256), 0, st, a);
-    else                hipLaunchKernelGGL((convDepthwise3x3Kernel<2, CPL>), grid, dim3(256), 0, st, a);
+    const int blocks = static_cast<int>(gridFor(a.total, 256));
+    const dim3 grid((blocks + 7) / 8 * 8);
+    if (d->stride == 1) hipLaunchKernelGGL((convDepthwise3x3Kernel<1, CPL>), grid, dim3(256), 0, st, a, blocks);
+    else                hipLaunchKernelGGL((convDepthwise3x3Kernel<2, CPL>), grid, dim3(256), 0, st, a, blocks);
     MSNH_LAUNCH_CHECK();
     return 0;
 }

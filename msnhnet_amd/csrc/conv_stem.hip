@@ -66,14 +66,21 @@ __global__ __launch_bounds__(256) void convStemMfmaKernel(StemArgs a)
     const int lane = threadIdx.x & 63;
     const int n = lane & 31;
     const bool hi = lane >= 32;
-    const int wavesTotal = gridDim.x * 4;
-    const int wave0 = blockIdx.x * 4 + (threadIdx.x >> 6);
+    // A workgroup takes one contiguous run of pixel groups (its four wavefronts interleaved), and the hardware's round-robin of
+    // workgroup ids over the 8 XCDs is undone so that an XCD works on one contiguous run of image rows: the input rows that
+    // neighbouring output rows share are then read from memory once, not once per XCD that happens to need them.
+    const int nBlocks = static_cast<int>(gridDim.x);
+    const int perXcd = (nBlocks + 7) / 8;
+    const int logical = static_cast<int>(blockIdx.x % 8) * perXcd + static_cast<int>(blockIdx.x / 8);
+    const int perBlock = (a.nGroups + nBlocks - 1) / nBlocks;
+    const int gBegin = logical < nBlocks ? logical * perBlock : a.nGroups;
+    const int gEnd = min(a.nGroups, gBegin + perBlock);
     const int planes = a.cin * a.H * a.W;
 
     const bool lin = (a.act == MSNH_ACT_LEAKY || a.act == MSNH_ACT_RELU || a.act == MSNH_ACT_NONE);
     const float slope = a.act == MSNH_ACT_LEAKY ? a.actParam : (a.act == MSNH_ACT_RELU ? 0.f : 1.f);
 
-    for (int g = wave0; g < a.nGroups; g += wavesTotal)
+    for (int g = gBegin + static_cast<int>(threadIdx.x >> 6); g < gEnd; g += 4)
     {
         const int gx = g % a.groupsPerRow;
         const int row = g / a.groupsPerRow;
@@ -172,7 +179,7 @@ int launchStem(const StemArgs &a, unsigned blocks, hipStream_t st)
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
         if (e != hipSuccess) { setError("hipFuncSetAttribute: %s", hipGetErrorString(e)); return 1; }
     }
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), smem, st, a);
+    hipLaunchKernelGGL(kern, dim3((blocks + 7) / 8 * 8), dim3(256), smem, st, a);      // a multiple of 8: the XCD regrouping is a bijection then
     MSNH_LAUNCH_CHECK();
     return 0;
 }
@@ -234,15 +241,20 @@ __global__ __launch_bounds__(256) void convStemRowsKernel(StemRowsArgs a)
     const int lane = threadIdx.x & 63;
     const int n = lane & 31;
     const bool hi = lane >= 32;
-    const int wavesTotal = gridDim.x * 4;
-    const int wave0 = blockIdx.x * 4 + (threadIdx.x >> 6);
+    // (contiguous runs of pixel groups per workgroup, XCD by XCD: see convStemMfmaKernel)
+    const int nBlocks = static_cast<int>(gridDim.x);
+    const int perXcd = (nBlocks + 7) / 8;
+    const int logical = static_cast<int>(blockIdx.x % 8) * perXcd + static_cast<int>(blockIdx.x / 8);
+    const int perBlock = (a.nGroups + nBlocks - 1) / nBlocks;
+    const int gBegin = logical < nBlocks ? logical * perBlock : a.nGroups;
+    const int gEnd = min(a.nGroups, gBegin + perBlock);
     const int planes = 3 * a.H * a.W;
     const __amdgpu_buffer_rsrc_t rx = stemRsrc(a.x, a.xBytes);
 
     const bool lin = (a.act == MSNH_ACT_LEAKY || a.act == MSNH_ACT_RELU || a.act == MSNH_ACT_NONE);
     const float slope = a.act == MSNH_ACT_LEAKY ? a.actParam : (a.act == MSNH_ACT_RELU ? 0.f : 1.f);
 
-    for (int g = wave0; g < a.nGroups; g += wavesTotal)
+    for (int g = gBegin + static_cast<int>(threadIdx.x >> 6); g < gEnd; g += 4)
     {
         const int gx = g % a.groupsPerRow;
         const int row = g / a.groupsPerRow;
@@ -335,7 +347,7 @@ int launchStemRows(const StemRowsArgs &a, unsigned blocks, hipStream_t st)
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
         if (e != hipSuccess) { setError("hipFuncSetAttribute: %s", hipGetErrorString(e)); return 1; }
     }
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), smem, st, a);
+    hipLaunchKernelGGL(kern, dim3((blocks + 7) / 8 * 8), dim3(256), smem, st, a);      // a multiple of 8: the XCD regrouping is a bijection then
     MSNH_LAUNCH_CHECK();
     return 0;
 }

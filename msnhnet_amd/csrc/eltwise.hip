@@ -124,6 +124,61 @@ __global__ __launch_bounds__(256) void maxPoolKernel(const T *__restrict__ x, in
     storeVec<T, VEC>(y + p * yLd + c0, m);
 }
 
+// The same for the window sizes the shipped graphs use (2, 3, 5), with the window unrolled: every load of the window is issued
+// before the first comparison (a window position outside the image loads a clamped position and is ignored), where the loop
+// above waits for each load in turn -- 25 dependent round trips for a 5 x 5 window.  Workgroups are dealt to the 8 XCDs in
+// contiguous runs, so the rows that neighbouring output rows share are found in one L2.
+template <typename T, int VEC, int K>
+__global__ __launch_bounds__(256) void maxPoolUnrolledKernel(const T *__restrict__ x, int xLd, int H, int W, int c, int stride, int pad, int OH,
+                                                             int OW, T *__restrict__ y, int yLd, long long total, int blocks)
+{
+    const int perXcd = (blocks + 7) / 8;
+    const int logical = static_cast<int>(blockIdx.x % 8) * perXcd + static_cast<int>(blockIdx.x / 8);
+    if (logical >= blocks) return;
+    const long long idx = static_cast<long long>(logical) * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int cv = c / VEC;
+    const int c0 = static_cast<int>(idx % cv) * VEC;
+    const long long p = idx / cv;
+    const int ox = static_cast<int>(p % OW);
+    const long long t = p / OW;
+    const int oy = static_cast<int>(t % OH);
+    const long long b = t / OH;
+    const int y0 = oy * stride - pad, x0 = ox * stride - pad;
+    float m[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) m[i] = -FLT_MAX;
+    // one window row at a time: its K loads are in flight together, and the next row's are issued while this one is compared
+#pragma unroll
+    for (int ky = 0; ky < K; ++ky)
+    {
+        const int iy = y0 + ky;
+        const bool rowOk = iy >= 0 && iy < H;
+        const int cy = iy < 0 ? 0 : (iy >= H ? H - 1 : iy);
+        const T *row = x + (b * H + cy) * W * xLd + c0;
+        float v[K][VEC];
+        bool ok[K];
+#pragma unroll
+        for (int kx = 0; kx < K; ++kx)
+        {
+            const int ix = x0 + kx;
+            ok[kx] = rowOk && ix >= 0 && ix < W;
+            const int cx = ix < 0 ? 0 : (ix >= W ? W - 1 : ix);
+            loadVec<T, VEC>(row + static_cast<long long>(cx) * xLd, v[kx]);
+        }
+#pragma unroll
+        for (int kx = 0; kx < K; ++kx)
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) m[i] = (ok[kx] && v[kx][i] > m[i]) ? v[kx][i] : m[i];
+    }
+    if constexpr (sizeof(T) == 2)
+    {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) m[i] = m[i] < -65504.f ? -65504.f : m[i];
+    }
+    storeVec<T, VEC>(y + p * yLd + c0, m);
+}
+
 // ---- average pooling over valid elements -------------------------------------------------------------
 template <typename T, typename TOut, int VEC>
 __global__ __launch_bounds__(256) void avgPoolKernel(const T *__restrict__ x, int xLd, int H, int W, int c, int ksize, int stride,
@@ -577,6 +632,20 @@ int msnh_hip_maxpool(int dtype, int batch, int in_h, int in_w, int c, const void
     const int vec = pickVec(dtype, c, {x_ld, y_ld}, {x, y});
     const long long total = static_cast<long long>(batch) * out_h * out_w * (c / vec);
     dim3 grid(gridFor(total, 256));
+    if ((ksize == 2 || ksize == 3 || ksize == 5) && vec > 1)
+    {
+        const int blocks = static_cast<int>(grid.x);
+        const dim3 xgrid((blocks + 7) / 8 * 8);
+#define MSNH_MPU(T, V, K)                                                                                               \
+        hipLaunchKernelGGL((maxPoolUnrolledKernel<T, V, K>), xgrid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, in_h, in_w, c, stride, \
+                           pad, out_h, out_w, static_cast<T *>(y), y_ld, total, blocks)
+#define MSNH_MPUK(T, V) do { if (ksize == 2) MSNH_MPU(T, V, 2); else if (ksize == 3) MSNH_MPU(T, V, 3); else MSNH_MPU(T, V, 5); } while (0)
+        if (dtype == MSNH_F16) MSNH_MPUK(f16, 8); else MSNH_MPUK(float, 4);
+#undef MSNH_MPUK
+#undef MSNH_MPU
+        MSNH_LAUNCH_CHECK();
+        return 0;
+    }
 #define MSNH_MP(T, V)                                                                                                  \
     hipLaunchKernelGGL((maxPoolKernel<T, V>), grid, dim3(256), 0, st, static_cast<const T *>(x), x_ld, in_h, in_w, c, ksize, stride, \
                        pad, out_h, out_w, static_cast<T *>(y), y_ld, total)
