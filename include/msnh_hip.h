@@ -312,6 +312,11 @@ int msnh_hip_yolo_nms_static(int batch, int classes, const float *rows, int cand
  * float16 plan; no counterpart in the reference. */
 int msnh_hip_absmax(int dtype, long long pixels, int c, const void *x, int x_ld, float *result, msnh_stream_t s);
 
+/* Number of elements of an NHWC tensor that are infinite or NaN, added to *result (caller zeroes it).  With msnh_hip_absmax
+ * the run-time check of the float16 plan's range: a non-finite element of a float16 activation tensor means an input ran past
+ * the headroom of the calibrated scales.  No counterpart in the reference. */
+int msnh_hip_count_nonfinite(int dtype, long long pixels, int c, const void *x, int x_ld, unsigned *result, msnh_stream_t s);
+
 #ifdef __cplusplus
 }
 #endif

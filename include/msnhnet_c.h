@@ -113,6 +113,10 @@ int msnhnet_run_classify_gpu(msnhnet_t net, const float *img, long long n, float
 /* NetBuilder::runYoloGPU: counts[b] = boxes of image b; boxes = rows of 7 floats (x y w h conf bestClsConf
  * bestClsIdx), images back to back, at most cap_boxes rows are written; *total = sum of counts. */
 int msnhnet_run_yolo_gpu(msnhnet_t net, const float *img, long long n, int *counts, float *boxes, long long cap_boxes, long long *total);
+/* Range check of a float16 plan for one input (NetBuilder::fp16Headroom): runs the network once on img and writes the factor by which
+ * img could still grow before a float16 activation overflows; 0 means it already did (an input far hotter than the [0,1) image the
+ * scales were calibrated on).  float32 plans report infinity. */
+int msnhnet_fp16_headroom(msnhnet_t net, const float *img, long long n, float *headroom);
 /* Output of top-level layer `layer` from the last run with layer dumps on (batch-major NCHW). Returns its length. */
 long long msnhnet_layer_output(msnhnet_t net, int layer, float *dst, long long cap);
 /* Device-resident serving path: write the batch into the buffer returned by msnhnet_device_input (device memory,

@@ -504,6 +504,23 @@ __global__ __launch_bounds__(256) void absMaxKernel(const T *__restrict__ x, int
     if ((threadIdx.x & 63) == 0 && m > 0.f) atomicMax(reinterpret_cast<int *>(result), __float_as_int(m));
 }
 
+template <typename T>
+__global__ __launch_bounds__(256) void countNonFiniteKernel(const T *__restrict__ x, int xLd, int c, long long total, unsigned *__restrict__ result)
+{
+    unsigned n = 0;
+    for (long long idx = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+         idx += static_cast<long long>(gridDim.x) * blockDim.x)
+    {
+        const long long p = idx / c;
+        const int ch = static_cast<int>(idx - p * c);
+        const float v = fabsf(toF(x[p * xLd + ch]));
+        n += (v <= FLT_MAX) ? 0u : 1u;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) n += __shfl_xor(n, off, 64);
+    if ((threadIdx.x & 63) == 0 && n > 0) atomicAdd(result, n);
+}
+
 } // namespace msnh
 
 using namespace msnh;
@@ -686,6 +703,22 @@ extern "C" int msnh_hip_absmax(int dtype, long long pixels, int c, const void *x
         hipLaunchKernelGGL((absMaxKernel<f16>), grid, dim3(256), 0, resolveStream(s), static_cast<const f16 *>(x), x_ld, c, total, result);
     else
         hipLaunchKernelGGL((absMaxKernel<float>), grid, dim3(256), 0, resolveStream(s), static_cast<const float *>(x), x_ld, c, total, result);
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int msnh_hip_count_nonfinite(int dtype, long long pixels, int c, const void *x, int x_ld, unsigned *result, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype) && pixels >= 0 && c > 0 && x_ld >= c && x && result, "count_nonfinite: bad argument");
+    if (pixels == 0) return 0;
+    const long long total = pixels * c;
+    long long blocks = (total + 255) / 256;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    dim3 grid(static_cast<unsigned>(blocks));
+    if (dtype == MSNH_F16)
+        hipLaunchKernelGGL((countNonFiniteKernel<f16>), grid, dim3(256), 0, resolveStream(s), static_cast<const f16 *>(x), x_ld, c, total, result);
+    else
+        hipLaunchKernelGGL((countNonFiniteKernel<float>), grid, dim3(256), 0, resolveStream(s), static_cast<const float *>(x), x_ld, c, total, result);
     MSNH_LAUNCH_CHECK();
     return 0;
 }

@@ -122,6 +122,7 @@ public:
     void tuneConvs(msnh_stream_t s, const std::string &cacheFile = std::string());
     void run(size_t opBegin, size_t opEnd, msnh_stream_t s);
     void runAll(msnh_stream_t s) { run(0, ops.size(), s); }
+    float fp16Headroom(msnh_stream_t s);    // eager run on the current input: 65504 / largest stored float16 magnitude, 0 after an overflow
     void runCalibration(msnh_stream_t s);   // one eager run; absmax of every NHWC tensor taken right behind the launch that writes it
 
     int   root(int t) const;

@@ -66,6 +66,11 @@ public:
     // network's input size on the device.  mean / std: three floats each, only read by MSNH_PRE_TRANSFORMED.
     void setInputImage(int index, const unsigned char *rgbHwc, int width, int height, int preproc, const float *mean, const float *std, bool shuffleRGB);
 
+    // Range check of the float16 plan for one input (batch*C*H*W floats): the activation scales are fixed at load from one
+    // calibration image of values in [0,1) with a 32x margin; this runs the network once, launch by launch, on `img` and returns the
+    // factor by which `img` could still grow before a float16 activation overflows (0: it already did; the results are then wrong).
+    float fp16Headroom(const std::vector<float> &img);
+
     Point2I getInputSize();
     int getInputChannel();
     int getBatch() const;

@@ -360,6 +360,14 @@ int msnhnet_run_yolo_gpu(msnhnet_t net, const float *img, long long n, int *coun
     });
 }
 
+int msnhnet_fp16_headroom(msnhnet_t net, const float *img, long long n, float *headroom)
+{
+    return guarded([&] {
+        if (!img || n <= 0 || !headroom) MSNH_THROW("bad argument");
+        *headroom = nb(net).fp16Headroom(std::vector<float>(img, img + n));
+    });
+}
+
 long long msnhnet_layer_output(msnhnet_t net, int layer, float *dst, long long cap)
 {
     long long n = -1;

@@ -654,6 +654,14 @@ std::vector<std::vector<YoloBox>> NetBuilder::runYoloGPU(std::vector<float> img)
     return out;
 }
 
+float NetBuilder::fp16Headroom(const std::vector<float> &img)
+{
+    checkInput(img.size());
+    if (_inFlight > 0) MSNH_THROW("fetch the outstanding results first");
+    uploadInput(img);
+    return _net->plan->fp16Headroom(_stream);
+}
+
 // ---- getters ---------------------------------------------------------------------------------------------------------
 Point2I NetBuilder::getInputSize()
 {

@@ -300,6 +300,33 @@ void Plan::runCalibration(msnh_stream_t s)
     for (size_t t = 0; t < tensors.size(); ++t) tensors[t].amax = host[t];
 }
 
+// Eager run on the current input; for every float16 tensor the largest stored magnitude and the number of non-finite elements.
+// Returns 65504 / (largest stored float16 magnitude), 0 if any float16 tensor holds an infinite or NaN element: the factor by which
+// the input could still grow before a float16 activation overflows.
+float Plan::fp16Headroom(msnh_stream_t s)
+{
+    DeviceBuffer res(sizeof(float) * 2);
+    MSNH_DEV(msnh_hip_fill_zero(res.ptr(), sizeof(float) * 2, s));
+    if (yoloCandCnt.ptr()) MSNH_DEV(msnh_hip_fill_zero(yoloCandCnt.ptr(), yoloCandCnt.bytes(), s));
+    for (PlanOp &op : ops)
+    {
+        if (op.dead) continue;
+        launch(op, s);
+        if (op.out < 0) continue;
+        const PlanTensor &pt = tensors[static_cast<size_t>(op.out)];
+        if (pt.layout != PlanTensor::NHWC || pt.dtype != MSNH_F16 || op.kind == PlanOp::COPY) continue;
+        MSNH_DEV(msnh_hip_absmax(pt.dtype, pt.pixels(), pt.c, ptr(op.out), ld(op.out), res.as<float>(), s));
+        MSNH_DEV(msnh_hip_count_nonfinite(pt.dtype, pt.pixels(), pt.c, ptr(op.out), ld(op.out), res.as<unsigned>() + 1, s));
+    }
+    float host[2] = {0.f, 0.f};
+    MSNH_DEV(msnh_hip_memcpy_d2h(host, res.ptr(), sizeof(host), s));
+    MSNH_DEV(msnh_hip_stream_sync(s));
+    unsigned bad = 0;
+    std::memcpy(&bad, &host[1], sizeof(bad));
+    if (bad != 0) return 0.f;
+    return host[0] > 0.f ? 65504.f / host[0] : std::numeric_limits<float>::infinity();
+}
+
 void Plan::applyCalibration(const Plan &cal)
 {
     if (cal.tensors.size() != tensors.size()) MSNH_THROW("calibration plan does not match");

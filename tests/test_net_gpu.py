@@ -132,6 +132,37 @@ def test_fp16_final_outputs(arch, size, batch):
                 assert int(np.argmax(logits[b])) == int(np.argmax(r))
 
 
+@pytest.mark.parametrize("arch,size,batch", [("resnet18", 224, 2), ("yolov3", 160, 2)])
+def test_fp16_headroom_and_hot_input(arch, size, batch):
+    """The float16 scales are fixed at load from one calibration image in [0,1).  An input 4x hotter than that must still be inside
+    the tolerance, the range check must report how much room is left, and it must report 0 once an input has overflowed."""
+    net, binp, g = nu.model(arch, batch, size, seed=3)
+    x = zoo.seeded_input(batch, 3, size, size, seed=4)
+    m = netapi.Net(net, binp, fp16=True, dump_layers=True)
+    h1 = m.fp16_headroom(x)
+    h4 = m.fp16_headroom(4.0 * x)
+    print(arch, "headroom on the [0,1) input", h1, "on the 4x input", h4, flush=True)
+    assert h1 >= 8.0 and h4 >= 2.0 and h4 < h1
+    hot = (4.0 * x).astype(np.float32)
+    ref, ref_boxes = _oracle_layers(arch, size, binp, hot)
+    if arch.startswith("yolo"):
+        boxes = m.run_yolo(hot)
+        for i in range(m.num_layers()):
+            if m.layer_info(i)["type"] != "yolo":
+                continue
+            got = m.layer_output(i - 1).reshape(batch, -1)
+            for b in range(batch):
+                assert nu.rel_err(got[b], ref[b][i - 1]) <= 2e-2
+        for b in range(batch):
+            assert abs(len(boxes[b]) - len(ref_boxes[b])) <= max(2, 0.02 * len(ref_boxes[b]))
+    else:
+        logits = m.run_classify(hot)
+        for b in range(batch):
+            assert nu.rel_err(logits[b], ref[b][-1]) <= 2e-2
+    assert m.fp16_headroom(4096.0 * x) < 1.0
+    assert netapi.Net(net, binp, fp16=False).fp16_headroom(4096.0 * x) == float("inf")
+
+
 import os
 GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_golden.npz"))
 MICRO = bytes(GOLD["micro/names"]).decode().split("\n")
