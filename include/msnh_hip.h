@@ -137,6 +137,8 @@ typedef struct msnh_conv_desc
  * speed per shape.  The host library times them per layer at load (the reference asks cuDNN for the fastest
  * algorithm the same way, src/layers/MsnhConvolutionalLayer.cpp:150-194). */
 int msnh_hip_conv2d_tile_count(void);
+/* Version of the layouts msnh_hip_conv2d_pack_weights writes: packed weights kept on disk are valid for the version they were made under. */
+int msnh_hip_conv2d_pack_layout_version(void);
 /* 1 if IGEMM tile configuration `tile` can run this shape (some configurations are specialised, e.g. for 3x3
  * stride-1 layers whose input patch fits in LDS), else 0.  Pure host function. */
 int msnh_hip_conv2d_tile_supported(const msnh_conv_desc *d, int tile);

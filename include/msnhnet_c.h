@@ -86,6 +86,8 @@ int msnhnet_set_device_nms(int mode);                     /* hard NMS: 0 = candi
                                                               PCIe; 1 (default) = on the device while the previous result had <= 2048 candidates per image */
 int msnhnet_set_tune_cache(int on);                       /* keep the per-layer tile search result in "<weights>.f16.tune" / ".f32.tune" next to the
                                                               .msnhbin file and reuse it on the next load (same graph, same device); off by default */
+int msnhnet_set_weight_cache(int on);                     /* keep the packed device-side kernels and the float16 calibration in "<weights>.f16.pack" /
+                                                            * ".f32.pack" next to the weights file (NetBuilder::setWeightCache); off by default */
 int msnhnet_set_use_winograd(int on);                     /* float16 builds: 3x3 stride-1 convolutions through Winograd F(2x2,3x3);
                                                              the reference keeps its own (ARM NEON, commented out) Winograd switch at
                                                              src/layers/MsnhConvolutionalLayer.cpp:1262 */
@@ -100,6 +102,7 @@ int msnhnet_num_layers(msnhnet_t net);
 int msnhnet_layer_info(msnhnet_t net, int layer, long long *info, char *name, int name_cap);
 long long msnhnet_layer_detail(msnhnet_t net, char *dst, long long cap);      /* returns the full length */
 long long msnhnet_plan_detail(msnhnet_t net, char *dst, long long cap);
+long long msnhnet_load_detail(msnhnet_t net, char *dst, long long cap);       /* wall-clock of the phases of the last load; state of the pack file */
 /* The parts of the weights file this graph expects, in `.msnhbin` order (NetBuilder::loadWeightsFromMsnhBin,
  * src/net/MsnhNetBuilder.cpp:624-663, and each layer's loadAllWeigths).  parts receives up to cap triples { what, count, fan_in }:
  * what = 0 convolution / deconvolution kernel, 1 batch-norm scale, 2 batch-norm shift, 3 running mean, 4 running variance,

@@ -339,6 +339,9 @@ extern "C" {
 
 int msnh_hip_conv2d_tile_count(void) { return igemmTileCount(); }
 
+// Bumped whenever msnh_hip_conv2d_pack_weights changes what it writes for some (descriptor, algorithm).
+int msnh_hip_conv2d_pack_layout_version(void) { return 1; }
+
 int msnh_hip_conv2d_tile_supported(const msnh_conv_desc *d, int tile)
 {
     if (!d || validate(d) || tile < 0 || tile > igemmTileCount()) return 0;

@@ -19,6 +19,7 @@
 #include <vector>
 #include "Msnhnet/config/MsnhnetCfg.h"
 #include "Msnhnet/core/MsnhDevice.h"
+#include "Msnhnet/core/MsnhPackFile.h"
 
 namespace Msnhnet
 {
@@ -114,9 +115,12 @@ public:
     void fuse();                            // passes 1
     void chainMaxPools();                   // stride-1 max-pools of one tensor (SPP): each larger window reads the next smaller one's result
     void aliasConcats();                    // pass 2
-    void applyCalibration(const Plan &calibrated);   // pass 3: take amax from an executed float32 twin
+    void applyCalibration(const std::vector<float> &amax);   // pass 3: amax per tensor, from an executed float32 twin (or from its record on disk)
+    std::vector<float> amaxOfTensors() const;
+    uint64_t structureHash() const;         // over ops and tensors as lowered and optimised (before placement): what a pack file must match
     void place();                           // pass 4 + arena allocation
-    void prepareWeights();                  // fold batch-norm, pick algorithms, pack and upload weights
+    // fold batch-norm, pick algorithms, pack and upload weights; packed kernels are taken from `from` where it holds them and recorded in `to`
+    void prepareWeights(PackFile *from = nullptr, PackFile *to = nullptr);
     // time every tile configuration / algorithm variant per conv launch, keep the fastest.  cacheFile (may be empty): choices of an
     // earlier search for the same plan on the same device are read from it instead of being timed again, and written to it otherwise
     void tuneConvs(msnh_stream_t s, const std::string &cacheFile = std::string());

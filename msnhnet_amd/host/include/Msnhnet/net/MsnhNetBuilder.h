@@ -33,6 +33,10 @@ public:
     static void setDeviceNms(const int &mode);
     static void setTuneCache(const bool &on);
     static bool tuneCache;
+    // keep the packed device-side kernels and the float16 calibration in "<weights>.f16.pack" / ".f32.pack" beside the weights file: the next
+    // load of the same weights into the same graph uploads them as they are (no calibration pass, no re-packing)
+    static void setWeightCache(const bool &on);
+    static bool weightCache;
     static void setUseWinograd(const bool &on);   // float16 plans: 3x3 stride-1 convolutions through Winograd F(2x2,3x3)
     static bool useWinograd;
     static bool autoTune;
@@ -93,6 +97,7 @@ public:
     const std::vector<std::vector<float>> &layerOutputs() const { return _layerOutputs; }
     void setWriteDumpFiles(bool on) { _writeDumpFiles = on; }
     std::string getPlanDetail() const;
+    std::string getLoadDetail() const;      // wall-clock of the phases of the last load, and what happened to the pack file
     double getConvFlops() const;              // 2*MACs of all conv/connected launches of one forward (whole batch)
     // Times `reps` eager passes over the live ops of one kind (PlanOp::Kind, or -1 for all) with device events on
     // the builder's stream; returns the total milliseconds and the number of launches timed.  The ops run on
@@ -104,6 +109,9 @@ public:
 private:
     void finalizePlan();
     std::string _weightsPath;               // set while loadWeightsFromMsnhBin runs: where the tune cache goes
+    uint64_t _weightsHash = 0;
+    float _readMs = 0.f;
+    std::string _loadDetail;
     std::unique_ptr<Plan> lowerNetwork(int dtype);
     void uploadInput(const std::vector<float> &img);
     void runLayersEager();

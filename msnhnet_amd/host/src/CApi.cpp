@@ -246,6 +246,7 @@ int msnhnet_set_use_fp16(int on) { return guarded([&] { NetBuilder::setUseFp16(o
 int msnhnet_set_use_winograd(int on) { return guarded([&] { NetBuilder::setUseWinograd(on != 0); }); }
 int msnhnet_set_device_nms(int mode) { return guarded([&] { NetBuilder::setDeviceNms(mode); }); }
 int msnhnet_set_tune_cache(int on) { return guarded([&] { NetBuilder::setTuneCache(on != 0); }); }
+int msnhnet_set_weight_cache(int on) { return guarded([&] { NetBuilder::setWeightCache(on != 0); }); }
 int msnhnet_set_keep_class_scores(int on) { return guarded([&] { NetBuilder::setKeepClassScores(on != 0); }); }
 int msnhnet_set_save_layer_output(msnhnet_t net, int on) { return guarded([&] { nb(net).setSaveLayerOutput(on != 0); }); }
 int msnhnet_build(msnhnet_t net, const char *path) { return guarded([&] { if (!path) MSNH_THROW("path is NULL"); nb(net).buildNetFromMsnhNet(path); }); }
@@ -301,6 +302,13 @@ long long msnhnet_plan_detail(msnhnet_t net, char *dst, long long cap)
 {
     long long n = -1;
     guarded([&] { n = copyText(nb(net).getPlanDetail(), dst, cap); });
+    return n;
+}
+
+long long msnhnet_load_detail(msnhnet_t net, char *dst, long long cap)
+{
+    long long n = -1;
+    guarded([&] { n = copyText(nb(net).getLoadDetail(), dst, cap); });
     return n;
 }
 

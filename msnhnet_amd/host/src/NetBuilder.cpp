@@ -4,6 +4,7 @@
 // is new.
 #include <cstdlib>
 #include "Msnhnet/net/MsnhNetBuilder.h"
+#include <chrono>
 #include <cmath>
 #include <cstring>
 #include <fstream>
@@ -51,6 +52,8 @@ bool NetBuilder::autoTune = true;
 void NetBuilder::setAutoTune(const bool &on) { autoTune = on; }
 bool NetBuilder::tuneCache = false;
 void NetBuilder::setTuneCache(const bool &on) { tuneCache = on; }
+bool NetBuilder::weightCache = false;
+void NetBuilder::setWeightCache(const bool &on) { weightCache = on; }
 bool NetBuilder::useWinograd = false;
 void NetBuilder::setUseWinograd(const bool &on) { useWinograd = on; }
 
@@ -287,8 +290,11 @@ void NetBuilder::buildNetFromMsnhNet(const std::string &path)
 void NetBuilder::loadWeightsFromMsnhBin(const std::string &path)
 {
     if (BaseLayer::isPreviewMode) MSNH_THROW("Can not load weights in preview mode !");
+    const auto t0 = std::chrono::steady_clock::now();
     _parser->readMsnhBin(path);
     _weightsPath = path;
+    _weightsHash = weightCache ? PackFile::hash(_parser->msnhF32Weights.data(), _parser->msnhF32Weights.size() * sizeof(float)) : 0;
+    _readMs = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
     loadWeightsFromVector(_parser->msnhF32Weights);
     _weightsPath.clear();
     std::vector<float>().swap(_parser->msnhF32Weights);
@@ -311,6 +317,7 @@ void NetBuilder::loadWeightsFromVector(const std::vector<float> &all)
         ptr += n;
     }
     if (ptr != all.size()) MSNH_THROW("Load weights err, need != given. Needed :" + std::to_string(ptr) + " given :" + std::to_string(all.size()));
+    if (_weightsPath.empty()) _readMs = 0.f;
     finalizePlan();
 }
 
@@ -384,13 +391,29 @@ void NetBuilder::finalizePlan()
     _nextSlot = 0;
     _inFlight = 0;
 
+    using Clock = std::chrono::steady_clock;
+    const auto msSince = [](Clock::time_point t) { return std::chrono::duration<float, std::milli>(Clock::now() - t).count(); };
+    Clock::time_point t0 = Clock::now();
     const int dtype = BaseLayer::useFp16 ? MSNH_F16 : MSNH_F32;
     std::unique_ptr<Plan> plan = lowerNetwork(dtype);
     plan->fuse();
     plan->chainMaxPools();
     plan->aliasConcats();
+    const float lowerMs = msSince(t0);
 
-    if (dtype == MSNH_F16)
+    // The packed kernels and the calibration of an earlier load of these weights into this graph, if asked for and still valid
+    const bool winograd = useWinograd && dtype == MSNH_F16;
+    const std::string packPath = (weightCache && !_weightsPath.empty()) ? _weightsPath + (dtype == MSNH_F16 ? ".f16.pack" : ".f32.pack") : std::string();
+    const std::string packLine = PackFile::headerLine(dtype, winograd);
+    const uint64_t graphHash = packPath.empty() ? 0 : plan->structureHash();
+    PackFile kept, fresh;
+    t0 = Clock::now();
+    const bool haveKept = !packPath.empty() && kept.open(packPath, packLine, _weightsHash, graphHash, plan->tensors.size());
+    const float openMs = msSince(t0);
+
+    t0 = Clock::now();
+    if (dtype == MSNH_F16 && haveKept) plan->applyCalibration(kept.amax());
+    else if (dtype == MSNH_F16)
     {
         // One float32 pass over a fixed pseudo-random U[0,1) input fixes the power-of-two scale of every
         // float16 tensor.  The float32 twin is lowered and optimised identically, so tensor ids line up.
@@ -411,14 +434,34 @@ void NetBuilder::finalizePlan()
         MSNH_DEV(msnh_hip_memcpy_h2d(_inputDev.ptr(), host, inBytes, _stream));
         if (cal->yoloCandCnt.ptr()) MSNH_DEV(msnh_hip_fill_zero(cal->yoloCandCnt.ptr(), cal->yoloCandCnt.bytes(), _stream));
         cal->runCalibration(_stream);
-        plan->applyCalibration(*cal);
+        plan->applyCalibration(cal->amaxOfTensors());
     }
+    const float calMs = msSince(t0);
+    t0 = Clock::now();
     plan->place();
     setupYoloBuffers(*plan, _net->batch);
-    plan->preferWinograd = useWinograd && dtype == MSNH_F16;
+    plan->preferWinograd = winograd;
     plan->sparseYolo = !_saveLayerOutput;         // layer dumps read the whole decoded tensors
-    plan->prepareWeights();
+    const bool writing = !packPath.empty() && !haveKept && fresh.create(packPath, packLine, _weightsHash, graphHash, plan->amaxOfTensors());
+    plan->prepareWeights(haveKept ? &kept : nullptr, writing ? &fresh : nullptr);
+    const char *packState = packPath.empty() ? "off" : "read";
+    if (writing) packState = fresh.commit() ? "written" : "not writable";
+    else if (haveKept && kept.stale())
+    {
+        // the file lacks a blob this plan asked for (the kernels were packed afresh): drop it, the next load writes a whole one
+        std::remove(packPath.c_str());
+        packState = "stale, removed";
+    }
+    const float packMs = msSince(t0);
+    t0 = Clock::now();
     if (autoTune) plan->tuneConvs(_stream, (tuneCache && !_weightsPath.empty()) ? _weightsPath + (dtype == MSNH_F16 ? ".f16.tune" : ".f32.tune") : std::string());
+    const float tuneMs = msSince(t0);
+    {
+        std::ostringstream os;
+        os << "load: read+hash " << _readMs << " ms, lower " << lowerMs << " ms, pack file open " << openMs << " ms, calibrate " << calMs << " ms, place+pack+upload "
+           << packMs << " ms, tune " << tuneMs << " ms; pack file " << packState;
+        _loadDetail = os.str();
+    }
 
     // hand every layer its slice of the op list
     for (size_t i = 0; i < _net->layers.size(); ++i)
@@ -809,6 +852,7 @@ std::string NetBuilder::profileEachOp(int reps)
     return os.str();
 }
 
+std::string NetBuilder::getLoadDetail() const { return _loadDetail; }
 std::string NetBuilder::getPlanDetail() const { return _net->plan ? _net->plan->describe() : std::string(); }
 double NetBuilder::getConvFlops() const { return _net->plan ? _net->plan->totalConvFlops() : 0.0; }
 }

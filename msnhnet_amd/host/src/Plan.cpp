@@ -327,9 +327,29 @@ float Plan::fp16Headroom(msnh_stream_t s)
     return host[0] > 0.f ? 65504.f / host[0] : std::numeric_limits<float>::infinity();
 }
 
-void Plan::applyCalibration(const Plan &cal)
+std::vector<float> Plan::amaxOfTensors() const
 {
-    if (cal.tensors.size() != tensors.size()) MSNH_THROW("calibration plan does not match");
+    std::vector<float> a(tensors.size());
+    for (size_t t = 0; t < tensors.size(); ++t) a[t] = tensors[t].amax;
+    return a;
+}
+
+uint64_t Plan::structureHash() const
+{
+    std::ostringstream os;
+    for (const PlanTensor &t : tensors)
+        os << t.n << ' ' << t.h << ' ' << t.w << ' ' << t.c << ' ' << t.dtype << ' ' << static_cast<int>(t.layout) << ' ' << t.parent << ' ' << t.chanOffset << ';';
+    for (const PlanOp &op : ops)
+        os << static_cast<int>(op.kind) << ' ' << op.in0 << ' ' << op.in1 << ' ' << op.out << ' ' << op.dead << ' ' << op.layerIndex << ' ' << op.ksize << ' ' << op.stride << ' '
+           << op.pad << ' ' << op.dilation << ' ' << op.groups << ' ' << static_cast<int>(op.act) << ' ' << static_cast<int>(op.act2) << ' ' << op.in1Sign << ' ' << (op.src2 != nullptr)
+           << ' ' << op.dstChanOffset << ';';
+    const std::string text = os.str();
+    return PackFile::hash(text.data(), text.size());
+}
+
+void Plan::applyCalibration(const std::vector<float> &calAmax)
+{
+    if (calAmax.size() != tensors.size()) MSNH_THROW("calibration plan does not match");
     // tensors that must share one scale: views with their parent, pooling / upsample inputs with outputs
     std::vector<int> group(tensors.size());
     std::iota(group.begin(), group.end(), 0);
@@ -343,7 +363,7 @@ void Plan::applyCalibration(const Plan &cal)
     for (size_t t = 0; t < tensors.size(); ++t)
     {
         const int g = find(static_cast<int>(t));
-        gmax[static_cast<size_t>(g)] = std::max(gmax[static_cast<size_t>(g)], cal.tensors[t].amax);
+        gmax[static_cast<size_t>(g)] = std::max(gmax[static_cast<size_t>(g)], calAmax[t]);
     }
     // Keep the calibrated maximum at or below 2^11: a 32x margin to the half maximum for inputs that run
     // hotter than the calibration image, while staying far above the subnormal range.
@@ -351,7 +371,7 @@ void Plan::applyCalibration(const Plan &cal)
     for (size_t t = 0; t < tensors.size(); ++t)
     {
         PlanTensor &pt = tensors[t];
-        pt.amax = cal.tensors[t].amax;
+        pt.amax = calAmax[t];
         const float m = gmax[static_cast<size_t>(find(static_cast<int>(t)))];
         pt.scaleExp = 0;
         if (pt.dtype == MSNH_F16 && pt.layout == PlanTensor::NHWC && m > target)
@@ -452,11 +472,12 @@ static msnh_conv_desc convDesc(const Plan &plan, const PlanOp &op)
 
 static std::vector<uint16_t> toHalf(const std::vector<float> &v);
 
-void Plan::prepareWeights()
+void Plan::prepareWeights(PackFile *from, PackFile *to)
 {
     size_t workspace = 0;
-    for (PlanOp &op : ops)
+    for (size_t opIndex = 0; opIndex < ops.size(); ++opIndex)
     {
+        PlanOp &op = ops[opIndex];
         if (op.dead) continue;
         if (op.kind == PlanOp::CONV)
         {
@@ -485,9 +506,15 @@ void Plan::prepareWeights()
             if (w.size() != expect) MSNH_THROW("conv weights are not loaded (" + op.name + ")");
             const size_t elems = msnh_hip_conv2d_packed_weight_elems(&d, op.algo);
             const size_t el = d.dtype == MSNH_F16 ? 2 : 4;
-            std::vector<unsigned char> packed(elems * el);
-            MSNH_DEV(msnh_hip_conv2d_pack_weights(&d, op.algo, w.data(), packed.data()));
-            op.wDev.upload(packed.data(), packed.size());
+            const unsigned char *kept = from ? from->blob(static_cast<uint32_t>(opIndex), static_cast<uint32_t>(op.algo), elems * el) : nullptr;
+            if (kept) op.wDev.upload(kept, elems * el);
+            else
+            {
+                std::vector<unsigned char> packed(elems * el);
+                MSNH_DEV(msnh_hip_conv2d_pack_weights(&d, op.algo, w.data(), packed.data()));
+                op.wDev.upload(packed.data(), packed.size());
+                if (to) to->add(static_cast<uint32_t>(opIndex), static_cast<uint32_t>(op.algo), packed.data(), packed.size());
+            }
 
             std::vector<float> scale, shift;
             op.src->foldedAffine(scale, shift);
@@ -538,9 +565,13 @@ void Plan::prepareWeights()
             // (src/layers/MsnhConnectedLayer.cpp:187 on an NCHW buffer); on the device the pixel's channels are contiguous.
             std::vector<float> permuted;
             const int hw = in.layout == PlanTensor::NHWC ? in.h * in.w : 1;
-            if (hw > 1)
+            // (the record's algorithm field of a connected launch: 100 + dtype + 10 if the weights were permuted to pixel-major)
+            const uint32_t packKind = 100u + static_cast<uint32_t>(in.dtype) + (hw > 1 ? 10u : 0u);
+            const size_t packBytes = w0.size() * (in.dtype == MSNH_F16 ? 2u : 4u);
+            const unsigned char *kept = from ? from->blob(static_cast<uint32_t>(opIndex), packKind, packBytes) : nullptr;
+            if (hw > 1 && ld(op.in0) != in.c) MSNH_THROW("connect: an image input needs a channel count that is a multiple of 8 (" + op.name + ")");
+            if (hw > 1 && !kept)
             {
-                if (ld(op.in0) != in.c) MSNH_THROW("connect: an image input needs a channel count that is a multiple of 8 (" + op.name + ")");
                 const size_t inputs = static_cast<size_t>(hw) * in.c;
                 if (w0.size() % inputs != 0) MSNH_THROW("connect: weight count does not match the input (" + op.name + ")");
                 const size_t outputs = w0.size() / inputs;
@@ -550,13 +581,19 @@ void Plan::prepareWeights()
                         for (int p = 0; p < hw; ++p)
                             permuted[o * inputs + static_cast<size_t>(p) * in.c + ch] = w0[o * inputs + static_cast<size_t>(ch) * hw + p];
             }
-            const std::vector<float> &w = hw > 1 ? permuted : w0;
-            if (in.dtype == MSNH_F16)
+            const std::vector<float> &w = hw > 1 && !kept ? permuted : w0;
+            if (kept) op.wDev.upload(kept, packBytes);
+            else if (in.dtype == MSNH_F16)
             {
                 const std::vector<uint16_t> h = toHalf(w);
                 op.wDev.upload(h.data(), h.size() * 2);
+                if (to) to->add(static_cast<uint32_t>(opIndex), packKind, h.data(), h.size() * 2);
             }
-            else op.wDev.upload(w.data(), w.size() * sizeof(float));
+            else
+            {
+                op.wDev.upload(w.data(), w.size() * sizeof(float));
+                if (to) to->add(static_cast<uint32_t>(opIndex), packKind, w.data(), w.size() * sizeof(float));
+            }
             std::vector<float> scale, shift;
             op.src->foldedAffine(scale, shift);
             if (!shift.empty()) op.shiftDev.upload(shift.data(), shift.size() * sizeof(float));

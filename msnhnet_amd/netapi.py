@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libMsnhnet.so")
 
 SYMBOLS = [
     "initMsnhnet", "buildMsnhnet", "runClassifyNoPred", "runYoloNoPred", "runClassifyList", "runYoloList", "dispose", "withGPU", "withCUDNN", "getCpuForwardTime",
-    "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16", "msnhnet_set_use_winograd", "msnhnet_set_tune_cache", "msnhnet_set_device_nms", "msnhnet_set_input_image_u8", "msnhnet_set_input_image", "msnhnet_boxes_to_image",
+    "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16", "msnhnet_set_use_winograd", "msnhnet_set_tune_cache", "msnhnet_set_weight_cache", "msnhnet_load_detail", "msnhnet_set_device_nms", "msnhnet_set_input_image_u8", "msnhnet_set_input_image", "msnhnet_boxes_to_image",
     "msnhnet_set_keep_class_scores", "msnhnet_set_save_layer_output", "msnhnet_build", "msnhnet_load", "msnhnet_load_from_memory",
     "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops", "msnhnet_weight_layout", "msnhnet_fp16_headroom",
     "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
@@ -71,6 +71,7 @@ def lib():
     L.msnhnet_set_use_fp16.argtypes = [ci]
     L.msnhnet_set_use_winograd.argtypes = [ci]
     L.msnhnet_set_tune_cache.argtypes = [ci]
+    L.msnhnet_set_weight_cache.argtypes = [ci]
     L.msnhnet_set_device_nms.argtypes = [ci]
     L.msnhnet_set_input_image_u8.argtypes = [vp, ci, ctypes.POINTER(ctypes.c_ubyte), ci, ci, ci, ci]
     L.msnhnet_set_input_image.argtypes = [vp, ci, ctypes.POINTER(ctypes.c_ubyte), ci, ci, ci, fp, fp, ci]
@@ -83,7 +84,7 @@ def lib():
     L.msnhnet_input_dims.argtypes = [vp, ip, ip, ip, ip]
     L.msnhnet_num_layers.argtypes = [vp]
     L.msnhnet_layer_info.argtypes = [vp, ci, llp, cp, ci]
-    for n in ("msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_time_detail"):
+    for n in ("msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_time_detail", "msnhnet_load_detail"):
         getattr(L, n).argtypes = [vp, cp, ll]
         getattr(L, n).restype = ll
     L.msnhnet_conv_flops.argtypes = [vp]
@@ -140,6 +141,10 @@ def set_device_nms(mode):
 
 def set_tune_cache(on):
     _check(lib().msnhnet_set_tune_cache(1 if on else 0))
+
+
+def set_weight_cache(on):
+    _check(lib().msnhnet_set_weight_cache(1 if on else 0))
 
 
 def set_use_winograd(on):
@@ -242,6 +247,9 @@ class Net:
 
     def plan_detail(self):
         return self._text(self.L.msnhnet_plan_detail)
+
+    def load_detail(self):
+        return self._text(self.L.msnhnet_load_detail)
 
     def time_detail(self):
         return self._text(self.L.msnhnet_time_detail)

@@ -224,3 +224,17 @@ def test_boxes_to_image_matches_the_oracle():
                 assert np.array_equal(got[i, 4:], boxes[i, 4:])
     with pytest.raises(netapi.MsnhnetError):
         netapi.boxes_to_image(boxes, 0, 608, 10, 10)
+
+
+def test_pack_file_round_trip_and_rejections(tmp_path):
+    """the packed-constants file beside a weights file: what was written comes back byte for byte, and a file that belongs to other
+    weights, another plan or another library build, or that is cut short, is refused (tests/cpp/packfile_check.cpp, host code only)"""
+    import subprocess
+    exe = str(tmp_path / "packfile_check")
+    lib = os.path.join(ROOT, "msnhnet_amd", "lib")
+    cmd = ["g++", "-std=c++17", "-O1", "-I" + os.path.join(ROOT, "msnhnet_amd", "host", "include"), os.path.join(ROOT, "tests", "cpp", "packfile_check.cpp"),
+           "-o", exe, "-L" + lib, "-lMsnhnet", "-lmsnh_hip", "-Wl,-rpath," + lib]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout
+    r = subprocess.run([exe, str(tmp_path)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout

@@ -321,6 +321,82 @@ def test_tune_cache(tmp_path):
         netapi.set_tune_cache(False)
 
 
+def test_weight_cache(tmp_path):
+    """the packed kernels and the float16 calibration are kept beside the weights file when asked for: the next load of the same
+    weights into the same graph takes them from the file (same plan, bit-identical outputs, no calibration pass); other weights under
+    the same name, another graph, a cut file or the other Winograd preference make the file count for nothing and it is rewritten"""
+    import shutil
+    arch, size, batch = "yolov3", 96, 2
+    net0, bin0, g = nu.model(arch, batch, size, seed=3)
+    net, binp = str(tmp_path / "m.msnhnet"), str(tmp_path / "m.msnhbin")
+    shutil.copy(net0, net)
+    shutil.copy(bin0, binp)
+    x = zoo.seeded_input(batch, 3, size, size, seed=4)
+    pack = binp + ".f16.pack"
+    plain = netapi.Net(net, binp, fp16=True)
+    assert not os.path.exists(pack) and plain.load_detail().endswith("pack file off")
+    netapi.set_tune_cache(True)          # the same tiles on every load below, so that outputs can be compared bit for bit
+    netapi.set_weight_cache(True)
+    try:
+        a = netapi.Net(net, binp, fp16=True)
+        assert a.load_detail().endswith("pack file written") and os.path.exists(pack) and not os.path.exists(pack + ".tmp")
+        blob = open(pack, "rb").read()
+        assert blob.startswith(b"msnhpack 1 layout ") and b" winograd 0 dtype 1\n" in blob[:100] and len(blob) > os.path.getsize(binp) // 4
+        b = netapi.Net(net, binp, fp16=True)
+        print(a.load_detail(), b.load_detail(), sep="\n", flush=True)
+        assert b.load_detail().endswith("pack file read") and open(pack, "rb").read() == blob
+        assert b.plan_detail() == a.plan_detail()
+        ya, yb = a.run_yolo(x), b.run_yolo(x)
+        for i in range(batch):
+            assert len(ya[i]) > 0 and np.array_equal(ya[i], yb[i])
+        # other weights under the same name (same size): the hash in the file does not fit, the file is rewritten
+        _, bin7, _ = nu.model(arch, batch, size, seed=7)
+        shutil.copy(bin7, binp)
+        c = netapi.Net(net, binp, fp16=True)
+        assert c.load_detail().endswith("pack file written") and open(pack, "rb").read() != blob
+        netapi.set_weight_cache(False)
+        d = netapi.Net(net, binp, fp16=True)
+        netapi.set_weight_cache(True)
+        e = netapi.Net(net, binp, fp16=True)
+        assert d.load_detail().endswith("pack file off") and e.load_detail().endswith("pack file read")
+        yc, yd, ye = c.run_yolo(x), d.run_yolo(x), e.run_yolo(x)
+        for i in range(batch):
+            assert np.array_equal(yc[i], yd[i]) and np.array_equal(ye[i], yd[i])
+            assert not np.array_equal(yc[i], ya[i])
+        # a cut file
+        blob = open(pack, "rb").read()
+        open(pack, "wb").write(blob[:len(blob) // 2])
+        f = netapi.Net(net, binp, fp16=True)
+        assert f.load_detail().endswith("pack file written") and open(pack, "rb").read() == blob
+        # the same weights in another graph (batch 1): not this plan's file
+        g1 = zoo.ARCHS[arch](batch=1, size=size)
+        net1 = str(tmp_path / "m1.msnhnet")
+        open(net1, "w").write(g1.text())
+        h = netapi.Net(net1, binp, fp16=True)
+        assert h.load_detail().endswith("pack file written")
+        y1 = h.run_yolo(x[:1])
+        assert abs(len(y1[0]) - len(yd[0])) <= max(2, 0.02 * len(yd[0]))
+        # float32 plans keep their own file; the Winograd preference is part of the first line
+        k = netapi.Net(net, binp, fp16=False)
+        assert k.load_detail().endswith("pack file written") and os.path.exists(binp + ".f32.pack")
+        assert netapi.Net(net, binp, fp16=False).load_detail().endswith("pack file read")
+        netapi.Net(net, binp, fp16=True)
+        netapi.set_use_winograd(True)
+        try:
+            w = netapi.Net(net, binp, fp16=True)
+            assert w.load_detail().endswith("pack file written") and b" winograd 1 " in open(pack, "rb").read()[:100]
+            w2 = netapi.Net(net, binp, fp16=True)
+            assert w2.load_detail().endswith("pack file read") and "winograd" in w2.plan_detail()
+            yw, yw2 = w.run_yolo(x), w2.run_yolo(x)
+            for i in range(batch):
+                assert np.array_equal(yw[i], yw2[i])
+        finally:
+            netapi.set_use_winograd(False)
+    finally:
+        netapi.set_weight_cache(False)
+        netapi.set_tune_cache(False)
+
+
 @pytest.mark.parametrize("arch,size,batch", [("yolov3", 224, 3), ("yolov3_tiny", 160, 2), ("yolov5s", 128, 2)])
 def test_device_nms_equals_host_nms(arch, size, batch):
     """same network, same input: boxes from the device's NMS (the default) and from the host's sort + NMS are identical,
