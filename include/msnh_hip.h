@@ -291,10 +291,15 @@ int msnh_hip_yolo_gather(int batch, int classes, const float *decoded, long long
  * kept_cnt[1 + b] != 0 says that image b was NOT processed completely: a class with more candidates in that image than the
  * kernels take (6144 with a workspace, 1024 without) or a NaN score.  The caller then runs the reference's procedure on
  * that image's rows itself and ignores its records.
+ * A workspace of msnh_hip_yolo_nms_pair_workspace_bytes() bytes (16-byte aligned) gives the same results faster when a class has
+ * thousands of members: the pair tests of such a class are then spread over the whole device as a bit matrix (a pool of at most
+ * 64 MiB inside the workspace; a class whose matrix does not fit into what is left of it is handled by one workgroup as with the
+ * plain workspace).
  * A record = { row[0..7], score of the class's best-scoring candidate, that candidate's cell index, pick order inside the
  * class, image index }, in no particular order.  The reference's output order of an image is: classes by (record[8]
  * descending, record[9] ascending), inside a class by record[10] ascending. */
 size_t msnh_hip_yolo_nms_workspace_bytes(int batch, int classes, int cand_cap);
+size_t msnh_hip_yolo_nms_pair_workspace_bytes(int batch, int classes, int cand_cap);
 int msnh_hip_yolo_nms(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept,
                       int kept_cap, int *kept_cnt, void *workspace, size_t workspace_bytes, msnh_stream_t s);
 

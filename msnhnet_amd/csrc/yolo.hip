@@ -186,6 +186,7 @@ __global__ __launch_bounds__(256) void yoloRowsKernel(const T *__restrict__ x, i
 // the compact row, the (score, cell) of the class's first member in the global list -- the host orders classes by it --,
 // the pick order inside the class and the image index.
 constexpr int NMS_CAP = 1024;           // members of one class in one image; more -> the image is flagged for the caller
+constexpr int NMS_PAIR_MIN = 256;       // with the pair workspace, classes with more members than this go through the bit matrix
 
 __device__ __forceinline__ unsigned orderedBits(float f)
 {
@@ -222,9 +223,35 @@ __device__ __forceinline__ bool iouAbove(float kx1, float ky1, float kx2, float 
     return 1.f * inter / uni > thr;
 }
 
+// One LDS atomic per wavefront instead of one per lane: the lanes with `pred` get consecutive slots from *counter (-1 for the others).
+// Every lane of the wavefront must make the call.
+__device__ __forceinline__ int waveSlot(bool pred, int *counter)
+{
+    const unsigned long long mask = __ballot(pred);
+    if (mask == 0ull) return -1;
+    const int lane = threadIdx.x & 63;
+    const int leader = __ffsll(static_cast<long long>(mask)) - 1;
+    int first = 0;
+    if (lane == leader) first = atomicAdd(counter, __popcll(mask));
+    first = __shfl(first, leader, 64);
+    return pred ? first + __popcll(mask & ((1ull << lane) - 1ull)) : -1;
+}
+
+__device__ __forceinline__ unsigned long long waveMax64(unsigned long long v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+    {
+        const unsigned lo = __shfl_xor(static_cast<unsigned>(v), o, 64), hi = __shfl_xor(static_cast<unsigned>(v >> 32), o, 64);
+        const unsigned long long other = (static_cast<unsigned long long>(hi) << 32) | lo;
+        v = other > v ? other : v;
+    }
+    return v;
+}
+
 __global__ __launch_bounds__(256) void yoloNmsKernel(const float *__restrict__ rows, int candCap, const int *__restrict__ candCnt, float thr,
                                                      float *__restrict__ kept, int keptCap, int *__restrict__ keptCnt, int *__restrict__ bigCnt,
-                                                     int *__restrict__ wsUsed)
+                                                     int *__restrict__ wsUsed, unsigned long long *__restrict__ pairHdr, int deferAbove)
 {
 #pragma clang fp contract(off)
     __shared__ unsigned long long keyA[NMS_CAP];
@@ -241,22 +268,24 @@ __global__ __launch_bounds__(256) void yoloNmsKernel(const float *__restrict__ r
     const float *r = rows + static_cast<size_t>(b) * candCap * 8;
     if (tid == 0) { nMem = 0; bad = 0; top = 0ull; }
     if (wsUsed != nullptr && cls == 0 && tid == 0) wsUsed[b] = 0;       // yoloNmsBigKernel's cursor into the image's workspace
+    if (pairHdr != nullptr && cls == 0 && b == 0 && tid == 0) { pairHdr[0] = 0ull; pairHdr[1] = 0ull; }    // pool cursor, list length
     __syncthreads();
-    for (int k = tid; k < n; k += 256)
-        if (static_cast<int>(r[static_cast<size_t>(k) * 8 + 6]) == cls)
-        {
-            const int slot = atomicAdd(&nMem, 1);
-            if (slot < NMS_CAP) member[slot] = k;
-        }
+    for (int k0 = 0; k0 < n; k0 += 256)
+    {
+        const int k = k0 + tid;
+        const int slot = waveSlot(k < n && static_cast<int>(r[static_cast<size_t>(k < n ? k : 0) * 8 + 6]) == cls, &nMem);
+        if (slot >= 0 && slot < NMS_CAP) member[slot] = k;
+    }
     __syncthreads();
     const int m = nMem;
     if (bigCnt != nullptr && tid == 0) bigCnt[b * gridDim.x + cls] = m;
     if (m == 0) return;
-    if (m > NMS_CAP)
+    if (m > deferAbove)                                  // (<= NMS_CAP)
     {
         if (bigCnt == nullptr && tid == 0) atomicOr(&keptCnt[1 + b], 1);    // (else yoloNmsBigKernel takes the class)
         return;
     }
+    unsigned long long best = 0ull;
     for (int i = tid; i < m; i += 256)
     {
         const float *q = r + static_cast<size_t>(member[i]) * 8;
@@ -266,8 +295,11 @@ __global__ __launch_bounds__(256) void yoloNmsKernel(const float *__restrict__ r
         const unsigned sb = orderedBits(score), cell = ~static_cast<unsigned>(q[7]);
         keyA[i] = (static_cast<unsigned long long>(orderedBits(conf)) << 32) | sb;
         keyB[i] = cell;
-        atomicMax(&top, (static_cast<unsigned long long>(sb) << 32) | cell);
+        const unsigned long long key = (static_cast<unsigned long long>(sb) << 32) | cell;
+        best = key > best ? key : best;
     }
+    best = waveMax64(best);
+    if ((tid & 63) == 0 && best != 0ull) atomicMax(&top, best);
     __syncthreads();
     if (bad)
     {
@@ -324,24 +356,46 @@ __global__ __launch_bounds__(256) void yoloNmsKernel(const float *__restrict__ r
     }
 }
 
-// The same procedure for a class with more than NMS_CAP members in an image (up to NMS_BIG): the members are sorted by a
-// bitonic network in LDS (keys and row indices, 128 KiB), the sorted row indices go to the workspace, then the corner
-// coordinates of all members take the keys' place in LDS and the whole workgroup runs the greedy pass (one barrier per pick).
-// state[i]: 0xffff = erased, 0xfffe = not visited yet, else the pick order.
-constexpr int NMS_BIG = 6144, NMS_SORT = 8192, NMS_SLOTS = NMS_BIG / 256;
-constexpr int NMS_BIG_LDS = NMS_SORT * 16 + NMS_BIG * 2;        // max(sort: 8+4+4 bytes per slot, boxes: 20 bytes per member) + state
+// The same procedure for a class with more than NMS_CAP members in an image (up to NMS_BIG), one workgroup of 16 wavefronts per class:
+//   1. the members are sorted by a bitonic network in LDS (keys and row indices, 128 KiB); the sorted row indices go to the workspace;
+//   2. the corner coordinates of the sorted members take the keys' place in LDS;
+//   3. the greedy pass runs over chunks of 64 members in sorted order.  A member survives iff no box kept before it overlaps it, so a
+//      chunk is first tested against everything kept so far (lane = member, the kept boxes dealt over the wavefronts, LDS broadcast
+//      reads) and against its own earlier members (a 64 x 64 bit block, 4 columns per wavefront); the first wavefront then resolves the
+//      block with bit operations only (ascending, an alive member erases the later members of its column) and appends the survivors to
+//      the kept list, which grows in place over the coordinates of members already visited (kept <= visited).
+// Two barriers per chunk instead of one per pick, and the pair tests of a chunk use the whole workgroup.
+constexpr int NMS_BIG = 6144, NMS_SORT = 8192, NMS_BIG_THREADS = 1024;
+constexpr int NMS_BIG_LDS = NMS_SORT * 16 + NMS_BIG * 2;        // max(sort: 8+4+4 bytes per slot, boxes: 20 bytes per member) + kept positions
 
-__global__ __launch_bounds__(256) void yoloNmsBigKernel(const float *__restrict__ rows, int candCap, const int *__restrict__ candCnt, float thr,
-                                                        float *__restrict__ kept, int keptCap, int *__restrict__ keptCnt,
-                                                        const int *__restrict__ bigCnt, int *__restrict__ wsSorted, int *__restrict__ wsUsed)
+// With the larger workspace (msnh_hip_yolo_nms_pair_workspace_bytes) step 3 of a large class leaves its workgroup: the sorted members'
+// corners go to the workspace, the class is entered in a list, yoloNmsPairKernel fills a bit matrix (row = a member, bit = a later
+// member it would erase) with the whole chip, and yoloNmsScanKernel walks it (bit operations only).  A class whose matrix does not fit
+// into what is left of the pool keeps to its own workgroup.
+struct NmsPairWs
+{
+    unsigned long long *hdr;            // [0] words of the pool handed out, [1] classes in the list (both zeroed by yoloNmsKernel)
+    int *list;                          // [maxList][8]: image, class, members, offset of the class in the image's sorted rows, matrix offset lo / hi,
+                                        //               score bits and cell of the class's best-scoring member (the record's fields 8, 9)
+    float *boxes;                       // [batch * candCap][8]: x1, y1, x2, y2, area of the sorted members, at the place of their sorted row
+    unsigned long long *pool;
+    unsigned long long poolWords;
+    int maxList;
+};
+
+__global__ __launch_bounds__(NMS_BIG_THREADS) void yoloNmsBigKernel(const float *__restrict__ rows, int candCap, const int *__restrict__ candCnt, float thr,
+                                                                    float *__restrict__ kept, int keptCap, int *__restrict__ keptCnt,
+                                                                    const int *__restrict__ bigCnt, int *__restrict__ wsSorted, int *__restrict__ wsUsed,
+                                                                    NmsPairWs pw, int deferAbove)
 {
 #pragma clang fp contract(off)
+    constexpr int NT = NMS_BIG_THREADS, NW = NT / 64, COLS = 64 / NW;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    __shared__ unsigned long long top;
-    __shared__ int nMem, bad, base, off;
+    __shared__ unsigned long long top, erasedBits, blockBits[64], matOff;
+    __shared__ int nMem, bad, base, off, nKept, usePair;
     const int cls = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
     const int m = bigCnt[b * gridDim.x + cls];
-    if (m <= NMS_CAP) return;
+    if (m <= deferAbove) return;
     if (m > NMS_BIG)
     {
         if (tid == 0) atomicOr(&keptCnt[1 + b], 1);
@@ -353,14 +407,16 @@ __global__ __launch_bounds__(256) void yoloNmsBigKernel(const float *__restrict_
     int n = candCnt[b];
     n = n < candCap ? n : candCap;
     const float *r = rows + static_cast<size_t>(b) * candCap * 8;
-    if (tid == 0) { nMem = 0; bad = 0; top = 0ull; off = atomicAdd(&wsUsed[b], m); }
+    if (tid == 0) { nMem = 0; bad = 0; top = 0ull; erasedBits = 0ull; nKept = 0; off = atomicAdd(&wsUsed[b], m); }
+    if (tid < 64) blockBits[tid] = 0ull;
     __syncthreads();
-    for (int k = tid; k < n; k += 256)
+    unsigned long long best = 0ull;
+    for (int k0 = 0; k0 < n; k0 += NT)
     {
-        const float *q = r + static_cast<size_t>(k) * 8;
-        if (static_cast<int>(q[6]) != cls) continue;
-        const int slot = atomicAdd(&nMem, 1);
-        if (slot >= NMS_SORT) continue;
+        const int k = k0 + tid;
+        const float *q = r + static_cast<size_t>(k < n ? k : 0) * 8;
+        const int slot = waveSlot(k < n && static_cast<int>(q[6]) == cls, &nMem);
+        if (slot < 0 || slot >= NMS_SORT) continue;
         const float conf = q[4];
         const float score = conf * q[5];
         if (!(score == score) || !(conf == conf)) bad = 1;
@@ -368,22 +424,25 @@ __global__ __launch_bounds__(256) void yoloNmsBigKernel(const float *__restrict_
         kA[slot] = (static_cast<unsigned long long>(orderedBits(conf)) << 32) | sb;
         kB[slot] = cell;
         ix[slot] = k;
-        atomicMax(&top, (static_cast<unsigned long long>(sb) << 32) | cell);
+        const unsigned long long key = (static_cast<unsigned long long>(sb) << 32) | cell;
+        best = key > best ? key : best;
     }
+    best = waveMax64(best);
+    if ((tid & 63) == 0 && best != 0ull) atomicMax(&top, best);
     __syncthreads();
     if (bad || nMem != m || off + m > candCap)
     {
         if (tid == 0) atomicOr(&keptCnt[1 + b], bad ? 2 : 4);
         return;
     }
-    int S = 2048;
+    int S = 512;
     while (S < m) S <<= 1;
-    for (int i = m + tid; i < S; i += 256) { kA[i] = 0ull; kB[i] = 0u; ix[i] = -1; }       // below every real key (objectness > 0)
+    for (int i = m + tid; i < S; i += NT) { kA[i] = 0ull; kB[i] = 0u; ix[i] = -1; }       // below every real key (objectness > 0)
     for (int k2 = 2; k2 <= S; k2 <<= 1)
         for (int j = k2 >> 1; j > 0; j >>= 1)
         {
             __syncthreads();
-            for (int t = tid; t < S / 2; t += 256)
+            for (int t = tid; t < S / 2; t += NT)
             {
                 const int lo = ((t / j) * 2 * j) + (t % j), hi = lo + j;
                 const unsigned long long a0 = kA[lo], a1 = kA[hi];
@@ -399,63 +458,332 @@ __global__ __launch_bounds__(256) void yoloNmsBigKernel(const float *__restrict_
         }
     __syncthreads();
     int *sortedRow = wsSorted + static_cast<size_t>(b) * candCap + off;
-    for (int i = tid; i < m; i += 256) sortedRow[i] = ix[i];
-    __syncthreads();                                             // the keys are dead from here on
-    float *x1 = reinterpret_cast<float *>(smem), *y1 = x1 + NMS_BIG, *x2 = y1 + NMS_BIG, *y2 = x2 + NMS_BIG, *area = y2 + NMS_BIG;
-    volatile unsigned short *state = reinterpret_cast<unsigned short *>(smem + NMS_SORT * 16);
-    // Every thread keeps its members (sorted positions tid, tid + 256, ...) in registers, so that the test against a pick is
-    // arithmetic only; LDS holds the same coordinates for the broadcast of the pick and the erased / picked state.
-    float rx1[NMS_SLOTS], ry1[NMS_SLOTS], rx2[NMS_SLOTS], ry2[NMS_SLOTS], rar[NMS_SLOTS];
-    unsigned alive = 0u;
-#pragma unroll
-    for (int t = 0; t < NMS_SLOTS; ++t)
+    for (int i = tid; i < m; i += NT) sortedRow[i] = ix[i];
+    if (tid == 0)
     {
-        const int i = t * 256 + tid;
-        rx1[t] = ry1[t] = rx2[t] = ry2[t] = rar[t] = 0.f;
-        if (i >= m) continue;
+        usePair = 0;
+        if (pw.pool != nullptr)
+        {
+            const unsigned long long W64 = static_cast<unsigned long long>((m + 63) / 64);
+            const unsigned long long need = (static_cast<unsigned long long>(m) + 64ull) * W64;      // rows, then the transposed diagonal blocks
+            const unsigned long long at = atomicAdd(&pw.hdr[0], need);
+            if (at + need <= pw.poolWords)
+            {
+                const int e = atomicAdd(reinterpret_cast<int *>(&pw.hdr[1]), 1);
+                if (e < pw.maxList)
+                {
+                    int *ent = pw.list + static_cast<size_t>(e) * 8;
+                    ent[0] = b; ent[1] = cls; ent[2] = m; ent[3] = off;
+                    ent[4] = static_cast<int>(at & 0xffffffffull); ent[5] = static_cast<int>(at >> 32);
+                    ent[6] = static_cast<int>(top >> 32); ent[7] = static_cast<int>(top & 0xffffffffull);
+                    usePair = 1;
+                }
+            }
+        }
+    }
+    __syncthreads();                                             // the keys are dead from here on
+    if (usePair)
+    {
+        float *bx8 = pw.boxes + (static_cast<size_t>(b) * candCap + off) * 8;
+        for (int i = tid; i < m; i += NT)
+        {
+            const float *q = r + static_cast<size_t>(ix[i]) * 8;
+            const float bx = q[0], by = q[1], bw = q[2], bh = q[3];
+            const float ax1 = bx - bw / 2.f, ax2 = bx + bw / 2.f, ay1 = by - bh / 2.f, ay2 = by + bh / 2.f;
+            *reinterpret_cast<float4 *>(bx8 + static_cast<size_t>(i) * 8) = make_float4(ax1, ay1, ax2, ay2);
+            bx8[static_cast<size_t>(i) * 8 + 4] = (ax2 - ax1 + 1) * (ay2 - ay1 + 1);
+        }
+        return;
+    }
+    float *x1 = reinterpret_cast<float *>(smem), *y1 = x1 + NMS_BIG, *x2 = y1 + NMS_BIG, *y2 = x2 + NMS_BIG, *area = y2 + NMS_BIG;
+    unsigned short *keptPos = reinterpret_cast<unsigned short *>(smem + NMS_SORT * 16);
+    __syncthreads();
+    for (int i = tid; i < m; i += NT)
+    {
         const float *q = r + static_cast<size_t>(sortedRow[i]) * 8;
         const float bx = q[0], by = q[1], bw = q[2], bh = q[3];
         const float ax1 = bx - bw / 2.f, ax2 = bx + bw / 2.f, ay1 = by - bh / 2.f, ay2 = by + bh / 2.f;
-        const float ar = (ax2 - ax1 + 1) * (ay2 - ay1 + 1);
-        x1[i] = ax1; x2[i] = ax2; y1[i] = ay1; y2[i] = ay2; area[i] = ar;
-        rx1[t] = ax1; rx2[t] = ax2; ry1[t] = ay1; ry2[t] = ay2; rar[t] = ar;
-        state[i] = 0xfffe;
-        alive |= 1u << t;
+        x1[i] = ax1; x2[i] = ax2; y1[i] = ay1; y2[i] = ay2;
+        area[i] = (ax2 - ax1 + 1) * (ay2 - ay1 + 1);
     }
     __syncthreads();
-    int picks = 0;
-    for (int i = 0;; ++i)
+    const int lane = tid & 63, wave = tid >> 6;
+    for (int c0 = 0; c0 < m; c0 += 64)
     {
-        while (i < m && state[i] == 0xffff) ++i;                 // same answer in every thread: writes end at the barrier below
-        if (i >= m) break;
-        const float kx1 = x1[i], ky1 = y1[i], kx2 = x2[i], ky2 = y2[i], karea = area[i];
+        const int j = c0 + lane;
+        const bool valid = j < m;
+        const int K = nKept;                                     // <= c0: the kept list never reaches the members still to visit
+        float jx1 = 0.f, jy1 = 0.f, jx2 = 0.f, jy2 = 0.f, jar = 0.f;
+        if (valid) { jx1 = x1[j]; jy1 = y1[j]; jx2 = x2[j]; jy2 = y2[j]; jar = area[j]; }
+        bool erased = false;
+        if (valid)
+            for (int k = wave; k < K; k += NW)
+                if (iouAbove(x1[k], y1[k], x2[k], y2[k], area[k], jx1, jy1, jx2, jy2, jar, thr)) { erased = true; break; }
+        unsigned long long word = 0ull;
+        if (valid && !erased)
 #pragma unroll
-        for (int t = 0; t < NMS_SLOTS; ++t)
+            for (int t = 0; t < COLS; ++t)
+            {
+                const int i = wave * COLS + t;
+                if (i < lane && iouAbove(x1[c0 + i], y1[c0 + i], x2[c0 + i], y2[c0 + i], area[c0 + i], jx1, jy1, jx2, jy2, jar, thr)) word |= 1ull << i;
+            }
+        const unsigned long long eb = __ballot(erased);
+        if (lane == 0 && eb != 0ull) atomicOr(&erasedBits, eb);
+        if (word != 0ull) atomicOr(&blockBits[lane], word);
+        __syncthreads();
+        if (wave == 0)
         {
-            if (t * 256 + 255 <= i || t * 256 >= m) continue;    // (uniform) nothing of this slot lies behind the pick
-            const int j = t * 256 + tid;
-            if (j <= i || !((alive >> t) & 1u)) continue;
-            if (iouAbove(kx1, ky1, kx2, ky2, karea, rx1[t], ry1[t], rx2[t], ry2[t], rar[t], thr)) { alive &= ~(1u << t); state[j] = 0xffff; }
+            unsigned long long alive = __ballot(valid) & ~erasedBits;
+            const unsigned long long mine = blockBits[lane];     // bit i: member i of this chunk, if kept, erases this lane's member
+            unsigned long long rest = alive;
+            while (rest != 0ull)
+            {
+                const int i = __ffsll(static_cast<long long>(rest)) - 1;
+                alive &= ~__ballot(((mine >> i) & 1ull) != 0ull);
+                rest = alive & ~((2ull << i) - 1ull);            // (2 << 63 wraps to 0: nothing is left behind the last member)
+            }
+            if ((alive >> lane) & 1ull)
+            {
+                const int p = K + __popcll(alive & ((1ull << lane) - 1ull));
+                x1[p] = jx1; y1[p] = jy1; x2[p] = jx2; y2[p] = jy2; area[p] = jar;
+                keptPos[p] = static_cast<unsigned short>(j);
+            }
+            blockBits[lane] = 0ull;
+            if (lane == 0) { nKept = K + __popcll(alive); erasedBits = 0ull; }
         }
         __syncthreads();
-        if (tid == 0) state[i] = static_cast<unsigned short>(picks);
-        ++picks;
     }
+    const int picks = nKept;
     if (tid == 0) base = atomicAdd(&keptCnt[0], picks);
     __syncthreads();
     const unsigned long long t = top;
     const float topScore = __uint_as_float((static_cast<unsigned>(t >> 32) & 0x80000000u) ? (static_cast<unsigned>(t >> 32) & 0x7fffffffu) : ~static_cast<unsigned>(t >> 32));
     const float topCell = static_cast<float>(~static_cast<unsigned>(t & 0xffffffffull));
-    for (int i = tid; i < m; i += 256)
+    for (int k = tid; k < picks; k += NT)
     {
-        const unsigned short st = state[i];
-        if (st == 0xffff) continue;
-        const int pos = base + st;
+        const int pos = base + k;
         if (pos >= keptCap) continue;
-        const float4 *q = reinterpret_cast<const float4 *>(r + static_cast<size_t>(sortedRow[i]) * 8);
+        const float4 *q = reinterpret_cast<const float4 *>(r + static_cast<size_t>(sortedRow[keptPos[k]]) * 8);
         float4 *o = reinterpret_cast<float4 *>(kept + static_cast<size_t>(pos) * 12);
         o[0] = q[0]; o[1] = q[1];
-        o[2] = make_float4(topScore, topCell, static_cast<float>(st), static_cast<float>(b));
+        o[2] = make_float4(topScore, topCell, static_cast<float>(k), static_cast<float>(b));
+    }
+}
+
+// Bit matrix of the listed classes: bit v - 64 w of M[i][w] says that member i, if kept, erases the later member v (64 w <= v < 64 w + 64).
+// Work item = one wavefront: the 64 rows of chunk rc (lane = row) against up to NMS_PAIR_GROUP words w >= rc (a lone wavefront needs
+// some 400 cycles per victim, so a longer item would be the kernel's critical path); the victims' corners are the same for
+// every lane: lane l loads victim l and the loop reads lane j's registers, so the item needs neither LDS nor a barrier.  The item holding a diagonal word (w = rc)
+// also writes that block transposed (lane = victim j, bit i = member 64 rc + i erases it) behind the rows: the scan resolves a chunk
+// from it.  The items of all classes form one sequence that the wavefronts of the grid stride through.
+constexpr int NMS_PAIR_GRID = 1024, NMS_PAIR_GROUP = 2;
+
+__device__ __forceinline__ long long nmsPairItems(int W)        // sum over rc < W of ceil((W - rc) / GROUP)
+{
+    const long long q = W / NMS_PAIR_GROUP, r = W % NMS_PAIR_GROUP;
+    return NMS_PAIR_GROUP * q * (q + 1) / 2 + r * (q + 1);
+}
+
+__global__ __launch_bounds__(256) void yoloNmsPairKernel(const unsigned long long *__restrict__ hdr, const int *__restrict__ list, int maxList,
+                                                         const float *__restrict__ boxes, unsigned long long *__restrict__ pool, int candCap, float thr)
+{
+#pragma clang fp contract(off)
+    const int lane = threadIdx.x & 63;
+    const long long nWaves = static_cast<long long>(gridDim.x) * 4;
+    int nList = static_cast<int>(hdr[1]);
+    nList = nList < maxList ? nList : maxList;
+    for (long long t = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.x * 4 + (threadIdx.x >> 6)));; t += nWaves)
+    {
+        long long left = t;
+        int e = 0;
+        for (; e < nList; ++e)
+        {
+            const long long items = nmsPairItems((list[e * 8 + 2] + 63) / 64);
+            if (left < items) break;
+            left -= items;
+        }
+        if (e >= nList) break;                                  // past the last item: every wavefront gets here
+        const int b = list[e * 8], m = list[e * 8 + 2], off = list[e * 8 + 3];
+        const int W = (m + 63) / 64;
+        int rc = 0;
+        for (;; ++rc)
+        {
+            const int groups = (W - rc + NMS_PAIR_GROUP - 1) / NMS_PAIR_GROUP;
+            if (left < groups) break;
+            left -= groups;
+        }
+        const int w0 = rc + static_cast<int>(left) * NMS_PAIR_GROUP;
+        const int w1 = w0 + NMS_PAIR_GROUP < W ? w0 + NMS_PAIR_GROUP : W;
+        const unsigned long long at = (static_cast<unsigned long long>(static_cast<unsigned>(list[e * 8 + 5])) << 32) | static_cast<unsigned>(list[e * 8 + 4]);
+        const float *bx8 = boxes + (static_cast<size_t>(b) * candCap + off) * 8;
+        const int i = rc * 64 + lane;
+        const int iSafe = i < m ? i : m - 1;
+        const float4 k4 = *reinterpret_cast<const float4 *>(bx8 + static_cast<size_t>(iSafe) * 8);
+        const float ka = bx8[static_cast<size_t>(iSafe) * 8 + 4];
+        // the 64 victims of a word: lane l loads victim l (one coalesced read, the next word's under way while this one is worked on);
+        // the loop takes victim j out of lane j's registers
+        const auto victim = [&](int w, float4 &c, float &a) {
+            const int v = w * 64 + lane;
+            const float *q = bx8 + static_cast<size_t>(v < m ? v : m - 1) * 8;
+            c = *reinterpret_cast<const float4 *>(q);
+            a = q[4];
+        };
+        float4 vcNext;
+        float vaNext;
+        victim(w0, vcNext, vaNext);
+        for (int w = w0; w < w1; ++w)
+        {
+            const float4 vc = vcNext;
+            const float va = vaNext;
+            if (w + 1 < w1) victim(w + 1, vcNext, vaNext);
+            unsigned long long word = 0ull, col = 0ull;
+            const int jEnd = m - w * 64 < 64 ? m - w * 64 : 64;
+            for (int j = 0; j < jEnd; ++j)
+            {
+                const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(vc.x), j));
+                const float c1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(vc.y), j));
+                const float c2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(vc.z), j));
+                const float c3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(vc.w), j));
+                const float c4 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(va), j));
+                if (w * 64 + j > i && iouAbove(k4.x, k4.y, k4.z, k4.w, ka, c0, c1, c2, c3, c4, thr)) word |= 1ull << j;
+                if (w == rc && j < lane && iouAbove(c0, c1, c2, c3, c4, k4.x, k4.y, k4.z, k4.w, ka, thr)) col |= 1ull << j;
+            }
+            if (i < m) pool[at + static_cast<unsigned long long>(i) * W + w] = word;
+            if (w == rc) pool[at + static_cast<unsigned long long>(m) * W + static_cast<unsigned long long>(i)] = i < m ? col : 0ull;
+        }
+    }
+}
+
+// The greedy pass of one listed class over its bit matrix, 64 members (one word column) at a time, by a workgroup of four wavefronts.
+// Every wavefront keeps erased bits for all members in two registers per lane (lane l: words l and l + 64): the OR of the rows it has
+// folded in so far.  Per chunk: (1) the first wavefront ORs the four partial words of the chunk, and resolves the chunk from the
+// transposed diagonal block: alive' = candidates & ~{ j : an alive earlier member of the chunk erases j }, repeated until nothing
+// changes (the first t members are final after t rounds; the greedy result is the only fixed point); meanwhile the other three copy
+// the next chunk's rows from the pool to LDS; (2) the kept rows of the chunk are dealt over the four wavefronts and folded into their
+// erased bits, and each publishes its word of the next chunk.
+constexpr int NMS_SCAN_W = (NMS_BIG + 63) / 64;                 // 96 words per row at most
+constexpr int NMS_SCAN_LDS = 2 * 64 * NMS_SCAN_W * 8 + NMS_BIG * 2;
+
+__device__ __forceinline__ unsigned long long readLane64(unsigned long long v, int lane)
+{
+    const unsigned lo = __builtin_amdgcn_readlane(static_cast<int>(static_cast<unsigned>(v)), lane);
+    const unsigned hi = __builtin_amdgcn_readlane(static_cast<int>(static_cast<unsigned>(v >> 32)), lane);
+    return (static_cast<unsigned long long>(hi) << 32) | lo;
+}
+
+__global__ __launch_bounds__(256) void yoloNmsScanKernel(const unsigned long long *__restrict__ hdr, const int *__restrict__ list, int maxList,
+                                                         const unsigned long long *__restrict__ pool, const float *__restrict__ rows, int candCap,
+                                                         const int *__restrict__ wsSorted, float *__restrict__ kept, int keptCap, int *__restrict__ keptCnt)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    __shared__ unsigned long long partial[2][4], aliveSh;
+    __shared__ int nKept, base;
+    int nList = static_cast<int>(hdr[1]);
+    nList = nList < maxList ? nList : maxList;
+    const int e = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    if (e >= nList) return;
+    const int *ent = list + e * 8;
+    const int b = ent[0], m = ent[2], off = ent[3];
+    const int W = (m + 63) / 64;
+    const unsigned long long *M = pool + ((static_cast<unsigned long long>(static_cast<unsigned>(ent[5])) << 32) | static_cast<unsigned>(ent[4]));
+    const unsigned long long *diagT = M + static_cast<unsigned long long>(m) * W;
+    unsigned long long *buf0 = reinterpret_cast<unsigned long long *>(smem), *buf1 = buf0 + 64 * NMS_SCAN_W;
+    unsigned short *keptPos = reinterpret_cast<unsigned short *>(smem + 2 * 64 * NMS_SCAN_W * 8);
+    // rows of chunk c, words c + 1 .. W - 1 (what the later chunks need); wavefront q of nq takes rows q, q + nq, ...; all its loads are
+    // in flight before the first is stored.  Rows past the last member are never folded in and are skipped.
+    const auto fetch = [&](int c, unsigned long long *dst, int q, int nq) {
+        constexpr int R = 22;                                   // ceil(64 / 3)
+        unsigned long long v0[R], v1[R];
+        const int wa = c + 1 + lane, wb = c + 65 + lane;
+#pragma unroll
+        for (int t = 0; t < R; ++t)
+        {
+            const int row = q + t * nq, i = c * 64 + row;
+            const bool ok = row < 64 && i < m;
+            v0[t] = ok && wa < W ? M[static_cast<unsigned long long>(i) * W + wa] : 0ull;
+            v1[t] = ok && wb < W ? M[static_cast<unsigned long long>(i) * W + wb] : 0ull;
+        }
+#pragma unroll
+        for (int t = 0; t < R; ++t)
+        {
+            const int row = q + t * nq;
+            if (row < 64 && wa < W) dst[row * W + wa] = v0[t];
+            if (row < 64 && wb < W) dst[row * W + wb] = v1[t];
+        }
+    };
+    if (wave != 0) fetch(0, buf0, wave - 1, 3);
+    if (tid < 8) partial[tid >> 2][tid & 3] = 0ull;
+    unsigned long long r0 = 0ull, r1 = 0ull;
+    int K = 0;
+    unsigned long long colNext = diagT[lane];                   // (rows past the end hold 0)
+    for (int c = 0; c < W; ++c)
+    {
+        __syncthreads();                                        // the partial words of chunk c are out; (c > 0) its rows are in LDS
+        unsigned long long *cur = (c & 1) ? buf1 : buf0, *nxt = (c & 1) ? buf0 : buf1;
+        if (wave == 0)
+        {
+            const unsigned long long col = colNext;
+            if (c + 1 < W) colNext = diagT[(c + 1) * 64 + lane];
+            const unsigned long long erased = (partial[c & 1][0] | partial[c & 1][1]) | (partial[c & 1][2] | partial[c & 1][3]);
+            const unsigned long long cand = __ballot(c * 64 + lane < m) & ~erased;
+            unsigned long long alive = cand;
+            for (;;)
+            {
+                const unsigned long long next = cand & ~__ballot((col & alive) != 0ull);
+                if (next == alive) break;
+                alive = next;
+            }
+            if ((alive >> lane) & 1ull) keptPos[K + __popcll(alive & ((1ull << lane) - 1ull))] = static_cast<unsigned short>(c * 64 + lane);
+            K += __popcll(alive);
+            if (lane == 0) aliveSh = alive;
+        }
+        else if (c + 1 < W && c > 0) fetch(c, cur, wave - 1, 3);     // (chunk 0 was fetched before the loop)
+        __syncthreads();                                        // the kept members of chunk c are known, its rows are in LDS
+        if (c + 1 >= W) break;
+        unsigned long long it = aliveSh;
+        const bool mine0 = lane > c && lane < W, mine1 = 64 + lane > c && 64 + lane < W;
+        // this wavefront's share: the kept members among rows 16 wave .. 16 wave + 15 of the chunk, four rows per round so that their
+        // LDS reads are in flight together
+        it = (it >> (16 * wave)) & 0xffffull;
+        while (it != 0ull)
+        {
+            int idx[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+            {
+                idx[u] = it != 0ull ? __builtin_amdgcn_readfirstlane(__ffsll(static_cast<long long>(it)) - 1) + 16 * wave : -1;
+                it &= it - 1ull;
+            }
+            unsigned long long a0[4], a1[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+            {
+                a0[u] = (idx[u] >= 0 && mine0) ? cur[idx[u] * W + lane] : 0ull;
+                a1[u] = (idx[u] >= 0 && mine1) ? cur[idx[u] * W + 64 + lane] : 0ull;
+            }
+            r0 |= (a0[0] | a0[1]) | (a0[2] | a0[3]);
+            r1 |= (a1[0] | a1[1]) | (a1[2] | a1[3]);
+        }
+        const unsigned long long mineNext = c + 1 < 64 ? readLane64(r0, c + 1) : readLane64(r1, c + 1 - 64);
+        if (lane == 0) partial[(c + 1) & 1][wave] = mineNext;
+        (void)nxt;
+    }
+    if (tid == 0) { nKept = K; base = atomicAdd(&keptCnt[0], K); }
+    __syncthreads();
+    const int picks = nKept;
+    const unsigned sbTop = static_cast<unsigned>(ent[6]), cellTop = static_cast<unsigned>(ent[7]);
+    const float topScore = __uint_as_float((sbTop & 0x80000000u) ? (sbTop & 0x7fffffffu) : ~sbTop);
+    const float topCell = static_cast<float>(~cellTop);
+    const float *r = rows + static_cast<size_t>(b) * candCap * 8;
+    const int *sortedRow = wsSorted + static_cast<size_t>(b) * candCap + off;
+    for (int k = tid; k < picks; k += 256)
+    {
+        const int pos = base + k;
+        if (pos >= keptCap) continue;
+        const float4 *q = reinterpret_cast<const float4 *>(r + static_cast<size_t>(sortedRow[keptPos[k]]) * 8);
+        float4 *o = reinterpret_cast<float4 *>(kept + static_cast<size_t>(pos) * 12);
+        o[0] = q[0]; o[1] = q[1];
+        o[2] = make_float4(topScore, topCell, static_cast<float>(k), static_cast<float>(b));
     }
 }
 
@@ -603,24 +931,69 @@ extern "C" size_t msnh_hip_yolo_nms_workspace_bytes(int batch, int classes, int 
     return sizeof(int) * (static_cast<size_t>(batch) * classes + static_cast<size_t>(batch) * cand_cap + static_cast<size_t>(batch));
 }
 
-// The two launches of the device NMS; ws = [batch*classes] class sizes | [batch*cand_cap] sorted rows | [batch] cursors, or NULL
-// (small classes only).
+// What follows the plain workspace in the larger one: header (2 x 8 bytes), class list, boxes, pool.
+namespace {
+constexpr size_t kPairPoolMax = static_cast<size_t>(64) << 20;
+size_t pairBase(int batch, int classes, int cand_cap) { return (msnh_hip_yolo_nms_workspace_bytes(batch, classes, cand_cap) + 15) & ~static_cast<size_t>(15); }
+int pairMaxList(int batch, int classes, int cand_cap)
+{
+    const long long perImage = std::min<long long>(classes, cand_cap / (NMS_PAIR_MIN + 1));
+    return static_cast<int>(std::min<long long>(perImage * batch, 4096));
+}
+size_t pairFixed(int batch, int classes, int cand_cap)
+{
+    return pairBase(batch, classes, cand_cap) + 16 + static_cast<size_t>(pairMaxList(batch, classes, cand_cap)) * 32 + static_cast<size_t>(batch) * cand_cap * 32;
+}
+}
+
+extern "C" size_t msnh_hip_yolo_nms_pair_workspace_bytes(int batch, int classes, int cand_cap)
+{
+    if (batch <= 0 || classes <= 0 || cand_cap <= 0) return 0;
+    if (cand_cap <= NMS_PAIR_MIN) return msnh_hip_yolo_nms_workspace_bytes(batch, classes, cand_cap);      // no class can be large
+    // all large classes of an image together have at most cand_cap members, each row at most NMS_BIG / 64 words
+    const size_t rowWords = (static_cast<size_t>(std::min(cand_cap, NMS_BIG)) + 63) / 64;
+    const size_t worst = static_cast<size_t>(batch) * cand_cap * (rowWords + 2) * 8;       // (+ the transposed diagonal blocks, 64 words per chunk)
+    return pairFixed(batch, classes, cand_cap) + std::min(worst, kPairPoolMax);
+}
+
+// The launches of the device NMS; ws = [batch*classes] class sizes | [batch*cand_cap] sorted rows | [batch] cursors, or NULL (small
+// classes only); with wsBytes beyond that part (16-byte aligned): | header | class list | boxes | matrix pool.
 static int launchYoloNms(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept, int kept_cap,
-                         int *kept_cnt, int *ws, bool bigKernelReady, hipStream_t st)
+                         int *kept_cnt, int *ws, size_t wsBytes, bool kernelsReady, hipStream_t st)
 {
     int *bigCnt = ws;
     int *wsSorted = bigCnt ? bigCnt + static_cast<size_t>(batch) * classes : nullptr;
     int *wsUsed = bigCnt ? wsSorted + static_cast<size_t>(batch) * cand_cap : nullptr;
-    hipLaunchKernelGGL(yoloNmsKernel, dim3(classes, batch), dim3(256), 0, st, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, bigCnt, wsUsed);
+    NmsPairWs pw = {nullptr, nullptr, nullptr, nullptr, 0ull, 0};
+    if (ws != nullptr && cand_cap > NMS_PAIR_MIN && wsBytes >= pairFixed(batch, classes, cand_cap) + (static_cast<size_t>(1) << 20) &&
+        reinterpret_cast<uintptr_t>(ws) % 16 == 0)
+    {
+        unsigned char *p = reinterpret_cast<unsigned char *>(ws) + pairBase(batch, classes, cand_cap);
+        pw.hdr = reinterpret_cast<unsigned long long *>(p);
+        pw.maxList = pairMaxList(batch, classes, cand_cap);
+        pw.list = reinterpret_cast<int *>(p + 16);
+        pw.boxes = reinterpret_cast<float *>(p + 16 + static_cast<size_t>(pw.maxList) * 32);
+        pw.pool = reinterpret_cast<unsigned long long *>(reinterpret_cast<unsigned char *>(ws) + pairFixed(batch, classes, cand_cap));
+        pw.poolWords = (wsBytes - pairFixed(batch, classes, cand_cap)) / 8;
+    }
+    hipLaunchKernelGGL(yoloNmsKernel, dim3(classes, batch), dim3(256), 0, st, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, bigCnt, wsUsed, pw.hdr,
+                       pw.pool ? NMS_PAIR_MIN : NMS_CAP);
     MSNH_LAUNCH_CHECK();
     if (ws == nullptr) return 0;
-    if (!bigKernelReady)
+    if (!kernelsReady)
     {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsBigKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_BIG_LDS);
+        if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsScanKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_SCAN_LDS);
         if (e != hipSuccess) { setError("hipFuncSetAttribute: %s", hipGetErrorString(e)); return 1; }
     }
-    hipLaunchKernelGGL(yoloNmsBigKernel, dim3(classes, batch), dim3(256), NMS_BIG_LDS, st, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt,
-                       bigCnt, wsSorted, wsUsed);
+    hipLaunchKernelGGL(yoloNmsBigKernel, dim3(classes, batch), dim3(NMS_BIG_THREADS), NMS_BIG_LDS, st, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt,
+                       bigCnt, wsSorted, wsUsed, pw, pw.pool ? NMS_PAIR_MIN : NMS_CAP);
+    MSNH_LAUNCH_CHECK();
+    if (pw.pool == nullptr) return 0;
+    hipLaunchKernelGGL(yoloNmsPairKernel, dim3(NMS_PAIR_GRID), dim3(256), 0, st, pw.hdr, pw.list, pw.maxList, pw.boxes, pw.pool, cand_cap, nms_thresh);
+    MSNH_LAUNCH_CHECK();
+    hipLaunchKernelGGL(yoloNmsScanKernel, dim3(pw.maxList), dim3(256), NMS_SCAN_LDS, st, pw.hdr, pw.list, pw.maxList, pw.pool, rows, cand_cap, wsSorted, kept, kept_cap,
+                       kept_cnt);
     MSNH_LAUNCH_CHECK();
     return 0;
 }
@@ -639,7 +1012,8 @@ extern "C" int msnh_hip_yolo_nms(int batch, int classes, const float *rows, int 
     if (int rc = checkYoloNmsArgs(batch, classes, rows, cand_cap, cand_cnt, kept, kept_cap, kept_cnt)) return rc;
     MSNH_REQUIRE(workspace == nullptr || (workspace_bytes >= msnh_hip_yolo_nms_workspace_bytes(batch, classes, cand_cap) && reinterpret_cast<uintptr_t>(workspace) % 4 == 0),
                  "yolo_nms: workspace too small (msnh_hip_yolo_nms_workspace_bytes)");
-    return launchYoloNms(batch, classes, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, static_cast<int *>(workspace), false, resolveStream(s));
+    return launchYoloNms(batch, classes, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, static_cast<int *>(workspace), workspace ? workspace_bytes : 0, false,
+                         resolveStream(s));
 }
 
 // ---- the same call for callers that cannot allocate ------------------------------------------------------------------------------
@@ -666,6 +1040,7 @@ int yoloNmsSetupDevice()
     MSNH_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
     MSNH_REQUIRE(p != nullptr, "yolo_nms_static: the scratch array has no address on device %d", dev);
     MSNH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsBigKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_BIG_LDS));
+    MSNH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsScanKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_SCAN_LDS));
     g_scratchPtr[dev] = static_cast<int *>(p);
     return 0;
 }
@@ -688,7 +1063,7 @@ extern "C" int msnh_hip_yolo_nms_static(int batch, int classes, const float *row
         if (int rc = yoloNmsSetupDevice()) return rc;        // (msnh_hip_init does this for the device it selects)
     // Nothing in the workspace has to start at zero: the first kernel writes every class size and resets every image's cursor,
     // and the sorted rows are written before they are read.
-    return launchYoloNms(batch, classes, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, g_scratchPtr[dev], true, resolveStream(s));
+    return launchYoloNms(batch, classes, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, g_scratchPtr[dev], need, true, resolveStream(s));
 }
 
 extern "C" int msnh_hip_absmax(int dtype, long long pixels, int c, const void *x, int x_ld, float *result, msnh_stream_t s)

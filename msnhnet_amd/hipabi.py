@@ -40,7 +40,7 @@ SYMBOLS = [
     "msnh_hip_conv2d_packed_weight_elems", "msnh_hip_conv2d_pack_weights", "msnh_hip_conv2d_workspace_bytes", "msnh_hip_conv2d", "msnh_hip_letterbox_u8", "msnh_hip_image_u8_to_input",
     "msnh_hip_affine_act", "msnh_hip_add_act", "msnh_hip_copy_channels", "msnh_hip_maxpool", "msnh_hip_avgpool",
     "msnh_hip_upsample_nearest", "msnh_hip_pad", "msnh_hip_slice", "msnh_hip_upsample_bilinear", "msnh_hip_softmax", "msnh_hip_deconv_col2im", "msnh_hip_connected", "msnh_hip_nchw_to_nhwc", "msnh_hip_nhwc_to_nchw", "msnh_hip_yolo_decode", "msnh_hip_yolo_decode_candidates",
-    "msnh_hip_yolo_gather", "msnh_hip_yolo_nms", "msnh_hip_yolo_nms_workspace_bytes", "msnh_hip_yolo_nms_static", "msnh_hip_yolo_nms_static_max_bytes", "msnh_hip_absmax", "msnh_hip_count_nonfinite",
+    "msnh_hip_yolo_gather", "msnh_hip_yolo_nms", "msnh_hip_yolo_nms_workspace_bytes", "msnh_hip_yolo_nms_pair_workspace_bytes", "msnh_hip_yolo_nms_static", "msnh_hip_yolo_nms_static_max_bytes", "msnh_hip_absmax", "msnh_hip_count_nonfinite",
 ]
 
 
@@ -108,6 +108,8 @@ def lib():
     L.msnh_hip_yolo_nms.argtypes = [ci, ci, vp, ci, vp, cf, vp, ci, vp, vp, sz, vp]
     L.msnh_hip_yolo_nms_workspace_bytes.argtypes = [ci, ci, ci]
     L.msnh_hip_yolo_nms_workspace_bytes.restype = sz
+    L.msnh_hip_yolo_nms_pair_workspace_bytes.argtypes = [ci, ci, ci]
+    L.msnh_hip_yolo_nms_pair_workspace_bytes.restype = sz
     L.msnh_hip_yolo_nms_static.argtypes = [ci, ci, vp, ci, vp, cf, vp, ci, vp, vp]
     L.msnh_hip_yolo_nms_static_max_bytes.argtypes = []
     L.msnh_hip_yolo_nms_static_max_bytes.restype = sz

@@ -359,11 +359,10 @@ public:
     std::vector<std::vector<YoloBox>> finalOut;
     static bool keepClassScores;           // also fill YoloBox::classesVal (costs an extra device->host copy)
     // hard NMS on the device (only the kept boxes are copied back): 0 = never (sort + NMS on the host), 2 = always,
-    // 1 = while the previous result of this network had at most kDeviceNmsCandidates candidates in every image (default): the
-    // device kernels give one workgroup to a class of an image, which beats the host for the hundreds of candidates real
-    // detections have and loses to its threads when a class has thousands.
+    // 1 = while the previous result of this network had at most kDeviceNmsCandidates candidates in every image (default): that is
+    // the largest class the device kernels take (msnh_hip_yolo_nms), so no image of such a batch can fall back to the host.
     static int deviceNms;
-    static const int kDeviceNmsCandidates = 2048;
+    static const int kDeviceNmsCandidates = 6144;
 
     // host post-processing of the compacted candidate rows of one image (8 floats per row, see msnh_hip_yolo_gather)
     std::vector<YoloBox> boxesFromRows(const float *rows, int count, const float *decodedOfImage) const;
@@ -386,10 +385,12 @@ private:
         msnh_event_t event = nullptr, ready = nullptr;
         bool pending = false, onDevice = false;
         size_t rowsCopied = 0;             // row slots per image that the asynchronous copy brings to the host
+        size_t quick = 0;                  // device NMS: records that the asynchronous copy brings to the host
     };
     std::vector<YoloBox> boxesFromKept(std::vector<const float *> &records) const;
     msnh_stream_t _copyStream = nullptr, _fetchStream = nullptr;
     int _lastMaxCandidates = 0;            // largest per-image candidate count of the previous result
+    size_t _lastKept = 0;                  // records the device NMS kept for the previous batch
     Slot _slots[2];
 };
 }

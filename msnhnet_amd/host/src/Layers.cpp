@@ -1171,7 +1171,7 @@ int YoloLayer::lower(Plan &plan, int in, int layerIndex)
 bool YoloOutLayer::keepClassScores = false;
 int YoloOutLayer::deviceNms = 1;
 static const size_t kRecordBytes = 12 * sizeof(float);     // one record of msnh_hip_yolo_nms
-static const size_t kQuickRecords = 2048;                   // records copied back with the counters, before their number is known
+static const size_t kQuickRecords = 2048;                   // least number of records copied back with the counters, before their number is known
 
 YoloOutLayer::YoloOutLayer(const int &batch, const int &orgWidth, const int &orgHeight, std::vector<int> &yoloIndexes, std::vector<YoloInfo> &yoloLayersInfo,
                            const float &confThresh, const float &nmsThresh, const int &useSotfNms, const YoloType &yoloType)
@@ -1453,21 +1453,24 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
     sl.onDevice = !_useSoftNms && (deviceNms == 2 || (deviceNms == 1 && _lastMaxCandidates <= kDeviceNmsCandidates));
     if (sl.onDevice)
     {
-        // NMS on the snapshot, on the copy stream: it overlaps the next forward, and what crosses PCIe is the kept boxes
-        // (the first kQuickRecords of them with the counters; finish() fetches the rest if there are more)
+        // NMS on the snapshot, on the copy stream: it overlaps the next forward, and what crosses PCIe is the kept boxes.  The records
+        // leave with the counters, as many as the previous result had and half as many again: a copy asked for in finish() would
+        // queue behind whatever the device runs by then (the next forward), and the host would wait for that instead of working
+        // beside it.  finish() fetches the rest only if there are more.
         const size_t keptCntBytes = sizeof(int) * (1 + static_cast<size_t>(_batch));
         const size_t keptCap = cells * static_cast<size_t>(_batch);
         if (sl.devKeptCnt.bytes() < keptCntBytes) sl.devKeptCnt.alloc(keptCntBytes);
         if (sl.devKept.bytes() < keptCap * kRecordBytes) sl.devKept.alloc(keptCap * kRecordBytes);
         sl.keptCnt.reserve(keptCntBytes);
-        sl.kept.reserve(std::min(keptCap, kQuickRecords) * kRecordBytes);
+        sl.quick = std::min(keptCap, std::max(kQuickRecords, _lastKept + _lastKept / 2 + 1024));
+        sl.kept.reserve(sl.quick * kRecordBytes);
         MSNH_DEV(msnh_hip_fill_zero(sl.devKeptCnt.ptr(), keptCntBytes, _copyStream));
-        const size_t wsBytes = msnh_hip_yolo_nms_workspace_bytes(_batch, _channel - 5, pl.yoloCells);
+        const size_t wsBytes = msnh_hip_yolo_nms_pair_workspace_bytes(_batch, _channel - 5, pl.yoloCells);
         if (sl.devNmsWs.bytes() < wsBytes) sl.devNmsWs.alloc(wsBytes);
         MSNH_DEV(msnh_hip_yolo_nms(_batch, _channel - 5, sl.devRows.as<float>(), pl.yoloCells, sl.devCnt.as<int>(), _nmsThresh, sl.devKept.as<float>(),
                                    static_cast<int>(keptCap), sl.devKeptCnt.as<int>(), sl.devNmsWs.ptr(), wsBytes, _copyStream));
         MSNH_DEV(msnh_hip_memcpy_d2h(sl.keptCnt.ptr(), sl.devKeptCnt.ptr(), keptCntBytes, _copyStream));
-        MSNH_DEV(msnh_hip_memcpy_d2h(sl.kept.ptr(), sl.devKept.ptr(), std::min(keptCap, kQuickRecords) * kRecordBytes, _copyStream));
+        MSNH_DEV(msnh_hip_memcpy_d2h(sl.kept.ptr(), sl.devKept.ptr(), sl.quick * kRecordBytes, _copyStream));
     }
     else
     {
@@ -1531,17 +1534,19 @@ void YoloOutLayer::finish(int slot)
         const size_t total = static_cast<size_t>(keptCnt[0]);
         // (its own stream: the copy stream may already hold the next forward's work)
         if (_fetchStream == nullptr) MSNH_DEV(msnh_hip_stream_create(&_fetchStream));
-        if (total > kQuickRecords)
+        _lastKept = total;
+        const size_t quick = sl.quick;
+        if (total > quick)
         {
             PinnedBuffer &rest = sl.rows;                                  // the host path's buffer doubles as the overflow area
-            rest.reserve((total - kQuickRecords) * kRecordBytes);
-            MSNH_DEV(msnh_hip_memcpy_d2h(rest.ptr(), sl.devKept.as<char>() + kQuickRecords * kRecordBytes, (total - kQuickRecords) * kRecordBytes, _fetchStream));
+            rest.reserve((total - quick) * kRecordBytes);
+            MSNH_DEV(msnh_hip_memcpy_d2h(rest.ptr(), sl.devKept.as<char>() + quick * kRecordBytes, (total - quick) * kRecordBytes, _fetchStream));
             MSNH_DEV(msnh_hip_stream_sync(_fetchStream));
         }
         std::vector<std::vector<const float *>> perImage(static_cast<size_t>(_batch));
         for (size_t i = 0; i < total; ++i)
         {
-            const float *r = i < kQuickRecords ? sl.kept.as<float>() + i * 12 : sl.rows.as<float>() + (i - kQuickRecords) * 12;
+            const float *r = i < quick ? sl.kept.as<float>() + i * 12 : sl.rows.as<float>() + (i - quick) * 12;
             const int b = static_cast<int>(r[11]);
             if (b < 0 || b >= _batch) MSNH_THROW("YoloOut: device NMS record names image " + std::to_string(b));
             perImage[static_cast<size_t>(b)].push_back(r);

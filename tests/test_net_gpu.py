@@ -397,10 +397,11 @@ def test_weight_cache(tmp_path):
         netapi.set_tune_cache(False)
 
 
-@pytest.mark.parametrize("arch,size,batch", [("yolov3", 224, 3), ("yolov3_tiny", 160, 2), ("yolov5s", 128, 2)])
+@pytest.mark.parametrize("arch,size,batch", [("yolov3", 224, 3), ("yolov3_tiny", 160, 2), ("yolov5s", 128, 2), ("yolov3", 704, 1)])
 def test_device_nms_equals_host_nms(arch, size, batch):
     """same network, same input: boxes from the device's NMS (the default) and from the host's sort + NMS are identical,
-    eagerly and with two forwards in flight"""
+    eagerly and with two forwards in flight; the 704 x 704 case has a class with more than 5000 members in the image (the
+    large-class kernel)"""
     net, binp, g = nu.model(arch, batch, size, seed=3)
     xs = [zoo.seeded_input(batch, 3, size, size, seed=s) for s in (4, 5, 6)]
     print("device nms", arch, size, batch, flush=True)
@@ -419,6 +420,9 @@ def test_device_nms_equals_host_nms(arch, size, batch):
     got += auto
     want += want
     assert sum(len(b) for w in want for b in w) > 0
+    if size == 704:
+        for w in want[:3]:
+            assert 5000 <= np.bincount(w[0][:, 6].astype(np.int64)).max() <= 6144
     for g_, w_ in zip(got, want):
         for b in range(batch):
             assert np.array_equal(g_[b], w_[b], equal_nan=True)

@@ -458,14 +458,23 @@ def test_yolo_nms():
     rows[3, 7, 5] = np.nan             # image 3: a NaN class score
     rd, cd = gu.dev(rows), gu.dev(cnt)
     nbytes = abi.lib().msnh_hip_yolo_nms_workspace_bytes(7, cls, cells)
-    ws = torch.full((nbytes // 4,), 0x55555555, dtype=torch.int32).cuda()
+    # the larger workspace (pair tests of the large classes as a bit matrix over the whole device), whole and with a pool that only
+    # takes the 1200-member class, so that the 6100-member one stays with its own workgroup
+    pbytes = abi.lib().msnh_hip_yolo_nms_pair_workspace_bytes(7, cls, cells)
+    pool = min(7 * cells * 98 * 8, 64 << 20)
+    assert pbytes > nbytes + pool
+    ws = torch.full((pbytes // 4 + 4,), 0x55555555, dtype=torch.int32).cuda()
     print("yolo_nms", cnt.tolist(), flush=True)
-    for with_ws, flags in ((True, [0, 0, 0, 2, 0, 0, 1]), (False, [0, 1, 0, 2, 0, 1, 1])):
+    for ws_bytes, flags in ((nbytes, [0, 0, 0, 2, 0, 0, 1]), (0, [0, 1, 0, 2, 0, 1, 1]), (pbytes, [0, 0, 0, 2, 0, 0, 1]),
+                            (pbytes - pool + (5 << 18), [0, 0, 0, 2, 0, 0, 1])):
+        with_ws = ws_bytes > 0
+        ws.fill_(0x55555555)
         keptd = torch.zeros((7 * cells, 12), dtype=torch.float32).cuda()
         kcd = torch.zeros(8, dtype=torch.int32).cuda()
         gu.sync()
+        print("yolo_nms workspace", ws_bytes, flush=True)
         abi.check(abi.lib().msnh_hip_yolo_nms(7, cls, gu.ptr(rd), cells, gu.ptr(cd), nms_t, gu.ptr(keptd), 7 * cells, gu.ptr(kcd),
-                                              gu.ptr(ws) if with_ws else None, nbytes if with_ws else 0, None))
+                                              gu.ptr(ws) if with_ws else None, ws_bytes, None))
         gu.sync()
         kc = kcd.cpu().numpy()
         kept = keptd.cpu().numpy()
