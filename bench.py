@@ -75,7 +75,11 @@ def cpu_baseline(arch, size, tmp, seed, budget_s=30.0):
 # HBM bytes per convolution launch (fetch + write), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script,
 # each scaled by what the same counter reads for a plain copy kernel of known size (fetch x2.0, write x1.0); the runs
 # and their summary are in profiles/conv_igemm_yolov3_608_f16_b8.md.  None for workloads that were not profiled.
-HBM_BYTES_PER_CONV_LAUNCH = {("yolov3", "f16", 8): int((40.24 + 19.06) * 2**20)}
+HBM_BYTES_PER_CONV_LAUNCH = {("yolov3", "f16", 8): int((38.80 + 18.00) * 2**20)}
+# The same for the depthwise launches (the dominant bandwidth-bound kernel of a network that has them); runs and summary in
+# profiles/hbm_kernels_mobilenetv2_b64_yolov4_b16.md.
+HBM_BYTES_PER_DEPTHWISE_LAUNCH = {("mobilenetv2", "f16", 64): int((27.07 + 16.53) * 2**20)}
+MSNH_CONV_DEPTHWISE = 3
 
 
 def conv_shape_mode(a):
@@ -286,13 +290,24 @@ def main():
     # roofline of the dominant kernel family: the convolution launches, timed with device events on the
     # library's stream; algorithmic FLOPs = 2*B*Cout*OH*OW*(Cin/g)*k*k per launch (direct-convolution count)
     marker()
-    conv_ms, launches, flops = net.profile_ops(0, 10)
+    conv_ms, launches, flops, conv_bytes = net.profile_ops_bytes(0, 10)
     marker()
     achieved = flops / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else 0.0
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK[dtype], "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK[dtype], 4), "traffic": HBM_BYTES_PER_CONV_LAUNCH.get((a.workload, dtype, batch)),
                 "kernel": "convolution launches (implicit-GEMM MFMA + stem)", "launches_per_step": launches // 10,
-                "avg_launch_us": round(conv_ms * 1e3 / max(launches, 1), 2), "flops_per_step": flops / 10}
+                "avg_launch_us": round(conv_ms * 1e3 / max(launches, 1), 2), "flops_per_step": flops / 10,
+                "least_bytes_per_launch": int(conv_bytes / max(launches, 1))}
+
+    # a network with depthwise convolutions is judged against the HBM roof as well: those launches move
+    # (input + output + weights) bytes each and compute next to nothing
+    roofline_hbm = None
+    dw_ms, dw_n, _, dw_bytes = net.profile_ops_bytes(1000 + MSNH_CONV_DEPTHWISE, 10)
+    if dw_n > 0:
+        gbs = dw_bytes / (dw_ms * 1e-3) / 1e9
+        roofline_hbm = {"bound": "hbm", "achieved": round(gbs, 1), "peak": 8000.0, "unit": "GB/s", "frac": round(gbs / 8000.0, 4),
+                        "traffic": HBM_BYTES_PER_DEPTHWISE_LAUNCH.get((a.workload, dtype, batch)), "kernel": "convDepthwise3x3Kernel",
+                        "launches_per_step": dw_n // 10, "avg_launch_us": round(dw_ms * 1e3 / dw_n, 2), "bytes_per_step": dw_bytes / 10}
 
     res = {"metric": f"images/sec on 1 MI355X ({a.workload} {size} {dtype} b{batch})", "value": round(batch / (ms_per_step * 1e-3), 2),
            "unit": "images/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4),
@@ -302,6 +317,8 @@ def main():
                       "input": a.input, "seed": a.seed, "ms_per_step_median": round(ms_median, 4), "device_launches_per_step": n_all // 10,
                       "device_ms_per_step_eager": round(gpu_only_ms, 4), "host_f32_images_per_s": host_rate},
            "roofline": roofline}
+    if roofline_hbm is not None:
+        res["roofline_hbm"] = roofline_hbm
     if detect:
         res["config"]["boxes_per_image"] = [int(len(b)) for b in out]
         res["config"]["nms"] = a.nms

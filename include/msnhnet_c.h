@@ -135,6 +135,9 @@ long long msnhnet_yolo_max_boxes(msnhnet_t net);
  * 4 maxpool, 5 avgpool, 6 upsample, 7 connected, 8 input cast, 9 yolo decode, -1 all).  Outputs the total
  * milliseconds, the number of launches timed and their algorithmic FLOPs (2*MACs; 0 for non-GEMM kinds). */
 int msnhnet_profile_ops(msnhnet_t net, int kind, int reps, float *ms_total, int *launches, double *flops);
+/* The same with kind = 1000 + a also accepted (the convolution launches of algorithm a: 3 depthwise, 5 first layer, ...), and with
+ * the bytes those launches must move at least (input + output + fused residual + weights) in *bytes. */
+int msnhnet_profile_ops_bytes(msnhnet_t net, int kind, int reps, float *ms_total, int *launches, double *flops, double *bytes);
 /* Per-launch timing table (text): every live launch of the plan timed on its own, `reps` repetitions each. */
 long long msnhnet_profile_each_op(msnhnet_t net, int reps, char *dst, long long cap);
 float msnhnet_gpu_inference_time(msnhnet_t net);          /* NetBuilder::getGpuInferenceTime, ms */

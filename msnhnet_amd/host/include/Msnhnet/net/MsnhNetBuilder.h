@@ -101,8 +101,9 @@ public:
     double getConvFlops() const;              // 2*MACs of all conv/connected launches of one forward (whole batch)
     // Times `reps` eager passes over the live ops of one kind (PlanOp::Kind, or -1 for all) with device events on
     // the builder's stream; returns the total milliseconds and the number of launches timed.  The ops run on
-    // whatever the buffers currently hold, so this is a timing tool, not a forward.
-    float profileOps(int kind, int reps, int *launches, double *flops);
+    // whatever the buffers currently hold, so this is a timing tool, not a forward.  kind 1000 + a: the convolution launches of
+    // algorithm a (MSNH_CONV_*).  bytes (optional): what those launches must move at least (input + output + residual + weights).
+    float profileOps(int kind, int reps, int *launches, double *flops, double *bytes = nullptr);
     // One line per live op: layer, kind, shapes, algorithm, microseconds per launch (mean of `reps`), TFLOP/s, GB/s.
     std::string profileEachOp(int reps);
 

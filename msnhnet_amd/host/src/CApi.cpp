@@ -415,6 +415,14 @@ int msnhnet_profile_ops(msnhnet_t net, int kind, int reps, float *ms_total, int 
     });
 }
 
+int msnhnet_profile_ops_bytes(msnhnet_t net, int kind, int reps, float *ms_total, int *launches, double *flops, double *bytes)
+{
+    return guarded([&] {
+        if (reps <= 0 || !ms_total) MSNH_THROW("bad argument");
+        *ms_total = nb(net).profileOps(kind, reps, launches, flops, bytes);
+    });
+}
+
 long long msnhnet_profile_each_op(msnhnet_t net, int reps, char *dst, long long cap)
 {
     static thread_local std::string cache;

@@ -776,7 +776,16 @@ void NetBuilder::setSaveLayerOutput(bool v)
     if (_planReady) finalizePlan();
 }
 
-float NetBuilder::profileOps(int kind, int reps, int *launches, double *flops)
+static double opBytes(const Plan &plan, const PlanOp &op)
+{
+    // what the launch must move at least: its input, its output, a fused residual, its weights
+    const PlanTensor &in = plan.tensors[static_cast<size_t>(op.in0)];
+    const PlanTensor &out = plan.tensors[static_cast<size_t>(op.out)];
+    const double oe = static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4);
+    return static_cast<double>(in.elems()) * (in.dtype == MSNH_F16 ? 2 : 4) + oe + (op.in1 >= 0 ? oe : 0.0) + static_cast<double>(op.wDev.bytes());
+}
+
+float NetBuilder::profileOps(int kind, int reps, int *launches, double *flops, double *bytes)
 {
     if (!_planReady) MSNH_THROW("weights are not loaded");
     Plan &plan = *_net->plan;
@@ -784,16 +793,19 @@ float NetBuilder::profileOps(int kind, int reps, int *launches, double *flops)
     MSNH_DEV(msnh_hip_event_create(&e0));
     MSNH_DEV(msnh_hip_event_create(&e1));
     int n = 0;
-    double f = 0;
+    double f = 0, by = 0;
     MSNH_DEV(msnh_hip_event_record(e0, _stream));
     for (int r = 0; r < reps; ++r)
         for (size_t i = 0; i < plan.ops.size(); ++i)
         {
             const PlanOp &op = plan.ops[i];
-            if (op.dead || (kind >= 0 && static_cast<int>(op.kind) != kind)) continue;
+            // kind: a PlanOp::Kind, -1 for every launch, or 1000 + a convolution algorithm (MSNH_CONV_*)
+            if (op.dead) continue;
+            if (kind >= 1000 ? (op.kind != PlanOp::CONV || op.algo != kind - 1000) : (kind >= 0 && static_cast<int>(op.kind) != kind)) continue;
             plan.run(i, i + 1, _stream);
             ++n;
             f += op.flops;
+            by += opBytes(plan, op);
         }
     MSNH_DEV(msnh_hip_event_record(e1, _stream));
     MSNH_DEV(msnh_hip_event_sync(e1));
@@ -803,6 +815,7 @@ float NetBuilder::profileOps(int kind, int reps, int *launches, double *flops)
     msnh_hip_event_destroy(e1);
     if (launches) *launches = n;
     if (flops) *flops = f;
+    if (bytes) *bytes = by;
     return ms;
 }
 

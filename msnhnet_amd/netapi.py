@@ -18,7 +18,7 @@ SYMBOLS = [
     "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops", "msnhnet_weight_layout", "msnhnet_fp16_headroom",
     "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
     "msnhnet_enqueue", "msnhnet_sync", "msnhnet_fetch_classify", "msnhnet_fetch_yolo", "msnhnet_gpu_inference_time", "msnhnet_time_detail",
-    "msnhnet_profile_ops", "msnhnet_profile_each_op", "msnhnet_yolo_max_boxes", "msnhnet_nms",
+    "msnhnet_profile_ops", "msnhnet_profile_ops_bytes", "msnhnet_profile_each_op", "msnhnet_yolo_max_boxes", "msnhnet_nms",
 ]
 
 LAYER_TYPE = {0: "conv", 1: "deconv", 2: "connect", 3: "maxpool", 4: "localavgpool", 5: "globalavgpool", 6: "softmax", 8: "route", 9: "varop",
@@ -103,6 +103,7 @@ def lib():
     L.msnhnet_fetch_classify.argtypes = [vp, fp, ll, llp]
     L.msnhnet_fetch_yolo.argtypes = [vp, ip, fp, ll, llp]
     L.msnhnet_profile_ops.argtypes = [vp, ci, ci, fp, ip, ctypes.POINTER(ctypes.c_double)]
+    L.msnhnet_profile_ops_bytes.argtypes = [vp, ci, ci, fp, ip, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     L.msnhnet_profile_each_op.argtypes = [vp, ci, cp, ll]
     L.msnhnet_profile_each_op.restype = ll
     L.msnhnet_nms.argtypes = [fp, ll, ctypes.c_float, ci, fp, ll, llp]
@@ -345,6 +346,12 @@ class Net:
         ms, n, f = ctypes.c_float(), ctypes.c_int(), ctypes.c_double()
         _check(self.L.msnhnet_profile_ops(self.h, kind, reps, ctypes.byref(ms), ctypes.byref(n), ctypes.byref(f)))
         return ms.value, n.value, f.value
+
+    def profile_ops_bytes(self, kind, reps):
+        """-> (total ms, launches, algorithmic FLOPs, least bytes moved); kind as profile_ops, or 1000 + a convolution algorithm"""
+        ms, n, f, b = ctypes.c_float(), ctypes.c_int(), ctypes.c_double(), ctypes.c_double()
+        _check(self.L.msnhnet_profile_ops_bytes(self.h, kind, reps, ctypes.byref(ms), ctypes.byref(n), ctypes.byref(f), ctypes.byref(b)))
+        return ms.value, n.value, f.value, b.value
 
     def profile_each_op(self, reps=20):
         n = self.L.msnhnet_profile_each_op(self.h, reps, None, 0)
