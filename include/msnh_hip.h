@@ -59,9 +59,11 @@ enum msnh_conv_algo
     MSNH_CONV_POINTWISE = 7,   /* 1x1 stride 1, float16, in_c and out_c <= 128 and multiples of 8: weights resident in LDS, pixels
                                   straight from memory into MFMA fragments, no tiles (tile must be 0).  IGEMM weight packing.
                                   Never chosen by AUTO. */
-    MSNH_CONV_IGEMM_SPLITK = 6 /* IGEMM with the K loop cut into up to 8 slices on separate workgroups, float32 partial sums in
+    MSNH_CONV_IGEMM_SPLITK = 6,/* IGEMM with the K loop cut into up to 8 slices on separate workgroups, float32 partial sums in
                                   the workspace summed in slice order (deterministic); for launches with few output tiles.
                                   Same weight packing as IGEMM.  Never chosen by AUTO. */
+    MSNH_CONV_STEM_DOWN = 8    /* not an algorithm of msnh_hip_conv2d: the label of a launch of msnh_hip_conv_stem_down (first layer
+                                  and first stride-2 layer as one), so that plans and timing tables can name it */
 };
 
 /* ------------------------------------------------------------------------------------------------
@@ -160,6 +162,20 @@ size_t msnh_hip_conv2d_workspace_bytes(const msnh_conv_desc *d, int algo);
  * residual: NHWC d->dtype with pixel stride res_ld, or NULL; y: NHWC d->out_dtype with pixel stride out_ld. */
 int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
                     const void *residual, void *y, void *workspace, size_t workspace_bytes, msnh_stream_t s);
+
+/* The first two convolutions of the Darknet-53 / CSPDarknet-53 trunks as one launch, float16: a 3x3 stride-1 pad-1 convolution with 32
+ * filters over the 3-channel NCHW float32 network input, then a 3x3 stride-2 pad-1 convolution with c2 = 32 / 64 / 128 filters
+ * (two ConvolutionalLayer::forwardGPU calls, src/layers/MsnhConvolutionalLayer.cpp:984-1169, with the full-resolution 32-channel tensor
+ * in device memory between them; here it stays in LDS).  y = out_mul * act2(scale2 * conv2(mid) + shift2) with
+ * mid = float16(mid_mul * act1(scale1 * conv1(x) + shift1)); scale2 must undo mid_mul.  y: NHWC float16 [batch][(h+1)/2][(w+1)/2] with pixel
+ * stride y_ld.  w1: [32][3][3][3], w2: [c2][32][3][3] float32 in `.msnhbin` order, packed by msnh_hip_conv_stem_down_pack into
+ * msnh_hip_conv_stem_down_packed_elems(c2, 0 | 1) float16 elements each (upload them afterwards).  _supported: pure host function. */
+int msnh_hip_conv_stem_down_supported(int in_c, int c1, int k1, int s1, int p1, int c2, int k2, int s2, int p2);
+size_t msnh_hip_conv_stem_down_packed_elems(int c2, int which);
+int msnh_hip_conv_stem_down_pack(const float *w1, int c2, const float *w2, void *packed1, void *packed2);
+int msnh_hip_conv_stem_down(int batch, int h, int w, const float *x, const void *packed1, const float *scale1, const float *shift1, int act1,
+                            float act1_param, float mid_mul, int c2, const void *packed2, const float *scale2, const float *shift2, int act2,
+                            float act2_param, float out_mul, void *y, int y_ld, msnh_stream_t s);
 
 /* ------------------------------------------------------------------------------------------------
  * Element-wise / bandwidth-bound layers (all NHWC, any ld).

@@ -73,6 +73,7 @@ struct PlanOp
     int  tile = 0;                          // CONV/IGEMM: tile configuration chosen by Plan::tuneConvs (0 = library default)
     BaseLayer *src = nullptr;               // layer that owns the host weights of this op
     BaseLayer *src2 = nullptr;              // batch-norm layer folded into a CONV
+    int  stemOp = -1;                       // CONV 3x3 stride 2: the (dead) first-layer op computed in front of it by the same launch (Plan::fuse c)
 
     // YOLO_DECODE
     std::array<float, 6> anchors{};
@@ -83,6 +84,7 @@ struct PlanOp
 
     // device-side constants, filled by Plan::prepareWeights
     DeviceBuffer wDev, scaleDev, shiftDev;
+    DeviceBuffer wDev2, scaleDev2, shiftDev2;   // stemOp >= 0: the first layer's
     double flops = 0;                       // 2*MACs of this launch (conv / connected)
 };
 
@@ -94,6 +96,7 @@ public:
     int computeDtype;
     bool sparseYolo = false;                // yolo heads decode only the rows of their candidates (nobody reads the full decoded tensors)
     bool yoloKeepDecoded = true;            // sparseYolo: also write the candidates' full decoded rows (only YoloBox::classesVal needs them)
+    bool fuseStemDown = true;               // float16: first layer + first stride-2 layer as one launch where msnh_hip_conv_stem_down takes the pair
     bool preferWinograd = false;            // 3x3 stride-1 float16 convs take the Winograd path where the kernel accepts the shape
     std::vector<PlanTensor> tensors;
     std::vector<PlanOp>     ops;

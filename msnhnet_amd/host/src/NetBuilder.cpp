@@ -396,6 +396,7 @@ void NetBuilder::finalizePlan()
     Clock::time_point t0 = Clock::now();
     const int dtype = BaseLayer::useFp16 ? MSNH_F16 : MSNH_F32;
     std::unique_ptr<Plan> plan = lowerNetwork(dtype);
+    plan->fuseStemDown = std::getenv("MSNH_NO_STEM_DOWN") == nullptr;
     plan->fuse();
     plan->chainMaxPools();
     plan->aliasConcats();
@@ -824,7 +825,7 @@ std::string NetBuilder::profileEachOp(int reps)
     if (!_planReady) MSNH_THROW("weights are not loaded");
     Plan &plan = *_net->plan;
     static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode", "pad", "slice", "bilinear", "softmax", "col2im"};
-    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk", "pointwise"};
+    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk", "pointwise", "stem+down"};
     msnh_event_t e0 = nullptr, e1 = nullptr;
     MSNH_DEV(msnh_hip_event_create(&e0));
     MSNH_DEV(msnh_hip_event_create(&e1));

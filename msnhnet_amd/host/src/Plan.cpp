@@ -187,6 +187,32 @@ void Plan::fuse()
             break;
         }
     }
+    // (c) float16: first layer (3x3 stride 1, 32 filters, over the NCHW network input) -> 3x3 stride-2 convolution that is its only
+    // consumer: one launch; the full-resolution 32-channel tensor between them stays on the chip (it keeps its place in the tensor
+    // list: its calibrated scale is the scale of the values in LDS)
+    if (computeDtype == MSNH_F16 && fuseStemDown)
+        for (size_t i = 0; i < ops.size(); ++i)
+        {
+            PlanOp &first = ops[i];
+            if (first.dead || first.kind != PlanOp::CONV || first.in1 >= 0 || first.groups != 1 || first.dilation != 1) continue;
+            const PlanTensor &in = tensors[static_cast<size_t>(first.in0)];
+            const PlanTensor &mid = tensors[static_cast<size_t>(first.out)];
+            if (in.layout != PlanTensor::NCHW_INPUT || mid.pinned || mid.persistent || mid.parent >= 0 || mid.dtype != MSNH_F16 || consumerCount(first.out) != 1) continue;
+            for (size_t k = i + 1; k < ops.size(); ++k)
+            {
+                PlanOp &down = ops[k];
+                if (down.dead || down.in0 != first.out) continue;
+                const PlanTensor &out = tensors[static_cast<size_t>(down.out)];
+                if (down.kind == PlanOp::CONV && down.in1 < 0 && down.groups == 1 && down.dilation == 1 && out.dtype == MSNH_F16 && out.layout == PlanTensor::NHWC &&
+                    msnh_hip_conv_stem_down_supported(in.c, mid.c, first.ksize, first.stride, first.pad, out.c, down.ksize, down.stride, down.pad))
+                {
+                    down.stemOp = static_cast<int>(i);
+                    down.in0 = first.in0;
+                    first.dead = true;
+                }
+                break;
+            }
+        }
 }
 
 // ---- pass 1b: stride-1 max-pools over one tensor (SPP blocks: 5, 9, 13) ---------------------------------------------
@@ -342,7 +368,7 @@ uint64_t Plan::structureHash() const
     for (const PlanOp &op : ops)
         os << static_cast<int>(op.kind) << ' ' << op.in0 << ' ' << op.in1 << ' ' << op.out << ' ' << op.dead << ' ' << op.layerIndex << ' ' << op.ksize << ' ' << op.stride << ' '
            << op.pad << ' ' << op.dilation << ' ' << op.groups << ' ' << static_cast<int>(op.act) << ' ' << static_cast<int>(op.act2) << ' ' << op.in1Sign << ' ' << (op.src2 != nullptr)
-           << ' ' << op.dstChanOffset << ';';
+           << ' ' << op.dstChanOffset << ' ' << op.stemOp << ';';
     const std::string text = os.str();
     return PackFile::hash(text.data(), text.size());
 }
@@ -479,6 +505,45 @@ void Plan::prepareWeights(PackFile *from, PackFile *to)
     {
         PlanOp &op = ops[opIndex];
         if (op.dead) continue;
+        if (op.kind == PlanOp::CONV && op.stemOp >= 0)
+        {
+            // the fused pair: both kernels packed into MFMA lane order, both batch-norms folded; the second layer's scale undoes the
+            // power-of-two scale of the values the first layer leaves in LDS
+            const PlanOp &first = ops[static_cast<size_t>(op.stemOp)];
+            const PlanTensor &mid = tensors[static_cast<size_t>(first.out)];
+            const PlanTensor &out = tensors[static_cast<size_t>(op.out)];
+            const std::vector<float> &w1 = first.src->kernelWeights(), &w2 = op.src->kernelWeights();
+            if (w1.size() != static_cast<size_t>(mid.c) * 27 || w2.size() != static_cast<size_t>(out.c) * mid.c * 9) MSNH_THROW("conv weights are not loaded (" + op.name + ")");
+            std::vector<uint16_t> p1(msnh_hip_conv_stem_down_packed_elems(out.c, 0)), p2(msnh_hip_conv_stem_down_packed_elems(out.c, 1));
+            MSNH_DEV(msnh_hip_conv_stem_down_pack(w1.data(), out.c, w2.data(), p1.data(), p2.data()));
+            op.wDev2.upload(p1.data(), p1.size() * 2);
+            op.wDev.upload(p2.data(), p2.size() * 2);
+            const auto affine = [&](const PlanOp &o, int channels, float inMul, DeviceBuffer &scaleDev, DeviceBuffer &shiftDev) {
+                std::vector<float> scale, shift;
+                o.src->foldedAffine(scale, shift);
+                if (o.src2)
+                {
+                    std::vector<float> s2, h2;
+                    o.src2->foldedAffine(s2, h2);
+                    if (scale.empty()) scale.assign(static_cast<size_t>(channels), 1.f);
+                    if (shift.empty()) shift.assign(static_cast<size_t>(channels), 0.f);
+                    for (size_t c = 0; c < static_cast<size_t>(channels); ++c) { scale[c] = s2[c] * scale[c]; shift[c] = s2[c] * shift[c] + h2[c]; }
+                }
+                if (inMul != 1.f)
+                {
+                    if (scale.empty()) scale.assign(static_cast<size_t>(channels), 1.f);
+                    for (float &v : scale) v *= inMul;
+                }
+                if (!scale.empty()) scaleDev.upload(scale.data(), scale.size() * sizeof(float));
+                if (!shift.empty()) shiftDev.upload(shift.data(), shift.size() * sizeof(float));
+            };
+            affine(first, mid.c, 1.f, op.scaleDev2, op.shiftDev2);
+            affine(op, out.c, mulOf(first.out), op.scaleDev, op.shiftDev);
+            op.algo = MSNH_CONV_STEM_DOWN;
+            const PlanTensor &img = tensors[static_cast<size_t>(op.in0)];
+            op.flops = 2.0 * img.n * (static_cast<double>(mid.c) * mid.h * mid.w * img.c * 9 + static_cast<double>(out.c) * out.h * out.w * mid.c * 9);
+            continue;
+        }
         if (op.kind == PlanOp::CONV)
         {
             const PlanTensor &in = tensors[static_cast<size_t>(op.in0)];
@@ -843,6 +908,14 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
     {
     case PlanOp::CONV:
     {
+        if (op.stemOp >= 0)
+        {
+            const PlanOp &first = ops[static_cast<size_t>(op.stemOp)];
+            MSNH_DEV(msnh_hip_conv_stem_down(in.n, in.h, in.w, static_cast<const float *>(ptr(op.in0)), op.wDev2.ptr(), op.scaleDev2.as<float>(), op.shiftDev2.as<float>(),
+                                             static_cast<int>(first.act), first.actParam, 1.f / mulOf(first.out), out.c, op.wDev.ptr(), op.scaleDev.as<float>(),
+                                             op.shiftDev.as<float>(), static_cast<int>(op.act), op.actParam, 1.f / mulOf(op.out), ptr(op.out), ld(op.out), s));
+            break;
+        }
         const msnh_conv_desc d = convDesc(*this, op);
         if (op.wDev.bytes() != msnh_hip_conv2d_packed_weight_elems(&d, op.algo) * (d.dtype == MSNH_F16 ? 2u : 4u))
             MSNH_THROW("conv weights on the device are not packed for the algorithm of this launch (" + op.name + ")");
@@ -958,7 +1031,7 @@ void Plan::exportTensor(int t, std::vector<float> &dst, msnh_stream_t s)
 std::string Plan::describe() const
 {
     static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode", "pad", "slice", "bilinear", "softmax", "col2im"};
-    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk", "pointwise"};
+    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk", "pointwise", "stem+down"};
     std::ostringstream os;
     os << "plan: " << liveOps() << " launches, " << tensors.size() << " tensors, arena " << _arena.bytes() / (1024.0 * 1024.0) << " MiB, dtype "
        << (computeDtype == MSNH_F16 ? "f16" : "f32") << "\n";

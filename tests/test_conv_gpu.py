@@ -2,6 +2,8 @@
 
 Tolerances: float32 1e-5 of max|ref| (only the accumulation order differs); float16 2e-3 of max|ref| with the
 oracle fed the same float16-rounded inputs and weights (accumulation is float32, the output is rounded once)."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -378,3 +380,47 @@ def test_conv_rejects_bad_shapes():
     assert b"IGEMM" in L.msnh_hip_last_error()
     d = abi.ConvDesc(abi.F16, abi.F16, 1, 8, 8, 16, 16, 16, 9, 8, 16, 3, 1, 1, 1, 1, 22, 0.1, 0, 16, 22, 0.1, 1.0, 1.0, 0, 0)
     assert L.msnh_hip_conv2d(ctypes.byref(d), 16, 16, None, None, None, 16, None, 0, None) != 0      # wrong out_h
+
+
+@pytest.mark.parametrize("b,h,w,c2,act", [(2, 32, 64, 64, "leaky"), (1, 37, 45, 32, "mish"), (3, 16, 16, 128, "relu"), (1, 608, 608, 64, "leaky")])
+def test_conv_stem_down(b, h, w, c2, act):
+    """first layer (3x3 stride 1, 32 filters, NCHW float32 in) + 3x3 stride-2 layer as one launch: equal to the two layers run one
+    after the other with the intermediate rounded to float16 (odd sizes exercise ragged tiles and the zero padding of the
+    intermediate at all four borders; mid_mul / out_mul are the power-of-two scales of a float16 plan)"""
+    import torch
+
+    import gpuutil as gu
+    gu.init()
+    L = abi.lib()
+    rng = np.random.default_rng(b * 1000 + h + c2)
+    x = rng.random((b, 3, h, w), dtype=np.float32)
+    w1 = rng.standard_normal((32, 3, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / 27))
+    w2 = rng.standard_normal((c2, 32, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / 288))
+    s1, h1 = rng.uniform(0.5, 1.5, 32).astype(np.float32), (rng.standard_normal(32) * 0.1).astype(np.float32)
+    s2, h2 = rng.uniform(0.5, 1.5, c2).astype(np.float32), (rng.standard_normal(c2) * 0.1).astype(np.float32)
+    mid_mul, out_mul = 0.25, 2.0
+    assert L.msnh_hip_conv_stem_down_supported(3, 32, 3, 1, 1, c2, 3, 2, 1) == 1
+    assert L.msnh_hip_conv_stem_down_supported(3, 64, 3, 1, 1, c2, 3, 2, 1) == 0 and L.msnh_hip_conv_stem_down_supported(3, 32, 3, 1, 1, 96, 3, 2, 1) == 0
+    p1 = np.zeros(L.msnh_hip_conv_stem_down_packed_elems(c2, 0), np.float16)
+    p2 = np.zeros(L.msnh_hip_conv_stem_down_packed_elems(c2, 1), np.float16)
+    abi.check(L.msnh_hip_conv_stem_down_pack(w1.ctypes.data_as(ctypes.c_void_p), c2, w2.ctypes.data_as(ctypes.c_void_p), p1.ctypes.data_as(ctypes.c_void_p),
+                                             p2.ctypes.data_as(ctypes.c_void_p)))
+    oh, ow = (h - 1) // 2 + 1, (w - 1) // 2 + 1
+    ld = c2 + 8
+    xd, p1d, p2d = gu.dev(x), gu.dev(p1), gu.dev(p2)
+    s1d, h1d, s2d, h2d = gu.dev(s1), gu.dev(h1), gu.dev(s2 / np.float32(mid_mul)), gu.dev(h2)
+    yd = torch.full((b, oh, ow, ld), 3.0, dtype=torch.float16).cuda()
+    gu.sync()
+    print("conv_stem_down", b, h, w, c2, act, flush=True)
+    abi.check(L.msnh_hip_conv_stem_down(b, h, w, gu.ptr(xd), gu.ptr(p1d), gu.ptr(s1d), gu.ptr(h1d), abi.ACT[act], 0.1, mid_mul, c2, gu.ptr(p2d), gu.ptr(s2d),
+                                        gu.ptr(h2d), abi.ACT[act], 0.1, out_mul, gu.ptr(yd), ld, None))
+    gu.sync()
+    got = gu.nchw_host(yd, c2)
+    assert (yd[..., c2:].float().cpu().numpy() == 3.0).all(), "kernel wrote outside its channel slice"
+    # the same in two steps: image and weights rounded to float16 as the matrix cores see them, the intermediate stored as
+    # float16(mid_mul * value) and multiplied back by the second layer's scale
+    mid = _ref(gu.round_f16(x), gu.round_f16(w1), 1, 1, 1, 1, s1, h1, act, 0.1, None, "none", 1.0, mid_mul)
+    mid = gu.round_f16(mid)
+    ref = _ref(mid, gu.round_f16(w2), 2, 1, 1, 1, s2 / np.float32(mid_mul), h2, act, 0.1, None, "none", 1.0, out_mul)
+    assert got.shape == ref.shape
+    assert gu.rel_err(got, ref) <= 2e-3
