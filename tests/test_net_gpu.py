@@ -321,6 +321,26 @@ def test_tune_cache(tmp_path):
         netapi.set_tune_cache(False)
 
 
+def test_first_pair_runs_as_one_launch():
+    """float16 plans of the Darknet trunks run the first layer and the first stride-2 layer as one launch (the full-resolution tensor
+    between them stays on the chip); float32 plans, layer-dump runs and networks that open differently keep their own launches; the
+    results are those of the layer-by-layer run to float16 accuracy"""
+    size, batch = 160, 2
+    net, binp, g = nu.model("yolov3", batch, size, seed=3)
+    x = zoo.seeded_input(batch, 3, size, size, seed=4)
+    fused = netapi.Net(net, binp, fp16=True)
+    assert "stem+down" in fused.plan_detail() and "conv[stem " not in fused.plan_detail()
+    assert "stem+down" not in netapi.Net(net, binp, fp16=False).plan_detail()
+    slow = netapi.Net(net, binp, fp16=True, dump_layers=True)
+    assert "stem+down" not in slow.plan_detail() and "conv[stem " in slow.plan_detail()
+    a, b = fused.run_yolo(x), slow.run_yolo(x)
+    for i in range(batch):
+        assert abs(len(a[i]) - len(b[i])) <= max(2, 0.02 * len(b[i]))
+        assert nu.boxes_matched_fraction(a[i], b[i], 2e-2) >= 0.95
+    r50, rbin, _ = nu.model("resnet50", 2, 224, seed=3)
+    assert "stem+down" not in netapi.Net(r50, rbin, fp16=True).plan_detail()
+
+
 def test_weight_cache(tmp_path):
     """the packed kernels and the float16 calibration are kept beside the weights file when asked for: the next load of the same
     weights into the same graph takes them from the file (same plan, bit-identical outputs, no calibration pass); other weights under
