@@ -118,10 +118,15 @@ def conv_shape_mode(a):
         d.tile = a.tile
         if not L.msnh_hip_conv2d_tile_supported(ctypes.byref(d), a.tile):
             sys.exit(f"tile {a.tile} does not take this shape")
+        import time
+        run()
+        abi.check(L.msnh_hip_stream_sync(None))
+        t0 = time.perf_counter()
         for _ in range(a.reps):
             run()
         abi.check(L.msnh_hip_stream_sync(None))
-        print(f"tile {a.tile}: {a.reps} launches of {a.conv_shape}")
+        us = (time.perf_counter() - t0) / a.reps * 1e6
+        print(f"tile {a.tile}: {a.reps} launches of {a.conv_shape}, {us:.2f} us per launch back to back (host clock)")
         return
     e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
     abi.check(L.msnh_hip_event_create(ctypes.byref(e0)))
