@@ -237,6 +237,8 @@ def main():
                 net.set_input_image_u8(i, host_u8[i])
         net.enqueue(None)
 
+    on_device = [0]
+
     def run_steps(k, stamps=None, host=None):
         """k forwards + k result fetches.  Detection keeps two batches in flight: while the host sorts and
         suppresses the boxes of batch i the device already runs batch i+1.  stamps collects the time at which each
@@ -253,8 +255,10 @@ def main():
                 feed()
                 out = net.fetch_yolo()
                 tick()
+                on_device[0] += net.last_nms_on_device()
             out = net.fetch_yolo()
             tick()
+            on_device[0] += net.last_nms_on_device()
         else:
             for _ in range(k):
                 feed()
@@ -271,6 +275,7 @@ def main():
     marker()
     torch.cuda.synchronize()
     stamps = []
+    on_device[0] = 0
     import gc
     gc.collect()
     gc.disable()          # a collection in the middle of the host stage would be timed as a step of several milliseconds
@@ -279,6 +284,7 @@ def main():
     net.sync()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    steps_on_device = on_device[0]
     gc.enable()
     slow = [i for i, v in enumerate(np.diff(np.array([t0] + stamps)) * 1e3) if v > 5.0]
     marker()
@@ -338,6 +344,7 @@ def main():
     if detect:
         res["config"]["boxes_per_image"] = [int(len(b)) for b in out]
         res["config"]["nms"] = a.nms
+        res["config"]["steps_with_nms_on_device"] = steps_on_device
     if a.per_op:
         with open(a.per_op, "w") as f:
             f.write(net.profile_each_op(20))

@@ -83,7 +83,8 @@ int msnhnet_create(msnhnet_t *net);                       /* NetBuilder() */
 int msnhnet_destroy(msnhnet_t net);
 int msnhnet_set_use_fp16(int on);                         /* NetBuilder::setUseFp16, process-wide, before build */
 int msnhnet_set_device_nms(int mode);                     /* hard NMS: 0 = candidates copied back, sort + NMS on the host; 2 = on the device, only kept boxes cross
-                                                              PCIe; 1 (default) = on the device while the previous result had <= 2048 candidates per image */
+                                                              PCIe; 1 (default) = chosen per batch from the previous result: on the device up to 2048 candidates per
+                                                              image, and up to 6144 unless forwards are pipelined and the host keeps up with them */
 int msnhnet_set_tune_cache(int on);                       /* keep the per-layer tile search result in "<weights>.f16.tune" / ".f32.tune" next to the
                                                               .msnhbin file and reuse it on the next load (same graph, same device); off by default */
 int msnhnet_set_weight_cache(int on);                     /* keep the packed device-side kernels and the float16 calibration in "<weights>.f16.pack" /
@@ -116,6 +117,8 @@ int msnhnet_run_classify_gpu(msnhnet_t net, const float *img, long long n, float
 /* NetBuilder::runYoloGPU: counts[b] = boxes of image b; boxes = rows of 7 floats (x y w h conf bestClsConf
  * bestClsIdx), images back to back, at most cap_boxes rows are written; *total = sum of counts. */
 int msnhnet_run_yolo_gpu(msnhnet_t net, const float *img, long long n, int *counts, float *boxes, long long cap_boxes, long long *total);
+/* Where the hard NMS of the detection result fetched last ran: 1 on the device, 0 on the host (msnhnet_set_device_nms). */
+int msnhnet_last_nms_on_device(msnhnet_t net, int *on_device);
 /* Range check of a float16 plan for one input (NetBuilder::fp16Headroom): runs the network once on img and writes the factor by which
  * img could still grow before a float16 activation overflows; 0 means it already did (an input far hotter than the [0,1) image the
  * scales were calibrated on).  float32 plans report infinity. */

@@ -628,6 +628,11 @@ __global__ __launch_bounds__(256) void yoloNmsPairKernel(const unsigned long lon
             c = *reinterpret_cast<const float4 *>(q);
             a = q[4];
         };
+        // A pair whose boxes are more than a unit apart in x or y has no intersection (inter = 0, never above a threshold >= 0): most
+        // pairs of a real image, decided with four comparisons.  The margin of 2 instead of the "+ 1" of the extents keeps the skip
+        // on the safe side of any rounding; NaN or infinite corners never skip (every comparison with them is false).
+        const float kx2p = k4.z + 2.f, ky2p = k4.w + 2.f;
+        const bool skipOk = thr >= 0.f;
         float4 vcNext;
         float vaNext;
         victim(w0, vcNext, vaNext);
@@ -636,17 +641,23 @@ __global__ __launch_bounds__(256) void yoloNmsPairKernel(const unsigned long lon
             const float4 vc = vcNext;
             const float va = vaNext;
             if (w + 1 < w1) victim(w + 1, vcNext, vaNext);
+            const float vx2p = vc.z + 2.f, vy2p = vc.w + 2.f;
             unsigned long long word = 0ull, col = 0ull;
             const int jEnd = m - w * 64 < 64 ? m - w * 64 : 64;
             for (int j = 0; j < jEnd; ++j)
             {
                 const float c0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(vc.x), j));
                 const float c1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(vc.y), j));
+                const float c2p = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(vx2p), j));
+                const float c3p = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(vy2p), j));
+                const bool apart = skipOk && (c0 > kx2p || k4.x > c2p || c1 > ky2p || k4.y > c3p);
+                const bool later = w * 64 + j > i, earlier = w == rc && j < lane;
+                if (!__any(!apart && (later || earlier))) continue;
                 const float c2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(vc.z), j));
                 const float c3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(vc.w), j));
                 const float c4 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(va), j));
-                if (w * 64 + j > i && iouAbove(k4.x, k4.y, k4.z, k4.w, ka, c0, c1, c2, c3, c4, thr)) word |= 1ull << j;
-                if (w == rc && j < lane && iouAbove(c0, c1, c2, c3, c4, k4.x, k4.y, k4.z, k4.w, ka, thr)) col |= 1ull << j;
+                if (later && !apart && iouAbove(k4.x, k4.y, k4.z, k4.w, ka, c0, c1, c2, c3, c4, thr)) word |= 1ull << j;
+                if (earlier && !apart && iouAbove(c0, c1, c2, c3, c4, k4.x, k4.y, k4.z, k4.w, ka, thr)) col |= 1ull << j;
             }
             if (i < m) pool[at + static_cast<unsigned long long>(i) * W + w] = word;
             if (w == rc) pool[at + static_cast<unsigned long long>(m) * W + static_cast<unsigned long long>(i)] = i < m ? col : 0ull;

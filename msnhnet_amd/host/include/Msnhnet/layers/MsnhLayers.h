@@ -358,10 +358,13 @@ public:
     std::vector<bool> batchHasBox;
     std::vector<std::vector<YoloBox>> finalOut;
     static bool keepClassScores;           // also fill YoloBox::classesVal (costs an extra device->host copy)
+    bool lastOnDevice = false;             // where the NMS of the result fetched last ran
     // hard NMS on the device (only the kept boxes are copied back): 0 = never (sort + NMS on the host), 2 = always,
-    // 1 = while the previous result of this network had at most kDeviceNmsCandidates candidates in every image (default): that is
-    // the largest class the device kernels take (msnh_hip_yolo_nms), so no image of such a batch can fall back to the host.
+    // 1 (default) = chosen per batch from the previous result: up to kDeviceNmsFew candidates per image on the device; up to
+    // kDeviceNmsCandidates (the largest class the device kernels take) on the device as well, except while forwards are pipelined and
+    // the host stage keeps up with them -- the host then does it for free beside the next forward; more than that on the host.
     static int deviceNms;
+    static const int kDeviceNmsFew = 2048;
     static const int kDeviceNmsCandidates = 6144;
 
     // host post-processing of the compacted candidate rows of one image (8 floats per row, see msnh_hip_yolo_gather)
@@ -391,6 +394,8 @@ private:
     msnh_stream_t _copyStream = nullptr, _fetchStream = nullptr;
     int _lastMaxCandidates = 0;            // largest per-image candidate count of the previous result
     size_t _lastKept = 0;                  // records the device NMS kept for the previous batch
+    int _hostBoundRuns = 0;                // batches in a row for which the host path did not have to wait for the device
+    bool _hostBound = false;
     Slot _slots[2];
 };
 }

@@ -78,6 +78,7 @@ public:
     Point2I getInputSize();
     int getInputChannel();
     int getBatch() const;
+    bool lastNmsOnDevice() const;           // detection networks: where the NMS of the result fetched last ran (see YoloOutLayer::deviceNms)
     void clearLayers();
     float getInferenceTime();
     std::string getLayerDetail();

@@ -368,6 +368,14 @@ int msnhnet_run_yolo_gpu(msnhnet_t net, const float *img, long long n, int *coun
     });
 }
 
+int msnhnet_last_nms_on_device(msnhnet_t net, int *on_device)
+{
+    return guarded([&] {
+        if (!on_device) MSNH_THROW("bad argument");
+        *on_device = nb(net).lastNmsOnDevice() ? 1 : 0;
+    });
+}
+
 int msnhnet_fp16_headroom(msnhnet_t net, const float *img, long long n, float *headroom)
 {
     return guarded([&] {

@@ -1450,7 +1450,12 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
     MSNH_DEV(msnh_hip_event_record(sl.ready, s));
     MSNH_DEV(msnh_hip_stream_wait_event(_copyStream, sl.ready));
     MSNH_DEV(msnh_hip_memcpy_d2h(sl.cnt.ptr(), sl.devCnt.ptr(), cntBytes, _copyStream));
-    sl.onDevice = !_useSoftNms && (deviceNms == 2 || (deviceNms == 1 && _lastMaxCandidates <= kDeviceNmsCandidates));
+    // auto: few candidates (real detections) -> the device; thousands per image -> the device too unless a second forward is in flight
+    // (the host's sort + NMS then runs beside that forward and costs the device nothing, whereas the device NMS takes about 0.1 ms of
+    // device time per batch from it) and the host stage has kept up with the device so far
+    const bool pipelined = _slots[(slot ^ 1) & 1].pending;
+    const bool autoDevice = _lastMaxCandidates <= kDeviceNmsFew || (_lastMaxCandidates <= kDeviceNmsCandidates && (!pipelined || _hostBound));
+    sl.onDevice = !_useSoftNms && (deviceNms == 2 || (deviceNms == 1 && autoDevice));
     if (sl.onDevice)
     {
         // NMS on the snapshot, on the copy stream: it overlaps the next forward, and what crosses PCIe is the kept boxes.  The records
@@ -1523,6 +1528,7 @@ void YoloOutLayer::finish(int slot)
     MSNH_DEV(msnh_hip_event_sync(sl.event));
     const float dbgWait = TimeUtil::getElapsedTime(dbg0);
     sl.pending = false;
+    lastOnDevice = sl.onDevice;
     const int cells = plan->yoloCells;
     const int per = _channel;
     const int *cnt = sl.cnt.as<int>();
@@ -1629,6 +1635,14 @@ void YoloOutLayer::finish(int slot)
         }
     }
     for (int b = 0; b < _batch; ++b) batchHasBox[static_cast<size_t>(b)] = cnt[b] > 0;
+    {
+        // did the device make the host wait?  If it has not for eight batches in a row, the host stage is what bounds the pipeline, and
+        // the automatic mode moves the NMS to the device (until a batch with few candidates resets the question)
+        const double stage = TimeUtil::getElapsedTime(dbg0) - dbgWait;
+        if (_lastMaxCandidates <= kDeviceNmsFew) { _hostBoundRuns = 0; _hostBound = false; }
+        else if (dbgWait < 0.05 * stage) { if (++_hostBoundRuns >= 8) _hostBound = true; }
+        else _hostBoundRuns = 0;
+    }
     if (std::getenv("MSNH_DEBUG_TIMING"))
         std::fprintf(stderr, "yoloout finish: wait %.3f ms, host %.3f ms (candidates %.3f, suppression %.3f, output %.3f)\n", dbgWait,
                      TimeUtil::getElapsedTime(dbg0) - dbgWait, dbgA - dbgWait, dbgB - dbgA, TimeUtil::getElapsedTime(dbg0) - dbgB);

@@ -722,6 +722,11 @@ int NetBuilder::getInputChannel()
 }
 
 int NetBuilder::getBatch() const { return _net->batch; }
+bool NetBuilder::lastNmsOnDevice() const
+{
+    BaseLayer *last = _net->layers.empty() ? nullptr : _net->layers.back();
+    return last && last->type() == LayerType::YOLO_OUT && static_cast<YoloOutLayer *>(last)->lastOnDevice;
+}
 
 float NetBuilder::getInferenceTime()
 {

@@ -15,7 +15,7 @@ SYMBOLS = [
     "initMsnhnet", "buildMsnhnet", "runClassifyNoPred", "runYoloNoPred", "runClassifyList", "runYoloList", "dispose", "withGPU", "withCUDNN", "getCpuForwardTime",
     "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16", "msnhnet_set_use_winograd", "msnhnet_set_tune_cache", "msnhnet_set_weight_cache", "msnhnet_load_detail", "msnhnet_set_device_nms", "msnhnet_set_input_image_u8", "msnhnet_set_input_image", "msnhnet_boxes_to_image",
     "msnhnet_set_keep_class_scores", "msnhnet_set_save_layer_output", "msnhnet_build", "msnhnet_load", "msnhnet_load_from_memory",
-    "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops", "msnhnet_weight_layout", "msnhnet_fp16_headroom",
+    "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops", "msnhnet_weight_layout", "msnhnet_fp16_headroom", "msnhnet_last_nms_on_device",
     "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
     "msnhnet_enqueue", "msnhnet_sync", "msnhnet_fetch_classify", "msnhnet_fetch_yolo", "msnhnet_gpu_inference_time", "msnhnet_time_detail",
     "msnhnet_profile_ops", "msnhnet_profile_ops_bytes", "msnhnet_profile_each_op", "msnhnet_yolo_max_boxes", "msnhnet_nms",
@@ -91,6 +91,7 @@ def lib():
     L.msnhnet_weight_layout.argtypes = [vp, llp, ll]
     L.msnhnet_weight_layout.restype = ll
     L.msnhnet_fp16_headroom.argtypes = [vp, fp, ll, fp]
+    L.msnhnet_last_nms_on_device.argtypes = [vp, ip]
     L.msnhnet_conv_flops.restype = ctypes.c_double
     L.msnhnet_run_classify.argtypes = [vp, fp, ll, fp, ll, llp]
     L.msnhnet_run_classify_gpu.argtypes = [vp, fp, ll, fp, ll, llp]
@@ -196,6 +197,11 @@ class Net:
     def load_array(self, w):
         w = np.ascontiguousarray(w, np.float32)
         _check(self.L.msnhnet_load_from_memory(self.h, _fp(w), w.size))
+
+    def last_nms_on_device(self):
+        v = ctypes.c_int()
+        _check(self.L.msnhnet_last_nms_on_device(self.h, ctypes.byref(v)))
+        return bool(v.value)
 
     def fp16_headroom(self, x):
         """factor by which input x could grow before a float16 activation overflows (0: it did); see msnhnet_fp16_headroom"""

@@ -10,6 +10,7 @@ Tolerances (max|a-b| / max|ref| per layer output):
 """
 import numpy as np
 import pytest
+import torch
 
 import msnh_oracle_net as on
 import netutil as nu
@@ -446,6 +447,38 @@ def test_device_nms_equals_host_nms(arch, size, batch):
     for g_, w_ in zip(got, want):
         for b in range(batch):
             assert np.array_equal(g_[b], w_[b], equal_nan=True)
+
+
+def test_auto_nms_placement():
+    """the automatic mode: thousands of candidates per image go to the device for a caller that runs one forward at a time (shorter
+    latency) and to the host while forwards are pipelined and the host keeps up (no device time taken from the next forward); few
+    candidates always go to the device; the boxes are the same wherever they were suppressed"""
+    size, batch = 352, 2
+    net, binp, g = nu.model("yolov3", batch, size, seed=3)
+    x = zoo.seeded_input(batch, 3, size, size, seed=4)
+    xd = torch.from_numpy(x).cuda()
+    netapi.set_device_nms(1)
+    m = netapi.Net(net, binp, fp16=True)
+    first = m.run_yolo(x)                    # (nothing known about the candidate count yet)
+    n = max(len(b) for b in first)
+    assert 2048 < n <= 6144, n               # the regime this test is about (boxes <= candidates)
+    one = m.run_yolo(x)
+    assert m.last_nms_on_device()
+    m.enqueue(xd.data_ptr())
+    m.enqueue(xd.data_ptr())
+    a = m.fetch_yolo()
+    assert m.last_nms_on_device()            # (enqueued while nothing else was in flight)
+    m.enqueue(xd.data_ptr())
+    b = m.fetch_yolo()
+    assert not m.last_nms_on_device()        # enqueued beside another forward
+    c = m.fetch_yolo()
+    for i in range(batch):
+        for other in (a, b, c):
+            assert np.array_equal(one[i], other[i], equal_nan=True)
+    few = np.zeros_like(x)
+    m.run_yolo(few)
+    m.run_yolo(few)
+    assert m.last_nms_on_device()
 
 
 def test_yolo_rows_copied_in_part():
