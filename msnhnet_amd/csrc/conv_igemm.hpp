@@ -16,6 +16,7 @@
 // power-of-two output scale on the float32 accumulators and stores 8 consecutive channels per lane.
 #pragma once
 #include "common.hpp"
+#include <algorithm>
 #include <type_traits>
 
 namespace msnh {
@@ -329,6 +330,38 @@ __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[
     });
 }
 
+// Epilogue of the kernels whose wavefronts come in two groups that multiplied different k-blocks of the same 64 x 64 wave tile
+// (kg = group, wt = wave tile index): group g keeps pixel block g of the tile, parks the other block's partial sums in LDS for
+// its partner and adds what the partner parked for it; then the ordinary epilogue runs over 64 x 32 per wavefront.
+// LDS: 8 KiB per wavefront (igemmSwapLds).
+template <int NW> constexpr size_t igemmSwapLds() { return static_cast<size_t>(NW) * 2 * 16 * 64 * sizeof(float); }
+
+template <typename T, typename TOut, int BM, int BN>
+__device__ __forceinline__ void igemmEpilogueSwap(const IgemmArgs &a, f32x16 (&acc)[2][2], unsigned char *smemRaw, float chScale, float chShift,
+                                                  int m0, int p0, int wm, int wn, int kg, int wt, int wave, int lane, int g)
+{
+    constexpr int XW = 2 * 16 * 64;                   // floats a wavefront parks
+    float *xch = reinterpret_cast<float *>(smemRaw);
+    f32x16 mine[2][1];
+    auto swap = [&](auto gTag) {
+        constexpr int q = decltype(gTag)::value;
+        float *put = xch + (wt * 2 + q) * XW + lane;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) put[(i * 16 + r) * 64] = acc[i][1 - q][r];
+        __syncthreads();
+        const float *get = xch + (wt * 2 + (1 - q)) * XW + lane;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mine[i][0][r] = acc[i][q][r] + get[(i * 16 + r) * 64];
+    };
+    if (kg == 0) swap(std::integral_constant<int, 0>()); else swap(std::integral_constant<int, 1>());
+    __syncthreads();
+    igemmEpilogue<T, TOut, BM, BN, 64, 32>(a, mine, smemRaw, chScale, chShift, m0, p0, wm, wn * 2 + kg, wave, lane, g);
+}
+
 // Register budget: two workgroups per CU (one wave of each per SIMD) so that one workgroup's barrier and epilogue
 // are covered by the other's MFMAs; smaller tiles, which serve the short-K bandwidth-bound layers, get three to six.
 constexpr int igemmWavesPerSimd(int bm, int bn, int kv = 8, int ns = 3, int nw = 4)
@@ -369,15 +402,19 @@ __device__ __forceinline__ i32x4 makeRsrcWords(const void *base, unsigned bytes)
     return r;
 }
 
-template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int NS>
-__global__ __launch_bounds__(64 * WM * WN)
-__attribute__((amdgpu_waves_per_eu(igemmWavesPerSimd(BM, BN, KV, NS, WM * WN), igemmWavesPerSimd(BM, BN, KV, NS, WM * WN))))
+// KG = 2: two groups of wavefronts share the WM x WN grid of (then 64 x 64) wave tiles and split the k-blocks of every tile step
+// between them, which takes a third off the LDS fragment reads per MFMA against 32 x 64 wave tiles of the same workgroup tile.
+template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int NS, int KG = 1>
+__global__ __launch_bounds__(64 * WM * WN * KG)
+__attribute__((amdgpu_waves_per_eu(KG == 2 ? (WM * WN * KG) / 4 : igemmWavesPerSimd(BM, BN, KV, NS, WM * WN),
+                                   KG == 2 ? (WM * WN * KG == 4 ? 3 : (WM * WN * KG) / 4) : igemmWavesPerSimd(BM, BN, KV, NS, WM * WN))))
 void convIgemmKernel(IgemmArgs a)
 {
     typedef typename Frag<T>::V V;
     constexpr int VEC   = Frag<T>::VEC;
     constexpr int BK    = KV * VEC;               // K elements per tile step
-    constexpr int NT    = 64 * WM * WN;           // threads: 4, 8 or 12 wavefronts
+    constexpr int NWT   = WM * WN;                // wave tiles
+    constexpr int NT    = 64 * NWT * KG;          // threads: 4, 8 or 12 wavefronts
     constexpr int RPP   = NT / KV;                // rows loaded per pass of the workgroup
     constexpr int BML   = (BM + RPP - 1) / RPP * RPP; // A rows held in LDS: BM rounded up to whole passes (the surplus rows load nothing)
     constexpr int AROWS = BML / RPP;              // A rows (16-byte chunks) per thread per tile step
@@ -388,13 +425,14 @@ void convIgemmKernel(IgemmArgs a)
     constexpr int TN    = BN / WN;
     constexpr int MB    = TM / 32;
     constexpr int NB    = TN / 32;
-    constexpr int S     = KV / 2;                 // MFMA k-steps per tile step (one k-block = two 16-byte chunks)
+    constexpr int S     = KV / 2 / KG;            // MFMA k-steps per tile step and wavefront (one k-block = two 16-byte chunks)
     constexpr unsigned ES = sizeof(T);
     constexpr int ROWB  = KV * 16;                // bytes per LDS row: unpadded
     constexpr int SWDIV = 16 / KV;                // rows per 256 bytes of LDS
     constexpr int A_BYTES = BML * ROWB;
     constexpr unsigned STAGE = (BML + BNL) * ROWB; // one LDS stage: A rows, then B rows
-    static_assert(TM % 32 == 0 && TN % 32 == 0 && (WM * WN == 4 || WM * WN == 8 || WM * WN == 12) && S % 2 == 0, "wave grid");
+    static_assert(TM % 32 == 0 && TN % 32 == 0 && (NT == 256 || NT == 512 || NT == 768) && S % 2 == 0, "wave grid");
+    static_assert(KG == 1 || (KG == 2 && TM == 64 && TN == 64), "the K-split variant works on 64 x 64 wave tiles");
     static_assert(NS >= 2 && NS <= 8, "LDS stages");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smemRaw[];
@@ -403,8 +441,9 @@ void convIgemmKernel(IgemmArgs a)
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm   = wave / WN;
-    const int wn   = wave % WN;
+    const int kg   = wave / NWT;                  // which k-blocks of a tile step this wavefront multiplies
+    const int wm   = (wave % NWT) / WN;
+    const int wn   = (wave % NWT) % WN;
     const int g    = blockIdx.z;
     // Workgroup -> tile mapping.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its own
     // L2.  Ids are therefore first regrouped per XCD (id % 8 selects the XCD, id / 8 the position inside it), and
@@ -505,7 +544,7 @@ void convIgemmKernel(IgemmArgs a)
 #pragma unroll
     for (int kb = 0; kb < S; ++kb)
     {
-        const unsigned off = fragRow * ROWB + (((2 * kb + (lane >> 5)) ^ fragSw) * 16);
+        const unsigned off = fragRow * ROWB + (((2 * (kg * S + kb) + (lane >> 5)) ^ fragSw) * 16);
         aAddr[kb] = wm * TM * ROWB + off;
         bAddr[kb] = A_BYTES + wn * TN * ROWB + off;
     }
@@ -612,10 +651,12 @@ void convIgemmKernel(IgemmArgs a)
         e.y = a.ws + static_cast<size_t>(blockIdx.y) * a.P * a.wsLd;
         e.outLd = a.wsLd;
         e.vecOk = (a.wsLd % 8 == 0) && (a.coutG % 8 == 0 || gridDim.z == 1);
-        igemmEpilogue<T, float, BM, BN, TM, TN>(e, acc, smemRaw, 1.f, 0.f, m0, p0, wm, wn, wave, lane, g);
+        if constexpr (KG == 2) igemmEpilogueSwap<T, float, BM, BN>(e, acc, smemRaw, 1.f, 0.f, m0, p0, wm, wn, kg, wave % NWT, wave, lane, g);
+        else igemmEpilogue<T, float, BM, BN, TM, TN>(e, acc, smemRaw, 1.f, 0.f, m0, p0, wm, wn, wave, lane, g);
         return;
     }
-    igemmEpilogue<T, TOut, BM, BN, TM, TN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, wave, lane, g);
+    if constexpr (KG == 2) igemmEpilogueSwap<T, TOut, BM, BN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, kg, wave % NWT, wave, lane, g);
+    else igemmEpilogue<T, TOut, BM, BN, TM, TN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, wave, lane, g);
 }
 
 // Split-K reduction: sums the K slices in slice order (so the result does not depend on timing) and applies the
@@ -646,7 +687,7 @@ __global__ __launch_bounds__(256) void splitKReduceKernel(IgemmArgs a, int outC,
 
 constexpr int kSplitKMax = 8;
 
-template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int NS = 3>
+template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int NS = 3, int KG = 1>
 inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
 {
     constexpr int VEC = Frag<T>::VEC;
@@ -659,9 +700,9 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
         setError("conv2d: the implicit GEMM needs at most 64 filter taps and tensors below 2 GiB");
         return 3;
     }
-    constexpr int RPP = 64 * WM * WN / KV;
+    constexpr int RPP = 64 * WM * WN * KG / KV;
     const size_t smemLoop = static_cast<size_t>(NS) * ((BM + RPP - 1) / RPP * RPP + (BN + RPP - 1) / RPP * RPP) * KV * 16;
-    const size_t smemEpi  = igemmEpilogueLds<BM, BM / WM, WM * WN>();
+    const size_t smemEpi  = std::max(igemmEpilogueLds<BM, BM / WM, WM * WN * KG>(), KG == 2 ? igemmSwapLds<WM * WN * KG>() : size_t(0));
     const size_t smem = smemLoop > smemEpi ? smemLoop : smemEpi;
     a.mTiles = (a.coutG + BM - 1) / BM;
     const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
@@ -681,14 +722,14 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
     }
     dim3 grid((tiles + 7) / 8 * 8, a.splitK, groups);
     if (a.dryRun) return 0;
-    auto kern = convIgemmKernel<T, TOut, BM, BN, KV, WM, WN, NS>;
+    auto kern = convIgemmKernel<T, TOut, BM, BN, KV, WM, WN, NS, KG>;
     if (smem > 48 * 1024)
     {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            static_cast<int>(smem));
         if (e != hipSuccess) { setError("hipFuncSetAttribute: %s", hipGetErrorString(e)); return 1; }
     }
-    hipLaunchKernelGGL(kern, grid, dim3(64 * WM * WN), smem, st, a);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * WM * WN * KG), smem, st, a);
     MSNH_LAUNCH_CHECK();
     if (a.splitK > 1)
     {
@@ -710,7 +751,7 @@ namespace msnh {
 // Tile configurations (BM x BN output tile, KV 16-byte vectors of K per step, WM x WN wavefront grid).
 // Index 0 is "choose for me"; the others can be forced through msnh_conv_desc::tile, which is how the host
 // library's per-layer search picks the fastest one at load time.
-constexpr int kIgemmTiles = 51;
+constexpr int kIgemmTiles = 62;
 
 template <typename T, typename TOut>
 int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
@@ -782,6 +823,20 @@ int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
     case 49: return launchPatch8<T, TOut, 128, 256, 4, 2, 3, 1>(a, groups, st);
     case 50: return launchPatch8<T, TOut, 64, 192, 2, 2, 4, 2>(a, groups, st);
     case 51: return launchPatch8<T, TOut, 128, 384, 2, 4, 3, 2>(a, groups, st);
+    // the same with the k-blocks of a tap step split between two groups of wavefronts over 64 x 64 wave tiles (the numbers are
+    // the grid of wave tiles; twice as many wavefronts run)
+    case 52: return launchPatch8<T, TOut, 64, 384, 1, 6, 3, 1, 0, 2>(a, groups, st);
+    case 53: return launchPatch8<T, TOut, 128, 192, 2, 3, 3, 1, 0, 2>(a, groups, st);
+    case 54: return launchPatch8<T, TOut, 64, 256, 1, 4, 4, 1, 0, 2>(a, groups, st);
+    case 55: return launchPatch8<T, TOut, 128, 128, 2, 2, 4, 1, 0, 2>(a, groups, st);
+    case 56: return launchPatch8<T, TOut, 64, 384, 1, 6, 4, 1, 0, 2>(a, groups, st);
+    // the generic kernel with the same split (numbers: tile, 16-byte vectors of K per step, grid of 64 x 64 wave tiles, LDS stages)
+    case 57: return launchIgemm<T, TOut, 128, 192, 8, 2, 3, 3, 2>(a, groups, st);
+    case 58: return launchIgemm<T, TOut, 128, 128, 8, 2, 2, 4, 2>(a, groups, st);
+    case 59: return launchIgemm<T, TOut, 64, 128, 8, 1, 2, 4, 2>(a, groups, st);
+    case 60: return launchIgemm<T, TOut, 128, 64, 8, 2, 1, 4, 2>(a, groups, st);
+    case 61: return launchIgemm<T, TOut, 64, 256, 8, 1, 4, 3, 2>(a, groups, st);
+    case 62: return launchIgemm<T, TOut, 64, 384, 8, 1, 6, 2, 2>(a, groups, st);
     default: break;
     }
     setError("igemm: unknown tile %d", tile);

@@ -24,30 +24,38 @@ namespace msnh {
 
 // DBG (timing experiments only, results are then meaningless; 0 in every instantiation the library ships): bit 0 leaves out the
 // loads of the main loop, bit 1 its LDS fragment reads, bit 2 its barrier, bit 3 its MFMAs, bit 4 the epilogue, bit 5 the prologue's loads.
-template <typename T, typename TOut, int BM, int BN, int WM, int WN, int NSA, int PS, int DBG = 0>
-__global__ __launch_bounds__(64 * WM * WN) __attribute__((amdgpu_waves_per_eu(WM * WN / 4, WM * WN / 4)))
+//
+// KG = 2 splits the four k-blocks of every tap step between two groups of wavefronts that share the same WM x WN grid of wave
+// tiles: a wavefront then owns a 64 x 64 tile over half of K instead of a 32 x 64 tile over all of it, which takes a third off
+// the LDS fragment reads per MFMA (2 A + 2 B fragments per 4 MFMAs instead of 1 A + 2 B per 2); LDS is the busiest unit of this
+// loop on the 38x38 and 19x19 layers.  After the loop the groups swap halves of their partial sums through LDS and each
+// finishes one 32-pixel block of the wave tile.
+template <typename T, typename TOut, int BM, int BN, int WM, int WN, int NSA, int PS, int DBG = 0, int KG = 1>
+__global__ __launch_bounds__(64 * WM * WN * KG) __attribute__((amdgpu_waves_per_eu(WM * WN * KG / 4, WM * WN * KG / 4)))
 void convPatch8Kernel(IgemmArgs a)
 {
     typedef typename Frag<T>::V V;
     constexpr int VEC   = Frag<T>::VEC;
     constexpr int KV    = 8;
     constexpr int BK    = KV * VEC;
-    constexpr int NW    = WM * WN;
+    constexpr int NWT   = WM * WN;                    // wave tiles
+    constexpr int NW    = NWT * KG;
     constexpr int NT    = 64 * NW;
     constexpr int RPP   = NT / KV;                    // weight rows per load pass of the workgroup
-    constexpr int BML   = (BM + RPP - 1) / RPP * RPP; // weight rows held in LDS (whole passes; the surplus rows load nothing)
-    constexpr int AL    = BML / RPP;                  // weight loads per thread per tap step
+    constexpr int AL    = (BM + RPP - 1) / RPP;       // weight loads per thread per tap step (whole passes of the workgroup)
     constexpr int NL    = AL + PS;                    // loads per thread per tap step
     constexpr int TM    = BM / WM;
     constexpr int TN    = BN / WN;
     constexpr int MB    = TM / 32;
     constexpr int NB    = TN / 32;
-    constexpr int S     = KV / 2;                     // MFMA k-blocks per tap step
+    constexpr int S     = KV / 2 / KG;                // MFMA k-blocks per tap step and wavefront
     constexpr unsigned ES = sizeof(T);
     constexpr int ROWB  = KV * 16;
-    constexpr unsigned A_STAGE = BML * ROWB;
+    constexpr unsigned A_STAGE = BM * ROWB;           // the wavefronts whose rows of the last pass lie past BM aim at the zero area
+    static_assert(BM % 8 == 0, "a wavefront's load covers eight weight rows");
     constexpr int PSTEPS = 11 - NSA;                  // tap steps of a chunk that bring in slices of the next chunk's patch
     static_assert(TM % 32 == 0 && TN % 32 == 0 && (NW == 4 || NW == 8 || NW == 12), "tile shape");
+    static_assert(KG == 1 || (KG == 2 && TM == 64 && TN == 64), "the K-split variant works on 64 x 64 wave tiles");
     static_assert(NSA >= 3 && NSA <= 5, "weight stages");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smemRaw[];
@@ -61,8 +69,9 @@ void convPatch8Kernel(IgemmArgs a)
     const int tid  = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm   = wave / WN;
-    const int wn   = wave % WN;
+    const int kg   = wave / NWT;                      // which k-blocks of a tap step this wavefront multiplies
+    const int wm   = (wave % NWT) / WN;
+    const int wn   = (wave % NWT) % WN;
     const int nTilesP = (a.P + BN - 1) / BN;
     const int total   = a.mTiles * nTilesP;
     const int perXcd  = (total + 7) / 8;
@@ -114,7 +123,8 @@ void convPatch8Kernel(IgemmArgs a)
     const unsigned waveLds = ldsBase + wave * 1024;
     auto issueA = [&](auto lTag, unsigned sA, bool cut, unsigned stageOff) {
         constexpr int l = decltype(lTag)::value;
-        dmaLoad16(rw, cut ? kOobOffset : aOff[l], sA, waveLds + stageOff + l * RPP * ROWB);
+        const bool real = wave * 8 + l * RPP < BM;    // else every lane's offset is out of range already: zeros onto zeros
+        dmaLoad16(rw, cut ? kOobOffset : aOff[l], sA, real ? waveLds + stageOff + l * RPP * ROWB : waveDump);
     };
 
     // ---- fragments ----------------------------------------------------------------------------------------------------------
@@ -122,7 +132,8 @@ void convPatch8Kernel(IgemmArgs a)
     const int fragSw  = (fragRow / 2) % KV;
     unsigned aAddr[S];
 #pragma unroll
-    for (int kb = 0; kb < S; ++kb) aAddr[kb] = wm * TM * ROWB + fragRow * ROWB + (((2 * kb + (lane >> 5)) ^ fragSw) * 16);
+    for (int kb = 0; kb < S; ++kb) aAddr[kb] = wm * TM * ROWB + fragRow * ROWB + (((2 * (kg * S + kb) + (lane >> 5)) ^ fragSw) * 16);
+    const unsigned kvBase = 2 * kg * S + (lane >> 5); // this lane's 16-byte k-vector of local k-block 0
     // per 32-pixel block j of the wave tile: which of the nine taps lie inside the image for this lane's pixel
     unsigned tapOk[NB];
 #pragma unroll
@@ -158,7 +169,7 @@ void convPatch8Kernel(IgemmArgs a)
         constexpr int kb = decltype(kbTag)::value;
         const unsigned row = bRow0 + tapRow;
         const unsigned sw = (row / 2) % KV;
-        const unsigned addr = pOff + row * ROWB + (((2 * kb + (lane >> 5)) ^ sw) * 16);
+        const unsigned addr = pOff + row * ROWB + (((2 * kb + kvBase) ^ sw) * 16);
         const unsigned bit = 1u << tap;
 #pragma unroll
         for (int j = 0; j < NB; ++j)
@@ -286,22 +297,25 @@ void convPatch8Kernel(IgemmArgs a)
         if (sum == 123.456f) static_cast<float *>(a.y)[0] = sum;
         return;
     }
-    igemmEpilogue<T, TOut, BM, BN, TM, TN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, wave, lane, 0);
+    if constexpr (KG == 1)
+        igemmEpilogue<T, TOut, BM, BN, TM, TN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, wave, lane, 0);
+    else
+        igemmEpilogueSwap<T, TOut, BM, BN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, kg, wave % NWT, wave, lane, 0);
 }
 
 // Host-side check shared by launch and tile enumeration.
-template <typename T, int BM, int BN, int WM, int WN, int NSA, int PS>
+template <typename T, int BM, int BN, int WM, int WN, int NSA, int PS, int KG = 1>
 inline bool patch8Fits(const IgemmArgs &a, size_t *smemOut, int *slicesOut)
 {
-    constexpr int NW = WM * WN;
-    constexpr int RPP = 64 * NW / 8;
-    constexpr int BML = (BM + RPP - 1) / RPP * RPP;
+    constexpr int NW = WM * WN * KG;
     constexpr int BK = 8 * Frag<T>::VEC;
     const int R = BN + 2 * a.W + 2;
     const int slices = (R + 7) / 8;
     const int stages = a.cinG > BK ? 2 : 1;
-    const size_t loop = static_cast<size_t>(NSA) * BML * 128 + static_cast<size_t>(stages) * slices * 1024 + 1024;
-    const size_t epi = igemmEpilogueLds<BM, BM / WM, NW>();
+    const size_t loop = static_cast<size_t>(NSA) * BM * 128 + static_cast<size_t>(stages) * slices * 1024 + 1024;
+    const size_t swap = KG == 2 ? igemmSwapLds<NW>() : 0;
+    const size_t epiOnly = igemmEpilogueLds<BM, BM / WM, NW>();
+    const size_t epi = epiOnly > swap ? epiOnly : swap;
     const size_t smem = loop > epi ? loop : epi;
     if (smemOut) *smemOut = smem;
     if (slicesOut) *slicesOut = slices;
@@ -309,14 +323,14 @@ inline bool patch8Fits(const IgemmArgs &a, size_t *smemOut, int *slicesOut)
     return a.patchOk && a.buffersOk && smem <= 160 * 1024 && (stages == 1 || slices <= (11 - NSA) * NW * PS);
 }
 
-template <typename T, typename TOut, int BM, int BN, int WM, int WN, int NSA, int PS, int DBG = 0>
+template <typename T, typename TOut, int BM, int BN, int WM, int WN, int NSA, int PS, int DBG = 0, int KG = 1>
 inline int launchPatch8(IgemmArgs &a, int groups, hipStream_t st)
 {
     constexpr int VEC = Frag<T>::VEC;
     constexpr int BK  = 8 * VEC;
     size_t smem = 0;
     int slices = 0;
-    if (groups != 1 || a.splitMax > 1 || !patch8Fits<T, BM, BN, WM, WN, NSA, PS>(a, &smem, &slices))
+    if (groups != 1 || a.splitMax > 1 || !patch8Fits<T, BM, BN, WM, WN, NSA, PS, KG>(a, &smem, &slices))
     {
         setError("conv2d: this tile needs a 3x3 stride-1 pad-1 ungrouped convolution whose input patch fits in LDS");
         return 3;
@@ -330,13 +344,13 @@ inline int launchPatch8(IgemmArgs &a, int groups, hipStream_t st)
     a.splitK  = 1;
     const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
     dim3 grid((tiles + 7) / 8 * 8, 1, 1);
-    auto kern = convPatch8Kernel<T, TOut, BM, BN, WM, WN, NSA, PS, DBG>;
+    auto kern = convPatch8Kernel<T, TOut, BM, BN, WM, WN, NSA, PS, DBG, KG>;
     if (smem > 48 * 1024)
     {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(smem));
         if (e != hipSuccess) { setError("hipFuncSetAttribute: %s", hipGetErrorString(e)); return 1; }
     }
-    hipLaunchKernelGGL(kern, grid, dim3(64 * WM * WN), smem, st, a);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * WM * WN * KG), smem, st, a);
     MSNH_LAUNCH_CHECK();
     return 0;
 }
