@@ -20,7 +20,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-Wno-unused-command-line-argument", "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(PKG, "csrc")]
-HOST_FLAGS = ["-O3", "-march=x86-64-v3", "-ffp-contract=off", "-std=c++17", "-fPIC", "-fopenmp", "-Wall", "-Wextra", "-I" + os.path.join(ROOT, "include"),
+HOST_FLAGS = ["-O3", "-march=x86-64-v3", "-ffp-contract=off", "-std=c++17", "-fPIC", "-fopenmp-simd", "-Wall", "-Wextra", "-I" + os.path.join(ROOT, "include"),
               "-I" + os.path.join(PKG, "host", "include")]
 
 
@@ -73,7 +73,7 @@ def build_host(verbose=True):
                 print(out)
     os.makedirs(LIB, exist_ok=True)
     _run(["g++", "-shared", "-fPIC", "-o", os.path.join(LIB, "libMsnhnet.so"), *objs,
-          "-L" + LIB, "-lmsnh_hip", "-Wl,-rpath,$ORIGIN", "-fopenmp", "-lpthread"])
+          "-L" + LIB, "-lmsnh_hip", "-Wl,-rpath,$ORIGIN", "-lpthread"])
     return os.path.join(LIB, "libMsnhnet.so")
 
 

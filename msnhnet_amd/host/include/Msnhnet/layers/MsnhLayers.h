@@ -363,9 +363,12 @@ public:
     // 1 (default) = chosen per batch from the previous result: up to kDeviceNmsFew candidates per image on the device; up to
     // kDeviceNmsCandidates (the largest class the device kernels take) on the device as well, except while forwards are pipelined and
     // the host stage keeps up with them -- the host then does it for free beside the next forward; more than that on the host.
+    // "Keeps up" is measured: when the host stage stops waiting for the device, kTrialBatches batches run on the device and the
+    // placement with the shorter time between results stays.
     static int deviceNms;
     static const int kDeviceNmsFew = 2048;
     static const int kDeviceNmsCandidates = 6144;
+    static const int kTrialBatches = 16;
 
     // host post-processing of the compacted candidate rows of one image (8 floats per row, see msnh_hip_yolo_gather)
     std::vector<YoloBox> boxesFromRows(const float *rows, int count, const float *decodedOfImage) const;
@@ -387,6 +390,7 @@ private:
         DeviceBuffer devCnt, devRows, devKept, devKeptCnt, devNmsWs;
         msnh_event_t event = nullptr, ready = nullptr;
         bool pending = false, onDevice = false;
+        bool trial = false;                // part of a device trial of the automatic placement
         size_t rowsCopied = 0;             // row slots per image that the asynchronous copy brings to the host
         size_t quick = 0;                  // device NMS: records that the asynchronous copy brings to the host
     };
@@ -395,7 +399,12 @@ private:
     int _lastMaxCandidates = 0;            // largest per-image candidate count of the previous result
     size_t _lastKept = 0;                  // records the device NMS kept for the previous batch
     int _hostBoundRuns = 0;                // batches in a row for which the host path did not have to wait for the device
-    bool _hostBound = false;
+    bool _hostBound = false;               // a device trial gave results faster than the host stage: stay on the device
+    int _trialLeft = 0, _trialSeen = 0, _trialSamples = 0;   // device trial: batches to enqueue / finished / intervals measured
+    double _trialSum = 0.0, _hostInterval = 0.0;             // ms between results: sum over the trial, moving mean of the host mode
+    std::chrono::steady_clock::time_point _lastFinish;
+    bool _haveLastFinish = false, _lastFinishHost = false;
+    void noteResult(const Slot &sl, bool pipelined);
     Slot _slots[2];
 };
 }

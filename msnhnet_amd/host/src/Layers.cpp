@@ -10,6 +10,7 @@
 #include <cstring>
 #include "Msnhnet/net/MsnhNetwork.h"
 #include "Msnhnet/utils/MsnhExVector.h"
+#include "Msnhnet/utils/MsnhTaskPool.h"
 
 namespace Msnhnet
 {
@@ -1454,7 +1455,10 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
     // (the host's sort + NMS then runs beside that forward and costs the device nothing, whereas the device NMS takes about 0.1 ms of
     // device time per batch from it) and the host stage has kept up with the device so far
     const bool pipelined = _slots[(slot ^ 1) & 1].pending;
-    const bool autoDevice = _lastMaxCandidates <= kDeviceNmsFew || (_lastMaxCandidates <= kDeviceNmsCandidates && (!pipelined || _hostBound));
+    const bool mid = _lastMaxCandidates > kDeviceNmsFew && _lastMaxCandidates <= kDeviceNmsCandidates;
+    sl.trial = deviceNms == 1 && !_useSoftNms && mid && pipelined && !_hostBound && _trialLeft > 0;
+    if (sl.trial) --_trialLeft;
+    const bool autoDevice = _lastMaxCandidates <= kDeviceNmsFew || (mid && (!pipelined || _hostBound || sl.trial));
     sl.onDevice = !_useSoftNms && (deviceNms == 2 || (deviceNms == 1 && autoDevice));
     if (sl.onDevice)
     {
@@ -1520,6 +1524,39 @@ std::vector<YoloBox> YoloOutLayer::boxesFromKept(std::vector<const float *> &rec
     return out;
 }
 
+// Time between consecutive results while two batches are in flight: a moving mean for the host placement, a plain mean over a
+// device trial (its first four results still carry the change-over).  At the end of a trial the faster placement stays; a
+// trial that lost is not repeated for a thousand batches.
+void YoloOutLayer::noteResult(const Slot &sl, bool pipelined)
+{
+    const std::chrono::steady_clock::time_point now = std::chrono::steady_clock::now();
+    const bool usable = _haveLastFinish && pipelined;
+    const double ms = usable ? std::chrono::duration<double, std::milli>(now - _lastFinish).count() : 0.0;
+    if (!sl.onDevice)
+    {
+        if (usable && _lastFinishHost) _hostInterval = _hostInterval > 0.0 ? _hostInterval + (ms - _hostInterval) / 8.0 : ms;
+    }
+    else if (sl.trial)
+    {
+        ++_trialSeen;
+        if (usable && _trialSeen > 4) { _trialSum += ms; ++_trialSamples; }
+        if (_trialSeen == kTrialBatches)
+        {
+            const bool faster = _trialSamples >= kTrialBatches / 2 && _trialSum / _trialSamples < 0.97 * _hostInterval;
+            if (std::getenv("MSNH_DEBUG_TIMING"))
+                std::fprintf(stderr, "yoloout placement trial: device %.3f ms (%d results), host %.3f ms between results -> %s\n",
+                             _trialSamples ? _trialSum / _trialSamples : 0.0, _trialSamples, _hostInterval, faster ? "device" : "host");
+            _hostBound = faster;
+            _hostBoundRuns = faster ? 0 : -1000;
+            _trialSeen = 0;
+            _trialLeft = 0;
+        }
+    }
+    _lastFinish = now;
+    _haveLastFinish = true;
+    _lastFinishHost = !sl.onDevice;
+}
+
 void YoloOutLayer::finish(int slot)
 {
     Slot &sl = _slots[slot & 1];
@@ -1529,6 +1566,7 @@ void YoloOutLayer::finish(int slot)
     const float dbgWait = TimeUtil::getElapsedTime(dbg0);
     sl.pending = false;
     lastOnDevice = sl.onDevice;
+    noteResult(sl, _slots[(slot ^ 1) & 1].pending);
     const int cells = plan->yoloCells;
     const int per = _channel;
     const int *cnt = sl.cnt.as<int>();
@@ -1559,9 +1597,9 @@ void YoloOutLayer::finish(int slot)
         }
         batchHasBox.assign(static_cast<size_t>(_batch), false);
         finalOut.assign(static_cast<size_t>(_batch), std::vector<YoloBox>());
-#pragma omp parallel for schedule(dynamic)
-        for (int b = 0; b < _batch; ++b)
+        TaskPool::instance().parallelFor(_batch, [&](int b) {
             if (keptCnt[1 + b] == 0) finalOut[static_cast<size_t>(b)] = boxesFromKept(perImage[static_cast<size_t>(b)]);
+        });
         std::vector<float> hostRows;
         for (int b = 0; b < _batch; ++b)
         {
@@ -1598,15 +1636,14 @@ void YoloOutLayer::finish(int slot)
     // independent, and a batch has far fewer images than the host has cores; concatenation per image
     std::vector<std::vector<YoloBox>> cand(static_cast<size_t>(_batch));
     std::vector<std::vector<std::vector<int>>> groups(static_cast<size_t>(_batch));
-#pragma omp parallel for schedule(dynamic)
-    for (int b = 0; b < _batch; ++b)
-    {
+    TaskPool &pool = TaskPool::instance();
+    pool.parallelFor(_batch, [&](int b) {
         const int n = std::min(cnt[b], cells);
         const float *dec = decodedHost ? decodedHost + static_cast<size_t>(b) * cells * per : nullptr;
         cand[static_cast<size_t>(b)] = boxesFromRows(sl.rows.as<float>() + static_cast<size_t>(b) * cells * 8, n, dec);
         if (_useSoftNms) finalOut[static_cast<size_t>(b)] = nms(cand[static_cast<size_t>(b)], _nmsThresh, true);
         else groups[static_cast<size_t>(b)] = groupByClass(cand[static_cast<size_t>(b)]);
-    }
+    });
     const double dbgA = TimeUtil::getElapsedTime(dbg0);
     double dbgB = dbgA;
     if (!_useSoftNms)
@@ -1619,29 +1656,28 @@ void YoloOutLayer::finish(int slot)
             return groups[static_cast<size_t>(x.first)][static_cast<size_t>(x.second)].size() > groups[static_cast<size_t>(y.first)][static_cast<size_t>(y.second)].size();
         });
         const int nTasks = static_cast<int>(tasks.size());
-#pragma omp parallel for schedule(dynamic, 1)
-        for (int t = 0; t < nTasks; ++t)
-        {
+        pool.parallelFor(nTasks, [&](int t) {
             const size_t b = static_cast<size_t>(tasks[static_cast<size_t>(t)].first);
             nmsClass(cand[b], groups[b][static_cast<size_t>(tasks[static_cast<size_t>(t)].second)], _nmsThresh);
-        }
+        });
         dbgB = TimeUtil::getElapsedTime(dbg0);
-#pragma omp parallel for schedule(dynamic)
-        for (int b = 0; b < _batch; ++b)
-        {
+        pool.parallelFor(_batch, [&](int b) {
             std::vector<YoloBox> &out = finalOut[static_cast<size_t>(b)];
             for (const std::vector<int> &m : groups[static_cast<size_t>(b)])
                 for (int j : m) out.push_back(cand[static_cast<size_t>(b)][static_cast<size_t>(j)]);
-        }
+        });
     }
     for (int b = 0; b < _batch; ++b) batchHasBox[static_cast<size_t>(b)] = cnt[b] > 0;
     {
-        // did the device make the host wait?  If it has not for eight batches in a row, the host stage is what bounds the pipeline, and
-        // the automatic mode moves the NMS to the device (until a batch with few candidates resets the question)
+        // did the device make the host wait?  If it has not for eight batches in a row, the host stage may be what bounds the
+        // pipeline: the automatic mode then tries the device for kTrialBatches batches (noteResult() compares the two)
         const double stage = TimeUtil::getElapsedTime(dbg0) - dbgWait;
         if (_lastMaxCandidates <= kDeviceNmsFew) { _hostBoundRuns = 0; _hostBound = false; }
-        else if (dbgWait < 0.05 * stage) { if (++_hostBoundRuns >= 8) _hostBound = true; }
-        else _hostBoundRuns = 0;
+        else if (dbgWait < 0.05 * stage)
+        {
+            if (++_hostBoundRuns >= 8 && _trialLeft == 0 && _trialSeen == 0 && _hostInterval > 0.0) { _trialLeft = kTrialBatches; _trialSum = 0.0; _trialSamples = 0; }
+        }
+        else if (_hostBoundRuns > 0) _hostBoundRuns = 0;
     }
     if (std::getenv("MSNH_DEBUG_TIMING"))
         std::fprintf(stderr, "yoloout finish: wait %.3f ms, host %.3f ms (candidates %.3f, suppression %.3f, output %.3f)\n", dbgWait,

@@ -238,3 +238,17 @@ def test_pack_file_round_trip_and_rejections(tmp_path):
     assert r.returncode == 0, r.stdout
     r = subprocess.run([exe, str(tmp_path)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
     assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout
+
+
+def test_task_pool(tmp_path):
+    """the worker pool of the box stage (tests/cpp/taskpool_check.cpp, host code only): each index once, exceptions propagate,
+    idle workers use no CPU time -- a spinning team exhausts a container's CPU allowance and stalls the thread that feeds the GPU"""
+    import subprocess
+    exe = str(tmp_path / "taskpool_check")
+    lib = os.path.join(ROOT, "msnhnet_amd", "lib")
+    cmd = ["g++", "-std=c++17", "-O1", "-I" + os.path.join(ROOT, "msnhnet_amd", "host", "include"), os.path.join(ROOT, "tests", "cpp", "taskpool_check.cpp"),
+           "-o", exe, "-L" + lib, "-lMsnhnet", "-lmsnh_hip", "-Wl,-rpath," + lib, "-lpthread"]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout
+    r = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout
