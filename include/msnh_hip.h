@@ -291,6 +291,24 @@ int msnh_hip_yolo_decode_candidates(int dtype, int batch, int h, int w, int clas
                                     const float *anchors6, float ratio, int yolo_version, float *decoded,
                                     long long decoded_batch_stride, float conf_thresh, int *cand_idx, int cand_cap, int cand_base,
                                     int *cand_cnt, float *rows, msnh_stream_t s);
+/* msnh_hip_yolo_decode_candidates for all heads of a network in two launches instead of two per head (YoloLayer::forwardGPU of every head,
+ * src/layers/MsnhYoloLayer.cpp:164-185, plus the candidate threshold of src/layers/MsnhYoloOutLayer.cpp:216-260): same list (as
+ * a set: the order inside the list is arbitrary in both) and same rows.  heads[k].cand_base must be the sum of 3*h*w of the heads
+ * before it (the cells of an image are numbered head after head); at most 4 heads; decoded may be NULL.  cand_cnt is
+ * incremented by the number of candidates found (caller zeroes it). */
+typedef struct msnh_yolo_head
+{
+    const void *x;          /* head logits NHWC, as for msnh_hip_yolo_decode */
+    int x_ld;
+    float x_mul;
+    int h, w;
+    float anchors[6];
+    float ratio;
+    int cand_base;
+} msnh_yolo_head;
+int msnh_hip_yolo_decode_candidates_heads(int dtype, int batch, int classes, int n_heads, const msnh_yolo_head *heads, int yolo_version,
+                                          float *decoded, long long decoded_batch_stride, float conf_thresh, int *cand_idx, int cand_cap,
+                                          int *cand_cnt, float *rows, msnh_stream_t s);
 /* Candidate compaction for YoloOutLayer (the per-box part of src/layers/MsnhYoloOutLayer.cpp:120-170 done on
  * the device so that only surviving boxes cross PCIe): for image b and k < min(cand_cnt[b], cand_cap) reads
  * the decoded row of cell cand_idx[b][k] (rows are `5+classes` floats, row r of image b at

@@ -176,6 +176,127 @@ __global__ __launch_bounds__(256) void yoloRowsKernel(const T *__restrict__ x, i
     }
 }
 
+// All heads of a network in two launches instead of two per head: an objectness scan over the cells of an image numbered over
+// the heads in list order (which is the numbering of the candidate list), then the rows of the listed candidates, each decoded
+// from the head its cell number falls into.  Same logistic, same threshold test and same per-value decode as the per-head
+// kernels, so list (as a set) and rows are identical.  (Decoding a workgroup's own candidates right after its scan, in one
+// launch, was slower: where objectness is dense a few workgroups hold most of the candidates.)
+constexpr int YOLO_MAX_HEADS = 4;
+struct YoloHeads
+{
+    const void *x[YOLO_MAX_HEADS];
+    int xLd[YOLO_MAX_HEADS], W[YOLO_MAX_HEADS], HW[YOLO_MAX_HEADS], base[YOLO_MAX_HEADS];
+    float xMul[YOLO_MAX_HEADS], ratio[YOLO_MAX_HEADS];
+    Anchors an[YOLO_MAX_HEADS];
+    int n, cells;
+};
+
+__device__ __forceinline__ int yoloHeadOf(const YoloHeads &hd, int cellG)
+{
+    int k = 0;
+#pragma unroll
+    for (int i = 1; i < YOLO_MAX_HEADS; ++i)
+        if (i < hd.n && cellG >= hd.base[i]) k = i;
+    return k;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void yoloHeadsScanKernel(YoloHeads hd, float confThresh, int *__restrict__ candIdx, int candCap, int *__restrict__ candCnt, int per)
+{
+    __shared__ int found[256];
+    __shared__ int nFound, base;
+    const int b = blockIdx.y;
+    if (threadIdx.x == 0) nFound = 0;
+    __syncthreads();
+    const int cellG = blockIdx.x * 256 + threadIdx.x;
+    if (cellG < hd.cells)
+    {
+        const int k = yoloHeadOf(hd, cellG);
+        const int cell = cellG - hd.base[k];
+        const int HW = hd.HW[k];
+        const int a = cell / HW, p = cell - a * HW;
+        const float v = hd.xMul[k] * toF(static_cast<const T *>(hd.x[k])[(static_cast<size_t>(b) * HW + p) * hd.xLd[k] + a * per + 4]);
+        if (logisticF(v) > confThresh) found[atomicAdd(&nFound, 1)] = cellG;
+    }
+    __syncthreads();
+    if (nFound == 0) return;
+    if (threadIdx.x == 0) base = atomicAdd(candCnt + b, nFound);
+    __syncthreads();
+    if (static_cast<int>(threadIdx.x) < nFound && base + static_cast<int>(threadIdx.x) < candCap)
+        candIdx[static_cast<size_t>(b) * candCap + base + threadIdx.x] = found[threadIdx.x];
+}
+
+template <typename T, bool V5>
+__global__ __launch_bounds__(256) void yoloHeadsRowsKernel(YoloHeads hd, float *__restrict__ decoded, long long decStride, const int *__restrict__ candIdx,
+                                                           int candCap, const int *__restrict__ candCnt, float *__restrict__ rows, int per)
+{
+    const int b = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int sub = lane & 15;
+    const int groupLane0 = lane & 48;
+    const int group = threadIdx.x >> 4;
+    int n = candCnt[b];
+    n = n < candCap ? n : candCap;
+    for (int slot = blockIdx.x * 16 + group; slot < n; slot += gridDim.x * 16)
+    {
+        const int cellG = candIdx[static_cast<size_t>(b) * candCap + slot];
+        if (cellG < 0 || cellG >= hd.cells) continue;
+        const int k = yoloHeadOf(hd, cellG);
+        const int cell = cellG - hd.base[k];
+        const int HW = hd.HW[k], W = hd.W[k];
+        const int a = cell / HW, p = cell - a * HW;
+        const int py = p / W, px = p - py * W;
+        const T *xr = static_cast<const T *>(hd.x[k]) + (static_cast<size_t>(b) * HW + p) * hd.xLd[k] + a * per;
+        float *dr = decoded + static_cast<size_t>(b) * decStride + static_cast<size_t>(cellG) * per;
+        const float xMul = hd.xMul[k], ratio = hd.ratio[k];
+        const Anchors an = hd.an[k];
+        float first = 0.f;
+        float bv = -3.402823466e38f * 2.f;
+        int bi = 0x7fffffff;
+        // all loads of the row first (the stores into `decoded` below may alias the head tensor as far as the compiler knows, and
+        // a load per round trip would make the row cost one memory latency per sixteen values)
+        constexpr int ROUNDS = 8;
+        float raw[ROUNDS];
+#pragma unroll
+        for (int it = 0; it < ROUNDS; ++it)
+        {
+            const int m = sub + 16 * it;
+            raw[it] = m < per ? toF(xr[m]) : 0.f;
+        }
+#pragma unroll
+        for (int it = 0; it < ROUNDS; ++it)
+        {
+            const int m = sub + 16 * it;
+            if (m >= per) break;
+            const float v = yoloDecodeOne<V5>(xMul * raw[it], m, px, py, a, an, ratio);
+            if (decoded != nullptr) dr[m] = v;
+            if (it == 0) first = v;
+            if (m >= 5 && v > bv) { bv = v; bi = m - 5; }
+        }
+        for (int m = sub + 16 * ROUNDS; m < per; m += 16)        // more than 123 classes
+        {
+            const float v = yoloDecodeOne<V5>(xMul * toF(xr[m]), m, px, py, a, an, ratio);
+            if (decoded != nullptr) dr[m] = v;
+            if (v > bv) { bv = v; bi = m - 5; }
+        }
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1)
+        {
+            const float ov = __shfl_xor(bv, off, 64);
+            const int oi = __shfl_xor(bi, off, 64);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
+        const float c0v = __shfl(first, groupLane0 + 5, 64);
+        if (c0v != c0v) { bv = c0v; bi = 0; }
+        if (bi == 0x7fffffff) bi = 0;
+        float *o = rows + (static_cast<size_t>(b) * candCap + slot) * 8;
+        if (sub < 5) o[sub] = first;
+        else if (sub == 5) o[5] = bv;
+        else if (sub == 6) o[6] = static_cast<float>(bi);
+        else if (sub == 7) o[7] = static_cast<float>(cellG);
+    }
+}
+
 // ---- per-class greedy NMS on the device (src/layers/MsnhYoloOutLayer.cpp:175-194 sort, :381-461 nms) -------------------
 // One workgroup per (class, image).  The reference sorts all candidates of an image by objectness * best class score
 // (descending; here ties keep cell order), visits the classes in the order of their first appearance in that list and,
@@ -920,6 +1041,49 @@ extern "C" int msnh_hip_yolo_decode_candidates(int dtype, int batch, int h, int 
     } while (0)
     if (dtype == MSNH_F16) MSNH_YC(f16); else MSNH_YC(float);
 #undef MSNH_YC
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int msnh_hip_yolo_decode_candidates_heads(int dtype, int batch, int classes, int n_heads, const msnh_yolo_head *heads, int yolo_version,
+                                                     float *decoded, long long decoded_batch_stride, float conf_thresh, int *cand_idx, int cand_cap,
+                                                     int *cand_cnt, float *rows, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "yolo_decode_candidates_heads: bad dtype");
+    MSNH_REQUIRE(batch > 0 && batch <= 65535 && classes > 0, "yolo_decode_candidates_heads: bad geometry");
+    MSNH_REQUIRE(n_heads >= 1 && n_heads <= YOLO_MAX_HEADS && heads, "yolo_decode_candidates_heads: 1 to 4 heads");
+    MSNH_REQUIRE(yolo_version == 3 || yolo_version == 4 || yolo_version == 5, "yolo_decode_candidates_heads: yolo_version must be 3, 4 or 5");
+    MSNH_REQUIRE(rows && cand_idx && cand_cnt && cand_cap > 0, "yolo_decode_candidates_heads: bad argument");
+    const int per = 5 + classes;
+    YoloHeads hd;
+    std::memset(&hd, 0, sizeof(hd));
+    hd.n = n_heads;
+    int cells = 0;
+    for (int k = 0; k < n_heads; ++k)
+    {
+        const msnh_yolo_head &h = heads[k];
+        MSNH_REQUIRE(h.x && h.h > 0 && h.w > 0 && h.x_ld >= 3 * per, "yolo_decode_candidates_heads: bad head");
+        MSNH_REQUIRE(h.cand_base == cells, "yolo_decode_candidates_heads: the heads' cell numbers must follow one another from 0");
+        hd.x[k] = h.x; hd.xLd[k] = h.x_ld; hd.xMul[k] = h.x_mul; hd.W[k] = h.w; hd.HW[k] = h.h * h.w; hd.base[k] = cells; hd.ratio[k] = h.ratio;
+        for (int i = 0; i < 6; ++i) hd.an[k].v[i] = h.anchors[i];
+        cells += 3 * h.h * h.w;
+    }
+    hd.cells = cells;
+    MSNH_REQUIRE(decoded == nullptr || decoded_batch_stride >= static_cast<long long>(cells) * per, "yolo_decode_candidates_heads: decoded_batch_stride too small");
+    hipStream_t st = resolveStream(s);
+    dim3 sgrid((cells + 255) / 256, batch), rgrid(256, batch);
+#define MSNH_YH(T)                                                                                                                                   \
+    do {                                                                                                                                             \
+        hipLaunchKernelGGL((yoloHeadsScanKernel<T>), sgrid, dim3(256), 0, st, hd, conf_thresh, cand_idx, cand_cap, cand_cnt, per);                   \
+        if (yolo_version == 5)                                                                                                                       \
+            hipLaunchKernelGGL((yoloHeadsRowsKernel<T, true>), rgrid, dim3(256), 0, st, hd, decoded, decoded_batch_stride, cand_idx, cand_cap,       \
+                               cand_cnt, rows, per);                                                                                                 \
+        else                                                                                                                                         \
+            hipLaunchKernelGGL((yoloHeadsRowsKernel<T, false>), rgrid, dim3(256), 0, st, hd, decoded, decoded_batch_stride, cand_idx, cand_cap,      \
+                               cand_cnt, rows, per);                                                                                                 \
+    } while (0)
+    if (dtype == MSNH_F16) MSNH_YH(f16); else MSNH_YH(float);
+#undef MSNH_YH
     MSNH_LAUNCH_CHECK();
     return 0;
 }

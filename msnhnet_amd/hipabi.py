@@ -39,9 +39,15 @@ SYMBOLS = [
     "msnh_hip_graph_end", "msnh_hip_graph_launch", "msnh_hip_graph_destroy", "msnh_hip_conv_stem_down_supported", "msnh_hip_conv_stem_down_packed_elems", "msnh_hip_conv_stem_down_pack", "msnh_hip_conv_stem_down", "msnh_hip_conv2d_tile_count", "msnh_hip_conv2d_pack_layout_version", "msnh_hip_conv2d_tile_supported", "msnh_hip_conv2d_select_algo",
     "msnh_hip_conv2d_packed_weight_elems", "msnh_hip_conv2d_pack_weights", "msnh_hip_conv2d_workspace_bytes", "msnh_hip_conv2d", "msnh_hip_letterbox_u8", "msnh_hip_image_u8_to_input",
     "msnh_hip_affine_act", "msnh_hip_add_act", "msnh_hip_copy_channels", "msnh_hip_maxpool", "msnh_hip_avgpool",
-    "msnh_hip_upsample_nearest", "msnh_hip_pad", "msnh_hip_slice", "msnh_hip_upsample_bilinear", "msnh_hip_softmax", "msnh_hip_deconv_col2im", "msnh_hip_connected", "msnh_hip_nchw_to_nhwc", "msnh_hip_nhwc_to_nchw", "msnh_hip_yolo_decode", "msnh_hip_yolo_decode_candidates",
+    "msnh_hip_upsample_nearest", "msnh_hip_pad", "msnh_hip_slice", "msnh_hip_upsample_bilinear", "msnh_hip_softmax", "msnh_hip_deconv_col2im", "msnh_hip_connected", "msnh_hip_nchw_to_nhwc", "msnh_hip_nhwc_to_nchw", "msnh_hip_yolo_decode", "msnh_hip_yolo_decode_candidates", "msnh_hip_yolo_decode_candidates_heads",
     "msnh_hip_yolo_gather", "msnh_hip_yolo_nms", "msnh_hip_yolo_nms_workspace_bytes", "msnh_hip_yolo_nms_pair_workspace_bytes", "msnh_hip_yolo_nms_static", "msnh_hip_yolo_nms_static_max_bytes", "msnh_hip_absmax", "msnh_hip_count_nonfinite",
 ]
+
+
+class YoloHead(ctypes.Structure):
+    """msnh_yolo_head of include/msnh_hip.h"""
+    _fields_ = [("x", ctypes.c_void_p), ("x_ld", ctypes.c_int), ("x_mul", ctypes.c_float), ("h", ctypes.c_int), ("w", ctypes.c_int),
+                ("anchors", ctypes.c_float * 6), ("ratio", ctypes.c_float), ("cand_base", ctypes.c_int)]
 
 
 def lib():
@@ -104,6 +110,7 @@ def lib():
     L.msnh_hip_nhwc_to_nchw.argtypes = [ci, ci, ci, ci, ci, vp, ci, cf, vp, vp]
     L.msnh_hip_yolo_decode.argtypes = [ci, ci, ci, ci, ci, vp, ci, cf, fp, cf, ci, vp, ll, cf, vp, ci, ci, vp, vp]
     L.msnh_hip_yolo_decode_candidates.argtypes = [ci, ci, ci, ci, ci, vp, ci, cf, fp, cf, ci, vp, ll, cf, vp, ci, ci, vp, vp, vp]
+    L.msnh_hip_yolo_decode_candidates_heads.argtypes = [ci, ci, ci, ci, ctypes.POINTER(YoloHead), ci, vp, ll, cf, vp, ci, vp, vp, vp]
     L.msnh_hip_yolo_gather.argtypes = [ci, ci, vp, ll, vp, ci, vp, vp, vp]
     L.msnh_hip_yolo_nms.argtypes = [ci, ci, vp, ci, vp, cf, vp, ci, vp, vp, sz, vp]
     L.msnh_hip_yolo_nms_workspace_bytes.argtypes = [ci, ci, ci]

@@ -96,6 +96,9 @@ public:
     int computeDtype;
     bool sparseYolo = false;                // yolo heads decode only the rows of their candidates (nobody reads the full decoded tensors)
     bool yoloKeepDecoded = true;            // sparseYolo: also write the candidates' full decoded rows (only YoloBox::classesVal needs them)
+    std::vector<size_t> yoloHeadOps;        // sparseYolo: the heads' decode ops in cell order when one launch (issued at the last of them in
+                                            // op order) can decode them all; empty = one launch pair per head
+    void findYoloHeads();                   // fills yoloHeadOps; call once the heads' cell numbers are assigned
     bool fuseStemDown = true;               // float16: first layer + first stride-2 layer as one launch where msnh_hip_conv_stem_down takes the pair
     bool preferWinograd = false;            // 3x3 stride-1 float16 convs take the Winograd path where the kernel accepts the shape
     std::vector<PlanTensor> tensors;

@@ -376,6 +376,7 @@ static void setupYoloBuffers(Plan &plan, int batch)
     plan.yoloCandIdx.alloc(sizeof(int) * cells * static_cast<size_t>(batch));
     plan.yoloCandCnt.alloc(sizeof(int) * static_cast<size_t>(std::max(batch, 64)));
     plan.yoloRows.alloc(sizeof(float) * 8 * cells * static_cast<size_t>(batch));
+    plan.findYoloHeads();
 }
 
 void NetBuilder::finalizePlan()

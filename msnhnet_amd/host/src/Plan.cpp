@@ -426,6 +426,15 @@ void Plan::place()
         if (op.dead) continue;
         touch(op.in0, i); touch(op.in1, i); touch(op.out, i);
     }
+    {
+        // the heads of a detector may all be decoded by one launch where the last of them stands (findYoloHeads): their inputs
+        // stay alive until then
+        int lastHead = -1;
+        for (int i = 0; i < nOps; ++i)
+            if (!ops[static_cast<size_t>(i)].dead && ops[static_cast<size_t>(i)].kind == PlanOp::YOLO_DECODE) lastHead = i;
+        for (int i = 0; i < lastHead; ++i)
+            if (!ops[static_cast<size_t>(i)].dead && ops[static_cast<size_t>(i)].kind == PlanOp::YOLO_DECODE) touch(ops[static_cast<size_t>(i)].in0, lastHead);
+    }
     for (int t = 0; t < nT; ++t)
     {
         if (!tensors[static_cast<size_t>(t)].persistent && !tensors[static_cast<size_t>(t)].pinned) continue;
@@ -992,7 +1001,26 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
         const int per = 5 + op.classes;
         float *decoded = yoloDecoded.as<float>() + static_cast<size_t>(op.cellBase) * per;
         const bool cand = op.confThresh < 1.5f;
-        if (sparseYolo && cand)
+        if (sparseYolo && cand && !yoloHeadOps.empty())
+        {
+            // all heads in one launch, issued where the last of them stands in the plan (nothing between the heads reads their lists)
+            size_t last = 0;
+            for (size_t i : yoloHeadOps) last = std::max(last, i);
+            if (&op != &ops[last]) break;
+            msnh_yolo_head heads[4];
+            for (size_t k = 0; k < yoloHeadOps.size(); ++k)
+            {
+                const PlanOp &h = ops[yoloHeadOps[k]];
+                const PlanTensor &t = tensors[static_cast<size_t>(h.in0)];
+                heads[k].x = ptr(h.in0); heads[k].x_ld = ld(h.in0); heads[k].x_mul = mulOf(h.in0); heads[k].h = t.h; heads[k].w = t.w;
+                for (int i = 0; i < 6; ++i) heads[k].anchors[i] = h.anchors[static_cast<size_t>(i)];
+                heads[k].ratio = h.ratio; heads[k].cand_base = h.cellBase;
+            }
+            MSNH_DEV(msnh_hip_yolo_decode_candidates_heads(in.dtype, in.n, op.classes, static_cast<int>(yoloHeadOps.size()), heads, op.yoloVersion,
+                                                           yoloKeepDecoded ? yoloDecoded.as<float>() : nullptr, static_cast<long long>(yoloCells) * per,
+                                                           op.confThresh, yoloCandIdx.as<int>(), yoloCells, yoloCandCnt.as<int>(), yoloRows.as<float>(), s));
+        }
+        else if (sparseYolo && cand)
             MSNH_DEV(msnh_hip_yolo_decode_candidates(in.dtype, in.n, in.h, in.w, op.classes, ptr(op.in0), ld(op.in0), mulOf(op.in0), op.anchors.data(),
                                                      op.ratio, op.yoloVersion, yoloKeepDecoded ? decoded : nullptr, static_cast<long long>(yoloCells) * per, op.confThresh,
                                                      yoloCandIdx.as<int>(), yoloCells, op.cellBase, yoloCandCnt.as<int>(), yoloRows.as<float>(), s));
@@ -1003,6 +1031,33 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
         break;
     }
     }
+}
+
+// One launch can decode all heads when there are at most four, they agree in everything but geometry and anchors, and their cell
+// numbers follow one another from 0 (the candidate list numbers the cells of an image head after head).
+void Plan::findYoloHeads()
+{
+    yoloHeadOps.clear();
+    if (std::getenv("MSNH_YOLO_HEAD_LAUNCHES")) return;
+    std::vector<size_t> heads;
+    for (size_t i = 0; i < ops.size(); ++i)
+        if (ops[i].kind == PlanOp::YOLO_DECODE && !ops[i].dead) heads.push_back(i);
+    if (heads.size() < 2 || heads.size() > 4) return;
+    std::sort(heads.begin(), heads.end(), [this](size_t a, size_t b) { return ops[a].cellBase < ops[b].cellBase; });
+    const PlanOp &first = ops[heads[0]];
+    int cells = 0;
+    for (size_t i : heads)
+    {
+        const PlanOp &h = ops[i];
+        const PlanTensor &t = tensors[static_cast<size_t>(h.in0)];
+        const PlanTensor &t0 = tensors[static_cast<size_t>(first.in0)];
+        if (h.cellBase != cells || h.classes != first.classes || h.yoloVersion != first.yoloVersion || h.confThresh != first.confThresh ||
+            h.confThresh >= 1.5f || t.dtype != t0.dtype || t.n != t0.n)
+            return;
+        cells += 3 * t.h * t.w;
+    }
+    if (cells != yoloCells) return;
+    yoloHeadOps = heads;
 }
 
 void Plan::run(size_t opBegin, size_t opEnd, msnh_stream_t s)

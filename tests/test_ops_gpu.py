@@ -403,6 +403,90 @@ def test_yolo_decode(dtype, version):
             assert int(rows[b, k, 6]) == int(np.argmax(r[5:]))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("version", [3, 5])
+@pytest.mark.parametrize("keep_decoded,cls", [(False, 20), (True, 20), (True, 130)])
+def test_yolo_decode_candidates_all_heads(dtype, version, keep_decoded, cls):
+    """one call over all heads of a network gives the candidate list (as a set), the compact rows and -- when asked for -- the
+    decoded rows that one msnh_hip_yolo_decode_candidates call per head gives, bit for bit; checked for three heads of different
+    sizes (one of them with more cells than a workgroup scans, one with none above the threshold) and a list shorter than the
+    number of candidates"""
+    import gpuutil as gu
+    gu.init()
+    L = abi.lib()
+    rng = np.random.default_rng(14)
+    per = 5 + cls
+    ld = (3 * per + 7) // 8 * 8
+    shapes = [(3, 4), (6, 8), (13, 11)]
+    anchors = [np.array([116, 90, 156, 198, 373, 326], np.float32), np.array([30, 61, 62, 45, 59, 119], np.float32), np.array([10, 13, 16, 30, 33, 23], np.float32)]
+    ratios = [32.0, 16.0, 8.0]
+    batch = 3
+    xs = []
+    for i, (h, w) in enumerate(shapes):
+        x = (rng.standard_normal((batch, 3 * per, h, w)) * 3).astype(np.float32)
+        if i == 1:
+            x[:, 4::per] = -9.0                  # this head has no candidate at all
+        if dtype == abi.F16:
+            x = gu.round_f16(x)
+        xs.append(gu.nhwc_dev(x, dtype, ld))
+    cells = sum(3 * h * w for h, w in shapes)
+    fp = ctypes.POINTER(ctypes.c_float)
+    for cap in (cells, 40):
+        def buffers():
+            return (torch.full((batch, cap), -1, dtype=torch.int32).cuda(), torch.zeros(batch, dtype=torch.int32).cuda(),
+                    torch.zeros((batch, cap, 8), dtype=torch.float32).cuda(), torch.full((batch, cells, per), -7.0, dtype=torch.float32).cuda())
+        ci1, cc1, rows1, dec1 = buffers()
+        ci2, cc2, rows2, dec2 = buffers()
+        gu.sync()
+        base = 0
+        for i, (h, w) in enumerate(shapes):
+            abi.check(L.msnh_hip_yolo_decode_candidates(dtype, batch, h, w, cls, gu.ptr(xs[i]), ld, 0.5, anchors[i].ctypes.data_as(fp), ratios[i], version,
+                                                        ctypes.c_void_p(dec1.data_ptr() + base * per * 4) if keep_decoded else None, cells * per, 0.6, gu.ptr(ci1), cap, base,
+                                                        gu.ptr(cc1), gu.ptr(rows1), None))
+            base += 3 * h * w
+        heads = (abi.YoloHead * 3)()
+        base = 0
+        for i, (h, w) in enumerate(shapes):
+            heads[i].x = xs[i].data_ptr(); heads[i].x_ld = ld; heads[i].x_mul = 0.5; heads[i].h = h; heads[i].w = w
+            for k in range(6):
+                heads[i].anchors[k] = float(anchors[i][k])
+            heads[i].ratio = ratios[i]; heads[i].cand_base = base
+            base += 3 * h * w
+        abi.check(L.msnh_hip_yolo_decode_candidates_heads(dtype, batch, cls, 3, heads, version, gu.ptr(dec2) if keep_decoded else None, cells * per, 0.6,
+                                                          gu.ptr(ci2), cap, gu.ptr(cc2), gu.ptr(rows2), None))
+        gu.sync()
+        assert np.array_equal(cc1.cpu().numpy(), cc2.cpu().numpy())
+        assert int(cc1.max()) > 40 and int(cc1.min()) > 0
+        if cap == cells:
+            for b in range(batch):
+                n = int(cc1[b])
+                assert sorted(ci1[b, :n].cpu().numpy().tolist()) == sorted(ci2[b, :n].cpu().numpy().tolist())
+                a1 = rows1[b, :n].cpu().numpy(); a2 = rows2[b, :n].cpu().numpy()
+                assert np.array_equal(a1[np.argsort(a1[:, 7])], a2[np.argsort(a2[:, 7])], equal_nan=True)
+                assert np.array_equal(ci2[b, :n].cpu().numpy().astype(np.float32), a2[:, 7])
+            assert np.array_equal(dec1.cpu().numpy(), dec2.cpu().numpy(), equal_nan=True)
+            assert keep_decoded == bool((dec2.cpu().numpy() != -7.0).any())
+        else:
+            # a list that is too short holds some `cap` of the candidates (which ones depends on timing in both paths): every
+            # entry must be a real candidate with its own row
+            full_idx, full_rows = want_full
+            for b in range(batch):
+                got = ci2[b].cpu().numpy()
+                assert len(set(got.tolist())) == cap and set(got.tolist()) <= set(full_idx[b].tolist())
+                r = rows2[b].cpu().numpy()
+                lookup = {int(c): full_rows[b][k] for k, c in enumerate(full_idx[b])}
+                for k in range(cap):
+                    assert np.array_equal(r[k], lookup[int(got[k])], equal_nan=True)
+        if cap == cells:
+            want_full = ([ci2[b, :int(cc2[b])].cpu().numpy() for b in range(batch)], [rows2[b, :int(cc2[b])].cpu().numpy() for b in range(batch)])
+    bad = (abi.YoloHead * 2)()
+    for i in range(2):
+        bad[i].x = xs[i].data_ptr(); bad[i].x_ld = ld; bad[i].x_mul = 1.0; bad[i].h, bad[i].w = shapes[i]; bad[i].ratio = 8.0; bad[i].cand_base = 5 * i
+    ci2, cc2, rows2, dec2 = buffers()
+    assert L.msnh_hip_yolo_decode_candidates_heads(dtype, batch, cls, 2, bad, version, None, cells * per, 0.6, gu.ptr(ci2), cap, gu.ptr(cc2), gu.ptr(rows2), None) != 0
+    assert L.msnh_hip_yolo_decode_candidates_heads(dtype, batch, cls, 5, bad, version, None, cells * per, 0.6, gu.ptr(ci2), cap, gu.ptr(cc2), gu.ptr(rows2), None) != 0
+
+
 def _ordered_records(kept, total, image):
     rec = kept[:total]
     rec = rec[rec[:, 11] == image]
