@@ -321,6 +321,16 @@ def main():
                 "avg_launch_us": round(conv_ms * 1e3 / max(launches, 1), 2), "flops_per_step": flops / 10,
                 "least_bytes_per_launch": int(conv_bytes / max(launches, 1))}
 
+    # what the matrix cores of this part sustain with nothing in their way (pure MFMA loops, three wavefronts per SIMD as in the
+    # convolution kernels), and the shader clock they hold meanwhile: `peak` above is the published figure at the maximum clock
+    if dtype == "f16":
+        import ctypes
+        from msnhnet_amd import hipabi
+        tf, mhz, sec = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+        hipabi.check(hipabi.lib().msnh_hip_mfma_probe(3, 20000, ctypes.byref(tf), ctypes.byref(mhz), ctypes.byref(sec), None))
+        roofline["mfma_probe"] = {"sustained": round(tf.value, 1), "unit": "TFLOP/s", "shader_mhz": round(mhz.value), "ms": round(sec.value * 1e3, 3),
+                                  "frac_of_sustained": round(achieved / tf.value, 4) if tf.value > 0 else None}
+
     # a network with depthwise convolutions is judged against the HBM roof as well: those launches move
     # (input + output + weights) bytes each and compute next to nothing
     roofline_hbm = None

@@ -348,6 +348,13 @@ size_t msnh_hip_yolo_nms_static_max_bytes(void);
 int msnh_hip_yolo_nms_static(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept,
                              int kept_cap, int *kept_cnt, msnh_stream_t s);
 
+/* Matrix-core ceiling probe (measurement only, no counterpart in the reference): every SIMD runs `iters` rounds of four independent
+ * 32x32x16 float16 MFMAs per wavefront with waves_per_simd (1..8) wavefronts resident, no memory traffic.  Reports the rate
+ * achieved (dense TFLOP/s), the shader clock held meanwhile (shader cycles per tick of the 100 MHz constant clock, read by the
+ * first wavefront) and the launch's duration.  The rate a fully loaded part sustains, not the published peak at the maximum
+ * engine clock, is the practical ceiling of the convolution kernels. */
+int msnh_hip_mfma_probe(int waves_per_simd, int iters, double *tflops, double *shader_mhz, double *seconds, msnh_stream_t s);
+
 /* max |x| over the finite elements of an NHWC tensor, combined into *result with an atomic max
  * (caller zeroes *result).  Used once at load time to calibrate the power-of-two activation scales of the
  * float16 plan; no counterpart in the reference. */

@@ -40,7 +40,7 @@ SYMBOLS = [
     "msnh_hip_conv2d_packed_weight_elems", "msnh_hip_conv2d_pack_weights", "msnh_hip_conv2d_workspace_bytes", "msnh_hip_conv2d", "msnh_hip_letterbox_u8", "msnh_hip_image_u8_to_input",
     "msnh_hip_affine_act", "msnh_hip_add_act", "msnh_hip_copy_channels", "msnh_hip_maxpool", "msnh_hip_avgpool",
     "msnh_hip_upsample_nearest", "msnh_hip_pad", "msnh_hip_slice", "msnh_hip_upsample_bilinear", "msnh_hip_softmax", "msnh_hip_deconv_col2im", "msnh_hip_connected", "msnh_hip_nchw_to_nhwc", "msnh_hip_nhwc_to_nchw", "msnh_hip_yolo_decode", "msnh_hip_yolo_decode_candidates", "msnh_hip_yolo_decode_candidates_heads",
-    "msnh_hip_yolo_gather", "msnh_hip_yolo_nms", "msnh_hip_yolo_nms_workspace_bytes", "msnh_hip_yolo_nms_pair_workspace_bytes", "msnh_hip_yolo_nms_static", "msnh_hip_yolo_nms_static_max_bytes", "msnh_hip_absmax", "msnh_hip_count_nonfinite",
+    "msnh_hip_yolo_gather", "msnh_hip_yolo_nms", "msnh_hip_yolo_nms_workspace_bytes", "msnh_hip_yolo_nms_pair_workspace_bytes", "msnh_hip_yolo_nms_static", "msnh_hip_yolo_nms_static_max_bytes", "msnh_hip_absmax", "msnh_hip_count_nonfinite", "msnh_hip_mfma_probe",
 ]
 
 
@@ -111,6 +111,7 @@ def lib():
     L.msnh_hip_yolo_decode.argtypes = [ci, ci, ci, ci, ci, vp, ci, cf, fp, cf, ci, vp, ll, cf, vp, ci, ci, vp, vp]
     L.msnh_hip_yolo_decode_candidates.argtypes = [ci, ci, ci, ci, ci, vp, ci, cf, fp, cf, ci, vp, ll, cf, vp, ci, ci, vp, vp, vp]
     L.msnh_hip_yolo_decode_candidates_heads.argtypes = [ci, ci, ci, ci, ctypes.POINTER(YoloHead), ci, vp, ll, cf, vp, ci, vp, vp, vp]
+    L.msnh_hip_mfma_probe.argtypes = [ci, ci, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), vp]
     L.msnh_hip_yolo_gather.argtypes = [ci, ci, vp, ll, vp, ci, vp, vp, vp]
     L.msnh_hip_yolo_nms.argtypes = [ci, ci, vp, ci, vp, cf, vp, ci, vp, vp, sz, vp]
     L.msnh_hip_yolo_nms_workspace_bytes.argtypes = [ci, ci, ci]
