@@ -23,7 +23,8 @@
 namespace msnh {
 
 // DBG (timing experiments only, results are then meaningless; 0 in every instantiation the library ships): bit 0 leaves out the
-// loads of the main loop, bit 1 its LDS fragment reads, bit 2 its barrier, bit 3 its MFMAs, bit 4 the epilogue, bit 5 the prologue's loads.
+// loads of the main loop, bit 1 its LDS fragment reads, bit 2 its barrier, bit 3 its MFMAs, bit 4 the epilogue, bit 5 the prologue's loads;
+// bit 6 makes the first wavefront write the shader-clock and constant-clock ticks its main loop took to IgemmArgs::ws (two 64-bit words).
 //
 // KG = 2 splits the four k-blocks of every tap step between two groups of wavefronts that share the same WM x WN grid of wave
 // tiles: a wavefront then owns a 64 x 64 tile over half of K instead of a 32 x 64 tile over all of it, which takes a third off
@@ -215,6 +216,8 @@ void convPatch8Kernel(IgemmArgs a)
     readA(0, std::integral_constant<int, 0>());
     readB(patchOff0, 0, 0u, std::integral_constant<int, 0>());
 
+    unsigned long long dbgT0 = 0, dbgR0 = 0;
+    if constexpr (DBG & 64) { dbgT0 = __builtin_readcyclecounter(); dbgR0 = __builtin_amdgcn_s_memrealtime(); }
     unsigned curA = 0, nxtA = A_STAGE, nnA = (NSA - 1) * A_STAGE;
     unsigned curP = patchOff0, othP = patchStages > 1 ? patchOff0 + patchBytes : patchOff0;
     int it = 0;
@@ -288,6 +291,15 @@ void convPatch8Kernel(IgemmArgs a)
     }
     dmaWait<0>();
     __syncthreads();
+    if constexpr (DBG & 64)
+    {
+        const unsigned long long t1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+        if (logical == 0 && tid == 0)
+        {
+            reinterpret_cast<unsigned long long *>(a.ws)[0] = t1 - dbgT0;
+            reinterpret_cast<unsigned long long *>(a.ws)[1] = r1 - dbgR0;
+        }
+    }
 
     if constexpr (DBG & 16)
     {
