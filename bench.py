@@ -75,7 +75,7 @@ def cpu_baseline(arch, size, tmp, seed, budget_s=30.0):
 # HBM bytes per convolution launch (fetch + write), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script,
 # each scaled by what the same counter reads for a plain copy kernel of known size (fetch x2.0, write x1.0); the runs
 # and their summary are in profiles/conv_igemm_yolov3_608_f16_b8.md.  None for workloads that were not profiled.
-HBM_BYTES_PER_CONV_LAUNCH = {("yolov3", "f16", 8): int((38.80 + 18.00) * 2**20)}
+HBM_BYTES_PER_CONV_LAUNCH = {("yolov3", "f16", 8): int((36.68 + 18.10) * 2**20)}
 # The same for the depthwise launches (the dominant bandwidth-bound kernel of a network that has them); runs and summary in
 # profiles/hbm_kernels_mobilenetv2_b64_yolov4_b16.md.
 HBM_BYTES_PER_DEPTHWISE_LAUNCH = {("mobilenetv2", "f16", 64): int((27.07 + 16.53) * 2**20)}
