@@ -7,6 +7,9 @@ A step is one forward of one batch through NetBuilder's device-resident path (in
 launch of the planned graph, and for detection networks the candidate compaction on the device plus copy-back,
 sort and NMS on the host, so that a step ends with the boxes (or logits) in host memory.  Prints ONE JSON line.
 `value` is the whole-job rate over the K timed steps; the median of the per-step times is reported beside it.
+By default the K steps are dealt round-robin to two instances of the network (--instances; each a NetBuilder with its own
+stream, driven by its own host thread, two batches in flight each), which is how a server keeps the device busy across
+the gaps between the launches of one forward; `one_instance_images_per_s` of the same line is the rate of one instance alone.
 
     python bench.py --conv-shape b,c,h,w,oc,k,stride [--tile n] [--reps 20] [--residual] [--conv-dtype f16|f32]
 
@@ -171,6 +174,11 @@ def main():
     ap.add_argument("--nms", default="auto", choices=["host", "auto", "device"],
                     help="detection workloads: sort + NMS on the host, on the device, or (library default) on the device while the "
                          "previous result had at most 2048 candidates per image -- the seeded weights give 11k, so auto means host here")
+    ap.add_argument("--instances", type=int, default=2,
+                    help="network instances on the GPU, each with its own stream, arena and packed weights, fed round-robin by one host thread each "
+                         "(netapi.NetGroup; device-resident input only).  The device runs their forwards side by side, which fills the launch gaps, "
+                         "prologues and write bursts that a single stream leaves open.  1 = one instance, two batches in flight on one stream")
+    ap.add_argument("--depth", type=int, default=2, help="--instances > 1: batches in flight per instance (detectors; a classifier has one)")
     ap.add_argument("--per-op", default=None, metavar="FILE",
                     help="also write the per-launch table (every launch of the plan timed on its own with device events: microseconds, "
                          "algorithmic TFLOP/s and GB/s with every tensor counted once) to FILE")
@@ -192,7 +200,12 @@ def main():
     tmp = tempfile.mkdtemp(prefix="msnh_bench_")
     netp, binp, g = zoo.write_model(a.workload, tmp, batch, size, seed=a.seed)
     netapi.set_device_nms({"host": 0, "auto": 1, "device": 2}[a.nms])
-    net = netapi.Net(netp, binp, fp16=(dtype == "f16"))
+    group = None
+    if a.instances > 1 and a.input == "device":
+        group = netapi.NetGroup(netp, binp, instances=a.instances, depth=a.depth, fp16=(dtype == "f16"))
+        net = group.nets[0]
+    else:
+        net = netapi.Net(netp, binp, fp16=(dtype == "f16"))
     detect = a.workload.startswith("yolo")
 
     if a.copy_probe:
@@ -227,7 +240,9 @@ def main():
 
     # device-resident input: the batch is written once into the network's own input buffer (msnhnet_device_input, the documented
     # serving path: a producer on the device writes there) and every step runs on it; no copy of the input inside the timed region
-    if host_u8 is None and host_x is None:
+    if group is not None:
+        group.prime(dev_in)
+    elif host_u8 is None and host_x is None:
         net.enqueue(dev_in)
         _ = net.fetch_yolo() if detect else net.fetch_classify()
 
@@ -239,13 +254,22 @@ def main():
 
     on_device = [0]
 
-    def run_steps(k, stamps=None, host=None):
+    def run_steps(k, stamps=None, host=None, use_group=True):
         """k forwards + k result fetches.  Detection keeps two batches in flight: while the host sorts and
         suppresses the boxes of batch i the device already runs batch i+1.  stamps collects the time at which each
         step's result reached the host."""
         out = None
         tick = (lambda: stamps.append(time.perf_counter())) if stamps is not None else (lambda: None)
-        if host is not None:
+        if group is not None and use_group and host is None:
+            # every instance's thread keeps `depth` batches in flight; results come back in submission order
+            for _ in range(k):
+                group.submit(None)
+            group.flush()
+            for _ in range(k):
+                out = group.fetch()
+                tick()
+            on_device[0] = None
+        elif host is not None:
             for _ in range(k):
                 out = net.run_yolo(host) if detect else net.run_classify(host)
                 tick()
@@ -285,11 +309,25 @@ def main():
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     steps_on_device = on_device[0]
+    single_rate = None
+    if group is not None:
+        # the same run with one instance alone (two batches in flight on one stream), for comparison
+        on_device[0] = 0
+        k1 = min(a.steps, 100)
+        ts = time.perf_counter()
+        run_steps(k1, use_group=False)
+        net.sync()
+        single_rate = round(batch * k1 / (time.perf_counter() - ts), 2)
     gc.enable()
-    slow = [i for i, v in enumerate(np.diff(np.array([t0] + stamps)) * 1e3) if v > 5.0]
     marker()
     ms_per_step = dt / a.steps * 1e3
     per_step = np.diff(np.array([t0] + stamps)) * 1e3
+    if group is not None and len(stamps) > 2 * a.instances:
+        # results of different instances arrive in bursts (they are handed out in submission order): the time between results is
+        # taken over one round of the instances
+        st = np.array([t0] + stamps)
+        per_step = (st[a.instances:] - st[:-a.instances]) / a.instances * 1e3
+    slow = [i for i, v in enumerate(per_step) if v > 5.0]
     # (pipelined detection: the first interval holds two forwards, every later one is a steady-state step)
     ms_median = float(np.median(per_step[1:])) if len(per_step) > 1 else float(per_step[0])
     steady = per_step[1:] if len(per_step) > 1 else per_step
@@ -345,7 +383,10 @@ def main():
            "unit": "images/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4),
            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
            "config": {"workload": f"{a.workload}-{size} {dtype} batch {batch}, seeded He-normal weights, U[0,1) input, "
-                                  f"{'input resident in the network input buffer on the device' if a.input == 'device' else a.input + ' input'} -> {'boxes' if detect else 'logits'} on host",
+                                  f"{'input resident in the network input buffer on the device' if a.input == 'device' else a.input + ' input'} -> {'boxes' if detect else 'logits'} on host"
+                                  + (f"; {a.instances} network instances fed round-robin, {group.depth} batch(es) in flight each, a step = one batch of one instance "
+                                     f"(ms_per_step = time between results)" if group is not None else ""),
+                      "instances": a.instances if group is not None else 1, "one_instance_images_per_s": single_rate, "batches_in_flight": (a.instances * group.depth) if group is not None else (2 if detect else 1),
                       "input": a.input, "seed": a.seed, "ms_per_step_median": round(ms_median, 4), "ms_per_step_percentiles_0_10_50_90_99_100": ms_spread, "steps_over_5ms": slow, "device_launches_per_step": n_all // 10,
                       "device_ms_per_step_eager": round(gpu_only_ms, 4), "host_f32_images_per_s": host_rate},
            "roofline": roofline}
@@ -358,6 +399,8 @@ def main():
     if a.per_op:
         with open(a.per_op, "w") as f:
             f.write(net.profile_each_op(20))
+    if group is not None:
+        group.close()
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(a.workload, size, tmp, a.seed)
     print(json.dumps(res))

@@ -8,6 +8,7 @@
 #include <fstream>
 #include <functional>
 #include <limits>
+#include <map>
 #include <mutex>
 #include <numeric>
 #include <sstream>
@@ -727,13 +728,17 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
     std::vector<size_t> tunedOps;
     for (size_t i = 0; i < ops.size(); ++i)
         if (tunable(ops[i])) tunedOps.push_back(i);
-    if (!cacheFile.empty())
-    {
+    // A recorded search: header, then "<signature> | <algo> <tile>" per tunable launch in plan order; any mismatch discards it.
+    // Two sources: what an earlier load of a plan with the same launches found in this process (instances of one network then run
+    // the same kernels and give the same bits), and the cache file beside the weights.
+    static std::mutex memoMutex;
+    static std::map<std::string, std::string> memoText;
+    const std::string memoKey = tuneHeader(nTiles, preferWinograd) + " " + std::to_string(structureHash());
+    const auto adopt = [&](std::istream &f) -> bool {
         // file: header, then "<signature> | <algo> <tile>" per tunable launch in plan order; any mismatch discards the file
-        std::ifstream f(cacheFile);
         std::string line;
         std::vector<std::pair<int, int>> picks;
-        bool ok = f.is_open() && std::getline(f, line) && line == tuneHeader(nTiles, preferWinograd);
+        bool ok = static_cast<bool>(std::getline(f, line)) && line == tuneHeader(nTiles, preferWinograd);
         for (size_t k = 0; ok && k < tunedOps.size(); ++k)
         {
             ok = static_cast<bool>(std::getline(f, line));
@@ -765,9 +770,44 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
             if (ok)
             {
                 if (need > _convWorkspace.bytes()) _convWorkspace.alloc(need);
-                return;
+                return true;
             }
             for (size_t k = 0; k < tunedOps.size(); ++k) { ops[tunedOps[k]].algo = before[k].first; ops[tunedOps[k]].tile = before[k].second; }
+        }
+        return false;
+    };
+    if (!cacheFile.empty())
+    {
+        std::ifstream f(cacheFile);
+        if (f.is_open() && adopt(f))
+        {
+            std::ifstream again(cacheFile);
+            std::ostringstream all;
+            all << again.rdbuf();
+            std::lock_guard<std::mutex> lk(memoMutex);
+            memoText[memoKey] = all.str();
+            return;
+        }
+    }
+    {
+        std::string text;
+        {
+            std::lock_guard<std::mutex> lk(memoMutex);
+            const auto it = memoText.find(memoKey);
+            if (it != memoText.end()) text = it->second;
+        }
+        if (!text.empty())
+        {
+            std::istringstream f(text);
+            if (adopt(f))
+            {
+                if (!cacheFile.empty())
+                {
+                    std::ofstream out(cacheFile, std::ios::trunc);
+                    if (out.is_open()) out << text;
+                }
+                return;
+            }
         }
     }
 
@@ -863,18 +903,21 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
     }
     msnh_hip_event_destroy(e0);
     msnh_hip_event_destroy(e1);
+    std::ostringstream text;
+    text << tuneHeader(nTiles, preferWinograd) << "\n";
+    for (size_t i : tunedOps)
+    {
+        // (the signature is taken with the searched choice in place: it does not depend on algo / tile)
+        text << tuneSignature(*this, ops[i]) << " | " << ops[i].algo << ' ' << ops[i].tile << "\n";
+    }
+    {
+        std::lock_guard<std::mutex> lk(memoMutex);
+        memoText[memoKey] = text.str();
+    }
     if (!cacheFile.empty())
     {
         std::ofstream f(cacheFile, std::ios::trunc);
-        if (f.is_open())
-        {
-            f << tuneHeader(nTiles, preferWinograd) << "\n";
-            for (size_t i : tunedOps)
-            {
-                // (the signature is taken with the searched choice in place: it does not depend on algo / tile)
-                f << tuneSignature(*this, ops[i]) << " | " << ops[i].algo << ' ' << ops[i].tile << "\n";
-            }
-        }
+        if (f.is_open()) f << text.str();
     }
 }
 

@@ -369,3 +369,98 @@ class Net:
 
     def gpu_inference_time_ms(self):
         return float(self.L.msnhnet_gpu_inference_time(self.h))
+
+
+class NetGroup:
+    """Several instances of one network on one GPU, fed round-robin: a throughput configuration for serving.
+
+    Each instance is a NetBuilder of its own (own stream, activation arena, captured graph and packed weights), driven by one host
+    thread that enqueues a batch and fetches the result of an earlier one, so that `instances * depth` batches are in flight.  The
+    device then runs the forwards of different instances side by side: the launch gaps, prologues and write bursts of one
+    forward's kernels are filled by another's, which a single stream cannot do.  Results come back in submission order.
+
+    submit(ptr) hands the next batch to the next instance: `ptr` is a device pointer to the float32 NCHW batch (copied into the
+    instance's input buffer on its stream) or None to run on what that buffer holds (prime() fills every instance's buffer once).
+    fetch() returns the oldest outstanding result (boxes per image for a detector, logits for a classifier)."""
+
+    def __init__(self, msnhnet_path, msnhbin_path, instances=2, depth=2, fp16=False):
+        import queue
+        import threading
+        self.nets = [Net(msnhnet_path, msnhbin_path, fp16=fp16) for _ in range(instances)]
+        last = self.nets[0].layer_info(self.nets[0].num_layers() - 1)["type"]
+        self.detect = last == "yoloout"
+        self.depth = max(1, depth if self.detect else 1)      # a classifier's result is read from its output tensor: one forward at a time
+        self._in = [queue.Queue() for _ in self.nets]
+        self._out = [queue.Queue() for _ in self.nets]
+        self._submitted = 0
+        self._fetched = 0
+        self._threads = [threading.Thread(target=self._drive, args=(i,), daemon=True) for i in range(instances)]
+        for t in self._threads:
+            t.start()
+
+    def _drive(self, i):
+        net, inq, outq = self.nets[i], self._in[i], self._out[i]
+        fetch = net.fetch_yolo if self.detect else net.fetch_classify
+        in_flight = 0
+        while True:
+            job = inq.get()
+            try:
+                if job == "stop" or job == "flush":
+                    while in_flight:
+                        outq.put(fetch())
+                        in_flight -= 1
+                    if job == "stop":
+                        return
+                    outq.put("flushed")
+                    continue
+                net.enqueue(job[0])
+                in_flight += 1
+                if in_flight == self.depth:
+                    outq.put(fetch())
+                    in_flight -= 1
+            except Exception as e:         # hand the error to whoever waits for the result
+                outq.put(e)
+                if job == "stop":
+                    return
+
+    def prime(self, device_ptr):
+        """One forward of the batch at device_ptr on every instance (its input buffer then holds that batch); returns the results."""
+        return [self._one(n, device_ptr) for n in self.nets]
+
+    def _one(self, net, device_ptr):
+        net.enqueue(device_ptr)
+        return net.fetch_yolo() if self.detect else net.fetch_classify()
+
+    def submit(self, device_ptr=None):
+        self._in[self._submitted % len(self.nets)].put((device_ptr,))
+        self._submitted += 1
+
+    def flush(self):
+        """Makes every instance fetch what it still has in flight (otherwise an instance keeps depth - 1 results back until more work comes)."""
+        for q in self._in:
+            q.put("flush")
+
+    def fetch(self):
+        if self._fetched >= self._submitted:
+            raise RuntimeError("nothing outstanding")
+        q = self._out[self._fetched % len(self.nets)]
+        while True:
+            r = q.get()
+            if isinstance(r, str):          # a flush marker: everything submitted before it has been delivered
+                continue
+            break
+        if isinstance(r, Exception):
+            raise r
+        self._fetched += 1
+        return r
+
+    def last_nms_on_device(self):
+        return sum(n.last_nms_on_device() for n in self.nets)
+
+    def close(self):
+        for q in self._in:
+            q.put("stop")
+        for t in self._threads:
+            t.join(timeout=30)
+        for n in self.nets:
+            n.close()

@@ -553,3 +553,49 @@ def test_cpu_entry_points_refuse():
         m.run_classify_cpu(np.zeros(3 * 224 * 224, np.float32))
     with pytest.raises(netapi.MsnhnetError, match="input image size err. Needed :150528 given :10"):
         m.run_classify(np.zeros(10, np.float32))
+
+
+@pytest.mark.parametrize("arch,size,batch,instances,depth", [("yolov3", 96, 2, 2, 2), ("yolov3", 96, 2, 3, 1), ("resnet18", 224, 2, 2, 2)])
+def test_net_group_results_in_submission_order(arch, size, batch, instances, depth):
+    """netapi.NetGroup: several instances of a network fed round-robin by one host thread each return, in submission order, exactly
+    what one instance returns for each of the submitted batches (distinct inputs, so a swapped or repeated result shows), also for the
+    batches an instance still holds in flight when flush() is called; an error inside a worker surfaces in fetch()"""
+    net, binp, g = nu.model(arch, batch, size, seed=11)
+    xs = [zoo.seeded_input(batch, 3, size, size, seed=20 + i) for i in range(7)]
+    xd = [torch.from_numpy(x).cuda() for x in xs]
+    one = netapi.Net(net, binp, fp16=True)
+    detect = arch.startswith("yolo")
+    want = [one.run_yolo(x) if detect else one.run_classify(x) for x in xs]
+    grp = netapi.NetGroup(net, binp, instances=instances, depth=depth, fp16=True)
+    try:
+        assert grp.detect == detect and len(grp.nets) == instances
+        first = grp.prime(xd[0].data_ptr())
+        for r in first:
+            if detect:
+                assert all(np.array_equal(a, b, equal_nan=True) for a, b in zip(r, want[0]))
+            else:
+                assert np.array_equal(r, want[0])
+        for rounds in range(2):
+            for t in xd:
+                grp.submit(t.data_ptr())
+            grp.flush()
+            for i in range(len(xd)):
+                got = grp.fetch()
+                if detect:
+                    assert len(got) == batch
+                    for a, b in zip(got, want[i]):
+                        assert np.array_equal(a, b, equal_nan=True), (rounds, i)
+                else:
+                    assert np.array_equal(got, want[i]), (rounds, i)
+        with pytest.raises(RuntimeError):
+            grp.fetch()                      # nothing outstanding
+        # on what the input buffers hold: instance k saw batch 6 - ((7 - 1 - k) % instances) ... simply: every result is one of the submitted ones
+        grp.submit(None)
+        grp.flush()
+        got = grp.fetch()
+        if detect:
+            assert any(all(np.array_equal(a, b, equal_nan=True) for a, b in zip(got, w)) for w in want)
+        else:
+            assert any(np.array_equal(got, w) for w in want)
+    finally:
+        grp.close()
