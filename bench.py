@@ -7,7 +7,7 @@ A step is one forward of one batch through NetBuilder's device-resident path (in
 launch of the planned graph, and for detection networks the candidate compaction on the device plus copy-back,
 sort and NMS on the host, so that a step ends with the boxes (or logits) in host memory.  Prints ONE JSON line.
 `value` is the whole-job rate over the K timed steps; the median of the per-step times is reported beside it.
-By default the K steps are dealt round-robin to two instances of the network (--instances; each a NetBuilder with its own
+By default the K steps are dealt round-robin to three instances of the network (--instances; each a NetBuilder with its own
 stream, driven by its own host thread, two batches in flight each), which is how a server keeps the device busy across
 the gaps between the launches of one forward; `one_instance_images_per_s` of the same line is the rate of one instance alone.
 
@@ -174,7 +174,7 @@ def main():
     ap.add_argument("--nms", default="auto", choices=["host", "auto", "device"],
                     help="detection workloads: sort + NMS on the host, on the device, or (library default) on the device while the "
                          "previous result had at most 2048 candidates per image -- the seeded weights give 11k, so auto means host here")
-    ap.add_argument("--instances", type=int, default=2,
+    ap.add_argument("--instances", type=int, default=3,
                     help="network instances on the GPU, each with its own stream, arena and packed weights, fed round-robin by one host thread each "
                          "(netapi.NetGroup; device-resident input only).  The device runs their forwards side by side, which fills the launch gaps, "
                          "prologues and write bursts that a single stream leaves open.  1 = one instance, two batches in flight on one stream")
