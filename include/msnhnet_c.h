@@ -163,6 +163,30 @@ int msnhnet_set_input_image(msnhnet_t net, int index, const unsigned char *rgb_h
 int msnhnet_boxes_to_image(float *boxes, long long count, int net_w, int net_h, int org_w, int org_h, int padded);
 long long msnhnet_time_detail(msnhnet_t net, char *dst, long long cap);       /* NetBuilder::getTimeDetail */
 
+/* Several instances of one network on one GPU, fed round-robin: the throughput arrangement for serving (no counterpart in the
+ * reference, whose callers would create several NetBuilder objects and threads themselves).  Each instance is a NetBuilder with
+ * its own stream, arena, graph and packed weights, driven by its own host thread with `depth` batches in flight (detectors 1 or
+ * 2, classifiers 1); the device runs the forwards of different instances side by side, which fills the gaps between the launches
+ * of one forward.  The switches of msnhnet_set_* apply as for msnhnet_create + build + load.
+ *   msnhnet_group_prime  : one forward of the device-resident float32 NCHW batch on every instance, on the calling thread
+ *                          (fills each instance's input buffer, captures its graph); call once before submitting.
+ *   msnhnet_group_submit : hands the next batch to the next instance; device_input as for msnhnet_enqueue (NULL = run on what
+ *                          the instance's input buffer holds), valid until the batch's result has been fetched.
+ *   msnhnet_group_flush  : every instance fetches what it still holds in flight (it otherwise keeps depth - 1 results back).
+ *   msnhnet_group_fetch_*: the oldest outstanding result, outputs as for msnhnet_fetch_*; blocks until it is there; an error
+ *                          raised inside an instance's thread is reported by the fetch of the batch it belongs to.
+ *   msnhnet_group_instance: the NetBuilder of instance i (owned by the group) for the query calls: dims, plan detail, profiles. */
+typedef void *msnhnet_group_t;
+int msnhnet_group_create(const char *msnhnet_path, const char *msnhbin_path, int instances, int depth, msnhnet_group_t *group);
+int msnhnet_group_destroy(msnhnet_group_t group);
+int msnhnet_group_info(msnhnet_group_t group, int *instances, int *depth, int *is_detector);
+int msnhnet_group_instance(msnhnet_group_t group, int i, msnhnet_t *net);
+int msnhnet_group_prime(msnhnet_group_t group, const float *device_input);
+int msnhnet_group_submit(msnhnet_group_t group, const float *device_input);
+int msnhnet_group_flush(msnhnet_group_t group);
+int msnhnet_group_fetch_classify(msnhnet_group_t group, float *out, long long cap, long long *n_out);
+int msnhnet_group_fetch_yolo(msnhnet_group_t group, int *counts, float *boxes, long long cap_boxes, long long *total);
+
 #ifdef __cplusplus
 }
 #endif

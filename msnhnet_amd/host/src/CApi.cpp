@@ -6,6 +6,7 @@
 #include <memory>
 #include <string>
 #include "Msnhnet/net/MsnhNetBuilder.h"
+#include "Msnhnet/net/MsnhNetGroup.h"
 
 using namespace Msnhnet;
 
@@ -506,6 +507,59 @@ float msnhnet_gpu_inference_time(msnhnet_t net)
     float t = -1.f;
     guarded([&] { t = nb(net).getGpuInferenceTime(); });
     return t;
+}
+
+}
+
+extern "C" {
+
+static NetGroup &ng(msnhnet_group_t g)
+{
+    if (g == nullptr) MSNH_THROW("group handle is NULL");
+    return *static_cast<NetGroup *>(g);
+}
+
+int msnhnet_group_create(const char *msnhnet_path, const char *msnhbin_path, int instances, int depth, msnhnet_group_t *group)
+{
+    return guarded([&] {
+        if (!msnhnet_path || !msnhbin_path || !group) MSNH_THROW("NULL argument");
+        *group = new NetGroup(msnhnet_path, msnhbin_path, instances, depth);
+    });
+}
+
+int msnhnet_group_destroy(msnhnet_group_t group) { return guarded([&] { delete static_cast<NetGroup *>(group); }); }
+
+int msnhnet_group_info(msnhnet_group_t group, int *instances, int *depth, int *is_detector)
+{
+    return guarded([&] {
+        NetGroup &g = ng(group);
+        if (instances) *instances = g.instances();
+        if (depth) *depth = g.depth();
+        if (is_detector) *is_detector = g.isDetector() ? 1 : 0;
+    });
+}
+
+int msnhnet_group_instance(msnhnet_group_t group, int i, msnhnet_t *net)
+{
+    return guarded([&] {
+        if (!net) MSNH_THROW("net pointer is NULL");
+        if (i < 0 || i >= ng(group).instances()) MSNH_THROW("no such instance");
+        *net = &ng(group).instance(i);
+    });
+}
+
+int msnhnet_group_prime(msnhnet_group_t group, const float *device_input) { return guarded([&] { ng(group).prime(device_input); }); }
+int msnhnet_group_submit(msnhnet_group_t group, const float *device_input) { return guarded([&] { ng(group).submit(device_input); }); }
+int msnhnet_group_flush(msnhnet_group_t group) { return guarded([&] { ng(group).flush(); }); }
+
+int msnhnet_group_fetch_classify(msnhnet_group_t group, float *out, long long cap, long long *n_out)
+{
+    return guarded([&] { copyOut(ng(group).fetchClassify(), out, cap, n_out); });
+}
+
+int msnhnet_group_fetch_yolo(msnhnet_group_t group, int *counts, float *boxes, long long cap_boxes, long long *total)
+{
+    return guarded([&] { packBoxes(ng(group).fetchYolo(), counts, boxes, cap_boxes, total); });
 }
 
 }

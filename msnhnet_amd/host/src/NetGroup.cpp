@@ -1,0 +1,157 @@
+#include "Msnhnet/net/MsnhNetGroup.h"
+#include "Msnhnet/layers/MsnhLayers.h"
+
+namespace Msnhnet
+{
+NetGroup::NetGroup(const std::string &msnhnetPath, const std::string &msnhbinPath, int instances, int depth)
+{
+    if (instances < 1 || instances > 16) MSNH_THROW("NetGroup: 1 to 16 instances");
+    for (int i = 0; i < instances; ++i)
+    {
+        std::unique_ptr<Lane> lane(new Lane());
+        lane->net.reset(new NetBuilder());
+        lane->net->buildNetFromMsnhNet(msnhnetPath);
+        lane->net->loadWeightsFromMsnhBin(msnhbinPath);
+        _lanes.push_back(std::move(lane));
+    }
+    Network *n = _lanes[0]->net->getNet();
+    _detect = !n->layers.empty() && n->layers.back()->type() == LayerType::YOLO_OUT;
+    _depth = _detect ? std::max(1, std::min(depth, 2)) : 1;
+    for (std::unique_ptr<Lane> &lane : _lanes)
+    {
+        Lane *l = lane.get();
+        l->thread = std::thread([this, l] { drive(*l); });
+    }
+}
+
+NetGroup::~NetGroup()
+{
+    for (std::unique_ptr<Lane> &lane : _lanes)
+    {
+        {
+            std::lock_guard<std::mutex> lk(lane->m);
+            lane->in.push_back({2, nullptr});
+        }
+        lane->cvIn.notify_one();
+    }
+    for (std::unique_ptr<Lane> &lane : _lanes)
+        if (lane->thread.joinable()) lane->thread.join();
+}
+
+// The instance's thread: enqueue the next batch, and once `depth` are in flight fetch the oldest.
+void NetGroup::drive(Lane &lane)
+{
+    int inFlight = 0;
+    const auto fetchOne = [&] {
+        Result r;
+        try
+        {
+            if (_detect) r.boxes = lane.net->fetchYolo();
+            else r.logits = lane.net->fetchClassify();
+        }
+        catch (...) { r.error = std::current_exception(); }
+        --inFlight;
+        {
+            std::lock_guard<std::mutex> lk(lane.m);
+            lane.out.push_back(std::move(r));
+        }
+        lane.cvOut.notify_one();
+    };
+    for (;;)
+    {
+        Job job;
+        {
+            std::unique_lock<std::mutex> lk(lane.m);
+            lane.cvIn.wait(lk, [&] { return !lane.in.empty(); });
+            job = lane.in.front();
+            lane.in.pop_front();
+        }
+        if (job.kind != 0)
+        {
+            while (inFlight > 0) fetchOne();
+            if (job.kind == 2) return;
+            continue;
+        }
+        try
+        {
+            lane.net->enqueueForward(job.input);
+            ++inFlight;
+        }
+        catch (...)
+        {
+            // the batch has no result of its own: its place in the order carries the error
+            Result r;
+            r.error = std::current_exception();
+            {
+                std::lock_guard<std::mutex> lk(lane.m);
+                lane.out.push_back(std::move(r));
+            }
+            lane.cvOut.notify_one();
+            continue;
+        }
+        if (inFlight == _depth) fetchOne();
+    }
+}
+
+void NetGroup::prime(const float *deviceInput)
+{
+    if (outstanding() != 0) MSNH_THROW("NetGroup: fetch the outstanding results before prime()");
+    for (std::unique_ptr<Lane> &lane : _lanes)
+    {
+        lane->net->enqueueForward(deviceInput);
+        if (_detect) lane->net->fetchYolo();
+        else lane->net->fetchClassify();
+    }
+}
+
+void NetGroup::submit(const float *deviceInput)
+{
+    Lane &lane = *_lanes[static_cast<size_t>(_submitted % static_cast<long long>(_lanes.size()))];
+    {
+        std::lock_guard<std::mutex> lk(lane.m);
+        lane.in.push_back({0, deviceInput});
+    }
+    lane.cvIn.notify_one();
+    ++_submitted;
+}
+
+void NetGroup::flush()
+{
+    for (std::unique_ptr<Lane> &lane : _lanes)
+    {
+        {
+            std::lock_guard<std::mutex> lk(lane->m);
+            lane->in.push_back({1, nullptr});
+        }
+        lane->cvIn.notify_one();
+    }
+}
+
+NetGroup::Result NetGroup::take()
+{
+    if (outstanding() <= 0) MSNH_THROW("NetGroup: nothing outstanding");
+    Lane &lane = *_lanes[static_cast<size_t>(_fetched % static_cast<long long>(_lanes.size()))];
+    Result r;
+    {
+        std::unique_lock<std::mutex> lk(lane.m);
+        lane.cvOut.wait(lk, [&] { return !lane.out.empty(); });
+        r = std::move(lane.out.front());
+        lane.out.pop_front();
+    }
+    ++_fetched;
+    if (r.error) std::rethrow_exception(r.error);
+    return r;
+}
+
+std::vector<std::vector<YoloBox>> NetGroup::fetchYolo()
+{
+    if (!_detect) MSNH_THROW("not a yolo net");
+    return take().boxes;
+}
+
+std::vector<float> NetGroup::fetchClassify()
+{
+    if (_detect) MSNH_THROW("NetGroup: a detector's results are fetched with fetchYolo");
+    return take().logits;
+}
+}

@@ -19,6 +19,8 @@ SYMBOLS = [
     "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
     "msnhnet_enqueue", "msnhnet_sync", "msnhnet_fetch_classify", "msnhnet_fetch_yolo", "msnhnet_gpu_inference_time", "msnhnet_time_detail",
     "msnhnet_profile_ops", "msnhnet_profile_ops_bytes", "msnhnet_profile_each_op", "msnhnet_yolo_max_boxes", "msnhnet_nms",
+    "msnhnet_group_create", "msnhnet_group_destroy", "msnhnet_group_info", "msnhnet_group_instance", "msnhnet_group_prime", "msnhnet_group_submit",
+    "msnhnet_group_flush", "msnhnet_group_fetch_classify", "msnhnet_group_fetch_yolo",
 ]
 
 LAYER_TYPE = {0: "conv", 1: "deconv", 2: "connect", 3: "maxpool", 4: "localavgpool", 5: "globalavgpool", 6: "softmax", 8: "route", 9: "varop",
@@ -103,6 +105,15 @@ def lib():
     L.msnhnet_sync.argtypes = [vp]
     L.msnhnet_fetch_classify.argtypes = [vp, fp, ll, llp]
     L.msnhnet_fetch_yolo.argtypes = [vp, ip, fp, ll, llp]
+    L.msnhnet_group_create.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ci, ci, ctypes.POINTER(vp)]
+    L.msnhnet_group_destroy.argtypes = [vp]
+    L.msnhnet_group_info.argtypes = [vp, ip, ip, ip]
+    L.msnhnet_group_instance.argtypes = [vp, ci, ctypes.POINTER(vp)]
+    L.msnhnet_group_prime.argtypes = [vp, vp]
+    L.msnhnet_group_submit.argtypes = [vp, vp]
+    L.msnhnet_group_flush.argtypes = [vp]
+    L.msnhnet_group_fetch_classify.argtypes = [vp, fp, ll, llp]
+    L.msnhnet_group_fetch_yolo.argtypes = [vp, ip, fp, ll, llp]
     L.msnhnet_profile_ops.argtypes = [vp, ci, ci, fp, ip, ctypes.POINTER(ctypes.c_double)]
     L.msnhnet_profile_ops_bytes.argtypes = [vp, ci, ci, fp, ip, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     L.msnhnet_profile_each_op.argtypes = [vp, ci, cp, ll]
@@ -177,9 +188,19 @@ class Net:
         if msnhbin_path:
             self.load(msnhbin_path)
 
+    @classmethod
+    def borrowed(cls, handle):
+        """A view of a NetBuilder that somebody else owns (an instance of a NetGroup): every query works, close() leaves it alone."""
+        self = cls.__new__(cls)
+        self.L = lib()
+        self.h = handle
+        self._borrowed = True
+        return self
+
     def close(self):
         if self.h:
-            self.L.msnhnet_destroy(self.h)
+            if not getattr(self, "_borrowed", False):
+                self.L.msnhnet_destroy(self.h)
             self.h = ctypes.c_void_p()
 
     def __del__(self):
@@ -372,95 +393,78 @@ class Net:
 
 
 class NetGroup:
-    """Several instances of one network on one GPU, fed round-robin: a throughput configuration for serving.
+    """Several instances of one network on one GPU, fed round-robin: a throughput configuration for serving (msnhnet_group_* of
+    include/msnhnet_c.h; the host threads and queues live in the library).
 
     Each instance is a NetBuilder of its own (own stream, activation arena, captured graph and packed weights), driven by one host
     thread that enqueues a batch and fetches the result of an earlier one, so that `instances * depth` batches are in flight.  The
     device then runs the forwards of different instances side by side: the launch gaps, prologues and write bursts of one
     forward's kernels are filled by another's, which a single stream cannot do.  Results come back in submission order.
 
-    submit(ptr) hands the next batch to the next instance: `ptr` is a device pointer to the float32 NCHW batch (copied into the
-    instance's input buffer on its stream) or None to run on what that buffer holds (prime() fills every instance's buffer once).
-    fetch() returns the oldest outstanding result (boxes per image for a detector, logits for a classifier)."""
+    prime(ptr) runs the device-resident float32 NCHW batch at `ptr` once on every instance (call it before the first submit).
+    submit(ptr) hands the next batch to the next instance: a device pointer (copied into the instance's input buffer on its
+    stream; keep it valid until the result is fetched) or None to run on what that buffer holds.  flush() makes the instances
+    deliver what they still hold in flight.  fetch() returns the oldest outstanding result (boxes per image for a detector,
+    logits for a classifier); an error raised inside an instance's thread surfaces in the fetch of its batch."""
 
     def __init__(self, msnhnet_path, msnhbin_path, instances=2, depth=2, fp16=False):
-        import queue
-        import threading
-        self.nets = [Net(msnhnet_path, msnhbin_path, fp16=fp16) for _ in range(instances)]
-        last = self.nets[0].layer_info(self.nets[0].num_layers() - 1)["type"]
-        self.detect = last == "yoloout"
-        self.depth = max(1, depth if self.detect else 1)      # a classifier's result is read from its output tensor: one forward at a time
-        self._in = [queue.Queue() for _ in self.nets]
-        self._out = [queue.Queue() for _ in self.nets]
+        self.L = lib()
+        set_use_fp16(fp16)
+        self.g = ctypes.c_void_p()
+        _check(self.L.msnhnet_group_create(msnhnet_path.encode(), msnhbin_path.encode(), instances, depth, ctypes.byref(self.g)))
+        n, d, det = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        _check(self.L.msnhnet_group_info(self.g, ctypes.byref(n), ctypes.byref(d), ctypes.byref(det)))
+        self.depth, self.detect = d.value, bool(det.value)
+        self.nets = []
+        for i in range(n.value):
+            h = ctypes.c_void_p()
+            _check(self.L.msnhnet_group_instance(self.g, i, ctypes.byref(h)))
+            self.nets.append(Net.borrowed(h))
         self._submitted = 0
         self._fetched = 0
-        self._threads = [threading.Thread(target=self._drive, args=(i,), daemon=True) for i in range(instances)]
-        for t in self._threads:
-            t.start()
-
-    def _drive(self, i):
-        net, inq, outq = self.nets[i], self._in[i], self._out[i]
-        fetch = net.fetch_yolo if self.detect else net.fetch_classify
-        in_flight = 0
-        while True:
-            job = inq.get()
-            try:
-                if job == "stop" or job == "flush":
-                    while in_flight:
-                        outq.put(fetch())
-                        in_flight -= 1
-                    if job == "stop":
-                        return
-                    outq.put("flushed")
-                    continue
-                net.enqueue(job[0])
-                in_flight += 1
-                if in_flight == self.depth:
-                    outq.put(fetch())
-                    in_flight -= 1
-            except Exception as e:         # hand the error to whoever waits for the result
-                outq.put(e)
-                if job == "stop":
-                    return
+        self._batch = self.nets[0].dims()[0]
+        if self.detect:
+            self._boxes = np.zeros((max(int(self.L.msnhnet_yolo_max_boxes(self.nets[0].h)), 1), 7), np.float32)
+        else:
+            self._outputs = self.nets[0].layer_info(self.nets[0].num_layers() - 1)["outputNum"]
 
     def prime(self, device_ptr):
-        """One forward of the batch at device_ptr on every instance (its input buffer then holds that batch); returns the results."""
-        return [self._one(n, device_ptr) for n in self.nets]
-
-    def _one(self, net, device_ptr):
-        net.enqueue(device_ptr)
-        return net.fetch_yolo() if self.detect else net.fetch_classify()
+        _check(self.L.msnhnet_group_prime(self.g, ctypes.c_void_p(device_ptr) if device_ptr else None))
 
     def submit(self, device_ptr=None):
-        self._in[self._submitted % len(self.nets)].put((device_ptr,))
+        _check(self.L.msnhnet_group_submit(self.g, ctypes.c_void_p(device_ptr) if device_ptr else None))
         self._submitted += 1
 
     def flush(self):
-        """Makes every instance fetch what it still has in flight (otherwise an instance keeps depth - 1 results back until more work comes)."""
-        for q in self._in:
-            q.put("flush")
+        _check(self.L.msnhnet_group_flush(self.g))
 
     def fetch(self):
         if self._fetched >= self._submitted:
             raise RuntimeError("nothing outstanding")
-        q = self._out[self._fetched % len(self.nets)]
-        while True:
-            r = q.get()
-            if isinstance(r, str):          # a flush marker: everything submitted before it has been delivered
-                continue
-            break
-        if isinstance(r, Exception):
-            raise r
-        self._fetched += 1
-        return r
-
-    def last_nms_on_device(self):
-        return sum(n.last_nms_on_device() for n in self.nets)
+        self._fetched += 1               # (a batch whose fetch reports an error is consumed as well)
+        if self.detect:
+            counts = (ctypes.c_int * self._batch)()
+            total = ctypes.c_longlong()
+            _check(self.L.msnhnet_group_fetch_yolo(self.g, counts, _fp(self._boxes), self._boxes.shape[0], ctypes.byref(total)))
+            out, at = [], 0
+            for i in range(self._batch):
+                out.append(self._boxes[at:at + counts[i]].copy())
+                at += counts[i]
+            return out
+        out = np.empty(self._batch * self._outputs, np.float32)
+        n = ctypes.c_longlong()
+        _check(self.L.msnhnet_group_fetch_classify(self.g, _fp(out), out.size, ctypes.byref(n)))
+        return out[:n.value].reshape(self._batch, -1)
 
     def close(self):
-        for q in self._in:
-            q.put("stop")
-        for t in self._threads:
-            t.join(timeout=30)
         for n in self.nets:
             n.close()
+        if self.g:
+            self.L.msnhnet_group_destroy(self.g)
+            self.g = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

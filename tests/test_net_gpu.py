@@ -569,12 +569,7 @@ def test_net_group_results_in_submission_order(arch, size, batch, instances, dep
     grp = netapi.NetGroup(net, binp, instances=instances, depth=depth, fp16=True)
     try:
         assert grp.detect == detect and len(grp.nets) == instances
-        first = grp.prime(xd[0].data_ptr())
-        for r in first:
-            if detect:
-                assert all(np.array_equal(a, b, equal_nan=True) for a, b in zip(r, want[0]))
-            else:
-                assert np.array_equal(r, want[0])
+        grp.prime(xd[0].data_ptr())
         for rounds in range(2):
             for t in xd:
                 grp.submit(t.data_ptr())
@@ -589,7 +584,7 @@ def test_net_group_results_in_submission_order(arch, size, batch, instances, dep
                     assert np.array_equal(got, want[i]), (rounds, i)
         with pytest.raises(RuntimeError):
             grp.fetch()                      # nothing outstanding
-        # on what the input buffers hold: instance k saw batch 6 - ((7 - 1 - k) % instances) ... simply: every result is one of the submitted ones
+        # on what an instance's input buffer holds (one of the submitted batches)
         grp.submit(None)
         grp.flush()
         got = grp.fetch()
