@@ -157,8 +157,8 @@ def conv_shape_mode(a):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--conv-shape", default=None, help="b,c,h,w,oc,k,stride: time this one convolution shape instead of a workload")
     ap.add_argument("--tile", type=int, default=0, help="--conv-shape: launch only this tile configuration, --reps times, untimed")
     ap.add_argument("--reps", type=int, default=20)
