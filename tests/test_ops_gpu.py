@@ -640,3 +640,22 @@ def test_image_u8_to_input(h, w, nw, nh):
     assert abi.lib().msnh_hip_image_u8_to_input(gu.ptr(src), w, h, nw, nh, 3, None, None, 0, gu.ptr(dst), None) != 0
     assert b"mean or std" in abi.lib().msnh_hip_last_error()
     assert abi.lib().msnh_hip_image_u8_to_input(gu.ptr(src), w, h, nw, nh, 9, None, None, 0, gu.ptr(dst), None) != 0
+
+
+def test_mfma_probe():
+    """the matrix-core ceiling probe reports a rate below the data-sheet peak and above half of it, a plausible shader clock, and
+    refuses nonsense arguments"""
+    import gpuutil as gu
+    gu.init()
+    L = abi.lib()
+    tf, mhz, sec = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+    abi.check(L.msnh_hip_mfma_probe(3, 4000, ctypes.byref(tf), ctypes.byref(mhz), ctypes.byref(sec), None))
+    print(f"mfma probe: {tf.value:.0f} TFLOP/s at {mhz.value:.0f} MHz in {sec.value * 1e3:.3f} ms", flush=True)
+    assert 1000.0 < tf.value < 2600.0
+    assert 800.0 < mhz.value < 2600.0
+    assert 0.0 < sec.value < 0.1
+    # the rate follows from the clock: 256 CUs x 4 SIMDs x 1024 FLOP per clock, within what a short run's ramp allows
+    assert 0.6 < tf.value / (mhz.value * 1e6 * 256 * 4 * 1024 / 1e12) < 1.05
+    assert L.msnh_hip_mfma_probe(0, 100, ctypes.byref(tf), ctypes.byref(mhz), ctypes.byref(sec), None) != 0
+    assert L.msnh_hip_mfma_probe(3, 0, ctypes.byref(tf), ctypes.byref(mhz), ctypes.byref(sec), None) != 0
+    assert L.msnh_hip_mfma_probe(3, 100, None, ctypes.byref(mhz), ctypes.byref(sec), None) != 0
