@@ -376,7 +376,7 @@ def main():
     if dw_n > 0:
         gbs = dw_bytes / (dw_ms * 1e-3) / 1e9
         roofline_hbm = {"bound": "hbm", "achieved": round(gbs, 1), "peak": 8000.0, "unit": "GB/s", "frac": round(gbs / 8000.0, 4),
-                        "traffic": HBM_BYTES_PER_DEPTHWISE_LAUNCH.get((a.workload, dtype, batch)), "kernel": "convDepthwise3x3Kernel",
+                        "traffic": HBM_BYTES_PER_DEPTHWISE_LAUNCH.get((a.workload, dtype, batch)), "kernel": "convDepthwise3x3FastKernel",
                         "launches_per_step": dw_n // 10, "avg_launch_us": round(dw_ms * 1e3 / dw_n, 2), "bytes_per_step": dw_bytes / 10}
 
     res = {"metric": f"images/sec on 1 MI355X ({a.workload} {size} {dtype} b{batch})", "value": round(batch / (ms_per_step * 1e-3), 2),

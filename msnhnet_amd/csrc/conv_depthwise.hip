@@ -8,6 +8,7 @@
 // Consecutive lanes take consecutive channel vectors of the same strip, so every load instruction of a wavefront
 // covers whole pixels.
 #include "common.hpp"
+#include <cstdlib>
 
 namespace msnh {
 
@@ -127,6 +128,137 @@ __global__ __launch_bounds__(256) void convDepthwise3x3Kernel(DwArgs a, int bloc
     }
 }
 
+
+// ---- the same strip kernel with 32-bit index arithmetic -------------------------------------------------------------------------
+// With two channels per lane a lane produces eight outputs, and the kernel above spends more vector instructions on finding out
+// which eight (three 64-bit divisions of the lane index, 64-bit address arithmetic for nine weight vectors and four stores) than on
+// the 72 multiply-adds: it is bound by the vector ALU, not by memory.  Where everything fits 32 bits (lane count, input, output
+// and weight bytes below 2^31 -- checked on the host) the divisions become multiplications by precomputed reciprocals
+// (Granlund & Montgomery, "Division by invariant integers using multiplication", figure 4.1), every address a 32-bit buffer offset,
+// and the stores past the row's end out-of-range offsets instead of branches.
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+struct FastDiv { unsigned m, s1, s2, d; };
+
+inline FastDiv makeFastDiv(unsigned d)
+{
+    unsigned l = 0;
+    while ((1ull << l) < d) ++l;                     // ceil(log2 d)
+    FastDiv f;
+    f.m = static_cast<unsigned>(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+    f.s1 = l < 1 ? l : 1;
+    f.s2 = l > 1 ? l - 1 : 0;
+    f.d = d;
+    return f;
+}
+
+__device__ __forceinline__ unsigned fastDiv(unsigned n, const FastDiv &f)
+{
+    const unsigned t = __umulhi(f.m, n);
+    return (t + ((n - t) >> f.s1)) >> f.s2;
+}
+
+struct DwFastArgs
+{
+    DwArgs d;
+    FastDiv byCv, byStrips, byOH;
+    unsigned wBytes, yBytes;
+};
+
+template <int STRIDE, int CPL>
+__global__ __launch_bounds__(256) void convDepthwise3x3FastKernel(DwFastArgs g, int blocks)
+{
+    constexpr int COLS = 3 * STRIDE + 3;
+    typedef f16 HV __attribute__((ext_vector_type(CPL)));
+    const DwArgs &a = g.d;
+    const int perXcd = (blocks + 7) / 8;
+    const int logical = static_cast<int>(blockIdx.x % 8) * perXcd + static_cast<int>(blockIdx.x / 8);
+    if (logical >= blocks) return;
+    const unsigned idx = static_cast<unsigned>(logical) * 256u + threadIdx.x;
+    if (idx >= static_cast<unsigned>(a.total)) return;
+    const unsigned q1 = fastDiv(idx, g.byCv);
+    const int c0 = static_cast<int>(idx - q1 * g.byCv.d) * CPL;
+    const unsigned q2 = fastDiv(q1, g.byStrips);
+    const int sx = static_cast<int>(q1 - q2 * g.byStrips.d);
+    const unsigned q3 = fastDiv(q2, g.byOH);
+    const int oy = static_cast<int>(q2 - q3 * g.byOH.d);
+    const int b = static_cast<int>(q3);
+    const int ox0 = sx * 4;
+    const int iy0 = oy * STRIDE - a.pad;
+    const int ix0 = ox0 * STRIDE - a.pad;
+
+    const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<f16 *>(a.x), 0, static_cast<int>(a.xBytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<f16 *>(a.w), 0, static_cast<int>(g.wBytes), 0x00020000);
+    const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, static_cast<int>(g.yBytes), 0x00020000);
+
+    HV wv[9];
+#pragma unroll
+    for (int k = 0; k < 9; ++k)
+    {
+        const int off = static_cast<int>(static_cast<unsigned>(k * a.C + c0) * 2u);
+        if constexpr (CPL == 4) wv[k] = __builtin_bit_cast(HV, __builtin_amdgcn_raw_buffer_load_b64(rw, off, 0, 0));
+        else wv[k] = __builtin_bit_cast(HV, __builtin_amdgcn_raw_buffer_load_b32(rw, off, 0, 0));
+    }
+
+    // byte offset of input pixel (iy0, ix0), channel c0, modulo 2^32: it may lie in front of the tensor and comes back into range
+    // once a valid tap's offset is added
+    const unsigned base = (static_cast<unsigned>((b * a.H + iy0) * a.W + ix0) * static_cast<unsigned>(a.inLd) + static_cast<unsigned>(c0)) * 2u;
+    const unsigned pixB = static_cast<unsigned>(a.inLd) * 2u;
+    const unsigned rowB = static_cast<unsigned>(a.W) * pixB;
+    HV xv[3][COLS];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+    {
+        const bool rowOk = static_cast<unsigned>(iy0 + r) < static_cast<unsigned>(a.H);
+#pragma unroll
+        for (int c = 0; c < COLS; ++c)
+        {
+            const bool ok = rowOk && static_cast<unsigned>(ix0 + c) < static_cast<unsigned>(a.W);
+            const unsigned off = ok ? base + static_cast<unsigned>(r) * rowB + static_cast<unsigned>(c) * pixB : kOob;
+            if constexpr (CPL == 4) xv[r][c] = __builtin_bit_cast(HV, __builtin_amdgcn_raw_buffer_load_b64(rx, static_cast<int>(off), 0, 0));
+            else xv[r][c] = __builtin_bit_cast(HV, __builtin_amdgcn_raw_buffer_load_b32(rx, static_cast<int>(off), 0, 0));
+        }
+    }
+    float acc[4][CPL];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) acc[j][e] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int kx = 0; kx < 3; ++kx)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int e = 0; e < CPL; ++e)
+                    acc[j][e] += static_cast<float>(xv[r][j * STRIDE + kx][e]) * static_cast<float>(wv[r * 3 + kx][e]);
+
+    float sc[CPL], sh[CPL];
+#pragma unroll
+    for (int e = 0; e < CPL; ++e)
+    {
+        sc[e] = a.scale ? a.scale[c0 + e] : 1.f;
+        sh[e] = a.shift ? a.shift[c0 + e] : 0.f;
+    }
+    float v[4 * CPL];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) v[j * CPL + e] = acc[j][e] * sc[e] + sh[e];
+    activateArray<4 * CPL>(v, a.act, a.actParam);
+    const unsigned obase = (static_cast<unsigned>((b * a.OH + oy) * a.OW + ox0) * static_cast<unsigned>(a.outLd) + static_cast<unsigned>(c0)) * 2u;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+    {
+        HV o;
+#pragma unroll
+        for (int e = 0; e < CPL; ++e) o[e] = static_cast<f16>(a.outMul * v[j * CPL + e]);
+        const unsigned off = ox0 + j < a.OW ? obase + static_cast<unsigned>(j * a.outLd) * 2u : kOob;
+        if constexpr (CPL == 4) __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, o), ry, static_cast<int>(off), 0, 0);
+        else __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, o), ry, static_cast<int>(off), 0, 0);
+    }
+}
+
 } // namespace
 
 bool depthwise3x3Ok(const msnh_conv_desc *d, const void *x, const void *w, const void *y)
@@ -153,6 +285,24 @@ int convDepthwise3x3(const msnh_conv_desc *d, const void *x, const void *w, cons
     a.act = d->act; a.actParam = d->act_param; a.outMul = d->out_mul;
     const int blocks = static_cast<int>(gridFor(a.total, 256));
     const dim3 grid((blocks + 7) / 8 * 8);
+    // everything below 2^31: the 32-bit form (d->tile == 1 keeps the general one, for comparison)
+    const unsigned long long yBytes = ((static_cast<unsigned long long>(d->batch) * d->out_h * d->out_w - 1) * d->out_ld + d->in_c) * 2ull;
+    const unsigned long long wBytes = 9ull * d->in_c * 2ull;
+    static const bool generalOnly = std::getenv("MSNH_DEPTHWISE_GENERAL") != nullptr;      // (for A/B timing of whole networks)
+    if (d->tile != 1 && !generalOnly && a.total < 0x7fffff00ll && yBytes < 0x7fffffffull && wBytes < 0x7fffffffull)
+    {
+        DwFastArgs g;
+        g.d = a;
+        g.byCv = makeFastDiv(static_cast<unsigned>(d->in_c / CPL));
+        g.byStrips = makeFastDiv(static_cast<unsigned>(a.strips));
+        g.byOH = makeFastDiv(static_cast<unsigned>(d->out_h));
+        g.wBytes = static_cast<unsigned>(wBytes);
+        g.yBytes = static_cast<unsigned>(yBytes);
+        if (d->stride == 1) hipLaunchKernelGGL((convDepthwise3x3FastKernel<1, 2>), grid, dim3(256), 0, st, g, blocks);
+        else                hipLaunchKernelGGL((convDepthwise3x3FastKernel<2, 2>), grid, dim3(256), 0, st, g, blocks);
+        MSNH_LAUNCH_CHECK();
+        return 0;
+    }
     if (d->stride == 1) hipLaunchKernelGGL((convDepthwise3x3Kernel<1, CPL>), grid, dim3(256), 0, st, a, blocks);
     else                hipLaunchKernelGGL((convDepthwise3x3Kernel<2, CPL>), grid, dim3(256), 0, st, a, blocks);
     MSNH_LAUNCH_CHECK();

@@ -199,6 +199,29 @@ def test_conv_depthwise(c, h, w, k, stride, pad, dtype):
     assert gu.rel_err(y, ref) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("b,c,h,w,stride", [(2, 32, 14, 14, 1), (1, 144, 9, 21, 1), (2, 24, 7, 7, 1), (1, 960, 7, 7, 1), (3, 64, 33, 18, 2), (1, 8, 5, 70, 1),
+                                            (2, 384, 14, 14, 2), (1, 32, 112, 112, 1), (2, 96, 15, 13, 2), (1, 16, 1, 1, 1), (1, 40, 3, 2, 2)])
+@pytest.mark.parametrize("act", ["relu6", "leaky"])
+def test_conv_depthwise_index_forms(b, c, h, w, stride, act):
+    """3x3 depthwise float16: the kernel with 32-bit index arithmetic and reciprocal-multiplication divisions (the default where every
+    size is below 2^31) and the general one (tile 1) agree with the reference convolution and with each other bit for bit; sizes that
+    are not multiples of the strip, one-pixel images, an output stride wider than the channel count"""
+    import gpuutil as gu
+    rng = np.random.default_rng(c * h + w)
+    x, wt = _case(rng, b, c, h, w, c, 3, groups=c)
+    scale = rng.uniform(0.5, 1.5, c).astype(np.float32)
+    shift = (rng.standard_normal(c) * 0.1).astype(np.float32)
+    x, wt = gu.round_f16(x), gu.round_f16(wt)
+    ref = _ref(x, wt, stride, 1, 1, c, scale, shift, act, 0.1, None, "none", 1.0, 1.0)
+    outs = []
+    for tile in (1, 0):
+        y, used = gu.conv2d(x, wt, dtype=abi.F16, stride=stride, pad=1, groups=c, scale=scale, shift=shift, act=act, tile=tile, out_ld=(c + 15) // 8 * 8)
+        assert used == "depthwise"
+        assert gu.rel_err(y, ref) <= TOL[abi.F16], tile
+        outs.append(y)
+    assert np.array_equal(outs[0], outs[1])
+
+
 @pytest.mark.parametrize("out_dtype", [abi.F32, abi.F16])
 @pytest.mark.parametrize("h,w,oc,k,stride,pad", [(33, 31, 32, 3, 1, 1), (40, 40, 64, 7, 2, 3), (25, 27, 32, 3, 2, 1), (70, 100, 64, 3, 1, 1),
                                                  (37, 45, 64, 7, 2, 3), (30, 70, 32, 7, 1, 3), (21, 19, 128, 7, 2, 0), (224, 224, 64, 7, 2, 3),
