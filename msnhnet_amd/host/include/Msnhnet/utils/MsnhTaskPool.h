@@ -22,8 +22,9 @@ public:
     static TaskPool &instance();
     // fn(i) for every i in [0, n), indices handed out one at a time in ascending order (big tasks first: sort before calling);
     // the caller works along and returns when every index is done -- it waits for tasks, not for workers: a worker that wakes up
-    // late finds nothing left and goes back to sleep.  The first exception thrown by fn is rethrown here.  One call at a time
-    // (concurrent callers queue up).
+    // late finds nothing left and goes back to sleep.  The first exception thrown by fn is rethrown here.  Calls from several
+    // threads run side by side (the instances of a NetGroup each have a host stage): a worker takes indices of whichever job has
+    // some left.
     void parallelFor(int n, const std::function<void(int)> &fn);
     int threads() const { return static_cast<int>(_threads.size()) + 1; }
     ~TaskPool();
@@ -40,10 +41,9 @@ private:
     void worker();
     void drain(Job &job);
     std::vector<std::thread> _threads;
-    std::mutex _callers, _m;
+    std::mutex _m;
     std::condition_variable _cvWork, _cvDone;
-    std::shared_ptr<Job> _current;
-    uint64_t _jobId = 0;
+    std::vector<std::shared_ptr<Job>> _jobs;        // jobs that may still have indices to hand out
     bool _stop = false;
 };
 }

@@ -58,16 +58,19 @@ void TaskPool::drain(Job &job)
 
 void TaskPool::worker()
 {
-    uint64_t seen = 0;
     std::unique_lock<std::mutex> lk(_m);
     for (;;)
     {
-        _cvWork.wait(lk, [&] { return _stop || _jobId != seen; });
+        std::shared_ptr<Job> job;
+        _cvWork.wait(lk, [&] {
+            if (_stop) return true;
+            for (const std::shared_ptr<Job> &j : _jobs)
+                if (j->next.load(std::memory_order_relaxed) < j->n) { job = j; return true; }
+            return false;
+        });
         if (_stop) return;
-        seen = _jobId;
-        std::shared_ptr<Job> job = _current;      // empty when the job was finished before this worker woke up
         lk.unlock();
-        if (job) drain(*job);
+        drain(*job);
         job.reset();
         lk.lock();
     }
@@ -81,14 +84,12 @@ void TaskPool::parallelFor(int n, const std::function<void(int)> &fn)
         for (int i = 0; i < n; ++i) fn(i);
         return;
     }
-    std::lock_guard<std::mutex> one(_callers);
     std::shared_ptr<Job> job = std::make_shared<Job>();
     job->fn = &fn;
     job->n = n;
     {
         std::lock_guard<std::mutex> lk(_m);
-        _current = job;
-        ++_jobId;
+        _jobs.push_back(job);
     }
     // as many workers as there are tasks beside the caller's
     const int wake = std::min(n - 1, static_cast<int>(_threads.size()));
@@ -97,7 +98,8 @@ void TaskPool::parallelFor(int n, const std::function<void(int)> &fn)
     drain(*job);
     std::unique_lock<std::mutex> lk(_m);
     _cvDone.wait(lk, [&] { return job->done.load(std::memory_order_acquire) == n; });
-    _current.reset();
+    for (size_t i = 0; i < _jobs.size(); ++i)
+        if (_jobs[i] == job) { _jobs.erase(_jobs.begin() + static_cast<long>(i)); break; }
     if (job->error) std::rethrow_exception(job->error);
 }
 }

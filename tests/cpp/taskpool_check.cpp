@@ -41,6 +41,25 @@ int main()
     ran = 0;
     pool.parallelFor(16, [&](int) { ++ran; });
     if (ran != 16) { std::printf("after exception: %d\n", ran.load()); return 1; }
+    // several callers at once (the instances of a group): every job completes with every index once
+    {
+        std::vector<std::thread> callers;
+        std::atomic<int> wrong{0};
+        for (int c = 0; c < 4; ++c)
+            callers.emplace_back([&, c] {
+                for (int rep = 0; rep < 300; ++rep)
+                {
+                    const int n = 5 + (rep + c) % 40;
+                    std::vector<std::atomic<int>> hits(static_cast<size_t>(n));
+                    for (auto &h : hits) h = 0;
+                    pool.parallelFor(n, [&](int i) { ++hits[static_cast<size_t>(i)]; });
+                    for (int i = 0; i < n; ++i)
+                        if (hits[static_cast<size_t>(i)] != 1) ++wrong;
+                }
+            });
+        for (std::thread &t : callers) t.join();
+        if (wrong != 0) { std::printf("concurrent callers: %d wrong counts\n", wrong.load()); return 1; }
+    }
     // idle workers sleep
     const double c0 = cpuSeconds();
     std::this_thread::sleep_for(std::chrono::milliseconds(300));
