@@ -314,10 +314,15 @@ def main():
         # the same run with one instance alone (two batches in flight on one stream), for comparison
         on_device[0] = 0
         k1 = min(a.steps, 100)
+        if detect:
+            net.set_copy_on_forward_stream(False)       # as a NetBuilder on its own runs: copy-back on a stream beside the next forward
+            run_steps(4, use_group=False)
         ts = time.perf_counter()
         run_steps(k1, use_group=False)
         net.sync()
         single_rate = round(batch * k1 / (time.perf_counter() - ts), 2)
+        if detect:
+            net.set_copy_on_forward_stream(True)
     gc.enable()
     marker()
     ms_per_step = dt / a.steps * 1e3

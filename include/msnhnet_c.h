@@ -117,6 +117,11 @@ int msnhnet_run_classify_gpu(msnhnet_t net, const float *img, long long n, float
 /* NetBuilder::runYoloGPU: counts[b] = boxes of image b; boxes = rows of 7 floats (x y w h conf bestClsConf
  * bestClsIdx), images back to back, at most cap_boxes rows are written; *total = sum of counts. */
 int msnhnet_run_yolo_gpu(msnhnet_t net, const float *img, long long n, int *counts, float *boxes, long long cap_boxes, long long *total);
+/* Detectors: put the copy-back of the candidates (and the device NMS) on the forward's own stream instead of a stream of their own.
+ * Off by default for a NetBuilder on its own (the copy of one batch then runs beside the next forward); the instances of a group
+ * have it on (one busy stream per instance: a process has four hardware queues, and a copy stream that shares one with another
+ * instance's forward waits behind that forward).  Set while nothing is in flight. */
+int msnhnet_set_copy_on_forward_stream(msnhnet_t net, int on);
 /* Where the hard NMS of the detection result fetched last ran: 1 on the device, 0 on the host (msnhnet_set_device_nms). */
 int msnhnet_last_nms_on_device(msnhnet_t net, int *on_device);
 /* Range check of a float16 plan for one input (NetBuilder::fp16Headroom): runs the network once on img and writes the factor by which

@@ -359,6 +359,7 @@ public:
     std::vector<std::vector<YoloBox>> finalOut;
     static bool keepClassScores;           // also fill YoloBox::classesVal (costs an extra device->host copy)
     bool lastOnDevice = false;             // where the NMS of the result fetched last ran
+    bool copyOnForwardStream = false;      // copy-back (and device NMS) on the forward's stream instead of a stream of their own (NetGroup)
     // hard NMS on the device (only the kept boxes are copied back): 0 = never (sort + NMS on the host), 2 = always,
     // 1 (default) = chosen per batch from the previous result: up to kDeviceNmsFew candidates per image on the device; up to
     // kDeviceNmsCandidates (the largest class the device kernels take) on the device as well, except while forwards are pipelined and

@@ -7,6 +7,7 @@
 #include <string>
 #include "Msnhnet/net/MsnhNetBuilder.h"
 #include "Msnhnet/net/MsnhNetGroup.h"
+#include "Msnhnet/layers/MsnhLayers.h"
 
 using namespace Msnhnet;
 
@@ -401,6 +402,15 @@ long long msnhnet_layer_output(msnhnet_t net, int layer, float *dst, long long c
 int msnhnet_device_input(msnhnet_t net, float **device_ptr)
 {
     return guarded([&] { if (!device_ptr) MSNH_THROW("pointer is NULL"); *device_ptr = nb(net).deviceInputBuffer(); });
+}
+
+int msnhnet_set_copy_on_forward_stream(msnhnet_t net, int on)
+{
+    return guarded([&] {
+        Network *n = nb(net).getNet();
+        if (n == nullptr || n->layers.empty() || n->layers.back()->type() != LayerType::YOLO_OUT) MSNH_THROW("not a yolo net");
+        static_cast<YoloOutLayer *>(n->layers.back())->copyOnForwardStream = on != 0;
+    });
 }
 
 int msnhnet_enqueue(msnhnet_t net, const float *device_input) { return guarded([&] { nb(net).enqueueForward(device_input); }); }

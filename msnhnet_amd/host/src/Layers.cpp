@@ -1442,15 +1442,21 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
     }
     // Snapshot on the device (microseconds), then cross PCIe on a second stream: the next forward does not wait for
     // the copy (several MiB: every cell has a row slot, the count is only known on the device).
-    if (_copyStream == nullptr) MSNH_DEV(msnh_hip_stream_create(&_copyStream));
+    // copyOnForwardStream (the instances of a NetGroup): everything below goes onto the forward's own stream.  A process has four
+    // hardware queues; three instances with a copy stream each are six busy streams, and a copy stream that shares a queue with
+    // another instance's forward waits behind that forward's kernels (measured: 4150-4750 images/s depending on nothing but the
+    // order in which the streams were created).  On its own stream the copy sits between two forwards of the instance, and the
+    // other instances fill the gap.
+    if (!copyOnForwardStream && _copyStream == nullptr) MSNH_DEV(msnh_hip_stream_create(&_copyStream));
+    const msnh_stream_t cs = copyOnForwardStream ? s : _copyStream;
     if (sl.ready == nullptr) MSNH_DEV(msnh_hip_event_create(&sl.ready));
     if (sl.devCnt.bytes() < cntBytes) sl.devCnt.alloc(cntBytes);
     if (sl.devRows.bytes() < rowBytes) sl.devRows.alloc(rowBytes);
     MSNH_DEV(msnh_hip_memcpy_d2d(sl.devCnt.ptr(), pl.yoloCandCnt.ptr(), cntBytes, s));
     MSNH_DEV(msnh_hip_memcpy_d2d(sl.devRows.ptr(), pl.yoloRows.ptr(), rowBytes, s));
     MSNH_DEV(msnh_hip_event_record(sl.ready, s));
-    MSNH_DEV(msnh_hip_stream_wait_event(_copyStream, sl.ready));
-    MSNH_DEV(msnh_hip_memcpy_d2h(sl.cnt.ptr(), sl.devCnt.ptr(), cntBytes, _copyStream));
+    if (!copyOnForwardStream) MSNH_DEV(msnh_hip_stream_wait_event(cs, sl.ready));
+    MSNH_DEV(msnh_hip_memcpy_d2h(sl.cnt.ptr(), sl.devCnt.ptr(), cntBytes, cs));
     // auto: few candidates (real detections) -> the device; thousands per image -> the device too unless a second forward is in flight
     // (the host's sort + NMS then runs beside that forward and costs the device nothing, whereas the device NMS takes about 0.1 ms of
     // device time per batch from it) and the host stage has kept up with the device so far
@@ -1473,13 +1479,13 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
         sl.keptCnt.reserve(keptCntBytes);
         sl.quick = std::min(keptCap, std::max(kQuickRecords, _lastKept + _lastKept / 2 + 1024));
         sl.kept.reserve(sl.quick * kRecordBytes);
-        MSNH_DEV(msnh_hip_fill_zero(sl.devKeptCnt.ptr(), keptCntBytes, _copyStream));
+        MSNH_DEV(msnh_hip_fill_zero(sl.devKeptCnt.ptr(), keptCntBytes, cs));
         const size_t wsBytes = msnh_hip_yolo_nms_pair_workspace_bytes(_batch, _channel - 5, pl.yoloCells);
         if (sl.devNmsWs.bytes() < wsBytes) sl.devNmsWs.alloc(wsBytes);
         MSNH_DEV(msnh_hip_yolo_nms(_batch, _channel - 5, sl.devRows.as<float>(), pl.yoloCells, sl.devCnt.as<int>(), _nmsThresh, sl.devKept.as<float>(),
-                                   static_cast<int>(keptCap), sl.devKeptCnt.as<int>(), sl.devNmsWs.ptr(), wsBytes, _copyStream));
-        MSNH_DEV(msnh_hip_memcpy_d2h(sl.keptCnt.ptr(), sl.devKeptCnt.ptr(), keptCntBytes, _copyStream));
-        MSNH_DEV(msnh_hip_memcpy_d2h(sl.kept.ptr(), sl.devKept.ptr(), sl.quick * kRecordBytes, _copyStream));
+                                   static_cast<int>(keptCap), sl.devKeptCnt.as<int>(), sl.devNmsWs.ptr(), wsBytes, cs));
+        MSNH_DEV(msnh_hip_memcpy_d2h(sl.keptCnt.ptr(), sl.devKeptCnt.ptr(), keptCntBytes, cs));
+        MSNH_DEV(msnh_hip_memcpy_d2h(sl.kept.ptr(), sl.devKept.ptr(), sl.quick * kRecordBytes, cs));
     }
     else
     {
@@ -1490,15 +1496,15 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
         if (const char *forced = std::getenv("MSNH_YOLO_ROWS_PREFIX")) guess = static_cast<size_t>(std::max(1L, std::atol(forced)));    // (tests)
         sl.rowsCopied = std::min(guess, cells);
         if (sl.rowsCopied == cells)
-            MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.ptr(), sl.devRows.ptr(), rowBytes, _copyStream));
+            MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.ptr(), sl.devRows.ptr(), rowBytes, cs));
         else
             for (int b = 0; b < _batch; ++b)
             {
                 const size_t off = static_cast<size_t>(b) * cells * 8;
-                MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.as<float>() + off, sl.devRows.as<float>() + off, sizeof(float) * 8 * sl.rowsCopied, _copyStream));
+                MSNH_DEV(msnh_hip_memcpy_d2h(sl.rows.as<float>() + off, sl.devRows.as<float>() + off, sizeof(float) * 8 * sl.rowsCopied, cs));
             }
     }
-    MSNH_DEV(msnh_hip_event_record(sl.event, _copyStream));
+    MSNH_DEV(msnh_hip_event_record(sl.event, cs));
     sl.pending = true;
 }
 

@@ -12,6 +12,13 @@ NetGroup::NetGroup(const std::string &msnhnetPath, const std::string &msnhbinPat
         lane->net.reset(new NetBuilder());
         lane->net->buildNetFromMsnhNet(msnhnetPath);
         lane->net->loadWeightsFromMsnhBin(msnhbinPath);
+        if (instances > 1)
+        {
+            // one stream per instance: see YoloOutLayer::copyOnForwardStream
+            Network *net = lane->net->getNet();
+            if (!net->layers.empty() && net->layers.back()->type() == LayerType::YOLO_OUT)
+                static_cast<YoloOutLayer *>(net->layers.back())->copyOnForwardStream = true;
+        }
         _lanes.push_back(std::move(lane));
     }
     Network *n = _lanes[0]->net->getNet();

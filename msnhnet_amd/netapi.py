@@ -15,7 +15,7 @@ SYMBOLS = [
     "initMsnhnet", "buildMsnhnet", "runClassifyNoPred", "runYoloNoPred", "runClassifyList", "runYoloList", "dispose", "withGPU", "withCUDNN", "getCpuForwardTime",
     "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16", "msnhnet_set_use_winograd", "msnhnet_set_tune_cache", "msnhnet_set_weight_cache", "msnhnet_load_detail", "msnhnet_set_device_nms", "msnhnet_set_input_image_u8", "msnhnet_set_input_image", "msnhnet_boxes_to_image",
     "msnhnet_set_keep_class_scores", "msnhnet_set_save_layer_output", "msnhnet_build", "msnhnet_load", "msnhnet_load_from_memory",
-    "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops", "msnhnet_weight_layout", "msnhnet_fp16_headroom", "msnhnet_last_nms_on_device",
+    "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops", "msnhnet_weight_layout", "msnhnet_fp16_headroom", "msnhnet_last_nms_on_device", "msnhnet_set_copy_on_forward_stream",
     "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
     "msnhnet_enqueue", "msnhnet_sync", "msnhnet_fetch_classify", "msnhnet_fetch_yolo", "msnhnet_gpu_inference_time", "msnhnet_time_detail",
     "msnhnet_profile_ops", "msnhnet_profile_ops_bytes", "msnhnet_profile_each_op", "msnhnet_yolo_max_boxes", "msnhnet_nms",
@@ -105,6 +105,7 @@ def lib():
     L.msnhnet_sync.argtypes = [vp]
     L.msnhnet_fetch_classify.argtypes = [vp, fp, ll, llp]
     L.msnhnet_fetch_yolo.argtypes = [vp, ip, fp, ll, llp]
+    L.msnhnet_set_copy_on_forward_stream.argtypes = [vp, ci]
     L.msnhnet_group_create.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ci, ci, ctypes.POINTER(vp)]
     L.msnhnet_group_destroy.argtypes = [vp]
     L.msnhnet_group_info.argtypes = [vp, ip, ip, ip]
@@ -218,6 +219,10 @@ class Net:
     def load_array(self, w):
         w = np.ascontiguousarray(w, np.float32)
         _check(self.L.msnhnet_load_from_memory(self.h, _fp(w), w.size))
+
+    def set_copy_on_forward_stream(self, on):
+        """detectors: copy-back on the forward's own stream (what the instances of a NetGroup use) or on a stream of its own (default)"""
+        _check(self.L.msnhnet_set_copy_on_forward_stream(self.h, 1 if on else 0))
 
     def last_nms_on_device(self):
         v = ctypes.c_int()

@@ -594,3 +594,34 @@ def test_net_group_results_in_submission_order(arch, size, batch, instances, dep
             assert any(np.array_equal(got, w) for w in want)
     finally:
         grp.close()
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_copy_on_forward_stream_same_results(mode):
+    """copy-back (and device NMS) on the forward's own stream, as the instances of a group run, returns what the copy stream beside
+    the next forward returns, pipelined and one at a time, for every NMS placement"""
+    size, batch = 160, 2
+    net, binp, g = nu.model("yolov3", batch, size, seed=5)
+    xs = [zoo.seeded_input(batch, 3, size, size, seed=30 + i) for i in range(3)]
+    xd = [torch.from_numpy(x).cuda() for x in xs]
+    netapi.set_device_nms(mode)
+    try:
+        m = netapi.Net(net, binp, fp16=True)
+        want = [m.run_yolo(x) for x in xs]
+        m.set_copy_on_forward_stream(True)
+        for rounds in range(2):
+            m.enqueue(xd[0].data_ptr())
+            for i in range(1, 3):
+                m.enqueue(xd[i].data_ptr())
+                got = m.fetch_yolo()
+                assert all(np.array_equal(a, b, equal_nan=True) for a, b in zip(got, want[i - 1]))
+            got = m.fetch_yolo()
+            assert all(np.array_equal(a, b, equal_nan=True) for a, b in zip(got, want[2]))
+        m.set_copy_on_forward_stream(False)
+        got = m.run_yolo(xs[1])
+        assert all(np.array_equal(a, b, equal_nan=True) for a, b in zip(got, want[1]))
+        cls = netapi.Net(*nu.model("resnet18", 1, 224, seed=3)[:2], fp16=True)
+        with pytest.raises(netapi.MsnhnetError):
+            cls.set_copy_on_forward_stream(True)
+    finally:
+        netapi.set_device_nms(1)
