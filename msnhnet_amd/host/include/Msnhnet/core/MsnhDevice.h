@@ -30,10 +30,10 @@ public:
     ~DeviceBuffer() { release(); }
     DeviceBuffer(const DeviceBuffer &) = delete;
     DeviceBuffer &operator=(const DeviceBuffer &) = delete;
-    DeviceBuffer(DeviceBuffer &&o) noexcept : _ptr(o._ptr), _bytes(o._bytes) { o._ptr = nullptr; o._bytes = 0; }
+    DeviceBuffer(DeviceBuffer &&o) noexcept : _ptr(o._ptr), _bytes(o._bytes), _owned(o._owned) { o._ptr = nullptr; o._bytes = 0; o._owned = true; }
     DeviceBuffer &operator=(DeviceBuffer &&o) noexcept
     {
-        if (this != &o) { release(); _ptr = o._ptr; _bytes = o._bytes; o._ptr = nullptr; o._bytes = 0; }
+        if (this != &o) { release(); _ptr = o._ptr; _bytes = o._bytes; _owned = o._owned; o._ptr = nullptr; o._bytes = 0; o._owned = true; }
         return *this;
     }
     void alloc(size_t bytes)
@@ -45,9 +45,18 @@ public:
     }
     void release()
     {
-        if (_ptr) msnh_hip_free(_ptr);
+        if (_ptr && _owned) msnh_hip_free(_ptr);
         _ptr = nullptr;
         _bytes = 0;
+        _owned = true;
+    }
+    // A view of another buffer's memory: nothing is freed when this object goes away; the owner must outlive it.
+    void aliasOf(const DeviceBuffer &o)
+    {
+        release();
+        _ptr = o._ptr;
+        _bytes = o._bytes;
+        _owned = false;
     }
     void upload(const void *host, size_t bytes, msnh_stream_t s = nullptr)
     {
@@ -62,6 +71,7 @@ public:
 private:
     void  *_ptr = nullptr;
     size_t _bytes = 0;
+    bool   _owned = true;
 };
 
 class PinnedBuffer
