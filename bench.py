@@ -175,7 +175,7 @@ def main():
                     help="detection workloads: sort + NMS on the host, on the device, or (library default) on the device while the "
                          "previous result had at most 2048 candidates per image -- the seeded weights give 11k, so auto means host here")
     ap.add_argument("--instances", type=int, default=3,
-                    help="network instances on the GPU, each with its own stream, arena and packed weights, fed round-robin by one host thread each "
+                    help="network instances on the GPU, each with its own stream and arena, fed round-robin by one host thread each "
                          "(netapi.NetGroup; device-resident input only).  The device runs their forwards side by side, which fills the launch gaps, "
                          "prologues and write bursts that a single stream leaves open.  1 = one instance, two batches in flight on one stream")
     ap.add_argument("--depth", type=int, default=2, help="--instances > 1: batches in flight per instance (detectors; a classifier has one)")

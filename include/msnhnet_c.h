@@ -170,7 +170,7 @@ long long msnhnet_time_detail(msnhnet_t net, char *dst, long long cap);       /*
 
 /* Several instances of one network on one GPU, fed round-robin: the throughput arrangement for serving (no counterpart in the
  * reference, whose callers would create several NetBuilder objects and threads themselves).  Each instance is a NetBuilder with
- * its own stream, arena, graph and packed weights, driven by its own host thread with `depth` batches in flight (detectors 1 or
+ * its own stream, arena and graph (one packed copy of the weights serves all), driven by its own host thread with `depth` batches in flight (detectors 1 or
  * 2, classifiers 1); the device runs the forwards of different instances side by side, which fills the gaps between the launches
  * of one forward.  The switches of msnhnet_set_* apply as for msnhnet_create + build + load.
  *   msnhnet_group_prime  : one forward of the device-resident float32 NCHW batch on every instance, on the calling thread

@@ -16,7 +16,7 @@ namespace Msnhnet
 //
 // A forward is a chain of dependent launches; the launch gaps, prologues and write bursts of its kernels leave much of the device idle
 // and nothing in the same stream can fill them.  Another forward on another stream can.  Each instance is a NetBuilder of its own (stream,
-// activation arena, captured graph, packed weights; the per-layer tile choices of the first are reused by the others, so all instances run
+// activation arena, captured graph; the per-layer tile choices and the packed weights of the first are used by the others, so all instances run
 // the same kernels), driven by its own host thread, which enqueues a batch and fetches the result of an earlier one so that `depth`
 // batches per instance are in flight.  Results come back in submission order.  No counterpart in the reference, whose callers would
 // create several NetBuilder objects and threads themselves.

@@ -401,7 +401,7 @@ class NetGroup:
     """Several instances of one network on one GPU, fed round-robin: a throughput configuration for serving (msnhnet_group_* of
     include/msnhnet_c.h; the host threads and queues live in the library).
 
-    Each instance is a NetBuilder of its own (own stream, activation arena, captured graph and packed weights), driven by one host
+    Each instance is a NetBuilder of its own (own stream, activation arena and captured graph; one packed copy of the weights serves all), driven by one host
     thread that enqueues a batch and fetches the result of an earlier one, so that `instances * depth` batches are in flight.  The
     device then runs the forwards of different instances side by side: the launch gaps, prologues and write bursts of one
     forward's kernels are filled by another's, which a single stream cannot do.  Results come back in submission order.
