@@ -362,7 +362,10 @@ def main():
                 "frac": round(achieved / PEAK[dtype], 4), "traffic": HBM_BYTES_PER_CONV_LAUNCH.get((a.workload, dtype, batch)),
                 "kernel": "convolution launches (implicit-GEMM MFMA + stem)", "launches_per_step": launches // 10,
                 "avg_launch_us": round(conv_ms * 1e3 / max(launches, 1), 2), "flops_per_step": flops / 10,
-                "least_bytes_per_launch": int(conv_bytes / max(launches, 1))}
+                "least_bytes_per_launch": int(conv_bytes / max(launches, 1)),
+                # the same FLOPs over the time between results of the timed region (everything included: the other launches, decode, copy-back,
+                # host stage, several instances overlapping): what the job as a whole extracts from the matrix cores
+                "whole_job_tflops": round(flops / 10 / (ms_per_step * 1e-3) / 1e12, 2), "whole_job_frac": round(flops / 10 / (ms_per_step * 1e-3) / 1e12 / PEAK[dtype], 4)}
 
     # what the matrix cores of this part sustain with nothing in their way (pure MFMA loops, three wavefronts per SIMD as in the
     # convolution kernels), and the shader clock they hold meanwhile: `peak` above is the published figure at the maximum clock
