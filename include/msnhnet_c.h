@@ -177,7 +177,8 @@ long long msnhnet_time_detail(msnhnet_t net, char *dst, long long cap);       /*
  *                          (fills each instance's input buffer, captures its graph); call once before submitting.
  *   msnhnet_group_submit : hands the next batch to the next instance; device_input as for msnhnet_enqueue (NULL = run on what
  *                          the instance's input buffer holds), valid until the batch's result has been fetched.
- *   msnhnet_group_flush  : every instance fetches what it still holds in flight (it otherwise keeps depth - 1 results back).
+ *   msnhnet_group_flush  : every instance fetches what it still holds in flight now (it otherwise keeps depth - 1 results back
+ *                          until more work comes or a fetch asks for one of them).  Calls on one group come from one thread.
  *   msnhnet_group_fetch_*: the oldest outstanding result, outputs as for msnhnet_fetch_*; blocks until it is there; an error
  *                          raised inside an instance's thread is reported by the fetch of the batch it belongs to.
  *   msnhnet_group_instance: the NetBuilder of instance i (owned by the group) for the query calls: dims, plan detail, profiles. */

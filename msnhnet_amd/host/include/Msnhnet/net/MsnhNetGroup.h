@@ -40,9 +40,11 @@ public:
     // Hands the next batch to the next instance.  deviceInput: device pointer to the batch (copied into the instance's input buffer on
     // its stream; must stay valid until the result has been fetched) or nullptr to run on what that buffer holds.
     void submit(const float *deviceInput);
-    // Makes every instance fetch what it still holds in flight (an instance otherwise keeps depth - 1 results back until more work comes).
+    // Makes every instance fetch what it still holds in flight now (an instance otherwise keeps depth - 1 results back until more work
+    // comes or one of them is asked for).
     void flush();
     // The oldest outstanding result; blocks until it is there.  An exception thrown inside an instance's thread is rethrown here.
+    // prime, submit, flush and the fetches are for one calling thread (or callers that serialise them).
     std::vector<std::vector<YoloBox>> fetchYolo();
     std::vector<float> fetchClassify();
     long long outstanding() const { return _submitted - _fetched; }
@@ -63,8 +65,10 @@ private:
         std::condition_variable cvIn, cvOut;
         std::deque<Job> in;
         std::deque<Result> out;
+        long long submitted = 0, taken = 0;                // by the caller's thread only
     };
     void drive(Lane &lane);
+    void stop();
     Result take();
     std::vector<std::unique_ptr<Lane>> _lanes;
     int _depth = 1;

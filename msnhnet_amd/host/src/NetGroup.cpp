@@ -48,14 +48,24 @@ NetGroup::NetGroup(const std::string &msnhnetPath, const std::string &msnhbinPat
     Network *n = _lanes[0]->net->getNet();
     _detect = !n->layers.empty() && n->layers.back()->type() == LayerType::YOLO_OUT;
     _depth = _detect ? std::max(1, std::min(depth, 2)) : 1;
-    for (std::unique_ptr<Lane> &lane : _lanes)
+    try
     {
-        Lane *l = lane.get();
-        l->thread = std::thread([this, l] { drive(*l); });
+        for (std::unique_ptr<Lane> &lane : _lanes)
+        {
+            Lane *l = lane.get();
+            l->thread = std::thread([this, l] { drive(*l); });
+        }
+    }
+    catch (...)
+    {
+        stop();                                             // a thread that could not be started: end the ones that were
+        throw;
     }
 }
 
-NetGroup::~NetGroup()
+NetGroup::~NetGroup() { stop(); }
+
+void NetGroup::stop()
 {
     for (std::unique_ptr<Lane> &lane : _lanes)
     {
@@ -143,6 +153,7 @@ void NetGroup::submit(const float *deviceInput)
         lane.in.push_back({0, deviceInput});
     }
     lane.cvIn.notify_one();
+    ++lane.submitted;
     ++_submitted;
 }
 
@@ -165,10 +176,18 @@ NetGroup::Result NetGroup::take()
     Result r;
     {
         std::unique_lock<std::mutex> lk(lane.m);
+        // The instance hands out its j-th result when batch j + depth - 1 arrives.  If that batch has not been submitted, the result
+        // asked for would wait for it for ever: make the instance fetch what it holds.
+        if (lane.submitted < lane.taken + _depth)
+        {
+            lane.in.push_back({1, nullptr});
+            lane.cvIn.notify_one();
+        }
         lane.cvOut.wait(lk, [&] { return !lane.out.empty(); });
         r = std::move(lane.out.front());
         lane.out.pop_front();
     }
+    ++lane.taken;
     ++_fetched;
     if (r.error) std::rethrow_exception(r.error);
     return r;

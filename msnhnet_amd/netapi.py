@@ -409,7 +409,7 @@ class NetGroup:
     prime(ptr) runs the device-resident float32 NCHW batch at `ptr` once on every instance (call it before the first submit).
     submit(ptr) hands the next batch to the next instance: a device pointer (copied into the instance's input buffer on its
     stream; keep it valid until the result is fetched) or None to run on what that buffer holds.  flush() makes the instances
-    deliver what they still hold in flight.  fetch() returns the oldest outstanding result (boxes per image for a detector,
+    deliver what they still hold in flight now (a fetch of a held-back result asks for it by itself).  fetch() returns the oldest outstanding result (boxes per image for a detector,
     logits for a classifier); an error raised inside an instance's thread surfaces in the fetch of its batch."""
 
     def __init__(self, msnhnet_path, msnhbin_path, instances=2, depth=2, fp16=False):
@@ -442,6 +442,9 @@ class NetGroup:
 
     def flush(self):
         _check(self.L.msnhnet_group_flush(self.g))
+
+    def outstanding(self):
+        return self._submitted - self._fetched
 
     def fetch(self):
         if self._fetched >= self._submitted:

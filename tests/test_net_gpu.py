@@ -584,6 +584,21 @@ def test_net_group_results_in_submission_order(arch, size, batch, instances, dep
                     assert np.array_equal(got, want[i]), (rounds, i)
         with pytest.raises(RuntimeError):
             grp.fetch()                      # nothing outstanding
+        # as a serving loop runs: a window of batches outstanding, one fetched for each one submitted, and the tail fetched without
+        # flush() (a result that its instance would hold back until more work comes is asked for by the fetch itself)
+        window = min(instances * depth, len(xd) - 1)
+        for t in xd[:window]:
+            grp.submit(t.data_ptr())
+        for i in range(len(xd)):
+            got = grp.fetch()
+            if i + window < len(xd):
+                grp.submit(xd[i + window].data_ptr())
+            if detect:
+                for a, b in zip(got, want[i]):
+                    assert np.array_equal(a, b, equal_nan=True), ("window", i)
+            else:
+                assert np.array_equal(got, want[i]), ("window", i)
+        assert grp.outstanding() == 0
         # on what an instance's input buffer holds (one of the submitted batches)
         grp.submit(None)
         grp.flush()
