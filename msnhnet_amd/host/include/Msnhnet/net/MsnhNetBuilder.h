@@ -51,6 +51,9 @@ public:
     // img holds batch*C*H*W floats, batch-major NCHW (one image when the graph's batch is 1, as in the reference).
     std::vector<float> runClassifyGPU(std::vector<float> img);
     std::vector<std::vector<YoloBox>> runYoloGPU(std::vector<float> img);
+    // the same two calls on a caller's buffer of `count` floats (what the C ABI holds: no vector is built from it)
+    std::vector<float> runClassifyGPU(const float *img, size_t count);
+    std::vector<std::vector<YoloBox>> runYoloGPU(const float *img, size_t count);
 
     // Steady-state serving path: the input already lives on the device (NCHW float32, batch*C*H*W floats).
     // Enqueues one forward on the builder's stream; results are fetched with fetchClassify / fetchYolo.
@@ -115,7 +118,7 @@ private:
     float _readMs = 0.f;
     std::string _loadDetail;
     std::unique_ptr<Plan> lowerNetwork(int dtype);
-    void uploadInput(const std::vector<float> &img);
+    void uploadInput(const float *img, size_t count);
     void runLayersEager();
     void checkInput(size_t given) const;
 

@@ -358,7 +358,7 @@ int msnhnet_run_classify_gpu(msnhnet_t net, const float *img, long long n, float
 {
     return guarded([&] {
         if (!img || n <= 0) MSNH_THROW("bad argument");
-        copyOut(nb(net).runClassifyGPU(std::vector<float>(img, img + n)), out, cap, n_out);
+        copyOut(nb(net).runClassifyGPU(img, static_cast<size_t>(n)), out, cap, n_out);
     });
 }
 
@@ -366,7 +366,7 @@ int msnhnet_run_yolo_gpu(msnhnet_t net, const float *img, long long n, int *coun
 {
     return guarded([&] {
         if (!img || n <= 0) MSNH_THROW("bad argument");
-        packBoxes(nb(net).runYoloGPU(std::vector<float>(img, img + n)), counts, boxes, cap_boxes, total);
+        packBoxes(nb(net).runYoloGPU(img, static_cast<size_t>(n)), counts, boxes, cap_boxes, total);
     });
 }
 
