@@ -117,6 +117,48 @@ def conv_shape_mode(a):
         abi.check(L.msnh_hip_conv2d(ctypes.byref(d), ptr(x), ptr(wt), ptr(sc), ptr(sh), ptr(res), ptr(y), None, 0, None))
 
     torch.cuda.synchronize()
+    if a.switches:
+        # the LDS-patch kernel with parts switched off (timing diagnostics library): where a launch's time goes and what clock the part
+        # holds under each mix of work
+        from msnhnet_amd import diag
+        if a.tile not in (46, 52) or k != 3 or stride != 1 or a.conv_dtype != "f16" or a.residual:
+            sys.exit("--switches: --tile 46 or 52, a 3x3 stride-1 float16 shape, no --residual")
+        D = diag.lib()
+        e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+        abi.check(L.msnh_hip_event_create(ctypes.byref(e0)))
+        abi.check(L.msnh_hip_event_create(ctypes.byref(e1)))
+        clocks = torch.zeros(2, dtype=torch.int64, device="cuda")
+        torch.cuda.synchronize()
+
+        def timed(fn):
+            fn()
+            fn()
+            abi.check(L.msnh_hip_event_record(e0, None))
+            for _ in range(a.reps):
+                fn()
+            abi.check(L.msnh_hip_event_record(e1, None))
+            abi.check(L.msnh_hip_event_sync(e1))
+            ms = ctypes.c_float()
+            abi.check(L.msnh_hip_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+            return ms.value * 1e3 / a.reps
+
+        for sw in diag.switches():
+            def one():
+                rc = D.msnh_hip_diag_patch8(a.tile, sw, b, c, h, w, oc, ptr(x), ptr(wt), ptr(sc), ptr(sh), ptr(y), ptr(clocks), None)
+                if rc:
+                    sys.exit(f"msnh_hip_diag_patch8: error {rc} (tile {a.tile}, switches {sw}): {L.msnh_hip_last_error()}")
+            us = timed(one)
+            line = f"tile {a.tile} switches {sw:2d} {diag.describe(sw):78s} {us:8.2f} us per launch"
+            if sw & 64:
+                t = clocks.cpu().numpy()
+                line += f"; main loop {int(t[0])} shader ticks in {t[1] / 100:.2f} us = {t[0] / max(int(t[1]), 1) * 100:.0f} MHz"
+            print(line, flush=True)
+        for blocks, threads in ((256, 768), (256, 256), (2048, 256)):
+            us = timed(lambda: D.msnh_hip_diag_empty_launch(blocks, threads, None))
+            print(f"empty kernel {blocks} x {threads}: {us:8.2f} us per launch", flush=True)
+        L.msnh_hip_event_destroy(e0)
+        L.msnh_hip_event_destroy(e1)
+        return
     if a.tile > 0:
         d.tile = a.tile
         if not L.msnh_hip_conv2d_tile_supported(ctypes.byref(d), a.tile):
@@ -162,6 +204,9 @@ def main():
     ap.add_argument("--conv-shape", default=None, help="b,c,h,w,oc,k,stride: time this one convolution shape instead of a workload")
     ap.add_argument("--tile", type=int, default=0, help="--conv-shape: launch only this tile configuration, --reps times, untimed")
     ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--switches", action="store_true",
+                    help="--conv-shape with --tile 46 or 52: the LDS-patch kernel timed with parts of it switched off and with the shader clock read inside "
+                         "(timing diagnostics library, include/msnh_hip_diag.h)")
     ap.add_argument("--residual", action="store_true", help="--conv-shape: with a fused residual add")
     ap.add_argument("--conv-dtype", default="f16", choices=["f16", "f32"])
     ap.add_argument("--workload", default="yolov3", choices=sorted(WORKLOADS))

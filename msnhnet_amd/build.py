@@ -1,7 +1,8 @@
-"""Builds the two shared libraries of the package in-tree:
+"""Builds the shared libraries of the package in-tree:
 
   msnhnet_amd/lib/libmsnh_hip.so   HIP kernels + C ABI (include/msnh_hip.h), hipcc --offload-arch=gfx950
   msnhnet_amd/lib/libMsnhnet.so    C++ host side (NetBuilder, Parser, layers) + C facade (include/msnhnet_c.h)
+  msnhnet_amd/lib/libmsnh_diag.so  timing diagnostics (include/msnh_hip_diag.h; measurement only, nothing in the product loads it)
 
 Run as `python -m msnhnet_amd.build` or through `__graft_entry__.build()`.
 """
@@ -53,12 +54,17 @@ def _compile(src, obj, flags, compiler):
 def build_hip(verbose=True):
     srcs = sorted(glob.glob(os.path.join(PKG, "csrc", "*.hip")))
     objs = [os.path.join(OBJ, "hip", os.path.basename(s) + ".o") for s in srcs]
+    diag_srcs = sorted(glob.glob(os.path.join(PKG, "csrc", "diag", "*.hip")))
+    diag_objs = [os.path.join(OBJ, "hip", "diag_" + os.path.basename(s) + ".o") for s in diag_srcs]
     with ThreadPoolExecutor(max_workers=8) as ex:
-        for out in ex.map(lambda so: _compile(so[0], so[1], HIP_FLAGS, HIPCC), zip(srcs, objs)):
+        for out in ex.map(lambda so: _compile(so[0], so[1], HIP_FLAGS, HIPCC), zip(srcs + diag_srcs, objs + diag_objs)):
             if verbose and out.strip():
                 print(out)
     os.makedirs(LIB, exist_ok=True)
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", os.path.join(LIB, "libmsnh_hip.so"), *objs])
+    if diag_objs:
+        _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", os.path.join(LIB, "libmsnh_diag.so"), *diag_objs,
+              "-L" + LIB, "-lmsnh_hip", "-Wl,-rpath,$ORIGIN"])
     return os.path.join(LIB, "libmsnh_hip.so")
 
 

@@ -32,6 +32,16 @@ def test_kernel_library_exports_every_declared_symbol():
     assert set(hipabi.SYMBOLS) == set(names) - {"msnh_hip_conv_desc"}
 
 
+def test_diagnostics_library_exports_every_declared_symbol():
+    from msnhnet_amd import diag
+    names = _declared("msnh_hip_diag.h")
+    ctypes.CDLL(hipabi.LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+    lib = ctypes.CDLL(diag.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert set(diag.SYMBOLS) == set(names)
+
+
 def test_host_library_exports_every_declared_symbol():
     names = [n for n in _declared("msnhnet_c.h") if n != "msnhnet_t"]
     lib = ctypes.CDLL(netapi.LIB_PATH)

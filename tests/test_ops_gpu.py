@@ -659,3 +659,61 @@ def test_mfma_probe():
     assert L.msnh_hip_mfma_probe(0, 100, ctypes.byref(tf), ctypes.byref(mhz), ctypes.byref(sec), None) != 0
     assert L.msnh_hip_mfma_probe(3, 0, ctypes.byref(tf), ctypes.byref(mhz), ctypes.byref(sec), None) != 0
     assert L.msnh_hip_mfma_probe(3, 100, None, ctypes.byref(mhz), ctypes.byref(sec), None) != 0
+
+
+@pytest.mark.parametrize("tile", [46, 52])
+def test_timing_diagnostics_patch_kernel(tile):
+    """the timing diagnostics library: with every switch off, and with only the clock read-out on, its instantiation of the LDS-patch
+    kernel returns bit for bit what the kernel library returns for the same tile; the clock read-out gives a plausible shader
+    clock; every listed switch combination launches and finishes; combinations that are not instantiated and bad shapes are refused"""
+    import gpuutil as gu
+    import torch
+    from msnhnet_amd import diag
+    gu.init()
+    L, D = abi.lib(), diag.lib()
+    b, c, h, w, oc = 2, 128, 38, 38, 128
+    rng = np.random.default_rng(tile)
+    x = gu.round_f16(rng.standard_normal((b, c, h, w), dtype=np.float32))
+    wt = gu.round_f16(rng.standard_normal((oc, c, 3, 3), dtype=np.float32) * np.float32(0.05))
+    scale = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    shift = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    d = abi.ConvDesc(abi.F16, abi.F16, b, h, w, c, c, oc, h, w, oc, 3, 1, 1, 1, 1, abi.ACT["leaky"], 0.1, 0, oc, abi.ACT["none"], 0.1, 1.0, 1.0,
+                     abi.ALGO["igemm"], tile)
+    assert L.msnh_hip_conv2d_tile_supported(ctypes.byref(d), tile)
+    want, used = gu.conv2d(x, wt, dtype=abi.F16, stride=1, pad=1, scale=scale, shift=shift, act="leaky", algo="igemm", tile=tile)
+    assert used == "igemm"
+    xd = torch.from_numpy(np.ascontiguousarray(x.transpose(0, 2, 3, 1))).cuda().half()
+    packed = np.zeros(L.msnh_hip_conv2d_packed_weight_elems(ctypes.byref(d), abi.ALGO["igemm"]), np.float16)
+    abi.check(L.msnh_hip_conv2d_pack_weights(ctypes.byref(d), abi.ALGO["igemm"], np.ascontiguousarray(wt, np.float32).ctypes.data_as(ctypes.POINTER(ctypes.c_float)),
+                                             packed.ctypes.data_as(ctypes.c_void_p)))
+    assert packed.size == oc * 9 * c
+    wd = torch.from_numpy(packed).cuda()
+    sc, sh = torch.from_numpy(scale).cuda(), torch.from_numpy(shift).cuda()
+    clocks = torch.zeros(2, dtype=torch.int64, device="cuda")
+    torch.cuda.synchronize()
+
+    def run(sw, y):
+        return D.msnh_hip_diag_patch8(tile, sw, b, c, h, w, oc, gu.ptr(xd), gu.ptr(wd), gu.ptr(sc), gu.ptr(sh), gu.ptr(y), gu.ptr(clocks), None)
+
+    for sw in (0, 64):
+        y = torch.full((b, h, w, oc), 3.0, dtype=torch.float16, device="cuda")
+        assert run(sw, y) == 0
+        abi.check(L.msnh_hip_stream_sync(None))
+        got = y.float().cpu().numpy().transpose(0, 3, 1, 2)
+        assert np.array_equal(got, want), sw
+    t = clocks.cpu().numpy()
+    assert t[0] > 0 and t[1] > 0
+    assert 500.0 < t[0] / t[1] * 100.0 < 2600.0             # shader ticks per 100 MHz tick
+    y = torch.empty((b, h, w, oc), dtype=torch.float16, device="cuda")
+    listed = diag.switches()
+    assert 0 in listed and 64 in listed
+    for sw in listed:
+        assert run(sw, y) == 0, sw
+    abi.check(L.msnh_hip_stream_sync(None))
+    assert run(6, y) != 0                                   # not instantiated
+    assert D.msnh_hip_diag_patch8(45, 0, b, c, h, w, oc, gu.ptr(xd), gu.ptr(wd), gu.ptr(sc), gu.ptr(sh), gu.ptr(y), gu.ptr(clocks), None) != 0
+    assert D.msnh_hip_diag_patch8(tile, 0, b, 96, h, w, oc, gu.ptr(xd), gu.ptr(wd), gu.ptr(sc), gu.ptr(sh), gu.ptr(y), gu.ptr(clocks), None) != 0
+    assert D.msnh_hip_diag_patch8(tile, 64, b, c, h, w, oc, gu.ptr(xd), gu.ptr(wd), gu.ptr(sc), gu.ptr(sh), gu.ptr(y), None, None) != 0
+    assert D.msnh_hip_diag_empty_launch(256, 256, None) == 0
+    assert D.msnh_hip_diag_empty_launch(0, 256, None) != 0
+    abi.check(L.msnh_hip_stream_sync(None))
