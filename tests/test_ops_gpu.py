@@ -697,6 +697,7 @@ def test_timing_diagnostics_patch_kernel(tile):
 
     for sw in (0, 64):
         y = torch.full((b, h, w, oc), 3.0, dtype=torch.float16, device="cuda")
+        torch.cuda.synchronize()                            # (the fill runs on torch's stream, the kernel on the library's)
         assert run(sw, y) == 0
         abi.check(L.msnh_hip_stream_sync(None))
         got = y.float().cpu().numpy().transpose(0, 3, 1, 2)
@@ -705,6 +706,7 @@ def test_timing_diagnostics_patch_kernel(tile):
     assert t[0] > 0 and t[1] > 0
     assert 500.0 < t[0] / t[1] * 100.0 < 2600.0             # shader ticks per 100 MHz tick
     y = torch.empty((b, h, w, oc), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
     listed = diag.switches()
     assert 0 in listed and 64 in listed
     for sw in listed:
