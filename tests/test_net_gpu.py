@@ -555,7 +555,7 @@ def test_cpu_entry_points_refuse():
         m.run_classify(np.zeros(10, np.float32))
 
 
-@pytest.mark.parametrize("arch,size,batch,instances,depth", [("yolov3", 96, 2, 2, 2), ("yolov3", 96, 2, 3, 1), ("resnet18", 224, 2, 2, 2)])
+@pytest.mark.parametrize("arch,size,batch,instances,depth", [("yolov3", 96, 2, 2, 2), ("yolov3", 96, 2, 3, 1), ("resnet18", 224, 2, 2, 2), ("yolov3", 96, 2, 1, 2)])
 def test_net_group_results_in_submission_order(arch, size, batch, instances, depth):
     """netapi.NetGroup: several instances of a network fed round-robin by one host thread each return, in submission order, exactly
     what one instance returns for each of the submitted batches (distinct inputs, so a swapped or repeated result shows), also for the
@@ -607,6 +607,26 @@ def test_net_group_results_in_submission_order(arch, size, batch, instances, dep
             assert any(all(np.array_equal(a, b, equal_nan=True) for a, b in zip(got, w)) for w in want)
         else:
             assert any(np.array_equal(got, w) for w in want)
+    finally:
+        grp.close()
+
+
+def test_net_group_refuses_bad_arguments(tmp_path):
+    """a group that cannot be built reports the error of the step that failed and leaves nothing running"""
+    net, binp, g = nu.model("yolov3", 2, 96, seed=3)
+    with pytest.raises(netapi.MsnhnetError, match="1 to 16 instances"):
+        netapi.NetGroup(net, binp, instances=0, depth=2, fp16=True)
+    with pytest.raises(netapi.MsnhnetError):
+        netapi.NetGroup(os.path.join(str(tmp_path), "missing.msnhnet"), binp, instances=2, depth=2, fp16=True)
+    with pytest.raises(netapi.MsnhnetError):
+        netapi.NetGroup(net, os.path.join(str(tmp_path), "missing.msnhbin"), instances=2, depth=2, fp16=True)
+    grp = netapi.NetGroup(net, binp, instances=2, depth=2, fp16=True)      # and the library still builds one afterwards
+    try:
+        x = torch.from_numpy(zoo.seeded_input(2, 3, 96, 96, seed=4)).cuda()
+        torch.cuda.synchronize()
+        grp.prime(x.data_ptr())
+        grp.submit(x.data_ptr())
+        assert len(grp.fetch()) == 2
     finally:
         grp.close()
 
