@@ -406,6 +406,7 @@ private:
     std::chrono::steady_clock::time_point _lastFinish;
     bool _haveLastFinish = false, _lastFinishHost = false;
     void noteResult(const Slot &sl, bool pipelined);
+    void prepareSlot(Slot &sl, bool deviceNmsBuffers);
     Slot _slots[2];
 };
 }

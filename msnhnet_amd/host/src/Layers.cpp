@@ -1415,6 +1415,33 @@ void YoloOutLayer::enqueueGather(msnh_stream_t s)
                                   pl.yoloCandIdx.as<int>(), pl.yoloCells, pl.yoloCandCnt.as<int>(), pl.yoloRows.as<float>(), s));
 }
 
+// Everything a slot needs, at its full size, before the slot is first used.  An allocation or a free of device or pinned memory
+// waits for the whole device: in the middle of a run, with other instances' forwards in flight, one such call stalls them all
+// for tens of milliseconds.  Both slots are prepared with the first forward (later calls find everything in place).
+void YoloOutLayer::prepareSlot(Slot &sl, bool deviceNmsBuffers)
+{
+    Plan &pl = *plan;
+    const size_t cells = static_cast<size_t>(pl.yoloCells);
+    const size_t cntBytes = sizeof(int) * static_cast<size_t>(_batch);
+    const size_t rowBytes = sizeof(float) * 8 * cells * static_cast<size_t>(_batch);
+    sl.cnt.reserve(cntBytes);
+    sl.rows.reserve(rowBytes);
+    if (sl.event == nullptr) MSNH_DEV(msnh_hip_event_create(&sl.event));
+    if (keepClassScores) return;
+    if (sl.ready == nullptr) MSNH_DEV(msnh_hip_event_create(&sl.ready));
+    if (sl.devCnt.bytes() < cntBytes) sl.devCnt.alloc(cntBytes);
+    if (sl.devRows.bytes() < rowBytes) sl.devRows.alloc(rowBytes);
+    if (!deviceNmsBuffers) return;
+    const size_t keptCntBytes = sizeof(int) * (1 + static_cast<size_t>(_batch));
+    const size_t keptCap = cells * static_cast<size_t>(_batch);
+    if (sl.devKeptCnt.bytes() < keptCntBytes) sl.devKeptCnt.alloc(keptCntBytes);
+    if (sl.devKept.bytes() < keptCap * kRecordBytes) sl.devKept.alloc(keptCap * kRecordBytes);
+    sl.keptCnt.reserve(keptCntBytes);
+    sl.kept.reserve(keptCap * kRecordBytes);
+    const size_t wsBytes = msnh_hip_yolo_nms_pair_workspace_bytes(_batch, _channel - 5, pl.yoloCells);
+    if (sl.devNmsWs.bytes() < wsBytes) sl.devNmsWs.alloc(wsBytes);
+}
+
 void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
 {
     Plan &pl = *plan;
@@ -1422,9 +1449,9 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
     if (sl.pending) MSNH_THROW("YoloOut: the results of the previous forward in this slot were not fetched");
     sl.onDevice = false;
     const size_t cells = static_cast<size_t>(pl.yoloCells);
-    sl.cnt.reserve(sizeof(int) * static_cast<size_t>(_batch));
-    sl.rows.reserve(sizeof(float) * 8 * cells * static_cast<size_t>(_batch));
-    if (sl.event == nullptr) MSNH_DEV(msnh_hip_event_create(&sl.event));
+    const bool mayUseDevice = deviceNms != 0 && !_useSoftNms && !keepClassScores;
+    prepareSlot(_slots[0], mayUseDevice);
+    prepareSlot(_slots[1], mayUseDevice);
     const size_t cntBytes = sizeof(int) * static_cast<size_t>(_batch);
     const size_t rowBytes = sizeof(float) * 8 * cells * static_cast<size_t>(_batch);
     if (keepClassScores)
@@ -1449,9 +1476,6 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
     // other instances fill the gap.
     if (!copyOnForwardStream && _copyStream == nullptr) MSNH_DEV(msnh_hip_stream_create(&_copyStream));
     const msnh_stream_t cs = copyOnForwardStream ? s : _copyStream;
-    if (sl.ready == nullptr) MSNH_DEV(msnh_hip_event_create(&sl.ready));
-    if (sl.devCnt.bytes() < cntBytes) sl.devCnt.alloc(cntBytes);
-    if (sl.devRows.bytes() < rowBytes) sl.devRows.alloc(rowBytes);
     MSNH_DEV(msnh_hip_memcpy_d2d(sl.devCnt.ptr(), pl.yoloCandCnt.ptr(), cntBytes, s));
     MSNH_DEV(msnh_hip_memcpy_d2d(sl.devRows.ptr(), pl.yoloRows.ptr(), rowBytes, s));
     MSNH_DEV(msnh_hip_event_record(sl.ready, s));
@@ -1462,9 +1486,11 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
     // device time per batch from it) and the host stage has kept up with the device so far
     const bool pipelined = _slots[(slot ^ 1) & 1].pending;
     const bool mid = _lastMaxCandidates > kDeviceNmsFew && _lastMaxCandidates <= kDeviceNmsCandidates;
-    sl.trial = deviceNms == 1 && !_useSoftNms && mid && pipelined && !_hostBound && _trialLeft > 0;
+    sl.trial = deviceNms == 1 && !_useSoftNms && mid && pipelined && !_hostBound && _trialLeft > 0 && !copyOnForwardStream;
     if (sl.trial) --_trialLeft;
-    const bool autoDevice = _lastMaxCandidates <= kDeviceNmsFew || (mid && (!pipelined || _hostBound || sl.trial));
+    // (on the forward's own stream the device NMS would sit in front of the instance's next forward: the instances of a group keep
+    //  thousands of candidates on the host, which works beside the other instances' forwards)
+    const bool autoDevice = _lastMaxCandidates <= kDeviceNmsFew || (mid && !copyOnForwardStream && (!pipelined || _hostBound || sl.trial));
     sl.onDevice = !_useSoftNms && (deviceNms == 2 || (deviceNms == 1 && autoDevice));
     if (sl.onDevice)
     {
@@ -1474,14 +1500,9 @@ void YoloOutLayer::enqueueCopyBack(msnh_stream_t s, int slot)
         // beside it.  finish() fetches the rest only if there are more.
         const size_t keptCntBytes = sizeof(int) * (1 + static_cast<size_t>(_batch));
         const size_t keptCap = cells * static_cast<size_t>(_batch);
-        if (sl.devKeptCnt.bytes() < keptCntBytes) sl.devKeptCnt.alloc(keptCntBytes);
-        if (sl.devKept.bytes() < keptCap * kRecordBytes) sl.devKept.alloc(keptCap * kRecordBytes);
-        sl.keptCnt.reserve(keptCntBytes);
         sl.quick = std::min(keptCap, std::max(kQuickRecords, _lastKept + _lastKept / 2 + 1024));
-        sl.kept.reserve(sl.quick * kRecordBytes);
         MSNH_DEV(msnh_hip_fill_zero(sl.devKeptCnt.ptr(), keptCntBytes, cs));
         const size_t wsBytes = msnh_hip_yolo_nms_pair_workspace_bytes(_batch, _channel - 5, pl.yoloCells);
-        if (sl.devNmsWs.bytes() < wsBytes) sl.devNmsWs.alloc(wsBytes);
         MSNH_DEV(msnh_hip_yolo_nms(_batch, _channel - 5, sl.devRows.as<float>(), pl.yoloCells, sl.devCnt.as<int>(), _nmsThresh, sl.devKept.as<float>(),
                                    static_cast<int>(keptCap), sl.devKeptCnt.as<int>(), sl.devNmsWs.ptr(), wsBytes, cs));
         MSNH_DEV(msnh_hip_memcpy_d2h(sl.keptCnt.ptr(), sl.devKeptCnt.ptr(), keptCntBytes, cs));
