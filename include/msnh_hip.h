@@ -342,8 +342,13 @@ int msnh_hip_yolo_nms(int batch, int classes, const float *rows, int cand_cap, c
  * the workspace is a device array inside the library: msnh_hip_yolo_nms_static_max_bytes() = 4 MiB per GPU the library runs on, held
  * until the process ends.  A geometry whose msnh_hip_yolo_nms_workspace_bytes() exceeds that is refused with an error (YOLOv3 / YOLOv4
  * at 608 x 608 with 80 classes, 22743 candidate slots per image, fit up to batch 45).  The call itself allocates and frees nothing; its one-time set-up per device runs
- * in msnh_hip_init (or in the first call on a device that msnh_hip_init did not select).  Every call on a GPU shares that GPU's
- * array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream follow each other safely. */
+ * in msnh_hip_init (or in the first call on a device that msnh_hip_init did not select; a failure of that set-up is reported by this
+ * call, not by msnh_hip_init).  Every call on a GPU shares that GPU's array, so the library puts the calls on a GPU in order: they
+ * are enqueued one at a time (a lock), and a call on another stream than the call before it makes its stream wait, on the device,
+ * for that call's end; the host does not block.  Calls from several threads or streams are therefore safe but run one after the
+ * other.  The exception is a stream under graph capture: a captured call neither waits for earlier calls nor is waited for
+ * (events cannot cross a capture's boundary), so a caller who captures this call keeps the replays of that graph apart from every
+ * other use of the entry point on the same GPU. */
 size_t msnh_hip_yolo_nms_static_max_bytes(void);
 int msnh_hip_yolo_nms_static(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept,
                              int kept_cap, int *kept_cnt, msnh_stream_t s);

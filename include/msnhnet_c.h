@@ -58,8 +58,11 @@ int runClassifyNoPred(char **msg, const float *data, const int len, int *bestInd
 int runYoloNoPred(char **msg, const float *data, const int len, BBoxContainer *bboxContainer, int *detectedNum, int runGPU);
 /* One 8-bit image (HWC, `channel` bytes per pixel, host memory) -> pre-processing named by preDataType (a PredDataType) on the
  * device -> forward -> index of the largest logit.  MsnhnetLib.h:44-46; the reference's own implementation needs its OpenCV
- * build (MsnhnetLib.cpp:97-...), here the in-tree CVUtil variants are followed (src/utils/MsnhCVUtil.cpp:91-375).  swapRGB
- * exchanges the first and third channel.  mean / std: three floats each, read only by PRE_DATA_TRANSFORMED_FC3.  Errors as the
+ * build (MsnhnetLib.cpp:97-...), here the facade of the build without OpenCV is followed (MsnhnetLib.cpp:540-905 over
+ * src/utils/MsnhCVUtil.cpp:91-375), including what swapRGB means there: that facade exchanges the first and third channel itself
+ * when swapRGB == 0 (:562, :771) and CVUtil exchanges them again by default for every variant except the letterbox, so the
+ * network sees the caller's channel order when swapRGB == 0 -- except with PRE_DATA_PADDING_ZERO_FC3 and in runYoloList, where it
+ * sees it when swapRGB != 0.  mean / std: three floats each, read only by PRE_DATA_TRANSFORMED_FC3.  Errors as the
  * reference's: "channel must be 1 or 3", "channel 1 must preprocess with F32_C1", "preDataType can't be none",
  * "mean or std can't be null"; 1-channel images and runGPU == 0 fail (no gray path, no CPU path in this build). */
 int runClassifyList(char **msg, unsigned char *imageData, const int width, const int height, const int channel, int *bestIndex,

@@ -13,7 +13,7 @@ namespace msnh {
 // ---- error reporting ------------------------------------------------------------------------------
 void setError(const char *fmt, ...);
 hipStream_t resolveStream(msnh_stream_t s);
-int yoloNmsSetupDevice();            // per-device set-up of msnh_hip_yolo_nms_static (csrc/yolo.hip), on the current device
+void yoloNmsSetupDevice();           // per-device set-up of the device NMS (csrc/yolo.hip) on the current device; failures are reported by the calls that need it
 
 #define MSNH_HIP_CHECK(expr)                                                                      \
     do {                                                                                          \

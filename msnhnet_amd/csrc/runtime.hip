@@ -50,7 +50,8 @@ int msnh_hip_init(int device)
         MSNH_HIP_CHECK(hipStreamCreateWithFlags(&g_defaultStream, hipStreamNonBlocking));
         g_device = device;
     }
-    return yoloNmsSetupDevice();
+    yoloNmsSetupDevice();
+    return 0;
 }
 
 int msnh_hip_device_count(int *count)

@@ -1134,7 +1134,7 @@ extern "C" size_t msnh_hip_yolo_nms_pair_workspace_bytes(int batch, int classes,
 // The launches of the device NMS; ws = [batch*classes] class sizes | [batch*cand_cap] sorted rows | [batch] cursors, or NULL (small
 // classes only); with wsBytes beyond that part (16-byte aligned): | header | class list | boxes | matrix pool.
 static int launchYoloNms(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept, int kept_cap,
-                         int *kept_cnt, int *ws, size_t wsBytes, bool kernelsReady, hipStream_t st)
+                         int *kept_cnt, int *ws, size_t wsBytes, hipStream_t st)
 {
     int *bigCnt = ws;
     int *wsSorted = bigCnt ? bigCnt + static_cast<size_t>(batch) * classes : nullptr;
@@ -1155,12 +1155,6 @@ static int launchYoloNms(int batch, int classes, const float *rows, int cand_cap
                        pw.pool ? NMS_PAIR_MIN : NMS_CAP);
     MSNH_LAUNCH_CHECK();
     if (ws == nullptr) return 0;
-    if (!kernelsReady)
-    {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsBigKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_BIG_LDS);
-        if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsScanKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_SCAN_LDS);
-        if (e != hipSuccess) { setError("hipFuncSetAttribute: %s", hipGetErrorString(e)); return 1; }
-    }
     hipLaunchKernelGGL(yoloNmsBigKernel, dim3(classes, batch), dim3(NMS_BIG_THREADS), NMS_BIG_LDS, st, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt,
                        bigCnt, wsSorted, wsUsed, pw, pw.pool ? NMS_PAIR_MIN : NMS_CAP);
     MSNH_LAUNCH_CHECK();
@@ -1181,16 +1175,6 @@ static int checkYoloNmsArgs(int batch, int classes, const float *rows, int cand_
     return 0;
 }
 
-extern "C" int msnh_hip_yolo_nms(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept,
-                                 int kept_cap, int *kept_cnt, void *workspace, size_t workspace_bytes, msnh_stream_t s)
-{
-    if (int rc = checkYoloNmsArgs(batch, classes, rows, cand_cap, cand_cnt, kept, kept_cap, kept_cnt)) return rc;
-    MSNH_REQUIRE(workspace == nullptr || (workspace_bytes >= msnh_hip_yolo_nms_workspace_bytes(batch, classes, cand_cap) && reinterpret_cast<uintptr_t>(workspace) % 4 == 0),
-                 "yolo_nms: workspace too small (msnh_hip_yolo_nms_workspace_bytes)");
-    return launchYoloNms(batch, classes, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, static_cast<int *>(workspace), workspace ? workspace_bytes : 0, false,
-                         resolveStream(s));
-}
-
 // ---- the same call for callers that cannot allocate ------------------------------------------------------------------------------
 // The workspace lives in a device array of this module: 4 MiB per GPU the library runs on, held until the process ends.  The
 // array's name is only a host-side stand-in; its device address is asked for once per device and kept.
@@ -1198,27 +1182,90 @@ namespace {
 constexpr size_t kNmsScratchInts = static_cast<size_t>(1) << 20;
 constexpr int kMaxDevices = 64;
 static __device__ __align__(256) int scratch[kNmsScratchInts];
-int *g_scratchPtr[kMaxDevices] = {};
-std::mutex g_scratchMutex;
+struct NmsDeviceState
+{
+    bool attrsTried = false, attrsOk = false;       // the large-class kernels' LDS limits (both entry points need them)
+    bool scratchTried = false;
+    int *scratchPtr = nullptr;                      // device address of `scratch` on this device
+    hipEvent_t done = nullptr;                      // end of the last msnh_hip_yolo_nms_static call on this device
+    bool haveDone = false;
+    hipStream_t lastStream = nullptr;
+    char error[256] = {0};                          // why the set-up failed, reported by the calls that need it
+};
+NmsDeviceState g_nms[kMaxDevices];
+std::mutex g_nmsMutex;                              // guards g_nms and orders the static entry point's calls
+
+int currentDevice(int *dev)
+{
+    MSNH_HIP_CHECK(hipGetDevice(dev));
+    MSNH_REQUIRE(*dev >= 0 && *dev < kMaxDevices, "yolo_nms: device index %d is beyond the %d this library keeps state for", *dev, kMaxDevices);
+    return 0;
+}
+
+// (g_nmsMutex held) once per device: the LDS limits of the large-class kernels
+bool ensureNmsAttributes(NmsDeviceState &st)
+{
+    if (st.attrsTried) return st.attrsOk;
+    st.attrsTried = true;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsBigKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_BIG_LDS);
+    if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsScanKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_SCAN_LDS);
+    if (e != hipSuccess)
+    {
+        std::snprintf(st.error, sizeof(st.error), "yolo_nms: hipFuncSetAttribute for the large-class kernels: %s", hipGetErrorString(e));
+        (void)hipGetLastError();
+    }
+    st.attrsOk = e == hipSuccess;
+    return st.attrsOk;
+}
+
+// (g_nmsMutex held) once per device: the scratch array's address there and the event that orders the calls
+bool ensureNmsScratch(NmsDeviceState &st)
+{
+    if (st.scratchTried) return st.scratchPtr != nullptr;
+    st.scratchTried = true;
+    void *p = nullptr;
+    hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e == hipSuccess && p == nullptr) e = hipErrorInvalidSymbol;
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&st.done, hipEventDisableTiming);
+    if (e != hipSuccess)
+    {
+        std::snprintf(st.error, sizeof(st.error), "yolo_nms_static: set-up of the built-in workspace: %s", hipGetErrorString(e));
+        (void)hipGetLastError();
+        return false;
+    }
+    st.scratchPtr = static_cast<int *>(p);
+    return true;
+}
 }
 
 namespace msnh {
-// One-time set-up on the current device: the scratch array's address there, and the large-class kernel's LDS limit.
-int yoloNmsSetupDevice()
+// One-time set-up on the current device, called by msnh_hip_init.  A failure here does not fail the library's initialisation: it is
+// kept and reported by the calls that need what could not be set up (msnh_hip_yolo_nms_static, the large-class path).
+void yoloNmsSetupDevice()
 {
     int dev = -1;
-    MSNH_HIP_CHECK(hipGetDevice(&dev));
-    MSNH_REQUIRE(dev >= 0 && dev < kMaxDevices, "yolo_nms_static: device index %d is beyond the %d this library keeps state for", dev, kMaxDevices);
-    std::lock_guard<std::mutex> lock(g_scratchMutex);
-    if (g_scratchPtr[dev] != nullptr) return 0;
-    void *p = nullptr;
-    MSNH_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
-    MSNH_REQUIRE(p != nullptr, "yolo_nms_static: the scratch array has no address on device %d", dev);
-    MSNH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsBigKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_BIG_LDS));
-    MSNH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(yoloNmsScanKernel), hipFuncAttributeMaxDynamicSharedMemorySize, NMS_SCAN_LDS));
-    g_scratchPtr[dev] = static_cast<int *>(p);
-    return 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) { (void)hipGetLastError(); return; }
+    std::lock_guard<std::mutex> lock(g_nmsMutex);
+    ensureNmsAttributes(g_nms[dev]);
+    ensureNmsScratch(g_nms[dev]);
 }
+}
+
+extern "C" int msnh_hip_yolo_nms(int batch, int classes, const float *rows, int cand_cap, const int *cand_cnt, float nms_thresh, float *kept,
+                                 int kept_cap, int *kept_cnt, void *workspace, size_t workspace_bytes, msnh_stream_t s)
+{
+    if (int rc = checkYoloNmsArgs(batch, classes, rows, cand_cap, cand_cnt, kept, kept_cap, kept_cnt)) return rc;
+    MSNH_REQUIRE(workspace == nullptr || (workspace_bytes >= msnh_hip_yolo_nms_workspace_bytes(batch, classes, cand_cap) && reinterpret_cast<uintptr_t>(workspace) % 4 == 0),
+                 "yolo_nms: workspace too small (msnh_hip_yolo_nms_workspace_bytes)");
+    if (workspace != nullptr)
+    {
+        int dev = -1;
+        if (int rc = currentDevice(&dev)) return rc;
+        std::lock_guard<std::mutex> lock(g_nmsMutex);
+        MSNH_REQUIRE(ensureNmsAttributes(g_nms[dev]), "%s", g_nms[dev].error);
+    }
+    return launchYoloNms(batch, classes, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, static_cast<int *>(workspace), workspace ? workspace_bytes : 0,
+                         resolveStream(s));
 }
 
 extern "C" size_t msnh_hip_yolo_nms_static_max_bytes(void) { return kNmsScratchInts * sizeof(int); }
@@ -1232,13 +1279,30 @@ extern "C" int msnh_hip_yolo_nms_static(int batch, int classes, const float *row
                  "yolo_nms_static: batch %d x (%d classes + %d candidate slots + 1) needs %zu bytes of workspace, the built-in one holds %zu; "
                  "use msnh_hip_yolo_nms with a workspace of the caller", batch, classes, cand_cap, need, kNmsScratchInts * sizeof(int));
     int dev = -1;
-    MSNH_HIP_CHECK(hipGetDevice(&dev));
-    MSNH_REQUIRE(dev >= 0 && dev < kMaxDevices, "yolo_nms_static: device index %d is beyond the %d this library keeps state for", dev, kMaxDevices);
-    if (g_scratchPtr[dev] == nullptr)
-        if (int rc = yoloNmsSetupDevice()) return rc;        // (msnh_hip_init does this for the device it selects)
+    if (int rc = currentDevice(&dev)) return rc;
+    // Every call on a device works in that device's one array.  The calls are put in order here: enqueued one at a time (the lock),
+    // and a call on another stream than the call before it first makes its stream wait for that call's end (an event recorded behind
+    // its launches) -- on the device, the host does not block.  A stream under graph capture cannot wait for an event recorded
+    // outside the capture nor record one for later calls: captured calls are ordered by the graph's own edges, and keeping them
+    // apart from other users of the array is left to the caller.
+    std::lock_guard<std::mutex> lock(g_nmsMutex);
+    NmsDeviceState &st = g_nms[dev];
+    MSNH_REQUIRE(ensureNmsScratch(st) && ensureNmsAttributes(st), "%s", st.error);
+    const hipStream_t stream = resolveStream(s);
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capture) != hipSuccess) { capture = hipStreamCaptureStatusNone; (void)hipGetLastError(); }
+    const bool ordered = capture == hipStreamCaptureStatusNone;
+    if (ordered && st.haveDone && st.lastStream != stream) MSNH_HIP_CHECK(hipStreamWaitEvent(stream, st.done, 0));
     // Nothing in the workspace has to start at zero: the first kernel writes every class size and resets every image's cursor,
     // and the sorted rows are written before they are read.
-    return launchYoloNms(batch, classes, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, g_scratchPtr[dev], need, true, resolveStream(s));
+    const int rc = launchYoloNms(batch, classes, rows, cand_cap, cand_cnt, nms_thresh, kept, kept_cap, kept_cnt, st.scratchPtr, need, stream);
+    if (ordered)
+    {
+        MSNH_HIP_CHECK(hipEventRecord(st.done, stream));
+        st.haveDone = true;
+        st.lastStream = stream;
+    }
+    return rc;
 }
 
 extern "C" int msnh_hip_absmax(int dtype, long long pixels, int c, const void *x, int x_ld, float *result, msnh_stream_t s)

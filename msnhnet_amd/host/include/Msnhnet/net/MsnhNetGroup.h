@@ -56,7 +56,7 @@ private:
         std::vector<float> logits;
         std::exception_ptr error;
     };
-    struct Job { int kind; const float *input; };          // kind 0 = forward, 1 = flush, 2 = stop
+    struct Job { int kind; const float *input; bool fail; };          // kind 0 = forward, 1 = flush, 2 = stop; fail: see submit()
     struct Lane
     {
         std::unique_ptr<NetBuilder> net;

@@ -148,6 +148,14 @@ static int preprocOf(int preDataType, int channel)
     MSNH_THROW("preDataType can't be none");
 }
 
+// Whether the network sees the first and third channel of the caller's image exchanged.  The reference's facade (its build without
+// OpenCV) exchanges them itself when swapRGB == 0 (src/c_api/MsnhnetLib.cpp:562-565, :771-774) and then calls the CVUtil function
+// with its default needShuffleRGB, which exchanges them once more for every variant but the letterbox
+// (include/Msnhnet/utils/MsnhCVUtil.h:23-38: true for getImgDataF32C3 / getGoogLenetF32C3 / getTransformedF32C3 / getCaffeModeF32C3,
+// false for getPaddingZeroF32C3).  Net effect: exchanged when swapRGB != 0, except for the letterbox, where it is exchanged when
+// swapRGB == 0.
+static bool facadeShuffle(int kind, int swapRGB) { return kind == MSNH_PRE_PADDING_ZERO ? swapRGB == 0 : swapRGB != 0; }
+
 int runClassifyList(char **msg, unsigned char *imageData, const int width, const int height, const int channel, int *bestIndex, int preDataType,
                     const int swapRGB, int runGPU, const float *mean, const float *std)
 {
@@ -158,7 +166,7 @@ int runClassifyList(char **msg, unsigned char *imageData, const int width, const
         if (kind == MSNH_PRE_TRANSFORMED && (mean == nullptr || std == nullptr)) MSNH_THROW("mean or std can't be null");
         if (!runGPU) g_net->runClassify(std::vector<float>());           // throws: this build has no CPU path
         if (g_net->getBatch() != 1) MSNH_THROW("runClassifyList takes one image: build the graph with batch 1");
-        g_net->setInputImage(0, imageData, width, height, kind, mean, std, swapRGB != 0);
+        g_net->setInputImage(0, imageData, width, height, kind, mean, std, facadeShuffle(kind, swapRGB));
         g_net->enqueueForward(nullptr);
         const std::vector<float> out = g_net->fetchClassify();
         *bestIndex = static_cast<int>(std::distance(out.begin(), std::max_element(out.begin(), out.end())));
@@ -175,7 +183,7 @@ int runYoloList(char **msg, unsigned char *imageData, const int width, const int
         if (channel == 1) MSNH_THROW("1-channel images are outside the convolutional path this build implements");
         if (!runGPU) g_net->runYolo(std::vector<float>());               // throws: this build has no CPU path
         if (g_net->getBatch() != 1) MSNH_THROW("runYoloList takes one image: build the graph with batch 1");
-        g_net->setInputImage(0, imageData, width, height, MSNH_PRE_PADDING_ZERO, nullptr, nullptr, swapRGB != 0);
+        g_net->setInputImage(0, imageData, width, height, MSNH_PRE_PADDING_ZERO, nullptr, nullptr, facadeShuffle(MSNH_PRE_PADDING_ZERO, swapRGB));
         g_net->enqueueForward(nullptr);
         const std::vector<std::vector<YoloBox>> out = g_net->fetchYolo();
         const std::vector<YoloBox> &b0 = out.at(0);

@@ -71,7 +71,7 @@ void NetGroup::stop()
     {
         {
             std::lock_guard<std::mutex> lk(lane->m);
-            lane->in.push_back({2, nullptr});
+            lane->in.push_back({2, nullptr, false});
         }
         lane->cvIn.notify_one();
     }
@@ -115,14 +115,17 @@ void NetGroup::drive(Lane &lane)
         }
         try
         {
+            if (job.fail) MSNH_THROW("NetGroup: enqueue failure requested by MSNH_GROUP_FAIL_ENQUEUE");
             lane.net->enqueueForward(job.input);
             ++inFlight;
         }
         catch (...)
         {
-            // the batch has no result of its own: its place in the order carries the error
+            // the batch has no result of its own: its place in the order carries the error.  The results of the batches
+            // enqueued before it come first, so that every fetch still returns what belongs to its own submission.
             Result r;
             r.error = std::current_exception();
+            while (inFlight > 0) fetchOne();
             {
                 std::lock_guard<std::mutex> lk(lane.m);
                 lane.out.push_back(std::move(r));
@@ -150,7 +153,9 @@ void NetGroup::submit(const float *deviceInput)
     Lane &lane = *_lanes[static_cast<size_t>(_submitted % static_cast<long long>(_lanes.size()))];
     {
         std::lock_guard<std::mutex> lk(lane.m);
-        lane.in.push_back({0, deviceInput});
+        // (tests) MSNH_GROUP_FAIL_ENQUEUE = n: the n-th submission of the group fails when its instance tries to enqueue it
+        const char *failAt = std::getenv("MSNH_GROUP_FAIL_ENQUEUE");
+        lane.in.push_back({0, deviceInput, failAt != nullptr && std::atoll(failAt) == _submitted});
     }
     lane.cvIn.notify_one();
     ++lane.submitted;
@@ -163,7 +168,7 @@ void NetGroup::flush()
     {
         {
             std::lock_guard<std::mutex> lk(lane->m);
-            lane->in.push_back({1, nullptr});
+            lane->in.push_back({1, nullptr, false});
         }
         lane->cvIn.notify_one();
     }
@@ -180,7 +185,7 @@ NetGroup::Result NetGroup::take()
         // asked for would wait for it for ever: make the instance fetch what it holds.
         if (lane.submitted < lane.taken + _depth)
         {
-            lane.in.push_back({1, nullptr});
+            lane.in.push_back({1, nullptr, false});
             lane.cvIn.notify_one();
         }
         lane.cvOut.wait(lk, [&] { return !lane.out.empty(); });

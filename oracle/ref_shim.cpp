@@ -7,7 +7,8 @@
 //   NetBuilder::loadWeightsFromMsnhBin (src/net/MsnhNetBuilder.cpp:624-663)
 //   the layer loop of runClassify/runYolo (src/net/MsnhNetBuilder.cpp:686-728, 763-806),
 //   restated here only so that every layer's output can be captured the way the reference's own
-//   setSaveLayerOutput dump does (src/net/MsnhNetBuilder.cpp:704-720).
+//   setSaveLayerOutput dump does (src/net/MsnhNetBuilder.cpp:704-720);
+//   the C facade runClassifyList / runYoloList (src/c_api/MsnhnetLib.cpp:540-905) through ref_facade_*.
 #include <vector>
 #include <string>
 #include <cstring>
@@ -19,6 +20,7 @@
 #include <map>
 #include <algorithm>
 #include <chrono>
+#include <cstdint>
 
 #define private public      // NetBuilder::_netState has no getter; the capture loop needs the pools
 #include "Msnhnet/net/MsnhNetBuilder.h"
@@ -316,6 +318,63 @@ void ref_bbox_resize2org(float *xywh, int curW, int curH, int orgW, int orgH, in
     else      YoloOutLayer::bboxResize2Org(b, Point2I(curW, curH), Point2I(orgW, orgH));
     xywh[0] = b.xywhBox.x; xywh[1] = b.xywhBox.y; xywh[2] = b.xywhBox.w; xywh[3] = b.xywhBox.h;
 }
+
+// ---- the reference's own C facade (src/c_api/MsnhnetLib.cpp, the build without OpenCV: :463-905), compiled from its source by
+// oracle/Makefile.  Its functions are declared here by hand: its header pulls in the umbrella header of the whole project.
+// The facade keeps one process-wide network (MsnhnetLib.cpp:3); the wrappers below drive it on the CPU (runGPU = 0).
+struct RefFacadeBBox { float x, y, w, h, conf, bestClsConf; uint32_t bestClsIdx; float angle; };      // MsnhnetLib.h:22-32
+struct RefFacadeBBoxContainer { RefFacadeBBox boxes[1024]; };                                            // MsnhnetLib.h:9, :34-37
+int initMsnhnet();
+int buildMsnhnet(char **msg, const char *msnhnet, const char *msnhbin, int useFp16, int useCudaOnly);
+int runClassifyList(char **msg, unsigned char *imageData, const int width, const int height, const int channel, int *bestIndex,
+                    int preDataType, const int swapRGB, int runGPU, const float *mean, const float *std);
+int runYoloList(char **msg, unsigned char *imageData, const int width, const int height, const int channel,
+                RefFacadeBBoxContainer *bboxContainer, int *detectedNum, const int swapRGB, const int runGPU);
+int dispose();
+
+// initMsnhnet + buildMsnhnet; scalarMode as for ref_create.  Returns the facade's own code (1 = success).
+int ref_facade_build(const char *msnhnetPath, const char *msnhbinPath, int scalarMode)
+{
+    std::streambuf *old = std::cout.rdbuf(nullptr);
+    initMsnhnet();
+    std::cout.rdbuf(old);
+    if(scalarMode)
+    {
+        BaseLayer::supportAvx = false;
+        BaseLayer::supportFma = false;
+    }
+    char *msg = nullptr;                // on failure the facade leaves a pointer into a destroyed vector here (:29-31): never read
+    return buildMsnhnet(&msg, msnhnetPath, msnhbinPath, 0, 0);
+}
+
+// runClassifyList on a private copy of a 3-channel image (the facade converts its argument in place, :562-565)
+int ref_facade_classify_list(const unsigned char *img, int width, int height, int preDataType, int swapRGB, const float *mean,
+                             const float *stdv, int *bestIndex)
+{
+    std::vector<unsigned char> copy(img, img + static_cast<size_t>(width) * height * 3);
+    char *msg = nullptr;
+    return runClassifyList(&msg, copy.data(), width, height, 3, bestIndex, preDataType, swapRGB, 0, mean, stdv);
+}
+
+// runYoloList likewise; dst receives rows of 7 floats (x y w h conf bestClsConf bestClsIdx), *count the number of boxes
+int ref_facade_yolo_list(const unsigned char *img, int width, int height, int swapRGB, float *dst, int capBoxes, int *count)
+{
+    std::vector<unsigned char> copy(img, img + static_cast<size_t>(width) * height * 3);
+    std::unique_ptr<RefFacadeBBoxContainer> box(new RefFacadeBBoxContainer());
+    char *msg = nullptr;
+    *count = 0;
+    const int rc = runYoloList(&msg, copy.data(), width, height, 3, box.get(), count, swapRGB, 0);
+    if(rc != 1) return rc;
+    for(int i = 0; i < *count && i < capBoxes; ++i)
+    {
+        const RefFacadeBBox &q = box->boxes[i];
+        float *o = dst + 7 * i;
+        o[0] = q.x; o[1] = q.y; o[2] = q.w; o[3] = q.h; o[4] = q.conf; o[5] = q.bestClsConf; o[6] = static_cast<float>(q.bestClsIdx);
+    }
+    return rc;
+}
+
+int ref_facade_dispose() { return dispose(); }
 
 void ref_set_threads_note(int *ompMax)
 {

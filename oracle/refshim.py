@@ -49,6 +49,10 @@ def lib():
         L.ref_letterbox_u8.argtypes = [u8p, ci, ci, ci, ci, ci, ci, fp, cp, ci]
         L.ref_bbox_resize2org.argtypes = [fp, ci, ci, ci, ci, ci]
         L.ref_preproc_u8.argtypes = [u8p, ci, ci, ci, ci, ci, fp, fp, ci, fp, cp, ci]
+        ip = ctypes.POINTER(ci)
+        L.ref_facade_build.argtypes = [cp, cp, ci]
+        L.ref_facade_classify_list.argtypes = [u8p, ci, ci, ci, ci, fp, fp, ip]
+        L.ref_facade_yolo_list.argtypes = [u8p, ci, ci, ci, fp, ci, ip]
         _lib = L
     return _lib
 
@@ -173,3 +177,44 @@ def bbox_resize2org(xywh, cur_w, cur_h, org_w, org_h, no_pad=False):
     b = np.array(xywh, np.float32)
     lib().ref_bbox_resize2org(b.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), cur_w, cur_h, org_w, org_h, int(no_pad))
     return b
+
+
+class RefFacade:
+    """The reference's own C facade (src/c_api/MsnhnetLib.cpp, the build without OpenCV) on its CPU path: initMsnhnet + buildMsnhnet,
+    then runClassifyList / runYoloList on 8-bit HWC images.  One process-wide network, as in the reference."""
+    PRE = {"none": 0, "c1": 1, "f32c3": 2, "googlenet": 3, "padding_zero": 4, "transformed": 5, "caffe": 6}      # PredDataType
+
+    def __init__(self, msnhnet, msnhbin, scalar=True):
+        self.L = lib()
+        if self.L.ref_facade_build(msnhnet.encode(), msnhbin.encode(), 1 if scalar else 0) != 1:
+            raise RefError("the reference's buildMsnhnet failed")
+
+    def classify_list(self, img, pre, swap_rgb, mean=None, std=None):
+        a = np.ascontiguousarray(img, np.uint8)
+        h, w, c = a.shape
+        assert c == 3
+        fp = ctypes.POINTER(ctypes.c_float)
+        m = None if mean is None else np.ascontiguousarray(mean, np.float32)
+        sd = None if std is None else np.ascontiguousarray(std, np.float32)
+        best = ctypes.c_int(-1)
+        rc = self.L.ref_facade_classify_list(a.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte)), w, h, self.PRE[pre], int(swap_rgb),
+                                             None if m is None else m.ctypes.data_as(fp), None if sd is None else sd.ctypes.data_as(fp),
+                                             ctypes.byref(best))
+        if rc != 1:
+            raise RefError(f"the reference's runClassifyList returned {rc}")
+        return best.value
+
+    def yolo_list(self, img, swap_rgb):
+        a = np.ascontiguousarray(img, np.uint8)
+        h, w, c = a.shape
+        assert c == 3
+        out = np.empty((1024, 7), np.float32)
+        n = ctypes.c_int(0)
+        rc = self.L.ref_facade_yolo_list(a.ctypes.data_as(ctypes.POINTER(ctypes.c_ubyte)), w, h, int(swap_rgb),
+                                         out.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), 1024, ctypes.byref(n))
+        if rc != 1:
+            raise RefError(f"the reference's runYoloList returned {rc}")
+        return out[:n.value].copy()
+
+    def close(self):
+        self.L.ref_facade_dispose()

@@ -30,6 +30,14 @@ def batch1_graph(arch, size, **kw):
     return path
 
 
+def facade_shuffle(pre, swap_rgb):
+    """whether the network behind the reference's C facade (the build without OpenCV) sees the first and third channel of the caller's
+    image exchanged: the facade exchanges them when swapRGB == 0 (src/c_api/MsnhnetLib.cpp:562, :771), CVUtil's default needShuffleRGB
+    (include/Msnhnet/utils/MsnhCVUtil.h:23-38) exchanges them again for every form but the letterbox.  tests/test_ref_facade_cpu.py
+    checks this table against the reference's facade itself."""
+    return (not swap_rgb) if pre == "padding_zero" else bool(swap_rgb)
+
+
 def rel_err(a, b):
     """max|a-b|/max|b| over entries finite in the reference; non-finite entries must agree in class and sign."""
     a = np.asarray(a, np.float64).ravel()

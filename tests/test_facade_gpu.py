@@ -116,13 +116,14 @@ def test_facade_classify_success_path(tmp_path):
     kinds = {"f32c3": "f32c3", "googlenet": "googlenet", "transformed": "transformed", "caffe": "caffe"}
     for pre, kind in kinds.items():
         for swap in (0, 1):
-            xin = on.preproc_u8(img, size, size, kind, mean, std, bool(swap))
+            xin = on.preproc_u8(img, size, size, kind, mean, std, nu.facade_shuffle(pre, swap))
             want = int(np.argmax(o.run(xin)[-1]))
             assert L.runClassifyList(ctypes.byref(msg), _u8p(img), 260, 180, 3, ctypes.byref(best), PRE[pre], swap, 1, _fp(mean), _fp(std)) == 1, msg.value
             assert best.value == want, (pre, swap)
-    xin = on.letterbox_u8(img, size, size)
-    assert L.runClassifyList(ctypes.byref(msg), _u8p(img), 260, 180, 3, ctypes.byref(best), PRE["padding_zero"], 0, 1, None, None) == 1
-    assert best.value == int(np.argmax(o.run(xin)[-1]))
+    for swap in (0, 1):
+        xin = on.letterbox_u8(img, size, size, False, nu.facade_shuffle("padding_zero", swap))
+        assert L.runClassifyList(ctypes.byref(msg), _u8p(img), 260, 180, 3, ctypes.byref(best), PRE["padding_zero"], swap, 1, None, None) == 1
+        assert best.value == int(np.argmax(o.run(xin)[-1])), ("padding_zero", swap)
     # the reference's argument errors
     for args, text in (((3, PRE["none"], None, None), b"preDataType can't be none"), ((2, PRE["f32c3"], None, None), b"channel must be 1 or 3"),
                        ((1, PRE["f32c3"], None, None), b"channel 1 must preprocess with F32_C1"), ((3, PRE["c1"], None, None), b"channel 1 can't preprocess with F32_C1"),
@@ -171,7 +172,7 @@ def test_facade_yolo_success_path(tmp_path):
     assert L.initMsnhnet() == 1
     assert L.buildMsnhnet(ctypes.byref(msg), net.encode(), binp.encode(), 0, 0) == 1, msg.value
     for swap in (0, 1):
-        o.run(on.letterbox_u8(img, size, size, False, bool(swap)))
+        o.run(on.letterbox_u8(img, size, size, False, nu.facade_shuffle("padding_zero", swap)))
         ref = o.boxes
         rc = L.runYoloList(ctypes.byref(msg), _u8p(img), 120, 70, 3, ctypes.byref(boxes), ctypes.byref(n), swap, 1)
         if len(ref) > 1024:
@@ -186,3 +187,52 @@ def test_facade_yolo_success_path(tmp_path):
     assert L.runYoloList(ctypes.byref(msg), _u8p(img), 120, 70, 3, ctypes.byref(boxes), ctypes.byref(n), 0, 0) == -1
     assert b"Gpu mode , can not run with cpu" in msg.value
     assert L.dispose() == 1
+
+
+@pytest.mark.gpu
+def test_facade_against_the_reference_facade(tmp_path):
+    """runClassifyList / runYoloList of this library against the reference's own facade (src/c_api/MsnhnetLib.cpp compiled into
+    oracle/_ref, CPU path) on the same 8-bit image, every PredDataType, swapRGB 0 and 1: same class index, same boxes"""
+    import refshim
+    from test_ref_facade_cpu import _image, small_detector
+    if not refshim.available():
+        pytest.skip("reference build not present")
+    L = netapi.lib()
+    msg = ctypes.c_char_p()
+    size = 64
+    net, binp, g = nu.model("resnet18", 1, size, seed=3)
+    ref = refshim.RefFacade(nu.batch1_graph("resnet18", size), binp)
+    img = _image(31, 50, 70)
+    mean, std = np.array([0.4, 0.5, 0.6], np.float32), np.array([0.2, 0.3, 0.25], np.float32)
+    assert L.initMsnhnet() == 1
+    assert L.buildMsnhnet(ctypes.byref(msg), net.encode(), binp.encode(), 0, 0) == 1, msg.value
+    best = ctypes.c_int(-1)
+    seen = set()
+    for pre in ("f32c3", "googlenet", "transformed", "caffe", "padding_zero"):
+        for swap in (0, 1):
+            want = ref.classify_list(img, pre, swap, mean, std)
+            print("facade", pre, swap, flush=True)
+            assert L.runClassifyList(ctypes.byref(msg), _u8p(img), 70, 50, 3, ctypes.byref(best), PRE[pre], swap, 1, _fp(mean), _fp(std)) == 1, msg.value
+            assert best.value == want, (pre, swap)
+            seen.add((pre, want))
+    assert len(seen) > 5                 # swapRGB changes the prediction for this image: the polarity is really tested
+    assert L.dispose() == 1
+    ref.close()
+
+    net, binp, size = small_detector(tmp_path)
+    ref = refshim.RefFacade(net, binp)
+    img = _image(33, 3 * size, 4 * size)
+    assert L.initMsnhnet() == 1
+    assert L.buildMsnhnet(ctypes.byref(msg), net.encode(), binp.encode(), 0, 0) == 1, msg.value
+    boxes = netapi.BBoxContainer()
+    n = ctypes.c_int(-1)
+    res = []
+    for swap in (0, 1):
+        want = ref.yolo_list(img, swap)
+        assert L.runYoloList(ctypes.byref(msg), _u8p(img), 4 * size, 3 * size, 3, ctypes.byref(boxes), ctypes.byref(n), swap, 1) == 1, msg.value
+        got = np.array([[b.x, b.y, b.w, b.h, b.conf, b.bestClsConf, b.bestClsIdx] for b in boxes.boxes[:n.value]], np.float32).reshape(-1, 7)
+        assert len(want) > 0 and nu.boxes_err(got, want) <= 1e-4, swap
+        res.append(want)
+    assert not np.array_equal(res[0], res[1])
+    assert L.dispose() == 1
+    ref.close()

@@ -262,3 +262,31 @@ def test_task_pool(tmp_path):
     assert r.returncode == 0, r.stdout
     r = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
     assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout
+
+
+def test_host_threads_under_sanitizers(tmp_path):
+    """the multi-threaded host code -- the worker pool (tests/cpp/taskpool_check.cpp) and the box stage's parallel per-(image, class)
+    suppression over it (tests/cpp/nms_pool_check.cpp, which also checks it against the reference-shaped loop) -- built from the host
+    library's sources with -fsanitize=thread and with -fsanitize=address,undefined and run: no report, exit status 0"""
+    import glob
+    import subprocess
+    host = os.path.join(ROOT, "msnhnet_amd", "host")
+    lib = os.path.join(ROOT, "msnhnet_amd", "lib")
+    inc = ["-I" + os.path.join(host, "include"), "-I" + os.path.join(ROOT, "include")]
+    srcs = sorted(glob.glob(os.path.join(host, "src", "*.cpp")))
+    builds = []
+    for tag, san in (("tsan", "-fsanitize=thread"), ("asan", "-fsanitize=address,undefined")):
+        common = ["g++", "-std=c++17", "-O1", "-g", san, "-fno-sanitize-recover=undefined", "-fopenmp-simd"] + inc
+        tp = str(tmp_path / f"taskpool_{tag}")
+        nm = str(tmp_path / f"nms_pool_{tag}")
+        builds.append((tp, subprocess.Popen(common + [os.path.join(ROOT, "tests", "cpp", "taskpool_check.cpp"), os.path.join(host, "src", "TaskPool.cpp"), "-o", tp, "-lpthread"],
+                                            stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        builds.append((nm, subprocess.Popen(common + [os.path.join(ROOT, "tests", "cpp", "nms_pool_check.cpp")] + srcs + ["-o", nm, "-L" + lib, "-lmsnh_hip", "-Wl,-rpath," + lib, "-lpthread"],
+                                            stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+    for exe, p in builds:
+        out, _ = p.communicate(timeout=600)
+        assert p.returncode == 0, out[-3000:]
+    env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1 exitcode=66", ASAN_OPTIONS="detect_leaks=1 exitcode=67", UBSAN_OPTIONS="print_stacktrace=1")
+    for exe, _ in builds:
+        r = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300, env=env)
+        assert r.returncode == 0 and r.stdout.strip().endswith("ok") and "Sanitizer" not in r.stdout, (exe, r.stdout[-3000:])

@@ -631,6 +631,38 @@ def test_net_group_refuses_bad_arguments(tmp_path):
         grp.close()
 
 
+@pytest.mark.parametrize("instances,fail_at", [(1, 2), (2, 4), (2, 5)])
+def test_net_group_enqueue_error_keeps_the_order(instances, fail_at, monkeypatch):
+    """a batch whose enqueue fails while an earlier batch of the same instance is still in flight (depth 2): the earlier batch's
+    result is handed out first, the failed submission's own fetch raises, and every later fetch returns what belongs to it"""
+    size, batch = 96, 2
+    net, binp, g = nu.model("yolov3", batch, size, seed=11)
+    xs = [zoo.seeded_input(batch, 3, size, size, seed=40 + i) for i in range(8)]
+    xd = [torch.from_numpy(x).cuda() for x in xs]
+    torch.cuda.synchronize()
+    one = netapi.Net(net, binp, fp16=True)
+    want = [one.run_yolo(x) for x in xs]
+    grp = netapi.NetGroup(net, binp, instances=instances, depth=2, fp16=True)
+    try:
+        grp.prime(xd[0].data_ptr())
+        monkeypatch.setenv("MSNH_GROUP_FAIL_ENQUEUE", str(fail_at))
+        for t in xd:
+            grp.submit(t.data_ptr())
+        monkeypatch.delenv("MSNH_GROUP_FAIL_ENQUEUE")
+        grp.flush()
+        for i in range(len(xd)):
+            if i == fail_at:
+                with pytest.raises(RuntimeError, match="MSNH_GROUP_FAIL_ENQUEUE"):
+                    grp.fetch()
+                continue
+            got = grp.fetch()
+            for a, b in zip(got, want[i]):
+                assert np.array_equal(a, b, equal_nan=True), i
+        assert grp.outstanding() == 0
+    finally:
+        grp.close()
+
+
 @pytest.mark.parametrize("mode", [0, 1, 2])
 def test_copy_on_forward_stream_same_results(mode):
     """copy-back (and device NMS) on the forward's own stream, as the instances of a group run, returns what the copy stream beside

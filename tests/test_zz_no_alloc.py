@@ -75,3 +75,49 @@ def test_yolo_nms_static_equals_workspace_variant():
     rd = torch.zeros(16, dtype=torch.float32).cuda()
     assert L.msnh_hip_yolo_nms_static(64, 80, gu.ptr(rd), 22743, gu.ptr(kc), thr, gu.ptr(rd), 64 * 22743, gu.ptr(kc), None) != 0
     assert b"built-in one holds" in L.msnh_hip_last_error()
+
+
+def test_yolo_nms_static_calls_on_two_streams_are_put_in_order():
+    """two calls issued back to back on two different streams, and two calls from two host threads, all on the one built-in workspace:
+    the library makes each wait for the one before it on the device, so every result equals the caller-workspace variant's"""
+    import ctypes
+    import threading
+    import gpuutil as gu
+    gu.init()
+    L = abi.lib()
+    rng = np.random.default_rng(78)
+    classes, thr = 6, 0.45
+    cases = []
+    for batch, cells, crowded in ((4, 6912, {0: 2500, 2: 1800}), (3, 4000, {1: 1300}), (4, 6912, {3: 3000}), (2, 3000, {0: 1100})):
+        rows, cnt = _rows(rng, batch, cells, classes, crowded)
+        (kept_a, kc_a), _ = _both(batch, classes, cells, rows, cnt, thr)
+        cases.append((batch, cells, gu.dev(rows), gu.dev(cnt), _records(kept_a, kc_a), kc_a))
+    streams = []
+    for _ in range(2):
+        s = ctypes.c_void_p()
+        abi.check(L.msnh_hip_stream_create(ctypes.byref(s)))
+        streams.append(s)
+    outs = [(torch.zeros((b * c, 12), dtype=torch.float32).cuda(), torch.zeros(1 + b, dtype=torch.int32).cuda()) for b, c, *_ in cases]
+    gu.sync()
+
+    def call(i, stream):
+        b, c, rd, cd, _, _ = cases[i]
+        kept, kc = outs[i]
+        abi.check(L.msnh_hip_yolo_nms_static(b, classes, gu.ptr(rd), c, gu.ptr(cd), thr, gu.ptr(kept), b * c, gu.ptr(kc), stream))
+
+    print("yolo_nms_static on two streams", flush=True)
+    call(0, streams[0])
+    call(1, streams[1])                 # enqueued while the first may still run: waits for it on the device
+    threads = [threading.Thread(target=call, args=(2, streams[0])), threading.Thread(target=call, args=(3, streams[1]))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for s in streams:
+        abi.check(L.msnh_hip_stream_sync(s))
+    for i, (b, c, rd, cd, want, want_kc) in enumerate(cases):
+        kept, kc = outs[i][0].cpu().numpy(), outs[i][1].cpu().numpy()
+        assert np.array_equal(kc, want_kc), (i, kc, want_kc)
+        assert np.array_equal(_records(kept, kc), want), i
+    for s in streams:
+        abi.check(L.msnh_hip_stream_destroy(s))
