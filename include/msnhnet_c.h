@@ -133,6 +133,15 @@ int msnhnet_last_nms_on_device(msnhnet_t net, int *on_device);
 int msnhnet_fp16_headroom(msnhnet_t net, const float *img, long long n, float *headroom);
 /* Output of top-level layer `layer` from the last run with layer dumps on (batch-major NCHW). Returns its length. */
 long long msnhnet_layer_output(msnhnet_t net, int layer, float *dst, long long cap);
+/* Detectors, for parity checks of the production path (no layer dumps needed).  After a fetched result:
+ * msnhnet_yolo_head_logits: the input tensor of detection head `head` (heads in the order of the yoloout layer's `layers:` list) as
+ *   batch-major NCHW float32, what YoloLayer::forward reads (src/layers/MsnhYoloLayer.cpp:61-142); returns its length.
+ * msnhnet_yolo_candidates: the candidate rows of image `image` before sorting and suppression -- what the reference's scan keeps at
+ *   src/layers/MsnhYoloOutLayer.cpp:120-170 -- 8 floats each (x y w h objectness, best class score, best class, cell number in the
+ *   reference's scan order: head by head, anchor, then pixel), in no particular order; returns their number.  Available when the
+ *   sort + NMS of that result ran on the host (msnhnet_set_device_nms(0)). */
+long long msnhnet_yolo_head_logits(msnhnet_t net, int head, float *dst, long long cap);
+long long msnhnet_yolo_candidates(msnhnet_t net, int image, float *dst, long long cap_rows);
 /* Device-resident serving path: write the batch into the buffer returned by msnhnet_device_input (device memory,
  * NCHW float32) or pass another device pointer, enqueue, then sync / fetch. */
 int msnhnet_device_input(msnhnet_t net, float **device_ptr);
@@ -156,6 +165,10 @@ float msnhnet_gpu_inference_time(msnhnet_t net);          /* NetBuilder::getGpuI
  * bestClsIdx), already in the order the layer would pass them; fast = 0 runs the reference-shaped greedy loop,
  * fast = 1 the sorted variant the library uses.  Writes at most cap rows, *n_out = number of surviving boxes. */
 int msnhnet_nms(const float *rows, long long n, float nms_thresh, int fast, float *out, long long cap, long long *n_out);
+/* The whole host stage of YoloOutLayer on candidate rows as msnhnet_yolo_candidates returns them (8 floats each, any order): back into
+ * scan order by cell number, sorted by objectness * class score (src/layers/MsnhYoloOutLayer.cpp:175-194), then msnhnet_nms.  Pure
+ * host code. */
+int msnhnet_boxes_from_candidates(const float *rows8, long long n, float nms_thresh, int fast, float *out, long long cap, long long *n_out);
 
 /* The step either side of the graph.
  * msnhnet_set_input_image_u8: letterbox one 8-bit RGB image (HWC, host memory) on the device into slot `index` of the

@@ -6,8 +6,9 @@
 //
 // File: one text line (format version, packing layout version of the kernel library, number of tile configurations, Winograd preference,
 // dtype), then binary little-endian: hash of the weights file, hash of the plan's structure, tensor count, the calibrated absolute maximum
-// of every tensor, then one record per packed blob { op index, algorithm, byte count, bytes padded to 8 } and a closing record that holds
-// the number of blobs.  A file whose line or hashes differ, that is cut short, or that lacks a blob the plan asks for is ignored and rewritten.
+// of every tensor, then one record per packed blob { op index, algorithm, byte count, hash of the bytes, bytes padded to 8 } and a closing record that holds
+// the number of blobs.  A file whose line or hashes differ, that is cut short, that holds a blob whose bytes no longer hash to the recorded
+// value, or that lacks a blob the plan asks for is ignored and rewritten.
 #pragma once
 #include <cstdint>
 #include <cstdio>
@@ -32,7 +33,7 @@ public:
     bool stale() const { return _stale; }
     size_t blobsServed() const { return _served; }
 
-    // writing: into "<path>.tmp", renamed over `path` by commit()
+    // writing: into "<path>.tmp.<pid>.<n>", renamed over `path` by commit()
     bool create(const std::string &path, const std::string &header, uint64_t weightsHash, uint64_t graphHash, const std::vector<float> &amax);
     void add(uint32_t op, uint32_t algo, const void *data, size_t bytes);
     bool commit();
@@ -45,7 +46,7 @@ private:
     bool _stale = false;
     size_t _served = 0;
     std::FILE *_out = nullptr;
-    std::string _path;
+    std::string _path, _tmp;
     uint32_t _written = 0;
     bool _failed = false;
 };

@@ -373,6 +373,13 @@ public:
 
     // host post-processing of the compacted candidate rows of one image (8 floats per row, see msnh_hip_yolo_gather)
     std::vector<YoloBox> boxesFromRows(const float *rows, int count, const float *decodedOfImage) const;
+    // the same as a function of the rows alone: candidates back in scan order (by cell number), then sorted by objectness * class score,
+    // descending, ties in scan order (src/layers/MsnhYoloOutLayer.cpp:120-194); decodedOfImage (may be NULL) supplies classesVal
+    static std::vector<YoloBox> sortedCandidates(const float *rows, int count, const float *decodedOfImage, int channel);
+    // the candidate rows of image `image` in the result fetched last, as the device wrote them (8 floats each: x y w h objectness, best
+    // class score, best class, cell number in scan order; any order) -- what the reference's scan keeps before sorting
+    // (src/layers/MsnhYoloOutLayer.cpp:120-170).  Only after a result whose sort + NMS ran on the host.
+    std::vector<float> lastCandidateRows(int image) const;
     static std::vector<std::vector<int>> groupByClass(const std::vector<YoloBox> &bboxes);
     static void nmsClass(const std::vector<YoloBox> &bboxes, std::vector<int> &members, float nmsThresh);
 
@@ -398,6 +405,7 @@ private:
     std::vector<YoloBox> boxesFromKept(std::vector<const float *> &records) const;
     msnh_stream_t _copyStream = nullptr, _fetchStream = nullptr;
     int _lastMaxCandidates = 0;            // largest per-image candidate count of the previous result
+    int _lastSlot = -1;                    // slot of the result fetched last
     size_t _lastKept = 0;                  // records the device NMS kept for the previous batch
     int _hostBoundRuns = 0;                // batches in a row for which the host path did not have to wait for the device
     bool _hostBound = false;               // a device trial gave results faster than the host stage: stay on the device

@@ -76,6 +76,12 @@ public:
     // Range check of the float16 plan for one input (batch*C*H*W floats): the activation scales are fixed at load from one
     // calibration image of values in [0,1) with a 32x margin; this runs the network once, launch by launch, on `img` and returns the
     // factor by which `img` could still grow before a float16 activation overflows (0: it already did; the results are then wrong).
+    // Detectors, after a fetched result: the input of detection head `head` (heads in the order of the yoloout layer's `layers:` list)
+    // as batch-major NCHW float32 -- the tensor the reference's YoloLayer::forward reads (src/layers/MsnhYoloLayer.cpp:61-142) -- and the
+    // candidate rows of one image before sorting and suppression (YoloOutLayer::lastCandidateRows).  For parity checks of the
+    // production path: which cells passed the objectness test, and on which logits.
+    std::vector<float> yoloHeadLogits(int head);
+    std::vector<float> yoloLastCandidates(int image);
     float fp16Headroom(const std::vector<float> &img);
 
     Point2I getInputSize();
@@ -114,7 +120,7 @@ public:
 private:
     void finalizePlan();
     std::string _weightsPath;               // set while loadWeightsFromMsnhBin runs: where the tune cache goes
-    uint64_t _weightsHash = 0;
+    uint64_t _graphTextHash = 0, _weightsHash = 0;
     float _readMs = 0.f;
     std::string _loadDetail;
     std::unique_ptr<Plan> lowerNetwork(int dtype);

@@ -407,6 +407,28 @@ long long msnhnet_layer_output(msnhnet_t net, int layer, float *dst, long long c
     return n;
 }
 
+long long msnhnet_yolo_head_logits(msnhnet_t net, int head, float *dst, long long cap)
+{
+    long long n = -1;
+    guarded([&] {
+        const std::vector<float> v = nb(net).yoloHeadLogits(head);
+        n = static_cast<long long>(v.size());
+        if (dst && cap > 0) std::memcpy(dst, v.data(), sizeof(float) * static_cast<size_t>(std::min(cap, n)));
+    });
+    return n;
+}
+
+long long msnhnet_yolo_candidates(msnhnet_t net, int image, float *dst, long long cap_rows)
+{
+    long long n = -1;
+    guarded([&] {
+        const std::vector<float> v = nb(net).yoloLastCandidates(image);
+        n = static_cast<long long>(v.size() / 8);
+        if (dst && cap_rows > 0) std::memcpy(dst, v.data(), sizeof(float) * 8 * static_cast<size_t>(std::min(cap_rows, n)));
+    });
+    return n;
+}
+
 int msnhnet_device_input(msnhnet_t net, float **device_ptr)
 {
     return guarded([&] { if (!device_ptr) MSNH_THROW("pointer is NULL"); *device_ptr = nb(net).deviceInputBuffer(); });
@@ -499,6 +521,17 @@ int msnhnet_boxes_to_image(float *boxes, long long count, int net_w, int net_h, 
             else        YoloOutLayer::bboxResize2OrgNoPad(b, Point2I(net_w, net_h), Point2I(org_w, org_h));
             r[0] = b.xywhBox.x; r[1] = b.xywhBox.y; r[2] = b.xywhBox.w; r[3] = b.xywhBox.h;
         }
+    });
+}
+
+int msnhnet_boxes_from_candidates(const float *rows8, long long n, float nms_thresh, int fast, float *out, long long cap, long long *n_out)
+{
+    return guarded([&] {
+        if ((!rows8 && n > 0) || n < 0 || n > (1LL << 30)) MSNH_THROW("bad argument");
+        const std::vector<YoloBox> in = YoloOutLayer::sortedCandidates(rows8, static_cast<int>(n), nullptr, 0);
+        std::vector<std::vector<YoloBox>> res(1);
+        res[0] = fast ? YoloOutLayer::nmsSorted(in, nms_thresh) : YoloOutLayer::nms(in, nms_thresh, false);
+        packBoxes(res, nullptr, out, cap, n_out);
     });
 }
 

@@ -1220,6 +1220,11 @@ int YoloOutLayer::lower(Plan &plan, int, int layerIndex)
 
 std::vector<YoloBox> YoloOutLayer::boxesFromRows(const float *rows, int count, const float *decodedOfImage) const
 {
+    return sortedCandidates(rows, count, decodedOfImage, _channel);
+}
+
+std::vector<YoloBox> YoloOutLayer::sortedCandidates(const float *rows, int count, const float *decodedOfImage, int channel)
+{
     // Candidates arrive in arbitrary order; the reference scans cells in ascending order
     // (src/layers/MsnhYoloOutLayer.cpp:120-170), so restore that first.
     std::vector<int> order(static_cast<size_t>(count));
@@ -1237,8 +1242,8 @@ std::vector<YoloBox> YoloOutLayer::boxesFromRows(const float *rows, int count, c
         b.bestClsIdx = static_cast<int>(r[6]);
         if (decodedOfImage)
         {
-            const float *row = decodedOfImage + static_cast<size_t>(r[7]) * _channel;
-            b.classesVal.assign(row + 5, row + _channel);
+            const float *row = decodedOfImage + static_cast<size_t>(r[7]) * channel;
+            b.classesVal.assign(row + 5, row + channel);
         }
         keys[static_cast<size_t>(i)] = b.conf * b.bestClsConf;
     }
@@ -1592,6 +1597,7 @@ void YoloOutLayer::finish(int slot)
     MSNH_DEV(msnh_hip_event_sync(sl.event));
     const float dbgWait = TimeUtil::getElapsedTime(dbg0);
     sl.pending = false;
+    _lastSlot = slot & 1;
     lastOnDevice = sl.onDevice;
     noteResult(sl, _slots[(slot ^ 1) & 1].pending);
     const int cells = plan->yoloCells;
@@ -1709,6 +1715,18 @@ void YoloOutLayer::finish(int slot)
     if (std::getenv("MSNH_DEBUG_TIMING"))
         std::fprintf(stderr, "yoloout finish: wait %.3f ms, host %.3f ms (candidates %.3f, suppression %.3f, output %.3f)\n", dbgWait,
                      TimeUtil::getElapsedTime(dbg0) - dbgWait, dbgA - dbgWait, dbgB - dbgA, TimeUtil::getElapsedTime(dbg0) - dbgB);
+}
+
+std::vector<float> YoloOutLayer::lastCandidateRows(int image) const
+{
+    if (_lastSlot < 0) MSNH_THROW("YoloOut: no result was fetched yet");
+    if (image < 0 || image >= _batch) MSNH_THROW("YoloOut: no such image in the batch");
+    const Slot &sl = _slots[_lastSlot];
+    if (sl.onDevice) MSNH_THROW("YoloOut: the last result was suppressed on the device, its candidate rows did not come to the host (device NMS mode 0 keeps them)");
+    const size_t cells = static_cast<size_t>(plan->yoloCells);
+    const size_t n = static_cast<size_t>(std::min(sl.cnt.as<int>()[image], plan->yoloCells));
+    const float *rows = sl.rows.as<float>() + static_cast<size_t>(image) * cells * 8;
+    return std::vector<float>(rows, rows + n * 8);
 }
 
 void YoloOutLayer::forwardGPU(NetworkState &netState)

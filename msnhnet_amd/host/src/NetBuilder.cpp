@@ -80,6 +80,13 @@ void NetBuilder::clearLayers()
 void NetBuilder::buildNetFromMsnhNet(const std::string &path)
 {
     _parser->readCfg(path);
+    {
+        // every parameter of the graph (activation slopes, batch-norm eps, anchors, thresholds, ...) takes part in what a packed-constants
+        // file must match: the file keeps a float16 calibration that depends on them
+        std::ifstream f(path, std::ios::binary);
+        const std::string text((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+        _graphTextHash = PackFile::hash(text.data(), text.size());
+    }
     clearLayers();
     if (BaseLayer::onlyUseGpu && BaseLayer::onlyUseCpu) MSNH_THROW("Gpu only mode and cpu only mode can not use at the same time!");
 
@@ -408,7 +415,7 @@ void NetBuilder::finalizePlan()
     const bool winograd = useWinograd && dtype == MSNH_F16;
     const std::string packPath = (weightCache && !_weightsPath.empty()) ? _weightsPath + (dtype == MSNH_F16 ? ".f16.pack" : ".f32.pack") : std::string();
     const std::string packLine = PackFile::headerLine(dtype, winograd);
-    const uint64_t graphHash = packPath.empty() ? 0 : plan->structureHash();
+    const uint64_t graphHash = packPath.empty() ? 0 : plan->structureHash() ^ (_graphTextHash * 0x9E3779B97F4A7C15ull);
     PackFile kept, fresh;
     t0 = Clock::now();
     const bool haveKept = !packPath.empty() && kept.open(packPath, packLine, _weightsHash, graphHash, plan->tensors.size());
@@ -672,6 +679,33 @@ std::vector<std::vector<YoloBox>> NetBuilder::fetchYolo()
     yout->finish(slot);
     --_inFlight;
     return yout->finalOut;
+}
+
+std::vector<float> NetBuilder::yoloHeadLogits(int head)
+{
+    if (!_planReady) MSNH_THROW("weights are not loaded");
+    if (_inFlight > 0) MSNH_THROW("fetch the outstanding results first");
+    Plan &plan = *_net->plan;
+    std::vector<size_t> heads = plan.yoloHeadOps;
+    if (heads.empty())
+    {
+        // heads decoded one by one: their inputs are only kept to the end of the forward while layer dumps pin them
+        if (!_saveLayerOutput) MSNH_THROW("the head tensors of this plan do not outlive the forward (run with layer dumps on)");
+        for (size_t i = 0; i < plan.ops.size(); ++i)
+            if (plan.ops[i].kind == PlanOp::YOLO_DECODE && !plan.ops[i].dead) heads.push_back(i);
+        std::sort(heads.begin(), heads.end(), [&plan](size_t a, size_t b) { return plan.ops[a].cellBase < plan.ops[b].cellBase; });
+    }
+    if (head < 0 || static_cast<size_t>(head) >= heads.size()) MSNH_THROW("no such detection head");
+    std::vector<float> out;
+    plan.exportTensor(plan.ops[heads[static_cast<size_t>(head)]].in0, out, _stream);
+    return out;
+}
+
+std::vector<float> NetBuilder::yoloLastCandidates(int image)
+{
+    BaseLayer *last = _net->layers.empty() ? nullptr : _net->layers.back();
+    if (last == nullptr || last->type() != LayerType::YOLO_OUT) MSNH_THROW("not a yolo net");
+    return static_cast<YoloOutLayer *>(last)->lastCandidateRows(image);
 }
 
 std::vector<float> NetBuilder::runClassifyGPU(std::vector<float> img) { return runClassifyGPU(img.data(), img.size()); }

@@ -1,15 +1,23 @@
 // Reader and writer of the packed-constants file of a plan (layout in MsnhPackFile.h).
 #include "Msnhnet/core/MsnhPackFile.h"
+#include <atomic>
 #include <cstring>
+#include <unistd.h>
 #include "msnh_hip.h"
 
 namespace Msnhnet
 {
 namespace
 {
-constexpr int kFormat = 1;
+constexpr int kFormat = 2;
 constexpr uint32_t kClosing = 0xFFFFFFFFu;
-struct Record { uint32_t op, algo; uint64_t bytes; };
+struct Record { uint32_t op, algo; uint64_t bytes, hash; };          // hash: PackFile::hash of the blob (the closing record: 0)
+// two processes (or two NetBuilders of one process) that write the file of the same weights at the same time each use a name of their own
+std::string tempName(const std::string &path)
+{
+    static std::atomic<unsigned> counter{0};
+    return path + ".tmp." + std::to_string(static_cast<long long>(getpid())) + "." + std::to_string(counter++);
+}
 }
 
 PackFile::~PackFile()
@@ -17,7 +25,7 @@ PackFile::~PackFile()
     if (_out)
     {
         std::fclose(_out);
-        std::remove((_path + ".tmp").c_str());
+        std::remove(_tmp.c_str());
     }
 }
 
@@ -92,11 +100,13 @@ bool PackFile::open(const std::string &path, const std::string &header, uint64_t
             if (r.op == kClosing)
             {
                 closed = true;
-                ok = r.algo == _entries.size() && r.bytes == 0 && at == rest;
+                ok = r.algo == _entries.size() && r.bytes == 0 && r.hash == 0 && at == rest;
                 break;
             }
             const size_t padded = (static_cast<size_t>(r.bytes) + 7) & ~static_cast<size_t>(7);
             ok = r.bytes <= rest && at + padded <= rest;
+            // a blob that does not hash to what was recorded (a flipped bit on disk) must not reach the device as weights
+            ok = ok && hash(_file.get() + at, static_cast<size_t>(r.bytes)) == r.hash;
             if (ok) _entries.push_back({r.op, r.algo, at, static_cast<size_t>(r.bytes)});
             at += padded;
         }
@@ -128,7 +138,8 @@ const unsigned char *PackFile::blob(uint32_t op, uint32_t algo, size_t bytes)
 bool PackFile::create(const std::string &path, const std::string &header, uint64_t weightsHash, uint64_t graphHash, const std::vector<float> &amax)
 {
     _path = path;
-    _out = std::fopen((path + ".tmp").c_str(), "wb");
+    _tmp = tempName(path);
+    _out = std::fopen(_tmp.c_str(), "wb");
     if (!_out) return false;
     const uint64_t three[3] = {weightsHash, graphHash, amax.size()};
     _failed = std::fwrite(header.data(), 1, header.size(), _out) != header.size() || std::fputc('\n', _out) == EOF ||
@@ -139,7 +150,7 @@ bool PackFile::create(const std::string &path, const std::string &header, uint64
 void PackFile::add(uint32_t op, uint32_t algo, const void *data, size_t bytes)
 {
     if (!_out || _failed) return;
-    const Record r = {op, algo, bytes};
+    const Record r = {op, algo, bytes, hash(data, bytes)};
     const unsigned char zeros[8] = {0};
     const size_t pad = ((bytes + 7) & ~static_cast<size_t>(7)) - bytes;
     _failed = std::fwrite(&r, sizeof(r), 1, _out) != 1 || std::fwrite(data, 1, bytes, _out) != bytes || std::fwrite(zeros, 1, pad, _out) != pad;
@@ -149,14 +160,13 @@ void PackFile::add(uint32_t op, uint32_t algo, const void *data, size_t bytes)
 bool PackFile::commit()
 {
     if (!_out) return false;
-    const Record r = {kClosing, _written, 0};
+    const Record r = {kClosing, _written, 0, 0};
     _failed = _failed || std::fwrite(&r, sizeof(r), 1, _out) != 1;
     _failed = std::fclose(_out) != 0 || _failed;
     _out = nullptr;
-    const std::string tmp = _path + ".tmp";
-    if (_failed || std::rename(tmp.c_str(), _path.c_str()) != 0)
+    if (_failed || std::rename(_tmp.c_str(), _path.c_str()) != 0)
     {
-        std::remove(tmp.c_str());
+        std::remove(_tmp.c_str());
         return false;
     }
     return true;

@@ -16,9 +16,9 @@ SYMBOLS = [
     "getGpuForwardTime", "getInputDim", "msnhnet_last_error", "msnhnet_create", "msnhnet_destroy", "msnhnet_set_use_fp16", "msnhnet_set_use_winograd", "msnhnet_set_tune_cache", "msnhnet_set_weight_cache", "msnhnet_load_detail", "msnhnet_set_device_nms", "msnhnet_set_input_image_u8", "msnhnet_set_input_image", "msnhnet_boxes_to_image",
     "msnhnet_set_keep_class_scores", "msnhnet_set_save_layer_output", "msnhnet_build", "msnhnet_load", "msnhnet_load_from_memory",
     "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops", "msnhnet_weight_layout", "msnhnet_fp16_headroom", "msnhnet_last_nms_on_device", "msnhnet_set_copy_on_forward_stream",
-    "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_device_input",
+    "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_yolo_head_logits", "msnhnet_yolo_candidates", "msnhnet_device_input",
     "msnhnet_enqueue", "msnhnet_sync", "msnhnet_fetch_classify", "msnhnet_fetch_yolo", "msnhnet_gpu_inference_time", "msnhnet_time_detail",
-    "msnhnet_profile_ops", "msnhnet_profile_ops_bytes", "msnhnet_profile_each_op", "msnhnet_yolo_max_boxes", "msnhnet_nms",
+    "msnhnet_profile_ops", "msnhnet_profile_ops_bytes", "msnhnet_profile_each_op", "msnhnet_yolo_max_boxes", "msnhnet_nms", "msnhnet_boxes_from_candidates",
     "msnhnet_group_create", "msnhnet_group_destroy", "msnhnet_group_info", "msnhnet_group_instance", "msnhnet_group_prime", "msnhnet_group_submit",
     "msnhnet_group_flush", "msnhnet_group_fetch_classify", "msnhnet_group_fetch_yolo",
 ]
@@ -93,6 +93,10 @@ def lib():
     L.msnhnet_weight_layout.argtypes = [vp, llp, ll]
     L.msnhnet_weight_layout.restype = ll
     L.msnhnet_fp16_headroom.argtypes = [vp, fp, ll, fp]
+    L.msnhnet_yolo_head_logits.argtypes = [vp, ci, fp, ll]
+    L.msnhnet_yolo_head_logits.restype = ll
+    L.msnhnet_yolo_candidates.argtypes = [vp, ci, fp, ll]
+    L.msnhnet_yolo_candidates.restype = ll
     L.msnhnet_last_nms_on_device.argtypes = [vp, ip]
     L.msnhnet_conv_flops.restype = ctypes.c_double
     L.msnhnet_run_classify.argtypes = [vp, fp, ll, fp, ll, llp]
@@ -120,6 +124,7 @@ def lib():
     L.msnhnet_profile_each_op.argtypes = [vp, ci, cp, ll]
     L.msnhnet_profile_each_op.restype = ll
     L.msnhnet_nms.argtypes = [fp, ll, ctypes.c_float, ci, fp, ll, llp]
+    L.msnhnet_boxes_from_candidates.argtypes = [fp, ll, ctypes.c_float, ci, fp, ll, llp]
     L.msnhnet_yolo_max_boxes.argtypes = [vp]
     L.msnhnet_yolo_max_boxes.restype = ll
     L.msnhnet_gpu_inference_time.argtypes = [vp]
@@ -171,6 +176,16 @@ def nms(rows, thresh, fast=True):
     out = np.zeros_like(rows)
     n = ctypes.c_longlong()
     _check(lib().msnhnet_nms(_fp(rows), len(rows), thresh, 1 if fast else 0, _fp(out), len(rows), ctypes.byref(n)))
+    return out[:n.value]
+
+
+def boxes_from_candidates(rows8, thresh, fast=True):
+    """the host stage of YoloOutLayer on candidate rows [n, 8] (x y w h objectness, class score, class, cell; any order): scan order,
+    sort by objectness * class score, per-class NMS; returns rows of 7 floats.  Host only."""
+    rows8 = np.ascontiguousarray(rows8, np.float32).reshape(-1, 8)
+    out = np.zeros((len(rows8), 7), np.float32)
+    n = ctypes.c_longlong()
+    _check(lib().msnhnet_boxes_from_candidates(_fp(rows8), len(rows8), thresh, 1 if fast else 0, _fp(out), len(rows8), ctypes.byref(n)))
     return out[:n.value]
 
 
@@ -329,6 +344,25 @@ class Net:
         a = np.empty(n, np.float32)
         if n:
             self.L.msnhnet_layer_output(self.h, i, _fp(a), n)
+        return a
+
+    def yolo_head_logits(self, head):
+        """input of detection head `head` after the last fetched result, batch-major NCHW float32 (flat)"""
+        n = self.L.msnhnet_yolo_head_logits(self.h, head, None, 0)
+        if n < 0:
+            _check(1)
+        a = np.empty(n, np.float32)
+        self.L.msnhnet_yolo_head_logits(self.h, head, _fp(a), n)
+        return a
+
+    def yolo_candidates(self, image):
+        """candidate rows [n, 8] of one image of the last fetched result (x y w h objectness, class score, class, cell number)"""
+        n = self.L.msnhnet_yolo_candidates(self.h, image, None, 0)
+        if n < 0:
+            _check(1)
+        a = np.empty((n, 8), np.float32)
+        if n:
+            self.L.msnhnet_yolo_candidates(self.h, image, _fp(a), n)
         return a
 
     def device_input_ptr(self):

@@ -1,5 +1,6 @@
 // Round trip and rejection cases of the pack file (host code only; no device call).  Prints "ok" or the first failed check.
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <fstream>
 #include <string>
@@ -27,7 +28,7 @@ int main(int argc, char **argv)
     if (argc < 2) return 2;
     const std::string path = std::string(argv[1]) + "/w.msnhbin.f16.pack";
     const std::string line = PackFile::headerLine(1, false);
-    CHECK(line.rfind("msnhpack 1 layout ", 0) == 0 && line != PackFile::headerLine(1, true) && line != PackFile::headerLine(0, false));
+    CHECK(line.rfind("msnhpack 2 layout ", 0) == 0 && line != PackFile::headerLine(1, true) && line != PackFile::headerLine(0, false));
 
     // the hash sees every byte, the length and the order
     std::vector<unsigned char> data(1000003);
@@ -85,6 +86,15 @@ int main(int argc, char **argv)
         PackFile r;
         CHECK(!r.open(path, line, 11, 22, amax.size()));
     }
+    // one flipped bit inside a blob: the blob's checksum refuses the whole file
+    for (size_t at : {whole.size() - 16 - 24 - 40, whole.size() / 2})
+    {
+        std::vector<unsigned char> flipped = whole;
+        flipped[at] ^= 0x10;
+        spill(path, flipped, flipped.size());
+        PackFile r;
+        CHECK(!r.open(path, line, 11, 22, amax.size()));
+    }
     // an abandoned writer leaves neither the file nor its temporary
     std::remove(path.c_str());
     {
@@ -92,7 +102,17 @@ int main(int argc, char **argv)
         CHECK(w.create(path, line, 1, 2, amax));
         w.add(0, 2, data.data(), 100);
     }
-    CHECK(!std::ifstream(path).good() && !std::ifstream(path + ".tmp").good());
+    CHECK(!std::ifstream(path).good());
+    {
+        // (temporaries are named "<path>.tmp.<pid>.<n>": none may be left in the directory)
+        const std::string dir = path.substr(0, path.find_last_of('/'));
+        const std::string cmd = "ls " + dir + " | grep -c '\\.tmp\\.' > " + dir + "/count.txt";
+        (void)std::system(cmd.c_str());
+        std::ifstream c(dir + "/count.txt");
+        int n = -1;
+        c >> n;
+        CHECK(n == 0);
+    }
     std::printf("ok\n");
     return 0;
 }

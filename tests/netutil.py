@@ -30,6 +30,13 @@ def batch1_graph(arch, size, **kw):
     return path
 
 
+def thresholds(arch):
+    """(confThresh, nmsThresh) the generated graph of a detector carries"""
+    import inspect
+    sig = inspect.signature(zoo.ARCHS[arch]).parameters
+    return float(sig["conf"].default), float(sig["nms"].default)
+
+
 def facade_shuffle(pre, swap_rgb):
     """whether the network behind the reference's C facade (the build without OpenCV) sees the first and third channel of the caller's
     image exchanged: the facade exchanges them when swapRGB == 0 (src/c_api/MsnhnetLib.cpp:562, :771), CVUtil's default needShuffleRGB
@@ -172,3 +179,151 @@ def stats_err(got, want):
     if ok.any():
         e = max(e, float(np.abs(got[6:][ok] - want[6:][ok]).max()) / rng)
     return float(e)
+
+
+# ---- detection candidates cell by cell ----------------------------------------------------------------------------------------------
+def yolo_scan(decoded_heads, per, conf_thresh):
+    """the reference's candidate scan (src/layers/MsnhYoloOutLayer.cpp:120-170) over decoded head tensors, each flat [3*per, H*W]:
+    rows [n, 8] = x y w h objectness, best class score, first-maximum class, cell number, in scan order (cells ascending: head by
+    head, anchor, pixel); the test is objectness > conf_thresh on the decoded value"""
+    rows, base = [], 0
+    for d in decoded_heads:
+        hw = d.size // (3 * per)
+        v = np.asarray(d, np.float32).reshape(3, per, hw).transpose(0, 2, 1).reshape(3 * hw, per)
+        c = np.nonzero(v[:, 4] > conf_thresh)[0]
+        r = np.zeros((len(c), 8), np.float32)
+        r[:, :5] = v[c, :5]
+        if len(c):
+            r[:, 5] = v[c, 5:].max(1)
+            r[:, 6] = v[c, 5:].argmax(1)
+        r[:, 7] = c + base
+        rows.append(r)
+        base += 3 * hw
+    return np.concatenate(rows) if rows else np.zeros((0, 8), np.float32)
+
+
+def head_logits_by_cell(logit_heads, per):
+    """head logit tensors (each flat [3*per, H*W], NCHW) -> [cells, per] in the scan's cell order, and the head of every cell"""
+    out, head = [], []
+    for k, t in enumerate(logit_heads):
+        hw = t.size // (3 * per)
+        out.append(np.asarray(t, np.float64).reshape(3, per, hw).transpose(0, 2, 1).reshape(3 * hw, per))
+        head.append(np.full(3 * hw, k, np.int64))
+    return np.concatenate(out), np.concatenate(head)
+
+
+def same_box_set(a, b):
+    """two sets of 7-float boxes are the same multiset, bit for bit (NaN equal to NaN)"""
+    a, b = sort_boxes(a), sort_boxes(b)
+    return a.shape == b.shape and np.array_equal(a, b, equal_nan=True)
+
+
+def attribute_candidates(dev_rows, ref_rows, near, tol=2e-2):
+    """Compares the candidate rows of the device with the reference's, cell by cell.
+
+    dev_rows, ref_rows: [n, 8] rows as yolo_scan returns them (any order).  near(cells, channel) -> bool array: whether the reference's
+    logit of that cell and channel (0 x, 1 y, 2 w, 3 h, 4 objectness, 5+j class j) lies within the float16 logit error of a point where
+    the decoded value jumps (zero for the logistic outputs, the range where exp is finite for w and h).
+
+    Returns (only_dev, only_ref, differing, unexplained): cells that are a candidate on one side only, common cells whose rows differ
+    (a finite column beyond tol * max|reference column|, another inf / NaN pattern, another class), and a list of descriptions of every
+    difference that `near` does not explain -- empty when every difference is attributed to a logit next to a decision point."""
+    dev_rows = np.asarray(dev_rows, np.float32).reshape(-1, 8)
+    ref_rows = np.asarray(ref_rows, np.float32).reshape(-1, 8)
+    dcell, rcell = dev_rows[:, 7].astype(np.int64), ref_rows[:, 7].astype(np.int64)
+    assert len(np.unique(dcell)) == len(dcell) and len(np.unique(rcell)) == len(rcell), "a cell appears twice"
+    only_dev = np.setdiff1d(dcell, rcell)
+    only_ref = np.setdiff1d(rcell, dcell)
+    unexplained = []
+    for cells, side in ((only_dev, "device only"), (only_ref, "reference only")):
+        if len(cells):
+            ok = near(cells, np.full(len(cells), 4))
+            unexplained += [f"cell {c}: candidate on the {side}, objectness logit not near zero" for c in cells[~ok]]
+    common, di, ri = np.intersect1d(dcell, rcell, return_indices=True)
+    d, r = dev_rows[di].astype(np.float64), ref_rows[ri].astype(np.float64)
+    differing = np.zeros(len(common), bool)
+    for col in range(6):
+        chan = np.full(len(common), col) if col < 5 else 5 + r[:, 6].astype(np.int64)
+        fin = np.isfinite(r[:, col])
+        scale = max(np.abs(r[fin, col]).max(), 1e-30) if fin.any() else 1.0
+        with np.errstate(invalid="ignore"):
+            bad = np.where(fin, ~(np.abs(d[:, col] - r[:, col]) <= tol * scale), ~((d[:, col] == r[:, col]) | (np.isnan(d[:, col]) & np.isnan(r[:, col]))))
+        bad &= d[:, 6] == r[:, 6]              # (rows of another class are handled below: their class score belongs to another channel)
+        if bad.any():
+            ok = near(common[bad], chan[bad])
+            unexplained += [f"cell {c} column {col}: {a} vs {b}" for c, a, b in zip(common[bad][~ok], d[bad][~ok, col], r[bad][~ok, col])]
+            differing |= bad
+    cls_bad = d[:, 6] != r[:, 6]
+    for i in np.nonzero(cls_bad)[0]:
+        # first-maximum class: it can only move if a class up to the later of the two has a logit next to zero (scores saturate at 1)
+        hi = int(max(d[i, 6], r[i, 6]))
+        if not near(np.full(hi + 1, common[i]), 5 + np.arange(hi + 1)).any():
+            unexplained.append(f"cell {common[i]}: class {int(d[i, 6])} vs {int(r[i, 6])}")
+    differing |= cls_bad
+    return only_dev, only_ref, common[differing], unexplained
+
+
+def attribute_against_reference(dev_rows, dev_logit_heads, ref_decoded_heads, ref_logit_heads, per, conf_thresh, bar=2e-2):
+    """The float16 candidates of one image against the reference's, every difference attributed.
+
+    dev_rows: candidate rows of the device [n, 8]; dev_logit_heads / ref_logit_heads: per head the logit tensor of this image (flat NCHW);
+    ref_decoded_heads: the reference's decoded head tensors.  Checks that the measured logit error of every head is within
+    bar * max|reference logits| and that every candidate-set or row difference sits on a reference logit no farther from a jump of the
+    decode than that head's measured error (+ 90: the width of the range where exp() is finite and the logistic is not yet exactly 0 or 1).
+    Returns (ref_rows, only_dev, only_ref, differing_cells, head_errors)."""
+    ref_rows = yolo_scan(ref_decoded_heads, per, conf_thresh)
+    ref_l, head = head_logits_by_cell(ref_logit_heads, per)
+    dev_l, _ = head_logits_by_cell(dev_logit_heads, per)
+    assert ref_l.shape == dev_l.shape
+    fin = np.isfinite(ref_l)
+    assert (np.isfinite(dev_l) == fin).all()
+    err = np.zeros(len(ref_logit_heads))
+    for k in range(len(ref_logit_heads)):
+        sel = head == k
+        d = np.abs(np.where(fin[sel], dev_l[sel] - ref_l[sel], 0.0))
+        err[k] = d.max()
+        assert err[k] <= bar * np.abs(ref_l[sel][fin[sel]]).max(), (k, err[k])
+
+    def near(cells, chans):
+        return np.abs(ref_l[cells, chans]) <= err[head[cells]] + 90.0
+
+    only_dev, only_ref, differing, unexplained = attribute_candidates(dev_rows, ref_rows, near, bar)
+    assert not unexplained, unexplained[:10]
+    # a cell that is a candidate on one side only: the two objectness logits lie on opposite sides of the threshold, so the
+    # reference's is no farther from it than the two are apart
+    for cells in (only_dev, only_ref):
+        if len(cells):
+            assert (np.abs(ref_l[cells, 4]) <= np.abs(dev_l[cells, 4] - ref_l[cells, 4]) + 1e-3).all()
+    return ref_rows, only_dev, only_ref, differing, err
+
+
+def _iou_plus1(a, b):
+    """Box::iou with the reference's +1 extents (include/Msnhnet/utils/MsnhTypes.h:123-140) on rows x y w h"""
+    ax1, ax2, ay1, ay2 = a[0] - a[2] / 2, a[0] + a[2] / 2, a[1] - a[3] / 2, a[1] + a[3] / 2
+    bx1, bx2, by1, by2 = b[0] - b[2] / 2, b[0] + b[2] / 2, b[1] - b[3] / 2, b[1] + b[3] / 2
+    iw = max(min(ax2, bx2) - max(ax1, bx1) + 1, 0.0)
+    ih = max(min(ay2, by2) - max(ay1, by1) + 1, 0.0)
+    inter = iw * ih
+    return inter / ((ax2 - ax1 + 1) * (ay2 - ay1 + 1) + (bx2 - bx1 + 1) * (by2 - by1 + 1) - inter)
+
+
+def box_sets_equal_up_to_ties(got, ref, nms_thresh):
+    """Two NMS results over the same candidates are the same multiset of boxes bit for bit, except where the reference's own result is
+    not determined by its input: it orders the candidates with std::sort (include/Msnhnet/utils/MsnhExVector.h:57-74), which leaves the
+    order of candidates with equal objectness * class score unspecified, and among candidates of equal objectness the greedy loop keeps
+    whichever comes first.  A box present on one side only must therefore have a partner on the other side only with the same class,
+    objectness and class score that it overlaps by more than the threshold (either suppresses the other).  Returns the number of such
+    swapped pairs; raises AssertionError otherwise."""
+    got = np.asarray(got, np.float32).reshape(-1, 7)
+    ref = np.asarray(ref, np.float32).reshape(-1, 7)
+    assert len(got) == len(ref), (len(got), len(ref))
+    key = lambda r: tuple(np.nan_to_num(r.astype(np.float64), nan=-7e300).tolist())
+    from collections import Counter
+    cg, cr = Counter(key(r) for r in got), Counter(key(r) for r in ref)
+    only_g, only_r = list((cg - cr).elements()), list((cr - cg).elements())
+    assert len(only_g) == len(only_r)
+    for a in only_g:
+        j = next((j for j, b in enumerate(only_r) if a[4:7] == b[4:7] and _iou_plus1(a, b) > nms_thresh), None)
+        assert j is not None, f"box {a} has no tied, overlapping partner among {only_r[:5]}"
+        only_r.pop(j)
+    return len(only_g)

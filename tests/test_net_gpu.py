@@ -111,18 +111,32 @@ def test_fp16_final_outputs(arch, size, batch):
     print("running fp16", arch, size, batch, flush=True)
     m = netapi.Net(net, binp, fp16=True, dump_layers=True)
     if arch.startswith("yolo"):
-        boxes = m.run_yolo(x)
+        netapi.set_device_nms(0)                # sort + NMS on the host: the candidate rows come to the host with the result
+        try:
+            boxes = m.run_yolo(x)
+            rows = [m.yolo_candidates(b) for b in range(batch)]
+        finally:
+            netapi.set_device_nms(1)
         # final logits = inputs of the yolo layers
-        for i in range(m.num_layers()):
-            if m.layer_info(i)["type"] != "yolo":
-                continue
-            got = m.layer_output(i - 1).reshape(batch, -1)
+        yolo = [i for i in range(m.num_layers()) if m.layer_info(i)["type"] == "yolo"]
+        per = m.layer_info(yolo[0])["outC"] // 3
+        conf_t, nms_t = nu.thresholds(arch)
+        logits = [m.layer_output(i - 1).reshape(batch, -1) for i in yolo]
+        for k, i in enumerate(yolo):
             for b in range(batch):
-                e = nu.rel_err(got[b], ref[b][i - 1])
+                e = nu.rel_err(logits[k][b], ref[b][i - 1])
                 assert e <= 2e-2, f"{arch} head logits before layer {i}, image {b}: {e}"
         for b in range(batch):
-            # objectness logits closer to the threshold than the float16 error may legitimately flip
-            assert abs(len(boxes[b]) - len(ref_boxes[b])) <= max(2, 0.02 * len(ref_boxes[b]))
+            # every candidate that differs from the reference's -- present on one side only, or a row beyond 2e-2 -- sits on a reference
+            # logit no farther from a jump of the decode than the measured float16 error of its head; the box count differs by no more
+            # than the number of such cells; and the boxes are the reference's NMS of the returned candidates
+            ref_rows, only_dev, only_ref, differing, herr = nu.attribute_against_reference(
+                rows[b], [l[b] for l in logits], [ref[b][i] for i in yolo], [ref[b][i - 1] for i in yolo], per, conf_t)
+            attributed = len(only_dev) + len(only_ref) + len(differing)
+            print(f"{arch} image {b}: candidates {len(rows[b])} reference {len(ref_rows)}, attributed cells {attributed}, boxes {len(boxes[b])} reference {len(ref_boxes[b])}", flush=True)
+            assert abs(len(boxes[b]) - len(ref_boxes[b])) <= attributed
+            assert nu.same_box_set(netapi.boxes_from_candidates(rows[b], nms_t, fast=False), boxes[b])
+            nu.box_sets_equal_up_to_ties(netapi.boxes_from_candidates(ref_rows, nms_t, fast=True), ref_boxes[b], nms_t)
     else:
         logits = m.run_classify(x)
         for b in range(batch):
@@ -360,9 +374,9 @@ def test_weight_cache(tmp_path):
     netapi.set_weight_cache(True)
     try:
         a = netapi.Net(net, binp, fp16=True)
-        assert a.load_detail().endswith("pack file written") and os.path.exists(pack) and not os.path.exists(pack + ".tmp")
+        assert a.load_detail().endswith("pack file written") and os.path.exists(pack) and not [f for f in os.listdir(str(tmp_path)) if ".tmp" in f]
         blob = open(pack, "rb").read()
-        assert blob.startswith(b"msnhpack 1 layout ") and b" winograd 0 dtype 1\n" in blob[:100] and len(blob) > os.path.getsize(binp) // 4
+        assert blob.startswith(b"msnhpack 2 layout ") and b" winograd 0 dtype 1\n" in blob[:100] and len(blob) > os.path.getsize(binp) // 4
         b = netapi.Net(net, binp, fp16=True)
         print(a.load_detail(), b.load_detail(), sep="\n", flush=True)
         assert b.load_detail().endswith("pack file read") and open(pack, "rb").read() == blob
@@ -389,6 +403,22 @@ def test_weight_cache(tmp_path):
         open(pack, "wb").write(blob[:len(blob) // 2])
         f = netapi.Net(net, binp, fp16=True)
         assert f.load_detail().endswith("pack file written") and open(pack, "rb").read() == blob
+        # one flipped bit inside a packed kernel: its checksum refuses the file
+        bad = bytearray(blob)
+        bad[len(bad) * 3 // 4] ^= 0x04
+        open(pack, "wb").write(bytes(bad))
+        f2 = netapi.Net(net, binp, fp16=True)
+        assert f2.load_detail().endswith("pack file written") and open(pack, "rb").read() == blob
+        # the same graph with another activation parameter (the float16 calibration depends on it): not this graph's file
+        text = open(net).read()
+        assert "leaky" in text
+        net_slope = str(tmp_path / "m_slope.msnhnet")
+        open(net_slope, "w").write(text.replace("activation: leaky", "activation: leaky,0.3"))
+        f3 = netapi.Net(net_slope, binp, fp16=True)
+        assert f3.load_detail().endswith("pack file written")
+        f4 = netapi.Net(net, binp, fp16=True)
+        assert f4.load_detail().endswith("pack file written")
+        blob = open(pack, "rb").read()
         # the same weights in another graph (batch 1): not this plan's file
         g1 = zoo.ARCHS[arch](batch=1, size=size)
         net1 = str(tmp_path / "m1.msnhnet")
