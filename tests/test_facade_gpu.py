@@ -199,7 +199,7 @@ def test_facade_against_the_reference_facade(tmp_path):
         pytest.skip("reference build not present")
     L = netapi.lib()
     msg = ctypes.c_char_p()
-    size = 64
+    size = 224            # (the 7x7 average pool of this library needs the full-size feature map)
     net, binp, g = nu.model("resnet18", 1, size, seed=3)
     ref = refshim.RefFacade(nu.batch1_graph("resnet18", size), binp)
     img = _image(31, 50, 70)
