@@ -75,13 +75,82 @@ def cpu_baseline(arch, size, tmp, seed, budget_s=30.0):
                       f"({best:.2f} s per image incl. its NMS)"}
 
 
-# HBM bytes per convolution launch (fetch + write), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script,
-# each scaled by what the same counter reads for a plain copy kernel of known size (fetch x2.0, write x1.0); the runs
-# and their summary are in profiles/conv_igemm_yolov3_608_f16_b8.md.  None for workloads that were not profiled.
-HBM_BYTES_PER_CONV_LAUNCH = {("yolov3", "f16", 8): int((36.68 + 18.10) * 2**20)}
-# The same for the depthwise launches (the dominant bandwidth-bound kernel of a network that has them); runs and summary in
-# profiles/hbm_kernels_mobilenetv2_b64_yolov4_b16.md.
-HBM_BYTES_PER_DEPTHWISE_LAUNCH = {("mobilenetv2", "f16", 64): int((27.07 + 16.53) * 2**20)}
+# HBM bytes per launch (fetch + write) of the dominant kernels, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script and kept in profiles/hbm_traffic.json, one entry per (workload, dtype, batch) with the hash of the plan it was measured
+# on (launch kinds, algorithms and shapes; not the tile choices, which the per-layer search may settle differently from run to
+# run).  A plan that hashes differently -- a kernel or a fusion changed since -- reports null instead of a stale figure.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+HBM_PEAK = 8000.0           # GB/s
+
+
+def plan_hash(plan_text):
+    """hash of a plan description without its tile numbers and arena size"""
+    import hashlib
+    import re
+    # (which of the GEMM-type kernels and which tile runs a layer is the per-layer search's choice and may differ between two runs)
+    lines = [re.sub(r"\[(igemm_splitk|igemm|pointwise)", "[gemm", re.sub(r" t\d+", "", l)) for l in plan_text.splitlines()[1:]]
+    return hashlib.sha256("\n".join(lines).encode()).hexdigest()[:16]
+
+
+def measured_traffic(workload, dtype, batch, plan_text, key):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None
+    e = table.get(f"{workload}|{dtype}|{batch}")
+    if not e or e.get("plan_hash") != plan_hash(plan_text):
+        return None
+    return e.get(key)
+
+
+def attainable(rows, peak_tflops):
+    """rows: netapi.Net.profile_each_op_values().  For every convolution / connected launch the time it cannot beat is
+    t_min = max(FLOPs / MFMA peak, least bytes / HBM peak); returns the sums that say how far the measured launches are from that
+    bound, split by which roof binds."""
+    out = {"mfma_bound": {"launches": 0, "us": 0.0, "us_min": 0.0, "tflops": 0.0}, "hbm_bound": {"launches": 0, "us": 0.0, "us_min": 0.0, "gbs": 0.0}}
+    flops_m = bytes_h = 0.0
+    for kind, algo, layer, tile, flops, nbytes, us, ks in rows:
+        if int(kind) not in (0, 7) or int(algo) == MSNH_CONV_DEPTHWISE:
+            continue
+        t_m = flops / (peak_tflops * 1e12) * 1e6
+        t_h = nbytes / (HBM_PEAK * 1e9) * 1e6
+        c = out["mfma_bound"] if t_m >= t_h else out["hbm_bound"]
+        c["launches"] += 1
+        c["us"] += us
+        c["us_min"] += max(t_m, t_h)
+        if t_m >= t_h:
+            flops_m += flops
+        else:
+            bytes_h += nbytes
+    m, h = out["mfma_bound"], out["hbm_bound"]
+    m["tflops"] = round(flops_m / m["us"] * 1e-6, 1) if m["us"] else None
+    h["gbs"] = round(bytes_h / h["us"] * 1e-3, 1) if h["us"] else None
+    m["frac_of_mfma_peak"] = round(m["tflops"] / peak_tflops, 4) if m["us"] else None
+    h["frac_of_hbm_peak"] = round(h["gbs"] / HBM_PEAK, 4) if h["us"] else None
+    total_us, total_min = m["us"] + h["us"], m["us_min"] + h["us_min"]
+    for c in (m, h):
+        c["us"], c["us_min"] = round(c["us"], 1), round(c["us_min"], 1)
+    return round(total_min / total_us, 4) if total_us else None, out
+
+
+def bandwidth_kinds(rows):
+    """the bandwidth-bound launches of the plan by kind (depthwise, pools, upsample, copies, decode, ...): GB/s on least bytes"""
+    names = {1: "affine", 2: "add", 3: "copy", 4: "maxpool", 5: "avgpool", 6: "upsample", 8: "input_cast", 9: "yolo_decode", 10: "pad", 11: "slice",
+             12: "bilinear", 13: "softmax", 14: "col2im"}
+    acc = {}
+    for kind, algo, layer, tile, flops, nbytes, us, ks in rows:
+        name = "depthwise" if (int(kind) == 0 and int(algo) == MSNH_CONV_DEPTHWISE) else names.get(int(kind))
+        if name is None:
+            continue
+        a = acc.setdefault(name, [0, 0.0, 0.0])
+        a[0] += 1
+        a[1] += nbytes
+        a[2] += us
+    return {k: {"launches": v[0], "us": round(v[2], 1), "gbs": round(v[1] / v[2] * 1e-3, 1), "frac_of_hbm_peak": round(v[1] / v[2] * 1e-3 / HBM_PEAK, 4)}
+            for k, v in acc.items() if v[2] > 0}
+
+
 MSNH_CONV_DEPTHWISE = 3
 
 
@@ -399,18 +468,26 @@ def main():
 
     # roofline of the dominant kernel family: the convolution launches, timed with device events on the
     # library's stream; algorithmic FLOPs = 2*B*Cout*OH*OW*(Cin/g)*k*k per launch (direct-convolution count)
+    plan_text = net.plan_detail()
     marker()
     conv_ms, launches, flops, conv_bytes = net.profile_ops_bytes(0, 10)
     marker()
     achieved = flops / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else 0.0
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK[dtype], "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK[dtype], 4), "traffic": HBM_BYTES_PER_CONV_LAUNCH.get((a.workload, dtype, batch)),
+                "frac": round(achieved / PEAK[dtype], 4), "traffic": measured_traffic(a.workload, dtype, batch, plan_text, "conv_hbm_bytes_per_launch"),
                 "kernel": "convolution launches (implicit-GEMM MFMA + stem)", "launches_per_step": launches // 10,
                 "avg_launch_us": round(conv_ms * 1e3 / max(launches, 1), 2), "flops_per_step": flops / 10,
                 "least_bytes_per_launch": int(conv_bytes / max(launches, 1)),
                 # the same FLOPs over the time between results of the timed region (everything included: the other launches, decode, copy-back,
                 # host stage, several instances overlapping): what the job as a whole extracts from the matrix cores
                 "whole_job_tflops": round(flops / 10 / (ms_per_step * 1e-3) / 1e12, 2), "whole_job_frac": round(flops / 10 / (ms_per_step * 1e-3) / 1e12 / PEAK[dtype], 4)}
+
+    # How far the launches are from the roof that binds each of them: a launch cannot beat max(FLOPs / MFMA peak, least bytes / HBM
+    # peak).  Every launch is timed on its own here (back-to-back repetitions), so the sums are a little below the in-order pass above.
+    rows = net.profile_each_op_values(20)
+    roofline["attainable_frac"], roofline["by_binding_roof"] = attainable(rows, PEAK[dtype])
+    roofline["plan_hash"] = plan_hash(plan_text)
+    bw = bandwidth_kinds(rows)
 
     # what the matrix cores of this part sustain with nothing in their way (pure MFMA loops, three wavefronts per SIMD as in the
     # convolution kernels), and the shader clock they hold meanwhile: `peak` above is the published figure at the maximum clock
@@ -429,7 +506,7 @@ def main():
     if dw_n > 0:
         gbs = dw_bytes / (dw_ms * 1e-3) / 1e9
         roofline_hbm = {"bound": "hbm", "achieved": round(gbs, 1), "peak": 8000.0, "unit": "GB/s", "frac": round(gbs / 8000.0, 4),
-                        "traffic": HBM_BYTES_PER_DEPTHWISE_LAUNCH.get((a.workload, dtype, batch)), "kernel": "convDepthwise3x3FastKernel",
+                        "traffic": measured_traffic(a.workload, dtype, batch, plan_text, "depthwise_hbm_bytes_per_launch"), "kernel": "convDepthwise3x3FastKernel",
                         "launches_per_step": dw_n // 10, "avg_launch_us": round(dw_ms * 1e3 / dw_n, 2), "bytes_per_step": dw_bytes / 10}
 
     res = {"metric": f"images/sec on 1 MI355X ({a.workload} {size} {dtype} b{batch})", "value": round(batch / (ms_per_step * 1e-3), 2),
@@ -445,6 +522,8 @@ def main():
            "roofline": roofline}
     if roofline_hbm is not None:
         res["roofline_hbm"] = roofline_hbm
+    if bw:
+        res["bandwidth_launches"] = bw
     if detect:
         res["config"]["boxes_per_image"] = [int(len(b)) for b in out]
         res["config"]["nms"] = a.nms

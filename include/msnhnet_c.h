@@ -160,6 +160,10 @@ int msnhnet_profile_ops(msnhnet_t net, int kind, int reps, float *ms_total, int 
 int msnhnet_profile_ops_bytes(msnhnet_t net, int kind, int reps, float *ms_total, int *launches, double *flops, double *bytes);
 /* Per-launch timing table (text): every live launch of the plan timed on its own, `reps` repetitions each. */
 long long msnhnet_profile_each_op(msnhnet_t net, int reps, char *dst, long long cap);
+/* The same measurement as numbers: 8 doubles per live launch, in plan order -- kind (as msnhnet_profile_ops), convolution algorithm,
+ * layer index, tile, algorithmic FLOPs, least bytes (input + output + fused residual + weights), microseconds per launch,
+ * ksize * 100 + stride.  At most cap_rows rows are written; returns the number of launches. */
+long long msnhnet_profile_each_op_values(msnhnet_t net, int reps, double *dst, long long cap_rows);
 float msnhnet_gpu_inference_time(msnhnet_t net);          /* NetBuilder::getGpuInferenceTime, ms */
 /* YoloOutLayer::nms on its own (pure host code, no GPU needed): rows of 7 floats in (x y w h conf bestClsConf
  * bestClsIdx), already in the order the layer would pass them; fast = 0 runs the reference-shaped greedy loop,

@@ -115,7 +115,9 @@ public:
     // algorithm a (MSNH_CONV_*).  bytes (optional): what those launches must move at least (input + output + residual + weights).
     float profileOps(int kind, int reps, int *launches, double *flops, double *bytes = nullptr);
     // One line per live op: layer, kind, shapes, algorithm, microseconds per launch (mean of `reps`), TFLOP/s, GB/s.
-    std::string profileEachOp(int reps);
+    // every live launch of the plan timed on its own (reps back-to-back repetitions); values (optional) receives 8 numbers per launch:
+    // kind, algorithm, layer index, tile, algorithmic FLOPs, least bytes (input + output + fused residual + weights), microseconds, ksize * 100 + stride
+    std::string profileEachOp(int reps, std::vector<double> *values = nullptr);
 
 private:
     void finalizePlan();

@@ -472,6 +472,18 @@ int msnhnet_profile_ops_bytes(msnhnet_t net, int kind, int reps, float *ms_total
     });
 }
 
+long long msnhnet_profile_each_op_values(msnhnet_t net, int reps, double *dst, long long cap_rows)
+{
+    long long n = -1;
+    guarded([&] {
+        std::vector<double> v;
+        nb(net).profileEachOp(reps > 0 ? reps : 1, &v);
+        n = static_cast<long long>(v.size() / 8);
+        if (dst && cap_rows > 0) std::memcpy(dst, v.data(), sizeof(double) * 8 * static_cast<size_t>(std::min(cap_rows, n)));
+    });
+    return n;
+}
+
 long long msnhnet_profile_each_op(msnhnet_t net, int reps, char *dst, long long cap)
 {
     static thread_local std::string cache;

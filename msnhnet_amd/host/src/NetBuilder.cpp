@@ -881,7 +881,7 @@ float NetBuilder::profileOps(int kind, int reps, int *launches, double *flops, d
     return ms;
 }
 
-std::string NetBuilder::profileEachOp(int reps)
+std::string NetBuilder::profileEachOp(int reps, std::vector<double> *values)
 {
     if (!_planReady) MSNH_THROW("weights are not loaded");
     Plan &plan = *_net->plan;
@@ -911,6 +911,12 @@ std::string NetBuilder::profileEachOp(int reps)
         MSNH_DEV(msnh_hip_event_elapsed_ms(e0, e1, &ms));
         const double us = ms * 1e3 / reps;
         totalUs += us;
+        if (values)
+        {
+            const double row[8] = {static_cast<double>(op.kind), static_cast<double>(op.algo), static_cast<double>(op.layerIndex), static_cast<double>(op.tile),
+                                   op.flops, opBytes(plan, op), us, static_cast<double>(op.ksize * 100 + op.stride)};
+            values->insert(values->end(), row, row + 8);
+        }
         const PlanTensor &in = plan.tensors[static_cast<size_t>(op.in0)];
         const PlanTensor &out = plan.tensors[static_cast<size_t>(op.out)];
         const double bytes = static_cast<double>(in.elems()) * (in.dtype == MSNH_F16 ? 2 : 4) + static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4) +

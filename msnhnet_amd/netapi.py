@@ -18,7 +18,7 @@ SYMBOLS = [
     "msnhnet_input_dims", "msnhnet_num_layers", "msnhnet_layer_info", "msnhnet_layer_detail", "msnhnet_plan_detail", "msnhnet_conv_flops", "msnhnet_weight_layout", "msnhnet_fp16_headroom", "msnhnet_last_nms_on_device", "msnhnet_set_copy_on_forward_stream",
     "msnhnet_run_classify", "msnhnet_run_classify_gpu", "msnhnet_run_yolo_gpu", "msnhnet_layer_output", "msnhnet_yolo_head_logits", "msnhnet_yolo_candidates", "msnhnet_device_input",
     "msnhnet_enqueue", "msnhnet_sync", "msnhnet_fetch_classify", "msnhnet_fetch_yolo", "msnhnet_gpu_inference_time", "msnhnet_time_detail",
-    "msnhnet_profile_ops", "msnhnet_profile_ops_bytes", "msnhnet_profile_each_op", "msnhnet_yolo_max_boxes", "msnhnet_nms", "msnhnet_boxes_from_candidates",
+    "msnhnet_profile_ops", "msnhnet_profile_ops_bytes", "msnhnet_profile_each_op", "msnhnet_profile_each_op_values", "msnhnet_yolo_max_boxes", "msnhnet_nms", "msnhnet_boxes_from_candidates",
     "msnhnet_group_create", "msnhnet_group_destroy", "msnhnet_group_info", "msnhnet_group_instance", "msnhnet_group_prime", "msnhnet_group_submit",
     "msnhnet_group_flush", "msnhnet_group_fetch_classify", "msnhnet_group_fetch_yolo",
 ]
@@ -123,6 +123,8 @@ def lib():
     L.msnhnet_profile_ops_bytes.argtypes = [vp, ci, ci, fp, ip, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]
     L.msnhnet_profile_each_op.argtypes = [vp, ci, cp, ll]
     L.msnhnet_profile_each_op.restype = ll
+    L.msnhnet_profile_each_op_values.argtypes = [vp, ci, ctypes.POINTER(ctypes.c_double), ll]
+    L.msnhnet_profile_each_op_values.restype = ll
     L.msnhnet_nms.argtypes = [fp, ll, ctypes.c_float, ci, fp, ll, llp]
     L.msnhnet_boxes_from_candidates.argtypes = [fp, ll, ctypes.c_float, ci, fp, ll, llp]
     L.msnhnet_yolo_max_boxes.argtypes = [vp]
@@ -418,6 +420,14 @@ class Net:
         ms, n, f, b = ctypes.c_float(), ctypes.c_int(), ctypes.c_double(), ctypes.c_double()
         _check(self.L.msnhnet_profile_ops_bytes(self.h, kind, reps, ctypes.byref(ms), ctypes.byref(n), ctypes.byref(f), ctypes.byref(b)))
         return ms.value, n.value, f.value, b.value
+
+    def profile_each_op_values(self, reps=20):
+        """[launches, 8]: kind, algorithm, layer, tile, FLOPs, least bytes, microseconds, ksize * 100 + stride of every live launch"""
+        a = np.zeros((4096, 8), np.float64)                 # (one call: the measurement itself is what takes time)
+        n = self.L.msnhnet_profile_each_op_values(self.h, reps, a.ctypes.data_as(ctypes.POINTER(ctypes.c_double)), len(a))
+        if n < 0:
+            _check(1)
+        return a[:n].copy()
 
     def profile_each_op(self, reps=20):
         n = self.L.msnhnet_profile_each_op(self.h, reps, None, 0)

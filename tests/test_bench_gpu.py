@@ -41,3 +41,14 @@ def test_bench_prints_one_json_line_with_the_contract_keys(workload, instances):
     assert abs(rf["frac"] - rf["achieved"] / rf["peak"]) < 2e-4
     # achieved = FLOPs of one pass over the convolution launches / their summed duration
     assert abs(rf["achieved"] - rf["flops_per_step"] / (rf["launches_per_step"] * rf["avg_launch_us"] * 1e-6) / 1e12) <= 0.01 * rf["achieved"]
+    # the attainable bound: every convolution launch against max(FLOPs / MFMA peak, least bytes / HBM peak), split by the binding roof
+    assert 0 < rf["attainable_frac"] <= 1.0 and len(rf["plan_hash"]) == 16
+    split = rf["by_binding_roof"]
+    n = split["mfma_bound"]["launches"] + split["hbm_bound"]["launches"]
+    assert n >= rf["launches_per_step"] - 1 and n <= rf["launches_per_step"] + 2          # (+ the connected layer where it is not lowered to a convolution)
+    t = split["mfma_bound"]["us"] + split["hbm_bound"]["us"]
+    t_min = split["mfma_bound"]["us_min"] + split["hbm_bound"]["us_min"]
+    assert abs(rf["attainable_frac"] - t_min / t) < 5e-3
+    for c in ("mfma_bound", "hbm_bound"):
+        assert split[c]["us_min"] <= split[c]["us"]
+    assert rf["traffic"] is None or rf["traffic"] > 0
