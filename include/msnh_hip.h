@@ -196,6 +196,14 @@ int msnh_hip_copy_channels(int dtype, long long pixels, int c, const void *x, in
  * cudnnPoolingForward, src/layers/MsnhMaxPoolLayer.cpp:460-463). */
 int msnh_hip_maxpool(int dtype, int batch, int in_h, int in_w, int c, const void *x, int x_ld, int ksize, int stride,
                      int pad, int out_h, int out_w, void *y, int y_ld, msnh_stream_t s);
+/* `steps` (2 or 3) stride-1 max-pools of window ksize (3 or 5) and padding ksize / 2, the first over x, each further one over the
+ * result of the one before it, in one launch; pool i writes y[i] (row stride y_ld[i]).  What the reference runs as separate layers
+ * over one tensor in its SPP blocks -- windows 5, 9 and 13 (src/layers/MsnhMaxPoolLayer.cpp:293-345 called three times from
+ * src/layers/MsnhConcatBlockLayer.cpp:255-355) are 5 over 5 over 5 -- with the same results as msnh_hip_maxpool called per pool.
+ * msnh_hip_maxpool_chain_supported says whether the geometry is taken (the H x W tile of an image must fit LDS). */
+int msnh_hip_maxpool_chain_supported(int dtype, int in_h, int in_w, int c, int ksize, int steps);
+int msnh_hip_maxpool_chain(int dtype, int batch, int in_h, int in_w, int c, int ksize, int steps, const void *x, int x_ld, void *const *y,
+                           const int *y_ld, msnh_stream_t s);
 /* Average over the valid window elements (localAvgPoolNormalKernel, src/layers/cuda/MsnhLocalAvgPoolLayerGPU.cu:5;
  * CPU semantics src/layers/MsnhLocalAvgPoolLayer.cpp:286-344).  y = out_mul * mean. */
 int msnh_hip_avgpool(int dtype, int out_dtype, int batch, int in_h, int in_w, int c, const void *x, int x_ld, int ksize,

@@ -179,6 +179,110 @@ __global__ __launch_bounds__(256) void maxPoolUnrolledKernel(const T *__restrict
     storeVec<T, VEC>(y + p * yLd + c0, m);
 }
 
+// A chain of stride-1 "same" max-pools of one window size, each reading the result of the one before it (the SPP block of the YOLOv4 /
+// YOLOv5 graphs: windows 5, 9 and 13 over one tensor are 5 over 5 over 5), in ONE launch: a workgroup holds the H x W tile of one
+// image for CG channels in LDS, runs every pool of the chain as a row pass and a column pass over it (the maximum over a window is
+// the maximum over its rows of the row maxima) and writes each result straight to its own destination.  The input crosses memory
+// once instead of once per pool, and one launch replaces three whose 25-tap windows were bound by load latency on 6 MB tensors.
+// Results are those of the separate launches bit for bit: a value replaces the running maximum only if it compares greater (a NaN
+// never does), positions outside the image are ignored, a window without any usable value gives -FLT_MAX, float16 stores clamp that
+// to the most negative finite half -- and each pool of the chain sees its predecessor's stored values.
+template <typename T, int VEC, int K>
+__global__ __launch_bounds__(1024) void maxPoolChainKernel(const T *__restrict__ x, int xLd, int H, int W, int c, int cg, int steps, int blocks, T *__restrict__ y0, int y0Ld,
+                                                           T *__restrict__ y1, int y1Ld, T *__restrict__ y2, int y2Ld)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char poolSmem[];
+    T *bufA = reinterpret_cast<T *>(poolSmem);
+    T *bufB = bufA + static_cast<size_t>(H) * W * cg;
+    const int groups = (c + cg - 1) / cg;
+    // workgroups are dealt to the 8 XCDs in contiguous runs: the channel groups of one image, which share every 128-byte line of
+    // the tensor between two of them, meet in one L2
+    const int perXcd = (blocks + 7) / 8;
+    const int logical = static_cast<int>(blockIdx.x % 8) * perXcd + static_cast<int>(blockIdx.x / 8);
+    if (logical >= blocks) return;
+    const int b = logical / groups;
+    const int c0 = (logical % groups) * cg;
+    const int cw = ((c - c0 < cg) ? c - c0 : cg) / VEC;           // channel vectors of a pixel in this group
+    const int pixels = H * W;
+    const int items = pixels * cw;                                // at most 4 per thread (host)
+    const long long img = static_cast<long long>(b) * pixels;
+    constexpr int R = K / 2;
+    constexpr int MAXI = 4;
+    typedef typename VecOf<T, VEC>::type V;
+    // a thread keeps the same (pixel, channel vector) items through every pass: where they sit in LDS, which neighbours of their row
+    // and column exist (bit d + R of a mask), where they go in memory -- the divisions are paid once
+    int ldsOff[MAXI], chan[MAXI], pix[MAXI];
+    unsigned rowMask[MAXI], colMask[MAXI];
+#pragma unroll
+    for (int k = 0; k < MAXI; ++k)
+    {
+        const int i = threadIdx.x + k * 1024;
+        ldsOff[k] = -1;
+        chan[k] = pix[k] = 0;
+        rowMask[k] = colMask[k] = 0u;
+        if (i < items)
+        {
+            const int p = i / cw, v = i - p * cw;
+            const int py = p / W, px = p - py * W;
+            ldsOff[k] = p * cg + v * VEC;
+            pix[k] = p;
+            chan[k] = v * VEC;
+#pragma unroll
+            for (int d = -R; d <= R; ++d)
+            {
+                if (px + d >= 0 && px + d < W) rowMask[k] |= 1u << (d + R);
+                if (py + d >= 0 && py + d < H) colMask[k] |= 1u << (d + R);
+            }
+            *reinterpret_cast<V *>(bufA + ldsOff[k]) = *reinterpret_cast<const V *>(x + (img + p) * xLd + c0 + v * VEC);
+        }
+    }
+    __syncthreads();
+    const int rowStep = cg, colStep = W * cg;
+    auto pass = [&](const T *src, int step, unsigned mask, int off, float (&m)[VEC]) {
+        float t[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) m[e] = -FLT_MAX;
+#pragma unroll
+        for (int d = -R; d <= R; ++d)
+        {
+            if (!(mask & (1u << (d + R)))) continue;
+            loadVec<T, VEC>(src + off + d * step, t);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) m[e] = t[e] > m[e] ? t[e] : m[e];
+        }
+        if constexpr (sizeof(T) == 2)
+        {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) m[e] = m[e] < -65504.f ? -65504.f : m[e];
+        }
+    };
+    for (int s = 0; s < steps; ++s)
+    {
+        float m[VEC];
+        // rows: A -> B
+#pragma unroll
+        for (int k = 0; k < MAXI; ++k)
+            if (ldsOff[k] >= 0)
+            {
+                pass(bufA, rowStep, rowMask[k], ldsOff[k], m);
+                storeVec<T, VEC>(bufB + ldsOff[k], m);
+            }
+        __syncthreads();
+        // columns: B -> this pool's destination, and back into A for the next pool
+        T *y = s == 0 ? y0 : (s == 1 ? y1 : y2);
+        const int yLd = s == 0 ? y0Ld : (s == 1 ? y1Ld : y2Ld);
+#pragma unroll
+        for (int k = 0; k < MAXI; ++k)
+            if (ldsOff[k] >= 0)
+            {
+                pass(bufB, colStep, colMask[k], ldsOff[k], m);
+                storeVec<T, VEC>(y + (img + pix[k]) * yLd + c0 + chan[k], m);
+                if (s + 1 < steps) storeVec<T, VEC>(bufA + ldsOff[k], m);
+            }
+        __syncthreads();
+    }
+}
+
 // ---- average pooling over valid elements -------------------------------------------------------------
 template <typename T, typename TOut, int VEC>
 __global__ __launch_bounds__(256) void avgPoolKernel(const T *__restrict__ x, int xLd, int H, int W, int c, int ksize, int stride,
@@ -652,6 +756,52 @@ int msnh_hip_maxpool(int dtype, int batch, int in_h, int in_w, int c, const void
     if (dtype == MSNH_F16) { if (vec == 8) MSNH_MP(f16, 8); else MSNH_MP(f16, 1); }
     else { if (vec == 4) MSNH_MP(float, 4); else MSNH_MP(float, 1); }
 #undef MSNH_MP
+    MSNH_LAUNCH_CHECK();
+    return 0;
+}
+
+// channels per workgroup of the chained max-pool for this geometry (two H x W tiles of them must fit 48 KiB of LDS); 0 = not taken
+static int poolChainGroup(int dtype, int in_h, int in_w, int c, int ksize, int steps)
+{
+    const int vec = dtype == MSNH_F16 ? 8 : 4;
+    const size_t es = dtype == MSNH_F16 ? 2 : 4;
+    if (!(ksize == 3 || ksize == 5) || steps < 2 || steps > 3 || c % vec != 0) return 0;
+    // two tiles in at most 48 KiB of LDS, and at most 4 (pixel, channel vector) items for each of the 1024 threads
+    for (int cg = 64; cg >= vec; cg /= 2)
+        if (2 * static_cast<size_t>(in_h) * in_w * cg * es <= 48 * 1024 && static_cast<long long>(in_h) * in_w * (cg / vec) <= 4096) return cg;
+    return 0;
+}
+
+int msnh_hip_maxpool_chain_supported(int dtype, int in_h, int in_w, int c, int ksize, int steps)
+{
+    return dtypeOk(dtype) && in_h > 0 && in_w > 0 && c > 0 && poolChainGroup(dtype, in_h, in_w, c, ksize, steps) > 0 ? 1 : 0;
+}
+
+int msnh_hip_maxpool_chain(int dtype, int batch, int in_h, int in_w, int c, int ksize, int steps, const void *x, int x_ld, void *const *y,
+                           const int *y_ld, msnh_stream_t s)
+{
+    MSNH_REQUIRE(dtypeOk(dtype), "maxpool_chain: bad dtype");
+    MSNH_REQUIRE(batch > 0 && in_h > 0 && in_w > 0 && c > 0 && x && y && y_ld && x_ld >= c, "maxpool_chain: bad argument");
+    const int cg = poolChainGroup(dtype, in_h, in_w, c, ksize, steps);
+    MSNH_REQUIRE(cg > 0, "maxpool_chain: windows of 3 or 5, 2 or 3 pools, channels a multiple of the 16-byte vector, and an H x W tile that fits LDS "
+                         "(msnh_hip_maxpool_chain_supported)");
+    const int vec = dtype == MSNH_F16 ? 8 : 4;
+    MSNH_REQUIRE(x_ld % vec == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0, "maxpool_chain: input must be 16-byte aligned with a row stride of whole vectors");
+    for (int i = 0; i < steps; ++i)
+        MSNH_REQUIRE(y[i] && y_ld[i] >= c && y_ld[i] % vec == 0 && reinterpret_cast<uintptr_t>(y[i]) % 16 == 0,
+                     "maxpool_chain: every destination must be 16-byte aligned with a row stride of whole vectors");
+    const long long blocks = static_cast<long long>(batch) * ((c + cg - 1) / cg);
+    MSNH_REQUIRE(blocks < (1LL << 31), "maxpool_chain: too many tiles");
+    hipStream_t st = resolveStream(s);
+    const size_t smem = 2 * static_cast<size_t>(in_h) * in_w * cg * (dtype == MSNH_F16 ? 2 : 4);
+    void *y2 = steps > 2 ? y[2] : y[1];
+    const int y2Ld = steps > 2 ? y_ld[2] : y_ld[1];
+#define MSNH_MPC(T, V, K)                                                                                              \
+    hipLaunchKernelGGL((maxPoolChainKernel<T, V, K>), dim3(static_cast<unsigned>((blocks + 7) / 8 * 8)), dim3(1024), smem, st, static_cast<const T *>(x), x_ld, in_h, in_w, c, cg, \
+                       steps, static_cast<int>(blocks), static_cast<T *>(y[0]), y_ld[0], static_cast<T *>(y[1]), y_ld[1], static_cast<T *>(y2), y2Ld)
+    if (dtype == MSNH_F16) { if (ksize == 3) MSNH_MPC(f16, 8, 3); else MSNH_MPC(f16, 8, 5); }
+    else { if (ksize == 3) MSNH_MPC(float, 4, 3); else MSNH_MPC(float, 4, 5); }
+#undef MSNH_MPC
     MSNH_LAUNCH_CHECK();
     return 0;
 }

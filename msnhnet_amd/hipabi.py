@@ -38,7 +38,7 @@ SYMBOLS = [
     "msnh_hip_event_destroy", "msnh_hip_event_record", "msnh_hip_stream_wait_event", "msnh_hip_event_sync", "msnh_hip_event_elapsed_ms", "msnh_hip_graph_begin",
     "msnh_hip_graph_end", "msnh_hip_graph_launch", "msnh_hip_graph_destroy", "msnh_hip_conv_stem_down_supported", "msnh_hip_conv_stem_down_packed_elems", "msnh_hip_conv_stem_down_pack", "msnh_hip_conv_stem_down", "msnh_hip_conv2d_tile_count", "msnh_hip_conv2d_pack_layout_version", "msnh_hip_conv2d_tile_supported", "msnh_hip_conv2d_select_algo",
     "msnh_hip_conv2d_packed_weight_elems", "msnh_hip_conv2d_pack_weights", "msnh_hip_conv2d_workspace_bytes", "msnh_hip_conv2d", "msnh_hip_letterbox_u8", "msnh_hip_image_u8_to_input",
-    "msnh_hip_affine_act", "msnh_hip_add_act", "msnh_hip_copy_channels", "msnh_hip_maxpool", "msnh_hip_avgpool",
+    "msnh_hip_affine_act", "msnh_hip_add_act", "msnh_hip_copy_channels", "msnh_hip_maxpool", "msnh_hip_maxpool_chain", "msnh_hip_maxpool_chain_supported", "msnh_hip_avgpool",
     "msnh_hip_upsample_nearest", "msnh_hip_pad", "msnh_hip_slice", "msnh_hip_upsample_bilinear", "msnh_hip_softmax", "msnh_hip_deconv_col2im", "msnh_hip_connected", "msnh_hip_nchw_to_nhwc", "msnh_hip_nhwc_to_nchw", "msnh_hip_yolo_decode", "msnh_hip_yolo_decode_candidates", "msnh_hip_yolo_decode_candidates_heads",
     "msnh_hip_yolo_gather", "msnh_hip_yolo_nms", "msnh_hip_yolo_nms_workspace_bytes", "msnh_hip_yolo_nms_pair_workspace_bytes", "msnh_hip_yolo_nms_static", "msnh_hip_yolo_nms_static_max_bytes", "msnh_hip_absmax", "msnh_hip_count_nonfinite", "msnh_hip_mfma_probe",
 ]
@@ -98,6 +98,8 @@ def lib():
     L.msnh_hip_add_act.argtypes = [ci, ll, ci, vp, ci, cf, vp, ci, cf, ci, cf, cf, vp, ci, vp]
     L.msnh_hip_copy_channels.argtypes = [ci, ll, ci, vp, ci, cf, vp, ci, vp]
     L.msnh_hip_maxpool.argtypes = [ci, ci, ci, ci, ci, vp, ci, ci, ci, ci, ci, ci, vp, ci, vp]
+    L.msnh_hip_maxpool_chain_supported.argtypes = [ci, ci, ci, ci, ci, ci]
+    L.msnh_hip_maxpool_chain.argtypes = [ci, ci, ci, ci, ci, ci, ci, vp, ci, ctypes.POINTER(vp), ctypes.POINTER(ci), vp]
     L.msnh_hip_avgpool.argtypes = [ci, ci, ci, ci, ci, ci, vp, ci, ci, ci, ci, ci, ci, cf, vp, ci, vp]
     L.msnh_hip_upsample_nearest.argtypes = [ci, ci, ci, ci, ci, vp, ci, ci, cf, vp, ci, vp]
     L.msnh_hip_pad.argtypes = [ci, ci, ci, ci, ci, vp, ci, ci, ci, ci, ci, cf, cf, vp, ci, vp]

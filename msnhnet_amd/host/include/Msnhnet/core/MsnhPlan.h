@@ -73,6 +73,8 @@ struct PlanOp
     int  tile = 0;                          // CONV/IGEMM: tile configuration chosen by Plan::tuneConvs (0 = library default)
     BaseLayer *src = nullptr;               // layer that owns the host weights of this op
     BaseLayer *src2 = nullptr;              // batch-norm layer folded into a CONV
+    int  chainHead = -1;                    // MAXPOOL: >= 0 = this pool's result is written by the launch of op chainHead (a chain of stride-1 pools in one launch)
+    int  chainNext = -1;                    // MAXPOOL at the head or inside such a chain: the op whose pool follows
     int  stemOp = -1;                       // CONV 3x3 stride 2: the (dead) first-layer op computed in front of it by the same launch (Plan::fuse c)
 
     // YOLO_DECODE
@@ -144,7 +146,7 @@ public:
     void  exportTensor(int t, std::vector<float> &dst, msnh_stream_t s);
 
     size_t arenaBytes() const { return _arena.bytes(); }
-    size_t liveOps() const;
+    size_t liveOps() const;                 // launches of one forward
     double totalConvFlops() const;
     std::string describe() const;           // one line per live op: kind, shapes, algorithm
 

@@ -843,7 +843,8 @@ static double opBytes(const Plan &plan, const PlanOp &op)
     // what the launch must move at least: its input, its output, a fused residual, its weights
     const PlanTensor &in = plan.tensors[static_cast<size_t>(op.in0)];
     const PlanTensor &out = plan.tensors[static_cast<size_t>(op.out)];
-    const double oe = static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4);
+    double oe = static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4);
+    for (int nx = op.chainNext; nx >= 0; nx = plan.ops[static_cast<size_t>(nx)].chainNext) oe += static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4);   // one launch, every pool's result
     return static_cast<double>(in.elems()) * (in.dtype == MSNH_F16 ? 2 : 4) + oe + (op.in1 >= 0 ? oe : 0.0) + static_cast<double>(op.wDev.bytes());
 }
 
@@ -862,7 +863,7 @@ float NetBuilder::profileOps(int kind, int reps, int *launches, double *flops, d
         {
             const PlanOp &op = plan.ops[i];
             // kind: a PlanOp::Kind, -1 for every launch, or 1000 + a convolution algorithm (MSNH_CONV_*)
-            if (op.dead) continue;
+            if (op.dead || op.chainHead >= 0) continue;
             if (kind >= 1000 ? (op.kind != PlanOp::CONV || op.algo != kind - 1000) : (kind >= 0 && static_cast<int>(op.kind) != kind)) continue;
             plan.run(i, i + 1, _stream);
             ++n;
@@ -895,7 +896,7 @@ std::string NetBuilder::profileEachOp(int reps, std::vector<double> *values)
     for (size_t i = 0; i < plan.ops.size(); ++i)
     {
         const PlanOp &op = plan.ops[i];
-        if (op.dead) continue;
+        if (op.dead || op.chainHead >= 0) continue;
         plan.run(i, i + 1, _stream);
         const bool yolo = op.kind == PlanOp::YOLO_DECODE && plan.yoloCandCnt.ptr();
         MSNH_DEV(msnh_hip_event_record(e0, _stream));

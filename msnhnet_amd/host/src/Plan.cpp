@@ -80,7 +80,7 @@ int Plan::consumerCount(int tensor) const
 size_t Plan::liveOps() const
 {
     size_t n = 0;
-    for (const PlanOp &op : ops) n += op.dead ? 0 : 1;
+    for (const PlanOp &op : ops) n += (op.dead || op.chainHead >= 0) ? 0 : 1;
     return n;
 }
 
@@ -264,6 +264,19 @@ void Plan::chainMaxPools()
             cur.pad = cur.ksize / 2;
             prevK = k;
         }
+        // pools of one window size over one tile that fits LDS run as ONE launch, issued where the first of them stands
+        // (msnh_hip_maxpool_chain): the others keep their place in the op list -- their outputs, lifetimes and calibration
+        // stay what they are -- but launch nothing
+        bool sameK = slots.size() <= 3;
+        for (size_t q = 1; q < slots.size(); ++q) sameK = sameK && ops[slots[q]].ksize == ops[slots[0]].ksize;
+        const PlanTensor &in = tensors[static_cast<size_t>(ops[slots[0]].in0)];
+        if (sameK && in.layout == PlanTensor::NHWC && !std::getenv("MSNH_NO_POOL_CHAIN") &&
+            msnh_hip_maxpool_chain_supported(in.dtype, in.h, in.w, in.c, ops[slots[0]].ksize, static_cast<int>(slots.size())))
+            for (size_t q = 1; q < slots.size(); ++q)
+            {
+                ops[slots[q]].chainHead = static_cast<int>(slots[0]);
+                ops[slots[q - 1]].chainNext = static_cast<int>(slots[q]);
+            }
     }
 }
 
@@ -369,7 +382,7 @@ uint64_t Plan::structureHash() const
     for (const PlanOp &op : ops)
         os << static_cast<int>(op.kind) << ' ' << op.in0 << ' ' << op.in1 << ' ' << op.out << ' ' << op.dead << ' ' << op.layerIndex << ' ' << op.ksize << ' ' << op.stride << ' '
            << op.pad << ' ' << op.dilation << ' ' << op.groups << ' ' << static_cast<int>(op.act) << ' ' << static_cast<int>(op.act2) << ' ' << op.in1Sign << ' ' << (op.src2 != nullptr)
-           << ' ' << op.dstChanOffset << ' ' << op.stemOp << ';';
+           << ' ' << op.dstChanOffset << ' ' << op.stemOp << ' ' << op.chainHead << ';';
     const std::string text = os.str();
     return PackFile::hash(text.data(), text.size());
 }
@@ -426,6 +439,7 @@ void Plan::place()
         const PlanOp &op = ops[static_cast<size_t>(i)];
         if (op.dead) continue;
         touch(op.in0, i); touch(op.in1, i); touch(op.out, i);
+        if (op.chainHead >= 0) touch(op.out, op.chainHead);      // written by the launch of the chain's first pool
     }
     {
         // the heads of a detector may all be decoded by one launch where the last of them stands (findYoloHeads): their inputs
@@ -991,6 +1005,20 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
         break;
     }
     case PlanOp::MAXPOOL:
+        if (op.chainHead >= 0) break;                            // done by the launch of the chain's first pool
+        if (op.chainNext >= 0)
+        {
+            void *ys[3] = {ptr(op.out), nullptr, nullptr};
+            int lds[3] = {ld(op.out), 0, 0};
+            int steps = 1;
+            for (int nx = op.chainNext; nx >= 0 && steps < 3; nx = ops[static_cast<size_t>(nx)].chainNext, ++steps)
+            {
+                ys[steps] = ptr(ops[static_cast<size_t>(nx)].out);
+                lds[steps] = ld(ops[static_cast<size_t>(nx)].out);
+            }
+            MSNH_DEV(msnh_hip_maxpool_chain(in.dtype, in.n, in.h, in.w, in.c, op.ksize, steps, ptr(op.in0), ld(op.in0), ys, lds, s));
+            break;
+        }
         MSNH_DEV(msnh_hip_maxpool(in.dtype, in.n, in.h, in.w, in.c, ptr(op.in0), ld(op.in0), op.ksize, op.stride, op.pad, out.h, out.w,
                                   ptr(op.out), ld(op.out), s));
         break;
@@ -1142,7 +1170,8 @@ std::string Plan::describe() const
         os << "  L" << op.layerIndex << " " << kinds[op.kind];
         if (op.kind == PlanOp::CONV)
             os << "[" << algos[op.algo] << (op.tile ? " t" + std::to_string(op.tile) : std::string()) << " k" << op.ksize << " s" << op.stride << " g" << op.groups << (op.in1 >= 0 ? " +res" : "") << (op.src2 ? " +bn" : "") << "]";
-        if (op.kind == PlanOp::MAXPOOL || op.kind == PlanOp::AVGPOOL) os << "[k" << op.ksize << " s" << op.stride << " p" << op.pad << "]";
+        if (op.kind == PlanOp::MAXPOOL || op.kind == PlanOp::AVGPOOL)
+            os << "[k" << op.ksize << " s" << op.stride << " p" << op.pad << (op.chainHead >= 0 ? " in the launch of the pool before it" : "") << "]";
         os << " " << in.n << "x" << in.h << "x" << in.w << "x" << in.c << " -> " << out.h << "x" << out.w << "x" << out.c
            << (out.dtype == MSNH_F16 ? " f16" : " f32") << " e" << out.scaleExp;
         if (out.parent >= 0) os << " (slice@" << chanOffsetInRoot(op.out) << " of " << tensors[static_cast<size_t>(root(op.out))].c << ")";

@@ -544,13 +544,32 @@ def test_yolo_rows_copied_in_part():
 
 
 def test_spp_maxpools_run_as_a_chain():
-    """the 5 / 9 / 13 pools of an SPP block become three 5-wide pools, each reading the one before (same results: the
-    per-layer and final-output parity tests of yolov4 and yolov5s run through this plan)"""
+    """the 5 / 9 / 13 pools of an SPP block become three 5-wide pools, each reading the one before, and where the tile of an image
+    fits LDS they are one launch (same results: the per-layer and final-output parity tests of yolov4 and yolov5s run through this
+    plan; with MSNH_NO_POOL_CHAIN the separate launches give the same boxes bit for bit)"""
     for arch, size in (("yolov4", 160), ("yolov5s", 160)):
-        net, binp, g = nu.model(arch, 1, size, seed=3)
-        m = netapi.Net(net, binp, fp16=True)
-        pools = [ln for ln in m.plan_detail().splitlines() if " maxpool[" in ln and " s1 " in ln]
-        assert len(pools) == 3 and all("[k5 s1 p2]" in ln for ln in pools), pools
+        net, binp, g = nu.model(arch, 2, size, seed=3)
+        x = zoo.seeded_input(2, 3, size, size, seed=4)
+        netapi.set_tune_cache(True)                 # the same tiles in both builds below
+        try:
+            m = netapi.Net(net, binp, fp16=True)
+            pools = [ln for ln in m.plan_detail().splitlines() if " maxpool[" in ln and " s1 " in ln]
+            assert len(pools) == 3 and all("[k5 s1 p2" in ln for ln in pools), pools
+            assert sum("in the launch of the pool before it" in ln for ln in pools) == 2, pools
+            launches = int(m.plan_detail().split(" launches")[0].split()[-1])
+            fused = m.run_yolo(x)
+            os.environ["MSNH_NO_POOL_CHAIN"] = "1"
+            try:
+                m2 = netapi.Net(net, binp, fp16=True)
+            finally:
+                del os.environ["MSNH_NO_POOL_CHAIN"]
+            assert "in the launch of the pool before it" not in m2.plan_detail()
+            assert int(m2.plan_detail().split(" launches")[0].split()[-1]) == launches + 2
+            apart = m2.run_yolo(x)
+            for a, b in zip(fused, apart):
+                assert len(a) > 0 and np.array_equal(a, b, equal_nan=True)
+        finally:
+            netapi.set_tune_cache(False)
 
 
 def test_image_in_boxes_out():

@@ -109,6 +109,53 @@ def test_maxpool_windows_compose(h, w, dtype):
     assert torch.equal(out["5o5"], out["9"]) and torch.equal(out["5o9"], out["13"])
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("h,w,c,k,steps", [(19, 19, 512, 5, 3), (13, 13, 72, 5, 3), (7, 5, 24, 5, 2), (16, 16, 256, 3, 3), (2, 2, 8, 5, 3)])
+def test_maxpool_chain(h, w, c, k, steps, dtype):
+    """the pools of an SPP block in one launch (msnh_hip_maxpool_chain): every pool's result equals the oracle's max-pool with the
+    composed window (k, 2k-1, 3k-2) and the separate launches bit for bit, also into channel slices of a wider tensor (the concat
+    the block writes), with NaN, infinities and a window that holds nothing usable in the input"""
+    import ctypes
+    import gpuutil as gu
+    gu.init()
+    L = abi.lib()
+    assert L.msnh_hip_maxpool_chain_supported(dtype, h, w, c, k, steps) == 1
+    rng = np.random.default_rng(h * 131 + c)
+    batch = 3
+    x = _x(rng, (batch, c, h, w), dtype)
+    x[0, 0, 0, 0] = np.nan
+    x[1, 1, :, :] = -np.inf                      # a channel without any value that compares greater than -FLT_MAX
+    x[2, 2, h // 2, w // 2] = np.inf
+    xd = gu.nhwc_dev(x, dtype)
+    ld = (steps + 1) * c + 8
+    cat = torch.full((batch, h, w, ld), 3.0, dtype=gu.TORCH_DT[dtype]).cuda()          # [pool_steps .. pool_1, (x), 8 spare channels]
+    es = 2 if dtype == abi.F16 else 4
+    ys = (ctypes.c_void_p * steps)(*[cat.data_ptr() + (steps - 1 - i) * c * es for i in range(steps)])
+    lds = (ctypes.c_int * steps)(*([ld] * steps))
+    gu.sync()
+    abi.check(L.msnh_hip_maxpool_chain(dtype, batch, h, w, c, k, steps, gu.ptr(xd), c, ys, lds, None))
+    gu.sync()
+    got = cat.cpu()
+    assert (got[..., steps * c:] == 3.0).all(), "wrote outside its slices"
+    src = xd
+    for i in range(steps):
+        sep = torch.zeros((batch, h, w, c), dtype=gu.TORCH_DT[dtype]).cuda()
+        abi.check(L.msnh_hip_maxpool(dtype, batch, h, w, c, gu.ptr(src), c, k, 1, k // 2, h, w, gu.ptr(sep), c, None))
+        gu.sync()
+        mine = got[..., (steps - 1 - i) * c:(steps - i) * c]
+        assert torch.equal(mine.contiguous().view(torch.int16 if dtype == abi.F16 else torch.int32),
+                           sep.cpu().view(torch.int16 if dtype == abi.F16 else torch.int32)), f"pool {i} differs from the separate launch"
+        kk = (i + 1) * (k - 1) + 1
+        finite = np.isfinite(x).all(axis=(2, 3))          # (the oracle comparison on the channels without special values)
+        want = on.maxpool(x, kk, 1, kk // 2)
+        have = mine.float().numpy().transpose(0, 3, 1, 2)
+        assert np.array_equal(have[finite], want[finite])
+        src = sep
+    # geometries it does not take are refused
+    assert L.msnh_hip_maxpool_chain_supported(dtype, 76, 76, 256, 5, 3) == 0
+    assert L.msnh_hip_maxpool_chain_supported(dtype, h, w, c, 7, 3) == 0
+
+
 @pytest.mark.parametrize("dtype,out_dtype", [(abi.F32, abi.F32), (abi.F16, abi.F16), (abi.F16, abi.F32)])
 @pytest.mark.parametrize("c,h,w,k,s,p", [(512, 7, 7, 7, 1, 0), (24, 9, 9, 3, 2, 1)])
 def test_avgpool(c, h, w, k, s, p, dtype, out_dtype):
