@@ -171,9 +171,12 @@ def conv_shape_mode(a):
     L = abi.lib()
     abi.check(L.msnh_hip_init(0))
     d = abi.ConvDesc(dt, dt, b, h, w, c, c, oc, oh, ow, oc, k, stride, pad, 1, 1, abi.ACT["leaky"], 0.1, 1 if a.residual else 0, oc,
-                     abi.ACT["none"], 0.1, 1.0, 1.0, abi.ALGO["igemm"], 0)
+                     abi.ACT["none"], 0.1, 1.0, 1.0, abi.ALGO[a.conv_algo], 0)
     x = torch.randn(b, h, w, c, dtype=tdt, device="cuda")
-    wt = torch.randn(oc, k * k, c, dtype=tdt, device="cuda") * 0.05
+    # (random values in the packed layout of the algorithm: tap-major filters, or the 16 transformed filter matrices of Winograd F(2x2,3x3))
+    wt = torch.randn(int(L.msnh_hip_conv2d_packed_weight_elems(ctypes.byref(d), abi.ALGO[a.conv_algo])), dtype=tdt, device="cuda") * 0.05
+    ws_bytes = int(L.msnh_hip_conv2d_workspace_bytes(ctypes.byref(d), abi.ALGO[a.conv_algo]))
+    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device="cuda")
     y = torch.empty(b, oh, ow, oc, dtype=tdt, device="cuda")
     res = torch.randn(b, oh, ow, oc, dtype=tdt, device="cuda") if a.residual else None
     sc = torch.ones(oc, device="cuda")
@@ -183,7 +186,7 @@ def conv_shape_mode(a):
         return ctypes.c_void_p(t.data_ptr()) if t is not None else None
 
     def run():
-        abi.check(L.msnh_hip_conv2d(ctypes.byref(d), ptr(x), ptr(wt), ptr(sc), ptr(sh), ptr(res), ptr(y), None, 0, None))
+        abi.check(L.msnh_hip_conv2d(ctypes.byref(d), ptr(x), ptr(wt), ptr(sc), ptr(sh), ptr(res), ptr(y), ptr(ws), ws_bytes, None))
 
     torch.cuda.synchronize()
     if a.switches:
@@ -278,6 +281,9 @@ def main():
                          "(timing diagnostics library, include/msnh_hip_diag.h)")
     ap.add_argument("--residual", action="store_true", help="--conv-shape: with a fused residual add")
     ap.add_argument("--conv-dtype", default="f16", choices=["f16", "f32"])
+    ap.add_argument("--conv-algo", default="igemm", choices=["igemm", "winograd"],
+                    help="--conv-shape: the implicit GEMM (default) or the three-launch Winograd F(2x2,3x3) form (input transform, 16 GEMMs as one grouped launch "
+                         "with the tile given, output transform)")
     ap.add_argument("--workload", default="yolov3", choices=sorted(WORKLOADS))
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")

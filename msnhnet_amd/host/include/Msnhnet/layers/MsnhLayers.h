@@ -380,6 +380,8 @@ public:
     // class score, best class, cell number in scan order; any order) -- what the reference's scan keeps before sorting
     // (src/layers/MsnhYoloOutLayer.cpp:120-170).  Only after a result whose sort + NMS ran on the host.
     std::vector<float> lastCandidateRows(int image) const;
+    // one line for NetBuilder::getTimeDetail: where the sort + NMS of the last result ran and what the automatic placement has measured
+    std::string placementDetail() const;
     static std::vector<std::vector<int>> groupByClass(const std::vector<YoloBox> &bboxes);
     static void nmsClass(const std::vector<YoloBox> &bboxes, std::vector<int> &members, float nmsThresh);
 

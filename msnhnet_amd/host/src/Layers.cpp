@@ -1729,6 +1729,22 @@ std::vector<float> YoloOutLayer::lastCandidateRows(int image) const
     return std::vector<float>(rows, rows + n * 8);
 }
 
+std::string YoloOutLayer::placementDetail() const
+{
+    if (_lastSlot < 0) return "YoloOut NMS     : no result yet\n";
+    std::string d = std::string("YoloOut NMS     : last result on the ") + (lastOnDevice ? "device" : "host") + ", mode " +
+                    (_useSoftNms ? "soft (host)" : (deviceNms == 0 ? "host" : (deviceNms == 2 ? "device" : "auto"))) + ", " + std::to_string(_lastMaxCandidates) +
+                    " candidates in the fullest image";
+    if (deviceNms == 1 && !_useSoftNms)
+    {
+        d += fmt("; host stage between results %.3f ms", _hostInterval);
+        if (_trialLeft > 0 || _trialSeen > 0) d += fmt("; device trial running (%d of %d batches seen)", _trialSeen, kTrialBatches);
+        else if (_hostBound) d += "; a device trial won: thousands of candidates stay on the device";
+        else if (_hostBoundRuns < 0) d += "; a device trial lost: not repeated for a thousand batches";
+    }
+    return d + "\n";
+}
+
 void YoloOutLayer::forwardGPU(NetworkState &netState)
 {
     enqueueGather(netState.stream);

@@ -817,7 +817,9 @@ std::string NetBuilder::getTimeDetail()
         d += _net->layers[i]->getLayerName() + " : " + index3(i) + "     " + std::to_string(t).substr(0, 6) + " ms         " +
              std::to_string(static_cast<int>(t / total * 1000) / 10.f).substr(0, 4) + "%\n";
     }
-    d += "=========================================================\nMsnhnet inference time : " + std::to_string(total) + " ms";
+    d += "=========================================================\n";
+    if (!_net->layers.empty() && _net->layers.back()->type() == LayerType::YOLO_OUT) d += static_cast<YoloOutLayer *>(_net->layers.back())->placementDetail();
+    d += "Msnhnet inference time : " + std::to_string(total) + " ms";
     return d;
 }
 
@@ -845,7 +847,8 @@ static double opBytes(const Plan &plan, const PlanOp &op)
     const PlanTensor &out = plan.tensors[static_cast<size_t>(op.out)];
     double oe = static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4);
     for (int nx = op.chainNext; nx >= 0; nx = plan.ops[static_cast<size_t>(nx)].chainNext) oe += static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4);   // one launch, every pool's result
-    return static_cast<double>(in.elems()) * (in.dtype == MSNH_F16 ? 2 : 4) + oe + (op.in1 >= 0 ? oe : 0.0) + static_cast<double>(op.wDev.bytes());
+    return static_cast<double>(in.elems()) * (in.dtype == MSNH_F16 ? 2 : 4) + oe + (op.in1 >= 0 ? static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4) : 0.0) +
+           static_cast<double>(op.wDev.bytes());
 }
 
 float NetBuilder::profileOps(int kind, int reps, int *launches, double *flops, double *bytes)

@@ -501,6 +501,7 @@ def test_auto_nms_placement():
     m.enqueue(xd.data_ptr())
     b = m.fetch_yolo()
     assert not m.last_nms_on_device()        # enqueued beside another forward
+    assert "YoloOut NMS     : last result on the host, mode auto" in m.time_detail()          # the choice is on record in getTimeDetail
     c = m.fetch_yolo()
     for i in range(batch):
         for other in (a, b, c):
@@ -509,6 +510,7 @@ def test_auto_nms_placement():
     m.run_yolo(few)
     m.run_yolo(few)
     assert m.last_nms_on_device()
+    assert "YoloOut NMS     : last result on the device, mode auto, 0 candidates" in m.time_detail()
 
 
 def test_yolo_rows_copied_in_part():
