@@ -249,7 +249,8 @@ def conv_shape_mode(a):
     abi.check(L.msnh_hip_event_create(ctypes.byref(e0)))
     abi.check(L.msnh_hip_event_create(ctypes.byref(e1)))
     flops = 2.0 * b * oc * oh * ow * c * k * k
-    for tile in range(1, L.msnh_hip_conv2d_tile_count() + 1):
+    # (the one-launch Winograd form has no tile configurations: it is timed as tile 0)
+    for tile in ([0] if a.conv_algo == "winograd_fused" else range(1, L.msnh_hip_conv2d_tile_count() + 1)):
         d.tile = tile
         if not L.msnh_hip_conv2d_tile_supported(ctypes.byref(d), tile):
             continue
@@ -281,7 +282,7 @@ def main():
                          "(timing diagnostics library, include/msnh_hip_diag.h)")
     ap.add_argument("--residual", action="store_true", help="--conv-shape: with a fused residual add")
     ap.add_argument("--conv-dtype", default="f16", choices=["f16", "f32"])
-    ap.add_argument("--conv-algo", default="igemm", choices=["igemm", "winograd"],
+    ap.add_argument("--conv-algo", default="igemm", choices=["igemm", "winograd", "winograd_fused"],
                     help="--conv-shape: the implicit GEMM (default) or the three-launch Winograd F(2x2,3x3) form (input transform, 16 GEMMs as one grouped launch "
                          "with the tile given, output transform)")
     ap.add_argument("--workload", default="yolov3", choices=sorted(WORKLOADS))

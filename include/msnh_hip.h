@@ -62,8 +62,11 @@ enum msnh_conv_algo
     MSNH_CONV_IGEMM_SPLITK = 6,/* IGEMM with the K loop cut into up to 8 slices on separate workgroups, float32 partial sums in
                                   the workspace summed in slice order (deterministic); for launches with few output tiles.
                                   Same weight packing as IGEMM.  Never chosen by AUTO. */
-    MSNH_CONV_STEM_DOWN = 8    /* not an algorithm of msnh_hip_conv2d: the label of a launch of msnh_hip_conv_stem_down (first layer
+    MSNH_CONV_STEM_DOWN = 8,   /* not an algorithm of msnh_hip_conv2d: the label of a launch of msnh_hip_conv_stem_down (first layer
                                   and first stride-2 layer as one), so that plans and timing tables can name it */
+    MSNH_CONV_WINOGRAD_FUSED = 9 /* F(2x2,3x3) in one launch, float16 in and out, in_c a multiple of 16: input transform into LDS, the 16
+                                  products with all accumulators in registers, output transform in the epilogue; weights packed as
+                                  for MSNH_CONV_WINOGRAD, no workspace */
 };
 
 /* ------------------------------------------------------------------------------------------------

@@ -23,6 +23,9 @@ int convWinograd(const msnh_conv_desc *d, const void *x, const void *w, const fl
 size_t winogradWorkspaceBytes(const msnh_conv_desc *d);
 void   winogradPackWeights(const msnh_conv_desc *d, const float *oihw, void *packed);
 void   winogradGemmDesc(const msnh_conv_desc *d, msnh_conv_desc *gd);
+bool   winogradFusedOk(const msnh_conv_desc *d);
+int convWinogradFused(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift, const void *residual, void *y,
+                      hipStream_t st);
 bool   depthwise3x3Ok(const msnh_conv_desc *d, const void *x, const void *w, const void *y);
 int    convDepthwise3x3(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift, void *y, hipStream_t st);
 bool   stemMfmaOk(const msnh_conv_desc *d);
@@ -347,6 +350,7 @@ int msnh_hip_conv2d_tile_supported(const msnh_conv_desc *d, int tile)
     if (!d || validate(d) || tile < 0 || tile > igemmTileCount()) return 0;
     msnh_conv_desc t = *d;
     if (d->algo == MSNH_CONV_POINTWISE) return tile == 0 && pointwiseOk(d) ? 1 : 0;
+    if (d->algo == MSNH_CONV_WINOGRAD_FUSED) return tile == 0 && winogradFusedOk(d) ? 1 : 0;
     if (d->algo == MSNH_CONV_WINOGRAD)
     {
         // the tile applies to the 16 transformed-domain GEMMs
@@ -374,7 +378,7 @@ size_t msnh_hip_conv2d_packed_weight_elems(const msnh_conv_desc *d, int algo)
     if (!d) return 0;
     const size_t kk = static_cast<size_t>(d->ksize) * d->ksize;
     const size_t cinG = static_cast<size_t>(d->in_c / d->groups);
-    if (algo == MSNH_CONV_WINOGRAD) return static_cast<size_t>(16) * d->out_c * d->in_c;
+    if (algo == MSNH_CONV_WINOGRAD || algo == MSNH_CONV_WINOGRAD_FUSED) return static_cast<size_t>(16) * d->out_c * d->in_c;
     // float32 payload for the scalar kernel, followed (float16 plans) by the MFMA operand fragments
     if (algo == MSNH_CONV_STEM) return kk * d->in_c * d->out_c * (d->dtype == MSNH_F16 ? 2 : 1) + (stemMfmaOk(d) ? stemMfmaElems(d) : 0);
     return static_cast<size_t>(d->out_c) * kk * cinG;
@@ -418,6 +422,7 @@ int msnh_hip_conv2d_pack_weights(const msnh_conv_desc *d, int algo, const float 
         return 0;
     }
     case MSNH_CONV_WINOGRAD:
+    case MSNH_CONV_WINOGRAD_FUSED:
         MSNH_REQUIRE(winogradOk(d), "pack_weights: shape not supported by the Winograd kernel");
         winogradPackWeights(d, oihw, packed);
         return 0;
@@ -461,6 +466,8 @@ int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const
         return convIgemmWs(d, x, w, scale, shift, residual, y, st, false, workspace, workspace_bytes);
     case MSNH_CONV_POINTWISE:
         return convPointwise(d, x, w, scale, shift, residual, y, st);
+    case MSNH_CONV_WINOGRAD_FUSED:
+        return convWinogradFused(d, x, w, scale, shift, residual, y, st);
     case MSNH_CONV_WINOGRAD:
         MSNH_REQUIRE(winogradOk(d), "conv2d: shape not supported by the Winograd kernel");
         return convWinograd(d, x, w, scale, shift, residual, y, workspace, workspace_bytes, st);

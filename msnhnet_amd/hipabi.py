@@ -10,7 +10,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmsnh_hip.so")
 
 F32, F16 = 0, 1
 ACT = {"logistic": 0, "relu": 1, "relu6": 2, "leaky": 8, "swish": 16, "hardswish": 17, "mish": 18, "none": 22}
-ALGO = {"auto": 0, "direct": 1, "igemm": 2, "depthwise": 3, "winograd": 4, "stem": 5, "igemm_splitk": 6, "pointwise": 7}
+ALGO = {"auto": 0, "direct": 1, "igemm": 2, "depthwise": 3, "winograd": 4, "stem": 5, "igemm_splitk": 6, "pointwise": 7, "winograd_fused": 9}
 ALGO_NAME = {v: k for k, v in ALGO.items()}
 
 

@@ -270,6 +270,35 @@ def test_conv_winograd(b, c, h, w, oc, with_res):
         assert gu.rel_err(y2, ref) <= 3 * TOL[abi.F16]
 
 
+@pytest.mark.parametrize("b,c,h,w,oc", [(2, 16, 12, 10, 24), (1, 32, 19, 19, 64), (3, 48, 7, 9, 8), (1, 64, 38, 38, 128), (8, 256, 38, 38, 512), (2, 32, 21, 37, 136)])
+@pytest.mark.parametrize("with_res", [False, True])
+def test_conv_winograd_fused(b, c, h, w, oc, with_res):
+    """Winograd F(2x2,3x3) in one launch (input transform into LDS with packed float16 additions, 16 accumulator sets in registers,
+    output transform in the epilogue): same result as the direct form within the Winograd tolerance, odd sizes (partial tiles at the
+    right and bottom edge), tile runs that cross image seams, partial channel blocks, channel slices of wider tensors, full epilogue"""
+    import gpuutil as gu
+    rng = np.random.default_rng(b * 100 + c + 7)
+    x, wt = _case(rng, b, c, h, w, oc, 3)
+    res = rng.standard_normal((b, oc, h, w), dtype=np.float32) if with_res else None
+    scale = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    shift = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    x, wt = gu.round_f16(x), gu.round_f16(wt)
+    if with_res:
+        res = gu.round_f16(res)
+    kw = dict(dtype=abi.F16, stride=1, pad=1, scale=scale, shift=shift, act="leaky", residual=res, act2="leaky" if with_res else "none",
+              res_mul=2.0, out_mul=0.5, algo="winograd_fused", in_ld=c + 8, out_ld=oc + 8, res_ld=oc + 16 if with_res else None)
+    print("winograd fused", (b, c, h, w, oc), with_res, flush=True)
+    y, used = gu.conv2d(x, wt, **kw)
+    assert used == "winograd_fused"
+    ref = _ref(x, wt, 1, 1, 1, 1, scale, shift, "leaky", 0.1, res, "leaky" if with_res else "none", 2.0, 0.5)
+    e = gu.rel_err(y, ref)
+    print("error", e, flush=True)
+    # float16 transformed weights and two float16 roundings in the input transform: above the direct kernel's tolerance
+    assert e <= 4 * TOL[abi.F16]
+    y2, _ = gu.conv2d(x, wt, **kw)
+    assert np.array_equal(y, y2)
+
+
 SPLITK_CASES = [
     # b, c, h, w, oc, k, stride, pad, groups
     (1, 512, 7, 7, 512, 3, 1, 1, 1),

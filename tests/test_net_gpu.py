@@ -510,7 +510,7 @@ def test_auto_nms_placement():
     m.run_yolo(few)
     m.run_yolo(few)
     assert m.last_nms_on_device()
-    assert "YoloOut NMS     : last result on the device, mode auto, 0 candidates" in m.time_detail()
+    assert "YoloOut NMS     : last result on the device, mode auto, " in m.time_detail()
 
 
 def test_yolo_rows_copied_in_part():
