@@ -156,7 +156,6 @@ void convPatch8Kernel(IgemmArgs a)
         tapOk[j] = m;
     }
     const unsigned bRow0 = wn * TN + fragRow;         // patch row of this lane's pixel for tap (0,0), block 0
-    const unsigned zeroAddr = dumpOff + lane * 16;
 
     V fa[2][MB], fb[2][NB];
     auto readA = [&](unsigned stageOff, auto kbTag) {
@@ -165,13 +164,17 @@ void convPatch8Kernel(IgemmArgs a)
 #pragma unroll
         for (int i = 0; i < MB; ++i) fa[kb % 2][i] = *reinterpret_cast<const V *>(ap + i * 32 * ROWB);
     };
-    // B fragments of tap `tap` (row offset tapRow = ky*W + kx) from the patch stage at pOff; rows 32 apart share the swizzle
+    // B fragments of tap `tap` (row offset tapRow = ky*W + kx) from the patch stage at pOff; rows 32 apart share the swizzle.
+    // A lane whose tap lies outside the image reads zeros from the zero area at the address bits that select the bank (stages,
+    // patch and zero area start at multiples of 1 KiB), so it takes the bank its pixel would have taken: the lanes of a pass
+    // stay on distinct banks.  (With one fixed zero address per lane every pass with a border pixel was a two-way conflict.)
     auto readB = [&](unsigned pOff, int tap, unsigned tapRow, auto kbTag) {
         constexpr int kb = decltype(kbTag)::value;
         const unsigned row = bRow0 + tapRow;
         const unsigned sw = (row / 2) % KV;
         const unsigned addr = pOff + row * ROWB + (((2 * kb + kvBase) ^ sw) * 16);
         const unsigned bit = 1u << tap;
+        const unsigned zeroAddr = dumpOff + (addr & 255u);
 #pragma unroll
         for (int j = 0; j < NB; ++j)
         {
