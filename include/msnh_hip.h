@@ -64,9 +64,11 @@ enum msnh_conv_algo
                                   Same weight packing as IGEMM.  Never chosen by AUTO. */
     MSNH_CONV_STEM_DOWN = 8,   /* not an algorithm of msnh_hip_conv2d: the label of a launch of msnh_hip_conv_stem_down (first layer
                                   and first stride-2 layer as one), so that plans and timing tables can name it */
-    MSNH_CONV_WINOGRAD_FUSED = 9 /* F(2x2,3x3) in one launch, float16 in and out, in_c a multiple of 16: input transform into LDS, the 16
+    MSNH_CONV_WINOGRAD_FUSED = 9, /* F(2x2,3x3) in one launch, float16 in and out, in_c a multiple of 16: input transform into LDS, the 16
                                   products with all accumulators in registers, output transform in the epilogue; weights packed as
                                   for MSNH_CONV_WINOGRAD, no workspace */
+    MSNH_CONV_MBCONV = 10      /* not an algorithm of msnh_hip_conv2d: the label of a launch of msnh_hip_mbconv (1x1 expand, 3x3 depthwise
+                                  and 1x1 project convolution of an inverted-residual block as one) */
 };
 
 /* ------------------------------------------------------------------------------------------------
@@ -179,6 +181,38 @@ int msnh_hip_conv_stem_down_pack(const float *w1, int c2, const float *w2, void 
 int msnh_hip_conv_stem_down(int batch, int h, int w, const float *x, const void *packed1, const float *scale1, const float *shift1, int act1,
                             float act1_param, float mid_mul, int c2, const void *packed2, const float *scale2, const float *shift2, int act2,
                             float act2_param, float out_mul, void *y, int y_ld, msnh_stream_t s);
+
+/* The inverted-residual block of MobileNetV2 as one launch, float16 NHWC: 1x1 convolution in_c -> exp_c, 3x3 depthwise convolution
+ * (stride 1 or 2, pad 1) over the exp_c channels, 1x1 convolution exp_c -> out_c, each with its folded batch-norm and activation, then the
+ * block's residual add (three ConvolutionalLayer::forwardGPU calls, src/layers/MsnhConvolutionalLayer.cpp:984-1169, the second with
+ * groups == channels, inside a Res2BlockLayer / AddBlockLayer, src/layers/MsnhRes2BlockLayer.cpp forwardGPU; in the reference the
+ * widened tensors live in device memory between the calls, here they stay in LDS):
+ *   e = float16(mul1 * act1(scale1 * conv1x1(x) + shift1));   d = float16(mul2 * act2(scale2 * dw3x3(e) + shift2));
+ *   y = out_mul * act4(act3(scale3 * conv1x1(d) + shift3) + res_mul * residual)      (without a residual: out_mul * act3(...))
+ * scale2 must undo mul1 and scale3 must undo mul2 (the power-of-two scales of the two widened tensors).
+ * Limits: in_c, out_c <= 96, all channel counts and pixel strides multiples of 8; _supported is a pure host function. */
+typedef struct msnh_mbconv_desc {
+    int batch, in_h, in_w, in_c, in_ld;
+    int exp_c, stride;
+    int out_c, out_h, out_w, out_ld;
+    int act1, act2, act3, act4;
+    float act1_param, act2_param, act3_param, act4_param;
+    int has_residual, res_ld;
+    float mul1, mul2, out_mul, res_mul;
+} msnh_mbconv_desc;
+int msnh_hip_mbconv_supported(const msnh_mbconv_desc *d);
+/* Bytes of the packed weights (0: block not supported). */
+size_t msnh_hip_mbconv_packed_bytes(const msnh_mbconv_desc *d);
+/* w_expand: [exp_c][in_c], w_dw: [exp_c][3][3], w_project: [out_c][exp_c] float32 in `.msnhbin` order; scale1 / shift1 / scale2 / shift2:
+ * float32[exp_c] or NULL (1 / 0).  `packed` is host memory of msnh_hip_mbconv_packed_bytes() bytes; upload it afterwards.  The packed record
+ * depends on the channel counts, act1, act2, mul1 and mul2 of the descriptor (the scales of the widened tensors are folded into the first
+ * two affines where the activation allows it): pack with the descriptor the launch will use. */
+int msnh_hip_mbconv_pack(const msnh_mbconv_desc *d, const float *w_expand, const float *scale1, const float *shift1, const float *w_dw,
+                         const float *scale2, const float *shift2, const float *w_project, void *packed);
+/* x: NHWC float16 [batch][in_h][in_w] with pixel stride in_ld; scale3 / shift3: float32[out_c] on the device or NULL; residual: NHWC float16
+ * with the output's geometry and pixel stride res_ld, or NULL; y: NHWC float16 with pixel stride out_ld. */
+int msnh_hip_mbconv(const msnh_mbconv_desc *d, const void *x, const void *packed, const float *scale3, const float *shift3, const void *residual,
+                    void *y, msnh_stream_t s);
 
 /* ------------------------------------------------------------------------------------------------
  * Element-wise / bandwidth-bound layers (all NHWC, any ld).

@@ -76,6 +76,8 @@ struct PlanOp
     int  chainHead = -1;                    // MAXPOOL: >= 0 = this pool's result is written by the launch of op chainHead (a chain of stride-1 pools in one launch)
     int  chainNext = -1;                    // MAXPOOL at the head or inside such a chain: the op whose pool follows
     int  stemOp = -1;                       // CONV 3x3 stride 2: the (dead) first-layer op computed in front of it by the same launch (Plan::fuse c)
+    int  mbExpand = -1, mbDw = -1;          // CONV 1x1 closing an inverted-residual block: the (dead) 1x1 expand and 3x3 depthwise ops computed in front of
+                                            // it by the same launch (Plan::fuse d, msnh_hip_mbconv)
 
     // YOLO_DECODE
     std::array<float, 6> anchors{};
@@ -101,6 +103,7 @@ public:
     std::vector<size_t> yoloHeadOps;        // sparseYolo: the heads' decode ops in cell order when one launch (issued at the last of them in
                                             // op order) can decode them all; empty = one launch pair per head
     void findYoloHeads();                   // fills yoloHeadOps; call once the heads' cell numbers are assigned
+    bool fuseMbconv = true;                 // float16: 1x1 expand -> 3x3 depthwise -> 1x1 project as one launch where msnh_hip_mbconv takes the block
     bool fuseStemDown = true;               // float16: first layer + first stride-2 layer as one launch where msnh_hip_conv_stem_down takes the pair
     bool preferWinograd = false;            // 3x3 stride-1 float16 convs take the Winograd path where the kernel accepts the shape
     std::vector<PlanTensor> tensors;

@@ -406,6 +406,7 @@ void NetBuilder::finalizePlan()
     const int dtype = BaseLayer::useFp16 ? MSNH_F16 : MSNH_F32;
     std::unique_ptr<Plan> plan = lowerNetwork(dtype);
     plan->fuseStemDown = std::getenv("MSNH_NO_STEM_DOWN") == nullptr;
+    plan->fuseMbconv = std::getenv("MSNH_NO_MBCONV") == nullptr;
     plan->fuse();
     plan->chainMaxPools();
     plan->aliasConcats();
@@ -890,7 +891,7 @@ std::string NetBuilder::profileEachOp(int reps, std::vector<double> *values)
     if (!_planReady) MSNH_THROW("weights are not loaded");
     Plan &plan = *_net->plan;
     static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode", "pad", "slice", "bilinear", "softmax", "col2im"};
-    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk", "pointwise", "stem+down"};
+    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk", "pointwise", "stem+down", "winograd_fused", "mbconv"};
     msnh_event_t e0 = nullptr, e1 = nullptr;
     MSNH_DEV(msnh_hip_event_create(&e0));
     MSNH_DEV(msnh_hip_event_create(&e1));

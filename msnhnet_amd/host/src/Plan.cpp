@@ -214,6 +214,50 @@ void Plan::fuse()
                 break;
             }
         }
+    // (d) float16: 1x1 convolution -> 3x3 depthwise convolution -> 1x1 convolution, each the only consumer of the one before (the
+    // inverted-residual block of MobileNetV2; the closing convolution may already carry the block's residual add from (b)): one launch,
+    // the two widened tensors stay on the chip.  They keep their places in the tensor list: their calibrated scales are the scales of
+    // the values in LDS.
+    if (computeDtype == MSNH_F16 && fuseMbconv)
+        for (size_t i = 0; i < ops.size(); ++i)
+        {
+            PlanOp &proj = ops[i];
+            if (proj.dead || proj.kind != PlanOp::CONV || proj.ksize != 1 || proj.stride != 1 || proj.pad != 0 || proj.groups != 1 || proj.stemOp >= 0) continue;
+            const auto inner = [&](int t) {
+                const PlanTensor &pt = tensors[static_cast<size_t>(t)];
+                return !pt.pinned && !pt.persistent && !pt.external && pt.parent < 0 && pt.dtype == MSNH_F16 && pt.layout == PlanTensor::NHWC && consumerCount(t) == 1;
+            };
+            const int pd = producerOf(proj.in0);
+            if (pd < 0 || !inner(proj.in0)) continue;
+            PlanOp &dw = ops[static_cast<size_t>(pd)];
+            const PlanTensor &wide = tensors[static_cast<size_t>(dw.in0)];
+            if (dw.kind != PlanOp::CONV || dw.ksize != 3 || dw.pad != 1 || dw.dilation != 1 || (dw.stride != 1 && dw.stride != 2) || dw.in1 >= 0 || dw.stemOp >= 0 ||
+                dw.groups != wide.c || tensors[static_cast<size_t>(dw.out)].c != wide.c)
+                continue;
+            const int pe = producerOf(dw.in0);
+            if (pe < 0 || !inner(dw.in0)) continue;
+            PlanOp &ex = ops[static_cast<size_t>(pe)];
+            if (ex.kind != PlanOp::CONV || ex.ksize != 1 || ex.stride != 1 || ex.pad != 0 || ex.groups != 1 || ex.in1 >= 0 || ex.stemOp >= 0 || ex.mbExpand >= 0) continue;
+            const PlanTensor &in = tensors[static_cast<size_t>(ex.in0)];
+            const PlanTensor &out = tensors[static_cast<size_t>(proj.out)];
+            if (in.layout != PlanTensor::NHWC || in.dtype != MSNH_F16 || out.dtype != MSNH_F16 || out.layout != PlanTensor::NHWC) continue;
+            // the residual must exist when the fused launch runs, which is where the closing convolution stands: it does
+            msnh_mbconv_desc d;
+            std::memset(&d, 0, sizeof(d));
+            const auto up8 = [](int c) { return (c + 7) / 8 * 8; };
+            d.batch = in.n; d.in_h = in.h; d.in_w = in.w; d.in_c = in.c; d.in_ld = up8(in.c);
+            d.exp_c = wide.c; d.stride = dw.stride;
+            d.out_c = out.c; d.out_h = out.h; d.out_w = out.w; d.out_ld = up8(out.c);
+            d.act1 = static_cast<int>(ex.act); d.act2 = static_cast<int>(dw.act); d.act3 = static_cast<int>(proj.act); d.act4 = static_cast<int>(proj.act2);
+            d.has_residual = proj.in1 >= 0 ? 1 : 0; d.res_ld = up8(out.c);
+            d.mul1 = d.mul2 = d.out_mul = d.res_mul = 1.f;
+            if (!msnh_hip_mbconv_supported(&d)) continue;
+            proj.mbExpand = pe;
+            proj.mbDw = pd;
+            proj.in0 = ex.in0;
+            ex.dead = true;
+            dw.dead = true;
+        }
 }
 
 // ---- pass 1b: stride-1 max-pools over one tensor (SPP blocks: 5, 9, 13) ---------------------------------------------
@@ -382,7 +426,7 @@ uint64_t Plan::structureHash() const
     for (const PlanOp &op : ops)
         os << static_cast<int>(op.kind) << ' ' << op.in0 << ' ' << op.in1 << ' ' << op.out << ' ' << op.dead << ' ' << op.layerIndex << ' ' << op.ksize << ' ' << op.stride << ' '
            << op.pad << ' ' << op.dilation << ' ' << op.groups << ' ' << static_cast<int>(op.act) << ' ' << static_cast<int>(op.act2) << ' ' << op.in1Sign << ' ' << (op.src2 != nullptr)
-           << ' ' << op.dstChanOffset << ' ' << op.stemOp << ' ' << op.chainHead << ';';
+           << ' ' << op.dstChanOffset << ' ' << op.stemOp << ' ' << op.chainHead << ' ' << op.mbExpand << ';';
     const std::string text = os.str();
     return PackFile::hash(text.data(), text.size());
 }
@@ -520,6 +564,50 @@ static msnh_conv_desc convDesc(const Plan &plan, const PlanOp &op)
     return d;
 }
 
+static msnh_mbconv_desc mbconvDesc(const Plan &plan, const PlanOp &op)
+{
+    const PlanOp &ex = plan.ops[static_cast<size_t>(op.mbExpand)];
+    const PlanOp &dw = plan.ops[static_cast<size_t>(op.mbDw)];
+    const PlanTensor &in = plan.tensors[static_cast<size_t>(op.in0)];
+    const PlanTensor &wide = plan.tensors[static_cast<size_t>(ex.out)];
+    const PlanTensor &out = plan.tensors[static_cast<size_t>(op.out)];
+    msnh_mbconv_desc d;
+    std::memset(&d, 0, sizeof(d));
+    d.batch = in.n; d.in_h = in.h; d.in_w = in.w; d.in_c = in.c; d.in_ld = plan.ld(op.in0);
+    d.exp_c = wide.c; d.stride = dw.stride;
+    d.out_c = out.c; d.out_h = out.h; d.out_w = out.w; d.out_ld = plan.ld(op.out);
+    d.act1 = static_cast<int>(ex.act); d.act2 = static_cast<int>(dw.act); d.act3 = static_cast<int>(op.act); d.act4 = static_cast<int>(op.act2);
+    d.act1_param = ex.actParam; d.act2_param = dw.actParam; d.act3_param = op.actParam; d.act4_param = op.act2Param;
+    d.has_residual = op.in1 >= 0 ? 1 : 0;
+    d.res_ld = op.in1 >= 0 ? plan.ld(op.in1) : out.c;
+    d.mul1 = 1.f / plan.mulOf(ex.out);
+    d.mul2 = 1.f / plan.mulOf(dw.out);
+    d.out_mul = 1.f / plan.mulOf(op.out);
+    d.res_mul = op.in1 >= 0 ? op.in1Sign * plan.mulOf(op.in1) : 1.f;
+    return d;
+}
+
+// folded affine of a convolution op (its own bias / batch-norm, a batch-norm layer fused behind it, the power-of-two scale of its input);
+// empty vectors mean 1 and 0
+static void foldAffine(const PlanOp &o, int channels, float inMul, std::vector<float> &scale, std::vector<float> &shift)
+{
+    scale.clear(); shift.clear();
+    o.src->foldedAffine(scale, shift);
+    if (o.src2)
+    {
+        std::vector<float> s2, h2;
+        o.src2->foldedAffine(s2, h2);
+        if (scale.empty()) scale.assign(static_cast<size_t>(channels), 1.f);
+        if (shift.empty()) shift.assign(static_cast<size_t>(channels), 0.f);
+        for (size_t c = 0; c < static_cast<size_t>(channels); ++c) { scale[c] = s2[c] * scale[c]; shift[c] = s2[c] * shift[c] + h2[c]; }
+    }
+    if (inMul != 1.f)
+    {
+        if (scale.empty()) scale.assign(static_cast<size_t>(channels), 1.f);
+        for (float &v : scale) v *= inMul;
+    }
+}
+
 static std::vector<uint16_t> toHalf(const std::vector<float> &v);
 
 void Plan::prepareWeights(PackFile *from, PackFile *to)
@@ -566,6 +654,34 @@ void Plan::prepareWeights(PackFile *from, PackFile *to)
             op.algo = MSNH_CONV_STEM_DOWN;
             const PlanTensor &img = tensors[static_cast<size_t>(op.in0)];
             op.flops = 2.0 * img.n * (static_cast<double>(mid.c) * mid.h * mid.w * img.c * 9 + static_cast<double>(out.c) * out.h * out.w * mid.c * 9);
+            continue;
+        }
+        if (op.kind == PlanOp::CONV && op.mbExpand >= 0)
+        {
+            // the fused inverted-residual block: both 1x1 filters in fragment order, the depthwise taps and the first two affines in one
+            // packed record per 64 widened channels; each stage's scale undoes the power-of-two scale of the tensor it reads
+            const PlanOp &ex = ops[static_cast<size_t>(op.mbExpand)];
+            const PlanOp &dw = ops[static_cast<size_t>(op.mbDw)];
+            const msnh_mbconv_desc d = mbconvDesc(*this, op);
+            const std::vector<float> &w1 = ex.src->kernelWeights(), &w2 = dw.src->kernelWeights(), &w3 = op.src->kernelWeights();
+            if (w1.size() != static_cast<size_t>(d.exp_c) * d.in_c || w2.size() != static_cast<size_t>(d.exp_c) * 9 || w3.size() != static_cast<size_t>(d.out_c) * d.exp_c)
+                MSNH_THROW("conv weights are not loaded (" + op.name + ")");
+            std::vector<float> s1, h1, s2, h2, s3, h3;
+            foldAffine(ex, d.exp_c, mulOf(op.in0), s1, h1);
+            foldAffine(dw, d.exp_c, mulOf(ex.out), s2, h2);
+            foldAffine(op, d.out_c, mulOf(dw.out), s3, h3);
+            std::vector<unsigned char> packed(msnh_hip_mbconv_packed_bytes(&d));
+            if (packed.empty()) MSNH_THROW("mbconv: the block is not supported after placement (" + op.name + ")");
+            MSNH_DEV(msnh_hip_mbconv_pack(&d, w1.data(), s1.empty() ? nullptr : s1.data(), h1.empty() ? nullptr : h1.data(), w2.data(), s2.empty() ? nullptr : s2.data(),
+                                          h2.empty() ? nullptr : h2.data(), w3.data(), packed.data()));
+            op.wDev.upload(packed.data(), packed.size());
+            if (!s3.empty()) op.scaleDev.upload(s3.data(), s3.size() * sizeof(float));
+            if (!h3.empty()) op.shiftDev.upload(h3.data(), h3.size() * sizeof(float));
+            op.algo = MSNH_CONV_MBCONV;
+            const PlanTensor &wide = tensors[static_cast<size_t>(ex.out)];
+            const PlanTensor &narrow = tensors[static_cast<size_t>(dw.out)];
+            op.flops = 2.0 * d.batch * (static_cast<double>(wide.h) * wide.w * d.exp_c * d.in_c + static_cast<double>(narrow.h) * narrow.w * d.exp_c * 9 +
+                                        static_cast<double>(d.out_h) * d.out_w * d.out_c * d.exp_c);
             continue;
         }
         if (op.kind == PlanOp::CONV)
@@ -982,6 +1098,13 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
                                              op.shiftDev.as<float>(), static_cast<int>(op.act), op.actParam, 1.f / mulOf(op.out), ptr(op.out), ld(op.out), s));
             break;
         }
+        if (op.mbExpand >= 0)
+        {
+            const msnh_mbconv_desc md = mbconvDesc(*this, op);
+            if (op.wDev.bytes() != msnh_hip_mbconv_packed_bytes(&md)) MSNH_THROW("mbconv weights on the device do not fit this launch (" + op.name + ")");
+            MSNH_DEV(msnh_hip_mbconv(&md, ptr(op.in0), op.wDev.ptr(), op.scaleDev.as<float>(), op.shiftDev.as<float>(), op.in1 >= 0 ? ptr(op.in1) : nullptr, ptr(op.out), s));
+            break;
+        }
         const msnh_conv_desc d = convDesc(*this, op);
         if (op.wDev.bytes() != msnh_hip_conv2d_packed_weight_elems(&d, op.algo) * (d.dtype == MSNH_F16 ? 2u : 4u))
             MSNH_THROW("conv weights on the device are not packed for the algorithm of this launch (" + op.name + ")");
@@ -1157,7 +1280,7 @@ void Plan::exportTensor(int t, std::vector<float> &dst, msnh_stream_t s)
 std::string Plan::describe() const
 {
     static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode", "pad", "slice", "bilinear", "softmax", "col2im"};
-    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk", "pointwise", "stem+down"};
+    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk", "pointwise", "stem+down", "winograd_fused", "mbconv"};
     std::ostringstream os;
     os << "plan: " << liveOps() << " launches, " << tensors.size() << " tensors, arena " << _arena.bytes() / (1024.0 * 1024.0) << " MiB, dtype "
        << (computeDtype == MSNH_F16 ? "f16" : "f32") << "\n";
