@@ -1,8 +1,8 @@
 """GPU parity of msnh_hip_mbconv (1x1 expand, 3x3 depthwise, 1x1 project of an inverted-residual block as one launch) against the
 three layers composed from the plain-C oracle convolution, with the two widened tensors rounded to float16 where the launch rounds them.
 
-Tolerance: 4e-3 of max|ref| -- the single-layer float16 bar (2e-3) twice, since a widened value that sits on a float16 rounding
-boundary may round the other way on the device (float32 summation order) and the projection then sums up to 576 of them."""
+Tolerance: 1e-3 of max|ref| (measured 2-4e-4) -- half the single-layer float16 bar: a widened value that sits on a float16 rounding
+boundary may round the other way on the device (float32 summation order), and the projection sums up to 576 of them."""
 import ctypes
 
 import numpy as np
@@ -97,7 +97,7 @@ def test_mbconv_block(case):
     ref = _reference(*args)
     e = gu.rel_err(y, ref)
     print("error", e, flush=True)
-    assert e <= 4e-3
+    assert e <= 1e-3
     assert np.array_equal(y, run_mbconv(*args, in_ld=cin + 8, out_ld=cout + 8, res_ld=cout + 16))
 
 
@@ -121,7 +121,7 @@ def test_mbconv_activations_and_limits():
         args = (x, we, wd, wp, one, zero + 0.3, one, zero - 0.1, s3, h3, 1, acts, 1.0, 1.0, 1.0, res, 1.0)
         e = gu.rel_err(run_mbconv(*args), _reference(*args))
         print("error", e, flush=True)
-        assert e <= 4e-3
+        assert e <= 1e-3
     bad = [dict(in_c=104), dict(out_c=104), dict(in_c=12), dict(stride=3), dict(out_h=5), dict(in_ld=20)]
     for change in bad:
         d = abi.MbconvDesc(1, 14, 14, 32, 32, 192, 1, 32, 14, 14, 32, abi.ACT["relu6"], abi.ACT["relu6"], abi.ACT["none"], abi.ACT["none"],

@@ -574,6 +574,35 @@ def test_spp_maxpools_run_as_a_chain():
             netapi.set_tune_cache(False)
 
 
+def test_inverted_residual_blocks_run_as_one_launch():
+    """float16 MobileNetV2: every expand -> depthwise -> project block whose channel counts the kernel takes is one launch
+    (msnh_hip_mbconv); the block's residual add rides in it.  Against the three-launch plan (MSNH_NO_MBCONV) the logits agree to
+    float16 accuracy (the widened tensors are rounded to float16 at the same points with the same scales; only the float32 summation
+    order of the projection differs), and the per-layer / final parity tests of mobilenetv2 run through the fused plan."""
+    for batch, size in ((3, 224),):                             # (the 7x7 average pool needs the full-size feature map; tiles cut by image edges: tests/test_mbconv_gpu.py)
+        net, binp, g = nu.model("mobilenetv2", batch, size, seed=3)
+        x = zoo.seeded_input(batch, 3, size, size, seed=4)
+        m = netapi.Net(net, binp, fp16=True)
+        detail = m.plan_detail()
+        fused_lines = [ln for ln in detail.splitlines() if "conv[mbconv" in ln]
+        assert len(fused_lines) == 12, detail                   # 17 blocks: the first has no expand, four have 160 / 320 channels
+        assert sum("+res" in ln for ln in fused_lines) == 8, fused_lines
+        launches = int(detail.split(" launches")[0].split()[-1])
+        fused = m.run_classify(x)
+        os.environ["MSNH_NO_MBCONV"] = "1"
+        try:
+            m2 = netapi.Net(net, binp, fp16=True)
+        finally:
+            del os.environ["MSNH_NO_MBCONV"]
+        assert "mbconv" not in m2.plan_detail()
+        assert int(m2.plan_detail().split(" launches")[0].split()[-1]) == launches + 24
+        apart = m2.run_classify(x)
+        err = np.abs(fused - apart).max() / np.abs(apart).max()
+        print("fused against three launches:", size, err, flush=True)
+        assert err <= 2e-3
+        assert np.array_equal(fused, m.run_classify(x))
+
+
 def test_image_in_boxes_out():
     """8-bit images of different shapes -> device letterbox -> forward -> boxes in original-image pixels: equals the
     float path fed with the restatement's letterbox, followed by the restatement's rescale."""
