@@ -269,12 +269,64 @@ def conv_shape_mode(a):
     L.msnh_hip_event_destroy(e1)
 
 
+def mbconv_shape_mode(a):
+    """One inverted-residual block (1x1 expand, 3x3 depthwise, 1x1 project, relu6 twice, optional residual) through msnh_hip_mbconv,
+    --reps launches back to back after one warm-up launch.  Random inputs and weights; results are not checked here (tests/test_mbconv_gpu.py
+    does that)."""
+    import ctypes
+    import time
+
+    import numpy as np
+    import torch
+
+    from msnhnet_amd import hipabi as abi
+    b, cin, h, w, cexp, cout, stride, with_res = (int(v) for v in a.mbconv_shape.split(","))
+    L = abi.lib()
+    abi.check(L.msnh_hip_init(0))
+    oh, ow = (h - 1) // stride + 1, (w - 1) // stride + 1
+    d = abi.MbconvDesc(b, h, w, cin, cin, cexp, stride, cout, oh, ow, cout, abi.ACT["relu6"], abi.ACT["relu6"], abi.ACT["none"], abi.ACT["none"],
+                       0.1, 0.1, 0.1, 0.1, 1 if with_res else 0, cout, 1.0, 1.0, 1.0, 1.0)
+    if not L.msnh_hip_mbconv_supported(ctypes.byref(d)):
+        sys.exit("msnh_hip_mbconv does not take this block")
+    rng = np.random.default_rng(a.seed)
+    we = rng.standard_normal((cexp, cin), dtype=np.float32) * np.float32(0.2)
+    wd = rng.standard_normal((cexp, 9), dtype=np.float32) * np.float32(0.3)
+    wp = rng.standard_normal((cout, cexp), dtype=np.float32) * np.float32(0.1)
+    packed = np.zeros(L.msnh_hip_mbconv_packed_bytes(ctypes.byref(d)), np.uint8)
+    hp = lambda arr: arr.ctypes.data_as(ctypes.c_void_p)
+    abi.check(L.msnh_hip_mbconv_pack(ctypes.byref(d), hp(we), None, None, hp(wd), None, None, hp(wp), hp(packed)))
+    x = torch.randn(b, h, w, cin, dtype=torch.float16, device="cuda")
+    y = torch.empty(b, oh, ow, cout, dtype=torch.float16, device="cuda")
+    r = torch.randn(b, oh, ow, cout, dtype=torch.float16, device="cuda") if with_res else None
+    pd = torch.from_numpy(packed).cuda()
+    dp = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    torch.cuda.synchronize()
+
+    def run():
+        abi.check(L.msnh_hip_mbconv(ctypes.byref(d), dp(x), dp(pd), None, None, dp(r), dp(y), None))
+
+    run()
+    abi.check(L.msnh_hip_stream_sync(None))
+    t0 = time.perf_counter()
+    for _ in range(a.reps):
+        run()
+    abi.check(L.msnh_hip_stream_sync(None))
+    us = (time.perf_counter() - t0) / a.reps * 1e6
+    flops = 2.0 * b * (h * w * cexp * cin + oh * ow * cexp * 9 + oh * ow * cout * cexp)
+    nbytes = 2.0 * b * (h * w * cin + oh * ow * cout * (2 if with_res else 1))
+    print(f"mbconv {a.mbconv_shape}: {a.reps} launches, {us:.2f} us per launch back to back (host clock), {flops / us * 1e-6:.1f} TFLOP/s, "
+          f"{nbytes / us * 1e-3:.0f} GB/s on input + output" + (" + residual" if with_res else ""))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--conv-shape", default=None, help="b,c,h,w,oc,k,stride: time this one convolution shape instead of a workload")
+    ap.add_argument("--mbconv-shape", default=None,
+                    help="b,in_c,h,w,exp_c,out_c,stride,residual(0|1): launch this one inverted-residual block (msnh_hip_mbconv) --reps times and "
+                         "print the time per launch (the form to put behind rocprofv3 --pmc)")
     ap.add_argument("--tile", type=int, default=0, help="--conv-shape: launch only this tile configuration, --reps times, untimed")
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--switches", action="store_true",
@@ -315,6 +367,9 @@ def main():
         sys.exit("bench.py: no GPU visible; the hot path has no CPU fallback")
     if a.conv_shape:
         conv_shape_mode(a)
+        return
+    if a.mbconv_shape:
+        mbconv_shape_mode(a)
         return
 
     dtype, batch, size = WORKLOADS[a.workload]

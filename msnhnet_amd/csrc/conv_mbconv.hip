@@ -413,7 +413,7 @@ int msnh_hip_mbconv(const msnh_mbconv_desc *d, const void *x, const void *packed
     a.cap1 = 6.f * d->mul1; a.cap2 = 6.f * d->mul2;
     const size_t lds = mbLdsBytes(d);
     const unsigned blocks = static_cast<unsigned>((total + 7) / 8 * 8);
-    hipStream_t st = static_cast<hipStream_t>(s);
+    hipStream_t st = resolveStream(s);
     if (d->stride == 1)
     {
         static bool raised = false;
