@@ -67,6 +67,8 @@ enum msnh_conv_algo
     MSNH_CONV_WINOGRAD_FUSED = 9, /* F(2x2,3x3) in one launch, float16 in and out, in_c a multiple of 16: input transform into LDS, the 16
                                   products with all accumulators in registers, output transform in the epilogue; weights packed as
                                   for MSNH_CONV_WINOGRAD, no workspace */
+    MSNH_CONV_IGEMM_TAIL = 11, /* not an algorithm of msnh_hip_conv2d: the label of a launch of msnh_hip_conv2d_tail (a convolution and the 1x1
+                                  convolution that reads its result) */
     MSNH_CONV_MBCONV = 10      /* not an algorithm of msnh_hip_conv2d: the label of a launch of msnh_hip_mbconv (1x1 expand, 3x3 depthwise
                                   and 1x1 project convolution of an inverted-residual block as one) */
 };
@@ -167,6 +169,28 @@ size_t msnh_hip_conv2d_workspace_bytes(const msnh_conv_desc *d, int algo);
  * residual: NHWC d->dtype with pixel stride res_ld, or NULL; y: NHWC d->out_dtype with pixel stride out_ld. */
 int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
                     const void *residual, void *y, void *workspace, size_t workspace_bytes, msnh_stream_t s);
+
+/* A convolution and the 1x1 stride-1 pad-0 convolution that reads its result, as one launch, float16: the 3x3 convolution that closes a
+ * Darknet residual block together with the 1x1 convolution that opens the next block (two ConvolutionalLayer::forwardGPU calls,
+ * src/layers/MsnhConvolutionalLayer.cpp:984-1169, inside ResBlockLayer::forwardGPU, src/layers/MsnhResBlockLayer.cpp:215-302, with the
+ * block's output read back from device memory between them).  d describes the first convolution as for msnh_hip_conv2d (algo MSNH_CONV_IGEMM,
+ * ungrouped, out_c <= 256 and a multiple of 8; d->tile: 0 or one of the tiles that carry a tail, the last msnh_hip_conv2d_tile_count() -
+ * msnh_hip_conv2d_tail_tile_first() + 1 ones); y is written as by msnh_hip_conv2d unless t->write_y is 0 (nobody else reads it).  Then
+ * z = out_mul * act(scale2 * (w2 . y) + shift2) with y as rounded to float16, so that z carries the bits a separate launch reading y
+ * would compute in the same k order.  w2: the 1x1 filters packed as for MSNH_CONV_IGEMM, [t->out_c][d->out_c] float16; t->out_c <= 128
+ * and a multiple of 8; z: NHWC float16 with pixel stride t->out_ld (a multiple of 8), 16-byte aligned.  _supported: pure host function. */
+typedef struct msnh_conv_tail_desc
+{
+    int   out_c, out_ld;
+    int   act;          /* msnh_act of the 1x1 convolution */
+    float act_param;
+    float out_mul;
+    int   write_y;
+} msnh_conv_tail_desc;
+int msnh_hip_conv2d_tail_tile_first(void);
+int msnh_hip_conv2d_tail_supported(const msnh_conv_desc *d, const msnh_conv_tail_desc *t, int tile);
+int msnh_hip_conv2d_tail(const msnh_conv_desc *d, const msnh_conv_tail_desc *t, const void *x, const void *w, const float *scale, const float *shift,
+                         const void *residual, void *y, const void *w2, const float *scale2, const float *shift2, void *z, msnh_stream_t s);
 
 /* The first two convolutions of the Darknet-53 / CSPDarknet-53 trunks as one launch, float16: a 3x3 stride-1 pad-1 convolution with 32
  * filters over the 3-channel NCHW float32 network input, then a 3x3 stride-2 pad-1 convolution with c2 = 32 / 64 / 128 filters

@@ -11,6 +11,9 @@ namespace msnh {
 
 int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
               const void *residual, void *y, hipStream_t st, bool dryRun);
+int convIgemmTail(const msnh_conv_desc *d, const msnh_conv_tail_desc *tail, const void *x, const void *w, const float *scale, const float *shift,
+                  const void *residual, void *y, const void *w2, const float *scale2, const float *shift2, void *z, hipStream_t st, bool dryRun);
+int igemmTailTileFirst();
 int convIgemmWs(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
                 const void *residual, void *y, hipStream_t st, bool dryRun, void *splitWs, size_t splitWsBytes);
 size_t igemmSplitKWorkspaceBytes(const msnh_conv_desc *d);
@@ -361,6 +364,38 @@ int msnh_hip_conv2d_tile_supported(const msnh_conv_desc *d, int tile)
     if (tile == 0 && d->algo != MSNH_CONV_IGEMM_SPLITK) return 1;
     t.tile = tile;
     return convIgemm(&t, d, d, nullptr, nullptr, nullptr, &t, nullptr, true) == 0 ? 1 : 0;      // pointers unused in a dry run
+}
+
+int msnh_hip_conv2d_tail_tile_first(void) { return igemmTailTileFirst(); }
+
+static bool tailDescOk(const msnh_conv_desc *d, const msnh_conv_tail_desc *t)
+{
+    return d && t && !validate(d) && igemmOk(d) && d->dtype == MSNH_F16 && d->out_dtype == MSNH_F16 && d->groups == 1 &&
+           (d->algo == MSNH_CONV_IGEMM || d->algo == MSNH_CONV_AUTO) && d->out_c % 8 == 0 && d->out_ld % 8 == 0 && (!d->has_residual || d->res_ld % 8 == 0) &&
+           t->out_c > 0 && t->out_c % 8 == 0 && t->out_ld >= t->out_c && t->out_ld % 8 == 0 && actOk(t->act);
+}
+
+int msnh_hip_conv2d_tail_supported(const msnh_conv_desc *d, const msnh_conv_tail_desc *t, int tile)
+{
+    if (!tailDescOk(d, t) || tile < 0 || tile > igemmTileCount() || (tile != 0 && tile < igemmTailTileFirst())) return 0;
+    msnh_conv_desc c = *d;
+    c.algo = MSNH_CONV_IGEMM;
+    c.tile = tile;
+    return convIgemmTail(&c, t, d, d, nullptr, nullptr, d, &c, d, nullptr, nullptr, &c, nullptr, true) == 0 ? 1 : 0;      // pointers unused in a dry run
+}
+
+int msnh_hip_conv2d_tail(const msnh_conv_desc *d, const msnh_conv_tail_desc *t, const void *x, const void *w, const float *scale, const float *shift,
+                         const void *residual, void *y, const void *w2, const float *scale2, const float *shift2, void *z, msnh_stream_t s)
+{
+    MSNH_REQUIRE(tailDescOk(d, t), "conv2d_tail: a float16 ungrouped IGEMM convolution followed by a 1x1 convolution, channel counts and pixel strides multiples of 8");
+    MSNH_REQUIRE(x && w && y && w2 && z, "conv2d_tail: NULL tensor pointer");
+    MSNH_REQUIRE(!d->has_residual || residual, "conv2d_tail: has_residual without a residual tensor");
+    MSNH_REQUIRE(d->in_ld >= d->in_c, "conv2d_tail: in_ld < in_c");
+    MSNH_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
+                 (!d->has_residual || reinterpret_cast<uintptr_t>(residual) % 16 == 0), "conv2d_tail: 16-byte aligned tensors");
+    msnh_conv_desc c = *d;
+    c.algo = MSNH_CONV_IGEMM;
+    return convIgemmTail(&c, t, x, w, scale, shift, residual, y, w2, scale2, shift2, z, resolveStream(s), false);
 }
 
 int msnh_hip_conv2d_select_algo(const msnh_conv_desc *d)

@@ -16,16 +16,25 @@ int igemmHeuristicTile(const msnh_conv_desc *d)
 }
 
 int igemmTileCount() { return kIgemmTiles; }
+int igemmTailTileFirst() { return kIgemmTailTileFirst; }
 
 size_t igemmSplitKWorkspaceBytes(const msnh_conv_desc *d)
 {
     return static_cast<size_t>(kSplitKMax) * d->batch * d->out_h * d->out_w * d->out_c * sizeof(float);
 }
 
-int convIgemmWs(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
-                const void *residual, void *y, hipStream_t st, bool dryRun, void *splitWs, size_t splitWsBytes)
+// tail != nullptr: the launch also computes the 1x1 convolution described there (msnh_hip_conv2d_tail); d->tile then names one of the
+// tiles that carry a tail, 0 the first of them that takes the shape.
+static int convIgemmAny(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
+                        const void *residual, void *y, hipStream_t st, bool dryRun, void *splitWs, size_t splitWsBytes,
+                        const msnh_conv_tail_desc *tail, const void *w2, const float *scale2, const float *shift2, void *z)
 {
     IgemmArgs a;
+    a.tailOn = tail ? 1 : 0;
+    a.w2 = w2; a.scale2 = scale2; a.shift2 = shift2; a.z = z;
+    a.cout2 = tail ? tail->out_c : 0; a.zLd = tail ? tail->out_ld : 0; a.act3 = tail ? tail->act : MSNH_ACT_NONE; a.writeY = tail ? (tail->write_y ? 1 : 0) : 1;
+    a.act3Param = tail ? tail->act_param : 0.f; a.zMul = tail ? tail->out_mul : 1.f;
+    a.w2Bytes = tail ? static_cast<unsigned>(tail->out_c) * static_cast<unsigned>(d->out_c) * 2u : 0u;
     a.x = x; a.w = w; a.scale = scale; a.shift = shift; a.res = residual; a.y = y;
     a.batch = d->batch; a.H = d->in_h; a.W = d->in_w; a.inLd = d->in_ld;
     a.OH = d->out_h; a.OW = d->out_w; a.outLd = d->out_ld; a.resLd = d->res_ld;
@@ -64,11 +73,32 @@ int convIgemmWs(const msnh_conv_desc *d, const void *x, const void *w, const flo
         a.ws = static_cast<float *>(splitWs);
     }
     int tile = d->tile;
+    if (tail)
+    {
+        MSNH_REQUIRE(d->dtype == MSNH_F16 && d->out_dtype == MSNH_F16 && d->groups == 1 && d->algo != MSNH_CONV_IGEMM_SPLITK, "conv2d_tail: float16, ungrouped, unsplit");
+        if (tile <= 0) tile = d->out_c > 128 ? kIgemmTailTileFirst : kIgemmTailTileFirst + 1;
+        MSNH_REQUIRE(tile >= kIgemmTailTileFirst && tile <= kIgemmTiles, "conv2d_tail: tile %d carries no tail", tile);
+        if (!dryRun)
+            MSNH_REQUIRE(reinterpret_cast<uintptr_t>(z) % 16 == 0 && reinterpret_cast<uintptr_t>(w2) % 16 == 0, "conv2d_tail: z and w2 must be 16-byte aligned");
+        else a.vecOk = (d->out_ld % 8 == 0) && (d->out_c % 8 == 0) && (!d->has_residual || d->res_ld % 8 == 0);
+    }
     if (tile <= 0 || tile > kIgemmTiles) tile = igemmHeuristicTile(d);
     if (d->dtype == MSNH_F16)
         return d->out_dtype == MSNH_F16 ? igemmF16F16(a, d->groups, tile, st) : igemmF16F32(a, d->groups, tile, st);
     MSNH_REQUIRE(d->out_dtype == MSNH_F32, "igemm: float32 input needs float32 output");
     return igemmF32F32(a, d->groups, tile, st);
+}
+
+int convIgemmWs(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,
+                const void *residual, void *y, hipStream_t st, bool dryRun, void *splitWs, size_t splitWsBytes)
+{
+    return convIgemmAny(d, x, w, scale, shift, residual, y, st, dryRun, splitWs, splitWsBytes, nullptr, nullptr, nullptr, nullptr, nullptr);
+}
+
+int convIgemmTail(const msnh_conv_desc *d, const msnh_conv_tail_desc *tail, const void *x, const void *w, const float *scale, const float *shift,
+                  const void *residual, void *y, const void *w2, const float *scale2, const float *shift2, void *z, hipStream_t st, bool dryRun)
+{
+    return convIgemmAny(d, x, w, scale, shift, residual, y, st, dryRun, nullptr, 0, tail, w2, scale2, shift2, z);
 }
 
 int convIgemm(const msnh_conv_desc *d, const void *x, const void *w, const float *scale, const float *shift,

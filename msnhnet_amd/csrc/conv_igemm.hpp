@@ -48,6 +48,15 @@ struct IgemmArgs
     int buffersOk;          // both extents fit a buffer resource
     int act, act2, hasRes, vecOk;
     float actParam, act2Param, resMul, outMul;
+    // tail (tiles with TAIL = 1 only): a 1x1 stride-1 convolution z = zMul * act3(scale2 * (W2 . y) + shift2) of this convolution's
+    // float16 result y, computed by the same workgroup from the copy of its y tile in LDS
+    int tailOn;             // the launch carries a tail (set by the tail entry point, also for dry runs)
+    const void  *w2;        // [cout2][coutG] float16, K contiguous
+    const float *scale2, *shift2;
+    void        *z;         // NHWC float16 with pixel stride zLd
+    int cout2, zLd, act3, writeY;
+    float act3Param, zMul;
+    unsigned w2Bytes;
 };
 
 template <typename T> struct Frag;
@@ -402,9 +411,270 @@ __device__ __forceinline__ i32x4 makeRsrcWords(const void *base, unsigned bytes)
     return r;
 }
 
+// Epilogue of the tiles that carry a tail: the workgroup's tile covers every output channel of the convolution (one channel tile), so
+// the 1x1 convolution that reads this convolution's result can be computed from the tile itself.
+//   1. the residual tile arrives in LDS by direct-to-LDS loads, in the layout of the result tile: [pixel][BM channels] float16, rows
+//      unpadded, 16-byte chunk c of row r at position c ^ (r % chunks per row); the main loop has asked for it already (resIssued)
+//      unless its K loop is a single step;
+//   2. affine + activation on the accumulators in place; then every lane adds the residual values under its accumulators (it reads
+//      them from LDS as 8-byte pieces: 4 consecutive channels of a pixel), applies the block activation and the output scale, rounds
+//      to float16 and writes the result back to the same place -- the LDS tile now holds exactly the bytes of y;
+//   3. y leaves for memory as 16-byte vectors, a pixel's channels from consecutive lanes (skipped when nobody else reads y);
+//   4. second GEMM: wavefront (channel block of 32, group of pixel blocks) multiplies W2 (fragments straight from global memory, asked
+//      for before step 3) with the y tile (B fragments from LDS) in k order, as a separate 1x1 launch would;
+//   5. its epilogue stages z as float16 in LDS the same way and stores 16-byte vectors.
+// The rounding points are those of two separate launches: y is rounded to float16 before the second GEMM reads it.
+// LDS map (the main loop of these tiles has two stages of STAGE bytes at [0, 2 STAGE); 160 KiB in all): 4 KiB of per-channel affines at 0; the y
+// tile's last UPROWS pixel rows behind the loop's stages, where the residual can arrive while the loop still runs; its first LOWROWS rows
+// (if the space behind the stages does not hold the whole tile) 4 KiB into the loop stage that the last tile step does not use -- that stage is
+// free from the barrier of the last step but one, and the residual rows are asked for right there; the z tile 4 KiB into the other stage (into
+// the first one when the y tile lies behind the stages entirely).
+constexpr int kTailMaxOut = 128;                   // output channels of the tail convolution
+template <int BM, int BN, unsigned STAGE> struct TailLds
+{
+    static constexpr unsigned TOTAL = 160 * 1024;
+    static constexpr unsigned HEAD  = 4096;
+    static constexpr int YROWB   = BM * 2;                                   // bytes per pixel row of the y tile
+    static constexpr int RPS     = 1024 / YROWB;                             // rows per 1 KiB delivery
+    static constexpr int FITROWS = static_cast<int>((TOTAL - 2 * STAGE) / YROWB) / RPS * RPS;
+    static constexpr int UPROWS  = FITROWS > BN ? BN : FITROWS;
+    static constexpr int LOWROWS = BN - UPROWS;
+    static constexpr unsigned UPOFF = 2 * STAGE;
+    static constexpr unsigned ZBYTES = BN * kTailMaxOut * 2;
+    static_assert(1024 % YROWB == 0 && LOWROWS % RPS == 0, "whole deliveries");
+    static_assert(HEAD + LOWROWS * YROWB <= STAGE && (LOWROWS == 0 ? HEAD + ZBYTES <= UPOFF : HEAD + ZBYTES <= STAGE), "tail tiles fit the loop's stages");
+    static_assert(UPOFF + UPROWS * YROWB <= TOTAL, "y tile fits behind the stages");
+    __device__ static unsigned lowOff(int freeStage) { return static_cast<unsigned>(freeStage) * STAGE + HEAD; }
+    __device__ static unsigned zOff(int freeStage) { return (LOWROWS == 0 ? 0u : static_cast<unsigned>(1 - freeStage) * STAGE) + HEAD; }
+    // byte offset of row 0 of the part that holds `row` (a row's address is this + row * YROWB)
+    __device__ static unsigned partBase(int row, unsigned low) { return row < LOWROWS ? low : UPOFF - LOWROWS * YROWB; }
+    static constexpr size_t bytes() { return LOWROWS > 0 ? TOTAL : (UPOFF + static_cast<size_t>(UPROWS) * YROWB); }
+};
+
+// The residual rows [LOWROWS, BN) (upper) or [0, LOWROWS) of the tile at pixel p0, straight into their places in the y tile: 1 KiB per wave
+// instruction, chunk c of row r at position c ^ (r % chunks per row).  Rows past the tensor and channels past out_c arrive as zeros.
+template <int BM, int BN, unsigned STAGE, int NW>
+__device__ __forceinline__ void tailIssueResidual(const IgemmArgs &a, int p0, unsigned ldsBase, int wave, int lane, bool upper, unsigned low)
+{
+    typedef TailLds<BM, BN, STAGE> L;
+    constexpr int YC = BM / 8;
+    const int npix = min(a.P - p0, BN);
+    const i32x4 rr = makeRsrcWords(static_cast<const f16 *>(a.res) + static_cast<size_t>(p0) * a.resLd, static_cast<unsigned>(npix) * a.resLd * 2u);
+    const int sBegin = (upper ? L::LOWROWS : 0) / L::RPS, sEnd = (upper ? BN : L::LOWROWS) / L::RPS;
+    const unsigned base = ldsBase + (upper ? L::UPOFF - L::LOWROWS * L::YROWB : low);
+    for (int s = sBegin + wave; s < sEnd; s += NW)
+    {
+        const int row = s * L::RPS + lane / YC;
+        const int c = (lane % YC) ^ (row % YC);
+        // (the address is the same in every lane; said explicitly, because it has to travel in a scalar register)
+        const unsigned ldsAddr = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(base + static_cast<unsigned>(s) * 1024u)));
+        dmaLoad16(rr, c * 8 < a.coutG ? static_cast<unsigned>(row * a.resLd + c * 8) * 2u : kOobOffset, 0u, ldsAddr);
+    }
+}
+
+template <int BM, int BN, int WM, int WN, unsigned STAGE>
+__device__ __forceinline__ void igemmTailEpilogue(const IgemmArgs &a, f32x16 (&acc)[BM / WM / 32][BN / WN / 32], unsigned char *smemRaw, unsigned ldsBase,
+                                                  float chScale, float chShift, float sc2, float sh2, int p0, int wm, int wn, int wave, int lane,
+                                                  bool resIssued, int freeStage)
+{
+    typedef TailLds<BM, BN, STAGE> L;
+    constexpr int NW    = WM * WN;
+    constexpr int NT    = 64 * NW;
+    constexpr int TM    = BM / WM, TN = BN / WN;
+    constexpr int MB    = TM / 32, NB = TN / 32;
+    constexpr int YROWB = BM * 2;                     // bytes per pixel row of the y tile
+    constexpr int YC    = BM / 8;                     // 16-byte chunks per row
+    constexpr int ZROWB = kTailMaxOut * 2, ZC = kTailMaxOut / 8;
+    const unsigned LOW = L::lowOff(freeStage);
+    const unsigned ZOFF = L::zOff(freeStage);
+    constexpr int PG    = NW / 4;                     // groups of pixel blocks in the second GEMM (4 channel blocks of 32)
+    constexpr int TN2   = BN / PG;
+    constexpr int NB2   = TN2 / 32;
+    constexpr int KB2   = BM / 16;                    // k-blocks of the second GEMM
+    static_assert(NW % 4 == 0 && BN % PG == 0 && TN2 % 32 == 0 && (BN * YC) % NT == 0 && (BN * ZC) % NT == 0, "tail geometry");
+    static_assert((2 * BM + 2 * kTailMaxOut) * 4 <= L::HEAD, "the affines fit in front of the tiles");
+
+    float *ss = reinterpret_cast<float *>(smemRaw);   // [BM] scale, [BM] shift, [128] scale2, [128] shift2
+    const int tid = wave * 64 + lane;
+    const int npix = min(a.P - p0, BN);
+    const int half = lane >> 5;
+    if (tid < BM) { ss[tid] = chScale; ss[BM + tid] = chShift; }
+    if (tid < kTailMaxOut) { ss[2 * BM + tid] = sc2; ss[2 * BM + kTailMaxOut + tid] = sh2; }
+
+    // 1. residual tile -> LDS, unless the main loop asked for it
+    if (a.hasRes && !resIssued)
+    {
+        tailIssueResidual<BM, BN, STAGE, NW>(a, p0, ldsBase, wave, lane, true, LOW);
+        if (L::LOWROWS > 0) tailIssueResidual<BM, BN, STAGE, NW>(a, p0, ldsBase, wave, lane, false, LOW);
+    }
+    __syncthreads();                                  // affines visible
+
+    // 2a. affine + activation in place
+    float slope1, slope2, slope3;
+    const bool lin1 = actIsSlope(a.act, a.actParam, slope1);
+    const bool lin2 = actIsSlope(a.act2, a.act2Param, slope2);
+    const bool lin3 = actIsSlope(a.act3, a.act3Param, slope3);
+    staticFor<0, NB>([&](auto jTag) {
+        constexpr int j = decltype(jTag)::value;
+        float t[MB * 16];
+        staticFor<0, MB * 4>([&](auto iqTag) {
+            constexpr int iq = decltype(iqTag)::value;
+            constexpr int i = iq / 4, q = iq % 4;
+            const int ml = wm * TM + i * 32 + q * 8 + half * 4;
+            const f32x4 sc = *reinterpret_cast<const f32x4 *>(ss + ml);
+            const f32x4 sh = *reinterpret_cast<const f32x4 *>(ss + BM + ml);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) t[iq * 4 + e] = acc[i][j][q * 4 + e] * sc[e] + sh[e];
+        });
+        if (lin1)
+        {
+#pragma unroll
+            for (int e = 0; e < MB * 16; ++e) t[e] = activateSel<true>(t[e], slope1, a.act, a.actParam);
+        }
+        else activateArray<MB * 16>(t, a.act, a.actParam);
+        staticFor<0, MB * 16>([&](auto eTag) { constexpr int e = decltype(eTag)::value; acc[e / 16][j][e % 16] = t[e]; });
+    });
+    dmaWait<0>();
+    __syncthreads();                                  // residual tile complete
+
+    // 2b. residual, block activation, scale, rounding; the y tile replaces the residual tile
+    staticFor<0, NB>([&](auto jTag) {
+        constexpr int j = decltype(jTag)::value;
+        const int row = wn * TN + j * 32 + (lane & 31);
+        unsigned char *rowPtr = smemRaw + L::partBase(row, LOW) + row * YROWB + half * 8;
+        const int sw = row % YC;
+        staticFor<0, MB * 4>([&](auto iqTag) {
+            constexpr int iq = decltype(iqTag)::value;
+            constexpr int i = iq / 4, q = iq % 4;
+            const int c = (wm * TM + i * 32) / 8 + q;
+            f16x4 *cell = reinterpret_cast<f16x4 *>(rowPtr + ((c ^ sw) * 16));
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[i][j][q * 4 + e];
+            if (a.hasRes)
+            {
+                const f16x4 r = *cell;
+                if (lin2)
+                {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = activateSel<true>(v[e] + a.resMul * static_cast<float>(r[e]), slope2, a.act2, a.act2Param);
+                }
+                else
+                {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] += a.resMul * static_cast<float>(r[e]);
+                    activateArray<4>(v, a.act2, a.act2Param);
+                }
+            }
+            f16x4 h;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) h[e] = static_cast<f16>(v[e] * a.outMul);
+            *cell = h;
+        });
+    });
+
+    // 4a. fragments of W2 for this wavefront's 32 output channels, all k-blocks (the accumulators' registers are free now)
+    const int wm2 = wave % 4, wn2 = wave / 4;
+    const __amdgpu_buffer_rsrc_t rw2 = makeRsrc(a.w2, a.w2Bytes);
+    f16x8 fa2[KB2];
+    {
+        const int m2 = wm2 * 32 + (lane & 31);
+#pragma unroll
+        for (int kb = 0; kb < KB2; ++kb)
+        {
+            const int c = 2 * kb + half;
+            fa2[kb] = bufferLoad16<f16x8>(rw2, (m2 < a.cout2 && c * 8 < a.coutG) ? static_cast<unsigned>(m2 * a.coutG + c * 8) * 2u : kOobOffset, 0u);
+        }
+    }
+    __syncthreads();                                  // y tile complete
+
+    // 3. y -> memory
+    if (a.writeY)
+    {
+        const __amdgpu_buffer_rsrc_t ry = makeRsrc(static_cast<f16 *>(a.y) + static_cast<size_t>(p0) * a.outLd, static_cast<unsigned>(npix) * a.outLd * 2u);
+#pragma unroll
+        for (int k = 0; k < BN * YC / NT; ++k)
+        {
+            const int v = tid + NT * k;
+            const int row = v / YC, c = v % YC;
+            const i32x4 d = *reinterpret_cast<const i32x4 *>(smemRaw + L::partBase(row, LOW) + row * YROWB + ((c ^ (row % YC)) * 16));
+            __builtin_amdgcn_raw_buffer_store_b128(d, ry, c * 8 < a.coutG ? (row * a.outLd + c * 8) * 2 : static_cast<int>(kOobOffset), 0, 0);
+        }
+    }
+
+    // 4b. z tile = W2 . y tile
+    f32x16 acc2[NB2];
+#pragma unroll
+    for (int j = 0; j < NB2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc2[j][r] = 0.f;
+    const unsigned char *bBase[NB2];
+    int bSw[NB2];
+#pragma unroll
+    for (int j = 0; j < NB2; ++j)
+    {
+        const int row = wn2 * TN2 + j * 32 + (lane & 31);
+        bBase[j] = smemRaw + L::partBase(row, LOW) + row * YROWB;
+        bSw[j] = row % YC;
+    }
+    staticFor<0, KB2>([&](auto kbTag) {
+        constexpr int kb = decltype(kbTag)::value;
+        f16x8 fb[NB2];
+#pragma unroll
+        for (int j = 0; j < NB2; ++j) fb[j] = *reinterpret_cast<const f16x8 *>(bBase[j] + (((2 * kb + half) ^ bSw[j]) * 16));
+#pragma unroll
+        for (int j = 0; j < NB2; ++j) mfmaBlock(fa2[kb], fb[j], acc2[j]);
+    });
+
+    // 5. z: affine, activation, scale, float16, staged in LDS, stored as 16-byte vectors
+    staticFor<0, NB2>([&](auto jTag) {
+        constexpr int j = decltype(jTag)::value;
+        const int row = wn2 * TN2 + j * 32 + (lane & 31);
+        unsigned char *rowPtr = smemRaw + ZOFF + row * ZROWB + half * 8;
+        float t[16];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const int mch = wm2 * 32 + q * 8 + half * 4;
+            const f32x4 sc = *reinterpret_cast<const f32x4 *>(ss + 2 * BM + mch);
+            const f32x4 sh = *reinterpret_cast<const f32x4 *>(ss + 2 * BM + kTailMaxOut + mch);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) t[q * 4 + e] = acc2[j][q * 4 + e] * sc[e] + sh[e];
+        }
+        if (lin3)
+        {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) t[e] = activateSel<true>(t[e], slope3, a.act3, a.act3Param);
+        }
+        else activateArray<16>(t, a.act3, a.act3Param);
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            f16x4 h;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) h[e] = static_cast<f16>(t[q * 4 + e] * a.zMul);
+            *reinterpret_cast<f16x4 *>(rowPtr + (((wm2 * 4 + q) ^ (row % ZC)) * 16)) = h;
+        }
+    });
+    __syncthreads();
+    {
+        const __amdgpu_buffer_rsrc_t rz = makeRsrc(static_cast<f16 *>(a.z) + static_cast<size_t>(p0) * a.zLd, static_cast<unsigned>(npix) * a.zLd * 2u);
+#pragma unroll
+        for (int k = 0; k < BN * ZC / NT; ++k)
+        {
+            const int v = tid + NT * k;
+            const int row = v / ZC, c = v % ZC;
+            const i32x4 d = *reinterpret_cast<const i32x4 *>(smemRaw + ZOFF + row * ZROWB + ((c ^ (row % ZC)) * 16));
+            __builtin_amdgcn_raw_buffer_store_b128(d, rz, c * 8 < a.cout2 ? (row * a.zLd + c * 8) * 2 : static_cast<int>(kOobOffset), 0, 0);
+        }
+    }
+}
+
+
 // KG = 2: two groups of wavefronts share the WM x WN grid of (then 64 x 64) wave tiles and split the k-blocks of every tile step
 // between them, which takes a third off the LDS fragment reads per MFMA against 32 x 64 wave tiles of the same workgroup tile.
-template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int NS, int KG = 1>
+// TAIL = 1: the epilogue also computes the 1x1 convolution that reads this one's result (igemmTailEpilogue); float16 only.
+template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int NS, int KG = 1, int TAIL = 0>
 __global__ __launch_bounds__(64 * WM * WN * KG)
 __attribute__((amdgpu_waves_per_eu(KG == 2 ? (WM * WN * KG) / 4 : igemmWavesPerSimd(BM, BN, KV, NS, WM * WN),
                                    KG == 2 ? (WM * WN * KG == 4 ? 3 : (WM * WN * KG) / 4) : igemmWavesPerSimd(BM, BN, KV, NS, WM * WN))))
@@ -464,6 +734,13 @@ void convIgemmKernel(IgemmArgs a)
 
     float chScale, chShift;
     loadChannelAffine(a, g, m0, tid, BM, chScale, chShift);
+    float sc2 = 1.f, sh2 = 0.f;                       // TAIL: the second convolution's affine of channel tid
+    if constexpr (TAIL != 0)
+        if (tid < kTailMaxOut && tid < a.cout2)
+        {
+            if (a.scale2) sc2 = a.scale2[tid];
+            if (a.shift2) sh2 = a.shift2[tid];
+        }
 
     // LDS layout of a stage: rows of KV 16-byte chunks without padding; chunk c of row r sits at chunk position
     // c ^ ((r / SWDIV) % KV).  With that XOR the 16 lanes the LDS serves per cycle hit 16 different 16-byte bank
@@ -529,8 +806,9 @@ void convIgemmKernel(IgemmArgs a)
     };
     int tapNext = 0, chunkNext = 0;              // the tile step whose loads were issued last
     unsigned sANext = 0, sBNext = 0;
-    bool cutNext = false;
+    bool cutNext = false, pastEndNext = false;
     auto advance = [&](bool pastEnd) {
+        pastEndNext = pastEnd;
         if (++chunkNext == a.cChunks) { chunkNext = 0; ++tapNext; if (tapNext < a.taps) setTap(tapNext); }
         sANext = (static_cast<unsigned>(tapNext) * a.cinG + chunkNext * BK) * ES;
         sBNext = static_cast<unsigned>(chunkNext * BK) * ES;
@@ -592,6 +870,7 @@ void convIgemmKernel(IgemmArgs a)
     // split-K: this workgroup multiplies tile steps [itBegin, itBegin + nLocal) of the K loop
     const int itBegin = a.splitK > 1 ? static_cast<int>(static_cast<long long>(blockIdx.y) * a.nIter / a.splitK) : 0;
     const int nLocal  = a.splitK > 1 ? static_cast<int>(static_cast<long long>(blockIdx.y + 1) * a.nIter / a.splitK) - itBegin : a.nIter;
+    const bool tailPrefetch = TAIL != 0 && a.hasRes && nLocal >= 2;
     tapNext = itBegin / a.cChunks;
     chunkNext = itBegin - tapNext * a.cChunks - 1;            // advance() steps onto the first tile step
     setTap(tapNext);
@@ -622,6 +901,14 @@ void convIgemmKernel(IgemmArgs a)
                 {
                     dmaWait<INFLIGHT>();         // all of step it+1 has landed; younger loads may be in flight
                     __syncthreads();
+                    if constexpr (TAIL != 0)
+                    {
+                        // the residual tile of the epilogue: the rows that lie behind the loop's stages right away, the others into the
+                        // stage of this step -- free from here on -- in the last step but one
+                        if (tailPrefetch && it == 0) tailIssueResidual<BM, BN, STAGE, NT / 64>(a, p0, ldsBase, wave, lane, true, 0u);
+                        if (tailPrefetch && it == nLocal - 2 && TailLds<BM, BN, STAGE>::LOWROWS > 0)
+                            tailIssueResidual<BM, BN, STAGE, NT / 64>(a, p0, ldsBase, wave, lane, false, TailLds<BM, BN, STAGE>::lowOff(nLocal & 1));
+                    }
                     readFrags(nxt, std::integral_constant<int, 0>());
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -632,7 +919,9 @@ void convIgemmKernel(IgemmArgs a)
                 // loads l with LBASE + l * LSPAN / NL == gi
                 constexpr int first = ((gi - LBASE) * NL + LSPAN - 1) / LSPAN;
                 constexpr int last  = ((gi - LBASE + 1) * NL + LSPAN - 1) / LSPAN;
-                staticFor<first, last>([&](auto lTag) { issueLoad(lTag, sANext, sBNext, cutNext, nn); });
+                // (TAIL: the stages that steps past the end of K would zero receive residual rows instead)
+                if (!(TAIL != 0 && pastEndNext))
+                    staticFor<first, last>([&](auto lTag) { issueLoad(lTag, sANext, sBNext, cutNext, nn); });
             }
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -643,6 +932,12 @@ void convIgemmKernel(IgemmArgs a)
     dmaWait<0>();
     __syncthreads();
 
+    if constexpr (TAIL != 0)
+    {
+        static_assert(KG == 1 && NS == 2 && std::is_same<T, f16>::value && std::is_same<TOut, f16>::value, "the tail is a float16 epilogue of the unsplit two-stage kernel");
+        igemmTailEpilogue<BM, BN, WM, WN, STAGE>(a, acc, smemRaw, ldsBase, chScale, chShift, sc2, sh2, p0, wm, wn, wave, lane, tailPrefetch, tailPrefetch ? (nLocal & 1) : 0);
+        return;
+    }
     if (a.splitK > 1)
     {
         // raw float32 partial sums of this K slice; affine, activation and residual follow in the reduction pass
@@ -687,11 +982,21 @@ __global__ __launch_bounds__(256) void splitKReduceKernel(IgemmArgs a, int outC,
 
 constexpr int kSplitKMax = 8;
 
-template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int NS = 3, int KG = 1>
+template <typename T, typename TOut, int BM, int BN, int KV, int WM, int WN, int NS = 3, int KG = 1, int TAIL = 0>
 inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
 {
     constexpr int VEC = Frag<T>::VEC;
     constexpr int BK  = KV * VEC;
+    if (TAIL != 0 || a.tailOn)
+    {
+        // a launch with a tail needs a tile that has one, and the other way round; the tile must hold every output channel
+        if (!(TAIL != 0 && a.tailOn) || groups != 1 || a.splitMax > 1 || a.coutG > BM || a.coutG % 8 != 0 || a.cout2 > kTailMaxOut || a.cout2 % 8 != 0 ||
+            a.cout2 <= 0 || a.outLd % 8 != 0 || a.zLd % 8 != 0 || (a.hasRes && a.resLd % 8 != 0) || !a.vecOk)
+        {
+            setError("conv2d: this tile needs a 1x1 convolution behind it (msnh_hip_conv2d_tail), the others take none; ungrouped, channel counts that fit one tile");
+            return 3;
+        }
+    }
     a.cChunks = (a.cinG + BK - 1) / BK;
     a.nIter   = a.taps * a.cChunks;
     a.ragged  = (a.cinG % BK) != 0;
@@ -702,7 +1007,13 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
     }
     constexpr int RPP = 64 * WM * WN * KG / KV;
     const size_t smemLoop = static_cast<size_t>(NS) * ((BM + RPP - 1) / RPP * RPP + (BN + RPP - 1) / RPP * RPP) * KV * 16;
-    const size_t smemEpi  = std::max(igemmEpilogueLds<BM, BM / WM, WM * WN * KG>(), KG == 2 ? igemmSwapLds<WM * WN * KG>() : size_t(0));
+    size_t smemEpi = 0;
+    if constexpr (TAIL != 0)
+    {
+        constexpr unsigned STAGE = static_cast<unsigned>(((BM + RPP - 1) / RPP * RPP + (BN + RPP - 1) / RPP * RPP) * KV * 16);
+        smemEpi = TailLds<BM, BN, STAGE>::bytes();
+    }
+    else smemEpi = std::max(igemmEpilogueLds<BM, BM / WM, WM * WN * KG>(), KG == 2 ? igemmSwapLds<WM * WN * KG>() : size_t(0));
     const size_t smem = smemLoop > smemEpi ? smemLoop : smemEpi;
     a.mTiles = (a.coutG + BM - 1) / BM;
     const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
@@ -722,7 +1033,7 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
     }
     dim3 grid((tiles + 7) / 8 * 8, a.splitK, groups);
     if (a.dryRun) return 0;
-    auto kern = convIgemmKernel<T, TOut, BM, BN, KV, WM, WN, NS, KG>;
+    auto kern = convIgemmKernel<T, TOut, BM, BN, KV, WM, WN, NS, KG, TAIL>;
     if (smem > 48 * 1024)
     {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -751,7 +1062,8 @@ namespace msnh {
 // Tile configurations (BM x BN output tile, KV 16-byte vectors of K per step, WM x WN wavefront grid).
 // Index 0 is "choose for me"; the others can be forced through msnh_conv_desc::tile, which is how the host
 // library's per-layer search picks the fastest one at load time.
-constexpr int kIgemmTiles = 62;
+constexpr int kIgemmTiles = 64;
+constexpr int kIgemmTailTileFirst = 63;         // tiles from here on carry a tail (msnh_hip_conv2d_tail)
 
 template <typename T, typename TOut>
 int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
@@ -837,6 +1149,20 @@ int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
     case 60: return launchIgemm<T, TOut, 128, 64, 8, 2, 1, 4, 2>(a, groups, st);
     case 61: return launchIgemm<T, TOut, 64, 256, 8, 1, 4, 3, 2>(a, groups, st);
     case 62: return launchIgemm<T, TOut, 64, 384, 8, 1, 6, 2, 2>(a, groups, st);
+    // tiles whose epilogue also computes the 1x1 convolution that follows (msnh_hip_conv2d_tail only; float16): the tile holds every
+    // output channel of the first convolution (at most 256 / 128)
+    case 63:
+    case 64:
+        if constexpr (std::is_same<T, f16>::value && std::is_same<TOut, f16>::value)
+        {
+            if (tile == 63) return launchIgemm<T, TOut, 256, 192, 8, 4, 3, 2, 1, 1>(a, groups, st);
+            return launchIgemm<T, TOut, 128, 192, 8, 4, 3, 2, 1, 1>(a, groups, st);
+        }
+        else
+        {
+            setError("conv2d: this tile needs float16 tensors and a 1x1 convolution behind it (msnh_hip_conv2d_tail)");
+            return 3;
+        }
     default: break;
     }
     setError("igemm: unknown tile %d", tile);

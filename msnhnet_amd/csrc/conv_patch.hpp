@@ -269,7 +269,7 @@ inline int launchPatch(IgemmArgs &a, int groups, hipStream_t st)
     constexpr int BK  = KV * VEC;
     size_t smem = 0;
     int slices = 0;
-    if (groups != 1 || a.splitMax > 1 || !patchFits<T, BM, BN, KV, WM, WN, PS>(a, &smem, &slices))
+    if (groups != 1 || a.splitMax > 1 || a.tailOn || !patchFits<T, BM, BN, KV, WM, WN, PS>(a, &smem, &slices))
     {
         setError("conv2d: this tile needs a 3x3 stride-1 pad-1 ungrouped convolution whose input patch fits in LDS");
         return 3;

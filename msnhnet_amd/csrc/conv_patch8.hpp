@@ -345,7 +345,7 @@ inline int launchPatch8(IgemmArgs &a, int groups, hipStream_t st)
     constexpr int BK  = 8 * VEC;
     size_t smem = 0;
     int slices = 0;
-    if (groups != 1 || a.splitMax > 1 || !patch8Fits<T, BM, BN, WM, WN, NSA, PS, KG>(a, &smem, &slices))
+    if (groups != 1 || a.splitMax > 1 || a.tailOn || !patch8Fits<T, BM, BN, WM, WN, NSA, PS, KG>(a, &smem, &slices))
     {
         setError("conv2d: this tile needs a 3x3 stride-1 pad-1 ungrouped convolution whose input patch fits in LDS");
         return 3;

@@ -10,7 +10,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmsnh_hip.so")
 
 F32, F16 = 0, 1
 ACT = {"logistic": 0, "relu": 1, "relu6": 2, "leaky": 8, "swish": 16, "hardswish": 17, "mish": 18, "none": 22}
-ALGO = {"auto": 0, "direct": 1, "igemm": 2, "depthwise": 3, "winograd": 4, "stem": 5, "igemm_splitk": 6, "pointwise": 7, "stem_down": 8, "winograd_fused": 9, "mbconv": 10}
+ALGO = {"auto": 0, "direct": 1, "igemm": 2, "depthwise": 3, "winograd": 4, "stem": 5, "igemm_splitk": 6, "pointwise": 7, "stem_down": 8, "winograd_fused": 9, "mbconv": 10, "igemm_tail": 11}
 ALGO_NAME = {v: k for k, v in ALGO.items()}
 
 
@@ -22,6 +22,12 @@ class ConvDesc(ctypes.Structure):
                 ("act", ctypes.c_int), ("act_param", ctypes.c_float),
                 ("has_residual", ctypes.c_int), ("res_ld", ctypes.c_int), ("act2", ctypes.c_int), ("act2_param", ctypes.c_float),
                 ("res_mul", ctypes.c_float), ("out_mul", ctypes.c_float), ("algo", ctypes.c_int), ("tile", ctypes.c_int)]
+
+
+class ConvTailDesc(ctypes.Structure):
+    """msnh_conv_tail_desc of include/msnh_hip.h"""
+    _fields_ = [("out_c", ctypes.c_int), ("out_ld", ctypes.c_int), ("act", ctypes.c_int), ("act_param", ctypes.c_float), ("out_mul", ctypes.c_float),
+                ("write_y", ctypes.c_int)]
 
 
 class MbconvDesc(ctypes.Structure):
@@ -48,7 +54,8 @@ SYMBOLS = [
     "msnh_hip_fill_zero", "msnh_hip_stream_create", "msnh_hip_stream_destroy", "msnh_hip_stream_sync", "msnh_hip_event_create",
     "msnh_hip_event_destroy", "msnh_hip_event_record", "msnh_hip_stream_wait_event", "msnh_hip_event_sync", "msnh_hip_event_elapsed_ms", "msnh_hip_graph_begin",
     "msnh_hip_graph_end", "msnh_hip_graph_launch", "msnh_hip_graph_destroy", "msnh_hip_conv_stem_down_supported", "msnh_hip_conv_stem_down_packed_elems", "msnh_hip_conv_stem_down_pack", "msnh_hip_conv_stem_down", "msnh_hip_mbconv_supported", "msnh_hip_mbconv_packed_bytes", "msnh_hip_mbconv_pack", "msnh_hip_mbconv", "msnh_hip_conv2d_tile_count", "msnh_hip_conv2d_pack_layout_version", "msnh_hip_conv2d_tile_supported", "msnh_hip_conv2d_select_algo",
-    "msnh_hip_conv2d_packed_weight_elems", "msnh_hip_conv2d_pack_weights", "msnh_hip_conv2d_workspace_bytes", "msnh_hip_conv2d", "msnh_hip_letterbox_u8", "msnh_hip_image_u8_to_input",
+    "msnh_hip_conv2d_packed_weight_elems", "msnh_hip_conv2d_pack_weights", "msnh_hip_conv2d_workspace_bytes", "msnh_hip_conv2d",
+    "msnh_hip_conv2d_tail_tile_first", "msnh_hip_conv2d_tail_supported", "msnh_hip_conv2d_tail", "msnh_hip_letterbox_u8", "msnh_hip_image_u8_to_input",
     "msnh_hip_affine_act", "msnh_hip_add_act", "msnh_hip_copy_channels", "msnh_hip_maxpool", "msnh_hip_maxpool_chain", "msnh_hip_maxpool_chain_supported", "msnh_hip_avgpool",
     "msnh_hip_upsample_nearest", "msnh_hip_pad", "msnh_hip_slice", "msnh_hip_upsample_bilinear", "msnh_hip_softmax", "msnh_hip_deconv_col2im", "msnh_hip_connected", "msnh_hip_nchw_to_nhwc", "msnh_hip_nhwc_to_nchw", "msnh_hip_yolo_decode", "msnh_hip_yolo_decode_candidates", "msnh_hip_yolo_decode_candidates_heads",
     "msnh_hip_yolo_gather", "msnh_hip_yolo_nms", "msnh_hip_yolo_nms_workspace_bytes", "msnh_hip_yolo_nms_pair_workspace_bytes", "msnh_hip_yolo_nms_static", "msnh_hip_yolo_nms_static_max_bytes", "msnh_hip_absmax", "msnh_hip_count_nonfinite", "msnh_hip_mfma_probe",
@@ -105,6 +112,8 @@ def lib():
     L.msnh_hip_conv2d_workspace_bytes.argtypes = [cdp, ci]
     L.msnh_hip_conv2d_workspace_bytes.restype = sz
     L.msnh_hip_conv2d.argtypes = [cdp, vp, vp, vp, vp, vp, vp, vp, sz, vp]
+    L.msnh_hip_conv2d_tail_supported.argtypes = [cdp, ctypes.POINTER(ConvTailDesc), ci]
+    L.msnh_hip_conv2d_tail.argtypes = [cdp, ctypes.POINTER(ConvTailDesc), vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]
     L.msnh_hip_affine_act.argtypes = [ci, ci, ll, ci, vp, ci, vp, vp, ci, cf, cf, vp, ci, vp]
     L.msnh_hip_add_act.argtypes = [ci, ll, ci, vp, ci, cf, vp, ci, cf, ci, cf, cf, vp, ci, vp]
     L.msnh_hip_copy_channels.argtypes = [ci, ll, ci, vp, ci, cf, vp, ci, vp]

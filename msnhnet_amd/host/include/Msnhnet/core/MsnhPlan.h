@@ -79,6 +79,12 @@ struct PlanOp
     int  mbExpand = -1, mbDw = -1;          // CONV 1x1 closing an inverted-residual block: the (dead) 1x1 expand and 3x3 depthwise ops computed in front of
                                             // it by the same launch (Plan::fuse d, msnh_hip_mbconv)
 
+    int  tail = -1;                         // CONV: the 1x1 convolution op that reads this one's result and that the same launch can compute
+                                            // (Plan::fuse e); it does when the search set algo to MSNH_CONV_IGEMM_TAIL, and the 1x1 op is then dead
+    int  tailOf = -1;                       // CONV 1x1: the op whose launch may compute it
+    double ownFlops = 0;                    // CONV with a tail: flops without the tail's
+    bool tailSkipY = false;                 // CONV computing its tail: nothing but the tail reads this op's own result, which therefore is not written
+
     // YOLO_DECODE
     std::array<float, 6> anchors{};
     int   classes = 0;
@@ -104,6 +110,9 @@ public:
                                             // op order) can decode them all; empty = one launch pair per head
     void findYoloHeads();                   // fills yoloHeadOps; call once the heads' cell numbers are assigned
     bool fuseMbconv = true;                 // float16: 1x1 expand -> 3x3 depthwise -> 1x1 project as one launch where msnh_hip_mbconv takes the block
+    bool fuseTail = false;                  // float16: a convolution whose tile holds all its output channels also computes the 1x1 convolution that
+                                            // reads its result (msnh_hip_conv2d_tail), where the per-layer search finds that faster than two launches
+    bool forceTail = false;                 // ... wherever the library takes the pair, whatever the timing says (tests)
     bool fuseStemDown = true;               // float16: first layer + first stride-2 layer as one launch where msnh_hip_conv_stem_down takes the pair
     bool preferWinograd = false;            // 3x3 stride-1 float16 convs take the Winograd path where the kernel accepts the shape
     std::vector<PlanTensor> tensors;
@@ -155,6 +164,8 @@ public:
 
 private:
     void launch(PlanOp &op, msnh_stream_t s);
+    void applyTails();                      // after the search: the 1x1 ops computed by their producer's launch become dead, the others alive
     DeviceBuffer _arena, _exportScratch, _convWorkspace;
+    bool _tailWriteAll = false;             // runs that look at every tensor (calibration, float16 headroom): tailSkipY is ignored
 };
 }

@@ -407,6 +407,10 @@ void NetBuilder::finalizePlan()
     std::unique_ptr<Plan> plan = lowerNetwork(dtype);
     plan->fuseStemDown = std::getenv("MSNH_NO_STEM_DOWN") == nullptr;
     plan->fuseMbconv = std::getenv("MSNH_NO_MBCONV") == nullptr;
+    // (measured level with two launches inside a forward, so not the default: MSNH_CONV_TAIL=1 lets the load-time search decide per pair,
+    // MSNH_FORCE_CONV_TAIL=1 takes every pair the library accepts)
+    plan->forceTail = std::getenv("MSNH_FORCE_CONV_TAIL") != nullptr;
+    plan->fuseTail = plan->forceTail || std::getenv("MSNH_CONV_TAIL") != nullptr;
     plan->fuse();
     plan->chainMaxPools();
     plan->aliasConcats();
@@ -848,6 +852,12 @@ static double opBytes(const Plan &plan, const PlanOp &op)
     const PlanTensor &out = plan.tensors[static_cast<size_t>(op.out)];
     double oe = static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4);
     for (int nx = op.chainNext; nx >= 0; nx = plan.ops[static_cast<size_t>(nx)].chainNext) oe += static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4);   // one launch, every pool's result
+    if (op.algo == MSNH_CONV_IGEMM_TAIL && op.tail >= 0)
+    {
+        // ... and the 1x1 convolution computed by the same launch: its result and its filters
+        const PlanOp &b = plan.ops[static_cast<size_t>(op.tail)];
+        oe += static_cast<double>(plan.tensors[static_cast<size_t>(b.out)].elems()) * 2 + static_cast<double>(b.wDev.bytes());
+    }
     return static_cast<double>(in.elems()) * (in.dtype == MSNH_F16 ? 2 : 4) + oe + (op.in1 >= 0 ? static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4) : 0.0) +
            static_cast<double>(op.wDev.bytes());
 }
@@ -891,7 +901,7 @@ std::string NetBuilder::profileEachOp(int reps, std::vector<double> *values)
     if (!_planReady) MSNH_THROW("weights are not loaded");
     Plan &plan = *_net->plan;
     static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode", "pad", "slice", "bilinear", "softmax", "col2im"};
-    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk", "pointwise", "stem+down", "winograd_fused", "mbconv"};
+    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk", "pointwise", "stem+down", "winograd_fused", "mbconv", "igemm+1x1"};
     msnh_event_t e0 = nullptr, e1 = nullptr;
     MSNH_DEV(msnh_hip_event_create(&e0));
     MSNH_DEV(msnh_hip_event_create(&e1));

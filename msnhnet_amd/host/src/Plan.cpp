@@ -258,6 +258,30 @@ void Plan::fuse()
             ex.dead = true;
             dw.dead = true;
         }
+    // (e) float16: convolution -> 1x1 stride-1 convolution (the 3x3 that closes a Darknet residual block and the 1x1 that opens the next one,
+    // src/layers/MsnhResBlockLayer.cpp:215-302): where one tile of the first launch holds all its output channels (at most 256) and the 1x1 has at
+    // most 128 filters, the first launch can compute the 1x1 from its own result tile (msnh_hip_conv2d_tail).  Only marked here: both ops stay
+    // alive, the per-layer search times the pair both ways (tuneConvs), and the 1x1's result is placed from the first launch on.
+    if (computeDtype == MSNH_F16 && fuseTail)
+        for (size_t i = 0; i < ops.size(); ++i)
+        {
+            PlanOp &b = ops[i];
+            if (b.dead || b.kind != PlanOp::CONV || b.ksize != 1 || b.stride != 1 || b.pad != 0 || b.groups != 1 || b.in1 >= 0 || b.stemOp >= 0 || b.mbExpand >= 0 ||
+                b.tail >= 0 || b.tailOf >= 0)
+                continue;
+            const int pa = producerOf(b.in0);
+            if (pa < 0 || pa >= static_cast<int>(i)) continue;
+            PlanOp &a = ops[static_cast<size_t>(pa)];
+            if (a.kind != PlanOp::CONV || a.groups != 1 || a.dilation != 1 || a.stemOp >= 0 || a.mbExpand >= 0 || a.tail >= 0 || a.tailOf >= 0 || a.out != b.in0) continue;
+            const PlanTensor &x = tensors[static_cast<size_t>(a.in0)];
+            const PlanTensor &y = tensors[static_cast<size_t>(a.out)];
+            const PlanTensor &z = tensors[static_cast<size_t>(b.out)];
+            const auto f16Image = [](const PlanTensor &t) { return t.dtype == MSNH_F16 && t.layout == PlanTensor::NHWC; };
+            if (!f16Image(x) || !f16Image(y) || !f16Image(z) || x.c % 8 != 0 || y.c % 8 != 0 || y.c > 256 || z.c % 8 != 0 || z.c > 128) continue;
+            if (a.in1 >= 0 && !f16Image(tensors[static_cast<size_t>(a.in1)])) continue;
+            a.tail = static_cast<int>(i);
+            b.tailOf = pa;
+        }
 }
 
 // ---- pass 1b: stride-1 max-pools over one tensor (SPP blocks: 5, 9, 13) ---------------------------------------------
@@ -359,6 +383,7 @@ void Plan::aliasConcats()
 // ended up in its place, and with it a scale that flushes its own values to zero.)
 void Plan::runCalibration(msnh_stream_t s)
 {
+    struct WriteAll { bool &f; explicit WriteAll(bool &x) : f(x) { f = true; } ~WriteAll() { f = false; } } writeAll(_tailWriteAll);
     DeviceBuffer res(sizeof(float) * tensors.size());
     MSNH_DEV(msnh_hip_fill_zero(res.ptr(), sizeof(float) * tensors.size(), s));
     for (PlanOp &op : ops)
@@ -389,6 +414,7 @@ void Plan::runCalibration(msnh_stream_t s)
 // the input could still grow before a float16 activation overflows.
 float Plan::fp16Headroom(msnh_stream_t s)
 {
+    struct WriteAll { bool &f; explicit WriteAll(bool &x) : f(x) { f = true; } ~WriteAll() { f = false; } } writeAll(_tailWriteAll);
     DeviceBuffer res(sizeof(float) * 2);
     MSNH_DEV(msnh_hip_fill_zero(res.ptr(), sizeof(float) * 2, s));
     if (yoloCandCnt.ptr()) MSNH_DEV(msnh_hip_fill_zero(yoloCandCnt.ptr(), yoloCandCnt.bytes(), s));
@@ -424,9 +450,9 @@ uint64_t Plan::structureHash() const
     for (const PlanTensor &t : tensors)
         os << t.n << ' ' << t.h << ' ' << t.w << ' ' << t.c << ' ' << t.dtype << ' ' << static_cast<int>(t.layout) << ' ' << t.parent << ' ' << t.chanOffset << ';';
     for (const PlanOp &op : ops)
-        os << static_cast<int>(op.kind) << ' ' << op.in0 << ' ' << op.in1 << ' ' << op.out << ' ' << op.dead << ' ' << op.layerIndex << ' ' << op.ksize << ' ' << op.stride << ' '
+        os << static_cast<int>(op.kind) << ' ' << op.in0 << ' ' << op.in1 << ' ' << op.out << ' ' << (op.dead && op.tailOf < 0) << ' ' << op.layerIndex << ' ' << op.ksize << ' ' << op.stride << ' '
            << op.pad << ' ' << op.dilation << ' ' << op.groups << ' ' << static_cast<int>(op.act) << ' ' << static_cast<int>(op.act2) << ' ' << op.in1Sign << ' ' << (op.src2 != nullptr)
-           << ' ' << op.dstChanOffset << ' ' << op.stemOp << ' ' << op.chainHead << ' ' << op.mbExpand << ';';
+           << ' ' << op.dstChanOffset << ' ' << op.stemOp << ' ' << op.chainHead << ' ' << op.mbExpand << ' ' << op.tail << ';';
     const std::string text = os.str();
     return PackFile::hash(text.data(), text.size());
 }
@@ -484,6 +510,7 @@ void Plan::place()
         if (op.dead) continue;
         touch(op.in0, i); touch(op.in1, i); touch(op.out, i);
         if (op.chainHead >= 0) touch(op.out, op.chainHead);      // written by the launch of the chain's first pool
+        if (op.tail >= 0) touch(ops[static_cast<size_t>(op.tail)].out, i);   // may be written by this launch (msnh_hip_conv2d_tail)
     }
     {
         // the heads of a detector may all be decoded by one launch where the last of them stands (findYoloHeads): their inputs
@@ -827,7 +854,45 @@ static std::string tuneSignature(const Plan &plan, const PlanOp &op)
     os << static_cast<int>(op.kind) << ' ' << in.n << ' ' << in.h << ' ' << in.w << ' ' << in.c << ' ' << plan.ld(op.in0) << ' ' << out.c << ' '
        << plan.ld(op.out) << ' ' << op.ksize << ' ' << op.stride << ' ' << op.pad << ' ' << op.dilation << ' ' << op.groups << ' ' << (op.in1 >= 0) << ' '
        << in.dtype << ' ' << out.dtype;
+    if (op.tail >= 0) os << " tail " << plan.tensors[static_cast<size_t>(plan.ops[static_cast<size_t>(op.tail)].out)].c;
     return os.str();
+}
+
+static msnh_conv_tail_desc tailDesc(const Plan &plan, const PlanOp &op)
+{
+    const PlanOp &b = plan.ops[static_cast<size_t>(op.tail)];
+    msnh_conv_tail_desc t;
+    std::memset(&t, 0, sizeof(t));
+    t.out_c = plan.tensors[static_cast<size_t>(b.out)].c;
+    t.out_ld = plan.ld(b.out);
+    t.act = static_cast<int>(b.act);
+    t.act_param = b.actParam;
+    t.out_mul = 1.f / plan.mulOf(b.out);
+    t.write_y = op.tailSkipY ? 0 : 1;
+    return t;
+}
+
+// The choice between one launch and two is the first op's algorithm; the 1x1 op follows it.
+void Plan::applyTails()
+{
+    for (PlanOp &a : ops)
+    {
+        if (a.tail < 0) continue;
+        PlanOp &b = ops[static_cast<size_t>(a.tail)];
+        if (a.ownFlops == 0) a.ownFlops = a.flops;
+        const bool fused = !a.dead && a.algo == MSNH_CONV_IGEMM_TAIL;
+        b.dead = fused;
+        a.flops = a.ownFlops + (fused ? b.flops : 0.0);
+        // the first convolution's own result stays on the chip when the 1x1 is its only reader: a plain tensor (no view of or into
+        // another), not kept for the caller, read by no other live op
+        const PlanTensor &y = tensors[static_cast<size_t>(a.out)];
+        bool alone = fused && y.parent < 0 && !y.pinned && !y.persistent && !y.external && consumerCount(a.out) == 0;
+        for (size_t t = 0; alone && t < tensors.size(); ++t)
+            if (tensors[t].parent == a.out) alone = false;
+        for (size_t t = 0; alone && t < layerOut.size(); ++t)
+            if (layerOut[t] == a.out && t + 1 == layerOut.size()) alone = false;
+        a.tailSkipY = alone;
+    }
 }
 
 static std::string tuneHeader(int nTiles, bool preferWinograd)
@@ -863,7 +928,7 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
     // the same kernels and give the same bits), and the cache file beside the weights.
     static std::mutex memoMutex;
     static std::map<std::string, std::string> memoText;
-    const std::string memoKey = tuneHeader(nTiles, preferWinograd) + " " + std::to_string(structureHash());
+    const std::string memoKey = tuneHeader(nTiles, preferWinograd) + " " + std::to_string(structureHash()) + (forceTail ? " tails forced" : "");
     const auto adopt = [&](std::istream &f) -> bool {
         // file: header, then "<signature> | <algo> <tile>" per tunable launch in plan order; any mismatch discards the file
         std::string line;
@@ -876,7 +941,8 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
             ok = ok && bar != std::string::npos && line.substr(0, bar) == tuneSignature(*this, ops[tunedOps[k]]);
             int algo = 0, tile = 0;
             ok = ok && std::sscanf(line.c_str() + bar + 3, "%d %d", &algo, &tile) == 2 && tile >= 0 && tile <= nTiles &&
-                 (algo == MSNH_CONV_IGEMM || algo == MSNH_CONV_WINOGRAD || algo == MSNH_CONV_IGEMM_SPLITK || algo == MSNH_CONV_POINTWISE);
+                 (algo == MSNH_CONV_IGEMM || algo == MSNH_CONV_WINOGRAD || algo == MSNH_CONV_IGEMM_SPLITK || algo == MSNH_CONV_POINTWISE ||
+                  (algo == MSNH_CONV_IGEMM_TAIL && ops[tunedOps[k]].tail >= 0));
             if (ok) picks.emplace_back(algo, tile);
         }
         if (ok)
@@ -893,6 +959,15 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
                 if ((picks[k].first == MSNH_CONV_WINOGRAD) != (op.algo == MSNH_CONV_WINOGRAD)) ok = false;
                 op.algo = picks[k].first; op.tile = picks[k].second;
                 const msnh_conv_desc d = convDesc(*this, op);
+                if (op.algo == MSNH_CONV_IGEMM_TAIL)
+                {
+                    // one launch for this op and its 1x1 consumer: both were packed for the implicit GEMM
+                    const msnh_conv_tail_desc t = tailDesc(*this, op);
+                    msnh_conv_desc c = d;
+                    c.algo = MSNH_CONV_IGEMM;
+                    if (before.back().first != MSNH_CONV_IGEMM || ops[static_cast<size_t>(op.tail)].algo == MSNH_CONV_WINOGRAD || !msnh_hip_conv2d_tail_supported(&c, &t, op.tile)) ok = false;
+                    continue;
+                }
                 if (!msnh_hip_conv2d_tile_supported(&d, op.tile)) ok = false;
                 if (op.kind == PlanOp::CONV && op.wDev.bytes() != msnh_hip_conv2d_packed_weight_elems(&d, op.algo) * (d.dtype == MSNH_F16 ? 2u : 4u)) ok = false;
                 need = std::max(need, msnh_hip_conv2d_workspace_bytes(&d, op.algo));
@@ -900,6 +975,7 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
             if (ok)
             {
                 if (need > _convWorkspace.bytes()) _convWorkspace.alloc(need);
+                applyTails();
                 return true;
             }
             for (size_t k = 0; k < tunedOps.size(); ++k) { ops[tunedOps[k]].algo = before[k].first; ops[tunedOps[k]].tile = before[k].second; }
@@ -1031,6 +1107,56 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
         op.tile = best;
         memo.emplace_back(key, bestAlgo * 1000 + best);
     }
+    // Pairs marked by fuse (e): the two launches as chosen above, back to back, against one launch on every tile that carries a tail.
+    {
+        struct PairKey { std::string a, b; int tile; };
+        std::vector<PairKey> pairMemo;              // identical pairs share one comparison; tile 0 = two launches
+        for (PlanOp &a : ops)
+        {
+            if (a.dead || a.tail < 0 || a.kind != PlanOp::CONV || a.algo != MSNH_CONV_IGEMM) continue;
+            PlanOp &b = ops[static_cast<size_t>(a.tail)];
+            if (b.dead || (b.algo != MSNH_CONV_IGEMM && b.algo != MSNH_CONV_POINTWISE)) continue;
+            const std::string ka = tuneSignature(*this, a), kb = tuneSignature(*this, b);
+            const int twoTile = a.tile;
+            bool found = false;
+            for (const PairKey &m : pairMemo)
+                if (m.a == ka && m.b == kb)
+                {
+                    if (m.tile > 0) { a.algo = MSNH_CONV_IGEMM_TAIL; a.tile = m.tile; }
+                    found = true;
+                    break;
+                }
+            if (found) continue;
+            const auto timePair = [&](int reps) {
+                for (int r = 0; r < 2; ++r) { launch(a, s); if (a.algo != MSNH_CONV_IGEMM_TAIL) launch(b, s); }
+                MSNH_DEV(msnh_hip_event_record(e0, s));
+                for (int r = 0; r < reps; ++r) { launch(a, s); if (a.algo != MSNH_CONV_IGEMM_TAIL) launch(b, s); }
+                MSNH_DEV(msnh_hip_event_record(e1, s));
+                MSNH_DEV(msnh_hip_event_sync(e1));
+                float ms = 0.f;
+                MSNH_DEV(msnh_hip_event_elapsed_ms(e0, e1, &ms));
+                return ms / static_cast<float>(reps);
+            };
+            // One launch has to win by a margin: timed alone and repeated, the pair's second launch finds its input in the caches more
+            // reliably than it does inside a forward, and a tie here was a small loss there.
+            float bestMs = timePair(16) * (forceTail ? 1.f : 0.95f);
+            int bestTile = 0;
+            const msnh_conv_tail_desc t = tailDesc(*this, a);
+            for (int tile = msnh_hip_conv2d_tail_tile_first(); tile <= nTiles; ++tile)
+            {
+                msnh_conv_desc c = convDesc(*this, a);
+                c.algo = MSNH_CONV_IGEMM;
+                if (!msnh_hip_conv2d_tail_supported(&c, &t, tile)) continue;
+                a.algo = MSNH_CONV_IGEMM_TAIL; a.tile = tile;
+                const float ms = timePair(16);
+                if (ms < bestMs || (forceTail && bestTile == 0)) { bestMs = ms; bestTile = tile; }
+            }
+            if (bestTile > 0) { a.algo = MSNH_CONV_IGEMM_TAIL; a.tile = bestTile; }
+            else { a.algo = MSNH_CONV_IGEMM; a.tile = twoTile; }
+            pairMemo.push_back({ka, kb, bestTile});
+        }
+    }
+    applyTails();
     msnh_hip_event_destroy(e0);
     msnh_hip_event_destroy(e1);
     std::ostringstream text;
@@ -1103,6 +1229,20 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
             const msnh_mbconv_desc md = mbconvDesc(*this, op);
             if (op.wDev.bytes() != msnh_hip_mbconv_packed_bytes(&md)) MSNH_THROW("mbconv weights on the device do not fit this launch (" + op.name + ")");
             MSNH_DEV(msnh_hip_mbconv(&md, ptr(op.in0), op.wDev.ptr(), op.scaleDev.as<float>(), op.shiftDev.as<float>(), op.in1 >= 0 ? ptr(op.in1) : nullptr, ptr(op.out), s));
+            break;
+        }
+        if (op.algo == MSNH_CONV_IGEMM_TAIL)
+        {
+            if (op.tail < 0) MSNH_THROW("no 1x1 convolution follows this launch (" + op.name + ")");
+            const PlanOp &b = ops[static_cast<size_t>(op.tail)];
+            msnh_conv_desc c = convDesc(*this, op);
+            c.algo = MSNH_CONV_IGEMM;
+            msnh_conv_tail_desc t = tailDesc(*this, op);
+            if (_tailWriteAll) t.write_y = 1;
+            if (op.wDev.bytes() != msnh_hip_conv2d_packed_weight_elems(&c, MSNH_CONV_IGEMM) * 2u || b.wDev.bytes() != static_cast<size_t>(t.out_c) * c.out_c * 2u)
+                MSNH_THROW("conv weights on the device are not packed for the algorithm of this launch (" + op.name + ")");
+            MSNH_DEV(msnh_hip_conv2d_tail(&c, &t, ptr(op.in0), op.wDev.ptr(), op.scaleDev.as<float>(), op.shiftDev.as<float>(), op.in1 >= 0 ? ptr(op.in1) : nullptr,
+                                          ptr(op.out), b.wDev.ptr(), b.scaleDev.as<float>(), b.shiftDev.as<float>(), ptr(b.out), s));
             break;
         }
         const msnh_conv_desc d = convDesc(*this, op);
@@ -1280,7 +1420,7 @@ void Plan::exportTensor(int t, std::vector<float> &dst, msnh_stream_t s)
 std::string Plan::describe() const
 {
     static const char *kinds[] = {"conv", "affine", "add", "copy", "maxpool", "avgpool", "upsample", "connected", "input_cast", "yolo_decode", "pad", "slice", "bilinear", "softmax", "col2im"};
-    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk", "pointwise", "stem+down", "winograd_fused", "mbconv"};
+    static const char *algos[] = {"auto", "direct", "igemm", "depthwise", "winograd", "stem", "igemm_splitk", "pointwise", "stem+down", "winograd_fused", "mbconv", "igemm+1x1"};
     std::ostringstream os;
     os << "plan: " << liveOps() << " launches, " << tensors.size() << " tensors, arena " << _arena.bytes() / (1024.0 * 1024.0) << " MiB, dtype "
        << (computeDtype == MSNH_F16 ? "f16" : "f32") << "\n";

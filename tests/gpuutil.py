@@ -65,6 +65,54 @@ def rel_err(a, b):
     return float(np.abs(a[fb] - b[fb]).max() / max(np.abs(b[fb]).max(), 1e-30))
 
 
+def conv2d_tail(x, w_oihw, w2_oi, *, stride=1, pad=0, scale=None, shift=None, act="none", act_param=0.1, residual=None, act2="none", res_mul=1.0, out_mul=1.0,
+                scale2=None, shift2=None, act3="none", act3_param=0.1, z_mul=1.0, write_y=True, tile=0, in_ld=None, out_ld=None, res_ld=None, z_ld=None):
+    """msnh_hip_conv2d_tail, float16: x NCHW float32 numpy, w_oihw the first convolution's filters, w2_oi [out_c2][out_c] the 1x1 filters.
+    Returns (y, z) as NCHW float32 numpy; y is None when write_y is False (the buffer is then checked to be untouched)."""
+    init()
+    L = abi.lib()
+    b, c, h, wd = x.shape
+    oc, _, k, _ = w_oihw.shape
+    oc2 = w2_oi.shape[0]
+    oh = (h + 2 * pad - k) // stride + 1
+    ow = (wd + 2 * pad - k) // stride + 1
+    d = abi.ConvDesc(abi.F16, abi.F16, b, h, wd, c, in_ld or c, oc, oh, ow, out_ld or oc, k, stride, pad, 1, 1, abi.ACT[act], act_param,
+                     1 if residual is not None else 0, res_ld or oc, abi.ACT[act2], 0.1, res_mul, out_mul, abi.ALGO["igemm"], tile)
+    t = abi.ConvTailDesc(oc2, z_ld or oc2, abi.ACT[act3], act3_param, z_mul, 1 if write_y else 0)
+    if not L.msnh_hip_conv2d_tail_supported(ctypes.byref(d), ctypes.byref(t), tile):
+        return None
+    fp = ctypes.POINTER(ctypes.c_float)
+
+    def pack(desc, w4):
+        n = L.msnh_hip_conv2d_packed_weight_elems(ctypes.byref(desc), abi.ALGO["igemm"])
+        packed = np.zeros(n, np.float16)
+        wf = np.ascontiguousarray(w4, np.float32)
+        abi.check(L.msnh_hip_conv2d_pack_weights(ctypes.byref(desc), abi.ALGO["igemm"], wf.ctypes.data_as(fp), packed.ctypes.data_as(ctypes.c_void_p)))
+        return dev(packed)
+
+    wdev = pack(d, w_oihw)
+    d2 = abi.ConvDesc(abi.F16, abi.F16, b, oh, ow, oc, out_ld or oc, oc2, oh, ow, z_ld or oc2, 1, 1, 0, 1, 1, abi.ACT[act3], act3_param, 0, oc2, abi.ACT["none"], 0.1,
+                      1.0, z_mul, abi.ALGO["igemm"], 0)
+    w2dev = pack(d2, w2_oi.reshape(oc2, oc, 1, 1))
+    xdev = nhwc_dev(x, abi.F16, in_ld)
+    ydev = torch.full((b, oh, ow, out_ld or oc), 3.0, dtype=torch.float16).cuda()
+    zdev = torch.full((b, oh, ow, z_ld or oc2), 5.0, dtype=torch.float16).cuda()
+    mk = lambda v: dev(np.asarray(v, np.float32)) if v is not None else None
+    sdev, hdev, s2dev, h2dev = mk(scale), mk(shift), mk(scale2), mk(shift2)
+    rdev = nhwc_dev(residual, abi.F16, res_ld) if residual is not None else None
+    sync()
+    abi.check(L.msnh_hip_conv2d_tail(ctypes.byref(d), ctypes.byref(t), ptr(xdev), ptr(wdev), ptr(sdev), ptr(hdev), ptr(rdev), ptr(ydev), ptr(w2dev), ptr(s2dev),
+                                     ptr(h2dev), ptr(zdev), None))
+    sync()
+    if (out_ld or oc) > oc:
+        assert (ydev[..., oc:].float().cpu().numpy() == 3.0).all(), "kernel wrote outside y's channel slice"
+    if (z_ld or oc2) > oc2:
+        assert (zdev[..., oc2:].float().cpu().numpy() == 5.0).all(), "kernel wrote outside z's channel slice"
+    if not write_y:
+        assert (ydev.float().cpu().numpy() == 3.0).all(), "y was written although write_y is 0"
+    return (nchw_host(ydev, oc) if write_y else None), nchw_host(zdev, oc2)
+
+
 def conv2d(x, w_oihw, *, dtype, out_dtype=None, stride=1, pad=0, dil=1, groups=1, scale=None, shift=None, act="none",
            act_param=0.1, residual=None, act2="none", act2_param=0.1, res_mul=1.0, out_mul=1.0, algo="auto",
            in_ld=None, out_ld=None, res_ld=None, tile=0):

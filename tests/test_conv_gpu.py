@@ -476,3 +476,77 @@ def test_conv_stem_down(b, h, w, c2, act):
     ref = _ref(mid, gu.round_f16(w2), 2, 1, 1, 1, s2 / np.float32(mid_mul), h2, act, 0.1, None, "none", 1.0, out_mul)
     assert got.shape == ref.shape
     assert gu.rel_err(got, ref) <= 2e-3
+
+
+TAIL_CASES = [
+    # b, c, h, w, oc, k, stride, pad, oc2, residual
+    (2, 128, 19, 19, 256, 3, 1, 1, 128, True),       # the 76x76 residual stage of Darknet-53, reduced
+    (1, 64, 13, 17, 256, 3, 1, 1, 128, False),
+    (2, 128, 20, 20, 256, 3, 2, 1, 128, False),      # the stride-2 convolution in front of a stage
+    (1, 64, 9, 11, 200, 3, 1, 1, 72, True),          # channel counts below the tile's
+    (1, 256, 14, 14, 128, 1, 1, 0, 64, True),        # 1x1 in front
+    (3, 128, 16, 16, 128, 3, 1, 1, 128, True),       # the 128-channel tile
+    (1, 32, 30, 30, 64, 3, 1, 1, 32, False),
+]
+
+
+@pytest.mark.parametrize("case", TAIL_CASES)
+@pytest.mark.parametrize("write_y", [True, False])
+def test_conv_tail(case, write_y):
+    """msnh_hip_conv2d_tail (a convolution and the 1x1 convolution that reads its result, one launch) on every tile that carries a tail:
+    y and z against the oracle's two convolutions (y rounded to float16 in between, as two launches round it), and bit for bit against
+    msnh_hip_conv2d called twice."""
+    import gpuutil as gu
+    L = abi.lib()
+    b, c, h, w, oc, k, stride, pad, oc2, with_res = case
+    rng = np.random.default_rng(hash(case) % (2 ** 31))
+    x, wt = _case(rng, b, c, h, w, oc, k)
+    w2 = (rng.standard_normal((oc2, oc), dtype=np.float32) * np.float32(np.sqrt(2.0 / oc)))
+    oh, ow = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
+    res = gu.round_f16(rng.standard_normal((b, oc, oh, ow), dtype=np.float32)) if with_res else None
+    scale = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    shift = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    scale2 = rng.uniform(0.5, 1.5, oc2).astype(np.float32)
+    shift2 = (rng.standard_normal(oc2) * 0.1).astype(np.float32)
+    x, wt, w2 = gu.round_f16(x), gu.round_f16(wt), gu.round_f16(w2)
+    kw = dict(stride=stride, pad=pad, scale=scale, shift=shift, act="leaky", residual=res, act2="none", res_mul=2.0, out_mul=0.5)
+    ran = 0
+    first = L.msnh_hip_conv2d_tail_tile_first()
+    for tile in [0] + list(range(first, L.msnh_hip_conv2d_tile_count() + 1)):
+        got = gu.conv2d_tail(x, wt, w2, **kw, scale2=scale2, shift2=shift2, act3="leaky", z_mul=2.0, write_y=write_y, tile=tile,
+                             in_ld=c + 8, out_ld=oc + 8, res_ld=oc + 16 if with_res else None, z_ld=oc2 + 8)
+        if got is None:
+            continue
+        ran += 1
+        y, z = got
+        y_ref = gu.round_f16(_ref(x, wt, stride, pad, 1, 1, scale, shift, "leaky", 0.1, res, "none", 2.0, 0.5))
+        z_ref = _ref(y_ref, w2.reshape(oc2, oc, 1, 1), 1, 0, 1, 1, scale2, shift2, "leaky", 0.1, None, "none", 1.0, 2.0)
+        if write_y:
+            assert gu.rel_err(y, y_ref) <= TOL[abi.F16], tile
+        assert gu.rel_err(z, z_ref) <= 2 * TOL[abi.F16], tile     # z sees y's own rounding differences as well
+        # two launches of msnh_hip_conv2d: the same bits
+        y2, _ = gu.conv2d(x, wt, dtype=abi.F16, **kw, algo="igemm", tile=37 if oc > 128 else 38, in_ld=c + 8, out_ld=oc + 8, res_ld=oc + 16 if with_res else None)
+        z2, _ = gu.conv2d(y2, w2.reshape(oc2, oc, 1, 1), dtype=abi.F16, scale=scale2, shift=shift2, act="leaky", out_mul=2.0, algo="igemm", tile=38)
+        if write_y:
+            assert np.array_equal(y, y2), tile
+        assert np.array_equal(z, z2), tile
+    assert ran >= 1
+
+
+def test_conv_tail_rejects():
+    L = abi.lib()
+    mk = lambda **kw: abi.ConvDesc(**{**dict(dtype=abi.F16, out_dtype=abi.F16, batch=1, in_h=8, in_w=8, in_c=64, in_ld=64, out_c=128, out_h=8, out_w=8, out_ld=128,
+                                             ksize=3, stride=1, pad=1, dilation=1, groups=1, act=22, act_param=0.1, has_residual=0, res_ld=128, act2=22,
+                                             act2_param=0.1, res_mul=1.0, out_mul=1.0, algo=abi.ALGO["igemm"], tile=0), **kw})
+    tk = lambda **kw: abi.ConvTailDesc(**{**dict(out_c=64, out_ld=64, act=22, act_param=0.1, out_mul=1.0, write_y=1), **kw})
+    ok = lambda d, t, tile=0: L.msnh_hip_conv2d_tail_supported(ctypes.byref(d), ctypes.byref(t), tile)
+    assert ok(mk(), tk()) == 1
+    assert ok(mk(out_c=512, out_ld=512, res_ld=512), tk()) == 0          # more channels than a tile holds
+    assert ok(mk(), tk(out_c=256, out_ld=256)) == 0                      # more tail channels than the epilogue stages
+    assert ok(mk(), tk(out_c=60, out_ld=64)) == 0
+    assert ok(mk(groups=2), tk()) == 0
+    assert ok(mk(dtype=abi.F32, out_dtype=abi.F32), tk()) == 0
+    assert ok(mk(), tk(), 37) == 0                                       # a tile without a tail
+    # ... and a tile with a tail does not run a plain convolution
+    assert L.msnh_hip_conv2d_tile_supported(ctypes.byref(mk()), L.msnh_hip_conv2d_tail_tile_first()) == 0
+    assert L.msnh_hip_conv2d_tail(ctypes.byref(mk()), ctypes.byref(tk()), None, None, None, None, None, None, None, None, None, None, None) != 0

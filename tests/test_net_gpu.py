@@ -603,6 +603,41 @@ def test_inverted_residual_blocks_run_as_one_launch():
         assert np.array_equal(fused, m.run_classify(x))
 
 
+def test_conv_with_its_1x1_consumer_as_one_launch():
+    """float16 YOLOv3: a convolution whose tile holds all its output channels (the 3x3 convolutions with 256 filters and fewer) can compute
+    the 1x1 convolution that reads its result in the same launch (msnh_hip_conv2d_tail).  Off by default (it measured level with two
+    launches inside a forward); MSNH_CONV_TAIL=1 lets the load-time search decide per pair; forced on here (MSNH_FORCE_CONV_TAIL).
+    The launch itself returns the bits of two launches on the same tiles (tests/test_conv_gpu.py::test_conv_tail); two networks tuned
+    separately may settle on different tiles for a layer, which changes float32 summation orders, so the comparison of the whole network
+    with the default plan is to float16 accuracy: head logits within 5e-3 of their largest value (two default plans tuned separately
+    have been seen 2e-3 apart on this network), as many boxes to within 1 %."""
+    batch, size = 2, 160
+    net, binp, g = nu.model("yolov3", batch, size, seed=5)
+    x = zoo.seeded_input(batch, 3, size, size, seed=6)
+    m0 = netapi.Net(net, binp, fp16=True)
+    assert "igemm+1x1" not in m0.plan_detail()
+    launches = int(m0.plan_detail().split(" launches")[0].split()[-1])
+    want = m0.run_yolo(x)
+    want_heads = [m0.yolo_head_logits(h) for h in range(3)]
+    os.environ["MSNH_FORCE_CONV_TAIL"] = "1"
+    try:
+        m = netapi.Net(net, binp, fp16=True)
+    finally:
+        del os.environ["MSNH_FORCE_CONV_TAIL"]
+    detail = m.plan_detail()
+    fused = [ln for ln in detail.splitlines() if "conv[igemm+1x1" in ln]
+    assert len(fused) >= 10, detail
+    assert int(detail.split(" launches")[0].split()[-1]) == launches - len(fused)
+    got = m.run_yolo(x)
+    for h in range(3):
+        e = nu.rel_err(m.yolo_head_logits(h), want_heads[h])
+        print("head", h, "one launch per pair against two:", e, flush=True)
+        assert e <= 5e-3, h
+    for a, b in zip(got, want):
+        assert len(b) > 0 and abs(len(a) - len(b)) <= max(2, len(b) // 100)
+    assert all(np.array_equal(a, b, equal_nan=True) for a, b in zip(m.run_yolo(x), got))
+
+
 def test_image_in_boxes_out():
     """8-bit images of different shapes -> device letterbox -> forward -> boxes in original-image pixels: equals the
     float path fed with the restatement's letterbox, followed by the restatement's rescale."""
