@@ -147,6 +147,28 @@ inline bool actOk(int act)
            act == MSNH_ACT_SWISH || act == MSNH_ACT_HARD_SWISH || act == MSNH_ACT_MISH || act == MSNH_ACT_NONE;
 }
 
+// Division of a 32-bit unsigned by a divisor known on the host: multiplication by a precomputed reciprocal (Granlund & Montgomery,
+// "Division by invariant integers using multiplication", figure 4.1); exact for every 32-bit dividend.
+struct FastDiv { unsigned m, s1, s2, d; };
+
+inline FastDiv makeFastDiv(unsigned d)
+{
+    unsigned l = 0;
+    while ((1ull << l) < d) ++l;                     // ceil(log2 d)
+    FastDiv f;
+    f.m = static_cast<unsigned>(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+    f.s1 = l < 1 ? l : 1;
+    f.s2 = l > 1 ? l - 1 : 0;
+    f.d = d;
+    return f;
+}
+
+__device__ __forceinline__ unsigned fastDiv(unsigned n, const FastDiv &f)
+{
+    const unsigned t = __umulhi(f.m, n);
+    return (t + ((n - t) >> f.s1)) >> f.s2;
+}
+
 inline unsigned gridFor(long long n, int block)
 {
     long long g = (n + block - 1) / block;

@@ -137,25 +137,6 @@ __global__ __launch_bounds__(256) void convDepthwise3x3Kernel(DwArgs a, int bloc
 // (Granlund & Montgomery, "Division by invariant integers using multiplication", figure 4.1), every address a 32-bit buffer offset,
 // and the stores past the row's end out-of-range offsets instead of branches.
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
-struct FastDiv { unsigned m, s1, s2, d; };
-
-inline FastDiv makeFastDiv(unsigned d)
-{
-    unsigned l = 0;
-    while ((1ull << l) < d) ++l;                     // ceil(log2 d)
-    FastDiv f;
-    f.m = static_cast<unsigned>(((1ull << 32) * ((1ull << l) - d)) / d + 1);
-    f.s1 = l < 1 ? l : 1;
-    f.s2 = l > 1 ? l - 1 : 0;
-    f.d = d;
-    return f;
-}
-
-__device__ __forceinline__ unsigned fastDiv(unsigned n, const FastDiv &f)
-{
-    const unsigned t = __umulhi(f.m, n);
-    return (t + ((n - t) >> f.s1)) >> f.s2;
-}
 
 struct DwFastArgs
 {

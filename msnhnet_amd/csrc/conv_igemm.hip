@@ -41,6 +41,8 @@ static int convIgemmAny(const msnh_conv_desc *d, const void *x, const void *w, c
     a.cinG = d->in_c / d->groups; a.coutG = d->out_c / d->groups;
     a.taps = d->ksize * d->ksize; a.ksize = d->ksize; a.stride = d->stride; a.pad = d->pad; a.dil = d->dilation;
     a.P = d->batch * d->out_h * d->out_w;
+    a.byOW = makeFastDiv(static_cast<unsigned>(d->out_w));
+    a.byOH = makeFastDiv(static_cast<unsigned>(d->out_h));
     a.patchOk = (d->ksize == 3 && d->stride == 1 && d->pad == 1 && d->dilation == 1 && d->groups == 1 && d->out_h == d->in_h && d->out_w == d->in_w) ? 1 : 0;
     a.patchRows = 0; a.mTiles = 0; a.cChunks = 0; a.nIter = 0;
     a.dryRun = dryRun ? 1 : 0;

@@ -48,6 +48,7 @@ struct IgemmArgs
     int buffersOk;          // both extents fit a buffer resource
     int act, act2, hasRes, vecOk;
     float actParam, act2Param, resMul, outMul;
+    FastDiv byOW, byOH;     // pixel index -> (image, row, column) without hardware-less integer division
     // tail (tiles with TAIL = 1 only): a 1x1 stride-1 convolution z = zMul * act3(scale2 * (W2 . y) + shift2) of this convolution's
     // float16 result y, computed by the same workgroup from the copy of its y tile in LDS
     int tailOn;             // the launch carries a tail (set by the tail entry point, also for dry runs)
@@ -197,9 +198,12 @@ template <int I, int N, typename F> __device__ __forceinline__ void staticFor(F 
 
 template <int BM, int TM, int NW = 4> constexpr size_t igemmEpilogueLds() { return (2 * BM + NW * 32 * (TM + 4)) * sizeof(float); }
 
+// ssReady / stageOwn (the K-split epilogue): the affines already stand at ssReady, published by a barrier the caller has passed, and this
+// wavefront stages in stageOwn (32 x (TM + 4) floats of its own) -- then the epilogue meets no workgroup barrier at all.
 template <typename T, typename TOut, int BM, int BN, int TM, int TN>
 __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[TM / 32][TN / 32], unsigned char *smemRaw, float chScale,
-                                              float chShift, int m0, int p0, int wm, int wn, int wave, int lane, int g)
+                                              float chShift, int m0, int p0, int wm, int wn, int wave, int lane, int g,
+                                              float *ssReady = nullptr, float *stageOwn = nullptr)
 {
     constexpr int MB  = TM / 32;
     constexpr int NB  = TN / 32;
@@ -208,11 +212,14 @@ __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[
     constexpr int RPI = 64 / VPR;                     // pixels covered per pass of the wave
     constexpr int PASSES = 32 / RPI;
     static_assert(BM <= 256 && VPR <= 32, "epilogue geometry");
-    float *ss    = reinterpret_cast<float *>(smemRaw);                 // [BM] scale, [BM] shift
-    float *stage = ss + 2 * BM + wave * (32 * LDE);
+    float *ss    = ssReady ? ssReady : reinterpret_cast<float *>(smemRaw);                 // [BM] scale, [BM] shift
+    float *stage = stageOwn ? stageOwn : ss + 2 * BM + wave * (32 * LDE);
     const int tid = wave * 64 + lane;
-    if (tid < BM) { ss[tid] = chScale; ss[BM + tid] = chShift; }
-    __syncthreads();
+    if (!ssReady)
+    {
+        if (tid < BM) { ss[tid] = chScale; ss[BM + tid] = chShift; }
+        __syncthreads();
+    }
 
     const int chBase = g * a.coutG;
     const int vcol = (lane % VPR) * 8;
@@ -281,7 +288,12 @@ __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[
             }
         };
         if (lin1) stageBlock(std::true_type()); else stageBlock(std::false_type());
-        __syncthreads();
+        // the staging area belongs to this wavefront alone, and the LDS serves a wavefront's accesses in the order it issued them: the
+        // reads below see the writes above without a workgroup barrier (a barrier here kept the twelve wavefronts of a tile in step
+        // through their stores)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
         auto storeBlock = [&](auto slopeTag) {
             constexpr bool SL = decltype(slopeTag)::value;
@@ -335,40 +347,55 @@ __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[
             }
         };
         if (lin2) storeBlock(std::true_type()); else storeBlock(std::false_type());
-        if (j + 1 < NB) __syncthreads();
+        if (j + 1 < NB)
+        {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
     });
 }
 
 // Epilogue of the kernels whose wavefronts come in two groups that multiplied different k-blocks of the same 64 x 64 wave tile
 // (kg = group, wt = wave tile index): group g keeps pixel block g of the tile, parks the other block's partial sums in LDS for
 // its partner and adds what the partner parked for it; then the ordinary epilogue runs over 64 x 32 per wavefront.
-// LDS: 8 KiB per wavefront (igemmSwapLds).
-template <int NW> constexpr size_t igemmSwapLds() { return static_cast<size_t>(NW) * 2 * 16 * 64 * sizeof(float); }
+// One workgroup barrier in all: the affines are written in front of it, into the area behind the wavefronts' regions, and a wavefront stages
+// its block (32 pixels x 68 floats) in the region it has just emptied -- the one its partner filled for it, which nobody else touches.
+// LDS: 32 x 68 floats per wavefront + the affines (igemmSwapLds).
+constexpr int kSwapRegion = 32 * (64 + 4);         // floats per wavefront: the staging block of a 64-channel wave tile, which holds the 2048 parked sums
+template <int NW, int BM> constexpr size_t igemmSwapLds() { return (static_cast<size_t>(NW) * kSwapRegion + 2 * BM) * sizeof(float); }
 
 template <typename T, typename TOut, int BM, int BN>
 __device__ __forceinline__ void igemmEpilogueSwap(const IgemmArgs &a, f32x16 (&acc)[2][2], unsigned char *smemRaw, float chScale, float chShift,
-                                                  int m0, int p0, int wm, int wn, int kg, int wt, int wave, int lane, int g)
+                                                  int m0, int p0, int wm, int wn, int kg, int wt, int wave, int lane, int g, int nWaves)
 {
-    constexpr int XW = 2 * 16 * 64;                   // floats a wavefront parks
     float *xch = reinterpret_cast<float *>(smemRaw);
+    float *ss  = xch + nWaves * kSwapRegion;
+    const int tid = wave * 64 + lane;
+    if (tid < BM) { ss[tid] = chScale; ss[BM + tid] = chShift; }
     f32x16 mine[2][1];
+    float *stageOwn = nullptr;
     auto swap = [&](auto gTag) {
         constexpr int q = decltype(gTag)::value;
-        float *put = xch + (wt * 2 + q) * XW + lane;
+        float *put = xch + (wt * 2 + q) * kSwapRegion + lane;
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int r = 0; r < 16; ++r) put[(i * 16 + r) * 64] = acc[i][1 - q][r];
         __syncthreads();
-        const float *get = xch + (wt * 2 + (1 - q)) * XW + lane;
+        stageOwn = xch + (wt * 2 + (1 - q)) * kSwapRegion;
+        const float *get = stageOwn + lane;
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int r = 0; r < 16; ++r) mine[i][0][r] = acc[i][q][r] + get[(i * 16 + r) * 64];
     };
     if (kg == 0) swap(std::integral_constant<int, 0>()); else swap(std::integral_constant<int, 1>());
-    __syncthreads();
-    igemmEpilogue<T, TOut, BM, BN, 64, 32>(a, mine, smemRaw, chScale, chShift, m0, p0, wm, wn * 2 + kg, wave, lane, g);
+    // (the partner's sums are in registers before the staging writes below reach the same region: one wavefront's LDS accesses are served in order)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    igemmEpilogue<T, TOut, BM, BN, 64, 32>(a, mine, smemRaw, chScale, chShift, m0, p0, wm, wn * 2 + kg, wave, lane, g, ss, stageOwn);
 }
 
 // Register budget: two workgroups per CU (one wave of each per SIMD) so that one workgroup's barrier and epilogue
@@ -760,23 +787,26 @@ void convIgemmKernel(IgemmArgs a)
         const int p = p0 + ldRow + i * RPP;
         const bool ok = p < a.P && ldRow + i * RPP < BN;
         const int pp = ok ? p : 0;
-        const int ox = pp % a.OW;
-        const int t  = pp / a.OW;
-        const int oy = t % a.OH;
-        const int b  = t / a.OH;
+        const int t  = static_cast<int>(fastDiv(static_cast<unsigned>(pp), a.byOW));
+        const int ox = pp - t * a.OW;
+        const int b  = static_cast<int>(fastDiv(static_cast<unsigned>(t), a.byOH));
+        const int oy = t - b * a.OH;
         const int iy0 = oy * a.stride - a.pad;
         const int ix0 = ox * a.stride - a.pad;
         const long long pix = (static_cast<long long>(b) * a.H + iy0) * a.W + ix0;
         bOff[i] = static_cast<unsigned>((pix * a.inLd + ldVec * VEC) * static_cast<long long>(ES));
+        // a tap lies inside the image when its row does and its column does: ksize row tests and ksize column tests instead of ksize^2 of both
+        unsigned rowBits = 0, colBits = 0;
+        for (int k = 0; k < a.ksize; ++k)
+        {
+            const int iy = iy0 + k * a.dil, ix = ix0 + k * a.dil;
+            rowBits |= ((iy >= 0 && iy < a.H) ? 1u : 0u) << k;
+            colBits |= ((ix >= 0 && ix < a.W) ? 1u : 0u) << k;
+        }
         unsigned long long mask = 0;
-        if (ok)
-            for (int ki = 0; ki < a.ksize; ++ki)
-                for (int kj = 0; kj < a.ksize; ++kj)
-                {
-                    const int iy = iy0 + ki * a.dil, ix = ix0 + kj * a.dil;
-                    if (iy >= 0 && iy < a.H && ix >= 0 && ix < a.W) mask |= 1ull << (ki * a.ksize + kj);
-                }
-        bMask[i] = mask;
+        for (int ki = 0; ki < a.ksize; ++ki)
+            if ((rowBits >> ki) & 1u) mask |= static_cast<unsigned long long>(colBits) << (ki * a.ksize);
+        bMask[i] = ok ? mask : 0ull;
     }
     unsigned aOff[AROWS];
 #pragma unroll
@@ -946,11 +976,11 @@ void convIgemmKernel(IgemmArgs a)
         e.y = a.ws + static_cast<size_t>(blockIdx.y) * a.P * a.wsLd;
         e.outLd = a.wsLd;
         e.vecOk = (a.wsLd % 8 == 0) && (a.coutG % 8 == 0 || gridDim.z == 1);
-        if constexpr (KG == 2) igemmEpilogueSwap<T, float, BM, BN>(e, acc, smemRaw, 1.f, 0.f, m0, p0, wm, wn, kg, wave % NWT, wave, lane, g);
+        if constexpr (KG == 2) igemmEpilogueSwap<T, float, BM, BN>(e, acc, smemRaw, 1.f, 0.f, m0, p0, wm, wn, kg, wave % NWT, wave, lane, g, NT / 64);
         else igemmEpilogue<T, float, BM, BN, TM, TN>(e, acc, smemRaw, 1.f, 0.f, m0, p0, wm, wn, wave, lane, g);
         return;
     }
-    if constexpr (KG == 2) igemmEpilogueSwap<T, TOut, BM, BN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, kg, wave % NWT, wave, lane, g);
+    if constexpr (KG == 2) igemmEpilogueSwap<T, TOut, BM, BN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, kg, wave % NWT, wave, lane, g, NT / 64);
     else igemmEpilogue<T, TOut, BM, BN, TM, TN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, wave, lane, g);
 }
 
@@ -1013,7 +1043,7 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
         constexpr unsigned STAGE = static_cast<unsigned>(((BM + RPP - 1) / RPP * RPP + (BN + RPP - 1) / RPP * RPP) * KV * 16);
         smemEpi = TailLds<BM, BN, STAGE>::bytes();
     }
-    else smemEpi = std::max(igemmEpilogueLds<BM, BM / WM, WM * WN * KG>(), KG == 2 ? igemmSwapLds<WM * WN * KG>() : size_t(0));
+    else smemEpi = std::max(igemmEpilogueLds<BM, BM / WM, WM * WN * KG>(), KG == 2 ? igemmSwapLds<WM * WN * KG, BM>() : size_t(0));
     const size_t smem = smemLoop > smemEpi ? smemLoop : smemEpi;
     a.mTiles = (a.coutG + BM - 1) / BM;
     const int tiles = a.mTiles * ((a.P + BN - 1) / BN);

@@ -123,14 +123,11 @@ void convPatch3x3Kernel(IgemmArgs a)
         unsigned m = 0;
         if (p < a.P)
         {
-            const int x = p % W;
-            const int y = (p / W) % H;
-#pragma unroll
-            for (int t = 0; t < 9; ++t)
-            {
-                const int yy = y + t / 3 - 1, xx = x + t % 3 - 1;
-                if (yy >= 0 && yy < H && xx >= 0 && xx < W) m |= 1u << t;
-            }
+            const int t = static_cast<int>(fastDiv(static_cast<unsigned>(p), a.byOW));      // (same-size output: OW = W, OH = H)
+            const int x = p - t * W;
+            const int y = t - static_cast<int>(fastDiv(static_cast<unsigned>(t), a.byOH)) * H;
+            const unsigned cols = (x > 0 ? 1u : 0u) | 2u | (x < W - 1 ? 4u : 0u);
+            m = (y > 0 ? cols : 0u) | (cols << 3) | (y < H - 1 ? cols << 6 : 0u);
         }
         tapOk[j] = m;
     }

@@ -144,14 +144,12 @@ void convPatch8Kernel(IgemmArgs a)
         unsigned m = 0;
         if (p < a.P)
         {
-            const int x = p % W;
-            const int y = (p / W) % H;
-#pragma unroll
-            for (int t = 0; t < 9; ++t)
-            {
-                const int yy = y + t / 3 - 1, xx = x + t % 3 - 1;
-                if (yy >= 0 && yy < H && xx >= 0 && xx < W) m |= 1u << t;
-            }
+            const int t = static_cast<int>(fastDiv(static_cast<unsigned>(p), a.byOW));      // (same-size output: OW = W, OH = H)
+            const int x = p - t * W;
+            const int y = t - static_cast<int>(fastDiv(static_cast<unsigned>(t), a.byOH)) * H;
+            // tap (ky, kx) lies inside the image when row y + ky - 1 and column x + kx - 1 do
+            const unsigned cols = (x > 0 ? 1u : 0u) | 2u | (x < W - 1 ? 4u : 0u);
+            m = (y > 0 ? cols : 0u) | (cols << 3) | (y < H - 1 ? cols << 6 : 0u);
         }
         tapOk[j] = m;
     }
@@ -315,7 +313,7 @@ void convPatch8Kernel(IgemmArgs a)
     if constexpr (KG == 1)
         igemmEpilogue<T, TOut, BM, BN, TM, TN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, wave, lane, 0);
     else
-        igemmEpilogueSwap<T, TOut, BM, BN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, kg, wave % NWT, wave, lane, 0);
+        igemmEpilogueSwap<T, TOut, BM, BN>(a, acc, smemRaw, chScale, chShift, m0, p0, wm, wn, kg, wave % NWT, wave, lane, 0, NW);
 }
 
 // Host-side check shared by launch and tile enumeration.
@@ -328,7 +326,7 @@ inline bool patch8Fits(const IgemmArgs &a, size_t *smemOut, int *slicesOut)
     const int slices = (R + 7) / 8;
     const int stages = a.cinG > BK ? 2 : 1;
     const size_t loop = static_cast<size_t>(NSA) * BM * 128 + static_cast<size_t>(stages) * slices * 1024 + 1024;
-    const size_t swap = KG == 2 ? igemmSwapLds<NW>() : 0;
+    const size_t swap = KG == 2 ? igemmSwapLds<NW, BM>() : 0;
     const size_t epiOnly = igemmEpilogueLds<BM, BM / WM, NW>();
     const size_t epi = epiOnly > swap ? epiOnly : swap;
     const size_t smem = loop > epi ? loop : epi;

@@ -58,6 +58,8 @@ extern "C" int msnh_hip_diag_patch8(int tile, int switches, int batch, int c, in
     a.batch = batch; a.H = h; a.W = w; a.inLd = c; a.OH = h; a.OW = w; a.outLd = oc; a.resLd = oc;
     a.cinG = c; a.coutG = oc; a.taps = 9; a.ksize = 3; a.stride = 1; a.pad = 1; a.dil = 1;
     a.P = batch * h * w; a.patchOk = 1; a.buffersOk = 1;
+    a.byOW = makeFastDiv(static_cast<unsigned>(w));
+    a.byOH = makeFastDiv(static_cast<unsigned>(h));
     a.xBytes = static_cast<unsigned>(xBytes);
     a.wBytes = static_cast<unsigned>(wBytes);
     a.act = MSNH_ACT_LEAKY; a.act2 = MSNH_ACT_NONE; a.actParam = 0.1f; a.resMul = 1.f; a.outMul = 1.f; a.vecOk = 1; a.wsLd = oc;
