@@ -205,6 +205,19 @@ int msnh_hip_conv_stem_down_pack(const float *w1, int c2, const float *w2, void 
 int msnh_hip_conv_stem_down(int batch, int h, int w, const float *x, const void *packed1, const float *scale1, const float *shift1, int act1,
                             float act1_param, float mid_mul, int c2, const void *packed2, const float *scale2, const float *shift2, int act2,
                             float act2_param, float out_mul, void *y, int y_ld, msnh_stream_t s);
+/* The same launch followed, inside it, by the 1x1 stride-1 convolution with c3 = 32 filters that reads its result -- the opening of Darknet-53's
+ * first residual block (a third ConvolutionalLayer::forwardGPU call, src/layers/MsnhConvolutionalLayer.cpp:984-1169, inside
+ * ResBlockLayer::forwardGPU, src/layers/MsnhResBlockLayer.cpp:215-302): z = z_mul * act3(scale3 * (w3 . y) + shift3) over y as rounded to
+ * float16 and stored (y is written as by msnh_hip_conv_stem_down: the block's residual add reads it), k in channel order as a separate launch
+ * sums it.  w3: [32][c2] float32 in `.msnhbin` order, packed by msnh_hip_conv_stem_down_tail_pack into msnh_hip_conv_stem_down_tail_packed_elems(c2)
+ * float16 elements; z: NHWC float16 with pixel stride z_ld (a multiple of 8), 16-byte aligned.  _supported: pure host function. */
+int msnh_hip_conv_stem_down_tail_supported(int c2, int c3, int k3, int s3, int p3);
+size_t msnh_hip_conv_stem_down_tail_packed_elems(int c2);
+int msnh_hip_conv_stem_down_tail_pack(int c2, const float *w3, void *packed3);
+int msnh_hip_conv_stem_down_tail(int batch, int h, int w, const float *x, const void *packed1, const float *scale1, const float *shift1, int act1,
+                                 float act1_param, float mid_mul, int c2, const void *packed2, const float *scale2, const float *shift2, int act2,
+                                 float act2_param, float out_mul, void *y, int y_ld, const void *packed3, const float *scale3, const float *shift3,
+                                 int act3, float act3_param, float z_mul, void *z, int z_ld, msnh_stream_t s);
 
 /* The inverted-residual block of MobileNetV2 as one launch, float16 NHWC: 1x1 convolution in_c -> exp_c, 3x3 depthwise convolution
  * (stride 1 or 2, pad 1) over the exp_c channels, 1x1 convolution exp_c -> out_c, each with its folded batch-norm and activation, then the

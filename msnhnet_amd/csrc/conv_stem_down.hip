@@ -14,6 +14,11 @@
 //      its A fragments (weights in MFMA lane order) straight from global memory one tap ahead, and writes NHWC float16.
 // Both MFMA row orders are the channel permutation that makes a lane's 16 accumulators 16 consecutive channels (row 8q + 4h + e
 // computes channel 16h + 4q + e).
+//   3. (msnh_hip_conv_stem_down_tail) the 1x1 convolution with 32 filters that reads the pair's result -- the opening of Darknet-53's
+//      first residual block -- computed by the same wavefront from its own 32 pixels without leaving the registers: a lane holds 16
+//      consecutive channels of its pixel as float16, which is two 8-channel halves of the B operand of a 32x32x16 MFMA; the half the
+//      lane's own operand slot does not take is the one its partner lane (same pixel, other half-wave) needs, and the other way round:
+//      one v_permlane32_swap per register.  K runs over the channels in order, as a separate 1x1 launch would.
 #include "common.hpp"
 
 namespace msnh {
@@ -41,6 +46,12 @@ struct StemDownArgs
     int B, H, W, OH, OW, outLd, tilesX, tilesY, total;
     int act1, act2;
     float act1Param, act2Param, midMul, outMul;
+    // tail: z = zMul * act3(scale3 * (w3 . y) + shift3), 32 filters over the C2 channels of y
+    const f16 *w3;          // [C2/32][2][64][8]
+    const float *scale3, *shift3;
+    f16 *z;
+    int zLd, act3;
+    float act3Param, zMul;
 };
 
 __device__ __forceinline__ unsigned sdSlotAddr(int slot, int chunk)
@@ -48,11 +59,11 @@ __device__ __forceinline__ unsigned sdSlotAddr(int slot, int chunk)
     return static_cast<unsigned>(slot) * 64u + static_cast<unsigned>((chunk ^ ((slot >> 1) & 3)) * 16);
 }
 
-template <int MB2>
+template <int MB2, int TAIL = 0>
 __global__ __launch_bounds__(256) void convStemDownKernel(StemDownArgs a)
 {
     __shared__ __attribute__((aligned(16))) unsigned char smem[SD_IMG_BYTES + SD_TILE_BYTES];
-    __shared__ float aff[2 * 32 + 2 * SD_MAXC2];
+    __shared__ float aff[2 * 32 + 2 * SD_MAXC2 + 2 * 32];
     float *imgL = reinterpret_cast<float *>(smem);
     unsigned char *tileL = smem + SD_IMG_BYTES;
 
@@ -94,8 +105,24 @@ __global__ __launch_bounds__(256) void convStemDownKernel(StemDownArgs a)
     const float late1 = hom1 ? 1.f : a.midMul, late2 = hom2 ? 1.f : a.outMul;
     if (tid < 32) { aff[tid] = fold1 * (a.scale1 ? a.scale1[tid] : 1.f); aff[32 + tid] = fold1 * (a.shift1 ? a.shift1[tid] : 0.f); }
     if (tid < MB2 * 32) { aff[64 + tid] = fold2 * (a.scale2 ? a.scale2[tid] : 1.f); aff[64 + SD_MAXC2 + tid] = fold2 * (a.shift2 ? a.shift2[tid] : 0.f); }
+    const bool hom3 = a.act3 == MSNH_ACT_NONE || a.act3 == MSNH_ACT_RELU || a.act3 == MSNH_ACT_LEAKY;
+    const float fold3 = hom3 ? a.zMul : 1.f, late3 = hom3 ? 1.f : a.zMul;
+    if (TAIL != 0 && tid < 32)
+    {
+        aff[64 + 2 * SD_MAXC2 + tid] = fold3 * (a.scale3 ? a.scale3[tid] : 1.f);
+        aff[64 + 2 * SD_MAXC2 + 32 + tid] = fold3 * (a.shift3 ? a.shift3[tid] : 0.f);
+    }
     const f16x8 w1a0 = *reinterpret_cast<const f16x8 *>(a.w1 + static_cast<size_t>(lane) * 8);
     const f16x8 w1a1 = *reinterpret_cast<const f16x8 *>(a.w1 + static_cast<size_t>(64 + lane) * 8);
+    // the 1x1 tail's operand A, asked for here so that the epilogue does not wait for it
+    f16x8 wa3[TAIL != 0 ? MB2 : 1][2];
+    if constexpr (TAIL != 0)
+    {
+#pragma unroll
+        for (int mb = 0; mb < MB2; ++mb)
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) wa3[mb][kb] = *reinterpret_cast<const f16x8 *>(a.w3 + static_cast<size_t>((mb * 2 + kb) * 64 + lane) * 8);
+    }
     __syncthreads();
 
     // ---- 1. first layer over the 17 x 33 pixels under the tile ------------------------------------------------------------------
@@ -189,21 +216,59 @@ __global__ __launch_bounds__(256) void convStemDownKernel(StemDownArgs a)
         }
     }
     const int oy = ty0 + ty, ox = tx0 + tx;
-    if (oy < a.OH && ox < a.OW)
+    const bool store = oy < a.OH && ox < a.OW;
+    const size_t pix = (static_cast<size_t>(b) * a.OH + (store ? oy : 0)) * a.OW + (store ? ox : 0);
+    f16 *yp = a.y + pix * a.outLd + 16 * g;
+    f32x16 accT;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) accT[r] = 0.f;
+#pragma unroll
+    for (int mb = 0; mb < MB2; ++mb)
     {
-        f16 *yp = a.y + ((static_cast<size_t>(b) * a.OH + oy) * a.OW + ox) * a.outLd + 16 * g;
+        float t[16];
 #pragma unroll
-        for (int mb = 0; mb < MB2; ++mb)
+        for (int r = 0; r < 16; ++r) t[r] = acc2[mb][r] * aff[64 + mb * 32 + 16 * g + r] + aff[64 + SD_MAXC2 + mb * 32 + 16 * g + r];
+        activateArray<16>(t, a.act2, a.act2Param);
+        f16x8 o0, o1;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) { o0[r] = static_cast<f16>(t[r] * late2); o1[r] = static_cast<f16>(t[8 + r] * late2); }
+        if (store)
         {
-            float t[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) t[r] = acc2[mb][r] * aff[64 + mb * 32 + 16 * g + r] + aff[64 + SD_MAXC2 + mb * 32 + 16 * g + r];
-            activateArray<16>(t, a.act2, a.act2Param);
-            f16x8 o0, o1;
-#pragma unroll
-            for (int r = 0; r < 8; ++r) { o0[r] = static_cast<f16>(t[r] * late2); o1[r] = static_cast<f16>(t[8 + r] * late2); }
             *reinterpret_cast<f16x8 *>(yp + mb * 32) = o0;
             *reinterpret_cast<f16x8 *>(yp + mb * 32 + 8) = o1;
+        }
+        if constexpr (TAIL != 0)
+        {
+            // o0 / o1 = channels 16g .. 16g+7 / 16g+8 .. 16g+15 of this lane's pixel (within the 32 of block mb), as stored.  The B operand of
+            // k-block kb wants channels 16 kb + 8g .. +7 from lane (pixel, g): after the swap x0 is that for kb = 0 and x1 for kb = 1
+            // (g = 0 keeps o0 and receives its partner's o0 as x1; g = 1 keeps o1 and receives its partner's o1 as x0).
+            typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+            typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+            u32x4 x0 = __builtin_bit_cast(u32x4, o0), x1 = __builtin_bit_cast(u32x4, o1);
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+            {
+                const u32x2 sw = __builtin_amdgcn_permlane32_swap(x0[d], x1[d], false, false);
+                x0[d] = sw[0]; x1[d] = sw[1];
+            }
+            accT = __builtin_amdgcn_mfma_f32_32x32x16_f16(wa3[mb][0], __builtin_bit_cast(f16x8, x0), accT, 0, 0, 0);
+            accT = __builtin_amdgcn_mfma_f32_32x32x16_f16(wa3[mb][1], __builtin_bit_cast(f16x8, x1), accT, 0, 0, 0);
+        }
+    }
+    if constexpr (TAIL != 0)
+    {
+        float t[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) t[r] = accT[r] * aff[64 + 2 * SD_MAXC2 + 16 * g + r] + aff[64 + 2 * SD_MAXC2 + 32 + 16 * g + r];
+        activateArray<16>(t, a.act3, a.act3Param);
+        f16x8 o0, o1;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) { o0[r] = static_cast<f16>(t[r] * late3); o1[r] = static_cast<f16>(t[8 + r] * late3); }
+        if (store)
+        {
+            f16 *zp = a.z + pix * a.zLd + 16 * g;
+            *reinterpret_cast<f16x8 *>(zp) = o0;
+            *reinterpret_cast<f16x8 *>(zp + 8) = o1;
         }
     }
 }
@@ -264,14 +329,21 @@ extern "C" int msnh_hip_conv_stem_down_pack(const float *w1, int c2, const float
     return 0;
 }
 
-extern "C" int msnh_hip_conv_stem_down(int batch, int h, int w, const float *x, const void *packed1, const float *scale1, const float *shift1, int act1,
-                                       float act1_param, float mid_mul, int c2, const void *packed2, const float *scale2, const float *shift2, int act2,
-                                       float act2_param, float out_mul, void *y, int y_ld, msnh_stream_t s)
+namespace {
+
+int stemDownLaunch(int batch, int h, int w, const float *x, const void *packed1, const float *scale1, const float *shift1, int act1,
+                   float act1_param, float mid_mul, int c2, const void *packed2, const float *scale2, const float *shift2, int act2,
+                   float act2_param, float out_mul, void *y, int y_ld, const void *packed3, const float *scale3, const float *shift3, int act3,
+                   float act3_param, float z_mul, void *z, int z_ld, msnh_stream_t s)
 {
     MSNH_REQUIRE(batch > 0 && h > 0 && w > 0 && x && packed1 && packed2 && y, "conv_stem_down: bad argument");
     MSNH_REQUIRE(c2 == 32 || c2 == 64 || c2 == 128, "conv_stem_down: the second layer must have 32, 64 or 128 filters");
     MSNH_REQUIRE(y_ld >= c2 && y_ld % 8 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0 && reinterpret_cast<uintptr_t>(packed1) % 16 == 0 &&
                  reinterpret_cast<uintptr_t>(packed2) % 16 == 0, "conv_stem_down: output and weights must be 16-byte aligned, y_ld a multiple of 8");
+    const bool tail = packed3 != nullptr;
+    if (tail)
+        MSNH_REQUIRE(z && z_ld >= 32 && z_ld % 8 == 0 && reinterpret_cast<uintptr_t>(z) % 16 == 0 && reinterpret_cast<uintptr_t>(packed3) % 16 == 0 && actOk(act3),
+                     "conv_stem_down_tail: z and the 1x1 filters must be 16-byte aligned, z_ld a multiple of 8");
     StemDownArgs a;
     a.x = x;
     a.w1 = static_cast<const f16 *>(packed1); a.scale1 = scale1; a.shift1 = shift1;
@@ -286,11 +358,65 @@ extern "C" int msnh_hip_conv_stem_down(int batch, int h, int w, const float *x, 
     a.total = static_cast<int>(total);
     a.act1 = act1; a.act1Param = act1_param; a.act2 = act2; a.act2Param = act2_param;
     a.midMul = mid_mul; a.outMul = out_mul;
+    a.w3 = static_cast<const f16 *>(packed3); a.scale3 = scale3; a.shift3 = shift3; a.z = static_cast<f16 *>(z);
+    a.zLd = z_ld; a.act3 = tail ? act3 : MSNH_ACT_NONE; a.act3Param = act3_param; a.zMul = z_mul;
     const dim3 grid(static_cast<unsigned>((total + 7) / 8 * 8));
     hipStream_t st = resolveStream(s);
-    if (c2 == 32) hipLaunchKernelGGL((convStemDownKernel<1>), grid, dim3(256), 0, st, a);
+    if (tail)
+    {
+        if (c2 == 32) hipLaunchKernelGGL((convStemDownKernel<1, 1>), grid, dim3(256), 0, st, a);
+        else if (c2 == 64) hipLaunchKernelGGL((convStemDownKernel<2, 1>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((convStemDownKernel<4, 1>), grid, dim3(256), 0, st, a);
+    }
+    else if (c2 == 32) hipLaunchKernelGGL((convStemDownKernel<1>), grid, dim3(256), 0, st, a);
     else if (c2 == 64) hipLaunchKernelGGL((convStemDownKernel<2>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((convStemDownKernel<4>), grid, dim3(256), 0, st, a);
     MSNH_LAUNCH_CHECK();
     return 0;
+}
+
+} // namespace
+
+extern "C" int msnh_hip_conv_stem_down(int batch, int h, int w, const float *x, const void *packed1, const float *scale1, const float *shift1, int act1,
+                                       float act1_param, float mid_mul, int c2, const void *packed2, const float *scale2, const float *shift2, int act2,
+                                       float act2_param, float out_mul, void *y, int y_ld, msnh_stream_t s)
+{
+    return stemDownLaunch(batch, h, w, x, packed1, scale1, shift1, act1, act1_param, mid_mul, c2, packed2, scale2, shift2, act2, act2_param, out_mul, y, y_ld,
+                          nullptr, nullptr, nullptr, MSNH_ACT_NONE, 0.f, 1.f, nullptr, 0, s);
+}
+
+extern "C" int msnh_hip_conv_stem_down_tail_supported(int c2, int c3, int k3, int s3, int p3)
+{
+    return (c2 == 32 || c2 == 64 || c2 == 128) && c3 == 32 && k3 == 1 && s3 == 1 && p3 == 0;
+}
+
+extern "C" size_t msnh_hip_conv_stem_down_tail_packed_elems(int c2)
+{
+    return (c2 == 32 || c2 == 64 || c2 == 128) ? static_cast<size_t>(c2 / 32) * 2 * 64 * 8 : 0;
+}
+
+extern "C" int msnh_hip_conv_stem_down_tail_pack(int c2, const float *w3, void *packed3)
+{
+    MSNH_REQUIRE(w3 && packed3 && (c2 == 32 || c2 == 64 || c2 == 128), "conv_stem_down_tail_pack: bad argument");
+    // w3[32][c2] (filter, channel): operand A of k-block (mb, kb): lane (row, half) holds channels 32 mb + 16 kb + 8 half + 0..7 of filter sdChannelOfRow(row)
+    uint16_t *p3 = static_cast<uint16_t *>(packed3);
+    for (int mb = 0; mb < c2 / 32; ++mb)
+        for (int kb = 0; kb < 2; ++kb)
+            for (int lane = 0; lane < 64; ++lane)
+                for (int e = 0; e < 8; ++e)
+                {
+                    const int oc = sdChannelOfRow(lane & 31), ic = mb * 32 + kb * 16 + (lane >> 5) * 8 + e;
+                    p3[(static_cast<size_t>(mb * 2 + kb) * 64 + lane) * 8 + e] = sdHalf(w3[static_cast<size_t>(oc) * c2 + ic]);
+                }
+    return 0;
+}
+
+extern "C" int msnh_hip_conv_stem_down_tail(int batch, int h, int w, const float *x, const void *packed1, const float *scale1, const float *shift1, int act1,
+                                            float act1_param, float mid_mul, int c2, const void *packed2, const float *scale2, const float *shift2, int act2,
+                                            float act2_param, float out_mul, void *y, int y_ld, const void *packed3, const float *scale3, const float *shift3,
+                                            int act3, float act3_param, float z_mul, void *z, int z_ld, msnh_stream_t s)
+{
+    MSNH_REQUIRE(packed3 && z, "conv_stem_down_tail: NULL pointer");
+    return stemDownLaunch(batch, h, w, x, packed1, scale1, shift1, act1, act1_param, mid_mul, c2, packed2, scale2, shift2, act2, act2_param, out_mul, y, y_ld,
+                          packed3, scale3, shift3, act3, act3_param, z_mul, z, z_ld, s);
 }

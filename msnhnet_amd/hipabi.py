@@ -53,7 +53,7 @@ SYMBOLS = [
     "msnh_hip_host_alloc", "msnh_hip_host_free", "msnh_hip_memcpy_h2d", "msnh_hip_memcpy_d2h", "msnh_hip_memcpy_d2d",
     "msnh_hip_fill_zero", "msnh_hip_stream_create", "msnh_hip_stream_destroy", "msnh_hip_stream_sync", "msnh_hip_event_create",
     "msnh_hip_event_destroy", "msnh_hip_event_record", "msnh_hip_stream_wait_event", "msnh_hip_event_sync", "msnh_hip_event_elapsed_ms", "msnh_hip_graph_begin",
-    "msnh_hip_graph_end", "msnh_hip_graph_launch", "msnh_hip_graph_destroy", "msnh_hip_conv_stem_down_supported", "msnh_hip_conv_stem_down_packed_elems", "msnh_hip_conv_stem_down_pack", "msnh_hip_conv_stem_down", "msnh_hip_mbconv_supported", "msnh_hip_mbconv_packed_bytes", "msnh_hip_mbconv_pack", "msnh_hip_mbconv", "msnh_hip_conv2d_tile_count", "msnh_hip_conv2d_pack_layout_version", "msnh_hip_conv2d_tile_supported", "msnh_hip_conv2d_select_algo",
+    "msnh_hip_graph_end", "msnh_hip_graph_launch", "msnh_hip_graph_destroy", "msnh_hip_conv_stem_down_supported", "msnh_hip_conv_stem_down_packed_elems", "msnh_hip_conv_stem_down_pack", "msnh_hip_conv_stem_down", "msnh_hip_conv_stem_down_tail_supported", "msnh_hip_conv_stem_down_tail_packed_elems", "msnh_hip_conv_stem_down_tail_pack", "msnh_hip_conv_stem_down_tail", "msnh_hip_mbconv_supported", "msnh_hip_mbconv_packed_bytes", "msnh_hip_mbconv_pack", "msnh_hip_mbconv", "msnh_hip_conv2d_tile_count", "msnh_hip_conv2d_pack_layout_version", "msnh_hip_conv2d_tile_supported", "msnh_hip_conv2d_select_algo",
     "msnh_hip_conv2d_packed_weight_elems", "msnh_hip_conv2d_pack_weights", "msnh_hip_conv2d_workspace_bytes", "msnh_hip_conv2d",
     "msnh_hip_conv2d_tail_tile_first", "msnh_hip_conv2d_tail_supported", "msnh_hip_conv2d_tail", "msnh_hip_letterbox_u8", "msnh_hip_image_u8_to_input",
     "msnh_hip_affine_act", "msnh_hip_add_act", "msnh_hip_copy_channels", "msnh_hip_maxpool", "msnh_hip_maxpool_chain", "msnh_hip_maxpool_chain_supported", "msnh_hip_avgpool",
@@ -148,6 +148,11 @@ def lib():
     L.msnh_hip_conv_stem_down_packed_elems.restype = sz
     L.msnh_hip_conv_stem_down_pack.argtypes = [vp, ci, vp, vp, vp]
     L.msnh_hip_conv_stem_down.argtypes = [ci, ci, ci, vp, vp, vp, vp, ci, cf, cf, ci, vp, vp, vp, ci, cf, cf, vp, ci, vp]
+    L.msnh_hip_conv_stem_down_tail_supported.argtypes = [ci, ci, ci, ci, ci]
+    L.msnh_hip_conv_stem_down_tail_packed_elems.argtypes = [ci]
+    L.msnh_hip_conv_stem_down_tail_packed_elems.restype = sz
+    L.msnh_hip_conv_stem_down_tail_pack.argtypes = [ci, vp, vp]
+    L.msnh_hip_conv_stem_down_tail.argtypes = [ci, ci, ci, vp, vp, vp, vp, ci, cf, cf, ci, vp, vp, vp, ci, cf, cf, vp, ci, vp, vp, vp, ci, cf, cf, vp, ci, vp]
     L.msnh_hip_count_nonfinite.argtypes = [ci, ll, ci, vp, ci, vp, vp]
     L.msnh_hip_mbconv_supported.argtypes = [vp]
     L.msnh_hip_mbconv_packed_bytes.argtypes = [vp]

@@ -76,6 +76,8 @@ struct PlanOp
     int  chainHead = -1;                    // MAXPOOL: >= 0 = this pool's result is written by the launch of op chainHead (a chain of stride-1 pools in one launch)
     int  chainNext = -1;                    // MAXPOOL at the head or inside such a chain: the op whose pool follows
     int  stemOp = -1;                       // CONV 3x3 stride 2: the (dead) first-layer op computed in front of it by the same launch (Plan::fuse c)
+    int  stemTail = -1;                     // CONV with stemOp: the (dead) 1x1 convolution with 32 filters that reads this op's result, computed by the
+                                            // same launch (Plan::fuse c, msnh_hip_conv_stem_down_tail)
     int  mbExpand = -1, mbDw = -1;          // CONV 1x1 closing an inverted-residual block: the (dead) 1x1 expand and 3x3 depthwise ops computed in front of
                                             // it by the same launch (Plan::fuse d, msnh_hip_mbconv)
 
@@ -95,6 +97,7 @@ struct PlanOp
     // device-side constants, filled by Plan::prepareWeights
     DeviceBuffer wDev, scaleDev, shiftDev;
     DeviceBuffer wDev2, scaleDev2, shiftDev2;   // stemOp >= 0: the first layer's
+    DeviceBuffer wDev3, scaleDev3, shiftDev3;   // stemTail >= 0: the 1x1 convolution's
     double flops = 0;                       // 2*MACs of this launch (conv / connected)
 };
 
@@ -113,6 +116,7 @@ public:
     bool fuseTail = false;                  // float16: a convolution whose tile holds all its output channels also computes the 1x1 convolution that
                                             // reads its result (msnh_hip_conv2d_tail), where the per-layer search finds that faster than two launches
     bool forceTail = false;                 // ... wherever the library takes the pair, whatever the timing says (tests)
+    bool fuseStemTail = true;               // ... and the 1x1 convolution with 32 filters behind that pair in the same launch (msnh_hip_conv_stem_down_tail)
     bool fuseStemDown = true;               // float16: first layer + first stride-2 layer as one launch where msnh_hip_conv_stem_down takes the pair
     bool preferWinograd = false;            // 3x3 stride-1 float16 convs take the Winograd path where the kernel accepts the shape
     std::vector<PlanTensor> tensors;

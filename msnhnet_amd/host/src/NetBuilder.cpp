@@ -407,6 +407,7 @@ void NetBuilder::finalizePlan()
     std::unique_ptr<Plan> plan = lowerNetwork(dtype);
     plan->fuseStemDown = std::getenv("MSNH_NO_STEM_DOWN") == nullptr;
     plan->fuseMbconv = std::getenv("MSNH_NO_MBCONV") == nullptr;
+    plan->fuseStemTail = std::getenv("MSNH_NO_STEM_TAIL") == nullptr;
     // (measured level with two launches inside a forward, so not the default: MSNH_CONV_TAIL=1 lets the load-time search decide per pair,
     // MSNH_FORCE_CONV_TAIL=1 takes every pair the library accepts)
     plan->forceTail = std::getenv("MSNH_FORCE_CONV_TAIL") != nullptr;
@@ -852,6 +853,11 @@ static double opBytes(const Plan &plan, const PlanOp &op)
     const PlanTensor &out = plan.tensors[static_cast<size_t>(op.out)];
     double oe = static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4);
     for (int nx = op.chainNext; nx >= 0; nx = plan.ops[static_cast<size_t>(nx)].chainNext) oe += static_cast<double>(out.elems()) * (out.dtype == MSNH_F16 ? 2 : 4);   // one launch, every pool's result
+    if (op.stemTail >= 0)
+    {
+        const PlanOp &b = plan.ops[static_cast<size_t>(op.stemTail)];
+        oe += static_cast<double>(plan.tensors[static_cast<size_t>(b.out)].elems()) * 2 + static_cast<double>(op.wDev3.bytes());
+    }
     if (op.algo == MSNH_CONV_IGEMM_TAIL && op.tail >= 0)
     {
         // ... and the 1x1 convolution computed by the same launch: its result and its filters

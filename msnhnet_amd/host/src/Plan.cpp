@@ -210,6 +210,23 @@ void Plan::fuse()
                     down.stemOp = static_cast<int>(i);
                     down.in0 = first.in0;
                     first.dead = true;
+                    // ... and the 1x1 convolution with 32 filters that reads the pair's result (the opening of Darknet-53's first residual
+                    // block), if it is the next launch: computed by the pair's launch from its own registers.  The pair's result is still
+                    // written (the block's residual add reads it).
+                    for (size_t t = k + 1; fuseStemTail && t < ops.size(); ++t)
+                    {
+                        PlanOp &tail = ops[t];
+                        if (tail.dead) continue;
+                        const PlanTensor &z = tensors[static_cast<size_t>(tail.out)];
+                        if (tail.kind == PlanOp::CONV && tail.in0 == down.out && tail.in1 < 0 && tail.groups == 1 && tail.dilation == 1 && tail.stemOp < 0 &&
+                            tail.mbExpand < 0 && z.dtype == MSNH_F16 && z.layout == PlanTensor::NHWC &&
+                            msnh_hip_conv_stem_down_tail_supported(out.c, z.c, tail.ksize, tail.stride, tail.pad))
+                        {
+                            down.stemTail = static_cast<int>(t);
+                            tail.dead = true;
+                        }
+                        break;
+                    }
                 }
                 break;
             }
@@ -452,7 +469,7 @@ uint64_t Plan::structureHash() const
     for (const PlanOp &op : ops)
         os << static_cast<int>(op.kind) << ' ' << op.in0 << ' ' << op.in1 << ' ' << op.out << ' ' << (op.dead && op.tailOf < 0) << ' ' << op.layerIndex << ' ' << op.ksize << ' ' << op.stride << ' '
            << op.pad << ' ' << op.dilation << ' ' << op.groups << ' ' << static_cast<int>(op.act) << ' ' << static_cast<int>(op.act2) << ' ' << op.in1Sign << ' ' << (op.src2 != nullptr)
-           << ' ' << op.dstChanOffset << ' ' << op.stemOp << ' ' << op.chainHead << ' ' << op.mbExpand << ' ' << op.tail << ';';
+           << ' ' << op.dstChanOffset << ' ' << op.stemOp << ' ' << op.chainHead << ' ' << op.mbExpand << ' ' << op.tail << ' ' << op.stemTail << ';';
     const std::string text = os.str();
     return PackFile::hash(text.data(), text.size());
 }
@@ -511,6 +528,7 @@ void Plan::place()
         touch(op.in0, i); touch(op.in1, i); touch(op.out, i);
         if (op.chainHead >= 0) touch(op.out, op.chainHead);      // written by the launch of the chain's first pool
         if (op.tail >= 0) touch(ops[static_cast<size_t>(op.tail)].out, i);   // may be written by this launch (msnh_hip_conv2d_tail)
+        if (op.stemTail >= 0) touch(ops[static_cast<size_t>(op.stemTail)].out, i);   // written by this launch (msnh_hip_conv_stem_down_tail)
     }
     {
         // the heads of a detector may all be decoded by one launch where the last of them stands (findYoloHeads): their inputs
@@ -681,6 +699,18 @@ void Plan::prepareWeights(PackFile *from, PackFile *to)
             op.algo = MSNH_CONV_STEM_DOWN;
             const PlanTensor &img = tensors[static_cast<size_t>(op.in0)];
             op.flops = 2.0 * img.n * (static_cast<double>(mid.c) * mid.h * mid.w * img.c * 9 + static_cast<double>(out.c) * out.h * out.w * mid.c * 9);
+            if (op.stemTail >= 0)
+            {
+                const PlanOp &tail = ops[static_cast<size_t>(op.stemTail)];
+                const PlanTensor &z = tensors[static_cast<size_t>(tail.out)];
+                const std::vector<float> &w3 = tail.src->kernelWeights();
+                if (w3.size() != static_cast<size_t>(z.c) * out.c) MSNH_THROW("conv weights are not loaded (" + tail.name + ")");
+                std::vector<uint16_t> p3(msnh_hip_conv_stem_down_tail_packed_elems(out.c));
+                MSNH_DEV(msnh_hip_conv_stem_down_tail_pack(out.c, w3.data(), p3.data()));
+                op.wDev3.upload(p3.data(), p3.size() * 2);
+                affine(tail, z.c, mulOf(op.out), op.scaleDev3, op.shiftDev3);
+                op.flops += 2.0 * img.n * static_cast<double>(z.c) * z.h * z.w * out.c;
+            }
             continue;
         }
         if (op.kind == PlanOp::CONV && op.mbExpand >= 0)
@@ -1219,6 +1249,16 @@ void Plan::launch(PlanOp &op, msnh_stream_t s)
         if (op.stemOp >= 0)
         {
             const PlanOp &first = ops[static_cast<size_t>(op.stemOp)];
+            if (op.stemTail >= 0)
+            {
+                const PlanOp &tail = ops[static_cast<size_t>(op.stemTail)];
+                MSNH_DEV(msnh_hip_conv_stem_down_tail(in.n, in.h, in.w, static_cast<const float *>(ptr(op.in0)), op.wDev2.ptr(), op.scaleDev2.as<float>(),
+                                                      op.shiftDev2.as<float>(), static_cast<int>(first.act), first.actParam, 1.f / mulOf(first.out), out.c, op.wDev.ptr(),
+                                                      op.scaleDev.as<float>(), op.shiftDev.as<float>(), static_cast<int>(op.act), op.actParam, 1.f / mulOf(op.out),
+                                                      ptr(op.out), ld(op.out), op.wDev3.ptr(), op.scaleDev3.as<float>(), op.shiftDev3.as<float>(),
+                                                      static_cast<int>(tail.act), tail.actParam, 1.f / mulOf(tail.out), ptr(tail.out), ld(tail.out), s));
+                break;
+            }
             MSNH_DEV(msnh_hip_conv_stem_down(in.n, in.h, in.w, static_cast<const float *>(ptr(op.in0)), op.wDev2.ptr(), op.scaleDev2.as<float>(), op.shiftDev2.as<float>(),
                                              static_cast<int>(first.act), first.actParam, 1.f / mulOf(first.out), out.c, op.wDev.ptr(), op.scaleDev.as<float>(),
                                              op.shiftDev.as<float>(), static_cast<int>(op.act), op.actParam, 1.f / mulOf(op.out), ptr(op.out), ld(op.out), s));
@@ -1432,7 +1472,7 @@ std::string Plan::describe() const
         const PlanTensor &out = tensors[static_cast<size_t>(op.out)];
         os << "  L" << op.layerIndex << " " << kinds[op.kind];
         if (op.kind == PlanOp::CONV)
-            os << "[" << algos[op.algo] << (op.tile ? " t" + std::to_string(op.tile) : std::string()) << " k" << op.ksize << " s" << op.stride << " g" << op.groups << (op.in1 >= 0 ? " +res" : "") << (op.src2 ? " +bn" : "") << "]";
+            os << "[" << algos[op.algo] << (op.stemTail >= 0 ? "+1x1" : "") << (op.tile ? " t" + std::to_string(op.tile) : std::string()) << " k" << op.ksize << " s" << op.stride << " g" << op.groups << (op.in1 >= 0 ? " +res" : "") << (op.src2 ? " +bn" : "") << "]";
         if (op.kind == PlanOp::MAXPOOL || op.kind == PlanOp::AVGPOOL)
             os << "[k" << op.ksize << " s" << op.stride << " p" << op.pad << (op.chainHead >= 0 ? " in the launch of the pool before it" : "") << "]";
         os << " " << in.n << "x" << in.h << "x" << in.w << "x" << in.c << " -> " << out.h << "x" << out.w << "x" << out.c

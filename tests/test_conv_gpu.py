@@ -477,6 +477,32 @@ def test_conv_stem_down(b, h, w, c2, act):
     assert got.shape == ref.shape
     assert gu.rel_err(got, ref) <= 2e-3
 
+    # ... and with the 1x1 convolution behind it in the same launch (32 filters: the opening of Darknet-53's first residual block):
+    # y carries the same bits as without, z equals the oracle's 1x1 over y as stored, and msnh_hip_conv2d's over the device's y
+    assert L.msnh_hip_conv_stem_down_tail_supported(c2, 32, 1, 1, 0) == 1
+    assert L.msnh_hip_conv_stem_down_tail_supported(c2, 64, 1, 1, 0) == 0 and L.msnh_hip_conv_stem_down_tail_supported(c2, 32, 3, 1, 1) == 0
+    w3 = rng.standard_normal((32, c2), dtype=np.float32) * np.float32(np.sqrt(2.0 / c2))
+    s3, h3 = rng.uniform(0.5, 1.5, 32).astype(np.float32), (rng.standard_normal(32) * 0.1).astype(np.float32)
+    z_mul, zld = 0.5, 40
+    p3 = np.zeros(L.msnh_hip_conv_stem_down_tail_packed_elems(c2), np.float16)
+    abi.check(L.msnh_hip_conv_stem_down_tail_pack(c2, w3.ctypes.data_as(ctypes.c_void_p), p3.ctypes.data_as(ctypes.c_void_p)))
+    p3d, s3d, h3d = gu.dev(p3), gu.dev(s3 / np.float32(out_mul)), gu.dev(h3)
+    yd2 = torch.full((b, oh, ow, ld), 3.0, dtype=torch.float16).cuda()
+    zd = torch.full((b, oh, ow, zld), 5.0, dtype=torch.float16).cuda()
+    gu.sync()
+    abi.check(L.msnh_hip_conv_stem_down_tail(b, h, w, gu.ptr(xd), gu.ptr(p1d), gu.ptr(s1d), gu.ptr(h1d), abi.ACT[act], 0.1, mid_mul, c2, gu.ptr(p2d), gu.ptr(s2d),
+                                             gu.ptr(h2d), abi.ACT[act], 0.1, out_mul, gu.ptr(yd2), ld, gu.ptr(p3d), gu.ptr(s3d), gu.ptr(h3d), abi.ACT["leaky"], 0.1,
+                                             z_mul, gu.ptr(zd), zld, None))
+    gu.sync()
+    assert torch.equal(yd2, yd)
+    assert (zd[..., 32:].float().cpu().numpy() == 5.0).all(), "kernel wrote outside z's channel slice"
+    z = gu.nchw_host(zd, 32)
+    z_ref = _ref(got, gu.round_f16(w3).reshape(32, c2, 1, 1), 1, 0, 1, 1, s3 / np.float32(out_mul), h3, "leaky", 0.1, None, "none", 1.0, z_mul)
+    assert gu.rel_err(z, z_ref) <= 2e-3
+    z2, _ = gu.conv2d(got, gu.round_f16(w3).reshape(32, c2, 1, 1), dtype=abi.F16, scale=s3 / np.float32(out_mul), shift=h3, act="leaky", out_mul=z_mul, algo="igemm", tile=38)
+    print("z equals a separate launch bit for bit:", bool(np.array_equal(z, z2)), flush=True)
+    assert gu.rel_err(z, z2) <= 1e-3
+
 
 TAIL_CASES = [
     # b, c, h, w, oc, k, stride, pad, oc2, residual
