@@ -140,6 +140,10 @@ typedef struct msnh_conv_desc
     float out_mul;
     int   algo;         /* msnh_conv_algo */
     int   tile;         /* IGEMM only: 0 = library default, 1..msnh_hip_conv2d_tile_count() = forced tile configuration */
+    int   out_upsample; /* 0 or 1: y is [batch][out_h][out_w].  2 (MSNH_CONV_IGEMM only, no residual, out_c and out_ld multiples of 8): every
+                           result pixel is written to the 2 x 2 pixels it maps to under nearest-neighbour upsampling, y is
+                           [batch][2 out_h][2 out_w] -- the convolution in front of an UpSampleLayer (src/layers/MsnhUpSampleLayer.cpp:96-118,
+                           Blas::cpuUpSample with stride 2 and scale 1) writes the upsampled tensor itself */
 } msnh_conv_desc;
 
 /* Number of tile configurations of the IGEMM algorithm; any of them computes the same result, they differ in

@@ -307,6 +307,10 @@ static int validate(const msnh_conv_desc *d)
     const int ow = (d->in_w + 2 * d->pad - ext) / d->stride + 1;
     MSNH_REQUIRE(oh == d->out_h && ow == d->out_w, "conv: out size %dx%d does not match geometry (%dx%d)", d->out_h, d->out_w, oh, ow);
     MSNH_REQUIRE(d->out_ld >= d->out_c, "conv: out_ld < out_c");
+    MSNH_REQUIRE(d->out_upsample >= 0 && d->out_upsample <= 2, "conv: out_upsample is 0, 1 or 2");
+    MSNH_REQUIRE(d->out_upsample != 2 || ((d->algo == MSNH_CONV_IGEMM || d->algo == MSNH_CONV_AUTO) && !d->has_residual && d->out_c % 8 == 0 && d->out_ld % 8 == 0 &&
+                                         d->groups == 1 && static_cast<long long>(d->batch) * d->out_h * d->out_w * 4 * d->out_ld * 4 < 0x7fffffffLL),
+                 "conv: the upsampling epilogue belongs to the IGEMM algorithm, without residual, channel counts multiples of 8");
     MSNH_REQUIRE(!d->has_residual || d->res_ld >= d->out_c, "conv: res_ld < out_c");
     MSNH_REQUIRE(actOk(d->act) && (!d->has_residual || actOk(d->act2)), "conv: unsupported activation");
     MSNH_REQUIRE(static_cast<long long>(d->batch) * d->out_h * d->out_w < (1LL << 31), "conv: too many output pixels");
@@ -402,6 +406,7 @@ int msnh_hip_conv2d_select_algo(const msnh_conv_desc *d)
 {
     if (!d) return MSNH_CONV_DIRECT;
     if (d->algo != MSNH_CONV_AUTO) return d->algo;
+    if (d->out_upsample == 2) return MSNH_CONV_IGEMM;
     if (stemOk(d)) return MSNH_CONV_STEM;
     if (depthwiseOk(d)) return MSNH_CONV_DEPTHWISE;
     if (igemmOk(d)) return MSNH_CONV_IGEMM;
@@ -494,6 +499,7 @@ int msnh_hip_conv2d(const msnh_conv_desc *d, const void *x, const void *w, const
     case MSNH_CONV_IGEMM:
         MSNH_REQUIRE(igemmOk(d), "conv2d: IGEMM needs (in_c/groups) and in_ld to be multiples of %d", d->dtype == MSNH_F16 ? 8 : 4);
         MSNH_REQUIRE(reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0, "conv2d: IGEMM needs 16-byte aligned x and w");
+        MSNH_REQUIRE(d->out_upsample != 2 || reinterpret_cast<uintptr_t>(y) % 16 == 0, "conv2d: the upsampling epilogue needs a 16-byte aligned y");
         return convIgemm(d, x, w, scale, shift, residual, y, st, false);
     case MSNH_CONV_IGEMM_SPLITK:
         MSNH_REQUIRE(igemmOk(d), "conv2d: IGEMM needs (in_c/groups) and in_ld to be multiples of %d", d->dtype == MSNH_F16 ? 8 : 4);

@@ -41,6 +41,8 @@ static int convIgemmAny(const msnh_conv_desc *d, const void *x, const void *w, c
     a.cinG = d->in_c / d->groups; a.coutG = d->out_c / d->groups;
     a.taps = d->ksize * d->ksize; a.ksize = d->ksize; a.stride = d->stride; a.pad = d->pad; a.dil = d->dilation;
     a.P = d->batch * d->out_h * d->out_w;
+    a.up2 = d->out_upsample == 2 ? 1 : 0;
+    a.yBytes = a.up2 ? static_cast<unsigned>(static_cast<unsigned long long>(d->batch) * d->out_h * d->out_w * 4ull * d->out_ld * dtypeSize(d->out_dtype)) : 0u;
     a.byOW = makeFastDiv(static_cast<unsigned>(d->out_w));
     a.byOH = makeFastDiv(static_cast<unsigned>(d->out_h));
     a.patchOk = (d->ksize == 3 && d->stride == 1 && d->pad == 1 && d->dilation == 1 && d->groups == 1 && d->out_h == d->in_h && d->out_w == d->in_w) ? 1 : 0;
@@ -63,6 +65,7 @@ static int convIgemmAny(const msnh_conv_desc *d, const void *x, const void *w, c
               (reinterpret_cast<uintptr_t>(y) % (8 * outEl) == 0) &&
               (!a.hasRes || (d->res_ld % 8 == 0 && reinterpret_cast<uintptr_t>(residual) % 16 == 0));
     a.splitMax = 0; a.splitK = 1; a.ws = nullptr; a.wsLd = d->out_c;
+    if (a.up2) MSNH_REQUIRE(d->algo != MSNH_CONV_IGEMM_SPLITK && !tail, "conv2d: the upsampling epilogue goes with the plain implicit GEMM");
     if (d->algo == MSNH_CONV_IGEMM_SPLITK)
     {
         MSNH_REQUIRE(d->out_c % 4 == 0, "conv2d: split-K needs out_c to be a multiple of 4");

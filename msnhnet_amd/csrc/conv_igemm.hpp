@@ -49,6 +49,8 @@ struct IgemmArgs
     int act, act2, hasRes, vecOk;
     float actParam, act2Param, resMul, outMul;
     FastDiv byOW, byOH;     // pixel index -> (image, row, column) without hardware-less integer division
+    int up2;                // every result pixel goes to the 2 x 2 pixels of y it maps to under nearest-neighbour upsampling (y: [batch][2 OH][2 OW])
+    unsigned yBytes;        // up2: extent of y in bytes
     // tail (tiles with TAIL = 1 only): a 1x1 stride-1 convolution z = zMul * act3(scale2 * (W2 . y) + shift2) of this convolution's
     // float16 result y, computed by the same workgroup from the copy of its y tile in LDS
     int tailOn;             // the launch carries a tail (set by the tail entry point, also for dry runs)
@@ -230,7 +232,7 @@ __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[
     const int npix = min(a.P - p0, BN);
     TOut    *yBlock = static_cast<TOut *>(a.y) + static_cast<size_t>(p0) * a.outLd;
     const T *rBlock = static_cast<const T *>(a.res) + static_cast<size_t>(p0) * a.resLd;
-    const __amdgpu_buffer_rsrc_t ry = makeRsrc(yBlock, static_cast<unsigned>(npix) * a.outLd * sizeof(TOut));
+    const __amdgpu_buffer_rsrc_t ry = a.up2 ? makeRsrc(a.y, a.yBytes) : makeRsrc(yBlock, static_cast<unsigned>(npix) * a.outLd * sizeof(TOut));
     const __amdgpu_buffer_rsrc_t rr = makeRsrc(a.hasRes ? rBlock : nullptr, a.hasRes ? static_cast<unsigned>(npix) * a.resLd * sizeof(T) : 0u);
     float slope1, slope2;
     const bool lin1 = actIsSlope(a.act, a.actParam, slope1);
@@ -329,7 +331,22 @@ __device__ __forceinline__ void igemmEpilogue(const IgemmArgs &a, f32x16 (&acc)[
                     for (int e = 0; e < 8; ++e) v[e] *= a.outMul;
                     Raw8<TOut> o;
                     o.fromFloat(v);
-                    bufferStore8<TOut>(o, ry, (pl * a.outLd + ch) * static_cast<unsigned>(sizeof(TOut)));
+                    if (a.up2)
+                    {
+                        // pixel (image, row, column) -> the 2 x 2 pixels (2 row + dy, 2 column + dx) of the upsampled tensor
+                        const unsigned p = static_cast<unsigned>(p0) + pl;
+                        const unsigned t1 = fastDiv(p, a.byOW), bImg = fastDiv(t1, a.byOH);
+                        const unsigned ox = p - t1 * a.OW, oy = t1 - bImg * a.OH;
+                        const unsigned q = ((bImg * 2u * a.OH + 2u * oy) * 2u * a.OW + 2u * ox) * a.outLd + ch;
+                        const unsigned rowStep = 2u * a.OW * a.outLd;
+                        const unsigned es = static_cast<unsigned>(sizeof(TOut));
+                        const bool in = static_cast<int>(pl) < npix;
+                        bufferStore8<TOut>(o, ry, in ? q * es : kOobOffset);
+                        bufferStore8<TOut>(o, ry, in ? (q + a.outLd) * es : kOobOffset);
+                        bufferStore8<TOut>(o, ry, in ? (q + rowStep) * es : kOobOffset);
+                        bufferStore8<TOut>(o, ry, in ? (q + rowStep + a.outLd) * es : kOobOffset);
+                    }
+                    else bufferStore8<TOut>(o, ry, (pl * a.outLd + ch) * static_cast<unsigned>(sizeof(TOut)));
                 }
                 else if (chOk && static_cast<int>(pl) < npix)
                 {
@@ -1026,6 +1043,11 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
             setError("conv2d: this tile needs a 1x1 convolution behind it (msnh_hip_conv2d_tail), the others take none; ungrouped, channel counts that fit one tile");
             return 3;
         }
+    }
+    if (a.up2 && (TAIL != 0 || groups != 1 || a.hasRes || a.splitMax > 1 || (!a.vecOk && !a.dryRun) || a.coutG % 8 != 0))
+    {
+        setError("conv2d: the upsampling epilogue takes an ungrouped convolution without residual, channel counts multiples of 8");
+        return 3;
     }
     a.cChunks = (a.cinG + BK - 1) / BK;
     a.nIter   = a.taps * a.cChunks;

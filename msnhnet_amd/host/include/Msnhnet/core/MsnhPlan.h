@@ -76,6 +76,8 @@ struct PlanOp
     int  chainHead = -1;                    // MAXPOOL: >= 0 = this pool's result is written by the launch of op chainHead (a chain of stride-1 pools in one launch)
     int  chainNext = -1;                    // MAXPOOL at the head or inside such a chain: the op whose pool follows
     int  stemOp = -1;                       // CONV 3x3 stride 2: the (dead) first-layer op computed in front of it by the same launch (Plan::fuse c)
+    bool up2 = false;                       // CONV: the launch writes every result pixel to the 2 x 2 pixels of `out` it maps to (Plan::fuse f): `out` is the
+                                            // tensor of the (dead) nearest-neighbour upsample that read this convolution's result
     int  stemTail = -1;                     // CONV with stemOp: the (dead) 1x1 convolution with 32 filters that reads this op's result, computed by the
                                             // same launch (Plan::fuse c, msnh_hip_conv_stem_down_tail)
     int  mbExpand = -1, mbDw = -1;          // CONV 1x1 closing an inverted-residual block: the (dead) 1x1 expand and 3x3 depthwise ops computed in front of
@@ -116,6 +118,7 @@ public:
     bool fuseTail = false;                  // float16: a convolution whose tile holds all its output channels also computes the 1x1 convolution that
                                             // reads its result (msnh_hip_conv2d_tail), where the per-layer search finds that faster than two launches
     bool forceTail = false;                 // ... wherever the library takes the pair, whatever the timing says (tests)
+    bool fuseUpsample = true;               // a convolution whose only reader is a 2x nearest-neighbour upsample writes the upsampled tensor itself
     bool fuseStemTail = true;               // ... and the 1x1 convolution with 32 filters behind that pair in the same launch (msnh_hip_conv_stem_down_tail)
     bool fuseStemDown = true;               // float16: first layer + first stride-2 layer as one launch where msnh_hip_conv_stem_down takes the pair
     bool preferWinograd = false;            // 3x3 stride-1 float16 convs take the Winograd path where the kernel accepts the shape

@@ -408,6 +408,7 @@ void NetBuilder::finalizePlan()
     plan->fuseStemDown = std::getenv("MSNH_NO_STEM_DOWN") == nullptr;
     plan->fuseMbconv = std::getenv("MSNH_NO_MBCONV") == nullptr;
     plan->fuseStemTail = std::getenv("MSNH_NO_STEM_TAIL") == nullptr;
+    plan->fuseUpsample = std::getenv("MSNH_NO_CONV_UPSAMPLE") == nullptr;
     // (measured level with two launches inside a forward, so not the default: MSNH_CONV_TAIL=1 lets the load-time search decide per pair,
     // MSNH_FORCE_CONV_TAIL=1 takes every pair the library accepts)
     plan->forceTail = std::getenv("MSNH_FORCE_CONV_TAIL") != nullptr;
@@ -434,6 +435,7 @@ void NetBuilder::finalizePlan()
         // One float32 pass over a fixed pseudo-random U[0,1) input fixes the power-of-two scale of every
         // float16 tensor.  The float32 twin is lowered and optimised identically, so tensor ids line up.
         std::unique_ptr<Plan> cal = lowerNetwork(MSNH_F32);
+        cal->fuseUpsample = plan->fuseUpsample;
         cal->fuse();
         cal->chainMaxPools();
         cal->aliasConcats();

@@ -275,6 +275,30 @@ void Plan::fuse()
             ex.dead = true;
             dw.dead = true;
         }
+    // (f) convolution -> 2x nearest-neighbour upsample that is its only reader (the lateral branches of the detection necks,
+    // src/layers/MsnhUpSampleLayer.cpp:96-118 behind a 1x1 ConvolutionalLayer): the convolution's epilogue writes every result pixel to the
+    // four pixels it maps to (msnh_conv_desc::out_upsample), the 19x19 / 38x38 tensor in between is never stored and the upsample launch goes.
+    if (fuseUpsample)
+        for (size_t i = 0; i < ops.size(); ++i)
+        {
+            PlanOp &up = ops[i];
+            if (up.dead || up.kind != PlanOp::UPSAMPLE || up.stride != 2 || up.upScale != 1.f) continue;
+            const int pc = producerOf(up.in0);
+            if (pc < 0) continue;
+            PlanOp &conv = ops[static_cast<size_t>(pc)];
+            const PlanTensor &x = tensors[static_cast<size_t>(conv.in0)];
+            const PlanTensor &mid = tensors[static_cast<size_t>(up.in0)];
+            const PlanTensor &big = tensors[static_cast<size_t>(up.out)];
+            const int vec = x.dtype == MSNH_F16 ? 8 : 4;
+            if (conv.kind != PlanOp::CONV || conv.in1 >= 0 || conv.groups != 1 || conv.stemOp >= 0 || conv.mbExpand >= 0 || conv.up2 || conv.tail >= 0 ||
+                conv.tailOf >= 0 || x.layout != PlanTensor::NHWC || x.c % vec != 0 || x.c <= 4 || mid.c % 8 != 0 || mid.pinned || mid.persistent || mid.external ||
+                mid.parent >= 0 || consumerCount(up.in0) != 1 || mid.dtype != big.dtype || big.h != 2 * mid.h || big.w != 2 * mid.w ||
+                (x.dtype == MSNH_F32 && mid.dtype != MSNH_F32))
+                continue;
+            conv.out = up.out;
+            conv.up2 = true;
+            up.dead = true;
+        }
     // (e) float16: convolution -> 1x1 stride-1 convolution (the 3x3 that closes a Darknet residual block and the 1x1 that opens the next one,
     // src/layers/MsnhResBlockLayer.cpp:215-302): where one tile of the first launch holds all its output channels (at most 256) and the 1x1 has at
     // most 128 filters, the first launch can compute the 1x1 from its own result tile (msnh_hip_conv2d_tail).  Only marked here: both ops stay
@@ -284,12 +308,12 @@ void Plan::fuse()
         {
             PlanOp &b = ops[i];
             if (b.dead || b.kind != PlanOp::CONV || b.ksize != 1 || b.stride != 1 || b.pad != 0 || b.groups != 1 || b.in1 >= 0 || b.stemOp >= 0 || b.mbExpand >= 0 ||
-                b.tail >= 0 || b.tailOf >= 0)
+                b.tail >= 0 || b.tailOf >= 0 || b.up2)
                 continue;
             const int pa = producerOf(b.in0);
             if (pa < 0 || pa >= static_cast<int>(i)) continue;
             PlanOp &a = ops[static_cast<size_t>(pa)];
-            if (a.kind != PlanOp::CONV || a.groups != 1 || a.dilation != 1 || a.stemOp >= 0 || a.mbExpand >= 0 || a.tail >= 0 || a.tailOf >= 0 || a.out != b.in0) continue;
+            if (a.kind != PlanOp::CONV || a.groups != 1 || a.dilation != 1 || a.stemOp >= 0 || a.mbExpand >= 0 || a.tail >= 0 || a.tailOf >= 0 || a.up2 || a.out != b.in0) continue;
             const PlanTensor &x = tensors[static_cast<size_t>(a.in0)];
             const PlanTensor &y = tensors[static_cast<size_t>(a.out)];
             const PlanTensor &z = tensors[static_cast<size_t>(b.out)];
@@ -469,7 +493,7 @@ uint64_t Plan::structureHash() const
     for (const PlanOp &op : ops)
         os << static_cast<int>(op.kind) << ' ' << op.in0 << ' ' << op.in1 << ' ' << op.out << ' ' << (op.dead && op.tailOf < 0) << ' ' << op.layerIndex << ' ' << op.ksize << ' ' << op.stride << ' '
            << op.pad << ' ' << op.dilation << ' ' << op.groups << ' ' << static_cast<int>(op.act) << ' ' << static_cast<int>(op.act2) << ' ' << op.in1Sign << ' ' << (op.src2 != nullptr)
-           << ' ' << op.dstChanOffset << ' ' << op.stemOp << ' ' << op.chainHead << ' ' << op.mbExpand << ' ' << op.tail << ' ' << op.stemTail << ';';
+           << ' ' << op.dstChanOffset << ' ' << op.stemOp << ' ' << op.chainHead << ' ' << op.mbExpand << ' ' << op.tail << ' ' << op.stemTail << ' ' << op.up2 << ';';
     const std::string text = os.str();
     return PackFile::hash(text.data(), text.size());
 }
@@ -606,6 +630,7 @@ static msnh_conv_desc convDesc(const Plan &plan, const PlanOp &op)
     d.out_mul = 1.f / plan.mulOf(op.out);
     d.algo = op.algo;
     d.tile = op.tile;
+    if (op.up2) { d.out_h = out.h / 2; d.out_w = out.w / 2; d.out_upsample = 2; }
     return d;
 }
 
@@ -884,6 +909,7 @@ static std::string tuneSignature(const Plan &plan, const PlanOp &op)
     os << static_cast<int>(op.kind) << ' ' << in.n << ' ' << in.h << ' ' << in.w << ' ' << in.c << ' ' << plan.ld(op.in0) << ' ' << out.c << ' '
        << plan.ld(op.out) << ' ' << op.ksize << ' ' << op.stride << ' ' << op.pad << ' ' << op.dilation << ' ' << op.groups << ' ' << (op.in1 >= 0) << ' '
        << in.dtype << ' ' << out.dtype;
+    if (op.up2) os << " up2";
     if (op.tail >= 0) os << " tail " << plan.tensors[static_cast<size_t>(plan.ops[static_cast<size_t>(op.tail)].out)].c;
     return os.str();
 }
@@ -1050,7 +1076,7 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
     msnh_event_t e0 = nullptr, e1 = nullptr;
     MSNH_DEV(msnh_hip_event_create(&e0));
     MSNH_DEV(msnh_hip_event_create(&e1));
-    struct Key { int kind, b, h, w, c, inLd, oc, outLd, k, st, pad, dil, g, res, odt, algo; bool operator==(const Key &o) const { return std::memcmp(this, &o, sizeof(Key)) == 0; } };
+    struct Key { int kind, b, h, w, c, inLd, oc, outLd, k, st, pad, dil, g, res, odt, algo, up; bool operator==(const Key &o) const { return std::memcmp(this, &o, sizeof(Key)) == 0; } };
     std::vector<std::pair<Key, int>> memo;         // identical shapes share one search
     for (PlanOp &op : ops)
     {
@@ -1062,7 +1088,7 @@ void Plan::tuneConvs(msnh_stream_t s, const std::string &cacheFile)
         key.kind = static_cast<int>(op.kind);
         key.b = in.n; key.h = in.h; key.w = in.w; key.c = in.c; key.inLd = ld(op.in0); key.oc = out.c; key.outLd = ld(op.out);
         key.k = op.ksize; key.st = op.stride; key.pad = op.pad; key.dil = op.dilation; key.g = op.groups;
-        key.res = op.in1 >= 0; key.odt = out.dtype; key.algo = op.algo;
+        key.res = op.in1 >= 0; key.odt = out.dtype; key.algo = op.algo; key.up = op.up2 ? 1 : 0;
         bool found = false;
         for (const auto &m : memo)
         {
@@ -1472,7 +1498,7 @@ std::string Plan::describe() const
         const PlanTensor &out = tensors[static_cast<size_t>(op.out)];
         os << "  L" << op.layerIndex << " " << kinds[op.kind];
         if (op.kind == PlanOp::CONV)
-            os << "[" << algos[op.algo] << (op.stemTail >= 0 ? "+1x1" : "") << (op.tile ? " t" + std::to_string(op.tile) : std::string()) << " k" << op.ksize << " s" << op.stride << " g" << op.groups << (op.in1 >= 0 ? " +res" : "") << (op.src2 ? " +bn" : "") << "]";
+            os << "[" << algos[op.algo] << (op.stemTail >= 0 ? "+1x1" : "") << (op.tile ? " t" + std::to_string(op.tile) : std::string()) << " k" << op.ksize << " s" << op.stride << " g" << op.groups << (op.in1 >= 0 ? " +res" : "") << (op.src2 ? " +bn" : "") << (op.up2 ? " +up2" : "") << "]";
         if (op.kind == PlanOp::MAXPOOL || op.kind == PlanOp::AVGPOOL)
             os << "[k" << op.ksize << " s" << op.stride << " p" << op.pad << (op.chainHead >= 0 ? " in the launch of the pool before it" : "") << "]";
         os << " " << in.n << "x" << in.h << "x" << in.w << "x" << in.c << " -> " << out.h << "x" << out.w << "x" << out.c

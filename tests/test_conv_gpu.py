@@ -576,3 +576,44 @@ def test_conv_tail_rejects():
     # ... and a tile with a tail does not run a plain convolution
     assert L.msnh_hip_conv2d_tile_supported(ctypes.byref(mk()), L.msnh_hip_conv2d_tail_tile_first()) == 0
     assert L.msnh_hip_conv2d_tail(ctypes.byref(mk()), ctypes.byref(tk()), None, None, None, None, None, None, None, None, None, None, None) != 0
+
+
+@pytest.mark.parametrize("dtype", [abi.F16, abi.F32])
+@pytest.mark.parametrize("case", [(2, 64, 19, 19, 40, 1, 1, 0), (1, 32, 13, 11, 64, 3, 1, 1), (3, 128, 10, 10, 128, 1, 1, 0), (1, 64, 38, 38, 256, 3, 2, 1)])
+def test_conv_upsampling_epilogue(case, dtype):
+    """msnh_conv_desc::out_upsample = 2: the convolution writes every result pixel to the 2 x 2 pixels it maps to under nearest-neighbour
+    upsampling (the convolution in front of an UpSampleLayer writes the upsampled tensor itself), on every tile of the implicit GEMM that
+    takes the shape: equal to the oracle's convolution repeated 2 x 2, and bit for bit to the same tile without it followed by the repeat."""
+    import gpuutil as gu
+    L = abi.lib()
+    b, c, h, w, oc, k, stride, pad = case
+    rng = np.random.default_rng(hash(case) % (2 ** 31))
+    x, wt = _case(rng, b, c, h, w, oc, k)
+    scale = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    shift = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    if dtype == abi.F16:
+        x, wt = gu.round_f16(x), gu.round_f16(wt)
+    ref = _ref(x, wt, stride, pad, 1, 1, scale, shift, "leaky", 0.1, None, "none", 1.0, 0.5)
+    ref_up = ref.repeat(2, axis=2).repeat(2, axis=3)
+    ran = 0
+    for tile in range(0, L.msnh_hip_conv2d_tile_count() + 1):
+        kw = dict(dtype=dtype, stride=stride, pad=pad, scale=scale, shift=shift, act="leaky", out_mul=0.5, algo="igemm", tile=tile, in_ld=c + 8, out_ld=oc + 8)
+        try:
+            y, _ = gu.conv2d(x, wt, **kw, upsample=2)
+        except abi.HipError as e:
+            assert "this tile needs" in str(e) or "upsampling epilogue" in str(e), str(e)
+            continue
+        ran += 1
+        assert y.shape == ref_up.shape
+        assert gu.rel_err(y, ref_up) <= TOL[dtype], tile
+        plain, _ = gu.conv2d(x, wt, **kw)
+        assert np.array_equal(y, plain.repeat(2, axis=2).repeat(2, axis=3)), tile
+    assert ran >= 10
+    # not for the other algorithms, not with a residual
+    d = abi.ConvDesc(dtype, dtype, b, h, w, c, c, oc, (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1, oc, k, stride, pad, 1, 1, 22, 0.1, 0, oc, 22, 0.1,
+                     1.0, 1.0, abi.ALGO["direct"], 0, 2)
+    assert L.msnh_hip_conv2d_tile_supported(ctypes.byref(d), 0) == 0
+    d.algo = abi.ALGO["igemm"]
+    assert L.msnh_hip_conv2d_tile_supported(ctypes.byref(d), 0) == 1
+    d.has_residual = 1
+    assert L.msnh_hip_conv2d_tile_supported(ctypes.byref(d), 0) == 0

@@ -638,6 +638,37 @@ def test_conv_with_its_1x1_consumer_as_one_launch():
     assert all(np.array_equal(a, b, equal_nan=True) for a, b in zip(m.run_yolo(x), got))
 
 
+@pytest.mark.parametrize("fp16", [False, True])
+def test_conv_writes_the_upsampled_tensor(fp16):
+    """The 1x1 convolutions in front of the two nearest-neighbour upsample layers of YOLOv3's neck write the upsampled tensors themselves
+    (msnh_conv_desc::out_upsample; Plan::fuse f): no upsample launch is left in the plan, and the head logits equal those of the plan that
+    keeps the upsample launches (MSNH_NO_CONV_UPSAMPLE) -- to 1e-5 in float32, to 5e-3 in float16 (two separately tuned plans may sum in
+    different orders)."""
+    batch, size = 2, 160
+    net, binp, g = nu.model("yolov3", batch, size, seed=7)
+    x = zoo.seeded_input(batch, 3, size, size, seed=8)
+    m = netapi.Net(net, binp, fp16=fp16)
+    detail = m.plan_detail()
+    assert sum("+up2" in ln for ln in detail.splitlines()) == 2, detail
+    assert not any(" upsample" in ln for ln in detail.splitlines()), detail
+    got = m.run_yolo(x)
+    heads = [m.yolo_head_logits(h) for h in range(3)]
+    os.environ["MSNH_NO_CONV_UPSAMPLE"] = "1"
+    try:
+        m0 = netapi.Net(net, binp, fp16=fp16)
+    finally:
+        del os.environ["MSNH_NO_CONV_UPSAMPLE"]
+    d0 = m0.plan_detail()
+    assert "+up2" not in d0 and sum(" upsample" in ln for ln in d0.splitlines()) == 2, d0
+    want = m0.run_yolo(x)
+    for h in range(3):
+        e = nu.rel_err(heads[h], m0.yolo_head_logits(h))
+        print("head", h, "fp16" if fp16 else "fp32", e, flush=True)
+        assert e <= (5e-3 if fp16 else 1e-5), h
+    for a, b in zip(got, want):
+        assert len(b) > 0 and abs(len(a) - len(b)) <= (max(2, len(b) // 100) if fp16 else 0)
+
+
 def test_image_in_boxes_out():
     """8-bit images of different shapes -> device letterbox -> forward -> boxes in original-image pixels: equals the
     float path fed with the restatement's letterbox, followed by the restatement's rescale."""
