@@ -977,6 +977,7 @@ int msnh_hip_connected(int dtype, int batch, int inputs, int outputs, const void
         reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 32 == 0)
     {
         msnh_conv_desc d;
+        std::memset(&d, 0, sizeof(d));
         d.dtype = dtype; d.out_dtype = MSNH_F32;
         d.batch = batch; d.in_h = 1; d.in_w = 1; d.in_c = inputs; d.in_ld = inputs;
         d.out_c = outputs; d.out_h = 1; d.out_w = 1; d.out_ld = outputs;
