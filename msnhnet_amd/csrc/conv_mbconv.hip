@@ -156,17 +156,19 @@ __global__ __launch_bounds__(64 * MB_NW) void mbconvKernel(MbArgs a)
     dmaWait<0>();
     __syncthreads();
 
-    for (int c = 0; c < a.chunks; ++c)
-    {
-        const unsigned cur = bOff + static_cast<unsigned>(c & 1) * a.chunkBytes;
-        if (c + 1 < a.chunks) issueBlob(c + 1, bOff + static_cast<unsigned>((c + 1) & 1) * a.chunkBytes);
-        const unsigned char *rec = smem + cur;
+    // Per chunk of 64 widened channels: expand (matrix cores, all wavefronts) | barrier | depthwise (vector ALU) | barrier | project (matrix
+    // cores, the first 2 mb wavefronts) together with the expand of the NEXT chunk, which touches neither the depthwise output the projection
+    // reads nor anything the projection writes: two workgroup barriers per chunk, and the wavefronts without a projection block start the next
+    // expand at once (its items are dealt from the last wavefront down).  The record of chunk c + 1 is asked for behind the first barrier of
+    // chunk c -- its buffer held chunk c - 1, whose last reader, the projection, every wavefront has left by then -- and is complete at the
+    // second one.
+    const auto expandChunk = [&](int c) {
+        const unsigned char *rec = smem + bOff + static_cast<unsigned>(c & 1) * a.chunkBytes;
         const float *aff = reinterpret_cast<const float *>(rec + mbAffOff(a.ks, a.mb));
-
         const int left = a.cexp - c * MB_CH;          // widened channels from this chunk on: a last chunk may be partial
         // ---- 1. expand (a 32-channel block past exp_c is skipped) ---------------------------------------------------------------------
         const int nmb = left > 32 ? 2 : 1;
-        for (int it = wave; it < nmb * NE; it += MB_NW)
+        for (int it = MB_NW - 1 - wave; it < nmb * NE; it += MB_NW)
         {
             const int mblk = nmb == 2 ? (it & 1) : 0, j = nmb == 2 ? (it >> 1) : it;
             f32x16 acc;
@@ -205,7 +207,16 @@ __global__ __launch_bounds__(64 * MB_NW) void mbconvKernel(MbArgs a)
             *reinterpret_cast<f16x8 *>(ep) = o0;
             *reinterpret_cast<f16x8 *>(ep + 16) = o1;
         }
+    };
+    expandChunk(0);
+    for (int c = 0; c < a.chunks; ++c)
+    {
+        const unsigned cur = bOff + static_cast<unsigned>(c & 1) * a.chunkBytes;
+        const unsigned char *rec = smem + cur;
+        const float *aff = reinterpret_cast<const float *>(rec + mbAffOff(a.ks, a.mb));
+        const int left = a.cexp - c * MB_CH;
         __syncthreads();
+        if (c + 1 < a.chunks) issueBlob(c + 1, bOff + static_cast<unsigned>((c + 1) & 1) * a.chunkBytes);
 
         // ---- 2. depthwise (the threads share out the channel vectors that exist) ---------------------------------------------------------
         {
@@ -243,6 +254,7 @@ __global__ __launch_bounds__(64 * MB_NW) void mbconvKernel(MbArgs a)
                 *reinterpret_cast<f16x8 *>(smem + yOff + p * MB_ROW + v8 * 16) = o;
             }
         }
+        dmaWait<0>();
         __syncthreads();
 
         // ---- 3. project --------------------------------------------------------------------------------------------------------
@@ -255,8 +267,7 @@ __global__ __launch_bounds__(64 * MB_NW) void mbconvKernel(MbArgs a)
             for (int s = 0; s < MB_CH / 16; ++s)
                 mfmaBlock(*reinterpret_cast<const f16x8 *>(ap + s * 1024), *reinterpret_cast<const f16x8 *>(bp + s * 32), accP);
         }
-        dmaWait<0>();
-        __syncthreads();
+        if (c + 1 < a.chunks) expandChunk(c + 1);
     }
 
     // ---- epilogue: affine, activation, residual, second activation, scale; two 16-byte stores per lane ------------------------------
