@@ -144,6 +144,12 @@ typedef struct msnh_conv_desc
                            result pixel is written to the 2 x 2 pixels it maps to under nearest-neighbour upsampling, y is
                            [batch][2 out_h][2 out_w] -- the convolution in front of an UpSampleLayer (src/layers/MsnhUpSampleLayer.cpp:96-118,
                            Blas::cpuUpSample with stride 2 and scale 1) writes the upsampled tensor itself */
+    int   xcd_blocks;   /* IGEMM algorithms, ungrouped and unsplit: how the tiles of the launch are dealt to the 8 XCDs (each has an L2 of its
+                           own).  1: an XCD takes a run of pixel tiles with all their channel tiles (every input pixel is fetched into
+                           one L2, every filter into all eight).  2, 4, 8: the XCDs form a g x (8 / g) grid over (channel tiles, pixel
+                           tiles) and each fetches only its share of the filters and of the input.  0: the library takes the arrangement
+                           that fetches the fewest bytes (MSNH_NO_XCD_BLOCKS=1 in the environment: always 1).  Same result bits either
+                           way; no counterpart in the reference */
 } msnh_conv_desc;
 
 /* Number of tile configurations of the IGEMM algorithm; any of them computes the same result, they differ in

@@ -308,6 +308,7 @@ static int validate(const msnh_conv_desc *d)
     MSNH_REQUIRE(oh == d->out_h && ow == d->out_w, "conv: out size %dx%d does not match geometry (%dx%d)", d->out_h, d->out_w, oh, ow);
     MSNH_REQUIRE(d->out_ld >= d->out_c, "conv: out_ld < out_c");
     MSNH_REQUIRE(d->out_upsample >= 0 && d->out_upsample <= 2, "conv: out_upsample is 0, 1 or 2");
+    MSNH_REQUIRE(d->xcd_blocks == 0 || d->xcd_blocks == 1 || d->xcd_blocks == 2 || d->xcd_blocks == 4 || d->xcd_blocks == 8, "conv: xcd_blocks is 0, 1, 2, 4 or 8");
     MSNH_REQUIRE(d->out_upsample != 2 || ((d->algo == MSNH_CONV_IGEMM || d->algo == MSNH_CONV_AUTO) && !d->has_residual && d->out_c % 8 == 0 && d->out_ld % 8 == 0 &&
                                          d->groups == 1 && static_cast<long long>(d->batch) * d->out_h * d->out_w * 4 * d->out_ld * 4 < 0x7fffffffLL),
                  "conv: the upsampling epilogue belongs to the IGEMM algorithm, without residual, channel counts multiples of 8");

@@ -42,6 +42,7 @@ static int convIgemmAny(const msnh_conv_desc *d, const void *x, const void *w, c
     a.taps = d->ksize * d->ksize; a.ksize = d->ksize; a.stride = d->stride; a.pad = d->pad; a.dil = d->dilation;
     a.P = d->batch * d->out_h * d->out_w;
     a.up2 = d->out_upsample == 2 ? 1 : 0;
+    a.xcdGm = d->xcd_blocks;
     a.yBytes = a.up2 ? static_cast<unsigned>(static_cast<unsigned long long>(d->batch) * d->out_h * d->out_w * 4ull * d->out_ld * dtypeSize(d->out_dtype)) : 0u;
     a.byOW = makeFastDiv(static_cast<unsigned>(d->out_w));
     a.byOH = makeFastDiv(static_cast<unsigned>(d->out_h));

@@ -17,6 +17,7 @@
 #pragma once
 #include "common.hpp"
 #include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 
 namespace msnh {
@@ -49,6 +50,8 @@ struct IgemmArgs
     int act, act2, hasRes, vecOk;
     float actParam, act2Param, resMul, outMul;
     FastDiv byOW, byOH;     // pixel index -> (image, row, column) without hardware-less integer division
+    int xcdGm;              // > 1: the XCDs form an xcdGm x (8 / xcdGm) grid over (channel tiles, pixel tiles), see igemmTileOf
+    int xcdMPer, xcdPPer;   // channel tiles / pixel tiles per XCD in that arrangement
     int up2;                // every result pixel goes to the 2 x 2 pixels of y it maps to under nearest-neighbour upsampling (y: [batch][2 OH][2 OW])
     unsigned yBytes;        // up2: extent of y in bytes
     // tail (tiles with TAIL = 1 only): a 1x1 stride-1 convolution z = zMul * act3(scale2 * (W2 . y) + shift2) of this convolution's
@@ -61,6 +64,57 @@ struct IgemmArgs
     float act3Param, zMul;
     unsigned w2Bytes;
 };
+
+// Workgroup -> tile.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2: id % 8 selects
+// the XCD, id / 8 the position inside it.  Default arrangement (xcdGm <= 1): an XCD takes a contiguous run of tiles with the
+// channel tiles of one pixel tile back to back, so an input pixel is fetched into one L2 once instead of once per channel
+// tile and XCD -- and every XCD fetches every filter.  Where the filters outweigh the input (512 -> 1024 channels over
+// 19 x 19 pixels: 9.4 MB against 3 MB) the host asks for an xcdGm x (8 / xcdGm) arrangement instead: an XCD owns a block of
+// channel tiles and a block of pixel tiles and fetches only that share of the filters and that share of the input.
+__device__ __forceinline__ bool igemmTileOf(const IgemmArgs &a, int nTilesP, int &mTile, int &pTile)
+{
+    const int xcd = blockIdx.x % 8, idx = blockIdx.x / 8;
+    if (a.xcdGm <= 1)
+    {
+        const int total   = a.mTiles * nTilesP;
+        const int perXcd  = (total + 7) / 8;
+        const int logical = xcd * perXcd + idx;
+        mTile = logical % a.mTiles;
+        pTile = logical / a.mTiles;
+        return logical < total;                       // padding ids of the last round
+    }
+    const int lp = idx / a.xcdMPer;
+    mTile = (xcd % a.xcdGm) * a.xcdMPer + (idx - lp * a.xcdMPer);
+    pTile = (xcd / a.xcdGm) * a.xcdPPer + lp;
+    return lp < a.xcdPPer && mTile < a.mTiles && pTile < nTilesP;
+}
+
+// grid.x of a launch over a.mTiles x nTilesP tiles, and the XCD arrangement it runs under (see igemmTileOf).  a.xcdGm comes in as
+// the caller's wish (msnh_conv_desc::xcd_blocks): 1, 2, 4, 8 are taken as they are; 0 picks the arrangement that makes the eight
+// L2s fetch the fewest bytes, counted as (8 / g) x filters + g x input -- the default one stays unless another saves a quarter
+// of that without more workgroup slots per XCD.  Grouped and split-K launches (plainGrid false) keep the default.
+inline unsigned igemmGridX(IgemmArgs &a, int nTilesP, size_t es, bool plainGrid)
+{
+    static const bool off = std::getenv("MSNH_NO_XCD_BLOCKS") != nullptr;      // (for A/B timing of whole networks)
+    const int wish = a.xcdGm;
+    const int tiles = a.mTiles * nTilesP;
+    const unsigned plain = static_cast<unsigned>((tiles + 7) / 8 * 8);
+    a.xcdGm = 1; a.xcdMPer = a.mTiles; a.xcdPPer = nTilesP;
+    if (!plainGrid || wish == 1 || (wish == 0 && off)) return plain;
+    const double wB = static_cast<double>(a.coutG) * a.taps * a.cinG * es;
+    const double xB = static_cast<double>(a.batch) * a.H * a.W * a.cinG * es;
+    double best = 8 * wB + xB;
+    const double need = 0.75 * best;
+    unsigned grid = plain;
+    for (int gm = 2; gm <= 8; gm *= 2)
+    {
+        const int gp = 8 / gm, mPer = (a.mTiles + gm - 1) / gm, pPer = (nTilesP + gp - 1) / gp;
+        const double cost = gp * wB + gm * xB;
+        const bool take = wish == gm || (wish == 0 && 8 * mPer * pPer <= static_cast<int>(plain) && cost < need && cost < best);
+        if (take) { best = cost; a.xcdGm = gm; a.xcdMPer = mPer; a.xcdPPer = pPer; grid = 8u * mPer * pPer; }
+    }
+    return grid;
+}
 
 template <typename T> struct Frag;
 template <> struct Frag<f16>   { typedef f16x8 V; static constexpr int VEC = 8; };
@@ -759,17 +813,10 @@ void convIgemmKernel(IgemmArgs a)
     const int wm   = (wave % NWT) / WN;
     const int wn   = (wave % NWT) % WN;
     const int g    = blockIdx.z;
-    // Workgroup -> tile mapping.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its own
-    // L2.  Ids are therefore first regrouped per XCD (id % 8 selects the XCD, id / 8 the position inside it), and
-    // inside an XCD the channel tiles of one pixel tile run back to back, so an input pixel is fetched into one L2
-    // once instead of once per channel tile and XCD.
-    const int nTilesP = (a.P + BN - 1) / BN;
-    const int total   = a.mTiles * nTilesP;
-    const int perXcd  = (total + 7) / 8;
-    const int logical = (blockIdx.x % 8) * perXcd + blockIdx.x / 8;
-    if (logical >= total) return;                     // padding ids of the last round
-    const int m0   = (logical % a.mTiles) * BM;
-    const int p0   = (logical / a.mTiles) * BN;
+    int mTile, pTile;
+    if (!igemmTileOf(a, (a.P + BN - 1) / BN, mTile, pTile)) return;
+    const int m0   = mTile * BM;
+    const int p0   = pTile * BN;
 
     const unsigned gx = static_cast<unsigned>(g) * a.cinG * ES;
     const unsigned gw = static_cast<unsigned>(g) * a.coutG * a.taps * a.cinG * ES;
@@ -1083,7 +1130,7 @@ inline int launchIgemm(IgemmArgs &a, int groups, hipStream_t st)
         }
         a.splitK = want;
     }
-    dim3 grid((tiles + 7) / 8 * 8, a.splitK, groups);
+    dim3 grid(igemmGridX(a, (a.P + BN - 1) / BN, sizeof(T), a.splitK == 1 && groups == 1), a.splitK, groups);
     if (a.dryRun) return 0;
     auto kern = convIgemmKernel<T, TOut, BM, BN, KV, WM, WN, NS, KG, TAIL>;
     if (smem > 48 * 1024)

@@ -56,13 +56,10 @@ void convPatch3x3Kernel(IgemmArgs a)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm   = wave / WN;
     const int wn   = wave % WN;
-    const int nTilesP = (a.P + BN - 1) / BN;
-    const int total   = a.mTiles * nTilesP;
-    const int perXcd  = (total + 7) / 8;
-    const int logical = (blockIdx.x % 8) * perXcd + blockIdx.x / 8;
-    if (logical >= total) return;
-    const int m0 = (logical % a.mTiles) * BM;
-    const int p0 = (logical / a.mTiles) * BN;
+    int mTile, pTile;
+    if (!igemmTileOf(a, (a.P + BN - 1) / BN, mTile, pTile)) return;
+    const int m0 = mTile * BM;
+    const int p0 = pTile * BN;
 
     const i32x4 rx = makeRsrcWords(a.x, a.xBytes);
     const i32x4 rw = makeRsrcWords(a.w, a.wBytes);
@@ -278,8 +275,7 @@ inline int launchPatch(IgemmArgs &a, int groups, hipStream_t st)
     a.ragged  = (a.cinG % BK) != 0;
     a.mTiles  = (a.coutG + BM - 1) / BM;
     a.splitK  = 1;
-    const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
-    dim3 grid((tiles + 7) / 8 * 8, 1, 1);
+    dim3 grid(igemmGridX(a, (a.P + BN - 1) / BN, sizeof(T), true), 1, 1);
     auto kern = convPatch3x3Kernel<T, TOut, BM, BN, KV, WM, WN, PS>;
     if (smem > 48 * 1024)
     {

@@ -73,13 +73,10 @@ void convPatch8Kernel(IgemmArgs a)
     const int kg   = wave / NWT;                      // which k-blocks of a tap step this wavefront multiplies
     const int wm   = (wave % NWT) / WN;
     const int wn   = (wave % NWT) % WN;
-    const int nTilesP = (a.P + BN - 1) / BN;
-    const int total   = a.mTiles * nTilesP;
-    const int perXcd  = (total + 7) / 8;
-    const int logical = (blockIdx.x % 8) * perXcd + blockIdx.x / 8;
-    if (logical >= total) return;
-    const int m0 = (logical % a.mTiles) * BM;
-    const int p0 = (logical / a.mTiles) * BN;
+    int mTile, pTile;
+    if (!igemmTileOf(a, (a.P + BN - 1) / BN, mTile, pTile)) return;
+    const int m0 = mTile * BM;
+    const int p0 = pTile * BN;
 
     const i32x4 rx = makeRsrcWords(a.x, a.xBytes);
     const i32x4 rw = makeRsrcWords(a.w, a.wBytes);
@@ -295,7 +292,7 @@ void convPatch8Kernel(IgemmArgs a)
     if constexpr (DBG & 64)
     {
         const unsigned long long t1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
-        if (logical == 0 && tid == 0)
+        if (mTile == 0 && pTile == 0 && tid == 0)
         {
             reinterpret_cast<unsigned long long *>(a.ws)[0] = t1 - dbgT0;
             reinterpret_cast<unsigned long long *>(a.ws)[1] = r1 - dbgR0;
@@ -355,8 +352,7 @@ inline int launchPatch8(IgemmArgs &a, int groups, hipStream_t st)
     a.ragged  = (a.cinG % BK) != 0;
     a.mTiles  = (a.coutG + BM - 1) / BM;
     a.splitK  = 1;
-    const int tiles = a.mTiles * ((a.P + BN - 1) / BN);
-    dim3 grid((tiles + 7) / 8 * 8, 1, 1);
+    dim3 grid(igemmGridX(a, (a.P + BN - 1) / BN, sizeof(T), true), 1, 1);
     auto kern = convPatch8Kernel<T, TOut, BM, BN, WM, WN, NSA, PS, DBG, KG>;
     if (smem > 48 * 1024)
     {

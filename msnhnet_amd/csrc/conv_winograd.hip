@@ -188,6 +188,7 @@ void winogradGemmDesc(const msnh_conv_desc *d, msnh_conv_desc *gd)
     gd->act = MSNH_ACT_NONE; gd->act_param = 0.f; gd->has_residual = 0; gd->res_ld = 16 * g.OC; gd->act2 = MSNH_ACT_NONE; gd->act2_param = 0.f;
     gd->res_mul = 1.f; gd->out_mul = 1.f; gd->algo = MSNH_CONV_IGEMM; gd->tile = d->tile;
     gd->out_upsample = 0;
+    gd->xcd_blocks = 0;
 }
 
 size_t winogradWorkspaceBytes(const msnh_conv_desc *d)

@@ -21,7 +21,7 @@ class ConvDesc(ctypes.Structure):
                 ("ksize", ctypes.c_int), ("stride", ctypes.c_int), ("pad", ctypes.c_int), ("dilation", ctypes.c_int), ("groups", ctypes.c_int),
                 ("act", ctypes.c_int), ("act_param", ctypes.c_float),
                 ("has_residual", ctypes.c_int), ("res_ld", ctypes.c_int), ("act2", ctypes.c_int), ("act2_param", ctypes.c_float),
-                ("res_mul", ctypes.c_float), ("out_mul", ctypes.c_float), ("algo", ctypes.c_int), ("tile", ctypes.c_int), ("out_upsample", ctypes.c_int)]
+                ("res_mul", ctypes.c_float), ("out_mul", ctypes.c_float), ("algo", ctypes.c_int), ("tile", ctypes.c_int), ("out_upsample", ctypes.c_int), ("xcd_blocks", ctypes.c_int)]
 
 
 class ConvTailDesc(ctypes.Structure):

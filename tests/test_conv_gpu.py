@@ -144,6 +144,45 @@ def test_conv_multi_wavefront_tiles(k, stride, dtype):
 
 
 @pytest.mark.parametrize("dtype", [abi.F32, abi.F16])
+@pytest.mark.parametrize("k,stride", [(3, 1), (3, 2), (1, 1)])
+def test_conv_xcd_arrangements(k, stride, dtype):
+    """msnh_conv_desc::xcd_blocks only changes which workgroup computes which tile: every arrangement gives the bits of the default
+    one, for every tile configuration that takes the shape.  328 output channels and 3 x 23 x 21 pixels make channel-tile and
+    pixel-tile counts that the 2 x 4, 4 x 2 and 8 x 1 grids of XCDs do not divide (XCDs with fewer tiles, ids past the last tile);
+    the default arrangement is checked against the oracle, and so is the library's own choice (xcd_blocks = 0)."""
+    import gpuutil as gu
+    gu.init()
+    rng = np.random.default_rng(300 + 10 * k + stride)
+    b, c, h, w, oc = 3, 64, 23, 21, 328
+    x, wt = _case(rng, b, c, h, w, oc, k)
+    pad = k // 2
+    oh, ow = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
+    res = rng.standard_normal((b, oc, oh, ow), dtype=np.float32)
+    scale = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+    shift = (rng.standard_normal(oc) * 0.1).astype(np.float32)
+    if dtype == abi.F16:
+        x, wt, res = gu.round_f16(x), gu.round_f16(wt), gu.round_f16(res)
+    ref = _ref(x, wt, stride, pad, 1, 1, scale, shift, "leaky", 0.1, res, "none", 1.0, 1.0)
+    kw = dict(dtype=dtype, stride=stride, pad=pad, scale=scale, shift=shift, act="leaky", residual=res, algo="igemm")
+    ran = 0
+    for tile in range(1, abi.lib().msnh_hip_conv2d_tile_count() + 1):
+        print("xcd arrangements, tile", tile, k, stride, dtype, flush=True)
+        try:
+            y1, _ = gu.conv2d(x, wt, tile=tile, xcd_blocks=1, **kw)
+        except abi.HipError as e:
+            assert "this tile" in str(e)
+            continue
+        ran += 1
+        assert gu.rel_err(y1, ref) <= TOL[dtype], tile
+        for g in (0, 2, 4, 8):
+            yg, _ = gu.conv2d(x, wt, tile=tile, xcd_blocks=g, **kw)
+            assert np.array_equal(yg, y1), (tile, g)
+    assert ran >= 8
+    with pytest.raises(abi.HipError, match="xcd_blocks"):
+        gu.conv2d(x, wt, tile=1, xcd_blocks=3, **kw)
+
+
+@pytest.mark.parametrize("dtype", [abi.F32, abi.F16])
 @pytest.mark.parametrize("shape", [(2, 16, 19, 19, 40), (1, 64, 38, 38, 96), (3, 8, 7, 5, 16), (1, 32, 76, 76, 64), (2, 72, 13, 11, 136)])
 def test_conv_patch_tiles(shape, dtype):
     """3x3 stride-1 layers with the input patch resident in LDS: image borders, batch seams, ragged channel chunks"""
