@@ -1161,8 +1161,8 @@ namespace msnh {
 // Tile configurations (BM x BN output tile, KV 16-byte vectors of K per step, WM x WN wavefront grid).
 // Index 0 is "choose for me"; the others can be forced through msnh_conv_desc::tile, which is how the host
 // library's per-layer search picks the fastest one at load time.
-constexpr int kIgemmTiles = 64;
-constexpr int kIgemmTailTileFirst = 63;         // tiles from here on carry a tail (msnh_hip_conv2d_tail)
+constexpr int kIgemmTiles = 65;
+constexpr int kIgemmTailTileFirst = 64;         // tiles from here on carry a tail (msnh_hip_conv2d_tail)
 
 template <typename T, typename TOut>
 int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
@@ -1248,13 +1248,17 @@ int igemmDispatch(IgemmArgs &a, int groups, int tile, hipStream_t st)
     case 60: return launchIgemm<T, TOut, 128, 64, 8, 2, 1, 4, 2>(a, groups, st);
     case 61: return launchIgemm<T, TOut, 64, 256, 8, 1, 4, 3, 2>(a, groups, st);
     case 62: return launchIgemm<T, TOut, 64, 384, 8, 1, 6, 2, 2>(a, groups, st);
+    // the LDS-patch kernel over 256 channels x 192 pixels with twelve wavefronts: one round of tiles for the 76x76 128 -> 256 layers at batch 8
+    // like tile 37, with a third fewer bytes delivered to LDS per tap step.  It fits the LDS with two weight stages only, the weight
+    // tile of step it + 2 asked for behind the barrier of step it (see LATE in conv_patch8.hpp)
+    case 63: return launchPatch8<T, TOut, 256, 192, 4, 3, 2, 1>(a, groups, st);
     // tiles whose epilogue also computes the 1x1 convolution that follows (msnh_hip_conv2d_tail only; float16): the tile holds every
     // output channel of the first convolution (at most 256 / 128)
-    case 63:
     case 64:
+    case 65:
         if constexpr (std::is_same<T, f16>::value && std::is_same<TOut, f16>::value)
         {
-            if (tile == 63) return launchIgemm<T, TOut, 256, 192, 8, 4, 3, 2, 1, 1>(a, groups, st);
+            if (tile == 64) return launchIgemm<T, TOut, 256, 192, 8, 4, 3, 2, 1, 1>(a, groups, st);
             return launchIgemm<T, TOut, 128, 192, 8, 4, 3, 2, 1, 1>(a, groups, st);
         }
         else

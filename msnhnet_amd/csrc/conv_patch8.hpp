@@ -14,7 +14,7 @@
 // LDS: NSA weight stages of BM x 128 B | patch of the current chunk | patch of the next chunk | 1 KiB of zeros.
 // Data movement as in conv_igemm.hpp: 16-byte-per-lane buffer loads straight into LDS, XOR-swizzled unpadded rows, explicit
 // vmcnt waits, one barrier per tap step.  The patch of chunk c+1 arrives in 1 KiB slices (8 pixels x 128 B, one wave
-// instruction each), PS per wavefront and tap step over the first 11 - NSA taps of chunk c; every tap step issues the same number
+// instruction each), PS per wavefront and tap step over the first 11 - NSA taps of chunk c (8 with two weight stages); every tap step issues the same number
 // of loads per wavefront (slices that do not exist go, out of range and therefore as zeros, into the zero area), so the count
 // of loads in flight at each barrier is a compile-time constant.
 #pragma once
@@ -54,10 +54,11 @@ void convPatch8Kernel(IgemmArgs a)
     constexpr int ROWB  = KV * 16;
     constexpr unsigned A_STAGE = BM * ROWB;           // the wavefronts whose rows of the last pass lie past BM aim at the zero area
     static_assert(BM % 8 == 0, "a wavefront's load covers eight weight rows");
-    constexpr int PSTEPS = 11 - NSA;                  // tap steps of a chunk that bring in slices of the next chunk's patch
+    constexpr bool LATE = NSA == 2;                   // two weight stages: the tile of step it + 2 is asked for behind the barrier of step it, into the stage that barrier frees
+    constexpr int PSTEPS = LATE ? 8 : 11 - NSA;       // tap steps of a chunk that bring in slices of the next chunk's patch
     static_assert(TM % 32 == 0 && TN % 32 == 0 && (NW == 4 || NW == 8 || NW == 12), "tile shape");
     static_assert(KG == 1 || (KG == 2 && TM == 64 && TN == 64), "the K-split variant works on 64 x 64 wave tiles");
-    static_assert(NSA >= 3 && NSA <= 5, "weight stages");
+    static_assert(NSA >= 2 && NSA <= 5, "weight stages");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smemRaw[];
     const unsigned ldsBase = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char *)smemRaw));
@@ -192,7 +193,12 @@ void convPatch8Kernel(IgemmArgs a)
     // At the barrier of step `it` the weight tile of step it+1 must have landed: it was issued during step it+2-NSA, and the
     // loads of the NSA-2 steps since then may still be in flight.  Patch slices are issued during taps 0 .. PSTEPS-1 = 10-NSA and
     // are needed from the barrier of tap 8 on, NSA-2 steps later: covered by the same count.
-    constexpr int INFLIGHT = (NSA - 2) * NL;
+    // Two stages (LATE): the weight tile of step it+2 goes into the stage of step `it` itself, which is free once the barrier of
+    // step `it` is passed (the fragments of its last k-block are in registers by then): its loads follow that barrier, among the
+    // MFMAs of the last k-block, and have until the next barrier to land; the patch slices of a step are issued ahead of its barrier
+    // and may still be in flight there (the slices of taps 0 .. 7 are older than the weight tile that the barrier of tap 8 waits for).
+    constexpr int INFLIGHT = LATE ? PS : (NSA - 2) * NL;
+    constexpr int AHEADA = LATE ? 2 : NSA - 1;        // the weight loads issued during step `it` belong to step it + AHEADA
 
     // ---- prologue: whole patch of chunk 0, weight tiles of steps 0 .. NSA-2 -----------------------------------------------------
     if constexpr (!(DBG & 32))
@@ -203,7 +209,7 @@ void convPatch8Kernel(IgemmArgs a)
         sA = (static_cast<unsigned>(tapL) * a.cinG + chunkL * BK) * ES;
         cutA = stepIndex >= a.nIter || (a.ragged && (chunkL * BK + ldVec * VEC >= a.cinG));
     };
-    staticFor<0, NSA - 1>([&](auto stTag) {
+    staticFor<0, AHEADA>([&](auto stTag) {
         constexpr int st = decltype(stTag)::value;
         unsigned sA; bool cutA;
         advanceA(sA, cutA, st);
@@ -228,7 +234,7 @@ void convPatch8Kernel(IgemmArgs a)
             const unsigned tapRowN = static_cast<unsigned>((tapN / 3) * W + tapN % 3);
             const unsigned nextP = tap == 8 ? othP : curP;
             unsigned sA; bool cutA;
-            advanceA(sA, cutA, it + NSA - 1);         // the weight tile of step it + NSA - 1
+            advanceA(sA, cutA, it + AHEADA);          // the weight tile of step it + AHEADA
 
             if constexpr (!(DBG & 2))
             {
@@ -263,7 +269,7 @@ void convPatch8Kernel(IgemmArgs a)
                 }
                 if constexpr (!(DBG & 8)) mfmaBlock(fa[ks % 2][(gi % PER) / NB], fb[ks % 2][(gi % PER) % NB], acc[(gi % PER) / NB][(gi % PER) % NB]);
                 else asm volatile("" : "+v"(fa[ks % 2][(gi % PER) / NB]), "+v"(fb[ks % 2][(gi % PER) % NB]));
-                if constexpr (gi < LSPAN && !(DBG & 1))
+                if constexpr (!LATE && gi < LSPAN && !(DBG & 1))
                 {
                     // loads l with l * LSPAN / NL == gi: patch slices first, then the weight rows
                     constexpr int first = (gi * NL + LSPAN - 1) / LSPAN;
@@ -275,6 +281,26 @@ void convPatch8Kernel(IgemmArgs a)
                         else
                             issueA(std::integral_constant<int, l - PS>(), sA, cutA, nnA);
                     });
+                }
+                if constexpr (LATE && !(DBG & 1))
+                {
+                    if constexpr (gi < LSPAN)
+                    {
+                        // patch slices l with l * LSPAN / PS == gi, ahead of the barrier
+                        constexpr int first = (gi * PS + LSPAN - 1) / LSPAN;
+                        constexpr int last  = ((gi + 1) * PS + LSPAN - 1) / LSPAN;
+                        staticFor<first, last>([&](auto lTag) {
+                            constexpr int l = decltype(lTag)::value;
+                            issuePatch(tap < PSTEPS ? tap * PS + l : (1 << 20), chunk + 1, othP);
+                        });
+                    }
+                    else
+                    {
+                        // weight rows l with l * PER / AL == gi - LSPAN, behind the barrier, into the stage it has freed
+                        constexpr int first = ((gi - LSPAN) * AL + PER - 1) / PER;
+                        constexpr int last  = ((gi - LSPAN + 1) * AL + PER - 1) / PER;
+                        staticFor<first, last>([&](auto lTag) { issueA(lTag, sA, cutA, curA); });
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
@@ -329,8 +355,8 @@ inline bool patch8Fits(const IgemmArgs &a, size_t *smemOut, int *slicesOut)
     const size_t smem = loop > epi ? loop : epi;
     if (smemOut) *smemOut = smem;
     if (slicesOut) *slicesOut = slices;
-    // the first 11 - NSA taps of a chunk bring in the next patch: (11 - NSA) * PS slices per wavefront
-    return a.patchOk && a.buffersOk && smem <= 160 * 1024 && (stages == 1 || slices <= (11 - NSA) * NW * PS);
+    // the first 11 - NSA taps of a chunk (8 with two weight stages) bring in the next patch, PS slices per wavefront and tap
+    return a.patchOk && a.buffersOk && smem <= 160 * 1024 && (stages == 1 || slices <= (NSA == 2 ? 8 : 11 - NSA) * NW * PS);
 }
 
 template <typename T, typename TOut, int BM, int BN, int WM, int WN, int NSA, int PS, int DBG = 0, int KG = 1>
