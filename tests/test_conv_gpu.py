@@ -183,9 +183,10 @@ def test_conv_xcd_arrangements(k, stride, dtype):
 
 
 @pytest.mark.parametrize("dtype", [abi.F32, abi.F16])
-@pytest.mark.parametrize("shape", [(2, 16, 19, 19, 40), (1, 64, 38, 38, 96), (3, 8, 7, 5, 16), (1, 32, 76, 76, 64), (2, 72, 13, 11, 136)])
+@pytest.mark.parametrize("shape", [(2, 16, 19, 19, 40), (1, 64, 38, 38, 96), (3, 8, 7, 5, 16), (1, 32, 76, 76, 64), (2, 72, 13, 11, 136), (1, 200, 20, 20, 264)])
 def test_conv_patch_tiles(shape, dtype):
-    """3x3 stride-1 layers with the input patch resident in LDS: image borders, batch seams, ragged channel chunks"""
+    """3x3 stride-1 layers with the input patch resident in LDS: image borders, batch seams, ragged channel chunks; the last shape runs
+    four channel chunks (both patch stages in turn, the last chunk ragged) over two channel tiles"""
     import ctypes
     import gpuutil as gu
     gu.init()
